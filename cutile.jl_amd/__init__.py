@@ -1,0 +1,274 @@
+"""Host side of libmi355tile: hand-written gfx950 (MI355X) HIP kernels behind a C ABI that
+stand in for the kernels cuTile.jl's examples compile through Tile IR.
+
+The directory name contains a dot, so the package is imported under the module name
+``cutile_jl_amd`` (see ``__graft_entry__.load_package``).  Nothing here computes on the
+CPU: every kernel wrapper calls the shared library and raises if it is missing.
+
+Array convention.  The reference's arrays are Julia column-major arrays.  A Julia array of
+shape ``(d1, d2, ..., dn)`` is held here as a ``torch`` tensor of shape ``(dn, ..., d2, d1)``
+in row-major order, which is the same memory.  :func:`TileArray` turns such a tensor (or a
+strided view of one) into the descriptor the C ABI takes, with sizes and strides listed in
+the Julia order, mirroring ``ct.TileArray(arr)`` (reference: src/language/types.jl:350-357).
+"""
+from __future__ import annotations
+
+import ctypes
+import os
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "libmi355tile.so")
+
+MI_F32, MI_F64, MI_F16, MI_BF16, MI_F8E4M3FN, MI_I32, MI_I64 = range(7)
+MI_MAX_RANK = 4
+
+# error codes of include/mi355tile.h
+MI_OK = 0
+MI_E_NULL, MI_E_DTYPE, MI_E_RANK, MI_E_SHAPE, MI_E_STRIDE = -1, -2, -3, -4, -5
+MI_E_TILE, MI_E_GRID, MI_E_ALIGN, MI_E_ARG, MI_E_UNSUPPORTED = -6, -7, -8, -9, -10
+
+
+class MiTileArray(ctypes.Structure):
+    """ctypes mirror of ``mi_tile_array`` (include/mi355tile.h)."""
+
+    _fields_ = [
+        ("ptr", ctypes.c_void_p),
+        ("dtype", ctypes.c_int32),
+        ("ndim", ctypes.c_int32),
+        ("sizes", ctypes.c_int64 * MI_MAX_RANK),
+        ("strides", ctypes.c_int64 * MI_MAX_RANK),
+    ]
+
+
+class MiError(RuntimeError):
+    """A libmi355tile entry point returned a non-zero status."""
+
+    def __init__(self, fn: str, code: int, msg: str):
+        super().__init__(f"{fn} failed with status {code}: {msg}")
+        self.code = code
+
+
+_A = ctypes.POINTER(MiTileArray)
+_i = ctypes.c_int
+_vp = ctypes.c_void_p
+_SIGNATURES = {
+    "mi_version": ([], ctypes.c_int),
+    "mi_strerror": ([_i], ctypes.c_char_p),
+    "mi_last_variant": ([], ctypes.c_char_p),
+    "mi_vec_add_kernel_1d": ([_A, _A, _A, _i, _vp], _i),
+    "mi_vec_add_kernel_2d": ([_A, _A, _A, _i, _i, _vp], _i),
+    "mi_vec_add_kernel_1d_gather": ([_A, _A, _A, _i, _vp], _i),
+    "mi_transpose_kernel": ([_A, _A, _i, _i, _vp], _i),
+    "mi_matmul_kernel": ([_A, _A, _A, _i, _i, _i, _vp], _i),
+    "mi_batch_matmul_kernel": ([_A, _A, _A, _i, _i, _i, _vp], _i),
+    "mi_swizzle_2d": ([ctypes.c_int32] * 6 + [ctypes.POINTER(ctypes.c_int32)] * 2, None),
+    "mi_layer_norm_fwd": ([_A, _A, _A, _A, _A, _A, ctypes.c_float, _i, _vp], _i),
+    "mi_layer_norm_bwd_dx_partial_dwdb": ([_A] * 9 + [_i, _i, _vp], _i),
+    "mi_layer_norm_bwd_dwdb": ([_A, _A, _A, _A, _i, _i, _vp], _i),
+    "mi_softmax_tma_kernel": ([_A, _A, _i, _i, _vp], _i),
+    "mi_softmax_chunked_kernel": ([_A, _A, _i, _i, _i, _vp], _i),
+    "mi_fmha_kernel": ([_A, _A, _A, _A, ctypes.c_float, ctypes.c_int32, _i, _i, _i, _i, _i, _i, _i, _vp], _i),
+    "mi_moe_align_tile_size": (
+        [ctypes.POINTER(ctypes.c_int64), ctypes.c_int64, ctypes.c_int64, _i, _i,
+         ctypes.POINTER(ctypes.c_int32), ctypes.POINTER(ctypes.c_int32),
+         ctypes.POINTER(ctypes.c_int64)], _i),
+    "mi_fused_moe_kernel": ([_A] * 6 + [_i, _i, _i, _i, _i, _A, _vp], _i),
+    "mi_silu_and_mul_kernel": ([_A, _A, _A, _i, _vp], _i),
+    "mi_moe_sum_topk": ([_A, _A, _vp], _i),
+}
+EXPORTED_SYMBOLS = tuple(_SIGNATURES)
+
+_lib = None
+
+
+def lib() -> ctypes.CDLL:
+    """Load libmi355tile.so (built in-tree by ``__graft_entry__.build``).  Raises if absent."""
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise RuntimeError(
+                f"{LIB_PATH} is missing: build it with `make -C {os.path.join(_HERE, 'csrc')}` "
+                "(or python -c 'import __graft_entry__ as g; g.build()'). There is no CPU fallback.")
+        # torch ships its own HIP runtime with the same soname; importing it first makes the
+        # kernels and torch's allocator share one runtime (and therefore streams).
+        import torch  # noqa: F401
+        cdll = ctypes.CDLL(LIB_PATH)
+        for name, (argtypes, restype) in _SIGNATURES.items():
+            fn = getattr(cdll, name)  # AttributeError if the library lacks a declared symbol
+            fn.argtypes = argtypes
+            fn.restype = restype
+        _lib = cdll
+    return _lib
+
+
+def strerror(code: int) -> str:
+    return lib().mi_strerror(code).decode()
+
+
+def last_variant() -> str:
+    return lib().mi_last_variant().decode()
+
+
+def _dtype_code(t) -> int:
+    import torch
+    table = {
+        torch.float32: MI_F32, torch.float64: MI_F64, torch.float16: MI_F16,
+        torch.bfloat16: MI_BF16, torch.int32: MI_I32, torch.int64: MI_I64,
+        torch.float8_e4m3fn: MI_F8E4M3FN,
+    }
+    try:
+        return table[t]
+    except KeyError:
+        raise TypeError(f"unsupported dtype {t}") from None
+
+
+def TileArray(t, dtype: int | None = None) -> MiTileArray:
+    """Descriptor for a torch tensor holding a Julia array in reversed-shape row-major form."""
+    if t.dim() > MI_MAX_RANK:
+        raise ValueError("rank > 4")
+    d = MiTileArray()
+    d.ptr = t.data_ptr()
+    d.dtype = _dtype_code(t.dtype) if dtype is None else dtype
+    d.ndim = t.dim()
+    for i, (sz, st) in enumerate(zip(reversed(t.shape), reversed(t.stride()))):
+        d.sizes[i] = sz
+        d.strides[i] = st
+    return d
+
+
+def _stream(stream=None):
+    import torch
+    if stream is None:
+        stream = torch.cuda.current_stream()
+    return ctypes.c_void_p(stream.cuda_stream)
+
+
+def _ref(x):
+    return None if x is None else ctypes.byref(x if isinstance(x, MiTileArray) else TileArray(x))
+
+
+def _call(name: str, *args):
+    rc = getattr(lib(), name)(*args)
+    if rc != 0:
+        raise MiError(name, rc, strerror(rc))
+
+
+# ---- kernel wrappers: one per entry point, argument order of the reference kernels --------
+
+def vec_add_kernel_1d(a, b, c, tile: int, stream=None):
+    """examples/vadd.jl:10-17"""
+    _call("mi_vec_add_kernel_1d", _ref(a), _ref(b), _ref(c), tile, _stream(stream))
+
+
+def vec_add_kernel_2d(a, b, c, tile_x: int, tile_y: int, stream=None):
+    """examples/vadd.jl:20-28"""
+    _call("mi_vec_add_kernel_2d", _ref(a), _ref(b), _ref(c), tile_x, tile_y, _stream(stream))
+
+
+def vec_add_kernel_1d_gather(a, b, c, tile: int, stream=None):
+    """examples/vadd.jl:31-45"""
+    _call("mi_vec_add_kernel_1d_gather", _ref(a), _ref(b), _ref(c), tile, _stream(stream))
+
+
+def transpose_kernel(x, y, tm: int, tn: int, stream=None):
+    """examples/transpose.jl:11-19"""
+    _call("mi_transpose_kernel", _ref(x), _ref(y), tm, tn, _stream(stream))
+
+
+def matmul_kernel(A, B, C, tm: int, tn: int, tk: int, stream=None):
+    """examples/matmul.jl:28-60"""
+    _call("mi_matmul_kernel", _ref(A), _ref(B), _ref(C), tm, tn, tk, _stream(stream))
+
+
+def batch_matmul_kernel(A, B, C, tm: int, tn: int, tk: int, stream=None):
+    """examples/batchmatmul.jl:15-56"""
+    _call("mi_batch_matmul_kernel", _ref(A), _ref(B), _ref(C), tm, tn, tk, _stream(stream))
+
+
+def swizzle_2d(M, N, tm, tn, GROUP_SIZE_M, bid):
+    """examples/matmul.jl:13-24 — 1-based bid -> 1-based (bid_m, bid_n)."""
+    bm, bn = ctypes.c_int32(), ctypes.c_int32()
+    lib().mi_swizzle_2d(M, N, tm, tn, GROUP_SIZE_M, bid, ctypes.byref(bm), ctypes.byref(bn))
+    return bm.value, bn.value
+
+
+def layer_norm_fwd(X, W, B, Y, Mean, Rstd, eps: float, TILE_N: int, stream=None):
+    """examples/layernorm.jl:27-68"""
+    _call("mi_layer_norm_fwd", _ref(X), _ref(W), _ref(B), _ref(Y), _ref(Mean), _ref(Rstd),
+          ctypes.c_float(eps), TILE_N, _stream(stream))
+
+
+def layer_norm_bwd_dx_partial_dwdb(DX, DY, DW, DB, X, W, Mean, Rstd, Locks, GROUP_SIZE_M: int,
+                                   TILE_N: int, stream=None):
+    """examples/layernorm.jl:118-171"""
+    _call("mi_layer_norm_bwd_dx_partial_dwdb", _ref(DX), _ref(DY), _ref(DW), _ref(DB), _ref(X),
+          _ref(W), _ref(Mean), _ref(Rstd), _ref(Locks), GROUP_SIZE_M, TILE_N, _stream(stream))
+
+
+def layer_norm_bwd_dwdb(DW, DB, FINAL_DW, FINAL_DB, TILE_M: int, TILE_N: int, stream=None):
+    """examples/layernorm.jl:186-205"""
+    _call("mi_layer_norm_bwd_dwdb", _ref(DW), _ref(DB), _ref(FINAL_DW), _ref(FINAL_DB), TILE_M,
+          TILE_N, _stream(stream))
+
+
+def softmax_tma_kernel(output, input, TILE_SIZE: int, num_programs: int | None = None, stream=None):
+    """examples/softmax.jl:18-42"""
+    if num_programs is None:
+        num_programs = max(1, min(input.shape[0] if input.dim() == 2 else 1, (1 << 24) - 1))
+    _call("mi_softmax_tma_kernel", _ref(output), _ref(input), TILE_SIZE, num_programs, _stream(stream))
+
+
+def softmax_chunked_kernel(output, input, n_elems: int, TILE_SIZE: int,
+                           num_programs: int | None = None, stream=None):
+    """examples/softmax.jl:48-100"""
+    if num_programs is None:
+        num_programs = max(1, min(input.shape[0] if input.dim() == 2 else 1, (1 << 24) - 1))
+    _call("mi_softmax_chunked_kernel", _ref(output), _ref(input), n_elems, TILE_SIZE, num_programs,
+          _stream(stream))
+
+
+def fmha_kernel(Q, K, V, Out, qk_scale: float, input_pos: int, TILE_D: int, H: int, TILE_M: int,
+                TILE_N: int, QUERY_GROUP_SIZE: int, CAUSAL: bool, EVEN_K: bool, stream=None):
+    """examples/fmha.jl:20-139"""
+    _call("mi_fmha_kernel", _ref(Q), _ref(K), _ref(V), _ref(Out), ctypes.c_float(qk_scale),
+          ctypes.c_int32(input_pos), TILE_D, H, TILE_M, TILE_N, QUERY_GROUP_SIZE, int(bool(CAUSAL)),
+          int(bool(EVEN_K)), _stream(stream))
+
+
+def moe_align_tile_size(topk_ids, tile_m: int, num_experts: int):
+    """examples/moe.jl:142-183.  ``topk_ids``: CPU int64 tensor holding the Julia
+    (num_tokens, topk) matrix, i.e. torch shape (topk, num_tokens).  Returns CPU int32
+    tensors (sorted_token_ids, sorted_expert_ids), both 1-based."""
+    import torch
+    assert topk_ids.device.type == "cpu" and topk_ids.dtype == torch.int64 and topk_ids.dim() == 2
+    ids = topk_ids.contiguous()
+    topk, num_tokens = ids.shape
+    p = ctypes.cast(ids.data_ptr(), ctypes.POINTER(ctypes.c_int64))
+    nblk = ctypes.c_int64()
+    _call("mi_moe_align_tile_size", p, num_tokens, topk, tile_m, num_experts, None, None,
+          ctypes.byref(nblk))
+    tok = torch.empty(nblk.value * tile_m, dtype=torch.int32)
+    exp = torch.empty(nblk.value, dtype=torch.int32)
+    _call("mi_moe_align_tile_size", p, num_tokens, topk, tile_m, num_experts,
+          ctypes.cast(tok.data_ptr(), ctypes.POINTER(ctypes.c_int32)),
+          ctypes.cast(exp.data_ptr(), ctypes.POINTER(ctypes.c_int32)), ctypes.byref(nblk))
+    return tok, exp
+
+
+def fused_moe_kernel(A, B, C, topk_weights, sorted_token_ids, sorted_expert_ids,
+                     num_token_replicas: int, mul_routed_weight: bool, TILE_M: int, TILE_N: int,
+                     TILE_K: int, b_scale=None, stream=None):
+    """examples/moe.jl:45-105 (``b_scale``: per-(n, expert) fp32 scales of fp8 weights)."""
+    _call("mi_fused_moe_kernel", _ref(A), _ref(B), _ref(C), _ref(topk_weights),
+          _ref(sorted_token_ids), _ref(sorted_expert_ids), num_token_replicas,
+          int(bool(mul_routed_weight)), TILE_M, TILE_N, TILE_K, _ref(b_scale), _stream(stream))
+
+
+def silu_and_mul_kernel(A, B, C, TILE_N: int, stream=None):
+    """examples/moe.jl:110-128"""
+    _call("mi_silu_and_mul_kernel", _ref(A), _ref(B), _ref(C), TILE_N, _stream(stream))
+
+
+def moe_sum_topk(inp, out, stream=None):
+    """The ``sum(cache3; dims=2)`` of examples/moe.jl:256."""
+    _call("mi_moe_sum_topk", _ref(inp), _ref(out), _stream(stream))

@@ -1,0 +1,473 @@
+// LayerNorm forward and backward: stand-ins for layer_norm_fwd (examples/layernorm.jl:27-68),
+// layer_norm_bwd_dx_partial_dwdb (:118-171) and layer_norm_bwd_dwdb (:186-205).
+//
+// Arrays are (N, M) fp32 with the normalised dimension N contiguous; "row" below means the
+// N contiguous elements that belong to one m.
+//
+// Forward: one workgroup per row, the row held in registers, so X is read once and Y
+// written once (algorithmic traffic 2*M*N*4 + small vectors) instead of the reference's
+// three passes.  Mean and variance are still two separate passes over the cached row
+// (mean first, then the sum of squared deviations), biased variance, rstd = 1/sqrt(var+eps).
+//
+// Backward: workgroup (g, s) walks the rows m with m mod GROUP_SIZE_M == g in S interleaved
+// splits, keeps the row's X and DY in registers (read once), writes DX, and accumulates its
+// rows' dW/dB contributions in registers.  At the end it adds them into slot g of the
+// caller's zero-filled DW/DB partial buffers: a plain read-add-write when one workgroup
+// owns the slot (S == 1), device-scope float atomics otherwise.  No spin-lock: workgroups of
+// one grid have no forward-progress guarantee relative to each other on this hardware.
+#include "common.h"
+#include <math.h>
+
+namespace {
+
+using namespace mi;
+
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+
+// Block all-reduce (sum) of two floats at once.
+template <int NWAVES>
+__device__ __forceinline__ void block_sum2(float& a, float& b, float* red) {
+    a = wave_reduce(a, SumOp{});
+    b = wave_reduce(b, SumOp{});
+    if constexpr (NWAVES == 1) return;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    if (lane == 0) { red[wave] = a; red[NWAVES + wave] = b; }
+    __syncthreads();
+    float ra = (lane < NWAVES) ? red[lane] : 0.f;
+    float rb = (lane < NWAVES) ? red[NWAVES + lane] : 0.f;
+#pragma unroll
+    for (int off = NWAVES / 2; off >= 1; off >>= 1) {
+        ra += __shfl_xor(ra, off, 64);
+        rb += __shfl_xor(rb, off, 64);
+    }
+    a = __shfl(ra, 0, 64);
+    b = __shfl(rb, 0, 64);
+    __syncthreads();
+}
+
+// Load / store the lane's VPT 4-element groups of one row.  Out-of-range elements load 0.
+template <int BLOCK, int VPT, bool ALIGNED, bool NT>
+__device__ __forceinline__ void load_row(const float* __restrict__ p, int N, float (&r)[VPT][4]) {
+#pragma unroll
+    for (int v = 0; v < VPT; ++v) {
+        const int e0 = (threadIdx.x + v * BLOCK) * 4;
+        if (ALIGNED && e0 + 4 <= N) {
+            f32x4 t = NT ? __builtin_nontemporal_load(reinterpret_cast<const f32x4*>(p + e0))
+                         : *reinterpret_cast<const f32x4*>(p + e0);
+#pragma unroll
+            for (int q = 0; q < 4; ++q) r[v][q] = t[q];
+        } else {
+#pragma unroll
+            for (int q = 0; q < 4; ++q) r[v][q] = (e0 + q < N) ? p[e0 + q] : 0.f;
+        }
+    }
+}
+template <int BLOCK, int VPT, bool ALIGNED>
+__device__ __forceinline__ void store_row(float* __restrict__ p, int N, const float (&r)[VPT][4]) {
+#pragma unroll
+    for (int v = 0; v < VPT; ++v) {
+        const int e0 = (threadIdx.x + v * BLOCK) * 4;
+        if (ALIGNED && e0 + 4 <= N) {
+            f32x4 t;
+#pragma unroll
+            for (int q = 0; q < 4; ++q) t[q] = r[v][q];
+            __builtin_nontemporal_store(t, reinterpret_cast<f32x4*>(p + e0));
+        } else {
+#pragma unroll
+            for (int q = 0; q < 4; ++q)
+                if (e0 + q < N) p[e0 + q] = r[v][q];
+        }
+    }
+}
+
+// ---- forward ---------------------------------------------------------------------------
+template <int BLOCK, int VPT, bool ALIGNED>
+__global__ __launch_bounds__(BLOCK) void ln_fwd_kernel(const float* __restrict__ X, int64_t ldx,
+                                                       const float* __restrict__ W,
+                                                       const float* __restrict__ B,
+                                                       float* __restrict__ Y, int64_t ldy,
+                                                       float* __restrict__ Mean,
+                                                       float* __restrict__ Rstd, float eps, int N,
+                                                       int64_t M) {
+    constexpr int NW = BLOCK / 64;
+    __shared__ float red[NW > 1 ? NW : 1];
+    const float invN = 1.0f / (float)N;
+    for (int64_t m = blockIdx.x; m < M; m += gridDim.x) {
+        float x[VPT][4];
+        load_row<BLOCK, VPT, ALIGNED, true>(X + m * ldx, N, x);
+        float s = 0.f;
+#pragma unroll
+        for (int v = 0; v < VPT; ++v)
+#pragma unroll
+            for (int q = 0; q < 4; ++q) s += x[v][q];
+        const float mean = block_reduce<NW>(s, red, SumOp{}, 0.f) / (float)N;
+        float sq = 0.f;
+#pragma unroll
+        for (int v = 0; v < VPT; ++v) {
+            const int e0 = (threadIdx.x + v * BLOCK) * 4;
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                const float d = (e0 + q < N) ? x[v][q] - mean : 0.f;
+                sq += d * d;
+            }
+        }
+        const float var = block_reduce<NW>(sq, red, SumOp{}, 0.f) / (float)N;
+        const float rstd = 1.0f / sqrtf(var + eps);
+        if (threadIdx.x == 0) {
+            Mean[m] = mean;
+            Rstd[m] = rstd;
+        }
+        float w[VPT][4], b[VPT][4];
+        load_row<BLOCK, VPT, ALIGNED, false>(W, N, w);
+        load_row<BLOCK, VPT, ALIGNED, false>(B, N, b);
+#pragma unroll
+        for (int v = 0; v < VPT; ++v)
+#pragma unroll
+            for (int q = 0; q < 4; ++q) x[v][q] = ((x[v][q] - mean) * rstd) * w[v][q] + b[v][q];
+        store_row<BLOCK, VPT, ALIGNED>(Y + m * ldy, N, x);
+    }
+    (void)invN;
+}
+
+// Forward for rows longer than the register-cached variants hold: three passes, the second
+// and third re-reading the row (served by L2 for rows up to a few MB).
+template <int BLOCK>
+__global__ __launch_bounds__(BLOCK) void ln_fwd_3pass_kernel(const float* __restrict__ X, int64_t ldx,
+                                                             const float* __restrict__ W,
+                                                             const float* __restrict__ B,
+                                                             float* __restrict__ Y, int64_t ldy,
+                                                             float* __restrict__ Mean,
+                                                             float* __restrict__ Rstd, float eps,
+                                                             int64_t N, int64_t M) {
+    constexpr int NW = BLOCK / 64;
+    __shared__ float red[NW];
+    for (int64_t m = blockIdx.x; m < M; m += gridDim.x) {
+        const float* x = X + m * ldx;
+        float s = 0.f;
+        for (int64_t e = threadIdx.x; e < N; e += BLOCK) s += x[e];
+        const float mean = block_reduce<NW>(s, red, SumOp{}, 0.f) / (float)N;
+        float sq = 0.f;
+        for (int64_t e = threadIdx.x; e < N; e += BLOCK) {
+            const float d = x[e] - mean;
+            sq += d * d;
+        }
+        const float var = block_reduce<NW>(sq, red, SumOp{}, 0.f) / (float)N;
+        const float rstd = 1.0f / sqrtf(var + eps);
+        if (threadIdx.x == 0) {
+            Mean[m] = mean;
+            Rstd[m] = rstd;
+        }
+        float* y = Y + m * ldy;
+        for (int64_t e = threadIdx.x; e < N; e += BLOCK) y[e] = ((x[e] - mean) * rstd) * W[e] + B[e];
+    }
+}
+
+// ---- backward: dX + partial dW/dB ------------------------------------------------------
+template <int BLOCK, int VPT, bool ALIGNED>
+__global__ __launch_bounds__(BLOCK) void ln_bwd_kernel(float* __restrict__ DX, int64_t lddx,
+                                                       const float* __restrict__ DY, int64_t lddy,
+                                                       float* __restrict__ DW, int64_t lddw,
+                                                       float* __restrict__ DB, int64_t lddb,
+                                                       const float* __restrict__ X, int64_t ldx,
+                                                       const float* __restrict__ W,
+                                                       const float* __restrict__ Mean,
+                                                       const float* __restrict__ Rstd, int N,
+                                                       int64_t M, int G, int S) {
+    constexpr int NW = BLOCK / 64;
+    __shared__ float red[2 * NW];
+    const int g = blockIdx.x % G, s = blockIdx.x / G;
+    float w[VPT][4], dw[VPT][4], db[VPT][4];
+    load_row<BLOCK, VPT, ALIGNED, false>(W, N, w);
+#pragma unroll
+    for (int v = 0; v < VPT; ++v)
+#pragma unroll
+        for (int q = 0; q < 4; ++q) dw[v][q] = db[v][q] = 0.f;
+
+    for (int64_t m = g + (int64_t)G * s; m < M; m += (int64_t)G * S) {
+        float x[VPT][4], dy[VPT][4];
+        load_row<BLOCK, VPT, ALIGNED, true>(X + m * ldx, N, x);
+        load_row<BLOCK, VPT, ALIGNED, true>(DY + m * lddy, N, dy);
+        const float mean = Mean[m], rstd = Rstd[m];
+        float c1 = 0.f, c2 = 0.f;
+#pragma unroll
+        for (int v = 0; v < VPT; ++v) {
+            const int e0 = (threadIdx.x + v * BLOCK) * 4;
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                const bool in = e0 + q < N;
+                const float xhat = in ? (x[v][q] - mean) * rstd : 0.f;
+                const float wdy = in ? w[v][q] * dy[v][q] : 0.f;
+                x[v][q] = xhat;
+                c1 += xhat * wdy;
+                c2 += wdy;
+            }
+        }
+        block_sum2<NW>(c1, c2, red);
+        c1 /= (float)N;
+        c2 /= (float)N;
+#pragma unroll
+        for (int v = 0; v < VPT; ++v)
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                const float xhat = x[v][q], wdy = w[v][q] * dy[v][q];
+                dw[v][q] += dy[v][q] * xhat;
+                db[v][q] += dy[v][q];
+                x[v][q] = (wdy - (xhat * c1 + c2)) * rstd;
+            }
+        store_row<BLOCK, VPT, ALIGNED>(DX + m * lddx, N, x);
+    }
+    float* dwp = DW + (int64_t)g * lddw;
+    float* dbp = DB + (int64_t)g * lddb;
+#pragma unroll
+    for (int v = 0; v < VPT; ++v) {
+        const int e0 = (threadIdx.x + v * BLOCK) * 4;
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+            if (e0 + q < N) {
+                if (S == 1) {
+                    dwp[e0 + q] += dw[v][q];
+                    dbp[e0 + q] += db[v][q];
+                } else {
+                    unsafeAtomicAdd(dwp + e0 + q, dw[v][q]);
+                    unsafeAtomicAdd(dbp + e0 + q, db[v][q]);
+                }
+            }
+        }
+    }
+}
+
+// Backward for rows longer than the register-cached variants hold.
+template <int BLOCK>
+__global__ __launch_bounds__(BLOCK) void ln_bwd_long_kernel(float* __restrict__ DX, int64_t lddx,
+                                                            const float* __restrict__ DY, int64_t lddy,
+                                                            float* __restrict__ DW, int64_t lddw,
+                                                            float* __restrict__ DB, int64_t lddb,
+                                                            const float* __restrict__ X, int64_t ldx,
+                                                            const float* __restrict__ W,
+                                                            const float* __restrict__ Mean,
+                                                            const float* __restrict__ Rstd,
+                                                            int64_t N, int64_t M, int G) {
+    constexpr int NW = BLOCK / 64;
+    __shared__ float red[2 * NW];
+    for (int64_t m = blockIdx.x; m < M; m += gridDim.x) {
+        const float* x = X + m * ldx;
+        const float* dy = DY + m * lddy;
+        const float mean = Mean[m], rstd = Rstd[m];
+        float c1 = 0.f, c2 = 0.f;
+        for (int64_t e = threadIdx.x; e < N; e += BLOCK) {
+            const float xhat = (x[e] - mean) * rstd, wdy = W[e] * dy[e];
+            c1 += xhat * wdy;
+            c2 += wdy;
+        }
+        block_sum2<NW>(c1, c2, red);
+        c1 /= (float)N;
+        c2 /= (float)N;
+        float* dwp = DW + (m % G) * lddw;
+        float* dbp = DB + (m % G) * lddb;
+        float* dx = DX + m * lddx;
+        for (int64_t e = threadIdx.x; e < N; e += BLOCK) {
+            const float xhat = (x[e] - mean) * rstd, wdy = W[e] * dy[e];
+            dx[e] = (wdy - (xhat * c1 + c2)) * rstd;
+            unsafeAtomicAdd(dwp + e, dy[e] * xhat);
+            unsafeAtomicAdd(dbp + e, dy[e]);
+        }
+    }
+}
+
+// ---- backward: final reduction over the partial slots -----------------------------------
+// 64 consecutive n per workgroup; the 4 waves split the slots, LDS combines them.
+__global__ __launch_bounds__(256) void ln_dwdb_kernel(const float* __restrict__ DW, int64_t lddw,
+                                                      const float* __restrict__ DB, int64_t lddb,
+                                                      float* __restrict__ FDW, float* __restrict__ FDB,
+                                                      int64_t N, int G) {
+    __shared__ float part[2][4][64];
+    const int lane = threadIdx.x & 63, wq = threadIdx.x >> 6;
+    const int64_t n = (int64_t)blockIdx.x * 64 + lane;
+    float a = 0.f, b = 0.f;
+    if (n < N) {
+        for (int g = wq; g < G; g += 4) {
+            a += DW[n + g * lddw];
+            b += DB[n + g * lddb];
+        }
+    }
+    part[0][wq][lane] = a;
+    part[1][wq][lane] = b;
+    __syncthreads();
+    if (wq == 0 && n < N) {
+        FDW[n] = (part[0][0][lane] + part[0][1][lane]) + (part[0][2][lane] + part[0][3][lane]);
+        FDB[n] = (part[1][0][lane] + part[1][1][lane]) + (part[1][2][lane] + part[1][3][lane]);
+    }
+}
+
+int check_f32(const mi_tile_array* a, int ndim) {
+    MI_CHECK(check_array(a, ndim));
+    if (a->dtype != MI_F32) return MI_E_DTYPE;
+    for (int i = 0; i < ndim; ++i)
+        if (i == 0 && a->sizes[0] > 1 && a->strides[0] != 1) return MI_E_STRIDE;
+    return MI_OK;
+}
+
+bool rows_vec_ok(const mi_tile_array* a) {
+    return aligned(a->ptr, 16) && (a->ndim < 2 || a->sizes[1] <= 1 || a->strides[1] % 4 == 0);
+}
+
+constexpr int kMaxRegsN = 256 * 16 * 4;
+
+template <bool AL>
+void launch_fwd(int vecs, dim3 grid, hipStream_t s, const float* X, int64_t ldx, const float* W,
+                const float* B, float* Y, int64_t ldy, float* Mean, float* Rstd, float eps, int N,
+                int64_t M) {
+#define FWD(BL, VP)                                                                              \
+    hipLaunchKernelGGL((ln_fwd_kernel<BL, VP, AL>), grid, dim3(BL), 0, s, X, ldx, W, B, Y, ldy, \
+                       Mean, Rstd, eps, N, M)
+    if (vecs <= 64) { FWD(64, 1); set_variant("ln_fwd_regs_b64_v1"); }
+    else if (vecs <= 128) { FWD(64, 2); set_variant("ln_fwd_regs_b64_v2"); }
+    else if (vecs <= 256) { FWD(256, 1); set_variant("ln_fwd_regs_b256_v1"); }
+    else if (vecs <= 512) { FWD(256, 2); set_variant("ln_fwd_regs_b256_v2"); }
+    else if (vecs <= 1024) { FWD(256, 4); set_variant("ln_fwd_regs_b256_v4"); }
+    else if (vecs <= 2048) { FWD(256, 8); set_variant("ln_fwd_regs_b256_v8"); }
+    else { FWD(256, 16); set_variant("ln_fwd_regs_b256_v16"); }
+#undef FWD
+}
+
+template <bool AL>
+void launch_bwd(int vecs, dim3 grid, hipStream_t s, float* DX, int64_t lddx, const float* DY,
+                int64_t lddy, float* DW, int64_t lddw, float* DB, int64_t lddb, const float* X,
+                int64_t ldx, const float* W, const float* Mean, const float* Rstd, int N, int64_t M,
+                int G, int S) {
+#define BWD(BL, VP)                                                                            \
+    hipLaunchKernelGGL((ln_bwd_kernel<BL, VP, AL>), grid, dim3(BL), 0, s, DX, lddx, DY, lddy, \
+                       DW, lddw, DB, lddb, X, ldx, W, Mean, Rstd, N, M, G, S)
+    if (vecs <= 64) { BWD(64, 1); set_variant("ln_bwd_regs_b64_v1"); }
+    else if (vecs <= 256) { BWD(256, 1); set_variant("ln_bwd_regs_b256_v1"); }
+    else if (vecs <= 512) { BWD(256, 2); set_variant("ln_bwd_regs_b256_v2"); }
+    else if (vecs <= 1024) { BWD(256, 4); set_variant("ln_bwd_regs_b256_v4"); }
+    else if (vecs <= 2048) { BWD(512, 4); set_variant("ln_bwd_regs_b512_v4"); }
+    else { BWD(1024, 4); set_variant("ln_bwd_regs_b1024_v4"); }
+#undef BWD
+}
+
+}  // namespace
+
+extern "C" int mi_layer_norm_fwd(const mi_tile_array* X, const mi_tile_array* W,
+                                 const mi_tile_array* B, const mi_tile_array* Y,
+                                 const mi_tile_array* Mean, const mi_tile_array* Rstd, float eps,
+                                 int TILE_N, void* stream) {
+    MI_CHECK(check_f32(X, 2));
+    MI_CHECK(check_f32(Y, 2));
+    MI_CHECK(check_f32(W, 1));
+    MI_CHECK(check_f32(B, 1));
+    MI_CHECK(check_f32(Mean, 1));
+    MI_CHECK(check_f32(Rstd, 1));
+    if (!is_pow2(TILE_N)) return MI_E_TILE;
+    const int64_t N = X->sizes[0], M = X->sizes[1];
+    if (!same_shape(X, Y) || W->sizes[0] != N || B->sizes[0] != N || Mean->sizes[0] != M ||
+        Rstd->sizes[0] != M)
+        return MI_E_SHAPE;
+    if ((M > 1 && (Mean->strides[0] != 1 || Rstd->strides[0] != 1))) return MI_E_STRIDE;
+    if (M > MI_MAX_GRID_DIM) return MI_E_GRID;
+    if (M == 0) return MI_OK;
+    if (N == 0) return MI_E_SHAPE;
+    hipStream_t s = (hipStream_t)stream;
+    const float* x = (const float*)X->ptr;
+    float* y = (float*)Y->ptr;
+    dim3 grid((unsigned)M);
+    if (N > kMaxRegsN) {
+        hipLaunchKernelGGL((ln_fwd_3pass_kernel<256>), grid, dim3(256), 0, s, x, X->strides[1],
+                           (const float*)W->ptr, (const float*)B->ptr, y, Y->strides[1],
+                           (float*)Mean->ptr, (float*)Rstd->ptr, eps, N, M);
+        set_variant("ln_fwd_3pass_b256");
+        return launch_status();
+    }
+    const bool al = rows_vec_ok(X) && rows_vec_ok(Y) && rows_vec_ok(W) && rows_vec_ok(B);
+    const int vecs = (int)cld(N, 4);
+    if (al)
+        launch_fwd<true>(vecs, grid, s, x, X->strides[1], (const float*)W->ptr, (const float*)B->ptr,
+                         y, Y->strides[1], (float*)Mean->ptr, (float*)Rstd->ptr, eps, (int)N, M);
+    else
+        launch_fwd<false>(vecs, grid, s, x, X->strides[1], (const float*)W->ptr, (const float*)B->ptr,
+                          y, Y->strides[1], (float*)Mean->ptr, (float*)Rstd->ptr, eps, (int)N, M);
+    return launch_status();
+}
+
+extern "C" int mi_layer_norm_bwd_dx_partial_dwdb(
+    const mi_tile_array* DX, const mi_tile_array* DY, const mi_tile_array* DW, const mi_tile_array* DB,
+    const mi_tile_array* X, const mi_tile_array* W, const mi_tile_array* Mean,
+    const mi_tile_array* Rstd, const mi_tile_array* Locks, int GROUP_SIZE_M, int TILE_N,
+    void* stream) {
+    MI_CHECK(check_f32(DX, 2));
+    MI_CHECK(check_f32(DY, 2));
+    MI_CHECK(check_f32(DW, 2));
+    MI_CHECK(check_f32(DB, 2));
+    MI_CHECK(check_f32(X, 2));
+    MI_CHECK(check_f32(W, 1));
+    MI_CHECK(check_f32(Mean, 1));
+    MI_CHECK(check_f32(Rstd, 1));
+    if (Locks) {
+        MI_CHECK(check_array(Locks, 1));
+        if (Locks->dtype != MI_I64) return MI_E_DTYPE;
+        if (Locks->sizes[0] < GROUP_SIZE_M) return MI_E_SHAPE;
+    }
+    if (GROUP_SIZE_M < 1) return MI_E_ARG;
+    if (!is_pow2(TILE_N)) return MI_E_TILE;
+    const int64_t N = X->sizes[0], M = X->sizes[1];
+    const int G = GROUP_SIZE_M;
+    if (!same_shape(X, DX) || !same_shape(X, DY) || W->sizes[0] != N || Mean->sizes[0] != M ||
+        Rstd->sizes[0] != M || DW->sizes[0] != N || DB->sizes[0] != N || DW->sizes[1] < G ||
+        DB->sizes[1] < G)
+        return MI_E_SHAPE;
+    if ((M > 1 && (Mean->strides[0] != 1 || Rstd->strides[0] != 1))) return MI_E_STRIDE;
+    if (M > MI_MAX_GRID_DIM) return MI_E_GRID;
+    if (M == 0) return MI_OK;
+    if (N == 0) return MI_E_SHAPE;
+    hipStream_t s = (hipStream_t)stream;
+    if (N > kMaxRegsN) {
+        hipLaunchKernelGGL((ln_bwd_long_kernel<256>), dim3((unsigned)M), dim3(256), 0, s,
+                           (float*)DX->ptr, DX->strides[1], (const float*)DY->ptr, DY->strides[1],
+                           (float*)DW->ptr, DW->strides[1], (float*)DB->ptr, DB->strides[1],
+                           (const float*)X->ptr, X->strides[1], (const float*)W->ptr,
+                           (const float*)Mean->ptr, (const float*)Rstd->ptr, N, M, G);
+        set_variant("ln_bwd_long_b256");
+        return launch_status();
+    }
+    // Splits per slot: enough workgroups to cover the 256 CUs a few times over, but at
+    // least ~4 rows per workgroup so the register partials amortise the atomics.
+    const int64_t rows_per_slot = cld(M, (int64_t)G);
+    int64_t S = cld((int64_t)1024, (int64_t)G);
+    if (S > cld(rows_per_slot, (int64_t)4)) S = cld(rows_per_slot, (int64_t)4);
+    if (S < 1) S = 1;
+    const bool al = rows_vec_ok(X) && rows_vec_ok(DX) && rows_vec_ok(DY) && rows_vec_ok(W);
+    const int vecs = (int)cld(N, 4);
+    dim3 grid((unsigned)(G * S));
+#define ARGS                                                                                   \
+    vecs, grid, s, (float*)DX->ptr, DX->strides[1], (const float*)DY->ptr, DY->strides[1],     \
+        (float*)DW->ptr, DW->strides[1], (float*)DB->ptr, DB->strides[1], (const float*)X->ptr, \
+        X->strides[1], (const float*)W->ptr, (const float*)Mean->ptr, (const float*)Rstd->ptr,  \
+        (int)N, M, G, (int)S
+    if (al) launch_bwd<true>(ARGS);
+    else launch_bwd<false>(ARGS);
+#undef ARGS
+    return launch_status();
+}
+
+extern "C" int mi_layer_norm_bwd_dwdb(const mi_tile_array* DW, const mi_tile_array* DB,
+                                      const mi_tile_array* FINAL_DW, const mi_tile_array* FINAL_DB,
+                                      int TILE_M, int TILE_N, void* stream) {
+    MI_CHECK(check_f32(DW, 2));
+    MI_CHECK(check_f32(DB, 2));
+    MI_CHECK(check_f32(FINAL_DW, 1));
+    MI_CHECK(check_f32(FINAL_DB, 1));
+    if (!is_pow2(TILE_M) || !is_pow2(TILE_N)) return MI_E_TILE;
+    const int64_t N = DW->sizes[0], G = DW->sizes[1];
+    if (!same_shape(DW, DB) || FINAL_DW->sizes[0] != N || FINAL_DB->sizes[0] != N) return MI_E_SHAPE;
+    if (N > 1 && (FINAL_DW->strides[0] != 1 || FINAL_DB->strides[0] != 1)) return MI_E_STRIDE;
+    if (cld(N, (int64_t)TILE_N) > MI_MAX_GRID_DIM) return MI_E_GRID;
+    if (N == 0) return MI_OK;
+    if (G > 0x7fffffff) return MI_E_SHAPE;
+    hipLaunchKernelGGL(ln_dwdb_kernel, dim3((unsigned)cld(N, (int64_t)64)), dim3(256), 0,
+                       (hipStream_t)stream, (const float*)DW->ptr, DW->strides[1],
+                       (const float*)DB->ptr, DB->strides[1], (float*)FINAL_DW->ptr,
+                       (float*)FINAL_DB->ptr, N, (int)G);
+    set_variant("ln_dwdb_b256");
+    return launch_status();
+}

@@ -1,0 +1,258 @@
+// Column softmax: stand-ins for softmax_tma_kernel (examples/softmax.jl:18-42) and
+// softmax_chunked_kernel (examples/softmax.jl:48-100) of the reference.
+//
+// input/output are (N, M) with the softmax dimension N contiguous.  One workgroup owns one
+// column at a time.  The single-tile kernel keeps the whole column in registers, so HBM is
+// touched exactly once per element each way (algorithmic traffic 2*M*N*sizeof(T)): 16-byte
+// loads, wave64 shuffle reductions, one LDS exchange per reduction across the waves of the
+// workgroup.  The chunked kernel makes the reference's three passes over the column (max,
+// denominator, normalise); passes two and three re-read the column from L2.
+//
+// Numerics follow the reference: fp32 math, max ignores NaN, full-precision exp (not
+// exp2), IEEE division, padding rows read as -Inf and are never written.
+#include "common.h"
+#include <math.h>
+
+namespace {
+
+using namespace mi;
+
+template <typename T> struct Raw;  // 16-byte vectors of the storage type
+template <> struct Raw<float> {
+    typedef float V __attribute__((ext_vector_type(4)));
+    static constexpr int EV = 4;
+};
+template <> struct Raw<__half> {
+    typedef _Float16 V __attribute__((ext_vector_type(8)));
+    static constexpr int EV = 8;
+};
+template <> struct Raw<__hip_bfloat16> {
+    typedef unsigned short V __attribute__((ext_vector_type(8)));
+    static constexpr int EV = 8;
+};
+
+template <typename T> __device__ __forceinline__ float vget(const typename Raw<T>::V& v, int q);
+template <> __device__ __forceinline__ float vget<float>(const Raw<float>::V& v, int q) { return v[q]; }
+template <> __device__ __forceinline__ float vget<__half>(const Raw<__half>::V& v, int q) {
+    return (float)v[q];
+}
+template <> __device__ __forceinline__ float vget<__hip_bfloat16>(const Raw<__hip_bfloat16>::V& v, int q) {
+    return __uint_as_float(((unsigned)v[q]) << 16);
+}
+template <typename T> __device__ __forceinline__ void vset(typename Raw<T>::V& v, int q, float f);
+template <> __device__ __forceinline__ void vset<float>(Raw<float>::V& v, int q, float f) { v[q] = f; }
+template <> __device__ __forceinline__ void vset<__half>(Raw<__half>::V& v, int q, float f) {
+    v[q] = (_Float16)f;
+}
+template <> __device__ __forceinline__ void vset<__hip_bfloat16>(Raw<__hip_bfloat16>::V& v, int q, float f) {
+    __hip_bfloat16 h = __float2bfloat16(f);
+    v[q] = *reinterpret_cast<unsigned short*>(&h);
+}
+
+// ---- single-tile kernel: column cached in registers -----------------------------------
+// Capacity BLOCK*VPT*EV elements.  ALIGNED: column bases and L allow 16-byte vectors.
+template <typename T, int BLOCK, int VPT, bool ALIGNED>
+__global__ __launch_bounds__(BLOCK) void softmax_regs_kernel(T* __restrict__ out, int64_t ldo,
+                                                             const T* __restrict__ in, int64_t ldi,
+                                                             int L, int64_t M) {
+    constexpr int EV = Raw<T>::EV;
+    using V = typename Raw<T>::V;
+    constexpr int NW = BLOCK / 64;
+    __shared__ float red[NW > 1 ? NW : 1];
+    const float NEG_INF = -INFINITY;
+
+    for (int64_t col = blockIdx.x; col < M; col += gridDim.x) {
+        const T* ip = in + col * ldi;
+        T* op = out + col * ldo;
+        float x[VPT][EV];
+#pragma unroll
+        for (int v = 0; v < VPT; ++v) {
+            const int e0 = (threadIdx.x + v * BLOCK) * EV;
+            if (ALIGNED && e0 + EV <= L) {
+                V raw = __builtin_nontemporal_load(reinterpret_cast<const V*>(ip + e0));
+#pragma unroll
+                for (int q = 0; q < EV; ++q) x[v][q] = vget<T>(raw, q);
+            } else {
+#pragma unroll
+                for (int q = 0; q < EV; ++q) x[v][q] = (e0 + q < L) ? to_f32<T>(ip[e0 + q]) : NEG_INF;
+            }
+        }
+        float mx = NEG_INF;
+#pragma unroll
+        for (int v = 0; v < VPT; ++v)
+#pragma unroll
+            for (int q = 0; q < EV; ++q) mx = fmaxf(mx, x[v][q]);
+        mx = block_reduce<NW>(mx, red, MaxOp{}, NEG_INF);
+        float sum = 0.f;
+#pragma unroll
+        for (int v = 0; v < VPT; ++v)
+#pragma unroll
+            for (int q = 0; q < EV; ++q) {
+                x[v][q] = expf(x[v][q] - mx);
+                sum += x[v][q];
+            }
+        sum = block_reduce<NW>(sum, red, SumOp{}, 0.f);
+#pragma unroll
+        for (int v = 0; v < VPT; ++v) {
+            const int e0 = (threadIdx.x + v * BLOCK) * EV;
+            if (ALIGNED && e0 + EV <= L) {
+                V raw;
+#pragma unroll
+                for (int q = 0; q < EV; ++q) vset<T>(raw, q, x[v][q] / sum);
+                __builtin_nontemporal_store(raw, reinterpret_cast<V*>(op + e0));
+            } else {
+#pragma unroll
+                for (int q = 0; q < EV; ++q)
+                    if (e0 + q < L) op[e0 + q] = from_f32<T>(x[v][q] / sum);
+            }
+        }
+    }
+}
+
+// ---- three-pass kernel: any column length ---------------------------------------------
+template <typename T, int BLOCK, bool ALIGNED>
+__global__ __launch_bounds__(BLOCK) void softmax_3pass_kernel(T* __restrict__ out, int64_t ldo,
+                                                              const T* __restrict__ in, int64_t ldi,
+                                                              int64_t L, int64_t M) {
+    constexpr int EV = Raw<T>::EV;
+    using V = typename Raw<T>::V;
+    constexpr int NW = BLOCK / 64;
+    __shared__ float red[NW];
+    const float NEG_INF = -INFINITY;
+    const int64_t nvec = ALIGNED ? L / EV : 0;
+
+    for (int64_t col = blockIdx.x; col < M; col += gridDim.x) {
+        const T* ip = in + col * ldi;
+        T* op = out + col * ldo;
+        // pass 1: running maximum
+        float mx = NEG_INF;
+        for (int64_t v = threadIdx.x; v < nvec; v += BLOCK) {
+            V raw = *reinterpret_cast<const V*>(ip + v * EV);
+#pragma unroll
+            for (int q = 0; q < EV; ++q) mx = fmaxf(mx, vget<T>(raw, q));
+        }
+        for (int64_t e = nvec * EV + threadIdx.x; e < L; e += BLOCK) mx = fmaxf(mx, to_f32<T>(ip[e]));
+        mx = block_reduce<NW>(mx, red, MaxOp{}, NEG_INF);
+        // pass 2: per-lane partial denominators, one reduction at the end
+        float den = 0.f;
+        for (int64_t v = threadIdx.x; v < nvec; v += BLOCK) {
+            V raw = *reinterpret_cast<const V*>(ip + v * EV);
+#pragma unroll
+            for (int q = 0; q < EV; ++q) den += expf(vget<T>(raw, q) - mx);
+        }
+        for (int64_t e = nvec * EV + threadIdx.x; e < L; e += BLOCK) den += expf(to_f32<T>(ip[e]) - mx);
+        den = block_reduce<NW>(den, red, SumOp{}, 0.f);
+        // pass 3: normalise and store
+        for (int64_t v = threadIdx.x; v < nvec; v += BLOCK) {
+            V raw = *reinterpret_cast<const V*>(ip + v * EV);
+            V res;
+#pragma unroll
+            for (int q = 0; q < EV; ++q) vset<T>(res, q, expf(vget<T>(raw, q) - mx) / den);
+            __builtin_nontemporal_store(res, reinterpret_cast<V*>(op + v * EV));
+        }
+        for (int64_t e = nvec * EV + threadIdx.x; e < L; e += BLOCK)
+            op[e] = from_f32<T>(expf(to_f32<T>(ip[e]) - mx) / den);
+    }
+}
+
+int check(const mi_tile_array* output, const mi_tile_array* input, int TILE_SIZE, int num_programs) {
+    MI_CHECK(check_array(output, 2));
+    MI_CHECK(check_array(input, 2));
+    if (output->dtype != input->dtype) return MI_E_DTYPE;
+    if (input->dtype != MI_F32 && input->dtype != MI_F16 && input->dtype != MI_BF16) return MI_E_DTYPE;
+    if (!same_shape(output, input)) return MI_E_SHAPE;
+    if (!is_pow2(TILE_SIZE)) return MI_E_TILE;
+    if (num_programs < 1 || num_programs > MI_MAX_GRID_DIM) return MI_E_GRID;
+    if (input->sizes[0] > 1 && (input->strides[0] != 1 || output->strides[0] != 1)) return MI_E_STRIDE;
+    return MI_OK;
+}
+
+template <typename T>
+bool vec_ok(const mi_tile_array* output, const mi_tile_array* input) {
+    constexpr int EV = Raw<T>::EV;
+    return aligned(input->ptr, 16) && aligned(output->ptr, 16) &&
+           (input->sizes[1] <= 1 || (input->strides[1] % EV == 0 && output->strides[1] % EV == 0));
+}
+
+template <typename T, int BLOCK, int VPT>
+void launch_regs(const mi_tile_array* output, const mi_tile_array* input, int L, bool al,
+                 hipStream_t s) {
+    const int64_t M = input->sizes[1];
+    dim3 grid((unsigned)M), block(BLOCK);
+    if (al)
+        hipLaunchKernelGGL((softmax_regs_kernel<T, BLOCK, VPT, true>), grid, block, 0, s,
+                           (T*)output->ptr, output->strides[1], (const T*)input->ptr,
+                           input->strides[1], L, M);
+    else
+        hipLaunchKernelGGL((softmax_regs_kernel<T, BLOCK, VPT, false>), grid, block, 0, s,
+                           (T*)output->ptr, output->strides[1], (const T*)input->ptr,
+                           input->strides[1], L, M);
+}
+
+template <typename T>
+int launch_3pass(const mi_tile_array* output, const mi_tile_array* input, int64_t L, hipStream_t s) {
+    const int64_t M = input->sizes[1];
+    const bool al = vec_ok<T>(output, input);
+    dim3 grid((unsigned)M), block(256);
+    if (al)
+        hipLaunchKernelGGL((softmax_3pass_kernel<T, 256, true>), grid, block, 0, s, (T*)output->ptr,
+                           output->strides[1], (const T*)input->ptr, input->strides[1], L, M);
+    else
+        hipLaunchKernelGGL((softmax_3pass_kernel<T, 256, false>), grid, block, 0, s, (T*)output->ptr,
+                           output->strides[1], (const T*)input->ptr, input->strides[1], L, M);
+    set_variant("softmax_3pass_b256");
+    return launch_status();
+}
+
+template <typename T>
+int launch_tma(const mi_tile_array* output, const mi_tile_array* input, int TILE_SIZE, hipStream_t s) {
+    constexpr int EV = Raw<T>::EV;
+    const int64_t N = input->sizes[0];
+    const int64_t L64 = N < TILE_SIZE ? N : (int64_t)TILE_SIZE;
+    if (L64 > 256 * 16 * EV) return launch_3pass<T>(output, input, L64, s);
+    const int L = (int)L64;
+    const bool al = vec_ok<T>(output, input);
+    const int vecs = (int)cld(L, EV);
+    if (vecs <= 64) { launch_regs<T, 64, 1>(output, input, L, al, s); set_variant("softmax_regs_b64_v1"); }
+    else if (vecs <= 128) { launch_regs<T, 64, 2>(output, input, L, al, s); set_variant("softmax_regs_b64_v2"); }
+    else if (vecs <= 256) { launch_regs<T, 256, 1>(output, input, L, al, s); set_variant("softmax_regs_b256_v1"); }
+    else if (vecs <= 512) { launch_regs<T, 256, 2>(output, input, L, al, s); set_variant("softmax_regs_b256_v2"); }
+    else if (vecs <= 1024) { launch_regs<T, 256, 4>(output, input, L, al, s); set_variant("softmax_regs_b256_v4"); }
+    else if (vecs <= 2048) { launch_regs<T, 256, 8>(output, input, L, al, s); set_variant("softmax_regs_b256_v8"); }
+    else { launch_regs<T, 256, 16>(output, input, L, al, s); set_variant("softmax_regs_b256_v16"); }
+    return launch_status();
+}
+
+}  // namespace
+
+extern "C" int mi_softmax_tma_kernel(const mi_tile_array* output, const mi_tile_array* input,
+                                     int TILE_SIZE, int num_programs, void* stream) {
+    MI_CHECK(check(output, input, TILE_SIZE, num_programs));
+    if (input->sizes[0] == 0 || input->sizes[1] == 0) return MI_OK;
+    if (input->sizes[1] > 0x7fffffffLL) return MI_E_GRID;
+    hipStream_t s = (hipStream_t)stream;
+    switch (input->dtype) {
+        case MI_F32: return launch_tma<float>(output, input, TILE_SIZE, s);
+        case MI_F16: return launch_tma<__half>(output, input, TILE_SIZE, s);
+        default: return launch_tma<__hip_bfloat16>(output, input, TILE_SIZE, s);
+    }
+}
+
+extern "C" int mi_softmax_chunked_kernel(const mi_tile_array* output, const mi_tile_array* input,
+                                         int n_elems, int TILE_SIZE, int num_programs, void* stream) {
+    MI_CHECK(check(output, input, TILE_SIZE, num_programs));
+    if (n_elems < 0) return MI_E_ARG;
+    if (input->sizes[0] == 0 || input->sizes[1] == 0) return MI_OK;
+    if (input->sizes[1] > 0x7fffffffLL) return MI_E_GRID;
+    // The chunk loop visits rows 1 .. cld(n_elems, TILE_SIZE)*TILE_SIZE; rows past the
+    // array's end are padding (softmax.jl:58, 65-69).
+    int64_t L = cld((int64_t)n_elems, (int64_t)TILE_SIZE) * TILE_SIZE;
+    if (L > input->sizes[0]) L = input->sizes[0];
+    if (L == 0) return MI_OK;
+    hipStream_t s = (hipStream_t)stream;
+    switch (input->dtype) {
+        case MI_F32: return launch_3pass<float>(output, input, L, s);
+        case MI_F16: return launch_3pass<__half>(output, input, L, s);
+        default: return launch_3pass<__hip_bfloat16>(output, input, L, s);
+    }
+}

@@ -1,0 +1,253 @@
+// Vector / matrix addition kernels: stand-ins for vec_add_kernel_1d, vec_add_kernel_2d and
+// vec_add_kernel_1d_gather of the reference's examples/vadd.jl:10-45.
+//
+// The result of c = a + b does not depend on the tile constant (a partial last tile is
+// zero-padded on load and clipped on store, src/language/operations.jl:637-646,819-821), so
+// the physical mapping is chosen for HBM3E streaming: 16-byte accesses, several independent
+// loads in flight per lane before the first use, non-temporal hints because nothing is
+// re-read.  Algorithmic traffic: 3 * n * sizeof(T) bytes.
+#include "common.h"
+
+namespace {
+
+using namespace mi;
+
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef double f64x2 __attribute__((ext_vector_type(2)));
+typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
+typedef unsigned short u16x8 __attribute__((ext_vector_type(8)));
+
+// One 16-byte vector of T and its element-wise IEEE add.
+template <typename T> struct Vec16;
+template <> struct Vec16<float> {
+    using V = f32x4;
+    static constexpr int N = 4;
+    static __device__ __forceinline__ V add(V a, V b) { return a + b; }
+    static __device__ __forceinline__ float add1(float a, float b) { return a + b; }
+};
+template <> struct Vec16<double> {
+    using V = f64x2;
+    static constexpr int N = 2;
+    static __device__ __forceinline__ V add(V a, V b) { return a + b; }
+    static __device__ __forceinline__ double add1(double a, double b) { return a + b; }
+};
+template <> struct Vec16<_Float16> {
+    using V = f16x8;
+    static constexpr int N = 8;
+    static __device__ __forceinline__ V add(V a, V b) { return a + b; }
+    static __device__ __forceinline__ _Float16 add1(_Float16 a, _Float16 b) { return a + b; }
+};
+// bf16 stored as raw 16-bit words: widen to fp32, add, round to nearest even.
+struct bf16raw { unsigned short v; };
+__device__ __forceinline__ float bf16_to_f32(unsigned short h) {
+    return __uint_as_float(((unsigned)h) << 16);
+}
+__device__ __forceinline__ unsigned short f32_to_bf16_rne(float f) {
+    unsigned u = __float_as_uint(f);
+    if ((u & 0x7fffffffu) > 0x7f800000u) return (unsigned short)((u >> 16) | 0x40);  // quiet NaN
+    u += 0x7fffu + ((u >> 16) & 1u);
+    return (unsigned short)(u >> 16);
+}
+template <> struct Vec16<bf16raw> {
+    using V = u16x8;
+    static constexpr int N = 8;
+    static __device__ __forceinline__ unsigned short add1u(unsigned short a, unsigned short b) {
+        return f32_to_bf16_rne(bf16_to_f32(a) + bf16_to_f32(b));
+    }
+    static __device__ __forceinline__ V add(V a, V b) {
+        V r;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) r[i] = add1u(a[i], b[i]);
+        return r;
+    }
+    static __device__ __forceinline__ bf16raw add1(bf16raw a, bf16raw b) {
+        return bf16raw{add1u(a.v, b.v)};
+    }
+};
+
+constexpr int kBlock = 256;
+
+// Streaming kernel: block b owns UNROLL*kBlock consecutive 16-byte vectors.  All UNROLL
+// loads of a and of b are issued before the first add so that each lane keeps
+// 2*UNROLL*16 bytes in flight.
+template <typename T, int UNROLL>
+__global__ __launch_bounds__(kBlock) void vadd_vec_kernel(const T* __restrict__ a,
+                                                          const T* __restrict__ b,
+                                                          T* __restrict__ c, int64_t nvec) {
+    using VT = Vec16<T>;
+    using V = typename VT::V;
+    const V* av = reinterpret_cast<const V*>(a);
+    const V* bv = reinterpret_cast<const V*>(b);
+    V* cv = reinterpret_cast<V*>(c);
+    const int64_t base = (int64_t)blockIdx.x * (UNROLL * kBlock) + threadIdx.x;
+    if (base + (int64_t)(UNROLL - 1) * kBlock < nvec) {
+        V x[UNROLL], y[UNROLL];
+#pragma unroll
+        for (int u = 0; u < UNROLL; ++u) x[u] = __builtin_nontemporal_load(av + base + u * kBlock);
+#pragma unroll
+        for (int u = 0; u < UNROLL; ++u) y[u] = __builtin_nontemporal_load(bv + base + u * kBlock);
+#pragma unroll
+        for (int u = 0; u < UNROLL; ++u)
+            __builtin_nontemporal_store(VT::add(x[u], y[u]), cv + base + u * kBlock);
+    } else {
+#pragma unroll
+        for (int u = 0; u < UNROLL; ++u) {
+            const int64_t i = base + u * kBlock;
+            if (i < nvec) cv[i] = VT::add(av[i], bv[i]);
+        }
+    }
+}
+
+// Element-wise kernel with arbitrary element strides: the scalar tail of the streaming
+// path, misaligned or strided 1-D arrays, and the gather/scatter variant (each lane forms
+// its own 1-based index, reads 0 when it is out of bounds and drops its store).
+template <typename T>
+__global__ __launch_bounds__(kBlock) void vadd_elem_kernel(const T* __restrict__ a, int64_t sa,
+                                                           const T* __restrict__ b, int64_t sb,
+                                                           T* __restrict__ c, int64_t sc,
+                                                           int64_t first, int64_t n_a, int64_t n_b,
+                                                           int64_t n_c) {
+    const int64_t i = first + (int64_t)blockIdx.x * kBlock + threadIdx.x;
+    if (i >= n_c) return;
+    T x = i < n_a ? a[i * sa] : T{};
+    T y = i < n_b ? b[i * sb] : T{};
+    c[i * sc] = Vec16<T>::add1(x, y);
+}
+
+// 2-D strided kernel (dimension 0 contiguous or not); one thread per element, x fastest.
+template <typename T>
+__global__ __launch_bounds__(kBlock) void vadd_2d_kernel(const T* __restrict__ a, int64_t a0,
+                                                         int64_t a1, const T* __restrict__ b,
+                                                         int64_t b0, int64_t b1, T* __restrict__ c,
+                                                         int64_t c0, int64_t c1, int64_t m,
+                                                         int64_t n) {
+    const int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+    const int64_t j = blockIdx.y;
+    if (i >= m || j >= n) return;
+    c[i * c0 + j * c1] = Vec16<T>::add1(a[i * a0 + j * a1], b[i * b0 + j * b1]);
+}
+
+template <typename T>
+int launch_dense(const void* a, const void* b, void* c, int64_t n, hipStream_t s) {
+    constexpr int N = Vec16<T>::N;
+    constexpr int UNROLL = 4;
+    const bool al = aligned(a, 16) && aligned(b, 16) && aligned(c, 16);
+    const int64_t nvec = al ? n / N : 0;
+    if (nvec > 0) {
+        const int64_t blocks = cld(nvec, (int64_t)UNROLL * kBlock);
+        if (blocks > 0x7fffffffLL) return MI_E_GRID;
+        hipLaunchKernelGGL((vadd_vec_kernel<T, UNROLL>), dim3((unsigned)blocks), dim3(kBlock), 0, s,
+                           (const T*)a, (const T*)b, (T*)c, nvec);
+        set_variant("vadd_vec16_nt_x4");
+    }
+    const int64_t done = nvec * N;
+    if (done < n) {
+        const int64_t blocks = cld(n - done, (int64_t)kBlock);
+        if (blocks > 0x7fffffffLL) return MI_E_GRID;
+        hipLaunchKernelGGL((vadd_elem_kernel<T>), dim3((unsigned)blocks), dim3(kBlock), 0, s,
+                           (const T*)a, (int64_t)1, (const T*)b, (int64_t)1, (T*)c, (int64_t)1,
+                           done, n, n, n);
+        if (nvec == 0) set_variant("vadd_elem");
+    }
+    return launch_status();
+}
+
+template <typename T>
+int launch_elem(const mi_tile_array* a, const mi_tile_array* b, const mi_tile_array* c,
+                hipStream_t s) {
+    const int64_t n = c->sizes[0];
+    if (n == 0) return MI_OK;
+    const int64_t blocks = cld(n, (int64_t)kBlock);
+    if (blocks > 0x7fffffffLL) return MI_E_GRID;
+    hipLaunchKernelGGL((vadd_elem_kernel<T>), dim3((unsigned)blocks), dim3(kBlock), 0, s,
+                       (const T*)a->ptr, a->strides[0], (const T*)b->ptr, b->strides[0],
+                       (T*)c->ptr, c->strides[0], (int64_t)0, a->sizes[0], b->sizes[0], n);
+    set_variant("vadd_elem");
+    return launch_status();
+}
+
+template <typename T>
+int launch_2d(const mi_tile_array* a, const mi_tile_array* b, const mi_tile_array* c,
+              hipStream_t s) {
+    const int64_t m = c->sizes[0], n = c->sizes[1];
+    if (m == 0 || n == 0) return MI_OK;
+    if (n > 65535) return MI_E_UNSUPPORTED;
+    hipLaunchKernelGGL((vadd_2d_kernel<T>), dim3((unsigned)cld(m, (int64_t)kBlock), (unsigned)n),
+                       dim3(kBlock), 0, s, (const T*)a->ptr, a->strides[0], a->strides[1],
+                       (const T*)b->ptr, b->strides[0], b->strides[1], (T*)c->ptr, c->strides[0],
+                       c->strides[1], m, n);
+    set_variant("vadd_2d_strided");
+    return launch_status();
+}
+
+#define DISPATCH_DTYPE(dt, CALL)                         \
+    switch (dt) {                                        \
+        case MI_F32: return CALL(float);                 \
+        case MI_F64: return CALL(double);                \
+        case MI_F16: return CALL(_Float16);              \
+        case MI_BF16: return CALL(bf16raw);              \
+        default: return MI_E_DTYPE;                      \
+    }
+
+int check3(const mi_tile_array* a, const mi_tile_array* b, const mi_tile_array* c, int ndim) {
+    MI_CHECK(check_array(a, ndim));
+    MI_CHECK(check_array(b, ndim));
+    MI_CHECK(check_array(c, ndim));
+    if (a->dtype != b->dtype || a->dtype != c->dtype) return MI_E_DTYPE;
+    return MI_OK;
+}
+
+}  // namespace
+
+extern "C" int mi_vec_add_kernel_1d(const mi_tile_array* a, const mi_tile_array* b,
+                                    const mi_tile_array* c, int tile, void* stream) {
+    MI_CHECK(check3(a, b, c, 1));
+    if (!is_pow2(tile)) return MI_E_TILE;
+    if (!same_shape(a, c) || !same_shape(b, c)) return MI_E_SHAPE;
+    const int64_t n = c->sizes[0];
+    if (cld(n, (int64_t)tile) > MI_MAX_GRID_DIM) return MI_E_GRID;
+    if (n == 0) return MI_OK;
+    hipStream_t s = (hipStream_t)stream;
+    if (is_dense(a) && is_dense(b) && is_dense(c)) {
+#define CALL(T) launch_dense<T>(a->ptr, b->ptr, c->ptr, n, s)
+        DISPATCH_DTYPE(c->dtype, CALL)
+#undef CALL
+    }
+#define CALL(T) launch_elem<T>(a, b, c, s)
+    DISPATCH_DTYPE(c->dtype, CALL)
+#undef CALL
+}
+
+extern "C" int mi_vec_add_kernel_1d_gather(const mi_tile_array* a, const mi_tile_array* b,
+                                           const mi_tile_array* c, int tile, void* stream) {
+    // Sizes may differ here: every lane bounds-checks its index against each array
+    // separately, as gather/scatter do.
+    MI_CHECK(check3(a, b, c, 1));
+    if (!is_pow2(tile)) return MI_E_TILE;
+    const int64_t n = c->sizes[0];
+    if (cld(n, (int64_t)tile) > MI_MAX_GRID_DIM) return MI_E_GRID;
+    hipStream_t s = (hipStream_t)stream;
+#define CALL(T) launch_elem<T>(a, b, c, s)
+    DISPATCH_DTYPE(c->dtype, CALL)
+#undef CALL
+}
+
+extern "C" int mi_vec_add_kernel_2d(const mi_tile_array* a, const mi_tile_array* b,
+                                    const mi_tile_array* c, int tile_x, int tile_y, void* stream) {
+    MI_CHECK(check3(a, b, c, 2));
+    if (!is_pow2(tile_x) || !is_pow2(tile_y)) return MI_E_TILE;
+    if (!same_shape(a, c) || !same_shape(b, c)) return MI_E_SHAPE;
+    const int64_t m = c->sizes[0], n = c->sizes[1];
+    if (cld(m, (int64_t)tile_x) > MI_MAX_GRID_DIM || cld(n, (int64_t)tile_y) > MI_MAX_GRID_DIM)
+        return MI_E_GRID;
+    if (m * n == 0) return MI_OK;
+    hipStream_t s = (hipStream_t)stream;
+    if (is_dense(a) && is_dense(b) && is_dense(c)) {
+#define CALL(T) launch_dense<T>(a->ptr, b->ptr, c->ptr, m * n, s)
+        DISPATCH_DTYPE(c->dtype, CALL)
+#undef CALL
+    }
+#define CALL(T) launch_2d<T>(a, b, c, s)
+    DISPATCH_DTYPE(c->dtype, CALL)
+#undef CALL
+}

@@ -1,0 +1,63 @@
+"""Mirror of examples/layernorm.jl:211-332 (prepare / run / metric)."""
+from __future__ import annotations
+
+import numpy as np
+import torch
+
+import cutile_jl_amd as ct
+from ._harness import namespace, rand_normal, time_launches
+
+
+def prepare(*, benchmark: bool = False, M: int | None = None, N: int | None = None,
+            eps: float = 1e-5, GROUP_SIZE_M: int = 64, seed: int = 1):
+    """layernorm.jl:211-234.  Arrays are Julia (N, M) = torch (M, N).  Inputs follow the
+    measured configuration: X ~ N(0,1), W ~ N(1,0.1), B ~ N(0,0.1), DY ~ N(0,1)."""
+    M = (4096 if benchmark else 256) if M is None else M
+    N = (4096 if benchmark else 256) if N is None else N
+    rng = np.random.default_rng(seed)
+    f32 = torch.float32
+    X = rand_normal(rng, (N, M), f32)
+    W = rand_normal(rng, (N,), f32, mean=1.0, std=0.1)
+    B = rand_normal(rng, (N,), f32, mean=0.0, std=0.1)
+    DY = rand_normal(rng, (N, M), f32)
+    dev = X.device
+    e = lambda *jl: torch.empty(tuple(reversed(jl)), dtype=f32, device=dev)
+    return namespace(
+        X=X, W=W, B=B, Y=e(N, M), Mean=e(M), Rstd=e(M),
+        DY=DY, DX=e(N, M), DW_partial=e(N, GROUP_SIZE_M), DB_partial=e(N, GROUP_SIZE_M),
+        Locks=torch.empty(GROUP_SIZE_M, dtype=torch.int64, device=dev),
+        FINAL_DW=e(N), FINAL_DB=e(N), M=M, N=N, eps=eps, GROUP_SIZE_M=GROUP_SIZE_M)
+
+
+def run(data, *, TILE_N: int = 1024, TILE_M: int = 32, nruns: int = 1, warmup: int = 0):
+    """layernorm.jl:236-282: the backward timing includes the three fills and both kernels."""
+    d = data
+
+    def run_fwd():
+        ct.layer_norm_fwd(d.X, d.W, d.B, d.Y, d.Mean, d.Rstd, d.eps, TILE_N)
+
+    def run_bwd():
+        d.DW_partial.zero_()
+        d.DB_partial.zero_()
+        d.Locks.zero_()
+        ct.layer_norm_bwd_dx_partial_dwdb(d.DX, d.DY, d.DW_partial, d.DB_partial, d.X, d.W, d.Mean,
+                                          d.Rstd, d.Locks, d.GROUP_SIZE_M, TILE_N)
+        ct.layer_norm_bwd_dwdb(d.DW_partial, d.DB_partial, d.FINAL_DW, d.FINAL_DB, TILE_M, TILE_N)
+
+    def both():
+        run_fwd()
+        run_bwd()
+
+    for _ in range(warmup):
+        both()
+    torch.cuda.synchronize()
+    times_fwd = time_launches(run_fwd, nruns, 0)
+    times_bwd = time_launches(run_bwd, nruns, 0)
+    return namespace(Y=d.Y, Mean=d.Mean, Rstd=d.Rstd, DX=d.DX, FINAL_DW=d.FINAL_DW,
+                     FINAL_DB=d.FINAL_DB, times_fwd=times_fwd, times_bwd=times_bwd)
+
+
+def metric(data):
+    """layernorm.jl:324-332 (the reference's formula, which counts its L2-served re-reads)."""
+    MN = data.M * data.N * 4
+    return {"cuTile Fwd": (4 * MN, "GB/s"), "cuTile Bwd": (5 * MN, "GB/s")}

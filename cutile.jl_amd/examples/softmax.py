@@ -1,0 +1,59 @@
+"""Mirror of examples/softmax.jl:116-198 (prepare / run / metric)."""
+from __future__ import annotations
+
+import numpy as np
+import torch
+
+import cutile_jl_amd as ct
+from ._harness import namespace, rand_normal, time_launches
+
+
+def next_power_of_2(n: int) -> int:
+    """softmax.jl:107-114"""
+    if n <= 0:
+        return 1
+    p = 1
+    while p < n:
+        p <<= 1
+    return p
+
+
+def prepare(*, benchmark: bool = False, M: int | None = None, N: int | None = None,
+            T: torch.dtype = torch.float32, seed: int = 2, std: float = 2.0):
+    """softmax.jl:116-127: input Julia (N, M) = torch (M, N); measured configuration draws
+    N(0, sigma^2 = 4)."""
+    M = (4096 if benchmark else 256) if M is None else M
+    N = (4096 if benchmark else 256) if N is None else N
+    rng = np.random.default_rng(seed)
+    inp = rand_normal(rng, (N, M), T, std=std)
+    return namespace(input=inp, output_tma=torch.empty_like(inp),
+                     output_chunked=torch.empty_like(inp), M=M, N=N)
+
+
+def run(data, *, tile_tma: int | None = None, tile_chunked: int = 1024, nruns: int = 1,
+        warmup: int = 0):
+    """softmax.jl:129-173."""
+    d = data
+    if tile_tma is None:
+        tile_tma = next_power_of_2(d.N)
+
+    def run_tma():
+        ct.softmax_tma_kernel(d.output_tma, d.input, tile_tma, num_programs=d.M)
+
+    def run_chunked():
+        ct.softmax_chunked_kernel(d.output_chunked, d.input, d.N, tile_chunked, num_programs=d.M)
+
+    for _ in range(warmup):
+        run_tma()
+        run_chunked()
+    torch.cuda.synchronize()
+    times_tma = time_launches(run_tma, nruns, 0)
+    times_chunked = time_launches(run_chunked, nruns, 0)
+    return namespace(output_tma=d.output_tma, output_chunked=d.output_chunked,
+                     times={"cuTile TMA": times_tma, "cuTile Chunked": times_chunked})
+
+
+def metric(data):
+    """softmax.jl:190-198."""
+    MN = data.M * data.N * 4
+    return {"cuTile TMA": (2 * MN, "GB/s"), "cuTile Chunked": (4 * MN, "GB/s")}

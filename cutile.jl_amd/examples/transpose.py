@@ -1,0 +1,30 @@
+"""Mirror of examples/transpose.jl:25-66 (prepare / run / metric)."""
+from __future__ import annotations
+
+import numpy as np
+import torch
+
+import cutile_jl_amd as ct
+from ._harness import namespace, rand_uniform, time_launches
+
+
+def prepare(*, benchmark: bool = False, m: int | None = None, n: int | None = None,
+            T: torch.dtype = torch.float32, seed: int = 0):
+    """transpose.jl:25-36: x (m, n) ~ U[0,1), y (n, m)."""
+    m = (8192 if benchmark else 1024) if m is None else m
+    n = (8192 if benchmark else 512) if n is None else n
+    rng = np.random.default_rng(seed)
+    x = rand_uniform(rng, (m, n), T)
+    y = torch.empty((m, n), dtype=T, device=x.device)  # Julia (n, m)
+    return namespace(x=x, y=y, m=m, n=n)
+
+
+def run(data, *, tm: int = 64, tn: int = 64, nruns: int = 1, warmup: int = 0):
+    """transpose.jl:38-56."""
+    times = time_launches(lambda: ct.transpose_kernel(data.x, data.y, tm, tn), nruns, warmup)
+    return namespace(y=data.y, times=times)
+
+
+def metric(data):
+    """transpose.jl:62-66: 1 read + 1 write."""
+    return 2 * data.m * data.n * data.x.element_size(), "GB/s"

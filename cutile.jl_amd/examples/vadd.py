@@ -1,0 +1,41 @@
+"""Mirror of examples/vadd.jl:52-136 (prepare / run / metric)."""
+from __future__ import annotations
+
+import numpy as np
+import torch
+
+import cutile_jl_amd as ct
+from ._harness import namespace, rand_uniform, time_launches
+
+
+def prepare(*, benchmark: bool = False, shape=None, use_gather: bool = False,
+            T: torch.dtype = torch.float32, seed: int = 0):
+    """vadd.jl:52-63; a, b ~ U[0,1) from ``seed`` (the reference draws them with cuRAND)."""
+    if shape is None:
+        shape = (2 ** 27,) if benchmark else (1_024_000,)
+    rng = np.random.default_rng(seed)
+    a = rand_uniform(rng, shape, T)
+    b = rand_uniform(rng, shape, T)
+    return namespace(a=a, b=b, c=torch.empty_like(a), shape=tuple(shape), use_gather=use_gather)
+
+
+def run(data, *, tile=1024, nruns: int = 1, warmup: int = 0):
+    """vadd.jl:65-125."""
+    a, b, c = data.a, data.b, data.c
+    if len(data.shape) == 2:
+        tile_x, tile_y = tile if isinstance(tile, tuple) else (tile, tile)
+        launch = lambda: ct.vec_add_kernel_2d(a, b, c, tile_x, tile_y)
+    else:
+        tile_val = tile[0] if isinstance(tile, tuple) else tile
+        if data.use_gather:
+            launch = lambda: ct.vec_add_kernel_1d_gather(a, b, c, tile_val)
+        else:
+            launch = lambda: ct.vec_add_kernel_1d(a, b, c, tile_val)
+    times = time_launches(launch, nruns, warmup)
+    return namespace(c=c, times=times)
+
+
+def metric(data):
+    """vadd.jl:131-136: 2 reads + 1 write."""
+    n = int(np.prod(data.shape))
+    return 3 * n * data.a.element_size(), "GB/s"

@@ -1,0 +1,195 @@
+/*
+ * mi355tile.h — C ABI of libmi355tile.so
+ *
+ * Hand-written HIP kernels for AMD Instinct MI355X (gfx950 / CDNA4) that stand in for
+ * the kernels cuTile.jl's examples compile through NVIDIA Tile IR.  There is exactly one
+ * entry point per example kernel.  Each takes the example kernel's arguments in the
+ * example's own order:
+ *
+ *   - every `ct.TileArray{T,N}` argument becomes a `const mi_tile_array*`, a plain-data
+ *     mirror of the reference's array descriptor (pointer, sizes, strides in ELEMENTS,
+ *     first dimension fastest — Julia column-major; reference: src/language/types.jl:283-287,
+ *     flattened for launch at src/launch.jl:750-777);
+ *   - scalar arguments stay scalars;
+ *   - the `ct.Constant(...)` tile-size arguments become plain `int`s;
+ *   - a trailing `void* stream` is the hipStream_t to enqueue on (NULL = default stream).
+ *     The reference enqueues on the task-local CUDA stream (src/launch.jl:862).
+ *
+ * The grid is derived inside the library from sizes + tile constants with the formulas
+ * the examples use (`cld(M,tm)*cld(N,tn)` …).  Tile constants are semantic parameters
+ * (block → data mapping, padding contracts, accumulation grouping); the physical
+ * wave / LDS tiling is chosen by the library for CDNA4.
+ *
+ * Every call is asynchronous, allocates nothing and never throws.  Return value: 0 on
+ * success, a negative MI_E_* code for argument errors detected on the host, or a
+ * positive hipError_t reported by the launch.  The caller owns all buffers.
+ */
+#ifndef MI355TILE_H
+#define MI355TILE_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define MI355TILE_VERSION 100 /* major*10000 + minor*100 + patch */
+
+/* Element types of a mi_tile_array. */
+typedef enum mi_dtype {
+    MI_F32 = 0,
+    MI_F64 = 1,
+    MI_F16 = 2,
+    MI_BF16 = 3,
+    MI_F8E4M3FN = 4, /* OCP FP8 E4M3 "FN": bias 7, no Inf, NaN = S.1111.111, max 448
+                        (reference: ext/DLFP8TypesExt.jl:7-9) */
+    MI_I32 = 5,
+    MI_I64 = 6
+} mi_dtype;
+
+/* Error codes (negative).  Positive return values are hipError_t. */
+enum {
+    MI_OK = 0,
+    MI_E_NULL = -1,      /* a required pointer is NULL */
+    MI_E_DTYPE = -2,     /* unsupported or mismatching element type */
+    MI_E_RANK = -3,      /* wrong number of dimensions */
+    MI_E_SHAPE = -4,     /* sizes of the arguments do not agree */
+    MI_E_STRIDE = -5,    /* layout not supported (fastest dimension must have stride 1) */
+    MI_E_TILE = -6,      /* tile constant not a positive power of two, or unsupported */
+    MI_E_GRID = -7,      /* a grid dimension exceeds 2^24-1 (reference: src/launch.jl:743,801-807) */
+    MI_E_ALIGN = -8,     /* pointer not aligned to its element size */
+    MI_E_ARG = -9,       /* other invalid scalar argument */
+    MI_E_UNSUPPORTED = -10
+};
+
+#define MI_MAX_RANK 4
+
+/* Mirror of cuTile's TileArray{T,N} (src/language/types.jl:283-287): a device pointer with
+ * per-dimension sizes and element strides, dimension 0 here = Julia dimension 1. */
+typedef struct mi_tile_array {
+    void* ptr;
+    int32_t dtype; /* mi_dtype */
+    int32_t ndim;
+    int64_t sizes[MI_MAX_RANK];
+    int64_t strides[MI_MAX_RANK];
+} mi_tile_array;
+
+/* ---- library ---------------------------------------------------------------------- */
+int mi_version(void);
+const char* mi_strerror(int code);
+/* Name of the kernel variant chosen by the most recent successful launch on this thread
+ * (for profiles and tests; never NULL). */
+const char* mi_last_variant(void);
+
+/* ---- vadd: examples/vadd.jl ------------------------------------------------------- */
+/* vec_add_kernel_1d (vadd.jl:10-17): c = a + b; block `bid` owns elements
+ * (bid-1)*tile+1 … bid*tile.  f32 / f64 / f16 / bf16. */
+int mi_vec_add_kernel_1d(const mi_tile_array* a, const mi_tile_array* b, const mi_tile_array* c,
+                         int tile, void* stream);
+/* vec_add_kernel_2d (vadd.jl:20-28): same on (tile_x, tile_y) tiles of 2-D arrays. */
+int mi_vec_add_kernel_2d(const mi_tile_array* a, const mi_tile_array* b, const mi_tile_array* c,
+                         int tile_x, int tile_y, void* stream);
+/* vec_add_kernel_1d_gather (vadd.jl:31-45): same through per-element indexed gather/scatter;
+ * lanes whose index is out of bounds read 0 and their store is dropped
+ * (src/language/operations.jl:996-1009,1072-1085). */
+int mi_vec_add_kernel_1d_gather(const mi_tile_array* a, const mi_tile_array* b,
+                                const mi_tile_array* c, int tile, void* stream);
+
+/* ---- transpose: examples/transpose.jl --------------------------------------------- */
+/* transpose_kernel (transpose.jl:11-19): y[j,i] = x[i,j]; x is (m,n), y is (n,m). */
+int mi_transpose_kernel(const mi_tile_array* x, const mi_tile_array* y, int tm, int tn,
+                        void* stream);
+
+/* ---- matmul: examples/matmul.jl, examples/batchmatmul.jl --------------------------- */
+/* matmul_kernel (matmul.jl:28-60): C(M,N) = A(M,K)·B(K,N), fp32 accumulate, 1-D grid of
+ * cld(M,tm)*cld(N,tn) blocks ordered by swizzle_2d with GROUP_SIZE_M = 8, ragged edges
+ * zero-padded on load and clipped on store.  A,B: f16 / bf16 / f32; C: the input type or
+ * f32.  f32 inputs are multiplied in true fp32 (gfx950 has no TF32-class MFMA; the
+ * reference rounds f32 operands to TF32 at matmul.jl:49-52). */
+int mi_matmul_kernel(const mi_tile_array* A, const mi_tile_array* B, const mi_tile_array* C,
+                     int tm, int tn, int tk, void* stream);
+/* batch_matmul_kernel (batchmatmul.jl:15-56): C(M,N,b) = A(M,K,b)·B(K,N,b), grid
+ * (cld(M,tm), cld(N,tn), Batch). */
+int mi_batch_matmul_kernel(const mi_tile_array* A, const mi_tile_array* B,
+                           const mi_tile_array* C, int tm, int tn, int tk, void* stream);
+/* swizzle_2d (matmul.jl:13-24, moe.jl:20-31), host helper: 1-based block id →
+ * 1-based (bid_m, bid_n). */
+void mi_swizzle_2d(int32_t M, int32_t N, int32_t tm, int32_t tn, int32_t group_size_m,
+                   int32_t bid, int32_t* bid_m, int32_t* bid_n);
+
+/* ---- layernorm: examples/layernorm.jl ---------------------------------------------- */
+/* layer_norm_fwd (layernorm.jl:27-68).  X,Y (N,M) f32 with N contiguous; W,B (N,);
+ * Mean,Rstd (M,).  Two-pass mean / biased variance, rstd = 1/sqrt(var+eps). */
+int mi_layer_norm_fwd(const mi_tile_array* X, const mi_tile_array* W, const mi_tile_array* B,
+                      const mi_tile_array* Y, const mi_tile_array* Mean,
+                      const mi_tile_array* Rstd, float eps, int TILE_N, void* stream);
+/* layer_norm_bwd_dx_partial_dwdb (layernorm.jl:118-171).  Writes DX and ADDS partial
+ * dW/dB into the GROUP_SIZE_M slots of DW,DB (N, GROUP_SIZE_M), which the caller has
+ * zero-filled (layernorm.jl:245-247); row m contributes to slot m mod GROUP_SIZE_M.
+ * `Locks` (GROUP_SIZE_M,) i64 is accepted for signature compatibility and not touched:
+ * accumulation uses per-workgroup register partials plus device-scope float atomics
+ * instead of the reference's CAS spin-lock.  May be NULL. */
+int mi_layer_norm_bwd_dx_partial_dwdb(const mi_tile_array* DX, const mi_tile_array* DY,
+                                      const mi_tile_array* DW, const mi_tile_array* DB,
+                                      const mi_tile_array* X, const mi_tile_array* W,
+                                      const mi_tile_array* Mean, const mi_tile_array* Rstd,
+                                      const mi_tile_array* Locks, int GROUP_SIZE_M, int TILE_N,
+                                      void* stream);
+/* layer_norm_bwd_dwdb (layernorm.jl:186-205): FINAL_DW[n] = sum_g DW[n,g], same for DB. */
+int mi_layer_norm_bwd_dwdb(const mi_tile_array* DW, const mi_tile_array* DB,
+                           const mi_tile_array* FINAL_DW, const mi_tile_array* FINAL_DB,
+                           int TILE_M, int TILE_N, void* stream);
+
+/* ---- softmax: examples/softmax.jl -------------------------------------------------- */
+/* softmax_tma_kernel (softmax.jl:18-42): column softmax of input (N,M), one tile of
+ * TILE_SIZE rows per column (rows beyond TILE_SIZE are neither read nor written, as in
+ * the reference).  `num_programs` is the reference's launch grid (`blocks=M` at
+ * softmax.jl:136); any value >= 1 gives the same result. f32 / f16 / bf16 storage. */
+int mi_softmax_tma_kernel(const mi_tile_array* output, const mi_tile_array* input,
+                          int TILE_SIZE, int num_programs, void* stream);
+/* softmax_chunked_kernel (softmax.jl:48-100): 3-pass softmax over the first n_elems rows
+ * in chunks of TILE_SIZE. */
+int mi_softmax_chunked_kernel(const mi_tile_array* output, const mi_tile_array* input,
+                              int n_elems, int TILE_SIZE, int num_programs, void* stream);
+
+/* ---- FMHA: examples/fmha.jl --------------------------------------------------------- */
+/* fmha_kernel (fmha.jl:20-139).  Q (D,Sq,H,B), K (D,Skv,KVH,B), V (Dv,Skv,KVH,B),
+ * Out (Dv,Sq,H,B), f16 or bf16; online softmax in the exp2 domain with fp32 accumulation,
+ * P rounded to the storage type before P·V, causal tile skipping, GQA via
+ * QUERY_GROUP_SIZE, decode offset input_pos, ragged KV tail when !EVEN_K. */
+int mi_fmha_kernel(const mi_tile_array* Q, const mi_tile_array* K, const mi_tile_array* V,
+                   const mi_tile_array* Out, float qk_scale, int32_t input_pos, int TILE_D,
+                   int H, int TILE_M, int TILE_N, int QUERY_GROUP_SIZE, int CAUSAL, int EVEN_K,
+                   void* stream);
+
+/* ---- MoE: examples/moe.jl ------------------------------------------------------------ */
+/* moe_align_tile_size (moe.jl:142-183), HOST routine on host memory.  topk_ids is the
+ * Julia (num_tokens, topk) Int64 matrix of 1-based expert ids in column-major order.
+ * sorted_token_ids_out needs capacity for tile_m * sum_e cld(count_e, tile_m) entries
+ * (never more than num_tokens*topk + num_experts*(tile_m-1)); sorted_expert_ids_out one
+ * entry per block.  Passing NULL outputs only counts.  Returns 0 or MI_E_*. */
+int mi_moe_align_tile_size(const int64_t* topk_ids, int64_t num_tokens, int64_t topk, int tile_m,
+                           int num_experts, int32_t* sorted_token_ids_out,
+                           int32_t* sorted_expert_ids_out, int64_t* total_blocks_out);
+/* fused_moe_kernel (moe.jl:45-105).  A (K,num_tokens), B (K,N,E), C (N,total_tokens),
+ * topk_weights (total_tokens,), sorted_token_ids (M_padded,) i32 1-based with sentinel
+ * total_tokens+1, sorted_expert_ids (blocks,) i32 1-based.  A, C, topk_weights f16/bf16.
+ * B is f16/bf16, or MI_F8E4M3FN with `b_scale` (N,E) f32 per-output-channel scales
+ * (fp8 weights are an extension of this build; b_scale must be NULL otherwise). */
+int mi_fused_moe_kernel(const mi_tile_array* A, const mi_tile_array* B, const mi_tile_array* C,
+                        const mi_tile_array* topk_weights, const mi_tile_array* sorted_token_ids,
+                        const mi_tile_array* sorted_expert_ids, int num_token_replicas,
+                        int mul_routed_weight, int TILE_M, int TILE_N, int TILE_K,
+                        const mi_tile_array* b_scale, void* stream);
+/* silu_and_mul_kernel (moe.jl:110-128): C[:,t] = silu(A[:,t]) * B[:,t] in fp32. */
+int mi_silu_and_mul_kernel(const mi_tile_array* A, const mi_tile_array* B,
+                           const mi_tile_array* C, int TILE_N, void* stream);
+/* The top-k combine `sum(cache3; dims=2)` of cutile_moe (moe.jl:256), which the reference
+ * hands to CUDA.jl: out (H, tokens) = sum over dim 2 of in (H, topk, tokens), fp32
+ * accumulation in slot order. */
+int mi_moe_sum_topk(const mi_tile_array* in, const mi_tile_array* out, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* MI355TILE_H */

@@ -1,0 +1,349 @@
+"""CPU oracle for the cuTile.jl example kernels.  TEST INFRASTRUCTURE ONLY.
+
+This module restates, in numpy, the CPU checking code of the reference's examples (their
+``verify`` / ``ref_*`` functions and integer host helpers).  Only ``tests/``,
+``__graft_entry__.smoke()`` and ``bench.py``'s ``cpu_baseline`` leg may import it; the
+product (``cutile.jl_amd``) never does.
+
+Arrays are numpy arrays in the JULIA shape (first dimension fastest in the reference); use
+:func:`to_julia` / :func:`from_julia` to convert from / to the reversed-shape row-major
+torch tensors the product works on.
+
+Every function cites the reference lines it follows.  What pins each function (so that a
+plausible mistake fails a test) is listed in ``tests/test_oracle.py``; summary:
+
+=====================  ======================================================================
+function               pinned by
+=====================  ======================================================================
+vadd, transpose        closed form (IEEE add / permutation); brute force
+swizzle_2d             bijection onto the tile grid, brute force; C restatement cross-check
+matmul, batch_matmul   float64 ``@``; 64x16x64 case of test/device/tile.jl:1036-1066 by loops
+layer_norm_*           invariants (zero-mean/unit-var xhat, sum dx = 0, constant row);
+                       ``torch.nn.functional.layer_norm`` + autograd on CPU
+softmax                columns sum to 1, shift invariance, ``scipy.special.softmax``
+ref_fmha               row 1 of causal output == V[:,1]; brute-force loops on tiny shapes;
+                       ``torch.nn.functional.scaled_dot_product_attention`` on CPU
+moe_align_tile_size    permutation / grouping / padding invariants; brute force; C cross-check
+ref_moe                per-token dense loop on tiny shapes
+e4m3fn codec           16 round-trip vectors and fma vectors of
+                       test/extensions/DLFP8Types.jl:126-141; all 256 codes vs torch.float8_e4m3fn
+=====================  ======================================================================
+
+The reference's device rounding (fma contraction, exp2 / reciprocal approximations, f16
+rounding of P, atomics order) is produced by NVIDIA's closed ``tileiras`` compiler and is
+"parity unpinned" at the bit level; the reference itself only checks it to rtol 1e-2
+against the same CPU formulas restated here.
+"""
+from __future__ import annotations
+
+import math
+
+import numpy as np
+
+
+# ---- layout helpers ----------------------------------------------------------------------
+
+def to_julia(t) -> np.ndarray:
+    """torch tensor (reversed-shape, row-major) -> numpy array in the Julia shape."""
+    import torch
+    if t.dtype == torch.bfloat16:
+        return t.detach().cpu().to(torch.float32).numpy().T
+    return t.detach().cpu().numpy().T
+
+
+def from_julia(a: np.ndarray):
+    """numpy array in the Julia shape -> contiguous torch tensor of the reversed shape."""
+    import torch
+    return torch.from_numpy(np.ascontiguousarray(a.T))
+
+
+def cld(a: int, b: int) -> int:
+    return -(-a // b)
+
+
+# ---- vadd / transpose ----------------------------------------------------------------------
+
+def vadd(a: np.ndarray, b: np.ndarray) -> np.ndarray:
+    """examples/vadd.jl:127-129: ``Array(a) + Array(b)`` in the arrays' own type (IEEE add;
+    Julia's Float16 add widens to Float32 and rounds once, as numpy's float16 add does)."""
+    return a + b
+
+
+def vadd_gather(a: np.ndarray, b: np.ndarray, n_c: int) -> np.ndarray:
+    """vec_add_kernel_1d_gather (vadd.jl:31-45) with possibly different lengths: an index
+    past the end of ``a`` or ``b`` gathers 0 (src/language/operations.jl:996-1009)."""
+    out = np.zeros(n_c, dtype=a.dtype)
+    na, nb = min(n_c, a.shape[0]), min(n_c, b.shape[0])
+    out[:na] += a[:na]
+    out[:nb] += b[:nb]
+    return out
+
+
+def transpose(x: np.ndarray) -> np.ndarray:
+    """examples/transpose.jl:58-60: ``transpose(Array(x))``."""
+    return np.ascontiguousarray(x.T)
+
+
+# ---- swizzle -------------------------------------------------------------------------------
+
+def swizzle_2d(M, N, tm, tn, GROUP_SIZE_M, bid):
+    """examples/matmul.jl:13-24 (dup. examples/moe.jl:20-31): 1-based bid -> 1-based
+    (bid_m, bid_n), grouped ordering."""
+    num_bid_m = cld(M, tm)
+    num_bid_n = cld(N, tn)
+    num_bid_in_group = GROUP_SIZE_M * num_bid_n
+    bid0 = bid - 1
+    group_id = bid0 // num_bid_in_group
+    first_bid_m = group_id * GROUP_SIZE_M
+    group_size_m = min(num_bid_m - first_bid_m, GROUP_SIZE_M)
+    bid_m = first_bid_m + bid0 % group_size_m + 1
+    bid_n = (bid0 % num_bid_in_group) // group_size_m + 1
+    return bid_m, bid_n
+
+
+# ---- matmul --------------------------------------------------------------------------------
+
+def matmul(A: np.ndarray, B: np.ndarray, dtype=np.float64) -> np.ndarray:
+    """examples/matmul.jl:98-101: ``Array(A) * Array(B)``; evaluated in ``dtype``
+    (float64 = the fp32-reference the tolerances are stated against)."""
+    return A.astype(dtype) @ B.astype(dtype)
+
+
+def batch_matmul(A: np.ndarray, B: np.ndarray, dtype=np.float64) -> np.ndarray:
+    """examples/batchmatmul.jl:97-106: per batch ``A[:,:,b] * B[:,:,b]`` (batch is LAST)."""
+    M, K, nb = A.shape
+    N = B.shape[1]
+    out = np.empty((M, N, nb), dtype=dtype, order="F")
+    for b in range(nb):
+        out[:, :, b] = A[:, :, b].astype(dtype) @ B[:, :, b].astype(dtype)
+    return out
+
+
+# ---- layernorm -----------------------------------------------------------------------------
+
+def layer_norm_fwd(X, W, B, eps, dtype=np.float64):
+    """examples/layernorm.jl:284-302.  X is (N, M): reduce along dim 1 (axis 0).  Returns
+    (Y, mean (M,), rstd (M,))."""
+    X = X.astype(dtype); W = W.astype(dtype); B = B.astype(dtype)
+    N = X.shape[0]
+    mean = X.sum(axis=0, keepdims=True) / N
+    var = ((X - mean) ** 2).sum(axis=0, keepdims=True) / N
+    rstd = 1.0 / np.sqrt(var + dtype(eps))
+    xhat = (X - mean) * rstd
+    Y = xhat * W[:, None] + B[:, None]
+    return Y, mean[0], rstd[0]
+
+
+def layer_norm_bwd(X, W, DY, eps, dtype=np.float64):
+    """examples/layernorm.jl:303-313.  Returns (DX (N,M), DW (N,), DB (N,))."""
+    X = X.astype(dtype); W = W.astype(dtype); DY = DY.astype(dtype)
+    N = X.shape[0]
+    mean = X.sum(axis=0, keepdims=True) / N
+    var = ((X - mean) ** 2).sum(axis=0, keepdims=True) / N
+    rstd = 1.0 / np.sqrt(var + dtype(eps))
+    xhat = (X - mean) * rstd
+    wdy = W[:, None] * DY
+    c1 = (xhat * wdy).sum(axis=0, keepdims=True) / N
+    c2 = wdy.sum(axis=0, keepdims=True) / N
+    DX = (wdy - (xhat * c1 + c2)) * rstd
+    DW = (DY * xhat).sum(axis=1)
+    DB = DY.sum(axis=1)
+    return DX, DW, DB
+
+
+# ---- softmax -------------------------------------------------------------------------------
+
+def softmax(x: np.ndarray, dtype=np.float64, rows: int | None = None) -> np.ndarray:
+    """examples/softmax.jl:175-188: per column j, ``exp.(col .- max) ./ sum``.  x is (N, M).
+    ``rows`` limits the softmax to the first ``rows`` rows (a TILE_SIZE smaller than N:
+    the tile at index 1 covers rows 1..TILE_SIZE only, softmax.jl:29-38)."""
+    x = x.astype(dtype)
+    if rows is not None:
+        x = x[:rows]
+    mx = x.max(axis=0, keepdims=True)
+    e = np.exp(x - mx)
+    return e / e.sum(axis=0, keepdims=True)
+
+
+# ---- FMHA ----------------------------------------------------------------------------------
+
+def ref_fmha(Q, K, V, qk_scale=None, causal=False, dtype=np.float32):
+    """examples/fmha.jl:175-220.  Q (D,M,H,B), K (D,N,KH,B), V (Dv,N,KH,B) -> Out (Dv,M,H,B).
+    Causal mask: key j (1-based) > query i is -Inf (no input_pos offset in the reference)."""
+    Q = Q.astype(dtype); K = K.astype(dtype); V = V.astype(dtype)
+    D, M, H, B = Q.shape
+    _, N, KH, _ = K.shape
+    Dv = V.shape[0]
+    if qk_scale is None:
+        qk_scale = dtype(1.0 / math.sqrt(D))
+    out = np.zeros((Dv, M, H, B), dtype=dtype, order="F")
+    group = H // KH
+    for b in range(B):
+        for h in range(H):
+            kh = h // group  # 0-based form of cld(h, H ÷ KH) for 1-based h
+            q = Q[:, :, h, b]; k = K[:, :, kh, b]; v = V[:, :, kh, b]
+            scores = (q.T @ k) * dtype(qk_scale)  # (M, N)
+            if causal:
+                i = np.arange(M)[:, None]; j = np.arange(N)[None, :]
+                scores = np.where(j > i, -np.inf, scores)
+            smax = scores.max(axis=1, keepdims=True)
+            smax = np.where(np.isinf(smax), 0.0, smax)
+            e = np.exp(scores - smax)
+            attn = e / e.sum(axis=1, keepdims=True)
+            out[:, :, h, b] = v @ attn.T
+    return out
+
+
+def fmha_general(Q, K, V, qk_scale=None, causal=False, input_pos=0, dtype=np.float64):
+    """The kernel's own masking rule (fmha.jl:45-46,92-103): query row i (0-based) sits at
+    position ``input_pos + i`` and sees keys ``j <= input_pos + i``.  Equals ref_fmha when
+    input_pos == 0.  Used for the decode-offset cases the reference's ref_fmha cannot
+    express; pinned against ref_fmha at input_pos == 0 and by the all-keys-visible limit."""
+    Q = Q.astype(dtype); K = K.astype(dtype); V = V.astype(dtype)
+    D, M, H, B = Q.shape
+    _, N, KH, _ = K.shape
+    if qk_scale is None:
+        qk_scale = 1.0 / math.sqrt(D)
+    out = np.zeros((V.shape[0], M, H, B), dtype=dtype, order="F")
+    group = H // KH
+    for b in range(B):
+        for h in range(H):
+            kh = h // group
+            s = (Q[:, :, h, b].T @ K[:, :, kh, b]) * qk_scale
+            if causal:
+                i = np.arange(M)[:, None] + input_pos; j = np.arange(N)[None, :]
+                s = np.where(j > i, -np.inf, s)
+            mx = s.max(axis=1, keepdims=True)
+            mx = np.where(np.isinf(mx), 0.0, mx)
+            e = np.exp(s - mx)
+            out[:, :, h, b] = V[:, :, kh, b] @ (e / e.sum(axis=1, keepdims=True)).T
+    return out
+
+
+# ---- MoE -----------------------------------------------------------------------------------
+
+def moe_align_tile_size(topk_ids: np.ndarray, tile_m: int, num_experts: int):
+    """examples/moe.jl:142-183.  topk_ids (num_tokens, topk) of 1-based expert ids.
+    Returns (sorted_token_ids int32 1-based with sentinel total+1, sorted_expert_ids int32)."""
+    num_tokens, topk = topk_ids.shape
+    total = num_tokens * topk
+    flat = topk_ids.reshape(-1)  # row-major of (tokens, topk) == slot fastest (moe.jl:148)
+    perm = np.argsort(flat, kind="stable") + 1
+    counts = np.bincount(flat - 1, minlength=num_experts)
+    blocks = -(-counts // tile_m)
+    total_blocks = int(blocks.sum())
+    tok = np.full(total_blocks * tile_m, total + 1, dtype=np.int32)
+    exp = np.zeros(total_blocks, dtype=np.int32)
+    cur_block = 0
+    cur_tok = 0
+    for e in range(num_experts):
+        tc, bc = int(counts[e]), int(blocks[e])
+        exp[cur_block:cur_block + bc] = e + 1
+        start = cur_block * tile_m
+        tok[start:start + tc] = perm[cur_tok:cur_tok + tc]
+        cur_tok += tc
+        cur_block += bc
+    return tok, exp
+
+
+def silu_and_mul(a: np.ndarray, b: np.ndarray, dtype=np.float64) -> np.ndarray:
+    """examples/moe.jl:110-128: ``a / (1 + exp(-a)) * b``."""
+    a = a.astype(dtype); b = b.astype(dtype)
+    return a / (1.0 + np.exp(-a)) * b
+
+
+def ref_moe(hidden_states, w1, w2, topk_weights, topk_ids, dtype=np.float32):
+    """examples/moe.jl:264-304.  hidden_states (hidden, tokens); w1 (hidden, 2*inter, E);
+    w2 (inter, hidden, E); topk_weights, topk_ids (tokens, topk), ids 1-based."""
+    hs = hidden_states.astype(dtype); w1 = w1.astype(dtype); w2 = w2.astype(dtype)
+    tw = topk_weights.astype(dtype)
+    hidden, num_tokens = hs.shape
+    inter = w2.shape[0]
+    E = w1.shape[2]
+    result = np.zeros((hidden, num_tokens), dtype=dtype, order="F")
+    for eid in range(1, E + 1):
+        tok_idx, slot_idx = np.nonzero(topk_ids == eid)
+        if tok_idx.size == 0:
+            continue
+        tokens = hs[:, tok_idx]
+        w1e = w1[:, :, eid - 1]
+        gate_out = w1e[:, :inter].T @ tokens
+        up_out = w1e[:, inter:].T @ tokens
+        silu_out = gate_out / (1.0 + np.exp(-gate_out)) * up_out
+        expert_out = w2[:, :, eid - 1].T @ silu_out
+        for i, (t, s) in enumerate(zip(tok_idx, slot_idx)):
+            result[:, t] += expert_out[:, i] * tw[t, s]
+    return result
+
+
+def route_top2(logits: np.ndarray, topk: int = 2):
+    """Router of the measured MoE configuration: top-k experts of each token's logits
+    (ties to the lower expert id), softmax over the selected logits.  logits (tokens, E).
+    Returns (topk_weights float32 (tokens, topk), topk_ids int64 1-based (tokens, topk))."""
+    order = np.argsort(-logits, axis=1, kind="stable")[:, :topk]
+    sel = np.take_along_axis(logits, order, axis=1).astype(np.float64)
+    e = np.exp(sel - sel.max(axis=1, keepdims=True))
+    return (e / e.sum(axis=1, keepdims=True)).astype(np.float32), (order + 1).astype(np.int64)
+
+
+# ---- FP8 E4M3FN ----------------------------------------------------------------------------
+
+def e4m3fn_decode(code: np.ndarray) -> np.ndarray:
+    """OCP FP8 E4M3FN -> float32: 1 sign, 4 exponent (bias 7), 3 mantissa bits; no Inf;
+    S.1111.111 is NaN; exponent 0 is subnormal (2^-6 * m/8); max finite 448.  The type the
+    reference maps ``Float8_E4M3FN`` to (ext/DLFP8TypesExt.jl:7-9)."""
+    c = np.asarray(code, dtype=np.uint8).astype(np.int32)
+    s = np.where(c & 0x80, -1.0, 1.0)
+    e = (c >> 3) & 0xF
+    m = c & 0x7
+    val = np.where(e == 0, (m / 8.0) * 2.0 ** -6, (1.0 + m / 8.0) * np.exp2((e - 7).astype(np.float64)))
+    val = np.where((e == 15) & (m == 7), np.nan, val)
+    return (s * val).astype(np.float32)
+
+
+def e4m3fn_encode(x: np.ndarray) -> np.ndarray:
+    """float -> E4M3FN code, round to nearest even (the reference's default conversion
+    rounding, src/compiler/intrinsics/conversions.jl:197), saturating finite values above
+    the largest representable magnitude to NaN as the FN format has no Inf."""
+    x = np.asarray(x, dtype=np.float64)
+    sign = (np.signbit(x)).astype(np.uint8) << 7
+    a = np.abs(x)
+    out = np.zeros(x.shape, dtype=np.uint8)
+    nan = np.isnan(a)
+    with np.errstate(divide="ignore", invalid="ignore"):
+        e = np.floor(np.log2(np.where(a > 0, a, 1.0)))
+    e = np.clip(e, -6, 8)
+    quantum = np.exp2(e - 3)  # spacing of representable values in this binade
+    q = np.rint(a / quantum)  # rint = round half to even
+    val = q * quantum
+    # rounding may carry into the next binade; recompute fields from val
+    with np.errstate(divide="ignore", invalid="ignore"):
+        e2 = np.floor(np.log2(np.where(val > 0, val, 1.0)))
+    e2 = np.clip(e2, -6, 8)
+    is_sub = val < 2.0 ** -6
+    mant = np.where(is_sub, np.rint(val / 2.0 ** -9), np.rint(val / np.exp2(e2 - 3)) - 8)
+    expf = np.where(is_sub, 0, e2 + 7)
+    code = (expf.astype(np.int64) << 3) | mant.astype(np.int64)
+    overflow = val > 448.0
+    code = np.where(overflow | nan, 0x7F, code)
+    out = (code.astype(np.uint8) | sign).astype(np.uint8)
+    return out
+
+
+def quantize_e4m3fn_per_channel(w: np.ndarray):
+    """Weight quantisation of the fp8 MoE configuration: w (K, N, E) -> codes (K, N, E) uint8
+    and scale (N, E) float32 with scale = amax over K / 448 (1 where the channel is zero)."""
+    amax = np.abs(w.astype(np.float32)).max(axis=0)
+    scale = np.where(amax > 0, amax / np.float32(448.0), np.float32(1.0)).astype(np.float32)
+    codes = e4m3fn_encode(w.astype(np.float32) / scale[None])
+    return codes, scale
+
+
+# ---- example verify() criteria -------------------------------------------------------------
+
+def isapprox(x: np.ndarray, y: np.ndarray, rtol: float, atol: float = 0.0) -> bool:
+    """Julia's ``isapprox`` for arrays: ``norm(x-y) <= max(atol, rtol*max(norm(x), norm(y)))``
+    with the 2-norm (used by every example's verify)."""
+    x = np.asarray(x, dtype=np.float64); y = np.asarray(y, dtype=np.float64)
+    d = np.linalg.norm((x - y).ravel())
+    return bool(d <= max(atol, rtol * max(np.linalg.norm(x.ravel()), np.linalg.norm(y.ravel()))))

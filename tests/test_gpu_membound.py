@@ -1,0 +1,239 @@
+"""GPU parity tests for the memory-bound kernels (vadd, transpose, softmax, LayerNorm),
+through the C ABI, against the CPU oracle.  The shape lists are those of the reference
+examples' ``main()`` (vadd.jl:219-248, transpose.jl:137-146, layernorm.jl:340-348,
+softmax.jl:248-256) plus ragged / strided / empty edge cases.
+
+Tolerances.  vadd and transpose: bit-exact.  fp32 kernels: |got - ref| <= 1e-5 * (|ref| +
+max|ref|) element-wise against a float64 evaluation of the reference's formulas (that is,
+relative 1e-5 for elements near the array's scale, and 1e-5 of that scale in absolute
+terms for elements near zero).
+"""
+import numpy as np
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+from cutile_jl_amd.examples import vadd, transpose, layernorm, softmax  # noqa: E402
+
+
+def close_f32(got, ref, tol=1e-5):
+    got = np.asarray(got, dtype=np.float64); ref = np.asarray(ref, dtype=np.float64)
+    scale = np.abs(ref).max()
+    err = np.abs(got - ref)
+    bound = tol * (np.abs(ref) + scale)
+    assert np.all(err <= bound), f"max err {err.max():.3e} (scale {scale:.3e}), worst ratio {np.max(err / bound):.2f}"
+
+
+# ---- vadd ---------------------------------------------------------------------------------
+
+@pytest.mark.parametrize("shape,tile,T,gather", [
+    ((1_024_000,), 1024, torch.float32, False), ((2 ** 20,), 512, torch.float32, False),
+    ((2 ** 18,), 512, torch.float64, False), ((1_024_000,), 1024, torch.float16, False),
+    ((2048, 1024), (32, 32), torch.float32, False), ((1024, 2048), (64, 64), torch.float32, False),
+    ((1024, 512), (32, 32), torch.float64, False), ((1024, 1024), (64, 64), torch.float16, False),
+    ((1_024_000,), 1024, torch.float32, True), ((2 ** 20,), 512, torch.float32, True),
+    ((1_000_003,), 1024, torch.float32, False), ((1001,), 256, torch.float16, False), ((3,), 1, torch.float64, False),
+    ((1000, 37), (32, 32), torch.float32, False), ((70_001,), 1024, torch.bfloat16, False),
+])
+def test_vadd_bit_exact(orc, shape, tile, T, gather):
+    d = vadd.prepare(shape=shape, use_gather=gather, T=T)
+    r = vadd.run(d, tile=tile)
+    ref = orc.from_julia(orc.vadd(orc.to_julia(d.a), orc.to_julia(d.b))) if T != torch.bfloat16 else (d.a.cpu().float() + d.b.cpu().float()).to(T)
+    assert torch.equal(r.c.cpu(), ref.to(T))
+
+
+def test_vadd_strided_views_and_misaligned(ct, orc):
+    rng = np.random.default_rng(0)
+    base = torch.from_numpy(rng.random(4099 * 3, dtype=np.float32)).cuda()
+    a, b = base[1::3], base[2::3]         # stride 3, misaligned start
+    c = torch.zeros(a.shape[0] * 2, device="cuda")[::2]
+    ct.vec_add_kernel_1d(a, b, c, 1024)
+    assert torch.equal(c, a + b)
+    a2 = base[1:4098]; b2 = base[5000:5000 + 4097]; c2 = torch.empty(4097 + 1, device="cuda")[1:]
+    ct.vec_add_kernel_1d(a2, b2, c2, 256)  # dense but only 4-byte aligned
+    assert torch.equal(c2, a2 + b2)
+    # 2-D column-strided view: Julia view(A, 1:100, :) of a (128, 50) array
+    A = torch.from_numpy(rng.random((50, 128), dtype=np.float32)).cuda()
+    B = torch.from_numpy(rng.random((50, 128), dtype=np.float32)).cuda()
+    C = torch.zeros(50, 128, device="cuda")
+    ct.vec_add_kernel_2d(A[:, :100], B[:, :100], C[:, :100], 32, 32)
+    assert torch.equal(C[:, :100], A[:, :100] + B[:, :100]) and torch.all(C[:, 100:] == 0)
+
+
+def test_vadd_gather_out_of_bounds_semantics(ct):
+    """test/device/gather_scatter.jl:75-113: an out-of-bounds gather lane reads 0, an
+    out-of-bounds scatter lane is dropped."""
+    a = torch.ones(16, device="cuda"); b = torch.full((32,), 2.0, device="cuda")
+    c = torch.zeros(32, device="cuda")
+    ct.vec_add_kernel_1d_gather(a, b, c, 32)
+    assert torch.all(c[:16] == 3.0) and torch.all(c[16:] == 2.0)
+    guard = torch.zeros(48, device="cuda")
+    c_small = guard[:16]
+    ct.vec_add_kernel_1d_gather(b, b, c_small, 32)
+    assert torch.all(guard[:16] == 4.0) and torch.all(guard[16:] == 0.0)
+
+
+def test_vadd_full_size_linearity():
+    """Benchmark size (2^27 f32): bit-exact against torch's own IEEE add on the device, and
+    (a+b)-b == a wherever that identity holds on the CPU for a sample."""
+    d = vadd.prepare(benchmark=True)
+    r = vadd.run(d)
+    assert torch.equal(r.c, d.a + d.b)
+    idx = torch.arange(0, 2 ** 27, 4099, device="cuda")
+    ref = d.a[idx].cpu().numpy() + d.b[idx].cpu().numpy()
+    assert np.array_equal(r.c[idx].cpu().numpy(), ref)
+
+
+# ---- transpose ----------------------------------------------------------------------------
+
+@pytest.mark.parametrize("m,n,tm,tn,T", [
+    (256, 256, 32, 32, torch.float32), (512, 512, 64, 64, torch.float32), (256, 512, 32, 64, torch.float32),
+    (1024, 1024, 64, 64, torch.float32), (1024, 512, 64, 64, torch.float32),
+    (100, 37, 32, 32, torch.float32), (1, 1, 64, 64, torch.float32), (65, 129, 64, 64, torch.float16),
+    (384, 200, 64, 64, torch.float16), (130, 66, 16, 16, torch.float64), (4, 1000, 64, 64, torch.float32),
+])
+def test_transpose_bit_exact(orc, m, n, tm, tn, T):
+    d = transpose.prepare(m=m, n=n, T=T)
+    r = transpose.run(d, tm=tm, tn=tn)
+    assert np.array_equal(orc.to_julia(r.y), orc.transpose(orc.to_julia(d.x)))
+
+
+def test_transpose_order_load_known_answer(ct):
+    """test/device/tile.jl:657-698: src = reshape(1:n^2, n, n), dst == transpose(src)."""
+    n = 64
+    src = torch.arange(1, n * n + 1, dtype=torch.float32, device="cuda").reshape(n, n)
+    dst = torch.zeros(n, n, device="cuda")
+    ct.transpose_kernel(src, dst, 16, 16)
+    assert torch.equal(dst, src.T.contiguous())
+
+
+def test_transpose_padded_leading_dimension(ct):
+    rng = np.random.default_rng(1)
+    big = torch.from_numpy(rng.random((40, 96), dtype=np.float32)).cuda()
+    x = big[:, :70]                     # Julia (70, 40) with column stride 96
+    ybig = torch.full((70, 48), -1.0, device="cuda")
+    y = ybig[:, :40]                    # Julia (40, 70) with column stride 48
+    ct.transpose_kernel(x, y, 64, 64)
+    assert torch.equal(y, x.T) and torch.all(ybig[:, 40:] == -1.0)
+
+
+def test_transpose_full_size_involution():
+    d = transpose.prepare(benchmark=True)
+    r = transpose.run(d)
+    assert torch.equal(r.y, d.x.T.contiguous())
+    import cutile_jl_amd as ct
+    back = torch.empty_like(d.x)
+    ct.transpose_kernel(r.y, back, 64, 64)
+    assert torch.equal(back, d.x)
+
+
+# ---- softmax ------------------------------------------------------------------------------
+
+@pytest.mark.parametrize("M,N,T", [(256, 256, torch.float32), (64, 1000, torch.float32), (33, 4096, torch.float32),
+                                   (17, 5000, torch.float32), (8, 16384, torch.float32), (4, 20000, torch.float32),
+                                   (5, 1, torch.float32), (3, 7, torch.float32), (128, 1024, torch.float16)])
+def test_softmax_both_kernels(orc, M, N, T):
+    d = softmax.prepare(M=M, N=N, T=T)
+    r = softmax.run(d)
+    ref = orc.softmax(orc.to_julia(d.input))
+    for got in (r.output_tma, r.output_chunked):
+        g = orc.to_julia(got).astype(np.float64)
+        if T == torch.float32:
+            close_f32(g, ref)
+            assert np.all(np.abs(g - ref) <= 1e-5 * ref + 1e-12)  # relative 1e-5 on every element
+        else:
+            assert np.all(np.abs(g - ref) <= 2e-2 * ref + 1e-7)
+        np.testing.assert_allclose(g.sum(axis=0), 1.0, rtol=1e-5 if T == torch.float32 else 2e-3)
+
+
+def test_softmax_tile_smaller_than_column_and_padding(ct, orc):
+    """A TILE_SIZE below N covers rows 1..TILE_SIZE only (softmax.jl:29-38); the chunked
+    kernel walks cld(n_elems, TILE)*TILE rows, clipped to the array."""
+    d = softmax.prepare(M=9, N=1000)
+    out = torch.full_like(d.input, -7.0)
+    ct.softmax_tma_kernel(out, d.input, 512)
+    close_f32(orc.to_julia(out)[:512], orc.softmax(orc.to_julia(d.input), rows=512))
+    assert torch.all(out[:, 512:] == -7.0)
+    out.fill_(-7.0)
+    ct.softmax_chunked_kernel(out, d.input, 300, 256)      # 2 chunks -> rows 1..512
+    close_f32(orc.to_julia(out)[:512], orc.softmax(orc.to_julia(d.input), rows=512))
+    assert torch.all(out[:, 512:] == -7.0)
+    # strided columns (padded leading dimension) and a different program count
+    big = torch.randn(9, 1100, device="cuda")
+    obig = torch.zeros(9, 1100, device="cuda")
+    ct.softmax_tma_kernel(obig[:, :1000], big[:, :1000], 1024, num_programs=4)
+    close_f32(orc.to_julia(obig[:, :1000]), orc.softmax(orc.to_julia(big[:, :1000])))
+    assert torch.all(obig[:, 1000:] == 0)
+
+
+def test_softmax_full_size_properties(orc):
+    d = softmax.prepare(benchmark=True)
+    r = softmax.run(d)
+    for out in (r.output_tma, r.output_chunked):
+        s = out.double().sum(dim=1)
+        assert torch.all((s - 1).abs() < 1e-5)
+        cols = [0, 1, 2047, 4095]
+        ref = orc.softmax(orc.to_julia(d.input[cols]))
+        close_f32(orc.to_julia(out[cols]), ref)
+    # shift invariance at full size
+    shifted = torch.empty_like(d.input)
+    import cutile_jl_amd as ct
+    ct.softmax_tma_kernel(shifted, d.input + 3.0, 4096)
+    assert torch.allclose(shifted, r.output_tma, rtol=2e-5, atol=1e-9)
+
+
+# ---- LayerNorm ----------------------------------------------------------------------------
+
+@pytest.mark.parametrize("M,N,TILE_N,G", [(256, 256, 256, 64), (512, 512, 512, 64), (1024, 1024, 1024, 64),
+                                          (100, 300, 128, 64), (7, 4096, 1024, 64), (130, 1000, 256, 16),
+                                          (64, 8192, 1024, 64), (5, 16384, 1024, 4), (3, 20000, 1024, 2),
+                                          (1000, 64, 64, 512), (1, 5, 8, 1)])
+def test_layernorm_fwd_bwd(orc, M, N, TILE_N, G):
+    d = layernorm.prepare(M=M, N=N, GROUP_SIZE_M=G)
+    r = layernorm.run(d, TILE_N=TILE_N)
+    X, W, B, DY = (orc.to_julia(t) for t in (d.X, d.W, d.B, d.DY))
+    Y, mean, rstd = orc.layer_norm_fwd(X, W, B, d.eps)
+    DX, DW, DB = orc.layer_norm_bwd(X, W, DY, d.eps)
+    close_f32(orc.to_julia(r.Y), Y)
+    close_f32(orc.to_julia(r.Mean), mean, tol=1e-5 if N > 1 else 1e-5)
+    close_f32(orc.to_julia(r.Rstd), rstd)
+    close_f32(orc.to_julia(r.DX), DX, tol=2e-5)
+    close_f32(orc.to_julia(r.FINAL_DW), DW)
+    close_f32(orc.to_julia(r.FINAL_DB), DB)
+    # the reference's own criterion (layernorm.jl:299,311-313)
+    for got, ref in ((r.Y, Y), (r.DX, DX), (r.FINAL_DW, DW), (r.FINAL_DB, DB)):
+        assert orc.isapprox(ref, orc.to_julia(got), rtol=1e-2)
+
+
+def test_layernorm_partials_accumulate_into_caller_buffers(ct, orc):
+    """The partial kernel ADDS into DW/DB (the reference's critical section loads, adds and
+    stores, layernorm.jl:159-163): pre-loading the slots shifts the final sums by exactly
+    that amount; slot g only receives rows m = g mod GROUP_SIZE_M."""
+    d = layernorm.prepare(M=40, N=256, GROUP_SIZE_M=8)
+    ct.layer_norm_fwd(d.X, d.W, d.B, d.Y, d.Mean, d.Rstd, d.eps, 256)
+    d.DW_partial.zero_(); d.DB_partial.zero_()
+    ct.layer_norm_bwd_dx_partial_dwdb(d.DX, d.DY, d.DW_partial, d.DB_partial, d.X, d.W, d.Mean, d.Rstd, None, 8, 256)
+    DY = orc.to_julia(d.DY).astype(np.float64)
+    db_slots = orc.to_julia(d.DB_partial)
+    for g in range(8):
+        close_f32(db_slots[:, g], DY[:, g::8].sum(axis=1))
+    d.DW_partial.fill_(1.0); d.DB_partial.fill_(2.0)
+    ct.layer_norm_bwd_dx_partial_dwdb(d.DX, d.DY, d.DW_partial, d.DB_partial, d.X, d.W, d.Mean, d.Rstd, d.Locks, 8, 256)
+    ct.layer_norm_bwd_dwdb(d.DW_partial, d.DB_partial, d.FINAL_DW, d.FINAL_DB, 32, 256)
+    _, DW, DB = orc.layer_norm_bwd(orc.to_julia(d.X), orc.to_julia(d.W), DY, d.eps)
+    close_f32(orc.to_julia(d.FINAL_DW), DW + 8.0)
+    close_f32(orc.to_julia(d.FINAL_DB), DB + 16.0)
+
+
+def test_layernorm_full_size(orc):
+    d = layernorm.prepare(benchmark=True)
+    r = layernorm.run(d)
+    X, W, B, DY = (orc.to_julia(t) for t in (d.X, d.W, d.B, d.DY))
+    Y, mean, rstd = orc.layer_norm_fwd(X, W, B, d.eps)
+    DX, DW, DB = orc.layer_norm_bwd(X, W, DY, d.eps)
+    close_f32(orc.to_julia(r.Y), Y)
+    close_f32(orc.to_julia(r.Rstd), rstd)
+    close_f32(orc.to_julia(r.DX), DX, tol=2e-5)
+    close_f32(orc.to_julia(r.FINAL_DW), DW)
+    close_f32(orc.to_julia(r.FINAL_DB), DB)

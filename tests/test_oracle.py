@@ -1,0 +1,314 @@
+"""Pins the CPU oracle (oracle/cutile_oracle.py, oracle/oracle_int.c) without a GPU.
+
+The reference ships no golden files (every reference test draws its inputs in-process), so
+the oracle is pinned by (a) the literal known-answer data the reference's tests do hold,
+(b) independent library routines already in this image (torch CPU, scipy), (c) invariants
+and brute-force loops chosen so that a dropped term, a wrong sign / index or a transposed
+operand fails.  None of these tests retypes the oracle's own formula.
+"""
+import ctypes
+import itertools
+import json
+import math
+import os
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import cutile_oracle as orc
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+ROOT = os.path.dirname(HERE)
+
+
+@pytest.fixture(scope="module")
+def corc():
+    path = os.path.join(ROOT, "oracle", "liboracle_int.so")
+    if not os.path.exists(path):
+        import subprocess
+        subprocess.check_call(["make", "-C", os.path.join(ROOT, "oracle")])
+    lib = ctypes.CDLL(path)
+    lib.oracle_e4m3fn_decode.restype = ctypes.c_float
+    lib.oracle_e4m3fn_decode.argtypes = [ctypes.c_uint8]
+    lib.oracle_e4m3fn_encode.restype = ctypes.c_uint8
+    lib.oracle_e4m3fn_encode.argtypes = [ctypes.c_float]
+    lib.oracle_moe_align_tile_size.restype = ctypes.c_int64
+    return lib
+
+
+# ---- swizzle_2d ---------------------------------------------------------------------------
+
+@pytest.mark.parametrize("M,N,tm,tn,G", [(4096, 4096, 64, 64, 8), (200, 100, 64, 64, 8),
+                                          (1000, 130, 32, 64, 8), (64, 64, 64, 64, 8),
+                                          (9 * 16, 5 * 16, 16, 16, 4), (17 * 8, 3 * 8, 8, 8, 8)])
+def test_swizzle_is_a_bijection_with_grouped_order(M, N, tm, tn, G):
+    nm, nn = orc.cld(M, tm), orc.cld(N, tn)
+    seen = [orc.swizzle_2d(M, N, tm, tn, G, bid) for bid in range(1, nm * nn + 1)]
+    assert sorted(seen) == sorted(itertools.product(range(1, nm + 1), range(1, nn + 1)))
+    # grouped ordering: within the first group the m index cycles fastest over min(G, nm) rows
+    g = min(G, nm)
+    assert [s[0] for s in seen[:g]] == list(range(1, g + 1))
+    assert all(s[1] == 1 for s in seen[:g])
+    # all blocks of group k come before any block of group k+1
+    groups = [(bm - 1) // G for bm, _ in seen]
+    assert groups == sorted(groups)
+
+
+def test_swizzle_c_restatement_agrees(corc):
+    bm, bn = ctypes.c_int32(), ctypes.c_int32()
+    for (M, N, tm, tn, G) in [(4096, 4096, 64, 64, 8), (200, 100, 64, 64, 8), (1000, 130, 32, 64, 8)]:
+        for bid in range(1, orc.cld(M, tm) * orc.cld(N, tn) + 1):
+            corc.oracle_swizzle_2d(M, N, tm, tn, G, bid, ctypes.byref(bm), ctypes.byref(bn))
+            assert (bm.value, bn.value) == orc.swizzle_2d(M, N, tm, tn, G, bid)
+
+
+# ---- matmul -------------------------------------------------------------------------------
+
+def test_matmul_known_case_by_loops():
+    """Shape of test/device/tile.jl:1036-1066 (M,K,N = 64,16,64), checked against scalar loops."""
+    rng = np.random.default_rng(0)
+    A = rng.random((64, 16), dtype=np.float32)
+    B = rng.random((16, 64), dtype=np.float32)
+    C = orc.matmul(A, B)
+    ref = np.zeros((64, 64))
+    for i in range(64):
+        for j in range(64):
+            ref[i, j] = sum(float(A[i, k]) * float(B[k, j]) for k in range(16))
+    np.testing.assert_allclose(C, ref, rtol=1e-12)
+    # not symmetric in its operands: a transposed-operand mistake fails
+    assert not np.allclose(orc.matmul(A, B), orc.matmul(B.T, A.T))
+
+
+def test_batch_matmul_batch_last():
+    rng = np.random.default_rng(1)
+    A = rng.standard_normal((5, 7, 3)); B = rng.standard_normal((7, 4, 3))
+    C = orc.batch_matmul(A, B)
+    assert C.shape == (5, 4, 3)
+    np.testing.assert_allclose(C, np.einsum("mkb,knb->mnb", A, B), rtol=1e-12)
+
+
+# ---- layernorm ----------------------------------------------------------------------------
+
+def test_layernorm_against_torch_autograd():
+    rng = np.random.default_rng(2)
+    N, M, eps = 48, 10, 1e-5
+    X = rng.standard_normal((N, M)); W = rng.standard_normal(N); B = rng.standard_normal(N)
+    DY = rng.standard_normal((N, M))
+    Y, mean, rstd = orc.layer_norm_fwd(X, W, B, eps)
+    DX, DW, DB = orc.layer_norm_bwd(X, W, DY, eps)
+    xt = torch.tensor(X.T.copy(), dtype=torch.float64, requires_grad=True)  # (M, N)
+    wt = torch.tensor(W, dtype=torch.float64, requires_grad=True)
+    bt = torch.tensor(B, dtype=torch.float64, requires_grad=True)
+    yt = torch.nn.functional.layer_norm(xt, (N,), wt, bt, eps)
+    yt.backward(torch.tensor(DY.T.copy()))
+    np.testing.assert_allclose(Y, yt.detach().numpy().T, rtol=1e-10, atol=1e-12)
+    np.testing.assert_allclose(DX, xt.grad.numpy().T, rtol=1e-9, atol=1e-11)
+    np.testing.assert_allclose(DW, wt.grad.numpy(), rtol=1e-10)
+    np.testing.assert_allclose(DB, bt.grad.numpy(), rtol=1e-10)
+    np.testing.assert_allclose(mean, X.mean(axis=0), rtol=1e-12)
+    np.testing.assert_allclose(rstd, 1 / np.sqrt(X.var(axis=0) + eps), rtol=1e-12)  # biased var
+
+
+def test_layernorm_invariants():
+    rng = np.random.default_rng(3)
+    N, M = 64, 6
+    X = rng.standard_normal((N, M)); DY = rng.standard_normal((N, M))
+    ones = np.ones(N)
+    DX, _, _ = orc.layer_norm_bwd(X, ones, DY, 0.0)
+    _, mean, rstd = orc.layer_norm_fwd(X, ones, np.zeros(N), 0.0)
+    xhat = (X - mean) * rstd
+    np.testing.assert_allclose(DX.sum(axis=0), 0, atol=1e-10)           # dx ⟂ 1
+    np.testing.assert_allclose((DX * xhat).sum(axis=0), 0, atol=1e-10)  # dx ⟂ xhat
+    # constant row: var = 0 -> rstd = 1/sqrt(eps), y = b
+    Xc = np.full((N, 2), 3.25)
+    Y, m, r = orc.layer_norm_fwd(Xc, ones, np.full(N, 0.5), 1e-5)
+    np.testing.assert_allclose(r, 1 / math.sqrt(1e-5))
+    np.testing.assert_allclose(Y, 0.5)
+
+
+# ---- softmax ------------------------------------------------------------------------------
+
+def test_softmax_against_scipy_and_invariants():
+    from scipy.special import softmax as sp_softmax
+    rng = np.random.default_rng(4)
+    x = rng.standard_normal((37, 9)) * 2
+    s = orc.softmax(x)
+    np.testing.assert_allclose(s, sp_softmax(x, axis=0), rtol=1e-12)
+    np.testing.assert_allclose(s.sum(axis=0), 1, rtol=1e-12)
+    np.testing.assert_allclose(orc.softmax(x + 5.0), s, rtol=1e-10)
+    part = orc.softmax(x, rows=16)
+    assert part.shape == (16, 9)
+    np.testing.assert_allclose(part, sp_softmax(x[:16], axis=0), rtol=1e-12)
+
+
+# ---- FMHA ---------------------------------------------------------------------------------
+
+def _fmha_loops(Q, K, V, scale, causal, input_pos=0):
+    D, M, H, B = Q.shape
+    N, KH = K.shape[1], K.shape[2]
+    out = np.zeros((V.shape[0], M, H, B))
+    for b in range(B):
+        for h in range(H):
+            kh = h // (H // KH)
+            for i in range(M):
+                s = np.array([sum(Q[d, i, h, b] * K[d, j, kh, b] for d in range(D)) * scale for j in range(N)])
+                if causal:
+                    s[np.arange(N) > i + input_pos] = -np.inf
+                p = np.exp(s - s.max()); p /= p.sum()
+                for j in range(N):
+                    out[:, i, h, b] += p[j] * V[:, j, kh, b]
+    return out
+
+
+@pytest.mark.parametrize("causal", [False, True])
+def test_ref_fmha_brute_force_tiny_gqa(causal):
+    rng = np.random.default_rng(5)
+    D, M, N, H, KH, B = 16, 8, 8, 4, 2, 1
+    Q = rng.standard_normal((D, M, H, B)); K = rng.standard_normal((D, N, KH, B)); V = rng.standard_normal((D, N, KH, B))
+    out = orc.ref_fmha(Q, K, V, causal=causal, dtype=np.float64)
+    np.testing.assert_allclose(out, _fmha_loops(Q, K, V, 1 / math.sqrt(D), causal), rtol=1e-10)
+    if causal:
+        np.testing.assert_allclose(out[:, 0, :, 0], V[:, 0, [0, 0, 1, 1], 0], rtol=1e-12)  # row 1 sees key 1 only
+
+
+def test_ref_fmha_against_torch_sdpa():
+    rng = np.random.default_rng(6)
+    D, M, H, B = 32, 24, 3, 2
+    Q = rng.standard_normal((D, M, H, B)); K = rng.standard_normal((D, M, H, B)); V = rng.standard_normal((D, M, H, B))
+    t = lambda a: torch.tensor(np.ascontiguousarray(a.T))  # (B,H,M,D)
+    for causal in (False, True):
+        ref = torch.nn.functional.scaled_dot_product_attention(t(Q), t(K), t(V), is_causal=causal)
+        np.testing.assert_allclose(orc.ref_fmha(Q, K, V, causal=causal, dtype=np.float64), ref.numpy().T, rtol=1e-9, atol=1e-12)
+
+
+def test_fmha_general_matches_ref_and_offset_limit():
+    rng = np.random.default_rng(7)
+    D, M, N, H, B = 16, 8, 24, 2, 1
+    Q = rng.standard_normal((D, M, H, B)); K = rng.standard_normal((D, N, H, B)); V = rng.standard_normal((D, N, H, B))
+    np.testing.assert_allclose(orc.fmha_general(Q, K, V, causal=True), orc.ref_fmha(Q, K, V, causal=True, dtype=np.float64), rtol=1e-12)
+    # decode offset: brute force, and with input_pos >= N every key is visible == non-causal
+    np.testing.assert_allclose(orc.fmha_general(Q, K, V, causal=True, input_pos=16),
+                               _fmha_loops(Q, K, V, 1 / math.sqrt(D), True, input_pos=16), rtol=1e-10)
+    np.testing.assert_allclose(orc.fmha_general(Q, K, V, causal=True, input_pos=N),
+                               orc.ref_fmha(Q, K, V, causal=False, dtype=np.float64), rtol=1e-12)
+
+
+# ---- MoE ----------------------------------------------------------------------------------
+
+def _random_topk_ids(rng, num_tokens, topk, E):
+    return np.stack([rng.permutation(E)[:topk] + 1 for _ in range(num_tokens)]).astype(np.int64)
+
+
+@pytest.mark.parametrize("num_tokens,topk,E,tile_m", [(48, 8, 64, 128), (7, 2, 4, 4), (256, 2, 32, 128), (5, 3, 3, 2)])
+def test_moe_align_invariants(num_tokens, topk, E, tile_m, corc):
+    rng = np.random.default_rng(8)
+    ids = _random_topk_ids(rng, num_tokens, topk, E)
+    tok, exp = orc.moe_align_tile_size(ids, tile_m, E)
+    total = num_tokens * topk
+    flat = ids.reshape(-1)
+    real = tok[tok != total + 1]
+    assert sorted(real.tolist()) == list(range(1, total + 1))          # each replica exactly once
+    counts = np.bincount(flat - 1, minlength=E)
+    assert len(tok) == tile_m * int(np.sum(-(-counts // tile_m))) and len(exp) * tile_m == len(tok)
+    for blk in range(len(exp)):
+        seg = tok[blk * tile_m:(blk + 1) * tile_m]
+        segr = seg[seg != total + 1]
+        assert np.all(flat[segr - 1] == exp[blk])                      # block holds one expert
+        assert np.all(np.diff(segr) > 0)                               # stable: ascending replica id
+        assert np.all(seg[len(segr):] == total + 1)                    # padding only at the tail
+    assert np.all(np.diff(exp) >= 0)
+    # C restatement (literal stable selection) agrees
+    ids_f = np.asfortranarray(ids)
+    tok_c = np.empty_like(tok); exp_c = np.empty_like(exp)
+    nb = corc.oracle_moe_align_tile_size(ids_f.ctypes.data_as(ctypes.c_void_p), ctypes.c_int64(num_tokens),
+                                         ctypes.c_int64(topk), ctypes.c_int32(tile_m), ctypes.c_int32(E),
+                                         tok_c.ctypes.data_as(ctypes.c_void_p), exp_c.ctypes.data_as(ctypes.c_void_p))
+    assert nb == len(exp)
+    assert np.array_equal(tok_c, tok) and np.array_equal(exp_c, exp)
+
+
+def test_ref_moe_per_token_dense_loop():
+    rng = np.random.default_rng(9)
+    hidden, inter, E, T, topk = 8, 6, 5, 7, 2
+    hs = rng.standard_normal((hidden, T)); w1 = rng.standard_normal((hidden, 2 * inter, E)) * 0.3
+    w2 = rng.standard_normal((inter, hidden, E)) * 0.3
+    ids = _random_topk_ids(rng, T, topk, E); tw = rng.random((T, topk))
+    ref = np.zeros((hidden, T))
+    for t in range(T):
+        for s in range(topk):
+            e = ids[t, s] - 1
+            gu = w1[:, :, e].T @ hs[:, t]
+            g, u = gu[:inter], gu[inter:]
+            act = g * (1 / (1 + np.exp(-g))) * u
+            ref[:, t] += tw[t, s] * (w2[:, :, e].T @ act)
+    np.testing.assert_allclose(orc.ref_moe(hs, w1, w2, tw, ids, dtype=np.float64), ref, rtol=1e-10)
+    np.testing.assert_allclose(orc.silu_and_mul(np.array([0.0, 1.0, -2.0]), np.array([3.0, 2.0, 1.0])),
+                               [0.0, 2 / (1 + math.exp(-1)), -2 / (1 + math.exp(2))], rtol=1e-12)
+
+
+def test_route_top2():
+    logits = np.array([[0.1, 2.0, -1.0, 1.0], [3.0, 3.0, 0.0, -5.0]])
+    w, ids = orc.route_top2(logits)
+    assert ids.tolist() == [[2, 4], [1, 2]]
+    np.testing.assert_allclose(w[0], np.exp([2.0, 1.0]) / np.exp([2.0, 1.0]).sum(), rtol=1e-6)
+    np.testing.assert_allclose(w[1], [0.5, 0.5])
+
+
+# ---- FP8 E4M3FN ---------------------------------------------------------------------------
+
+GOLDEN = json.load(open(os.path.join(HERE, "golden", "dlfp8_vectors.json")))
+
+
+def test_e4m3fn_reference_known_answers(corc):
+    """test/extensions/DLFP8Types.jl:126-141: 16 representable values round-trip bit for bit;
+    the fma vectors are exact in e4m3."""
+    rep = np.array(GOLDEN["representable"], dtype=np.float32)
+    assert np.array_equal(orc.e4m3fn_decode(orc.e4m3fn_encode(rep)), rep)
+    assert [corc.oracle_e4m3fn_decode(corc.oracle_e4m3fn_encode(float(v))) for v in rep] == rep.tolist()
+    a, b, c = (np.array(GOLDEN["fma"][k], dtype=np.float32) for k in ("a", "b", "c"))
+    q = lambda v: orc.e4m3fn_decode(orc.e4m3fn_encode(v))
+    assert np.array_equal(q(q(a) * q(b) + q(c)), a * b + c)
+
+
+def test_e4m3fn_all_codes_against_torch(corc):
+    codes = np.arange(256, dtype=np.uint8)
+    ref = torch.from_numpy(codes).view(torch.float8_e4m3fn).to(torch.float32).numpy()
+    dec = orc.e4m3fn_decode(codes)
+    assert np.array_equal(np.isnan(dec), np.isnan(ref))
+    assert np.array_equal(dec[~np.isnan(ref)], ref[~np.isnan(ref)])
+    cdec = np.array([corc.oracle_e4m3fn_decode(int(c)) for c in codes], dtype=np.float32)
+    assert np.array_equal(cdec[~np.isnan(ref)], ref[~np.isnan(ref)])
+    assert dec[0x7E] == 448.0 and dec[0x08] == 2.0 ** -6 and dec[0x01] == 2.0 ** -9
+    finite = codes[~np.isnan(ref)]
+    assert np.array_equal(orc.e4m3fn_encode(dec[finite]), finite)  # encode∘decode = id (incl. -0)
+
+
+def test_e4m3fn_encode_rne_against_torch_and_c(corc):
+    rng = np.random.default_rng(10)
+    x = np.concatenate([rng.standard_normal(4000) * 3, rng.standard_normal(2000) * 200,
+                        rng.standard_normal(2000) * 0.01,
+                        # exact midpoints between neighbours: ties must go to even
+                        np.array([0.5625 * 2, 1.0625, 1.1875, 2.0 ** -10, 3 * 2.0 ** -10, 17.0, 19.0, 464.0, 463.9, 448.0])]).astype(np.float32)
+    x = x[np.abs(x) < 480]
+    ref = torch.from_numpy(x).to(torch.float8_e4m3fn).view(torch.uint8).numpy()
+    got = orc.e4m3fn_encode(x)
+    assert np.array_equal(got & 0x7F, ref & 0x7F)
+    nz = got & 0x7F != 0
+    assert np.array_equal(got[nz], ref[nz])
+    sub = x[:: 37]
+    assert [corc.oracle_e4m3fn_encode(float(v)) for v in sub] == orc.e4m3fn_encode(sub).tolist()
+
+
+def test_quantize_per_channel_bound():
+    rng = np.random.default_rng(11)
+    w = (rng.standard_normal((64, 12, 3)) * 0.02).astype(np.float32)
+    codes, scale = orc.quantize_e4m3fn_per_channel(w)
+    deq = orc.e4m3fn_decode(codes) * scale[None]
+    assert np.all(np.abs(deq - w) <= np.abs(w) * 2.0 ** -4 + scale[None] * 2.0 ** -10)  # half-ulp of 3 mantissa bits
+    assert np.all(np.abs(orc.e4m3fn_decode(codes)).max(axis=0) == 448.0)
+
+
+def test_isapprox_is_normwise():
+    x = np.array([1.0, 0.0]); y = np.array([1.0, 0.005])
+    assert orc.isapprox(x, y, rtol=1e-2) and not orc.isapprox(x, y, rtol=1e-3)

@@ -1,0 +1,319 @@
+// Fused multi-head attention forward: stand-in for fmha_kernel of the reference's
+// examples/fmha.jl:20-139 (FlashAttention-2 style online softmax).
+//
+// Layout (Julia column-major): Q (D, Sq, H, B), K (D, Skv, KVH, B), V (D, Skv, KVH, B),
+// Out (D, Sq, H, B); D is contiguous, so a query / key / value vector is a contiguous run.
+//
+// Mapping to CDNA4.  A workgroup (4 waves) owns 128 consecutive queries of one (batch, head);
+// a wave owns 32 of them.  KV is walked in tiles of 64 keys staged in LDS.
+//   S^T (keys x queries) = K . Q : MFMA 32x32x16, row operand = K rows read as 16-byte
+//     D-contiguous fragments from an XOR-swizzled LDS tile, column operand = Q fragments
+//     held in registers for the whole kernel (lane % 32 = query).
+//   online softmax in the exp2 domain, entirely in registers: a query's scores live in the
+//     two lanes l and l^32, so row max / row sum need one cross-lane exchange each.
+//   O^T (D x queries) += V . P : the fp32 scores, rounded to the storage type (fmha.jl:124),
+//     are already in column-operand layout (lane % 32 = query, 8 keys per lane); the
+//     matching row operand is read from the V tile with the LDS transpose read, whose
+//     4-consecutive-row granularity matches the accumulator's 4-row groups, so P never
+//     moves between lanes.
+// Causal tile skipping: the KV loop stops at the workgroup's last query, and a wave skips
+// tiles that lie wholly above its own last query.  Masking and the ragged KV tail use -Inf
+// as in the reference (fmha.jl:92-103).
+//
+// FLOPs (causal-exact): 4 * B * H * D * Sq*(Sq+1)/2 for Sq == Skv.
+#include "common.h"
+#include <math.h>
+
+namespace {
+
+using namespace mi;
+
+typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef short s16x4 __attribute__((ext_vector_type(4)));
+typedef short s16x8 __attribute__((ext_vector_type(8)));
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+
+#define LDS_PTR(T, p) ((T __attribute__((address_space(3)))*)(p))
+
+struct F16 {
+    static __device__ __forceinline__ f32x16 mfma32(s16x8 a, s16x8 b, f32x16 c) {
+        return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, a), __builtin_bit_cast(f16x8, b), c, 0, 0, 0);
+    }
+    static __device__ __forceinline__ short cvt(float v) {
+        _Float16 h = (_Float16)v;
+        return __builtin_bit_cast(short, h);
+    }
+};
+struct BF16 {
+    static __device__ __forceinline__ f32x16 mfma32(s16x8 a, s16x8 b, f32x16 c) {
+        return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
+    }
+    static __device__ __forceinline__ short cvt(float v) {
+        unsigned u = __float_as_uint(v);
+        if ((u & 0x7fffffffu) > 0x7f800000u) return (short)((u >> 16) | 0x40);
+        u += 0x7fffu + ((u >> 16) & 1u);
+        return (short)(u >> 16);
+    }
+};
+
+constexpr int kQB = 128;  // queries per workgroup
+constexpr int kKV = 64;   // keys per LDS tile
+
+// Row operand for P.V from the V tile stored [key][d] (d contiguous, `pitch` elements per
+// key): lane l gets column d0 + l%32 and the 8 keys {4h+0..3, 8+4h+0..3} (h = l/32) of the
+// 16-key chunk starting at `base` — exactly the keys whose scores the lane holds in
+// accumulator registers 8c..8c+7 of a 32x32 S tile.
+__device__ __forceinline__ s16x8 lds_read_v_frag(const unsigned short* base, int pitch, int lane) {
+    const int g = lane >> 4, r = lane & 15;
+    const unsigned short* p = base + (4 * (g >> 1) + (r >> 2)) * pitch + 16 * (g & 1) + 4 * (r & 3);
+    s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16(LDS_PTR(s16x4, p));
+    s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(LDS_PTR(s16x4, p + 8 * pitch));
+    return __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+}
+
+struct Strides {
+    int64_t s1, s2, s3;  // element strides of dims 1..3 (dim 0 is contiguous)
+};
+
+template <typename E, int D, bool CAUSAL>
+__global__ __launch_bounds__(256) void fmha_fwd_kernel(const unsigned short* __restrict__ Q, Strides qs,
+                                                       const unsigned short* __restrict__ K, Strides ks,
+                                                       const unsigned short* __restrict__ V, Strides vs,
+                                                       unsigned short* __restrict__ O, Strides os, int Sq,
+                                                       int Skv, int H, int group, float scale2,
+                                                       int input_pos, bool vec_ok) {
+    constexpr int CH = D / 8;             // 16-byte chunks per row
+    constexpr int PER_T = kKV * CH / 256;  // chunks per thread per tile
+    constexpr int KSTEPS = D / 16;
+    constexpr int DT = D / 32;            // 32-wide d tiles of the output
+    constexpr int VP = D + 8;             // V tile pitch (elements): rows 4 apart hit distinct banks
+    __shared__ __attribute__((aligned(16))) unsigned short Ks[kKV * D];
+    __shared__ __attribute__((aligned(16))) unsigned short Vs[kKV * VP];
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, hb = lane >> 5;
+    const int nqb = gridDim.x;
+    const int qb = CAUSAL ? nqb - 1 - (int)blockIdx.x : (int)blockIdx.x;  // heavy tiles first
+    const int batch = blockIdx.y / H, head = blockIdx.y % H, kvh = head / group;
+    const int q0 = qb * kQB, qw0 = q0 + wave * 32;
+    Q += (int64_t)head * qs.s2 + (int64_t)batch * qs.s3;
+    O += (int64_t)head * os.s2 + (int64_t)batch * os.s3;
+    K += (int64_t)kvh * ks.s2 + (int64_t)batch * ks.s3;
+    V += (int64_t)kvh * vs.s2 + (int64_t)batch * vs.s3;
+
+    // Q fragments: lane holds query qw0 + lane%32, d = 16*s + 8*hb + 0..7 for every k-step s.
+    const int my_q = qw0 + (lane & 31);
+    s16x8 qf[KSTEPS];
+#pragma unroll
+    for (int s = 0; s < KSTEPS; ++s) {
+        s16x8 v = {0};
+        if (my_q < Sq) {
+            const unsigned short* p = Q + (int64_t)my_q * qs.s1 + 16 * s + 8 * hb;
+            if (vec_ok) v = *reinterpret_cast<const s16x8*>(p);
+            else
+#pragma unroll
+                for (int e = 0; e < 8; ++e) v[e] = (short)p[e];
+        }
+        qf[s] = v;
+    }
+
+    int kv_end = Skv;
+    if (CAUSAL) {
+        const int lim = input_pos + q0 + kQB;  // one past the last query position of the group
+        kv_end = lim < Skv ? lim : Skv;
+        if (kv_end < 0) kv_end = 0;
+    }
+    const int ntiles = (kv_end + kKV - 1) / kKV;
+    const int my_pos = input_pos + my_q;              // this lane's query position
+    const int wave_last_pos = input_pos + qw0 + 31;   // last query position of the wave
+
+    f32x16 o[DT];
+#pragma unroll
+    for (int t = 0; t < DT; ++t) o[t] = f32x16{0};
+    float m_i = -INFINITY, l_i = 0.f;
+
+    s16x8 kreg[PER_T], vreg[PER_T];
+    auto load_tile = [&](int t) {
+#pragma unroll
+        for (int i = 0; i < PER_T; ++i) {
+            const int id = tid + 256 * i, key = id / CH, c = id % CH;
+            const int gk = t * kKV + key;
+            s16x8 a = {0}, b = {0};
+            if (gk < Skv) {
+                const unsigned short* pk = K + (int64_t)gk * ks.s1 + 8 * c;
+                const unsigned short* pv = V + (int64_t)gk * vs.s1 + 8 * c;
+                if (vec_ok) {
+                    a = *reinterpret_cast<const s16x8*>(pk);
+                    b = *reinterpret_cast<const s16x8*>(pv);
+                } else {
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) { a[e] = (short)pk[e]; b[e] = (short)pv[e]; }
+                }
+            }
+            kreg[i] = a;
+            vreg[i] = b;
+        }
+    };
+    if (ntiles > 0) load_tile(0);
+
+    for (int t = 0; t < ntiles; ++t) {
+        __syncthreads();  // every wave has finished reading the previous tile
+#pragma unroll
+        for (int i = 0; i < PER_T; ++i) {
+            const int id = tid + 256 * i, key = id / CH, c = id % CH;
+            *reinterpret_cast<s16x8*>(&Ks[key * D + 8 * (c ^ (key & 7))]) = kreg[i];
+            *reinterpret_cast<s16x8*>(&Vs[key * VP + 8 * c]) = vreg[i];
+        }
+        __syncthreads();
+        if (t + 1 < ntiles) load_tile(t + 1);  // in flight while this tile is computed
+
+        const int kv0 = t * kKV;
+        if (CAUSAL && kv0 > wave_last_pos) continue;  // tile wholly above this wave's queries
+
+        // ---- S^T = K . Q ---------------------------------------------------------------
+        f32x16 s[2] = {f32x16{0}, f32x16{0}};
+#pragma unroll
+        for (int kt = 0; kt < 2; ++kt) {
+            const int key = 32 * kt + (lane & 31);
+#pragma unroll
+            for (int st = 0; st < KSTEPS; ++st) {
+                const int c = 2 * st + hb;
+                s16x8 kf = *reinterpret_cast<const s16x8*>(&Ks[key * D + 8 * (c ^ (key & 7))]);
+                s[kt] = E::mfma32(kf, qf[st], s[kt]);
+            }
+        }
+        // ---- mask: causal diagonal and ragged KV tail -------------------------------------
+        const bool need_mask = (CAUSAL && kv0 + kKV - 1 > input_pos + qw0) || (kv0 + kKV > Skv);
+        if (need_mask) {
+#pragma unroll
+            for (int kt = 0; kt < 2; ++kt)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) {
+                    const int key = kv0 + 32 * kt + 8 * (r >> 2) + 4 * hb + (r & 3);
+                    const bool ok = key < Skv && (!CAUSAL || key <= my_pos);
+                    s[kt][r] = ok ? s[kt][r] : -INFINITY;
+                }
+        }
+        // ---- online softmax (exp2 domain) ----------------------------------------------------
+        float mx = -INFINITY;
+#pragma unroll
+        for (int kt = 0; kt < 2; ++kt)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) mx = fmaxf(mx, s[kt][r]);
+        mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+        const float m_new = fmaxf(m_i, mx * scale2);
+        const float alpha = __builtin_amdgcn_exp2f(m_i - m_new);
+        float rs = 0.f;
+        s16x8 pf[2][2];
+#pragma unroll
+        for (int kt = 0; kt < 2; ++kt)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const float p = __builtin_amdgcn_exp2f(s[kt][r] * scale2 - m_new);
+                rs += p;
+                pf[kt][r >> 3][r & 7] = E::cvt(p);
+            }
+        rs += __shfl_xor(rs, 32, 64);
+        l_i = l_i * alpha + rs;
+        m_i = m_new;
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) o[dt][r] *= alpha;
+        // ---- O^T += V . P ------------------------------------------------------------------------
+#pragma unroll
+        for (int kt = 0; kt < 2; ++kt)
+#pragma unroll
+            for (int c = 0; c < 2; ++c)
+#pragma unroll
+                for (int dt = 0; dt < DT; ++dt) {
+                    s16x8 vf = lds_read_v_frag(&Vs[(32 * kt + 16 * c) * VP + 32 * dt], VP, lane);
+                    o[dt] = E::mfma32(vf, pf[kt][c], o[dt]);
+                }
+    }
+
+    // ---- epilogue: O / l (approximate reciprocal, fmha.jl:132-134), round, store -------------
+    if (my_q < Sq) {
+        const float inv = __builtin_amdgcn_rcpf(l_i);
+        unsigned short* op = O + (int64_t)my_q * os.s1;
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+            for (int g = 0; g < 4; ++g) {
+                s16x4 w;
+#pragma unroll
+                for (int e = 0; e < 4; ++e) w[e] = E::cvt(o[dt][4 * g + e] * inv);
+                unsigned short* dst = op + 32 * dt + 8 * g + 4 * hb;
+                if (vec_ok) *reinterpret_cast<s16x4*>(dst) = w;
+                else
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) dst[e] = (unsigned short)w[e];
+            }
+    }
+}
+
+bool vec16(const mi_tile_array* a) {
+    return aligned(a->ptr, 16) && a->strides[1] % 8 == 0 && a->strides[2] % 8 == 0 && a->strides[3] % 8 == 0;
+}
+
+template <typename E, int D>
+void launch(dim3 grid, hipStream_t s, bool causal, const mi_tile_array* Q, const mi_tile_array* K,
+            const mi_tile_array* V, const mi_tile_array* O, int H, int group, float scale2, int input_pos,
+            bool vec_ok) {
+    Strides qs{Q->strides[1], Q->strides[2], Q->strides[3]}, ks{K->strides[1], K->strides[2], K->strides[3]},
+        vs{V->strides[1], V->strides[2], V->strides[3]}, os{O->strides[1], O->strides[2], O->strides[3]};
+    const int Sq = (int)Q->sizes[1], Skv = (int)K->sizes[1];
+    if (causal)
+        hipLaunchKernelGGL((fmha_fwd_kernel<E, D, true>), grid, dim3(256), 0, s, (const unsigned short*)Q->ptr, qs,
+                           (const unsigned short*)K->ptr, ks, (const unsigned short*)V->ptr, vs,
+                           (unsigned short*)O->ptr, os, Sq, Skv, H, group, scale2, input_pos, vec_ok);
+    else
+        hipLaunchKernelGGL((fmha_fwd_kernel<E, D, false>), grid, dim3(256), 0, s, (const unsigned short*)Q->ptr, qs,
+                           (const unsigned short*)K->ptr, ks, (const unsigned short*)V->ptr, vs,
+                           (unsigned short*)O->ptr, os, Sq, Skv, H, group, scale2, input_pos, vec_ok);
+}
+
+}  // namespace
+
+extern "C" int mi_fmha_kernel(const mi_tile_array* Q, const mi_tile_array* K, const mi_tile_array* V,
+                              const mi_tile_array* Out, float qk_scale, int32_t input_pos, int TILE_D, int H,
+                              int TILE_M, int TILE_N, int QUERY_GROUP_SIZE, int CAUSAL, int EVEN_K, void* stream) {
+    MI_CHECK(check_array(Q, 4));
+    MI_CHECK(check_array(K, 4));
+    MI_CHECK(check_array(V, 4));
+    MI_CHECK(check_array(Out, 4));
+    const int dt = Q->dtype;
+    if (dt != MI_F16 && dt != MI_BF16) return MI_E_DTYPE;
+    if (K->dtype != dt || V->dtype != dt || Out->dtype != dt) return MI_E_DTYPE;
+    if (!is_pow2(TILE_D) || !is_pow2(TILE_M) || !is_pow2(TILE_N)) return MI_E_TILE;
+    if (QUERY_GROUP_SIZE < 1 || H < 1) return MI_E_ARG;
+    const int64_t D = Q->sizes[0], Sq = Q->sizes[1], Hq = Q->sizes[2], B = Q->sizes[3];
+    const int64_t Skv = K->sizes[1], KVH = K->sizes[2];
+    if (K->sizes[0] != D || V->sizes[0] != D || Out->sizes[0] != D || TILE_D != D) return MI_E_SHAPE;
+    if (Hq != H || KVH * QUERY_GROUP_SIZE != H || V->sizes[1] != Skv || V->sizes[2] != KVH) return MI_E_SHAPE;
+    if (K->sizes[3] != B || V->sizes[3] != B || Out->sizes[3] != B || Out->sizes[1] != Sq || Out->sizes[2] != H)
+        return MI_E_SHAPE;
+    if ((EVEN_K != 0) != (Skv % TILE_N == 0)) return MI_E_ARG;  // fmha.jl:153
+    if (input_pos < 0) return MI_E_ARG;
+    if (D != 64 && D != 128) return MI_E_UNSUPPORTED;
+    for (const mi_tile_array* a : {Q, K, V, Out})
+        if (a->strides[0] != 1) return MI_E_STRIDE;
+    if (Sq > 0x3fffffff || Skv > 0x3fffffff) return MI_E_SHAPE;
+    if (cld(Sq, (int64_t)TILE_M) > MI_MAX_GRID_DIM || B * H > 65535) return MI_E_GRID;
+    if (Sq == 0 || B == 0) return MI_OK;
+    if (Skv == 0) return MI_E_SHAPE;
+    const bool vec_ok = vec16(Q) && vec16(K) && vec16(V) && vec16(Out);
+    const float scale2 = qk_scale * 1.4426950408889634f;  // fmha.jl:41: fold 1/log(2) for exp2
+    dim3 grid((unsigned)cld(Sq, (int64_t)kQB), (unsigned)(B * H));
+    hipStream_t s = (hipStream_t)stream;
+    const bool causal = CAUSAL != 0;
+    if (dt == MI_F16) {
+        if (D == 64) launch<F16, 64>(grid, s, causal, Q, K, V, Out, H, QUERY_GROUP_SIZE, scale2, input_pos, vec_ok);
+        else launch<F16, 128>(grid, s, causal, Q, K, V, Out, H, QUERY_GROUP_SIZE, scale2, input_pos, vec_ok);
+    } else {
+        if (D == 64) launch<BF16, 64>(grid, s, causal, Q, K, V, Out, H, QUERY_GROUP_SIZE, scale2, input_pos, vec_ok);
+        else launch<BF16, 128>(grid, s, causal, Q, K, V, Out, H, QUERY_GROUP_SIZE, scale2, input_pos, vec_ok);
+    }
+    set_variant(D == 64 ? "fmha_q128_kv64_d64_mfma32" : "fmha_q128_kv64_d128_mfma32");
+    return launch_status();
+}

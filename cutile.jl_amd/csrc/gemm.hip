@@ -1,0 +1,331 @@
+// Matrix multiplication: stand-ins for matmul_kernel (examples/matmul.jl:28-60) and
+// batch_matmul_kernel (examples/batchmatmul.jl:15-56) of the reference.
+//
+// C(M,N) = A(M,K) * B(K,N), all column-major (first index contiguous), fp32 accumulation.
+// In memory A is "M-contiguous" (row k of A^T holds M consecutive values) and B is
+// "K-contiguous" (column n of B holds K consecutive values).  CDNA4 MFMA wants, for both
+// operands, the K values of one row/column packed in a lane; B has that shape already, A is
+// brought to it with the LDS transpose read ds_read_b64_tr_b16.  The MFMA's row operand
+// carries n and its column operand (lane % 32) carries m, so that the 32 lanes of a
+// half-wave hold 32 consecutive m of one column of C and every store is a full 128-byte
+// line.
+//
+// Kernels:
+//   gemm16_generic   f16/bf16, 64x64x32 workgroup tile, any shape / stride / alignment
+//                    (ragged edges are zero-padded on load and clipped on store, as
+//                    ct.load(padding_mode=Zero) / ct.store do).
+//   gemm16_big       f16/bf16, 256x256x64 workgroup tile, 4 waves of 128x128, direct
+//                    global->LDS loads, double-buffered LDS, XOR-swizzled LDS layouts;
+//                    used when M,N are multiples of 256, K of 64 and everything is 16-byte
+//                    aligned.
+//   gemm32           fp32 via v_mfma_f32_32x32x2_f32 (gfx950 has no TF32-class MFMA;
+//                    the reference rounds fp32 operands to TF32, matmul.jl:49-52).
+//
+// The (tm, tn, tk) tile constants of the reference only fix the block->data mapping and
+// the L2 swizzle; results do not depend on them, and the physical tiling above is chosen
+// for CDNA4.  FLOP count: 2*M*N*K per batch.
+#include "common.h"
+
+namespace {
+
+using namespace mi;
+
+typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
+typedef _Float16 f16x4 __attribute__((ext_vector_type(4)));
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef short s16x4 __attribute__((ext_vector_type(4)));
+typedef short s16x8 __attribute__((ext_vector_type(8)));
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
+
+#define LDS_PTR(T, p) ((T __attribute__((address_space(3)))*)(p))
+
+// 16-bit element traits: raw storage is `short`; the MFMA picks the interpretation.
+struct F16 {
+    static __device__ __forceinline__ f32x16 mfma32(s16x8 a, s16x8 b, f32x16 c) {
+        return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, a),
+                                                      __builtin_bit_cast(f16x8, b), c, 0, 0, 0);
+    }
+    static __device__ __forceinline__ unsigned short from_f32(float v) {
+        _Float16 h = (_Float16)v;
+        return __builtin_bit_cast(unsigned short, h);
+    }
+};
+struct BF16 {
+    static __device__ __forceinline__ f32x16 mfma32(s16x8 a, s16x8 b, f32x16 c) {
+        return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a),
+                                                       __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
+    }
+    static __device__ __forceinline__ unsigned short from_f32(float v) {
+        unsigned u = __float_as_uint(v);
+        if ((u & 0x7fffffffu) > 0x7f800000u) return (unsigned short)((u >> 16) | 0x40);
+        u += 0x7fffu + ((u >> 16) & 1u);
+        return (unsigned short)(u >> 16);
+    }
+};
+
+template <typename E, typename OutT> __device__ __forceinline__ OutT cvt_out(float v);
+template <> __device__ __forceinline__ float cvt_out<F16, float>(float v) { return v; }
+template <> __device__ __forceinline__ float cvt_out<BF16, float>(float v) { return v; }
+template <> __device__ __forceinline__ unsigned short cvt_out<F16, unsigned short>(float v) {
+    return F16::from_f32(v);
+}
+template <> __device__ __forceinline__ unsigned short cvt_out<BF16, unsigned short>(float v) {
+    return BF16::from_f32(v);
+}
+
+// Transposed LDS fragment read.  `base` points at element (row k0, column m0) of an LDS
+// tile stored [k][m] with m contiguous and `pitch` elements per row.  The wave gets the
+// MFMA column operand for columns m0..m0+31 and the 16 k rows k0..k0+15: lane l holds
+// column m0 + l%32 and rows k0 + 8*(l/32) + 0..7.  Two ds_read_b64_tr_b16 per lane: within
+// each group of 16 lanes, lane r reads 4 consecutive m of row (r/4) and receives the
+// 4 consecutive rows of column (group base + r).
+__device__ __forceinline__ s16x8 lds_read_tr_k16(const unsigned short* base, int pitch, int lane) {
+    const int g = lane >> 4, r = lane & 15;
+    const unsigned short* p = base + (8 * (g >> 1) + (r >> 2)) * pitch + 16 * (g & 1) + 4 * (r & 3);
+    s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16(LDS_PTR(s16x4, p));
+    s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(LDS_PTR(s16x4, p + 4 * pitch));
+    return __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+}
+
+// ---- generic 16-bit kernel ---------------------------------------------------------------
+// Workgroup tile 64(m) x 64(n), K step 32, 4 waves as 2x2 of 32x32.
+constexpr int GT = 64, GK = 32, GA_PITCH = GT + 8, GB_PITCH = GK + 8;
+
+template <typename E, typename OutT>
+__global__ __launch_bounds__(256) void gemm16_generic(
+    const unsigned short* __restrict__ A, int64_t lda, int64_t sa, const unsigned short* __restrict__ B,
+    int64_t ldb, int64_t sb, OutT* __restrict__ C, int64_t ldc, int64_t sc, int M, int N, int K,
+    int tiles_m, bool vecA, bool vecB) {
+    __shared__ __attribute__((aligned(16))) unsigned short As[GK * GA_PITCH];  // [k][m]
+    __shared__ __attribute__((aligned(16))) unsigned short Bs[GT * GB_PITCH];  // [n][k]
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int bm = blockIdx.x % tiles_m, bn = blockIdx.x / tiles_m;
+    const int64_t m0 = (int64_t)bm * GT, n0 = (int64_t)bn * GT;
+    A += (int64_t)blockIdx.z * sa;
+    B += (int64_t)blockIdx.z * sb;
+    C += (int64_t)blockIdx.z * sc;
+    const int wm = (wave & 1) * 32, wn = (wave >> 1) * 32;
+
+    const int ak = tid >> 3, am = (tid & 7) * 8;  // A tile: row k, 8 consecutive m
+    const int bnn = tid >> 2, bk = (tid & 3) * 8;  // B tile: column n, 8 consecutive k
+    f32x16 acc = {0};
+
+    for (int k0 = 0; k0 < K; k0 += GK) {
+        s16x8 va = {0}, vb = {0};
+        {
+            const int64_t gm = m0 + am;
+            const int gk = k0 + ak;
+            if (gk < K) {
+                const unsigned short* p = A + gm + (int64_t)gk * lda;
+                if (vecA && gm + 8 <= M) va = *reinterpret_cast<const s16x8*>(p);
+                else
+#pragma unroll
+                    for (int q = 0; q < 8; ++q) va[q] = (gm + q < M) ? (short)p[q] : (short)0;
+            }
+            const int64_t gn = n0 + bnn;
+            const int gk2 = k0 + bk;
+            if (gn < N) {
+                const unsigned short* p = B + gk2 + gn * ldb;
+                if (vecB && gk2 + 8 <= K) vb = *reinterpret_cast<const s16x8*>(p);
+                else
+#pragma unroll
+                    for (int q = 0; q < 8; ++q) vb[q] = (gk2 + q < K) ? (short)p[q] : (short)0;
+            }
+        }
+        __syncthreads();  // previous iteration's fragment reads are done
+        *reinterpret_cast<s16x8*>(&As[ak * GA_PITCH + am]) = va;
+        *reinterpret_cast<s16x8*>(&Bs[bnn * GB_PITCH + bk]) = vb;
+        __syncthreads();
+#pragma unroll
+        for (int ks = 0; ks < GK / 16; ++ks) {
+            s16x8 fn = *reinterpret_cast<const s16x8*>(&Bs[(wn + (lane & 31)) * GB_PITCH + ks * 16 + 8 * (lane >> 5)]);
+            s16x8 fm = lds_read_tr_k16(&As[(ks * 16) * GA_PITCH + wm], GA_PITCH, lane);
+            acc = E::mfma32(fn, fm, acc);
+        }
+    }
+    const int64_t gm = m0 + wm + (lane & 31);
+    if (gm < M) {
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+            const int64_t gn = n0 + wn + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
+            if (gn < N) C[gm + gn * ldc] = cvt_out<E, OutT>(acc[r]);
+        }
+    }
+}
+
+// ---- fp32 kernel ---------------------------------------------------------------------------
+// Workgroup tile 128(m) x 128(n), K step 16, 4 waves as 2x2 of 64x64 (2x2 MFMA 32x32x2).
+constexpr int FT = 128, FK = 16, F_PITCH = FT + 32;
+
+__global__ __launch_bounds__(256) void gemm32_kernel(const float* __restrict__ A, int64_t lda, int64_t sa,
+                                                     const float* __restrict__ B, int64_t ldb, int64_t sb,
+                                                     float* __restrict__ C, int64_t ldc, int64_t sc, int M,
+                                                     int N, int K, int tiles_m, bool vecA, bool vecB) {
+    __shared__ __attribute__((aligned(16))) float As[FK * F_PITCH];  // [k][m]
+    __shared__ __attribute__((aligned(16))) float Bs[FK * F_PITCH];  // [k][n]
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int bm = blockIdx.x % tiles_m, bn = blockIdx.x / tiles_m;
+    const int64_t m0 = (int64_t)bm * FT, n0 = (int64_t)bn * FT;
+    A += (int64_t)blockIdx.z * sa;
+    B += (int64_t)blockIdx.z * sb;
+    C += (int64_t)blockIdx.z * sc;
+    const int wm = (wave & 1) * 64, wn = (wave >> 1) * 64;
+    const int ak = tid >> 4, am = (tid & 15) * 8;  // A tile: row k, 8 consecutive m
+    const int bnn = tid >> 1, bk = (tid & 1) * 8;  // B tile: column n, 8 consecutive k
+    f32x16 acc[2][2] = {};
+
+    for (int k0 = 0; k0 < K; k0 += FK) {
+        float va[8], vb[8];
+        {
+            const int64_t gm = m0 + am;
+            const int gk = k0 + ak;
+            const float* p = A + gm + (int64_t)gk * lda;
+            if (gk < K && vecA && gm + 8 <= M) {
+                f32x4 t0 = *reinterpret_cast<const f32x4*>(p), t1 = *reinterpret_cast<const f32x4*>(p + 4);
+#pragma unroll
+                for (int q = 0; q < 4; ++q) { va[q] = t0[q]; va[4 + q] = t1[q]; }
+            } else {
+#pragma unroll
+                for (int q = 0; q < 8; ++q) va[q] = (gk < K && gm + q < M) ? p[q] : 0.f;
+            }
+            const int64_t gn = n0 + bnn;
+            const int gk2 = k0 + bk;
+            const float* pb = B + gk2 + gn * ldb;
+            if (gn < N && vecB && gk2 + 8 <= K) {
+                f32x4 t0 = *reinterpret_cast<const f32x4*>(pb), t1 = *reinterpret_cast<const f32x4*>(pb + 4);
+#pragma unroll
+                for (int q = 0; q < 4; ++q) { vb[q] = t0[q]; vb[4 + q] = t1[q]; }
+            } else {
+#pragma unroll
+                for (int q = 0; q < 8; ++q) vb[q] = (gn < N && gk2 + q < K) ? pb[q] : 0.f;
+            }
+        }
+        __syncthreads();
+#pragma unroll
+        for (int q = 0; q < 8; ++q) As[ak * F_PITCH + am + q] = va[q];
+#pragma unroll
+        for (int q = 0; q < 8; ++q) Bs[(bk + q) * F_PITCH + bnn] = vb[q];
+        __syncthreads();
+#pragma unroll
+        for (int kk = 0; kk < FK; kk += 2) {
+            float fm[2], fn[2];
+#pragma unroll
+            for (int i = 0; i < 2; ++i) {
+                fm[i] = As[(kk + (lane >> 5)) * F_PITCH + wm + 32 * i + (lane & 31)];
+                fn[i] = Bs[(kk + (lane >> 5)) * F_PITCH + wn + 32 * i + (lane & 31)];
+            }
+#pragma unroll
+            for (int i = 0; i < 2; ++i)
+#pragma unroll
+                for (int j = 0; j < 2; ++j)
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(fn[j], fm[i], acc[i][j], 0, 0, 0);
+        }
+    }
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+        const int64_t gm = m0 + wm + 32 * i + (lane & 31);
+        if (gm >= M) continue;
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const int64_t gn = n0 + wn + 32 * j + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
+                if (gn < N) C[gm + gn * ldc] = acc[i][j][r];
+            }
+    }
+}
+
+// ---- host side -------------------------------------------------------------------------------
+
+struct Problem {
+    const void *A, *B;
+    void* C;
+    int64_t lda, ldb, ldc, sa, sb, sc;
+    int M, N, K, batch;
+    int in_dtype, out_dtype;
+};
+
+int validate(const mi_tile_array* A, const mi_tile_array* B, const mi_tile_array* C, int ndim, int tm,
+             int tn, int tk, Problem* p) {
+    MI_CHECK(check_array(A, ndim));
+    MI_CHECK(check_array(B, ndim));
+    MI_CHECK(check_array(C, ndim));
+    if (A->dtype != B->dtype) return MI_E_DTYPE;
+    if (A->dtype != MI_F16 && A->dtype != MI_BF16 && A->dtype != MI_F32) return MI_E_DTYPE;
+    if (C->dtype != A->dtype && C->dtype != MI_F32) return MI_E_DTYPE;
+    if (!is_pow2(tm) || !is_pow2(tn) || !is_pow2(tk)) return MI_E_TILE;
+    const int64_t M = A->sizes[0], K = A->sizes[1], N = B->sizes[1];
+    if (B->sizes[0] != K || C->sizes[0] != M || C->sizes[1] != N) return MI_E_SHAPE;
+    int64_t batch = 1;
+    if (ndim == 3) {
+        batch = A->sizes[2];
+        if (B->sizes[2] != batch || C->sizes[2] != batch) return MI_E_SHAPE;
+        if (batch > 65535) return MI_E_GRID;
+    }
+    if (M > 0x7fffffffLL || N > 0x7fffffffLL || K > 0x7fffffffLL) return MI_E_SHAPE;
+    if (cld(M, (int64_t)tm) > MI_MAX_GRID_DIM || cld(N, (int64_t)tn) > MI_MAX_GRID_DIM ||
+        cld(M, (int64_t)tm) * cld(N, (int64_t)tn) > MI_MAX_GRID_DIM)
+        return MI_E_GRID;
+    if ((M > 1 && (A->strides[0] != 1 || C->strides[0] != 1)) || (K > 1 && B->strides[0] != 1))
+        return MI_E_STRIDE;
+    p->A = A->ptr; p->B = B->ptr; p->C = C->ptr;
+    p->lda = A->strides[1]; p->ldb = B->strides[1]; p->ldc = C->strides[1];
+    p->sa = ndim == 3 ? A->strides[2] : 0;
+    p->sb = ndim == 3 ? B->strides[2] : 0;
+    p->sc = ndim == 3 ? C->strides[2] : 0;
+    p->M = (int)M; p->N = (int)N; p->K = (int)K; p->batch = (int)batch;
+    p->in_dtype = A->dtype; p->out_dtype = C->dtype;
+    return MI_OK;
+}
+
+template <typename E, typename OutT>
+void launch_generic16(const Problem& p, hipStream_t s) {
+    const int tiles_m = (int)cld((int64_t)p.M, (int64_t)GT), tiles_n = (int)cld((int64_t)p.N, (int64_t)GT);
+    const bool vecA = aligned(p.A, 16) && p.lda % 8 == 0 && p.sa % 8 == 0;
+    const bool vecB = aligned(p.B, 16) && p.ldb % 8 == 0 && p.sb % 8 == 0;
+    hipLaunchKernelGGL((gemm16_generic<E, OutT>), dim3((unsigned)(tiles_m * tiles_n), 1, (unsigned)p.batch),
+                       dim3(256), 0, s, (const unsigned short*)p.A, p.lda, p.sa, (const unsigned short*)p.B,
+                       p.ldb, p.sb, (OutT*)p.C, p.ldc, p.sc, p.M, p.N, p.K, tiles_m, vecA, vecB);
+}
+
+int run(const Problem& p, hipStream_t s) {
+    if (p.M == 0 || p.N == 0 || p.batch == 0) return MI_OK;
+    if (p.in_dtype == MI_F32) {
+        const int tiles_m = (int)cld((int64_t)p.M, (int64_t)FT), tiles_n = (int)cld((int64_t)p.N, (int64_t)FT);
+        const bool vecA = aligned(p.A, 16) && p.lda % 4 == 0 && p.sa % 4 == 0;
+        const bool vecB = aligned(p.B, 16) && p.ldb % 4 == 0 && p.sb % 4 == 0;
+        hipLaunchKernelGGL(gemm32_kernel, dim3((unsigned)(tiles_m * tiles_n), 1, (unsigned)p.batch), dim3(256), 0, s,
+                           (const float*)p.A, p.lda, p.sa, (const float*)p.B, p.ldb, p.sb, (float*)p.C, p.ldc, p.sc,
+                           p.M, p.N, p.K, tiles_m, vecA, vecB);
+        set_variant("gemm32_128x128x16_mfma32x32x2");
+        return launch_status();
+    }
+    const bool f32out = p.out_dtype == MI_F32;
+    if (p.in_dtype == MI_F16) {
+        if (f32out) launch_generic16<F16, float>(p, s);
+        else launch_generic16<F16, unsigned short>(p, s);
+    } else {
+        if (f32out) launch_generic16<BF16, float>(p, s);
+        else launch_generic16<BF16, unsigned short>(p, s);
+    }
+    set_variant("gemm16_generic_64x64x32");
+    return launch_status();
+}
+
+}  // namespace
+
+extern "C" int mi_matmul_kernel(const mi_tile_array* A, const mi_tile_array* B, const mi_tile_array* C, int tm,
+                                int tn, int tk, void* stream) {
+    Problem p;
+    MI_CHECK(validate(A, B, C, 2, tm, tn, tk, &p));
+    return run(p, (hipStream_t)stream);
+}
+
+extern "C" int mi_batch_matmul_kernel(const mi_tile_array* A, const mi_tile_array* B, const mi_tile_array* C,
+                                      int tm, int tn, int tk, void* stream) {
+    Problem p;
+    MI_CHECK(validate(A, B, C, 3, tm, tn, tk, &p));
+    return run(p, (hipStream_t)stream);
+}

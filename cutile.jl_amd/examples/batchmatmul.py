@@ -1,0 +1,49 @@
+"""Mirror of examples/batchmatmul.jl:62-111 (prepare / run / metric)."""
+from __future__ import annotations
+
+import numpy as np
+import torch
+
+import cutile_jl_amd as ct
+from ._harness import namespace, rand_uniform, time_launches
+
+
+def prepare(*, benchmark: bool = False, M: int | None = None, K: int | None = None, N: int | None = None,
+            Batch: int | None = None, T: torch.dtype = torch.float32, seed: int = 4, lo: float = -1.0, hi: float = 1.0):
+    """batchmatmul.jl:62-73, batch-last: A (M,K,Batch) = torch (Batch,K,M) etc.  Inputs
+    U(lo,hi); the measured configuration uses U(-1,1) (the reference U[0,1))."""
+    M = (1024 if benchmark else 256) if M is None else M
+    K = (512 if benchmark else 128) if K is None else K
+    N = (2048 if benchmark else 256) if N is None else N
+    Batch = (8 if benchmark else 4) if Batch is None else Batch
+    rng = np.random.default_rng(seed)
+    A = rand_uniform(rng, (M, K, Batch), T, lo, hi)
+    B = rand_uniform(rng, (K, N, Batch), T, lo, hi)
+    C = torch.empty((Batch, N, M), dtype=T, device=A.device)
+    return namespace(A=A, B=B, C=C, M=M, K=K, N=N, Batch=Batch)
+
+
+def run(data, *, tm: int = 128, tn: int = 128, tk: int = 64, nruns: int = 1, warmup: int = 0):
+    """batchmatmul.jl:75-95."""
+    times = time_launches(lambda: ct.batch_matmul_kernel(data.A, data.B, data.C, tm, tn, tk), nruns, warmup)
+    return namespace(C=data.C, times=times)
+
+
+def metric(data):
+    """batchmatmul.jl:108-111."""
+    return 2 * data.M * data.K * data.N * data.Batch, "TFLOPS"
+
+
+def smoke(orc):
+    d = prepare(M=130, K=70, N=96, Batch=2)
+    r = run(d)
+    ref = orc.batch_matmul(orc.to_julia(d.A), orc.to_julia(d.B))
+    got = orc.to_julia(r.C).astype(np.float64)
+    assert np.abs(got - ref).max() <= 1e-5 * np.abs(ref).max()
+
+
+def bench(ct_, entry, event_times, nruns, warmup):
+    d = prepare(benchmark=True)
+    t = event_times(lambda: ct_.batch_matmul_kernel(d.A, d.B, d.C, 128, 128, 64), nruns, warmup)
+    return {"batchmatmul": entry("batched GEMM 8x(1024x512x2048) f32", t, metric(d)[0], "TFLOPS", "mfma", 157.3,
+                                 "f32", {"variant": ct_.last_variant()})}

@@ -1,0 +1,142 @@
+"""Mirror of examples/moe.jl:186-383 (invoke_* helpers, cutile_moe, prepare / run / metric)."""
+from __future__ import annotations
+
+import numpy as np
+import torch
+
+import cutile_jl_amd as ct
+from ._harness import namespace, rand_normal, time_launches
+
+
+def invoke_fused_moe_kernel(A, B, C, topk_weights, sorted_token_ids, sorted_expert_ids, *, mul_routed_weight,
+                            num_token_replicas, tile_m, tile_n, tile_k, b_scale=None):
+    """moe.jl:186-199.  ``topk_weights`` Julia (num_tokens, topk) = torch (topk, num_tokens);
+    flattened slot-fastest (moe.jl:193).  ``C`` Julia (dim, topk, num_tokens) is flattened to
+    (dim, total_tokens) (moe.jl:196)."""
+    topk_weights_flat = topk_weights.t().contiguous().reshape(-1)
+    C_flat = C.reshape(C.shape[0] * C.shape[1], C.shape[2]) if C.dim() == 3 else C
+    ct.fused_moe_kernel(A, B, C_flat, topk_weights_flat, sorted_token_ids, sorted_expert_ids, num_token_replicas,
+                        mul_routed_weight, tile_m, tile_n, tile_k, b_scale=b_scale)
+
+
+def invoke_silu_and_mul_kernel(AB, C):
+    """moe.jl:202-215: AB Julia (2*inter, total) = torch (total, 2*inter); halves along dim 1."""
+    inter = C.shape[1]
+    A_half = AB[:, :inter]
+    B_half = AB[:, inter:2 * inter]
+    tile_n = 1 << (inter - 1).bit_length()
+    ct.silu_and_mul_kernel(A_half, B_half, C, tile_n)
+
+
+def cutile_moe(hidden_states, w1, w2, topk_weights, topk_ids, tile_m, tile_n, tile_k, *, w1_scale=None,
+               w2_scale=None, aligned=None):
+    """moe.jl:218-257.  Torch shapes (reversed Julia): hidden_states (tokens, hidden); w1
+    (E, 2*inter, hidden); w2 (E, hidden, inter); topk_weights / topk_ids (topk, tokens), ids
+    1-based int64.  ``aligned`` may carry a precomputed (sorted_token_ids, sorted_expert_ids)
+    pair on the device to skip the host round trip of moe.jl:232-233."""
+    num_tokens, hidden_size = hidden_states.shape
+    num_experts, _, intermediate_size = w2.shape
+    topk = topk_ids.shape[0]
+    total_tokens = num_tokens * topk
+    T, dev = hidden_states.dtype, hidden_states.device
+    cache1 = torch.zeros((num_tokens, topk, intermediate_size * 2), dtype=T, device=dev)
+    cache2 = torch.zeros((total_tokens, intermediate_size), dtype=T, device=dev)
+    cache3 = torch.zeros((num_tokens, topk, hidden_size), dtype=T, device=dev)
+    if aligned is None:
+        tok, exp = ct.moe_align_tile_size(topk_ids.cpu(), tile_m, num_experts)
+        sorted_token_ids, sorted_expert_ids = tok.to(dev), exp.to(dev)
+    else:
+        sorted_token_ids, sorted_expert_ids = aligned
+    invoke_fused_moe_kernel(hidden_states, w1, cache1, topk_weights, sorted_token_ids, sorted_expert_ids,
+                            mul_routed_weight=False, num_token_replicas=topk, tile_m=tile_m, tile_n=tile_n,
+                            tile_k=tile_k, b_scale=w1_scale)
+    cache1_flat = cache1.reshape(total_tokens, intermediate_size * 2)
+    invoke_silu_and_mul_kernel(cache1_flat, cache2)
+    invoke_fused_moe_kernel(cache2, w2, cache3, topk_weights, sorted_token_ids, sorted_expert_ids,
+                            mul_routed_weight=True, num_token_replicas=1, tile_m=tile_m, tile_n=tile_n,
+                            tile_k=tile_k, b_scale=w2_scale)
+    out = torch.empty((num_tokens, hidden_size), dtype=T, device=dev)
+    ct.moe_sum_topk(cache3, out)  # sum(cache3; dims=2), moe.jl:256
+    return out
+
+
+def prepare(*, benchmark: bool = False, num_tokens: int | None = None, hidden_size: int | None = None,
+            num_experts: int | None = None, intermediate_size: int | None = None, topk: int = 8,
+            T: torch.dtype = torch.float16, seed: int = 6, router: str = "randperm", weight_std: float = 0.02):
+    """moe.jl:311-344.  ``router='randperm'``: the reference's unique random experts with softmax
+    of U(0,1) weights; ``'top2_logits'``: the measured configuration (logits ~ N(0,1), top-k,
+    softmax over the selected logits).  Activations ~ N(0,1), weights ~ N(0, weight_std)."""
+    num_tokens = (256 if benchmark else 48) if num_tokens is None else num_tokens
+    hidden_size = (1024 if benchmark else 512) if hidden_size is None else hidden_size
+    num_experts = (32 if benchmark else 64) if num_experts is None else num_experts
+    intermediate_size = (2048 if benchmark else 1024) if intermediate_size is None else intermediate_size
+    rng = np.random.default_rng(seed)
+    hidden_states = rand_normal(rng, (hidden_size, num_tokens), T)
+    w1 = rand_normal(rng, (hidden_size, intermediate_size * 2, num_experts), T, std=weight_std)
+    w2 = rand_normal(rng, (intermediate_size, hidden_size, num_experts), T, std=weight_std)
+    if router == "top2_logits":
+        logits = rng.standard_normal((num_tokens, num_experts)).astype(np.float32)
+        order = np.argsort(-logits, axis=1, kind="stable")[:, :topk]
+        sel = np.take_along_axis(logits, order, axis=1).astype(np.float64)
+        e = np.exp(sel - sel.max(axis=1, keepdims=True))
+        weights = (e / e.sum(axis=1, keepdims=True)).astype(np.float32)
+        ids = (order + 1).astype(np.int64)
+    else:
+        ids = np.stack([rng.permutation(num_experts)[:topk] + 1 for _ in range(num_tokens)]).astype(np.int64)
+        raw = np.exp(rng.random((num_tokens, topk), dtype=np.float32))
+        weights = raw / raw.sum(axis=1, keepdims=True)
+    dev = hidden_states.device
+    topk_weights = torch.from_numpy(np.ascontiguousarray(weights.T)).to(T).to(dev)  # Julia (tokens, topk)
+    topk_ids = torch.from_numpy(np.ascontiguousarray(ids.T)).to(dev)
+    return namespace(hidden_states=hidden_states, w1=w1, w2=w2, topk_weights=topk_weights, topk_ids=topk_ids,
+                     num_tokens=num_tokens, hidden_size=hidden_size, num_experts=num_experts,
+                     intermediate_size=intermediate_size, topk=topk, tile_m=128, tile_n=128, tile_k=64)
+
+
+def run(data, *, nruns: int = 1, warmup: int = 0, **kw):
+    """moe.jl:347-367: the timed region is the whole cutile_moe call."""
+    d = data
+    holder = {}
+
+    def call():
+        holder["out"] = cutile_moe(d.hidden_states, d.w1, d.w2, d.topk_weights, d.topk_ids, d.tile_m, d.tile_n,
+                                   d.tile_k, **kw)
+
+    times = time_launches(call, nruns, warmup)
+    return namespace(out=holder["out"], times=times)
+
+
+def metric(data):
+    """moe.jl:377-383."""
+    return 2 * data.num_tokens * data.topk * data.hidden_size * data.intermediate_size * 3, "TFLOPS"
+
+
+def smoke(orc):
+    d = prepare(num_tokens=24, hidden_size=256, num_experts=8, intermediate_size=256, topk=2, router="top2_logits")
+    r = run(d)
+    J = orc.to_julia
+    ref = orc.ref_moe(J(d.hidden_states), J(d.w1), J(d.w2), J(d.topk_weights), J(d.topk_ids))
+    got = J(r.out).astype(np.float32)
+    assert np.abs(got - ref).max() <= 2e-2 * np.abs(ref).max(), np.abs(got - ref).max()
+
+
+def bench(ct_, entry, event_times, nruns, warmup):
+    res = {}
+    d = prepare(benchmark=True, topk=2, router="top2_logits")
+    t = event_times(lambda: cutile_moe(d.hidden_states, d.w1, d.w2, d.topk_weights, d.topk_ids, 128, 128, 64),
+                    nruns, warmup)
+    wbytes = (d.w1.numel() + d.w2.numel()) * 2 + 2 * d.hidden_states.numel() * 2
+    flop = metric(d)[0]
+    e = entry("MoE f16 256tok/1024h/32e/2048i top-2 (whole cutile_moe incl. host align)", t, wbytes, "GB/s", "hbm",
+              8000.0, "f16", {"flop": flop, "tflops_at_min": round(flop / (min(t) * 1e-3) / 1e12, 2),
+                              "mfma_frac_at_min": round(flop / (min(t) * 1e-3) / 1e12 / 2500.0, 5)})
+    res["moe_f16"] = e
+    tok, exp = ct_.moe_align_tile_size(d.topk_ids.cpu(), 128, d.num_experts)
+    al = (tok.cuda(), exp.cuda())
+    t = event_times(lambda: cutile_moe(d.hidden_states, d.w1, d.w2, d.topk_weights, d.topk_ids, 128, 128, 64,
+                                       aligned=al), nruns, warmup)
+    res["moe_f16_device_only"] = entry("MoE f16 top-2 (device work only: zero-fill + 4 kernels)", t, wbytes, "GB/s",
+                                       "hbm", 8000.0, "f16",
+                                       {"flop": flop, "tflops_at_min": round(flop / (min(t) * 1e-3) / 1e12, 2),
+                                        "mfma_frac_at_min": round(flop / (min(t) * 1e-3) / 1e12 / 2500.0, 5)})
+    return res

@@ -1,0 +1,113 @@
+"""GPU parity tests for the fused attention kernel through the C ABI.
+
+Oracle: the numpy restatement of ``ref_fmha`` (examples/fmha.jl:175-220), evaluated in float64
+on the f16/bf16 inputs (the "fp32 reference" of the tolerance, at higher precision).  Shapes:
+the reference example's ``main()`` list (fmha.jl:314-325) plus GQA, decode offset
+(``input_pos``), ragged sequence lengths (EVEN_K = false), D = 128 and strided views.
+
+Tolerance: |err| <= 2e-2 * (|ref| + max|ref|) element-wise, and the reference's own
+``isapprox(rtol=1e-2, atol=1e-3)`` (fmha.jl:277-282).
+"""
+import numpy as np
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+from cutile_jl_amd.examples import fmha  # noqa: E402
+
+
+def check(orc, out, ref, tol=2e-2):
+    got = orc.to_julia(out).astype(np.float64)
+    err = np.abs(got - ref)
+    bound = tol * (np.abs(ref) + np.abs(ref).max())
+    assert np.all(err <= bound), f"max err {err.max():.3e}, worst ratio {np.max(err / bound):.3f}"
+    assert orc.isapprox(got, ref, rtol=1e-2, atol=1e-3)
+    return err.max()
+
+
+@pytest.mark.parametrize("batch,heads,sq,skv,d,causal,qg,T", [
+    (2, 8, 128, 128, 64, False, 1, torch.float16), (2, 8, 128, 128, 64, True, 1, torch.float16),
+    (4, 16, 256, 256, 64, True, 1, torch.float16),
+    (1, 4, 384, 384, 64, True, 2, torch.float16), (1, 8, 256, 512, 64, False, 4, torch.float16),
+    (2, 2, 200, 200, 64, True, 1, torch.float16), (1, 2, 77, 130, 64, False, 1, torch.float16),
+    (1, 2, 1, 1, 64, True, 1, torch.float16), (1, 2, 130, 64, 64, False, 1, torch.float16),
+    (2, 4, 256, 256, 128, True, 1, torch.float16), (1, 2, 100, 300, 128, False, 2, torch.float16),
+    (2, 4, 256, 256, 64, True, 1, torch.bfloat16), (1, 2, 192, 192, 128, False, 1, torch.bfloat16),
+])
+def test_fmha_against_ref(orc, batch, heads, sq, skv, d, causal, qg, T):
+    data = fmha.prepare(batch=batch, heads=heads, seq_q=sq, seq_kv=skv, d_k=d, d_v=d, query_group_size=qg,
+                        causal=causal, T=T)
+    r = fmha.run(data)
+    Q, K, V = (orc.to_julia(t) for t in (data.Q, data.K, data.V))
+    if causal and sq != skv:
+        pytest.skip("ref_fmha's causal mask assumes aligned positions")
+    ref = orc.ref_fmha(Q, K, V, causal=causal, dtype=np.float64)
+    check(orc, r.out, ref, 2e-2 if T == torch.float16 else 3e-2)
+
+
+def test_fmha_reference_input_distribution(orc):
+    """The reference's own inputs, U(-0.5, 0.5) (fmha.jl:240-242)."""
+    data = fmha.prepare(batch=2, heads=8, seq_q=256, seq_kv=256, dist="uniform")
+    r = fmha.run(data)
+    ref = orc.ref_fmha(*(orc.to_julia(t) for t in (data.Q, data.K, data.V)), causal=True, dtype=np.float64)
+    check(orc, r.out, ref)
+
+
+@pytest.mark.parametrize("sq,skv,pos", [(64, 256, 192), (1, 200, 199), (128, 300, 100), (130, 512, 300)])
+def test_fmha_decode_offset(orc, sq, skv, pos):
+    """input_pos shifts the query positions (fmha.jl:45-46,66): query i sees keys <= pos + i."""
+    data = fmha.prepare(batch=1, heads=4, seq_q=sq, seq_kv=skv, query_group_size=2)
+    out = fmha.cutile_fmha(data.Q, data.K, data.V, input_pos=pos, causal=True, query_group_size=2)
+    ref = orc.fmha_general(*(orc.to_julia(t) for t in (data.Q, data.K, data.V)), causal=True, input_pos=pos)
+    check(orc, out, ref)
+
+
+def test_fmha_causal_first_row_and_noncausal_limit(orc):
+    data = fmha.prepare(batch=1, heads=2, seq_q=256, seq_kv=256)
+    out = fmha.cutile_fmha(data.Q, data.K, data.V, causal=True)
+    # query 1 attends to key 1 only: output row equals V[:, 1] exactly (softmax weight 1.0)
+    assert torch.equal(out[:, :, 0, :], data.V[:, :, 0, :])
+    # with input_pos >= Skv the causal kernel sees every key: equals the non-causal kernel bit for bit
+    a = fmha.cutile_fmha(data.Q, data.K, data.V, causal=True, input_pos=256)
+    b = fmha.cutile_fmha(data.Q, data.K, data.V, causal=False)
+    assert torch.equal(a, b)
+
+
+def test_fmha_strided_views_and_scale(orc):
+    """Q/K/V as views of a packed (B, S, 3, H, D) buffer, and an explicit qk_scale."""
+    rng = np.random.default_rng(0)
+    B, S, H, D = 2, 192, 4, 64
+    packed = torch.from_numpy(rng.standard_normal((B, S, 3, H, D), dtype=np.float32)).to(torch.float16).cuda()
+    Q, K, V = (packed[:, :, i].permute(0, 2, 1, 3) for i in range(3))  # torch (B,H,S,D) views, D contiguous
+    out = fmha.cutile_fmha(Q, K, V, causal=True, qk_scale=0.2)
+    ref = orc.ref_fmha(orc.to_julia(Q), orc.to_julia(K), orc.to_julia(V), qk_scale=0.2, causal=True, dtype=np.float64)
+    check(orc, out, ref)
+
+
+def test_fmha_argument_errors(ct):
+    data = fmha.prepare(batch=1, heads=2, seq_q=128, seq_kv=128)
+    out = torch.empty_like(data.Q)
+    with pytest.raises(ct.MiError) as e:
+        ct.fmha_kernel(data.Q, data.K, data.V, out, 0.125, 0, 64, 2, 128, 128, 1, True, False)  # EVEN_K mismatch
+    assert e.value.code == ct.MI_E_ARG
+    with pytest.raises(ct.MiError) as e:
+        ct.fmha_kernel(data.Q, data.K, data.V, out, 0.125, 0, 32, 2, 128, 128, 1, True, True)   # TILE_D != D
+    assert e.value.code == ct.MI_E_SHAPE
+
+
+def test_fmha_full_size(orc):
+    """Benchmark shape 8x16x1024x64 causal: a sample of (batch, head) pairs against float64 and
+    the softmax-weights-sum-to-one property via V = ones."""
+    data = fmha.prepare(benchmark=True)
+    r = fmha.run(data)
+    Q, K, V = (orc.to_julia(t) for t in (data.Q, data.K, data.V))
+    got = orc.to_julia(r.out).astype(np.float64)
+    for (h, b) in [(0, 0), (15, 7), (7, 3)]:
+        ref = orc.ref_fmha(Q[:, :, h:h + 1, b:b + 1], K[:, :, h:h + 1, b:b + 1], V[:, :, h:h + 1, b:b + 1],
+                           causal=True, dtype=np.float64)
+        err = np.abs(got[:, :, h, b] - ref[:, :, 0, 0])
+        assert np.all(err <= 2e-2 * (np.abs(ref[:, :, 0, 0]) + np.abs(ref).max()))
+    ones = torch.ones_like(data.V)
+    out1 = fmha.cutile_fmha(data.Q, data.K, ones, causal=True)
+    assert torch.all((out1.float() - 1).abs() <= 2e-3)

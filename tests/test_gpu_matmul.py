@@ -1,0 +1,119 @@
+"""GPU parity tests for matmul / batch matmul through the C ABI against the float64 oracle.
+Shapes: the reference examples' ``main()`` lists (matmul.jl:156-165, batchmatmul.jl:161-169),
+the ragged 200x100x300 case of docs/src/tutorials/matmul.md:225-256, the 64x16x64 case of
+test/device/tile.jl:1036-1066, plus strided / misaligned / degenerate cases.
+
+Tolerances (stated against a float64 evaluation of ``A*B`` on the same inputs):
+  fp32 inputs : |err| <= 1e-5 * (|ref| + max|ref|)       (true fp32 MFMA, fp32 accumulate)
+  f16 / bf16  : |err| <= 2e-2 * (|ref| + max|ref|) when C is f32; the same plus one output
+                rounding (2^-11 / 2^-8 relative) when C is stored in the input type.
+"""
+import numpy as np
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+from cutile_jl_amd.examples import matmul, batchmatmul  # noqa: E402
+
+
+def check(got, ref, tol):
+    got = np.asarray(got, dtype=np.float64)
+    err = np.abs(got - ref)
+    bound = tol * (np.abs(ref) + np.abs(ref).max())
+    assert np.all(err <= bound), f"max err {err.max():.3e}, worst ratio {np.max(err / np.maximum(bound, 1e-300)):.3f}"
+
+
+@pytest.mark.parametrize("M,N,K,tm,tn,tk", [(256, 256, 256, 32, 32, 32), (512, 512, 512, 64, 64, 64),
+                                            (256, 512, 128, 32, 32, 32), (1024, 1024, 1024, 64, 64, 64),
+                                            (200, 100, 300, 64, 64, 64), (64, 64, 16, 32, 32, 16),
+                                            (1, 1, 1, 64, 64, 64), (129, 65, 33, 64, 64, 64), (5, 700, 9, 64, 64, 64)])
+def test_matmul_f32(orc, M, N, K, tm, tn, tk):
+    d = matmul.prepare(M=M, N=N, K=K)
+    r = matmul.run(d, tm=tm, tn=tn, tk=tk)
+    ref = orc.matmul(orc.to_julia(d.A), orc.to_julia(d.B))
+    check(orc.to_julia(r.C), ref, 1e-5)
+    assert orc.isapprox(orc.to_julia(r.C), ref, rtol=1e-2)  # matmul.jl:98-101
+
+
+@pytest.mark.parametrize("T", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("M,N,K", [(256, 256, 256), (512, 256, 1024), (200, 100, 300), (64, 64, 16), (33, 17, 41),
+                                   (1024, 768, 512), (256, 256, 64), (512, 1024, 192), (8, 8, 8)])
+@pytest.mark.parametrize("out32", [True, False])
+def test_matmul_16bit(orc, T, M, N, K, out32):
+    d = matmul.prepare(M=M, N=N, K=K, T=T, out_T=torch.float32 if out32 else None, dist="normal64")
+    r = matmul.run(d)
+    ref = orc.matmul(orc.to_julia(d.A), orc.to_julia(d.B))
+    extra = 0.0 if out32 else (2.0 ** -11 if T == torch.float16 else 2.0 ** -8)
+    check(orc.to_julia(r.C), ref, 2e-2 + extra)
+    # far tighter in practice: fp32 accumulation of exactly-representable products
+    assert np.abs(orc.to_julia(r.C).astype(np.float64) - ref).max() <= (1e-4 + 2 * extra) * np.abs(ref).max() + 1e-6
+
+
+def test_matmul_integer_valued_inputs_are_exact(ct, orc):
+    """Small-integer f16 operands: every product and partial sum is exact in fp32, so the
+    result must equal the integer matrix product bit for bit (catches any operand
+    permutation inside the MFMA / transpose-read path)."""
+    rng = np.random.default_rng(0)
+    for (M, N, K) in [(256, 256, 256), (96, 160, 80), (512, 512, 1024)]:
+        A = rng.integers(-4, 5, (M, K)).astype(np.float32); B = rng.integers(-4, 5, (K, N)).astype(np.float32)
+        At = orc.from_julia(A).to(torch.float16).cuda(); Bt = orc.from_julia(B).to(torch.float16).cuda()
+        C = torch.empty((N, M), dtype=torch.float32, device="cuda")
+        ct.matmul_kernel(At, Bt, C, 64, 64, 64)
+        assert np.array_equal(orc.to_julia(C), A @ B)
+
+
+def test_matmul_padded_leading_dims_and_misaligned(ct, orc):
+    rng = np.random.default_rng(1)
+    M, N, K = 100, 90, 70
+    Abig = torch.from_numpy(rng.standard_normal((K, 128), dtype=np.float32)).to(torch.float16).cuda()
+    Bbig = torch.from_numpy(rng.standard_normal((N, 77), dtype=np.float32)).to(torch.float16).cuda()
+    Cbig = torch.full((N, 111), -5.0, dtype=torch.float32, device="cuda")
+    A = Abig[:, 3:3 + M]      # Julia view(Abig, 4:103, :)  -> misaligned start, lda = 128
+    B = Bbig[:, 1:1 + K]      # ldb = 77 (odd)
+    C = Cbig[:, :M]
+    ct.matmul_kernel(A, B, C, 64, 64, 64)
+    ref = orc.matmul(orc.to_julia(A), orc.to_julia(B))
+    check(orc.to_julia(C), ref, 2e-2)
+    assert np.abs(orc.to_julia(C) - ref).max() < 1e-3
+    assert torch.all(Cbig[:, M:] == -5.0)
+
+
+@pytest.mark.parametrize("M,K,N,Batch,T", [(256, 128, 256, 4, torch.float32), (512, 256, 1024, 4, torch.float16),
+                                           (130, 70, 96, 3, torch.float32), (64, 32, 48, 1, torch.float16),
+                                           (100, 50, 60, 2, torch.bfloat16)])
+def test_batch_matmul(orc, M, K, N, Batch, T):
+    d = batchmatmul.prepare(M=M, K=K, N=N, Batch=Batch, T=T)
+    r = batchmatmul.run(d)
+    ref = orc.batch_matmul(orc.to_julia(d.A), orc.to_julia(d.B))
+    tol = 1e-5 if T == torch.float32 else 2e-2 + (2.0 ** -11 if T == torch.float16 else 2.0 ** -8)
+    check(orc.to_julia(r.C), ref, tol)
+    assert orc.isapprox(orc.to_julia(r.C), ref, rtol=1e-2)  # batchmatmul.jl:97-106
+
+
+def test_matmul_full_size_f16(orc):
+    """4096^3 f16 -> f32 (the measured configuration): sampled rows/columns against float64,
+    and linearity C(A, B1+B2) == C(A,B1) + C(A,B2) on integer-valued inputs (exact)."""
+    d = matmul.prepare(benchmark=True, T=torch.float16, out_T=torch.float32, dist="normal64")
+    r = matmul.run(d)
+    A = orc.to_julia(d.A).astype(np.float64); B = orc.to_julia(d.B).astype(np.float64)
+    C = orc.to_julia(r.C)
+    rows = [0, 1, 255, 256, 2049, 4095]; cols = [0, 31, 32, 1000, 4095]
+    ref_rows = A[rows] @ B
+    check(C[rows], ref_rows, 2e-2)
+    assert np.abs(C[rows] - ref_rows).max() <= 1e-4 * np.abs(ref_rows).max()
+    ref_cols = A @ B[:, cols]
+    assert np.abs(C[:, cols] - ref_cols).max() <= 1e-4 * np.abs(ref_cols).max()
+    # checksum of checksums: sum over all of C equals (column sums of A) . (row sums of B)
+    total = torch.sum(r.C.double()).item()
+    expect = float(A.sum(axis=0) @ B.sum(axis=1))
+    assert abs(total - expect) <= 1e-4 * np.abs(A).sum(axis=0) @ np.abs(B).sum(axis=1)
+
+
+def test_batch_matmul_full_size_f32(orc):
+    d = batchmatmul.prepare(benchmark=True)
+    r = batchmatmul.run(d)
+    A = orc.to_julia(d.A); B = orc.to_julia(d.B); C = orc.to_julia(r.C)
+    for b in (0, 7):
+        ref = A[:, :, b].astype(np.float64) @ B[:, :, b].astype(np.float64)
+        check(C[:, :, b], ref, 1e-5)

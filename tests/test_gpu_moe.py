@@ -1,0 +1,139 @@
+"""GPU parity tests for the MoE kernels through the C ABI.
+
+Oracle: numpy restatement of ``ref_moe`` (examples/moe.jl:264-304) in float64, plus per-kernel
+checks of the grouped GEMM, SiLU*mul and the top-k sum.  Shapes: the reference example's
+``main()`` list (moe.jl:402-410), the measured top-2 configuration at reduced width, expert
+counts that are not multiples of the tile (sentinel padding), and FP8-E4M3 weights.
+
+Tolerance: |err| <= 2e-2 * (|ref| + max|ref|), and the reference's
+``isapprox(rtol=1e-2, atol=1e-2)`` (moe.jl:370-374).  The f16 result is rounded to f16 three
+times on the way (cache1, cache2, cache3) exactly as in the reference.
+"""
+import numpy as np
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+from cutile_jl_amd.examples import moe  # noqa: E402
+
+
+def check(got, ref, tol=2e-2):
+    got = np.asarray(got, dtype=np.float64)
+    err = np.abs(got - ref)
+    bound = tol * (np.abs(ref) + np.abs(ref).max())
+    assert np.all(err <= bound), f"max err {err.max():.3e}, worst ratio {np.max(err / bound):.3f}"
+
+
+@pytest.mark.parametrize("tokens,hidden,experts,inter,topk,router", [
+    (48, 512, 64, 1024, 8, "randperm"), (128, 512, 32, 1024, 4, "randperm"), (64, 1024, 64, 2048, 8, "randperm"),
+    (256, 512, 32, 512, 2, "top2_logits"), (7, 256, 3, 128, 2, "randperm"), (300, 256, 2, 256, 2, "randperm"),
+    (1, 128, 4, 64, 1, "randperm"),
+])
+def test_moe_end_to_end(orc, tokens, hidden, experts, inter, topk, router):
+    d = moe.prepare(num_tokens=tokens, hidden_size=hidden, num_experts=experts, intermediate_size=inter, topk=topk,
+                    router=router)
+    r = moe.run(d)
+    J = orc.to_julia
+    ref = orc.ref_moe(J(d.hidden_states), J(d.w1), J(d.w2), J(d.topk_weights), J(d.topk_ids), dtype=np.float64)
+    check(J(r.out), ref)
+    assert orc.isapprox(J(r.out).astype(np.float64), ref, rtol=1e-2, atol=1e-2)
+
+
+def test_moe_bf16(orc):
+    d = moe.prepare(num_tokens=64, hidden_size=256, num_experts=8, intermediate_size=256, topk=2, T=torch.bfloat16)
+    r = moe.run(d)
+    J = orc.to_julia
+    ref = orc.ref_moe(J(d.hidden_states), J(d.w1), J(d.w2), J(d.topk_weights), J(d.topk_ids), dtype=np.float64)
+    check(J(r.out), ref, 5e-2)
+
+
+def test_fused_moe_kernel_alone_with_sentinels(ct, orc):
+    """One grouped GEMM against per-slot dot products; checks the replica -> token mapping
+    (cld(token_id, replicas)), the routed-weight scaling, that sentinel slots write nothing
+    and that untouched columns of C keep their contents."""
+    rng = np.random.default_rng(0)
+    K, N, E, tokens, topk, tile_m = 192, 160, 5, 9, 3, 16
+    A = rng.standard_normal((K, tokens)).astype(np.float16)
+    B = (rng.standard_normal((K, N, E)) * 0.1).astype(np.float16)
+    ids = np.stack([rng.permutation(E)[:topk] + 1 for _ in range(tokens)]).astype(np.int64)
+    w = rng.random((tokens, topk)).astype(np.float16)
+    tok, exp = orc.moe_align_tile_size(ids, tile_m, E)
+    total = tokens * topk
+    dev = "cuda"
+    C = torch.full((total + 2, N), 9.0, dtype=torch.float16, device=dev)  # two spare columns
+    wflat = torch.from_numpy(w.reshape(-1)).to(dev)
+    for mul in (False, True):
+        C.fill_(9.0)
+        ct.fused_moe_kernel(orc.from_julia(A).to(dev), orc.from_julia(B).to(dev), C[:total], wflat,
+                            torch.from_numpy(tok).to(dev), torch.from_numpy(exp).to(dev), topk, mul, tile_m, 128, 64)
+        got = orc.to_julia(C).astype(np.float64)
+        flat_e = ids.reshape(-1)
+        ref = np.zeros((N, total))
+        for f in range(total):
+            t = f // topk
+            ref[:, f] = B[:, :, flat_e[f] - 1].astype(np.float64).T @ A[:, t].astype(np.float64)
+            if mul:
+                ref[:, f] *= float(w.reshape(-1)[f])
+        check(got[:, :total], ref, 2e-2)
+        assert np.all(got[:, total:] == 9.0)
+
+
+def test_silu_and_mul_and_topk_sum(ct, orc):
+    rng = np.random.default_rng(1)
+    inter, total = 300, 37
+    AB = torch.from_numpy((rng.standard_normal((total, 2 * inter)) * 3).astype(np.float16)).cuda()
+    C = torch.zeros((total, inter), dtype=torch.float16, device="cuda")
+    moe.invoke_silu_and_mul_kernel(AB, C)
+    a = orc.to_julia(AB[:, :inter]); b = orc.to_julia(AB[:, inter:])
+    ref = orc.silu_and_mul(a, b)
+    check(orc.to_julia(C), ref, 2e-3)
+    x = torch.from_numpy(rng.standard_normal((19, 4, 130)).astype(np.float16)).cuda()  # Julia (130, 4, 19)
+    out = torch.empty((19, 130), dtype=torch.float16, device="cuda")
+    ct.moe_sum_topk(x, out)
+    assert torch.equal(out, x.float().sum(dim=1).to(torch.float16))
+
+
+def test_moe_fp8_weights(orc):
+    """E4M3FN expert weights with per-(n, expert) fp32 scales: the oracle is ref_moe on the
+    dequantised weights, so only accumulation order and the f16 cache roundings differ."""
+    d = moe.prepare(num_tokens=96, hidden_size=512, num_experts=8, intermediate_size=512, topk=2,
+                    router="top2_logits")
+    J = orc.to_julia
+    c1, s1 = orc.quantize_e4m3fn_per_channel(J(d.w1).astype(np.float32))
+    c2, s2 = orc.quantize_e4m3fn_per_channel(J(d.w2).astype(np.float32))
+    up = lambda c: orc.from_julia(c).cuda().view(torch.float8_e4m3fn)
+    out = moe.cutile_moe(d.hidden_states, up(c1), up(c2), d.topk_weights, d.topk_ids, 128, 128, 64,
+                         w1_scale=orc.from_julia(s1).cuda(), w2_scale=orc.from_julia(s2).cuda())
+    w1d = orc.e4m3fn_decode(c1) * s1[None]; w2d = orc.e4m3fn_decode(c2) * s2[None]
+    ref = orc.ref_moe(J(d.hidden_states), w1d, w2d, J(d.topk_weights), J(d.topk_ids), dtype=np.float64)
+    check(J(out), ref)
+
+
+def test_fp8_dequant_covers_every_code(ct, orc):
+    """Every finite E4M3FN code as a weight: K = 256 codes against a one-hot activation picks
+    each dequantised value out exactly (checks subnormals, signs and the exponent rebias)."""
+    codes = np.arange(256, dtype=np.uint8)
+    codes[0x7F] = 0; codes[0xFF] = 0x80  # the two NaN codes never occur in weights
+    K, N, E = 256, 32, 1
+    Bq = np.repeat(codes[:, None, None], N, axis=1)           # (K, N, E)
+    scale = np.linspace(0.5, 2.0, N, dtype=np.float32)[:, None]  # (N, E)
+    A = np.eye(K, dtype=np.float16)                           # token t = one-hot at k = t
+    ids = np.ones((K, 1), dtype=np.int64)
+    tok, exp = orc.moe_align_tile_size(ids, 128, E)
+    C = torch.zeros((K, N), dtype=torch.float16, device="cuda")
+    ct.fused_moe_kernel(orc.from_julia(A).cuda(), orc.from_julia(Bq).cuda().view(torch.float8_e4m3fn), C,
+                        torch.ones(K, dtype=torch.float16, device="cuda"), torch.from_numpy(tok).cuda(),
+                        torch.from_numpy(exp).cuda(), 1, False, 128, 128, 64,
+                        b_scale=orc.from_julia(scale).cuda())
+    ref = (orc.e4m3fn_decode(codes)[None, :] * scale).astype(np.float16)  # (N, K)
+    assert np.array_equal(orc.to_julia(C), ref)
+
+
+def test_moe_full_size_top2(orc):
+    """The measured configuration (256 tokens, hidden 1024, 32 experts, inter 2048, top-2)."""
+    d = moe.prepare(benchmark=True, topk=2, router="top2_logits")
+    r = moe.run(d)
+    J = orc.to_julia
+    ref = orc.ref_moe(J(d.hidden_states), J(d.w1), J(d.w2), J(d.topk_weights), J(d.topk_ids), dtype=np.float32)
+    check(J(r.out), ref.astype(np.float64))

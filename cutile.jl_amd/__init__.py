@@ -17,7 +17,8 @@ import ctypes
 import os
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(_HERE, "libmi355tile.so")
+# MI355TILE_LIB selects another build of the same library (e.g. an experimental variant).
+LIB_PATH = os.environ.get("MI355TILE_LIB") or os.path.join(_HERE, "libmi355tile.so")
 
 MI_F32, MI_F64, MI_F16, MI_BF16, MI_F8E4M3FN, MI_I32, MI_I64 = range(7)
 MI_MAX_RANK = 4

@@ -24,70 +24,12 @@
 // The (tm, tn, tk) tile constants of the reference only fix the block->data mapping and
 // the L2 swizzle; results do not depend on them, and the physical tiling above is chosen
 // for CDNA4.  FLOP count: 2*M*N*K per batch.
-#include "common.h"
+#include "gemm_common.h"
 
 namespace {
 
 using namespace mi;
-
-typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
-typedef _Float16 f16x4 __attribute__((ext_vector_type(4)));
-typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
-typedef short s16x4 __attribute__((ext_vector_type(4)));
-typedef short s16x8 __attribute__((ext_vector_type(8)));
-typedef float f32x16 __attribute__((ext_vector_type(16)));
-typedef float f32x4 __attribute__((ext_vector_type(4)));
-typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
-
-#define LDS_PTR(T, p) ((T __attribute__((address_space(3)))*)(p))
-
-// 16-bit element traits: raw storage is `short`; the MFMA picks the interpretation.
-struct F16 {
-    static __device__ __forceinline__ f32x16 mfma32(s16x8 a, s16x8 b, f32x16 c) {
-        return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, a),
-                                                      __builtin_bit_cast(f16x8, b), c, 0, 0, 0);
-    }
-    static __device__ __forceinline__ unsigned short from_f32(float v) {
-        _Float16 h = (_Float16)v;
-        return __builtin_bit_cast(unsigned short, h);
-    }
-};
-struct BF16 {
-    static __device__ __forceinline__ f32x16 mfma32(s16x8 a, s16x8 b, f32x16 c) {
-        return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a),
-                                                       __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
-    }
-    static __device__ __forceinline__ unsigned short from_f32(float v) {
-        unsigned u = __float_as_uint(v);
-        if ((u & 0x7fffffffu) > 0x7f800000u) return (unsigned short)((u >> 16) | 0x40);
-        u += 0x7fffu + ((u >> 16) & 1u);
-        return (unsigned short)(u >> 16);
-    }
-};
-
-template <typename E, typename OutT> __device__ __forceinline__ OutT cvt_out(float v);
-template <> __device__ __forceinline__ float cvt_out<F16, float>(float v) { return v; }
-template <> __device__ __forceinline__ float cvt_out<BF16, float>(float v) { return v; }
-template <> __device__ __forceinline__ unsigned short cvt_out<F16, unsigned short>(float v) {
-    return F16::from_f32(v);
-}
-template <> __device__ __forceinline__ unsigned short cvt_out<BF16, unsigned short>(float v) {
-    return BF16::from_f32(v);
-}
-
-// Transposed LDS fragment read.  `base` points at element (row k0, column m0) of an LDS
-// tile stored [k][m] with m contiguous and `pitch` elements per row.  The wave gets the
-// MFMA column operand for columns m0..m0+31 and the 16 k rows k0..k0+15: lane l holds
-// column m0 + l%32 and rows k0 + 8*(l/32) + 0..7.  Two ds_read_b64_tr_b16 per lane: within
-// each group of 16 lanes, lane r reads 4 consecutive m of row (r/4) and receives the
-// 4 consecutive rows of column (group base + r).
-__device__ __forceinline__ s16x8 lds_read_tr_k16(const unsigned short* base, int pitch, int lane) {
-    const int g = lane >> 4, r = lane & 15;
-    const unsigned short* p = base + (8 * (g >> 1) + (r >> 2)) * pitch + 16 * (g & 1) + 4 * (r & 3);
-    s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16(LDS_PTR(s16x4, p));
-    s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(LDS_PTR(s16x4, p + 4 * pitch));
-    return __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
-}
+using namespace mi::gemm;
 
 // ---- generic 16-bit kernel ---------------------------------------------------------------
 // Workgroup tile 64(m) x 64(n), K step 32, 4 waves as 2x2 of 32x32.
@@ -239,14 +181,6 @@ __global__ __launch_bounds__(256) void gemm32_kernel(const float* __restrict__ A
 
 // ---- host side -------------------------------------------------------------------------------
 
-struct Problem {
-    const void *A, *B;
-    void* C;
-    int64_t lda, ldb, ldc, sa, sb, sc;
-    int M, N, K, batch;
-    int in_dtype, out_dtype;
-};
-
 int validate(const mi_tile_array* A, const mi_tile_array* B, const mi_tile_array* C, int ndim, int tm,
              int tn, int tk, Problem* p) {
     MI_CHECK(check_array(A, ndim));
@@ -303,6 +237,10 @@ int run(const Problem& p, hipStream_t s) {
         return launch_status();
     }
     const bool f32out = p.out_dtype == MI_F32;
+    if (big16_applicable(p)) {
+        big16_launch(p, s);
+        return launch_status();
+    }
     if (p.in_dtype == MI_F16) {
         if (f32out) launch_generic16<F16, float>(p, s);
         else launch_generic16<F16, unsigned short>(p, s);

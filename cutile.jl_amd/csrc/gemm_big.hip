@@ -1,0 +1,268 @@
+// Large-tile f16/bf16 GEMM for MI355X: C(M,N) = A(M,K) * B(K,N), column-major, fp32 accumulate.
+//
+// Workgroup tile 256(m) x 256(n); 4 waves as 2x2, each 128x128 = 4x4 MFMA 32x32x16 tiles
+// (256 accumulator registers per lane, one wave per SIMD).  K is walked in steps of 32
+// through a ring of four LDS stages (4 x 32 KB) filled by direct global->LDS transfers
+// (global_load_lds, 16 bytes per lane, no staging registers).  The transfers for step s+3 /
+// s+4 are issued while step s is multiplied, a few at a time between the MFMAs, so the L2 /
+// fabric see a steady stream and every transfer has two to three steps (> 1 us) to land.
+// One workgroup barrier per step; the barrier waits only for the oldest stage in flight
+// (s_waitcnt vmcnt(16)), never for the stream to drain.
+//
+// LDS layouts (per stage):
+//   B tile [256 n][32 k]: row = 64 bytes = four 16-byte chunks; chunk c of row n sits at
+//     position c ^ ((n >> 2) & 3), so the 16 rows a quarter-wave reads with ds_read_b128 cover
+//     all 64 banks.
+//   A tile [32 k][256 m]: row = 512 bytes; chunk c of row k sits at position c ^ (4*(k & 3)),
+//     so the 4 rows x 32 bytes each 16-lane group of a transpose read (ds_read_b64_tr_b16)
+//     touches, and the two groups of a half-wave, land on 8 distinct 32-byte bank groups.
+//   Both swizzles are applied on the global side: the lane whose LDS slot is `pos` fetches
+//   the chunk that belongs there.
+//
+// The MFMA row operand carries n (B fragments, plain 16-byte reads), the column operand
+// (lane % 32) carries m (A fragments through the transpose read); a half-wave therefore
+// holds 32 consecutive m of one column of C and every store is a full 128-byte line.
+//
+// Workgroups are numbered so that the tiles resident on one XCD (ids congruent mod 8) form a
+// 4 x 8 block of tiles and share A row panels / B column panels in that XCD's L2.
+//
+// Requires M, N multiples of 256, K a multiple of 128 and >= 256, 16-byte aligned operands.
+#include "gemm_common.h"
+
+namespace {
+
+using namespace mi;
+using namespace mi::gemm;
+
+constexpr int BT = 256, BK = 32;
+constexpr int STAGE = BT * BK;  // elements per A or B stage (16 KB)
+
+#define SG_MFMA 0x008
+#define SG_VMEM 0x010
+#define SG_DSRD 0x100
+
+__device__ __forceinline__ void gload_lds16(const void* g, void* lds_wave_base) {
+    __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)g,
+                                     (__attribute__((address_space(3))) void*)lds_wave_base, 16, 0, 0);
+}
+
+struct Lane {
+    unsigned goffA, goffB;  // byte offset of this lane's 16-byte chunk within a wave-wide 1 KB transfer
+    unsigned fb[2];         // LDS element offset of the B fragment, k16 sub-step 0/1 (+ 32*j*BK for n tile j)
+    unsigned fa[4];         // LDS element offset of the A fragment, m tile i (+ 16*ks*BT for sub-step ks)
+};
+
+struct Frag {
+    s16x8 a[4], b[4];
+};
+
+// B stage: 256 rows x 64 B = 16 transfers of 1 KB (16 rows each); wave w takes transfers w, w+4, w+8, w+12.
+__device__ __forceinline__ void issue_B(const char* Bg, int64_t ldb2, unsigned short* Bs, int wave, const Lane& ln) {
+#pragma unroll
+    for (int j = 0; j < 4; ++j) gload_lds16(Bg + (int64_t)(64 * j) * ldb2 + ln.goffB, Bs + (wave + 4 * j) * 512);
+}
+// A stage: 32 rows x 512 B = 16 transfers of 1 KB (2 rows each).
+__device__ __forceinline__ void issue_A(const char* Ag, int64_t lda2, unsigned short* As, int wave, const Lane& ln) {
+#pragma unroll
+    for (int j = 0; j < 4; ++j) gload_lds16(Ag + (int64_t)(8 * j) * lda2 + ln.goffA, As + (wave + 4 * j) * 512);
+}
+
+__device__ __forceinline__ void load_frags(const unsigned short* As, const unsigned short* Bs, const Lane& ln, int ks,
+                                           Frag& f) {
+#pragma unroll
+    for (int j = 0; j < 4; ++j) f.b[j] = *reinterpret_cast<const s16x8*>(Bs + ln.fb[ks] + 32 * j * BK);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const unsigned short* p = As + ln.fa[i] + 16 * ks * BT;
+        s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16(LDS_PTR(s16x4, p));
+        s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(LDS_PTR(s16x4, p + 4 * BT));
+        f.a[i] = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+    }
+}
+
+template <typename E>
+__device__ __forceinline__ void mma16(const Frag& f, f32x16 (&acc)[4][4]) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) acc[i][j] = E::mfma32(f.b[j], f.a[i], acc[i][j]);
+}
+
+// Spread 12 LDS reads and (if DMA) 4 global->LDS transfers over 16 MFMAs.
+template <bool DMA, bool FRAGS>
+__device__ __forceinline__ void interleave16() {
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+        __builtin_amdgcn_sched_group_barrier(SG_MFMA, 1, 0);
+        if (FRAGS && i < 12) __builtin_amdgcn_sched_group_barrier(SG_DSRD, 1, 0);
+        if (DMA && (i & 3) == 1) __builtin_amdgcn_sched_group_barrier(SG_VMEM, 1, 0);
+    }
+    __builtin_amdgcn_sched_barrier(0);
+}
+
+template <int VMCNT>
+__device__ __forceinline__ void stage_barrier() {
+    // My reads of the current stage are done (lgkmcnt(0)) and my transfers into the next stage
+    // have landed (vmcnt leaves only the VMCNT youngest transfers in flight); then meet the
+    // other waves.  The wait is the builtin, not inline asm, so that the compiler's own
+    // wait-count bookkeeping sees it and does not add a full vmcnt(0) drain before the
+    // following LDS reads.  gfx9 encoding: vmcnt[3:0] | expcnt[6:4] | lgkmcnt[11:8] | vmcnt[15:14].
+    constexpr int imm = (VMCNT & 15) | (7 << 4) | (0 << 8) | ((VMCNT >> 4) << 14);
+    __builtin_amdgcn_s_waitcnt(imm);
+    asm volatile("" ::: "memory");
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+}
+
+// One K step of 32 on stage (AsX, BsX); the next step's data is in (AsY, BsY).
+//   first half : MFMAs of sub-step 0 | read sub-step 1 fragments | issue A transfers (into stage AsA)
+//   barrier
+//   second half: MFMAs of sub-step 1 | read next stage's sub-step 0 fragments | issue B transfers (into BsX)
+template <typename E, bool DMA_A, bool DMA_B, int VMCNT, bool LAST>
+__device__ __forceinline__ void k_step(const unsigned short* AsX, unsigned short* BsX, const unsigned short* AsY,
+                                       const unsigned short* BsY, unsigned short* AsA, const char* Ag_next3,
+                                       const char* Bg_next4, int64_t lda2, int64_t ldb2, int wave, const Lane& ln,
+                                       Frag& f0, Frag& f1, f32x16 (&acc)[4][4]) {
+    if (DMA_A) issue_A(Ag_next3, lda2, AsA, wave, ln);
+    load_frags(AsX, BsX, ln, 1, f1);
+    mma16<E>(f0, acc);
+    interleave16<DMA_A, true>();
+    if (!LAST) stage_barrier<VMCNT>();
+    if (DMA_B) issue_B(Bg_next4, ldb2, BsX, wave, ln);
+    if (!LAST) load_frags(AsY, BsY, ln, 0, f0);
+    mma16<E>(f1, acc);
+    interleave16<DMA_B, !LAST>();
+}
+
+template <typename E, typename OutT>
+__global__ __launch_bounds__(256) void gemm16_big(const unsigned short* __restrict__ A, int64_t lda, int64_t sa,
+                                                  const unsigned short* __restrict__ B, int64_t ldb, int64_t sb,
+                                                  OutT* __restrict__ C, int64_t ldc, int64_t sc, int K, int tiles_m,
+                                                  int tiles_n) {
+    __shared__ __attribute__((aligned(1024))) unsigned short As0[STAGE], As1[STAGE], As2[STAGE], As3[STAGE];
+    __shared__ __attribute__((aligned(1024))) unsigned short Bs0[STAGE], Bs1[STAGE], Bs2[STAGE], Bs3[STAGE];
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int total = tiles_m * tiles_n;
+    int L = blockIdx.x;
+    if (total % 8 == 0) L = (L & 7) * (total >> 3) + (L >> 3);
+    constexpr int GM = 4;
+    const int per_group = GM * tiles_n;
+    const int first_m = (L / per_group) * GM;
+    const int gsz = tiles_m - first_m < GM ? tiles_m - first_m : GM;
+    const int bm = first_m + (L % per_group) % gsz, bn = (L % per_group) / gsz;
+    const int wm = (wave & 1) * 128, wn = (wave >> 1) * 128;
+
+    Lane ln;
+    {
+        const int hb = lane >> 5, g = lane >> 4, r = lane & 15;
+        // B transfer: lane -> row lane/4 of its 16-row block, LDS position lane%4; rows n = 16*blk + lane/4
+        ln.goffB = (unsigned)(((int64_t)(lane >> 2) * ldb + 8 * ((lane & 3) ^ ((lane >> 4) & 3))) * 2);
+        // A transfer: lane -> row lane/32 of its 2-row block, LDS position lane%32; rows k = 2*blk + lane/32
+        const int ka = 2 * wave + (lane >> 5);
+        ln.goffA = (unsigned)(((int64_t)(lane >> 5) * lda + 8 * ((lane & 31) ^ (4 * (ka & 3)))) * 2);
+#pragma unroll
+        for (int ks = 0; ks < 2; ++ks) {
+            const int n = wn + (lane & 31);
+            ln.fb[ks] = n * BK + 8 * ((2 * ks + hb) ^ ((n >> 2) & 3));
+        }
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int k = 8 * (g >> 1) + (r >> 2);
+            const int m = wm + 32 * i + 16 * (g & 1) + 4 * (r & 3);
+            ln.fa[i] = k * BT + 8 * ((m >> 3) ^ (4 * (r >> 2))) + (m & 7);
+        }
+    }
+    const int64_t lda2 = lda * 2, ldb2 = ldb * 2;
+    // wave-uniform byte pointers to this wave's first rows of the k = 0 stage
+    const char* Ab = (const char*)(A + (int64_t)blockIdx.z * sa + (int64_t)bm * BT) + (int64_t)(2 * wave) * lda2;
+    const char* Bb = (const char*)(B + (int64_t)blockIdx.z * sb + (int64_t)bn * BT * ldb) + (int64_t)(16 * wave) * ldb2;
+    C += (int64_t)blockIdx.z * sc;
+    const int64_t a_step = (int64_t)BK * lda2;  // next K step of A: 32 rows down
+    const int64_t b_step = (int64_t)BK * 2;     // next K step of B: 32 elements along the row
+
+    f32x16 acc[4][4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) acc[i][j] = f32x16{0};
+
+    const int KT = K / BK;  // multiple of 4, >= 8 (checked on the host)
+    Frag f0, f1;
+    // prologue: stages 0..2 and the B half of stage 3 (28 transfers per wave)
+    issue_B(Bb, ldb2, Bs0, wave, ln);
+    issue_A(Ab, lda2, As0, wave, ln);
+    issue_B(Bb + b_step, ldb2, Bs1, wave, ln);
+    issue_A(Ab + a_step, lda2, As1, wave, ln);
+    issue_B(Bb + 2 * b_step, ldb2, Bs2, wave, ln);
+    issue_A(Ab + 2 * a_step, lda2, As2, wave, ln);
+    issue_B(Bb + 3 * b_step, ldb2, Bs3, wave, ln);
+    stage_barrier<20>();
+    load_frags(As0, Bs0, ln, 0, f0);
+
+#define KSTEP(X, Y, AA, DA, DB, VM, LAST, s)                                                                      \
+    k_step<E, DA, DB, VM, LAST>(As##X, Bs##X, As##Y, Bs##Y, As##AA, Ab + (int64_t)((s) + 3) * a_step,            \
+                                Bb + (int64_t)((s) + 4) * b_step, lda2, ldb2, wave, ln, f0, f1, acc)
+    int s = 0;
+    for (; s + 8 <= KT; s += 4) {
+        KSTEP(0, 1, 3, true, true, 16, false, s);
+        KSTEP(1, 2, 0, true, true, 16, false, s + 1);
+        KSTEP(2, 3, 1, true, true, 16, false, s + 2);
+        KSTEP(3, 0, 2, true, true, 16, false, s + 3);
+    }
+    // last four steps: only the A half of the final stage is still to be requested
+    KSTEP(0, 1, 3, true, false, 16, false, s);
+    KSTEP(1, 2, 0, false, false, 8, false, s + 1);
+    KSTEP(2, 3, 1, false, false, 0, false, s + 2);
+    KSTEP(3, 0, 2, false, false, 0, true, s + 3);
+#undef KSTEP
+
+    // Epilogue.  The lane's own offset (m within the wave tile, plus its 4*hb rows of n) is a
+    // 32-bit element offset; the part of n that is uniform across the wave goes into the base.
+    const unsigned lane_off = (unsigned)((lane & 31) + (int64_t)(4 * (lane >> 5)) * ldc);
+    OutT* Cw = C + (int64_t)bm * BT + wm + ((int64_t)bn * BT + wn) * ldc;
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                OutT* cu = Cw + 32 * i + (int64_t)(32 * j + 8 * (r >> 2) + (r & 3)) * ldc;
+                __builtin_nontemporal_store(cvt_out<E, OutT>(acc[i][j][r]), cu + lane_off);
+            }
+}
+
+template <typename E, typename OutT>
+void launch(const Problem& p, hipStream_t s) {
+    const int tiles_m = p.M / BT, tiles_n = p.N / BT;
+    hipLaunchKernelGGL((gemm16_big<E, OutT>), dim3((unsigned)(tiles_m * tiles_n), 1, (unsigned)p.batch), dim3(256), 0,
+                       s, (const unsigned short*)p.A, p.lda, p.sa, (const unsigned short*)p.B, p.ldb, p.sb,
+                       (OutT*)p.C, p.ldc, p.sc, p.K, tiles_m, tiles_n);
+}
+
+}  // namespace
+
+namespace mi {
+namespace gemm {
+
+bool big16_applicable(const Problem& p) {
+    if (p.in_dtype != MI_F16 && p.in_dtype != MI_BF16) return false;
+    return p.M % BT == 0 && p.N % BT == 0 && p.K % 128 == 0 && p.K >= 256 && aligned(p.A, 16) && aligned(p.B, 16) &&
+           p.lda % 8 == 0 && p.ldb % 8 == 0 && p.sa % 8 == 0 && p.sb % 8 == 0 && p.ldc < (1 << 26) &&
+           p.lda < (1 << 26) && p.ldb < (1 << 26) && (int64_t)(p.M / BT) * (p.N / BT) * p.batch >= 64;
+}
+
+void big16_launch(const Problem& p, hipStream_t s) {
+    const bool f32out = p.out_dtype == MI_F32;
+    if (p.in_dtype == MI_F16) {
+        if (f32out) launch<F16, float>(p, s);
+        else launch<F16, unsigned short>(p, s);
+    } else {
+        if (f32out) launch<BF16, float>(p, s);
+        else launch<BF16, unsigned short>(p, s);
+    }
+    set_variant("gemm16_big_256x256x32_ring4");
+}
+
+}  // namespace gemm
+}  // namespace mi

@@ -63,6 +63,40 @@ def test_matmul_integer_valued_inputs_are_exact(ct, orc):
         assert np.array_equal(orc.to_julia(C), A @ B)
 
 
+@pytest.mark.parametrize("M,N,K,T,out32", [(2048, 2048, 256, torch.float16, True), (2048, 2048, 384, torch.float16, False),
+                                            (4096, 1024, 512, torch.bfloat16, True), (1024, 4096, 640, torch.bfloat16, False)])
+def test_matmul_large_tile_kernel_exact(ct, orc, M, N, K, T, out32):
+    """Shapes that take the 256x256 direct-to-LDS kernel (>= 64 tiles, K % 128 == 0), with
+    small-integer operands so the expected result is exact: checks the swizzled LDS layouts,
+    the ring of stages (K/32 = 8, 12, 16, 20 steps) and the tile -> workgroup mapping."""
+    rng = np.random.default_rng(7)
+    A = rng.integers(-1, 2, (M, K)).astype(np.float32); B = rng.integers(-2, 3, (K, N)).astype(np.float32)
+    At = orc.from_julia(A).to(T).cuda(); Bt = orc.from_julia(B).to(T).cuda()
+    C = torch.empty((N, M), dtype=torch.float32 if out32 else T, device="cuda")
+    ct.matmul_kernel(At, Bt, C, 64, 64, 64)
+    assert "big" in ct.last_variant()
+    ref = A @ B
+    assert out32 or np.abs(ref).max() <= 256  # integers up to 256 are exact in bf16's 8 bits as well
+    assert np.array_equal(orc.to_julia(C).astype(np.float32), ref)
+
+
+def test_batch_matmul_large_tile_kernel(ct, orc):
+    rng = np.random.default_rng(8)
+    M, K, N, Bn = 1024, 256, 1024, 4
+    A = rng.integers(-2, 3, (M, K, Bn)).astype(np.float32); B = rng.integers(-2, 3, (K, N, Bn)).astype(np.float32)
+    At = orc.from_julia(A).to(torch.float16).cuda(); Bt = orc.from_julia(B).to(torch.float16).cuda()
+    C = torch.empty((Bn, N, M), dtype=torch.float16, device="cuda")
+    ct.batch_matmul_kernel(At, Bt, C, 128, 128, 64)
+    assert "big" in ct.last_variant()
+    assert np.array_equal(orc.to_julia(C).astype(np.float32), np.einsum("mkb,knb->mnb", A, B))
+    # the same through padded leading dimensions (views of wider buffers)
+    Aw = torch.zeros((Bn, K, M + 64), dtype=torch.float16, device="cuda"); Aw[:, :, :M] = At
+    Bw = torch.zeros((Bn, N, K + 8), dtype=torch.float16, device="cuda"); Bw[:, :, :K] = Bt
+    C2 = torch.empty_like(C)
+    ct.batch_matmul_kernel(Aw[:, :, :M], Bw[:, :, :K], C2, 128, 128, 64)
+    assert "big" in ct.last_variant() and torch.equal(C, C2)
+
+
 def test_matmul_padded_leading_dims_and_misaligned(ct, orc):
     rng = np.random.default_rng(1)
     M, N, K = 100, 90, 70

@@ -252,6 +252,355 @@ __global__ __launch_bounds__(256) void fmha_fwd_kernel(const unsigned short* __r
     }
 }
 
+// ---- main kernel: direct global->LDS K/V tiles, double-buffered, 64 queries per wave ----------
+// Used when every row is 16-byte aligned.  A workgroup owns 128 queries of one (batch, head):
+// for D = 64 two waves of 64 queries (two 32-query MFMA column tiles each, so every K / V
+// fragment read from LDS feeds two MFMAs), for D = 128 four waves of 32 queries.  K and V tiles
+// of 64 keys travel global -> LDS with global_load_lds (no staging registers) into two stages;
+// the transfer of tile t+1 is issued right after the barrier that publishes tile t.
+//   K tile [key][d]: 16-byte chunk c of row `key` at position c ^ (key & 7)
+//   V tile [key][d]: chunk c at position c ^ ((D/32) * (key & 3)), which spreads the 4 rows x 32
+//     bytes of a transpose-read group over distinct banks.
+// Softmax bookkeeping per lane: running max m (shared by lanes l and l^32 after one exchange
+// per tile), running sum l of the lane's own half of the keys (the halves are added once at
+// the end), taken over the scores AFTER rounding to the storage type, i.e. over exactly the
+// weights that multiply V.  The accumulator is rescaled only on tiles where some row's max
+// actually rose.  Workgroups are numbered so that all query tiles of one (batch, head) run
+// on the same XCD and share its K/V in that XCD's L2.
+typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+
+template <typename E> struct Pack;
+template <> struct Pack<F16> {
+    static __device__ __forceinline__ unsigned pack(float a, float b) {
+        f16x2 v = {(_Float16)a, (_Float16)b};
+        return __builtin_bit_cast(unsigned, v);
+    }
+    static __device__ __forceinline__ float sum2(unsigned p, float acc) {
+        const f16x2 one = {(_Float16)1.0f, (_Float16)1.0f};
+        return __builtin_amdgcn_fdot2(__builtin_bit_cast(f16x2, p), one, acc, false);
+    }
+};
+template <> struct Pack<BF16> {
+    static __device__ __forceinline__ unsigned pack(float a, float b) {
+        bf16x2 v = {(__bf16)a, (__bf16)b};
+        return __builtin_bit_cast(unsigned, v);
+    }
+    static __device__ __forceinline__ float sum2(unsigned p, float acc) {
+        const bf16x2 one = {(__bf16)1.0f, (__bf16)1.0f};
+        return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2, p), one, acc, false);
+    }
+};
+
+typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
+
+__device__ __forceinline__ void gload_lds16(const void* g, void* lds_wave_base) {
+    __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)g,
+                                     (__attribute__((address_space(3))) void*)lds_wave_base, 16, 0, 0);
+}
+
+template <int D, int NW>
+struct DmaLane {
+    static constexpr int TPW = (D / 8) / NW;  // 1 KB transfers per wave per tile, for K and for V
+    unsigned koff[TPW], voff[TPW];            // byte offsets of the lane's chunk, relative to the tile's first key
+};
+
+template <typename E, int D, int JT, bool CAUSAL>
+struct FmhaDma {
+    static constexpr int NW = 4 / JT;          // waves per workgroup (128 queries)
+    static constexpr int KSTEPS = D / 16, DT = D / 32, CH = D / 8;
+    static constexpr int TPW = (D / 8) / NW;
+    static constexpr int TILE = kKV * D;       // elements per K or V stage
+
+    struct State {
+        s16x8 qf[JT][KSTEPS];
+        f32x16 o[JT][DT];
+        float m[JT], l[JT];
+        unsigned kfo[KSTEPS];  // K fragment element offsets per k-step (+ 32*kt*D)
+        unsigned vfo[DT];      // V fragment element offsets per d tile (+ (32*kt + 16*c)*D, + 8*D for the high half)
+        int my_pos[JT];     // position of this lane's query in column tile j
+        int first_pos[JT];  // position of the first query of column tile j
+    };
+
+    static __device__ __forceinline__ void issue(const char* Kg, const char* Vg, unsigned short* Ks,
+                                                 unsigned short* Vs, int wave, const DmaLane<D, NW>& dl) {
+#pragma unroll
+        for (int i = 0; i < TPW; ++i) gload_lds16(Kg + dl.koff[i], Ks + (wave + NW * i) * 512);
+#pragma unroll
+        for (int i = 0; i < TPW; ++i) gload_lds16(Vg + dl.voff[i], Vs + (wave + NW * i) * 512);
+    }
+
+    // JM: bit j set = column tile j takes part in this KV tile (a causal wave drops its early
+    // query tile once the keys pass that tile's diagonal).
+    template <int JM>
+    static __device__ __forceinline__ void compute(const unsigned short* Ks, const unsigned short* Vs, State& st,
+                                                   int kv0, int Skv, float scale2, int lane) {
+        const int hb = lane >> 5;
+        // ---- S^T = K . Q ---------------------------------------------------------------
+        f32x16 s[JT][2];
+#pragma unroll
+        for (int j = 0; j < JT; ++j) s[j][0] = s[j][1] = f32x16{0};
+#define ACT(j) ((JM >> (j)) & 1)
+#pragma unroll
+        for (int kt = 0; kt < 2; ++kt)
+#pragma unroll
+            for (int ks = 0; ks < KSTEPS; ++ks) {
+                s16x8 kf = *reinterpret_cast<const s16x8*>(Ks + st.kfo[ks] + 32 * kt * D);
+#pragma unroll
+                for (int j = 0; j < JT; ++j)
+                    if (ACT(j)) s[j][kt] = E::mfma32(kf, st.qf[j][ks], s[j][kt]);
+            }
+        // ---- mask (causal diagonal, ragged KV tail) ------------------------------------------
+#pragma unroll
+        for (int j = 0; j < JT; ++j) {
+            if (!ACT(j)) continue;
+            const bool need_mask = (CAUSAL && kv0 + kKV - 1 > st.first_pos[j]) || (kv0 + kKV > Skv);
+            if (need_mask) {
+                // last visible key, relative to this lane's first key of the tile
+                int lim = Skv - 1;
+                if (CAUSAL && st.my_pos[j] < lim) lim = st.my_pos[j];
+                lim -= kv0 + 4 * hb;
+#pragma unroll
+                for (int kt = 0; kt < 2; ++kt)
+#pragma unroll
+                    for (int r = 0; r < 16; ++r)
+                        s[j][kt][r] = (32 * kt + 8 * (r >> 2) + (r & 3) <= lim) ? s[j][kt][r] : -INFINITY;
+            }
+        }
+        // ---- online softmax ---------------------------------------------------------------------
+        unsigned pf[JT][2][2][4];  // [j][kt][16-key chunk][4 dwords = 8 packed values]
+#pragma unroll
+        for (int j = 0; j < JT; ++j) {
+            if (!ACT(j)) continue;
+            float mx = fmaxf(s[j][0][0], s[j][1][0]);
+#pragma unroll
+            for (int r = 1; r < 16; ++r) mx = fmaxf(fmaxf(mx, s[j][0][r]), s[j][1][r]);
+            mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+            const float m_new = fmaxf(st.m[j], mx * scale2);
+            if (__any(m_new > st.m[j])) {  // some row's max rose: rescale the wave's accumulators
+                const float alpha = __builtin_amdgcn_exp2f(st.m[j] - m_new);
+                st.l[j] *= alpha;
+#pragma unroll
+                for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+                    for (int r = 0; r < 16; ++r) st.o[j][dt][r] *= alpha;
+                st.m[j] = m_new;
+            }
+            const float mj = st.m[j];
+            float lsum = st.l[j];
+#pragma unroll
+            for (int kt = 0; kt < 2; ++kt)
+#pragma unroll
+                for (int r = 0; r < 16; r += 2) {
+                    const float p0 = __builtin_amdgcn_exp2f(s[j][kt][r] * scale2 - mj);
+                    const float p1 = __builtin_amdgcn_exp2f(s[j][kt][r + 1] * scale2 - mj);
+                    const unsigned pk = Pack<E>::pack(p0, p1);
+                    lsum = Pack<E>::sum2(pk, lsum);
+                    pf[j][kt][r >> 3][(r & 7) >> 1] = pk;
+                }
+            st.l[j] = lsum;
+        }
+        // ---- O^T += V . P ------------------------------------------------------------------------
+#pragma unroll
+        for (int kt = 0; kt < 2; ++kt)
+#pragma unroll
+            for (int c = 0; c < 2; ++c)
+#pragma unroll
+                for (int dt = 0; dt < DT; ++dt) {
+                    const unsigned short* p = Vs + st.vfo[dt] + (32 * kt + 16 * c) * D;
+                    s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16(LDS_PTR(s16x4, p));
+                    s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(LDS_PTR(s16x4, p + 8 * D));
+                    s16x8 vf = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+#pragma unroll
+                    for (int j = 0; j < JT; ++j) {
+                        if (!ACT(j)) continue;
+                        u32x4 pw = {pf[j][kt][c][0], pf[j][kt][c][1], pf[j][kt][c][2], pf[j][kt][c][3]};
+                        st.o[j][dt] = E::mfma32(vf, __builtin_bit_cast(s16x8, pw), st.o[j][dt]);
+                    }
+                }
+#undef ACT
+    }
+};
+
+__device__ __forceinline__ void tile_barrier() {
+    // own LDS reads done, own transfers landed; gfx9 s_waitcnt encoding of vmcnt(0) lgkmcnt(0)
+    __builtin_amdgcn_s_waitcnt(0x0070);
+    asm volatile("" ::: "memory");
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+}
+
+// Query tiles of 32 are dealt to the waves as follows.  Non-causal: wave w of workgroup qb
+// takes the JT adjacent tiles starting at JT*(NW*qb + w).  Causal (JT == 2): the work of a
+// tile grows with its index, so a wave takes one early and one late tile, u and NT-1-u with
+// u = 2*qb + w; every wave then has the same number of MFMAs, and the two waves of a workgroup
+// need the same KV range.  The early tile simply drops out of the KV loop after its diagonal.
+template <typename E, int D, int JT, bool CAUSAL>
+__global__ __launch_bounds__(128 * 2 / JT) __attribute__((amdgpu_waves_per_eu(2, 2))) void fmha_fwd_dma_kernel(
+    const unsigned short* __restrict__ Q, Strides qs, const unsigned short* __restrict__ K, Strides ks,
+    const unsigned short* __restrict__ V, Strides vs, unsigned short* __restrict__ O, Strides os, int Sq, int Skv,
+    int H, int group, float scale2, int input_pos, int nqb, int nbh) {
+    using F = FmhaDma<E, D, JT, CAUSAL>;
+    constexpr int NW = F::NW, KSTEPS = F::KSTEPS, DT = F::DT, CH = F::CH, TPW = F::TPW;
+    constexpr bool PAIRED = CAUSAL && JT == 2;
+    __shared__ __attribute__((aligned(1024))) unsigned short Ks0[F::TILE], Ks1[F::TILE], Vs0[F::TILE], Vs1[F::TILE];
+
+    const int tid = threadIdx.x, lane = tid & 63, hb = lane >> 5;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    // Workgroup -> (query block, batch*head): ids congruent mod 8 share an XCD; give each XCD
+    // whole (batch, head) pairs so their K/V stay in that XCD's L2.  Low block index = most work.
+    int qb, bh;
+    {
+        const int L = blockIdx.x;
+        if (nbh % 8 == 0) {
+            const int idx = L >> 3;
+            bh = (L & 7) + 8 * (idx / nqb);
+            qb = idx % nqb;
+        } else {
+            bh = L / nqb;
+            qb = L % nqb;
+        }
+        if (CAUSAL && !PAIRED) qb = nqb - 1 - qb;
+    }
+    const int batch = bh / H, head = bh % H, kvh = head / group;
+    Q += (int64_t)head * qs.s2 + (int64_t)batch * qs.s3;
+    O += (int64_t)head * os.s2 + (int64_t)batch * os.s3;
+    const char* Kg = (const char*)(K + (int64_t)kvh * ks.s2 + (int64_t)batch * ks.s3);
+    const char* Vg = (const char*)(V + (int64_t)kvh * vs.s2 + (int64_t)batch * vs.s3);
+
+    const int NT = (Sq + 31) / 32;  // query tiles of 32
+    int tq[JT];                     // this wave's query tiles (wave-uniform); -1 = none
+    int wg_last_tile;               // highest query tile of the workgroup (bounds the causal KV loop)
+    if (PAIRED) {
+        const int u = 2 * qb + wave;
+        const int hi = NT - 1 - u;
+        tq[0] = (u < hi) ? u : -1;
+        tq[JT - 1] = (u <= hi) ? hi : -1;
+        wg_last_tile = NT - 1 - 2 * qb;
+    } else {
+#pragma unroll
+        for (int j = 0; j < JT; ++j) {
+            const int t = JT * (NW * qb + wave) + j;
+            tq[j] = t < NT ? t : -1;
+        }
+        wg_last_tile = JT * NW * (qb + 1) - 1;
+        if (wg_last_tile > NT - 1) wg_last_tile = NT - 1;
+    }
+
+    typename F::State st;
+    int my_q[JT], last_pos[JT];
+#pragma unroll
+    for (int j = 0; j < JT; ++j) {
+        my_q[j] = tq[j] >= 0 ? 32 * tq[j] + (lane & 31) : Sq;
+        st.my_pos[j] = input_pos + my_q[j];
+        st.first_pos[j] = input_pos + 32 * tq[j];
+        last_pos[j] = tq[j] >= 0 ? st.first_pos[j] + 31 : -1;
+#pragma unroll
+        for (int s = 0; s < KSTEPS; ++s) {
+            s16x8 v = {0};
+            if (my_q[j] < Sq) v = *reinterpret_cast<const s16x8*>(Q + (int64_t)my_q[j] * qs.s1 + 16 * s + 8 * hb);
+            st.qf[j][s] = v;
+        }
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt) st.o[j][dt] = f32x16{0};
+        st.m[j] = -INFINITY;
+        st.l[j] = 0.f;
+    }
+    {
+        const int key = lane & 31;
+#pragma unroll
+        for (int s = 0; s < KSTEPS; ++s) st.kfo[s] = key * D + 8 * ((2 * s + hb) ^ (key & 7));
+        const int g = lane >> 4, r = lane & 15;
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt) {
+            const int row = 4 * (g >> 1) + (r >> 2);
+            const int col = 32 * dt + 16 * (g & 1) + 4 * (r & 3);
+            st.vfo[dt] = row * D + 8 * ((col >> 3) ^ ((D / 32) * (r >> 2))) + (col & 7);
+        }
+    }
+    DmaLane<D, NW> dl;
+#pragma unroll
+    for (int i = 0; i < TPW; ++i) {
+        const int t = wave + NW * i;  // transfer index: rows (512/D)*t ... of the tile
+        const int key = (512 / D) * t + lane / CH, pos = lane % CH;
+        dl.koff[i] = (unsigned)(((int64_t)key * ks.s1 + 8 * (pos ^ (key & 7))) * 2);
+        dl.voff[i] = (unsigned)(((int64_t)key * vs.s1 + 8 * (pos ^ ((D / 32) * (key & 3)))) * 2);
+    }
+
+    int kv_end = Skv;
+    if (CAUSAL) {
+        const int lim = input_pos + 32 * (wg_last_tile + 1);  // one past the workgroup's last query position
+        kv_end = lim < Skv ? lim : Skv;
+        if (kv_end < 0) kv_end = 0;
+    }
+    const int ntiles = (kv_end + kKV - 1) / kKV;
+    const int64_t k_tile_bytes = (int64_t)kKV * ks.s1 * 2, v_tile_bytes = (int64_t)kKV * vs.s1 * 2;
+
+    // Rows past the end of K / V in the last tile are never dereferenced: their lanes re-read
+    // the last valid row (the masked scores make the values irrelevant, and finite).
+    auto issue_tile = [&](int t, unsigned short* Ksx, unsigned short* Vsx) {
+        if ((t + 1) * kKV <= Skv) {
+            F::issue(Kg + t * k_tile_bytes, Vg + t * v_tile_bytes, Ksx, Vsx, wave, dl);
+        } else {
+            DmaLane<D, NW> cl;
+#pragma unroll
+            for (int i = 0; i < TPW; ++i) {
+                const int tr = wave + NW * i;
+                int key = (512 / D) * tr + lane / CH;
+                const int pos = lane % CH;
+                const int swk = key & 7, swv = key & 3;
+                if (t * kKV + key >= Skv) key = Skv - 1 - t * kKV;
+                cl.koff[i] = (unsigned)(((int64_t)key * ks.s1 + 8 * (pos ^ swk)) * 2);
+                cl.voff[i] = (unsigned)(((int64_t)key * vs.s1 + 8 * (pos ^ ((D / 32) * swv))) * 2);
+            }
+            F::issue(Kg + t * k_tile_bytes, Vg + t * v_tile_bytes, Ksx, Vsx, wave, cl);
+        }
+    };
+    // Which of the wave's column tiles still see keys of the tile starting at kv0.
+    auto run_tile = [&](const unsigned short* Ksx, const unsigned short* Vsx, int kv0) {
+        if (JT == 2) {
+            const bool a0 = tq[0] >= 0 && (!CAUSAL || kv0 <= last_pos[0]);
+            const bool a1 = tq[JT - 1] >= 0 && (!CAUSAL || kv0 <= last_pos[JT - 1]);
+            if (a0 && a1) F::template compute<3>(Ksx, Vsx, st, kv0, Skv, scale2, lane);
+            else if (a1) F::template compute<2>(Ksx, Vsx, st, kv0, Skv, scale2, lane);
+            else if (a0) F::template compute<1>(Ksx, Vsx, st, kv0, Skv, scale2, lane);
+        } else {
+            if (tq[0] >= 0 && (!CAUSAL || kv0 <= last_pos[0])) F::template compute<1>(Ksx, Vsx, st, kv0, Skv, scale2, lane);
+        }
+    };
+
+    if (ntiles > 0) issue_tile(0, Ks0, Vs0);
+    for (int t = 0; t < ntiles; t += 2) {
+        tile_barrier();  // tile t has landed for every wave; every wave is done with the other stage
+        if (t + 1 < ntiles) issue_tile(t + 1, Ks1, Vs1);
+        run_tile(Ks0, Vs0, t * kKV);
+        if (t + 1 < ntiles) {
+            tile_barrier();
+            if (t + 2 < ntiles) issue_tile(t + 2, Ks0, Vs0);
+            run_tile(Ks1, Vs1, (t + 1) * kKV);
+        }
+    }
+
+    // ---- epilogue: add the two half-row sums, O / l (approximate reciprocal), round, store -----
+#pragma unroll
+    for (int j = 0; j < JT; ++j) {
+        const float l_tot = st.l[j] + __shfl_xor(st.l[j], 32, 64);
+        if (my_q[j] < Sq) {
+            const float inv = __builtin_amdgcn_rcpf(l_tot);
+            unsigned short* op = O + (int64_t)my_q[j] * os.s1;
+#pragma unroll
+            for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+                for (int g = 0; g < 4; ++g) {
+                    s16x4 w;
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) w[e] = E::cvt(st.o[j][dt][4 * g + e] * inv);
+                    *reinterpret_cast<s16x4*>(op + 32 * dt + 8 * g + 4 * hb) = w;
+                }
+        }
+    }
+}
+
 bool vec16(const mi_tile_array* a) {
     return aligned(a->ptr, 16) && a->strides[1] % 8 == 0 && a->strides[2] % 8 == 0 && a->strides[3] % 8 == 0;
 }
@@ -263,6 +612,21 @@ void launch(dim3 grid, hipStream_t s, bool causal, const mi_tile_array* Q, const
     Strides qs{Q->strides[1], Q->strides[2], Q->strides[3]}, ks{K->strides[1], K->strides[2], K->strides[3]},
         vs{V->strides[1], V->strides[2], V->strides[3]}, os{O->strides[1], O->strides[2], O->strides[3]};
     const int Sq = (int)Q->sizes[1], Skv = (int)K->sizes[1];
+    if (vec_ok && K->strides[1] < (1 << 24) && V->strides[1] < (1 << 24)) {
+        constexpr int JT = D == 64 ? 2 : 1;
+        const int nqb = (int)grid.x, nbh = (int)grid.y;
+        dim3 g1((unsigned)(nqb * nbh)), blk(128 * 2 / JT);
+        if (causal)
+            hipLaunchKernelGGL((fmha_fwd_dma_kernel<E, D, JT, true>), g1, blk, 0, s, (const unsigned short*)Q->ptr, qs,
+                               (const unsigned short*)K->ptr, ks, (const unsigned short*)V->ptr, vs,
+                               (unsigned short*)O->ptr, os, Sq, Skv, H, group, scale2, input_pos, nqb, nbh);
+        else
+            hipLaunchKernelGGL((fmha_fwd_dma_kernel<E, D, JT, false>), g1, blk, 0, s, (const unsigned short*)Q->ptr, qs,
+                               (const unsigned short*)K->ptr, ks, (const unsigned short*)V->ptr, vs,
+                               (unsigned short*)O->ptr, os, Sq, Skv, H, group, scale2, input_pos, nqb, nbh);
+        set_variant(D == 64 ? "fmha_dma_q128_kv64_d64_w64q" : "fmha_dma_q128_kv64_d128_w32q");
+        return;
+    }
     if (causal)
         hipLaunchKernelGGL((fmha_fwd_kernel<E, D, true>), grid, dim3(256), 0, s, (const unsigned short*)Q->ptr, qs,
                            (const unsigned short*)K->ptr, ks, (const unsigned short*)V->ptr, vs,
@@ -271,6 +635,7 @@ void launch(dim3 grid, hipStream_t s, bool causal, const mi_tile_array* Q, const
         hipLaunchKernelGGL((fmha_fwd_kernel<E, D, false>), grid, dim3(256), 0, s, (const unsigned short*)Q->ptr, qs,
                            (const unsigned short*)K->ptr, ks, (const unsigned short*)V->ptr, vs,
                            (unsigned short*)O->ptr, os, Sq, Skv, H, group, scale2, input_pos, vec_ok);
+    set_variant(D == 64 ? "fmha_regstage_q128_kv64_d64" : "fmha_regstage_q128_kv64_d128");
 }
 
 }  // namespace
@@ -314,6 +679,5 @@ extern "C" int mi_fmha_kernel(const mi_tile_array* Q, const mi_tile_array* K, co
         if (D == 64) launch<BF16, 64>(grid, s, causal, Q, K, V, Out, H, QUERY_GROUP_SIZE, scale2, input_pos, vec_ok);
         else launch<BF16, 128>(grid, s, causal, Q, K, V, Out, H, QUERY_GROUP_SIZE, scale2, input_pos, vec_ok);
     }
-    set_variant(D == 64 ? "fmha_q128_kv64_d64_mfma32" : "fmha_q128_kv64_d128_mfma32");
     return launch_status();
 }

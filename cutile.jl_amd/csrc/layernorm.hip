@@ -17,6 +17,7 @@
 // one grid have no forward-progress guarantee relative to each other on this hardware.
 #include "common.h"
 #include <math.h>
+#include <stdlib.h>
 
 namespace {
 
@@ -175,6 +176,7 @@ __global__ __launch_bounds__(BLOCK) void ln_bwd_kernel(float* __restrict__ DX, i
                                                        int64_t M, int G, int S) {
     constexpr int NW = BLOCK / 64;
     __shared__ float red[2 * NW];
+    __shared__ float stage[BLOCK * VPT * 4];
     const int g = blockIdx.x % G, s = blockIdx.x / G;
     float w[VPT][4], dw[VPT][4], db[VPT][4];
     load_row<BLOCK, VPT, ALIGNED, false>(W, N, w);
@@ -216,23 +218,28 @@ __global__ __launch_bounds__(BLOCK) void ln_bwd_kernel(float* __restrict__ DX, i
             }
         store_row<BLOCK, VPT, ALIGNED>(DX + m * lddx, N, x);
     }
+    // Flush through LDS so that consecutive lanes add to consecutive addresses: a float atomic
+    // instruction then covers 256 contiguous bytes instead of 64 scattered words (memory-side
+    // float atomics are the scarce resource here, not bandwidth).
     float* dwp = DW + (int64_t)g * lddw;
     float* dbp = DB + (int64_t)g * lddb;
 #pragma unroll
-    for (int v = 0; v < VPT; ++v) {
-        const int e0 = (threadIdx.x + v * BLOCK) * 4;
+    for (int pass = 0; pass < 2; ++pass) {
 #pragma unroll
-        for (int q = 0; q < 4; ++q) {
-            if (e0 + q < N) {
-                if (S == 1) {
-                    dwp[e0 + q] += dw[v][q];
-                    dbp[e0 + q] += db[v][q];
-                } else {
-                    unsafeAtomicAdd(dwp + e0 + q, dw[v][q]);
-                    unsafeAtomicAdd(dbp + e0 + q, db[v][q]);
-                }
+        for (int v = 0; v < VPT; ++v)
+#pragma unroll
+            for (int q = 0; q < 4; ++q) stage[(threadIdx.x + v * BLOCK) * 4 + q] = pass == 0 ? dw[v][q] : db[v][q];
+        __syncthreads();
+        float* dst = pass == 0 ? dwp : dbp;
+        for (int c = threadIdx.x; c < N; c += BLOCK) {
+            if (S == 1) dst[c] += stage[c];
+            else {
+#ifndef EXP_NOATOMIC
+                unsafeAtomicAdd(dst + c, stage[c]);
+#endif
             }
         }
+        __syncthreads();
     }
 }
 
@@ -275,17 +282,19 @@ __global__ __launch_bounds__(BLOCK) void ln_bwd_long_kernel(float* __restrict__ 
 }
 
 // ---- backward: final reduction over the partial slots -----------------------------------
-// 64 consecutive n per workgroup; the 4 waves split the slots, LDS combines them.
-__global__ __launch_bounds__(256) void ln_dwdb_kernel(const float* __restrict__ DW, int64_t lddw,
-                                                      const float* __restrict__ DB, int64_t lddb,
-                                                      float* __restrict__ FDW, float* __restrict__ FDB,
-                                                      int64_t N, int G) {
-    __shared__ float part[2][4][64];
+// 64 consecutive n per workgroup; its 16 waves split the slots (independent loads, one round
+// trip for GROUP_SIZE_M <= 64), LDS combines them in a fixed order.
+__global__ __launch_bounds__(1024) void ln_dwdb_kernel(const float* __restrict__ DW, int64_t lddw,
+                                                       const float* __restrict__ DB, int64_t lddb,
+                                                       float* __restrict__ FDW, float* __restrict__ FDB,
+                                                       int64_t N, int G) {
+    __shared__ float part[2][16][64];
     const int lane = threadIdx.x & 63, wq = threadIdx.x >> 6;
     const int64_t n = (int64_t)blockIdx.x * 64 + lane;
     float a = 0.f, b = 0.f;
     if (n < N) {
-        for (int g = wq; g < G; g += 4) {
+#pragma unroll 4
+        for (int g = wq; g < G; g += 16) {
             a += DW[n + g * lddw];
             b += DB[n + g * lddb];
         }
@@ -293,9 +302,11 @@ __global__ __launch_bounds__(256) void ln_dwdb_kernel(const float* __restrict__ 
     part[0][wq][lane] = a;
     part[1][wq][lane] = b;
     __syncthreads();
-    if (wq == 0 && n < N) {
-        FDW[n] = (part[0][0][lane] + part[0][1][lane]) + (part[0][2][lane] + part[0][3][lane]);
-        FDB[n] = (part[1][0][lane] + part[1][1][lane]) + (part[1][2][lane] + part[1][3][lane]);
+    if (wq < 2 && n < N) {
+        float t = 0.f;
+#pragma unroll
+        for (int k = 0; k < 16; ++k) t += part[wq][k][lane];
+        (wq == 0 ? FDW : FDB)[n] = t;
     }
 }
 
@@ -430,12 +441,17 @@ extern "C" int mi_layer_norm_bwd_dx_partial_dwdb(
         set_variant("ln_bwd_long_b256");
         return launch_status();
     }
-    // Splits per slot: enough workgroups to cover the 256 CUs a few times over, but at
-    // least ~4 rows per workgroup so the register partials amortise the atomics.
+    // Splits per slot: about two workgroups per CU (measured optimum on MI355X: more
+    // workgroups cost more atomics, fewer leave HBM idle), and at least ~4 rows per workgroup
+    // so the register partials amortise the flush.
     const int64_t rows_per_slot = cld(M, (int64_t)G);
-    int64_t S = cld((int64_t)1024, (int64_t)G);
+    int64_t S = cld((int64_t)512, (int64_t)G);
     if (S > cld(rows_per_slot, (int64_t)4)) S = cld(rows_per_slot, (int64_t)4);
     if (S < 1) S = 1;
+    if (const char* env = getenv("MI_LN_BWD_SPLITS")) {  // tuning override: workgroups per partial slot
+        const long v = atol(env);
+        if (v >= 1 && v <= rows_per_slot) S = v;
+    }
     const bool al = rows_vec_ok(X) && rows_vec_ok(DX) && rows_vec_ok(DY) && rows_vec_ok(W);
     const int vecs = (int)cld(N, 4);
     dim3 grid((unsigned)(G * S));
@@ -464,10 +480,10 @@ extern "C" int mi_layer_norm_bwd_dwdb(const mi_tile_array* DW, const mi_tile_arr
     if (cld(N, (int64_t)TILE_N) > MI_MAX_GRID_DIM) return MI_E_GRID;
     if (N == 0) return MI_OK;
     if (G > 0x7fffffff) return MI_E_SHAPE;
-    hipLaunchKernelGGL(ln_dwdb_kernel, dim3((unsigned)cld(N, (int64_t)64)), dim3(256), 0,
+    hipLaunchKernelGGL(ln_dwdb_kernel, dim3((unsigned)cld(N, (int64_t)64)), dim3(1024), 0,
                        (hipStream_t)stream, (const float*)DW->ptr, DW->strides[1],
                        (const float*)DB->ptr, DB->strides[1], (float*)FINAL_DW->ptr,
                        (float*)FINAL_DB->ptr, N, (int)G);
-    set_variant("ln_dwdb_b256");
+    set_variant("ln_dwdb_b1024");
     return launch_status();
 }

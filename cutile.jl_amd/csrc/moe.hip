@@ -67,64 +67,83 @@ __device__ __forceinline__ unsigned e4m3x2_to_f16x2(unsigned w16) {
     return __builtin_bit_cast(unsigned, h);
 }
 
-constexpr int kNT = 128;  // output channels per workgroup (4 waves x 32)
-constexpr int kKT = 64;   // K step
-constexpr int kMaxMT = 4; // token tiles of 32 per workgroup (TILE_M <= 128)
+constexpr int kTT = 32;   // token slots per workgroup (one MFMA row tile)
 
 // E: activation/output element traits; W8: weights are E4M3FN bytes (else same type as A).
-template <typename E, bool W8>
+// NTW: waves side by side along n (workgroup strip = 32*NTW channels); the other 4/NTW waves
+// split each K step between them and their accumulators are added through LDS at the end.
+// kKT: K step.  Two shapes are used: (NTW=4, kKT=128) when N is large enough to give every CU
+// several strips, and (NTW=1, kKT=256) for small N, where 32-channel strips with a 4-way
+// in-workgroup K split keep ~4x more workgroups (and bytes) in flight.
+// Workgroup = (one tile of up to 32 consecutive sorted slots, one strip of 32*NTW channels).
+// With ~16 tokens per expert most 32-slot tiles of a TILE_M block hold only padding; their
+// workgroups leave at once, so the expert's weight strip is streamed by exactly as many
+// workgroups as it has (started) 32-token tiles.  Small register footprint -> many
+// workgroups per CU, each with the next weight tile already in flight.
+template <typename E, bool W8, int NTW, int kKT>
 __global__ __launch_bounds__(256) void fused_moe_kernel(
     const unsigned short* __restrict__ A, int64_t lda, int num_a_cols, const void* __restrict__ Bv, int64_t ldb,
     int64_t sbe, unsigned short* __restrict__ C, int64_t ldc, int total_tokens,
     const unsigned short* __restrict__ topk_weights, const int* __restrict__ sorted_token_ids, int num_slots,
     const int* __restrict__ sorted_expert_ids, const float* __restrict__ b_scale, int64_t ld_scale, int K, int N,
-    int num_experts, int replicas, bool mul_routed_weight, int TILE_M, int n_blocks, bool vecA, bool vecB) {
-    __shared__ __attribute__((aligned(16))) unsigned short Bs[kNT * kKT];          // [n][k], 16-byte chunks XOR-swizzled
-    __shared__ __attribute__((aligned(16))) unsigned short As[32 * kMaxMT * kKT];  // [slot][k], same swizzle
-    __shared__ int s_tok[32 * kMaxMT];
+    int num_experts, int replicas, bool mul_routed_weight, int TILE_M, int tile_slots, int n_blocks, bool vecA,
+    bool vecB) {
+    constexpr int kNT = 32 * NTW, KW = 4 / NTW;
+    __shared__ __attribute__((aligned(16))) unsigned short Bs[kNT * kKT];  // [n][k], 16-byte chunks XOR-swizzled
+    __shared__ __attribute__((aligned(16))) unsigned short As[kTT * kKT];  // [slot][k], same swizzle
+    __shared__ int s_tok[kTT];
+    __shared__ int s_any;
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, hb = lane >> 5;
-    // consecutive workgroups share the token block (and therefore the activations in L2)
-    const int bid_m = blockIdx.x / n_blocks, bid_n = blockIdx.x % n_blocks;
+    const int wn = wave % NTW, wk = wave / NTW;  // position along n / along the K split
+    // consecutive workgroups share the token tile (and therefore the activations in L2)
+    const int tile = blockIdx.x / n_blocks, bid_n = blockIdx.x % n_blocks;
     const int n0 = bid_n * kNT;
-    const int slot0 = bid_m * TILE_M;
-    const int expert = sorted_expert_ids[bid_m] - 1;
-    const bool expert_ok = expert >= 0 && expert < num_experts;
+    const int slot0 = tile * tile_slots;            // tile_slots = min(TILE_M, 32) divides TILE_M
+    const int expert = sorted_expert_ids[slot0 / TILE_M] - 1;
 
-    for (int i = tid; i < TILE_M; i += 256) {
-        const int s = slot0 + i;
-        s_tok[i] = s < num_slots ? sorted_token_ids[s] : 0;  // 1-based; 0 / >total = no token
+    if (tid == 0) s_any = 0;
+    __syncthreads();
+    if (tid < kTT) {
+        const int sl = slot0 + tid;
+        int t = (tid < tile_slots && sl < num_slots) ? sorted_token_ids[sl] : 0;  // 1-based; 0 / >total = no token
+        if (t < 1 || t > total_tokens) t = 0;
+        s_tok[tid] = t;
+        if (t) s_any = 1;
     }
     __syncthreads();
-    // number of 32-slot tiles that contain at least one real token
-    int mt_used = 0;
-    for (int i = 0; i < TILE_M; ++i) {
-        const int t = s_tok[i];
-        if (t >= 1 && t <= total_tokens) mt_used = i / 32 + 1;
-    }
-    if (mt_used == 0 || !expert_ok) return;  // uniform across the workgroup
+    if (!s_any || expert < 0 || expert >= num_experts) return;  // uniform across the workgroup
 
     const unsigned char* B8 = (const unsigned char*)Bv + (int64_t)expert * sbe;
     const unsigned short* B16 = (const unsigned short*)Bv + (int64_t)expert * sbe;
 
-    f32x16 acc[kMaxMT];
+    f32x16 acc = f32x16{0};
+    // staging registers for the next B tile (128 n x kKT k) and A tile (32 slots x kKT k)
+    constexpr int CPR = kKT / 8;            // 16-byte chunks per tile row
+    constexpr int NB = kNT * CPR / 256;     // B chunks per thread
+    constexpr int NA = kTT * CPR / 256;     // A chunks per thread
+    s16x8 breg[NB], areg[NA];
+    int a_col[NA];
 #pragma unroll
-    for (int i = 0; i < kMaxMT; ++i) acc[i] = f32x16{0};
-
-    // staging registers: B tile 128 n x 64 k = 1024 chunks of 8 elements -> 4 per thread;
-    // A tile up to 128 slots x 64 k -> up to 4 per thread.
-    s16x8 breg[4], areg[kMaxMT];
+    for (int i = 0; i < NA; ++i) {
+        a_col[i] = -1;
+        const int tok = s_tok[(tid + 256 * i) / CPR];
+        if (tok) {
+            const int col = (tok + replicas - 1) / replicas - 1;  // cld(token_id, replicas), 0-based
+            if (col < num_a_cols) a_col[i] = col;
+        }
+    }
     auto load_tiles = [&](int k0) {
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            const int id = tid + 256 * i, n = id >> 3, c = id & 7;
+        for (int i = 0; i < NB; ++i) {
+            const int id = tid + 256 * i, n = id / CPR, c = id % CPR;
             const int gn = n0 + n, gk = k0 + 8 * c;
             s16x8 v = {0};
             if (gn < N && gk < K) {
                 if (W8) {
                     const unsigned char* p = B8 + gk + (int64_t)gn * ldb;
                     u32x2 raw = {0, 0};
-                    if (vecB && gk + 8 <= K) raw = *reinterpret_cast<const u32x2*>(p);
+                    if (vecB && gk + 8 <= K) raw = __builtin_nontemporal_load(reinterpret_cast<const u32x2*>(p));
                     else {
                         unsigned long long acc8 = 0;
                         for (int e = 0; e < 8; ++e)
@@ -140,7 +159,7 @@ __global__ __launch_bounds__(256) void fused_moe_kernel(
                     v = __builtin_bit_cast(s16x8, w);
                 } else {
                     const unsigned short* p = B16 + gk + (int64_t)gn * ldb;
-                    if (vecB && gk + 8 <= K) v = *reinterpret_cast<const s16x8*>(p);
+                    if (vecB && gk + 8 <= K) v = __builtin_nontemporal_load(reinterpret_cast<const s16x8*>(p));
                     else
 #pragma unroll
                         for (int e = 0; e < 8; ++e) v[e] = (gk + e < K) ? (short)p[e] : (short)0;
@@ -149,22 +168,15 @@ __global__ __launch_bounds__(256) void fused_moe_kernel(
             breg[i] = v;
         }
 #pragma unroll
-        for (int i = 0; i < kMaxMT; ++i) {
+        for (int i = 0; i < NA; ++i) {
             s16x8 v = {0};
-            if (i < mt_used) {
-                const int id = tid + 256 * i, slot = id >> 3, c = id & 7;
-                const int tok = slot < TILE_M ? s_tok[slot] : 0;
-                const int gk = k0 + 8 * c;
-                if (tok >= 1 && tok <= total_tokens && gk < K) {
-                    const int col = (tok + replicas - 1) / replicas - 1;  // cld(token_id, replicas), 0-based
-                    if (col < num_a_cols) {
-                        const unsigned short* p = A + gk + (int64_t)col * lda;
-                        if (vecA && gk + 8 <= K) v = *reinterpret_cast<const s16x8*>(p);
-                        else
+            const int gk = k0 + 8 * ((tid + 256 * i) % CPR);
+            if (a_col[i] >= 0 && gk < K) {
+                const unsigned short* p = A + gk + (int64_t)a_col[i] * lda;
+                if (vecA && gk + 8 <= K) v = *reinterpret_cast<const s16x8*>(p);
+                else
 #pragma unroll
-                            for (int e = 0; e < 8; ++e) v[e] = (gk + e < K) ? (short)p[e] : (short)0;
-                    }
-                }
+                    for (int e = 0; e < 8; ++e) v[e] = (gk + e < K) ? (short)p[e] : (short)0;
             }
             areg[i] = v;
         }
@@ -174,53 +186,59 @@ __global__ __launch_bounds__(256) void fused_moe_kernel(
     for (int k0 = 0; k0 < K; k0 += kKT) {
         __syncthreads();
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            const int id = tid + 256 * i, n = id >> 3, c = id & 7;
+        for (int i = 0; i < NB; ++i) {
+            const int id = tid + 256 * i, n = id / CPR, c = id % CPR;
             *reinterpret_cast<s16x8*>(&Bs[n * kKT + 8 * (c ^ (n & 7))]) = breg[i];
         }
 #pragma unroll
-        for (int i = 0; i < kMaxMT; ++i)
-            if (i < mt_used) {
-                const int id = tid + 256 * i, slot = id >> 3, c = id & 7;
-                *reinterpret_cast<s16x8*>(&As[slot * kKT + 8 * (c ^ (slot & 7))]) = areg[i];
-            }
+        for (int i = 0; i < NA; ++i) {
+            const int id = tid + 256 * i, sl = id / CPR, c = id % CPR;
+            *reinterpret_cast<s16x8*>(&As[sl * kKT + 8 * (c ^ (sl & 7))]) = areg[i];
+        }
         __syncthreads();
         if (k0 + kKT < K) load_tiles(k0 + kKT);
 #pragma unroll
-        for (int ks = 0; ks < kKT / 16; ++ks) {
+        for (int kq = 0; kq < kKT / 16 / KW; ++kq) {
+            const int ks = wk * (kKT / 16 / KW) + kq;
             const int c = 2 * ks + hb;
-            const int n = wave * 32 + (lane & 31);
+            const int n = wn * 32 + (lane & 31);
+            const int slot = lane & 31;
             s16x8 bf = *reinterpret_cast<const s16x8*>(&Bs[n * kKT + 8 * (c ^ (n & 7))]);
-#pragma unroll
-            for (int mt = 0; mt < kMaxMT; ++mt)
-                if (mt < mt_used) {
-                    const int slot = 32 * mt + (lane & 31);
-                    s16x8 af = *reinterpret_cast<const s16x8*>(&As[slot * kKT + 8 * (c ^ (slot & 7))]);
-                    acc[mt] = E::mfma32(af, bf, acc[mt]);
-                }
+            s16x8 af = *reinterpret_cast<const s16x8*>(&As[slot * kKT + 8 * (c ^ (slot & 7))]);
+            acc = E::mfma32(af, bf, acc);
         }
     }
+    if (KW > 1) {  // add the K-split partial accumulators: wave (wn, wk) -> wave (wn, 0)
+        __syncthreads();
+        float* red = reinterpret_cast<float*>(Bs);  // 4 waves x 64 lanes x 16 floats = 16 KB <= sizeof(Bs)
+        static_assert(KW == 1 || sizeof(unsigned short) * kNT * kKT >= 4 * 64 * 16 * sizeof(float), "reduction buffer");
+        if (wk > 0) {
+#pragma unroll
+            for (int r = 0; r < 16; ++r) red[(wave * 16 + r) * 64 + lane] = acc[r];
+        }
+        __syncthreads();
+        if (wk > 0) return;
+#pragma unroll
+        for (int q = 1; q < KW; ++q)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[r] += red[((wn + NTW * q) * 16 + r) * 64 + lane];
+    }
 
-    // epilogue: rows = token slots 8*(r/4) + 4*hb + r%4, column = channel n0 + wave*32 + lane%32
-    const int gn = n0 + wave * 32 + (lane & 31);
+    // epilogue: rows = token slots 8*(r/4) + 4*hb + r%4, column = channel n0 + wn*32 + lane%32
+    const int gn = n0 + wn * 32 + (lane & 31);
     if (gn >= N) return;
     float ch_scale = 1.f;
     if (W8) ch_scale = b_scale[gn + (int64_t)expert * ld_scale];
 #pragma unroll
-    for (int mt = 0; mt < kMaxMT; ++mt)
-        if (mt < mt_used) {
-#pragma unroll
-            for (int r = 0; r < 16; ++r) {
-                const int slot = 32 * mt + 8 * (r >> 2) + 4 * hb + (r & 3);
-                if (slot >= TILE_M) continue;
-                const int tok = s_tok[slot];
-                if (tok < 1 || tok > total_tokens) continue;
-                float v = acc[mt][r];
-                if (W8) v *= ch_scale;
-                if (mul_routed_weight) v *= E::widen(topk_weights[tok - 1]);
-                C[gn + (int64_t)(tok - 1) * ldc] = E::cvt(v);
-            }
-        }
+    for (int r = 0; r < 16; ++r) {
+        const int slot = 8 * (r >> 2) + 4 * hb + (r & 3);
+        const int tok = s_tok[slot];
+        if (!tok) continue;
+        float v = acc[r];
+        if (W8) v *= ch_scale;
+        if (mul_routed_weight) v *= E::widen(topk_weights[tok - 1]);
+        C[gn + (int64_t)(tok - 1) * ldc] = E::cvt(v);
+    }
 }
 
 // ---- SiLU(a) * b -------------------------------------------------------------------------------
@@ -285,7 +303,6 @@ extern "C" int mi_fused_moe_kernel(const mi_tile_array* A, const mi_tile_array* 
     if (w8 != (b_scale != nullptr)) return MI_E_ARG;
     if (sorted_token_ids->dtype != MI_I32 || sorted_expert_ids->dtype != MI_I32) return MI_E_DTYPE;
     if (!is_pow2(TILE_M) || !is_pow2(TILE_N) || !is_pow2(TILE_K)) return MI_E_TILE;
-    if (TILE_M > 32 * kMaxMT) return MI_E_UNSUPPORTED;
     if (num_token_replicas < 1) return MI_E_ARG;
     const int64_t K = B->sizes[0], N = B->sizes[1], E = B->sizes[2];
     if (A->sizes[0] != K || C->sizes[0] != N) return MI_E_SHAPE;
@@ -306,29 +323,41 @@ extern "C" int mi_fused_moe_kernel(const mi_tile_array* A, const mi_tile_array* 
     if (K > 0x7fffffff || N > 0x7fffffff || total > 0x7ffffffe || slots > 0x7fffffff) return MI_E_SHAPE;
     if (m_blocks * cld(N, (int64_t)TILE_N) > MI_MAX_GRID_DIM) return MI_E_GRID;
     if (m_blocks == 0 || N == 0) return MI_OK;
-    const int n_blocks = (int)cld(N, (int64_t)kNT);
-    if (m_blocks * n_blocks > 0x7fffffffLL) return MI_E_GRID;
+    const int tile_slots = TILE_M < kTT ? TILE_M : kTT;
+    const int64_t tiles = m_blocks * (TILE_M / tile_slots);
+    // Wide strips (128 channels) when they already give the chip >= ~3 workgroups per CU,
+    // counting one started 32-slot tile per TILE_M block; otherwise 32-channel strips with an
+    // in-workgroup K split.
+    const bool narrow = m_blocks * cld(N, (int64_t)128) < 768 && K >= 512;
+    const int n_blocks = (int)cld(N, (int64_t)(narrow ? 32 : 128));
+    if (tiles * n_blocks > 0x7fffffffLL) return MI_E_GRID;
     const bool vecA = aligned(A->ptr, 16) && A->strides[1] % 8 == 0;
-    const int bdiv = w8 ? 8 : 8;
-    const bool vecB = aligned(B->ptr, w8 ? 8 : 16) && B->strides[1] % bdiv == 0 && B->strides[2] % bdiv == 0;
-    dim3 grid((unsigned)(m_blocks * n_blocks));
+    const bool vecB = aligned(B->ptr, w8 ? 8 : 16) && B->strides[1] % 8 == 0 && B->strides[2] % 8 == 0;
+    dim3 grid((unsigned)(tiles * n_blocks));
     hipStream_t s = (hipStream_t)stream;
-#define LAUNCH(ET, W8)                                                                                              \
-    hipLaunchKernelGGL((fused_moe_kernel<ET, W8>), grid, dim3(256), 0, s, (const unsigned short*)A->ptr,           \
+#define LAUNCH(ET, W8, NTW, KT)                                                                                     \
+    hipLaunchKernelGGL((fused_moe_kernel<ET, W8, NTW, KT>), grid, dim3(256), 0, s, (const unsigned short*)A->ptr,   \
                        A->strides[1], (int)A->sizes[1], (const void*)B->ptr, B->strides[1], B->strides[2],          \
                        (unsigned short*)C->ptr, C->strides[1], (int)total, (const unsigned short*)topk_weights->ptr, \
                        (const int*)sorted_token_ids->ptr, (int)slots, (const int*)sorted_expert_ids->ptr,           \
                        w8 ? (const float*)b_scale->ptr : nullptr, w8 ? b_scale->strides[1] : 0, (int)K, (int)N,     \
-                       (int)E, num_token_replicas, mul_routed_weight != 0, TILE_M, n_blocks, vecA, vecB)
+                       (int)E, num_token_replicas, mul_routed_weight != 0, TILE_M, tile_slots, n_blocks, vecA, vecB)
+#define LAUNCH_SHAPE(ET, W8)                   \
+    do {                                       \
+        if (narrow) LAUNCH(ET, W8, 1, 256);    \
+        else LAUNCH(ET, W8, 4, 128);           \
+    } while (0)
     if (A->dtype == MI_F16) {
-        if (w8) LAUNCH(F16, true);
-        else LAUNCH(F16, false);
+        if (w8) LAUNCH_SHAPE(F16, true);
+        else LAUNCH_SHAPE(F16, false);
     } else {
-        if (w8) LAUNCH(BF16, true);
-        else LAUNCH(BF16, false);
+        if (w8) LAUNCH_SHAPE(BF16, true);
+        else LAUNCH_SHAPE(BF16, false);
     }
+#undef LAUNCH_SHAPE
 #undef LAUNCH
-    set_variant(w8 ? "fused_moe_n128_k64_w8a16" : "fused_moe_n128_k64");
+    if (narrow) set_variant(w8 ? "fused_moe_t32_n32_k256_ksplit4_w8a16" : "fused_moe_t32_n32_k256_ksplit4");
+    else set_variant(w8 ? "fused_moe_t32_n128_k128_w8a16" : "fused_moe_t32_n128_k128");
     return launch_status();
 }
 

@@ -8,6 +8,7 @@
 // dimension.  Workgroups are numbered so that consecutive ids walk down x's contiguous
 // dimension.  Algorithmic traffic: 2 * m * n * sizeof(T) bytes.
 #include "common.h"
+#include <stdlib.h>
 
 namespace {
 
@@ -77,6 +78,99 @@ __global__ __launch_bounds__(kBlock) void transpose_kernel(const T* __restrict__
     }
 }
 
+// ---- 4-byte elements, every dimension a multiple of 4: 4x4 register micro-transpose ----------
+// A lane loads a 4(m) x 4(n) block as four 16-byte vectors along m, transposes it in registers,
+// and passes four 16-byte vectors along n through an LDS tile L[m][n] whose 16-byte slots are
+// XOR-swizzled with (m >> 2) so that both the writes (lanes differ in m) and the reads (lanes
+// differ in n) of a quarter-wave cover all 64 banks.  All LDS traffic is 128-bit.
+// ORDER selects how workgroup ids walk the tile grid (the workgroups that run at the same
+// time decide how large the contiguous spans are that DRAM sees on each side).
+typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
+
+template <int TM, int TN>
+__global__ __launch_bounds__(256) void transpose4_kernel(const unsigned* __restrict__ x, int64_t ldx,
+                                                         unsigned* __restrict__ y, int64_t ldy, int64_t m,
+                                                         int64_t n, int tiles_m, int tiles_n, int order) {
+    __shared__ __attribute__((aligned(16))) unsigned lds[TM * TN];
+    constexpr int MB = TM * TN / (16 * 256);  // 4x4 micro-blocks per lane
+    constexpr int SLOTS = TN / 4;             // 16-byte slots per LDS row
+    int bm, bn;
+    {
+        const int id = blockIdx.x;
+        if (order == 0) { bm = id % tiles_m; bn = id / tiles_m; }
+        else if (order == 1) { bn = id % tiles_n; bm = id / tiles_n; }
+        else {  // 8 x 8 super-tiles, m fastest inside
+            const int sm = (tiles_m + 7) / 8;
+            const int st = id / 64, in = id % 64;
+            bm = (st % sm) * 8 + (in % 8);
+            bn = (st / sm) * 8 + (in / 8);
+            if (bm >= tiles_m || bn >= tiles_n) return;
+        }
+    }
+    const int64_t m0 = (int64_t)bm * TM, n0 = (int64_t)bn * TN;
+#pragma unroll
+    for (int k = 0; k < MB; ++k) {
+        const int b = threadIdx.x + 256 * k;
+        const int i4 = b % (TM / 4), j4 = b / (TM / 4);
+        const int64_t gm = m0 + 4 * i4, gn = n0 + 4 * j4;
+        u32x4 r[4] = {};
+        if (gm < m) {
+#pragma unroll
+            for (int c = 0; c < 4; ++c)
+                if (gn + c < n) r[c] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(x + gm + (gn + c) * ldx));
+        }
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+            u32x4 t = {r[0][q], r[1][q], r[2][q], r[3][q]};  // x[m+q, n..n+3]
+            const int row = 4 * i4 + q;
+            *reinterpret_cast<u32x4*>(&lds[row * TN + 4 * (j4 ^ (i4 & (SLOTS - 1)))]) = t;
+        }
+    }
+    __syncthreads();
+#pragma unroll
+    for (int k = 0; k < 4 * MB; ++k) {
+        const int b = threadIdx.x + 256 * k;
+        const int j4 = b % SLOTS, row = b / SLOTS;
+        const int64_t gn = n0 + 4 * j4, gm = m0 + row;
+        if (gn < n && gm < m) {
+            u32x4 t = *reinterpret_cast<const u32x4*>(&lds[row * TN + 4 * (j4 ^ ((row >> 2) & (SLOTS - 1)))]);
+            __builtin_nontemporal_store(t, reinterpret_cast<u32x4*>(y + gn + gm * ldy));
+        }
+    }
+}
+
+int launch4(const mi_tile_array* x, const mi_tile_array* y, hipStream_t s) {
+    const int64_t m = x->sizes[0], n = x->sizes[1];
+    int tile = 2, order = 2;  // measured best on MI355X for 8192^2 fp32: 64(m) x 128(n) tiles, 8x8 super-tiles
+    if (const char* e = getenv("MI_TRANSPOSE_TILE")) tile = atoi(e);    // tuning overrides
+    if (const char* e = getenv("MI_TRANSPOSE_ORDER")) order = atoi(e);
+    int TM = 64, TN = 128;
+    if (tile == 128) { TM = 128; TN = 128; }
+    else if (tile == 2) { TM = 64; TN = 128; }
+    else if (tile == 3) { TM = 128; TN = 64; }
+    else if (tile == 4) { TM = 32; TN = 256; }
+    else if (tile == 5) { TM = 64; TN = 256; }
+    else if (tile == 6) { TM = 32; TN = 128; }
+    else if (tile == 64) { TM = 64; TN = 64; }
+    const int64_t tm_ = cld(m, (int64_t)TM), tn_ = cld(n, (int64_t)TN);
+    int64_t blocks = tm_ * tn_;
+    if (order == 2) blocks = ((tm_ + 7) / 8) * ((tn_ + 7) / 8) * 64;
+    if (blocks > 0x7fffffffLL || tm_ > 0x3fffffff || tn_ > 0x3fffffff) return MI_E_GRID;
+#define T4(A, B)                                                                                          \
+    hipLaunchKernelGGL((transpose4_kernel<A, B>), dim3((unsigned)blocks), dim3(256), 0, s,                \
+                       (const unsigned*)x->ptr, x->strides[1], (unsigned*)y->ptr, y->strides[1], m, n,    \
+                       (int)tm_, (int)tn_, order)
+    if (TM == 64 && TN == 64) { T4(64, 64); set_variant("transpose4_64x64_regmicro"); }
+    else if (TM == 128 && TN == 128) { T4(128, 128); set_variant("transpose4_128x128_regmicro"); }
+    else if (TM == 32 && TN == 256) { T4(32, 256); set_variant("transpose4_32x256_regmicro"); }
+    else if (TM == 64 && TN == 256) { T4(64, 256); set_variant("transpose4_64x256_regmicro"); }
+    else if (TM == 32 && TN == 128) { T4(32, 128); set_variant("transpose4_32x128_regmicro"); }
+    else if (TM == 64) { T4(64, 128); set_variant("transpose4_64x128_regmicro"); }
+    else { T4(128, 64); set_variant("transpose4_128x64_regmicro"); }
+#undef T4
+    return launch_status();
+}
+
 template <typename T>
 int launch(const mi_tile_array* x, const mi_tile_array* y, hipStream_t s) {
     constexpr int V = 16 / sizeof(T);
@@ -118,7 +212,11 @@ extern "C" int mi_transpose_kernel(const mi_tile_array* x, const mi_tile_array* 
     switch (dtype_size(x->dtype)) {
         case 1: return launch<uint8_t>(x, y, s);
         case 2: return launch<uint16_t>(x, y, s);
-        case 4: return launch<uint32_t>(x, y, s);
+        case 4:
+            if (m % 4 == 0 && n % 4 == 0 && x->strides[1] % 4 == 0 && y->strides[1] % 4 == 0 && aligned(x->ptr, 16) &&
+                aligned(y->ptr, 16))
+                return launch4(x, y, s);
+            return launch<uint32_t>(x, y, s);
         case 8: return launch<uint64_t>(x, y, s);
         default: return MI_E_DTYPE;
     }

@@ -2,22 +2,29 @@
 """Benchmark of the hot path on one MI355X: the kernels of cuTile.jl's examples, through the
 C ABI of libmi355tile.so.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME] [--no-cpu] [--table]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--kernels LIST|all|none] [--no-cpu] [--table]
 
-Prints ONE JSON line on stdout.  A "step" is one pass of the headline workload over one
-batch of synthetic, seeded input already resident in HBM:
+Prints ONE JSON line on stdout.  A "step" is one pass of the headline workload over one batch
+of synthetic, seeded input already resident in HBM:
 
-    headline workload (default) = "layernorm_softmax": LayerNorm fwd + bwd and the column
-    softmax on 4096x4096 fp32 (the second entry of BASELINE.json's configs);
-    ``value`` = algorithmic bytes of the step / time per step, in GB/s.
+    headline workload = the second entry of BASELINE.json's configs: row LayerNorm fwd + bwd
+    (y, dx, dgamma, dbeta) and the row softmax on 4096x4096 fp32.
+    ``value`` = algorithmic bytes of the step / wall time per step, in GB/s, timed over
+    exactly ``--steps`` steps between two device synchronisations.
 
-Every other configuration of BASELINE.json (vadd, transpose, GEMM, batched GEMM, FMHA, MoE)
-is measured in the same run with the reference's protocol (examples/benchmarks.jl:12-13:
-5 warm-up launches, 20 timed launches, min and mean) and reported under ``"kernels"``, each
-with absolute GB/s or TFLOP/s and its fraction of the MI355X roofline (HBM 8 TB/s; dense
-MFMA f16 2.5 PFLOP/s, fp8 5.0 PFLOP/s, fp32 157.3 TFLOP/s).  ``roofline`` on the top level
-is the dominant kernel of the headline workload.  ``cpu_baseline`` times the numpy/OpenBLAS
-restatement of the reference's CPU path for the headline workload on a bounded sample.
+Every other configuration of BASELINE.json (vadd, transpose, GEMM, batched GEMM, FMHA, MoE f16
+and fp8) is measured in the same run and reported under ``"kernels"``:
+  * ``min_ms`` / ``mean_ms``: the reference's protocol (examples/benchmarks.jl:12-13: 5 warm-up
+    launches, 20 launches each bracketed by its own pair of events on the launch stream);
+  * ``avg_ms``: 20 launches back to back between ONE pair of events (no per-launch event
+    and host overhead; this is what agrees with a profiler's average kernel duration);
+  * ``achieved`` (from ``avg_ms``) in GB/s or TFLOP/s and ``frac`` of the MI355X roofline
+    (HBM 8 TB/s; dense MFMA f16 2.5 PFLOP/s, fp8 5.0 PFLOP/s, fp32 157.3 TFLOP/s);
+  * ``cpu_ms``: the numpy/OpenBLAS restatement of the reference's CPU path for the same
+    configuration (or a stated sample of it), timed on this host.
+The top-level ``roofline`` is the dominant kernel of the headline workload, with its average
+launch duration measured by events inside the timed region; ``cpu_baseline`` is the CPU
+restatement of the headline workload on a bounded sample.
 """
 from __future__ import annotations
 
@@ -31,11 +38,11 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0
-MFMA_PEAK_TFLOPS = {"f16": 2500.0, "bf16": 2500.0, "fp8": 5000.0, "f32": 157.3}
 NRUNS, WARMUP = 20, 5  # examples/benchmarks.jl:12-13
 
 
 def _event_times(fn, nruns, warmup):
+    """Reference protocol: each launch bracketed by its own events; returns ms per launch."""
     import torch
     for _ in range(warmup):
         fn()
@@ -48,103 +55,256 @@ def _event_times(fn, nruns, warmup):
     return out
 
 
-def _entry(name, times_ms, work, unit, bound, peak, dtype, extra=None):
-    tmin = min(times_ms); tmean = sum(times_ms) / len(times_ms)
+def _back_to_back(fn, nruns):
+    """nruns launches between one pair of events; returns average ms per launch."""
+    import torch
+    torch.cuda.synchronize()
+    e0 = torch.cuda.Event(enable_timing=True); e1 = torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(nruns):
+        fn()
+    e1.record(); e1.synchronize()
+    return e0.elapsed_time(e1) / nruns
+
+
+def _entry(name, fn, work, unit, bound, peak, dtype, nruns, warmup, extra=None):
+    t = _event_times(fn, nruns, warmup)
+    avg = _back_to_back(fn, nruns)
     scale = 1e9 if unit == "GB/s" else 1e12
-    ach_min = work / (tmin * 1e-3) / scale
-    ach_mean = work / (tmean * 1e-3) / scale
-    e = {"name": name, "min_ms": round(tmin, 5), "mean_ms": round(tmean, 5), "work": work,
-         "achieved": round(ach_mean, 2), "achieved_at_min": round(ach_min, 2), "unit": unit if unit == "GB/s" else "TFLOP/s",
-         "bound": bound, "peak": peak, "frac": round(ach_mean / peak, 4), "frac_at_min": round(ach_min / peak, 4),
-         "dtype": dtype}
+    ach = work / (avg * 1e-3) / scale
+    e = {"name": name, "min_ms": round(min(t), 5), "mean_ms": round(sum(t) / len(t), 5), "avg_ms": round(avg, 5),
+         "work": work, "achieved": round(ach, 2), "unit": "GB/s" if unit == "GB/s" else "TFLOP/s", "bound": bound,
+         "peak": peak, "frac": round(ach / peak, 4), "dtype": dtype}
     if extra:
         e.update(extra)
     return e
 
 
-def bench_kernels(ct, which, nruns=NRUNS, warmup=WARMUP):
-    """Measure each configuration; returns {name: entry}."""
+def _cpu_time(fn, repeats=3):
+    fn()  # warm-up
+    best = float("inf")
+    for _ in range(repeats):
+        t0 = time.perf_counter(); fn(); best = min(best, time.perf_counter() - t0)
+    return best * 1e3
+
+
+def bench_kernels(ct, which, cpu, nruns=NRUNS, warmup=WARMUP):
+    """Measure each configuration; returns {key: entry}."""
+    import numpy as np
     import torch
-    from cutile_jl_amd import examples  # noqa: F401
-    import importlib
+    from oracle import cutile_oracle as orc
+    from cutile_jl_amd.examples import vadd, transpose, layernorm, softmax, matmul, batchmatmul, fmha, moe
     res = {}
+    ncores = os.cpu_count()
 
     def want(n):
         return which is None or n in which
 
     if want("vadd"):
-        m = importlib.import_module("cutile_jl_amd.examples.vadd")
-        d = m.prepare(benchmark=True)
-        t = _event_times(lambda: ct.vec_add_kernel_1d(d.a, d.b, d.c, 1024), nruns, warmup)
-        res["vadd"] = _entry("vadd 2^27 f32", t, m.metric(d)[0], "GB/s", "hbm", HBM_PEAK_GBS, "f32",
-                             {"variant": ct.last_variant()})
+        d = vadd.prepare(benchmark=True)
+        A, B, C = ct.TileArray(d.a), ct.TileArray(d.b), ct.TileArray(d.c)
+        e = _entry("vadd 2^27 f32", lambda: ct.vec_add_kernel_1d(A, B, C, 1024), vadd.metric(d)[0], "GB/s", "hbm",
+                   HBM_PEAK_GBS, "f32", nruns, warmup, {"variant": None})
+        e["variant"] = ct.last_variant()
+        if cpu:
+            a, b = d.a.cpu().numpy(), d.b.cpu().numpy()
+            e["cpu_ms"] = round(_cpu_time(lambda: a + b), 2); e["cpu_note"] = "numpy a+b, 1 thread"
+        res["vadd"] = e
         del d
     if want("transpose"):
-        m = importlib.import_module("cutile_jl_amd.examples.transpose")
-        d = m.prepare(benchmark=True)
-        t = _event_times(lambda: ct.transpose_kernel(d.x, d.y, 64, 64), nruns, warmup)
-        res["transpose"] = _entry("transpose 8192^2 f32", t, m.metric(d)[0], "GB/s", "hbm", HBM_PEAK_GBS, "f32",
-                                  {"variant": ct.last_variant()})
+        d = transpose.prepare(benchmark=True)
+        X, Y = ct.TileArray(d.x), ct.TileArray(d.y)
+        e = _entry("transpose 8192^2 f32", lambda: ct.transpose_kernel(X, Y, 64, 64), transpose.metric(d)[0], "GB/s",
+                   "hbm", HBM_PEAK_GBS, "f32", nruns, warmup)
+        e["variant"] = ct.last_variant()
+        if cpu:
+            x = d.x.cpu().numpy()
+            e["cpu_ms"] = round(_cpu_time(lambda: np.ascontiguousarray(x.T)), 2); e["cpu_note"] = "numpy transpose copy, 1 thread"
+        res["transpose"] = e
         del d
     if want("layernorm"):
-        m = importlib.import_module("cutile_jl_amd.examples.layernorm")
-        d = m.prepare(benchmark=True)
-        r = m.run(d, nruns=nruns, warmup=warmup)
-        MN4 = d.M * d.N * 4
-        fwd_bytes = 2 * MN4 + (2 * d.N + 2 * d.M) * 4
-        bwd_bytes = 3 * MN4 + (d.N + 2 * d.M) * 4 + 4 * d.N * d.GROUP_SIZE_M * 4 + 2 * d.N * 4
-        res["layernorm_fwd"] = _entry("LayerNorm fwd 4096^2 f32", r.times_fwd, fwd_bytes, "GB/s", "hbm", HBM_PEAK_GBS,
-                                      "f32", {"reference_formula_bytes": 4 * MN4})
-        res["layernorm_bwd"] = _entry("LayerNorm bwd 4096^2 f32 (3 fills + 2 kernels)", r.times_bwd, bwd_bytes, "GB/s",
-                                      "hbm", HBM_PEAK_GBS, "f32", {"reference_formula_bytes": 5 * MN4})
-        del d, r
+        for G in (64, 256):
+            d = layernorm.prepare(benchmark=True, GROUP_SIZE_M=G)
+            D = {k: ct.TileArray(getattr(d, k)) for k in ("X", "W", "B", "Y", "Mean", "Rstd", "DY", "DX", "DW_partial",
+                                                          "DB_partial", "Locks", "FINAL_DW", "FINAL_DB")}
+            MN4 = d.M * d.N * 4
+
+            def fwd():
+                ct.layer_norm_fwd(D["X"], D["W"], D["B"], D["Y"], D["Mean"], D["Rstd"], d.eps, 1024)
+
+            def bwd():
+                d.DW_partial.zero_(); d.DB_partial.zero_(); d.Locks.zero_()
+                ct.layer_norm_bwd_dx_partial_dwdb(D["DX"], D["DY"], D["DW_partial"], D["DB_partial"], D["X"], D["W"],
+                                                  D["Mean"], D["Rstd"], D["Locks"], G, 1024)
+                ct.layer_norm_bwd_dwdb(D["DW_partial"], D["DB_partial"], D["FINAL_DW"], D["FINAL_DB"], 32, 1024)
+
+            fwd_bytes = 2 * MN4 + (2 * d.N + 2 * d.M) * 4
+            bwd_bytes = 3 * MN4 + (d.N + 2 * d.M) * 4 + 4 * d.N * G * 4 + 2 * d.N * 4
+            if G == 64:
+                res["layernorm_fwd"] = _entry("LayerNorm fwd 4096^2 f32", fwd, fwd_bytes, "GB/s", "hbm", HBM_PEAK_GBS,
+                                              "f32", nruns, warmup, {"reference_formula_bytes": 4 * MN4})
+                fwd(); res["layernorm_fwd"]["variant"] = ct.last_variant()
+            key = "layernorm_bwd" if G == 64 else "layernorm_bwd_G256"
+            res[key] = _entry(f"LayerNorm bwd 4096^2 f32, GROUP_SIZE_M={G} (3 fills + 2 kernels)", bwd, bwd_bytes,
+                              "GB/s", "hbm", HBM_PEAK_GBS, "f32", nruns, warmup, {"reference_formula_bytes": 5 * MN4})
+            if cpu and G == 64:
+                X, W, B, DY = (orc.to_julia(t) for t in (d.X, d.W, d.B, d.DY))
+                sub = slice(0, 512)
+                res["layernorm_fwd"]["cpu_ms"] = round(_cpu_time(lambda: orc.layer_norm_fwd(X[:, sub], W, B, d.eps, dtype=np.float32)) * 8, 1)
+                res["layernorm_fwd"]["cpu_note"] = "numpy 1 thread, 512 of 4096 rows x8"
+                res[key]["cpu_ms"] = round(_cpu_time(lambda: orc.layer_norm_bwd(X[:, sub], W, DY[:, sub], d.eps, dtype=np.float32)) * 8, 1)
+                res[key]["cpu_note"] = "numpy 1 thread, 512 of 4096 rows x8"
+            del d, D
     if want("softmax"):
-        m = importlib.import_module("cutile_jl_amd.examples.softmax")
-        d = m.prepare(benchmark=True)
-        r = m.run(d, nruns=nruns, warmup=warmup)
+        d = softmax.prepare(benchmark=True)
+        I, O1, O2 = ct.TileArray(d.input), ct.TileArray(d.output_tma), ct.TileArray(d.output_chunked)
         MN4 = d.M * d.N * 4
-        res["softmax_tma"] = _entry("softmax (single tile) 4096^2 f32", r.times["cuTile TMA"], 2 * MN4, "GB/s", "hbm",
-                                    HBM_PEAK_GBS, "f32")
-        res["softmax_chunked"] = _entry("softmax (chunked) 4096^2 f32", r.times["cuTile Chunked"], 2 * MN4, "GB/s",
-                                        "hbm", HBM_PEAK_GBS, "f32", {"reference_formula_bytes": 4 * MN4})
-        del d, r
-    for name in ("matmul", "batchmatmul", "fmha", "moe"):
-        if not want(name):
-            continue
+        res["softmax_tma"] = _entry("softmax (single tile) 4096^2 f32", lambda: ct.softmax_tma_kernel(O1, I, 4096, d.M),
+                                    2 * MN4, "GB/s", "hbm", HBM_PEAK_GBS, "f32", nruns, warmup)
+        res["softmax_tma"]["variant"] = ct.last_variant()
+        res["softmax_chunked"] = _entry("softmax (chunked) 4096^2 f32",
+                                        lambda: ct.softmax_chunked_kernel(O2, I, d.N, 1024, d.M), 2 * MN4, "GB/s", "hbm",
+                                        HBM_PEAK_GBS, "f32", nruns, warmup, {"reference_formula_bytes": 4 * MN4})
+        if cpu:
+            x = orc.to_julia(d.input)
+            res["softmax_tma"]["cpu_ms"] = round(_cpu_time(lambda: orc.softmax(x[:, :512], dtype=np.float32)) * 8, 1)
+            res["softmax_tma"]["cpu_note"] = "numpy 1 thread, 512 of 4096 columns x8"
+        del d
+    if want("matmul"):
+        d = matmul.prepare(benchmark=True, T=torch.float16, out_T=torch.float32, dist="normal64")
+        A, B, C = ct.TileArray(d.A), ct.TileArray(d.B), ct.TileArray(d.C)
+        e = _entry("GEMM 4096^3 f16 -> f32", lambda: ct.matmul_kernel(A, B, C, 64, 64, 64), matmul.metric(d)[0],
+                   "TFLOPS", "mfma", 2500.0, "f16", nruns, warmup)
+        e["variant"] = ct.last_variant()
+        if cpu:
+            a = orc.to_julia(d.A).astype(np.float32); b = orc.to_julia(d.B).astype(np.float32)
+            e["cpu_ms"] = round(_cpu_time(lambda: a @ b, repeats=2), 1); e["cpu_note"] = f"numpy/OpenBLAS sgemm on widened inputs, {ncores} threads"
+        res["matmul"] = e
+        del d
+    if want("batchmatmul"):
+        d = batchmatmul.prepare(benchmark=True)
+        A, B, C = ct.TileArray(d.A), ct.TileArray(d.B), ct.TileArray(d.C)
+        e = _entry("batched GEMM 8x(1024x512x2048) f32", lambda: ct.batch_matmul_kernel(A, B, C, 128, 128, 64),
+                   batchmatmul.metric(d)[0], "TFLOPS", "mfma", 157.3, "f32", nruns, warmup)
+        e["variant"] = ct.last_variant()
+        if cpu:
+            a = orc.to_julia(d.A); b = orc.to_julia(d.B)
+            e["cpu_ms"] = round(_cpu_time(lambda: orc.batch_matmul(a, b, dtype=np.float32), repeats=2), 1)
+            e["cpu_note"] = f"numpy/OpenBLAS sgemm per batch, {ncores} threads"
+        res["batchmatmul"] = e
+        del d
+    if want("fmha"):
+        d = fmha.prepare(benchmark=True)
+        out = torch.empty_like(d.Q)
+        Q, K, V, O = (ct.TileArray(t) for t in (d.Q, d.K, d.V, out))
+        scale = float(np.float32(1.0 / np.sqrt(d.d_k)))
+        e = _entry("causal FMHA 8x16x1024x64 f16",
+                   lambda: ct.fmha_kernel(Q, K, V, O, scale, 0, d.d_k, d.heads, 128, 128, 1, True, True),
+                   fmha.causal_flops(d), "TFLOPS", "mfma", 2500.0, "f16", nruns, warmup)
+        e["variant"] = ct.last_variant()
+        e["dense_count_flop"] = fmha.metric(d)[0]
+        e["tflops_dense_count"] = round(fmha.metric(d)[0] / (e["avg_ms"] * 1e-3) / 1e12, 2)
+        if cpu:
+            q, k, v = (orc.to_julia(t)[:, :, :, :1] for t in (d.Q, d.K, d.V))
+            e["cpu_ms"] = round(_cpu_time(lambda: orc.ref_fmha(q[:, :, :4], k[:, :, :4], v[:, :, :4], causal=True), repeats=2) * 32, 1)
+            e["cpu_note"] = f"numpy restatement of ref_fmha, 4 of 128 (batch, head) pairs x32, BLAS {ncores} threads"
+        res["fmha"] = e
+        del d
+    if want("moe"):
+        d = moe.prepare(benchmark=True, topk=2, router="top2_logits")
+        flop = moe.metric(d)[0]
+        wbytes = (d.w1.numel() + d.w2.numel()) * 2 + 2 * d.hidden_states.numel() * 2
+        tok, exp = ct.moe_align_tile_size(d.topk_ids.cpu(), 128, d.num_experts)
+        al = (tok.cuda(), exp.cuda())
+
+        def graph_of(fn):
+            """Replayable HIP graph of the device work (zero-fills are fill kernels, no memset nodes)."""
+            s = torch.cuda.Stream()
+            s.wait_stream(torch.cuda.current_stream())
+            with torch.cuda.stream(s):
+                fn()
+            torch.cuda.current_stream().wait_stream(s)
+            g = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(g):
+                outv = fn()
+            return g, outv
+
+        def extra(e):
+            e["flop"] = flop
+            e["tflops"] = round(flop / (e["avg_ms"] * 1e-3) / 1e12, 2)
+            e["mfma_frac"] = round(e["tflops"] / 2500.0, 5)
+            return e
+
+        whole = lambda: moe.cutile_moe(d.hidden_states, d.w1, d.w2, d.topk_weights, d.topk_ids, 128, 128, 64)
+        res["moe_f16"] = extra(_entry("MoE f16 256tok/1024h/32e/2048i top-2, whole cutile_moe (host align + H2D/D2H inside)",
+                                      whole, wbytes, "GB/s", "hbm", HBM_PEAK_GBS, "f16", nruns, warmup))
+        dev = lambda: moe.cutile_moe(d.hidden_states, d.w1, d.w2, d.topk_weights, d.topk_ids, 128, 128, 64, aligned=al)
+        ref_out = dev()
         try:
-            m = importlib.import_module(f"cutile_jl_amd.examples.{name}")
-        except ModuleNotFoundError:
-            continue
-        res.update(m.bench(ct, _entry, _event_times, nruns, warmup))
+            g, gout = graph_of(dev)
+            g.replay(); torch.cuda.synchronize()
+            assert torch.equal(gout, ref_out), "graph replay differs from eager"
+            res["moe_f16_device"] = extra(_entry("MoE f16 top-2, device work only (3 zero-fills + 4 kernels, HIP graph replay)",
+                                                 g.replay, wbytes, "GB/s", "hbm", HBM_PEAK_GBS, "f16", nruns, warmup))
+        except Exception as ex:  # graph capture unavailable: fall back to eager launches
+            res["moe_f16_device"] = extra(_entry(f"MoE f16 top-2, device work only (eager; graph failed: {type(ex).__name__})",
+                                                 dev, wbytes, "GB/s", "hbm", HBM_PEAK_GBS, "f16", nruns, warmup))
+        if cpu:
+            J = orc.to_julia
+            args = (J(d.hidden_states), J(d.w1), J(d.w2), J(d.topk_weights), J(d.topk_ids))
+            res["moe_f16"]["cpu_ms"] = round(_cpu_time(lambda: orc.ref_moe(*args), repeats=1), 1)
+            res["moe_f16"]["cpu_note"] = f"numpy restatement of ref_moe, BLAS {ncores} threads"
+        # fp8 weights (per-channel fp32 scales)
+        J = orc.to_julia
+        c1, s1 = orc.quantize_e4m3fn_per_channel(J(d.w1).astype(np.float32))
+        c2, s2 = orc.quantize_e4m3fn_per_channel(J(d.w2).astype(np.float32))
+        w1q = orc.from_julia(c1).cuda().view(torch.float8_e4m3fn); w2q = orc.from_julia(c2).cuda().view(torch.float8_e4m3fn)
+        s1t, s2t = orc.from_julia(s1).cuda(), orc.from_julia(s2).cuda()
+        w8bytes = c1.size + c2.size + (s1.size + s2.size) * 4 + 2 * d.hidden_states.numel() * 2
+        dev8 = lambda: moe.cutile_moe(d.hidden_states, w1q, w2q, d.topk_weights, d.topk_ids, 128, 128, 64, w1_scale=s1t,
+                                      w2_scale=s2t, aligned=al)
+        dev8()
+        try:
+            g8, _ = graph_of(dev8)
+            res["moe_fp8_device"] = extra(_entry("MoE e4m3 weights top-2, device work only (HIP graph replay)", g8.replay,
+                                                 w8bytes, "GB/s", "hbm", HBM_PEAK_GBS, "fp8 weights / f16 MFMA", nruns, warmup))
+        except Exception as ex:
+            res["moe_fp8_device"] = extra(_entry(f"MoE e4m3 weights top-2, device work only (eager; {type(ex).__name__})", dev8,
+                                                 w8bytes, "GB/s", "hbm", HBM_PEAK_GBS, "fp8 weights / f16 MFMA", nruns, warmup))
+        del d
     torch.cuda.synchronize()
     return res
 
 
 def headline(ct, steps, warmup):
-    """configs[1]: LayerNorm fwd+bwd and softmax on 4096x4096 fp32; returns timing + per-kernel
-    durations measured with events on the launch stream inside the timed region."""
+    """configs[1]: LayerNorm fwd+bwd and softmax on 4096x4096 fp32.  Returns seconds per step,
+    per-stage average durations from events inside the timed region, and algorithmic bytes."""
     import torch
     from cutile_jl_amd.examples import layernorm, softmax
     dl = layernorm.prepare(benchmark=True)
     ds = softmax.prepare(benchmark=True)
+    D = {k: ct.TileArray(getattr(dl, k)) for k in ("X", "W", "B", "Y", "Mean", "Rstd", "DY", "DX", "DW_partial",
+                                                   "DB_partial", "Locks", "FINAL_DW", "FINAL_DB")}
+    SI, SO = ct.TileArray(ds.input), ct.TileArray(ds.output_tma)
+    G = dl.GROUP_SIZE_M
 
     def ln_fwd():
-        ct.layer_norm_fwd(dl.X, dl.W, dl.B, dl.Y, dl.Mean, dl.Rstd, dl.eps, 1024)
+        ct.layer_norm_fwd(D["X"], D["W"], D["B"], D["Y"], D["Mean"], D["Rstd"], dl.eps, 1024)
 
-    def ln_bwd_fill():
+    def fills():
         dl.DW_partial.zero_(); dl.DB_partial.zero_(); dl.Locks.zero_()
 
     def ln_bwd_main():
-        ct.layer_norm_bwd_dx_partial_dwdb(dl.DX, dl.DY, dl.DW_partial, dl.DB_partial, dl.X, dl.W, dl.Mean, dl.Rstd,
-                                          dl.Locks, dl.GROUP_SIZE_M, 1024)
+        ct.layer_norm_bwd_dx_partial_dwdb(D["DX"], D["DY"], D["DW_partial"], D["DB_partial"], D["X"], D["W"], D["Mean"],
+                                          D["Rstd"], D["Locks"], G, 1024)
 
     def ln_bwd_final():
-        ct.layer_norm_bwd_dwdb(dl.DW_partial, dl.DB_partial, dl.FINAL_DW, dl.FINAL_DB, 32, 1024)
+        ct.layer_norm_bwd_dwdb(D["DW_partial"], D["DB_partial"], D["FINAL_DW"], D["FINAL_DB"], 32, 1024)
 
     def sm():
-        ct.softmax_tma_kernel(ds.output_tma, ds.input, 4096, num_programs=ds.M)
+        ct.softmax_tma_kernel(SO, SI, 4096, ds.M)
 
-    stages = [("layer_norm_fwd", ln_fwd), ("fills", ln_bwd_fill), ("layer_norm_bwd_dx_partial_dwdb", ln_bwd_main),
+    stages = [("layer_norm_fwd", ln_fwd), ("fills", fills), ("layer_norm_bwd_dx_partial_dwdb", ln_bwd_main),
               ("layer_norm_bwd_dwdb", ln_bwd_final), ("softmax_tma_kernel", sm)]
     for _ in range(warmup):
         for _, f in stages:
@@ -165,8 +325,8 @@ def headline(ct, steps, warmup):
     MN4 = dl.M * dl.N * 4
     work = {
         "layer_norm_fwd": 2 * MN4 + (2 * dl.N + 2 * dl.M) * 4,
-        "layer_norm_bwd_dx_partial_dwdb": 3 * MN4 + (dl.N + 2 * dl.M) * 4 + 2 * dl.N * dl.GROUP_SIZE_M * 4,
-        "layer_norm_bwd_dwdb": 2 * dl.N * dl.GROUP_SIZE_M * 4 + 2 * dl.N * 4,
+        "layer_norm_bwd_dx_partial_dwdb": 3 * MN4 + (dl.N + 2 * dl.M) * 4 + 2 * dl.N * G * 4,
+        "layer_norm_bwd_dwdb": 2 * dl.N * G * 4 + 2 * dl.N * 4,
         "softmax_tma_kernel": 2 * MN4,
         "fills": 0,
     }
@@ -176,7 +336,7 @@ def headline(ct, steps, warmup):
 def cpu_baseline_headline(sample_rows=512):
     """numpy restatement of the reference's CPU path (Julia Base broadcast + reductions,
     examples/layernorm.jl:284-313 and softmax.jl:175-188) on `sample_rows` of the 4096 rows,
-    single-threaded as Julia's broadcasting is.  Returns GB/s on the same byte count."""
+    single-threaded as Julia's broadcasting is.  GB/s on the same per-row byte count."""
     import numpy as np
     from oracle import cutile_oracle as orc
     rng = np.random.default_rng(1)
@@ -195,7 +355,8 @@ def cpu_baseline_headline(sample_rows=512):
     MN4 = M * N * 4
     work = (2 * MN4) + (3 * MN4) + (2 * MN4)
     return {"value": round(work / best / 1e9, 3), "unit": "GB/s", "cores": 1, "kind": "port",
-            "sample": f"{sample_rows} of 4096 rows (N=4096 f32) of LayerNorm fwd+bwd and softmax, numpy single-threaded, min of 3"}
+            "sample": f"{sample_rows} of 4096 rows (N=4096 f32) of LayerNorm fwd+bwd and softmax, numpy restatement of the "
+                      "examples' verify() formulas, single-threaded, min of 3"}
 
 
 def main():
@@ -223,7 +384,7 @@ def main():
     dom = max((k for k in work if work[k] > 0), key=lambda k: per_stage[k])
     ach = work[dom] / (per_stage[dom] * 1e-3) / 1e9
     out = {
-        "metric": "LayerNorm fwd+bwd + softmax 4096x4096 f32, algorithmic GB/s (norm/softmax leg of: FMHA/MoE/GEMM TFLOPS + norm/softmax GB/s, % of MI355X roofline)",
+        "metric": "LayerNorm fwd+bwd + softmax 4096x4096 f32, algorithmic GB/s (the norm/softmax leg of: FMHA/MoE/GEMM TFLOPS + norm/softmax GB/s, % of MI355X roofline; the other legs are under 'kernels')",
         "value": round(total_work / sec_per_step / 1e9, 2), "unit": "GB/s", "n_gpus": 1, "steps": args.steps,
         "warmup": args.warmup, "ms_per_step": round(sec_per_step * 1e3, 5), "higher_is_better": True,
         "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
@@ -234,15 +395,16 @@ def main():
                      "avg_launch_ms": round(per_stage[dom], 5), "algorithmic_bytes": work[dom]},
         "stages_ms": {k: round(v, 5) for k, v in per_stage.items()},
     }
-    if args.kernels != "none":
-        which = None if args.kernels == "all" else set(args.kernels.split(","))
-        out["kernels"] = bench_kernels(ct, which)
     if not args.no_cpu:
         out["cpu_baseline"] = cpu_baseline_headline()
+    if args.kernels != "none":
+        which = None if args.kernels == "all" else set(args.kernels.split(","))
+        out["kernels"] = bench_kernels(ct, which, cpu=not args.no_cpu)
     if args.table and "kernels" in out:
         for k, e in out["kernels"].items():
-            print(f"{e['name']:<50} min {e['min_ms']:9.4f} ms  mean {e['mean_ms']:9.4f} ms  "
-                  f"{e['achieved']:10.1f} {e['unit']:<8} {100 * e['frac']:6.2f}% of {e['bound']} peak", file=sys.stderr)
+            cpu = f"  cpu {e['cpu_ms']:10.1f} ms" if "cpu_ms" in e else ""
+            print(f"{e['name'][:72]:<72} min {e['min_ms']:8.4f}  avg {e['avg_ms']:8.4f} ms  "
+                  f"{e['achieved']:9.1f} {e['unit']:<8} {100 * e['frac']:6.2f}% of {e['bound']} peak{cpu}", file=sys.stderr)
     print(json.dumps(out))
 
 

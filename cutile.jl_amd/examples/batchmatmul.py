@@ -41,9 +41,3 @@ def smoke(orc):
     got = orc.to_julia(r.C).astype(np.float64)
     assert np.abs(got - ref).max() <= 1e-5 * np.abs(ref).max()
 
-
-def bench(ct_, entry, event_times, nruns, warmup):
-    d = prepare(benchmark=True)
-    t = event_times(lambda: ct_.batch_matmul_kernel(d.A, d.B, d.C, 128, 128, 64), nruns, warmup)
-    return {"batchmatmul": entry("batched GEMM 8x(1024x512x2048) f32", t, metric(d)[0], "TFLOPS", "mfma", 157.3,
-                                 "f32", {"variant": ct_.last_variant()})}

@@ -74,11 +74,3 @@ def smoke(orc):
     got = orc.to_julia(r.out).astype(np.float32)
     assert np.abs(got - ref).max() <= 2e-2 * np.abs(ref).max(), np.abs(got - ref).max()
 
-
-def bench(ct_, entry, event_times, nruns, warmup):
-    d = prepare(benchmark=True)
-    out = torch.empty_like(d.Q)
-    t = event_times(lambda: cutile_fmha(d.Q, d.K, d.V, causal=True, out=out), nruns, warmup)
-    return {"fmha": entry("causal FMHA 8x16x1024x64 f16", t, causal_flops(d), "TFLOPS", "mfma", 2500.0, "f16",
-                          {"variant": ct_.last_variant(), "dense_count_flop": metric(d)[0],
-                           "tflops_dense_count_at_min": round(metric(d)[0] / (min(t) * 1e-3) / 1e12, 2)})}

@@ -44,9 +44,3 @@ def smoke(orc):
     got = orc.to_julia(r.C).astype(np.float64)
     assert np.all(np.abs(got - ref) <= 2e-2 * np.abs(ref) + 2e-2 * np.abs(ref).max() * 1e-2), np.abs(got - ref).max()
 
-
-def bench(ct_, entry, event_times, nruns, warmup):
-    d = prepare(benchmark=True, T=torch.float16, out_T=torch.float32, dist="normal64")
-    t = event_times(lambda: ct_.matmul_kernel(d.A, d.B, d.C, 64, 64, 64), nruns, warmup)
-    return {"matmul": entry("GEMM 4096^3 f16 -> f32", t, metric(d)[0], "TFLOPS", "mfma", 2500.0, "f16",
-                            {"variant": ct_.last_variant()})}

@@ -119,24 +119,3 @@ def smoke(orc):
     got = J(r.out).astype(np.float32)
     assert np.abs(got - ref).max() <= 2e-2 * np.abs(ref).max(), np.abs(got - ref).max()
 
-
-def bench(ct_, entry, event_times, nruns, warmup):
-    res = {}
-    d = prepare(benchmark=True, topk=2, router="top2_logits")
-    t = event_times(lambda: cutile_moe(d.hidden_states, d.w1, d.w2, d.topk_weights, d.topk_ids, 128, 128, 64),
-                    nruns, warmup)
-    wbytes = (d.w1.numel() + d.w2.numel()) * 2 + 2 * d.hidden_states.numel() * 2
-    flop = metric(d)[0]
-    e = entry("MoE f16 256tok/1024h/32e/2048i top-2 (whole cutile_moe incl. host align)", t, wbytes, "GB/s", "hbm",
-              8000.0, "f16", {"flop": flop, "tflops_at_min": round(flop / (min(t) * 1e-3) / 1e12, 2),
-                              "mfma_frac_at_min": round(flop / (min(t) * 1e-3) / 1e12 / 2500.0, 5)})
-    res["moe_f16"] = e
-    tok, exp = ct_.moe_align_tile_size(d.topk_ids.cpu(), 128, d.num_experts)
-    al = (tok.cuda(), exp.cuda())
-    t = event_times(lambda: cutile_moe(d.hidden_states, d.w1, d.w2, d.topk_weights, d.topk_ids, 128, 128, 64,
-                                       aligned=al), nruns, warmup)
-    res["moe_f16_device_only"] = entry("MoE f16 top-2 (device work only: zero-fill + 4 kernels)", t, wbytes, "GB/s",
-                                       "hbm", 8000.0, "f16",
-                                       {"flop": flop, "tflops_at_min": round(flop / (min(t) * 1e-3) / 1e12, 2),
-                                        "mfma_frac_at_min": round(flop / (min(t) * 1e-3) / 1e12 / 2500.0, 5)})
-    return res

@@ -391,7 +391,10 @@ def main():
         "config": {"workload": "configs[1]: row LayerNorm fwd+bwd (y, dx, dgamma, dbeta) + row softmax on 4096x4096 Float32",
                    "M": 4096, "N": 4096, "eps": 1e-5, "GROUP_SIZE_M": 64, "bytes_per_step": total_work},
         "roofline": {"bound": "hbm", "achieved": round(ach, 2), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": round(ach / HBM_PEAK_GBS, 4), "traffic": None, "kernel": dom,
+                     "frac": round(ach / HBM_PEAK_GBS, 4),
+                     # HBM bytes per launch from rocprofv3 FETCH_SIZE (x2.000) + WRITE_SIZE (x1.000) counter runs,
+                     # calibrated on vadd; summary: profiles/membound_kernels_hbm_traffic_pmc.txt
+                     "traffic": 218972979 if dom == "layer_norm_bwd_dx_partial_dwdb" else None, "kernel": dom,
                      "avg_launch_ms": round(per_stage[dom], 5), "algorithmic_bytes": work[dom]},
         "stages_ms": {k: round(v, 5) for k, v in per_stage.items()},
     }

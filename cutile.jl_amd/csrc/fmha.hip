@@ -4,18 +4,26 @@
 // Layout (Julia column-major): Q (D, Sq, H, B), K (D, Skv, KVH, B), V (D, Skv, KVH, B),
 // Out (D, Sq, H, B); D is contiguous, so a query / key / value vector is a contiguous run.
 //
-// Mapping to CDNA4.  A workgroup (4 waves) owns 128 consecutive queries of one (batch, head);
-// a wave owns 32 of them.  KV is walked in tiles of 64 keys staged in LDS.
+// Mapping to CDNA4 (fmha_fwd_dma_kernel; fmha_fwd_kernel below is the register-staged
+// fallback for inputs that are not 16-byte aligned, one 32-query tile per wave).
+// A workgroup owns 128 consecutive queries of one (batch, head): 2 waves x 64 queries for
+// D = 64, 4 waves x 32 for D = 128.  A wave's queries are two 32-query MFMA column tiles
+// which share every K / V fragment read.  KV is walked in tiles of 64 keys, double-buffered
+// in LDS by direct global->LDS loads (XOR swizzle applied on the global-address side).
 //   S^T (keys x queries) = K . Q : MFMA 32x32x16, row operand = K rows read as 16-byte
-//     D-contiguous fragments from an XOR-swizzled LDS tile, column operand = Q fragments
+//     D-contiguous fragments from the swizzled LDS tile, column operand = Q fragments
 //     held in registers for the whole kernel (lane % 32 = query).
 //   online softmax in the exp2 domain, entirely in registers: a query's scores live in the
-//     two lanes l and l^32, so row max / row sum need one cross-lane exchange each.
+//     two lanes l and l^32, so the row max needs one cross-lane exchange per tile; the
+//     accumulator is rescaled only on tiles where some row max rose; row sums are taken
+//     over the rounded P values with v_dot2 and combined across the lane pair at the end.
 //   O^T (D x queries) += V . P : the fp32 scores, rounded to the storage type (fmha.jl:124),
 //     are already in column-operand layout (lane % 32 = query, 8 keys per lane); the
 //     matching row operand is read from the V tile with the LDS transpose read, whose
 //     4-consecutive-row granularity matches the accumulator's 4-row groups, so P never
 //     moves between lanes.
+// Causal balance: with causal masking a wave takes the 32-query tiles u and NT-1-u, so every
+// wave walks the same number of KV tiles.  All query tiles of a (batch, head) run on one XCD.
 // Causal tile skipping: the KV loop stops at the workgroup's last query, and a wave skips
 // tiles that lie wholly above its own last query.  Masking and the ragged KV tail use -Inf
 // as in the reference (fmha.jl:92-103).

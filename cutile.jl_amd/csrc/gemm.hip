@@ -14,10 +14,10 @@
 //   gemm16_generic   f16/bf16, 64x64x32 workgroup tile, any shape / stride / alignment
 //                    (ragged edges are zero-padded on load and clipped on store, as
 //                    ct.load(padding_mode=Zero) / ct.store do).
-//   gemm16_big       f16/bf16, 256x256x64 workgroup tile, 4 waves of 128x128, direct
-//                    global->LDS loads, double-buffered LDS, XOR-swizzled LDS layouts;
-//                    used when M,N are multiples of 256, K of 64 and everything is 16-byte
-//                    aligned.
+//   gemm16_big       (gemm_big.hip) f16/bf16, 256x256 workgroup tile, 4 waves of 128x128,
+//                    K step 32 through a ring of four LDS stages filled by direct
+//                    global->LDS loads, XOR-swizzled LDS layouts; used when M,N are
+//                    multiples of 256, K of 128 and everything is 16-byte aligned.
 //   gemm32           fp32 via v_mfma_f32_32x32x2_f32 (gfx950 has no TF32-class MFMA;
 //                    the reference rounds fp32 operands to TF32, matmul.jl:49-52).
 //

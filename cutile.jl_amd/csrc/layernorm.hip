@@ -233,11 +233,7 @@ __global__ __launch_bounds__(BLOCK) void ln_bwd_kernel(float* __restrict__ DX, i
         float* dst = pass == 0 ? dwp : dbp;
         for (int c = threadIdx.x; c < N; c += BLOCK) {
             if (S == 1) dst[c] += stage[c];
-            else {
-#ifndef EXP_NOATOMIC
-                unsafeAtomicAdd(dst + c, stage[c]);
-#endif
-            }
+            else unsafeAtomicAdd(dst + c, stage[c]);
         }
         __syncthreads();
     }

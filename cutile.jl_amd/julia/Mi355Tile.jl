@@ -1,0 +1,261 @@
+# Mi355Tile.jl — Julia binding of libmi355tile.so (the C ABI in include/mi355tile.h).
+#
+# One Julia function per example kernel of cuTile.jl, with the kernel's own name and argument
+# order, so an example's host code changes only at the launch line:
+#
+#     @cuda backend=cuTile blocks=grid matmul_kernel(A, B, C, ct.Constant(tm), ct.Constant(tn), ct.Constant(tk))
+# becomes
+#     Mi355Tile.matmul_kernel(A, B, C, tm, tn, tk)
+#
+# Arrays are anything that answers `pointer`, `size`, `strides` and `eltype` with a DEVICE
+# pointer: `AMDGPU.ROCArray`, views of it (`SubArray`/`reshape`), or the `DevicePtrArray`
+# below for memory obtained from hipMalloc directly.  The default stream argument is the HIP
+# null stream; pass `AMDGPU.stream().stream` (a `hipStream_t`) to enqueue on the task's stream,
+# which is what the reference does with the task-local CUDA stream (src/launch.jl:862).
+#
+# This file has not been executed: the build image has no Julia.  It is the binding a
+# maintainer would add; the same entry points are exercised through Python ctypes by the
+# test-suite.
+
+module Mi355Tile
+
+const libmi355tile = get(ENV, "MI355TILE_LIB",
+                         joinpath(@__DIR__, "..", "libmi355tile.so"))
+
+# ---- mi_tile_array (include/mi355tile.h) -------------------------------------------------
+
+const MI_MAX_RANK = 4
+
+struct MiTileArray
+    ptr::Ptr{Cvoid}
+    dtype::Int32
+    ndim::Int32
+    sizes::NTuple{MI_MAX_RANK,Int64}
+    strides::NTuple{MI_MAX_RANK,Int64}
+end
+
+mi_dtype(::Type{Float32}) = Int32(0)
+mi_dtype(::Type{Float64}) = Int32(1)
+mi_dtype(::Type{Float16}) = Int32(2)
+mi_dtype(::Type{Int32})   = Int32(5)
+mi_dtype(::Type{Int64})   = Int32(6)
+# BFloat16 (BFloat16s.jl / Core.BFloat16) = 3 and Float8_E4M3FN (DLFP8Types.jl) = 4: add the
+# methods in a package extension, the way ext/DLFP8TypesExt.jl adds the cuTile mapping.
+mi_dtype(T::Type) = T === UInt8 ? Int32(4) :   # raw e4m3fn bytes
+                    error("Mi355Tile: unsupported element type $T")
+
+"A bare device allocation viewed as an N-d column-major array (no GPU package needed)."
+struct DevicePtrArray{T,N}
+    ptr::Ptr{T}
+    dims::NTuple{N,Int}
+end
+Base.pointer(a::DevicePtrArray) = a.ptr
+Base.size(a::DevicePtrArray) = a.dims
+Base.strides(a::DevicePtrArray{T,N}) where {T,N} =
+    ntuple(i -> prod(a.dims[1:i-1]; init=1), N)
+Base.eltype(::DevicePtrArray{T}) where {T} = T
+
+pad4(t::NTuple{N,<:Integer}, fill) where {N} =
+    ntuple(i -> i <= N ? Int64(t[i]) : Int64(fill), MI_MAX_RANK)
+
+"Descriptor of `a` — the same (ptr, sizes, strides-in-elements) triple that the reference's
+`TileArray(arr)` builds (src/language/types.jl:314-357)."
+function descriptor(a; dtype::Int32=mi_dtype(eltype(a)))
+    N = length(size(a))
+    N <= MI_MAX_RANK || error("Mi355Tile: rank $N > $MI_MAX_RANK")
+    MiTileArray(Ptr{Cvoid}(UInt(pointer(a))), dtype, Int32(N),
+                pad4(size(a), 1), pad4(strides(a), 0))
+end
+descriptor(::Nothing; kwargs...) = nothing
+
+struct MiError <: Exception
+    code::Cint
+    msg::String
+end
+Base.showerror(io::IO, e::MiError) = print(io, "mi355tile error ", e.code, ": ", e.msg)
+
+function check(rc::Cint)
+    rc == 0 && return nothing
+    msg = unsafe_string(ccall((:mi_strerror, libmi355tile), Cstring, (Cint,), rc))
+    throw(MiError(rc, msg))
+end
+
+ref(d::MiTileArray) = Ref(d)
+const NULLDESC = Ptr{MiTileArray}(C_NULL)
+
+version() = ccall((:mi_version, libmi355tile), Cint, ())
+last_variant() = unsafe_string(ccall((:mi_last_variant, libmi355tile), Cstring, ()))
+
+# ---- examples/vadd.jl ---------------------------------------------------------------------
+
+function vec_add_kernel_1d(a, b, c, tile::Integer; stream::Ptr{Cvoid}=C_NULL)
+    da, db, dc = ref(descriptor(a)), ref(descriptor(b)), ref(descriptor(c))
+    GC.@preserve a b c check(ccall((:mi_vec_add_kernel_1d, libmi355tile), Cint,
+        (Ref{MiTileArray}, Ref{MiTileArray}, Ref{MiTileArray}, Cint, Ptr{Cvoid}),
+        da, db, dc, tile, stream))
+end
+
+function vec_add_kernel_2d(a, b, c, tile_x::Integer, tile_y::Integer; stream::Ptr{Cvoid}=C_NULL)
+    da, db, dc = ref(descriptor(a)), ref(descriptor(b)), ref(descriptor(c))
+    GC.@preserve a b c check(ccall((:mi_vec_add_kernel_2d, libmi355tile), Cint,
+        (Ref{MiTileArray}, Ref{MiTileArray}, Ref{MiTileArray}, Cint, Cint, Ptr{Cvoid}),
+        da, db, dc, tile_x, tile_y, stream))
+end
+
+function vec_add_kernel_1d_gather(a, b, c, tile::Integer; stream::Ptr{Cvoid}=C_NULL)
+    da, db, dc = ref(descriptor(a)), ref(descriptor(b)), ref(descriptor(c))
+    GC.@preserve a b c check(ccall((:mi_vec_add_kernel_1d_gather, libmi355tile), Cint,
+        (Ref{MiTileArray}, Ref{MiTileArray}, Ref{MiTileArray}, Cint, Ptr{Cvoid}),
+        da, db, dc, tile, stream))
+end
+
+# ---- examples/transpose.jl ----------------------------------------------------------------
+
+function transpose_kernel(x, y, tm::Integer, tn::Integer; stream::Ptr{Cvoid}=C_NULL)
+    dx, dy = ref(descriptor(x)), ref(descriptor(y))
+    GC.@preserve x y check(ccall((:mi_transpose_kernel, libmi355tile), Cint,
+        (Ref{MiTileArray}, Ref{MiTileArray}, Cint, Cint, Ptr{Cvoid}),
+        dx, dy, tm, tn, stream))
+end
+
+# ---- examples/matmul.jl, examples/batchmatmul.jl ------------------------------------------
+
+function matmul_kernel(A, B, C, tm::Integer, tn::Integer, tk::Integer; stream::Ptr{Cvoid}=C_NULL)
+    dA, dB, dC = ref(descriptor(A)), ref(descriptor(B)), ref(descriptor(C))
+    GC.@preserve A B C check(ccall((:mi_matmul_kernel, libmi355tile), Cint,
+        (Ref{MiTileArray}, Ref{MiTileArray}, Ref{MiTileArray}, Cint, Cint, Cint, Ptr{Cvoid}),
+        dA, dB, dC, tm, tn, tk, stream))
+end
+
+function batch_matmul_kernel(A, B, C, tm::Integer, tn::Integer, tk::Integer; stream::Ptr{Cvoid}=C_NULL)
+    dA, dB, dC = ref(descriptor(A)), ref(descriptor(B)), ref(descriptor(C))
+    GC.@preserve A B C check(ccall((:mi_batch_matmul_kernel, libmi355tile), Cint,
+        (Ref{MiTileArray}, Ref{MiTileArray}, Ref{MiTileArray}, Cint, Cint, Cint, Ptr{Cvoid}),
+        dA, dB, dC, tm, tn, tk, stream))
+end
+
+function swizzle_2d(M, N, tm, tn, GROUP_SIZE_M, bid)
+    bm, bn = Ref{Int32}(0), Ref{Int32}(0)
+    ccall((:mi_swizzle_2d, libmi355tile), Cvoid,
+          (Int32, Int32, Int32, Int32, Int32, Int32, Ref{Int32}, Ref{Int32}),
+          M, N, tm, tn, GROUP_SIZE_M, bid, bm, bn)
+    return bm[], bn[]
+end
+
+# ---- examples/layernorm.jl ----------------------------------------------------------------
+
+function layer_norm_fwd(X, W, B, Y, Mean, Rstd, eps::Real, TILE_N::Integer; stream::Ptr{Cvoid}=C_NULL)
+    d = map(a -> ref(descriptor(a)), (X, W, B, Y, Mean, Rstd))
+    GC.@preserve X W B Y Mean Rstd check(ccall((:mi_layer_norm_fwd, libmi355tile), Cint,
+        (Ref{MiTileArray}, Ref{MiTileArray}, Ref{MiTileArray}, Ref{MiTileArray},
+         Ref{MiTileArray}, Ref{MiTileArray}, Cfloat, Cint, Ptr{Cvoid}),
+        d[1], d[2], d[3], d[4], d[5], d[6], Float32(eps), TILE_N, stream))
+end
+
+# The caller zero-fills DW and DB first, as the reference's run_bwd does (layernorm.jl:245-246).
+# `Locks` is accepted and ignored (pass the array or `nothing`).
+function layer_norm_bwd_dx_partial_dwdb(DX, DY, DW, DB, X, W, Mean, Rstd, Locks,
+                                        GROUP_SIZE_M::Integer, TILE_N::Integer;
+                                        stream::Ptr{Cvoid}=C_NULL)
+    d = map(a -> ref(descriptor(a)), (DX, DY, DW, DB, X, W, Mean, Rstd))
+    dl = Locks === nothing ? nothing : ref(descriptor(Locks))
+    GC.@preserve DX DY DW DB X W Mean Rstd Locks check(ccall(
+        (:mi_layer_norm_bwd_dx_partial_dwdb, libmi355tile), Cint,
+        (Ref{MiTileArray}, Ref{MiTileArray}, Ref{MiTileArray}, Ref{MiTileArray},
+         Ref{MiTileArray}, Ref{MiTileArray}, Ref{MiTileArray}, Ref{MiTileArray},
+         Ptr{MiTileArray}, Cint, Cint, Ptr{Cvoid}),
+        d[1], d[2], d[3], d[4], d[5], d[6], d[7], d[8],
+        dl === nothing ? NULLDESC : Base.unsafe_convert(Ptr{MiTileArray}, dl),
+        GROUP_SIZE_M, TILE_N, stream))
+end
+
+function layer_norm_bwd_dwdb(DW, DB, FINAL_DW, FINAL_DB, TILE_M::Integer, TILE_N::Integer;
+                             stream::Ptr{Cvoid}=C_NULL)
+    d = map(a -> ref(descriptor(a)), (DW, DB, FINAL_DW, FINAL_DB))
+    GC.@preserve DW DB FINAL_DW FINAL_DB check(ccall((:mi_layer_norm_bwd_dwdb, libmi355tile), Cint,
+        (Ref{MiTileArray}, Ref{MiTileArray}, Ref{MiTileArray}, Ref{MiTileArray}, Cint, Cint, Ptr{Cvoid}),
+        d[1], d[2], d[3], d[4], TILE_M, TILE_N, stream))
+end
+
+# ---- examples/softmax.jl ------------------------------------------------------------------
+
+function softmax_tma_kernel(output, input, TILE_SIZE::Integer; blocks::Integer=size(input, 2),
+                            stream::Ptr{Cvoid}=C_NULL)
+    dout, din = ref(descriptor(output)), ref(descriptor(input))
+    GC.@preserve output input check(ccall((:mi_softmax_tma_kernel, libmi355tile), Cint,
+        (Ref{MiTileArray}, Ref{MiTileArray}, Cint, Cint, Ptr{Cvoid}),
+        dout, din, TILE_SIZE, blocks, stream))
+end
+
+function softmax_chunked_kernel(output, input, n_elems::Integer, TILE_SIZE::Integer;
+                                blocks::Integer=size(input, 2), stream::Ptr{Cvoid}=C_NULL)
+    dout, din = ref(descriptor(output)), ref(descriptor(input))
+    GC.@preserve output input check(ccall((:mi_softmax_chunked_kernel, libmi355tile), Cint,
+        (Ref{MiTileArray}, Ref{MiTileArray}, Cint, Cint, Cint, Ptr{Cvoid}),
+        dout, din, n_elems, TILE_SIZE, blocks, stream))
+end
+
+# ---- examples/fmha.jl ---------------------------------------------------------------------
+
+function fmha_kernel(Q, K, V, Out, qk_scale::Real, input_pos::Integer, TILE_D::Integer,
+                     H::Integer, TILE_M::Integer, TILE_N::Integer, QUERY_GROUP_SIZE::Integer,
+                     CAUSAL::Bool, EVEN_K::Bool; stream::Ptr{Cvoid}=C_NULL)
+    d = map(a -> ref(descriptor(a)), (Q, K, V, Out))
+    GC.@preserve Q K V Out check(ccall((:mi_fmha_kernel, libmi355tile), Cint,
+        (Ref{MiTileArray}, Ref{MiTileArray}, Ref{MiTileArray}, Ref{MiTileArray}, Cfloat, Int32,
+         Cint, Cint, Cint, Cint, Cint, Cint, Cint, Ptr{Cvoid}),
+        d[1], d[2], d[3], d[4], Float32(qk_scale), Int32(input_pos), TILE_D, H, TILE_M, TILE_N,
+        QUERY_GROUP_SIZE, CAUSAL, EVEN_K, stream))
+end
+
+# ---- examples/moe.jl ----------------------------------------------------------------------
+
+"Host routine; `topk_ids` is the (num_tokens, topk) Int64 matrix of 1-based expert ids
+(examples/moe.jl:142-183).  Returns (sorted_token_ids, sorted_expert_ids) as host Int32 vectors."
+function moe_align_tile_size(topk_ids::Matrix{Int64}, tile_m::Integer, num_experts::Integer)
+    nt, topk = size(topk_ids)
+    nblocks = Ref{Int64}(0)
+    check(ccall((:mi_moe_align_tile_size, libmi355tile), Cint,
+        (Ptr{Int64}, Int64, Int64, Cint, Cint, Ptr{Int32}, Ptr{Int32}, Ref{Int64}),
+        topk_ids, nt, topk, tile_m, num_experts, C_NULL, C_NULL, nblocks))
+    ids = Vector{Int32}(undef, nblocks[] * tile_m)
+    experts = Vector{Int32}(undef, nblocks[])
+    check(ccall((:mi_moe_align_tile_size, libmi355tile), Cint,
+        (Ptr{Int64}, Int64, Int64, Cint, Cint, Ptr{Int32}, Ptr{Int32}, Ref{Int64}),
+        topk_ids, nt, topk, tile_m, num_experts, ids, experts, nblocks))
+    return ids, experts
+end
+
+# `b_scale` (N, E) Float32 goes with e4m3fn weights only; `nothing` otherwise.
+function fused_moe_kernel(A, B, C, topk_weights, sorted_token_ids, sorted_expert_ids,
+                          num_token_replicas::Integer, mul_routed_weight::Bool,
+                          TILE_M::Integer, TILE_N::Integer, TILE_K::Integer;
+                          b_scale=nothing, stream::Ptr{Cvoid}=C_NULL)
+    d = map(a -> ref(descriptor(a)), (A, B, C, topk_weights, sorted_token_ids, sorted_expert_ids))
+    ds = b_scale === nothing ? nothing : ref(descriptor(b_scale))
+    GC.@preserve A B C topk_weights sorted_token_ids sorted_expert_ids b_scale check(ccall(
+        (:mi_fused_moe_kernel, libmi355tile), Cint,
+        (Ref{MiTileArray}, Ref{MiTileArray}, Ref{MiTileArray}, Ref{MiTileArray},
+         Ref{MiTileArray}, Ref{MiTileArray}, Cint, Cint, Cint, Cint, Cint,
+         Ptr{MiTileArray}, Ptr{Cvoid}),
+        d[1], d[2], d[3], d[4], d[5], d[6], num_token_replicas, mul_routed_weight,
+        TILE_M, TILE_N, TILE_K,
+        ds === nothing ? NULLDESC : Base.unsafe_convert(Ptr{MiTileArray}, ds), stream))
+end
+
+function silu_and_mul_kernel(A, B, C, TILE_N::Integer; stream::Ptr{Cvoid}=C_NULL)
+    d = map(a -> ref(descriptor(a)), (A, B, C))
+    GC.@preserve A B C check(ccall((:mi_silu_and_mul_kernel, libmi355tile), Cint,
+        (Ref{MiTileArray}, Ref{MiTileArray}, Ref{MiTileArray}, Cint, Ptr{Cvoid}),
+        d[1], d[2], d[3], TILE_N, stream))
+end
+
+"out (H, tokens) = sum over dim 2 of in (H, topk, tokens): the `sum(cache3; dims=2)` of
+cutile_moe (examples/moe.jl:256)."
+function moe_sum_topk(in, out; stream::Ptr{Cvoid}=C_NULL)
+    d = map(a -> ref(descriptor(a)), (in, out))
+    GC.@preserve in out check(ccall((:mi_moe_sum_topk, libmi355tile), Cint,
+        (Ref{MiTileArray}, Ref{MiTileArray}, Ptr{Cvoid}), d[1], d[2], stream))
+end
+
+end # module

@@ -78,6 +78,13 @@ def test_tilearray_descriptor_follows_julia_order(ct):
     assert dv.ptr == t.data_ptr() + 2 * 4
 
 
+def test_descriptor_struct_layout_matches_header(ct):
+    # struct mi_tile_array: void* ptr; int32 dtype; int32 ndim; int64 sizes[4]; int64 strides[4]
+    M = ct.MiTileArray
+    assert ctypes.sizeof(M) == 80
+    assert (M.ptr.offset, M.dtype.offset, M.ndim.offset, M.sizes.offset, M.strides.offset) == (0, 8, 12, 16, 48)
+
+
 def test_host_swizzle_matches_oracle(ct, orc):
     for (M, N, tm, tn) in [(4096, 4096, 64, 64), (200, 100, 64, 64), (1000, 130, 32, 64), (4096, 512, 128, 128)]:
         for bid in range(1, orc.cld(M, tm) * orc.cld(N, tn) + 1):

@@ -29,41 +29,15 @@
 // as in the reference (fmha.jl:92-103).
 //
 // FLOPs (causal-exact): 4 * B * H * D * Sq*(Sq+1)/2 for Sq == Skv.
-#include "common.h"
-#include <math.h>
+#include "fmha_common.h"
+#include <stdlib.h>
+#include <string.h>
 
 namespace {
 
 using namespace mi;
+using namespace mi::fmha;
 
-typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
-typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
-typedef short s16x4 __attribute__((ext_vector_type(4)));
-typedef short s16x8 __attribute__((ext_vector_type(8)));
-typedef float f32x16 __attribute__((ext_vector_type(16)));
-
-#define LDS_PTR(T, p) ((T __attribute__((address_space(3)))*)(p))
-
-struct F16 {
-    static __device__ __forceinline__ f32x16 mfma32(s16x8 a, s16x8 b, f32x16 c) {
-        return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, a), __builtin_bit_cast(f16x8, b), c, 0, 0, 0);
-    }
-    static __device__ __forceinline__ short cvt(float v) {
-        _Float16 h = (_Float16)v;
-        return __builtin_bit_cast(short, h);
-    }
-};
-struct BF16 {
-    static __device__ __forceinline__ f32x16 mfma32(s16x8 a, s16x8 b, f32x16 c) {
-        return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
-    }
-    static __device__ __forceinline__ short cvt(float v) {
-        unsigned u = __float_as_uint(v);
-        if ((u & 0x7fffffffu) > 0x7f800000u) return (short)((u >> 16) | 0x40);
-        u += 0x7fffu + ((u >> 16) & 1u);
-        return (short)(u >> 16);
-    }
-};
 
 constexpr int kQB = 128;  // queries per workgroup
 constexpr int kKV = 64;   // keys per LDS tile
@@ -80,9 +54,6 @@ __device__ __forceinline__ s16x8 lds_read_v_frag(const unsigned short* base, int
     return __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
 }
 
-struct Strides {
-    int64_t s1, s2, s3;  // element strides of dims 1..3 (dim 0 is contiguous)
-};
 
 template <typename E, int D, bool CAUSAL>
 __global__ __launch_bounds__(256) void fmha_fwd_kernel(const unsigned short* __restrict__ Q, Strides qs,
@@ -275,32 +246,6 @@ __global__ __launch_bounds__(256) void fmha_fwd_kernel(const unsigned short* __r
 // weights that multiply V.  The accumulator is rescaled only on tiles where some row's max
 // actually rose.  Workgroups are numbered so that all query tiles of one (batch, head) run
 // on the same XCD and share its K/V in that XCD's L2.
-typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
-typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
-
-template <typename E> struct Pack;
-template <> struct Pack<F16> {
-    static __device__ __forceinline__ unsigned pack(float a, float b) {
-        f16x2 v = {(_Float16)a, (_Float16)b};
-        return __builtin_bit_cast(unsigned, v);
-    }
-    static __device__ __forceinline__ float sum2(unsigned p, float acc) {
-        const f16x2 one = {(_Float16)1.0f, (_Float16)1.0f};
-        return __builtin_amdgcn_fdot2(__builtin_bit_cast(f16x2, p), one, acc, false);
-    }
-};
-template <> struct Pack<BF16> {
-    static __device__ __forceinline__ unsigned pack(float a, float b) {
-        bf16x2 v = {(__bf16)a, (__bf16)b};
-        return __builtin_bit_cast(unsigned, v);
-    }
-    static __device__ __forceinline__ float sum2(unsigned p, float acc) {
-        const bf16x2 one = {(__bf16)1.0f, (__bf16)1.0f};
-        return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2, p), one, acc, false);
-    }
-};
-
-typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
 
 __device__ __forceinline__ void gload_lds16(const void* g, void* lds_wave_base) {
     __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)g,
@@ -679,7 +624,20 @@ extern "C" int mi_fmha_kernel(const mi_tile_array* Q, const mi_tile_array* K, co
     const float scale2 = qk_scale * 1.4426950408889634f;  // fmha.jl:41: fold 1/log(2) for exp2
     dim3 grid((unsigned)cld(Sq, (int64_t)kQB), (unsigned)(B * H));
     hipStream_t s = (hipStream_t)stream;
-    const bool causal = CAUSAL != 0;
+    // A decode offset that already exposes every key to the first query makes the mask a no-op.
+    const bool causal = CAUSAL != 0 && input_pos < Skv - 1;
+    {
+        // MI_FMHA_KERNEL=dma keeps the double-buffered kernel below for every shape (comparison runs).
+        static const bool no_pipe = [] {
+            const char* e = getenv("MI_FMHA_KERNEL");
+            return e && strcmp(e, "dma") == 0;
+        }();
+        fmha::Problem pr{Q, K, V, Out, H, QUERY_GROUP_SIZE, scale2, input_pos, causal, dt == MI_BF16};
+        if (!no_pipe && fmha::pipe_applicable(pr)) {
+            fmha::pipe_launch(pr, s);
+            return launch_status();
+        }
+    }
     if (dt == MI_F16) {
         if (D == 64) launch<F16, 64>(grid, s, causal, Q, K, V, Out, H, QUERY_GROUP_SIZE, scale2, input_pos, vec_ok);
         else launch<F16, 128>(grid, s, causal, Q, K, V, Out, H, QUERY_GROUP_SIZE, scale2, input_pos, vec_ok);

@@ -1,0 +1,83 @@
+// Shared pieces of the fused-attention kernels: vector types, per-storage-type MFMA /
+// conversion traits, array strides.
+#pragma once
+#include "common.h"
+#include <math.h>
+
+namespace mi {
+namespace fmha {
+
+typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef short s16x4 __attribute__((ext_vector_type(4)));
+typedef short s16x8 __attribute__((ext_vector_type(8)));
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+
+#define LDS_PTR(T, p) ((T __attribute__((address_space(3)))*)(p))
+
+struct F16 {
+    static __device__ __forceinline__ f32x16 mfma32(s16x8 a, s16x8 b, f32x16 c) {
+        return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, a), __builtin_bit_cast(f16x8, b), c, 0, 0, 0);
+    }
+    static __device__ __forceinline__ short cvt(float v) {
+        _Float16 h = (_Float16)v;
+        return __builtin_bit_cast(short, h);
+    }
+};
+struct BF16 {
+    static __device__ __forceinline__ f32x16 mfma32(s16x8 a, s16x8 b, f32x16 c) {
+        return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
+    }
+    static __device__ __forceinline__ short cvt(float v) {
+        unsigned u = __float_as_uint(v);
+        if ((u & 0x7fffffffu) > 0x7f800000u) return (short)((u >> 16) | 0x40);
+        u += 0x7fffu + ((u >> 16) & 1u);
+        return (short)(u >> 16);
+    }
+};
+
+struct Strides {
+    int64_t s1, s2, s3;  // element strides of dims 1..3 (dim 0 is contiguous)
+};
+
+typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+
+template <typename E> struct Pack;
+template <> struct Pack<F16> {
+    static __device__ __forceinline__ unsigned pack(float a, float b) {
+        f16x2 v = {(_Float16)a, (_Float16)b};
+        return __builtin_bit_cast(unsigned, v);
+    }
+    static __device__ __forceinline__ float sum2(unsigned p, float acc) {
+        const f16x2 one = {(_Float16)1.0f, (_Float16)1.0f};
+        return __builtin_amdgcn_fdot2(__builtin_bit_cast(f16x2, p), one, acc, false);
+    }
+};
+template <> struct Pack<BF16> {
+    static __device__ __forceinline__ unsigned pack(float a, float b) {
+        bf16x2 v = {(__bf16)a, (__bf16)b};
+        return __builtin_bit_cast(unsigned, v);
+    }
+    static __device__ __forceinline__ float sum2(unsigned p, float acc) {
+        const bf16x2 one = {(__bf16)1.0f, (__bf16)1.0f};
+        return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2, p), one, acc, false);
+    }
+};
+
+typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
+
+// Software-pipelined kernel for head dimension 64 (fmha_pipe.hip).  `pipe_applicable` says
+// whether the problem has the shape that kernel is written for; `pipe_launch` enqueues it.
+struct Problem {
+    const mi_tile_array *Q, *K, *V, *O;
+    int H, group;     // query heads, query heads per KV head
+    float scale2;     // qk_scale / ln 2
+    int input_pos;
+    bool causal, bf16;
+};
+bool pipe_applicable(const Problem& p);
+void pipe_launch(const Problem& p, hipStream_t stream);
+
+}  // namespace fmha
+}  // namespace mi

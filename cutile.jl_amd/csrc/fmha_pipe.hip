@@ -9,17 +9,17 @@
 // after its diagonal.
 //
 // K and V travel in halves of 32 keys (4 KB each) through two rings of four LDS slots, filled
-// by direct global->LDS loads three steps ahead of their use.  One step handles one half:
-//     barrier (publishes the half issued three steps ago)
-//     issue loads of K half j+5 and V half j+3
-//     S(j+1) = K(j+1) . Q          8 MFMA, K fragments already in registers
-//     read K(j+2) and V(j) fragments from LDS
-//     softmax of S(j)              VALU, overlaps the MFMAs above
-//     O += V(j) . P(j)             8 MFMA
-// so the matrix pipe works on the next half's scores while the vector pipe exponentiates this
-// half's.  The two score buffers swap roles every step (the loops are unrolled by two), so no
-// register copies are needed.  The global->LDS loads are issued from inline assembly and waited
-// for with explicit vmcnt counts; the compiler sees only the LDS reads.
+// by direct global->LDS loads three steps ahead of their use.  One step handles one half j:
+//     raise the running maxima if the maxima of S(j) (taken in the previous step) demand it
+//     barrier (publishes the halves issued three steps ago), issue loads of K half j+5, V half j+3
+//     read the V(j) fragments
+//     S(j+1) = K(j+1) . Q   (K fragments already in registers)   |  interleaved, one MFMA per
+//     weights P(j) = exp2(S(j) - m), packed, row sums            |  issue slot, with the
+//     O += V(j) . P(j)      as soon as a 16-key chunk of P exists|  vector work
+//     read the K(j+2) fragments; row maxima of S(j+1)
+// The two score buffers swap roles every step (the loops are unrolled by two), so no register
+// copies are needed.  The global->LDS loads are issued from inline assembly and waited for with
+// explicit vmcnt counts; the compiler sees only the LDS reads.
 //
 // Online softmax in the exp2 domain (fmha.jl:41,106-127).  The running maximum m of a row is
 // only raised when the new maximum exceeds it by more than 8 (a factor 256 in the weights):
@@ -73,38 +73,44 @@ __device__ __forceinline__ float xhalf_sum(float v) {
 
 struct Lane {
     // wave-uniform
-    const char *Kg, *Vg;            // first key of this (batch, kv head)
+    const char *kptr, *vptr;        // next K / V half to be transferred
+    int k_left, v_left;             // halves not yet transferred (the last one is re-sent once they run out)
     int64_t k_half_bytes, v_half_bytes;
     unsigned ks_base, vs_base;      // LDS byte addresses of the rings
     int wave, nh;                   // halves walked by this workgroup
-    float scale2;
+    float scale2, inv_scale2;
     // per lane
-    unsigned kdma[2], vdma[2];      // byte offsets of the lane's 16 bytes in transfers wave, wave+2
+    unsigned kdma, vdma;            // byte offset of the lane's 16 bytes in transfer `wave` (transfer wave+2: 16 keys on)
     unsigned kfo[4];                // K fragment element offsets inside a slot, per k-step
     unsigned vfo[2];                // V fragment element offsets inside a slot, per d tile
-    int lim[2];                     // last visible key of the lane's query minus 4*(lane/32), per stream
+    int lim0;                       // (lane % 32) - 4 * (lane / 32)
+    int q0[2];                      // first query of each stream (wave-uniform)
 };
+
 
 template <typename E>
 struct Acc {
     s16x8 qf[2][4];
     f32x16 o[2][2];
-    float m[2], l[2];
+    float m[2], l[2];  // running maximum (exp2 domain) and sum of the lane's half of the keys
+    float thr[2];      // raw score above which m is raised: (m + kRaise) / scale2
 };
 
-__device__ __forceinline__ void issue_k(const Lane& c, int h, int slot) {
-    const int hc = h < c.nh ? h : c.nh - 1;  // past the end: reload the last half into a free slot
-    const char* g = c.Kg + hc * c.k_half_bytes;
+// Transfers the next K (V) half into ring slot `slot`.  Past the last half the same half is sent
+// again into a slot nobody reads, which keeps the count of outstanding transfers uniform.
+__device__ __forceinline__ void issue_k(Lane& c, int slot) {
     const unsigned lds = c.ks_base + slot * kSlotBytes + c.wave * 1024;
-    dma16(c.kdma[0], g, lds);
-    dma16(c.kdma[1], g, lds + 2048);
+    dma16(c.kdma, c.kptr, lds);
+    dma16(c.kdma, c.kptr + (c.k_half_bytes >> 1), lds + 2048);
+    c.k_left -= 1;
+    if (c.k_left > 0) c.kptr += c.k_half_bytes;
 }
-__device__ __forceinline__ void issue_v(const Lane& c, int h, int slot) {
-    const int hc = h < c.nh ? h : c.nh - 1;
-    const char* g = c.Vg + hc * c.v_half_bytes;
+__device__ __forceinline__ void issue_v(Lane& c, int slot) {
     const unsigned lds = c.vs_base + slot * kSlotBytes + c.wave * 1024;
-    dma16(c.vdma[0], g, lds);
-    dma16(c.vdma[1], g, lds + 2048);
+    dma16(c.vdma, c.vptr, lds);
+    dma16(c.vdma, c.vptr + (c.v_half_bytes >> 1), lds + 2048);
+    c.v_left -= 1;
+    if (c.v_left > 0) c.vptr += c.v_half_bytes;
 }
 
 __device__ __forceinline__ void read_k_frags(const unsigned short* Ks, const Lane& c, int slot, s16x8 (&kf)[4]) {
@@ -113,57 +119,72 @@ __device__ __forceinline__ void read_k_frags(const unsigned short* Ks, const Lan
 }
 
 // First part of the softmax of one stream's 32x32 score tile: apply the causal mask and return
-// the row maximum in the exp2 domain.
+// the row maximum of the raw scores (before the exp2-domain scale).
 template <bool MASK>
-__device__ __forceinline__ float masked_row_max(f32x16& s, int lim, float scale2) {
+__device__ __forceinline__ float masked_row_max(f32x16& s, int lim) {
     if (MASK) {
 #pragma unroll
         for (int r = 0; r < 16; ++r) s[r] = (8 * (r >> 2) + (r & 3) <= lim) ? s[r] : -INFINITY;
     }
-    float mx = fmaxf(s[0], s[1]);
+    float mx = fmaxf(fmaxf(s[0], s[1]), s[2]);
 #pragma unroll
-    for (int r = 2; r < 16; r += 2) mx = fmaxf(fmaxf(mx, s[r]), s[r + 1]);
-    return xhalf_max(mx) * scale2;
+    for (int r = 3; r < 15; r += 2) mx = fmaxf(fmaxf(mx, s[r]), s[r + 1]);
+    return xhalf_max(fmaxf(mx, s[15]));
 }
 
-// Second part: weights relative to the (possibly stale) running maximum, rounded and packed for
-// the P.V MFMAs, and their row sum.
+// The weights of one score pair (2h, 2h+1), h = 0..7, are made in two stages that the step below
+// places in consecutive issue slots, so that no instruction waits for the one just before it:
+// stage 1: 2 fma + 2 exp2 relative to the (possibly stale) running maximum;
+// stage 2: round and pack for the P.V MFMAs, add to the row sum.
+__device__ __forceinline__ void exp_stage1(const f32x16& s, int h, float nm, float scale2, float (&p)[2]) {
+    p[0] = __builtin_amdgcn_exp2f(__builtin_fmaf(s[2 * h], scale2, nm));
+    p[1] = __builtin_amdgcn_exp2f(__builtin_fmaf(s[2 * h + 1], scale2, nm));
+}
 template <typename E>
-__device__ __forceinline__ void exp_pack(const f32x16& s, float m, float& l, float scale2, unsigned (&pf)[2][4]) {
-    const float nm = -m;
-    float lsum = l;
-#pragma unroll
-    for (int r = 0; r < 16; r += 2) {
-        const float p0 = __builtin_amdgcn_exp2f(__builtin_fmaf(s[r], scale2, nm));
-        const float p1 = __builtin_amdgcn_exp2f(__builtin_fmaf(s[r + 1], scale2, nm));
-        const unsigned pk = Pack<E>::pack(p0, p1);
-        lsum = Pack<E>::sum2(pk, lsum);
-        pf[r >> 3][(r & 7) >> 1] = pk;
-    }
-    l = lsum;
+__device__ __forceinline__ void exp_stage2(const float (&p)[2], int h, float& l, unsigned (&pf)[2][4]) {
+    const unsigned pk = Pack<E>::pack(p[0], p[1]);
+    l = Pack<E>::sum2(pk, l);
+    pf[h >> 2][h & 3] = pk;
 }
 
-// One step.  CUR / NEXT: bit jj set = stream jj takes part in half j / half j+1.
-// MASKJ: stream whose diagonal may cross half j (-1: none).
-template <typename E, int CUR, int NEXT, int MASKJ>
-__device__ __forceinline__ void half_step(const unsigned short* Ks, const unsigned short* Vs, const Lane& c, Acc<E>& a,
-                                          int j, f32x16 (&s_cur)[2], f32x16 (&s_next)[2], s16x8 (&kf)[4]) {
-    // ---- row maxima of S(j); raise the running maxima if some row outgrew its own by 2^kRaise ----
+// Closes an issue slot: nothing is scheduled across it.
+__device__ __forceinline__ void slot_end() {
+    __builtin_amdgcn_sched_barrier(0);
+}
+
+constexpr int popcount2(int m) { return (m & 1) + ((m >> 1) & 1); }
+// k-th stream (0-based) of a non-empty 2-bit stream mask
+constexpr int nth_stream(int m, int k) { return (m & 1) ? k : 1; }
+
+// One step.  CUR / NEXT: bit jj set = stream jj takes part in half j / half j+1 (NEXT is a
+// subset of CUR).  MASKN: stream whose diagonal may cross half j+1 (-1: none).
+// On entry cand[jj] holds the raw row maxima of S(j); on exit those of S(j+1).
+//
+// A wave issues in order, so the body is laid out as issue slots -- one MFMA followed by the
+// vector work that fits in its shadow, closed by a scheduling barrier -- instead of leaving
+// the interleaving to the compiler:
+//   A: [S(j+1) MFMA] + two exp_pair pieces        while key chunk 0 of every stream is weighted
+//   B: [S(j+1) or P.V MFMA] + one exp_pair piece   while key chunk 1 is weighted; P.V MFMAs of a
+//                                                  chunk follow as soon as its weights exist
+//   C: remaining P.V MFMAs, each followed by the row maxima of one stream of S(j+1)
+template <typename E, int CUR, int NEXT, int MASKN>
+__device__ __forceinline__ void half_step(const unsigned short* Ks, const unsigned short* Vs, Lane& c, Acc<E>& a,
+                                          int j, f32x16 (&s_cur)[2], f32x16 (&s_next)[2], s16x8 (&kf)[4],
+                                          float (&cand)[2]) {
+    constexpr int nC = popcount2(CUR), nN = popcount2(NEXT);
+    constexpr int nQ = 4 * nN;   // S(j+1) MFMAs, k-step major over the NEXT streams
+    constexpr int nP = 2 * nC;   // P.V MFMAs per 16-key chunk, stream major
+    // ---- raise the running maxima if some row outgrew its own by 2^kRaise ---------------------------
     // (Every row sees key 0 in the first half, so a raised maximum is finite.)
-    float cand[2];
     bool raise = false;
 #pragma unroll
-    for (int jj = 0; jj < 2; ++jj) {
-        if (!((CUR >> jj) & 1)) continue;
-        cand[jj] = MASKJ == jj ? masked_row_max<true>(s_cur[jj], c.lim[jj] - kHK * j, c.scale2)
-                               : masked_row_max<false>(s_cur[jj], 0, c.scale2);
-        raise = raise || cand[jj] > a.m[jj] + kRaise;
-    }
+    for (int jj = 0; jj < 2; ++jj)
+        if ((CUR >> jj) & 1) raise = raise || cand[jj] > a.thr[jj];
     if (__any(raise)) {
 #pragma unroll
         for (int jj = 0; jj < 2; ++jj) {
             if (!((CUR >> jj) & 1)) continue;
-            const float m_new = fmaxf(a.m[jj], cand[jj]);
+            const float m_new = fmaxf(a.m[jj], cand[jj] * c.scale2);
             const float alpha = __builtin_amdgcn_exp2f(a.m[jj] - m_new);
             a.l[jj] *= alpha;
 #pragma unroll
@@ -171,23 +192,13 @@ __device__ __forceinline__ void half_step(const unsigned short* Ks, const unsign
 #pragma unroll
                 for (int r = 0; r < 16; ++r) a.o[jj][dt][r] *= alpha;
             a.m[jj] = m_new;
+            a.thr[jj] = (m_new + kRaise) * c.inv_scale2;
         }
     }
     wait_and_barrier<kWaitVm8>();
-    issue_k(c, j + 5, (j + 1) & 3);
-    issue_v(c, j + 3, (j + 3) & 3);
-
-    // ---- S(j+1) = K(j+1) . Q ------------------------------------------------------------------
-    if (NEXT) {
-#pragma unroll
-        for (int ks = 0; ks < 4; ++ks)
-#pragma unroll
-            for (int jj = 0; jj < 2; ++jj)
-                if ((NEXT >> jj) & 1) s_next[jj] = E::mfma32(kf[ks], a.qf[jj][ks], ks == 0 ? f32x16{0} : s_next[jj]);
-    }
-    // ---- fragment reads: K(j+2) for the next step, V(j) for this one ----------------------------
-    s16x8 kn[4];
-    if (NEXT) read_k_frags(Ks, c, (j + 2) & 3, kn);
+    issue_k(c, (j + 1) & 3);  // half j+5
+    issue_v(c, (j + 3) & 3);  // half j+3
+    // ---- V(j) fragments ------------------------------------------------------------------------------
     s16x8 vf[2][2];  // [16-key chunk][d tile]
     {
         const unsigned short* vb = Vs + (j & 3) * kSlot;
@@ -201,27 +212,83 @@ __device__ __forceinline__ void half_step(const unsigned short* Ks, const unsign
                 vf[ch][dt] = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
             }
     }
-    // ---- weights of S(j), then O += V(j) . P(j) ---------------------------------------------------
+    float nm[2];
+#pragma unroll
+    for (int jj = 0; jj < 2; ++jj) nm[jj] = -a.m[jj];
     unsigned pf[2][2][4];
+    slot_end();
+
+    int qi = 0, p0 = 0, p1 = 0, xi = 0, mi = 0;  // next S MFMA, next P.V MFMA of chunk 0 / 1, next exp piece, next maxima
+    auto mfma_q = [&]() {
+        constexpr int nNd = nN ? nN : 1;  // (never called when NEXT is empty)
+        const int ks = qi / nNd, jj = nth_stream(NEXT, qi % nNd);
+        s_next[jj] = E::mfma32(kf[ks], a.qf[jj][ks], ks == 0 ? f32x16{0} : s_next[jj]);
+        ++qi;
+    };
+    auto mfma_p = [&](int ch, int k) {
+        const int jj = nth_stream(CUR, k / 2), dt = k % 2;
+        u32x4 pw = {pf[jj][ch][0], pf[jj][ch][1], pf[jj][ch][2], pf[jj][ch][3]};
+        a.o[jj][dt] = E::mfma32(vf[ch][dt], __builtin_bit_cast(s16x8, pw), a.o[jj][dt]);
+    };
+    // exp pieces run chunk 0 of every stream, then chunk 1: piece x -> (chunk, stream, pair).
+    // piece() starts piece xi and finishes piece xi-1.
+    float pa[2], pb[2];  // stage-1 results in flight, used alternately
+    auto stage1 = [&](int x, float (&p)[2]) {
+        const int ch = x / (4 * nC), jj = nth_stream(CUR, (x / 4) % nC), h = 4 * ch + x % 4;
+        exp_stage1(s_cur[jj], h, nm[jj], c.scale2, p);
+    };
+    auto stage2 = [&](int x, const float (&p)[2]) {
+        const int ch = x / (4 * nC), jj = nth_stream(CUR, (x / 4) % nC), h = 4 * ch + x % 4;
+        exp_stage2<E>(p, h, a.l[jj], pf[jj]);
+    };
+    auto piece = [&]() {
+        if (xi % 2 == 0) {
+            if (xi < 8 * nC) stage1(xi, pa);
+            if (xi > 0) stage2(xi - 1, pb);
+        } else {
+            if (xi < 8 * nC) stage1(xi, pb);
+            stage2(xi - 1, pa);
+        }
+        ++xi;
+    };
+    auto maxima = [&]() {
+        const int jn = nth_stream(NEXT, mi);
+        cand[jn] = MASKN == jn ? masked_row_max<true>(s_next[jn], c.q0[jn] + c.lim0 - kHK * (j + 1))
+                               : masked_row_max<false>(s_next[jn], 0);
+        ++mi;
+    };
+    // A: chunk 0 of every stream
 #pragma unroll
-    for (int jj = 0; jj < 2; ++jj) {
-        if (!((CUR >> jj) & 1)) continue;
-        exp_pack<E>(s_cur[jj], a.m[jj], a.l[jj], c.scale2, pf[jj]);
+    for (int sl = 0; sl < 2 * nC; ++sl) {
+        if (qi < nQ) mfma_q();
+        piece();
+        piece();
+        slot_end();
+    }
+    // B: chunk 1; P.V MFMAs of chunk 0 alternate with the remaining S MFMAs, then those P.V MFMAs
+    // of chunk 1 whose weights are complete
+#pragma unroll
+    for (int sl = 0; sl < 4 * nC; ++sl) {
+        if (qi < nQ && (sl % 2 == 0 || p0 == nP)) mfma_q();
+        else if (p0 < nP && xi > 4 * ((p0 / 2) + 1)) mfma_p(0, p0++);
+        else if (p1 < nP && xi > 4 * nC + 4 * (p1 / 2 + 1)) mfma_p(1, p1++);
+        piece();
+        slot_end();
+    }
+    piece();  // finishes the last pair
+    // C
+    if (NEXT) read_k_frags(Ks, c, (j + 2) & 3, kf);  // every S MFMA has been issued: the old fragments are free
+#pragma unroll
+    for (int sl = 0; sl < 2 * nQ + 2 * nP; ++sl) {
+        if (qi < nQ) mfma_q();
+        else if (p0 < nP) mfma_p(0, p0++);
+        else if (p1 < nP) mfma_p(1, p1++);
+        else break;
+        if (qi == nQ && mi < nN && (sl % 2 == 1 || p1 == nP)) maxima();
+        slot_end();
     }
 #pragma unroll
-    for (int ch = 0; ch < 2; ++ch)
-#pragma unroll
-        for (int dt = 0; dt < 2; ++dt)
-#pragma unroll
-            for (int jj = 0; jj < 2; ++jj) {
-                if (!((CUR >> jj) & 1)) continue;
-                u32x4 pw = {pf[jj][ch][0], pf[jj][ch][1], pf[jj][ch][2], pf[jj][ch][3]};
-                a.o[jj][dt] = E::mfma32(vf[ch][dt], __builtin_bit_cast(s16x8, pw), a.o[jj][dt]);
-            }
-    if (NEXT) {
-#pragma unroll
-        for (int ks = 0; ks < 4; ++ks) kf[ks] = kn[ks];
-    }
+    while (mi < nN) maxima();
 }
 
 template <typename E, bool CAUSAL>
@@ -263,21 +330,27 @@ __global__ __launch_bounds__(128) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     }
 
     Lane c;
-    c.Kg = (const char*)(K + (int64_t)kvh * ks.s2 + (int64_t)batch * ks.s3);
-    c.Vg = (const char*)(V + (int64_t)kvh * vs.s2 + (int64_t)batch * vs.s3);
+    c.kptr = (const char*)(K + (int64_t)kvh * ks.s2 + (int64_t)batch * ks.s3);
+    c.vptr = (const char*)(V + (int64_t)kvh * vs.s2 + (int64_t)batch * vs.s3);
     c.k_half_bytes = (int64_t)kHK * ks.s1 * 2;
     c.v_half_bytes = (int64_t)kHK * vs.s1 * 2;
     c.ks_base = (unsigned)(size_t)Ks;
     c.vs_base = (unsigned)(size_t)Vs;
     c.wave = wave;
     c.nh = CAUSAL ? NT - 2 * qb : NT;
+    c.k_left = c.v_left = c.nh;
     c.scale2 = scale2;
-#pragma unroll
-    for (int i = 0; i < 2; ++i) {
-        const int key = 8 * (wave + 2 * i) + (lane >> 3), pos = lane & 7;
-        c.kdma[i] = (unsigned)(((int64_t)key * ks.s1 + 8 * (pos ^ (key & 7))) * 2);
-        c.vdma[i] = (unsigned)(((int64_t)key * vs.s1 + 8 * (pos ^ (2 * (key & 3)))) * 2);
+    c.inv_scale2 = 1.0f / scale2;
+    {
+        // transfer `wave` of a half covers keys 8*wave .. 8*wave+7; transfer wave+2 the keys 16 further on,
+        // whose swizzle (a function of key % 8 resp. key % 4) is the same
+        const int key = 8 * wave + (lane >> 3), pos = lane & 7;
+        c.kdma = (unsigned)(((int64_t)key * ks.s1 + 8 * (pos ^ (key & 7))) * 2);
+        c.vdma = (unsigned)(((int64_t)key * vs.s1 + 8 * (pos ^ (2 * (key & 3)))) * 2);
     }
+    c.lim0 = (lane & 31) - 4 * hb;
+    c.q0[0] = 32 * tq[0];
+    c.q0[1] = 32 * tq[1];
     {
         const int key = lane & 31;
 #pragma unroll
@@ -296,74 +369,42 @@ __global__ __launch_bounds__(128) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
 #pragma unroll
     for (int jj = 0; jj < 2; ++jj) {
         my_q[jj] = 32 * tq[jj] + (lane & 31);
-        c.lim[jj] = my_q[jj] - 4 * hb;
 #pragma unroll
         for (int s = 0; s < 4; ++s)
             a.qf[jj][s] = *reinterpret_cast<const s16x8*>(Q + (int64_t)my_q[jj] * qs.s1 + 16 * s + 8 * hb);
 #pragma unroll
         for (int dt = 0; dt < 2; ++dt) a.o[jj][dt] = f32x16{0};
         a.m[jj] = -INFINITY;
+        a.thr[jj] = -INFINITY;
         a.l[jj] = 0.f;
     }
 
     // ---- prologue: fill the rings, compute S(0), fetch the K(1) fragments -----------------------
-    issue_k(c, 0, 0);
-    issue_k(c, 1, 1);
-    issue_k(c, 2, 2);
-    issue_v(c, 0, 0);
-    issue_k(c, 3, 3);
-    issue_v(c, 1, 1);
+    issue_k(c, 0);
+    issue_k(c, 1);
+    issue_k(c, 2);
+    issue_v(c, 0);
+    issue_k(c, 3);
+    issue_v(c, 1);
     wait_and_barrier<kWaitVm4>();  // K(0..2), V(0) have landed
     f32x16 sa[2], sb[2];
     s16x8 kf[4];
+    float cand[2];
     read_k_frags(Ks, c, 0, kf);
 #pragma unroll
     for (int s = 0; s < 4; ++s)
 #pragma unroll
         for (int jj = 0; jj < 2; ++jj) sa[jj] = E::mfma32(kf[s], a.qf[jj][s], s == 0 ? f32x16{0} : sa[jj]);
-    {
-        s16x8 k1[4];
-        read_k_frags(Ks, c, 1, k1);
+    read_k_frags(Ks, c, 1, kf);
 #pragma unroll
-        for (int s = 0; s < 4; ++s) kf[s] = k1[s];
-    }
+    for (int jj = 0; jj < 2; ++jj)  // tile 0 has its diagonal in half 0
+        cand[jj] = CAUSAL ? masked_row_max<true>(sa[jj], c.q0[jj] + c.lim0) : masked_row_max<false>(sa[jj], 0);
     wait_and_barrier<kWaitVm4>();  // every wave has read its K(0) fragments: slot 0 is free
-    issue_k(c, 4, 0);
-    issue_v(c, 2, 2);
+    issue_k(c, 0);  // half 4
+    issue_v(c, 2);
 
-    // ---- main loops: two steps per trip, the score buffers swap roles --------------------------------
-    const int nh = c.nh;
-    int j = 0;
-    if (CAUSAL) {
-        const int n1 = 2 * qb + 2;  // steps in which stream 0 takes part; its diagonal is in the last two
-        for (; j < n1 - 2; j += 2) {
-            half_step<E, 3, 3, -1>(Ks, Vs, c, a, j, sa, sb, kf);
-            half_step<E, 3, 3, -1>(Ks, Vs, c, a, j + 1, sb, sa, kf);
-        }
-        half_step<E, 3, 3, 0>(Ks, Vs, c, a, j, sa, sb, kf);
-        half_step<E, 3, 2, 0>(Ks, Vs, c, a, j + 1, sb, sa, kf);
-        j += 2;
-        for (; j < nh - 2; j += 2) {
-            half_step<E, 2, 2, -1>(Ks, Vs, c, a, j, sa, sb, kf);
-            half_step<E, 2, 2, -1>(Ks, Vs, c, a, j + 1, sb, sa, kf);
-        }
-        half_step<E, 2, 2, 1>(Ks, Vs, c, a, j, sa, sb, kf);
-        half_step<E, 2, 0, 1>(Ks, Vs, c, a, j + 1, sb, sa, kf);
-    } else {
-        for (; j < nh - 2; j += 2) {
-            half_step<E, 3, 3, -1>(Ks, Vs, c, a, j, sa, sb, kf);
-            half_step<E, 3, 3, -1>(Ks, Vs, c, a, j + 1, sb, sa, kf);
-        }
-        half_step<E, 3, 3, -1>(Ks, Vs, c, a, j, sa, sb, kf);
-        half_step<E, 3, 0, -1>(Ks, Vs, c, a, j + 1, sb, sa, kf);
-    }
-    // Transfers issued for halves past the end are still in flight: let them land before the
-    // workgroup's LDS can be handed to another workgroup.
-    __builtin_amdgcn_s_waitcnt(kWaitVm0);
-
-    // ---- epilogue: add the two half-row sums, O / l (approximate reciprocal), round, store --------
-#pragma unroll
-    for (int jj = 0; jj < 2; ++jj) {
+    // Epilogue of one stream: add the two half-row sums, O / l (approximate reciprocal), round, store.
+    auto store_tile = [&](int jj) {
         const float inv = __builtin_amdgcn_rcpf(xhalf_sum(a.l[jj]));
         unsigned short* op = O + (int64_t)my_q[jj] * os.s1;
 #pragma unroll
@@ -375,7 +416,54 @@ __global__ __launch_bounds__(128) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
                 for (int e = 0; e < 4; ++e) w[e] = E::cvt(a.o[jj][dt][4 * g + e] * inv);
                 *reinterpret_cast<s16x4*>(op + 32 * dt + 8 * g + 4 * hb) = w;
             }
+    };
+
+    // ---- main loops: two steps per trip, the score buffers swap roles --------------------------------
+#define STEP(CUR, NEXT, MASKN, jx, s0, s1) half_step<E, CUR, NEXT, MASKN>(Ks, Vs, c, a, jx, s0, s1, kf, cand)
+    const int nh = c.nh;
+    int j = 0;
+    if (CAUSAL) {
+        // Stream 0 takes part in steps 0..n1-1 and has its diagonal in halves n1-2, n1-1 (one per
+        // wave); stream 1 runs to the end and has its diagonal in halves nh-2, nh-1.  A half is
+        // masked when its row maxima are taken, i.e. one step before it is consumed.
+        const int n1 = 2 * qb + 2;
+        for (; j < n1 - 4; j += 2) {
+            STEP(3, 3, -1, j, sa, sb);
+            STEP(3, 3, -1, j + 1, sb, sa);
+        }
+        for (; j < n1 - 2; j += 2) {  // at most one trip; masking half n1-3 as well is harmless
+            STEP(3, 3, 0, j, sa, sb);
+            STEP(3, 3, 0, j + 1, sb, sa);
+        }
+        STEP(3, 3, 0, j, sa, sb);
+        STEP(3, 2, 1, j + 1, sb, sa);  // (stream 1's mask only bites when its diagonal is two halves away)
+        j += 2;
+        store_tile(0);  // stream 0 is complete: its registers are free for the rest of the walk
+        for (; j < nh - 4; j += 2) {
+            STEP(2, 2, -1, j, sa, sb);
+            STEP(2, 2, -1, j + 1, sb, sa);
+        }
+        for (; j < nh - 2; j += 2) {  // at most one trip
+            STEP(2, 2, 1, j, sa, sb);
+            STEP(2, 2, 1, j + 1, sb, sa);
+        }
+        STEP(2, 2, 1, j, sa, sb);
+        STEP(2, 0, -1, j + 1, sb, sa);
+    } else {
+        for (; j < nh - 2; j += 2) {
+            STEP(3, 3, -1, j, sa, sb);
+            STEP(3, 3, -1, j + 1, sb, sa);
+        }
+        STEP(3, 3, -1, j, sa, sb);
+        STEP(3, 0, -1, j + 1, sb, sa);
     }
+#undef STEP
+    // Transfers issued for halves past the end are still in flight: let them land before the
+    // workgroup's LDS can be handed to another workgroup.
+    __builtin_amdgcn_s_waitcnt(kWaitVm0);
+
+    if (!CAUSAL) store_tile(0);
+    store_tile(1);
 }
 
 bool vec16(const mi_tile_array* a) {
@@ -423,3 +511,4 @@ void pipe_launch(const Problem& p, hipStream_t stream) {
 
 }  // namespace fmha
 }  // namespace mi
+

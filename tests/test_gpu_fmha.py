@@ -85,6 +85,38 @@ def test_fmha_strided_views_and_scale(orc):
     check(orc, out, ref)
 
 
+@pytest.mark.parametrize("batch,heads,s,causal,qg,T", [
+    (1, 4, 512, True, 2, torch.float16), (1, 2, 640, True, 1, torch.float16), (1, 2, 640, False, 1, torch.float16),
+    (1, 2, 512, True, 1, torch.bfloat16), (3, 3, 256, True, 1, torch.float16), (1, 8, 1024, False, 8, torch.float16),
+])
+def test_fmha_pipelined_kernel_shapes(ct, orc, batch, heads, s, causal, qg, T):
+    """Shapes served by the software-pipelined D = 64 kernel (Sq == Skv, multiple of 128): odd numbers
+    of 128-query blocks, (batch*heads) not a multiple of 8, GQA, bf16, and both mask settings."""
+    data = fmha.prepare(batch=batch, heads=heads, seq_q=s, seq_kv=s, query_group_size=qg, causal=causal, T=T)
+    r = fmha.run(data)
+    assert ct.last_variant().startswith("fmha_pipe")
+    ref = orc.ref_fmha(*(orc.to_julia(t) for t in (data.Q, data.K, data.V)), causal=causal, dtype=np.float64)
+    check(orc, r.out, ref, 2e-2 if T == torch.float16 else 3e-2)
+
+
+@pytest.mark.parametrize("causal", [True, False])
+def test_fmha_running_maximum_keeps_rising(ct, orc, causal):
+    """Scores that grow with the key index by far more than the kernel's lazy-rescale threshold:
+    the running maximum has to be raised again and again, and early keys end up with weights
+    far below the smallest f16 subnormal."""
+    rng = np.random.default_rng(11)
+    D, S, H, B = 64, 512, 2, 1
+    q = rng.standard_normal((D, S, H, B)).astype(np.float32) * 0.25 + 1.0
+    ramp = (1.0 + 6.0 * np.arange(S) / S)[None, :, None, None]
+    k = (rng.standard_normal((D, S, H, B)).astype(np.float32) * 0.25 + 1.0) * ramp
+    v = rng.standard_normal((D, S, H, B)).astype(np.float32)
+    Q, K, V = (orc.from_julia(x).to(torch.float16).cuda() for x in (q, k, v))
+    out = fmha.cutile_fmha(Q, K, V, causal=causal)
+    assert ct.last_variant().startswith("fmha_pipe")
+    ref = orc.ref_fmha(*(orc.to_julia(t) for t in (Q, K, V)), causal=causal, dtype=np.float64)
+    check(orc, out, ref)
+
+
 def test_fmha_argument_errors(ct):
     data = fmha.prepare(batch=1, heads=2, seq_q=128, seq_kv=128)
     out = torch.empty_like(data.Q)

@@ -55,17 +55,27 @@ struct BF16 {
     static __device__ __forceinline__ float widen(unsigned short h) { return __uint_as_float(((unsigned)h) << 16); }
 };
 
-// Two E4M3FN bytes (the low or high half of `w`) -> two f16, exactly.  The byte's 7 magnitude
-// bits land in f16's exponent/mantissa fields shifted by 7, which gives value * 2^-8 for
-// normals and subnormals alike (bias 7 vs 15); the factor 2^8 is applied by an exact f16
-// multiply.  (NaN codes never occur in weights.)
-__device__ __forceinline__ unsigned e4m3x2_to_f16x2(unsigned w16) {
-    const unsigned x = (w16 & 0xffu) | ((w16 & 0xff00u) << 8);       // bytes at bits 0-7 and 16-23
-    const unsigned bits = ((x & 0x007f007fu) << 7) | ((x & 0x00800080u) << 8);
-    f16x2 h = __builtin_bit_cast(f16x2, bits);
-    h = h * (f16x2){(_Float16)256.0f, (_Float16)256.0f};
-    return __builtin_bit_cast(unsigned, h);
-}
+// Four E4M3FN bytes -> four values of the activation type.  gfx950's FP8 is the OCP E4M3FN
+// format; its conversion instruction with scale 1 is exact for f16 (every e4m3 value,
+// subnormals included, is an f16 value).  For bf16 activations the f16 pair is widened and
+// truncated, also exactly (e4m3 has 3 mantissa bits).
+template <typename E> struct Fp8;
+template <> struct Fp8<F16> {
+    static __device__ __forceinline__ void cvt4(unsigned w, unsigned& lo, unsigned& hi) {
+        lo = __builtin_bit_cast(unsigned, __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(w, 1.0f, false));
+        hi = __builtin_bit_cast(unsigned, __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(w, 1.0f, true));
+    }
+};
+template <> struct Fp8<BF16> {
+    static __device__ __forceinline__ unsigned f16x2_to_bf16x2(f16x2 h) {
+        const unsigned a = __float_as_uint((float)h[0]) >> 16, b = __float_as_uint((float)h[1]) & 0xffff0000u;
+        return a | b;
+    }
+    static __device__ __forceinline__ void cvt4(unsigned w, unsigned& lo, unsigned& hi) {
+        lo = f16x2_to_bf16x2(__builtin_amdgcn_cvt_scalef32_pk_f16_fp8(w, 1.0f, false));
+        hi = f16x2_to_bf16x2(__builtin_amdgcn_cvt_scalef32_pk_f16_fp8(w, 1.0f, true));
+    }
+};
 
 constexpr int kTT = 32;   // token slots per workgroup (one MFMA row tile)
 
@@ -119,10 +129,13 @@ __global__ __launch_bounds__(256) void fused_moe_kernel(
 
     f32x16 acc = f32x16{0};
     // staging registers for the next B tile (128 n x kKT k) and A tile (32 slots x kKT k)
-    constexpr int CPR = kKT / 8;            // 16-byte chunks per tile row
-    constexpr int NB = kNT * CPR / 256;     // B chunks per thread
+    constexpr int CPR = kKT / 8;            // 16-byte chunks per LDS tile row
+    constexpr int EPB = W8 ? 16 : 8;        // weight elements per 16-byte global chunk
+    constexpr int CPRB = kKT / EPB;         // 16-byte global chunks per weight row
+    constexpr int NB = kNT * CPRB / 256;    // weight chunks per thread
     constexpr int NA = kTT * CPR / 256;     // A chunks per thread
-    s16x8 breg[NB], areg[NA];
+    u32x4 breg[NB];                         // raw bytes; e4m3 weights are widened on their way into LDS
+    s16x8 areg[NA];
     int a_col[NA];
 #pragma unroll
     for (int i = 0; i < NA; ++i) {
@@ -136,33 +149,22 @@ __global__ __launch_bounds__(256) void fused_moe_kernel(
     auto load_tiles = [&](int k0) {
 #pragma unroll
         for (int i = 0; i < NB; ++i) {
-            const int id = tid + 256 * i, n = id / CPR, c = id % CPR;
-            const int gn = n0 + n, gk = k0 + 8 * c;
-            s16x8 v = {0};
+            const int id = tid + 256 * i, n = id / CPRB, c = id % CPRB;
+            const int gn = n0 + n, gk = k0 + EPB * c;
+            u32x4 v = {0, 0, 0, 0};
             if (gn < N && gk < K) {
                 if (W8) {
                     const unsigned char* p = B8 + gk + (int64_t)gn * ldb;
-                    u32x2 raw = {0, 0};
-                    if (vecB && gk + 8 <= K) raw = __builtin_nontemporal_load(reinterpret_cast<const u32x2*>(p));
-                    else {
-                        unsigned long long acc8 = 0;
-                        for (int e = 0; e < 8; ++e)
-                            if (gk + e < K) acc8 |= (unsigned long long)p[e] << (8 * e);
-                        raw[0] = (unsigned)acc8;
-                        raw[1] = (unsigned)(acc8 >> 32);
-                    }
-                    u32x4 w;
-                    w[0] = e4m3x2_to_f16x2(raw[0] & 0xffffu);
-                    w[1] = e4m3x2_to_f16x2(raw[0] >> 16);
-                    w[2] = e4m3x2_to_f16x2(raw[1] & 0xffffu);
-                    w[3] = e4m3x2_to_f16x2(raw[1] >> 16);
-                    v = __builtin_bit_cast(s16x8, w);
+                    if (vecB && gk + 16 <= K) v = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(p));
+                    else
+                        for (int e = 0; e < 16; ++e)
+                            if (gk + e < K) v[e >> 2] |= (unsigned)p[e] << (8 * (e & 3));
                 } else {
                     const unsigned short* p = B16 + gk + (int64_t)gn * ldb;
-                    if (vecB && gk + 8 <= K) v = __builtin_nontemporal_load(reinterpret_cast<const s16x8*>(p));
+                    if (vecB && gk + 8 <= K) v = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(p));
                     else
-#pragma unroll
-                        for (int e = 0; e < 8; ++e) v[e] = (gk + e < K) ? (short)p[e] : (short)0;
+                        for (int e = 0; e < 8; ++e)
+                            if (gk + e < K) v[e >> 1] |= (unsigned)p[e] << (16 * (e & 1));
                 }
             }
             breg[i] = v;
@@ -187,8 +189,17 @@ __global__ __launch_bounds__(256) void fused_moe_kernel(
         __syncthreads();
 #pragma unroll
         for (int i = 0; i < NB; ++i) {
-            const int id = tid + 256 * i, n = id / CPR, c = id % CPR;
-            *reinterpret_cast<s16x8*>(&Bs[n * kKT + 8 * (c ^ (n & 7))]) = breg[i];
+            const int id = tid + 256 * i, n = id / CPRB, c = id % CPRB;
+            if (W8) {
+                unsigned w[8];
+#pragma unroll
+                for (int q = 0; q < 4; ++q) Fp8<E>::cvt4(breg[i][q], w[2 * q], w[2 * q + 1]);
+                const u32x4 lo = {w[0], w[1], w[2], w[3]}, hi = {w[4], w[5], w[6], w[7]};  // k elements 0-7, 8-15
+                *reinterpret_cast<u32x4*>(&Bs[n * kKT + 8 * ((2 * c) ^ (n & 7))]) = lo;
+                *reinterpret_cast<u32x4*>(&Bs[n * kKT + 8 * ((2 * c + 1) ^ (n & 7))]) = hi;
+            } else {
+                *reinterpret_cast<u32x4*>(&Bs[n * kKT + 8 * (c ^ (n & 7))]) = breg[i];
+            }
         }
 #pragma unroll
         for (int i = 0; i < NA; ++i) {
@@ -332,7 +343,7 @@ extern "C" int mi_fused_moe_kernel(const mi_tile_array* A, const mi_tile_array* 
     const int n_blocks = (int)cld(N, (int64_t)(narrow ? 32 : 128));
     if (tiles * n_blocks > 0x7fffffffLL) return MI_E_GRID;
     const bool vecA = aligned(A->ptr, 16) && A->strides[1] % 8 == 0;
-    const bool vecB = aligned(B->ptr, w8 ? 8 : 16) && B->strides[1] % 8 == 0 && B->strides[2] % 8 == 0;
+    const bool vecB = aligned(B->ptr, 16) && B->strides[1] % (w8 ? 16 : 8) == 0 && B->strides[2] % (w8 ? 16 : 8) == 0;
     dim3 grid((unsigned)(tiles * n_blocks));
     hipStream_t s = (hipStream_t)stream;
 #define LAUNCH(ET, W8, NTW, KT)                                                                                     \

@@ -1,6 +1,7 @@
 // Shared host/device helpers for libmi355tile (gfx950 only).
 #pragma once
 #include <hip/hip_runtime.h>
+#include <stdlib.h>
 #include <hip/hip_fp16.h>
 #include <hip/hip_bf16.h>
 #include <stdint.h>
@@ -132,6 +133,29 @@ template <> __device__ __forceinline__ float from_f32<float>(float v) { return v
 template <> __device__ __forceinline__ __half from_f32<__half>(float v) { return __float2half_rn(v); }
 template <> __device__ __forceinline__ __hip_bfloat16 from_f32<__hip_bfloat16>(float v) {
     return __float2bfloat16(v);
+}
+
+// Streaming (non-temporal) or cached global access, chosen per launch.  A working set that fits
+// the 256 MB memory-side cache is better served by ordinary accesses when the same buffers
+// are used launch after launch; anything larger should not evict it on its way through.
+template <bool STREAM, typename V>
+__device__ __forceinline__ V ld_global(const V* p) {
+    return STREAM ? __builtin_nontemporal_load(p) : *p;
+}
+template <bool STREAM, typename V>
+__device__ __forceinline__ void st_global(V v, V* p) {
+    if (STREAM) __builtin_nontemporal_store(v, p);
+    else *p = v;
+}
+// Host side of the choice: stream when the bytes one launch touches exceed what the memory-side
+// cache can keep next to other tenants.  MI_STREAM_HINT=0 / 1 forces one way (measurements).
+inline bool stream_hint(int64_t bytes_touched) {
+    static const int forced = [] {
+        const char* e = getenv("MI_STREAM_HINT");
+        return e ? (e[0] == '0' ? 0 : 1) : -1;
+    }();
+    if (forced >= 0) return forced != 0;
+    return bytes_touched > (224ll << 20);
 }
 
 }  // namespace mi

@@ -53,8 +53,7 @@ __device__ __forceinline__ void load_row(const float* __restrict__ p, int N, flo
     for (int v = 0; v < VPT; ++v) {
         const int e0 = (threadIdx.x + v * BLOCK) * 4;
         if (ALIGNED && e0 + 4 <= N) {
-            f32x4 t = NT ? __builtin_nontemporal_load(reinterpret_cast<const f32x4*>(p + e0))
-                         : *reinterpret_cast<const f32x4*>(p + e0);
+            f32x4 t = ld_global<NT>(reinterpret_cast<const f32x4*>(p + e0));
 #pragma unroll
             for (int q = 0; q < 4; ++q) r[v][q] = t[q];
         } else {
@@ -63,7 +62,7 @@ __device__ __forceinline__ void load_row(const float* __restrict__ p, int N, flo
         }
     }
 }
-template <int BLOCK, int VPT, bool ALIGNED>
+template <int BLOCK, int VPT, bool ALIGNED, bool NT>
 __device__ __forceinline__ void store_row(float* __restrict__ p, int N, const float (&r)[VPT][4]) {
 #pragma unroll
     for (int v = 0; v < VPT; ++v) {
@@ -72,7 +71,7 @@ __device__ __forceinline__ void store_row(float* __restrict__ p, int N, const fl
             f32x4 t;
 #pragma unroll
             for (int q = 0; q < 4; ++q) t[q] = r[v][q];
-            __builtin_nontemporal_store(t, reinterpret_cast<f32x4*>(p + e0));
+            st_global<NT>(t, reinterpret_cast<f32x4*>(p + e0));
         } else {
 #pragma unroll
             for (int q = 0; q < 4; ++q)
@@ -82,7 +81,7 @@ __device__ __forceinline__ void store_row(float* __restrict__ p, int N, const fl
 }
 
 // ---- forward ---------------------------------------------------------------------------
-template <int BLOCK, int VPT, bool ALIGNED>
+template <int BLOCK, int VPT, bool ALIGNED, bool STREAM>
 __global__ __launch_bounds__(BLOCK) void ln_fwd_kernel(const float* __restrict__ X, int64_t ldx,
                                                        const float* __restrict__ W,
                                                        const float* __restrict__ B,
@@ -94,8 +93,11 @@ __global__ __launch_bounds__(BLOCK) void ln_fwd_kernel(const float* __restrict__
     __shared__ float red[NW > 1 ? NW : 1];
     const float invN = 1.0f / (float)N;
     for (int64_t m = blockIdx.x; m < M; m += gridDim.x) {
-        float x[VPT][4];
-        load_row<BLOCK, VPT, ALIGNED, true>(X + m * ldx, N, x);
+        float x[VPT][4], w[VPT][4], b[VPT][4];
+        load_row<BLOCK, VPT, ALIGNED, STREAM>(X + m * ldx, N, x);
+        // W and B come from L2; asked for now, they arrive while the row is being reduced
+        load_row<BLOCK, VPT, ALIGNED, false>(W, N, w);
+        load_row<BLOCK, VPT, ALIGNED, false>(B, N, b);
         float s = 0.f;
 #pragma unroll
         for (int v = 0; v < VPT; ++v)
@@ -118,14 +120,11 @@ __global__ __launch_bounds__(BLOCK) void ln_fwd_kernel(const float* __restrict__
             Mean[m] = mean;
             Rstd[m] = rstd;
         }
-        float w[VPT][4], b[VPT][4];
-        load_row<BLOCK, VPT, ALIGNED, false>(W, N, w);
-        load_row<BLOCK, VPT, ALIGNED, false>(B, N, b);
 #pragma unroll
         for (int v = 0; v < VPT; ++v)
 #pragma unroll
             for (int q = 0; q < 4; ++q) x[v][q] = ((x[v][q] - mean) * rstd) * w[v][q] + b[v][q];
-        store_row<BLOCK, VPT, ALIGNED>(Y + m * ldy, N, x);
+        store_row<BLOCK, VPT, ALIGNED, STREAM>(Y + m * ldy, N, x);
     }
     (void)invN;
 }
@@ -164,7 +163,7 @@ __global__ __launch_bounds__(BLOCK) void ln_fwd_3pass_kernel(const float* __rest
 }
 
 // ---- backward: dX + partial dW/dB ------------------------------------------------------
-template <int BLOCK, int VPT, bool ALIGNED>
+template <int BLOCK, int VPT, bool ALIGNED, bool STREAM>
 __global__ __launch_bounds__(BLOCK) void ln_bwd_kernel(float* __restrict__ DX, int64_t lddx,
                                                        const float* __restrict__ DY, int64_t lddy,
                                                        float* __restrict__ DW, int64_t lddw,
@@ -187,8 +186,8 @@ __global__ __launch_bounds__(BLOCK) void ln_bwd_kernel(float* __restrict__ DX, i
 
     for (int64_t m = g + (int64_t)G * s; m < M; m += (int64_t)G * S) {
         float x[VPT][4], dy[VPT][4];
-        load_row<BLOCK, VPT, ALIGNED, true>(X + m * ldx, N, x);
-        load_row<BLOCK, VPT, ALIGNED, true>(DY + m * lddy, N, dy);
+        load_row<BLOCK, VPT, ALIGNED, STREAM>(X + m * ldx, N, x);
+        load_row<BLOCK, VPT, ALIGNED, STREAM>(DY + m * lddy, N, dy);
         const float mean = Mean[m], rstd = Rstd[m];
         float c1 = 0.f, c2 = 0.f;
 #pragma unroll
@@ -216,7 +215,7 @@ __global__ __launch_bounds__(BLOCK) void ln_bwd_kernel(float* __restrict__ DX, i
                 db[v][q] += dy[v][q];
                 x[v][q] = (wdy - (xhat * c1 + c2)) * rstd;
             }
-        store_row<BLOCK, VPT, ALIGNED>(DX + m * lddx, N, x);
+        store_row<BLOCK, VPT, ALIGNED, STREAM>(DX + m * lddx, N, x);
     }
     // Flush through LDS so that consecutive lanes add to consecutive addresses: a float atomic
     // instruction then covers 256 contiguous bytes instead of 64 scattered words (memory-side
@@ -320,12 +319,12 @@ bool rows_vec_ok(const mi_tile_array* a) {
 
 constexpr int kMaxRegsN = 256 * 16 * 4;
 
-template <bool AL>
+template <bool AL, bool ST>
 void launch_fwd(int vecs, dim3 grid, hipStream_t s, const float* X, int64_t ldx, const float* W,
                 const float* B, float* Y, int64_t ldy, float* Mean, float* Rstd, float eps, int N,
                 int64_t M) {
 #define FWD(BL, VP)                                                                              \
-    hipLaunchKernelGGL((ln_fwd_kernel<BL, VP, AL>), grid, dim3(BL), 0, s, X, ldx, W, B, Y, ldy, \
+    hipLaunchKernelGGL((ln_fwd_kernel<BL, VP, AL, ST>), grid, dim3(BL), 0, s, X, ldx, W, B, Y, ldy, \
                        Mean, Rstd, eps, N, M)
     if (vecs <= 64) { FWD(64, 1); set_variant("ln_fwd_regs_b64_v1"); }
     else if (vecs <= 128) { FWD(64, 2); set_variant("ln_fwd_regs_b64_v2"); }
@@ -337,13 +336,13 @@ void launch_fwd(int vecs, dim3 grid, hipStream_t s, const float* X, int64_t ldx,
 #undef FWD
 }
 
-template <bool AL>
+template <bool AL, bool ST>
 void launch_bwd(int vecs, dim3 grid, hipStream_t s, float* DX, int64_t lddx, const float* DY,
                 int64_t lddy, float* DW, int64_t lddw, float* DB, int64_t lddb, const float* X,
                 int64_t ldx, const float* W, const float* Mean, const float* Rstd, int N, int64_t M,
                 int G, int S) {
 #define BWD(BL, VP)                                                                            \
-    hipLaunchKernelGGL((ln_bwd_kernel<BL, VP, AL>), grid, dim3(BL), 0, s, DX, lddx, DY, lddy, \
+    hipLaunchKernelGGL((ln_bwd_kernel<BL, VP, AL, ST>), grid, dim3(BL), 0, s, DX, lddx, DY, lddy, \
                        DW, lddw, DB, lddb, X, ldx, W, Mean, Rstd, N, M, G, S)
     if (vecs <= 64) { BWD(64, 1); set_variant("ln_bwd_regs_b64_v1"); }
     else if (vecs <= 256) { BWD(256, 1); set_variant("ln_bwd_regs_b256_v1"); }
@@ -388,12 +387,13 @@ extern "C" int mi_layer_norm_fwd(const mi_tile_array* X, const mi_tile_array* W,
     }
     const bool al = rows_vec_ok(X) && rows_vec_ok(Y) && rows_vec_ok(W) && rows_vec_ok(B);
     const int vecs = (int)cld(N, 4);
-    if (al)
-        launch_fwd<true>(vecs, grid, s, x, X->strides[1], (const float*)W->ptr, (const float*)B->ptr,
-                         y, Y->strides[1], (float*)Mean->ptr, (float*)Rstd->ptr, eps, (int)N, M);
-    else
-        launch_fwd<false>(vecs, grid, s, x, X->strides[1], (const float*)W->ptr, (const float*)B->ptr,
-                          y, Y->strides[1], (float*)Mean->ptr, (float*)Rstd->ptr, eps, (int)N, M);
+#define ARGS                                                                                      \
+    vecs, grid, s, x, X->strides[1], (const float*)W->ptr, (const float*)B->ptr, y, Y->strides[1], \
+        (float*)Mean->ptr, (float*)Rstd->ptr, eps, (int)N, M
+    if (!al) launch_fwd<false, false>(ARGS);
+    else if (stream_hint(2 * M * N * (int64_t)sizeof(float))) launch_fwd<true, true>(ARGS);
+    else launch_fwd<true, false>(ARGS);
+#undef ARGS
     return launch_status();
 }
 
@@ -456,8 +456,9 @@ extern "C" int mi_layer_norm_bwd_dx_partial_dwdb(
         (float*)DW->ptr, DW->strides[1], (float*)DB->ptr, DB->strides[1], (const float*)X->ptr, \
         X->strides[1], (const float*)W->ptr, (const float*)Mean->ptr, (const float*)Rstd->ptr,  \
         (int)N, M, G, (int)S
-    if (al) launch_bwd<true>(ARGS);
-    else launch_bwd<false>(ARGS);
+    if (!al) launch_bwd<false, false>(ARGS);
+    else if (stream_hint(3 * M * N * (int64_t)sizeof(float))) launch_bwd<true, true>(ARGS);
+    else launch_bwd<true, false>(ARGS);
 #undef ARGS
     return launch_status();
 }

@@ -47,7 +47,7 @@ __global__ __launch_bounds__(kBlock) void transpose_kernel(const T* __restrict__
         const int64_t gi = m0 + vi * V, gj = n0 + j;
         if constexpr (VEC) {
             if (gi < m && gj < n) {
-                VT v = __builtin_nontemporal_load(reinterpret_cast<const VT*>(x + gi + gj * ldx));
+                VT v = ld_global<true>(reinterpret_cast<const VT*>(x + gi + gj * ldx));
 #pragma unroll
                 for (int q = 0; q < V; ++q) lds[(vi * V + q) * kPitch + j] = v[q];
             }
@@ -68,7 +68,7 @@ __global__ __launch_bounds__(kBlock) void transpose_kernel(const T* __restrict__
                 VT v;
 #pragma unroll
                 for (int q = 0; q < V; ++q) v[q] = lds[i * kPitch + vi * V + q];
-                __builtin_nontemporal_store(v, reinterpret_cast<VT*>(y + gj + gi * ldy));
+                st_global<true>(v, reinterpret_cast<VT*>(y + gj + gi * ldy));
             }
         } else {
 #pragma unroll
@@ -87,7 +87,7 @@ __global__ __launch_bounds__(kBlock) void transpose_kernel(const T* __restrict__
 // time decide how large the contiguous spans are that DRAM sees on each side).
 typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
 
-template <int TM, int TN>
+template <int TM, int TN, bool STREAM = true>
 __global__ __launch_bounds__(256) void transpose4_kernel(const unsigned* __restrict__ x, int64_t ldx,
                                                          unsigned* __restrict__ y, int64_t ldy, int64_t m,
                                                          int64_t n, int tiles_m, int tiles_n, int order) {
@@ -117,7 +117,7 @@ __global__ __launch_bounds__(256) void transpose4_kernel(const unsigned* __restr
         if (gm < m) {
 #pragma unroll
             for (int c = 0; c < 4; ++c)
-                if (gn + c < n) r[c] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(x + gm + (gn + c) * ldx));
+                if (gn + c < n) r[c] = ld_global<STREAM>(reinterpret_cast<const u32x4*>(x + gm + (gn + c) * ldx));
         }
 #pragma unroll
         for (int q = 0; q < 4; ++q) {
@@ -134,7 +134,7 @@ __global__ __launch_bounds__(256) void transpose4_kernel(const unsigned* __restr
         const int64_t gn = n0 + 4 * j4, gm = m0 + row;
         if (gn < n && gm < m) {
             u32x4 t = *reinterpret_cast<const u32x4*>(&lds[row * TN + 4 * (j4 ^ ((row >> 2) & (SLOTS - 1)))]);
-            __builtin_nontemporal_store(t, reinterpret_cast<u32x4*>(y + gn + gm * ldy));
+            st_global<STREAM>(t, reinterpret_cast<u32x4*>(y + gn + gm * ldy));
         }
     }
 }
@@ -165,7 +165,12 @@ int launch4(const mi_tile_array* x, const mi_tile_array* y, hipStream_t s) {
     else if (TM == 32 && TN == 256) { T4(32, 256); set_variant("transpose4_32x256_regmicro"); }
     else if (TM == 64 && TN == 256) { T4(64, 256); set_variant("transpose4_64x256_regmicro"); }
     else if (TM == 32 && TN == 128) { T4(32, 128); set_variant("transpose4_32x128_regmicro"); }
-    else if (TM == 64) { T4(64, 128); set_variant("transpose4_64x128_regmicro"); }
+    else if (TM == 64 && !stream_hint(2 * m * n * (int64_t)sizeof(unsigned))) {
+        hipLaunchKernelGGL((transpose4_kernel<64, 128, false>), dim3((unsigned)blocks), dim3(256), 0, s,
+                           (const unsigned*)x->ptr, x->strides[1], (unsigned*)y->ptr, y->strides[1], m, n,
+                           (int)tm_, (int)tn_, order);
+        set_variant("transpose4_64x128_regmicro_cached");
+    } else if (TM == 64) { T4(64, 128); set_variant("transpose4_64x128_regmicro"); }
     else { T4(128, 64); set_variant("transpose4_128x64_regmicro"); }
 #undef T4
     return launch_status();

@@ -70,7 +70,7 @@ constexpr int kBlock = 256;
 // Streaming kernel: block b owns UNROLL*kBlock consecutive 16-byte vectors.  All UNROLL
 // loads of a and of b are issued before the first add so that each lane keeps
 // 2*UNROLL*16 bytes in flight.
-template <typename T, int UNROLL>
+template <typename T, int UNROLL, bool STREAM>
 __global__ __launch_bounds__(kBlock) void vadd_vec_kernel(const T* __restrict__ a,
                                                           const T* __restrict__ b,
                                                           T* __restrict__ c, int64_t nvec) {
@@ -83,12 +83,12 @@ __global__ __launch_bounds__(kBlock) void vadd_vec_kernel(const T* __restrict__ 
     if (base + (int64_t)(UNROLL - 1) * kBlock < nvec) {
         V x[UNROLL], y[UNROLL];
 #pragma unroll
-        for (int u = 0; u < UNROLL; ++u) x[u] = __builtin_nontemporal_load(av + base + u * kBlock);
+        for (int u = 0; u < UNROLL; ++u) x[u] = ld_global<STREAM>(av + base + u * kBlock);
 #pragma unroll
-        for (int u = 0; u < UNROLL; ++u) y[u] = __builtin_nontemporal_load(bv + base + u * kBlock);
+        for (int u = 0; u < UNROLL; ++u) y[u] = ld_global<STREAM>(bv + base + u * kBlock);
 #pragma unroll
         for (int u = 0; u < UNROLL; ++u)
-            __builtin_nontemporal_store(VT::add(x[u], y[u]), cv + base + u * kBlock);
+            st_global<STREAM>(VT::add(x[u], y[u]), cv + base + u * kBlock);
     } else {
 #pragma unroll
         for (int u = 0; u < UNROLL; ++u) {
@@ -136,9 +136,15 @@ int launch_dense(const void* a, const void* b, void* c, int64_t n, hipStream_t s
     if (nvec > 0) {
         const int64_t blocks = cld(nvec, (int64_t)UNROLL * kBlock);
         if (blocks > 0x7fffffffLL) return MI_E_GRID;
-        hipLaunchKernelGGL((vadd_vec_kernel<T, UNROLL>), dim3((unsigned)blocks), dim3(kBlock), 0, s,
-                           (const T*)a, (const T*)b, (T*)c, nvec);
-        set_variant("vadd_vec16_nt_x4");
+        if (stream_hint(3 * n * (int64_t)sizeof(T))) {
+            hipLaunchKernelGGL((vadd_vec_kernel<T, UNROLL, true>), dim3((unsigned)blocks), dim3(kBlock), 0, s,
+                               (const T*)a, (const T*)b, (T*)c, nvec);
+            set_variant("vadd_vec16_nt_x4");
+        } else {
+            hipLaunchKernelGGL((vadd_vec_kernel<T, UNROLL, false>), dim3((unsigned)blocks), dim3(kBlock), 0, s,
+                               (const T*)a, (const T*)b, (T*)c, nvec);
+            set_variant("vadd_vec16_x4");
+        }
     }
     const int64_t done = nvec * N;
     if (done < n) {

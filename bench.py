@@ -288,21 +288,16 @@ def headline(ct, steps, warmup):
     SI, SO = ct.TileArray(ds.input), ct.TileArray(ds.output_tma)
     G = dl.GROUP_SIZE_M
 
-    def ln_fwd():
-        ct.layer_norm_fwd(D["X"], D["W"], D["B"], D["Y"], D["Mean"], D["Rstd"], dl.eps, 1024)
+    # Pre-bound launches (arguments converted once): at ~20 us per kernel the Python side of an
+    # ordinary wrapper call would be the bottleneck of the timed loop.
+    ln_fwd = ct.bind("mi_layer_norm_fwd", D["X"], D["W"], D["B"], D["Y"], D["Mean"], D["Rstd"], dl.eps, 1024)
+    ln_bwd_main = ct.bind("mi_layer_norm_bwd_dx_partial_dwdb", D["DX"], D["DY"], D["DW_partial"], D["DB_partial"],
+                          D["X"], D["W"], D["Mean"], D["Rstd"], D["Locks"], G, 1024)
+    ln_bwd_final = ct.bind("mi_layer_norm_bwd_dwdb", D["DW_partial"], D["DB_partial"], D["FINAL_DW"], D["FINAL_DB"], 32, 1024)
+    sm = ct.bind("mi_softmax_tma_kernel", SO, SI, 4096, ds.M)
 
-    def fills():
+    def fills():  # the host code's three fill! calls before every backward (layernorm.jl:245-247)
         dl.DW_partial.zero_(); dl.DB_partial.zero_(); dl.Locks.zero_()
-
-    def ln_bwd_main():
-        ct.layer_norm_bwd_dx_partial_dwdb(D["DX"], D["DY"], D["DW_partial"], D["DB_partial"], D["X"], D["W"], D["Mean"],
-                                          D["Rstd"], D["Locks"], G, 1024)
-
-    def ln_bwd_final():
-        ct.layer_norm_bwd_dwdb(D["DW_partial"], D["DB_partial"], D["FINAL_DW"], D["FINAL_DB"], 32, 1024)
-
-    def sm():
-        ct.softmax_tma_kernel(SO, SI, 4096, ds.M)
 
     stages = [("layer_norm_fwd", ln_fwd), ("fills", fills), ("layer_norm_bwd_dx_partial_dwdb", ln_bwd_main),
               ("layer_norm_bwd_dwdb", ln_bwd_final), ("softmax_tma_kernel", sm)]

@@ -154,6 +154,24 @@ def _call(name: str, *args):
         raise MiError(name, rc, strerror(rc))
 
 
+def bind(name: str, *args, stream=None):
+    """Pre-bound launch: converts the arguments of entry point ``name`` once (arrays to descriptors,
+    the stream handle) and returns a zero-argument callable that only makes the C call.  For
+    launch loops where Python's per-call argument handling would otherwise outweigh a 20 us
+    kernel.  ``args`` are the entry point's arguments without the trailing stream."""
+    fn = getattr(lib(), name)
+    keep = [a if isinstance(a, MiTileArray) or not hasattr(a, "data_ptr") else TileArray(a) for a in args]
+    cargs = tuple(ctypes.byref(a) if isinstance(a, MiTileArray) else (int(a) if isinstance(a, bool) else a)
+                  for a in keep) + (_stream(stream),)
+
+    def call():
+        rc = fn(*cargs)
+        if rc != 0:
+            raise MiError(name, rc, strerror(rc))
+    call._keep = keep
+    return call
+
+
 # ---- kernel wrappers: one per entry point, argument order of the reference kernels --------
 
 def vec_add_kernel_1d(a, b, c, tile: int, stream=None):

@@ -71,7 +71,7 @@ __device__ __forceinline__ void store_row(float* __restrict__ p, int N, const fl
             f32x4 t;
 #pragma unroll
             for (int q = 0; q < 4; ++q) t[q] = r[v][q];
-            st_global<NT>(t, reinterpret_cast<f32x4*>(p + e0));
+            st_global<true>(t, reinterpret_cast<f32x4*>(p + e0));
         } else {
 #pragma unroll
             for (int q = 0; q < 4; ++q)

@@ -102,7 +102,7 @@ __global__ __launch_bounds__(BLOCK) void softmax_regs_kernel(T* __restrict__ out
                 V raw;
 #pragma unroll
                 for (int q = 0; q < EV; ++q) vset<T>(raw, q, x[v][q] * rsum);
-                st_global<STREAM>(raw, reinterpret_cast<V*>(op + e0));
+                st_global<true>(raw, reinterpret_cast<V*>(op + e0));
             } else {
 #pragma unroll
                 for (int q = 0; q < EV; ++q)

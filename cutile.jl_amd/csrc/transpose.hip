@@ -134,7 +134,7 @@ __global__ __launch_bounds__(256) void transpose4_kernel(const unsigned* __restr
         const int64_t gn = n0 + 4 * j4, gm = m0 + row;
         if (gn < n && gm < m) {
             u32x4 t = *reinterpret_cast<const u32x4*>(&lds[row * TN + 4 * (j4 ^ ((row >> 2) & (SLOTS - 1)))]);
-            st_global<STREAM>(t, reinterpret_cast<u32x4*>(y + gn + gm * ldy));
+            st_global<true>(t, reinterpret_cast<u32x4*>(y + gn + gm * ldy));
         }
     }
 }

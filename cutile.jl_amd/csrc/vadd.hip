@@ -88,7 +88,7 @@ __global__ __launch_bounds__(kBlock) void vadd_vec_kernel(const T* __restrict__ 
         for (int u = 0; u < UNROLL; ++u) y[u] = ld_global<STREAM>(bv + base + u * kBlock);
 #pragma unroll
         for (int u = 0; u < UNROLL; ++u)
-            st_global<STREAM>(VT::add(x[u], y[u]), cv + base + u * kBlock);
+            st_global<true>(VT::add(x[u], y[u]), cv + base + u * kBlock);
     } else {
 #pragma unroll
         for (int u = 0; u < UNROLL; ++u) {

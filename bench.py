@@ -133,7 +133,7 @@ def bench_kernels(ct, which, cpu, nruns=NRUNS, warmup=WARMUP):
                 ct.layer_norm_fwd(D["X"], D["W"], D["B"], D["Y"], D["Mean"], D["Rstd"], d.eps, 1024)
 
             def bwd():
-                d.DW_partial.zero_(); d.DB_partial.zero_(); d.Locks.zero_()
+                d.partials.zero_()
                 ct.layer_norm_bwd_dx_partial_dwdb(D["DX"], D["DY"], D["DW_partial"], D["DB_partial"], D["X"], D["W"],
                                                   D["Mean"], D["Rstd"], D["Locks"], G, 1024)
                 ct.layer_norm_bwd_dwdb(D["DW_partial"], D["DB_partial"], D["FINAL_DW"], D["FINAL_DB"], 32, 1024)
@@ -145,7 +145,7 @@ def bench_kernels(ct, which, cpu, nruns=NRUNS, warmup=WARMUP):
                                               "f32", nruns, warmup, {"reference_formula_bytes": 4 * MN4})
                 fwd(); res["layernorm_fwd"]["variant"] = ct.last_variant()
             key = "layernorm_bwd" if G == 64 else "layernorm_bwd_G256"
-            res[key] = _entry(f"LayerNorm bwd 4096^2 f32, GROUP_SIZE_M={G} (3 fills + 2 kernels)", bwd, bwd_bytes,
+            res[key] = _entry(f"LayerNorm bwd 4096^2 f32, GROUP_SIZE_M={G} (1 fill + 2 kernels)", bwd, bwd_bytes,
                               "GB/s", "hbm", HBM_PEAK_GBS, "f32", nruns, warmup, {"reference_formula_bytes": 5 * MN4})
             if cpu and G == 64:
                 X, W, B, DY = (orc.to_julia(t) for t in (d.X, d.W, d.B, d.DY))
@@ -244,7 +244,7 @@ def bench_kernels(ct, which, cpu, nruns=NRUNS, warmup=WARMUP):
             g, gout = graph_of(dev)
             g.replay(); torch.cuda.synchronize()
             assert torch.equal(gout, ref_out), "graph replay differs from eager"
-            res["moe_f16_device"] = extra(_entry("MoE f16 top-2, device work only (3 zero-fills + 4 kernels, HIP graph replay)",
+            res["moe_f16_device"] = extra(_entry("MoE f16 top-2, device work only (1 zero-fill + 4 kernels, HIP graph replay)",
                                                  g.replay, wbytes, "GB/s", "hbm", HBM_PEAK_GBS, "f16", nruns, warmup))
         except Exception as ex:  # graph capture unavailable: fall back to eager launches
             res["moe_f16_device"] = extra(_entry(f"MoE f16 top-2, device work only (eager; graph failed: {type(ex).__name__})",
@@ -296,8 +296,8 @@ def headline(ct, steps, warmup):
     ln_bwd_final = ct.bind("mi_layer_norm_bwd_dwdb", D["DW_partial"], D["DB_partial"], D["FINAL_DW"], D["FINAL_DB"], 32, 1024)
     sm = ct.bind("mi_softmax_tma_kernel", SO, SI, 4096, ds.M)
 
-    def fills():  # the host code's three fill! calls before every backward (layernorm.jl:245-247)
-        dl.DW_partial.zero_(); dl.DB_partial.zero_(); dl.Locks.zero_()
+    def fills():  # the host code's fill! of the partials before every backward (layernorm.jl:245-246), one launch
+        dl.partials.zero_()
 
     stages = [("layer_norm_fwd", ln_fwd), ("fills", fills), ("layer_norm_bwd_dx_partial_dwdb", ln_bwd_main),
               ("layer_norm_bwd_dwdb", ln_bwd_final), ("softmax_tma_kernel", sm)]

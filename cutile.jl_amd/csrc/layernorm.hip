@@ -238,6 +238,123 @@ __global__ __launch_bounds__(BLOCK) void ln_bwd_kernel(float* __restrict__ DX, i
     }
 }
 
+// Backward with two row groups per workgroup (512 lanes for rows of up to 4096 elements, 16-byte
+// aligned): the halves of the workgroup walk different rows of the same partial slot and add
+// their dW/dB partials in LDS before the flush, which halves the number of memory-side float
+// atomics -- the scarce resource of this kernel -- at the same number of rows in flight.
+// Workgroup (g, s): group h handles rows m = g + G*(2*s + h), stepping by 2*G*S.
+template <int VPT, bool STREAM>
+__global__ __launch_bounds__(512) void ln_bwd_rg2_kernel(float* __restrict__ DX, int64_t lddx,
+                                                         const float* __restrict__ DY, int64_t lddy,
+                                                         float* __restrict__ DW, int64_t lddw,
+                                                         float* __restrict__ DB, int64_t lddb,
+                                                         const float* __restrict__ X, int64_t ldx,
+                                                         const float* __restrict__ W,
+                                                         const float* __restrict__ Mean,
+                                                         const float* __restrict__ Rstd, int N,
+                                                         int64_t M, int G, int S) {
+    constexpr int BLOCK = 256, NW = 4;
+    __shared__ float red[2][2 * NW];
+    __shared__ float stage[BLOCK * VPT * 4];
+    const int g = blockIdx.x % G, s = blockIdx.x / G;
+    const int h = threadIdx.x >> 8, lt = threadIdx.x & 255, lane = lt & 63, wave = lt >> 6;
+    auto vec = [&](int v) { return (lt + v * BLOCK) * 4; };
+    float w[VPT][4], dw[VPT][4], db[VPT][4];
+#pragma unroll
+    for (int v = 0; v < VPT; ++v) {
+        const f32x4 t = vec(v) < N ? *reinterpret_cast<const f32x4*>(W + vec(v)) : f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+            w[v][q] = t[q];
+            dw[v][q] = db[v][q] = 0.f;
+        }
+    }
+    const int64_t step = (int64_t)2 * G * S, m0 = g + (int64_t)G * (2 * s + h);
+    const int64_t trips = (M - (g + (int64_t)G * 2 * s) + step - 1) / step;  // of group 0; group 1 may idle in the last
+    for (int64_t it = 0; it < trips; ++it) {
+        const int64_t m = m0 + it * step;
+        const bool live = m < M;  // uniform per group; both groups keep meeting at the barriers
+        float x[VPT][4], dy[VPT][4];
+#pragma unroll
+        for (int v = 0; v < VPT; ++v) {
+            f32x4 tx = {0.f, 0.f, 0.f, 0.f}, ty = tx;
+            if (live && vec(v) < N) {
+                tx = ld_global<STREAM>(reinterpret_cast<const f32x4*>(X + m * ldx + vec(v)));
+                ty = ld_global<STREAM>(reinterpret_cast<const f32x4*>(DY + m * lddy + vec(v)));
+            }
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                x[v][q] = tx[q];
+                dy[v][q] = ty[q];
+            }
+        }
+        const float mean = live ? Mean[m] : 0.f, rstd = live ? Rstd[m] : 0.f;
+        float c1 = 0.f, c2 = 0.f;
+#pragma unroll
+        for (int v = 0; v < VPT; ++v) {
+            const bool in = vec(v) < N;  // N % 4 == 0 here
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                const float xhat = in ? (x[v][q] - mean) * rstd : 0.f;
+                const float wdy = w[v][q] * dy[v][q];
+                x[v][q] = xhat;
+                c1 += xhat * wdy;
+                c2 += wdy;
+            }
+        }
+        c1 = wave_reduce(c1, SumOp{});
+        c2 = wave_reduce(c2, SumOp{});
+        if (lane == 0) {
+            red[h][wave] = c1;
+            red[h][NW + wave] = c2;
+        }
+        __syncthreads();
+        c1 = (red[h][0] + red[h][1]) + (red[h][2] + red[h][3]);
+        c2 = (red[h][NW] + red[h][NW + 1]) + (red[h][NW + 2] + red[h][NW + 3]);
+        __syncthreads();
+        c1 /= (float)N;
+        c2 /= (float)N;
+#pragma unroll
+        for (int v = 0; v < VPT; ++v) {
+            f32x4 t;
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                const float xhat = x[v][q], wdy = w[v][q] * dy[v][q];
+                dw[v][q] += dy[v][q] * xhat;
+                db[v][q] += dy[v][q];
+                t[q] = (wdy - (xhat * c1 + c2)) * rstd;
+            }
+            if (live && vec(v) < N) st_global<true>(t, reinterpret_cast<f32x4*>(DX + m * lddx + vec(v)));
+        }
+    }
+    // group 1 hands its partials to group 0 through LDS; group 0 flushes with coalesced atomics
+    float* dwp = DW + (int64_t)g * lddw;
+    float* dbp = DB + (int64_t)g * lddb;
+#pragma unroll
+    for (int pass = 0; pass < 2; ++pass) {
+        if (h == 1) {
+#pragma unroll
+            for (int v = 0; v < VPT; ++v)
+#pragma unroll
+                for (int q = 0; q < 4; ++q) stage[vec(v) + q] = pass == 0 ? dw[v][q] : db[v][q];
+        }
+        __syncthreads();
+        if (h == 0) {
+#pragma unroll
+            for (int v = 0; v < VPT; ++v)
+#pragma unroll
+                for (int q = 0; q < 4; ++q) stage[vec(v) + q] += pass == 0 ? dw[v][q] : db[v][q];
+        }
+        __syncthreads();
+        float* dst = pass == 0 ? dwp : dbp;
+        for (int c = threadIdx.x; c < N; c += 512) {
+            if (S == 1) dst[c] += stage[c];
+            else unsafeAtomicAdd(dst + c, stage[c]);
+        }
+        __syncthreads();
+    }
+}
+
 // Backward for rows longer than the register-cached variants hold.
 template <int BLOCK>
 __global__ __launch_bounds__(BLOCK) void ln_bwd_long_kernel(float* __restrict__ DX, int64_t lddx,
@@ -456,8 +573,23 @@ extern "C" int mi_layer_norm_bwd_dx_partial_dwdb(
         (float*)DW->ptr, DW->strides[1], (float*)DB->ptr, DB->strides[1], (const float*)X->ptr, \
         X->strides[1], (const float*)W->ptr, (const float*)Mean->ptr, (const float*)Rstd->ptr,  \
         (int)N, M, G, (int)S
-    if (!al) launch_bwd<false, false>(ARGS);
-    else if (stream_hint(3 * M * N * (int64_t)sizeof(float))) launch_bwd<true, true>(ARGS);
+    const bool stream_in = stream_hint(3 * M * N * (int64_t)sizeof(float));
+    static const bool no_rg2 = [] { const char* e = getenv("MI_LN_BWD_RG"); return e && e[0] == '1'; }();
+    if (al && N % 4 == 0 && vecs > 512 && vecs <= 1024 && S % 2 == 0 && !no_rg2) {
+        // two row groups per workgroup: same rows in flight, half the atomics
+        const int S2 = (int)S / 2;
+        dim3 grid2((unsigned)(G * S2));
+#define RG2(ST)                                                                                              \
+    hipLaunchKernelGGL((ln_bwd_rg2_kernel<4, ST>), grid2, dim3(512), 0, s, (float*)DX->ptr, DX->strides[1],    \
+                       (const float*)DY->ptr, DY->strides[1], (float*)DW->ptr, DW->strides[1], (float*)DB->ptr, \
+                       DB->strides[1], (const float*)X->ptr, X->strides[1], (const float*)W->ptr,               \
+                       (const float*)Mean->ptr, (const float*)Rstd->ptr, (int)N, M, G, S2)
+        if (stream_in) RG2(true);
+        else RG2(false);
+#undef RG2
+        set_variant("ln_bwd_regs_b512_v4_rg2");
+    } else if (!al) launch_bwd<false, false>(ARGS);
+    else if (stream_in) launch_bwd<true, true>(ARGS);
     else launch_bwd<true, false>(ARGS);
 #undef ARGS
     return launch_status();

@@ -238,13 +238,17 @@ def bench_kernels(ct, which, cpu, nruns=NRUNS, warmup=WARMUP):
         whole = lambda: moe.cutile_moe(d.hidden_states, d.w1, d.w2, d.topk_weights, d.topk_ids, 128, 128, 64)
         res["moe_f16"] = extra(_entry("MoE f16 256tok/1024h/32e/2048i top-2, whole cutile_moe (host align + H2D/D2H inside)",
                                       whole, wbytes, "GB/s", "hbm", HBM_PEAK_GBS, "f16", nruns, warmup))
-        dev = lambda: moe.cutile_moe(d.hidden_states, d.w1, d.w2, d.topk_weights, d.topk_ids, 128, 128, 64, aligned=al)
+        whole_dev = lambda: moe.cutile_moe(d.hidden_states, d.w1, d.w2, d.topk_weights, d.topk_ids, 128, 128, 64,
+                                           device_align=True)
+        res["moe_f16_device_align"] = extra(_entry("MoE f16 top-2, whole cutile_moe with the token sort on the GPU (no host round trip; eager launches)",
+                                                   whole_dev, wbytes, "GB/s", "hbm", HBM_PEAK_GBS, "f16", nruns, warmup))
+        dev = whole_dev
         ref_out = dev()
         try:
             g, gout = graph_of(dev)
             g.replay(); torch.cuda.synchronize()
             assert torch.equal(gout, ref_out), "graph replay differs from eager"
-            res["moe_f16_device"] = extra(_entry("MoE f16 top-2, device work only (1 zero-fill + 4 kernels, HIP graph replay)",
+            res["moe_f16_device"] = extra(_entry("MoE f16 top-2, whole cutile_moe on the device (zero-fill + token sort + 4 kernels), HIP graph replay",
                                                  g.replay, wbytes, "GB/s", "hbm", HBM_PEAK_GBS, "f16", nruns, warmup))
         except Exception as ex:  # graph capture unavailable: fall back to eager launches
             res["moe_f16_device"] = extra(_entry(f"MoE f16 top-2, device work only (eager; graph failed: {type(ex).__name__})",
@@ -262,11 +266,11 @@ def bench_kernels(ct, which, cpu, nruns=NRUNS, warmup=WARMUP):
         s1t, s2t = orc.from_julia(s1).cuda(), orc.from_julia(s2).cuda()
         w8bytes = c1.size + c2.size + (s1.size + s2.size) * 4 + 2 * d.hidden_states.numel() * 2
         dev8 = lambda: moe.cutile_moe(d.hidden_states, w1q, w2q, d.topk_weights, d.topk_ids, 128, 128, 64, w1_scale=s1t,
-                                      w2_scale=s2t, aligned=al)
+                                      w2_scale=s2t, device_align=True)
         dev8()
         try:
             g8, _ = graph_of(dev8)
-            res["moe_fp8_device"] = extra(_entry("MoE e4m3 weights top-2, device work only (HIP graph replay)", g8.replay,
+            res["moe_fp8_device"] = extra(_entry("MoE e4m3 weights top-2, whole cutile_moe on the device, HIP graph replay", g8.replay,
                                                  w8bytes, "GB/s", "hbm", HBM_PEAK_GBS, "fp8 weights / f16 MFMA", nruns, warmup))
         except Exception as ex:
             res["moe_fp8_device"] = extra(_entry(f"MoE e4m3 weights top-2, device work only (eager; {type(ex).__name__})", dev8,

@@ -69,6 +69,7 @@ _SIGNATURES = {
     "mi_softmax_tma_kernel": ([_A, _A, _i, _i, _vp], _i),
     "mi_softmax_chunked_kernel": ([_A, _A, _i, _i, _i, _vp], _i),
     "mi_fmha_kernel": ([_A, _A, _A, _A, ctypes.c_float, ctypes.c_int32, _i, _i, _i, _i, _i, _i, _i, _vp], _i),
+    "mi_moe_align_tile_size_device": ([_A, _i, _i, _A, _A, _vp], _i),
     "mi_moe_align_tile_size": (
         [ctypes.POINTER(ctypes.c_int64), ctypes.c_int64, ctypes.c_int64, _i, _i,
          ctypes.POINTER(ctypes.c_int32), ctypes.POINTER(ctypes.c_int32),
@@ -272,6 +273,30 @@ def moe_align_tile_size(topk_ids, tile_m: int, num_experts: int):
           ctypes.cast(tok.data_ptr(), ctypes.POINTER(ctypes.c_int32)),
           ctypes.cast(exp.data_ptr(), ctypes.POINTER(ctypes.c_int32)), ctypes.byref(nblk))
     return tok, exp
+
+
+def moe_align_capacity(num_tokens: int, topk: int, tile_m: int, num_experts: int):
+    """(blocks, slots) that always hold the result of ``moe_align_tile_size`` for these sizes."""
+    total = num_tokens * topk
+    blocks = -(-(total + min(total, num_experts) * (tile_m - 1)) // tile_m)
+    return blocks, blocks * tile_m
+
+
+def moe_align_tile_size_device(topk_ids, tile_m: int, num_experts: int, sorted_token_ids=None,
+                               sorted_expert_ids=None, stream=None):
+    """On-device ``moe_align_tile_size`` (no host round trip).  ``topk_ids``: device int64 tensor
+    of torch shape (topk, num_tokens).  Returns device int32 tensors of fixed capacity
+    (``moe_align_capacity``); unused slots hold the sentinel, unused blocks expert 0."""
+    import torch
+    topk, num_tokens = topk_ids.shape
+    blocks, slots = moe_align_capacity(num_tokens, topk, tile_m, num_experts)
+    if sorted_token_ids is None:
+        sorted_token_ids = torch.empty(slots, dtype=torch.int32, device=topk_ids.device)
+    if sorted_expert_ids is None:
+        sorted_expert_ids = torch.empty(blocks, dtype=torch.int32, device=topk_ids.device)
+    _call("mi_moe_align_tile_size_device", _ref(topk_ids), tile_m, num_experts, _ref(sorted_token_ids),
+          _ref(sorted_expert_ids), _stream(stream))
+    return sorted_token_ids, sorted_expert_ids
 
 
 def fused_moe_kernel(A, B, C, topk_weights, sorted_token_ids, sorted_expert_ids,

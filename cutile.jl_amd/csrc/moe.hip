@@ -372,6 +372,111 @@ extern "C" int mi_fused_moe_kernel(const mi_tile_array* A, const mi_tile_array* 
     return launch_status();
 }
 
+// ---- on-device moe_align_tile_size ------------------------------------------------------------
+// One workgroup of four waves.  Counting sort by expert of the replica ids (slot-fastest
+// flattening of topk_ids, examples/moe.jl:148-150): LDS histogram, serial scan over the experts,
+// then placement in super-blocks of 256 consecutive replicas.  A replica's slot is
+//     cursor[e] + (replicas of e in earlier waves of the super-block) + (those in earlier lanes),
+// the last term from ballots alone, so ids of one expert ascend exactly as the stable sortperm
+// of moe.jl:150 orders them.  The outputs have fixed capacity: unused slots hold the sentinel
+// total+1, unused blocks expert 0, which the GEMM kernel skips.
+constexpr int kAlignMaxExperts = 1024;
+__global__ __launch_bounds__(256) void moe_align_kernel(const long long* __restrict__ topk_ids, int64_t ld_slot,
+                                                        int num_tokens, int topk, int tile_m, int num_experts,
+                                                        int* __restrict__ sorted_token_ids, int cap_slots,
+                                                        int* __restrict__ sorted_expert_ids, int cap_blocks) {
+    __shared__ int cursor[kAlignMaxExperts];      // histogram, then next free slot of every expert
+    __shared__ int tbl[4][kAlignMaxExperts];      // replicas per (wave, expert) of the current super-block
+    __shared__ int s_blocks;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, total = num_tokens * topk;
+    for (int e = tid; e < num_experts; e += 256) {
+        cursor[e] = 0;
+        tbl[0][e] = tbl[1][e] = tbl[2][e] = tbl[3][e] = 0;
+    }
+    for (int i = tid; i < cap_slots; i += 256) sorted_token_ids[i] = total + 1;
+    __syncthreads();
+    for (int r = tid; r < total; r += 256) {
+        const long long e = topk_ids[(r / topk) + (int64_t)(r % topk) * ld_slot];
+        if (e >= 1 && e <= num_experts) atomicAdd(&cursor[(int)e - 1], 1);
+    }
+    __syncthreads();
+    if (tid == 0) {
+        int blk = 0;
+        for (int e = 0; e < num_experts; ++e) {
+            const int nb = (cursor[e] + tile_m - 1) / tile_m;
+            cursor[e] = blk * tile_m;  // first slot of the expert
+            for (int b = 0; b < nb && blk < cap_blocks; ++b) sorted_expert_ids[blk++] = e + 1;
+        }
+        s_blocks = blk;
+    }
+    __syncthreads();
+    for (int b = s_blocks + tid; b < cap_blocks; b += 256) sorted_expert_ids[b] = 0;
+
+    const unsigned long long lt = lane ? (~0ull >> (64 - lane)) : 0ull;
+    for (int r0 = 0; r0 < total; r0 += 256) {
+        const int r = r0 + tid;
+        int e = -1;
+        if (r < total) {
+            const long long v = topk_ids[(r / topk) + (int64_t)(r % topk) * ld_slot];
+            if (v >= 1 && v <= num_experts) e = (int)v - 1;
+        }
+        int rank = 0;
+        unsigned long long todo = __ballot(e >= 0);
+        while (todo) {  // one trip per distinct expert of the wave's 64 replicas
+            const int leader = __ffsll((long long)todo) - 1;
+            const int el = __shfl(e, leader, 64);
+            const unsigned long long m = __ballot(e == el);
+            if (e == el) rank = __popcll(m & lt);
+            if (lane == leader) tbl[wave][el] = __popcll(m);
+            todo &= ~m;
+        }
+        __syncthreads();
+        if (e >= 0) {
+            int pos = cursor[e] + rank;
+            for (int w = 0; w < wave; ++w) pos += tbl[w][e];
+            if (pos < cap_slots) sorted_token_ids[pos] = r + 1;
+        }
+        __syncthreads();
+        // advance the cursors and clear the table: the entries touched are those of this super-block's experts
+        if (e >= 0 && rank == 0) {  // first lane of its expert within the wave
+            atomicAdd(&cursor[e], tbl[wave][e]);
+        }
+        __syncthreads();
+        if (e >= 0 && rank == 0) tbl[wave][e] = 0;
+        __syncthreads();
+    }
+}
+
+extern "C" int mi_moe_align_tile_size_device(const mi_tile_array* topk_ids, int tile_m, int num_experts,
+                                             const mi_tile_array* sorted_token_ids,
+                                             const mi_tile_array* sorted_expert_ids, void* stream) {
+    MI_CHECK(check_array(topk_ids, 2));
+    MI_CHECK(check_array(sorted_token_ids, 1));
+    MI_CHECK(check_array(sorted_expert_ids, 1));
+    if (topk_ids->dtype != MI_I64 || sorted_token_ids->dtype != MI_I32 || sorted_expert_ids->dtype != MI_I32)
+        return MI_E_DTYPE;
+    if (!is_pow2(tile_m)) return MI_E_TILE;
+    if (num_experts < 1) return MI_E_ARG;
+    if (num_experts > kAlignMaxExperts) return MI_E_UNSUPPORTED;
+    const int64_t num_tokens = topk_ids->sizes[0], topk = topk_ids->sizes[1], total = num_tokens * topk;
+    if (total > (1 << 22)) return MI_E_UNSUPPORTED;  // one workgroup sorts; larger batches use the host routine
+    if (num_tokens > 1 && topk_ids->strides[0] != 1) return MI_E_STRIDE;
+    const int64_t cap_blocks = sorted_expert_ids->sizes[0], cap_slots = sorted_token_ids->sizes[0];
+    // worst case: every expert's last block is one replica short of empty
+    const int64_t used = total < num_experts ? total : (int64_t)num_experts;
+    const int64_t need_blocks = cld(total + used * (tile_m - 1), (int64_t)tile_m);
+    if (cap_blocks < need_blocks || cap_slots < cap_blocks * tile_m) return MI_E_SHAPE;
+    if ((cap_slots > 1 && sorted_token_ids->strides[0] != 1) || (cap_blocks > 1 && sorted_expert_ids->strides[0] != 1))
+        return MI_E_STRIDE;
+    if (cap_slots > 0x7fffffff) return MI_E_SHAPE;
+    if (cap_blocks == 0) return MI_OK;
+    hipLaunchKernelGGL(moe_align_kernel, dim3(1), dim3(256), 0, (hipStream_t)stream, (const long long*)topk_ids->ptr,
+                       topk > 1 ? topk_ids->strides[1] : 0, (int)num_tokens, (int)topk, tile_m, num_experts,
+                       (int*)sorted_token_ids->ptr, (int)cap_slots, (int*)sorted_expert_ids->ptr, (int)cap_blocks);
+    set_variant("moe_align_device_1wg");
+    return launch_status();
+}
+
 extern "C" int mi_silu_and_mul_kernel(const mi_tile_array* A, const mi_tile_array* B, const mi_tile_array* C,
                                       int TILE_N, void* stream) {
     MI_CHECK(check_array(A, 2));

@@ -29,11 +29,12 @@ def invoke_silu_and_mul_kernel(AB, C):
 
 
 def cutile_moe(hidden_states, w1, w2, topk_weights, topk_ids, tile_m, tile_n, tile_k, *, w1_scale=None,
-               w2_scale=None, aligned=None):
+               w2_scale=None, aligned=None, device_align=False):
     """moe.jl:218-257.  Torch shapes (reversed Julia): hidden_states (tokens, hidden); w1
     (E, 2*inter, hidden); w2 (E, hidden, inter); topk_weights / topk_ids (topk, tokens), ids
     1-based int64.  ``aligned`` may carry a precomputed (sorted_token_ids, sorted_expert_ids)
-    pair on the device to skip the host round trip of moe.jl:232-233."""
+    pair on the device to skip the host round trip of moe.jl:232-233; ``device_align`` sorts on
+    the GPU instead (fixed-capacity outputs, nothing leaves the device)."""
     num_tokens, hidden_size = hidden_states.shape
     num_experts, _, intermediate_size = w2.shape
     topk = topk_ids.shape[0]
@@ -46,7 +47,9 @@ def cutile_moe(hidden_states, w1, w2, topk_weights, topk_ids, tile_m, tile_n, ti
     cache1 = caches[:n1].view(num_tokens, topk, intermediate_size * 2)
     cache2 = caches[n1:n1 + n2].view(total_tokens, intermediate_size)
     cache3 = caches[n1 + n2:].view(num_tokens, topk, hidden_size)
-    if aligned is None:
+    if aligned is None and device_align:
+        sorted_token_ids, sorted_expert_ids = ct.moe_align_tile_size_device(topk_ids, tile_m, num_experts)
+    elif aligned is None:
         tok, exp = ct.moe_align_tile_size(topk_ids.cpu(), tile_m, num_experts)
         sorted_token_ids, sorted_expert_ids = tok.to(dev), exp.to(dev)
     else:

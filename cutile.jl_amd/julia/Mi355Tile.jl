@@ -226,6 +226,18 @@ function moe_align_tile_size(topk_ids::Matrix{Int64}, tile_m::Integer, num_exper
     return ids, experts
 end
 
+"Device counterpart: `topk_ids` (num_tokens, topk) Int64 on the device; fills the fixed-capacity
+device vectors `sorted_token_ids` (Int32, `tile_m` per block) and `sorted_expert_ids` (Int32, at least
+cld(total + min(total, num_experts)*(tile_m-1), tile_m) blocks).  Unused blocks get expert 0."
+function moe_align_tile_size_device(topk_ids, tile_m::Integer, num_experts::Integer,
+                                    sorted_token_ids, sorted_expert_ids; stream::Ptr{Cvoid}=C_NULL)
+    d = map(a -> ref(descriptor(a)), (topk_ids, sorted_token_ids, sorted_expert_ids))
+    GC.@preserve topk_ids sorted_token_ids sorted_expert_ids check(ccall(
+        (:mi_moe_align_tile_size_device, libmi355tile), Cint,
+        (Ref{MiTileArray}, Cint, Cint, Ref{MiTileArray}, Ref{MiTileArray}, Ptr{Cvoid}),
+        d[1], tile_m, num_experts, d[2], d[3], stream))
+end
+
 # `b_scale` (N, E) Float32 goes with e4m3fn weights only; `nothing` otherwise.
 function fused_moe_kernel(A, B, C, topk_weights, sorted_token_ids, sorted_expert_ids,
                           num_token_replicas::Integer, mul_routed_weight::Bool,

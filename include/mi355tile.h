@@ -171,6 +171,18 @@ int mi_fmha_kernel(const mi_tile_array* Q, const mi_tile_array* K, const mi_tile
 int mi_moe_align_tile_size(const int64_t* topk_ids, int64_t num_tokens, int64_t topk, int tile_m,
                            int num_experts, int32_t* sorted_token_ids_out,
                            int32_t* sorted_expert_ids_out, int64_t* total_blocks_out);
+/* Device counterpart of moe_align_tile_size: the same stable counting sort, run by one workgroup
+ * on `stream`, so that cutile_moe needs no host round trip (the reference copies topk_ids to the
+ * host, sorts there and copies the result back: moe.jl:232-233).  topk_ids (num_tokens, topk)
+ * i64 on the device.  The outputs have fixed capacity, since the block count is only known on
+ * the device: sorted_expert_ids needs at least
+ * cld(total + min(total, num_experts)*(tile_m-1), tile_m) entries and sorted_token_ids
+ * tile_m times as many; unused slots get the sentinel total+1 and unused blocks expert 0, which
+ * mi_fused_moe_kernel skips.  Expert ids outside 1..num_experts are dropped (the host routine
+ * reports MI_E_ARG for them).  At most 1024 experts and 2^22 replicas. */
+int mi_moe_align_tile_size_device(const mi_tile_array* topk_ids, int tile_m, int num_experts,
+                                  const mi_tile_array* sorted_token_ids,
+                                  const mi_tile_array* sorted_expert_ids, void* stream);
 /* fused_moe_kernel (moe.jl:45-105).  A (K,num_tokens), B (K,N,E), C (N,total_tokens),
  * topk_weights (total_tokens,), sorted_token_ids (M_padded,) i32 1-based with sentinel
  * total_tokens+1, sorted_expert_ids (blocks,) i32 1-based.  A, C, topk_weights f16/bf16.

@@ -137,3 +137,36 @@ def test_moe_full_size_top2(orc):
     J = orc.to_julia
     ref = orc.ref_moe(J(d.hidden_states), J(d.w1), J(d.w2), J(d.topk_weights), J(d.topk_ids), dtype=np.float32)
     check(J(r.out), ref.astype(np.float64))
+
+
+@pytest.mark.parametrize("num_tokens,topk,E,tile_m", [(256, 2, 32, 128), (48, 8, 64, 16), (7, 3, 5, 4), (1, 1, 1, 128),
+                                                      (1000, 4, 9, 32), (130, 2, 1000, 8)])
+def test_device_align_matches_host_routine(ct, orc, num_tokens, topk, E, tile_m):
+    """The one-workgroup counting sort gives the host routine's arrays (stable per-expert order,
+    sentinel padding) in the leading part of its fixed-capacity outputs, and marks the rest unused."""
+    rng = np.random.default_rng(num_tokens + topk)
+    ids = rng.integers(1, E + 1, size=(topk, num_tokens), dtype=np.int64)   # torch layout of Julia (tokens, topk)
+    ids_t = torch.from_numpy(ids)
+    tok_h, exp_h = ct.moe_align_tile_size(ids_t, tile_m, E)
+    tok_d, exp_d = ct.moe_align_tile_size_device(ids_t.cuda(), tile_m, E)
+    nb = exp_h.numel()
+    blocks, slots = ct.moe_align_capacity(num_tokens, topk, tile_m, E)
+    assert tok_d.numel() == slots and exp_d.numel() == blocks and nb <= blocks
+    assert torch.equal(exp_d[:nb].cpu(), exp_h) and torch.all(exp_d[nb:] == 0)
+    assert torch.equal(tok_d[:nb * tile_m].cpu(), tok_h) and torch.all(tok_d[nb * tile_m:] == num_tokens * topk + 1)
+    # oracle as a third opinion
+    tok_o, exp_o = orc.moe_align_tile_size(ids.T, tile_m, E)
+    assert np.array_equal(tok_h.numpy(), tok_o) and np.array_equal(exp_h.numpy(), exp_o)
+
+
+def test_moe_end_to_end_with_device_align(orc):
+    """cutile_moe with the sort on the GPU equals the version that sorts on the host, bit for bit
+    (the extra, unused blocks change nothing)."""
+    d = moe.prepare(benchmark=True, topk=2, router="top2_logits")
+    a = moe.cutile_moe(d.hidden_states, d.w1, d.w2, d.topk_weights, d.topk_ids, 128, 128, 64)
+    b = moe.cutile_moe(d.hidden_states, d.w1, d.w2, d.topk_weights, d.topk_ids, 128, 128, 64, device_align=True)
+    assert torch.equal(a, b)
+    d = moe.prepare(num_tokens=33, hidden_size=256, num_experts=7, intermediate_size=128, topk=3)
+    a = moe.cutile_moe(d.hidden_states, d.w1, d.w2, d.topk_weights, d.topk_ids, 16, 128, 64)
+    b = moe.cutile_moe(d.hidden_states, d.w1, d.w2, d.topk_weights, d.topk_ids, 16, 128, 64, device_align=True)
+    assert torch.equal(a, b)

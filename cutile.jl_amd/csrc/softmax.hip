@@ -5,8 +5,9 @@
 // column at a time.  The single-tile kernel keeps the whole column in registers, so HBM is
 // touched exactly once per element each way (algorithmic traffic 2*M*N*sizeof(T)): 16-byte
 // loads, wave64 shuffle reductions, one LDS exchange per reduction across the waves of the
-// workgroup.  The chunked kernel makes the reference's three passes over the column (max,
-// denominator, normalise); passes two and three re-read the column from L2.
+// workgroup.  Columns too long for that (more than 16384 elements per 256 lanes' registers) take
+// the reference's three passes (max, denominator, normalise), re-reading the column from L2;
+// softmax_chunked_kernel uses the register kernel too whenever its column fits.
 //
 // Numerics follow the reference: fp32 math, max ignores NaN, full-precision exp (not
 // exp2), IEEE division, padding rows read as -Inf and are never written.
@@ -206,11 +207,11 @@ int launch_3pass(const mi_tile_array* output, const mi_tile_array* input, int64_
     return launch_status();
 }
 
+// Softmax over the first L64 rows of every column: the register kernel when the column fits
+// (one HBM pass), otherwise three passes.
 template <typename T>
-int launch_tma(const mi_tile_array* output, const mi_tile_array* input, int TILE_SIZE, hipStream_t s) {
+int launch_len(const mi_tile_array* output, const mi_tile_array* input, int64_t L64, hipStream_t s) {
     constexpr int EV = Raw<T>::EV;
-    const int64_t N = input->sizes[0];
-    const int64_t L64 = N < TILE_SIZE ? N : (int64_t)TILE_SIZE;
     if (L64 > 256 * 16 * EV) return launch_3pass<T>(output, input, L64, s);
     const int L = (int)L64;
     const bool al = vec_ok<T>(output, input);
@@ -233,10 +234,11 @@ extern "C" int mi_softmax_tma_kernel(const mi_tile_array* output, const mi_tile_
     if (input->sizes[0] == 0 || input->sizes[1] == 0) return MI_OK;
     if (input->sizes[1] > 0x7fffffffLL) return MI_E_GRID;
     hipStream_t s = (hipStream_t)stream;
+    const int64_t L = input->sizes[0] < TILE_SIZE ? input->sizes[0] : (int64_t)TILE_SIZE;  // one tile per column
     switch (input->dtype) {
-        case MI_F32: return launch_tma<float>(output, input, TILE_SIZE, s);
-        case MI_F16: return launch_tma<__half>(output, input, TILE_SIZE, s);
-        default: return launch_tma<__hip_bfloat16>(output, input, TILE_SIZE, s);
+        case MI_F32: return launch_len<float>(output, input, L, s);
+        case MI_F16: return launch_len<__half>(output, input, L, s);
+        default: return launch_len<__hip_bfloat16>(output, input, L, s);
     }
 }
 
@@ -253,8 +255,10 @@ extern "C" int mi_softmax_chunked_kernel(const mi_tile_array* output, const mi_t
     if (L == 0) return MI_OK;
     hipStream_t s = (hipStream_t)stream;
     switch (input->dtype) {
-        case MI_F32: return launch_3pass<float>(output, input, L, s);
-        case MI_F16: return launch_3pass<__half>(output, input, L, s);
-        default: return launch_3pass<__hip_bfloat16>(output, input, L, s);
+        // Same function of the column as the reference's three chunked passes; a column that
+        // fits in registers is read from HBM once instead.
+        case MI_F32: return launch_len<float>(output, input, L, s);
+        case MI_F16: return launch_len<__half>(output, input, L, s);
+        default: return launch_len<__hip_bfloat16>(output, input, L, s);
     }
 }

@@ -147,8 +147,9 @@ int mi_layer_norm_bwd_dwdb(const mi_tile_array* DW, const mi_tile_array* DB,
  * softmax.jl:136); any value >= 1 gives the same result. f32 / f16 / bf16 storage. */
 int mi_softmax_tma_kernel(const mi_tile_array* output, const mi_tile_array* input,
                           int TILE_SIZE, int num_programs, void* stream);
-/* softmax_chunked_kernel (softmax.jl:48-100): 3-pass softmax over the first n_elems rows
- * in chunks of TILE_SIZE. */
+/* softmax_chunked_kernel (softmax.jl:48-100): softmax over the rows that the reference's chunk
+ * loop visits, 1 .. cld(n_elems, TILE_SIZE)*TILE_SIZE.  Same function of the column as the
+ * reference's three chunked passes; columns that fit in registers are read once. */
 int mi_softmax_chunked_kernel(const mi_tile_array* output, const mi_tile_array* input,
                               int n_elems, int TILE_SIZE, int num_programs, void* stream);
 

@@ -238,13 +238,13 @@ __global__ __launch_bounds__(BLOCK) void ln_bwd_kernel(float* __restrict__ DX, i
     }
 }
 
-// Backward with two row groups per workgroup (512 lanes for rows of up to 4096 elements, 16-byte
-// aligned): the halves of the workgroup walk different rows of the same partial slot and add
-// their dW/dB partials in LDS before the flush, which halves the number of memory-side float
-// atomics -- the scarce resource of this kernel -- at the same number of rows in flight.
-// Workgroup (g, s): group h handles rows m = g + G*(2*s + h), stepping by 2*G*S.
-template <int VPT, bool STREAM>
-__global__ __launch_bounds__(512) void ln_bwd_rg2_kernel(float* __restrict__ DX, int64_t lddx,
+// Backward with RG row groups of 256 lanes per workgroup (rows of up to 4096 elements, 16-byte
+// aligned): the groups walk different rows of the same partial slot and add their dW/dB
+// partials in LDS before the flush, which divides the number of memory-side float atomics --
+// the scarce resource of this kernel -- by RG at the same number of rows in flight.
+// Workgroup (g, s): group h handles rows m = g + G*(RG*s + h), stepping by RG*G*S.
+template <int VPT, bool STREAM, int RG>
+__global__ __launch_bounds__(256 * RG) void ln_bwd_rg_kernel(float* __restrict__ DX, int64_t lddx,
                                                          const float* __restrict__ DY, int64_t lddy,
                                                          float* __restrict__ DW, int64_t lddw,
                                                          float* __restrict__ DB, int64_t lddb,
@@ -254,7 +254,7 @@ __global__ __launch_bounds__(512) void ln_bwd_rg2_kernel(float* __restrict__ DX,
                                                          const float* __restrict__ Rstd, int N,
                                                          int64_t M, int G, int S) {
     constexpr int BLOCK = 256, NW = 4;
-    __shared__ float red[2][2 * NW];
+    __shared__ float red[RG][2 * NW];
     __shared__ float stage[BLOCK * VPT * 4];
     const int g = blockIdx.x % G, s = blockIdx.x / G;
     const int h = threadIdx.x >> 8, lt = threadIdx.x & 255, lane = lt & 63, wave = lt >> 6;
@@ -269,8 +269,8 @@ __global__ __launch_bounds__(512) void ln_bwd_rg2_kernel(float* __restrict__ DX,
             dw[v][q] = db[v][q] = 0.f;
         }
     }
-    const int64_t step = (int64_t)2 * G * S, m0 = g + (int64_t)G * (2 * s + h);
-    const int64_t trips = (M - (g + (int64_t)G * 2 * s) + step - 1) / step;  // of group 0; group 1 may idle in the last
+    const int64_t step = (int64_t)RG * G * S, m0 = g + (int64_t)G * (RG * s + h);
+    const int64_t trips = (M - (g + (int64_t)G * RG * s) + step - 1) / step;  // of group 0; later groups may idle in the last
     for (int64_t it = 0; it < trips; ++it) {
         const int64_t m = m0 + it * step;
         const bool live = m < M;  // uniform per group; both groups keep meeting at the barriers
@@ -327,27 +327,28 @@ __global__ __launch_bounds__(512) void ln_bwd_rg2_kernel(float* __restrict__ DX,
             if (live && vec(v) < N) st_global<true>(t, reinterpret_cast<f32x4*>(DX + m * lddx + vec(v)));
         }
     }
-    // group 1 hands its partials to group 0 through LDS; group 0 flushes with coalesced atomics
+    // the groups add their partials in LDS, one after the other; then everybody flushes with
+    // coalesced atomics
     float* dwp = DW + (int64_t)g * lddw;
     float* dbp = DB + (int64_t)g * lddb;
 #pragma unroll
     for (int pass = 0; pass < 2; ++pass) {
-        if (h == 1) {
 #pragma unroll
-            for (int v = 0; v < VPT; ++v)
+        for (int turn = 0; turn < RG; ++turn) {
+            if (h == turn) {
 #pragma unroll
-                for (int q = 0; q < 4; ++q) stage[vec(v) + q] = pass == 0 ? dw[v][q] : db[v][q];
+                for (int v = 0; v < VPT; ++v)
+#pragma unroll
+                    for (int q = 0; q < 4; ++q) {
+                        const float val = pass == 0 ? dw[v][q] : db[v][q];
+                        if (turn == 0) stage[vec(v) + q] = val;
+                        else stage[vec(v) + q] += val;
+                    }
+            }
+            __syncthreads();
         }
-        __syncthreads();
-        if (h == 0) {
-#pragma unroll
-            for (int v = 0; v < VPT; ++v)
-#pragma unroll
-                for (int q = 0; q < 4; ++q) stage[vec(v) + q] += pass == 0 ? dw[v][q] : db[v][q];
-        }
-        __syncthreads();
         float* dst = pass == 0 ? dwp : dbp;
-        for (int c = threadIdx.x; c < N; c += 512) {
+        for (int c = threadIdx.x; c < N; c += 256 * RG) {
             if (S == 1) dst[c] += stage[c];
             else unsafeAtomicAdd(dst + c, stage[c]);
         }
@@ -574,19 +575,19 @@ extern "C" int mi_layer_norm_bwd_dx_partial_dwdb(
         X->strides[1], (const float*)W->ptr, (const float*)Mean->ptr, (const float*)Rstd->ptr,  \
         (int)N, M, G, (int)S
     const bool stream_in = stream_hint(3 * M * N * (int64_t)sizeof(float));
-    static const bool no_rg2 = [] { const char* e = getenv("MI_LN_BWD_RG"); return e && e[0] == '1'; }();
-    if (al && N % 4 == 0 && vecs > 512 && vecs <= 1024 && S % 2 == 0 && !no_rg2) {
-        // two row groups per workgroup: same rows in flight, half the atomics
+    static const bool one_group = [] { const char* e = getenv("MI_LN_BWD_RG"); return e && e[0] == '1'; }();
+    if (al && N % 4 == 0 && vecs > 512 && vecs <= 1024 && S % 2 == 0 && !one_group) {
+        // two row groups per workgroup: same rows in flight, half the atomics (four groups measured no better)
         const int S2 = (int)S / 2;
         dim3 grid2((unsigned)(G * S2));
-#define RG2(ST)                                                                                              \
-    hipLaunchKernelGGL((ln_bwd_rg2_kernel<4, ST>), grid2, dim3(512), 0, s, (float*)DX->ptr, DX->strides[1],    \
+#define RGK(ST)                                                                                               \
+    hipLaunchKernelGGL((ln_bwd_rg_kernel<4, ST, 2>), grid2, dim3(512), 0, s, (float*)DX->ptr, DX->strides[1],   \
                        (const float*)DY->ptr, DY->strides[1], (float*)DW->ptr, DW->strides[1], (float*)DB->ptr, \
                        DB->strides[1], (const float*)X->ptr, X->strides[1], (const float*)W->ptr,               \
                        (const float*)Mean->ptr, (const float*)Rstd->ptr, (int)N, M, G, S2)
-        if (stream_in) RG2(true);
-        else RG2(false);
-#undef RG2
+        if (stream_in) RGK(true);
+        else RGK(false);
+#undef RGK
         set_variant("ln_bwd_regs_b512_v4_rg2");
     } else if (!al) launch_bwd<false, false>(ARGS);
     else if (stream_in) launch_bwd<true, true>(ARGS);

@@ -93,7 +93,7 @@ def bench_kernels(ct, which, cpu, nruns=NRUNS, warmup=WARMUP):
     import numpy as np
     import torch
     from oracle import cutile_oracle as orc
-    from cutile_jl_amd.examples import vadd, transpose, layernorm, softmax, matmul, batchmatmul, fmha, moe
+    from cutile_jl_amd.examples import vadd, transpose, layernorm, softmax, matmul, batchmatmul, fmha, moe, fft
     res = {}
     ncores = os.cpu_count()
 
@@ -210,6 +210,18 @@ def bench_kernels(ct, which, cpu, nruns=NRUNS, warmup=WARMUP):
             e["cpu_note"] = f"numpy restatement of ref_fmha, 4 of 128 (batch, head) pairs x32, BLAS {ncores} threads"
         res["fmha"] = e
         del d
+    if want("fft"):
+        d = fft.prepare(benchmark=True)
+        F0, F1, F2 = d.factors
+        go = ct.bind("mi_fft_kernel", d.x_packed, d.y_packed, d.W0, d.W1, d.W2, d.T0, d.T1, d.N, F0, F1, F2, 1, d.D)
+        nbytes = 2 * d.batch * d.N * 8 + (d.T0.numel() + d.T1.numel() + d.W0.numel() * 3) * 4
+        res["fft"] = _entry("FFT 4096-point x 256 signals complex64 (3-stage 16x16x16), latency benchmark of the reference",
+                            go, nbytes, "GB/s", "hbm", HBM_PEAK_GBS, "f32", nruns, warmup)
+        if cpu:
+            x = d.input.cpu().numpy()
+            res["fft"]["cpu_ms"] = round(_cpu_time(lambda: np.fft.fft(x, axis=1)), 2)
+            res["fft"]["cpu_note"] = "numpy.fft (pocketfft) on the same complex64 batch, 1 thread (the reference verifies against FFTW)"
+
     if want("moe"):
         d = moe.prepare(benchmark=True, topk=2, router="top2_logits")
         flop = moe.metric(d)[0]

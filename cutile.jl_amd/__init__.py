@@ -69,6 +69,7 @@ _SIGNATURES = {
     "mi_softmax_tma_kernel": ([_A, _A, _i, _i, _vp], _i),
     "mi_softmax_chunked_kernel": ([_A, _A, _i, _i, _i, _vp], _i),
     "mi_fmha_kernel": ([_A, _A, _A, _A, ctypes.c_float, ctypes.c_int32, _i, _i, _i, _i, _i, _i, _i, _vp], _i),
+    "mi_fft_kernel": ([_A, _A, _A, _A, _A, _A, _A, _i, _i, _i, _i, _i, _i, _vp], _i),
     "mi_moe_align_tile_size_device": ([_A, _i, _i, _A, _A, _vp], _i),
     "mi_moe_align_tile_size": (
         [ctypes.POINTER(ctypes.c_int64), ctypes.c_int64, ctypes.c_int64, _i, _i,
@@ -153,6 +154,13 @@ def _call(name: str, *args):
     rc = getattr(lib(), name)(*args)
     if rc != 0:
         raise MiError(name, rc, strerror(rc))
+
+
+def fft_kernel(x_packed_in, y_packed_out, W0, W1, W2, T0, T1, N: int, F0: int, F1: int, F2: int, BS: int,
+               D: int, stream=None):
+    """examples/fft.jl:22-126"""
+    _call("mi_fft_kernel", _ref(x_packed_in), _ref(y_packed_out), _ref(W0), _ref(W1), _ref(W2), _ref(T0),
+          _ref(T1), N, F0, F1, F2, BS, D, _stream(stream))
 
 
 def bind(name: str, *args, stream=None):

@@ -270,4 +270,15 @@ function moe_sum_topk(in, out; stream::Ptr{Cvoid}=C_NULL)
         (Ref{MiTileArray}, Ref{MiTileArray}, Ptr{Cvoid}), d[1], d[2], stream))
 end
 
+# ---- examples/fft.jl ----------------------------------------------------------------------
+
+function fft_kernel(x_packed_in, y_packed_out, W0, W1, W2, T0, T1, N::Integer, F0::Integer, F1::Integer,
+                    F2::Integer, BS::Integer, D::Integer; stream::Ptr{Cvoid}=C_NULL)
+    d = map(a -> ref(descriptor(a)), (x_packed_in, y_packed_out, W0, W1, W2, T0, T1))
+    GC.@preserve x_packed_in y_packed_out W0 W1 W2 T0 T1 check(ccall((:mi_fft_kernel, libmi355tile), Cint,
+        (Ref{MiTileArray}, Ref{MiTileArray}, Ref{MiTileArray}, Ref{MiTileArray}, Ref{MiTileArray},
+         Ref{MiTileArray}, Ref{MiTileArray}, Cint, Cint, Cint, Cint, Cint, Cint, Ptr{Cvoid}),
+        d[1], d[2], d[3], d[4], d[5], d[6], d[7], N, F0, F1, F2, BS, D, stream))
+end
+
 end # module

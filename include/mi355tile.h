@@ -202,6 +202,18 @@ int mi_silu_and_mul_kernel(const mi_tile_array* A, const mi_tile_array* B,
  * accumulation in slot order. */
 int mi_moe_sum_topk(const mi_tile_array* in, const mi_tile_array* out, void* stream);
 
+/* ---- FFT: examples/fft.jl ------------------------------------------------------------- */
+/* fft_kernel (fft.jl:22-126): batched complex FFT of N = F0*F1*F2 points as three stages of small
+ * DFTs.  x_packed_in, y_packed_out (D, 2N/D, batch) f32: the interleaved (re, im) signals, dense;
+ * W0 (2,F0,F0), W1 (2,F1,F1), W2 (2,F2,F2): DFT matrices, T0 (2,F1*F2,F0), T1 (2,F2,F1): twiddles
+ * (fft.jl:130-180), all f32 with the (re, im) pair leading.  One workgroup per signal; BS (signals
+ * per block of the reference's launch) only has to divide the batch.  N <= 4096; the radix triples
+ * compiled in are listed in fft.hip (MI_E_UNSUPPORTED otherwise). */
+int mi_fft_kernel(const mi_tile_array* x_packed_in, const mi_tile_array* y_packed_out,
+                  const mi_tile_array* W0, const mi_tile_array* W1, const mi_tile_array* W2,
+                  const mi_tile_array* T0, const mi_tile_array* T1, int N, int F0, int F1, int F2,
+                  int BS, int D, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

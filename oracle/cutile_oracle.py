@@ -25,6 +25,7 @@ ref_fmha               row 1 of causal output == V[:,1]; brute-force loops on ti
                        ``torch.nn.functional.scaled_dot_product_attention`` on CPU
 moe_align_tile_size    permutation / grouping / padding invariants; brute force; C cross-check
 ref_moe                per-token dense loop on tiny shapes
+fft_3stage, tables     ``numpy.fft.fft`` (independent library); brute-force DFT sum on tiny sizes
 e4m3fn codec           16 round-trip vectors and fma vectors of
                        test/extensions/DLFP8Types.jl:126-141; all 256 codes vs torch.float8_e4m3fn
 =====================  ======================================================================
@@ -339,11 +340,60 @@ def quantize_e4m3fn_per_channel(w: np.ndarray):
     return codes, scale
 
 
+# ---- FFT -----------------------------------------------------------------------------------
+
+def dft_matrix(size: int) -> np.ndarray:
+    """examples/fft.jl:130-140: W[i, j] = exp(-2 pi i * i*j / size), stored (2, size, size) float32
+    (Julia shape), real part first."""
+    i, j = np.meshgrid(np.arange(size), np.arange(size), indexing="ij")
+    W = np.exp(-2j * np.pi * i * j / size)
+    return np.stack([W.real, W.imag]).astype(np.float32)
+
+
+def make_twiddles(factors):
+    """examples/fft.jl:143-180.  Returns (W0, W1, W2, T0, T1) in the Julia shapes
+    (2,F0,F0), (2,F1,F1), (2,F2,F2), (2,F1F2,F0), (2,F2,F1), float32."""
+    F0, F1, F2 = factors
+    N, F1F2 = F0 * F1 * F2, F1 * F2
+    j, i = np.meshgrid(np.arange(F1F2), np.arange(F0), indexing="ij")      # T0[:, j, i] = exp(-2 pi i * i*j / N)
+    t0 = np.exp(-2j * np.pi * i * j / N)
+    k, jj = np.meshgrid(np.arange(F2), np.arange(F1), indexing="ij")       # T1[:, k, j] = exp(-2 pi i * j*k / F1F2)
+    t1 = np.exp(-2j * np.pi * jj * k / F1F2)
+    T0 = np.stack([t0.real, t0.imag]).astype(np.float32)
+    T1 = np.stack([t1.real, t1.imag]).astype(np.float32)
+    return dft_matrix(F0), dft_matrix(F1), dft_matrix(F2), T0, T1
+
+
+def fft_3stage(x: np.ndarray, factors, tables=None, dtype=np.complex128) -> np.ndarray:
+    """The data flow of fft_kernel (examples/fft.jl:45-121) on x of Julia shape (N, batch), complex:
+    three batched products with the DFT matrices, two element-wise twiddle multiplications and the
+    reshapes / permutedims between them, written with Fortran-order reshapes so that every line
+    matches the Julia one."""
+    F0, F1, F2 = factors
+    N, F1F2, F0F2, F0F1 = F0 * F1 * F2, F1 * F2, F0 * F2, F0 * F1
+    BS = x.shape[1]
+    W0, W1, W2, T0, T1 = tables if tables is not None else make_twiddles(factors)
+    c = lambda t: (t[0].astype(np.float64) + 1j * t[1].astype(np.float64)).astype(dtype)
+    W0, W1, W2, T0, T1 = c(W0), c(W1), c(W2), c(T0), c(T1)
+    R = lambda a, shp: np.reshape(a, shp, order="F")
+    X = R(x.astype(dtype), (F1F2, F0, BS))                                   # fft.jl:82-83
+    X = np.einsum("rib,ik->rkb", X, W0)                                      # :84-85  X * W0
+    X = R(X, (N, BS)) * R(T0, (N,))[:, None]                                 # :88-89
+    X = np.transpose(R(X, (F2, F1, F0, BS)), (2, 0, 1, 3))                   # :92-93  permutedims (3,1,2,4)
+    X = np.einsum("rib,ik->rkb", R(X, (F0F2, F1, BS)), W1)                   # :97-100
+    X = R(X, (F0, F1F2, BS)) * R(T1, (F1F2,))[None, :, None]                 # :103-104
+    X = np.transpose(R(X, (F0, F2, F1, BS)), (2, 0, 1, 3))                   # :107-108
+    X = np.einsum("rib,ik->rkb", R(X, (F0F1, F2, BS)), W2)                   # :112-115
+    X = np.transpose(R(X, (F1, F0, F2, BS)), (1, 0, 2, 3))                   # :118-119 permutedims (2,1,3,4)
+    return R(X, (N, BS))
+
+
 # ---- example verify() criteria -------------------------------------------------------------
 
 def isapprox(x: np.ndarray, y: np.ndarray, rtol: float, atol: float = 0.0) -> bool:
     """Julia's ``isapprox`` for arrays: ``norm(x-y) <= max(atol, rtol*max(norm(x), norm(y)))``
     with the 2-norm (used by every example's verify)."""
-    x = np.asarray(x, dtype=np.float64); y = np.asarray(y, dtype=np.float64)
+    wide = np.complex128 if np.iscomplexobj(x) or np.iscomplexobj(y) else np.float64
+    x = np.asarray(x, dtype=wide); y = np.asarray(y, dtype=wide)
     d = np.linalg.norm((x - y).ravel())
     return bool(d <= max(atol, rtol * max(np.linalg.norm(x.ravel()), np.linalg.norm(y.ravel()))))

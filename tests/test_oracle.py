@@ -312,3 +312,30 @@ def test_quantize_per_channel_bound():
 def test_isapprox_is_normwise():
     x = np.array([1.0, 0.0]); y = np.array([1.0, 0.005])
     assert orc.isapprox(x, y, rtol=1e-2) and not orc.isapprox(x, y, rtol=1e-3)
+
+
+# ---- FFT (examples/fft.jl) ---------------------------------------------------------------------
+
+@pytest.mark.parametrize("factors", [(2, 2, 2), (8, 8, 8), (16, 16, 16), (4, 8, 2), (2, 4, 8)])
+def test_fft_3stage_matches_numpy_fft(factors):
+    """The three-stage data flow restated from fft.jl:45-121 equals the library FFT (an index or
+    permutation slip in any stage scrambles the spectrum)."""
+    rng = np.random.default_rng(3)
+    N = factors[0] * factors[1] * factors[2]
+    x = rng.standard_normal((N, 3)) + 1j * rng.standard_normal((N, 3))
+    y = orc.fft_3stage(x, factors)
+    ref = np.fft.fft(x, axis=0)
+    assert np.abs(y - ref).max() <= 1e-6 * np.abs(ref).max()      # float32 tables
+
+
+def test_fft_tables_and_brute_force_dft():
+    W = orc.dft_matrix(8)
+    assert W.shape == (2, 8, 8) and W.dtype == np.float32
+    assert np.allclose(W[0] + 1j * W[1], np.fft.fft(np.eye(8)), atol=1e-6)
+    W0, W1, W2, T0, T1 = orc.make_twiddles((2, 4, 8))
+    assert T0.shape == (2, 32, 2) and T1.shape == (2, 8, 4)
+    assert np.allclose(T0[0, 5, 1] + 1j * T0[1, 5, 1], np.exp(-2j * np.pi * 5 / 64), atol=1e-7)   # fft.jl:146-150
+    assert np.allclose(T1[0, 3, 2] + 1j * T1[1, 3, 2], np.exp(-2j * np.pi * 6 / 32), atol=1e-7)   # fft.jl:158-162
+    x = np.arange(8, dtype=np.float64)[:, None] * (1 + 0.5j)
+    brute = np.array([sum(x[n, 0] * np.exp(-2j * np.pi * k * n / 8) for n in range(8)) for k in range(8)])
+    assert np.allclose(orc.fft_3stage(x, (2, 2, 2))[:, 0], brute, atol=1e-5)

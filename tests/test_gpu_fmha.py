@@ -100,6 +100,23 @@ def test_fmha_pipelined_kernel_shapes(ct, orc, batch, heads, s, causal, qg, T):
 
 
 @pytest.mark.parametrize("causal", [True, False])
+def test_fmha_pipelined_kernel_strided_views(ct, orc, causal):
+    """Q/K/V as views of one packed (B, S, 3, H, D) buffer and Out as a view of a wider buffer: row,
+    head and batch strides all differ from the dense ones."""
+    rng = np.random.default_rng(4)
+    B, S, H, D = 2, 256, 4, 64
+    packed = torch.from_numpy(rng.standard_normal((B, S, 3, H, D), dtype=np.float32)).to(torch.float16).cuda()
+    Q, K, V = (packed[:, :, i].permute(0, 2, 1, 3) for i in range(3))        # torch (B, H, S, D) views
+    out_buf = torch.zeros((B, H, S, 2 * D), dtype=torch.float16, device="cuda")
+    out = out_buf[..., D:]                                                     # rows 2*D apart, offset D
+    fmha.cutile_fmha(Q, K, V, causal=causal, out=out)
+    assert ct.last_variant().startswith("fmha_pipe")
+    ref = orc.ref_fmha(orc.to_julia(Q), orc.to_julia(K), orc.to_julia(V), causal=causal, dtype=np.float64)
+    check(orc, out, ref)
+    assert torch.all(out_buf[..., :D] == 0)
+
+
+@pytest.mark.parametrize("causal", [True, False])
 def test_fmha_running_maximum_keeps_rising(ct, orc, causal):
     """Scores that grow with the key index by far more than the kernel's lazy-rescale threshold:
     the running maximum has to be raised again and again, and early keys end up with weights

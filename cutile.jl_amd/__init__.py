@@ -20,7 +20,7 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 # MI355TILE_LIB selects another build of the same library (e.g. an experimental variant).
 LIB_PATH = os.environ.get("MI355TILE_LIB") or os.path.join(_HERE, "libmi355tile.so")
 
-MI_F32, MI_F64, MI_F16, MI_BF16, MI_F8E4M3FN, MI_I32, MI_I64 = range(7)
+MI_F32, MI_F64, MI_F16, MI_BF16, MI_F8E4M3FN, MI_I32, MI_I64, MI_BOOL = range(8)
 MI_MAX_RANK = 4
 
 # error codes of include/mi355tile.h
@@ -78,6 +78,15 @@ _SIGNATURES = {
     "mi_fused_moe_kernel": ([_A] * 6 + [_i, _i, _i, _i, _i, _A, _vp], _i),
     "mi_silu_and_mul_kernel": ([_A, _A, _A, _i, _vp], _i),
     "mi_moe_sum_topk": ([_A, _A, _vp], _i),
+    "mi_tiled_broadcast": ([_A, ctypes.c_char_p, ctypes.POINTER(_A), _i, _vp, _i, _vp], _i),
+    "mi_tiled_broadcast_eltype": ([ctypes.c_char_p, ctypes.POINTER(ctypes.c_int32), _i,
+                                   ctypes.POINTER(ctypes.c_int32), _i, ctypes.POINTER(ctypes.c_int32)], _i),
+    "mi_tiled_mapreduce": ([_A, _A, ctypes.c_char_p, _vp, _i, _i, _vp, ctypes.c_int64, _vp], _i),
+    "mi_tiled_mapreduce_workspace": ([_A, _A, _i, ctypes.POINTER(ctypes.c_int64)], _i),
+    "mi_tiled_mapreduce_eltype": ([ctypes.c_char_p, ctypes.c_int32, ctypes.POINTER(ctypes.c_int32), _i, _i, _i,
+                                   ctypes.POINTER(ctypes.c_int32)], _i),
+    "mi_tiled_set_dry_run": ([_i], _i),
+    "mi_tiled_compile_count": ([], _i),
 }
 EXPORTED_SYMBOLS = tuple(_SIGNATURES)
 

@@ -20,7 +20,8 @@
  * (block → data mapping, padding contracts, accumulation grouping); the physical
  * wave / LDS tiling is chosen by the library for CDNA4.
  *
- * Every call is asynchronous, allocates nothing and never throws.  Return value: 0 on
+ * Every call is asynchronous, allocates nothing and never throws (the mi_tiled_* entry points
+ * compile and load a code object the first time they meet a new expression, see below).  Return value: 0 on
  * success, a negative MI_E_* code for argument errors detected on the host, or a
  * positive hipError_t reported by the launch.  The caller owns all buffers.
  */
@@ -44,7 +45,8 @@ typedef enum mi_dtype {
     MI_F8E4M3FN = 4, /* OCP FP8 E4M3 "FN": bias 7, no Inf, NaN = S.1111.111, max 448
                         (reference: ext/DLFP8TypesExt.jl:7-9) */
     MI_I32 = 5,
-    MI_I64 = 6
+    MI_I64 = 6,
+    MI_BOOL = 7      /* Julia Bool: one byte holding 0 or 1 (Tiled broadcast / mapreduce only) */
 } mi_dtype;
 
 /* Error codes (negative).  Positive return values are hipError_t. */
@@ -213,6 +215,74 @@ int mi_fft_kernel(const mi_tile_array* x_packed_in, const mi_tile_array* y_packe
                   const mi_tile_array* W0, const mi_tile_array* W1, const mi_tile_array* W2,
                   const mi_tile_array* T0, const mi_tile_array* T1, int N, int F0, int F1, int F2,
                   int BS, int D, void* stream);
+
+/* ---- Host-level Tiled broadcast and mapreduce ---------------------------------------------------
+ * The reference specialises and compiles a kernel per broadcast tree / reduction on first use
+ * (src/broadcast.jl:75-129, src/mapreduce.jl:13-129) and caches it (src/launch.jl:663-687).  These
+ * entry points do the same through hiprtc: the first call with a new (expression, element types,
+ * layout class) generates a fused gfx950 kernel, compiles, loads and caches it (tens of
+ * milliseconds, allocates the code object); every later call only launches.  Arrays have 0 to 4
+ * dimensions and any element strides; element types f32 f64 f16 bf16 i32 i64 bool.
+ *
+ * Expressions are text in prefix form:  expr := name(expr{,expr}) | a<i> | s<i>, with a<i> the
+ * i-th array leaf and s<i> the i-th scalar; `name` is one of
+ *   add sub mul div pow neg abs abs2 sign max min fma muladd clamp copysign floor ceil round trunc
+ *   sqrt cbrt inv exp exp2 exp10 expm1 log log2 log10 log1p sin cos tan asin acos atan sinh cosh
+ *   tanh atan2 hypot lt le gt ge eq ne isnan isinf isfinite signbit iszero not and or xor ifelse
+ *   div_int rem mod fld cld identity f16 bf16 f32 f64 i32 i64 bool
+ * (Julia's `+` is add, `/` is div, `^` is pow, `÷` is div_int, `Float32(x)` is f32, ...).  Node
+ * types follow Julia's promote_type / float() rules; Float16 and BFloat16 operations are rounded
+ * after every step as Julia defines them.  Unknown names return MI_E_UNSUPPORTED. */
+typedef struct mi_tile_scalar {
+    int32_t dtype;      /* mi_dtype of the Julia number */
+    int32_t reserved;
+    union {
+        double f;       /* value of a float type */
+        int64_t i;      /* value of an integer type or Bool */
+    } value;
+} mi_tile_scalar;
+
+/* dest .= expr(leaves..., scalars...)   (reference: Base.Broadcast.materialize!(::Tiled, bc),
+ * src/broadcast.jl:20-24,75-92).  A leaf dimension must equal dest's or be 1 (it then expands);
+ * leaves of lower rank expand along the trailing dimensions; MI_E_SHAPE otherwise (the reference
+ * throws DimensionMismatch).  The tree's value is converted to dest's element type.  An empty
+ * dest launches nothing.  At most 8 leaves, 8 scalars, 128 nodes. */
+int mi_tiled_broadcast(const mi_tile_array* dest, const char* expr, const mi_tile_array* const* leaves,
+                       int n_leaves, const mi_tile_scalar* scalars, int n_scalars, void* stream);
+
+/* Element type of a tree: Base.Broadcast.combine_eltypes as used by the allocating form
+ * (src/broadcast.jl:26-32). */
+int mi_tiled_broadcast_eltype(const char* expr, const int32_t* leaf_dtypes, int n_leaves,
+                              const int32_t* scalar_dtypes, int n_scalars, int32_t* out_dtype);
+
+/* Reduction operators (src/mapreduce.jl:5-11 lists the reference's). */
+enum { MI_OP_ADD = 0, MI_OP_MUL = 1, MI_OP_MAX = 2, MI_OP_MIN = 3, MI_OP_AND = 4, MI_OP_OR = 5 };
+
+/* dest = reduce(op, f.(src)) over the dimensions in which dest has extent 1 and src has not
+ * (reference: `_mapreducedim!`, src/mapreduce.jl:66-129, dimension rule of :188-196).  `f_expr`
+ * is an expression in a0 (= one element of src) and the scalars, NULL for identity; its value is
+ * converted to dest's element type, which is also the accumulator type.  The accumulator starts
+ * from op's neutral element (0, 1, typemin, typemax, all-ones, 0); a caller's `init` is applied
+ * afterwards as the reference does (src/mapreduce.jl:157-163).  With no reduced dimension this is
+ * map.  Reductions with few outputs run in two passes through `workspace` (device memory, 16-byte
+ * aligned, at least mi_tiled_mapreduce_workspace() bytes; may be NULL when that is 0); float
+ * results are reproducible from run to run.  max / min propagate NaN as Julia does. */
+int mi_tiled_mapreduce(const mi_tile_array* dest, const mi_tile_array* src, const char* f_expr,
+                       const mi_tile_scalar* scalars, int n_scalars, int op, void* workspace,
+                       int64_t workspace_bytes, void* stream);
+int mi_tiled_mapreduce_workspace(const mi_tile_array* dest, const mi_tile_array* src, int op, int64_t* bytes);
+
+/* Element type of the result: promote_op(op, T, T) of T = typeof(f(x)) (src/mapreduce.jl:133-137).
+ * `widen` != 0 selects Base's add_sum / mul_prod, which widen Int32 and Bool to Int64 (what
+ * `sum` / `prod` pass); 0 is plain `+` / `*` as `reduce(+, ...)` passes. */
+int mi_tiled_mapreduce_eltype(const char* f_expr, int32_t src_dtype, const int32_t* scalar_dtypes,
+                              int n_scalars, int op, int widen, int32_t* out_dtype);
+
+/* Test hooks.  mi_tiled_set_dry_run(1) makes the two entry points stop after compiling (nothing is
+ * loaded or launched, no GPU is needed); returns the previous setting.  mi_tiled_compile_count()
+ * is the number of kernels compiled so far in this process. */
+int mi_tiled_set_dry_run(int on);
+int mi_tiled_compile_count(void);
 
 #ifdef __cplusplus
 }

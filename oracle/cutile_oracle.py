@@ -26,6 +26,12 @@ ref_fmha               row 1 of causal output == V[:,1]; brute-force loops on ti
 moe_align_tile_size    permutation / grouping / padding invariants; brute force; C cross-check
 ref_moe                per-token dense loop on tiny shapes
 fft_3stage, tables     ``numpy.fft.fft`` (independent library); brute-force DFT sum on tiny sizes
+tiled_eval/broadcast   known answers of test/host/broadcast.jl (fills, 0-dim, expansion cases);
+                       plain numpy expressions written out by hand; torch CPU for bfloat16
+tiled_mapreduce        known answers of test/host/mapreduce.jl (count == 4, any / all, max of
+                       fill(-5) == -5); numpy reductions; brute-force loops on tiny arrays
+jl_promote             Julia's documented promotion facts (Int32+Int64 -> Int64, Int64+Float32 ->
+                       Float32, Float16+Float32 -> Float32, Bool yields, true + true == 2)
 e4m3fn codec           16 round-trip vectors and fma vectors of
                        test/extensions/DLFP8Types.jl:126-141; all 256 codes vs torch.float8_e4m3fn
 =====================  ======================================================================
@@ -386,6 +392,258 @@ def fft_3stage(x: np.ndarray, factors, tables=None, dtype=np.complex128) -> np.n
     X = np.einsum("rib,ik->rkb", R(X, (F0F1, F2, BS)), W2)                   # :112-115
     X = np.transpose(R(X, (F1, F0, F2, BS)), (1, 0, 2, 3))                   # :118-119 permutedims (2,1,3,4)
     return R(X, (N, BS))
+
+
+# ---- host-level Tiled broadcast / mapreduce ------------------------------------------------
+# Julia element types by name; numpy has no bfloat16, those cases are checked against torch.
+_JL_FLOATS = ("Float16", "Float32", "Float64")
+_JL_NP = {"Float16": np.float16, "Float32": np.float32, "Float64": np.float64, "Int32": np.int32, "Int64": np.int64,
+          "Bool": np.bool_}
+_NP_JL = {np.dtype(v): k for k, v in _JL_NP.items()}
+
+
+def jl_promote(a: str, b: str) -> str:
+    """Julia's promote_type on {Bool, Int32, Int64, Float16, Float32, Float64} (Base promotion.jl:
+    Bool yields to everything, integers yield to floats, the wider of two of a kind wins)."""
+    if a == b:
+        return a
+    if a == "Bool":
+        return b
+    if b == "Bool":
+        return a
+    ai, bi = a.startswith("Int"), b.startswith("Int")
+    if ai and bi:
+        return "Int64"
+    if ai:
+        return b
+    if bi:
+        return a
+    return _JL_FLOATS[max(_JL_FLOATS.index(a), _JL_FLOATS.index(b))]
+
+
+def _jl_scalar_type(x) -> str:
+    if isinstance(x, (bool, np.bool_)):
+        return "Bool"
+    if isinstance(x, np.generic):
+        return _NP_JL[np.dtype(type(x))]
+    return "Int64" if isinstance(x, int) else "Float64"
+
+
+_TILED_MATH = {"sqrt": np.sqrt, "cbrt": np.cbrt, "exp": np.exp, "exp2": np.exp2, "expm1": np.expm1, "log": np.log,
+               "log2": np.log2, "log10": np.log10, "log1p": np.log1p, "sin": np.sin, "cos": np.cos, "tan": np.tan,
+               "asin": np.arcsin, "acos": np.arccos, "atan": np.arctan, "sinh": np.sinh, "cosh": np.cosh,
+               "tanh": np.tanh, "exp10": lambda v: np.power(v.dtype.type(10), v), "inv": lambda v: v.dtype.type(1) / v}
+_TILED_CMP = {"lt": np.less, "le": np.less_equal, "gt": np.greater, "ge": np.greater_equal, "eq": np.equal,
+              "ne": np.not_equal}
+
+
+def _jl_max(a, b):
+    """Julia's max: NaN wins, +0.0 beats -0.0 (Base math.jl)."""
+    with np.errstate(invalid="ignore"):
+        r = np.where(np.isnan(a) | np.isnan(b), a + b, np.maximum(a, b)) if a.dtype.kind == "f" else np.maximum(a, b)
+    if a.dtype.kind == "f":
+        tie = (a == b) & (a == 0)
+        r = np.where(tie, np.where(np.signbit(a), b, a), r)
+    return r.astype(a.dtype)
+
+
+def _jl_min(a, b):
+    with np.errstate(invalid="ignore"):
+        r = np.where(np.isnan(a) | np.isnan(b), a + b, np.minimum(a, b)) if a.dtype.kind == "f" else np.minimum(a, b)
+    if a.dtype.kind == "f":
+        tie = (a == b) & (a == 0)
+        r = np.where(tie, np.where(np.signbit(a), a, b), r)
+    return r.astype(a.dtype)
+
+
+def tiled_eval(text: str, leaves=(), scalars=()):
+    """Value and Julia element type of a broadcast tree in the text form of the Tiled API
+    (`name(args...)`, `a<i>`, `s<i>`), evaluated like Base.Broadcast does on the CPU: every node in
+    its Julia result type (reference: `_eval_bc`, src/broadcast.jl:101-113; element types
+    Base.Broadcast.combine_eltypes as used in src/broadcast.jl:28).  `leaves` are numpy arrays in the
+    Julia shape; lower-rank leaves expand along trailing dimensions."""
+    pos = 0
+    rank = max([np.ndim(a) for a in leaves] + [0])
+
+    def parse():
+        nonlocal pos
+        j = pos
+        while pos < len(text) and (text[pos].isalnum() or text[pos] == "_"):
+            pos += 1
+        name = text[j:pos]
+        if pos < len(text) and text[pos] == "(":
+            pos += 1
+            args = [parse()]
+            while text[pos] == ",":
+                pos += 1
+                args.append(parse())
+            assert text[pos] == ")"
+            pos += 1
+            return apply(name, args)
+        if name[0] == "a":
+            a = np.asarray(leaves[int(name[1:])])
+            a = a.reshape(a.shape + (1,) * (rank - a.ndim))
+            return a, _NP_JL[a.dtype]
+        x = scalars[int(name[1:])]
+        t = _jl_scalar_type(x)
+        return np.asarray(x, dtype=_JL_NP[t]), t
+
+    def conv(v, t):
+        return v[0].astype(_JL_NP[t]) if v[1] != t else v[0]
+
+    def apply(name, args):
+        T = args[0][1]
+        for a in args[1:]:
+            T = jl_promote(T, a[1])
+        isf = T in _JL_FLOATS
+        if name in ("add", "sub"):
+            R = "Int64" if T == "Bool" else T
+            f = np.add if name == "add" else np.subtract
+            return f(conv(args[0], R), conv(args[1], R)).astype(_JL_NP[R]), R
+        if name == "mul":
+            a, b = conv(args[0], T), conv(args[1], T)
+            return (np.logical_and(a, b) if T == "Bool" else (a * b).astype(_JL_NP[T])), T
+        if name == "div":
+            R = T if isf else "Float64"
+            return (conv(args[0], R) / conv(args[1], R)).astype(_JL_NP[R]), R
+        if name == "neg":
+            R = "Int64" if T == "Bool" else T
+            return (-conv(args[0], R)).astype(_JL_NP[R]), R
+        if name == "pow":
+            b, x = args
+            R = b[1] if (b[1] in _JL_FLOATS and x[1] not in _JL_FLOATS) else T
+            if R in _JL_FLOATS:
+                return np.power(conv(b, R), conv(x, R)).astype(_JL_NP[R]), R
+            return np.power(conv(b, R), conv(x, R)).astype(_JL_NP[R]), R
+        if name in _TILED_MATH or name in ("atan2", "hypot"):
+            R = T if isf else "Float64"
+            # Julia evaluates Float16 functions in Float32 and rounds once (Base math.jl)
+            W = "Float32" if R == "Float16" else R
+            if name == "atan2":
+                r = np.arctan2(conv(args[0], W), conv(args[1], W))
+            elif name == "hypot":
+                r = np.hypot(conv(args[0], W), conv(args[1], W))
+            else:
+                r = _TILED_MATH[name](conv(args[0], W))
+            return np.asarray(r).astype(_JL_NP[R]), R
+        if name in _TILED_CMP:
+            return _TILED_CMP[name](conv(args[0], T), conv(args[1], T)), "Bool"
+        if name in ("abs", "abs2", "sign", "floor", "ceil", "round", "trunc", "identity"):
+            v = conv(args[0], T)
+            if T == "Bool" or name == "identity":
+                return v, T
+            f = {"abs": np.abs, "abs2": lambda q: q * q, "sign": np.sign, "floor": np.floor, "ceil": np.ceil,
+                 "round": np.rint, "trunc": np.trunc}[name]
+            return (f(v) if isf or name in ("abs", "abs2", "sign") else v).astype(_JL_NP[T]), T
+        if name in ("max", "min"):
+            return (_jl_max if name == "max" else _jl_min)(*np.broadcast_arrays(conv(args[0], T), conv(args[1], T))), T
+        if name in ("fma", "muladd"):
+            a, b, c = (conv(v, T) for v in args)
+            if isf and T != "Float64":   # one rounding: exact in float64 for Float32 / Float16 operands, then round
+                return (a.astype(np.float64) * b.astype(np.float64) + c.astype(np.float64)).astype(_JL_NP[T]), T
+            return (a * b + c).astype(_JL_NP[T]), T
+        if name == "clamp":
+            x, lo, hi = (conv(v, T) for v in args)
+            return np.where(x > hi, hi, np.where(x < lo, lo, x)).astype(_JL_NP[T]), T
+        if name == "copysign":
+            R = args[0][1]
+            a, b = conv(args[0], R), conv(args[1], R)
+            if R in _JL_FLOATS:
+                return np.copysign(a, b), R
+            return np.where(b < 0, -np.abs(a), np.abs(a)).astype(_JL_NP[R]), R
+        if name in ("isnan", "isinf", "isfinite", "signbit", "iszero"):
+            v = args[0][0]
+            if name == "iszero":
+                return v == 0, "Bool"
+            if v.dtype.kind != "f":
+                return np.broadcast_to({"isnan": False, "isinf": False, "isfinite": True}.get(name, False), v.shape) \
+                    if name != "signbit" else (v < 0 if v.dtype.kind == "i" else np.zeros(v.shape, bool)), "Bool"
+            return {"isnan": np.isnan, "isinf": np.isinf, "isfinite": np.isfinite, "signbit": np.signbit}[name](v), "Bool"
+        if name == "not":
+            v = conv(args[0], T)
+            return (np.logical_not(v) if T == "Bool" else np.invert(v)), T
+        if name in ("and", "or", "xor"):
+            assert not isf
+            f = {"and": np.bitwise_and, "or": np.bitwise_or, "xor": np.bitwise_xor}[name]
+            return f(conv(args[0], T), conv(args[1], T)), T
+        if name == "ifelse":
+            R = jl_promote(args[1][1], args[2][1])
+            return np.where(args[0][0], conv(args[1], R), conv(args[2], R)).astype(_JL_NP[R]), R
+        if name in ("div_int", "rem", "mod", "fld", "cld"):
+            R = "Int64" if T == "Bool" else T
+            a, b = conv(args[0], R), conv(args[1], R)
+            if R in _JL_FLOATS:
+                r = {"div_int": lambda: np.trunc(a / b), "rem": lambda: np.fmod(a, b), "mod": lambda: np.mod(a, b),
+                     "fld": lambda: np.floor(a / b), "cld": lambda: np.ceil(a / b)}[name]()
+            else:
+                q = np.floor_divide(a, b)
+                r = {"div_int": lambda: np.trunc(a / b).astype(a.dtype), "rem": lambda: np.fmod(a, b),
+                     "mod": lambda: np.mod(a, b), "fld": lambda: q,
+                     "cld": lambda: -np.floor_divide(-a, b)}[name]()
+            return np.asarray(r).astype(_JL_NP[R]), R
+        conv_names = {"f16": "Float16", "f32": "Float32", "f64": "Float64", "i32": "Int32", "i64": "Int64", "bool": "Bool"}
+        if name in conv_names:
+            R = conv_names[name]
+            v = args[0][0]
+            if R.startswith("Int") and v.dtype.kind == "f":
+                v = np.trunc(v)
+            return (v != 0 if R == "Bool" else v.astype(_JL_NP[R])), R
+        raise KeyError(name)
+
+    value, jl = parse()
+    assert pos == len(text)
+    return value, jl
+
+
+def tiled_broadcast(dest_shape, dest_type: str, text: str, leaves=(), scalars=()):
+    """`dest .= tree` for a destination of Julia shape `dest_shape` and element type `dest_type`
+    (src/broadcast.jl:75-92): axes must match or be 1 (DimensionMismatch -> ValueError), the value is
+    converted to the destination's type."""
+    rank = len(dest_shape)
+    for a in leaves:
+        sh = tuple(np.shape(a)) + (1,) * (rank - np.ndim(a))
+        for d, v in enumerate(sh):
+            if v != 1 and (d >= rank or v != dest_shape[d]):
+                raise ValueError("DimensionMismatch")
+    value, _ = tiled_eval(text, leaves, scalars)
+    value = np.asarray(value)
+    value = value.reshape(value.shape + (1,) * (rank - value.ndim)) if value.ndim <= rank else value.reshape(dest_shape)
+    return np.broadcast_to(value, dest_shape).astype(_JL_NP[dest_type])
+
+
+def tiled_mapreduce(f_text, op: str, A: np.ndarray, dims=None, init=None, scalars=()):
+    """`mapreduce(f, op, A; dims, init)` with the reference's result-type and `dims` rules
+    (src/mapreduce.jl:131-172): T = typeof(f(x)), ET = promote_op(op, T, T) -- `+` turns Bool into
+    Int64, "add_sum" / "mul_prod" (what sum / prod pass) also widen Int32 -- dimensions outside
+    1:ndims are ignored, reduced dimensions keep extent 1, `dims=None` (Julia's `:`) returns a
+    scalar.  Returns (value, Julia element type)."""
+    v, T = tiled_eval(f_text, (A,), scalars) if f_text else (np.asarray(A), _NP_JL[np.asarray(A).dtype])
+    v = np.broadcast_to(v, np.shape(A))
+    ET = T
+    if op in ("+", "add_sum") and T == "Bool":
+        ET = "Int64"
+    if op in ("add_sum", "mul_prod") and T in ("Int32", "Bool"):
+        ET = "Int64"
+    v = v.astype(_JL_NP[ET])
+    N = v.ndim
+    region = tuple(range(1, N + 1)) if dims is None else ((dims,) if isinstance(dims, (int, np.integer)) else tuple(dims))
+    axes = tuple(d - 1 for d in range(1, N + 1) if d in region)
+    if op in ("max", "min"):
+        # numpy's max / min propagate NaN like Julia's; ties between +-0.0 are not distinguished by value
+        r = (np.max if op == "max" else np.min)(v, axis=axes, keepdims=True) if axes else v
+    else:
+        f = {"+": np.add, "add_sum": np.add, "*": np.multiply, "mul_prod": np.multiply, "&": np.bitwise_and,
+             "|": np.bitwise_or}[op]
+        acc = np.float64 if ET in ("Float16", "Float32") else _JL_NP[ET]
+        r = f.reduce(v.astype(acc), axis=axes, keepdims=True).astype(_JL_NP[ET]) if axes else v
+    if init is not None:
+        i = _JL_NP[ET](init)
+        g = {"+": np.add, "add_sum": np.add, "*": np.multiply, "mul_prod": np.multiply, "max": np.maximum,
+             "min": np.minimum, "&": np.bitwise_and, "|": np.bitwise_or}[op]
+        r = g(i, r).astype(_JL_NP[ET])
+    if dims is None:
+        return r.reshape(-1)[0], ET
+    return r, ET
 
 
 # ---- example verify() criteria -------------------------------------------------------------

@@ -339,3 +339,92 @@ def test_fft_tables_and_brute_force_dft():
     x = np.arange(8, dtype=np.float64)[:, None] * (1 + 0.5j)
     brute = np.array([sum(x[n, 0] * np.exp(-2j * np.pi * k * n / 8) for n in range(8)) for k in range(8)])
     assert np.allclose(orc.fft_3stage(x, (2, 2, 2))[:, 0], brute, atol=1e-5)
+
+
+# ---- host-level Tiled broadcast / mapreduce ---------------------------------------------------------
+
+def test_jl_promote_known_julia_facts(orc):
+    """Facts of Julia's promotion (Base promotion.jl / bool.jl / float.jl), written out."""
+    facts = {("Int32", "Int64"): "Int64", ("Int64", "Float32"): "Float32", ("Int32", "Float16"): "Float16",
+             ("Float16", "Float32"): "Float32", ("Float32", "Float64"): "Float64", ("Bool", "Int32"): "Int32",
+             ("Bool", "Float16"): "Float16", ("Bool", "Bool"): "Bool", ("Int64", "Int64"): "Int64"}
+    for (a, b), want in facts.items():
+        assert orc.jl_promote(a, b) == want and orc.jl_promote(b, a) == want
+
+
+def test_tiled_eval_types_and_values_by_hand(orc):
+    a = np.array([1, -2, 3], np.int32)
+    b = np.array([2, 2, 2], np.int64)
+    v, t = orc.tiled_eval("div(a0,a1)", (a, b))
+    assert t == "Float64" and np.array_equal(v, [0.5, -1.0, 1.5])          # Int / Int is Float64
+    v, t = orc.tiled_eval("add(a0,a0)", (np.array([True, False]),))
+    assert t == "Int64" and np.array_equal(v, [2, 0])                      # true + true == 2
+    v, t = orc.tiled_eval("mul(a0,a1)", (np.array([True, False]), np.array([1.5, 2.5], np.float16)))
+    assert t == "Float16" and np.array_equal(v, np.array([1.5, 0], np.float16))
+    v, t = orc.tiled_eval("add(a0,s0)", (np.array([0.1], np.float32),), (1.0,))
+    assert t == "Float64" and v[0] == np.float64(np.float32(0.1)) + 1.0    # Float32 .+ 1.0 is Float64
+    v, t = orc.tiled_eval("add(a0,s0)", (np.array([0.1], np.float32),), (np.float32(1),))
+    assert t == "Float32" and v[0] == np.float32(0.1) + np.float32(1)
+    # Julia: div rounds toward zero, fld down, cld up, rem takes the dividend's sign, mod the divisor's
+    x, y = np.array([7, -7, 7, -7], np.int64), np.array([2, 2, -2, -2], np.int64)
+    for name, want in (("div_int", [3, -3, -3, 3]), ("fld", [3, -4, -4, 3]), ("cld", [4, -3, -3, 4]),
+                       ("rem", [1, -1, 1, -1]), ("mod", [1, 1, -1, -1])):
+        v, t = orc.tiled_eval(f"{name}(a0,a1)", (x, y))
+        assert t == "Int64" and np.array_equal(v, want), name
+    # max / min: NaN wins, +0.0 > -0.0
+    v, _ = orc.tiled_eval("max(a0,a1)", (np.array([np.nan, 1, -0.0], np.float32), np.array([1, np.nan, 0.0], np.float32)))
+    assert np.isnan(v[0]) and np.isnan(v[1]) and not np.signbit(v[2])
+    v, _ = orc.tiled_eval("min(a0,a1)", (np.array([-0.0], np.float32), np.array([0.0], np.float32)))
+    assert np.signbit(v[0])
+    # Float16 arithmetic rounds after every operation: (2048 + 1) + 1 stays 2048, 2048 + (1 + 1) is 2050
+    h = np.array([2048], np.float16)
+    one = np.array([1], np.float16)
+    assert orc.tiled_eval("add(add(a0,a1),a1)", (h, one))[0][0] == 2048
+    assert orc.tiled_eval("add(a0,add(a1,a1))", (h, one))[0][0] == 2050
+
+
+def test_tiled_broadcast_reference_cases(orc):
+    """Known answers of test/host/broadcast.jl: scalar fills (:175-183), 0-dim (:194-203), size-1
+    expansion only (:138-144), allocating with expansion (:166-173), shape mismatch (:112-122)."""
+    assert np.all(orc.tiled_broadcast((1000,), "Float32", "s0", (), (0,)) == 0)
+    assert np.all(orc.tiled_broadcast((33, 65), "Float32", "s0", (), (np.float32(2.5),)) == 2.5)
+    assert orc.tiled_broadcast((), "Float32", "add(a0,s0)", (np.array(2.0, np.float32),), (np.float32(1),))[()] == 3.0
+    A = np.arange(512, dtype=np.float32).reshape(1, 512)
+    got = orc.tiled_broadcast((32, 512), "Float32", "add(a0,s0)", (A,), (np.float32(1),))
+    assert np.array_equal(got, np.repeat(A + 1, 32, axis=0))
+    row, col = np.arange(128, dtype=np.float32).reshape(1, 128), np.arange(64, dtype=np.float32).reshape(64, 1)
+    v, _ = orc.tiled_eval("add(a0,a1)", (row, col))
+    assert v.shape == (64, 128) and v[5, 7] == 12
+    vec, mat = np.arange(64, dtype=np.float32), np.ones((64, 128), np.float32)
+    v, _ = orc.tiled_eval("add(a0,a1)", (vec, mat))                       # rank expansion along trailing dims
+    assert v.shape == (64, 128) and v[9, 100] == 10
+    for bad_dest, leaf in (((10,), np.zeros(11, np.float32)), ((8, 8), np.zeros((8, 16), np.float32))):
+        with pytest.raises(ValueError):
+            orc.tiled_broadcast(bad_dest, "Float32", "a0", (leaf,))
+
+
+def test_tiled_mapreduce_reference_cases_and_brute_force(orc):
+    """Known answers of test/host/mapreduce.jl (count == 4 :153-160, any / all :131-151, max of
+    fill(-5) == -5 :97-104, out-of-range dims ignored :47-57) and brute-force loops on a tiny array."""
+    c = np.zeros(1024, bool)
+    c[[0, 99, 499, 998]] = True
+    assert orc.tiled_mapreduce(None, "add_sum", c) == (4, "Int64")
+    assert orc.tiled_mapreduce(None, "|", np.zeros(1024, bool))[0] == False          # noqa: E712
+    assert orc.tiled_mapreduce(None, "|", c)[0] == True                             # noqa: E712
+    assert orc.tiled_mapreduce(None, "&", ~c)[0] == False                           # noqa: E712
+    assert orc.tiled_mapreduce(None, "max", np.full(1000, -5, np.float32)) == (-5.0, "Float32")
+    rng = np.random.default_rng(0)
+    A = rng.standard_normal((3, 4, 5)).astype(np.float32)
+    r, t = orc.tiled_mapreduce(None, "add_sum", A, dims=(2, 7))
+    assert t == "Float32" and r.shape == (3, 1, 5)
+    for i in range(3):
+        for k in range(5):
+            assert abs(r[i, 0, k] - sum(float(A[i, j, k]) for j in range(4))) < 1e-5
+    r, _ = orc.tiled_mapreduce("abs(a0)", "max", A, dims=(1, 3))
+    for j in range(4):
+        assert r[0, j, 0] == max(abs(A[i, j, k]) for i in range(3) for k in range(5))
+    assert orc.tiled_mapreduce(None, "add_sum", np.array([2**31 - 1, 1], np.int32)) == (2**31, "Int64")   # sum widens
+    assert orc.tiled_mapreduce(None, "+", np.array([3, 4], np.int32))[1] == "Int32"                       # reduce(+) does not
+    r, _ = orc.tiled_mapreduce(None, "mul_prod", np.full(17, 2, np.int32), dims=())
+    assert r.shape == (17,) and np.all(r == 2)                                      # no reduced dimension: map
+    assert orc.tiled_mapreduce(None, "add_sum", A, init=100.0)[0] == pytest.approx(100 + A.astype(np.float64).sum(), rel=1e-6)

@@ -222,6 +222,34 @@ def bench_kernels(ct, which, cpu, nruns=NRUNS, warmup=WARMUP):
             res["fft"]["cpu_ms"] = round(_cpu_time(lambda: np.fft.fft(x, axis=1)), 2)
             res["fft"]["cpu_note"] = "numpy.fft (pocketfft) on the same complex64 batch, 1 thread (the reference verifies against FFTW)"
 
+    if want("tiled"):
+        # Host-level Tiled broadcast / mapreduce (src/broadcast.jl, src/mapreduce.jl): kernels generated at run time.
+        from cutile_jl_amd import tiled as T
+        n = 1 << 27
+        A = torch.rand(n, device="cuda"); B = torch.rand(n, device="cuda"); C = torch.empty(n, device="cuda")
+        M, Cm = A.view(8192, 16384), C.view(8192, 16384)          # Julia (16384, 8192)
+        row = torch.rand(8192, 1, device="cuda")                  # Julia (1, 8192)
+        legs = [
+            ("tiled_broadcast_add", "Tiled(C) .= Tiled(A) .+ Tiled(B), 2^27 f32", lambda: T.Tiled(C).assign(T.Tiled(A) + T.Tiled(B)), 12 * n),
+            ("tiled_broadcast_fused", "Tiled(C) .= A .+ A .* sin.(B), 2^27 f32, one fused kernel",
+             lambda: T.Tiled(C).assign(T.Tiled(A) + T.Tiled(A) * T.sin(T.Tiled(B))), 12 * n),
+            ("tiled_broadcast_expand", "Tiled(C) .= M .+ row, M (16384, 8192), row (1, 8192) f32", lambda: T.Tiled(Cm).assign(T.Tiled(M) + T.Tiled(row)), 8 * n),
+            ("tiled_sum_all", "sum(Tiled(A); dims=1), 2^27 f32 (two passes)", lambda: T.sum(T.Tiled(A), dims=1), 4 * n),
+            ("tiled_sum_dims1", "sum(Tiled(M); dims=1), (16384, 8192) f32: contiguous runs", lambda: T.sum(T.Tiled(M), dims=1), 4 * n),
+            ("tiled_sum_dims2", "sum(Tiled(M); dims=2), (16384, 8192) f32: strided (two passes)", lambda: T.sum(T.Tiled(M), dims=2), 4 * n),
+            ("tiled_maximum_dims2", "maximum(Tiled(M); dims=2), NaN-propagating", lambda: T.maximum(T.Tiled(M), dims=2), 4 * n),
+        ]
+        for key, name, fn, nbytes in legs:
+            res[key] = _entry(name, fn, nbytes, "GB/s", "hbm", HBM_PEAK_GBS, "f32", nruns, warmup)
+            res[key]["variant"] = ct.last_variant()
+        if cpu:
+            a, b = A[: n // 16].cpu().numpy(), B[: n // 16].cpu().numpy()
+            res["tiled_broadcast_fused"]["cpu_ms"] = round(_cpu_time(lambda: a + a * np.sin(b)) * 16, 1)
+            res["tiled_broadcast_fused"]["cpu_note"] = "numpy a + a*sin(b) on 1/16 of the elements x16, 1 thread"
+            res["tiled_sum_all"]["cpu_ms"] = round(_cpu_time(lambda: a.sum()) * 16, 1)
+            res["tiled_sum_all"]["cpu_note"] = "numpy sum on 1/16 of the elements x16, 1 thread"
+        del A, B, C, M, Cm
+
     if want("moe"):
         d = moe.prepare(benchmark=True, topk=2, router="top2_logits")
         flop = moe.metric(d)[0]

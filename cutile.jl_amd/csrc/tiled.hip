@@ -279,22 +279,26 @@ int broadcast_impl(const mi_tile_array* dest, const char* text, const mi_tile_ar
         if (keep0[i]) { snprintf(buf, sizeof buf, "    L%d r%d[U][V] = {};\n", i, i); g += buf; }
         else { snprintf(buf, sizeof buf, "    const car<%s> c%d = to_car(ldg<false>(p%d));\n", tag(leaf_dt[i]), i, i); g += buf; }
     }
-    g += "#pragma unroll\n    for (int u = 0; u < U; ++u) {\n"
-         "        const long long i0 = (((long long)bx * U + u) * TX + tx) * V;\n"
-         "        if (i0 < n0) {\n";
-    for (int i = 0; i < e.leaves_used; ++i)
-        if (keep0[i]) {
-            snprintf(buf, sizeof buf, "            load_run<L%d, V, %s, NT>(p%d + i0 * A.leaf[%d].st[0], n0 - i0, A.leaf[%d].st[0], r%d[u]);\n", i,
-                     vec_l[i] ? "true" : "false", i, i, i, i);
-            g += buf;
-        }
-    g += "        }\n    }\n"
-         "#pragma unroll\n    for (int u = 0; u < U; ++u) {\n"
-         "        const long long i0 = (((long long)bx * U + u) * TX + tx) * V;\n"
-         "        if (i0 < n0) {\n"
-         "            DST o[V];\n"
-         "#pragma unroll\n            for (int q = 0; q < V; ++q) o[q] = to_sto<DST>(eval(";
-    {
+    // The block body is emitted twice: without predicates for blocks that lie wholly inside
+    // dimension 0 (all loads of a lane are issued before the first use), with them for the last one.
+    auto emit_block = [&](bool guard) {
+        const char* left = guard ? "n0 - i0" : "(long long)V";
+        g += "#pragma unroll\n        for (int u = 0; u < U; ++u) {\n"
+             "            const long long i0 = (((long long)bx * U + u) * TX + tx) * V;\n";
+        if (guard) g += "            if (i0 < n0) {\n";
+        for (int i = 0; i < e.leaves_used; ++i)
+            if (keep0[i]) {
+                snprintf(buf, sizeof buf, "            load_run<L%d, V, %s, NT>(p%d + i0 * A.leaf[%d].st[0], %s, A.leaf[%d].st[0], r%d[u]);\n", i,
+                         vec_l[i] ? "true" : "false", i, i, left, i, i);
+                g += buf;
+            }
+        if (guard) g += "            }\n";
+        g += "        }\n"
+             "#pragma unroll\n        for (int u = 0; u < U; ++u) {\n"
+             "            const long long i0 = (((long long)bx * U + u) * TX + tx) * V;\n";
+        if (guard) g += "            if (i0 < n0) {\n";
+        g += "            DST o[V];\n"
+             "#pragma unroll\n            for (int q = 0; q < V; ++q) o[q] = to_sto<DST>(eval(";
         bool first = true;
         for (int i = 0; i < e.leaves_used; ++i) {
             if (keep0[i]) snprintf(buf, sizeof buf, "%sto_car(r%d[u][q])", first ? "" : ", ", i);
@@ -303,10 +307,17 @@ int broadcast_impl(const mi_tile_array* dest, const char* text, const mi_tile_ar
             first = false;
         }
         for (int i = 0; i < e.scalars_used; ++i) { snprintf(buf, sizeof buf, "%ss%d", first ? "" : ", ", i); g += buf; first = false; }
-    }
-    g += "));\n"
-         "            store_run<DST, V, VECD, NT>(dp + i0 * A.dst[0], n0 - i0, A.dst[0], o);\n"
-         "        }\n    }\n}\n";
+        g += "));\n";
+        snprintf(buf, sizeof buf, "            store_run<DST, V, VECD, NT>(dp + i0 * A.dst[0], %s, A.dst[0], o);\n", left);
+        g += buf;
+        if (guard) g += "            }\n";
+        g += "        }\n";
+    };
+    g += "    if (((long long)bx + 1) * U * TX * V <= n0) {\n";
+    emit_block(false);
+    g += "    } else {\n";
+    emit_block(true);
+    g += "    }\n}\n";
 
     hipFunction_t fn = nullptr;
     MI_CHECK(compile(g, "tiled_bc", &fn));
@@ -338,6 +349,7 @@ struct MrArgs {
     long long P;
     long long nbx;
     long long nk;        // number of outputs (partials of split p start at nk * p in the column shape)
+    long long chunk;     // reduced indices per split: split p owns [p * chunk, (p + 1) * chunk)
     double sf[kMaxScalars];
     long long si[kMaxScalars];
 };
@@ -347,9 +359,14 @@ struct MrArgs {
 // order, the reduced index space over the reduced ones; both are unpacked with 32-bit divisions
 // that the compiler drops for dimensions of the other role.
 const char* const kRunKernel = R"SRC(
+// LANES lanes (a power of two up to the workgroup) share one output; a workgroup holds T / LANES outputs.
 extern "C" __global__ __launch_bounds__(T) void tiled_mr(Args A) {
+    constexpr int G = T / LANES;
     const unsigned P = (unsigned)A.P;
-    const unsigned p = blockIdx.x % P, o = blockIdx.x / P;
+    const unsigned p = blockIdx.x % P;
+    const unsigned o = (blockIdx.x / P) * G + threadIdx.x / LANES;
+    const unsigned lane = threadIdx.x % LANES;
+    const bool live = o < (unsigned long long)A.nk;
     long long soff = 0, doff = 0;
     {
         unsigned rest = o;
@@ -368,12 +385,15 @@ extern "C" __global__ __launch_bounds__(T) void tiled_mr(Args A) {
     unsigned long long nq = nvec0;
 #pragma unroll
     for (int d = 1; d < 4; ++d) if ((RMASK >> d) & 1) nq *= (unsigned long long)A.size[d];
+    unsigned long long qend = (unsigned long long)(p + 1) * (unsigned long long)A.chunk;
+    if (qend > nq) qend = nq;
+    if (!live) qend = 0;
     SCALARS
     AC acc[V];
 #pragma unroll
     for (int e = 0; e < V; ++e) acc[e] = neutral();
 #pragma unroll UNR
-    for (unsigned long long q = (unsigned long long)p * T + threadIdx.x; q < nq; q += (unsigned long long)P * T) {
+    for (unsigned long long q = (unsigned long long)p * (unsigned long long)A.chunk + lane; q < qend; q += LANES) {
         unsigned v0 = (unsigned)q;
         long long off = 0;
         if constexpr ((RMASK & 14) != 0) {
@@ -397,14 +417,14 @@ extern "C" __global__ __launch_bounds__(T) void tiled_mr(Args A) {
 #pragma unroll
     for (int e = 1; e < V; ++e) a = redop(a, acc[e]);
 #pragma unroll
-    for (int m = 32; m >= 1; m >>= 1) a = redop(a, xor_lane(a, m));
-    if constexpr (T > 64) {
+    for (int m = (LANES < 64 ? LANES : 64) / 2; m >= 1; m >>= 1) a = redop(a, xor_lane(a, m));
+    if constexpr (LANES > 64) {
         __shared__ AC sh[T / 64];
         if ((threadIdx.x & 63) == 0) sh[threadIdx.x >> 6] = a;
         __syncthreads();
-        if (threadIdx.x == 0) for (int w = 1; w < T / 64; ++w) a = redop(a, sh[w]);
+        if (lane == 0) for (int w = 1; w < LANES / 64; ++w) a = redop(a, sh[(threadIdx.x >> 6) + w]);
     }
-    if (threadIdx.x == 0) {
+    if (lane == 0 && live) {
         if constexpr (OUT_WS) ((AC*)A.dst)[p + (unsigned long long)P * o] = a;
         else ((DST*)A.dst)[doff] = to_sto<DST>(a);
     }
@@ -441,9 +461,11 @@ extern "C" __global__ __launch_bounds__(TX * TY) void tiled_mr(Args A) {
     AC acc[V];
 #pragma unroll
     for (int e = 0; e < V; ++e) acc[e] = neutral();
+    unsigned long long qend = (unsigned long long)(p + 1) * (unsigned long long)A.chunk;
+    if (qend > nq) qend = nq;
     if (live) {
 #pragma unroll UNR
-        for (unsigned long long q = (unsigned long long)p * TY + ty; q < nq; q += (unsigned long long)P * TY) {
+        for (unsigned long long q = (unsigned long long)p * (unsigned long long)A.chunk + ty; q < qend; q += TY) {
             unsigned rest = (unsigned)q;
             long long off = 0;
 #pragma unroll
@@ -523,10 +545,23 @@ struct MrShape {
     bool red(int d) const { return (rmask >> d) & 1; }
 };
 struct MrPlan {
-    int V, T, TX, TY, UNR;
+    int V, T, TX, TY, UNR, LANES;
     bool vec, vecd, nt;
-    int64_t P, nbx, blocks, nk;
+    int64_t P, nbx, blocks, nk, chunk;
 };
+
+// Tuning overrides (environment): workgroups a split reduction aims for, iterations a lane should
+// at least have, unroll factor of the accumulation loop.
+int knob(const char* name, int dflt) {
+    const char* e = getenv(name);
+    const int v = e ? atoi(e) : 0;
+    return v > 0 ? v : dflt;
+}
+int knob_blocks() { static const int v = knob("MI_TILED_BLOCKS", 2048); return v; }
+int knob_column_blocks() { static const int v = knob("MI_TILED_COLUMN_BLOCKS", 2048); return v; }
+int knob_min_tx() { static const int v = knob("MI_TILED_MIN_TX", 64); return v; }
+int knob_iters() { static const int v = knob("MI_TILED_ITERS", 8); return v; }
+int knob_unroll() { static const int v = knob("MI_TILED_UNROLL", 4); return v; }
 
 // Launch geometry of one pass; `allow_split` false for the pass over the partials.
 int plan_pass(const MrShape& sh, int src_dt, int acc_dt, const void* src, const void* dst, bool allow_split, MrPlan* pl) {
@@ -543,20 +578,38 @@ int plan_pass(const MrShape& sh, int src_dt, int acc_dt, const void* src, const 
     for (int d = 1; d < 4; ++d) (sh.red(d) ? nred : nkept) *= sh.size[d];
     for (int d = 0; d < 4; ++d) if (sh.size[d] > 0x7fffffffLL) return MI_E_GRID;
     pl->nt = stream_hint(srcn * es);
-    pl->UNR = 4;
+    pl->UNR = knob_unroll();
     pl->vecd = false;
     if (sh.run()) {
         const int64_t nq = nvec0 * nred, nk = nkept;
         if (nq >= (1ll << 32) || nk > 0x7fffffffLL) return MI_E_GRID;
-        pl->T = nq >= 1024 ? 256 : 64;
+        // lanes per output: at least four vectors each, more when there are too few outputs to
+        // fill the chip otherwise
+        int lanes = 1;
+        while (lanes < 256 && (int64_t)lanes * 8 <= nq) lanes <<= 1;
+        while (lanes < 256 && lanes < nq && nk * lanes < (int64_t)256 * 1024) lanes <<= 1;
+        pl->LANES = lanes;
+        pl->T = 256;
         pl->TX = pl->T; pl->TY = 1;
         int64_t P = 1;
-        if (allow_split) { P = cld(nq, (int64_t)pl->T * 8); const int64_t want = nk >= 2048 ? 1 : 2048 / (nk ? nk : 1); if (P > want) P = want; if (P < 1) P = 1; }
-        pl->P = P; pl->nbx = 1; pl->nk = nk; pl->blocks = nk * P;
+        if (allow_split && lanes == 256) {
+            P = cld(nq, (int64_t)lanes * knob_iters());
+            const int64_t want = nk >= knob_blocks() ? 1 : knob_blocks() / (nk ? nk : 1);
+            if (P > want) P = want;
+            if (P < 1) P = 1;
+        }
+        pl->chunk = cld(cld(nq, P), (int64_t)lanes) * lanes;
+        P = pl->chunk ? cld(nq, pl->chunk) : 1;
+        if (P < 1) P = 1;
+        pl->P = P; pl->nbx = 1; pl->nk = nk; pl->blocks = cld(nk, (int64_t)(pl->T / lanes)) * P;
     } else {
         const int64_t nq = nred, nk = sh.size[0] * nkept;
         if (nq >= (1ll << 32) || nkept > 0x7fffffffLL) return MI_E_GRID;
-        pl->TX = nvec0 >= 256 ? 256 : pow2ceil(nvec0);
+        // Lanes along dimension 0: as wide as the extent allows, narrowed (down to knob_min_tx) while
+        // that leaves the chip short of workgroups and the reduced range can use the freed rows.
+        int tx = nvec0 >= 256 ? 256 : pow2ceil(nvec0);
+        while (tx > knob_min_tx() && cld(nvec0, (int64_t)tx) * nkept < 512 && (int64_t)(256 / tx) * 2 <= nq) tx >>= 1;
+        pl->TX = tx;
         int ty = 256 / pl->TX;
         while (ty > 1 && ty > nq) ty >>= 1;
         pl->TY = ty;
@@ -565,8 +618,16 @@ int plan_pass(const MrShape& sh, int src_dt, int acc_dt, const void* src, const 
         if (pl->nbx < 1) pl->nbx = 1;
         const int64_t b0 = pl->nbx * nkept;
         int64_t P = 1;
-        if (allow_split) { P = cld(nq, (int64_t)pl->TY * 8); const int64_t want = b0 >= 2048 ? 1 : 2048 / (b0 ? b0 : 1); if (P > want) P = want; if (P < 1) P = 1; }
-        pl->P = P; pl->nk = nk; pl->blocks = b0 * P;
+        if (allow_split) {
+            P = cld(nq, (int64_t)pl->TY * knob_iters());
+            const int64_t want = b0 >= knob_column_blocks() ? 1 : knob_column_blocks() / (b0 ? b0 : 1);
+            if (P > want) P = want;
+            if (P < 1) P = 1;
+        }
+        pl->chunk = cld(cld(nq, P), (int64_t)pl->TY) * pl->TY;
+        P = pl->chunk ? cld(nq, pl->chunk) : 1;
+        if (P < 1) P = 1;
+        pl->P = P; pl->nk = nk; pl->blocks = b0 * P; pl->LANES = 1;
         const int dvb = V * ds < 16 ? V * ds : 16;
         pl->vecd = sh.dstr[0] == 1 && ((uintptr_t)dst) % (uintptr_t)dvb == 0;
         for (int d = 1; d < 4; ++d) if (!sh.red(d) && (sh.dstr[d] * ds) % dvb) pl->vecd = false;
@@ -603,14 +664,14 @@ std::string mr_source(const Expr& e, const int32_t* scal_dt, int src_dt, int acc
     std::string g;
     char buf[512];
     snprintf(buf, sizeof buf,
-             "constexpr int SRC = %s, ACC = %s, V = %d, T = %d, TX = %d, TY = %d, RMASK = %d;\n"
+             "constexpr int SRC = %s, ACC = %s, V = %d, T = %d, TX = %d, TY = %d, RMASK = %d, LANES = %d;\n"
              "constexpr bool NT = %s, VEC = %s, VECD = %s, OUT_WS = %s;\n#define UNR %d\n",
-             tag(src_dt), tag(acc_dt), pl.V, pl.T, pl.TX, pl.TY, sh.rmask, pl.nt ? "true" : "false", pl.vec ? "true" : "false",
+             tag(src_dt), tag(acc_dt), pl.V, pl.T, pl.TX, pl.TY, sh.rmask, pl.LANES, pl.nt ? "true" : "false", pl.vec ? "true" : "false",
              pl.vecd ? "true" : "false", out_ws ? "true" : "false", pl.UNR);
     g += buf;
     snprintf(buf, sizeof buf, "typedef %s SST;\ntypedef %s DST;\ntypedef car<ACC> AC;\n", storage(src_dt), storage(acc_dt));
     g += buf;
-    g += "struct Args { const void* src; void* dst; long long size[4]; long long sst[4]; long long dstr[4]; long long P; long long nbx; long long nk; "
+    g += "struct Args { const void* src; void* dst; long long size[4]; long long sst[4]; long long dstr[4]; long long P; long long nbx; long long nk; long long chunk; "
          "double sf[8]; long long si[8]; };\n";
     int32_t leaf_dt[1] = {src_dt};
     g += "__device__ __forceinline__ AC mapf(" + eval_params(e, leaf_dt, scal_dt) + ") {\n" + emit_body(e);
@@ -642,6 +703,7 @@ int run_pass(const Expr& e, const int32_t* scal_dt, const ScalarArgs& sa, int sr
     a.P = pl.P;
     a.nbx = pl.nbx;
     a.nk = pl.nk;
+    a.chunk = pl.chunk;
     memcpy(a.sf, sa.sf, sizeof a.sf);
     memcpy(a.si, sa.si, sizeof a.si);
     return launch(fn, pl.blocks, pl.T, &a, sizeof a, stream);
@@ -676,7 +738,7 @@ int mapreduce_impl(const mi_tile_array* dest, const mi_tile_array* src, const ch
 
     char buf[96];
     if (p1.P == 1) {
-        snprintf(buf, sizeof buf, "tiled_mr_%s_t%d_ty%d", sh.run() ? "run" : "column", p1.T, p1.TY);
+        snprintf(buf, sizeof buf, "tiled_mr_%s_l%d_ty%d", sh.run() ? "run" : "column", p1.LANES, p1.TY);
         set_variant_text(buf);
         return run_pass(e, scal_dt, sa, src->dtype, dest->dtype, op, sh, p1, src->ptr, dest->ptr, false, stream);
     }
@@ -703,7 +765,7 @@ int mapreduce_impl(const mi_tile_array* dest, const mi_tile_array* src, const ch
     MI_CHECK(parse_expr("a0", id));
     int32_t l2[1] = {cdt};
     MI_CHECK(infer_types(id, l2, 1, scal_dt, 0));
-    snprintf(buf, sizeof buf, "tiled_mr_%s_t%d_ty%d_split%lld", sh.run() ? "run" : "column", p1.T, p1.TY, (long long)p1.P);
+    snprintf(buf, sizeof buf, "tiled_mr_%s_l%d_ty%d_split%lld", sh.run() ? "run" : "column", p1.LANES, p1.TY, (long long)p1.P);
     set_variant_text(buf);
     ScalarArgs none;
     memset(&none, 0, sizeof none);

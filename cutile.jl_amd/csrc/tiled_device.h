@@ -137,11 +137,11 @@ template <int DT> __device__ __forceinline__ bool sgn(car<DT> a) {
     else return a < 0;
 }
 template <int DT> __device__ __forceinline__ car<DT> f_max(car<DT> a, car<DT> b) {
-    if constexpr (is_flt<DT>) { if (a != a) return a; if (b != b) return b; return a > b ? a : b > a ? b : sgn<DT>(a) ? b : a; }
+    if constexpr (is_flt<DT>) return __builtin_elementwise_maximum(a, b);   // IEEE 754-2019 maximum: v_maximum3_f32
     else return a > b ? a : b;
 }
 template <int DT> __device__ __forceinline__ car<DT> f_min(car<DT> a, car<DT> b) {
-    if constexpr (is_flt<DT>) { if (a != a) return a; if (b != b) return b; return a < b ? a : b < a ? b : sgn<DT>(a) ? a : b; }
+    if constexpr (is_flt<DT>) return __builtin_elementwise_minimum(a, b);
     else return a < b ? a : b;
 }
 template <int DT> __device__ __forceinline__ car<DT> f_fma(car<DT> a, car<DT> b, car<DT> c) {

@@ -39,6 +39,7 @@ mi_dtype(::Type{Float64}) = Int32(1)
 mi_dtype(::Type{Float16}) = Int32(2)
 mi_dtype(::Type{Int32})   = Int32(5)
 mi_dtype(::Type{Int64})   = Int32(6)
+mi_dtype(::Type{Bool})    = Int32(7)
 # BFloat16 (BFloat16s.jl / Core.BFloat16) = 3 and Float8_E4M3FN (DLFP8Types.jl) = 4: add the
 # methods in a package extension, the way ext/DLFP8TypesExt.jl adds the cuTile mapping.
 mi_dtype(T::Type) = T === UInt8 ? Int32(4) :   # raw e4m3fn bytes
@@ -279,6 +280,62 @@ function fft_kernel(x_packed_in, y_packed_out, W0, W1, W2, T0, T1, N::Integer, F
         (Ref{MiTileArray}, Ref{MiTileArray}, Ref{MiTileArray}, Ref{MiTileArray}, Ref{MiTileArray},
          Ref{MiTileArray}, Ref{MiTileArray}, Cint, Cint, Cint, Cint, Cint, Cint, Ptr{Cvoid}),
         d[1], d[2], d[3], d[4], d[5], d[6], d[7], N, F0, F1, F2, BS, D, stream))
+end
+
+# ---- host-level Tiled broadcast / mapreduce (src/broadcast.jl, src/mapreduce.jl) ---------
+
+# == struct mi_tile_scalar: dtype, reserved, 8-byte value (Float64 bits or Int64)
+struct MiTileScalar
+    dtype::Int32
+    reserved::Int32
+    bits::UInt64
+end
+MiTileScalar(x::AbstractFloat) = MiTileScalar(mi_dtype(typeof(x)), 0, reinterpret(UInt64, Float64(x)))
+MiTileScalar(x::Integer) = MiTileScalar(mi_dtype(typeof(x)), 0, reinterpret(UInt64, Int64(x)))
+MiTileScalar(x::Bool) = MiTileScalar(mi_dtype(Bool), 0, UInt64(x))
+
+const MI_OP_ADD, MI_OP_MUL, MI_OP_MAX, MI_OP_MIN, MI_OP_AND, MI_OP_OR = Int32.(0:5)
+opcode(::typeof(+)) = MI_OP_ADD
+opcode(::typeof(Base.add_sum)) = MI_OP_ADD
+opcode(::typeof(*)) = MI_OP_MUL
+opcode(::typeof(Base.mul_prod)) = MI_OP_MUL
+opcode(::typeof(max)) = MI_OP_MAX
+opcode(::typeof(min)) = MI_OP_MIN
+opcode(::typeof(&)) = MI_OP_AND
+opcode(::typeof(|)) = MI_OP_OR
+
+"`dest .= expr(leaves..., scalars...)`; `expr` is the prefix text form described in mi355tile.h."
+function tiled_broadcast(dest, expr::AbstractString, leaves::AbstractVector, scalars::AbstractVector{<:Number};
+                         stream::Ptr{Cvoid}=C_NULL)
+    descs = [descriptor(a) for a in leaves]
+    ptrs = [pointer(descs, i) for i in eachindex(descs)]
+    sc = MiTileScalar[MiTileScalar(x) for x in scalars]
+    d = ref(descriptor(dest))
+    GC.@preserve dest leaves descs ptrs sc check(ccall((:mi_tiled_broadcast, libmi355tile), Cint,
+        (Ref{MiTileArray}, Cstring, Ptr{Ptr{MiTileArray}}, Cint, Ptr{MiTileScalar}, Cint, Ptr{Cvoid}),
+        d, expr, ptrs, length(ptrs), sc, length(sc), stream))
+    return dest
+end
+
+"Bytes of device workspace `tiled_mapreduce` needs for these shapes (0 for most)."
+function tiled_mapreduce_workspace(dest, src, op::Integer)
+    n = Ref{Int64}(0)
+    check(ccall((:mi_tiled_mapreduce_workspace, libmi355tile), Cint,
+        (Ref{MiTileArray}, Ref{MiTileArray}, Cint, Ref{Int64}), ref(descriptor(dest)), ref(descriptor(src)), op, n))
+    return n[]
+end
+
+"`dest = reduce(op, f.(src))` over the dimensions where `dest` has extent 1; `f_expr === nothing` is identity."
+function tiled_mapreduce(dest, src, f_expr::Union{Nothing,AbstractString}, scalars::AbstractVector{<:Number}, op::Integer,
+                         workspace=nothing; stream::Ptr{Cvoid}=C_NULL)
+    sc = MiTileScalar[MiTileScalar(x) for x in scalars]
+    ws = workspace === nothing ? C_NULL : Ptr{Cvoid}(UInt(pointer(workspace)))
+    nws = workspace === nothing ? 0 : sizeof(workspace)
+    GC.@preserve dest src sc workspace check(ccall((:mi_tiled_mapreduce, libmi355tile), Cint,
+        (Ref{MiTileArray}, Ref{MiTileArray}, Cstring, Ptr{MiTileScalar}, Cint, Cint, Ptr{Cvoid}, Int64, Ptr{Cvoid}),
+        ref(descriptor(dest)), ref(descriptor(src)), f_expr === nothing ? C_NULL : f_expr, sc, length(sc), op, ws, nws,
+        stream))
+    return dest
 end
 
 end # module

@@ -226,15 +226,17 @@ def _mr(ct, dest, src, f, op, scalars=()):
 def test_generated_reduction_kernels_compile(ct, dry_run):
     z = torch.zeros
     rc, ws = _mr(ct, z(1), z(1024), None, T.MI_OP_ADD)
-    assert rc == 0 and ws == 0 and ct.last_variant() == "tiled_mr_run_t64_ty1"
+    assert rc == 0 and ws == 0 and ct.last_variant().startswith("tiled_mr_run_l256")
     rc, ws = _mr(ct, z(1), z(1 << 24), None, T.MI_OP_ADD)
-    assert rc == 0 and ws == 2048 * 4 and "split2048" in ct.last_variant()
+    assert rc == 0 and ws > 0 and ws % 4 == 0 and "split" in ct.last_variant()
     rc, ws = _mr(ct, z(256, 1), z(256, 128), None, T.MI_OP_ADD)             # Julia dims=1
     assert rc == 0 and ws == 0 and "run" in ct.last_variant()
     rc, ws = _mr(ct, z(1, 4096), z(100000, 4096), None, T.MI_OP_MAX)         # Julia dims=2
-    assert rc == 0 and ws == 512 * 4096 * 4 and "column" in ct.last_variant()
+    assert rc == 0 and ws > 0 and ws % (4096 * 4) == 0 and "column" in ct.last_variant()
     rc, _ = _mr(ct, z(1, 16, 1), z(8, 16, 32), "abs2(a0)", T.MI_OP_ADD)      # Julia dims=(1,3)
     assert rc == 0
+    rc, ws = _mr(ct, z(1 << 20, 1), z(1 << 20, 8), None, T.MI_OP_ADD)        # short runs: one lane per output
+    assert rc == 0 and ws == 0 and ct.last_variant().startswith("tiled_mr_run_l1_")
     rc, _ = _mr(ct, z(8, 1, 32), z(8, 16, 32), None, T.MI_OP_MIN)            # Julia dims=2
     assert rc == 0 and "column" in ct.last_variant()
     for dt, op in ((torch.int32, T.MI_OP_MUL), (torch.int64, T.MI_OP_AND), (torch.bool, T.MI_OP_OR), (torch.float64, T.MI_OP_MIN),

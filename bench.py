@@ -250,6 +250,22 @@ def bench_kernels(ct, which, cpu, nruns=NRUNS, warmup=WARMUP):
             res["tiled_sum_all"]["cpu_note"] = "numpy sum on 1/16 of the elements x16, 1 thread"
         del A, B, C, M, Cm
 
+    if want("rng"):
+        # Host-level Philox2x32-7 fills (src/language/random.jl:759-818): write-only streams.
+        from cutile_jl_amd import random as R
+        n = 1 << 27
+        out = torch.empty(n, device="cuda")
+        rng = R.RNG(42)
+        for key, name, fn in (("rng_rand_f32", "Random.rand!(RNG, A), 2^27 f32", lambda: R.rand_(rng, out)),
+                              ("rng_randn_f32", "Random.randn!(RNG, A), 2^27 f32 (Box-Muller)", lambda: R.randn_(rng, out))):
+            res[key] = _entry(name, fn, 4 * n, "GB/s", "hbm", HBM_PEAK_GBS, "u32" if "rand_f32" in key else "f32", nruns, warmup)
+            res[key]["variant"] = ct.last_variant()
+        if cpu:
+            g = np.random.Generator(np.random.Philox(42))
+            res["rng_rand_f32"]["cpu_ms"] = round(_cpu_time(lambda: g.random(n // 16, dtype=np.float32)) * 16, 1)
+            res["rng_rand_f32"]["cpu_note"] = "numpy Generator(Philox) float32 uniforms, 1/16 of the elements x16, 1 thread"
+        del out
+
     if want("moe"):
         d = moe.prepare(benchmark=True, topk=2, router="top2_logits")
         flop = moe.metric(d)[0]

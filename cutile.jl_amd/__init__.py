@@ -20,7 +20,7 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 # MI355TILE_LIB selects another build of the same library (e.g. an experimental variant).
 LIB_PATH = os.environ.get("MI355TILE_LIB") or os.path.join(_HERE, "libmi355tile.so")
 
-MI_F32, MI_F64, MI_F16, MI_BF16, MI_F8E4M3FN, MI_I32, MI_I64, MI_BOOL = range(8)
+MI_F32, MI_F64, MI_F16, MI_BF16, MI_F8E4M3FN, MI_I32, MI_I64, MI_BOOL, MI_I8, MI_I16 = range(10)
 MI_MAX_RANK = 4
 
 # error codes of include/mi355tile.h
@@ -85,6 +85,8 @@ _SIGNATURES = {
     "mi_tiled_mapreduce_workspace": ([_A, _A, _i, ctypes.POINTER(ctypes.c_int64)], _i),
     "mi_tiled_mapreduce_eltype": ([ctypes.c_char_p, ctypes.c_int32, ctypes.POINTER(ctypes.c_int32), _i, _i, _i,
                                    ctypes.POINTER(ctypes.c_int32)], _i),
+    "mi_rng_fill": ([_A, ctypes.c_uint32, ctypes.c_uint32, _i, _vp], _i),
+    "mi_rng_advance_counter": ([ctypes.POINTER(ctypes.c_uint32), ctypes.POINTER(ctypes.c_uint32), ctypes.c_int64], _i),
     "mi_tiled_set_dry_run": ([_i], _i),
     "mi_tiled_compile_count": ([], _i),
 }

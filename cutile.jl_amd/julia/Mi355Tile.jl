@@ -338,4 +338,21 @@ function tiled_mapreduce(dest, src, f_expr::Union{Nothing,AbstractString}, scala
     return dest
 end
 
+# ---- host-level RNG fills (src/language/random.jl:759-818) -------------------------------
+
+mi_dtype(::Type{Int8})  = Int32(8)
+mi_dtype(::Type{Int16}) = Int32(9)
+mi_dtype(::Type{UInt16}) = Int32(9)
+mi_dtype(::Type{UInt32}) = Int32(5)
+mi_dtype(::Type{UInt64}) = Int32(6)
+
+"Fill `A` with the Philox2x32-7 stream of `cuTile.RNG(seed, counter)`; dist 0 = rand, 1 = randn, 2 = randexp."
+function rng_fill(A, seed::UInt32, counter::UInt32, dist::Integer; stream::Ptr{Cvoid}=C_NULL)
+    T = eltype(A)
+    d = ref(descriptor(A; dtype = T === UInt8 ? Int32(8) : mi_dtype(T)))
+    GC.@preserve A check(ccall((:mi_rng_fill, libmi355tile), Cint,
+        (Ref{MiTileArray}, UInt32, UInt32, Cint, Ptr{Cvoid}), d, seed, counter, dist, stream))
+    return A
+end
+
 end # module

@@ -46,7 +46,9 @@ typedef enum mi_dtype {
                         (reference: ext/DLFP8TypesExt.jl:7-9) */
     MI_I32 = 5,
     MI_I64 = 6,
-    MI_BOOL = 7      /* Julia Bool: one byte holding 0 or 1 (Tiled broadcast / mapreduce only) */
+    MI_BOOL = 7,     /* Julia Bool: one byte holding 0 or 1 (Tiled broadcast / mapreduce only) */
+    MI_I8 = 8,       /* Int8 / UInt8 and */
+    MI_I16 = 9       /* Int16 / UInt16: RNG fills only (unsigned types share the codes of the signed ones) */
 } mi_dtype;
 
 /* Error codes (negative).  Positive return values are hipError_t. */
@@ -277,6 +279,20 @@ int mi_tiled_mapreduce_workspace(const mi_tile_array* dest, const mi_tile_array*
  * `sum` / `prod` pass); 0 is plain `+` / `*` as `reduce(+, ...)` passes. */
 int mi_tiled_mapreduce_eltype(const char* f_expr, int32_t src_dtype, const int32_t* scalar_dtypes,
                               int n_scalars, int op, int widen, int32_t* out_dtype);
+
+/* ---- Host-level RNG fills -----------------------------------------------------------------------
+ * Random.rand!(rng, A) / randn! / randexp! for rng = cuTile.RNG(seed, counter)
+ * (reference: src/language/random.jl:759-818 launching the fill kernels of :703-740).  Writes the
+ * reference's Philox2x32-7 stream value for value: block b of 512 outputs is keyed with
+ * (b * 0x9E3779B9) ^ seed and uses the counters counter + i.  `out` is any dense array, filled in
+ * linear order.  dist: 0 = rand (every element type: integers take the raw bits, floats lie in
+ * (0, 1]), 1 = randn, 2 = randexp (float types only, MI_E_DTYPE otherwise).  Integer results are
+ * bit-exact; randn / randexp go through this library's log / sin / cos. */
+int mi_rng_fill(const mi_tile_array* out, uint32_t seed, uint32_t counter, int dist, void* stream);
+
+/* advance_counter! after a fill of n_elements (src/language/random.jl:694-699,776-779): the counter
+ * moves by whole blocks of 512 and a wrap increments the seed. */
+int mi_rng_advance_counter(uint32_t* seed, uint32_t* counter, int64_t n_elements);
 
 /* Test hooks.  mi_tiled_set_dry_run(1) makes the two entry points stop after compiling (nothing is
  * loaded or launched, no GPU is needed); returns the previous setting.  mi_tiled_compile_count()

@@ -32,6 +32,9 @@ tiled_mapreduce        known answers of test/host/mapreduce.jl (count == 4, any 
                        fill(-5) == -5); numpy reductions; brute-force loops on tiny arrays
 jl_promote             Julia's documented promotion facts (Int32+Int64 -> Int64, Int64+Float32 ->
                        Float32, Float16+Float32 -> Float32, Bool yields, true + true == 2)
+philox2x32, rng_fill   Random123's published known-answer vectors for philox2x32 (7 and 10 rounds);
+                       slot layout by brute-force loops; the reference's own properties
+                       (test/device/random.jl:421-526: uniqueness, disjoint streams, counter carry)
 e4m3fn codec           16 round-trip vectors and fma vectors of
                        test/extensions/DLFP8Types.jl:126-141; all 256 codes vs torch.float8_e4m3fn
 =====================  ======================================================================
@@ -644,6 +647,135 @@ def tiled_mapreduce(f_text, op: str, A: np.ndarray, dims=None, init=None, scalar
     if dims is None:
         return r.reshape(-1)[0], ET
     return r, ET
+
+
+# ---- Philox2x32-7 host RNG fills ---------------------------------------------------------------
+PHILOX_M = 0xD256D193      # src/language/random.jl:93
+PHILOX_W = 0x9E3779B9      # src/language/random.jl:94 (Weyl key step)
+RAND_FILL_TILE = 512       # src/language/random.jl:701
+
+
+def philox2x32(c1, c2, key, rounds: int = 7):
+    """Philox2x32 with `rounds` rounds on uint32 arrays: per round (hi ^ k ^ c2, lo) of the 64-bit
+    product c1 * M, the key bumped by W between rounds (src/language/random.jl:100-122).  This is
+    Random123's philox2x32 (D. E. Shaw Research, Random123 1.14, `philox.h`); its published
+    known-answer vectors (`tests/kat_vectors`) pin this function in tests/test_oracle.py."""
+    c1 = np.asarray(c1, np.uint32).copy()
+    c2 = np.asarray(c2, np.uint32).copy()
+    k = np.broadcast_to(np.asarray(key, np.uint32), c1.shape).copy()
+    for r in range(rounds):
+        if r:
+            k = (k + np.uint32(PHILOX_W)).astype(np.uint32)
+        p = c1.astype(np.uint64) * np.uint64(PHILOX_M)
+        hi = (p >> np.uint64(32)).astype(np.uint32)
+        lo = (p & np.uint64(0xFFFFFFFF)).astype(np.uint32)
+        c1, c2 = hi ^ k ^ c2, lo
+    return c1, c2
+
+
+def _u01_f32(u):
+    """(u * 2^-32) + 2^-33 in Float32 (src/language/random.jl:136-142)."""
+    return (u.astype(np.float32) * np.float32(2.0 ** -32) + np.float32(2.0 ** -33)).astype(np.float32)
+
+
+def _u01_f64(u):
+    """Mantissa construction in [1, 2) minus 1, low bit forced (src/language/random.jl:169-174)."""
+    bits = (u >> np.uint64(12)) | np.uint64(0x3FF0000000000001)
+    return bits.view(np.float64) - 1.0
+
+
+def rng_advance_counter(seed: int, counter: int, n: int):
+    """`advance_counter!`: UInt32 counter += n, the carry bumps the seed (src/language/random.jl:694-699)."""
+    new = (counter + n) & 0xFFFFFFFF
+    if new < counter:
+        seed = (seed + 1) & 0xFFFFFFFF
+    return seed, new
+
+
+def rng_fill(kind: str, n: int, seed: int, counter: int, dist: str = "rand"):
+    """The `n` values a host fill writes for `cuTile.RNG(seed, counter)`: `rand!` / `randn!` /
+    `randexp!` (src/language/random.jl:759-818) launch one block per 512 outputs (:703-740); block b
+    (0-based) uses the Philox key (b * W) xor seed (:207-224, default stream) and counters
+    counter + i.  How a block's Philox outputs (c1, c2) land in its 512 slots depends on the width:
+    32-bit: 256 calls, c1 -> slots 0..255, c2 -> 256..511 (:262-286); 64-bit: 512 calls, c1 | c2 << 32
+    (:290-305); 16-bit: 128 calls give 256 words (c1 then c2), low halves -> 0..255, high halves ->
+    256..511 (:314-324); 8-bit: 64 calls give 128 words, byte q of word m -> slot 128 q + m
+    (:326-338).  Floats: `u01` (:136-174).  randn: Box-Muller on the (c1, c2) pair, r = sqrt(-2 log
+    u01(c2)), angle = 2 pi u01(c1) -> (r sin, r cos) in slots i and 256 + i, computed in Float32 for
+    the 16-bit floats (:369-398, 420-441); Float64 pairs counters i and 256 + i (:449-480).
+    randexp: -log(rand) (:500-501).
+    `kind`: u8 i8 u16 i16 u32 i32 u64 i64 f16 bf16 f32 f64; bf16 values are returned as float32."""
+    width = {"u8": 1, "i8": 1, "u16": 2, "i16": 2, "f16": 2, "bf16": 2, "u32": 4, "i32": 4, "f32": 4, "u64": 8, "i64": 8,
+             "f64": 8}[kind]
+    nb = cld(n, RAND_FILL_TILE)
+    b = np.arange(nb, dtype=np.uint64)
+    key = ((b * np.uint64(PHILOX_W)) & np.uint64(0xFFFFFFFF)).astype(np.uint32) ^ np.uint32(seed & 0xFFFFFFFF)
+
+    def calls(count, offset=0):
+        ctr = ((np.uint64(counter) + np.uint64(offset) + np.arange(count, dtype=np.uint64)) & np.uint64(0xFFFFFFFF)).astype(np.uint32)
+        c1, c2 = philox2x32(np.broadcast_to(ctr, (nb, count)), np.zeros((nb, count), np.uint32), key[:, None])
+        return c1, c2
+
+    if dist == "randn":
+        if width == 8:
+            a1, a2 = calls(256)
+            b1, b2 = calls(256, 256)
+            f1 = _u01_f64(a1.astype(np.uint64) | (a2.astype(np.uint64) << np.uint64(32)))
+            f2 = _u01_f64(b1.astype(np.uint64) | (b2.astype(np.uint64) << np.uint64(32)))
+            r = np.sqrt(-2.0 * np.log(f1))
+            ang = 2.0 * np.pi * f2
+        else:
+            c1, c2 = calls(256)
+            f1, f2 = _u01_f32(c1), _u01_f32(c2)
+            r = np.sqrt(np.float32(-2) * np.log(f2)).astype(np.float32)
+            ang = (np.float32(2 * np.pi) * f1).astype(np.float32)
+        out = np.concatenate([r * np.sin(ang), r * np.cos(ang)], axis=1)
+        if kind == "f16":
+            out = out.astype(np.float16)
+        elif kind == "bf16":
+            out = bf16_round(out.astype(np.float32))
+        return out.reshape(-1)[:n]
+
+    if width == 4:
+        c1, c2 = calls(256)
+        u = np.concatenate([c1, c2], axis=1)
+    elif width == 8:
+        c1, c2 = calls(512)
+        u = c1.astype(np.uint64) | (c2.astype(np.uint64) << np.uint64(32))
+    elif width == 2:
+        c1, c2 = calls(128)
+        raw = np.concatenate([c1, c2], axis=1)
+        u = np.concatenate([(raw & np.uint32(0xFFFF)).astype(np.uint16), (raw >> np.uint32(16)).astype(np.uint16)], axis=1)
+    else:
+        c1, c2 = calls(64)
+        raw = np.concatenate([c1, c2], axis=1)
+        u = np.concatenate([((raw >> np.uint32(8 * q)) & np.uint32(0xFF)).astype(np.uint8) for q in range(4)], axis=1)
+    u = u.reshape(-1)[:n]
+    if kind in ("u8", "u16", "u32", "u64"):
+        v = u
+    elif kind in ("i8", "i16", "i32", "i64"):
+        v = u.view({1: np.int8, 2: np.int16, 4: np.int32, 8: np.int64}[width])
+    elif kind == "f32":
+        v = _u01_f32(u)
+    elif kind == "f64":
+        v = _u01_f64(u)
+    elif kind == "f16":        # (u >> 6) | 0x3C01 as Float16, minus 1 (src/language/random.jl:148-154)
+        v = ((u >> np.uint16(6)) | np.uint16(0x3C01)).view(np.float16) - np.float16(1)
+    else:                      # bf16: (u >> 9) | 0x3F81 as BFloat16, minus 1 (:155-161); exact in float32
+        bits = ((u >> np.uint16(9)) | np.uint16(0x3F81)).astype(np.uint32) << np.uint32(16)
+        v = bits.view(np.float32) - np.float32(1)
+    if dist == "randexp":
+        if kind == "f64":
+            return -np.log(v)
+        return (-np.log(v.astype(np.float32))).astype(np.float16 if kind == "f16" else np.float32)
+    return v
+
+
+def bf16_round(x: np.ndarray) -> np.ndarray:
+    """float32 -> nearest-even BFloat16, returned as float32."""
+    u = np.asarray(x, np.float32).view(np.uint32)
+    r = (u + np.uint32(0x7FFF) + ((u >> np.uint32(16)) & np.uint32(1))) & np.uint32(0xFFFF0000)
+    return r.view(np.float32)
 
 
 # ---- example verify() criteria -------------------------------------------------------------

@@ -428,3 +428,75 @@ def test_tiled_mapreduce_reference_cases_and_brute_force(orc):
     r, _ = orc.tiled_mapreduce(None, "mul_prod", np.full(17, 2, np.int32), dims=())
     assert r.shape == (17,) and np.all(r == 2)                                      # no reduced dimension: map
     assert orc.tiled_mapreduce(None, "add_sum", A, init=100.0)[0] == pytest.approx(100 + A.astype(np.float64).sum(), rel=1e-6)
+
+
+# ---- Philox2x32-7 RNG fills -----------------------------------------------------------------------
+
+def test_philox2x32_random123_known_answers(orc):
+    """Random123 1.14 `tests/kat_vectors`, lines `philox2x32 7 ...` and `philox2x32 10 ...`
+    (counter words, key, expected output)."""
+    kat = [(7, 0x00000000, 0x00000000, 0x00000000, 0x257A3673, 0xCD26BE2A),
+           (7, 0xFFFFFFFF, 0xFFFFFFFF, 0xFFFFFFFF, 0xAB302C4D, 0x3DC9D239),
+           (7, 0x243F6A88, 0x85A308D3, 0x13198A2E, 0xBEDBBE6B, 0xE4C770B3),
+           (10, 0x00000000, 0x00000000, 0x00000000, 0xFF1DAE59, 0x6CD10DF2),
+           (10, 0xFFFFFFFF, 0xFFFFFFFF, 0xFFFFFFFF, 0x2C3F628B, 0xAB4FD7AD),
+           (10, 0x243F6A88, 0x85A308D3, 0x13198A2E, 0xDD7CE038, 0xF62A4C12)]
+    for rounds, c1, c2, k, o1, o2 in kat:
+        a, b = orc.philox2x32([c1], [c2], [k], rounds)
+        assert (int(a[0]), int(b[0])) == (o1, o2), rounds
+
+
+def test_rng_fill_layout_by_brute_force(orc):
+    """Slot placement of a block's Philox outputs for every width, element by element with scalar
+    loops (src/language/random.jl:262-338), on two blocks with a partial second one."""
+    seed, counter, n = 0x1234ABCD, 0xFFFFFFF0, 700          # the counter wraps inside the block
+
+    def call(b, i):
+        key = ((b * orc.PHILOX_W) & 0xFFFFFFFF) ^ seed
+        a, c = orc.philox2x32([(counter + i) & 0xFFFFFFFF], [0], [key])
+        return int(a[0]), int(c[0])
+    want32, want64, want16, want8 = [0] * 1024, [0] * 1024, [0] * 1024, [0] * 1024
+    for b in range(2):
+        for i in range(256):
+            c1, c2 = call(b, i)
+            want32[512 * b + i], want32[512 * b + 256 + i] = c1, c2
+        for i in range(512):
+            c1, c2 = call(b, i)
+            want64[512 * b + i] = c1 | (c2 << 32)
+        raw = [0] * 256
+        for i in range(128):
+            raw[i], raw[128 + i] = call(b, i)
+        for m in range(256):
+            want16[512 * b + m], want16[512 * b + 256 + m] = raw[m] & 0xFFFF, raw[m] >> 16
+        raw = [0] * 128
+        for i in range(64):
+            raw[i], raw[64 + i] = call(b, i)
+        for q in range(4):
+            for m in range(128):
+                want8[512 * b + 128 * q + m] = (raw[m] >> (8 * q)) & 0xFF
+    assert orc.rng_fill("u32", n, seed, counter).tolist() == want32[:n]
+    assert orc.rng_fill("u64", n, seed, counter).tolist() == want64[:n]
+    assert orc.rng_fill("u16", n, seed, counter).tolist() == want16[:n]
+    assert orc.rng_fill("u8", n, seed, counter).tolist() == want8[:n]
+    assert np.array_equal(orc.rng_fill("i32", n, seed, counter).view(np.uint32), orc.rng_fill("u32", n, seed, counter))
+
+
+def test_rng_float_conversions_and_reference_properties(orc):
+    """u01 end points (src/language/random.jl:129-174) and the properties the reference's tests assert
+    for the host RNG (test/device/random.jl:421-526)."""
+    assert orc._u01_f32(np.array([0, 0xFFFFFFFF], np.uint32)).tolist() == [2.0 ** -33, 1.0]
+    f64 = orc._u01_f64(np.array([0, 0xFFFFFFFFFFFFFFFF], np.uint64))
+    assert f64[0] == 2.0 ** -52 and f64[1] == 1.0 - 2.0 ** -52
+    f16 = orc.rng_fill("f16", 4096, 1, 0)
+    assert f16.min() > 0 and f16.max() < 1 and f16.dtype == np.float16
+    bf = orc.rng_fill("bf16", 4096, 1, 0)
+    assert bf.min() > 0 and bf.max() < 1 and np.array_equal(bf, orc.bf16_round(bf))
+    v = orc.rng_fill("u32", 2048, 42, 0)
+    assert len(np.unique(v)) == 2048
+    assert not set(v.tolist()) & set(orc.rng_fill("u32", 2048, 100, 0).tolist())
+    assert not set(v.tolist()) & set(orc.rng_fill("u32", 2048, 42, 2048).tolist())      # the next fill of the same RNG
+    assert orc.rng_advance_counter(7, 2 ** 32 - 4, 10) == (8, 6)                          # random.jl test :520-525
+    z = orc.rng_fill("f32", 1 << 16, 5, 0, "randn").astype(np.float64)
+    assert abs(z.mean()) < 0.02 and abs(z.var() - 1) < 0.03
+    e = orc.rng_fill("f64", 1 << 16, 5, 0, "randexp")
+    assert abs(e.mean() - 1) < 0.02 and e.min() > 0

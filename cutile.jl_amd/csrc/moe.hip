@@ -373,29 +373,31 @@ extern "C" int mi_fused_moe_kernel(const mi_tile_array* A, const mi_tile_array* 
 }
 
 // ---- on-device moe_align_tile_size ------------------------------------------------------------
-// One workgroup of four waves.  Counting sort by expert of the replica ids (slot-fastest
+// One workgroup of sixteen waves.  Counting sort by expert of the replica ids (slot-fastest
 // flattening of topk_ids, examples/moe.jl:148-150): LDS histogram, serial scan over the experts,
-// then placement in super-blocks of 256 consecutive replicas.  A replica's slot is
+// then placement in super-blocks of 1024 consecutive replicas (one per lane).  A replica's slot is
 //     cursor[e] + (replicas of e in earlier waves of the super-block) + (those in earlier lanes),
 // the last term from ballots alone, so ids of one expert ascend exactly as the stable sortperm
 // of moe.jl:150 orders them.  The outputs have fixed capacity: unused slots hold the sentinel
 // total+1, unused blocks expert 0, which the GEMM kernel skips.
 constexpr int kAlignMaxExperts = 1024;
-__global__ __launch_bounds__(256) void moe_align_kernel(const long long* __restrict__ topk_ids, int64_t ld_slot,
+constexpr int kAlignThreads = 1024, kAlignWaves = kAlignThreads / 64;
+__global__ __launch_bounds__(kAlignThreads) void moe_align_kernel(const long long* __restrict__ topk_ids, int64_t ld_slot,
                                                         int num_tokens, int topk, int tile_m, int num_experts,
                                                         int* __restrict__ sorted_token_ids, int cap_slots,
                                                         int* __restrict__ sorted_expert_ids, int cap_blocks) {
     __shared__ int cursor[kAlignMaxExperts];      // histogram, then next free slot of every expert
-    __shared__ int tbl[4][kAlignMaxExperts];      // replicas per (wave, expert) of the current super-block
+    __shared__ unsigned short tbl[kAlignWaves][kAlignMaxExperts];   // replicas per (wave, expert) of the current super-block (<= 64)
     __shared__ int s_blocks;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, total = num_tokens * topk;
-    for (int e = tid; e < num_experts; e += 256) {
+    for (int e = tid; e < num_experts; e += kAlignThreads) {
         cursor[e] = 0;
-        tbl[0][e] = tbl[1][e] = tbl[2][e] = tbl[3][e] = 0;
+#pragma unroll
+        for (int w = 0; w < kAlignWaves; ++w) tbl[w][e] = 0;
     }
-    for (int i = tid; i < cap_slots; i += 256) sorted_token_ids[i] = total + 1;
+    for (int i = tid; i < cap_slots; i += kAlignThreads) sorted_token_ids[i] = total + 1;
     __syncthreads();
-    for (int r = tid; r < total; r += 256) {
+    for (int r = tid; r < total; r += kAlignThreads) {
         const long long e = topk_ids[(r / topk) + (int64_t)(r % topk) * ld_slot];
         if (e >= 1 && e <= num_experts) atomicAdd(&cursor[(int)e - 1], 1);
     }
@@ -410,10 +412,10 @@ __global__ __launch_bounds__(256) void moe_align_kernel(const long long* __restr
         s_blocks = blk;
     }
     __syncthreads();
-    for (int b = s_blocks + tid; b < cap_blocks; b += 256) sorted_expert_ids[b] = 0;
+    for (int b = s_blocks + tid; b < cap_blocks; b += kAlignThreads) sorted_expert_ids[b] = 0;
 
     const unsigned long long lt = lane ? (~0ull >> (64 - lane)) : 0ull;
-    for (int r0 = 0; r0 < total; r0 += 256) {
+    for (int r0 = 0; r0 < total; r0 += kAlignThreads) {
         const int r = r0 + tid;
         int e = -1;
         if (r < total) {
@@ -427,7 +429,7 @@ __global__ __launch_bounds__(256) void moe_align_kernel(const long long* __restr
             const int el = __shfl(e, leader, 64);
             const unsigned long long m = __ballot(e == el);
             if (e == el) rank = __popcll(m & lt);
-            if (lane == leader) tbl[wave][el] = __popcll(m);
+            if (lane == leader) tbl[wave][el] = (unsigned short)__popcll(m);
             todo &= ~m;
         }
         __syncthreads();
@@ -439,7 +441,7 @@ __global__ __launch_bounds__(256) void moe_align_kernel(const long long* __restr
         __syncthreads();
         // advance the cursors and clear the table: the entries touched are those of this super-block's experts
         if (e >= 0 && rank == 0) {  // first lane of its expert within the wave
-            atomicAdd(&cursor[e], tbl[wave][e]);
+            atomicAdd(&cursor[e], (int)tbl[wave][e]);
         }
         __syncthreads();
         if (e >= 0 && rank == 0) tbl[wave][e] = 0;
@@ -470,7 +472,7 @@ extern "C" int mi_moe_align_tile_size_device(const mi_tile_array* topk_ids, int 
         return MI_E_STRIDE;
     if (cap_slots > 0x7fffffff) return MI_E_SHAPE;
     if (cap_blocks == 0) return MI_OK;
-    hipLaunchKernelGGL(moe_align_kernel, dim3(1), dim3(256), 0, (hipStream_t)stream, (const long long*)topk_ids->ptr,
+    hipLaunchKernelGGL(moe_align_kernel, dim3(1), dim3(kAlignThreads), 0, (hipStream_t)stream, (const long long*)topk_ids->ptr,
                        topk > 1 ? topk_ids->strides[1] : 0, (int)num_tokens, (int)topk, tile_m, num_experts,
                        (int*)sorted_token_ids->ptr, (int)cap_slots, (int*)sorted_expert_ids->ptr, (int)cap_blocks);
     set_variant("moe_align_device_1wg");

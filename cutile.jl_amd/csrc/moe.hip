@@ -91,7 +91,7 @@ constexpr int kTT = 32;   // token slots per workgroup (one MFMA row tile)
 // workgroups as it has (started) 32-token tiles.  Small register footprint -> many
 // workgroups per CU, each with the next weight tile already in flight.
 template <typename E, bool W8, int NTW, int kKT>
-__global__ __launch_bounds__(256) void fused_moe_kernel(
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4))) void fused_moe_kernel(
     const unsigned short* __restrict__ A, int64_t lda, int num_a_cols, const void* __restrict__ Bv, int64_t ldb,
     int64_t sbe, unsigned short* __restrict__ C, int64_t ldc, int total_tokens,
     const unsigned short* __restrict__ topk_weights, const int* __restrict__ sorted_token_ids, int num_slots,
@@ -99,10 +99,12 @@ __global__ __launch_bounds__(256) void fused_moe_kernel(
     int num_experts, int replicas, bool mul_routed_weight, int TILE_M, int tile_slots, int n_blocks, bool vecA,
     bool vecB) {
     constexpr int kNT = 32 * NTW, KW = 4 / NTW;
-    __shared__ __attribute__((aligned(16))) unsigned short Bs[kNT * kKT];  // [n][k], 16-byte chunks XOR-swizzled
+    // B tile [n][k], 16-byte chunks XOR-swizzled.  E4M3 weights stay raw bytes here (half the LDS
+    // traffic and footprint) and are widened after the fragment read; see b_offset8 below.
+    constexpr int kBsBytes = (W8 ? 1 : 2) * kNT * kKT, kRedBytes = KW > 1 ? 4 * 64 * 16 * 4 : 0;
+    __shared__ __attribute__((aligned(16))) unsigned char Bs_raw[kBsBytes > kRedBytes ? kBsBytes : kRedBytes];
+    unsigned short* Bs = reinterpret_cast<unsigned short*>(Bs_raw);
     __shared__ __attribute__((aligned(16))) unsigned short As[kTT * kKT];  // [slot][k], same swizzle
-    __shared__ int s_tok[kTT];
-    __shared__ int s_any;
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, hb = lane >> 5;
     const int wn = wave % NTW, wk = wave / NTW;  // position along n / along the K split
@@ -112,17 +114,17 @@ __global__ __launch_bounds__(256) void fused_moe_kernel(
     const int slot0 = tile * tile_slots;            // tile_slots = min(TILE_M, 32) divides TILE_M
     const int expert = sorted_expert_ids[slot0 / TILE_M] - 1;
 
-    if (tid == 0) s_any = 0;
-    __syncthreads();
-    if (tid < kTT) {
-        const int sl = slot0 + tid;
-        int t = (tid < tile_slots && sl < num_slots) ? sorted_token_ids[sl] : 0;  // 1-based; 0 / >total = no token
+    // The tile's 32 token ids live in registers, slot i in lanes i and i + 32 of every wave (LDS is
+    // exactly the two operand tiles, which is what lets a fourth workgroup fit on a CU).
+    int my_tok;
+    {
+        const int i = lane & 31, sl = slot0 + i;
+        int t = (i < tile_slots && sl < num_slots) ? sorted_token_ids[sl] : 0;  // 1-based; 0 / >total = no token
         if (t < 1 || t > total_tokens) t = 0;
-        s_tok[tid] = t;
-        if (t) s_any = 1;
+        my_tok = t;
     }
-    __syncthreads();
-    if (!s_any || expert < 0 || expert >= num_experts) return;  // uniform across the workgroup
+    auto tok_of = [&](int slot) { return __shfl(my_tok, slot, 64); };
+    if (__ballot(my_tok != 0) == 0ull || expert < 0 || expert >= num_experts) return;  // same in every wave
 
     const unsigned char* B8 = (const unsigned char*)Bv + (int64_t)expert * sbe;
     const unsigned short* B16 = (const unsigned short*)Bv + (int64_t)expert * sbe;
@@ -134,19 +136,22 @@ __global__ __launch_bounds__(256) void fused_moe_kernel(
     constexpr int CPRB = kKT / EPB;         // 16-byte global chunks per weight row
     constexpr int NB = kNT * CPRB / 256;    // weight chunks per thread
     constexpr int NA = kTT * CPR / 256;     // A chunks per thread
-    u32x4 breg[NB];                         // raw bytes; e4m3 weights are widened on their way into LDS
-    s16x8 areg[NA];
+    // Two staging sets for the e4m3 path (its raw tiles are half the size, so two tiles per
+    // workgroup can be in flight at the register cost of one f16 tile); one set otherwise.
+    constexpr int DEPTH = W8 ? 2 : 1;
+    u32x4 breg0[NB], breg1[DEPTH == 2 ? NB : 1];
+    s16x8 areg0[NA], areg1[DEPTH == 2 ? NA : 1];
     int a_col[NA];
 #pragma unroll
     for (int i = 0; i < NA; ++i) {
         a_col[i] = -1;
-        const int tok = s_tok[(tid + 256 * i) / CPR];
+        const int tok = tok_of((tid + 256 * i) / CPR);
         if (tok) {
             const int col = (tok + replicas - 1) / replicas - 1;  // cld(token_id, replicas), 0-based
             if (col < num_a_cols) a_col[i] = col;
         }
     }
-    auto load_tiles = [&](int k0) {
+    auto load_tiles = [&](int k0, u32x4* breg, s16x8* areg) {
 #pragma unroll
         for (int i = 0; i < NB; ++i) {
             const int id = tid + 256 * i, n = id / CPRB, c = id % CPRB;
@@ -183,20 +188,21 @@ __global__ __launch_bounds__(256) void fused_moe_kernel(
             areg[i] = v;
         }
     };
-    load_tiles(0);
+    // Raw-byte tile of the e4m3 path: row n = kKT bytes in 16-byte chunks.  Chunk c sits at
+    // c ^ sw(n) and its two 8-byte halves are swapped for rows with bit 4 set, which makes the
+    // 8-byte fragment reads of 32 lanes (rows n .. n+31, one half) cover all 64 banks exactly once.
+    auto b_sw = [](int n) { return kKT == 128 ? ((n >> 1) & 7) : (n & 15); };
 
-    for (int k0 = 0; k0 < K; k0 += kKT) {
+    // One K step: staged tile -> LDS, refill the staging set with the tile DEPTH steps ahead, MFMAs.
+    auto step = [&](int k0, u32x4* breg, s16x8* areg) {
         __syncthreads();
 #pragma unroll
         for (int i = 0; i < NB; ++i) {
             const int id = tid + 256 * i, n = id / CPRB, c = id % CPRB;
             if (W8) {
-                unsigned w[8];
-#pragma unroll
-                for (int q = 0; q < 4; ++q) Fp8<E>::cvt4(breg[i][q], w[2 * q], w[2 * q + 1]);
-                const u32x4 lo = {w[0], w[1], w[2], w[3]}, hi = {w[4], w[5], w[6], w[7]};  // k elements 0-7, 8-15
-                *reinterpret_cast<u32x4*>(&Bs[n * kKT + 8 * ((2 * c) ^ (n & 7))]) = lo;
-                *reinterpret_cast<u32x4*>(&Bs[n * kKT + 8 * ((2 * c + 1) ^ (n & 7))]) = hi;
+                const u32x4 v = breg[i];
+                const u32x4 sw = ((n >> 4) & 1) ? u32x4{v[2], v[3], v[0], v[1]} : v;
+                *reinterpret_cast<u32x4*>(&Bs_raw[n * kKT + 16 * (c ^ b_sw(n))]) = sw;
             } else {
                 *reinterpret_cast<u32x4*>(&Bs[n * kKT + 8 * (c ^ (n & 7))]) = breg[i];
             }
@@ -207,22 +213,40 @@ __global__ __launch_bounds__(256) void fused_moe_kernel(
             *reinterpret_cast<s16x8*>(&As[sl * kKT + 8 * (c ^ (sl & 7))]) = areg[i];
         }
         __syncthreads();
-        if (k0 + kKT < K) load_tiles(k0 + kKT);
+        if (k0 + DEPTH * kKT < K) load_tiles(k0 + DEPTH * kKT, breg, areg);
 #pragma unroll
         for (int kq = 0; kq < kKT / 16 / KW; ++kq) {
             const int ks = wk * (kKT / 16 / KW) + kq;
             const int c = 2 * ks + hb;
             const int n = wn * 32 + (lane & 31);
             const int slot = lane & 31;
-            s16x8 bf = *reinterpret_cast<const s16x8*>(&Bs[n * kKT + 8 * (c ^ (n & 7))]);
+            s16x8 bf;
+            if (W8) {   // k elements 16 ks + 8 hb .. +7 are half hb of chunk ks
+                const u32x2 raw = *reinterpret_cast<const u32x2*>(&Bs_raw[n * kKT + 16 * (ks ^ b_sw(n)) + 8 * (hb ^ ((n >> 4) & 1))]);
+                unsigned w0, w1, w2, w3;
+                Fp8<E>::cvt4(raw[0], w0, w1);
+                Fp8<E>::cvt4(raw[1], w2, w3);
+                bf = __builtin_bit_cast(s16x8, u32x4{w0, w1, w2, w3});
+            } else {
+                bf = *reinterpret_cast<const s16x8*>(&Bs[n * kKT + 8 * (c ^ (n & 7))]);
+            }
             s16x8 af = *reinterpret_cast<const s16x8*>(&As[slot * kKT + 8 * (c ^ (slot & 7))]);
             acc = E::mfma32(af, bf, acc);
         }
+    };
+    load_tiles(0, breg0, areg0);
+    if (DEPTH == 2) {
+        if (kKT < K) load_tiles(kKT, breg1, areg1);
+        for (int k0 = 0; k0 < K; k0 += 2 * kKT) {
+            step(k0, breg0, areg0);
+            if (k0 + kKT < K) step(k0 + kKT, breg1, areg1);
+        }
+    } else {
+        for (int k0 = 0; k0 < K; k0 += kKT) step(k0, breg0, areg0);
     }
     if (KW > 1) {  // add the K-split partial accumulators: wave (wn, wk) -> wave (wn, 0)
         __syncthreads();
-        float* red = reinterpret_cast<float*>(Bs);  // 4 waves x 64 lanes x 16 floats = 16 KB <= sizeof(Bs)
-        static_assert(KW == 1 || sizeof(unsigned short) * kNT * kKT >= 4 * 64 * 16 * sizeof(float), "reduction buffer");
+        float* red = reinterpret_cast<float*>(Bs_raw);  // 4 waves x 64 lanes x 16 floats = 16 KB <= sizeof(Bs_raw)
         if (wk > 0) {
 #pragma unroll
             for (int r = 0; r < 16; ++r) red[(wave * 16 + r) * 64 + lane] = acc[r];
@@ -237,13 +261,15 @@ __global__ __launch_bounds__(256) void fused_moe_kernel(
 
     // epilogue: rows = token slots 8*(r/4) + 4*hb + r%4, column = channel n0 + wn*32 + lane%32
     const int gn = n0 + wn * 32 + (lane & 31);
+    int toks[16];   // gathered while every lane of the wave is still active
+#pragma unroll
+    for (int r = 0; r < 16; ++r) toks[r] = tok_of(8 * (r >> 2) + 4 * hb + (r & 3));
     if (gn >= N) return;
     float ch_scale = 1.f;
     if (W8) ch_scale = b_scale[gn + (int64_t)expert * ld_scale];
 #pragma unroll
     for (int r = 0; r < 16; ++r) {
-        const int slot = 8 * (r >> 2) + 4 * hb + (r & 3);
-        const int tok = s_tok[slot];
+        const int tok = toks[r];
         if (!tok) continue;
         float v = acc[r];
         if (W8) v *= ch_scale;

@@ -80,6 +80,26 @@ int compile(const std::string& gen, const char* kernel, hipFunction_t* fn) {
     return MI_OK;
 }
 
+// Kernels already built, by a short key (expression text + the constants baked into the kernel), so
+// that a repeated call does not have to regenerate the source text just to find its kernel.
+std::unordered_map<std::string, hipFunction_t> g_by_key;
+
+template <typename MakeSource>
+int kernel_for(const std::string& key, const char* kernel, MakeSource make_source, hipFunction_t* fn) {
+    int dev = 0;
+    if (!g_dry_run && hipGetDevice(&dev) != hipSuccess) return (int)hipGetLastError();
+    const std::string k = std::to_string(dev) + "#" + key;
+    {
+        std::lock_guard<std::mutex> lock(g_mu);
+        auto it = g_by_key.find(k);
+        if (it != g_by_key.end()) { *fn = it->second; return MI_OK; }
+    }
+    MI_CHECK(compile(make_source(), kernel, fn));
+    std::lock_guard<std::mutex> lock(g_mu);
+    g_by_key.emplace(k, *fn);
+    return MI_OK;
+}
+
 int launch(hipFunction_t f, int64_t blocks, int threads, void* args, size_t bytes, hipStream_t s) {
     if (g_dry_run) return MI_OK;
     if (blocks <= 0) return MI_OK;
@@ -245,9 +265,17 @@ int broadcast_impl(const mi_tile_array* dest, const char* text, const mi_tile_ar
     const int64_t nbx = cld(nvec0, (int64_t)TX * U), nby = cld(rows, (int64_t)TY);
     if (nbx > 0x7fffffffLL || nbx * nby > 0x7fffffffLL) return MI_E_GRID;
 
-    // ---- source ----
-    std::string g;
+    // ---- kernel: looked up by what is baked into it, generated and compiled on a miss ----
     char buf[512];
+    std::string key = "bc|";
+    key += text;
+    snprintf(buf, sizeof buf, "|%d|%d,%d,%d,%d,%d,%d,%d|", dest->dtype, V, U, TX, TY, n, NT ? 1 : 0, vec_d ? 1 : 0);
+    key += buf;
+    for (int i = 0; i < e.leaves_used; ++i) { snprintf(buf, sizeof buf, "%d%c%c,", leaf_dt[i], keep0[i] ? 'k' : 'b', vec_l[i] ? 'v' : 's'); key += buf; }
+    key += "|";
+    for (int i = 0; i < e.scalars_used; ++i) { snprintf(buf, sizeof buf, "%d,", scal_dt[i]); key += buf; }
+    auto make_source = [&]() {
+    std::string g;
     snprintf(buf, sizeof buf, "constexpr int V = %d, U = %d, TX = %d, TY = %d, NDIM = %d;\nconstexpr bool NT = %s, VECD = %s;\n", V, U, TX, TY,
              n, NT ? "true" : "false", vec_d ? "true" : "false");
     g += buf;
@@ -319,8 +347,10 @@ int broadcast_impl(const mi_tile_array* dest, const char* text, const mi_tile_ar
     emit_block(true);
     g += "    }\n}\n";
 
+    return g;
+    };
     hipFunction_t fn = nullptr;
-    MI_CHECK(compile(g, "tiled_bc", &fn));
+    MI_CHECK(kernel_for(key, "tiled_bc", make_source, &fn));
     BcArgs a;
     memset(&a, 0, sizeof a);
     a.d = dest->ptr;
@@ -690,11 +720,17 @@ std::string mr_source(const Expr& e, const int32_t* scal_dt, int src_dt, int acc
     return g;
 }
 
-int run_pass(const Expr& e, const int32_t* scal_dt, const ScalarArgs& sa, int src_dt, int acc_dt, int op, const MrShape& sh, const MrPlan& pl,
-             const void* src, void* dst, bool out_ws, hipStream_t stream) {
-    const std::string g = mr_source(e, scal_dt, src_dt, acc_dt, op, sh, pl, out_ws);
+int run_pass(const Expr& e, const char* text, const int32_t* scal_dt, const ScalarArgs& sa, int src_dt, int acc_dt, int op, const MrShape& sh,
+             const MrPlan& pl, const void* src, void* dst, bool out_ws, hipStream_t stream) {
+    char kb[256];
+    snprintf(kb, sizeof kb, "|%d,%d,%d|%d,%d,%d,%d,%d,%d,%d|%d,%d,%d,%d|", src_dt, acc_dt, op, pl.V, pl.T, pl.TX, pl.TY, sh.rmask, pl.LANES, pl.UNR,
+             pl.nt ? 1 : 0, pl.vec ? 1 : 0, pl.vecd ? 1 : 0, out_ws ? 1 : 0);
+    std::string key = "mr|";
+    key += text;
+    key += kb;
+    for (int i = 0; i < e.scalars_used; ++i) { snprintf(kb, sizeof kb, "%d,", scal_dt[i]); key += kb; }
     hipFunction_t fn = nullptr;
-    MI_CHECK(compile(g, "tiled_mr", &fn));
+    MI_CHECK(kernel_for(key, "tiled_mr", [&]() { return mr_source(e, scal_dt, src_dt, acc_dt, op, sh, pl, out_ws); }, &fn));
     MrArgs a;
     memset(&a, 0, sizeof a);
     a.src = src;
@@ -740,11 +776,11 @@ int mapreduce_impl(const mi_tile_array* dest, const mi_tile_array* src, const ch
     if (p1.P == 1) {
         snprintf(buf, sizeof buf, "tiled_mr_%s_l%d_ty%d", sh.run() ? "run" : "column", p1.LANES, p1.TY);
         set_variant_text(buf);
-        return run_pass(e, scal_dt, sa, src->dtype, dest->dtype, op, sh, p1, src->ptr, dest->ptr, false, stream);
+        return run_pass(e, f_text ? f_text : "a0", scal_dt, sa, src->dtype, dest->dtype, op, sh, p1, src->ptr, dest->ptr, false, stream);
     }
     if (!workspace || workspace_bytes < need) return MI_E_ARG;
     if (((uintptr_t)workspace) % 16) return MI_E_ALIGN;
-    MI_CHECK(run_pass(e, scal_dt, sa, src->dtype, dest->dtype, op, sh, p1, src->ptr, workspace, true, stream));
+    MI_CHECK(run_pass(e, f_text ? f_text : "a0", scal_dt, sa, src->dtype, dest->dtype, op, sh, p1, src->ptr, workspace, true, stream));
     // Second pass: the P partials of every output, identity map.  The partials form a dense array
     // whose kept dimensions keep their place; P takes the place of dimension 0 (run shape: partials
     // of one output are adjacent) or of the first reduced dimension (column shape: P planes of nk).
@@ -769,7 +805,7 @@ int mapreduce_impl(const mi_tile_array* dest, const mi_tile_array* src, const ch
     set_variant_text(buf);
     ScalarArgs none;
     memset(&none, 0, sizeof none);
-    return run_pass(id, scal_dt, none, cdt, dest->dtype, op, s2, p2, workspace, dest->ptr, false, stream);
+    return run_pass(id, "a0", scal_dt, none, cdt, dest->dtype, op, s2, p2, workspace, dest->ptr, false, stream);
 }
 
 }  // namespace
@@ -824,7 +860,7 @@ int mi_tiled_mapreduce_eltype(const char* f_expr, int32_t src_dtype, const int32
 int mi_tiled_set_dry_run(int on) {
     std::lock_guard<std::mutex> lock(g_mu);
     const int old = g_dry_run ? 1 : 0;
-    if ((on != 0) != g_dry_run) g_cache.clear();   // entries of a dry run hold no loaded function
+    if ((on != 0) != g_dry_run) { g_cache.clear(); g_by_key.clear(); }   // entries of a dry run hold no loaded function
     g_dry_run = on != 0;
     return old;
 }

@@ -309,24 +309,31 @@ def bench_kernels(ct, which, cpu, nruns=NRUNS, warmup=WARMUP):
         except Exception as ex:  # graph capture unavailable: fall back to eager launches
             res["moe_f16_device"] = extra(_entry(f"MoE f16 top-2, device work only (eager; graph failed: {type(ex).__name__})",
                                                  dev, wbytes, "GB/s", "hbm", HBM_PEAK_GBS, "f16", nruns, warmup))
+        fused = lambda: moe.cutile_moe(d.hidden_states, d.w1, d.w2, d.topk_weights, d.topk_ids, 128, 128, 64,
+                                       device_align=True, fuse_silu=True)
+        assert torch.equal(fused(), ref_out), "fused SiLU epilogue differs from the separate kernels"
+        try:
+            gf, _ = graph_of(fused)
+            res["moe_f16_device_fused"] = extra(_entry("MoE f16 top-2 on the device, SiLU*up fused into the gate/up GEMM epilogue (3 kernels + sort), HIP graph replay",
+                                                       gf.replay, wbytes, "GB/s", "hbm", HBM_PEAK_GBS, "f16", nruns, warmup))
+        except Exception as ex:
+            res["moe_f16_device_fused"] = extra(_entry(f"MoE f16 top-2, fused SiLU epilogue (eager; graph failed: {type(ex).__name__})",
+                                                       fused, wbytes, "GB/s", "hbm", HBM_PEAK_GBS, "f16", nruns, warmup))
         if cpu:
             J = orc.to_julia
             args = (J(d.hidden_states), J(d.w1), J(d.w2), J(d.topk_weights), J(d.topk_ids))
             res["moe_f16"]["cpu_ms"] = round(_cpu_time(lambda: orc.ref_moe(*args), repeats=1), 1)
             res["moe_f16"]["cpu_note"] = f"numpy restatement of ref_moe, BLAS {ncores} threads"
         # fp8 weights (per-channel fp32 scales)
-        J = orc.to_julia
-        c1, s1 = orc.quantize_e4m3fn_per_channel(J(d.w1).astype(np.float32))
-        c2, s2 = orc.quantize_e4m3fn_per_channel(J(d.w2).astype(np.float32))
-        w1q = orc.from_julia(c1).cuda().view(torch.float8_e4m3fn); w2q = orc.from_julia(c2).cuda().view(torch.float8_e4m3fn)
-        s1t, s2t = orc.from_julia(s1).cuda(), orc.from_julia(s2).cuda()
-        w8bytes = c1.size + c2.size + (s1.size + s2.size) * 4 + 2 * d.hidden_states.numel() * 2
+        q = moe.quantize_weights(d)
+        w1q, w2q, s1t, s2t = q.w1, q.w2, q.w1_scale, q.w2_scale
+        w8bytes = w1q.numel() + w2q.numel() + (s1t.numel() + s2t.numel()) * 4 + 2 * d.hidden_states.numel() * 2
         dev8 = lambda: moe.cutile_moe(d.hidden_states, w1q, w2q, d.topk_weights, d.topk_ids, 128, 128, 64, w1_scale=s1t,
-                                      w2_scale=s2t, device_align=True)
+                                      w2_scale=s2t, device_align=True, fuse_silu=True)
         dev8()
         try:
             g8, _ = graph_of(dev8)
-            res["moe_fp8_device"] = extra(_entry("MoE e4m3 weights top-2, whole cutile_moe on the device, HIP graph replay", g8.replay,
+            res["moe_fp8_device"] = extra(_entry("MoE e4m3 weights top-2, whole cutile_moe on the device (fused SiLU epilogue), HIP graph replay", g8.replay,
                                                  w8bytes, "GB/s", "hbm", HBM_PEAK_GBS, "fp8 weights / f16 MFMA", nruns, warmup))
         except Exception as ex:
             res["moe_fp8_device"] = extra(_entry(f"MoE e4m3 weights top-2, device work only (eager; {type(ex).__name__})", dev8,

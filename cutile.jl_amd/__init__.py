@@ -76,6 +76,7 @@ _SIGNATURES = {
          ctypes.POINTER(ctypes.c_int32), ctypes.POINTER(ctypes.c_int32),
          ctypes.POINTER(ctypes.c_int64)], _i),
     "mi_fused_moe_kernel": ([_A] * 6 + [_i, _i, _i, _i, _i, _A, _vp], _i),
+    "mi_fused_moe_silu_kernel": ([_A] * 6 + [_i, _i, _i, _i, _i, _A, _vp], _i),
     "mi_silu_and_mul_kernel": ([_A, _A, _A, _i, _vp], _i),
     "mi_moe_sum_topk": ([_A, _A, _vp], _i),
     "mi_tiled_broadcast": ([_A, ctypes.c_char_p, ctypes.POINTER(_A), _i, _vp, _i, _vp], _i),
@@ -323,6 +324,16 @@ def fused_moe_kernel(A, B, C, topk_weights, sorted_token_ids, sorted_expert_ids,
                      TILE_K: int, b_scale=None, stream=None):
     """examples/moe.jl:45-105 (``b_scale``: per-(n, expert) fp32 scales of fp8 weights)."""
     _call("mi_fused_moe_kernel", _ref(A), _ref(B), _ref(C), _ref(topk_weights),
+          _ref(sorted_token_ids), _ref(sorted_expert_ids), num_token_replicas,
+          int(bool(mul_routed_weight)), TILE_M, TILE_N, TILE_K, _ref(b_scale), _stream(stream))
+
+
+def fused_moe_silu_kernel(A, B, C, topk_weights, sorted_token_ids, sorted_expert_ids,
+                          num_token_replicas: int, mul_routed_weight: bool, TILE_M: int, TILE_N: int,
+                          TILE_K: int, b_scale=None, stream=None):
+    """fused_moe_kernel (moe.jl:45-105) on the gate / up projection with silu_and_mul_kernel
+    (moe.jl:110-128) as its epilogue: ``C`` is (N/2, total_tokens)."""
+    _call("mi_fused_moe_silu_kernel", _ref(A), _ref(B), _ref(C), _ref(topk_weights),
           _ref(sorted_token_ids), _ref(sorted_expert_ids), num_token_replicas,
           int(bool(mul_routed_weight)), TILE_M, TILE_N, TILE_K, _ref(b_scale), _stream(stream))
 

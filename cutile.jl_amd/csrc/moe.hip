@@ -77,6 +77,17 @@ template <> struct Fp8<BF16> {
     }
 };
 
+// SiLU(x) * y in fp32 with the approximate reciprocal of moe.jl:117-124.  The barrier keeps the
+// fp32 product a value of its own: without it the compiler may fold the final multiply into the
+// conversion to f16 (one rounding instead of two) in one kernel and not in another, and the fused
+// and the separate path would differ in the last bit now and then.
+__device__ __forceinline__ float silu_mul(float x, float y) {
+    const float denom = 1.0f + expf(-x);
+    float p = x * __builtin_amdgcn_rcpf(denom) * y;
+    asm volatile("" : "+v"(p));
+    return p;
+}
+
 constexpr int kTT = 32;   // token slots per workgroup (one MFMA row tile)
 
 // E: activation/output element traits; W8: weights are E4M3FN bytes (else same type as A).
@@ -90,7 +101,11 @@ constexpr int kTT = 32;   // token slots per workgroup (one MFMA row tile)
 // workgroups leave at once, so the expert's weight strip is streamed by exactly as many
 // workgroups as it has (started) 32-token tiles.  Small register footprint -> many
 // workgroups per CU, each with the next weight tile already in flight.
-template <typename E, bool W8, int NTW, int kKT>
+// SILU (wide shape only): the workgroup's 128 weight rows are 64 gate channels [n0, n0 + 64) and
+// the 64 up channels N/2 + [n0, n0 + 64) of the gate / up projection; the epilogue rounds both
+// products to the activation type exactly as the separate kernels would, applies SiLU(gate) * up
+// (moe.jl:110-128) and writes N/2 channels, so the intermediate never goes to memory.
+template <typename E, bool W8, int NTW, int kKT, bool SILU = false>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4))) void fused_moe_kernel(
     const unsigned short* __restrict__ A, int64_t lda, int num_a_cols, const void* __restrict__ Bv, int64_t ldb,
     int64_t sbe, unsigned short* __restrict__ C, int64_t ldc, int total_tokens,
@@ -110,7 +125,12 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4))) void f
     const int wn = wave % NTW, wk = wave / NTW;  // position along n / along the K split
     // consecutive workgroups share the token tile (and therefore the activations in L2)
     const int tile = blockIdx.x / n_blocks, bid_n = blockIdx.x % n_blocks;
-    const int n0 = bid_n * kNT;
+    static_assert(!SILU || NTW == 4, "the fused SiLU epilogue pairs waves 0,1 (gate) with waves 2,3 (up)");
+    const int half_n = N / 2;
+    const int n0 = bid_n * (SILU ? kNT / 2 : kNT);
+    // global weight row of tile row n
+    auto row_of = [&](int n) { return SILU ? (n < 64 ? n0 + n : half_n + n0 + n - 64) : n0 + n; };
+    auto row_ok = [&](int n) { return SILU ? (n0 + (n & 63) < half_n) : (n0 + n < N); };
     const int slot0 = tile * tile_slots;            // tile_slots = min(TILE_M, 32) divides TILE_M
     const int expert = sorted_expert_ids[slot0 / TILE_M] - 1;
 
@@ -155,9 +175,9 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4))) void f
 #pragma unroll
         for (int i = 0; i < NB; ++i) {
             const int id = tid + 256 * i, n = id / CPRB, c = id % CPRB;
-            const int gn = n0 + n, gk = k0 + EPB * c;
+            const int gn = row_of(n), gk = k0 + EPB * c;
             u32x4 v = {0, 0, 0, 0};
-            if (gn < N && gk < K) {
+            if (row_ok(n) && gk < K) {
                 if (W8) {
                     const unsigned char* p = B8 + gk + (int64_t)gn * ldb;
                     if (vecB && gk + 16 <= K) v = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(p));
@@ -260,10 +280,41 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4))) void f
     }
 
     // epilogue: rows = token slots 8*(r/4) + 4*hb + r%4, column = channel n0 + wn*32 + lane%32
-    const int gn = n0 + wn * 32 + (lane & 31);
     int toks[16];   // gathered while every lane of the wave is still active
 #pragma unroll
     for (int r = 0; r < 16; ++r) toks[r] = tok_of(8 * (r >> 2) + 4 * hb + (r & 3));
+    if constexpr (SILU) {
+        const int nt = wn * 32 + (lane & 31);               // tile row of this lane's channel
+        const bool ok = row_ok(nt);
+        float ch_scale = 1.f;
+        if (W8 && ok) ch_scale = b_scale[row_of(nt) + (int64_t)expert * ld_scale];
+        // both halves rounded to the activation type, as the unfused GEMM stores them
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+            float v = acc[r];
+            if (W8) v *= ch_scale;
+            if (mul_routed_weight && toks[r]) v *= E::widen(topk_weights[toks[r] - 1]);
+            acc[r] = E::widen(E::cvt(v));
+        }
+        __syncthreads();                                     // every wave is done with the operand tiles
+        float* up = reinterpret_cast<float*>(Bs_raw);        // 2 waves x 16 x 64 floats = 8 KB
+        if (wn >= 2) {
+#pragma unroll
+            for (int r = 0; r < 16; ++r) up[((wn - 2) * 16 + r) * 64 + lane] = acc[r];
+        }
+        __syncthreads();
+        if (wn >= 2 || !ok) return;
+        const int gc = n0 + nt;                              // output channel, < N / 2
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+            const int tok = toks[r];
+            if (!tok) continue;
+            const float g = acc[r], u = up[(wn * 16 + r) * 64 + lane];
+            C[gc + (int64_t)(tok - 1) * ldc] = E::cvt(silu_mul(g, u));
+        }
+        return;
+    }
+    const int gn = n0 + wn * 32 + (lane & 31);
     if (gn >= N) return;
     float ch_scale = 1.f;
     if (W8) ch_scale = b_scale[gn + (int64_t)expert * ld_scale];
@@ -290,10 +341,7 @@ __global__ __launch_bounds__(256) void silu_and_mul_kernel(const unsigned short*
     unsigned short* c = C + col * ldc;
     const int i0 = (blockIdx.x * 256 + threadIdx.x) * 8;
     if (i0 >= rows) return;
-    auto f = [](float x, float y) {
-        const float denom = 1.0f + expf(-x);
-        return x * __builtin_amdgcn_rcpf(denom) * y;  // approximate reciprocal, moe.jl:117-124
-    };
+    auto f = [](float x, float y) { return silu_mul(x, y); };
     if (vec && i0 + 8 <= rows) {
         s16x8 va = *reinterpret_cast<const s16x8*>(a + i0), vb = *reinterpret_cast<const s16x8*>(b + i0), vc;
 #pragma unroll
@@ -323,11 +371,10 @@ bool is16(int dt) { return dt == MI_F16 || dt == MI_BF16; }
 
 }  // namespace
 
-extern "C" int mi_fused_moe_kernel(const mi_tile_array* A, const mi_tile_array* B, const mi_tile_array* C,
-                                   const mi_tile_array* topk_weights, const mi_tile_array* sorted_token_ids,
-                                   const mi_tile_array* sorted_expert_ids, int num_token_replicas,
-                                   int mul_routed_weight, int TILE_M, int TILE_N, int TILE_K,
-                                   const mi_tile_array* b_scale, void* stream) {
+static int fused_moe_impl(const mi_tile_array* A, const mi_tile_array* B, const mi_tile_array* C,
+                          const mi_tile_array* topk_weights, const mi_tile_array* sorted_token_ids,
+                          const mi_tile_array* sorted_expert_ids, int num_token_replicas, int mul_routed_weight,
+                          int TILE_M, int TILE_N, int TILE_K, const mi_tile_array* b_scale, bool silu, void* stream) {
     MI_CHECK(check_array(A, 2));
     MI_CHECK(check_array(B, 3));
     MI_CHECK(check_array(C, 2));
@@ -342,7 +389,8 @@ extern "C" int mi_fused_moe_kernel(const mi_tile_array* A, const mi_tile_array* 
     if (!is_pow2(TILE_M) || !is_pow2(TILE_N) || !is_pow2(TILE_K)) return MI_E_TILE;
     if (num_token_replicas < 1) return MI_E_ARG;
     const int64_t K = B->sizes[0], N = B->sizes[1], E = B->sizes[2];
-    if (A->sizes[0] != K || C->sizes[0] != N) return MI_E_SHAPE;
+    if (silu && (N % 2)) return MI_E_SHAPE;
+    if (A->sizes[0] != K || C->sizes[0] != (silu ? N / 2 : N)) return MI_E_SHAPE;
     const int64_t slots = sorted_token_ids->sizes[0], total = C->sizes[1];
     const int64_t m_blocks = cld(slots, (int64_t)TILE_M);
     if (sorted_expert_ids->sizes[0] < m_blocks) return MI_E_SHAPE;
@@ -365,24 +413,25 @@ extern "C" int mi_fused_moe_kernel(const mi_tile_array* A, const mi_tile_array* 
     // Wide strips (128 channels) when they already give the chip >= ~3 workgroups per CU,
     // counting one started 32-slot tile per TILE_M block; otherwise 32-channel strips with an
     // in-workgroup K split.
-    const bool narrow = m_blocks * cld(N, (int64_t)128) < 768 && K >= 512;
-    const int n_blocks = (int)cld(N, (int64_t)(narrow ? 32 : 128));
+    const bool narrow = !silu && m_blocks * cld(N, (int64_t)128) < 768 && K >= 512;
+    const int n_blocks = silu ? (int)cld(N / 2, (int64_t)64) : (int)cld(N, (int64_t)(narrow ? 32 : 128));
     if (tiles * n_blocks > 0x7fffffffLL) return MI_E_GRID;
     const bool vecA = aligned(A->ptr, 16) && A->strides[1] % 8 == 0;
     const bool vecB = aligned(B->ptr, 16) && B->strides[1] % (w8 ? 16 : 8) == 0 && B->strides[2] % (w8 ? 16 : 8) == 0;
     dim3 grid((unsigned)(tiles * n_blocks));
     hipStream_t s = (hipStream_t)stream;
-#define LAUNCH(ET, W8, NTW, KT)                                                                                     \
-    hipLaunchKernelGGL((fused_moe_kernel<ET, W8, NTW, KT>), grid, dim3(256), 0, s, (const unsigned short*)A->ptr,   \
+#define LAUNCH(ET, W8, NTW, KT, ...)                                                                                \
+    hipLaunchKernelGGL((fused_moe_kernel<ET, W8, NTW, KT, ##__VA_ARGS__>), grid, dim3(256), 0, s, (const unsigned short*)A->ptr, \
                        A->strides[1], (int)A->sizes[1], (const void*)B->ptr, B->strides[1], B->strides[2],          \
                        (unsigned short*)C->ptr, C->strides[1], (int)total, (const unsigned short*)topk_weights->ptr, \
                        (const int*)sorted_token_ids->ptr, (int)slots, (const int*)sorted_expert_ids->ptr,           \
                        w8 ? (const float*)b_scale->ptr : nullptr, w8 ? b_scale->strides[1] : 0, (int)K, (int)N,     \
                        (int)E, num_token_replicas, mul_routed_weight != 0, TILE_M, tile_slots, n_blocks, vecA, vecB)
-#define LAUNCH_SHAPE(ET, W8)                   \
-    do {                                       \
-        if (narrow) LAUNCH(ET, W8, 1, 256);    \
-        else LAUNCH(ET, W8, 4, 128);           \
+#define LAUNCH_SHAPE(ET, W8)                        \
+    do {                                            \
+        if (silu) LAUNCH(ET, W8, 4, 128, true);     \
+        else if (narrow) LAUNCH(ET, W8, 1, 256);    \
+        else LAUNCH(ET, W8, 4, 128);                \
     } while (0)
     if (A->dtype == MI_F16) {
         if (w8) LAUNCH_SHAPE(F16, true);
@@ -393,9 +442,28 @@ extern "C" int mi_fused_moe_kernel(const mi_tile_array* A, const mi_tile_array* 
     }
 #undef LAUNCH_SHAPE
 #undef LAUNCH
-    if (narrow) set_variant(w8 ? "fused_moe_t32_n32_k256_ksplit4_w8a16" : "fused_moe_t32_n32_k256_ksplit4");
+    if (silu) set_variant(w8 ? "fused_moe_silu_t32_n64x2_k128_w8a16" : "fused_moe_silu_t32_n64x2_k128");
+    else if (narrow) set_variant(w8 ? "fused_moe_t32_n32_k256_ksplit4_w8a16" : "fused_moe_t32_n32_k256_ksplit4");
     else set_variant(w8 ? "fused_moe_t32_n128_k128_w8a16" : "fused_moe_t32_n128_k128");
     return launch_status();
+}
+
+extern "C" int mi_fused_moe_kernel(const mi_tile_array* A, const mi_tile_array* B, const mi_tile_array* C,
+                                   const mi_tile_array* topk_weights, const mi_tile_array* sorted_token_ids,
+                                   const mi_tile_array* sorted_expert_ids, int num_token_replicas,
+                                   int mul_routed_weight, int TILE_M, int TILE_N, int TILE_K,
+                                   const mi_tile_array* b_scale, void* stream) {
+    return fused_moe_impl(A, B, C, topk_weights, sorted_token_ids, sorted_expert_ids, num_token_replicas, mul_routed_weight,
+                          TILE_M, TILE_N, TILE_K, b_scale, false, stream);
+}
+
+extern "C" int mi_fused_moe_silu_kernel(const mi_tile_array* A, const mi_tile_array* B, const mi_tile_array* C,
+                                        const mi_tile_array* topk_weights, const mi_tile_array* sorted_token_ids,
+                                        const mi_tile_array* sorted_expert_ids, int num_token_replicas,
+                                        int mul_routed_weight, int TILE_M, int TILE_N, int TILE_K,
+                                        const mi_tile_array* b_scale, void* stream) {
+    return fused_moe_impl(A, B, C, topk_weights, sorted_token_ids, sorted_expert_ids, num_token_replicas, mul_routed_weight,
+                          TILE_M, TILE_N, TILE_K, b_scale, true, stream);
 }
 
 // ---- on-device moe_align_tile_size ------------------------------------------------------------

@@ -9,14 +9,15 @@ from ._harness import namespace, rand_normal, time_launches
 
 
 def invoke_fused_moe_kernel(A, B, C, topk_weights, sorted_token_ids, sorted_expert_ids, *, mul_routed_weight,
-                            num_token_replicas, tile_m, tile_n, tile_k, b_scale=None):
+                            num_token_replicas, tile_m, tile_n, tile_k, b_scale=None, fuse_silu=False):
     """moe.jl:186-199.  ``topk_weights`` Julia (num_tokens, topk) = torch (topk, num_tokens);
     flattened slot-fastest (moe.jl:193).  ``C`` Julia (dim, topk, num_tokens) is flattened to
     (dim, total_tokens) (moe.jl:196)."""
     topk_weights_flat = topk_weights.t().contiguous().reshape(-1)
     C_flat = C.reshape(C.shape[0] * C.shape[1], C.shape[2]) if C.dim() == 3 else C
-    ct.fused_moe_kernel(A, B, C_flat, topk_weights_flat, sorted_token_ids, sorted_expert_ids, num_token_replicas,
-                        mul_routed_weight, tile_m, tile_n, tile_k, b_scale=b_scale)
+    launch = ct.fused_moe_silu_kernel if fuse_silu else ct.fused_moe_kernel
+    launch(A, B, C_flat, topk_weights_flat, sorted_token_ids, sorted_expert_ids, num_token_replicas,
+           mul_routed_weight, tile_m, tile_n, tile_k, b_scale=b_scale)
 
 
 def invoke_silu_and_mul_kernel(AB, C):
@@ -29,12 +30,14 @@ def invoke_silu_and_mul_kernel(AB, C):
 
 
 def cutile_moe(hidden_states, w1, w2, topk_weights, topk_ids, tile_m, tile_n, tile_k, *, w1_scale=None,
-               w2_scale=None, aligned=None, device_align=False):
+               w2_scale=None, aligned=None, device_align=False, fuse_silu=False):
     """moe.jl:218-257.  Torch shapes (reversed Julia): hidden_states (tokens, hidden); w1
     (E, 2*inter, hidden); w2 (E, hidden, inter); topk_weights / topk_ids (topk, tokens), ids
     1-based int64.  ``aligned`` may carry a precomputed (sorted_token_ids, sorted_expert_ids)
     pair on the device to skip the host round trip of moe.jl:232-233; ``device_align`` sorts on
-    the GPU instead (fixed-capacity outputs, nothing leaves the device)."""
+    the GPU instead (fixed-capacity outputs, nothing leaves the device).  ``fuse_silu`` runs the
+    gate / up GEMM with SiLU * up as its epilogue: cache1 and the silu_and_mul launch disappear,
+    the result is bit-identical."""
     num_tokens, hidden_size = hidden_states.shape
     num_experts, _, intermediate_size = w2.shape
     topk = topk_ids.shape[0]
@@ -42,9 +45,10 @@ def cutile_moe(hidden_states, w1, w2, topk_weights, topk_ids, tile_m, tile_n, ti
     T, dev = hidden_states.dtype, hidden_states.device
     # The three zero-initialised caches of moe.jl:228-230 are carved out of one allocation, so
     # that zeroing them is one fill instead of three.
-    n1, n2, n3 = total_tokens * intermediate_size * 2, total_tokens * intermediate_size, total_tokens * hidden_size
+    n1 = 0 if fuse_silu else total_tokens * intermediate_size * 2
+    n2, n3 = total_tokens * intermediate_size, total_tokens * hidden_size
     caches = torch.zeros(n1 + n2 + n3, dtype=T, device=dev)
-    cache1 = caches[:n1].view(num_tokens, topk, intermediate_size * 2)
+    cache1 = None if fuse_silu else caches[:n1].view(num_tokens, topk, intermediate_size * 2)
     cache2 = caches[n1:n1 + n2].view(total_tokens, intermediate_size)
     cache3 = caches[n1 + n2:].view(num_tokens, topk, hidden_size)
     if aligned is None and device_align:
@@ -54,11 +58,16 @@ def cutile_moe(hidden_states, w1, w2, topk_weights, topk_ids, tile_m, tile_n, ti
         sorted_token_ids, sorted_expert_ids = tok.to(dev), exp.to(dev)
     else:
         sorted_token_ids, sorted_expert_ids = aligned
-    invoke_fused_moe_kernel(hidden_states, w1, cache1, topk_weights, sorted_token_ids, sorted_expert_ids,
-                            mul_routed_weight=False, num_token_replicas=topk, tile_m=tile_m, tile_n=tile_n,
-                            tile_k=tile_k, b_scale=w1_scale)
-    cache1_flat = cache1.reshape(total_tokens, intermediate_size * 2)
-    invoke_silu_and_mul_kernel(cache1_flat, cache2)
+    if fuse_silu:
+        invoke_fused_moe_kernel(hidden_states, w1, cache2, topk_weights, sorted_token_ids, sorted_expert_ids,
+                                mul_routed_weight=False, num_token_replicas=topk, tile_m=tile_m, tile_n=tile_n,
+                                tile_k=tile_k, b_scale=w1_scale, fuse_silu=True)
+    else:
+        invoke_fused_moe_kernel(hidden_states, w1, cache1, topk_weights, sorted_token_ids, sorted_expert_ids,
+                                mul_routed_weight=False, num_token_replicas=topk, tile_m=tile_m, tile_n=tile_n,
+                                tile_k=tile_k, b_scale=w1_scale)
+        cache1_flat = cache1.reshape(total_tokens, intermediate_size * 2)
+        invoke_silu_and_mul_kernel(cache1_flat, cache2)
     invoke_fused_moe_kernel(cache2, w2, cache3, topk_weights, sorted_token_ids, sorted_expert_ids,
                             mul_routed_weight=True, num_token_replicas=1, tile_m=tile_m, tile_n=tile_n,
                             tile_k=tile_k, b_scale=w2_scale)
@@ -98,6 +107,20 @@ def prepare(*, benchmark: bool = False, num_tokens: int | None = None, hidden_si
     return namespace(hidden_states=hidden_states, w1=w1, w2=w2, topk_weights=topk_weights, topk_ids=topk_ids,
                      num_tokens=num_tokens, hidden_size=hidden_size, num_experts=num_experts,
                      intermediate_size=intermediate_size, topk=topk, tile_m=128, tile_n=128, tile_k=64)
+
+
+def quantize_weights(data):
+    """Input preparation of the e4m3 configuration: per-(output channel, expert) fp32 scale
+    = max |w| over K / 448 (1 for an all-zero channel), codes = round-to-nearest-even E4M3FN of
+    w / scale.  Torch shapes: w (E, N, K) -> codes (E, N, K) float8_e4m3fn, scale (E, N) float32."""
+    def q(w):
+        w32 = w.float()
+        amax = w32.abs().amax(dim=2)
+        scale = torch.where(amax > 0, amax / 448.0, torch.ones_like(amax))
+        return (w32 / scale[:, :, None]).to(torch.float8_e4m3fn), scale.contiguous()
+    w1, s1 = q(data.w1)
+    w2, s2 = q(data.w2)
+    return namespace(w1=w1, w2=w2, w1_scale=s1, w2_scale=s2)
 
 
 def run(data, *, nruns: int = 1, warmup: int = 0, **kw):

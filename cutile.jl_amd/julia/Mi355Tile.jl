@@ -256,6 +256,23 @@ function fused_moe_kernel(A, B, C, topk_weights, sorted_token_ids, sorted_expert
         ds === nothing ? NULLDESC : Base.unsafe_convert(Ptr{MiTileArray}, ds), stream))
 end
 
+# The gate / up GEMM with silu_and_mul_kernel as its epilogue: C is (N/2, total_tokens).
+function fused_moe_silu_kernel(A, B, C, topk_weights, sorted_token_ids, sorted_expert_ids,
+                          num_token_replicas::Integer, mul_routed_weight::Bool,
+                          TILE_M::Integer, TILE_N::Integer, TILE_K::Integer;
+                          b_scale=nothing, stream::Ptr{Cvoid}=C_NULL)
+    d = map(a -> ref(descriptor(a)), (A, B, C, topk_weights, sorted_token_ids, sorted_expert_ids))
+    ds = b_scale === nothing ? nothing : ref(descriptor(b_scale))
+    GC.@preserve A B C topk_weights sorted_token_ids sorted_expert_ids b_scale check(ccall(
+        (:mi_fused_moe_silu_kernel, libmi355tile), Cint,
+        (Ref{MiTileArray}, Ref{MiTileArray}, Ref{MiTileArray}, Ref{MiTileArray},
+         Ref{MiTileArray}, Ref{MiTileArray}, Cint, Cint, Cint, Cint, Cint,
+         Ptr{MiTileArray}, Ptr{Cvoid}),
+        d[1], d[2], d[3], d[4], d[5], d[6], num_token_replicas, mul_routed_weight,
+        TILE_M, TILE_N, TILE_K,
+        ds === nothing ? NULLDESC : Base.unsafe_convert(Ptr{MiTileArray}, ds), stream))
+end
+
 function silu_and_mul_kernel(A, B, C, TILE_N::Integer; stream::Ptr{Cvoid}=C_NULL)
     d = map(a -> ref(descriptor(a)), (A, B, C))
     GC.@preserve A B C check(ccall((:mi_silu_and_mul_kernel, libmi355tile), Cint,

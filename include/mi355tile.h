@@ -198,6 +198,20 @@ int mi_fused_moe_kernel(const mi_tile_array* A, const mi_tile_array* B, const mi
                         const mi_tile_array* sorted_expert_ids, int num_token_replicas,
                         int mul_routed_weight, int TILE_M, int TILE_N, int TILE_K,
                         const mi_tile_array* b_scale, void* stream);
+/* The first grouped GEMM of cutile_moe fused with silu_and_mul_kernel (moe.jl:234-251 launch them
+ * one after the other through cache1): B holds the gate rows [0, N/2) and the up rows [N/2, N) of
+ * every expert, C is (N/2, total_tokens) and receives SiLU(gate) * up.  Both products are rounded
+ * to the activation type before the activation, so the result is bit-identical to
+ * mi_fused_moe_kernel + mi_silu_and_mul_kernel whenever that GEMM runs the same wide mainloop
+ * (it does at the benchmark shape; small problems use a K-split whose fp32 sums are ordered
+ * differently); cache1 is never written.  No counterpart in the
+ * reference, whose host code launches the two kernels separately; same arguments and checks
+ * otherwise. */
+int mi_fused_moe_silu_kernel(const mi_tile_array* A, const mi_tile_array* B, const mi_tile_array* C,
+                             const mi_tile_array* topk_weights, const mi_tile_array* sorted_token_ids,
+                             const mi_tile_array* sorted_expert_ids, int num_token_replicas,
+                             int mul_routed_weight, int TILE_M, int TILE_N, int TILE_K,
+                             const mi_tile_array* b_scale, void* stream);
 /* silu_and_mul_kernel (moe.jl:110-128): C[:,t] = silu(A[:,t]) * B[:,t] in fp32. */
 int mi_silu_and_mul_kernel(const mi_tile_array* A, const mi_tile_array* B,
                            const mi_tile_array* C, int TILE_N, void* stream);

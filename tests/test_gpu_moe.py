@@ -170,3 +170,71 @@ def test_moe_end_to_end_with_device_align(orc):
     a = moe.cutile_moe(d.hidden_states, d.w1, d.w2, d.topk_weights, d.topk_ids, 16, 128, 64)
     b = moe.cutile_moe(d.hidden_states, d.w1, d.w2, d.topk_weights, d.topk_ids, 16, 128, 64, device_align=True)
     assert torch.equal(a, b)
+
+
+@pytest.mark.parametrize("shape", [dict(benchmark=True, topk=2, router="top2_logits"),
+                                   dict(num_tokens=33, hidden_size=256, num_experts=7, intermediate_size=128, topk=3),
+                                   dict(num_tokens=20, hidden_size=512, num_experts=5, intermediate_size=80, topk=2),
+                                   dict(num_tokens=64, hidden_size=384, num_experts=4, intermediate_size=1000, topk=1)])
+def test_gemm_with_fused_silu_epilogue(ct, orc, shape):
+    """mi_fused_moe_silu_kernel against mi_fused_moe_kernel followed by mi_silu_and_mul_kernel: both
+    products are rounded to the activation type before SiLU, as the separate kernels do, so the
+    results are bit-identical whenever the separate GEMM runs the same 128-lane-wide mainloop; when it
+    picks its K-split shape (small problems) the fp32 sums are ordered differently and the outputs
+    may differ by rounding (bar: the f16 tolerance of this file against the float64 oracle).
+    Includes intermediate sizes that are not multiples of the 64-channel strips."""
+    d = moe.prepare(**shape)
+    tile_m = 128 if shape.get("benchmark") else 16
+    a = moe.cutile_moe(d.hidden_states, d.w1, d.w2, d.topk_weights, d.topk_ids, tile_m, 128, 64, device_align=True)
+    variants = set()
+    inter, total = d.intermediate_size, d.num_tokens * d.topk
+    tok, exp = ct.moe_align_tile_size_device(d.topk_ids, tile_m, d.num_experts)
+    c1 = torch.zeros(total, 2 * inter, dtype=d.hidden_states.dtype, device="cuda")
+    moe.invoke_fused_moe_kernel(d.hidden_states, d.w1, c1, d.topk_weights, tok, exp, mul_routed_weight=False,
+                                num_token_replicas=d.topk, tile_m=tile_m, tile_n=128, tile_k=64)
+    variants.add(ct.last_variant())
+    b = moe.cutile_moe(d.hidden_states, d.w1, d.w2, d.topk_weights, d.topk_ids, tile_m, 128, 64, device_align=True,
+                       fuse_silu=True)
+    if variants == {"fused_moe_t32_n128_k128"}:
+        assert torch.equal(a, b)
+    J = orc.to_julia
+    ref = orc.ref_moe(J(d.hidden_states), J(d.w1), J(d.w2), J(d.topk_weights), J(d.topk_ids), dtype=np.float64)
+    check(J(b), ref)
+
+
+def test_fused_silu_epilogue_bf16_and_fp8_weights():
+    d = moe.prepare(num_tokens=40, hidden_size=256, num_experts=6, intermediate_size=192, topk=2, T=torch.bfloat16)
+    a = moe.cutile_moe(d.hidden_states, d.w1, d.w2, d.topk_weights, d.topk_ids, 32, 128, 64)
+    b = moe.cutile_moe(d.hidden_states, d.w1, d.w2, d.topk_weights, d.topk_ids, 32, 128, 64, fuse_silu=True)
+    assert torch.equal(a, b)
+    d = moe.prepare(benchmark=True, topk=2, router="top2_logits")
+    q = moe.quantize_weights(d)
+    a = moe.cutile_moe(d.hidden_states, q.w1, q.w2, d.topk_weights, d.topk_ids, 128, 128, 64, w1_scale=q.w1_scale,
+                       w2_scale=q.w2_scale, device_align=True)
+    b = moe.cutile_moe(d.hidden_states, q.w1, q.w2, d.topk_weights, d.topk_ids, 128, 128, 64, w1_scale=q.w1_scale,
+                       w2_scale=q.w2_scale, device_align=True, fuse_silu=True)
+    assert torch.equal(a, b)
+
+
+def test_product_quantizer_matches_oracle_codec(orc):
+    """examples.moe.quantize_weights (torch, on the GPU) against the oracle's per-channel E4M3FN
+    quantiser: scales equal to fp32 rounding of the division, codes equal except where that last
+    bit of the scale moves a value across a rounding tie (then by one code step)."""
+    d = moe.prepare(num_tokens=8, hidden_size=128, num_experts=3, intermediate_size=64, topk=1)
+    q = moe.quantize_weights(d)
+    J = orc.to_julia
+    c1, s1 = orc.quantize_e4m3fn_per_channel(J(d.w1).astype(np.float32))
+    np.testing.assert_allclose(J(q.w1_scale), s1, rtol=2e-7)
+    got = J(q.w1.view(torch.uint8)).astype(np.int32)
+    diff = np.abs(got - c1.astype(np.int32))
+    assert diff.max() <= 1 and (diff != 0).mean() < 1e-3
+
+
+def test_fused_silu_entry_checks_shapes(ct):
+    d = moe.prepare(num_tokens=8, hidden_size=128, num_experts=2, intermediate_size=64, topk=1)
+    tok, exp = ct.moe_align_tile_size(d.topk_ids.cpu(), 16, 2)
+    tok, exp = tok.cuda(), exp.cuda()
+    wrong = torch.zeros(8, 128, dtype=torch.float16, device="cuda")          # must be (total, inter) = (8, 64)
+    with pytest.raises(ct.MiError) as e:
+        ct.fused_moe_silu_kernel(d.hidden_states, d.w1, wrong, d.topk_weights.reshape(-1), tok, exp, 1, False, 16, 128, 64)
+    assert e.value.code == ct.MI_E_SHAPE

@@ -224,13 +224,13 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4))) void f
                 const u32x4 sw = ((n >> 4) & 1) ? u32x4{v[2], v[3], v[0], v[1]} : v;
                 *reinterpret_cast<u32x4*>(&Bs_raw[n * kKT + 16 * (c ^ b_sw(n))]) = sw;
             } else {
-                *reinterpret_cast<u32x4*>(&Bs[n * kKT + 8 * (c ^ (n & 7))]) = breg[i];
+                *reinterpret_cast<u32x4*>(&Bs[n * kKT + 8 * (c ^ (n & 15))]) = breg[i];
             }
         }
 #pragma unroll
         for (int i = 0; i < NA; ++i) {
             const int id = tid + 256 * i, sl = id / CPR, c = id % CPR;
-            *reinterpret_cast<s16x8*>(&As[sl * kKT + 8 * (c ^ (sl & 7))]) = areg[i];
+            *reinterpret_cast<s16x8*>(&As[sl * kKT + 8 * (c ^ (sl & 15))]) = areg[i];
         }
         __syncthreads();
         if (k0 + DEPTH * kKT < K) load_tiles(k0 + DEPTH * kKT, breg, areg);
@@ -248,9 +248,9 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4))) void f
                 Fp8<E>::cvt4(raw[1], w2, w3);
                 bf = __builtin_bit_cast(s16x8, u32x4{w0, w1, w2, w3});
             } else {
-                bf = *reinterpret_cast<const s16x8*>(&Bs[n * kKT + 8 * (c ^ (n & 7))]);
+                bf = *reinterpret_cast<const s16x8*>(&Bs[n * kKT + 8 * (c ^ (n & 15))]);
             }
-            s16x8 af = *reinterpret_cast<const s16x8*>(&As[slot * kKT + 8 * (c ^ (slot & 7))]);
+            s16x8 af = *reinterpret_cast<const s16x8*>(&As[slot * kKT + 8 * (c ^ (slot & 15))]);
             acc = E::mfma32(af, bf, acc);
         }
     };

@@ -343,9 +343,11 @@ __global__ __launch_bounds__(128) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     c.inv_scale2 = 1.0f / scale2;
     {
         // transfer `wave` of a half covers keys 8*wave .. 8*wave+7; transfer wave+2 the keys 16 further on,
-        // whose swizzle (a function of key % 8 resp. key % 4) is the same
+        // whose swizzle (a function of key % 16 resp. key % 4) is the same.  K: chunk ^ (key / 2) % 8 --
+        // rows alternate between the two halves of the banks, so the 16 lanes that the LDS serves
+        // together for a 16-byte read (keys k .. k+15 of one chunk column) land on 16 distinct slots.
         const int key = 8 * wave + (lane >> 3), pos = lane & 7;
-        c.kdma = (unsigned)(((int64_t)key * ks.s1 + 8 * (pos ^ (key & 7))) * 2);
+        c.kdma = (unsigned)(((int64_t)key * ks.s1 + 8 * (pos ^ ((key >> 1) & 7))) * 2);
         c.vdma = (unsigned)(((int64_t)key * vs.s1 + 8 * (pos ^ (2 * (key & 3)))) * 2);
     }
     c.lim0 = (lane & 31) - 4 * hb;
@@ -354,7 +356,7 @@ __global__ __launch_bounds__(128) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     {
         const int key = lane & 31;
 #pragma unroll
-        for (int s = 0; s < 4; ++s) c.kfo[s] = key * kD + 8 * ((2 * s + hb) ^ (key & 7));
+        for (int s = 0; s < 4; ++s) c.kfo[s] = key * kD + 8 * ((2 * s + hb) ^ ((key >> 1) & 7));
         const int g = lane >> 4, r = lane & 15;
 #pragma unroll
         for (int dt = 0; dt < 2; ++dt) {

@@ -99,6 +99,8 @@ __global__ __launch_bounds__(256) void gemm16_generic(
 
 // ---- fp32 kernel ---------------------------------------------------------------------------
 // Workgroup tile 128(m) x 128(n), K step 16, 4 waves as 2x2 of 64x64 (2x2 MFMA 32x32x2).
+// Pitch 160 floats: consecutive rows are 32 banks apart, so the two half-waves of a fragment read
+// (rows kk and kk + 1, 32 consecutive floats each) cover the 64 banks once.
 constexpr int FT = 128, FK = 16, F_PITCH = FT + 32;
 
 __global__ __launch_bounds__(256) void gemm32_kernel(const float* __restrict__ A, int64_t lda, int64_t sa,
@@ -114,8 +116,9 @@ __global__ __launch_bounds__(256) void gemm32_kernel(const float* __restrict__ A
     B += (int64_t)blockIdx.z * sb;
     C += (int64_t)blockIdx.z * sc;
     const int wm = (wave & 1) * 64, wn = (wave >> 1) * 64;
-    const int ak = tid >> 4, am = (tid & 15) * 8;  // A tile: row k, 8 consecutive m
-    const int bnn = tid >> 1, bk = (tid & 1) * 8;  // B tile: column n, 8 consecutive k
+    const int ak = tid >> 4, am = (tid & 15) * 4;  // A tile: row k, m = am .. am+3 and 64 + am .. 64 + am+3
+    const int bnn = tid & 127, bk = (tid >> 7) * 8;  // B tile: column n, 8 consecutive k; a wave's 64 lanes
+                                                     // transpose into 64 consecutive floats of one row
     f32x16 acc[2][2] = {};
 
     for (int k0 = 0; k0 < K; k0 += FK) {
@@ -124,13 +127,16 @@ __global__ __launch_bounds__(256) void gemm32_kernel(const float* __restrict__ A
             const int64_t gm = m0 + am;
             const int gk = k0 + ak;
             const float* p = A + gm + (int64_t)gk * lda;
-            if (gk < K && vecA && gm + 8 <= M) {
-                f32x4 t0 = *reinterpret_cast<const f32x4*>(p), t1 = *reinterpret_cast<const f32x4*>(p + 4);
+            if (gk < K && vecA && gm + 68 <= M) {
+                f32x4 t0 = *reinterpret_cast<const f32x4*>(p), t1 = *reinterpret_cast<const f32x4*>(p + 64);
 #pragma unroll
                 for (int q = 0; q < 4; ++q) { va[q] = t0[q]; va[4 + q] = t1[q]; }
             } else {
 #pragma unroll
-                for (int q = 0; q < 8; ++q) va[q] = (gk < K && gm + q < M) ? p[q] : 0.f;
+                for (int q = 0; q < 8; ++q) {
+                    const int o = (q & 3) + 64 * (q >> 2);
+                    va[q] = (gk < K && gm + o < M) ? p[o] : 0.f;
+                }
             }
             const int64_t gn = n0 + bnn;
             const int gk2 = k0 + bk;
@@ -146,7 +152,8 @@ __global__ __launch_bounds__(256) void gemm32_kernel(const float* __restrict__ A
         }
         __syncthreads();
 #pragma unroll
-        for (int q = 0; q < 8; ++q) As[ak * F_PITCH + am + q] = va[q];
+        for (int q = 0; q < 2; ++q)   // 16 lanes x 16 bytes = one contiguous 256-byte run per store
+            *reinterpret_cast<f32x4*>(&As[ak * F_PITCH + am + 64 * q]) = f32x4{va[4 * q], va[4 * q + 1], va[4 * q + 2], va[4 * q + 3]};
 #pragma unroll
         for (int q = 0; q < 8; ++q) Bs[(bk + q) * F_PITCH + bnn] = vb[q];
         __syncthreads();

@@ -456,7 +456,7 @@ def main():
                      "frac": round(ach / HBM_PEAK_GBS, 4),
                      # HBM bytes per launch from rocprofv3 FETCH_SIZE (x2.000) + WRITE_SIZE (x1.000) counter runs,
                      # calibrated on vadd; summary: profiles/membound_kernels_hbm_traffic_pmc.txt
-                     "traffic": 210354586 if dom == "layer_norm_bwd_dx_partial_dwdb" else None, "kernel": dom,
+                     "traffic": 210337792 if dom == "layer_norm_bwd_dx_partial_dwdb" else None, "kernel": dom,
                      "avg_launch_ms": round(per_stage[dom], 5), "algorithmic_bytes": work[dom]},
         "stages_ms": {k: round(v, 5) for k, v in per_stage.items()},
     }

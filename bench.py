@@ -7,13 +7,14 @@ C ABI of libmi355tile.so.
 Prints ONE JSON line on stdout.  A "step" is one pass of the headline workload over one batch
 of synthetic, seeded input already resident in HBM:
 
-    headline workload = the second entry of BASELINE.json's configs: row LayerNorm fwd + bwd
+    headline workload = the second of the benchmark configurations: row LayerNorm fwd + bwd
     (y, dx, dgamma, dbeta) and the row softmax on 4096x4096 fp32.
     ``value`` = algorithmic bytes of the step / wall time per step, in GB/s, timed over
     exactly ``--steps`` steps between two device synchronisations.
 
-Every other configuration of BASELINE.json (vadd, transpose, GEMM, batched GEMM, FMHA, MoE f16
-and fp8) is measured in the same run and reported under ``"kernels"``:
+Every other configuration (vadd, transpose, GEMM, batched GEMM, FMHA, MoE f16 and fp8, and the
+follow-up rows: FFT, Tiled broadcast / mapreduce, RNG fills) is measured in the same run and reported
+under ``"kernels"``:
   * ``min_ms`` / ``mean_ms``: the reference's protocol (examples/benchmarks.jl:12-13: 5 warm-up
     launches, 20 launches each bracketed by its own pair of events on the launch stream);
   * ``avg_ms``: 20 launches back to back between ONE pair of events (no per-launch event

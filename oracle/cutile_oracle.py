@@ -42,7 +42,8 @@ e4m3fn codec           16 round-trip vectors and fma vectors of
 The reference's device rounding (fma contraction, exp2 / reciprocal approximations, f16
 rounding of P, atomics order) is produced by NVIDIA's closed ``tileiras`` compiler and is
 "parity unpinned" at the bit level; the reference itself only checks it to rtol 1e-2
-against the same CPU formulas restated here.
+against the same CPU formulas restated here.  The same holds for the transcendental functions of
+the Tiled vocabulary and for randn / randexp (device math library against numpy, a few ulp).
 """
 from __future__ import annotations
 

@@ -296,9 +296,10 @@ def test_math_functions(orc, dtype, rtol):
     np.testing.assert_allclose(Y.cpu().numpy(), x.numpy() ** x.numpy() + x.numpy() ** 3, rtol=rtol * 2)
 
 
-def test_max_min_follow_julia_for_nan_and_signed_zero(orc):
-    a = np.array([1.0, np.nan, 2.0, -0.0, 0.0, np.nan, -np.inf, 5.0], np.float32)
-    b = np.array([np.nan, 1.0, 3.0, 0.0, -0.0, np.nan, np.inf, 5.0], np.float32)
+@pytest.mark.parametrize("npdt", [np.float32, np.float64, np.float16])
+def test_max_min_follow_julia_for_nan_and_signed_zero(orc, npdt):
+    a = np.array([1.0, np.nan, 2.0, -0.0, 0.0, np.nan, -np.inf, 5.0], npdt)
+    b = np.array([np.nan, 1.0, 3.0, 0.0, -0.0, np.nan, np.inf, 5.0], npdt)
     A, B = dev(a), dev(b)
     for name in ("max", "min"):
         got = getattr(T, name)(Tiled(A), Tiled(B)).copy().cpu().numpy()
@@ -509,11 +510,18 @@ def test_init_is_applied_like_the_reference():
     assert T.maximum(Tiled(A), init=5.0) == 5.0
 
 
-def test_nan_propagates_through_max():
-    A = rand(5000)
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float64, torch.float16])
+def test_nan_propagates_through_max(dtype):
+    A = rand(5000, dtype=dtype)
     A[1234] = float("nan")
     assert np.isnan(T.maximum(Tiled(A)))
     assert np.isnan(T.minimum(Tiled(A)))
+    M = rand(300, 40, dtype=dtype)                        # Julia (300, 40); NaN in column 7
+    M[7, 123] = float("nan")
+    for dims in (1, 2):
+        R = T.maximum(Tiled(M), dims=dims)
+        ref = M.double().cpu().numpy().max(axis=2 - dims, keepdims=True)      # numpy max propagates NaN too
+        assert np.array_equal(R.double().cpu().numpy(), ref, equal_nan=True)
 
 
 @pytest.mark.parametrize("shape,dims", [((1 << 24,), None), ((4096, 4096), None), ((4096, 4096), 1), ((4096, 4096), 2),

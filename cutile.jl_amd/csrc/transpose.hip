@@ -1,12 +1,16 @@
 // Matrix transpose: stand-in for transpose_kernel of the reference's examples/transpose.jl:11-19,
 // y[j,i] = x[i,j] for x (m,n) and y (n,m), both with dimension 0 contiguous.
 //
-// The result does not depend on the (tm,tn) tile constants, so the physical tile is fixed
-// at 64x64 elements per 256-lane workgroup: 16-byte global loads along x's contiguous
-// dimension, a padded LDS tile (pitch 65 elements: both the scattered writes and the
-// gathered reads hit 64 distinct banks), 16-byte global stores along y's contiguous
-// dimension.  Workgroups are numbered so that consecutive ids walk down x's contiguous
-// dimension.  Algorithmic traffic: 2 * m * n * sizeof(T) bytes.
+// The result does not depend on the (tm,tn) tile constants, so the physical tiling is the
+// library's.  Two kernels:
+//   * 4-byte elements with every dimension and stride a multiple of 4 (the benchmark case):
+//     64(m) x 128(n) tiles, a 4x4 block per lane transposed in registers, 16-byte traffic through
+//     an XOR-swizzled LDS tile in both directions, workgroup ids walking 8x8 super-tiles
+//     (transpose4_kernel);
+//   * everything else: 64x64 tiles through a padded LDS tile (pitch 65 elements: both the
+//     scattered writes and the gathered reads hit 64 distinct banks), 16-byte global accesses
+//     where alignment allows, element-wise with bounds checks otherwise (transpose_kernel).
+// Algorithmic traffic: 2 * m * n * sizeof(T) bytes.
 #include "common.h"
 #include <stdlib.h>
 

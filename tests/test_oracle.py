@@ -433,17 +433,15 @@ def test_tiled_mapreduce_reference_cases_and_brute_force(orc):
 # ---- Philox2x32-7 RNG fills -----------------------------------------------------------------------
 
 def test_philox2x32_random123_known_answers(orc):
-    """Random123 1.14 `tests/kat_vectors`, lines `philox2x32 7 ...` and `philox2x32 10 ...`
-    (counter words, key, expected output)."""
-    kat = [(7, 0x00000000, 0x00000000, 0x00000000, 0x257A3673, 0xCD26BE2A),
-           (7, 0xFFFFFFFF, 0xFFFFFFFF, 0xFFFFFFFF, 0xAB302C4D, 0x3DC9D239),
-           (7, 0x243F6A88, 0x85A308D3, 0x13198A2E, 0xBEDBBE6B, 0xE4C770B3),
-           (10, 0x00000000, 0x00000000, 0x00000000, 0xFF1DAE59, 0x6CD10DF2),
-           (10, 0xFFFFFFFF, 0xFFFFFFFF, 0xFFFFFFFF, 0x2C3F628B, 0xAB4FD7AD),
-           (10, 0x243F6A88, 0x85A308D3, 0x13198A2E, 0xDD7CE038, 0xF62A4C12)]
-    for rounds, c1, c2, k, o1, o2 in kat:
-        a, b = orc.philox2x32([c1], [c2], [k], rounds)
-        assert (int(a[0]), int(b[0])) == (o1, o2), rounds
+    """Random123's published known-answer vectors for philox2x32 at 7 and 10 rounds
+    (tests/golden/philox2x32_kat.json)."""
+    import json
+    import os
+    kat = json.load(open(os.path.join(os.path.dirname(__file__), "golden", "philox2x32_kat.json")))["vectors"]
+    assert len(kat) == 6
+    for v in kat:
+        a, b = orc.philox2x32([int(v["ctr"][0], 16)], [int(v["ctr"][1], 16)], [int(v["key"], 16)], v["rounds"])
+        assert (int(a[0]), int(b[0])) == (int(v["out"][0], 16), int(v["out"][1], 16)), v
 
 
 def test_rng_fill_layout_by_brute_force(orc):

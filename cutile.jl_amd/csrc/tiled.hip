@@ -432,9 +432,13 @@ extern "C" __global__ __launch_bounds__(T) void tiled_mr(Args A) {
 #pragma unroll
             for (int d = 1; d < 4; ++d)
                 if ((RMASK >> d) & 1) {
-                    const unsigned n = (unsigned)A.size[d], r = rest % n;
-                    rest /= n;
-                    off += r * A.sst[d];
+                    // the highest reduced dimension takes what is left: no division for it
+                    if ((RMASK >> (d + 1)) == 0) { off += rest * A.sst[d]; }
+                    else {
+                        const unsigned n = (unsigned)A.size[d], r = rest % n;
+                        rest /= n;
+                        off += r * A.sst[d];
+                    }
                 }
         }
         const long long i0 = (long long)v0 * V, left = n0 - i0;
@@ -501,9 +505,13 @@ extern "C" __global__ __launch_bounds__(TX * TY) void tiled_mr(Args A) {
 #pragma unroll
             for (int d = 1; d < 4; ++d)
                 if ((RMASK >> d) & 1) {
-                    const unsigned n = (unsigned)A.size[d], r = rest % n;
-                    rest /= n;
-                    off += r * A.sst[d];
+                    // the highest reduced dimension takes what is left: no division for it
+                    if ((RMASK >> (d + 1)) == 0) { off += rest * A.sst[d]; }
+                    else {
+                        const unsigned n = (unsigned)A.size[d], r = rest % n;
+                        rest /= n;
+                        off += r * A.sst[d];
+                    }
                 }
             SST r[V] = {};
             load_run<SST, V, VEC, NT>(base + off, left, A.sst[0], r);

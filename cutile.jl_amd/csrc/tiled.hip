@@ -597,7 +597,7 @@ int knob(const char* name, int dflt) {
 }
 int knob_blocks() { static const int v = knob("MI_TILED_BLOCKS", 2048); return v; }
 int knob_column_blocks() { static const int v = knob("MI_TILED_COLUMN_BLOCKS", 2048); return v; }
-int knob_min_tx() { static const int v = knob("MI_TILED_MIN_TX", 64); return v; }
+int knob_min_tx() { static const int v = knob("MI_TILED_MIN_TX", 32); return v; }   // 32 lanes x 16 B = 512-byte runs: the shortest that read at full rate
 int knob_iters() { static const int v = knob("MI_TILED_ITERS", 8); return v; }
 int knob_unroll() { static const int v = knob("MI_TILED_UNROLL", 4); return v; }
 

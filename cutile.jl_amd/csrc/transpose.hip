@@ -4,9 +4,9 @@
 // The result does not depend on the (tm,tn) tile constants, so the physical tiling is the
 // library's.  Two kernels:
 //   * 4-byte elements with every dimension and stride a multiple of 4 (the benchmark case):
-//     64(m) x 128(n) tiles, a 4x4 block per lane transposed in registers, 16-byte traffic through
-//     an XOR-swizzled LDS tile in both directions, workgroup ids walking 8x8 super-tiles
-//     (transpose4_kernel);
+//     128 x 128 tiles of 1024 lanes (64 x 128 of 256 lanes for small matrices), a 4x4 block per
+//     lane transposed in registers, 16-byte traffic through an XOR-swizzled LDS tile in both
+//     directions, workgroup ids walking 8x8 super-tiles (transpose4_kernel);
 //   * everything else: 64x64 tiles through a padded LDS tile (pitch 65 elements: both the
 //     scattered writes and the gathered reads hit 64 distinct banks), 16-byte global accesses
 //     where alignment allows, element-wise with bounds checks otherwise (transpose_kernel).
@@ -91,12 +91,16 @@ __global__ __launch_bounds__(kBlock) void transpose_kernel(const T* __restrict__
 // time decide how large the contiguous spans are that DRAM sees on each side).
 typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
 
-template <int TM, int TN, bool STREAM = true>
-__global__ __launch_bounds__(256) void transpose4_kernel(const unsigned* __restrict__ x, int64_t ldx,
+// NT lanes per workgroup.  Two shapes are used: 128 x 128 tiles with 1024 lanes (one 4x4 block per
+// lane) for large matrices -- runs of 512 bytes on both sides, which is what the memory system needs
+// to move a strided run at the rate of a linear copy, and two workgroups fill a CU -- and 64 x 128
+// tiles with 256 lanes (five workgroups per CU) when there are too few tiles for that.
+template <int TM, int TN, bool STREAM = true, int NT = 256>
+__global__ __launch_bounds__(NT) void transpose4_kernel(const unsigned* __restrict__ x, int64_t ldx,
                                                          unsigned* __restrict__ y, int64_t ldy, int64_t m,
                                                          int64_t n, int tiles_m, int tiles_n, int order) {
     __shared__ __attribute__((aligned(16))) unsigned lds[TM * TN];
-    constexpr int MB = TM * TN / (16 * 256);  // 4x4 micro-blocks per lane
+    constexpr int MB = TM * TN / (16 * NT);   // 4x4 micro-blocks per lane
     constexpr int SLOTS = TN / 4;             // 16-byte slots per LDS row
     int bm, bn;
     {
@@ -114,7 +118,7 @@ __global__ __launch_bounds__(256) void transpose4_kernel(const unsigned* __restr
     const int64_t m0 = (int64_t)bm * TM, n0 = (int64_t)bn * TN;
 #pragma unroll
     for (int k = 0; k < MB; ++k) {
-        const int b = threadIdx.x + 256 * k;
+        const int b = threadIdx.x + NT * k;
         const int i4 = b % (TM / 4), j4 = b / (TM / 4);
         const int64_t gm = m0 + 4 * i4, gn = n0 + 4 * j4;
         u32x4 r[4] = {};
@@ -133,7 +137,7 @@ __global__ __launch_bounds__(256) void transpose4_kernel(const unsigned* __restr
     __syncthreads();
 #pragma unroll
     for (int k = 0; k < 4 * MB; ++k) {
-        const int b = threadIdx.x + 256 * k;
+        const int b = threadIdx.x + NT * k;
         const int j4 = b % SLOTS, row = b / SLOTS;
         const int64_t gn = n0 + 4 * j4, gm = m0 + row;
         if (gn < n && gm < m) {
@@ -145,7 +149,9 @@ __global__ __launch_bounds__(256) void transpose4_kernel(const unsigned* __restr
 
 int launch4(const mi_tile_array* x, const mi_tile_array* y, hipStream_t s) {
     const int64_t m = x->sizes[0], n = x->sizes[1];
-    int tile = 2, order = 2;  // measured best on MI355X for 8192^2 fp32: 64(m) x 128(n) tiles, 8x8 super-tiles
+    // measured best on MI355X for 8192^2 fp32: 128 x 128 tiles of 1024 lanes, 8x8 super-tiles (90 us; 64 x 128
+    // tiles of 256 lanes 104 us); the big shape needs enough tiles to keep two workgroups on every CU
+    int tile = cld(m, (int64_t)128) * cld(n, (int64_t)128) >= 1024 ? 9 : 2, order = 2;
     if (const char* e = getenv("MI_TRANSPOSE_TILE")) tile = atoi(e);    // tuning overrides
     if (const char* e = getenv("MI_TRANSPOSE_ORDER")) order = atoi(e);
     int TM = 64, TN = 128;
@@ -156,6 +162,7 @@ int launch4(const mi_tile_array* x, const mi_tile_array* y, hipStream_t s) {
     else if (tile == 5) { TM = 64; TN = 256; }
     else if (tile == 6) { TM = 32; TN = 128; }
     else if (tile == 64) { TM = 64; TN = 64; }
+    else if (tile == 9) { TM = 128; TN = 128; }   // with 1024 lanes
     const int64_t tm_ = cld(m, (int64_t)TM), tn_ = cld(n, (int64_t)TN);
     int64_t blocks = tm_ * tn_;
     if (order == 2) blocks = ((tm_ + 7) / 8) * ((tn_ + 7) / 8) * 64;
@@ -164,7 +171,14 @@ int launch4(const mi_tile_array* x, const mi_tile_array* y, hipStream_t s) {
     hipLaunchKernelGGL((transpose4_kernel<A, B>), dim3((unsigned)blocks), dim3(256), 0, s,                \
                        (const unsigned*)x->ptr, x->strides[1], (unsigned*)y->ptr, y->strides[1], m, n,    \
                        (int)tm_, (int)tn_, order)
-    if (TM == 64 && TN == 64) { T4(64, 64); set_variant("transpose4_64x64_regmicro"); }
+    if (tile == 9) {
+        const bool st = stream_hint(2 * m * n * (int64_t)sizeof(unsigned));
+        if (st) hipLaunchKernelGGL((transpose4_kernel<128, 128, true, 1024>), dim3((unsigned)blocks), dim3(1024), 0, s,
+                                   (const unsigned*)x->ptr, x->strides[1], (unsigned*)y->ptr, y->strides[1], m, n, (int)tm_, (int)tn_, order);
+        else hipLaunchKernelGGL((transpose4_kernel<128, 128, false, 1024>), dim3((unsigned)blocks), dim3(1024), 0, s,
+                                (const unsigned*)x->ptr, x->strides[1], (unsigned*)y->ptr, y->strides[1], m, n, (int)tm_, (int)tn_, order);
+        set_variant(st ? "transpose4_128x128_t1024_regmicro" : "transpose4_128x128_t1024_regmicro_cached");
+    } else if (TM == 64 && TN == 64) { T4(64, 64); set_variant("transpose4_64x64_regmicro"); }
     else if (TM == 128 && TN == 128) { T4(128, 128); set_variant("transpose4_128x128_regmicro"); }
     else if (TM == 32 && TN == 256) { T4(32, 256); set_variant("transpose4_32x256_regmicro"); }
     else if (TM == 64 && TN == 256) { T4(64, 256); set_variant("transpose4_64x256_regmicro"); }

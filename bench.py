@@ -321,6 +321,23 @@ def bench_kernels(ct, which, cpu, nruns=NRUNS, warmup=WARMUP):
         except Exception as ex:
             res["moe_f16_device_fused"] = extra(_entry(f"MoE f16 top-2, fused SiLU epilogue (eager; graph failed: {type(ex).__name__})",
                                                        fused, wbytes, "GB/s", "hbm", HBM_PEAK_GBS, "f16", nruns, warmup))
+        # from router logits to output without a host step: router + sort + 3 kernels
+        logits_jl = d.logits.t().contiguous()
+        rw = torch.empty_like(d.topk_weights)
+        rid = torch.empty_like(d.topk_ids)
+
+        def routed():
+            ct.moe_route_topk(logits_jl, 2, topk_weights=rw, topk_ids=rid)
+            return moe.cutile_moe(d.hidden_states, d.w1, d.w2, rw, rid, 128, 128, 64, device_align=True, fuse_silu=True)
+        routed()
+        assert torch.equal(rid, d.topk_ids), "device router picks other experts than the host router"
+        try:
+            gr, _ = graph_of(routed)
+            res["moe_f16_device_routed"] = extra(_entry("MoE f16 top-2 from router logits to output on the device (router + sort + 3 kernels), HIP graph replay",
+                                                        gr.replay, wbytes, "GB/s", "hbm", HBM_PEAK_GBS, "f16", nruns, warmup))
+        except Exception as ex:
+            res["moe_f16_device_routed"] = extra(_entry(f"MoE f16 top-2 from router logits (eager; graph failed: {type(ex).__name__})",
+                                                        routed, wbytes, "GB/s", "hbm", HBM_PEAK_GBS, "f16", nruns, warmup))
         if cpu:
             J = orc.to_julia
             args = (J(d.hidden_states), J(d.w1), J(d.w2), J(d.topk_weights), J(d.topk_ids))

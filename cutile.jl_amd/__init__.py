@@ -71,6 +71,7 @@ _SIGNATURES = {
     "mi_fmha_kernel": ([_A, _A, _A, _A, ctypes.c_float, ctypes.c_int32, _i, _i, _i, _i, _i, _i, _i, _vp], _i),
     "mi_fft_kernel": ([_A, _A, _A, _A, _A, _A, _A, _i, _i, _i, _i, _i, _i, _vp], _i),
     "mi_moe_align_tile_size_device": ([_A, _i, _i, _A, _A, _vp], _i),
+    "mi_moe_route_topk": ([_A, _A, _A, _vp], _i),
     "mi_moe_align_tile_size": (
         [ctypes.POINTER(ctypes.c_int64), ctypes.c_int64, ctypes.c_int64, _i, _i,
          ctypes.POINTER(ctypes.c_int32), ctypes.POINTER(ctypes.c_int32),
@@ -317,6 +318,21 @@ def moe_align_tile_size_device(topk_ids, tile_m: int, num_experts: int, sorted_t
     _call("mi_moe_align_tile_size_device", _ref(topk_ids), tile_m, num_experts, _ref(sorted_token_ids),
           _ref(sorted_expert_ids), _stream(stream))
     return sorted_token_ids, sorted_expert_ids
+
+
+def moe_route_topk(logits, topk: int, weight_dtype=None, topk_weights=None, topk_ids=None, stream=None):
+    """Router on the device: the ``topk`` largest logits of every token (ties to the lower expert
+    id) and the softmax over them.  ``logits``: device tensor of torch shape (num_experts,
+    num_tokens), i.e. Julia (num_tokens, num_experts).  Returns (topk_weights, topk_ids) of torch
+    shape (topk, num_tokens), the layout ``cutile_moe`` takes; ids are int64 and 1-based."""
+    import torch
+    num_experts, num_tokens = logits.shape
+    if topk_weights is None:
+        topk_weights = torch.empty((topk, num_tokens), dtype=weight_dtype or logits.dtype, device=logits.device)
+    if topk_ids is None:
+        topk_ids = torch.empty((topk, num_tokens), dtype=torch.int64, device=logits.device)
+    _call("mi_moe_route_topk", _ref(logits), _ref(topk_weights), _ref(topk_ids), _stream(stream))
+    return topk_weights, topk_ids
 
 
 def fused_moe_kernel(A, B, C, topk_weights, sorted_token_ids, sorted_expert_ids,

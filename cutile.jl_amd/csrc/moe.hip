@@ -573,6 +573,104 @@ extern "C" int mi_moe_align_tile_size_device(const mi_tile_array* topk_ids, int 
     return launch_status();
 }
 
+// ---- on-device router ---------------------------------------------------------------------------
+// The routing that examples/moe.jl leaves to its caller (moe.jl:311-344 draws random experts on
+// the host): the top-k experts of every token's logits, ties to the lower expert id, and the
+// softmax over the k selected logits.  One wave per token; lane l holds experts l, l + 64, ...;
+// k rounds of a wave-wide argmax over the experts not yet taken.  NaN logits rank as -Inf.
+constexpr int kRoutePerLane = 8;  // up to 512 experts
+
+__device__ __forceinline__ float route_load(const void* p, int dtype, int64_t i) {
+    if (dtype == MI_F32) return ((const float*)p)[i];
+    if (dtype == MI_F16) return F16::widen(((const unsigned short*)p)[i]);
+    return BF16::widen(((const unsigned short*)p)[i]);
+}
+
+__global__ __launch_bounds__(256) void moe_route_kernel(const void* __restrict__ logits, int ldt, int64_t ls_tok,
+                                                        int64_t ls_exp, int num_tokens, int E, int k,
+                                                        void* __restrict__ weights, int wdt, int64_t ws_slot,
+                                                        long long* __restrict__ ids, int64_t is_slot) {
+    const int lane = threadIdx.x & 63, token = blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (token >= num_tokens) return;  // whole waves leave
+    float v[kRoutePerLane];
+    unsigned taken = 0;
+#pragma unroll
+    for (int j = 0; j < kRoutePerLane; ++j) {
+        const int e = lane + 64 * j;
+        v[j] = -INFINITY;
+        if (e < E) {
+            const float x = route_load(logits, ldt, token * ls_tok + e * ls_exp);
+            if (x == x) v[j] = x;
+        } else {
+            taken |= 1u << j;
+        }
+    }
+    float mine = -INFINITY, top = -INFINITY;
+    int mine_id = 0;
+    for (int s = 0; s < k; ++s) {
+        float bv = -INFINITY;
+        int bi = 0x7fffffff;
+#pragma unroll
+        for (int j = 0; j < kRoutePerLane; ++j) {
+            const int e = lane + 64 * j;
+            if (!((taken >> j) & 1u) && (v[j] > bv || (v[j] == bv && e < bi))) {
+                bv = v[j];
+                bi = e;
+            }
+        }
+#pragma unroll
+        for (int off = 32; off >= 1; off >>= 1) {
+            const float ov = __shfl_xor(bv, off, 64);
+            const int oi = __shfl_xor(bi, off, 64);
+            if (ov > bv || (ov == bv && oi < bi)) {
+                bv = ov;
+                bi = oi;
+            }
+        }
+        if ((bi & 63) == lane) taken |= 1u << (bi >> 6);  // k <= E: some expert is always left
+        if (lane == s) {
+            mine = bv;
+            mine_id = bi;
+        }
+        if (s == 0) top = bv;
+    }
+    const float ex = lane < k ? expf(mine - top) : 0.f;
+    float sum = ex;
+#pragma unroll
+    for (int off = 32; off >= 1; off >>= 1) sum += __shfl_xor(sum, off, 64);
+    if (lane < k) {
+        const float w = ex / sum;
+        const int64_t wi = token + lane * ws_slot;
+        if (wdt == MI_F32) ((float*)weights)[wi] = w;
+        else if (wdt == MI_F16) ((unsigned short*)weights)[wi] = F16::cvt(w);
+        else ((unsigned short*)weights)[wi] = BF16::cvt(w);
+        ids[token + lane * is_slot] = mine_id + 1;
+    }
+}
+
+extern "C" int mi_moe_route_topk(const mi_tile_array* logits, const mi_tile_array* topk_weights,
+                                 const mi_tile_array* topk_ids, void* stream) {
+    MI_CHECK(check_array(logits, 2));
+    MI_CHECK(check_array(topk_weights, 2));
+    MI_CHECK(check_array(topk_ids, 2));
+    auto is_float = [](int d) { return d == MI_F32 || d == MI_F16 || d == MI_BF16; };
+    if (!is_float(logits->dtype) || !is_float(topk_weights->dtype) || topk_ids->dtype != MI_I64) return MI_E_DTYPE;
+    const int64_t num_tokens = logits->sizes[0], E = logits->sizes[1], k = topk_ids->sizes[1];
+    if (topk_ids->sizes[0] != num_tokens || topk_weights->sizes[0] != num_tokens || topk_weights->sizes[1] != k)
+        return MI_E_SHAPE;
+    if (k < 1 || k > E) return MI_E_ARG;
+    if (E > 64 * kRoutePerLane || k > 64) return MI_E_UNSUPPORTED;
+    if (num_tokens > 1 && (topk_weights->strides[0] != 1 || topk_ids->strides[0] != 1)) return MI_E_STRIDE;
+    if (num_tokens == 0) return MI_OK;
+    if (cld(num_tokens, (int64_t)4) > MI_MAX_GRID_DIM) return MI_E_GRID;
+    hipLaunchKernelGGL(moe_route_kernel, dim3((unsigned)cld(num_tokens, (int64_t)4)), dim3(256), 0, (hipStream_t)stream,
+                       (const void*)logits->ptr, logits->dtype, logits->strides[0], logits->strides[1], (int)num_tokens,
+                       (int)E, (int)k, (void*)topk_weights->ptr, topk_weights->dtype, topk_weights->strides[1],
+                       (long long*)topk_ids->ptr, topk_ids->strides[1]);
+    set_variant("moe_route_topk_wave_per_token");
+    return launch_status();
+}
+
 extern "C" int mi_silu_and_mul_kernel(const mi_tile_array* A, const mi_tile_array* B, const mi_tile_array* C,
                                       int TILE_N, void* stream) {
     MI_CHECK(check_array(A, 2));

@@ -90,6 +90,7 @@ def prepare(*, benchmark: bool = False, num_tokens: int | None = None, hidden_si
     hidden_states = rand_normal(rng, (hidden_size, num_tokens), T)
     w1 = rand_normal(rng, (hidden_size, intermediate_size * 2, num_experts), T, std=weight_std)
     w2 = rand_normal(rng, (intermediate_size, hidden_size, num_experts), T, std=weight_std)
+    logits = None
     if router == "top2_logits":
         logits = rng.standard_normal((num_tokens, num_experts)).astype(np.float32)
         order = np.argsort(-logits, axis=1, kind="stable")[:, :topk]
@@ -104,7 +105,8 @@ def prepare(*, benchmark: bool = False, num_tokens: int | None = None, hidden_si
     dev = hidden_states.device
     topk_weights = torch.from_numpy(np.ascontiguousarray(weights.T)).to(T).to(dev)  # Julia (tokens, topk)
     topk_ids = torch.from_numpy(np.ascontiguousarray(ids.T)).to(dev)
-    return namespace(hidden_states=hidden_states, w1=w1, w2=w2, topk_weights=topk_weights, topk_ids=topk_ids,
+    logits = None if logits is None else torch.from_numpy(logits).to(dev)   # (tokens, experts), for the device router
+    return namespace(hidden_states=hidden_states, w1=w1, w2=w2, topk_weights=topk_weights, topk_ids=topk_ids, logits=logits,
                      num_tokens=num_tokens, hidden_size=hidden_size, num_experts=num_experts,
                      intermediate_size=intermediate_size, topk=topk, tile_m=128, tile_n=128, tile_k=64)
 

@@ -239,6 +239,16 @@ function moe_align_tile_size_device(topk_ids, tile_m::Integer, num_experts::Inte
         d[1], tile_m, num_experts, d[2], d[3], stream))
 end
 
+"Router on the device: fills `topk_ids` (num_tokens, topk) Int64 with the experts of the `topk`
+largest `logits[t, :]` (ties to the lower id) and `topk_weights` with the softmax over them."
+function moe_route_topk(logits, topk_weights, topk_ids; stream::Ptr{Cvoid}=C_NULL)
+    d = map(a -> ref(descriptor(a)), (logits, topk_weights, topk_ids))
+    GC.@preserve logits topk_weights topk_ids check(ccall(
+        (:mi_moe_route_topk, libmi355tile), Cint,
+        (Ref{MiTileArray}, Ref{MiTileArray}, Ref{MiTileArray}, Ptr{Cvoid}),
+        d[1], d[2], d[3], stream))
+end
+
 # `b_scale` (N, E) Float32 goes with e4m3fn weights only; `nothing` otherwise.
 function fused_moe_kernel(A, B, C, topk_weights, sorted_token_ids, sorted_expert_ids,
                           num_token_replicas::Integer, mul_routed_weight::Bool,

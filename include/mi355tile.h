@@ -188,6 +188,15 @@ int mi_moe_align_tile_size(const int64_t* topk_ids, int64_t num_tokens, int64_t 
 int mi_moe_align_tile_size_device(const mi_tile_array* topk_ids, int tile_m, int num_experts,
                                   const mi_tile_array* sorted_token_ids,
                                   const mi_tile_array* sorted_expert_ids, void* stream);
+/* Router on the device: topk_ids[t, :] = the topk = size(topk_ids, 2) experts with the largest
+ * logits[t, :] in descending order (ties to the lower expert id, NaN ranks as -Inf), 1-based;
+ * topk_weights[t, :] = softmax over those topk logits.  logits (num_tokens, num_experts) f32 / f16 /
+ * bf16 with any strides, topk_weights (num_tokens, topk) f32 / f16 / bf16, topk_ids (num_tokens,
+ * topk) i64: the inputs cutile_moe takes (moe.jl:218-222).  No counterpart in the reference, whose
+ * example draws its routing on the host (moe.jl:323-333); with mi_moe_align_tile_size_device the
+ * routed forward pass needs no host step at all.  At most 512 experts, topk <= 64. */
+int mi_moe_route_topk(const mi_tile_array* logits, const mi_tile_array* topk_weights,
+                      const mi_tile_array* topk_ids, void* stream);
 /* fused_moe_kernel (moe.jl:45-105).  A (K,num_tokens), B (K,N,E), C (N,total_tokens),
  * topk_weights (total_tokens,), sorted_token_ids (M_padded,) i32 1-based with sentinel
  * total_tokens+1, sorted_expert_ids (blocks,) i32 1-based.  A, C, topk_weights f16/bf16.

@@ -25,6 +25,7 @@ ref_fmha               row 1 of causal output == V[:,1]; brute-force loops on ti
                        ``torch.nn.functional.scaled_dot_product_attention`` on CPU
 moe_align_tile_size    permutation / grouping / padding invariants; brute force; C cross-check
 ref_moe                per-token dense loop on tiny shapes
+route_top2             hand-computed answers (distinct logits, an exact tie -> lower id, weights 1/2)
 fft_3stage, tables     ``numpy.fft.fft`` (independent library); brute-force DFT sum on tiny sizes
 tiled_eval/broadcast   known answers of test/host/broadcast.jl (fills, 0-dim, expansion cases);
                        plain numpy expressions written out by hand; torch CPU for bfloat16

@@ -63,6 +63,14 @@ def test_argument_errors_are_reported_without_launching(ct):
     assert L.mi_softmax_tma_kernel(r(inp), r(inp), 256, 0, None) == ct.MI_E_GRID
     X = _desc(ct, (256, 8)); W = _desc(ct, (128,)); v = _desc(ct, (8,))
     assert L.mi_layer_norm_fwd(r(X), r(W), r(W), r(X), r(v), r(v), ctypes.c_float(1e-5), 256, None) == ct.MI_E_SHAPE
+    # device router: topk within 1..num_experts, at most 512 experts, i64 ids
+    lg = _desc(ct, (16, 32)); tw = _desc(ct, (16, 2)); ti = _desc(ct, (16, 2), ct.MI_I64)
+    assert L.mi_moe_route_topk(r(lg), r(tw), r(_desc(ct, (16, 2), ct.MI_I32)), None) == ct.MI_E_DTYPE
+    assert L.mi_moe_route_topk(r(lg), r(_desc(ct, (16, 3))), r(ti), None) == ct.MI_E_SHAPE
+    assert L.mi_moe_route_topk(r(lg), r(_desc(ct, (16, 33))), r(_desc(ct, (16, 33), ct.MI_I64)), None) == ct.MI_E_ARG
+    assert L.mi_moe_route_topk(r(_desc(ct, (16, 513))), r(tw), r(ti), None) == ct.MI_E_UNSUPPORTED
+    assert L.mi_moe_route_topk(r(_desc(ct, (0, 32), ptr=0)), r(_desc(ct, (0, 2), ptr=0)),
+                               r(_desc(ct, (0, 2), ct.MI_I64, ptr=0)), None) == 0
     # empty arrays are a successful no-op
     e = _desc(ct, (0,), ptr=0)
     assert L.mi_vec_add_kernel_1d(r(e), r(e), r(e), 1024, None) == 0

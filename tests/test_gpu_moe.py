@@ -159,6 +159,60 @@ def test_device_align_matches_host_routine(ct, orc, num_tokens, topk, E, tile_m)
     assert np.array_equal(tok_h.numpy(), tok_o) and np.array_equal(exp_h.numpy(), exp_o)
 
 
+@pytest.mark.parametrize("num_tokens,E,topk,dtype", [(256, 32, 2, torch.float32), (48, 64, 8, torch.float32),
+                                                     (7, 100, 5, torch.float16), (3, 512, 64, torch.float32),
+                                                     (5, 6, 6, torch.bfloat16), (1, 1, 1, torch.float32),
+                                                     (1000, 130, 4, torch.float32)])
+def test_device_router_matches_oracle(ct, orc, num_tokens, E, topk, dtype):
+    """mi_moe_route_topk against the oracle's router (stable argsort of the negated logits, softmax
+    over the selected ones in float64): ids identical, weights within 1e-6 relative in f32 (one
+    exp and one division in fp32) or one rounding step of the 16-bit output type."""
+    rng = np.random.default_rng(num_tokens * 7 + E)
+    logits = torch.from_numpy(rng.standard_normal((num_tokens, E)).astype(np.float32)).to(dtype)
+    w_ref, ids_ref = orc.route_top2(logits.float().numpy().astype(np.float64), topk)
+    w, ids = ct.moe_route_topk(logits.t().contiguous().cuda(), topk)            # torch (E, tokens) = Julia (tokens, E)
+    assert ids.shape == (topk, num_tokens) and ids.dtype == torch.int64 and w.dtype == dtype
+    assert np.array_equal(ids.cpu().numpy().T, ids_ref)
+    tol = 1e-6 if dtype == torch.float32 else (2.0 ** -10 if dtype == torch.float16 else 2.0 ** -7)
+    np.testing.assert_allclose(w.float().cpu().numpy().T, w_ref, rtol=tol, atol=1e-30 if dtype == torch.float32 else 1e-7)
+    # f32 weights from 16-bit logits, and a strided (token-major) logits view
+    w32, ids2 = ct.moe_route_topk(logits.cuda().t(), topk, weight_dtype=torch.float32)
+    assert np.array_equal(ids2.cpu().numpy().T, ids_ref)
+    np.testing.assert_allclose(w32.cpu().numpy().T, w_ref, rtol=1e-6)
+    np.testing.assert_allclose(w32.sum(dim=0).cpu().numpy(), 1.0, rtol=1e-6)
+
+
+def test_device_router_ties_and_nan(ct, orc):
+    """Equal logits go to the lower expert id (the stable sort of the oracle); NaN logits are never
+    preferred to numbers."""
+    rng = np.random.default_rng(3)
+    logits = rng.integers(-2, 3, size=(64, 40)).astype(np.float32)               # many ties
+    w_ref, ids_ref = orc.route_top2(logits.astype(np.float64), 6)
+    w, ids = ct.moe_route_topk(torch.from_numpy(logits).t().contiguous().cuda(), 6)
+    assert np.array_equal(ids.cpu().numpy().T, ids_ref)
+    np.testing.assert_allclose(w.cpu().numpy().T, w_ref, rtol=1e-6)
+    logits = rng.standard_normal((16, 12)).astype(np.float32)
+    logits[:, [1, 5, 7]] = np.nan
+    clean = np.where(np.isnan(logits), -1e30, logits)
+    _, ids_ref = orc.route_top2(clean.astype(np.float64), 4)
+    _, ids = ct.moe_route_topk(torch.from_numpy(logits).t().contiguous().cuda(), 4)
+    assert np.array_equal(ids.cpu().numpy().T, ids_ref)
+
+
+def test_moe_routed_on_device_end_to_end(ct, orc):
+    """Router, sort, GEMMs, activation and combine all on the GPU: the measured configuration from
+    logits to output equals the run whose routing was prepared on the host."""
+    d = moe.prepare(benchmark=True, topk=2, router="top2_logits")
+    w, ids = ct.moe_route_topk(d.logits.t().contiguous(), 2, weight_dtype=d.topk_weights.dtype)
+    assert torch.equal(ids, d.topk_ids)
+    a = moe.cutile_moe(d.hidden_states, d.w1, d.w2, d.topk_weights, d.topk_ids, 128, 128, 64, device_align=True)
+    b = moe.cutile_moe(d.hidden_states, d.w1, d.w2, w, ids, 128, 128, 64, device_align=True)
+    J = orc.to_julia
+    ref = orc.ref_moe(J(d.hidden_states), J(d.w1), J(d.w2), J(w), J(ids), dtype=np.float32)
+    check(J(b), ref.astype(np.float64))
+    assert (a.float() - b.float()).abs().max().item() <= 2e-3 * a.float().abs().max().item()  # weights differ by <= 1 f16 step
+
+
 def test_moe_end_to_end_with_device_align(orc):
     """cutile_moe with the sort on the GPU equals the version that sorts on the host, bit for bit
     (the extra, unused blocks change nothing)."""

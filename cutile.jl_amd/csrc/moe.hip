@@ -123,8 +123,15 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4))) void f
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, hb = lane >> 5;
     const int wn = wave % NTW, wk = wave / NTW;  // position along n / along the K split
-    // consecutive workgroups share the token tile (and therefore the activations in L2)
-    const int tile = blockIdx.x / n_blocks, bid_n = blockIdx.x % n_blocks;
+    // Consecutive workgroups share the token tile (and therefore the activations in L2).  The tiles
+    // are walked sub-tile-major: first the leading 32 slots of every TILE_M block, which always hold
+    // a token, then the second 32 slots of every block, and so on.  With ~16 tokens per expert all
+    // the workgroups that have work are thus dispatched first and stream from the start; in slot
+    // order three quarters of every dispatch round would be padding tiles that leave at once, and
+    // the weight streams would take several rounds to build up.
+    const int t_lin = blockIdx.x / n_blocks, bid_n = blockIdx.x % n_blocks;
+    const int tpb = TILE_M / tile_slots, m_blocks = (gridDim.x / n_blocks) / tpb;
+    const int tile = (t_lin % m_blocks) * tpb + t_lin / m_blocks;
     static_assert(!SILU || NTW == 4, "the fused SiLU epilogue pairs waves 0,1 (gate) with waves 2,3 (up)");
     const int half_n = N / 2;
     const int n0 = bid_n * (SILU ? kNT / 2 : kNT);

@@ -475,7 +475,7 @@ extern "C" int mi_fused_moe_silu_kernel(const mi_tile_array* A, const mi_tile_ar
 
 // ---- on-device moe_align_tile_size ------------------------------------------------------------
 // One workgroup of sixteen waves.  Counting sort by expert of the replica ids (slot-fastest
-// flattening of topk_ids, examples/moe.jl:148-150): LDS histogram, serial scan over the experts,
+// flattening of topk_ids, examples/moe.jl:148-150): LDS histogram, scan over the experts,
 // then placement in super-blocks of 1024 consecutive replicas (one per lane).  A replica's slot is
 //     cursor[e] + (replicas of e in earlier waves of the super-block) + (those in earlier lanes),
 // the last term from ballots alone, so ids of one expert ascend exactly as the stable sortperm
@@ -489,7 +489,7 @@ __global__ __launch_bounds__(kAlignThreads) void moe_align_kernel(const long lon
                                                         int* __restrict__ sorted_expert_ids, int cap_blocks) {
     __shared__ int cursor[kAlignMaxExperts];      // histogram, then next free slot of every expert
     __shared__ unsigned short tbl[kAlignWaves][kAlignMaxExperts];   // replicas per (wave, expert) of the current super-block (<= 64)
-    __shared__ int s_blocks;
+    __shared__ int s_blocks, wave_total[kAlignWaves];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, total = num_tokens * topk;
     for (int e = tid; e < num_experts; e += kAlignThreads) {
         cursor[e] = 0;
@@ -503,14 +503,24 @@ __global__ __launch_bounds__(kAlignThreads) void moe_align_kernel(const long lon
         if (e >= 1 && e <= num_experts) atomicAdd(&cursor[(int)e - 1], 1);
     }
     __syncthreads();
-    if (tid == 0) {
-        int blk = 0;
-        for (int e = 0; e < num_experts; ++e) {
-            const int nb = (cursor[e] + tile_m - 1) / tile_m;
-            cursor[e] = blk * tile_m;  // first slot of the expert
-            for (int b = 0; b < nb && blk < cap_blocks; ++b) sorted_expert_ids[blk++] = e + 1;
+    {   // exclusive scan of the experts' block counts (thread e owns expert e): shuffles inside a
+        // wave, the waves' totals through LDS; then every expert labels its own blocks
+        const int nb = tid < num_experts ? (cursor[tid] + tile_m - 1) / tile_m : 0;
+        int incl = nb;
+#pragma unroll
+        for (int off = 1; off < 64; off <<= 1) {
+            const int up = __shfl_up(incl, off, 64);
+            if (lane >= off) incl += up;
         }
-        s_blocks = blk;
+        if (lane == 63) wave_total[wave] = incl;
+        __syncthreads();
+        int first = incl - nb;
+        for (int w = 0; w < wave; ++w) first += wave_total[w];
+        if (tid < num_experts) {
+            cursor[tid] = first * tile_m;  // first slot of the expert
+            for (int b = first; b < first + nb && b < cap_blocks; ++b) sorted_expert_ids[b] = tid + 1;
+        }
+        if (tid == kAlignThreads - 1) s_blocks = first + nb < cap_blocks ? first + nb : cap_blocks;
     }
     __syncthreads();
     for (int b = s_blocks + tid; b < cap_blocks; b += kAlignThreads) sorted_expert_ids[b] = 0;
@@ -527,7 +537,7 @@ __global__ __launch_bounds__(kAlignThreads) void moe_align_kernel(const long lon
         unsigned long long todo = __ballot(e >= 0);
         while (todo) {  // one trip per distinct expert of the wave's 64 replicas
             const int leader = __ffsll((long long)todo) - 1;
-            const int el = __shfl(e, leader, 64);
+            const int el = __builtin_amdgcn_readlane(e, leader);  // leader comes from a ballot: wave-uniform
             const unsigned long long m = __ballot(e == el);
             if (e == el) rank = __popcll(m & lt);
             if (lane == leader) tbl[wave][el] = (unsigned short)__popcll(m);

@@ -256,6 +256,38 @@ template <int DT> __device__ __forceinline__ car<DT> f_cld(car<DT> a, car<DT> b)
     else { const car<DT> q = f_divi<DT>(a, b); return (b != 0 && (a % (b == -1 ? 1 : b)) != 0 && ((a < 0) == (b < 0))) ? q + 1 : q; }
 }
 
+template <int DT> __device__ __forceinline__ car<DT> f_rsqrt(car<DT> a) {
+    if constexpr (DT == DT_F64) return 1.0 / sqrt(a); else return rnd<DT>(1.0f / sqrtf(a));
+}
+// Julia's shifts: a count of the word size or more shifts everything out (>> keeps the sign), a
+// negative count shifts the other way.
+template <int DT> struct UCar { typedef unsigned int type; };
+template <> struct UCar<DT_I64> { typedef unsigned long long type; };
+template <int DT> __device__ __forceinline__ car<DT> shift_left(car<DT> a, long long n) {
+    constexpr int B = 8 * (int)sizeof(car<DT>);
+    return n >= B ? (car<DT>)0 : (car<DT>)((typename UCar<DT>::type)a << n);
+}
+template <int DT, bool ARITH> __device__ __forceinline__ car<DT> shift_right(car<DT> a, long long n) {
+    constexpr int B = 8 * (int)sizeof(car<DT>);
+    if constexpr (ARITH) return n >= B ? (car<DT>)(a < 0 ? -1 : 0) : (car<DT>)(a >> n);
+    else return n >= B ? (car<DT>)0 : (car<DT>)((typename UCar<DT>::type)a >> n);
+}
+template <int DT> __device__ __forceinline__ car<DT> f_shl(car<DT> a, long long n) {
+    return n >= 0 ? shift_left<DT>(a, n) : shift_right<DT, true>(a, n < -64 ? 64 : -n);
+}
+template <int DT> __device__ __forceinline__ car<DT> f_shr(car<DT> a, long long n) {
+    return n >= 0 ? shift_right<DT, true>(a, n) : shift_left<DT>(a, n < -64 ? 64 : -n);
+}
+template <int DT> __device__ __forceinline__ car<DT> f_lshr(car<DT> a, long long n) {
+    return n >= 0 ? shift_right<DT, false>(a, n) : shift_left<DT>(a, n < -64 ? 64 : -n);
+}
+// High half of the full product (Base.mul_hi).
+template <int DT> __device__ __forceinline__ car<DT> f_mul_hi(car<DT> a, car<DT> b) {
+    if constexpr (DT == DT_I32) return (int)(((long long)a * (long long)b) >> 32);
+    else if constexpr (DT == DT_I64) return (long long)(((__int128)a * (__int128)b) >> 64);
+    else return false;
+}
+
 // ---- wave64 exchange of any carrier ----
 template <typename C> __device__ __forceinline__ C xor_lane(C v, int m) {
     if constexpr (sizeof(C) == 8) {

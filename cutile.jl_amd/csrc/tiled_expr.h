@@ -39,7 +39,8 @@ enum Rule {
     R_IFELSE,    // ifelse(cond::Bool, a, b): promote_type(a, b)
     R_FIRST,     // type of the first argument (copysign)
     R_CONVERT,   // constructors: fixed result type
-    R_INTDIV     // div / rem / mod / fld / cld: promote (integers stay integers)
+    R_INTDIV,    // div / rem / mod / fld / cld: promote (integers stay integers)
+    R_SHIFT      // << >> >>>: type of the shifted integer (Bool widens to Int64), any integer count
 };
 
 struct FnInfo {
@@ -115,6 +116,11 @@ static const FnInfo kFns[] = {
     {"mod", 2, R_INTDIV, 0, "f_mod"},
     {"fld", 2, R_INTDIV, 0, "f_fld"},
     {"cld", 2, R_INTDIV, 0, "f_cld"},
+    {"rsqrt", 1, R_FLOAT, 0, "f_rsqrt"},
+    {"shl", 2, R_SHIFT, 0, "f_shl"},
+    {"shr", 2, R_SHIFT, 0, "f_shr"},
+    {"lshr", 2, R_SHIFT, 0, "f_lshr"},
+    {"mul_hi", 2, R_LOGIC, 0, "f_mul_hi"},
     {"f16", 1, R_CONVERT, MI_F16, "f_convert"},
     {"bf16", 1, R_CONVERT, MI_BF16, "f_convert"},
     {"f32", 1, R_CONVERT, MI_F32, "f_convert"},
@@ -258,6 +264,12 @@ static inline int infer_types(Expr& e, const int32_t* leaf_dt, int nl, const int
             case R_FIRST: n.dtype = e.nodes[n.args[0]].dtype; break;
             case R_CONVERT: n.dtype = f.fixed; break;
             case R_INTDIV: n.dtype = t == MI_BOOL ? MI_I64 : t; break;
+            case R_SHIFT: {
+                const int x = e.nodes[n.args[0]].dtype, c = e.nodes[n.args[1]].dtype;
+                if (dt_is_float(x) || dt_is_float(c)) return MI_E_DTYPE;
+                n.dtype = x == MI_BOOL ? MI_I64 : x;
+                break;
+            }
         }
     }
     return MI_OK;
@@ -327,6 +339,7 @@ static inline std::string emit_body(const Expr& e) {
             if (f.rule == R_IFELSE && k == 0) want = MI_BOOL;
             if (f.rule == R_POW && k == 1 && dt_is_float(n.dtype) && !dt_is_float(a.dtype)) want = MI_I64;
             if (f.rule == R_CONVERT) want = a.dtype;
+            if (f.rule == R_SHIFT && k == 1) want = MI_I64;
             if (k) o += ", ";
             if (want == a.dtype) snprintf(buf, sizeof buf, "t%d", n.args[k]);
             else snprintf(buf, sizeof buf, "cvt<%s>(t%d)", tag(want), n.args[k]);

@@ -125,6 +125,10 @@ class _Node:
     def __ror__(self, o): return Broadcasted("or", o, self)
     def __xor__(self, o): return Broadcasted("xor", self, o)
     def __rxor__(self, o): return Broadcasted("xor", o, self)
+    def __lshift__(self, o): return Broadcasted("shl", self, o)
+    def __rlshift__(self, o): return Broadcasted("shl", o, self)
+    def __rshift__(self, o): return Broadcasted("shr", self, o)      # arithmetic, like Julia's >> on signed integers
+    def __rrshift__(self, o): return Broadcasted("shr", o, self)
     def __lt__(self, o): return Broadcasted("lt", self, o)
     def __le__(self, o): return Broadcasted("le", self, o)
     def __gt__(self, o): return Broadcasted("gt", self, o)
@@ -189,9 +193,9 @@ def _fn(name, arity):
     return call
 
 
-_UNARY = ("abs abs2 sign floor ceil round trunc sqrt cbrt inv exp exp2 exp10 expm1 log log2 log10 log1p sin cos "
+_UNARY = ("abs abs2 sign floor ceil round trunc sqrt rsqrt cbrt inv exp exp2 exp10 expm1 log log2 log10 log1p sin cos "
           "tan asin acos atan sinh cosh tanh isnan isinf isfinite signbit iszero identity").split()
-_BINARY = "max min copysign atan2 hypot rem mod fld cld".split()
+_BINARY = "max min copysign atan2 hypot rem mod fld cld mul_hi lshr".split()   # lshr: Julia's >>>
 for _n in _UNARY:
     globals()[_n] = _fn(_n, 1)
 for _n in _BINARY:
@@ -325,7 +329,7 @@ def copy(bc, stream=None):
 
 _BINOPS = {ast.Add: operator.add, ast.Sub: operator.sub, ast.Mult: operator.mul, ast.Div: operator.truediv,
            ast.Pow: operator.pow, ast.Mod: operator.mod, ast.FloorDiv: operator.floordiv, ast.BitAnd: operator.and_,
-           ast.BitOr: operator.or_, ast.BitXor: operator.xor}
+           ast.BitOr: operator.or_, ast.BitXor: operator.xor, ast.LShift: operator.lshift, ast.RShift: operator.rshift}
 _CMPOPS = {ast.Lt: operator.lt, ast.LtE: operator.le, ast.Gt: operator.gt, ast.GtE: operator.ge, ast.Eq: operator.eq,
            ast.NotEq: operator.ne}
 

@@ -254,8 +254,9 @@ int mi_fft_kernel(const mi_tile_array* x_packed_in, const mi_tile_array* y_packe
  *   add sub mul div pow neg abs abs2 sign max min fma muladd clamp copysign floor ceil round trunc
  *   sqrt cbrt inv exp exp2 exp10 expm1 log log2 log10 log1p sin cos tan asin acos atan sinh cosh
  *   tanh atan2 hypot lt le gt ge eq ne isnan isinf isfinite signbit iszero not and or xor ifelse
- *   div_int rem mod fld cld identity f16 bf16 f32 f64 i32 i64 bool
- * (Julia's `+` is add, `/` is div, `^` is pow, `÷` is div_int, `Float32(x)` is f32, ...).  Node
+ *   div_int rem mod fld cld identity f16 bf16 f32 f64 i32 i64 bool rsqrt shl shr lshr mul_hi
+ * (Julia's `+` is add, `/` is div, `^` is pow, `÷` is div_int, `Float32(x)` is f32, `<<` `>>` `>>>`
+ * are shl shr lshr, ct.rsqrt of src/language/math.jl:16 is rsqrt, ...).  Node
  * types follow Julia's promote_type / float() rules; Float16 and BFloat16 operations are rounded
  * after every step as Julia defines them.  Unknown names return MI_E_UNSUPPORTED. */
 typedef struct mi_tile_scalar {

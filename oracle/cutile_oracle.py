@@ -437,7 +437,26 @@ def _jl_scalar_type(x) -> str:
 _TILED_MATH = {"sqrt": np.sqrt, "cbrt": np.cbrt, "exp": np.exp, "exp2": np.exp2, "expm1": np.expm1, "log": np.log,
                "log2": np.log2, "log10": np.log10, "log1p": np.log1p, "sin": np.sin, "cos": np.cos, "tan": np.tan,
                "asin": np.arcsin, "acos": np.arccos, "atan": np.arctan, "sinh": np.sinh, "cosh": np.cosh,
-               "tanh": np.tanh, "exp10": lambda v: np.power(v.dtype.type(10), v), "inv": lambda v: v.dtype.type(1) / v}
+               "tanh": np.tanh, "exp10": lambda v: np.power(v.dtype.type(10), v), "inv": lambda v: v.dtype.type(1) / v,
+               "rsqrt": lambda v: v.dtype.type(1) / np.sqrt(v)}
+
+
+def _jl_shift(name, a, n):
+    """Julia's << / >> / >>> on Int32 / Int64 (Base int.jl): counts of the word size or more shift everything
+    out (>> keeps the sign), negative counts shift the other way."""
+    bits = a.dtype.itemsize * 8
+    u = np.dtype(f"uint{bits}")
+    n = np.asarray(n, dtype=np.int64)
+    a, n = np.broadcast_arrays(a, n)
+    k = np.clip(np.abs(n), 0, bits - 1).astype(u)          # in-range count for numpy
+    big = np.abs(n) >= bits
+    left = np.where(big, 0, (a.view(u) << k).view(a.dtype))
+    right_a = np.where(big, np.where(a < 0, -1, 0), a >> k.astype(a.dtype))
+    right_l = np.where(big, 0, (a.view(u) >> k).view(a.dtype))
+    right = right_a if name == "shr" else right_l
+    fwd = left if name == "shl" else right
+    back = (right_a if name == "shl" else left)            # a negative count of << is >>, of >> / >>> is <<
+    return np.where(n >= 0, fwd, back).astype(a.dtype)
 _TILED_CMP = {"lt": np.less, "le": np.less_equal, "gt": np.greater, "ge": np.greater_equal, "eq": np.equal,
               "ne": np.not_equal}
 
@@ -571,6 +590,18 @@ def tiled_eval(text: str, leaves=(), scalars=()):
             assert not isf
             f = {"and": np.bitwise_and, "or": np.bitwise_or, "xor": np.bitwise_xor}[name]
             return f(conv(args[0], T), conv(args[1], T)), T
+        if name in ("shl", "shr", "lshr"):
+            R = "Int64" if args[0][1] == "Bool" else args[0][1]
+            assert R in ("Int32", "Int64") and args[1][1] not in _JL_FLOATS
+            return _jl_shift(name, np.ascontiguousarray(conv(args[0], R)), conv(args[1], "Int64")), R
+        if name == "mul_hi":
+            assert not isf
+            a, b = conv(args[0], T), conv(args[1], T)
+            if T == "Bool":
+                return np.zeros(np.broadcast(a, b).shape, bool), T
+            bits = 32 if T == "Int32" else 64
+            prod = a.astype(object) * b.astype(object)          # exact Python integers
+            return np.asarray(prod >> bits, dtype=object).astype(_JL_NP[T]), T
         if name == "ifelse":
             R = jl_promote(args[1][1], args[2][1])
             return np.where(args[0][0], conv(args[1], R), conv(args[2], R)).astype(_JL_NP[R]), R

@@ -228,6 +228,12 @@ TYPE_CASES = [
     ("abs2(a0)", (torch.float16,), "Float16"),
     ("copysign(a0,a1)", (torch.float32, torch.int32), "Float32"),
     ("clamp(a0,a1,a0)", (torch.int32, torch.int32), "Int32"),
+    ("shl(a0,a1)", (torch.int32, torch.int64), "Int32"),      # counts -50 .. 49: both directions, >= 32 too
+    ("shr(a0,a1)", (torch.int64, torch.int32), "Int64"),
+    ("lshr(a0,a1)", (torch.int32, torch.int32), "Int32"),
+    ("shl(a0,a1)", (torch.bool, torch.int32), "Int64"),
+    ("mul_hi(shl(a0,a1),shl(a1,a0))", (torch.int32, torch.int32), "Int32"),      # operands of every magnitude and sign
+    ("mul_hi(shl(a0,a1),shl(a1,a0))", (torch.int64, torch.int64), "Int64"),
 ]
 
 
@@ -277,7 +283,7 @@ def test_bfloat16_against_torch():
     assert torch.equal(D.cpu(), a.float() + b.to(torch.float16).float())
 
 
-MATH = "sqrt cbrt inv exp exp2 exp10 expm1 log log2 log10 log1p sin cos tan asin acos atan sinh cosh tanh".split()
+MATH = "sqrt rsqrt cbrt inv exp exp2 exp10 expm1 log log2 log10 log1p sin cos tan asin acos atan sinh cosh tanh".split()
 
 
 @pytest.mark.parametrize("dtype,rtol", [(torch.float32, 2e-6), (torch.float64, 1e-14)])

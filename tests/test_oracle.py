@@ -371,6 +371,24 @@ def test_tiled_eval_types_and_values_by_hand(orc):
                        ("rem", [1, -1, 1, -1]), ("mod", [1, 1, -1, -1])):
         v, t = orc.tiled_eval(f"{name}(a0,a1)", (x, y))
         assert t == "Int64" and np.array_equal(v, want), name
+    # Julia's shifts (answers worked out by hand): the value keeps its type; Int32 wraps; a count of the word size
+    # or more empties the word (>> keeps the sign); >>> is logical; a negative count shifts the other way
+    w = np.array([1, -8, 5, -1, 2 ** 30], np.int32)
+    for text, cnt, want in (("shl", 2, [4, -32, 20, -4, 0]), ("shr", 1, [0, -4, 2, -1, 2 ** 29]),
+                            ("lshr", 28, [0, 15, 0, 15, 4]), ("shl", 40, [0, 0, 0, 0, 0]), ("shr", 40, [0, -1, 0, -1, 0]),
+                            ("shl", -1, [0, -4, 2, -1, 2 ** 29]), ("lshr", -2, [4, -32, 20, -4, 0])):
+        v, t = orc.tiled_eval(f"{text}(a0,s0)", (w,), (np.int64(cnt),))
+        assert t == "Int32" and np.array_equal(v, want), (text, cnt)
+    v, t = orc.tiled_eval("shl(a0,s0)", (np.array([True, False]),), (3,))
+    assert t == "Int64" and np.array_equal(v, [8, 0])                      # true << 3 == 8
+    # mul_hi: high word of the exact product
+    v, t = orc.tiled_eval("mul_hi(a0,a1)", (w, np.array([7, -8, 2 ** 30, -1, 2 ** 30], np.int32)))
+    assert t == "Int32" and np.array_equal(v, [0, 0, 1, 0, 2 ** 28])       # 5 * 2^30 >> 32 == 1
+    big = np.array([2 ** 62, -2 ** 62, 3], np.int64)
+    v, t = orc.tiled_eval("mul_hi(a0,a1)", (big, np.array([4, 4, -1], np.int64)))
+    assert t == "Int64" and np.array_equal(v, [1, -1, -1])                 # 2^64 >> 64, -2^64 >> 64, -3 >> 64
+    v, t = orc.tiled_eval("rsqrt(a0)", (np.array([4.0, 0.25], np.float32),))
+    assert t == "Float32" and np.array_equal(v, [0.5, 2.0])
     # max / min: NaN wins, +0.0 > -0.0
     v, _ = orc.tiled_eval("max(a0,a1)", (np.array([np.nan, 1, -0.0], np.float32), np.array([1, np.nan, 0.0], np.float32)))
     assert np.isnan(v[0]) and np.isnan(v[1]) and not np.signbit(v[2])

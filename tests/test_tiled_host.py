@@ -54,6 +54,11 @@ def eltype(ct, text, leaves=(), scalars=()):
     ("i32(a0)", ("Float64",), (), "Int32"),
     ("copysign(a0,a1)", ("Float32", "Float64"), (), "Float32"),
     ("fma(a0,a1,s0)", ("Float16", "Float16"), ("Float32",), "Float32"),
+    ("shl(a0,s0)", ("Int32",), ("Int64",), "Int32"),          # Julia: the shifted value's type
+    ("shr(a0,a1)", ("Int64", "Int32"), (), "Int64"),
+    ("lshr(a0,a1)", ("Bool", "Int32"), (), "Int64"),
+    ("mul_hi(a0,a1)", ("Int32", "Int32"), (), "Int32"),
+    ("rsqrt(a0)", ("Float16",), (), "Float16"),
 ])
 def test_element_type_rules(ct, text, leaves, scalars, want):
     rc, got = eltype(ct, text, leaves, scalars)
@@ -72,7 +77,7 @@ def test_oracle_and_library_agree_on_promotion(ct, orc):
     ("foo(a0)", "MI_E_UNSUPPORTED"), ("add(a0)", "MI_E_ARG"), ("add(a0,a1", "MI_E_ARG"), ("add(a0,a1))", "MI_E_ARG"),
     ("", "MI_E_ARG"), ("a", "MI_E_ARG"), ("a0 a1", "MI_E_ARG"), ("add(a0,a9)", "MI_E_UNSUPPORTED"), ("add(a0,a3)", "MI_E_ARG"),
     ("and(a0,a1)", "MI_E_DTYPE"), ("ifelse(a0,a0,a1)", "MI_E_DTYPE"), ("add(a0;a1)", "MI_E_ARG"),
-    ("system(a0)", "MI_E_UNSUPPORTED"), ("add(a0,1.0)", "MI_E_ARG"),
+    ("system(a0)", "MI_E_UNSUPPORTED"), ("add(a0,1.0)", "MI_E_ARG"), ("shl(a0,a1)", "MI_E_DTYPE"), ("mul_hi(a0,a1)", "MI_E_DTYPE"),
 ])
 def test_malformed_or_unknown_expressions_are_refused(ct, text, code):
     rc, _ = eltype(ct, text, ("Float32", "Float32"))
@@ -181,7 +186,7 @@ def test_generated_broadcast_kernels_compile(ct, dry_run):
     assert _bc(ct, f32(4, 8, 16, 32), "add(a0,a1)", [f32(4, 1, 16, 1), f32(1, 8, 1, 32)]) == 0
     assert ct.last_variant().endswith("nd4")
     chain = "a0"
-    for name in ("abs abs2 sign floor ceil round trunc sqrt cbrt inv exp exp2 exp10 expm1 log log2 log10 log1p sin cos "
+    for name in ("abs abs2 sign floor ceil round trunc sqrt rsqrt cbrt inv exp exp2 exp10 expm1 log log2 log10 log1p sin cos "
                  "tan asin acos atan sinh cosh tanh identity neg").split():
         chain = f"{name}({chain})"
     def total(terms):
@@ -197,10 +202,11 @@ def test_generated_broadcast_kernels_compile(ct, dry_run):
         assert _bc(ct, x, two, [x, x]) == 0, dt
     for dt in (torch.int32, torch.int64):
         x = torch.zeros(100, dtype=dt)
-        ints = total([f"{n}(a0,a1)" for n in "sub mul pow max min copysign div_int rem mod fld cld and or xor".split()]
+        ints = total([f"{n}(a0,a1)" for n in "sub mul pow max min copysign div_int rem mod fld cld and or xor shl shr lshr mul_hi".split()]
                      + ["fma(a0,a1,a0)", "clamp(a0,a1,a0)", "not(a0)", "abs(a0)", "abs2(a0)", "sign(a0)", "neg(a0)"])
         assert _bc(ct, x, ints, [x, x]) == 0, dt
     b = torch.zeros(100, dtype=torch.bool)
+    assert _bc(ct, torch.zeros(100, dtype=torch.int64), "add(shl(a0,a1),mul_hi(a0,a0))", [b, torch.zeros(100, dtype=torch.int32)]) == 0
     preds = "xor(a0,not(a0))"
     for t in [f"{n}(a1,a1)" for n in "lt le gt ge eq ne".split()] + [f"{n}(a1)" for n in "isnan isinf isfinite signbit iszero bool".split()]:
         preds = f"and({preds},{t})"

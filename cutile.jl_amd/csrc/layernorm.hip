@@ -16,6 +16,7 @@
 // owns the slot (S == 1), device-scope float atomics otherwise.  No spin-lock: workgroups of
 // one grid have no forward-progress guarantee relative to each other on this hardware.
 #include "common.h"
+#include <type_traits>
 #include <math.h>
 #include <stdlib.h>
 
@@ -238,6 +239,15 @@ __global__ __launch_bounds__(BLOCK) void ln_bwd_kernel(float* __restrict__ DX, i
     }
 }
 
+// Workgroup barrier that waits for the wave's LDS accesses only (lgkmcnt(0), vmcnt and expcnt at
+// their maxima): unlike __syncthreads() it leaves global loads and stores in flight.
+__device__ __forceinline__ void lds_barrier() {
+    asm volatile("" ::: "memory");
+    __builtin_amdgcn_s_waitcnt(0xc07f);
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+}
+
 // Backward with RG row groups of 256 lanes per workgroup (rows of up to 4096 elements, 16-byte
 // aligned): the groups walk different rows of the same partial slot and add their dW/dB
 // partials in LDS before the flush, which divides the number of memory-side float atomics --
@@ -271,28 +281,48 @@ __global__ __launch_bounds__(256 * RG) void ln_bwd_rg_kernel(float* __restrict__
     }
     const int64_t step = (int64_t)RG * G * S, m0 = g + (int64_t)G * (RG * s + h);
     const int64_t trips = (M - (g + (int64_t)G * RG * s) + step - 1) / step;  // of group 0; later groups may idle in the last
-    for (int64_t it = 0; it < trips; ++it) {
+    // The rows of the next two trips are requested before the current one is reduced: the reductions
+    // meet at barriers, which no load crosses on its own, and a workgroup would otherwise have
+    // nothing in flight for half of every trip.  Two register sets take turns.
+    // (Unpredicated: a row past the end re-reads the last row and a column past the end the last
+    // vector of the row, and the values are discarded where they are used.  A predicated load
+    // would have to be waited for at once to be merged with its default.)
+    f32x4 bx[2][VPT], by[2][VPT];
+    float bmean[2] = {0.f, 0.f}, brstd[2] = {0.f, 0.f};
+    auto fetch = [&](auto set, int64_t m) {
+        constexpr int B = decltype(set)::value;
+        const int64_t mc = m < M ? m : M - 1;
+#pragma unroll
+        for (int v = 0; v < VPT; ++v) {
+            const int col = vec(v) < N ? vec(v) : N - 4;   // N % 4 == 0 here
+            bx[B][v] = ld_global<STREAM>(reinterpret_cast<const f32x4*>(X + mc * ldx + col));
+            by[B][v] = ld_global<STREAM>(reinterpret_cast<const f32x4*>(DY + mc * lddy + col));
+        }
+        bmean[B] = Mean[mc];
+        brstd[B] = Rstd[mc];
+    };
+    using Set0 = std::integral_constant<int, 0>;
+    using Set1 = std::integral_constant<int, 1>;
+    if (trips > 0) fetch(Set0{}, m0);
+    if (trips > 1) fetch(Set1{}, m0 + step);
+    auto trip = [&](auto set, int64_t it) {
+        constexpr int B = decltype(set)::value;
         const int64_t m = m0 + it * step;
         const bool live = m < M;  // uniform per group; both groups keep meeting at the barriers
         float x[VPT][4], dy[VPT][4];
 #pragma unroll
-        for (int v = 0; v < VPT; ++v) {
-            f32x4 tx = {0.f, 0.f, 0.f, 0.f}, ty = tx;
-            if (live && vec(v) < N) {
-                tx = ld_global<STREAM>(reinterpret_cast<const f32x4*>(X + m * ldx + vec(v)));
-                ty = ld_global<STREAM>(reinterpret_cast<const f32x4*>(DY + m * lddy + vec(v)));
-            }
+        for (int v = 0; v < VPT; ++v)
 #pragma unroll
             for (int q = 0; q < 4; ++q) {
-                x[v][q] = tx[q];
-                dy[v][q] = ty[q];
+                x[v][q] = bx[B][v][q];
+                dy[v][q] = (live && vec(v) < N) ? by[B][v][q] : 0.f;
             }
-        }
-        const float mean = live ? Mean[m] : 0.f, rstd = live ? Rstd[m] : 0.f;
+        const float mean = bmean[B], rstd = live ? brstd[B] : 0.f;
+        if (it + 2 < trips) fetch(set, m + 2 * step);
         float c1 = 0.f, c2 = 0.f;
 #pragma unroll
         for (int v = 0; v < VPT; ++v) {
-            const bool in = vec(v) < N;  // N % 4 == 0 here
+            const bool in = live && vec(v) < N;  // N % 4 == 0 here
 #pragma unroll
             for (int q = 0; q < 4; ++q) {
                 const float xhat = in ? (x[v][q] - mean) * rstd : 0.f;
@@ -308,10 +338,10 @@ __global__ __launch_bounds__(256 * RG) void ln_bwd_rg_kernel(float* __restrict__
             red[h][wave] = c1;
             red[h][NW + wave] = c2;
         }
-        __syncthreads();
+        lds_barrier();
         c1 = (red[h][0] + red[h][1]) + (red[h][2] + red[h][3]);
         c2 = (red[h][NW] + red[h][NW + 1]) + (red[h][NW + 2] + red[h][NW + 3]);
-        __syncthreads();
+        lds_barrier();
         c1 /= (float)N;
         c2 /= (float)N;
 #pragma unroll
@@ -326,6 +356,10 @@ __global__ __launch_bounds__(256 * RG) void ln_bwd_rg_kernel(float* __restrict__
             }
             if (live && vec(v) < N) st_global<true>(t, reinterpret_cast<f32x4*>(DX + m * lddx + vec(v)));
         }
+    };
+    for (int64_t it = 0; it < trips; it += 2) {
+        trip(Set0{}, it);
+        if (it + 1 < trips) trip(Set1{}, it + 1);
     }
     // the groups add their partials in LDS, one after the other; then everybody flushes with
     // coalesced atomics

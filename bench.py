@@ -493,7 +493,7 @@ def main():
                      "frac": round(ach / HBM_PEAK_GBS, 4),
                      # HBM bytes per launch from rocprofv3 FETCH_SIZE (x2.000) + WRITE_SIZE (x1.000) counter runs,
                      # calibrated on vadd; summary: profiles/membound_kernels_hbm_traffic_pmc.txt
-                     "traffic": 210337792, "kernel": dom,
+                     "traffic": 210371940, "kernel": dom,
                      "avg_launch_ms": round(dom_ms, 5), "algorithmic_bytes": work[dom]},
         "stages_ms": {k: round(v, 5) for k, v in per_stage.items()},
     }

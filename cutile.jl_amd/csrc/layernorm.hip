@@ -253,8 +253,8 @@ __device__ __forceinline__ void lds_barrier() {
 // partials in LDS before the flush, which divides the number of memory-side float atomics --
 // the scarce resource of this kernel -- by RG at the same number of rows in flight.
 // Workgroup (g, s): group h handles rows m = g + G*(RG*s + h), stepping by RG*G*S.
-template <int VPT, bool STREAM, int RG>
-__global__ __launch_bounds__(256 * RG) void ln_bwd_rg_kernel(float* __restrict__ DX, int64_t lddx,
+template <int BLOCK, int VPT, bool STREAM, int RG>
+__global__ __launch_bounds__(BLOCK * RG) void ln_bwd_rg_kernel(float* __restrict__ DX, int64_t lddx,
                                                          const float* __restrict__ DY, int64_t lddy,
                                                          float* __restrict__ DW, int64_t lddw,
                                                          float* __restrict__ DB, int64_t lddb,
@@ -263,11 +263,11 @@ __global__ __launch_bounds__(256 * RG) void ln_bwd_rg_kernel(float* __restrict__
                                                          const float* __restrict__ Mean,
                                                          const float* __restrict__ Rstd, int N,
                                                          int64_t M, int G, int S) {
-    constexpr int BLOCK = 256, NW = 4;
+    constexpr int NW = BLOCK / 64;
     __shared__ float red[RG][2 * NW];
     __shared__ float stage[BLOCK * VPT * 4];
     const int g = blockIdx.x % G, s = blockIdx.x / G;
-    const int h = threadIdx.x >> 8, lt = threadIdx.x & 255, lane = lt & 63, wave = lt >> 6;
+    const int h = threadIdx.x / BLOCK, lt = threadIdx.x % BLOCK, lane = lt & 63, wave = lt >> 6;
     auto vec = [&](int v) { return (lt + v * BLOCK) * 4; };
     float w[VPT][4], dw[VPT][4], db[VPT][4];
 #pragma unroll
@@ -341,6 +341,10 @@ __global__ __launch_bounds__(256 * RG) void ln_bwd_rg_kernel(float* __restrict__
         lds_barrier();
         c1 = (red[h][0] + red[h][1]) + (red[h][2] + red[h][3]);
         c2 = (red[h][NW] + red[h][NW + 1]) + (red[h][NW + 2] + red[h][NW + 3]);
+        if constexpr (NW == 8) {
+            c1 += (red[h][4] + red[h][5]) + (red[h][6] + red[h][7]);
+            c2 += (red[h][NW + 4] + red[h][NW + 5]) + (red[h][NW + 6] + red[h][NW + 7]);
+        }
         lds_barrier();
         c1 /= (float)N;
         c2 /= (float)N;
@@ -382,7 +386,7 @@ __global__ __launch_bounds__(256 * RG) void ln_bwd_rg_kernel(float* __restrict__
             __syncthreads();
         }
         float* dst = pass == 0 ? dwp : dbp;
-        for (int c = threadIdx.x; c < N; c += 256 * RG) {
+        for (int c = threadIdx.x; c < N; c += BLOCK * RG) {
             if (S == 1) dst[c] += stage[c];
             else unsafeAtomicAdd(dst + c, stage[c]);
         }
@@ -610,19 +614,29 @@ extern "C" int mi_layer_norm_bwd_dx_partial_dwdb(
         (int)N, M, G, (int)S
     const bool stream_in = stream_hint(3 * M * N * (int64_t)sizeof(float));
     static const bool one_group = [] { const char* e = getenv("MI_LN_BWD_RG"); return e && e[0] == '1'; }();
-    if (al && N % 4 == 0 && vecs > 512 && vecs <= 1024 && S % 2 == 0 && !one_group) {
-        // two row groups per workgroup: same rows in flight, half the atomics (four groups measured no better)
-        const int S2 = (int)S / 2;
+    if (al && N % 4 == 0 && vecs <= 2048 && !one_group) {
+        // Row groups with two rows of look-ahead.  Up to 4096 elements a group is 256 lanes and two
+        // groups share a workgroup (same rows in flight, half the atomics; four groups measured no
+        // better); up to 8192 elements one group of 512 lanes.
+        const int rg = vecs <= 1024 ? 2 : 1;
+        const int S2 = (int)cld(S, (int64_t)rg);
         dim3 grid2((unsigned)(G * S2));
-#define RGK(ST)                                                                                               \
-    hipLaunchKernelGGL((ln_bwd_rg_kernel<4, ST, 2>), grid2, dim3(512), 0, s, (float*)DX->ptr, DX->strides[1],   \
+#define RGK(BL, VP, ST, R)                                                                                      \
+    hipLaunchKernelGGL((ln_bwd_rg_kernel<BL, VP, ST, R>), grid2, dim3(BL * R), 0, s, (float*)DX->ptr, DX->strides[1], \
                        (const float*)DY->ptr, DY->strides[1], (float*)DW->ptr, DW->strides[1], (float*)DB->ptr, \
                        DB->strides[1], (const float*)X->ptr, X->strides[1], (const float*)W->ptr,               \
                        (const float*)Mean->ptr, (const float*)Rstd->ptr, (int)N, M, G, S2)
-        if (stream_in) RGK(true);
-        else RGK(false);
+#define RGS(BL, VP, R)                 \
+    do {                               \
+        if (stream_in) RGK(BL, VP, true, R); \
+        else RGK(BL, VP, false, R);    \
+    } while (0)
+        if (vecs <= 256) { RGS(256, 1, 2); set_variant("ln_bwd_regs_b512_v1_rg2"); }
+        else if (vecs <= 512) { RGS(256, 2, 2); set_variant("ln_bwd_regs_b512_v2_rg2"); }
+        else if (vecs <= 1024) { RGS(256, 4, 2); set_variant("ln_bwd_regs_b512_v4_rg2"); }
+        else { RGS(512, 4, 1); set_variant("ln_bwd_regs_b512_v4_rg1"); }
+#undef RGS
 #undef RGK
-        set_variant("ln_bwd_regs_b512_v4_rg2");
     } else if (!al) launch_bwd<false, false>(ARGS);
     else if (stream_in) launch_bwd<true, true>(ARGS);
     else launch_bwd<true, false>(ARGS);

@@ -264,6 +264,7 @@ __global__ __launch_bounds__(BLOCK * RG) void ln_bwd_rg_kernel(float* __restrict
                                                          const float* __restrict__ Rstd, int N,
                                                          int64_t M, int G, int S) {
     constexpr int NW = BLOCK / 64;
+    static_assert(NW == 1 || NW == 4 || NW == 8, "the cross-wave sums are written out for 4 and 8 waves");
     __shared__ float red[RG][2 * NW];
     __shared__ float stage[BLOCK * VPT * 4];
     const int g = blockIdx.x % G, s = blockIdx.x / G;
@@ -334,18 +335,20 @@ __global__ __launch_bounds__(BLOCK * RG) void ln_bwd_rg_kernel(float* __restrict
         }
         c1 = wave_reduce(c1, SumOp{});
         c2 = wave_reduce(c2, SumOp{});
-        if (lane == 0) {
-            red[h][wave] = c1;
-            red[h][NW + wave] = c2;
+        if constexpr (NW > 1) {   // (a one-wave group is done after the shuffles)
+            if (lane == 0) {
+                red[h][wave] = c1;
+                red[h][NW + wave] = c2;
+            }
+            lds_barrier();
+            c1 = (red[h][0] + red[h][1]) + (red[h][2] + red[h][3]);
+            c2 = (red[h][NW] + red[h][NW + 1]) + (red[h][NW + 2] + red[h][NW + 3]);
+            if constexpr (NW == 8) {
+                c1 += (red[h][4] + red[h][5]) + (red[h][6] + red[h][7]);
+                c2 += (red[h][NW + 4] + red[h][NW + 5]) + (red[h][NW + 6] + red[h][NW + 7]);
+            }
+            lds_barrier();
         }
-        lds_barrier();
-        c1 = (red[h][0] + red[h][1]) + (red[h][2] + red[h][3]);
-        c2 = (red[h][NW] + red[h][NW + 1]) + (red[h][NW + 2] + red[h][NW + 3]);
-        if constexpr (NW == 8) {
-            c1 += (red[h][4] + red[h][5]) + (red[h][6] + red[h][7]);
-            c2 += (red[h][NW + 4] + red[h][NW + 5]) + (red[h][NW + 6] + red[h][NW + 7]);
-        }
-        lds_barrier();
         c1 /= (float)N;
         c2 /= (float)N;
 #pragma unroll
@@ -484,7 +487,7 @@ void launch_fwd(int vecs, dim3 grid, hipStream_t s, const float* X, int64_t ldx,
                        Mean, Rstd, eps, N, M)
     if (vecs <= 64) { FWD(64, 1); set_variant("ln_fwd_regs_b64_v1"); }
     else if (vecs <= 128) { FWD(64, 2); set_variant("ln_fwd_regs_b64_v2"); }
-    else if (vecs <= 256) { FWD(256, 1); set_variant("ln_fwd_regs_b256_v1"); }
+    else if (vecs <= 256) { FWD(64, 4); set_variant("ln_fwd_regs_b64_v4"); }   // one wave per row: no barriers (5.4 -> 6.3 TB/s at N = 1024)
     else if (vecs <= 512) { FWD(256, 2); set_variant("ln_fwd_regs_b256_v2"); }
     else if (vecs <= 1024) { FWD(256, 4); set_variant("ln_fwd_regs_b256_v4"); }
     else if (vecs <= 2048) { FWD(256, 8); set_variant("ln_fwd_regs_b256_v8"); }
@@ -618,7 +621,15 @@ extern "C" int mi_layer_norm_bwd_dx_partial_dwdb(
         // Row groups with two rows of look-ahead.  Up to 4096 elements a group is 256 lanes and two
         // groups share a workgroup (same rows in flight, half the atomics; four groups measured no
         // better); up to 8192 elements one group of 512 lanes.
-        const int rg = vecs <= 1024 ? 2 : 1;
+        // Up to 512 elements a group is a single wave (no barriers in the walk) and eight groups
+        // share a workgroup; there the chip wants four times as many groups in flight, since a
+        // group's rows are that much shorter.
+        const int rg = vecs <= 128 ? 8 : vecs <= 1024 ? 2 : 1;
+        if (vecs <= 128 && !getenv("MI_LN_BWD_SPLITS")) {
+            S = cld((int64_t)2048, (int64_t)G);
+            if (S > cld(rows_per_slot, (int64_t)4)) S = cld(rows_per_slot, (int64_t)4);
+            if (S < 1) S = 1;
+        }
         const int S2 = (int)cld(S, (int64_t)rg);
         dim3 grid2((unsigned)(G * S2));
 #define RGK(BL, VP, ST, R)                                                                                      \
@@ -631,7 +642,9 @@ extern "C" int mi_layer_norm_bwd_dx_partial_dwdb(
         if (stream_in) RGK(BL, VP, true, R); \
         else RGK(BL, VP, false, R);    \
     } while (0)
-        if (vecs <= 256) { RGS(256, 1, 2); set_variant("ln_bwd_regs_b512_v1_rg2"); }
+        if (vecs <= 64) { RGS(64, 1, 8); set_variant("ln_bwd_regs_b512_v1_rg8"); }
+        else if (vecs <= 128) { RGS(64, 2, 8); set_variant("ln_bwd_regs_b512_v2_rg8"); }
+        else if (vecs <= 256) { RGS(256, 1, 2); set_variant("ln_bwd_regs_b512_v1_rg2"); }
         else if (vecs <= 512) { RGS(256, 2, 2); set_variant("ln_bwd_regs_b512_v2_rg2"); }
         else if (vecs <= 1024) { RGS(256, 4, 2); set_variant("ln_bwd_regs_b512_v4_rg2"); }
         else { RGS(512, 4, 1); set_variant("ln_bwd_regs_b512_v4_rg1"); }

@@ -218,7 +218,7 @@ int launch_len(const mi_tile_array* output, const mi_tile_array* input, int64_t 
     const int vecs = (int)cld(L, EV);
     if (vecs <= 64) { launch_regs<T, 64, 1>(output, input, L, al, s); set_variant("softmax_regs_b64_v1"); }
     else if (vecs <= 128) { launch_regs<T, 64, 2>(output, input, L, al, s); set_variant("softmax_regs_b64_v2"); }
-    else if (vecs <= 256) { launch_regs<T, 256, 1>(output, input, L, al, s); set_variant("softmax_regs_b256_v1"); }
+    else if (vecs <= 256) { launch_regs<T, 64, 4>(output, input, L, al, s); set_variant("softmax_regs_b64_v4"); }   // one wave per column: no barriers
     else if (vecs <= 512) { launch_regs<T, 256, 2>(output, input, L, al, s); set_variant("softmax_regs_b256_v2"); }
     else if (vecs <= 1024) { launch_regs<T, 256, 4>(output, input, L, al, s); set_variant("softmax_regs_b256_v4"); }
     else if (vecs <= 2048) { launch_regs<T, 256, 8>(output, input, L, al, s); set_variant("softmax_regs_b256_v8"); }

@@ -48,13 +48,17 @@ __device__ __forceinline__ void block_sum2(float& a, float& b, float* red) {
 }
 
 // Load / store the lane's VPT 4-element groups of one row.  Out-of-range elements load 0.
+// ALIGNED: 16-byte aligned rows of a multiple of 4 elements, so a group is wholly inside the row or
+// wholly outside and there is no element-wise tail (whose second code path would keep twice the
+// registers alive).
 template <int BLOCK, int VPT, bool ALIGNED, bool NT>
 __device__ __forceinline__ void load_row(const float* __restrict__ p, int N, float (&r)[VPT][4]) {
 #pragma unroll
     for (int v = 0; v < VPT; ++v) {
         const int e0 = (threadIdx.x + v * BLOCK) * 4;
-        if (ALIGNED && e0 + 4 <= N) {
-            f32x4 t = ld_global<NT>(reinterpret_cast<const f32x4*>(p + e0));
+        if constexpr (ALIGNED) {
+            f32x4 t = {0.f, 0.f, 0.f, 0.f};
+            if (e0 < N) t = ld_global<NT>(reinterpret_cast<const f32x4*>(p + e0));
 #pragma unroll
             for (int q = 0; q < 4; ++q) r[v][q] = t[q];
         } else {
@@ -68,11 +72,11 @@ __device__ __forceinline__ void store_row(float* __restrict__ p, int N, const fl
 #pragma unroll
     for (int v = 0; v < VPT; ++v) {
         const int e0 = (threadIdx.x + v * BLOCK) * 4;
-        if (ALIGNED && e0 + 4 <= N) {
+        if constexpr (ALIGNED) {
             f32x4 t;
 #pragma unroll
             for (int q = 0; q < 4; ++q) t[q] = r[v][q];
-            st_global<true>(t, reinterpret_cast<f32x4*>(p + e0));
+            if (e0 < N) st_global<true>(t, reinterpret_cast<f32x4*>(p + e0));
         } else {
 #pragma unroll
             for (int q = 0; q < 4; ++q)
@@ -490,8 +494,9 @@ void launch_fwd(int vecs, dim3 grid, hipStream_t s, const float* X, int64_t ldx,
     else if (vecs <= 256) { FWD(64, 4); set_variant("ln_fwd_regs_b64_v4"); }   // one wave per row: no barriers (5.4 -> 6.3 TB/s at N = 1024)
     else if (vecs <= 512) { FWD(256, 2); set_variant("ln_fwd_regs_b256_v2"); }
     else if (vecs <= 1024) { FWD(256, 4); set_variant("ln_fwd_regs_b256_v4"); }
-    else if (vecs <= 2048) { FWD(256, 8); set_variant("ln_fwd_regs_b256_v8"); }
-    else { FWD(256, 16); set_variant("ln_fwd_regs_b256_v16"); }
+    else if (vecs <= 2048) { FWD(512, 4); set_variant("ln_fwd_regs_b512_v4"); }      // longer rows: more lanes, not more
+    else { FWD(1024, 4); set_variant("ln_fwd_regs_b1024_v4"); }                       // registers per lane
+
 #undef FWD
 }
 
@@ -544,7 +549,7 @@ extern "C" int mi_layer_norm_fwd(const mi_tile_array* X, const mi_tile_array* W,
         set_variant("ln_fwd_3pass_b256");
         return launch_status();
     }
-    const bool al = rows_vec_ok(X) && rows_vec_ok(Y) && rows_vec_ok(W) && rows_vec_ok(B);
+    const bool al = N % 4 == 0 && rows_vec_ok(X) && rows_vec_ok(Y) && rows_vec_ok(W) && rows_vec_ok(B);
     const int vecs = (int)cld(N, 4);
 #define ARGS                                                                                      \
     vecs, grid, s, x, X->strides[1], (const float*)W->ptr, (const float*)B->ptr, y, Y->strides[1], \
@@ -607,7 +612,7 @@ extern "C" int mi_layer_norm_bwd_dx_partial_dwdb(
         const long v = atol(env);
         if (v >= 1 && v <= rows_per_slot) S = v;
     }
-    const bool al = rows_vec_ok(X) && rows_vec_ok(DX) && rows_vec_ok(DY) && rows_vec_ok(W);
+    const bool al = N % 4 == 0 && rows_vec_ok(X) && rows_vec_ok(DX) && rows_vec_ok(DY) && rows_vec_ok(W);
     const int vecs = (int)cld(N, 4);
     dim3 grid((unsigned)(G * S));
 #define ARGS                                                                                   \

@@ -630,8 +630,9 @@ extern "C" int mi_layer_norm_bwd_dx_partial_dwdb(
         // share a workgroup; there the chip wants four times as many groups in flight, since a
         // group's rows are that much shorter.
         const int rg = vecs <= 128 ? 8 : vecs <= 1024 ? 2 : 1;
-        if (vecs <= 128 && !getenv("MI_LN_BWD_SPLITS")) {
-            S = cld((int64_t)2048, (int64_t)G);
+        if ((vecs <= 128 || vecs > 1024) && !getenv("MI_LN_BWD_SPLITS")) {
+            // (and a 512-lane group fills a CU by itself: one workgroup per CU, half the flushes)
+            S = cld((int64_t)(vecs <= 128 ? 2048 : 256), (int64_t)G);
             if (S > cld(rows_per_slot, (int64_t)4)) S = cld(rows_per_slot, (int64_t)4);
             if (S < 1) S = 1;
         }

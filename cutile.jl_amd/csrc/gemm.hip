@@ -14,6 +14,9 @@
 //   gemm16_generic   f16/bf16, 64x64x32 workgroup tile, any shape / stride / alignment
 //                    (ragged edges are zero-padded on load and clipped on store, as
 //                    ct.load(padding_mode=Zero) / ct.store do).
+//   gemm16_mid       f16/bf16, 128x128x32 workgroup tile with a register look-ahead of one K step, any
+//                    shape; used for larger problems that gemm16_big does not take (ragged or
+//                    unaligned: 4096 x 4096 x 4000 runs at 680 TFLOP/s against 460 with 64x64 tiles).
 //   gemm16_big       (gemm_big.hip) f16/bf16, 256x256 workgroup tile, 4 waves of 128x128,
 //                    K step 32 through a ring of four LDS stages filled by direct
 //                    global->LDS loads, XOR-swizzled LDS layouts; used when M,N are
@@ -94,6 +97,111 @@ __global__ __launch_bounds__(256) void gemm16_generic(
             const int64_t gn = n0 + wn + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
             if (gn < N) C[gm + gn * ldc] = cvt_out<E, OutT>(acc[r]);
         }
+    }
+}
+
+// ---- 128 x 128 16-bit kernel ----------------------------------------------------------------
+// Workgroup tile 128(m) x 128(n), K step 32, 4 waves as 2x2 of 64x64 (four 32x32x16 MFMAs per 16
+// k, one LDS fragment read per MFMA).  The next K step's operands are requested into registers
+// before the current step's MFMAs and cross the workgroup barriers in flight (the barriers wait
+// for LDS accesses only).  Any shape: workgroups whose tile is interior and 16-byte aligned load
+// without predicates; the others zero-pad element by element.
+constexpr int MT = 128, MA_PITCH = MT + 8, MB_PITCH = GK + 8;
+
+__device__ __forceinline__ void lds_barrier() {
+    asm volatile("" ::: "memory");
+    __builtin_amdgcn_s_waitcnt(0xc07f);   // lgkmcnt(0); vmcnt and expcnt at their maxima
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+}
+
+template <typename E, typename OutT>
+__global__ __launch_bounds__(256) void gemm16_mid(
+    const unsigned short* __restrict__ A, int64_t lda, int64_t sa, const unsigned short* __restrict__ B,
+    int64_t ldb, int64_t sb, OutT* __restrict__ C, int64_t ldc, int64_t sc, int M, int N, int K,
+    int tiles_m, bool vecA, bool vecB) {
+    __shared__ __attribute__((aligned(16))) unsigned short As[GK * MA_PITCH];  // [k][m]
+    __shared__ __attribute__((aligned(16))) unsigned short Bs[MT * MB_PITCH];  // [n][k]
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int bm = blockIdx.x % tiles_m, bn = blockIdx.x / tiles_m;
+    const int64_t m0 = (int64_t)bm * MT, n0 = (int64_t)bn * MT;
+    A += (int64_t)blockIdx.z * sa;
+    B += (int64_t)blockIdx.z * sb;
+    C += (int64_t)blockIdx.z * sc;
+    const int wm = (wave & 1) * 64, wn = (wave >> 1) * 64;
+    const int ak = tid >> 4, am = (tid & 15) * 8;   // A tile: rows k = ak and ak + 16, 8 consecutive m
+    const int bnn = tid >> 2, bk = (tid & 3) * 8;   // B tile: columns n = bnn and bnn + 64, 8 consecutive k
+    const bool interior = vecA && vecB && m0 + MT <= M && n0 + MT <= N;   // same for the whole workgroup
+
+    f32x16 acc[2][2] = {};
+    s16x8 va[2], vb[2];
+    auto gload = [&](int k0) {
+        if (interior && k0 + GK <= K) {
+#pragma unroll
+            for (int h = 0; h < 2; ++h) {
+                va[h] = *reinterpret_cast<const s16x8*>(A + m0 + am + (int64_t)(k0 + ak + 16 * h) * lda);
+                vb[h] = *reinterpret_cast<const s16x8*>(B + k0 + bk + (n0 + bnn + 64 * h) * ldb);
+            }
+            return;
+        }
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+            va[h] = vb[h] = s16x8{0};
+            const int64_t gm = m0 + am;
+            const int gk = k0 + ak + 16 * h;
+            if (gk < K) {
+                const unsigned short* p = A + gm + (int64_t)gk * lda;
+                if (vecA && gm + 8 <= M) va[h] = *reinterpret_cast<const s16x8*>(p);
+                else
+#pragma unroll
+                    for (int q = 0; q < 8; ++q) va[h][q] = (gm + q < M) ? (short)p[q] : (short)0;
+            }
+            const int64_t gn = n0 + bnn + 64 * h;
+            const int gk2 = k0 + bk;
+            if (gn < N) {
+                const unsigned short* p = B + gk2 + gn * ldb;
+                if (vecB && gk2 + 8 <= K) vb[h] = *reinterpret_cast<const s16x8*>(p);
+                else
+#pragma unroll
+                    for (int q = 0; q < 8; ++q) vb[h][q] = (gk2 + q < K) ? (short)p[q] : (short)0;
+            }
+        }
+    };
+    gload(0);
+    for (int k0 = 0; k0 < K; k0 += GK) {
+        lds_barrier();  // previous iteration's fragment reads are done
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+            *reinterpret_cast<s16x8*>(&As[(ak + 16 * h) * MA_PITCH + am]) = va[h];
+            *reinterpret_cast<s16x8*>(&Bs[(bnn + 64 * h) * MB_PITCH + bk]) = vb[h];
+        }
+        lds_barrier();
+        if (k0 + GK < K) gload(k0 + GK);
+#pragma unroll
+        for (int ks = 0; ks < GK / 16; ++ks) {
+            s16x8 fn[2], fm[2];
+#pragma unroll
+            for (int i = 0; i < 2; ++i) {
+                fn[i] = *reinterpret_cast<const s16x8*>(&Bs[(wn + 32 * i + (lane & 31)) * MB_PITCH + ks * 16 + 8 * (lane >> 5)]);
+                fm[i] = lds_read_tr_k16(&As[(ks * 16) * MA_PITCH + wm + 32 * i], MA_PITCH, lane);
+            }
+#pragma unroll
+            for (int i = 0; i < 2; ++i)
+#pragma unroll
+                for (int j = 0; j < 2; ++j) acc[i][j] = E::mfma32(fn[j], fm[i], acc[i][j]);
+        }
+    }
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+        const int64_t gm = m0 + wm + 32 * i + (lane & 31);
+        if (gm >= M) continue;
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const int64_t gn = n0 + wn + 32 * j + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
+                if (gn < N) C[gm + gn * ldc] = cvt_out<E, OutT>(acc[i][j][r]);
+            }
     }
 }
 
@@ -222,6 +330,16 @@ int validate(const mi_tile_array* A, const mi_tile_array* B, const mi_tile_array
 }
 
 template <typename E, typename OutT>
+void launch_mid16(const Problem& p, hipStream_t s) {
+    const int tiles_m = (int)cld((int64_t)p.M, (int64_t)MT), tiles_n = (int)cld((int64_t)p.N, (int64_t)MT);
+    const bool vecA = aligned(p.A, 16) && p.lda % 8 == 0 && p.sa % 8 == 0;
+    const bool vecB = aligned(p.B, 16) && p.ldb % 8 == 0 && p.sb % 8 == 0;
+    hipLaunchKernelGGL((gemm16_mid<E, OutT>), dim3((unsigned)(tiles_m * tiles_n), 1, (unsigned)p.batch), dim3(256), 0,
+                       s, (const unsigned short*)p.A, p.lda, p.sa, (const unsigned short*)p.B, p.ldb, p.sb,
+                       (OutT*)p.C, p.ldc, p.sc, p.M, p.N, p.K, tiles_m, vecA, vecB);
+}
+
+template <typename E, typename OutT>
 void launch_generic16(const Problem& p, hipStream_t s) {
     const int tiles_m = (int)cld((int64_t)p.M, (int64_t)GT), tiles_n = (int)cld((int64_t)p.N, (int64_t)GT);
     const bool vecA = aligned(p.A, 16) && p.lda % 8 == 0 && p.sa % 8 == 0;
@@ -244,8 +362,24 @@ int run(const Problem& p, hipStream_t s) {
         return launch_status();
     }
     const bool f32out = p.out_dtype == MI_F32;
-    if (big16_applicable(p)) {
+    static const int force = [] { const char* e = getenv("MI_GEMM_KERNEL"); return e ? atoi(e) : 0; }();   // 1 generic, 2 mid, 3 big
+    const int64_t tiles_mid = (int64_t)cld((int64_t)p.M, (int64_t)MT) * cld((int64_t)p.N, (int64_t)MT) * p.batch;
+    // The 256x256 kernel wherever it applies (aligned shapes: even with a quarter of the CUs busy it
+    // matches the 128x128 kernel); the 128x128 kernel for other shapes whose tiles give at least half
+    // the CUs work; the 64x64 kernel for what is left (small problems).
+    if (big16_applicable(p) && (force == 3 || force == 0)) {
         big16_launch(p, s);
+        return launch_status();
+    }
+    if (force == 2 || (force == 0 && tiles_mid >= 128)) {
+        if (p.in_dtype == MI_F16) {
+            if (f32out) launch_mid16<F16, float>(p, s);
+            else launch_mid16<F16, unsigned short>(p, s);
+        } else {
+            if (f32out) launch_mid16<BF16, float>(p, s);
+            else launch_mid16<BF16, unsigned short>(p, s);
+        }
+        set_variant("gemm16_mid_128x128x32");
         return launch_status();
     }
     if (p.in_dtype == MI_F16) {

@@ -63,6 +63,22 @@ def test_matmul_integer_valued_inputs_are_exact(ct, orc):
         assert np.array_equal(orc.to_julia(C), A @ B)
 
 
+@pytest.mark.parametrize("M,N,K,T,out32", [(1504, 1544, 200, torch.float16, True), (1500, 1540, 333, torch.float16, False),
+                                           (2048, 1100, 96, torch.bfloat16, True), (1536, 1536, 32, torch.float16, True)])
+def test_matmul_mid_tile_kernel_exact(ct, orc, M, N, K, T, out32):
+    """The 128x128 kernel (shapes the 256x256 kernel does not take, enough tiles to fill half the chip):
+    aligned interior tiles without predicates, ragged edges in M, N and K, rows that are not 16-byte
+    aligned (M = 1500), one and many K steps.  Integer-valued operands make every sum exact, so any
+    mistake in the tile mapping, the register look-ahead or the fragment reads changes the result."""
+    rng = np.random.default_rng(M + K)
+    A = rng.integers(-3, 4, (M, K)).astype(np.float32); B = rng.integers(-3, 4, (K, N)).astype(np.float32)
+    At = orc.from_julia(A).to(T).cuda(); Bt = orc.from_julia(B).to(T).cuda()
+    C = torch.empty((N, M), dtype=torch.float32 if out32 else T, device="cuda")
+    ct.matmul_kernel(At, Bt, C, 128, 128, 32)
+    assert ct.last_variant() == "gemm16_mid_128x128x32"
+    assert np.array_equal(orc.to_julia(C.float()), A @ B)      # (random sums of 333 terms stay far below 2048: exact in f16 too)
+
+
 @pytest.mark.parametrize("M,N,K,T,out32", [(2048, 2048, 256, torch.float16, True), (2048, 2048, 384, torch.float16, False),
                                             (4096, 1024, 512, torch.bfloat16, True), (1024, 4096, 640, torch.bfloat16, False)])
 def test_matmul_large_tile_kernel_exact(ct, orc, M, N, K, T, out32):

@@ -116,13 +116,20 @@ __global__ __launch_bounds__(NT) void transpose4_kernel(const unsigned* __restri
         }
     }
     const int64_t m0 = (int64_t)bm * TM, n0 = (int64_t)bn * TN;
+    // A tile that lies wholly inside the matrix is moved without predicates: a predicated load has
+    // to be waited for before the other side of its branch may write the same registers, which
+    // would leave a lane with one load in flight instead of four.
+    const bool interior = m0 + TM <= m && n0 + TN <= n;
 #pragma unroll
     for (int k = 0; k < MB; ++k) {
         const int b = threadIdx.x + NT * k;
         const int i4 = b % (TM / 4), j4 = b / (TM / 4);
         const int64_t gm = m0 + 4 * i4, gn = n0 + 4 * j4;
         u32x4 r[4] = {};
-        if (gm < m) {
+        if (interior) {
+#pragma unroll
+            for (int c = 0; c < 4; ++c) r[c] = ld_global<STREAM>(reinterpret_cast<const u32x4*>(x + gm + (gn + c) * ldx));
+        } else if (gm < m) {
 #pragma unroll
             for (int c = 0; c < 4; ++c)
                 if (gn + c < n) r[c] = ld_global<STREAM>(reinterpret_cast<const u32x4*>(x + gm + (gn + c) * ldx));
@@ -140,7 +147,7 @@ __global__ __launch_bounds__(NT) void transpose4_kernel(const unsigned* __restri
         const int b = threadIdx.x + NT * k;
         const int j4 = b % SLOTS, row = b / SLOTS;
         const int64_t gn = n0 + 4 * j4, gm = m0 + row;
-        if (gn < n && gm < m) {
+        if (interior || (gn < n && gm < m)) {
             u32x4 t = *reinterpret_cast<const u32x4*>(&lds[row * TN + 4 * (j4 ^ ((row >> 2) & (SLOTS - 1)))]);
             st_global<true>(t, reinterpret_cast<u32x4*>(y + gn + gm * ldy));
         }

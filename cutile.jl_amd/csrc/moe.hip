@@ -178,7 +178,27 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4))) void f
             if (col < num_a_cols) a_col[i] = col;
         }
     }
+    // Workgroups whose whole tile is inside the arrays (the usual case) load without predicates: a
+    // predicated load is waited for before the other side of its branch may write the same
+    // registers, which would leave a lane with one load in flight at a time.  Slots without a token
+    // read column 0 there; their accumulator rows are never stored.
+    const bool fast = vecA && vecB && K % kKT == 0 && (SILU ? n0 + kNT / 2 <= half_n : n0 + kNT <= N);
     auto load_tiles = [&](int k0, u32x4* breg, s16x8* areg) {
+        if (fast) {
+#pragma unroll
+            for (int i = 0; i < NB; ++i) {
+                const int id = tid + 256 * i, n = id / CPRB, c = id % CPRB;
+                const int64_t off = k0 + EPB * c + (int64_t)row_of(n) * ldb;
+                breg[i] = W8 ? __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(B8 + off))
+                             : __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(B16 + off));
+            }
+#pragma unroll
+            for (int i = 0; i < NA; ++i) {
+                const int gk = k0 + 8 * ((tid + 256 * i) % CPR);
+                areg[i] = *reinterpret_cast<const s16x8*>(A + gk + (int64_t)(a_col[i] < 0 ? 0 : a_col[i]) * lda);
+            }
+            return;
+        }
 #pragma unroll
         for (int i = 0; i < NB; ++i) {
             const int id = tid + 256 * i, n = id / CPRB, c = id % CPRB;

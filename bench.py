@@ -338,6 +338,24 @@ def bench_kernels(ct, which, cpu, nruns=NRUNS, warmup=WARMUP):
         except Exception as ex:
             res["moe_f16_device_routed"] = extra(_entry(f"MoE f16 top-2 from router logits (eager; graph failed: {type(ex).__name__})",
                                                         routed, wbytes, "GB/s", "hbm", HBM_PEAK_GBS, "f16", nruns, warmup))
+        # the reference example's own routing (moe.jl:311-344: top-8 of 32 experts, 64 tokens per expert on average)
+        d8 = moe.prepare(benchmark=True, topk=8)
+        flop8 = moe.metric(d8)[0]
+        top8 = lambda: moe.cutile_moe(d8.hidden_states, d8.w1, d8.w2, d8.topk_weights, d8.topk_ids, 128, 128, 64,
+                                      device_align=True, fuse_silu=True)
+        top8()
+        try:
+            g8k, _ = graph_of(top8)
+            e8 = _entry("MoE f16 top-8 (the reference example's routing) on the device, fused SiLU epilogue, HIP graph replay",
+                        g8k.replay, wbytes, "GB/s", "hbm", HBM_PEAK_GBS, "f16", nruns, warmup)
+        except Exception as ex:
+            e8 = _entry(f"MoE f16 top-8 on the device (eager; graph failed: {type(ex).__name__})", top8, wbytes, "GB/s", "hbm",
+                        HBM_PEAK_GBS, "f16", nruns, warmup)
+        e8["flop"] = flop8
+        e8["tflops"] = round(flop8 / (e8["avg_ms"] * 1e-3) / 1e12, 2)
+        e8["mfma_frac"] = round(e8["tflops"] / 2500.0, 5)
+        res["moe_f16_top8_device_fused"] = e8
+        del d8
         if cpu:
             J = orc.to_julia
             args = (J(d.hidden_states), J(d.w1), J(d.w2), J(d.topk_weights), J(d.topk_ids))

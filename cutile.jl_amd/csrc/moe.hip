@@ -105,8 +105,11 @@ constexpr int kTT = 32;   // token slots per workgroup (one MFMA row tile)
 // the 64 up channels N/2 + [n0, n0 + 64) of the gate / up projection; the epilogue rounds both
 // products to the activation type exactly as the separate kernels would, applies SiLU(gate) * up
 // (moe.jl:110-128) and writes N/2 channels, so the intermediate never goes to memory.
-template <typename E, bool W8, int NTW, int kKT, bool SILU = false>
-__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4))) void fused_moe_kernel(
+// TS: 32-slot tiles of one expert block that a workgroup multiplies with the same weight tile
+// (wide shapes only).  With more than 32 tokens per expert TS = 2 streams an expert's weights once
+// per 64 tokens instead of once per 32, at the price of one workgroup per CU less.
+template <typename E, bool W8, int NTW, int kKT, bool SILU = false, int TS = 1>
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(TS == 1 ? 4 : 3))) void fused_moe_kernel(
     const unsigned short* __restrict__ A, int64_t lda, int num_a_cols, const void* __restrict__ Bv, int64_t ldb,
     int64_t sbe, unsigned short* __restrict__ C, int64_t ldc, int total_tokens,
     const unsigned short* __restrict__ topk_weights, const int* __restrict__ sorted_token_ids, int num_slots,
@@ -119,7 +122,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4))) void f
     constexpr int kBsBytes = (W8 ? 1 : 2) * kNT * kKT, kRedBytes = KW > 1 ? 4 * 64 * 16 * 4 : 0;
     __shared__ __attribute__((aligned(16))) unsigned char Bs_raw[kBsBytes > kRedBytes ? kBsBytes : kRedBytes];
     unsigned short* Bs = reinterpret_cast<unsigned short*>(Bs_raw);
-    __shared__ __attribute__((aligned(16))) unsigned short As[kTT * kKT];  // [slot][k], same swizzle
+    constexpr int kTTS = kTT * TS;   // token slots per workgroup
+    __shared__ __attribute__((aligned(16))) unsigned short As[kTTS * kKT];  // [slot][k], same swizzle
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, hb = lane >> 5;
     const int wn = wave % NTW, wk = wave / NTW;  // position along n / along the K split
@@ -130,39 +134,44 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4))) void f
     // order three quarters of every dispatch round would be padding tiles that leave at once, and
     // the weight streams would take several rounds to build up.
     const int t_lin = blockIdx.x / n_blocks, bid_n = blockIdx.x % n_blocks;
-    const int tpb = TILE_M / tile_slots, m_blocks = (gridDim.x / n_blocks) / tpb;
-    const int tile = (t_lin % m_blocks) * tpb + t_lin / m_blocks;
+    const int gpb = TILE_M / tile_slots / TS, m_blocks = (gridDim.x / n_blocks) / gpb;   // groups of TS tiles per block
+    const int grp = (t_lin % m_blocks) * gpb + t_lin / m_blocks;
     static_assert(!SILU || NTW == 4, "the fused SiLU epilogue pairs waves 0,1 (gate) with waves 2,3 (up)");
     const int half_n = N / 2;
     const int n0 = bid_n * (SILU ? kNT / 2 : kNT);
     // global weight row of tile row n
     auto row_of = [&](int n) { return SILU ? (n < 64 ? n0 + n : half_n + n0 + n - 64) : n0 + n; };
     auto row_ok = [&](int n) { return SILU ? (n0 + (n & 63) < half_n) : (n0 + n < N); };
-    const int slot0 = tile * tile_slots;            // tile_slots = min(TILE_M, 32) divides TILE_M
+    const int slot0 = grp * tile_slots * TS;        // tile_slots = min(TILE_M, 32) divides TILE_M (32 when TS > 1)
     const int expert = sorted_expert_ids[slot0 / TILE_M] - 1;
 
-    // The tile's 32 token ids live in registers, slot i in lanes i and i + 32 of every wave (LDS is
+    // A tile's 32 token ids live in registers, slot i in lanes i and i + 32 of every wave (LDS is
     // exactly the two operand tiles, which is what lets a fourth workgroup fit on a CU).
-    int my_tok;
-    {
-        const int i = lane & 31, sl = slot0 + i;
+    int my_tok[TS];
+    unsigned live = 0;   // tiles of the workgroup that hold a token; the same in every wave
+#pragma unroll
+    for (int ts = 0; ts < TS; ++ts) {
+        const int i = lane & 31, sl = slot0 + kTT * ts + i;
         int t = (i < tile_slots && sl < num_slots) ? sorted_token_ids[sl] : 0;  // 1-based; 0 / >total = no token
         if (t < 1 || t > total_tokens) t = 0;
-        my_tok = t;
+        my_tok[ts] = t;
+        if (__ballot(t != 0) != 0ull) live |= 1u << ts;
     }
-    auto tok_of = [&](int slot) { return __shfl(my_tok, slot, 64); };
-    if (__ballot(my_tok != 0) == 0ull || expert < 0 || expert >= num_experts) return;  // same in every wave
+    auto tok_of = [&](int ts, int slot) { return __shfl(my_tok[ts], slot, 64); };
+    if (!live || expert < 0 || expert >= num_experts) return;
 
     const unsigned char* B8 = (const unsigned char*)Bv + (int64_t)expert * sbe;
     const unsigned short* B16 = (const unsigned short*)Bv + (int64_t)expert * sbe;
 
-    f32x16 acc = f32x16{0};
+    f32x16 acc[TS];
+#pragma unroll
+    for (int ts = 0; ts < TS; ++ts) acc[ts] = f32x16{0};
     // staging registers for the next B tile (128 n x kKT k) and A tile (32 slots x kKT k)
     constexpr int CPR = kKT / 8;            // 16-byte chunks per LDS tile row
     constexpr int EPB = W8 ? 16 : 8;        // weight elements per 16-byte global chunk
     constexpr int CPRB = kKT / EPB;         // 16-byte global chunks per weight row
     constexpr int NB = kNT * CPRB / 256;    // weight chunks per thread
-    constexpr int NA = kTT * CPR / 256;     // A chunks per thread
+    constexpr int NA = kTTS * CPR / 256;    // A chunks per thread
     // Two staging sets for the e4m3 path (its raw tiles are half the size, so two tiles per
     // workgroup can be in flight at the register cost of one f16 tile); one set otherwise.
     constexpr int DEPTH = W8 ? 2 : 1;
@@ -172,7 +181,12 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4))) void f
 #pragma unroll
     for (int i = 0; i < NA; ++i) {
         a_col[i] = -1;
-        const int tok = tok_of((tid + 256 * i) / CPR);
+        const int sl = (tid + 256 * i) / CPR;
+        int tok = tok_of(0, sl & 31);
+        if constexpr (TS == 2) {
+            const int tok1 = tok_of(1, sl & 31);
+            if (sl >= kTT) tok = tok1;
+        }
         if (tok) {
             const int col = (tok + replicas - 1) / replicas - 1;  // cld(token_id, replicas), 0-based
             if (col < num_a_cols) a_col[i] = col;
@@ -277,8 +291,12 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4))) void f
             } else {
                 bf = *reinterpret_cast<const s16x8*>(&Bs[n * kKT + 8 * (c ^ (n & 15))]);
             }
-            s16x8 af = *reinterpret_cast<const s16x8*>(&As[slot * kKT + 8 * (c ^ (slot & 15))]);
-            acc = E::mfma32(af, bf, acc);
+#pragma unroll
+            for (int ts = 0; ts < TS; ++ts) {
+                if (TS > 1 && !((live >> ts) & 1u)) continue;
+                s16x8 af = *reinterpret_cast<const s16x8*>(&As[(kTT * ts + slot) * kKT + 8 * (c ^ (slot & 15))]);
+                acc[ts] = E::mfma32(af, bf, acc[ts]);
+            }
         }
     };
     load_tiles(0, breg0, areg0);
@@ -291,68 +309,80 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4))) void f
     } else {
         for (int k0 = 0; k0 < K; k0 += kKT) step(k0, breg0, areg0);
     }
-    if (KW > 1) {  // add the K-split partial accumulators: wave (wn, wk) -> wave (wn, 0)
-        __syncthreads();
+    if (KW > 1) {  // add the K-split partial accumulators: wave (wn, wk) -> wave (wn, 0), one slot tile at a time
         float* red = reinterpret_cast<float*>(Bs_raw);  // 4 waves x 64 lanes x 16 floats = 16 KB <= sizeof(Bs_raw)
-        if (wk > 0) {
 #pragma unroll
-            for (int r = 0; r < 16; ++r) red[(wave * 16 + r) * 64 + lane] = acc[r];
+        for (int ts = 0; ts < TS; ++ts) {
+            if (!((live >> ts) & 1u)) continue;   // same decision in every wave
+            __syncthreads();                      // the operand tiles (or the previous exchange) are no longer read
+            if (wk > 0) {
+#pragma unroll
+                for (int r = 0; r < 16; ++r) red[(wave * 16 + r) * 64 + lane] = acc[ts][r];
+            }
+            __syncthreads();
+            if (wk == 0) {
+#pragma unroll
+                for (int q = 1; q < KW; ++q)
+#pragma unroll
+                    for (int r = 0; r < 16; ++r) acc[ts][r] += red[((wn + NTW * q) * 16 + r) * 64 + lane];
+            }
         }
-        __syncthreads();
         if (wk > 0) return;
-#pragma unroll
-        for (int q = 1; q < KW; ++q)
-#pragma unroll
-            for (int r = 0; r < 16; ++r) acc[r] += red[((wn + NTW * q) * 16 + r) * 64 + lane];
     }
 
     // epilogue: rows = token slots 8*(r/4) + 4*hb + r%4, column = channel n0 + wn*32 + lane%32
-    int toks[16];   // gathered while every lane of the wave is still active
 #pragma unroll
-    for (int r = 0; r < 16; ++r) toks[r] = tok_of(8 * (r >> 2) + 4 * hb + (r & 3));
-    if constexpr (SILU) {
-        const int nt = wn * 32 + (lane & 31);               // tile row of this lane's channel
-        const bool ok = row_ok(nt);
-        float ch_scale = 1.f;
-        if (W8 && ok) ch_scale = b_scale[row_of(nt) + (int64_t)expert * ld_scale];
-        // both halves rounded to the activation type, as the unfused GEMM stores them
+    for (int ts = 0; ts < TS; ++ts) {
+        if (!((live >> ts) & 1u)) continue;   // same decision in every wave
+        int toks[16];   // gathered with every lane of the wave active
 #pragma unroll
-        for (int r = 0; r < 16; ++r) {
-            float v = acc[r];
-            if (W8) v *= ch_scale;
-            if (mul_routed_weight && toks[r]) v *= E::widen(topk_weights[toks[r] - 1]);
-            acc[r] = E::widen(E::cvt(v));
+        for (int r = 0; r < 16; ++r) toks[r] = tok_of(ts, 8 * (r >> 2) + 4 * hb + (r & 3));
+        if constexpr (SILU) {
+            const int nt = wn * 32 + (lane & 31);               // tile row of this lane's channel
+            const bool ok = row_ok(nt);
+            float ch_scale = 1.f;
+            if (W8 && ok) ch_scale = b_scale[row_of(nt) + (int64_t)expert * ld_scale];
+            // both halves rounded to the activation type, as the unfused GEMM stores them
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                float v = acc[ts][r];
+                if (W8) v *= ch_scale;
+                if (mul_routed_weight && toks[r]) v *= E::widen(topk_weights[toks[r] - 1]);
+                acc[ts][r] = E::widen(E::cvt(v));
+            }
+            __syncthreads();   // every wave is done with the operand tiles (and with the previous tile's exchange)
+            float* up = reinterpret_cast<float*>(Bs_raw);        // 2 waves x 16 x 64 floats = 8 KB
+            if (wn >= 2) {
+#pragma unroll
+                for (int r = 0; r < 16; ++r) up[((wn - 2) * 16 + r) * 64 + lane] = acc[ts][r];
+            }
+            __syncthreads();
+            if (wn < 2 && ok) {
+                const int gc = n0 + nt;                          // output channel, < N / 2
+#pragma unroll
+                for (int r = 0; r < 16; ++r) {
+                    const int tok = toks[r];
+                    if (!tok) continue;
+                    const float g = acc[ts][r], u = up[(wn * 16 + r) * 64 + lane];
+                    C[gc + (int64_t)(tok - 1) * ldc] = E::cvt(silu_mul(g, u));
+                }
+            }
+        } else {
+            const int gn = n0 + wn * 32 + (lane & 31);
+            if (gn < N) {
+                float ch_scale = 1.f;
+                if (W8) ch_scale = b_scale[gn + (int64_t)expert * ld_scale];
+#pragma unroll
+                for (int r = 0; r < 16; ++r) {
+                    const int tok = toks[r];
+                    if (!tok) continue;
+                    float v = acc[ts][r];
+                    if (W8) v *= ch_scale;
+                    if (mul_routed_weight) v *= E::widen(topk_weights[tok - 1]);
+                    C[gn + (int64_t)(tok - 1) * ldc] = E::cvt(v);
+                }
+            }
         }
-        __syncthreads();                                     // every wave is done with the operand tiles
-        float* up = reinterpret_cast<float*>(Bs_raw);        // 2 waves x 16 x 64 floats = 8 KB
-        if (wn >= 2) {
-#pragma unroll
-            for (int r = 0; r < 16; ++r) up[((wn - 2) * 16 + r) * 64 + lane] = acc[r];
-        }
-        __syncthreads();
-        if (wn >= 2 || !ok) return;
-        const int gc = n0 + nt;                              // output channel, < N / 2
-#pragma unroll
-        for (int r = 0; r < 16; ++r) {
-            const int tok = toks[r];
-            if (!tok) continue;
-            const float g = acc[r], u = up[(wn * 16 + r) * 64 + lane];
-            C[gc + (int64_t)(tok - 1) * ldc] = E::cvt(silu_mul(g, u));
-        }
-        return;
-    }
-    const int gn = n0 + wn * 32 + (lane & 31);
-    if (gn >= N) return;
-    float ch_scale = 1.f;
-    if (W8) ch_scale = b_scale[gn + (int64_t)expert * ld_scale];
-#pragma unroll
-    for (int r = 0; r < 16; ++r) {
-        const int tok = toks[r];
-        if (!tok) continue;
-        float v = acc[r];
-        if (W8) v *= ch_scale;
-        if (mul_routed_weight) v *= E::widen(topk_weights[tok - 1]);
-        C[gn + (int64_t)(tok - 1) * ldc] = E::cvt(v);
     }
 }
 
@@ -442,10 +472,13 @@ static int fused_moe_impl(const mi_tile_array* A, const mi_tile_array* B, const 
     // in-workgroup K split.
     const bool narrow = !silu && m_blocks * cld(N, (int64_t)128) < 768 && K >= 512;
     const int n_blocks = silu ? (int)cld(N / 2, (int64_t)64) : (int)cld(N, (int64_t)(narrow ? 32 : 128));
+    // Two slot tiles per workgroup where an expert has more than 32 tokens on average (wide shapes).
+    // (not the e4m3 K-split shape: its two staging sets leave no registers for a second tile)
+    const int ts = (tile_slots == kTT && (TILE_M / kTT) % 2 == 0 && total >= (int64_t)kTT * E && !(narrow && w8)) ? 2 : 1;
     if (tiles * n_blocks > 0x7fffffffLL) return MI_E_GRID;
     const bool vecA = aligned(A->ptr, 16) && A->strides[1] % 8 == 0;
     const bool vecB = aligned(B->ptr, 16) && B->strides[1] % (w8 ? 16 : 8) == 0 && B->strides[2] % (w8 ? 16 : 8) == 0;
-    dim3 grid((unsigned)(tiles * n_blocks));
+    dim3 grid((unsigned)(tiles / ts * n_blocks));
     hipStream_t s = (hipStream_t)stream;
 #define LAUNCH(ET, W8, NTW, KT, ...)                                                                                \
     hipLaunchKernelGGL((fused_moe_kernel<ET, W8, NTW, KT, ##__VA_ARGS__>), grid, dim3(256), 0, s, (const unsigned short*)A->ptr, \
@@ -454,11 +487,14 @@ static int fused_moe_impl(const mi_tile_array* A, const mi_tile_array* B, const 
                        (const int*)sorted_token_ids->ptr, (int)slots, (const int*)sorted_expert_ids->ptr,           \
                        w8 ? (const float*)b_scale->ptr : nullptr, w8 ? b_scale->strides[1] : 0, (int)K, (int)N,     \
                        (int)E, num_token_replicas, mul_routed_weight != 0, TILE_M, tile_slots, n_blocks, vecA, vecB)
-#define LAUNCH_SHAPE(ET, W8)                        \
-    do {                                            \
-        if (silu) LAUNCH(ET, W8, 4, 128, true);     \
-        else if (narrow) LAUNCH(ET, W8, 1, 256);    \
-        else LAUNCH(ET, W8, 4, 128);                \
+#define LAUNCH_SHAPE(ET, W8)                                  \
+    do {                                                      \
+        if (silu && ts == 2) LAUNCH(ET, W8, 4, 128, true, 2); \
+        else if (silu) LAUNCH(ET, W8, 4, 128, true);          \
+        else if (narrow && ts == 2 && !W8) LAUNCH(ET, false, 1, 256, false, 2); \
+        else if (narrow) LAUNCH(ET, W8, 1, 256);              \
+        else if (ts == 2) LAUNCH(ET, W8, 4, 128, false, 2);   \
+        else LAUNCH(ET, W8, 4, 128);                          \
     } while (0)
     if (A->dtype == MI_F16) {
         if (w8) LAUNCH_SHAPE(F16, true);
@@ -469,8 +505,11 @@ static int fused_moe_impl(const mi_tile_array* A, const mi_tile_array* B, const 
     }
 #undef LAUNCH_SHAPE
 #undef LAUNCH
-    if (silu) set_variant(w8 ? "fused_moe_silu_t32_n64x2_k128_w8a16" : "fused_moe_silu_t32_n64x2_k128");
+    if (silu && ts == 2) set_variant(w8 ? "fused_moe_silu_t64_n64x2_k128_w8a16" : "fused_moe_silu_t64_n64x2_k128");
+    else if (silu) set_variant(w8 ? "fused_moe_silu_t32_n64x2_k128_w8a16" : "fused_moe_silu_t32_n64x2_k128");
+    else if (narrow && ts == 2) set_variant(w8 ? "fused_moe_t64_n32_k256_ksplit4_w8a16" : "fused_moe_t64_n32_k256_ksplit4");
     else if (narrow) set_variant(w8 ? "fused_moe_t32_n32_k256_ksplit4_w8a16" : "fused_moe_t32_n32_k256_ksplit4");
+    else if (ts == 2) set_variant(w8 ? "fused_moe_t64_n128_k128_w8a16" : "fused_moe_t64_n128_k128");
     else set_variant(w8 ? "fused_moe_t32_n128_k128_w8a16" : "fused_moe_t32_n128_k128");
     return launch_status();
 }

@@ -256,6 +256,51 @@ def test_gemm_with_fused_silu_epilogue(ct, orc, shape):
     check(J(b), ref)
 
 
+def test_dense_routing_two_slot_tiles_per_workgroup(ct, orc):
+    """More than 32 tokens per expert on average (the reference's own benchmark routing: 256 tokens, top-8 of 32
+    experts, moe.jl:311-344): a workgroup then multiplies two 32-slot tiles with the same weight tile.  The wide,
+    the fused-SiLU and the K-split mainloops all have that variant; every element is accumulated in the same order
+    as with one tile per workgroup, so fused and separate paths still agree bit for bit, and the result is checked
+    against the float64 oracle.  Includes a small problem (K-split shape) with unequal expert loads."""
+    d = moe.prepare(benchmark=True, topk=8)
+    tok, exp = ct.moe_align_tile_size_device(d.topk_ids, 128, d.num_experts)
+    c1 = torch.zeros(d.num_tokens * 8, 2 * d.intermediate_size, dtype=torch.float16, device="cuda")
+    moe.invoke_fused_moe_kernel(d.hidden_states, d.w1, c1, d.topk_weights, tok, exp, mul_routed_weight=False,
+                                num_token_replicas=8, tile_m=128, tile_n=128, tile_k=64)
+    assert ct.last_variant() == "fused_moe_t64_n128_k128"
+    c2 = torch.zeros(d.num_tokens * 8, d.intermediate_size, dtype=torch.float16, device="cuda")
+    moe.invoke_fused_moe_kernel(d.hidden_states, d.w1, c2, d.topk_weights, tok, exp, mul_routed_weight=False,
+                                num_token_replicas=8, tile_m=128, tile_n=128, tile_k=64, fuse_silu=True)
+    assert ct.last_variant() == "fused_moe_silu_t64_n64x2_k128"
+    c3 = torch.zeros(d.num_tokens * 8, d.hidden_size, dtype=torch.float16, device="cuda")
+    moe.invoke_fused_moe_kernel(c2, d.w2, c3, d.topk_weights, tok, exp, mul_routed_weight=True,
+                                num_token_replicas=1, tile_m=128, tile_n=128, tile_k=64)
+    assert ct.last_variant() == "fused_moe_t64_n32_k256_ksplit4"
+    a = moe.cutile_moe(d.hidden_states, d.w1, d.w2, d.topk_weights, d.topk_ids, 128, 128, 64, device_align=True)
+    b = moe.cutile_moe(d.hidden_states, d.w1, d.w2, d.topk_weights, d.topk_ids, 128, 128, 64, device_align=True, fuse_silu=True)
+    h = moe.cutile_moe(d.hidden_states, d.w1, d.w2, d.topk_weights, d.topk_ids, 128, 128, 64)      # host sort: exact block count
+    assert torch.equal(a, b) and torch.equal(a, h)
+    J = orc.to_julia
+    ref = orc.ref_moe(J(d.hidden_states), J(d.w1), J(d.w2), J(d.topk_weights), J(d.topk_ids), dtype=np.float32)
+    check(J(a), ref.astype(np.float64))
+    q = moe.quantize_weights(d)
+    f = moe.cutile_moe(d.hidden_states, q.w1, q.w2, d.topk_weights, d.topk_ids, 128, 128, 64, w1_scale=q.w1_scale,
+                       w2_scale=q.w2_scale, device_align=True, fuse_silu=True)
+    g = moe.cutile_moe(d.hidden_states, q.w1, q.w2, d.topk_weights, d.topk_ids, 128, 128, 64, w1_scale=q.w1_scale,
+                       w2_scale=q.w2_scale, device_align=True)
+    assert torch.equal(f, g)
+    w1d = orc.e4m3fn_decode(J(q.w1.view(torch.uint8))) * J(q.w1_scale)[None]
+    w2d = orc.e4m3fn_decode(J(q.w2.view(torch.uint8))) * J(q.w2_scale)[None]
+    check(J(f), orc.ref_moe(J(d.hidden_states), w1d, w2d, J(d.topk_weights), J(d.topk_ids), dtype=np.float32).astype(np.float64))
+    # small and uneven: 3 experts, 70 tokens, top-2 (about 47 tokens per expert, some tiles half empty)
+    d = moe.prepare(num_tokens=70, hidden_size=256, num_experts=3, intermediate_size=192, topk=2)
+    a = moe.cutile_moe(d.hidden_states, d.w1, d.w2, d.topk_weights, d.topk_ids, 128, 128, 64, device_align=True)
+    b = moe.cutile_moe(d.hidden_states, d.w1, d.w2, d.topk_weights, d.topk_ids, 64, 128, 64, fuse_silu=True)
+    ref = orc.ref_moe(J(d.hidden_states), J(d.w1), J(d.w2), J(d.topk_weights), J(d.topk_ids), dtype=np.float64)
+    check(J(a), ref)
+    check(J(b), ref)
+
+
 def test_fused_silu_epilogue_bf16_and_fp8_weights():
     d = moe.prepare(num_tokens=40, hidden_size=256, num_experts=6, intermediate_size=192, topk=2, T=torch.bfloat16)
     a = moe.cutile_moe(d.hidden_states, d.w1, d.w2, d.topk_weights, d.topk_ids, 32, 128, 64)

@@ -470,11 +470,13 @@ static int fused_moe_impl(const mi_tile_array* A, const mi_tile_array* B, const 
     // Wide strips (128 channels) when they already give the chip >= ~3 workgroups per CU,
     // counting one started 32-slot tile per TILE_M block; otherwise 32-channel strips with an
     // in-workgroup K split.
-    const bool narrow = !silu && m_blocks * cld(N, (int64_t)128) < 768 && K >= 512;
+    // Dense routing (more than 32 tokens per expert on average): two slot tiles per workgroup, and
+    // wide strips throughout -- every block then has two or more tiles with tokens, which gives the
+    // wide shape its workgroups, and a weight strip is streamed once per 64 tokens.
+    const bool dense = tile_slots == kTT && (TILE_M / kTT) % 2 == 0 && total >= (int64_t)kTT * E;
+    const bool narrow = !silu && !dense && m_blocks * cld(N, (int64_t)128) < 768 && K >= 512;
     const int n_blocks = silu ? (int)cld(N / 2, (int64_t)64) : (int)cld(N, (int64_t)(narrow ? 32 : 128));
-    // Two slot tiles per workgroup where an expert has more than 32 tokens on average (wide shapes).
-    // (not the e4m3 K-split shape: its two staging sets leave no registers for a second tile)
-    const int ts = (tile_slots == kTT && (TILE_M / kTT) % 2 == 0 && total >= (int64_t)kTT * E && !(narrow && w8)) ? 2 : 1;
+    const int ts = dense ? 2 : 1;
     if (tiles * n_blocks > 0x7fffffffLL) return MI_E_GRID;
     const bool vecA = aligned(A->ptr, 16) && A->strides[1] % 8 == 0;
     const bool vecB = aligned(B->ptr, 16) && B->strides[1] % (w8 ? 16 : 8) == 0 && B->strides[2] % (w8 ? 16 : 8) == 0;
@@ -491,7 +493,6 @@ static int fused_moe_impl(const mi_tile_array* A, const mi_tile_array* B, const 
     do {                                                      \
         if (silu && ts == 2) LAUNCH(ET, W8, 4, 128, true, 2); \
         else if (silu) LAUNCH(ET, W8, 4, 128, true);          \
-        else if (narrow && ts == 2 && !W8) LAUNCH(ET, false, 1, 256, false, 2); \
         else if (narrow) LAUNCH(ET, W8, 1, 256);              \
         else if (ts == 2) LAUNCH(ET, W8, 4, 128, false, 2);   \
         else LAUNCH(ET, W8, 4, 128);                          \
@@ -507,7 +508,6 @@ static int fused_moe_impl(const mi_tile_array* A, const mi_tile_array* B, const 
 #undef LAUNCH
     if (silu && ts == 2) set_variant(w8 ? "fused_moe_silu_t64_n64x2_k128_w8a16" : "fused_moe_silu_t64_n64x2_k128");
     else if (silu) set_variant(w8 ? "fused_moe_silu_t32_n64x2_k128_w8a16" : "fused_moe_silu_t32_n64x2_k128");
-    else if (narrow && ts == 2) set_variant(w8 ? "fused_moe_t64_n32_k256_ksplit4_w8a16" : "fused_moe_t64_n32_k256_ksplit4");
     else if (narrow) set_variant(w8 ? "fused_moe_t32_n32_k256_ksplit4_w8a16" : "fused_moe_t32_n32_k256_ksplit4");
     else if (ts == 2) set_variant(w8 ? "fused_moe_t64_n128_k128_w8a16" : "fused_moe_t64_n128_k128");
     else set_variant(w8 ? "fused_moe_t32_n128_k128_w8a16" : "fused_moe_t32_n128_k128");

@@ -259,9 +259,9 @@ def test_gemm_with_fused_silu_epilogue(ct, orc, shape):
 def test_dense_routing_two_slot_tiles_per_workgroup(ct, orc):
     """More than 32 tokens per expert on average (the reference's own benchmark routing: 256 tokens, top-8 of 32
     experts, moe.jl:311-344): a workgroup then multiplies two 32-slot tiles with the same weight tile.  The wide,
-    the fused-SiLU and the K-split mainloops all have that variant; every element is accumulated in the same order
+    and the fused-SiLU mainloops have that variant (dense routing always takes wide strips); every element is accumulated in the same order
     as with one tile per workgroup, so fused and separate paths still agree bit for bit, and the result is checked
-    against the float64 oracle.  Includes a small problem (K-split shape) with unequal expert loads."""
+    against the float64 oracle.  Includes a small problem with unequal expert loads."""
     d = moe.prepare(benchmark=True, topk=8)
     tok, exp = ct.moe_align_tile_size_device(d.topk_ids, 128, d.num_experts)
     c1 = torch.zeros(d.num_tokens * 8, 2 * d.intermediate_size, dtype=torch.float16, device="cuda")
@@ -275,7 +275,7 @@ def test_dense_routing_two_slot_tiles_per_workgroup(ct, orc):
     c3 = torch.zeros(d.num_tokens * 8, d.hidden_size, dtype=torch.float16, device="cuda")
     moe.invoke_fused_moe_kernel(c2, d.w2, c3, d.topk_weights, tok, exp, mul_routed_weight=True,
                                 num_token_replicas=1, tile_m=128, tile_n=128, tile_k=64)
-    assert ct.last_variant() == "fused_moe_t64_n32_k256_ksplit4"
+    assert ct.last_variant() == "fused_moe_t64_n128_k128"
     a = moe.cutile_moe(d.hidden_states, d.w1, d.w2, d.topk_weights, d.topk_ids, 128, 128, 64, device_align=True)
     b = moe.cutile_moe(d.hidden_states, d.w1, d.w2, d.topk_weights, d.topk_ids, 128, 128, 64, device_align=True, fuse_silu=True)
     h = moe.cutile_moe(d.hidden_states, d.w1, d.w2, d.topk_weights, d.topk_ids, 128, 128, 64)      # host sort: exact block count

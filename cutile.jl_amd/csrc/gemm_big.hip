@@ -26,7 +26,8 @@
 // Workgroups are numbered so that the tiles resident on one XCD (ids congruent mod 8) form a
 // 4 x 8 block of tiles and share A row panels / B column panels in that XCD's L2.
 //
-// Requires M, N multiples of 256, K a multiple of 128 and >= 256, 16-byte aligned operands.
+// Requires M a multiple of 8, K a multiple of 128 and >= 256, 16-byte aligned operands.  Tiles that
+// reach past M or N re-read the last valid rows / chunks on the way in and clip their stores.
 #include "gemm_common.h"
 
 namespace {
@@ -47,7 +48,8 @@ __device__ __forceinline__ void gload_lds16(const void* g, void* lds_wave_base) 
 }
 
 struct Lane {
-    unsigned goffA, goffB;  // byte offset of this lane's 16-byte chunk within a wave-wide 1 KB transfer
+    unsigned goffA;         // byte offset of this lane's 16-byte chunk within a wave-wide 1 KB transfer of A
+    int64_t goffB[4];       // the same for the wave's four B transfers (rows past the matrix edge re-read the last row)
     unsigned fb[2];         // LDS element offset of the B fragment, k16 sub-step 0/1 (+ 32*j*BK for n tile j)
     unsigned fa[4];         // LDS element offset of the A fragment, m tile i (+ 16*ks*BT for sub-step ks)
 };
@@ -59,7 +61,7 @@ struct Frag {
 // B stage: 256 rows x 64 B = 16 transfers of 1 KB (16 rows each); wave w takes transfers w, w+4, w+8, w+12.
 __device__ __forceinline__ void issue_B(const char* Bg, int64_t ldb2, unsigned short* Bs, int wave, const Lane& ln) {
 #pragma unroll
-    for (int j = 0; j < 4; ++j) gload_lds16(Bg + (int64_t)(64 * j) * ldb2 + ln.goffB, Bs + (wave + 4 * j) * 512);
+    for (int j = 0; j < 4; ++j) gload_lds16(Bg + ln.goffB[j], Bs + (wave + 4 * j) * 512);
 }
 // A stage: 32 rows x 512 B = 16 transfers of 1 KB (2 rows each).
 __device__ __forceinline__ void issue_A(const char* Ag, int64_t lda2, unsigned short* As, int wave, const Lane& ln) {
@@ -137,8 +139,8 @@ __device__ __forceinline__ void k_step(const unsigned short* AsX, unsigned short
 template <typename E, typename OutT>
 __global__ __launch_bounds__(256) void gemm16_big(const unsigned short* __restrict__ A, int64_t lda, int64_t sa,
                                                   const unsigned short* __restrict__ B, int64_t ldb, int64_t sb,
-                                                  OutT* __restrict__ C, int64_t ldc, int64_t sc, int K, int tiles_m,
-                                                  int tiles_n) {
+                                                  OutT* __restrict__ C, int64_t ldc, int64_t sc, int M, int N, int K,
+                                                  int tiles_m, int tiles_n) {
     __shared__ __attribute__((aligned(1024))) unsigned short As0[STAGE], As1[STAGE], As2[STAGE], As3[STAGE];
     __shared__ __attribute__((aligned(1024))) unsigned short Bs0[STAGE], Bs1[STAGE], Bs2[STAGE], Bs3[STAGE];
     const int tid = threadIdx.x, lane = tid & 63;
@@ -156,11 +158,24 @@ __global__ __launch_bounds__(256) void gemm16_big(const unsigned short* __restri
     Lane ln;
     {
         const int hb = lane >> 5, g = lane >> 4, r = lane & 15;
-        // B transfer: lane -> row lane/4 of its 16-row block, LDS position lane%4; rows n = 16*blk + lane/4
-        ln.goffB = (unsigned)(((int64_t)(lane >> 2) * ldb + 8 * ((lane & 3) ^ ((lane >> 4) & 3))) * 2);
-        // A transfer: lane -> row lane/32 of its 2-row block, LDS position lane%32; rows k = 2*blk + lane/32
+        // B transfer: lane -> row lane/4 of its 16-row block, LDS position lane%4; rows n = 16*blk + lane/4.
+        // In a tile that reaches past N the rows beyond the edge re-read row N-1 (their products land in
+        // accumulators that are never stored), so every transfer stays inside the matrix.
+        {
+            const int first = bn * BT + 16 * wave;               // first row of the wave's transfer 0
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                int row = 64 * j + (lane >> 2);                  // relative to `first`
+                if (first + row > N - 1) row = N - 1 - first;    // (may be negative: still inside the tile's rows)
+                ln.goffB[j] = ((int64_t)row * ldb + 8 * ((lane & 3) ^ ((lane >> 4) & 3))) * 2;
+            }
+        }
+        // A transfer: lane -> row lane/32 of its 2-row block, LDS position lane%32; rows k = 2*blk + lane/32.
+        // Chunks of 8 m past the edge re-read the last whole chunk (M is a multiple of 8).
         const int ka = 2 * wave + (lane >> 5);
-        ln.goffA = (unsigned)(((int64_t)(lane >> 5) * lda + 8 * ((lane & 31) ^ (4 * (ka & 3)))) * 2);
+        int ca = (lane & 31) ^ (4 * (ka & 3));
+        if (bm * BT + 8 * ca + 8 > M) ca = (M - bm * BT) / 8 - 1;
+        ln.goffA = (unsigned)(((int64_t)(lane >> 5) * lda + 8 * ca) * 2);
 #pragma unroll
         for (int ks = 0; ks < 2; ++ks) {
             const int n = wn + (lane & 31);
@@ -221,23 +236,43 @@ __global__ __launch_bounds__(256) void gemm16_big(const unsigned short* __restri
     // 32-bit element offset; the part of n that is uniform across the wave goes into the base.
     const unsigned lane_off = (unsigned)((lane & 31) + (int64_t)(4 * (lane >> 5)) * ldc);
     OutT* Cw = C + (int64_t)bm * BT + wm + ((int64_t)bn * BT + wn) * ldc;
+    if ((bm + 1) * BT <= M && (bn + 1) * BT <= N) {   // interior tile (same for the whole workgroup)
 #pragma unroll
-    for (int i = 0; i < 4; ++i)
+        for (int i = 0; i < 4; ++i)
 #pragma unroll
-        for (int j = 0; j < 4; ++j)
+            for (int j = 0; j < 4; ++j)
 #pragma unroll
-            for (int r = 0; r < 16; ++r) {
-                OutT* cu = Cw + 32 * i + (int64_t)(32 * j + 8 * (r >> 2) + (r & 3)) * ldc;
-                __builtin_nontemporal_store(cvt_out<E, OutT>(acc[i][j][r]), cu + lane_off);
-            }
+                for (int r = 0; r < 16; ++r) {
+                    OutT* cu = Cw + 32 * i + (int64_t)(32 * j + 8 * (r >> 2) + (r & 3)) * ldc;
+                    __builtin_nontemporal_store(cvt_out<E, OutT>(acc[i][j][r]), cu + lane_off);
+                }
+    } else {                                          // edge tile: clip to the matrix
+        int m_left = M - (bm * BT + wm + (lane & 31)), n_left = N - (bn * BT + wn + 4 * (lane >> 5));
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) {
+                    // the empty statement keeps each test next to its store (256 hoisted lane masks would
+                    // not fit the scalar registers)
+                    asm volatile("" : "+v"(m_left), "+v"(n_left));
+                    const int dn = 32 * j + 8 * (r >> 2) + (r & 3);
+                    if (32 * i < m_left && dn < n_left) {
+                        float v = acc[i][j][r];
+                        asm volatile("" : "+v"(v));   // convert after the test, not 256 values ahead of it
+                        __builtin_nontemporal_store(cvt_out<E, OutT>(v), Cw + 32 * i + (int64_t)dn * ldc + lane_off);
+                    }
+                }
+    }
 }
 
 template <typename E, typename OutT>
 void launch(const Problem& p, hipStream_t s) {
-    const int tiles_m = p.M / BT, tiles_n = p.N / BT;
+    const int tiles_m = (p.M + BT - 1) / BT, tiles_n = (p.N + BT - 1) / BT;
     hipLaunchKernelGGL((gemm16_big<E, OutT>), dim3((unsigned)(tiles_m * tiles_n), 1, (unsigned)p.batch), dim3(256), 0,
                        s, (const unsigned short*)p.A, p.lda, p.sa, (const unsigned short*)p.B, p.ldb, p.sb,
-                       (OutT*)p.C, p.ldc, p.sc, p.K, tiles_m, tiles_n);
+                       (OutT*)p.C, p.ldc, p.sc, p.M, p.N, p.K, tiles_m, tiles_n);
 }
 
 }  // namespace
@@ -247,9 +282,11 @@ namespace gemm {
 
 bool big16_applicable(const Problem& p) {
     if (p.in_dtype != MI_F16 && p.in_dtype != MI_BF16) return false;
-    return p.M % BT == 0 && p.N % BT == 0 && p.K % 128 == 0 && p.K >= 256 && aligned(p.A, 16) && aligned(p.B, 16) &&
+    // M a multiple of 8 (A moves in 16-byte chunks along m), any N; ragged tiles re-read edge rows
+    const int64_t tiles = (int64_t)((p.M + BT - 1) / BT) * ((p.N + BT - 1) / BT) * p.batch;
+    return p.M % 8 == 0 && p.M >= 8 && p.N >= 1 && p.K % 128 == 0 && p.K >= 256 && aligned(p.A, 16) && aligned(p.B, 16) &&
            p.lda % 8 == 0 && p.ldb % 8 == 0 && p.sa % 8 == 0 && p.sb % 8 == 0 && p.ldc < (1 << 26) &&
-           p.lda < (1 << 26) && p.ldb < (1 << 26) && (int64_t)(p.M / BT) * (p.N / BT) * p.batch >= 64;
+           p.lda < (1 << 26) && p.ldb < (1 << 26) && tiles >= 64;
 }
 
 void big16_launch(const Problem& p, hipStream_t s) {

@@ -96,6 +96,24 @@ def test_matmul_large_tile_kernel_exact(ct, orc, M, N, K, T, out32):
     assert np.array_equal(orc.to_julia(C).astype(np.float32), ref)
 
 
+@pytest.mark.parametrize("M,N,K,T,out32", [(2040, 2000, 256, torch.float16, True), (2056, 2311, 384, torch.bfloat16, False),
+                                            (4000, 4001, 256, torch.float16, False), (8, 16385, 256, torch.float16, True)])
+def test_matmul_large_tile_kernel_ragged_edges(ct, orc, M, N, K, T, out32):
+    """M (a multiple of 8) and N off the 256 grid on the 256x256 kernel: edge tiles re-read the last
+    valid rows on the way in and clip their stores.  Exact integer sums; C is a view of a wider,
+    taller buffer filled with a sentinel, which must come back untouched (remainders of 8 rows of m
+    and of 7 / 1 columns of n included)."""
+    rng = np.random.default_rng(M ^ N)
+    A = rng.integers(-1, 2, (M, K)).astype(np.float32); B = rng.integers(-2, 3, (K, N)).astype(np.float32)
+    At = orc.from_julia(A).to(T).cuda(); Bt = orc.from_julia(B).to(T).cuda()
+    buf = torch.full((N + 3, M + 24), -77.0, dtype=torch.float32 if out32 else T, device="cuda")
+    C = buf[:N, :M]
+    ct.matmul_kernel(At, Bt, C, 64, 64, 64)
+    assert "big" in ct.last_variant()
+    assert np.array_equal(orc.to_julia(C.contiguous()).astype(np.float32), A @ B)
+    assert bool((buf[N:] == -77.0).all()) and bool((buf[:, M:] == -77.0).all())
+
+
 def test_batch_matmul_large_tile_kernel(ct, orc):
     rng = np.random.default_rng(8)
     M, K, N, Bn = 1024, 256, 1024, 4

@@ -26,8 +26,10 @@
 // Workgroups are numbered so that the tiles resident on one XCD (ids congruent mod 8) form a
 // 4 x 8 block of tiles and share A row panels / B column panels in that XCD's L2.
 //
-// Requires M a multiple of 8, K a multiple of 128 and >= 256, 16-byte aligned operands.  Tiles that
-// reach past M or N re-read the last valid rows / chunks on the way in and clip their stores.
+// Requires M and K multiples of 8, K >= 256, 16-byte aligned operands.  Tiles that reach past M or N
+// re-read the last valid rows / chunks on the way in and clip their stores.  K is walked in whole
+// groups of four steps (128); in the last group the 16-byte chunks at k >= K are fetched from a
+// 16-byte block of zeros instead (both operands, so padding never meets a non-finite value).
 #include "gemm_common.h"
 
 namespace {
@@ -47,7 +49,11 @@ __device__ __forceinline__ void gload_lds16(const void* g, void* lds_wave_base) 
                                      (__attribute__((address_space(3))) void*)lds_wave_base, 16, 0, 0);
 }
 
+// Source of every chunk that lies past K.
+__device__ __attribute__((aligned(16))) const unsigned zeros16[4] = {0u, 0u, 0u, 0u};
+
 struct Lane {
+    int kA, kB;             // first k, within a stage, of the lane's chunk in A transfer 0 (transfer j: + 8*j) / in a B transfer
     unsigned goffA;         // byte offset of this lane's 16-byte chunk within a wave-wide 1 KB transfer of A
     int64_t goffB[4];       // the same for the wave's four B transfers (rows past the matrix edge re-read the last row)
     unsigned fb[2];         // LDS element offset of the B fragment, k16 sub-step 0/1 (+ 32*j*BK for n tile j)
@@ -59,14 +65,27 @@ struct Frag {
 };
 
 // B stage: 256 rows x 64 B = 16 transfers of 1 KB (16 rows each); wave w takes transfers w, w+4, w+8, w+12.
-__device__ __forceinline__ void issue_B(const char* Bg, int64_t ldb2, unsigned short* Bs, int wave, const Lane& ln) {
+// TAIL: k_left = K - (first k of the stage); chunks at or past it come from the zero block.
+template <bool TAIL = false>
+__device__ __forceinline__ void issue_B(const char* Bg, int64_t ldb2, unsigned short* Bs, int wave, const Lane& ln,
+                                        int k_left = 0) {
 #pragma unroll
-    for (int j = 0; j < 4; ++j) gload_lds16(Bg + ln.goffB[j], Bs + (wave + 4 * j) * 512);
+    for (int j = 0; j < 4; ++j) {
+        const char* g = Bg + ln.goffB[j];
+        if (TAIL && ln.kB >= k_left) g = (const char*)zeros16;
+        gload_lds16(g, Bs + (wave + 4 * j) * 512);
+    }
 }
 // A stage: 32 rows x 512 B = 16 transfers of 1 KB (2 rows each).
-__device__ __forceinline__ void issue_A(const char* Ag, int64_t lda2, unsigned short* As, int wave, const Lane& ln) {
+template <bool TAIL = false>
+__device__ __forceinline__ void issue_A(const char* Ag, int64_t lda2, unsigned short* As, int wave, const Lane& ln,
+                                        int k_left = 0) {
 #pragma unroll
-    for (int j = 0; j < 4; ++j) gload_lds16(Ag + (int64_t)(8 * j) * lda2 + ln.goffA, As + (wave + 4 * j) * 512);
+    for (int j = 0; j < 4; ++j) {
+        const char* g = Ag + (int64_t)(8 * j) * lda2 + ln.goffA;
+        if (TAIL && ln.kA + 8 * j >= k_left) g = (const char*)zeros16;
+        gload_lds16(g, As + (wave + 4 * j) * 512);
+    }
 }
 
 __device__ __forceinline__ void load_frags(const unsigned short* As, const unsigned short* Bs, const Lane& ln, int ks,
@@ -120,17 +139,18 @@ __device__ __forceinline__ void stage_barrier() {
 //   first half : MFMAs of sub-step 0 | read sub-step 1 fragments | issue A transfers (into stage AsA)
 //   barrier
 //   second half: MFMAs of sub-step 1 | read next stage's sub-step 0 fragments | issue B transfers (into BsX)
-template <typename E, bool DMA_A, bool DMA_B, int VMCNT, bool LAST>
+// TAIL: the stages requested here may reach past K; k_left3 = K - (first k of step s+3).
+template <typename E, bool DMA_A, bool DMA_B, int VMCNT, bool LAST, bool TAIL>
 __device__ __forceinline__ void k_step(const unsigned short* AsX, unsigned short* BsX, const unsigned short* AsY,
                                        const unsigned short* BsY, unsigned short* AsA, const char* Ag_next3,
                                        const char* Bg_next4, int64_t lda2, int64_t ldb2, int wave, const Lane& ln,
-                                       Frag& f0, Frag& f1, f32x16 (&acc)[4][4]) {
-    if (DMA_A) issue_A(Ag_next3, lda2, AsA, wave, ln);
+                                       Frag& f0, Frag& f1, f32x16 (&acc)[4][4], int k_left3) {
+    if (DMA_A) issue_A<TAIL>(Ag_next3, lda2, AsA, wave, ln, k_left3);
     load_frags(AsX, BsX, ln, 1, f1);
     mma16<E>(f0, acc);
     interleave16<DMA_A, true>();
     if (!LAST) stage_barrier<VMCNT>();
-    if (DMA_B) issue_B(Bg_next4, ldb2, BsX, wave, ln);
+    if (DMA_B) issue_B<TAIL>(Bg_next4, ldb2, BsX, wave, ln, k_left3 - BK);
     if (!LAST) load_frags(AsY, BsY, ln, 0, f0);
     mma16<E>(f1, acc);
     interleave16<DMA_B, !LAST>();
@@ -173,6 +193,8 @@ __global__ __launch_bounds__(256) void gemm16_big(const unsigned short* __restri
         // A transfer: lane -> row lane/32 of its 2-row block, LDS position lane%32; rows k = 2*blk + lane/32.
         // Chunks of 8 m past the edge re-read the last whole chunk (M is a multiple of 8).
         const int ka = 2 * wave + (lane >> 5);
+        ln.kA = ka;
+        ln.kB = 8 * ((lane & 3) ^ ((lane >> 4) & 3));
         int ca = (lane & 31) ^ (4 * (ka & 3));
         if (bm * BT + 8 * ca + 8 > M) ca = (M - bm * BT) / 8 - 1;
         ln.goffA = (unsigned)(((int64_t)(lane >> 5) * lda + 8 * ca) * 2);
@@ -202,7 +224,7 @@ __global__ __launch_bounds__(256) void gemm16_big(const unsigned short* __restri
 #pragma unroll
         for (int j = 0; j < 4; ++j) acc[i][j] = f32x16{0};
 
-    const int KT = K / BK;  // multiple of 4, >= 8 (checked on the host)
+    const int KT = 4 * ((K + 4 * BK - 1) / (4 * BK));  // steps, in whole groups of four; >= 8 (K >= 256 is checked on the host)
     Frag f0, f1;
     // prologue: stages 0..2 and the B half of stage 3 (28 transfers per wave)
     issue_B(Bb, ldb2, Bs0, wave, ln);
@@ -215,21 +237,28 @@ __global__ __launch_bounds__(256) void gemm16_big(const unsigned short* __restri
     stage_barrier<20>();
     load_frags(As0, Bs0, ln, 0, f0);
 
-#define KSTEP(X, Y, AA, DA, DB, VM, LAST, s)                                                                      \
-    k_step<E, DA, DB, VM, LAST>(As##X, Bs##X, As##Y, Bs##Y, As##AA, Ab + (int64_t)((s) + 3) * a_step,            \
-                                Bb + (int64_t)((s) + 4) * b_step, lda2, ldb2, wave, ln, f0, f1, acc)
+#define KSTEP(X, Y, AA, DA, DB, VM, LAST, TAIL, s)                                                                \
+    k_step<E, DA, DB, VM, LAST, TAIL>(As##X, Bs##X, As##Y, Bs##Y, As##AA, Ab + (int64_t)((s) + 3) * a_step,      \
+                                      Bb + (int64_t)((s) + 4) * b_step, lda2, ldb2, wave, ln, f0, f1, acc,       \
+                                      K - ((s) + 3) * BK)
     int s = 0;
-    for (; s + 8 <= KT; s += 4) {
-        KSTEP(0, 1, 3, true, true, 16, false, s);
-        KSTEP(1, 2, 0, true, true, 16, false, s + 1);
-        KSTEP(2, 3, 1, true, true, 16, false, s + 2);
-        KSTEP(3, 0, 2, true, true, 16, false, s + 3);
+    for (; s + 12 <= KT; s += 4) {
+        KSTEP(0, 1, 3, true, true, 16, false, false, s);
+        KSTEP(1, 2, 0, true, true, 16, false, false, s + 1);
+        KSTEP(2, 3, 1, true, true, 16, false, false, s + 2);
+        KSTEP(3, 0, 2, true, true, 16, false, false, s + 3);
     }
+    // the group that requests the last four stages (the only ones that can reach past K)
+    KSTEP(0, 1, 3, true, true, 16, false, true, s);
+    KSTEP(1, 2, 0, true, true, 16, false, true, s + 1);
+    KSTEP(2, 3, 1, true, true, 16, false, true, s + 2);
+    KSTEP(3, 0, 2, true, true, 16, false, true, s + 3);
+    s += 4;
     // last four steps: only the A half of the final stage is still to be requested
-    KSTEP(0, 1, 3, true, false, 16, false, s);
-    KSTEP(1, 2, 0, false, false, 8, false, s + 1);
-    KSTEP(2, 3, 1, false, false, 0, false, s + 2);
-    KSTEP(3, 0, 2, false, false, 0, true, s + 3);
+    KSTEP(0, 1, 3, true, false, 16, false, true, s);
+    KSTEP(1, 2, 0, false, false, 8, false, false, s + 1);
+    KSTEP(2, 3, 1, false, false, 0, false, false, s + 2);
+    KSTEP(3, 0, 2, false, false, 0, true, false, s + 3);
 #undef KSTEP
 
     // Epilogue.  The lane's own offset (m within the wave tile, plus its 4*hb rows of n) is a
@@ -282,9 +311,9 @@ namespace gemm {
 
 bool big16_applicable(const Problem& p) {
     if (p.in_dtype != MI_F16 && p.in_dtype != MI_BF16) return false;
-    // M a multiple of 8 (A moves in 16-byte chunks along m), any N; ragged tiles re-read edge rows
+    // M and K multiples of 8 (A and B move in 16-byte chunks along m and k), any N
     const int64_t tiles = (int64_t)((p.M + BT - 1) / BT) * ((p.N + BT - 1) / BT) * p.batch;
-    return p.M % 8 == 0 && p.M >= 8 && p.N >= 1 && p.K % 128 == 0 && p.K >= 256 && aligned(p.A, 16) && aligned(p.B, 16) &&
+    return p.M % 8 == 0 && p.M >= 8 && p.N >= 1 && p.K % 8 == 0 && p.K >= 256 && aligned(p.A, 16) && aligned(p.B, 16) &&
            p.lda % 8 == 0 && p.ldb % 8 == 0 && p.sa % 8 == 0 && p.sb % 8 == 0 && p.ldc < (1 << 26) &&
            p.lda < (1 << 26) && p.ldb < (1 << 26) && tiles >= 64;
 }

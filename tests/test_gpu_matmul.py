@@ -97,15 +97,22 @@ def test_matmul_large_tile_kernel_exact(ct, orc, M, N, K, T, out32):
 
 
 @pytest.mark.parametrize("M,N,K,T,out32", [(2040, 2000, 256, torch.float16, True), (2056, 2311, 384, torch.bfloat16, False),
-                                            (4000, 4001, 256, torch.float16, False), (8, 16385, 256, torch.float16, True)])
+                                            (4000, 4001, 256, torch.float16, False), (8, 16385, 256, torch.float16, True),
+                                            (2048, 2048, 264, torch.float16, True), (2040, 2000, 1000, torch.float16, False),
+                                            (2048, 2304, 376, torch.bfloat16, True), (4096, 4096, 4000, torch.float16, True)])
 def test_matmul_large_tile_kernel_ragged_edges(ct, orc, M, N, K, T, out32):
     """M (a multiple of 8) and N off the 256 grid on the 256x256 kernel: edge tiles re-read the last
-    valid rows on the way in and clip their stores.  Exact integer sums; C is a view of a wider,
-    taller buffer filled with a sentinel, which must come back untouched (remainders of 8 rows of m
-    and of 7 / 1 columns of n included)."""
+    valid rows on the way in and clip their stores.  K (a multiple of 8) off the 128 grid: the last
+    group of four steps takes zeros for k >= K (remainders of 8, 104, 120 and 32 here; A and B are
+    views of buffers whose cells past K hold NaN, which must not reach the result).  Exact integer
+    sums; C is a view of a wider, taller buffer filled with a sentinel, which must come back
+    untouched (remainders of 8 rows of m and of 7 / 1 columns of n included)."""
     rng = np.random.default_rng(M ^ N)
     A = rng.integers(-1, 2, (M, K)).astype(np.float32); B = rng.integers(-2, 3, (K, N)).astype(np.float32)
-    At = orc.from_julia(A).to(T).cuda(); Bt = orc.from_julia(B).to(T).cuda()
+    # A is (M, K) column-major = torch (K, M): rows past K hold NaN; B is (K, N) = torch (N, K): columns past K hold NaN
+    Abuf = torch.full((K + 128, M), float("nan"), dtype=T, device="cuda"); Bbuf = torch.full((N, K + 128), float("nan"), dtype=T, device="cuda")
+    Abuf[:K] = orc.from_julia(A).to(T).cuda(); Bbuf[:, :K] = orc.from_julia(B).to(T).cuda()
+    At, Bt = Abuf[:K], Bbuf[:, :K]
     buf = torch.full((N + 3, M + 24), -77.0, dtype=torch.float32 if out32 else T, device="cuda")
     C = buf[:N, :M]
     ct.matmul_kernel(At, Bt, C, 64, 64, 64)

@@ -37,8 +37,11 @@ namespace {
 using namespace mi;
 using namespace mi::gemm;
 
+// The tile is BT m x (64*J) n: J = 4 is the 256x256 tile described above, J = 2 a 256x128 tile (waves of
+// 128x64, half the B stage, half the accumulators) for problems that would otherwise give too few
+// workgroups to the chip.
 constexpr int BT = 256, BK = 32;
-constexpr int STAGE = BT * BK;  // elements per A or B stage (16 KB)
+constexpr int STAGE = BT * BK;  // elements per A stage, and per B stage at J = 4 (16 KB)
 
 #define SG_MFMA 0x008
 #define SG_VMEM 0x010
@@ -61,16 +64,16 @@ struct Lane {
 };
 
 struct Frag {
-    s16x8 a[4], b[4];
+    s16x8 a[4], b[4];   // (b[j] for j < J)
 };
 
-// B stage: 256 rows x 64 B = 16 transfers of 1 KB (16 rows each); wave w takes transfers w, w+4, w+8, w+12.
+// B stage: 64*J rows x 64 B = 4*J transfers of 1 KB (16 rows each); wave w takes transfers w, w+4, ...
 // TAIL: k_left = K - (first k of the stage); chunks at or past it come from the zero block.
-template <bool TAIL = false>
+template <int J, bool TAIL = false>
 __device__ __forceinline__ void issue_B(const char* Bg, int64_t ldb2, unsigned short* Bs, int wave, const Lane& ln,
                                         int k_left = 0) {
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
+    for (int j = 0; j < J; ++j) {
         const char* g = Bg + ln.goffB[j];
         if (TAIL && ln.kB >= k_left) g = (const char*)zeros16;
         gload_lds16(g, Bs + (wave + 4 * j) * 512);
@@ -88,10 +91,11 @@ __device__ __forceinline__ void issue_A(const char* Ag, int64_t lda2, unsigned s
     }
 }
 
+template <int J>
 __device__ __forceinline__ void load_frags(const unsigned short* As, const unsigned short* Bs, const Lane& ln, int ks,
                                            Frag& f) {
 #pragma unroll
-    for (int j = 0; j < 4; ++j) f.b[j] = *reinterpret_cast<const s16x8*>(Bs + ln.fb[ks] + 32 * j * BK);
+    for (int j = 0; j < J; ++j) f.b[j] = *reinterpret_cast<const s16x8*>(Bs + ln.fb[ks] + 32 * j * BK);
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
         const unsigned short* p = As + ln.fa[i] + 16 * ks * BT;
@@ -101,22 +105,34 @@ __device__ __forceinline__ void load_frags(const unsigned short* As, const unsig
     }
 }
 
-template <typename E>
-__device__ __forceinline__ void mma16(const Frag& f, f32x16 (&acc)[4][4]) {
+template <typename E, int J>
+__device__ __forceinline__ void mma16(const Frag& f, f32x16 (&acc)[4][J]) {
 #pragma unroll
     for (int i = 0; i < 4; ++i)
 #pragma unroll
-        for (int j = 0; j < 4; ++j) acc[i][j] = E::mfma32(f.b[j], f.a[i], acc[i][j]);
+        for (int j = 0; j < J; ++j) acc[i][j] = E::mfma32(f.b[j], f.a[i], acc[i][j]);
 }
 
-// Spread 12 LDS reads and (if DMA) 4 global->LDS transfers over 16 MFMAs.
-template <bool DMA, bool FRAGS>
+// Spread the 8 + J LDS reads and (if NDMA) the 4 (A) or J (B) global->LDS transfers of a half step
+// over its 4*J MFMAs.
+template <int J, int NDMA, bool FRAGS>
 __device__ __forceinline__ void interleave16() {
+    if constexpr (J == 4) {
 #pragma unroll
-    for (int i = 0; i < 16; ++i) {
-        __builtin_amdgcn_sched_group_barrier(SG_MFMA, 1, 0);
-        if (FRAGS && i < 12) __builtin_amdgcn_sched_group_barrier(SG_DSRD, 1, 0);
-        if (DMA && (i & 3) == 1) __builtin_amdgcn_sched_group_barrier(SG_VMEM, 1, 0);
+        for (int i = 0; i < 16; ++i) {
+            __builtin_amdgcn_sched_group_barrier(SG_MFMA, 1, 0);
+            if (FRAGS && i < 12) __builtin_amdgcn_sched_group_barrier(SG_DSRD, 1, 0);
+            if (NDMA && (i & 3) == 1) __builtin_amdgcn_sched_group_barrier(SG_VMEM, 1, 0);
+        }
+    } else {
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            __builtin_amdgcn_sched_group_barrier(SG_MFMA, 1, 0);
+            if (FRAGS) __builtin_amdgcn_sched_group_barrier(SG_DSRD, 1, 0);
+            if (FRAGS && i < 2) __builtin_amdgcn_sched_group_barrier(SG_DSRD, 1, 0);
+            if (NDMA == 4 && (i & 1) == 1) __builtin_amdgcn_sched_group_barrier(SG_VMEM, 1, 0);
+            if (NDMA == 2 && (i & 3) == 1) __builtin_amdgcn_sched_group_barrier(SG_VMEM, 1, 0);
+        }
     }
     __builtin_amdgcn_sched_barrier(0);
 }
@@ -140,29 +156,30 @@ __device__ __forceinline__ void stage_barrier() {
 //   barrier
 //   second half: MFMAs of sub-step 1 | read next stage's sub-step 0 fragments | issue B transfers (into BsX)
 // TAIL: the stages requested here may reach past K; k_left3 = K - (first k of step s+3).
-template <typename E, bool DMA_A, bool DMA_B, int VMCNT, bool LAST, bool TAIL>
+template <typename E, int J, bool DMA_A, bool DMA_B, int VMCNT, bool LAST, bool TAIL>
 __device__ __forceinline__ void k_step(const unsigned short* AsX, unsigned short* BsX, const unsigned short* AsY,
                                        const unsigned short* BsY, unsigned short* AsA, const char* Ag_next3,
                                        const char* Bg_next4, int64_t lda2, int64_t ldb2, int wave, const Lane& ln,
-                                       Frag& f0, Frag& f1, f32x16 (&acc)[4][4], int k_left3) {
+                                       Frag& f0, Frag& f1, f32x16 (&acc)[4][J], int k_left3) {
     if (DMA_A) issue_A<TAIL>(Ag_next3, lda2, AsA, wave, ln, k_left3);
-    load_frags(AsX, BsX, ln, 1, f1);
-    mma16<E>(f0, acc);
-    interleave16<DMA_A, true>();
+    load_frags<J>(AsX, BsX, ln, 1, f1);
+    mma16<E, J>(f0, acc);
+    interleave16<J, DMA_A ? 4 : 0, true>();
     if (!LAST) stage_barrier<VMCNT>();
-    if (DMA_B) issue_B<TAIL>(Bg_next4, ldb2, BsX, wave, ln, k_left3 - BK);
-    if (!LAST) load_frags(AsY, BsY, ln, 0, f0);
-    mma16<E>(f1, acc);
-    interleave16<DMA_B, !LAST>();
+    if (DMA_B) issue_B<J, TAIL>(Bg_next4, ldb2, BsX, wave, ln, k_left3 - BK);
+    if (!LAST) load_frags<J>(AsY, BsY, ln, 0, f0);
+    mma16<E, J>(f1, acc);
+    interleave16<J, DMA_B ? J : 0, !LAST>();
 }
 
-template <typename E, typename OutT>
+template <typename E, typename OutT, int J>
 __global__ __launch_bounds__(256) void gemm16_big(const unsigned short* __restrict__ A, int64_t lda, int64_t sa,
                                                   const unsigned short* __restrict__ B, int64_t ldb, int64_t sb,
                                                   OutT* __restrict__ C, int64_t ldc, int64_t sc, int M, int N, int K,
                                                   int tiles_m, int tiles_n) {
     __shared__ __attribute__((aligned(1024))) unsigned short As0[STAGE], As1[STAGE], As2[STAGE], As3[STAGE];
-    __shared__ __attribute__((aligned(1024))) unsigned short Bs0[STAGE], Bs1[STAGE], Bs2[STAGE], Bs3[STAGE];
+    constexpr int BTN = 64 * J, STAGE_B = BTN * BK;
+    __shared__ __attribute__((aligned(1024))) unsigned short Bs0[STAGE_B], Bs1[STAGE_B], Bs2[STAGE_B], Bs3[STAGE_B];
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int total = tiles_m * tiles_n;
@@ -173,7 +190,7 @@ __global__ __launch_bounds__(256) void gemm16_big(const unsigned short* __restri
     const int first_m = (L / per_group) * GM;
     const int gsz = tiles_m - first_m < GM ? tiles_m - first_m : GM;
     const int bm = first_m + (L % per_group) % gsz, bn = (L % per_group) / gsz;
-    const int wm = (wave & 1) * 128, wn = (wave >> 1) * 128;
+    const int wm = (wave & 1) * 128, wn = (wave >> 1) * (32 * J);
 
     Lane ln;
     {
@@ -182,9 +199,9 @@ __global__ __launch_bounds__(256) void gemm16_big(const unsigned short* __restri
         // In a tile that reaches past N the rows beyond the edge re-read row N-1 (their products land in
         // accumulators that are never stored), so every transfer stays inside the matrix.
         {
-            const int first = bn * BT + 16 * wave;               // first row of the wave's transfer 0
+            const int first = bn * BTN + 16 * wave;              // first row of the wave's transfer 0
 #pragma unroll
-            for (int j = 0; j < 4; ++j) {
+            for (int j = 0; j < J; ++j) {
                 int row = 64 * j + (lane >> 2);                  // relative to `first`
                 if (first + row > N - 1) row = N - 1 - first;    // (may be negative: still inside the tile's rows)
                 ln.goffB[j] = ((int64_t)row * ldb + 8 * ((lane & 3) ^ ((lane >> 4) & 3))) * 2;
@@ -213,50 +230,51 @@ __global__ __launch_bounds__(256) void gemm16_big(const unsigned short* __restri
     const int64_t lda2 = lda * 2, ldb2 = ldb * 2;
     // wave-uniform byte pointers to this wave's first rows of the k = 0 stage
     const char* Ab = (const char*)(A + (int64_t)blockIdx.z * sa + (int64_t)bm * BT) + (int64_t)(2 * wave) * lda2;
-    const char* Bb = (const char*)(B + (int64_t)blockIdx.z * sb + (int64_t)bn * BT * ldb) + (int64_t)(16 * wave) * ldb2;
+    const char* Bb = (const char*)(B + (int64_t)blockIdx.z * sb + (int64_t)bn * BTN * ldb) + (int64_t)(16 * wave) * ldb2;
     C += (int64_t)blockIdx.z * sc;
     const int64_t a_step = (int64_t)BK * lda2;  // next K step of A: 32 rows down
     const int64_t b_step = (int64_t)BK * 2;     // next K step of B: 32 elements along the row
 
-    f32x16 acc[4][4];
+    f32x16 acc[4][J];
 #pragma unroll
     for (int i = 0; i < 4; ++i)
 #pragma unroll
-        for (int j = 0; j < 4; ++j) acc[i][j] = f32x16{0};
+        for (int j = 0; j < J; ++j) acc[i][j] = f32x16{0};
 
     const int KT = 4 * ((K + 4 * BK - 1) / (4 * BK));  // steps, in whole groups of four; >= 8 (K >= 256 is checked on the host)
     Frag f0, f1;
-    // prologue: stages 0..2 and the B half of stage 3 (28 transfers per wave)
-    issue_B(Bb, ldb2, Bs0, wave, ln);
+    // prologue: stages 0..2 and the B half of stage 3 (4 + J transfers per wave and stage); wait for stage 0
+    issue_B<J>(Bb, ldb2, Bs0, wave, ln);
     issue_A(Ab, lda2, As0, wave, ln);
-    issue_B(Bb + b_step, ldb2, Bs1, wave, ln);
+    issue_B<J>(Bb + b_step, ldb2, Bs1, wave, ln);
     issue_A(Ab + a_step, lda2, As1, wave, ln);
-    issue_B(Bb + 2 * b_step, ldb2, Bs2, wave, ln);
+    issue_B<J>(Bb + 2 * b_step, ldb2, Bs2, wave, ln);
     issue_A(Ab + 2 * a_step, lda2, As2, wave, ln);
-    issue_B(Bb + 3 * b_step, ldb2, Bs3, wave, ln);
-    stage_barrier<20>();
-    load_frags(As0, Bs0, ln, 0, f0);
+    issue_B<J>(Bb + 3 * b_step, ldb2, Bs3, wave, ln);
+    constexpr int PER_STAGE = 4 + J;   // transfers per wave and stage: the waits below leave 2, 1 or 0 stages in flight
+    stage_barrier<2 * PER_STAGE + J>();
+    load_frags<J>(As0, Bs0, ln, 0, f0);
 
 #define KSTEP(X, Y, AA, DA, DB, VM, LAST, TAIL, s)                                                                \
-    k_step<E, DA, DB, VM, LAST, TAIL>(As##X, Bs##X, As##Y, Bs##Y, As##AA, Ab + (int64_t)((s) + 3) * a_step,      \
+    k_step<E, J, DA, DB, (VM) * PER_STAGE, LAST, TAIL>(As##X, Bs##X, As##Y, Bs##Y, As##AA, Ab + (int64_t)((s) + 3) * a_step,      \
                                       Bb + (int64_t)((s) + 4) * b_step, lda2, ldb2, wave, ln, f0, f1, acc,       \
                                       K - ((s) + 3) * BK)
     int s = 0;
     for (; s + 12 <= KT; s += 4) {
-        KSTEP(0, 1, 3, true, true, 16, false, false, s);
-        KSTEP(1, 2, 0, true, true, 16, false, false, s + 1);
-        KSTEP(2, 3, 1, true, true, 16, false, false, s + 2);
-        KSTEP(3, 0, 2, true, true, 16, false, false, s + 3);
+        KSTEP(0, 1, 3, true, true, 2, false, false, s);
+        KSTEP(1, 2, 0, true, true, 2, false, false, s + 1);
+        KSTEP(2, 3, 1, true, true, 2, false, false, s + 2);
+        KSTEP(3, 0, 2, true, true, 2, false, false, s + 3);
     }
     // the group that requests the last four stages (the only ones that can reach past K)
-    KSTEP(0, 1, 3, true, true, 16, false, true, s);
-    KSTEP(1, 2, 0, true, true, 16, false, true, s + 1);
-    KSTEP(2, 3, 1, true, true, 16, false, true, s + 2);
-    KSTEP(3, 0, 2, true, true, 16, false, true, s + 3);
+    KSTEP(0, 1, 3, true, true, 2, false, true, s);
+    KSTEP(1, 2, 0, true, true, 2, false, true, s + 1);
+    KSTEP(2, 3, 1, true, true, 2, false, true, s + 2);
+    KSTEP(3, 0, 2, true, true, 2, false, true, s + 3);
     s += 4;
     // last four steps: only the A half of the final stage is still to be requested
-    KSTEP(0, 1, 3, true, false, 16, false, true, s);
-    KSTEP(1, 2, 0, false, false, 8, false, false, s + 1);
+    KSTEP(0, 1, 3, true, false, 2, false, true, s);
+    KSTEP(1, 2, 0, false, false, 1, false, false, s + 1);
     KSTEP(2, 3, 1, false, false, 0, false, false, s + 2);
     KSTEP(3, 0, 2, false, false, 0, true, false, s + 3);
 #undef KSTEP
@@ -264,23 +282,23 @@ __global__ __launch_bounds__(256) void gemm16_big(const unsigned short* __restri
     // Epilogue.  The lane's own offset (m within the wave tile, plus its 4*hb rows of n) is a
     // 32-bit element offset; the part of n that is uniform across the wave goes into the base.
     const unsigned lane_off = (unsigned)((lane & 31) + (int64_t)(4 * (lane >> 5)) * ldc);
-    OutT* Cw = C + (int64_t)bm * BT + wm + ((int64_t)bn * BT + wn) * ldc;
-    if ((bm + 1) * BT <= M && (bn + 1) * BT <= N) {   // interior tile (same for the whole workgroup)
+    OutT* Cw = C + (int64_t)bm * BT + wm + ((int64_t)bn * BTN + wn) * ldc;
+    if ((bm + 1) * BT <= M && (bn + 1) * BTN <= N) {   // interior tile (same for the whole workgroup)
 #pragma unroll
         for (int i = 0; i < 4; ++i)
 #pragma unroll
-            for (int j = 0; j < 4; ++j)
+            for (int j = 0; j < J; ++j)
 #pragma unroll
                 for (int r = 0; r < 16; ++r) {
                     OutT* cu = Cw + 32 * i + (int64_t)(32 * j + 8 * (r >> 2) + (r & 3)) * ldc;
                     __builtin_nontemporal_store(cvt_out<E, OutT>(acc[i][j][r]), cu + lane_off);
                 }
     } else {                                          // edge tile: clip to the matrix
-        int m_left = M - (bm * BT + wm + (lane & 31)), n_left = N - (bn * BT + wn + 4 * (lane >> 5));
+        int m_left = M - (bm * BT + wm + (lane & 31)), n_left = N - (bn * BTN + wn + 4 * (lane >> 5));
 #pragma unroll
         for (int i = 0; i < 4; ++i)
 #pragma unroll
-            for (int j = 0; j < 4; ++j)
+            for (int j = 0; j < J; ++j)
 #pragma unroll
                 for (int r = 0; r < 16; ++r) {
                     // the empty statement keeps each test next to its store (256 hoisted lane masks would
@@ -296,10 +314,25 @@ __global__ __launch_bounds__(256) void gemm16_big(const unsigned short* __restri
     }
 }
 
-template <typename E, typename OutT>
+int64_t tiles_of(const Problem& p, int btn) {
+    return (int64_t)((p.M + BT - 1) / BT) * ((p.N + btn - 1) / btn) * p.batch;
+}
+
+// 256x128 or 256x256 tiles: whichever needs less time by "rounds of 256 workgroups x time of a round".
+// A K step of a 256x128 tile takes about 0.55 of one of a 256x256 tile (measured: 4096^3 takes 132 us
+// in two rounds against 122 us in one), so the smaller tile wins when it does not cost an extra
+// round: 2048^3 (64 / 128 tiles) 42 -> 29 us, 4096 x 2048 x 4096 85 -> 67 us; 3072^3 (144 / 288) stays.
+bool half_n(const Problem& p) {
+    static const int force = [] { const char* e = getenv("MI_GEMM_BIG_J"); return e ? atoi(e) : 0; }();   // 2 or 4
+    if (force == 2 || force == 4) return force == 2;
+    const int64_t rounds4 = (tiles_of(p, 256) + 255) / 256, rounds2 = (tiles_of(p, 128) + 255) / 256;
+    return rounds2 * 11 < rounds4 * 20;
+}
+
+template <typename E, typename OutT, int J>
 void launch(const Problem& p, hipStream_t s) {
-    const int tiles_m = (p.M + BT - 1) / BT, tiles_n = (p.N + BT - 1) / BT;
-    hipLaunchKernelGGL((gemm16_big<E, OutT>), dim3((unsigned)(tiles_m * tiles_n), 1, (unsigned)p.batch), dim3(256), 0,
+    const int tiles_m = (p.M + BT - 1) / BT, tiles_n = (p.N + 64 * J - 1) / (64 * J);
+    hipLaunchKernelGGL((gemm16_big<E, OutT, J>), dim3((unsigned)(tiles_m * tiles_n), 1, (unsigned)p.batch), dim3(256), 0,
                        s, (const unsigned short*)p.A, p.lda, p.sa, (const unsigned short*)p.B, p.ldb, p.sb,
                        (OutT*)p.C, p.ldc, p.sc, p.M, p.N, p.K, tiles_m, tiles_n);
 }
@@ -312,7 +345,7 @@ namespace gemm {
 bool big16_applicable(const Problem& p) {
     if (p.in_dtype != MI_F16 && p.in_dtype != MI_BF16) return false;
     // M and K multiples of 8 (A and B move in 16-byte chunks along m and k), any N
-    const int64_t tiles = (int64_t)((p.M + BT - 1) / BT) * ((p.N + BT - 1) / BT) * p.batch;
+    const int64_t tiles = tiles_of(p, 128);
     return p.M % 8 == 0 && p.M >= 8 && p.N >= 1 && p.K % 8 == 0 && p.K >= 256 && aligned(p.A, 16) && aligned(p.B, 16) &&
            p.lda % 8 == 0 && p.ldb % 8 == 0 && p.sa % 8 == 0 && p.sb % 8 == 0 && p.ldc < (1 << 26) &&
            p.lda < (1 << 26) && p.ldb < (1 << 26) && tiles >= 64;
@@ -320,14 +353,17 @@ bool big16_applicable(const Problem& p) {
 
 void big16_launch(const Problem& p, hipStream_t s) {
     const bool f32out = p.out_dtype == MI_F32;
+    const bool h = half_n(p);
+#define BIG(E, O) (h ? launch<E, O, 2>(p, s) : launch<E, O, 4>(p, s))
     if (p.in_dtype == MI_F16) {
-        if (f32out) launch<F16, float>(p, s);
-        else launch<F16, unsigned short>(p, s);
+        if (f32out) BIG(F16, float);
+        else BIG(F16, unsigned short);
     } else {
-        if (f32out) launch<BF16, float>(p, s);
-        else launch<BF16, unsigned short>(p, s);
+        if (f32out) BIG(BF16, float);
+        else BIG(BF16, unsigned short);
     }
-    set_variant("gemm16_big_256x256x32_ring4");
+#undef BIG
+    set_variant(h ? "gemm16_big_256x128x32_ring4" : "gemm16_big_256x256x32_ring4");
 }
 
 }  // namespace gemm

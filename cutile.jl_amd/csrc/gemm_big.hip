@@ -37,11 +37,11 @@ namespace {
 using namespace mi;
 using namespace mi::gemm;
 
-// The tile is BT m x (64*J) n: J = 4 is the 256x256 tile described above, J = 2 a 256x128 tile (waves of
-// 128x64, half the B stage, half the accumulators) for problems that would otherwise give too few
-// workgroups to the chip.
-constexpr int BT = 256, BK = 32;
-constexpr int STAGE = BT * BK;  // elements per A stage, and per B stage at J = 4 (16 KB)
+// The tile is (64*I) m x (64*J) n, a wave's part (32*I) x (32*J): I = J = 4 is the 256x256 tile described
+// above; 256x128 (I = 4, J = 2: half the B stage, half the accumulators) and 128x128 (I = J = 2: 64 KB of
+// LDS, two workgroups per CU) serve problems that would otherwise give too few workgroups to the chip.
+// An A stage of 32 k x (64*I) m moves as 4*I transfers of 1 KB, each 8/I rows of k; a row is 8*I chunks.
+constexpr int BK = 32;
 
 #define SG_MFMA 0x008
 #define SG_VMEM 0x010
@@ -56,11 +56,11 @@ __device__ __forceinline__ void gload_lds16(const void* g, void* lds_wave_base) 
 __device__ __attribute__((aligned(16))) const unsigned zeros16[4] = {0u, 0u, 0u, 0u};
 
 struct Lane {
-    int kA, kB;             // first k, within a stage, of the lane's chunk in A transfer 0 (transfer j: + 8*j) / in a B transfer
+    int kA, kB;             // first k, within a stage, of the lane's chunk in A transfer 0 (transfer j: + 32/I*j) / in a B transfer
     unsigned goffA;         // byte offset of this lane's 16-byte chunk within a wave-wide 1 KB transfer of A
     int64_t goffB[4];       // the same for the wave's four B transfers (rows past the matrix edge re-read the last row)
     unsigned fb[2];         // LDS element offset of the B fragment, k16 sub-step 0/1 (+ 32*j*BK for n tile j)
-    unsigned fa[4];         // LDS element offset of the A fragment, m tile i (+ 16*ks*BT for sub-step ks)
+    unsigned fa[4];         // LDS element offset of the A fragment, m tile i (+ 16*ks*64*I for sub-step ks)
 };
 
 struct Frag {
@@ -79,45 +79,54 @@ __device__ __forceinline__ void issue_B(const char* Bg, int64_t ldb2, unsigned s
         gload_lds16(g, Bs + (wave + 4 * j) * 512);
     }
 }
-// A stage: 32 rows x 512 B = 16 transfers of 1 KB (2 rows each).
-template <bool TAIL = false>
+// A stage: 32 rows x 128*I B = 4*I transfers of 1 KB (8/I rows each); wave w takes transfers w, w+4, ...
+template <int I, bool TAIL = false>
 __device__ __forceinline__ void issue_A(const char* Ag, int64_t lda2, unsigned short* As, int wave, const Lane& ln,
                                         int k_left = 0) {
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
-        const char* g = Ag + (int64_t)(8 * j) * lda2 + ln.goffA;
-        if (TAIL && ln.kA + 8 * j >= k_left) g = (const char*)zeros16;
+    for (int j = 0; j < I; ++j) {
+        const char* g = Ag + (int64_t)(32 / I * j) * lda2 + ln.goffA;
+        if (TAIL && ln.kA + 32 / I * j >= k_left) g = (const char*)zeros16;
         gload_lds16(g, As + (wave + 4 * j) * 512);
     }
 }
 
-template <int J>
+template <int I, int J>
 __device__ __forceinline__ void load_frags(const unsigned short* As, const unsigned short* Bs, const Lane& ln, int ks,
                                            Frag& f) {
+    constexpr int BTM = 64 * I;
 #pragma unroll
     for (int j = 0; j < J; ++j) f.b[j] = *reinterpret_cast<const s16x8*>(Bs + ln.fb[ks] + 32 * j * BK);
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-        const unsigned short* p = As + ln.fa[i] + 16 * ks * BT;
+    for (int i = 0; i < I; ++i) {
+        const unsigned short* p = As + ln.fa[i] + 16 * ks * BTM;
         s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16(LDS_PTR(s16x4, p));
-        s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(LDS_PTR(s16x4, p + 4 * BT));
+        s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(LDS_PTR(s16x4, p + 4 * BTM));
         f.a[i] = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
     }
 }
 
-template <typename E, int J>
-__device__ __forceinline__ void mma16(const Frag& f, f32x16 (&acc)[4][J]) {
+template <typename E, int I, int J>
+__device__ __forceinline__ void mma16(const Frag& f, f32x16 (&acc)[I][J]) {
 #pragma unroll
-    for (int i = 0; i < 4; ++i)
+    for (int i = 0; i < I; ++i)
 #pragma unroll
         for (int j = 0; j < J; ++j) acc[i][j] = E::mfma32(f.b[j], f.a[i], acc[i][j]);
 }
 
-// Spread the 8 + J LDS reads and (if NDMA) the 4 (A) or J (B) global->LDS transfers of a half step
-// over its 4*J MFMAs.
-template <int J, int NDMA, bool FRAGS>
+// Spread the 2*I + J LDS reads and (if NDMA) the I (A) or J (B) global->LDS transfers of a half step
+// over its I*J MFMAs.
+template <int I, int J, int NDMA, bool FRAGS>
 __device__ __forceinline__ void interleave16() {
-    if constexpr (J == 4) {
+    if constexpr (I == 2) {   // 4 MFMAs, 6 reads, 2 transfers
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            __builtin_amdgcn_sched_group_barrier(SG_MFMA, 1, 0);
+            if (FRAGS) __builtin_amdgcn_sched_group_barrier(SG_DSRD, 1, 0);
+            if (FRAGS && i < 2) __builtin_amdgcn_sched_group_barrier(SG_DSRD, 1, 0);
+            if (NDMA && (i & 1) == 1) __builtin_amdgcn_sched_group_barrier(SG_VMEM, 1, 0);
+        }
+    } else if constexpr (J == 4) {
 #pragma unroll
         for (int i = 0; i < 16; ++i) {
             __builtin_amdgcn_sched_group_barrier(SG_MFMA, 1, 0);
@@ -156,29 +165,29 @@ __device__ __forceinline__ void stage_barrier() {
 //   barrier
 //   second half: MFMAs of sub-step 1 | read next stage's sub-step 0 fragments | issue B transfers (into BsX)
 // TAIL: the stages requested here may reach past K; k_left3 = K - (first k of step s+3).
-template <typename E, int J, bool DMA_A, bool DMA_B, int VMCNT, bool LAST, bool TAIL>
+template <typename E, int I, int J, bool DMA_A, bool DMA_B, int VMCNT, bool LAST, bool TAIL>
 __device__ __forceinline__ void k_step(const unsigned short* AsX, unsigned short* BsX, const unsigned short* AsY,
                                        const unsigned short* BsY, unsigned short* AsA, const char* Ag_next3,
                                        const char* Bg_next4, int64_t lda2, int64_t ldb2, int wave, const Lane& ln,
-                                       Frag& f0, Frag& f1, f32x16 (&acc)[4][J], int k_left3) {
-    if (DMA_A) issue_A<TAIL>(Ag_next3, lda2, AsA, wave, ln, k_left3);
-    load_frags<J>(AsX, BsX, ln, 1, f1);
-    mma16<E, J>(f0, acc);
-    interleave16<J, DMA_A ? 4 : 0, true>();
+                                       Frag& f0, Frag& f1, f32x16 (&acc)[I][J], int k_left3) {
+    if (DMA_A) issue_A<I, TAIL>(Ag_next3, lda2, AsA, wave, ln, k_left3);
+    load_frags<I, J>(AsX, BsX, ln, 1, f1);
+    mma16<E, I, J>(f0, acc);
+    interleave16<I, J, DMA_A ? I : 0, true>();
     if (!LAST) stage_barrier<VMCNT>();
     if (DMA_B) issue_B<J, TAIL>(Bg_next4, ldb2, BsX, wave, ln, k_left3 - BK);
-    if (!LAST) load_frags<J>(AsY, BsY, ln, 0, f0);
-    mma16<E, J>(f1, acc);
-    interleave16<J, DMA_B ? J : 0, !LAST>();
+    if (!LAST) load_frags<I, J>(AsY, BsY, ln, 0, f0);
+    mma16<E, I, J>(f1, acc);
+    interleave16<I, J, DMA_B ? J : 0, !LAST>();
 }
 
-template <typename E, typename OutT, int J>
+template <typename E, typename OutT, int I, int J>
 __global__ __launch_bounds__(256) void gemm16_big(const unsigned short* __restrict__ A, int64_t lda, int64_t sa,
                                                   const unsigned short* __restrict__ B, int64_t ldb, int64_t sb,
                                                   OutT* __restrict__ C, int64_t ldc, int64_t sc, int M, int N, int K,
                                                   int tiles_m, int tiles_n) {
-    __shared__ __attribute__((aligned(1024))) unsigned short As0[STAGE], As1[STAGE], As2[STAGE], As3[STAGE];
-    constexpr int BTN = 64 * J, STAGE_B = BTN * BK;
+    constexpr int BTM = 64 * I, STAGE_A = BTM * BK, BTN = 64 * J, STAGE_B = BTN * BK;
+    __shared__ __attribute__((aligned(1024))) unsigned short As0[STAGE_A], As1[STAGE_A], As2[STAGE_A], As3[STAGE_A];
     __shared__ __attribute__((aligned(1024))) unsigned short Bs0[STAGE_B], Bs1[STAGE_B], Bs2[STAGE_B], Bs3[STAGE_B];
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -190,7 +199,7 @@ __global__ __launch_bounds__(256) void gemm16_big(const unsigned short* __restri
     const int first_m = (L / per_group) * GM;
     const int gsz = tiles_m - first_m < GM ? tiles_m - first_m : GM;
     const int bm = first_m + (L % per_group) % gsz, bn = (L % per_group) / gsz;
-    const int wm = (wave & 1) * 128, wn = (wave >> 1) * (32 * J);
+    const int wm = (wave & 1) * (32 * I), wn = (wave >> 1) * (32 * J);
 
     Lane ln;
     {
@@ -207,56 +216,56 @@ __global__ __launch_bounds__(256) void gemm16_big(const unsigned short* __restri
                 ln.goffB[j] = ((int64_t)row * ldb + 8 * ((lane & 3) ^ ((lane >> 4) & 3))) * 2;
             }
         }
-        // A transfer: lane -> row lane/32 of its 2-row block, LDS position lane%32; rows k = 2*blk + lane/32.
-        // Chunks of 8 m past the edge re-read the last whole chunk (M is a multiple of 8).
-        const int ka = 2 * wave + (lane >> 5);
+        // A transfer: lane -> row lane/(8*I) of its block of 8/I rows, LDS position lane%(8*I); rows
+        // k = 8/I*blk + lane/(8*I).  Chunks of 8 m past the edge re-read the last whole chunk (M is a multiple of 8).
+        const int ka = 8 / I * wave + lane / (8 * I);
         ln.kA = ka;
         ln.kB = 8 * ((lane & 3) ^ ((lane >> 4) & 3));
-        int ca = (lane & 31) ^ (4 * (ka & 3));
-        if (bm * BT + 8 * ca + 8 > M) ca = (M - bm * BT) / 8 - 1;
-        ln.goffA = (unsigned)(((int64_t)(lane >> 5) * lda + 8 * ca) * 2);
+        int ca = (lane % (8 * I)) ^ (4 * (ka & 3));
+        if (bm * BTM + 8 * ca + 8 > M) ca = (M - bm * BTM) / 8 - 1;
+        ln.goffA = (unsigned)(((int64_t)(lane / (8 * I)) * lda + 8 * ca) * 2);
 #pragma unroll
         for (int ks = 0; ks < 2; ++ks) {
             const int n = wn + (lane & 31);
             ln.fb[ks] = n * BK + 8 * ((2 * ks + hb) ^ ((n >> 2) & 3));
         }
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
+        for (int i = 0; i < I; ++i) {
             const int k = 8 * (g >> 1) + (r >> 2);
             const int m = wm + 32 * i + 16 * (g & 1) + 4 * (r & 3);
-            ln.fa[i] = k * BT + 8 * ((m >> 3) ^ (4 * (r >> 2))) + (m & 7);
+            ln.fa[i] = k * BTM + 8 * ((m >> 3) ^ (4 * (r >> 2))) + (m & 7);
         }
     }
     const int64_t lda2 = lda * 2, ldb2 = ldb * 2;
     // wave-uniform byte pointers to this wave's first rows of the k = 0 stage
-    const char* Ab = (const char*)(A + (int64_t)blockIdx.z * sa + (int64_t)bm * BT) + (int64_t)(2 * wave) * lda2;
+    const char* Ab = (const char*)(A + (int64_t)blockIdx.z * sa + (int64_t)bm * BTM) + (int64_t)(8 / I * wave) * lda2;
     const char* Bb = (const char*)(B + (int64_t)blockIdx.z * sb + (int64_t)bn * BTN * ldb) + (int64_t)(16 * wave) * ldb2;
     C += (int64_t)blockIdx.z * sc;
     const int64_t a_step = (int64_t)BK * lda2;  // next K step of A: 32 rows down
     const int64_t b_step = (int64_t)BK * 2;     // next K step of B: 32 elements along the row
 
-    f32x16 acc[4][J];
+    f32x16 acc[I][J];
 #pragma unroll
-    for (int i = 0; i < 4; ++i)
+    for (int i = 0; i < I; ++i)
 #pragma unroll
         for (int j = 0; j < J; ++j) acc[i][j] = f32x16{0};
 
     const int KT = 4 * ((K + 4 * BK - 1) / (4 * BK));  // steps, in whole groups of four; >= 8 (K >= 256 is checked on the host)
     Frag f0, f1;
-    // prologue: stages 0..2 and the B half of stage 3 (4 + J transfers per wave and stage); wait for stage 0
+    // prologue: stages 0..2 and the B half of stage 3 (I + J transfers per wave and stage); wait for stage 0
     issue_B<J>(Bb, ldb2, Bs0, wave, ln);
-    issue_A(Ab, lda2, As0, wave, ln);
+    issue_A<I>(Ab, lda2, As0, wave, ln);
     issue_B<J>(Bb + b_step, ldb2, Bs1, wave, ln);
-    issue_A(Ab + a_step, lda2, As1, wave, ln);
+    issue_A<I>(Ab + a_step, lda2, As1, wave, ln);
     issue_B<J>(Bb + 2 * b_step, ldb2, Bs2, wave, ln);
-    issue_A(Ab + 2 * a_step, lda2, As2, wave, ln);
+    issue_A<I>(Ab + 2 * a_step, lda2, As2, wave, ln);
     issue_B<J>(Bb + 3 * b_step, ldb2, Bs3, wave, ln);
-    constexpr int PER_STAGE = 4 + J;   // transfers per wave and stage: the waits below leave 2, 1 or 0 stages in flight
+    constexpr int PER_STAGE = I + J;   // transfers per wave and stage: the waits below leave 2, 1 or 0 stages in flight
     stage_barrier<2 * PER_STAGE + J>();
-    load_frags<J>(As0, Bs0, ln, 0, f0);
+    load_frags<I, J>(As0, Bs0, ln, 0, f0);
 
 #define KSTEP(X, Y, AA, DA, DB, VM, LAST, TAIL, s)                                                                \
-    k_step<E, J, DA, DB, (VM) * PER_STAGE, LAST, TAIL>(As##X, Bs##X, As##Y, Bs##Y, As##AA, Ab + (int64_t)((s) + 3) * a_step,      \
+    k_step<E, I, J, DA, DB, (VM) * PER_STAGE, LAST, TAIL>(As##X, Bs##X, As##Y, Bs##Y, As##AA, Ab + (int64_t)((s) + 3) * a_step,      \
                                       Bb + (int64_t)((s) + 4) * b_step, lda2, ldb2, wave, ln, f0, f1, acc,       \
                                       K - ((s) + 3) * BK)
     int s = 0;
@@ -282,10 +291,10 @@ __global__ __launch_bounds__(256) void gemm16_big(const unsigned short* __restri
     // Epilogue.  The lane's own offset (m within the wave tile, plus its 4*hb rows of n) is a
     // 32-bit element offset; the part of n that is uniform across the wave goes into the base.
     const unsigned lane_off = (unsigned)((lane & 31) + (int64_t)(4 * (lane >> 5)) * ldc);
-    OutT* Cw = C + (int64_t)bm * BT + wm + ((int64_t)bn * BTN + wn) * ldc;
-    if ((bm + 1) * BT <= M && (bn + 1) * BTN <= N) {   // interior tile (same for the whole workgroup)
+    OutT* Cw = C + (int64_t)bm * BTM + wm + ((int64_t)bn * BTN + wn) * ldc;
+    if ((bm + 1) * BTM <= M && (bn + 1) * BTN <= N) {   // interior tile (same for the whole workgroup)
 #pragma unroll
-        for (int i = 0; i < 4; ++i)
+        for (int i = 0; i < I; ++i)
 #pragma unroll
             for (int j = 0; j < J; ++j)
 #pragma unroll
@@ -294,9 +303,9 @@ __global__ __launch_bounds__(256) void gemm16_big(const unsigned short* __restri
                     __builtin_nontemporal_store(cvt_out<E, OutT>(acc[i][j][r]), cu + lane_off);
                 }
     } else {                                          // edge tile: clip to the matrix
-        int m_left = M - (bm * BT + wm + (lane & 31)), n_left = N - (bn * BTN + wn + 4 * (lane >> 5));
+        int m_left = M - (bm * BTM + wm + (lane & 31)), n_left = N - (bn * BTN + wn + 4 * (lane >> 5));
 #pragma unroll
-        for (int i = 0; i < 4; ++i)
+        for (int i = 0; i < I; ++i)
 #pragma unroll
             for (int j = 0; j < J; ++j)
 #pragma unroll
@@ -314,25 +323,28 @@ __global__ __launch_bounds__(256) void gemm16_big(const unsigned short* __restri
     }
 }
 
-int64_t tiles_of(const Problem& p, int btn) {
-    return (int64_t)((p.M + BT - 1) / BT) * ((p.N + btn - 1) / btn) * p.batch;
+int64_t tiles_of(const Problem& p, int btm, int btn) {
+    return (int64_t)((p.M + btm - 1) / btm) * ((p.N + btn - 1) / btn) * p.batch;
 }
 
-// 256x128 or 256x256 tiles: whichever needs less time by "rounds of 256 workgroups x time of a round".
-// A K step of a 256x128 tile takes about 0.55 of one of a 256x256 tile (measured: 4096^3 takes 132 us
-// in two rounds against 122 us in one), so the smaller tile wins when it does not cost an extra
-// round: 2048^3 (64 / 128 tiles) 42 -> 29 us, 4096 x 2048 x 4096 85 -> 67 us; 3072^3 (144 / 288) stays.
-bool half_n(const Problem& p) {
-    static const int force = [] { const char* e = getenv("MI_GEMM_BIG_J"); return e ? atoi(e) : 0; }();   // 2 or 4
-    if (force == 2 || force == 4) return force == 2;
-    const int64_t rounds4 = (tiles_of(p, 256) + 255) / 256, rounds2 = (tiles_of(p, 128) + 255) / 256;
-    return rounds2 * 11 < rounds4 * 20;
+// Tile size: whichever needs least time by "rounds of workgroups x time of a round".  Measured time of
+// one K step of a round (us): 256x256 0.63 (a quarter of the CUs busy) to 0.93 (all busy: the clock
+// drops); 256x128 0.42 to 0.51; 128x128 0.33 with one workgroup per CU, 0.58 when CUs hold two.
+// f16 examples (us, 256x256 / 256x128 / 128x128): 1024^3 23 / 15 / 10, 2048^3 40 / 27 / 21,
+// 2560^3 51 / 37 / 46, 4096 x 2048 x 4096 77 / 65 / 74, 3072^3 64 / 83 / 77, 4096^3 119 / 128 / 144.
+int pick_tile(const Problem& p) {
+    static const int force = [] { const char* e = getenv("MI_GEMM_BIG_TILE"); return e ? atoi(e) : 0; }();   // 44, 42 or 22
+    if (force == 44 || force == 42 || force == 22) return force;
+    const int64_t t44 = tiles_of(p, 256, 256), t42 = tiles_of(p, 256, 128), t22 = tiles_of(p, 128, 128);
+    const int64_t c44 = (t44 + 255) / 256 * 90, c42 = (t42 + 255) / 256 * 50;
+    const int64_t c22 = t22 <= 256 ? 33 : (t22 + 511) / 512 * 60;
+    return c22 <= c42 && c22 <= c44 ? 22 : c42 <= c44 ? 42 : 44;
 }
 
-template <typename E, typename OutT, int J>
+template <typename E, typename OutT, int I, int J>
 void launch(const Problem& p, hipStream_t s) {
-    const int tiles_m = (p.M + BT - 1) / BT, tiles_n = (p.N + 64 * J - 1) / (64 * J);
-    hipLaunchKernelGGL((gemm16_big<E, OutT, J>), dim3((unsigned)(tiles_m * tiles_n), 1, (unsigned)p.batch), dim3(256), 0,
+    const int tiles_m = (p.M + 64 * I - 1) / (64 * I), tiles_n = (p.N + 64 * J - 1) / (64 * J);
+    hipLaunchKernelGGL((gemm16_big<E, OutT, I, J>), dim3((unsigned)(tiles_m * tiles_n), 1, (unsigned)p.batch), dim3(256), 0,
                        s, (const unsigned short*)p.A, p.lda, p.sa, (const unsigned short*)p.B, p.ldb, p.sb,
                        (OutT*)p.C, p.ldc, p.sc, p.M, p.N, p.K, tiles_m, tiles_n);
 }
@@ -345,16 +357,16 @@ namespace gemm {
 bool big16_applicable(const Problem& p) {
     if (p.in_dtype != MI_F16 && p.in_dtype != MI_BF16) return false;
     // M and K multiples of 8 (A and B move in 16-byte chunks along m and k), any N
-    const int64_t tiles = tiles_of(p, 128);
+    const int64_t tiles = tiles_of(p, 128, 128);   // (from 16 tiles of 128x128 on, this kernel is no slower than 64x64 tiles)
     return p.M % 8 == 0 && p.M >= 8 && p.N >= 1 && p.K % 8 == 0 && p.K >= 256 && aligned(p.A, 16) && aligned(p.B, 16) &&
            p.lda % 8 == 0 && p.ldb % 8 == 0 && p.sa % 8 == 0 && p.sb % 8 == 0 && p.ldc < (1 << 26) &&
-           p.lda < (1 << 26) && p.ldb < (1 << 26) && tiles >= 64;
+           p.lda < (1 << 26) && p.ldb < (1 << 26) && tiles >= 16;
 }
 
 void big16_launch(const Problem& p, hipStream_t s) {
     const bool f32out = p.out_dtype == MI_F32;
-    const bool h = half_n(p);
-#define BIG(E, O) (h ? launch<E, O, 2>(p, s) : launch<E, O, 4>(p, s))
+    const int t = pick_tile(p);
+#define BIG(E, O) (t == 22 ? launch<E, O, 2, 2>(p, s) : t == 42 ? launch<E, O, 4, 2>(p, s) : launch<E, O, 4, 4>(p, s))
     if (p.in_dtype == MI_F16) {
         if (f32out) BIG(F16, float);
         else BIG(F16, unsigned short);
@@ -363,7 +375,7 @@ void big16_launch(const Problem& p, hipStream_t s) {
         else BIG(BF16, unsigned short);
     }
 #undef BIG
-    set_variant(h ? "gemm16_big_256x128x32_ring4" : "gemm16_big_256x256x32_ring4");
+    set_variant(t == 22 ? "gemm16_big_128x128x32_ring4" : t == 42 ? "gemm16_big_256x128x32_ring4" : "gemm16_big_256x256x32_ring4");
 }
 
 }  // namespace gemm

@@ -79,13 +79,16 @@ def test_matmul_mid_tile_kernel_exact(ct, orc, M, N, K, T, out32):
     assert np.array_equal(orc.to_julia(C.float()), A @ B)      # (random sums of 333 terms stay far below 2048: exact in f16 too)
 
 
-@pytest.mark.parametrize("M,N,K,T,out32,tile", [(2048, 2048, 256, torch.float16, True, "256x128"), (2048, 2048, 384, torch.float16, False, "256x128"),
-                                                 (4096, 1024, 512, torch.bfloat16, True, "256x128"), (1024, 4096, 640, torch.bfloat16, False, "256x128"),
+@pytest.mark.parametrize("M,N,K,T,out32,tile", [(2048, 2048, 256, torch.float16, True, "128x128"), (2048, 2048, 384, torch.float16, False, "128x128"),
+                                                 (4096, 1024, 512, torch.bfloat16, True, "128x128"), (1024, 4096, 640, torch.bfloat16, False, "128x128"),
+                                                 (512, 512, 768, torch.float16, True, "128x128"),
                                                  (4096, 4096, 256, torch.float16, False, "256x256"), (3072, 3072, 384, torch.bfloat16, True, "256x256"),
-                                                 (4096, 2048, 512, torch.float16, True, "256x128"), (8192, 2048, 640, torch.bfloat16, False, "256x256")])
+                                                 (8192, 2048, 640, torch.bfloat16, False, "256x256"),
+                                                 (4096, 2048, 512, torch.float16, True, "256x128"), (2560, 2560, 256, torch.bfloat16, False, "256x128"),
+                                                 (2048, 4096, 384, torch.float16, False, "256x128")])
 def test_matmul_large_tile_kernel_exact(ct, orc, M, N, K, T, out32, tile):
-    """Shapes that take the direct-to-LDS kernel (>= 64 tiles, K >= 256) in its two tile sizes (256x128
-    when that does not cost a further round of 256 workgroups), with small-integer operands so the
+    """Shapes that take the direct-to-LDS kernel (K >= 256) in each of its three tile sizes (chosen by
+    the number of workgroups the problem gives the 256 CUs), with small-integer operands so the
     expected result is exact: checks the swizzled LDS layouts, the ring of stages (K/32 = 8, 12, 16, 20
     steps) and the tile -> workgroup mapping."""
     rng = np.random.default_rng(7)
@@ -99,12 +102,12 @@ def test_matmul_large_tile_kernel_exact(ct, orc, M, N, K, T, out32, tile):
     assert np.array_equal(orc.to_julia(C).astype(np.float32), ref)
 
 
-@pytest.mark.parametrize("M,N,K,T,out32", [(2040, 2000, 256, torch.float16, True), (2056, 2311, 384, torch.bfloat16, False),
-                                            (4000, 4001, 256, torch.float16, False), (8, 16385, 256, torch.float16, True),
-                                            (2048, 2048, 264, torch.float16, True), (2040, 2000, 1000, torch.float16, False),
-                                            (2048, 2304, 376, torch.bfloat16, True), (4096, 4096, 4000, torch.float16, True),
-                                            (3072, 3081, 328, torch.bfloat16, False)])
-def test_matmul_large_tile_kernel_ragged_edges(ct, orc, M, N, K, T, out32):
+@pytest.mark.parametrize("M,N,K,T,out32,tile", [(2040, 2000, 256, torch.float16, True, "128x128"), (2056, 2311, 384, torch.bfloat16, False, "256x128"),
+                                                 (4000, 4001, 256, torch.float16, False, "256x256"), (8, 16385, 256, torch.float16, True, "128x128"),
+                                                 (2048, 2048, 264, torch.float16, True, "128x128"), (2040, 2000, 1000, torch.float16, False, "128x128"),
+                                                 (2048, 2304, 376, torch.bfloat16, True, "256x128"), (4096, 4096, 4000, torch.float16, True, "256x256"),
+                                                 (3072, 3081, 328, torch.bfloat16, False, "256x256"), (1096, 1001, 1064, torch.bfloat16, False, "128x128")])
+def test_matmul_large_tile_kernel_ragged_edges(ct, orc, M, N, K, T, out32, tile):
     """M (a multiple of 8) and N off the 256 grid on the 256x256 kernel: edge tiles re-read the last
     valid rows on the way in and clip their stores.  K (a multiple of 8) off the 128 grid: the last
     group of four steps takes zeros for k >= K (remainders of 8, 104, 120 and 32 here; A and B are
@@ -120,8 +123,7 @@ def test_matmul_large_tile_kernel_ragged_edges(ct, orc, M, N, K, T, out32):
     buf = torch.full((N + 3, M + 24), -77.0, dtype=torch.float32 if out32 else T, device="cuda")
     C = buf[:N, :M]
     ct.matmul_kernel(At, Bt, C, 64, 64, 64)
-    # both tile sizes of the kernel see ragged M, N and K
-    assert ct.last_variant() == ("gemm16_big_256x256x32_ring4" if M * N >= 3072 * 3072 else "gemm16_big_256x128x32_ring4")
+    assert ct.last_variant() == f"gemm16_big_{tile}x32_ring4"       # every tile size of the kernel sees ragged M, N and K
     assert np.array_equal(orc.to_julia(C.contiguous()).astype(np.float32), A @ B)
     assert bool((buf[N:] == -77.0).all()) and bool((buf[:, M:] == -77.0).all())
 

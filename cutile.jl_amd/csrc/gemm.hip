@@ -17,11 +17,11 @@
 //   gemm16_mid       f16/bf16, 128x128x32 workgroup tile with a register look-ahead of one K step, any
 //                    shape; used for larger problems that gemm16_big does not take (rows that are
 //                    not 16-byte aligned, K below 256).
-//   gemm16_big       (gemm_big.hip) f16/bf16, 256x256 workgroup tile, 4 waves of 128x128,
-//                    K step 32 through a ring of four LDS stages filled by direct
-//                    global->LDS loads, XOR-swizzled LDS layouts; used when M and K are
-//                    multiples of 8, K >= 256, everything is 16-byte aligned and there are at
-//                    least 64 tiles (ragged edges in M, N and K are handled on the way in).
+//   gemm16_big       (gemm_big.hip) f16/bf16, 256x256 workgroup tile, 4 waves of 128x128 (or 256x128 /
+//                    128x128 tiles for problems with few tiles), K step 32 through a ring of four LDS
+//                    stages filled by direct global->LDS loads, XOR-swizzled LDS layouts; used when M
+//                    and K are multiples of 8, K >= 256, everything is 16-byte aligned and there are
+//                    at least 16 tiles of 128x128 (ragged edges in M, N and K are handled on the way in).
 //   gemm32           fp32 via v_mfma_f32_32x32x2_f32 (gfx950 has no TF32-class MFMA;
 //                    the reference rounds fp32 operands to TF32, matmul.jl:49-52).
 //
@@ -365,9 +365,9 @@ int run(const Problem& p, hipStream_t s) {
     const bool f32out = p.out_dtype == MI_F32;
     static const int force = [] { const char* e = getenv("MI_GEMM_KERNEL"); return e ? atoi(e) : 0; }();   // 1 generic, 2 mid, 3 big
     const int64_t tiles_mid = (int64_t)cld((int64_t)p.M, (int64_t)MT) * cld((int64_t)p.N, (int64_t)MT) * p.batch;
-    // The 256x256 kernel wherever it applies (16-byte aligned rows: even with a quarter of the CUs busy it
-    // matches the 128x128 kernel); the 128x128 kernel for other shapes whose tiles give at least half
-    // the CUs work; the 64x64 kernel for what is left (small problems).
+    // The direct-to-LDS kernel wherever it applies (16-byte aligned rows; it picks its own tile size);
+    // the register-staged 128x128 kernel for other shapes whose tiles give at least half the CUs work;
+    // the 64x64 kernel for what is left (small problems).
     if (big16_applicable(p) && (force == 3 || force == 0)) {
         big16_launch(p, s);
         return launch_status();

@@ -66,7 +66,8 @@ def test_matmul_integer_valued_inputs_are_exact(ct, orc):
 @pytest.mark.parametrize("M,N,K,T,out32", [(1504, 1544, 200, torch.float16, True), (1500, 1540, 333, torch.float16, False),
                                            (2048, 1100, 96, torch.bfloat16, True), (1536, 1536, 32, torch.float16, True)])
 def test_matmul_mid_tile_kernel_exact(ct, orc, M, N, K, T, out32):
-    """The 128x128 kernel (shapes the 256x256 kernel does not take, enough tiles to fill half the chip):
+    """The register-staged 128x128 kernel (shapes the direct-to-LDS kernel does not take: rows that are not
+    16-byte aligned or K below 256; enough tiles to fill half the chip):
     aligned interior tiles without predicates, ragged edges in M, N and K, rows that are not 16-byte
     aligned (M = 1500), one and many K steps.  Integer-valued operands make every sum exact, so any
     mistake in the tile mapping, the register look-ahead or the fragment reads changes the result."""
@@ -108,7 +109,7 @@ def test_matmul_large_tile_kernel_exact(ct, orc, M, N, K, T, out32, tile):
                                                  (2048, 2304, 376, torch.bfloat16, True, "256x128"), (4096, 4096, 4000, torch.float16, True, "256x256"),
                                                  (3072, 3081, 328, torch.bfloat16, False, "256x256"), (1096, 1001, 1064, torch.bfloat16, False, "128x128")])
 def test_matmul_large_tile_kernel_ragged_edges(ct, orc, M, N, K, T, out32, tile):
-    """M (a multiple of 8) and N off the 256 grid on the 256x256 kernel: edge tiles re-read the last
+    """M (a multiple of 8) and N off the tile grid on the direct-to-LDS kernel: edge tiles re-read the last
     valid rows on the way in and clip their stores.  K (a multiple of 8) off the 128 grid: the last
     group of four steps takes zeros for k >= K (remainders of 8, 104, 120 and 32 here; A and B are
     views of buffers whose cells past K hold NaN, which must not reach the result).  Exact integer

@@ -129,6 +129,27 @@ def test_matmul_large_tile_kernel_ragged_edges(ct, orc, M, N, K, T, out32, tile)
     assert bool((buf[N:] == -77.0).all()) and bool((buf[:, M:] == -77.0).all())
 
 
+def test_matmul_direct_to_lds_kernel_shape_sweep(ct, orc):
+    """Thirty seeded shapes with M, K multiples of 8 (K >= 256) and any N, so that every tile size of the
+    direct-to-LDS kernel meets edges in M, N and K at many remainders; small-integer operands, exact sums."""
+    rng = np.random.default_rng(2024)
+    seen = set()
+    for case in range(30):
+        M = 8 * int(rng.integers(16, 420)); N = int(rng.integers(100, 3400)); K = 8 * int(rng.integers(32, 160))
+        T = torch.float16 if case % 2 == 0 else torch.bfloat16
+        out32 = case % 3 != 0
+        A = rng.integers(-1, 2, (M, K)).astype(np.float32); B = rng.integers(-2, 3, (K, N)).astype(np.float32)
+        At = orc.from_julia(A).to(T).cuda(); Bt = orc.from_julia(B).to(T).cuda()
+        C = torch.full((N, M), -77.0, dtype=torch.float32 if out32 else T, device="cuda")
+        ct.matmul_kernel(At, Bt, C, 64, 64, 64)
+        v = ct.last_variant()
+        if (-(-M // 128)) * (-(-N // 128)) >= 16:
+            assert v.startswith("gemm16_big_"), (M, N, K, v)
+        seen.add(v)
+        assert np.array_equal(orc.to_julia(C).astype(np.float32), A @ B), (M, N, K, v)
+    assert {"gemm16_big_128x128x32_ring4", "gemm16_big_256x128x32_ring4", "gemm16_big_256x256x32_ring4"} <= seen
+
+
 def test_batch_matmul_large_tile_kernel(ct, orc):
     rng = np.random.default_rng(8)
     M, K, N, Bn = 1024, 256, 1024, 4

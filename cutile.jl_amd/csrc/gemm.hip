@@ -352,7 +352,12 @@ void launch_generic16(const Problem& p, hipStream_t s) {
 
 int run(const Problem& p, hipStream_t s) {
     if (p.M == 0 || p.N == 0 || p.batch == 0) return MI_OK;
+    static const int force = [] { const char* e = getenv("MI_GEMM_KERNEL"); return e ? atoi(e) : 0; }();   // 1 generic, 2 mid, 3 big
     if (p.in_dtype == MI_F32) {
+        if (big32_applicable(p) && force != 1) {   // 16-byte aligned rows: the direct-to-LDS kernel
+            big32_launch(p, s);
+            return launch_status();
+        }
         const int tiles_m = (int)cld((int64_t)p.M, (int64_t)FT), tiles_n = (int)cld((int64_t)p.N, (int64_t)FT);
         const bool vecA = aligned(p.A, 16) && p.lda % 4 == 0 && p.sa % 4 == 0;
         const bool vecB = aligned(p.B, 16) && p.ldb % 4 == 0 && p.sb % 4 == 0;
@@ -363,7 +368,6 @@ int run(const Problem& p, hipStream_t s) {
         return launch_status();
     }
     const bool f32out = p.out_dtype == MI_F32;
-    static const int force = [] { const char* e = getenv("MI_GEMM_KERNEL"); return e ? atoi(e) : 0; }();   // 1 generic, 2 mid, 3 big
     const int64_t tiles_mid = (int64_t)cld((int64_t)p.M, (int64_t)MT) * cld((int64_t)p.N, (int64_t)MT) * p.batch;
     // The direct-to-LDS kernel wherever it applies (16-byte aligned rows; it picks its own tile size);
     // the register-staged 128x128 kernel for other shapes whose tiles give at least half the CUs work;

@@ -185,15 +185,20 @@ template <typename E, typename OutT, int I, int J>
 __global__ __launch_bounds__(256) void gemm16_big(const unsigned short* __restrict__ A, int64_t lda, int64_t sa,
                                                   const unsigned short* __restrict__ B, int64_t ldb, int64_t sb,
                                                   OutT* __restrict__ C, int64_t ldc, int64_t sc, int M, int N, int K,
-                                                  int tiles_m, int tiles_n) {
+                                                  int tiles_m, int tiles_n, int batch) {
     constexpr int BTM = 64 * I, STAGE_A = BTM * BK, BTN = 64 * J, STAGE_B = BTN * BK;
     __shared__ __attribute__((aligned(1024))) unsigned short As0[STAGE_A], As1[STAGE_A], As2[STAGE_A], As3[STAGE_A];
     __shared__ __attribute__((aligned(1024))) unsigned short Bs0[STAGE_B], Bs1[STAGE_B], Bs2[STAGE_B], Bs3[STAGE_B];
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int total = tiles_m * tiles_n;
+    // One-dimensional grid over (tile, batch).  Workgroups whose ids are congruent mod 8 share an XCD and
+    // its L2: give each XCD a contiguous run of (batch-major) tiles, so that it works on neighbouring
+    // tiles of as few batch entries as possible.
+    const int total = tiles_m * tiles_n, total_all = total * batch;
     int L = blockIdx.x;
-    if (total % 8 == 0) L = (L & 7) * (total >> 3) + (L >> 3);
+    if (total_all % 8 == 0) L = (L & 7) * (total_all >> 3) + (L >> 3);
+    const int bz = L / total;
+    L -= bz * total;
     constexpr int GM = 4;
     const int per_group = GM * tiles_n;
     const int first_m = (L / per_group) * GM;
@@ -238,9 +243,9 @@ __global__ __launch_bounds__(256) void gemm16_big(const unsigned short* __restri
     }
     const int64_t lda2 = lda * 2, ldb2 = ldb * 2;
     // wave-uniform byte pointers to this wave's first rows of the k = 0 stage
-    const char* Ab = (const char*)(A + (int64_t)blockIdx.z * sa + (int64_t)bm * BTM) + (int64_t)(8 / I * wave) * lda2;
-    const char* Bb = (const char*)(B + (int64_t)blockIdx.z * sb + (int64_t)bn * BTN * ldb) + (int64_t)(16 * wave) * ldb2;
-    C += (int64_t)blockIdx.z * sc;
+    const char* Ab = (const char*)(A + (int64_t)bz * sa + (int64_t)bm * BTM) + (int64_t)(8 / I * wave) * lda2;
+    const char* Bb = (const char*)(B + (int64_t)bz * sb + (int64_t)bn * BTN * ldb) + (int64_t)(16 * wave) * ldb2;
+    C += (int64_t)bz * sc;
     const int64_t a_step = (int64_t)BK * lda2;  // next K step of A: 32 rows down
     const int64_t b_step = (int64_t)BK * 2;     // next K step of B: 32 elements along the row
 
@@ -344,9 +349,9 @@ int pick_tile(const Problem& p) {
 template <typename E, typename OutT, int I, int J>
 void launch(const Problem& p, hipStream_t s) {
     const int tiles_m = (p.M + 64 * I - 1) / (64 * I), tiles_n = (p.N + 64 * J - 1) / (64 * J);
-    hipLaunchKernelGGL((gemm16_big<E, OutT, I, J>), dim3((unsigned)(tiles_m * tiles_n), 1, (unsigned)p.batch), dim3(256), 0,
+    hipLaunchKernelGGL((gemm16_big<E, OutT, I, J>), dim3((unsigned)(tiles_m * tiles_n * p.batch)), dim3(256), 0,
                        s, (const unsigned short*)p.A, p.lda, p.sa, (const unsigned short*)p.B, p.ldb, p.sb,
-                       (OutT*)p.C, p.ldc, p.sc, p.M, p.N, p.K, tiles_m, tiles_n);
+                       (OutT*)p.C, p.ldc, p.sc, p.M, p.N, p.K, tiles_m, tiles_n, p.batch);
 }
 
 }  // namespace
@@ -360,7 +365,7 @@ bool big16_applicable(const Problem& p) {
     const int64_t tiles = tiles_of(p, 128, 128);   // (from 16 tiles of 128x128 on, this kernel is no slower than 64x64 tiles)
     return p.M % 8 == 0 && p.M >= 8 && p.N >= 1 && p.K % 8 == 0 && p.K >= 256 && aligned(p.A, 16) && aligned(p.B, 16) &&
            p.lda % 8 == 0 && p.ldb % 8 == 0 && p.sa % 8 == 0 && p.sb % 8 == 0 && p.ldc < (1 << 26) &&
-           p.lda < (1 << 26) && p.ldb < (1 << 26) && tiles >= 16;
+           p.lda < (1 << 26) && p.ldb < (1 << 26) && tiles >= 16 && tiles < (1 << 30);
 }
 
 void big16_launch(const Problem& p, hipStream_t s) {

@@ -77,6 +77,9 @@ struct Problem {
 // gemm_big.hip: true if the 256x256 direct-to-LDS kernel applies to the problem / launches it.
 bool big16_applicable(const Problem& p);
 void big16_launch(const Problem& p, hipStream_t s);
+// gemm32_big.hip: the same for fp32 operands.
+bool big32_applicable(const Problem& p);
+void big32_launch(const Problem& p, hipStream_t s);
 
 }  // namespace gemm
 }  // namespace mi

@@ -150,6 +150,25 @@ def test_matmul_direct_to_lds_kernel_shape_sweep(ct, orc):
     assert {"gemm16_big_128x128x32_ring4", "gemm16_big_256x128x32_ring4", "gemm16_big_256x256x32_ring4"} <= seen
 
 
+@pytest.mark.parametrize("M,N,K,tile", [(2040, 2000, 256, "128x128"), (2056, 2311, 388, "256x128"), (4000, 4001, 132, "256x256"),
+                                         (4, 16385, 128, "128x128"), (3072, 3081, 196, "256x256"), (1096, 1001, 1060, "128x128"),
+                                         (2048, 2304, 376, "256x128"), (512, 512, 128, "128x128"), (4096, 4096, 320, "256x256")])
+def test_matmul_f32_direct_to_lds_kernel_exact(ct, orc, M, N, K, tile):
+    """The fp32 direct-to-LDS kernel in each tile size: M and K multiples of 4 off the tile / 64 grid, any
+    N.  Small-integer operands make every fp32 sum exact; A and B are views of buffers whose cells past K
+    hold NaN, C a view of a wider, taller buffer of sentinels that must come back untouched."""
+    rng = np.random.default_rng(M ^ N)
+    A = rng.integers(-3, 4, (M, K)).astype(np.float32); B = rng.integers(-3, 4, (K, N)).astype(np.float32)
+    Abuf = torch.full((K + 64, M), float("nan"), device="cuda"); Bbuf = torch.full((N, K + 64), float("nan"), device="cuda")
+    Abuf[:K] = orc.from_julia(A).cuda(); Bbuf[:, :K] = orc.from_julia(B).cuda()
+    buf = torch.full((N + 3, M + 12), -77.0, device="cuda")
+    C = buf[:N, :M]
+    ct.matmul_kernel(Abuf[:K], Bbuf[:, :K], C, 64, 64, 64)
+    assert ct.last_variant() == f"gemm32_big_{tile}x16_ring4"
+    assert np.array_equal(orc.to_julia(C.contiguous()), A @ B)
+    assert bool((buf[N:] == -77.0).all()) and bool((buf[:, M:] == -77.0).all())
+
+
 def test_batch_matmul_large_tile_kernel(ct, orc):
     rng = np.random.default_rng(8)
     M, K, N, Bn = 1024, 256, 1024, 4

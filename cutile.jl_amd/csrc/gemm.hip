@@ -23,7 +23,9 @@
 //                    and K are multiples of 8, K >= 256, everything is 16-byte aligned and there are
 //                    at least 16 tiles of 128x128 (ragged edges in M, N and K are handled on the way in).
 //   gemm32           fp32 via v_mfma_f32_32x32x2_f32 (gfx950 has no TF32-class MFMA;
-//                    the reference rounds fp32 operands to TF32, matmul.jl:49-52).
+//                    the reference rounds fp32 operands to TF32, matmul.jl:49-52), 128x128x16 tile,
+//                    any shape; gemm32_big (gemm32_big.hip), the fp32 sibling of gemm16_big, takes
+//                    the problems whose rows are 16-byte aligned (M, K multiples of 4, K >= 128).
 //
 // The (tm, tn, tk) tile constants of the reference only fix the block->data mapping and
 // the L2 swizzle; results do not depend on them, and the physical tiling above is chosen

@@ -186,6 +186,25 @@ def test_batch_matmul_large_tile_kernel(ct, orc):
     assert "big" in ct.last_variant() and torch.equal(C, C2)
 
 
+@pytest.mark.parametrize("T", [torch.float16, torch.float32])
+@pytest.mark.parametrize("M,K,N,Bn", [(1024, 512, 2048, 8), (520, 264, 1001, 3), (2048, 320, 2040, 5), (256, 256, 384, 16)])
+def test_batch_matmul_direct_to_lds_kernels_exact(ct, orc, T, M, K, N, Bn):
+    """Batched problems on the direct-to-LDS kernels (16-bit and fp32): the (tile, batch entry) -> workgroup
+    mapping with batch counts that are and are not multiples of 8, ragged tiles inside every entry, and
+    padded leading dimensions / batch strides (views of wider buffers).  Small-integer operands: exact."""
+    rng = np.random.default_rng(M + Bn)
+    A = rng.integers(-2, 3, (M, K, Bn)).astype(np.float32); B = rng.integers(-2, 3, (K, N, Bn)).astype(np.float32)
+    ref = np.stack([A[:, :, b] @ B[:, :, b] for b in range(Bn)], axis=2)
+    Aw = torch.zeros((Bn, K + 3, M + 16), dtype=T, device="cuda"); Aw[:, :K, :M] = orc.from_julia(A).to(T).cuda()
+    Bw = torch.zeros((Bn, N + 2, K + 8), dtype=T, device="cuda"); Bw[:, :N, :K] = orc.from_julia(B).to(T).cuda()
+    Cw = torch.full((Bn, N + 1, M + 4), -77.0, dtype=torch.float32, device="cuda")
+    C = Cw[:, :N, :M]
+    ct.batch_matmul_kernel(Aw[:, :K, :M], Bw[:, :N, :K], C, 128, 128, 64)
+    assert ct.last_variant().startswith("gemm32_big_" if T == torch.float32 else "gemm16_big_")
+    assert np.array_equal(orc.to_julia(C.contiguous()), ref)
+    assert bool((Cw[:, N:] == -77.0).all()) and bool((Cw[:, :, M:] == -77.0).all())
+
+
 def test_matmul_padded_leading_dims_and_misaligned(ct, orc):
     rng = np.random.default_rng(1)
     M, N, K = 100, 90, 70

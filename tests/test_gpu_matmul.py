@@ -194,7 +194,8 @@ def test_batch_matmul_direct_to_lds_kernels_exact(ct, orc, T, M, K, N, Bn):
     padded leading dimensions / batch strides (views of wider buffers).  Small-integer operands: exact."""
     rng = np.random.default_rng(M + Bn)
     A = rng.integers(-2, 3, (M, K, Bn)).astype(np.float32); B = rng.integers(-2, 3, (K, N, Bn)).astype(np.float32)
-    ref = np.stack([A[:, :, b] @ B[:, :, b] for b in range(Bn)], axis=2)
+    # (contiguous copies: numpy multiplies strided slices without BLAS, minutes at these sizes)
+    ref = np.stack([np.ascontiguousarray(A[:, :, b]) @ np.ascontiguousarray(B[:, :, b]) for b in range(Bn)], axis=2)
     Aw = torch.zeros((Bn, K + 3, M + 16), dtype=T, device="cuda"); Aw[:, :K, :M] = orc.from_julia(A).to(T).cuda()
     Bw = torch.zeros((Bn, N + 2, K + 8), dtype=T, device="cuda"); Bw[:, :N, :K] = orc.from_julia(B).to(T).cuda()
     Cw = torch.full((Bn, N + 1, M + 4), -77.0, dtype=torch.float32, device="cuda")

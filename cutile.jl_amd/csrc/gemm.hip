@@ -371,7 +371,9 @@ int run(const Problem& p, hipStream_t s) {
     }
     const bool f32out = p.out_dtype == MI_F32;
     const int64_t tiles_mid = (int64_t)cld((int64_t)p.M, (int64_t)MT) * cld((int64_t)p.N, (int64_t)MT) * p.batch;
-    // The direct-to-LDS kernel wherever it applies (16-byte aligned rows; it picks its own tile size);
+    // The direct-to-LDS kernel wherever it applies (16-byte aligned rows, K >= 256: with a shorter K the
+    // problem is bound by the stores of C and smaller workgroups in several rounds overlap them better;
+    // it picks its own tile size);
     // the register-staged 128x128 kernel for other shapes whose tiles give at least half the CUs work;
     // the 64x64 kernel for what is left (small problems).
     if (big16_applicable(p) && (force == 3 || force == 0)) {

@@ -24,7 +24,7 @@
 // Requires M and K multiples of 4, K >= 128, 16-byte aligned operands.  Tiles that reach past M or N
 // re-read the last valid rows / chunks on the way in and clip their stores; in the last group of four
 // steps the chunks at k >= K come from a 16-byte block of zeros (both operands).
-#include "gemm_common.h"
+#include "gemm_direct.h"
 
 namespace {
 
@@ -32,15 +32,6 @@ using namespace mi;
 using namespace mi::gemm;
 
 constexpr int BK = 16;
-
-#define SG_MFMA 0x008
-#define SG_VMEM 0x010
-#define SG_DSRD 0x100
-
-__device__ __forceinline__ void gload_lds16(const void* g, void* lds_wave_base) {
-    __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)g,
-                                     (__attribute__((address_space(3))) void*)lds_wave_base, 16, 0, 0);
-}
 
 // Source of every chunk that lies past K.
 __device__ __attribute__((aligned(16))) const unsigned zeros16[4] = {0u, 0u, 0u, 0u};
@@ -115,18 +106,6 @@ __device__ __forceinline__ void interleave() {
         if (NDMA && i % (NM / 4) == 1 && i / (NM / 4) < NDMA) __builtin_amdgcn_sched_group_barrier(SG_VMEM, 1, 0);
     }
     __builtin_amdgcn_sched_barrier(0);
-}
-
-template <int VMCNT>
-__device__ __forceinline__ void stage_barrier() {
-    // My reads of the current stage are done (lgkmcnt(0)) and my transfers into the next stage have
-    // landed (vmcnt leaves only the VMCNT youngest transfers in flight); then meet the other waves.
-    // gfx9 encoding: vmcnt[3:0] | expcnt[6:4] | lgkmcnt[11:8] | vmcnt[15:14].
-    constexpr int imm = (VMCNT & 15) | (7 << 4) | (0 << 8) | ((VMCNT >> 4) << 14);
-    __builtin_amdgcn_s_waitcnt(imm);
-    asm volatile("" ::: "memory");
-    __builtin_amdgcn_s_barrier();
-    asm volatile("" ::: "memory");
 }
 
 // One K step of 16 on stage (AsX, BsX); the next step's data is in (AsY, BsY).
@@ -297,22 +276,6 @@ __global__ __launch_bounds__(256) void gemm32_big(const float* __restrict__ A, i
     }
 }
 
-int64_t tiles_of(const Problem& p, int btm, int btn) {
-    return (int64_t)((p.M + btm - 1) / btm) * ((p.N + btn - 1) / btn) * p.batch;
-}
-
-// Tile size: whichever needs least time by "rounds of workgroups x time of a round" (a round is 256
-// workgroups of 256x256 or 256x128, or 512 of 128x128, two per CU); the relative times of a round
-// are those measured for the 16-bit kernel of the same structure.
-int pick_tile(const Problem& p) {
-    static const int force = [] { const char* e = getenv("MI_GEMM_BIG_TILE"); return e ? atoi(e) : 0; }();   // 44, 42 or 22
-    if (force == 44 || force == 42 || force == 22) return force;
-    const int64_t t44 = tiles_of(p, 256, 256), t42 = tiles_of(p, 256, 128), t22 = tiles_of(p, 128, 128);
-    const int64_t c44 = (t44 + 255) / 256 * 90, c42 = (t42 + 255) / 256 * 50;
-    const int64_t c22 = t22 <= 256 ? 33 : (t22 + 511) / 512 * 60;
-    return c22 <= c42 && c22 <= c44 ? 22 : c42 <= c44 ? 42 : 44;
-}
-
 template <int I, int J>
 void launch(const Problem& p, hipStream_t s) {
     const int tiles_m = (p.M + 64 * I - 1) / (64 * I), tiles_n = (p.N + 64 * J - 1) / (64 * J);
@@ -336,7 +299,7 @@ bool big32_applicable(const Problem& p) {
 }
 
 void big32_launch(const Problem& p, hipStream_t s) {
-    const int t = pick_tile(p);
+    const int t = pick_direct_tile(p);   // (the relative times of a round are those measured for the 16-bit kernel of the same structure)
     if (t == 22) launch<2, 2>(p, s);
     else if (t == 42) launch<4, 2>(p, s);
     else launch<4, 4>(p, s);

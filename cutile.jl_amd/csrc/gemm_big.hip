@@ -30,7 +30,7 @@
 // re-read the last valid rows / chunks on the way in and clip their stores.  K is walked in whole
 // groups of four steps (128); in the last group the 16-byte chunks at k >= K are fetched from a
 // 16-byte block of zeros instead (both operands, so padding never meets a non-finite value).
-#include "gemm_common.h"
+#include "gemm_direct.h"
 
 namespace {
 
@@ -42,15 +42,6 @@ using namespace mi::gemm;
 // LDS, two workgroups per CU) serve problems that would otherwise give too few workgroups to the chip.
 // An A stage of 32 k x (64*I) m moves as 4*I transfers of 1 KB, each 8/I rows of k; a row is 8*I chunks.
 constexpr int BK = 32;
-
-#define SG_MFMA 0x008
-#define SG_VMEM 0x010
-#define SG_DSRD 0x100
-
-__device__ __forceinline__ void gload_lds16(const void* g, void* lds_wave_base) {
-    __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)g,
-                                     (__attribute__((address_space(3))) void*)lds_wave_base, 16, 0, 0);
-}
 
 // Source of every chunk that lies past K.
 __device__ __attribute__((aligned(16))) const unsigned zeros16[4] = {0u, 0u, 0u, 0u};
@@ -144,20 +135,6 @@ __device__ __forceinline__ void interleave16() {
         }
     }
     __builtin_amdgcn_sched_barrier(0);
-}
-
-template <int VMCNT>
-__device__ __forceinline__ void stage_barrier() {
-    // My reads of the current stage are done (lgkmcnt(0)) and my transfers into the next stage
-    // have landed (vmcnt leaves only the VMCNT youngest transfers in flight); then meet the
-    // other waves.  The wait is the builtin, not inline asm, so that the compiler's own
-    // wait-count bookkeeping sees it and does not add a full vmcnt(0) drain before the
-    // following LDS reads.  gfx9 encoding: vmcnt[3:0] | expcnt[6:4] | lgkmcnt[11:8] | vmcnt[15:14].
-    constexpr int imm = (VMCNT & 15) | (7 << 4) | (0 << 8) | ((VMCNT >> 4) << 14);
-    __builtin_amdgcn_s_waitcnt(imm);
-    asm volatile("" ::: "memory");
-    __builtin_amdgcn_s_barrier();
-    asm volatile("" ::: "memory");
 }
 
 // One K step of 32 on stage (AsX, BsX); the next step's data is in (AsY, BsY).
@@ -328,24 +305,6 @@ __global__ __launch_bounds__(256) void gemm16_big(const unsigned short* __restri
     }
 }
 
-int64_t tiles_of(const Problem& p, int btm, int btn) {
-    return (int64_t)((p.M + btm - 1) / btm) * ((p.N + btn - 1) / btn) * p.batch;
-}
-
-// Tile size: whichever needs least time by "rounds of workgroups x time of a round".  Measured time of
-// one K step of a round (us): 256x256 0.63 (a quarter of the CUs busy) to 0.93 (all busy: the clock
-// drops); 256x128 0.42 to 0.51; 128x128 0.33 with one workgroup per CU, 0.58 when CUs hold two.
-// f16 examples (us, 256x256 / 256x128 / 128x128): 1024^3 23 / 15 / 10, 2048^3 40 / 27 / 21,
-// 2560^3 51 / 37 / 46, 4096 x 2048 x 4096 77 / 65 / 74, 3072^3 64 / 83 / 77, 4096^3 119 / 128 / 144.
-int pick_tile(const Problem& p) {
-    static const int force = [] { const char* e = getenv("MI_GEMM_BIG_TILE"); return e ? atoi(e) : 0; }();   // 44, 42 or 22
-    if (force == 44 || force == 42 || force == 22) return force;
-    const int64_t t44 = tiles_of(p, 256, 256), t42 = tiles_of(p, 256, 128), t22 = tiles_of(p, 128, 128);
-    const int64_t c44 = (t44 + 255) / 256 * 90, c42 = (t42 + 255) / 256 * 50;
-    const int64_t c22 = t22 <= 256 ? 33 : (t22 + 511) / 512 * 60;
-    return c22 <= c42 && c22 <= c44 ? 22 : c42 <= c44 ? 42 : 44;
-}
-
 template <typename E, typename OutT, int I, int J>
 void launch(const Problem& p, hipStream_t s) {
     const int tiles_m = (p.M + 64 * I - 1) / (64 * I), tiles_n = (p.N + 64 * J - 1) / (64 * J);
@@ -370,7 +329,7 @@ bool big16_applicable(const Problem& p) {
 
 void big16_launch(const Problem& p, hipStream_t s) {
     const bool f32out = p.out_dtype == MI_F32;
-    const int t = pick_tile(p);
+    const int t = pick_direct_tile(p);
 #define BIG(E, O) (t == 22 ? launch<E, O, 2, 2>(p, s) : t == 42 ? launch<E, O, 4, 2>(p, s) : launch<E, O, 4, 4>(p, s))
     if (p.in_dtype == MI_F16) {
         if (f32out) BIG(F16, float);

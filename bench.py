@@ -3,6 +3,7 @@
 C ABI of libmi355tile.so.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--kernels LIST|all|none] [--no-cpu] [--table]
+    (--kernels gemm_shapes: opt-in sweep of the GEMM entry points over other shapes, not part of 'all')
 
 Prints ONE JSON line on stdout.  A "step" is one pass of the headline workload over one batch
 of synthetic, seeded input already resident in HBM:
@@ -183,6 +184,31 @@ def bench_kernels(ct, which, cpu, nruns=NRUNS, warmup=WARMUP):
             e["cpu_ms"] = round(_cpu_time(lambda: a @ b, repeats=2), 1); e["cpu_note"] = f"numpy/OpenBLAS sgemm on widened inputs, {ncores} threads"
         res["matmul"] = e
         del d
+    if which is not None and "gemm_shapes" in which:
+        # Opt-in (not part of 'all'): the same entry points at other shapes, among them the size lists of the
+        # reference examples' main() (matmul.jl:156-165, batchmatmul.jl:161-169), shapes off the tile grid and
+        # problems with few tiles, where the direct-to-LDS kernels switch to 256x128 / 128x128 tiles.
+        shapes = [("f16", 1, 256, 256, 256), ("f16", 1, 512, 512, 512), ("f16", 1, 1024, 1024, 1024), ("f16", 1, 2048, 2048, 2048),
+                  ("f16", 1, 2560, 2560, 2560), ("f16", 1, 3072, 3072, 3072), ("f16", 1, 4096, 2048, 4096), ("f16", 1, 4000, 4000, 4000),
+                  ("f16", 1, 4096, 4096, 4000), ("f16", 1, 8192, 8192, 8192), ("f16", 4, 512, 1024, 256),
+                  ("f32", 1, 256, 256, 256), ("f32", 1, 512, 512, 512), ("f32", 1, 256, 512, 128), ("f32", 1, 1024, 1024, 1024),
+                  ("f32", 1, 2048, 2048, 2048), ("f32", 1, 4096, 4096, 4096), ("f32", 4, 256, 256, 128), ("f32", 4, 512, 512, 256)]
+        rows = []
+        for (dt, Bt, M, N, K) in shapes:
+            T = torch.float16 if dt == "f16" else torch.float32
+            a = (torch.randn(Bt, K, M, device="cuda") / 8).to(T); b = (torch.randn(Bt, N, K, device="cuda") / 8).to(T)
+            c = torch.empty(Bt, N, M, device="cuda", dtype=torch.float32)
+            if Bt == 1:
+                A, B, C = ct.TileArray(a[0]), ct.TileArray(b[0]), ct.TileArray(c[0])
+                fn = lambda: ct.matmul_kernel(A, B, C, 64, 64, 64)
+            else:
+                A, B, C = ct.TileArray(a), ct.TileArray(b), ct.TileArray(c)
+                fn = lambda: ct.batch_matmul_kernel(A, B, C, 64, 64, 64)
+            e = _entry(f"GEMM {dt} batch {Bt} M={M} N={N} K={K}", fn, 2.0 * Bt * M * N * K, "TFLOPS", "mfma",
+                       2500.0 if dt == "f16" else 157.3, dt, nruns, warmup)
+            e["variant"] = ct.last_variant()
+            rows.append(e)
+        res["gemm_shapes"] = {"name": "GEMM at other shapes (opt-in)", "rows": rows}
     if want("batchmatmul"):
         d = batchmatmul.prepare(benchmark=True)
         A, B, C = ct.TileArray(d.A), ct.TileArray(d.B), ct.TileArray(d.C)
@@ -521,7 +547,8 @@ def main():
         which = None if args.kernels == "all" else set(args.kernels.split(","))
         out["kernels"] = bench_kernels(ct, which, cpu=not args.no_cpu)
     if args.table and "kernels" in out:
-        for k, e in out["kernels"].items():
+        flat = [r for e in out["kernels"].values() for r in e.get("rows", [e])]
+        for e in flat:
             cpu = f"  cpu {e['cpu_ms']:10.1f} ms" if "cpu_ms" in e else ""
             print(f"{e['name'][:72]:<72} min {e['min_ms']:8.4f}  avg {e['avg_ms']:8.4f} ms  "
                   f"{e['achieved']:9.1f} {e['unit']:<8} {100 * e['frac']:6.2f}% of {e['bound']} peak{cpu}", file=sys.stderr)

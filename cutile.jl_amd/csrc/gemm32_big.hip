@@ -7,7 +7,9 @@
 // ring of four LDS stages filled by global_load_lds (16 bytes per lane, no staging registers), the
 // transfers for step s+3 / s+4 issued between the MFMAs of step s, one barrier per step that waits
 // only for the oldest stage in flight.  I = J = 4 is a 256x256 tile (256 accumulator registers, one
-// wave per SIMD); 256x128 and 128x128 serve problems with few tiles.
+// wave per SIMD); 256x128, 128x128 and 64x64 (I = J = 1, 32 KB of LDS) serve problems with few tiles:
+// the fp32 MFMA is slow enough (64 cycles for 32x32x2) that a small problem is bound by the MFMA work
+// of its busiest CU, so the tile that spreads the work over most CUs wins.
 //
 // LDS layouts (per stage):
 //   B tile [64*J n][16 k]: row = 64 bytes = four 16-byte chunks; chunk c of row n sits at position
@@ -98,12 +100,14 @@ __device__ __forceinline__ void mma(const Frag& f, f32x16 (&acc)[I][J]) {
 template <int I, int J, int NDMA, bool FRAGS>
 __device__ __forceinline__ void interleave() {
     constexpr int NM = 4 * I * J, ND = J + 4 * I;
-    static_assert(ND <= NM, "one read per MFMA slot");
+    static_assert(ND <= 2 * NM, "at most two reads per MFMA slot");
 #pragma unroll
     for (int i = 0; i < NM; ++i) {
         __builtin_amdgcn_sched_group_barrier(SG_MFMA, 1, 0);
         if (FRAGS && i < ND) __builtin_amdgcn_sched_group_barrier(SG_DSRD, 1, 0);
-        if (NDMA && i % (NM / 4) == 1 && i / (NM / 4) < NDMA) __builtin_amdgcn_sched_group_barrier(SG_VMEM, 1, 0);
+        if (FRAGS && i + NM < ND) __builtin_amdgcn_sched_group_barrier(SG_DSRD, 1, 0);
+        if (NDMA && NM >= 8 && i % (NM / 4) == 1 && i / (NM / 4) < NDMA) __builtin_amdgcn_sched_group_barrier(SG_VMEM, 1, 0);
+        if (NDMA && NM < 8 && i < NDMA) __builtin_amdgcn_sched_group_barrier(SG_VMEM, 1, 0);
     }
     __builtin_amdgcn_sched_barrier(0);
 }
@@ -294,16 +298,34 @@ bool big32_applicable(const Problem& p) {
     // M and K multiples of 4 (A and B move in 16-byte chunks along m and k), any N
     return p.M % 4 == 0 && p.M >= 4 && p.N >= 1 && p.K % 4 == 0 && p.K >= 128 && aligned(p.A, 16) && aligned(p.B, 16) &&
            p.lda % 4 == 0 && p.ldb % 4 == 0 && p.sa % 4 == 0 && p.sb % 4 == 0 && p.ldc < (1 << 26) &&
-           p.lda < (1 << 26) && p.ldb < (1 << 26) && tiles_of(p, 128, 128) >= 16 &&
-           tiles_of(p, 128, 128) < (1 << 30);
+           p.lda < (1 << 26) && p.ldb < (1 << 26) && tiles_of(p, 64, 64) >= 16 &&
+           tiles_of(p, 64, 64) < (1 << 30);
+}
+
+// Tile size for fp32.  The kernel is bound by MFMA time, so a candidate costs (rounds of 256 workgroups)
+// x (MFMAs per wave and step, I*J); co-resident workgroups of the small tiles simply add up.  The
+// smallest tile moves four times the bytes per flop of 128x128 through L2, so it is only taken when it
+// at least halves that cost (1024^3: 64 tiles of 128x128 take 63 us).  Ties go to the larger tile.
+int pick_tile32(const Problem& p) {
+    static const int force = [] { const char* e = getenv("MI_GEMM_BIG_TILE"); return e ? atoi(e) : 0; }();   // 44, 42, 22 or 11
+    if (force == 44 || force == 42 || force == 22 || force == 11) return force;
+    auto rounds = [&](int btm, int btn) { return (tiles_of(p, btm, btn) + 255) / 256; };
+    const int64_t c44 = rounds(256, 256) * 16, c42 = rounds(256, 128) * 8, c22 = rounds(128, 128) * 4, c11 = rounds(64, 64);
+    const int64_t best = c44 <= c42 && c44 <= c22 ? c44 : c42 <= c22 ? c42 : c22;
+    if (2 * c11 <= best) return 11;
+    return best == c44 ? 44 : best == c42 ? 42 : 22;
 }
 
 void big32_launch(const Problem& p, hipStream_t s) {
-    const int t = pick_direct_tile(p);   // (the relative times of a round are those measured for the 16-bit kernel of the same structure)
-    if (t == 22) launch<2, 2>(p, s);
+    const int t = pick_tile32(p);
+    if (t == 11) launch<1, 1>(p, s);
+    else if (t == 22) launch<2, 2>(p, s);
     else if (t == 42) launch<4, 2>(p, s);
     else launch<4, 4>(p, s);
-    set_variant(t == 22 ? "gemm32_big_128x128x16_ring4" : t == 42 ? "gemm32_big_256x128x16_ring4" : "gemm32_big_256x256x16_ring4");
+    set_variant(t == 11   ? "gemm32_big_64x64x16_ring4"
+                : t == 22 ? "gemm32_big_128x128x16_ring4"
+                : t == 42 ? "gemm32_big_256x128x16_ring4"
+                          : "gemm32_big_256x256x16_ring4");
 }
 
 }  // namespace gemm

@@ -151,8 +151,9 @@ def test_matmul_direct_to_lds_kernel_shape_sweep(ct, orc):
 
 
 @pytest.mark.parametrize("M,N,K,tile", [(2040, 2000, 256, "128x128"), (2056, 2311, 388, "256x128"), (4000, 4001, 132, "256x256"),
-                                         (4, 16385, 128, "128x128"), (3072, 3081, 196, "256x256"), (1096, 1001, 1060, "128x128"),
-                                         (2048, 2304, 376, "256x128"), (512, 512, 128, "128x128"), (4096, 4096, 320, "256x256")])
+                                         (4, 16385, 128, "64x64"), (3072, 3081, 196, "128x128"), (1096, 1001, 1060, "64x64"),
+                                         (2048, 2304, 376, "256x128"), (512, 512, 128, "64x64"), (4096, 4096, 320, "256x256"),
+                                         (260, 250, 132, "64x64")])
 def test_matmul_f32_direct_to_lds_kernel_exact(ct, orc, M, N, K, tile):
     """The fp32 direct-to-LDS kernel in each tile size: M and K multiples of 4 off the tile / 64 grid, any
     N.  Small-integer operands make every fp32 sum exact; A and B are views of buffers whose cells past K

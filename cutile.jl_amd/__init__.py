@@ -26,7 +26,7 @@ MI_MAX_RANK = 4
 # error codes of include/mi355tile.h
 MI_OK = 0
 MI_E_NULL, MI_E_DTYPE, MI_E_RANK, MI_E_SHAPE, MI_E_STRIDE = -1, -2, -3, -4, -5
-MI_E_TILE, MI_E_GRID, MI_E_ALIGN, MI_E_ARG, MI_E_UNSUPPORTED = -6, -7, -8, -9, -10
+MI_E_TILE, MI_E_GRID, MI_E_ALIGN, MI_E_ARG, MI_E_UNSUPPORTED, MI_E_SCRATCH = -6, -7, -8, -9, -10, -11
 
 
 class MiTileArray(ctypes.Structure):
@@ -66,6 +66,7 @@ _SIGNATURES = {
     "mi_layer_norm_fwd": ([_A, _A, _A, _A, _A, _A, ctypes.c_float, _i, _vp], _i),
     "mi_layer_norm_bwd_dx_partial_dwdb": ([_A] * 9 + [_i, _i, _vp], _i),
     "mi_layer_norm_bwd_dwdb": ([_A, _A, _A, _A, _i, _i, _vp], _i),
+    "mi_layer_norm_bwd_static": ([_A] * 8 + [_i, _i, _i, _vp], _i),
     "mi_softmax_tma_kernel": ([_A, _A, _i, _i, _vp], _i),
     "mi_softmax_chunked_kernel": ([_A, _A, _i, _i, _i, _vp], _i),
     "mi_fmha_kernel": ([_A, _A, _A, _A, ctypes.c_float, ctypes.c_int32, _i, _i, _i, _i, _i, _i, _i, _vp], _i),
@@ -250,6 +251,14 @@ def layer_norm_bwd_dwdb(DW, DB, FINAL_DW, FINAL_DB, TILE_M: int, TILE_N: int, st
     """examples/layernorm.jl:186-205"""
     _call("mi_layer_norm_bwd_dwdb", _ref(DW), _ref(DB), _ref(FINAL_DW), _ref(FINAL_DB), TILE_M,
           TILE_N, _stream(stream))
+
+
+def layer_norm_bwd_static(DX, DY, X, W, Mean, Rstd, FINAL_DW, FINAL_DB, GROUP_SIZE_M: int, TILE_M: int,
+                          TILE_N: int, stream=None):
+    """The whole backward of examples/layernorm.jl:245-251 in one call that allocates nothing: the
+    partial slots live in the library's static scratch (MiError with MI_E_SCRATCH beyond its size)."""
+    _call("mi_layer_norm_bwd_static", _ref(DX), _ref(DY), _ref(X), _ref(W), _ref(Mean), _ref(Rstd),
+          _ref(FINAL_DW), _ref(FINAL_DB), GROUP_SIZE_M, TILE_M, TILE_N, _stream(stream))
 
 
 def softmax_tma_kernel(output, input, TILE_SIZE: int, num_programs: int | None = None, stream=None):

@@ -29,6 +29,7 @@ extern "C" const char* mi_strerror(int code) {
         case MI_E_ALIGN: return "pointer is not aligned to its element size";
         case MI_E_ARG: return "invalid scalar argument";
         case MI_E_UNSUPPORTED: return "configuration not supported";
+        case MI_E_SCRATCH: return "problem exceeds the library's static scratch buffer";
         default: break;
     }
     if (code > 0) return hipGetErrorString((hipError_t)code);

@@ -468,6 +468,44 @@ __global__ __launch_bounds__(1024) void ln_dwdb_kernel(const float* __restrict__
     }
 }
 
+// ---- static scratch of the allocation-free backward ---------------------------------------
+// Partial dW / dB slots of mi_layer_norm_bwd_static: kScratchFloats floats for DW followed by as many
+// for DB (4 MiB in all).  Host code never uses the array's name as an address: the device address
+// is looked up once per device (scratch_ptr) and passed to the kernels like any other buffer.
+constexpr int64_t kScratchFloats = 512 * 1024;
+static __device__ __align__(256) float scratch[2 * kScratchFloats];
+
+constexpr int kMaxDevices = 64;
+float* g_scratch_ptr[kMaxDevices];
+bool g_scratch_known[kMaxDevices];
+
+// Device address of `scratch` on the current device; positive hipError_t on failure.
+int scratch_ptr(float** out) {
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return (int)e;
+    if (dev < 0 || dev >= kMaxDevices) return MI_E_UNSUPPORTED;
+    if (!__atomic_load_n(&g_scratch_known[dev], __ATOMIC_ACQUIRE)) {
+        float* p = nullptr;
+        e = hipGetSymbolAddress((void**)&p, HIP_SYMBOL(scratch));
+        if (e != hipSuccess) return (int)e;
+        if (!p) return MI_E_NULL;
+        g_scratch_ptr[dev] = p;   // every thread that gets here stores the same address
+        __atomic_store_n(&g_scratch_known[dev], true, __ATOMIC_RELEASE);
+    }
+    *out = g_scratch_ptr[dev];
+    return MI_OK;
+}
+
+// Zero fill as a kernel (a memset node would not survive stream capture and replay on this runtime).
+__global__ __launch_bounds__(256) void fill_zero_kernel(f32x4* __restrict__ a, f32x4* __restrict__ b, int64_t nvec) {
+    const f32x4 z = {0.f, 0.f, 0.f, 0.f};
+    for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < nvec; i += (int64_t)gridDim.x * 256) {
+        a[i] = z;
+        b[i] = z;
+    }
+}
+
 int check_f32(const mi_tile_array* a, int ndim) {
     MI_CHECK(check_array(a, ndim));
     if (a->dtype != MI_F32) return MI_E_DTYPE;
@@ -683,4 +721,46 @@ extern "C" int mi_layer_norm_bwd_dwdb(const mi_tile_array* DW, const mi_tile_arr
                        (float*)FINAL_DB->ptr, N, (int)G);
     set_variant("ln_dwdb_b1024");
     return launch_status();
+}
+
+// Backward in one call with the partial slots in the library's static scratch: zero fill,
+// layer_norm_bwd_dx_partial_dwdb, layer_norm_bwd_dwdb (layernorm.jl:245-251 issues the same three
+// steps on buffers its caller allocated, layernorm.jl:226-228).  Calls nothing that allocates.
+extern "C" int mi_layer_norm_bwd_static(const mi_tile_array* DX, const mi_tile_array* DY,
+                                        const mi_tile_array* X, const mi_tile_array* W,
+                                        const mi_tile_array* Mean, const mi_tile_array* Rstd,
+                                        const mi_tile_array* FINAL_DW, const mi_tile_array* FINAL_DB,
+                                        int GROUP_SIZE_M, int TILE_M, int TILE_N, void* stream) {
+    MI_CHECK(check_f32(X, 2));
+    MI_CHECK(check_f32(FINAL_DW, 1));
+    MI_CHECK(check_f32(FINAL_DB, 1));
+    if (GROUP_SIZE_M < 1) return MI_E_ARG;
+    const int64_t N = X->sizes[0], G = GROUP_SIZE_M;
+    if (FINAL_DW->sizes[0] != N || FINAL_DB->sizes[0] != N) return MI_E_SHAPE;
+    // rows of the slot matrices are padded to whole 16-byte vectors
+    const int64_t ld = (N + 3) / 4 * 4;
+    if (ld * G > kScratchFloats) return MI_E_SCRATCH;
+    float* base = nullptr;
+    MI_CHECK(scratch_ptr(&base));
+    mi_tile_array dw = {}, db = {};
+    dw.ptr = base;
+    db.ptr = base + kScratchFloats;
+    for (mi_tile_array* a : {&dw, &db}) {
+        a->dtype = MI_F32;
+        a->ndim = 2;
+        a->sizes[0] = N;
+        a->sizes[1] = G;
+        a->strides[0] = 1;
+        a->strides[1] = ld;
+    }
+    if (N > 0) {
+        const int64_t nvec = ld * G / 4;
+        const unsigned blocks = (unsigned)(nvec < 256 * 1024 ? cld(nvec, (int64_t)256) : 1024);
+        hipLaunchKernelGGL(fill_zero_kernel, dim3(blocks), dim3(256), 0, (hipStream_t)stream,
+                           (f32x4*)dw.ptr, (f32x4*)db.ptr, nvec);
+        MI_CHECK(launch_status());
+    }
+    MI_CHECK(mi_layer_norm_bwd_dx_partial_dwdb(DX, DY, &dw, &db, X, W, Mean, Rstd, nullptr, GROUP_SIZE_M,
+                                               TILE_N, stream));
+    return mi_layer_norm_bwd_dwdb(&dw, &db, FINAL_DW, FINAL_DB, TILE_M, TILE_N, stream);
 }

@@ -178,6 +178,20 @@ function layer_norm_bwd_dwdb(DW, DB, FINAL_DW, FINAL_DB, TILE_M::Integer, TILE_N
         d[1], d[2], d[3], d[4], TILE_M, TILE_N, stream))
 end
 
+# The whole backward (zero fill of the partials, layer_norm_bwd_dx_partial_dwdb, layer_norm_bwd_dwdb:
+# layernorm.jl:245-251) in one call that allocates nothing: the partial slots live in a static device
+# array of the library (N rounded up to a multiple of 4, times GROUP_SIZE_M, at most 524288 floats).
+# For callers that can not allocate; calls that overlap on one GPU share the array and race.
+function layer_norm_bwd_static(DX, DY, X, W, Mean, Rstd, FINAL_DW, FINAL_DB, GROUP_SIZE_M::Integer,
+                               TILE_M::Integer, TILE_N::Integer; stream::Ptr{Cvoid}=C_NULL)
+    d = map(a -> ref(descriptor(a)), (DX, DY, X, W, Mean, Rstd, FINAL_DW, FINAL_DB))
+    GC.@preserve DX DY X W Mean Rstd FINAL_DW FINAL_DB check(ccall(
+        (:mi_layer_norm_bwd_static, libmi355tile), Cint,
+        (Ref{MiTileArray}, Ref{MiTileArray}, Ref{MiTileArray}, Ref{MiTileArray}, Ref{MiTileArray},
+         Ref{MiTileArray}, Ref{MiTileArray}, Ref{MiTileArray}, Cint, Cint, Cint, Ptr{Cvoid}),
+        d[1], d[2], d[3], d[4], d[5], d[6], d[7], d[8], GROUP_SIZE_M, TILE_M, TILE_N, stream))
+end
+
 # ---- examples/softmax.jl ------------------------------------------------------------------
 
 function softmax_tma_kernel(output, input, TILE_SIZE::Integer; blocks::Integer=size(input, 2),

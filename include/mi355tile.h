@@ -63,7 +63,8 @@ enum {
     MI_E_GRID = -7,      /* a grid dimension exceeds 2^24-1 (reference: src/launch.jl:743,801-807) */
     MI_E_ALIGN = -8,     /* pointer not aligned to its element size */
     MI_E_ARG = -9,       /* other invalid scalar argument */
-    MI_E_UNSUPPORTED = -10
+    MI_E_UNSUPPORTED = -10,
+    MI_E_SCRATCH = -11   /* the problem needs more scratch memory than the library's static buffer holds */
 };
 
 #define MI_MAX_RANK 4
@@ -143,6 +144,20 @@ int mi_layer_norm_bwd_dx_partial_dwdb(const mi_tile_array* DX, const mi_tile_arr
 int mi_layer_norm_bwd_dwdb(const mi_tile_array* DW, const mi_tile_array* DB,
                            const mi_tile_array* FINAL_DW, const mi_tile_array* FINAL_DB,
                            int TILE_M, int TILE_N, void* stream);
+
+/* Whole backward in one call that allocates nothing.  No counterpart in the reference, whose host
+ * code allocates the partial buffers itself (layernorm.jl:226-228); for callers that can not
+ * allocate: code under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc.
+ * Same result as zero-filling DW / DB (N, GROUP_SIZE_M), mi_layer_norm_bwd_dx_partial_dwdb and
+ * mi_layer_norm_bwd_dwdb, with the partial slots held in a file-scope device array of the library
+ * (4 MiB per GPU, kept until the process ends).  Limit: cld(N,4)*4 * GROUP_SIZE_M <= 524288 floats
+ * (N = 8192 with 64 slots), MI_E_SCRATCH beyond.  Every call on a GPU uses that GPU's one array:
+ * calls that overlap on one GPU (different streams or threads) race. */
+int mi_layer_norm_bwd_static(const mi_tile_array* DX, const mi_tile_array* DY, const mi_tile_array* X,
+                             const mi_tile_array* W, const mi_tile_array* Mean,
+                             const mi_tile_array* Rstd, const mi_tile_array* FINAL_DW,
+                             const mi_tile_array* FINAL_DB, int GROUP_SIZE_M, int TILE_M, int TILE_N,
+                             void* stream);
 
 /* ---- softmax: examples/softmax.jl -------------------------------------------------- */
 /* softmax_tma_kernel (softmax.jl:18-42): column softmax of input (N,M), one tile of

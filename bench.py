@@ -184,6 +184,18 @@ def bench_kernels(ct, which, cpu, nruns=NRUNS, warmup=WARMUP):
             e["cpu_ms"] = round(_cpu_time(lambda: a @ b, repeats=2), 1); e["cpu_note"] = f"numpy/OpenBLAS sgemm on widened inputs, {ncores} threads"
         res["matmul"] = e
         del d
+    if want("matmul_fp8"):
+        # fp8 x fp8 operands (ext/DLFP8TypesExt.jl:15-19): the same 4096^3 problem on the fp8 matrix cores
+        g = torch.Generator().manual_seed(6)
+        for key, T8, nm in (("matmul_fp8", torch.float8_e4m3fn, "e4m3fn"), ("matmul_fp8_e5m2", torch.float8_e5m2, "e5m2")):
+            a8 = torch.randn(4096, 4096, generator=g).to(T8).cuda(); b8 = torch.randn(4096, 4096, generator=g).to(T8).cuda()
+            c8 = torch.empty(4096, 4096, device="cuda")
+            A, B, C = ct.TileArray(a8), ct.TileArray(b8), ct.TileArray(c8)
+            e = _entry(f"GEMM 4096^3 {nm} x {nm} -> f32 (inputs ~ N(0,1) rounded to fp8)", lambda: ct.matmul_kernel(A, B, C, 64, 64, 64),
+                       2.0 * 4096 ** 3, "TFLOPS", "mfma", 5000.0, "fp8", nruns, warmup)
+            e["variant"] = ct.last_variant()
+            res[key] = e
+            del a8, b8, c8
     if which is not None and "gemm_shapes" in which:
         # Opt-in (not part of 'all'): the same entry points at other shapes, among them the size lists of the
         # reference examples' main() (matmul.jl:156-165, batchmatmul.jl:161-169), shapes off the tile grid and

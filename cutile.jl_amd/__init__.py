@@ -20,7 +20,7 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 # MI355TILE_LIB selects another build of the same library (e.g. an experimental variant).
 LIB_PATH = os.environ.get("MI355TILE_LIB") or os.path.join(_HERE, "libmi355tile.so")
 
-MI_F32, MI_F64, MI_F16, MI_BF16, MI_F8E4M3FN, MI_I32, MI_I64, MI_BOOL, MI_I8, MI_I16 = range(10)
+MI_F32, MI_F64, MI_F16, MI_BF16, MI_F8E4M3FN, MI_I32, MI_I64, MI_BOOL, MI_I8, MI_I16, MI_F8E5M2 = range(11)
 MI_MAX_RANK = 4
 
 # error codes of include/mi355tile.h
@@ -131,7 +131,7 @@ def _dtype_code(t) -> int:
     table = {
         torch.float32: MI_F32, torch.float64: MI_F64, torch.float16: MI_F16,
         torch.bfloat16: MI_BF16, torch.int32: MI_I32, torch.int64: MI_I64,
-        torch.float8_e4m3fn: MI_F8E4M3FN,
+        torch.float8_e4m3fn: MI_F8E4M3FN, torch.float8_e5m2: MI_F8E5M2,
     }
     try:
         return table[t]

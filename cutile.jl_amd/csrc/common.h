@@ -21,6 +21,7 @@ static inline int dtype_size(int dt) {
         case MI_F16: return 2;
         case MI_BF16: return 2;
         case MI_F8E4M3FN: return 1;
+        case MI_F8E5M2: return 1;
         case MI_I32: return 4;
         case MI_I64: return 8;
         default: return 0;

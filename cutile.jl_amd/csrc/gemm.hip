@@ -305,8 +305,13 @@ int validate(const mi_tile_array* A, const mi_tile_array* B, const mi_tile_array
     MI_CHECK(check_array(B, ndim));
     MI_CHECK(check_array(C, ndim));
     if (A->dtype != B->dtype) return MI_E_DTYPE;
-    if (A->dtype != MI_F16 && A->dtype != MI_BF16 && A->dtype != MI_F32) return MI_E_DTYPE;
-    if (C->dtype != A->dtype && C->dtype != MI_F32) return MI_E_DTYPE;
+    const bool fp8 = A->dtype == MI_F8E4M3FN || A->dtype == MI_F8E5M2;
+    if (A->dtype != MI_F16 && A->dtype != MI_BF16 && A->dtype != MI_F32 && !fp8) return MI_E_DTYPE;
+    // fp8 operands accumulate in fp32 and store f32, f16 or bf16 (the accumulator types the reference
+    // allows are f16 and f32: ext/DLFP8TypesExt.jl:15-19)
+    if (fp8 ? (C->dtype != MI_F32 && C->dtype != MI_F16 && C->dtype != MI_BF16)
+            : (C->dtype != A->dtype && C->dtype != MI_F32))
+        return MI_E_DTYPE;
     if (!is_pow2(tm) || !is_pow2(tn) || !is_pow2(tk)) return MI_E_TILE;
     const int64_t M = A->sizes[0], K = A->sizes[1], N = B->sizes[1];
     if (B->sizes[0] != K || C->sizes[0] != M || C->sizes[1] != N) return MI_E_SHAPE;
@@ -355,6 +360,10 @@ void launch_generic16(const Problem& p, hipStream_t s) {
 int run(const Problem& p, hipStream_t s) {
     if (p.M == 0 || p.N == 0 || p.batch == 0) return MI_OK;
     static const int force = [] { const char* e = getenv("MI_GEMM_KERNEL"); return e ? atoi(e) : 0; }();   // 1 generic, 2 mid, 3 big
+    if (p.in_dtype == MI_F8E4M3FN || p.in_dtype == MI_F8E5M2) {
+        fp8_launch(p, s);
+        return launch_status();
+    }
     if (p.in_dtype == MI_F32) {
         if (big32_applicable(p) && force != 1) {   // 16-byte aligned rows: the direct-to-LDS kernel
             big32_launch(p, s);

@@ -298,6 +298,8 @@ bool big32_applicable(const Problem& p) {
     // M and K multiples of 4 (A and B move in 16-byte chunks along m and k), any N
     return p.M % 4 == 0 && p.M >= 4 && p.N >= 1 && p.K % 4 == 0 && p.K >= 128 && aligned(p.A, 16) && aligned(p.B, 16) &&
            p.lda % 4 == 0 && p.ldb % 4 == 0 && p.sa % 4 == 0 && p.sb % 4 == 0 && p.ldc < (1 << 26) &&
+           // (the kernel's 32-bit lane offsets assume rows that follow each other upwards in memory)
+           p.lda >= p.M && p.ldb >= p.K && p.ldc >= p.M && p.sa >= 0 && p.sb >= 0 && p.sc >= 0 &&
            p.lda < (1 << 26) && p.ldb < (1 << 26) && tiles_of(p, 64, 64) >= 16 &&
            tiles_of(p, 64, 64) < (1 << 30);
 }

@@ -324,6 +324,8 @@ bool big16_applicable(const Problem& p) {
     const int64_t tiles = tiles_of(p, 128, 128);   // (from 16 tiles of 128x128 on, this kernel is no slower than 64x64 tiles)
     return p.M % 8 == 0 && p.M >= 8 && p.N >= 1 && p.K % 8 == 0 && p.K >= 256 && aligned(p.A, 16) && aligned(p.B, 16) &&
            p.lda % 8 == 0 && p.ldb % 8 == 0 && p.sa % 8 == 0 && p.sb % 8 == 0 && p.ldc < (1 << 26) &&
+           // (the kernel's 32-bit lane offsets assume rows that follow each other upwards in memory)
+           p.lda >= p.M && p.ldb >= p.K && p.ldc >= p.M && p.sa >= 0 && p.sb >= 0 && p.sc >= 0 &&
            p.lda < (1 << 26) && p.ldb < (1 << 26) && tiles >= 16 && tiles < (1 << 30);
 }
 

@@ -80,6 +80,8 @@ void big16_launch(const Problem& p, hipStream_t s);
 // gemm32_big.hip: the same for fp32 operands.
 bool big32_applicable(const Problem& p);
 void big32_launch(const Problem& p, hipStream_t s);
+// gemm8.hip: fp8 (E4M3FN / E5M2) operands; picks its kernel itself.
+void fp8_launch(const Problem& p, hipStream_t s);
 
 }  // namespace gemm
 }  // namespace mi

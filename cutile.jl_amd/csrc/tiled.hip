@@ -116,7 +116,7 @@ void set_variant_text(const char* text) {
     set_variant(keep.c_str());
 }
 
-int tiled_dtype_size(int dt) { return dt == MI_BOOL ? 1 : (dt == MI_F8E4M3FN ? 0 : dtype_size(dt)); }
+int tiled_dtype_size(int dt) { return dt == MI_BOOL ? 1 : (dt == MI_F8E4M3FN || dt == MI_F8E5M2 ? 0 : dtype_size(dt)); }
 
 // Arrays of this API: 0 to 4 dimensions, any element strides, pointer aligned to the element.
 int check_tiled(const mi_tile_array* a) {

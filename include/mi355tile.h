@@ -48,7 +48,9 @@ typedef enum mi_dtype {
     MI_I64 = 6,
     MI_BOOL = 7,     /* Julia Bool: one byte holding 0 or 1 (Tiled broadcast / mapreduce only) */
     MI_I8 = 8,       /* Int8 / UInt8 and */
-    MI_I16 = 9       /* Int16 / UInt16: RNG fills only (unsigned types share the codes of the signed ones) */
+    MI_I16 = 9,      /* Int16 / UInt16: RNG fills only (unsigned types share the codes of the signed ones) */
+    MI_F8E5M2 = 10   /* OCP FP8 E5M2: bias 15, Inf and NaN as in IEEE (reference: ext/DLFP8TypesExt.jl:11-13);
+                        matmul operands only */
 } mi_dtype;
 
 /* Error codes (negative).  Positive return values are hipError_t. */
@@ -110,7 +112,10 @@ int mi_transpose_kernel(const mi_tile_array* x, const mi_tile_array* y, int tm, 
  * cld(M,tm)*cld(N,tn) blocks ordered by swizzle_2d with GROUP_SIZE_M = 8, ragged edges
  * zero-padded on load and clipped on store.  A,B: f16 / bf16 / f32; C: the input type or
  * f32.  f32 inputs are multiplied in true fp32 (gfx950 has no TF32-class MFMA; the
- * reference rounds f32 operands to TF32 at matmul.jl:49-52). */
+ * reference rounds f32 operands to TF32 at matmul.jl:49-52).  A,B both MI_F8E4M3FN or both
+ * MI_F8E5M2 (the reference's fp8 mma operands, ext/DLFP8TypesExt.jl:15-19; lhs and rhs must share
+ * the type, src/compiler/intrinsics/core.jl:589-604): multiplied on the fp8 matrix cores with fp32
+ * accumulation, C f32, f16 or bf16. */
 int mi_matmul_kernel(const mi_tile_array* A, const mi_tile_array* B, const mi_tile_array* C,
                      int tm, int tn, int tk, void* stream);
 /* batch_matmul_kernel (batchmatmul.jl:15-56): C(M,N,b) = A(M,K,b)·B(K,N,b), grid

@@ -38,6 +38,10 @@ philox2x32, rng_fill   Random123's published known-answer vectors for philox2x32
                        (test/device/random.jl:421-526: uniqueness, disjoint streams, counter carry)
 e4m3fn codec           16 round-trip vectors and fma vectors of
                        test/extensions/DLFP8Types.jl:126-141; all 256 codes vs torch.float8_e4m3fn
+e5m2 codec             the same 16 round-trip vectors (DLFP8Types.jl:126-134); all 256 codes and
+                       RNE encoding vs torch.float8_e5m2
+fp8_matmul             the exact mma case of test/extensions/DLFP8Types.jl:143-152 (operands in
+                       {0, 0.5, 1}: integer arithmetic by hand); float64 ``@`` on decoded operands
 =====================  ======================================================================
 
 The reference's device rounding (fma contraction, exp2 / reciprocal approximations, f16
@@ -340,6 +344,53 @@ def e4m3fn_encode(x: np.ndarray) -> np.ndarray:
     code = np.where(overflow | nan, 0x7F, code)
     out = (code.astype(np.uint8) | sign).astype(np.uint8)
     return out
+
+
+def e5m2_decode(code: np.ndarray) -> np.ndarray:
+    """OCP FP8 E5M2 -> float32: 1 sign, 5 exponent (bias 15), 2 mantissa bits; IEEE-style Inf
+    (S.11111.00) and NaN; exponent 0 is subnormal (2^-14 * m/4); max finite 57344.  The type the
+    reference maps ``Float8_E5M2`` to (ext/DLFP8TypesExt.jl:11-13)."""
+    c = np.asarray(code, dtype=np.uint8).astype(np.int32)
+    s = np.where(c & 0x80, -1.0, 1.0)
+    e = (c >> 2) & 0x1F
+    m = c & 0x3
+    val = np.where(e == 0, (m / 4.0) * 2.0 ** -14, (1.0 + m / 4.0) * np.exp2((e - 15).astype(np.float64)))
+    val = np.where(e == 31, np.where(m == 0, np.inf, np.nan), val)
+    return (s * val).astype(np.float32)
+
+
+def e5m2_encode(x: np.ndarray) -> np.ndarray:
+    """float -> E5M2 code, round to nearest even (src/compiler/intrinsics/conversions.jl:197);
+    values that round past the largest finite magnitude become Inf, as in IEEE formats."""
+    x = np.asarray(x, dtype=np.float64)
+    sign = (np.signbit(x)).astype(np.uint8) << 7
+    a = np.abs(x)
+    nan = np.isnan(a)
+    inf = np.isinf(a)
+    fin = np.where(nan | inf, 0.0, a)
+    with np.errstate(divide="ignore", invalid="ignore"):
+        e = np.floor(np.log2(np.where(fin > 0, fin, 1.0)))
+    e = np.clip(e, -14, 15)
+    quantum = np.exp2(e - 2)
+    val = np.rint(fin / quantum) * quantum
+    with np.errstate(divide="ignore", invalid="ignore"):
+        e2 = np.floor(np.log2(np.where(val > 0, val, 1.0)))
+    e2 = np.clip(e2, -14, 16)
+    is_sub = val < 2.0 ** -14
+    mant = np.where(is_sub, np.rint(val / 2.0 ** -16), np.rint(val / np.exp2(e2 - 2)) - 4)
+    expf = np.where(is_sub, 0, e2 + 15)
+    code = (expf.astype(np.int64) << 2) | mant.astype(np.int64)
+    code = np.where(inf | (val > 57344.0), 0x7C, code)
+    code = np.where(nan, 0x7F, code)
+    return (code.astype(np.uint8) | sign).astype(np.uint8)
+
+
+def fp8_matmul(A_codes: np.ndarray, B_codes: np.ndarray, fmt: str = "e4m3fn", dtype=np.float64) -> np.ndarray:
+    """``mma`` of fp8 operands (ext/DLFP8TypesExt.jl:15-19 allows them; the product is defined on
+    the decoded values, test/extensions/DLFP8Types.jl:143-152: ``Float32.(a) * Float32.(b)``).
+    A_codes (M, K) and B_codes (K, N) uint8, Julia shapes; (M, N) float64 out."""
+    dec = e4m3fn_decode if fmt == "e4m3fn" else e5m2_decode
+    return dec(A_codes).astype(dtype) @ dec(B_codes).astype(dtype)
 
 
 def quantize_e4m3fn_per_channel(w: np.ndarray):

@@ -7,6 +7,10 @@ Tolerances (stated against a float64 evaluation of ``A*B`` on the same inputs):
   fp32 inputs : |err| <= 1e-5 * (|ref| + max|ref|)       (true fp32 MFMA, fp32 accumulate)
   f16 / bf16  : |err| <= 2e-2 * (|ref| + max|ref|) when C is f32; the same plus one output
                 rounding (2^-11 / 2^-8 relative) when C is stored in the input type.
+  fp8 (E4M3FN / E5M2 operands, ext/DLFP8TypesExt.jl:15-19): the reference compares with ``==``
+                against ``Float32.(a) * Float32.(b)`` on exactly representable operands
+                (test/extensions/DLFP8Types.jl:143-152), and so do the tests here (products and fp32
+                sums are exact); random operands: 2e-2 as above against float64 on the decoded values.
 """
 import numpy as np
 import pytest
@@ -261,3 +265,151 @@ def test_batch_matmul_full_size_f32(orc):
     for b in (0, 7):
         ref = A[:, :, b].astype(np.float64) @ B[:, :, b].astype(np.float64)
         check(C[:, :, b], ref, 1e-5)
+
+
+# ---- fp8 operands ---------------------------------------------------------------------------------
+
+FP8 = {"e4m3fn": torch.float8_e4m3fn, "e5m2": torch.float8_e5m2}
+
+
+def fp8_tensor(orc, vals, fmt):
+    """Exactly representable values (numpy, Julia shape) -> (device tensor of the fp8 type, codes)."""
+    codes = (orc.e4m3fn_encode if fmt == "e4m3fn" else orc.e5m2_encode)(vals)
+    dec = (orc.e4m3fn_decode if fmt == "e4m3fn" else orc.e5m2_decode)(codes)
+    assert np.array_equal(dec, vals.astype(np.float32))
+    return orc.from_julia(codes).view(FP8[fmt]).cuda(), codes
+
+
+@pytest.mark.parametrize("fmt", ["e4m3fn", "e5m2"])
+@pytest.mark.parametrize("acc", [torch.float32, torch.float16])
+def test_matmul_fp8_reference_exact_case(ct, orc, fmt, acc):
+    """test/extensions/DLFP8Types.jl:143-152: 16 x 16 operands drawn from {0, 0.5, 1}, result compared
+    with ``==``, for both accumulator / result types the reference allows."""
+    rng = np.random.default_rng(3)
+    A = rng.integers(0, 3, (16, 16)) / 2.0; B = rng.integers(0, 3, (16, 16)) / 2.0
+    At, Ac = fp8_tensor(orc, A, fmt); Bt, Bc = fp8_tensor(orc, B, fmt)
+    C = torch.full((16, 16), -1.0, dtype=acc, device="cuda")
+    ct.matmul_kernel(At, Bt, C, 16, 16, 16)
+    assert ct.last_variant() == "gemm8_generic_64x64x64"
+    assert np.array_equal(orc.to_julia(C).astype(np.float64), orc.fp8_matmul(Ac, Bc, fmt))
+
+
+@pytest.mark.parametrize("fmt", ["e4m3fn", "e5m2"])
+@pytest.mark.parametrize("M,N,K", [(200, 100, 300), (33, 17, 41), (64, 64, 16), (1, 1, 1), (129, 65, 33), (5, 700, 9),
+                                   (512, 256, 1024), (256, 256, 64)])
+def test_matmul_fp8_generic_kernel_exact(ct, orc, fmt, M, N, K):
+    """Any shape on the register-staged fp8 kernel: ragged M, N, K, rows that are not 16-byte aligned
+    (views of wider buffers whose cells past the edges hold NaN codes), C inside a buffer of sentinels.
+    Operands are multiples of 1/2 up to 2 in magnitude: exact in both fp8 types, exact sums."""
+    rng = np.random.default_rng(M * 7 + K)
+    A = rng.integers(-4, 5, (M, K)) / 2.0; B = rng.integers(-4, 5, (K, N)) / 2.0
+    At, Ac = fp8_tensor(orc, A, fmt); Bt, Bc = fp8_tensor(orc, B, fmt)
+    nan = torch.full((1,), float("nan")).to(FP8[fmt]).view(torch.uint8).item()
+    Abuf = torch.full((K + 3, M + 5), nan, dtype=torch.uint8, device="cuda").view(FP8[fmt])
+    Bbuf = torch.full((N + 2, K + 7), nan, dtype=torch.uint8, device="cuda").view(FP8[fmt])
+    Abuf.view(torch.uint8)[:K, 1:1 + M] = At.view(torch.uint8); Bbuf.view(torch.uint8)[:N, 3:3 + K] = Bt.view(torch.uint8)
+    buf = torch.full((N + 3, M + 9), -77.0, device="cuda")
+    C = buf[:N, :M]
+    ct.matmul_kernel(Abuf[:K, 1:1 + M], Bbuf[:N, 3:3 + K], C, 64, 64, 64)
+    assert ct.last_variant() == "gemm8_generic_64x64x64"
+    assert np.array_equal(orc.to_julia(C.contiguous()).astype(np.float64), orc.fp8_matmul(Ac, Bc, fmt))
+    assert bool((buf[N:] == -77.0).all()) and bool((buf[:, M:] == -77.0).all())
+    # 16-byte aligned operands of the same problem take the vector loads of the same kernel
+    C2 = torch.empty((N, M), device="cuda")
+    ct.matmul_kernel(At, Bt, C2, 64, 64, 64)
+    assert torch.equal(C2, C)
+
+
+@pytest.mark.parametrize("M,N,K,fmt,out", [(4096, 4096, 512, "e4m3fn", torch.float32), (2048, 2304, 1040, "e5m2", torch.float16),
+                                           (4000, 4001, 528, "e4m3fn", torch.float16), (1024, 512, 2048, "e5m2", torch.float32),
+                                           (3072, 3081, 784, "e4m3fn", torch.bfloat16), (16, 16385, 512, "e5m2", torch.float32),
+                                           (2064, 2000, 1296, "e4m3fn", torch.float32)])
+def test_matmul_fp8_direct_to_lds_kernel_exact(ct, orc, M, N, K, fmt, out):
+    """The fp8 direct-to-LDS kernel (256 x 256 tiles of 32x32x64 MFMAs, ring of four stages): M and K
+    multiples of 16 off the tile / 256 grid, any N, K/64 = 8 ... 32 steps with remainders of 16, 48 and
+    16 bytes of K in the last group.  Operands in {-1, -1/2, 0, 1/2, 1}: every sum is exact, so any slip
+    in the byte-transposing LDS reads, the swizzles, the ring or the tile mapping changes the result.
+    Cells past K hold NaN codes; C is a view of a buffer of sentinels that must come back untouched."""
+    rng = np.random.default_rng(M ^ N ^ K)
+    A = rng.integers(-2, 3, (M, K)) / 2.0; B = rng.integers(-2, 3, (K, N)) / 2.0
+    At, Ac = fp8_tensor(orc, A, fmt); Bt, Bc = fp8_tensor(orc, B, fmt)
+    nan = torch.full((1,), float("nan")).to(FP8[fmt]).view(torch.uint8).item()
+    Abuf = torch.full((K + 128, M), nan, dtype=torch.uint8, device="cuda"); Bbuf = torch.full((N, K + 128), nan, dtype=torch.uint8, device="cuda")
+    Abuf[:K] = At.view(torch.uint8); Bbuf[:, :K] = Bt.view(torch.uint8)
+    buf = torch.full((N + 3, M + 48), -77.0, dtype=out, device="cuda")
+    C = buf[:N, :M]
+    ct.matmul_kernel(Abuf.view(FP8[fmt])[:K], Bbuf.view(FP8[fmt])[:, :K], C, 64, 64, 64)
+    assert ct.last_variant() == "gemm8_big_256x256x64_ring4"
+    ref = orc.fp8_matmul(Ac, Bc, fmt)
+    want = orc.to_julia(orc.from_julia(ref.astype(np.float32)).to(out).float())   # the exact fp32 sum, rounded once on the store
+    assert np.array_equal(orc.to_julia(C.contiguous().float()), want)
+    assert bool((buf[N:] == -77.0).all()) and bool((buf[:, M:] == -77.0).all())
+
+
+def test_matmul_fp8_direct_to_lds_kernel_shape_sweep(ct, orc):
+    """Sixteen seeded shapes with M, K multiples of 16 (K >= 512) and any N on the fp8 direct-to-LDS
+    kernel; exact sums."""
+    rng = np.random.default_rng(808)
+    for case in range(16):
+        M = 16 * int(rng.integers(32, 200)); N = int(rng.integers(600, 3000)); K = 16 * int(rng.integers(32, 120))
+        fmt = "e4m3fn" if case % 2 == 0 else "e5m2"
+        A = rng.integers(-2, 3, (M, K)) / 2.0; B = rng.integers(-2, 3, (K, N)) / 2.0
+        At, Ac = fp8_tensor(orc, A, fmt); Bt, Bc = fp8_tensor(orc, B, fmt)
+        C = torch.full((N, M), -77.0, device="cuda")
+        ct.matmul_kernel(At, Bt, C, 64, 64, 64)
+        v = ct.last_variant()
+        if (-(-M // 256)) * (-(-N // 256)) >= 8:
+            assert v == "gemm8_big_256x256x64_ring4", (M, N, K, v)
+        assert np.array_equal(orc.to_julia(C).astype(np.float64), orc.fp8_matmul(Ac, Bc, fmt)), (M, N, K, v)
+
+
+@pytest.mark.parametrize("M,K,N,Bn,big", [(512, 512, 512, 8, True), (528, 784, 1001, 3, True), (100, 70, 90, 5, False)])
+def test_batch_matmul_fp8_exact(ct, orc, M, K, N, Bn, big):
+    """batch_matmul_kernel on fp8 operands: both kernels, padded leading dimensions and batch strides."""
+    rng = np.random.default_rng(M + Bn)
+    A = rng.integers(-2, 3, (M, K, Bn)) / 2.0; B = rng.integers(-2, 3, (K, N, Bn)) / 2.0
+    At, Ac = fp8_tensor(orc, A, "e4m3fn"); Bt, Bc = fp8_tensor(orc, B, "e4m3fn")
+    ref = np.stack([orc.fp8_matmul(np.ascontiguousarray(Ac[:, :, b]), np.ascontiguousarray(Bc[:, :, b])) for b in range(Bn)], axis=2)
+    Aw = torch.zeros((Bn, K + 3, M + 16), dtype=torch.uint8, device="cuda"); Aw[:, :K, :M] = At.view(torch.uint8)
+    Bw = torch.zeros((Bn, N + 2, K + 16), dtype=torch.uint8, device="cuda"); Bw[:, :N, :K] = Bt.view(torch.uint8)
+    Cw = torch.full((Bn, N + 1, M + 4), -77.0, device="cuda")
+    C = Cw[:, :N, :M]
+    ct.batch_matmul_kernel(Aw.view(FP8["e4m3fn"])[:, :K, :M], Bw.view(FP8["e4m3fn"])[:, :N, :K], C, 128, 128, 64)
+    assert ct.last_variant() == ("gemm8_big_256x256x64_ring4" if big else "gemm8_generic_64x64x64")
+    assert np.array_equal(orc.to_julia(C.contiguous()).astype(np.float64), ref)
+    assert bool((Cw[:, N:] == -77.0).all()) and bool((Cw[:, :, M:] == -77.0).all())
+
+
+def test_matmul_fp8_rejects_mixed_operand_types(ct):
+    """lhs and rhs must share the type (src/compiler/intrinsics/core.jl:589-590); C may not be fp8."""
+    a = torch.zeros((64, 64), dtype=torch.uint8, device="cuda")
+    C = torch.empty((64, 64), device="cuda")
+    with pytest.raises(ct.MiError) as e:
+        ct.matmul_kernel(a.view(torch.float8_e4m3fn), a.view(torch.float8_e5m2), C, 64, 64, 64)
+    assert e.value.code == ct.MI_E_DTYPE
+    with pytest.raises(ct.MiError) as e:
+        ct.matmul_kernel(a.view(torch.float8_e4m3fn), a.view(torch.float8_e4m3fn), a.view(torch.float8_e4m3fn), 64, 64, 64)
+    assert e.value.code == ct.MI_E_DTYPE
+
+
+@pytest.mark.parametrize("fmt", ["e4m3fn", "e5m2"])
+def test_matmul_full_size_fp8(ct, orc, fmt):
+    """4096^3 fp8 -> f32: operands ~ N(0, 1) rounded to the fp8 type; sampled rows / columns against float64
+    on the decoded operands, and the checksum of checksums over all of C."""
+    rng = np.random.default_rng(9)
+    enc, dec = (orc.e4m3fn_encode, orc.e4m3fn_decode) if fmt == "e4m3fn" else (orc.e5m2_encode, orc.e5m2_decode)
+    Ac = enc(rng.standard_normal((4096, 4096), dtype=np.float32)); Bc = enc(rng.standard_normal((4096, 4096), dtype=np.float32))
+    At = orc.from_julia(Ac).view(FP8[fmt]).cuda(); Bt = orc.from_julia(Bc).view(FP8[fmt]).cuda()
+    Ct = torch.empty((4096, 4096), device="cuda")
+    ct.matmul_kernel(At, Bt, Ct, 64, 64, 64)
+    assert ct.last_variant() == "gemm8_big_256x256x64_ring4"
+    A = dec(Ac).astype(np.float64); B = dec(Bc).astype(np.float64); C = orc.to_julia(Ct)
+    rows = [0, 1, 255, 256, 2049, 4095]; cols = [0, 31, 32, 1000, 4095]
+    ref_rows = A[rows] @ B
+    check(C[rows], ref_rows, 2e-2)
+    assert np.abs(C[rows] - ref_rows).max() <= 1e-4 * np.abs(ref_rows).max()      # exact products, fp32 sums of 4096 terms
+    ref_cols = A @ B[:, cols]
+    assert np.abs(C[:, cols] - ref_cols).max() <= 1e-4 * np.abs(ref_cols).max()
+    total = torch.sum(Ct.double()).item()
+    expect = float(A.sum(axis=0) @ B.sum(axis=1))
+    assert abs(total - expect) <= 1e-4 * np.abs(A).sum(axis=0) @ np.abs(B).sum(axis=1)

@@ -284,6 +284,42 @@ def test_e4m3fn_all_codes_against_torch(corc):
     assert np.array_equal(orc.e4m3fn_encode(dec[finite]), finite)  # encode∘decode = id (incl. -0)
 
 
+def test_e5m2_codec_against_torch_and_reference_vectors():
+    """Every E5M2 code decodes as torch.float8_e5m2 does; encoding is round-to-nearest-even with
+    overflow to Inf (torch's conversion is an independent implementation); the reference's 16
+    exactly representable values round-trip (test/extensions/DLFP8Types.jl:126-134)."""
+    codes = np.arange(256, dtype=np.uint8)
+    ref = torch.from_numpy(codes).view(torch.float8_e5m2).to(torch.float32).numpy()
+    dec = orc.e5m2_decode(codes)
+    assert np.array_equal(np.isnan(dec), np.isnan(ref))
+    ok = ~np.isnan(ref)
+    assert np.array_equal(dec[ok], ref[ok]) and np.array_equal(np.signbit(dec[ok]), np.signbit(ref[ok]))
+    assert np.array_equal(orc.e5m2_encode(dec[ok]), codes[ok])          # encode . decode = id, -0 and Inf included
+    rng = np.random.default_rng(5)
+    x = np.concatenate([rng.standard_normal(20000).astype(np.float32) * np.float32(s) for s in (1e-5, 1e-3, 1.0, 300.0, 4e4)]
+                       + [dec[ok], (dec[ok][:-1] + dec[ok][1:])[np.isfinite(dec[ok][:-1] + dec[ok][1:])] / 2])   # ties
+    got = orc.e5m2_encode(x)
+    want = torch.from_numpy(x.astype(np.float32)).to(torch.float8_e5m2).view(torch.uint8).numpy()
+    assert np.array_equal(got, want)
+    with open(os.path.join(os.path.dirname(__file__), "golden", "dlfp8_vectors.json")) as f:
+        rep = np.array(json.load(f)["representable"], dtype=np.float32)
+    assert np.array_equal(orc.e5m2_decode(orc.e5m2_encode(rep)), rep)
+
+
+def test_fp8_matmul_reference_exact_case():
+    """The reference's own mma check (test/extensions/DLFP8Types.jl:143-152): operands drawn from
+    {0, 0.5, 1}, so twice every operand is an integer and 4 * (A * B) is an integer matrix product."""
+    rng = np.random.default_rng(11)
+    for fmt, enc in (("e4m3fn", orc.e4m3fn_encode), ("e5m2", orc.e5m2_encode)):
+        a2 = rng.integers(0, 3, (16, 16)); b2 = rng.integers(0, 3, (16, 16))
+        got = orc.fp8_matmul(enc(a2 / 2.0), enc(b2 / 2.0), fmt)
+        want = np.zeros((16, 16), dtype=np.int64)
+        for i in range(16):
+            for j in range(16):
+                want[i, j] = sum(int(a2[i, k]) * int(b2[k, j]) for k in range(16))
+        assert np.array_equal(got * 4, want)
+
+
 def test_e4m3fn_encode_rne_against_torch_and_c(corc):
     rng = np.random.default_rng(10)
     x = np.concatenate([rng.standard_normal(4000) * 3, rng.standard_normal(2000) * 200,

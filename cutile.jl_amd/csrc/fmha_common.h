@@ -23,6 +23,7 @@ struct F16 {
         _Float16 h = (_Float16)v;
         return __builtin_bit_cast(short, h);
     }
+    static __device__ __forceinline__ float to_f32(short v) { return (float)__builtin_bit_cast(_Float16, v); }
 };
 struct BF16 {
     static __device__ __forceinline__ f32x16 mfma32(s16x8 a, s16x8 b, f32x16 c) {
@@ -34,6 +35,7 @@ struct BF16 {
         u += 0x7fffu + ((u >> 16) & 1u);
         return (short)(u >> 16);
     }
+    static __device__ __forceinline__ float to_f32(short v) { return __uint_as_float((unsigned)(unsigned short)v << 16); }
 };
 
 struct Strides {

@@ -61,10 +61,18 @@ __device__ __forceinline__ void wait_and_barrier() {
     fence();
 }
 
+// max(a, b, c) as one instruction.  (fmaxf() is preceded by a quieting v_max_f32 x, x, x of every operand the
+// compiler can not prove to be no signalling NaN, and MFMA results are such operands.)
+__device__ __forceinline__ float max3(float a, float b, float c) {
+    float r;
+    asm("v_max3_f32 %0, %1, %2, %3" : "=v"(r) : "v"(a), "v"(b), "v"(c));
+    return r;
+}
+
 // max / sum over the lane pair (l, l ^ 32)
 __device__ __forceinline__ float xhalf_max(float v) {
     auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
-    return fmaxf(__uint_as_float(r[0]), __uint_as_float(r[1]));
+    return max3(__uint_as_float(r[0]), __uint_as_float(r[1]), __uint_as_float(r[1]));
 }
 __device__ __forceinline__ float xhalf_sum(float v) {
     auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
@@ -78,7 +86,7 @@ struct Lane {
     int64_t k_half_bytes, v_half_bytes;
     unsigned ks_base, vs_base;      // LDS byte addresses of the rings
     int wave, nh;                   // halves walked by this workgroup
-    float scale2, inv_scale2;
+    bool hb0;                       // lane of the lower half-wave (holds k = 0..7 of an MFMA operand)
     // per lane
     unsigned kdma, vdma;            // byte offset of the lane's 16 bytes in transfer `wave` (transfer wave+2: 16 keys on)
     unsigned kfo[4];                // K fragment element offsets inside a slot, per k-step
@@ -90,10 +98,15 @@ struct Lane {
 
 template <typename E>
 struct Acc {
-    s16x8 qf[2][4];
+    s16x8 qf[2][4];    // Q fragments, already multiplied by the exp2-domain scale
+    s16x8 qm[2];       // a fifth "k step" of the query operand: -(running maximum) at k = 0, zeros elsewhere.  Against
+                       // a key operand that is 1 at k = 0 it makes the S MFMAs deliver S - m, so the weights are a
+                       // bare exp2 of the accumulator (two MFMAs per step instead of 32 vector fma)
+    s16x8 ones;        // that key operand
     f32x16 o[2][2];
-    float m[2], l[2];  // running maximum (exp2 domain) and sum of the lane's half of the keys
-    float thr[2];      // raw score above which m is raised: (m + kRaise) / scale2
+    float m[2], l[2];  // running maximum (exp2 domain, a value of the storage type; -inf until the first half) and
+                       // sum of the lane's half of the keys
+    float thr[2];      // S - m above which m is raised: -inf until the first half, kRaise afterwards
 };
 
 // Transfers the next K (V) half into ring slot `slot`.  Past the last half the same half is sent
@@ -126,19 +139,19 @@ __device__ __forceinline__ float masked_row_max(f32x16& s, int lim) {
 #pragma unroll
         for (int r = 0; r < 16; ++r) s[r] = (8 * (r >> 2) + (r & 3) <= lim) ? s[r] : -INFINITY;
     }
-    float mx = fmaxf(fmaxf(s[0], s[1]), s[2]);
+    float mx = max3(s[0], s[1], s[2]);
 #pragma unroll
-    for (int r = 3; r < 15; r += 2) mx = fmaxf(fmaxf(mx, s[r]), s[r + 1]);
-    return xhalf_max(fmaxf(mx, s[15]));
+    for (int r = 3; r < 15; r += 2) mx = max3(mx, s[r], s[r + 1]);
+    return xhalf_max(max3(mx, s[15], s[15]));
 }
 
 // The weights of one score pair (2h, 2h+1), h = 0..7, are made in two stages that the step below
 // places in consecutive issue slots, so that no instruction waits for the one just before it:
-// stage 1: 2 fma + 2 exp2 relative to the (possibly stale) running maximum;
+// stage 1: 2 exp2 of scores that the MFMAs delivered relative to the (possibly stale) running maximum;
 // stage 2: round and pack for the P.V MFMAs, add to the row sum.
-__device__ __forceinline__ void exp_stage1(const f32x16& s, int h, float nm, float scale2, float (&p)[2]) {
-    p[0] = __builtin_amdgcn_exp2f(__builtin_fmaf(s[2 * h], scale2, nm));
-    p[1] = __builtin_amdgcn_exp2f(__builtin_fmaf(s[2 * h + 1], scale2, nm));
+__device__ __forceinline__ void exp_stage1(const f32x16& s, int h, float (&p)[2]) {
+    p[0] = __builtin_amdgcn_exp2f(s[2 * h]);
+    p[1] = __builtin_amdgcn_exp2f(s[2 * h + 1]);
 }
 template <typename E>
 __device__ __forceinline__ void exp_stage2(const float (&p)[2], int h, float& l, unsigned (&pf)[2][4]) {
@@ -172,7 +185,7 @@ __device__ __forceinline__ void half_step(const unsigned short* Ks, const unsign
                                           int j, f32x16 (&s_cur)[2], f32x16 (&s_next)[2], s16x8 (&kf)[4],
                                           float (&cand)[2]) {
     constexpr int nC = popcount2(CUR), nN = popcount2(NEXT);
-    constexpr int nQ = 4 * nN;   // S(j+1) MFMAs, k-step major over the NEXT streams
+    constexpr int nQ = 5 * nN;   // S(j+1) MFMAs, k-step major over the NEXT streams; "k step" 0 places -m
     constexpr int nP = 2 * nC;   // P.V MFMAs per 16-key chunk, stream major
     // ---- raise the running maxima if some row outgrew its own by 2^kRaise ---------------------------
     // (Every row sees key 0 in the first half, so a raised maximum is finite.)
@@ -184,15 +197,23 @@ __device__ __forceinline__ void half_step(const unsigned short* Ks, const unsign
 #pragma unroll
         for (int jj = 0; jj < 2; ++jj) {
             if (!((CUR >> jj) & 1)) continue;
-            const float m_new = fmaxf(a.m[jj], cand[jj] * c.scale2);
+            // the scores of this half were computed relative to `base` (0 before the first maximum); the new
+            // maximum is rounded to the storage type, in which the MFMA operand carries it
+            const float base = a.thr[jj] == -INFINITY ? 0.f : a.m[jj];
+            const short mh = E::cvt(fmaxf(a.m[jj], base + cand[jj]));
+            const float m_new = E::to_f32(mh);
             const float alpha = __builtin_amdgcn_exp2f(a.m[jj] - m_new);
+            const float shift = base - m_new;
             a.l[jj] *= alpha;
 #pragma unroll
             for (int dt = 0; dt < 2; ++dt)
 #pragma unroll
                 for (int r = 0; r < 16; ++r) a.o[jj][dt][r] *= alpha;
+#pragma unroll
+            for (int r = 0; r < 16; ++r) s_cur[jj][r] += shift;
+            a.qm[jj][0] = c.hb0 ? (short)(mh ^ (short)0x8000) : (short)0;
             a.m[jj] = m_new;
-            a.thr[jj] = (m_new + kRaise) * c.inv_scale2;
+            a.thr[jj] = kRaise;
         }
     }
     wait_and_barrier<kWaitVm8>();
@@ -212,9 +233,6 @@ __device__ __forceinline__ void half_step(const unsigned short* Ks, const unsign
                 vf[ch][dt] = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
             }
     }
-    float nm[2];
-#pragma unroll
-    for (int jj = 0; jj < 2; ++jj) nm[jj] = -a.m[jj];
     unsigned pf[2][2][4];
     slot_end();
 
@@ -222,7 +240,7 @@ __device__ __forceinline__ void half_step(const unsigned short* Ks, const unsign
     auto mfma_q = [&]() {
         constexpr int nNd = nN ? nN : 1;  // (never called when NEXT is empty)
         const int ks = qi / nNd, jj = nth_stream(NEXT, qi % nNd);
-        s_next[jj] = E::mfma32(kf[ks], a.qf[jj][ks], ks == 0 ? f32x16{0} : s_next[jj]);
+        s_next[jj] = ks == 0 ? E::mfma32(a.ones, a.qm[jj], f32x16{0}) : E::mfma32(kf[ks - 1], a.qf[jj][ks - 1], s_next[jj]);
         ++qi;
     };
     auto mfma_p = [&](int ch, int k) {
@@ -235,7 +253,7 @@ __device__ __forceinline__ void half_step(const unsigned short* Ks, const unsign
     float pa[2], pb[2];  // stage-1 results in flight, used alternately
     auto stage1 = [&](int x, float (&p)[2]) {
         const int ch = x / (4 * nC), jj = nth_stream(CUR, (x / 4) % nC), h = 4 * ch + x % 4;
-        exp_stage1(s_cur[jj], h, nm[jj], c.scale2, p);
+        exp_stage1(s_cur[jj], h, p);
     };
     auto stage2 = [&](int x, const float (&p)[2]) {
         const int ch = x / (4 * nC), jj = nth_stream(CUR, (x / 4) % nC), h = 4 * ch + x % 4;
@@ -277,13 +295,22 @@ __device__ __forceinline__ void half_step(const unsigned short* Ks, const unsign
     }
     piece();  // finishes the last pair
     // C
-    if (NEXT) read_k_frags(Ks, c, (j + 2) & 3, kf);  // every S MFMA has been issued: the old fragments are free
+    // the K(j+2) fragments are read once every S MFMA has been issued: the old fragments are free then
+    bool kread = !NEXT;
+    if (!kread && qi == nQ) {
+        read_k_frags(Ks, c, (j + 2) & 3, kf);
+        kread = true;
+    }
 #pragma unroll
     for (int sl = 0; sl < 2 * nQ + 2 * nP; ++sl) {
         if (qi < nQ) mfma_q();
         else if (p0 < nP) mfma_p(0, p0++);
         else if (p1 < nP) mfma_p(1, p1++);
         else break;
+        if (!kread && qi == nQ) {
+            read_k_frags(Ks, c, (j + 2) & 3, kf);
+            kread = true;
+        }
         if (qi == nQ && mi < nN && (sl % 2 == 1 || p1 == nP)) maxima();
         slot_end();
     }
@@ -339,8 +366,7 @@ __global__ __launch_bounds__(128) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     c.wave = wave;
     c.nh = CAUSAL ? NT - 2 * qb : NT;
     c.k_left = c.v_left = c.nh;
-    c.scale2 = scale2;
-    c.inv_scale2 = 1.0f / scale2;
+    c.hb0 = hb == 0;
     {
         // transfer `wave` of a half covers keys 8*wave .. 8*wave+7; transfer wave+2 the keys 16 further on,
         // whose swizzle (a function of key % 16 resp. key % 4) is the same.  K: chunk ^ (key / 2) % 8 --
@@ -367,15 +393,23 @@ __global__ __launch_bounds__(128) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     }
 
     Acc<E> a;
+    a.ones = s16x8{0};
+    a.ones[0] = hb == 0 ? E::cvt(1.0f) : (short)0;
     int my_q[2];
 #pragma unroll
     for (int jj = 0; jj < 2; ++jj) {
         my_q[jj] = 32 * tq[jj] + (lane & 31);
 #pragma unroll
-        for (int s = 0; s < 4; ++s)
-            a.qf[jj][s] = *reinterpret_cast<const s16x8*>(Q + (int64_t)my_q[jj] * qs.s1 + 16 * s + 8 * hb);
+        for (int s = 0; s < 4; ++s) {
+            // Q * (qk_scale / ln 2), rounded once to the storage type: the S MFMAs then deliver exp2-domain
+            // scores (fmha.jl:41,106-110 scales the fp32 products instead; the difference is one rounding of Q)
+            const s16x8 q = *reinterpret_cast<const s16x8*>(Q + (int64_t)my_q[jj] * qs.s1 + 16 * s + 8 * hb);
+#pragma unroll
+            for (int e = 0; e < 8; ++e) a.qf[jj][s][e] = E::cvt(E::to_f32(q[e]) * scale2);
+        }
 #pragma unroll
         for (int dt = 0; dt < 2; ++dt) a.o[jj][dt] = f32x16{0};
+        a.qm[jj] = s16x8{0};
         a.m[jj] = -INFINITY;
         a.thr[jj] = -INFINITY;
         a.l[jj] = 0.f;

@@ -61,7 +61,7 @@ __global__ __launch_bounds__(256) void fmha_fwd_kernel(const unsigned short* __r
                                                        const unsigned short* __restrict__ V, Strides vs,
                                                        unsigned short* __restrict__ O, Strides os, int Sq,
                                                        int Skv, int H, int group, float scale2,
-                                                       int input_pos, bool vec_ok) {
+                                                       int input_pos, bool vec_ok, int nqb) {
     constexpr int CH = D / 8;             // 16-byte chunks per row
     constexpr int PER_T = kKV * CH / 256;  // chunks per thread per tile
     constexpr int KSTEPS = D / 16;
@@ -71,9 +71,10 @@ __global__ __launch_bounds__(256) void fmha_fwd_kernel(const unsigned short* __r
     __shared__ __attribute__((aligned(16))) unsigned short Vs[kKV * VP];
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, hb = lane >> 5;
-    const int nqb = gridDim.x;
-    const int qb = CAUSAL ? nqb - 1 - (int)blockIdx.x : (int)blockIdx.x;  // heavy tiles first
-    const int batch = blockIdx.y / H, head = blockIdx.y % H, kvh = head / group;
+    // one-dimensional grid over (query block, batch * head), query blocks fastest
+    const int bh = (int)(blockIdx.x / (unsigned)nqb), qbx = (int)(blockIdx.x % (unsigned)nqb);
+    const int qb = CAUSAL ? nqb - 1 - qbx : qbx;  // heavy tiles first
+    const int batch = bh / H, head = bh % H, kvh = head / group;
     const int q0 = qb * kQB, qw0 = q0 + wave * 32;
     Q += (int64_t)head * qs.s2 + (int64_t)batch * qs.s3;
     O += (int64_t)head * os.s2 + (int64_t)batch * os.s3;
@@ -580,14 +581,15 @@ void launch(dim3 grid, hipStream_t s, bool causal, const mi_tile_array* Q, const
         set_variant(D == 64 ? "fmha_dma_q128_kv64_d64_w64q" : "fmha_dma_q128_kv64_d128_w32q");
         return;
     }
+    const dim3 g2((unsigned)(grid.x * grid.y));
     if (causal)
-        hipLaunchKernelGGL((fmha_fwd_kernel<E, D, true>), grid, dim3(256), 0, s, (const unsigned short*)Q->ptr, qs,
+        hipLaunchKernelGGL((fmha_fwd_kernel<E, D, true>), g2, dim3(256), 0, s, (const unsigned short*)Q->ptr, qs,
                            (const unsigned short*)K->ptr, ks, (const unsigned short*)V->ptr, vs,
-                           (unsigned short*)O->ptr, os, Sq, Skv, H, group, scale2, input_pos, vec_ok);
+                           (unsigned short*)O->ptr, os, Sq, Skv, H, group, scale2, input_pos, vec_ok, (int)grid.x);
     else
-        hipLaunchKernelGGL((fmha_fwd_kernel<E, D, false>), grid, dim3(256), 0, s, (const unsigned short*)Q->ptr, qs,
+        hipLaunchKernelGGL((fmha_fwd_kernel<E, D, false>), g2, dim3(256), 0, s, (const unsigned short*)Q->ptr, qs,
                            (const unsigned short*)K->ptr, ks, (const unsigned short*)V->ptr, vs,
-                           (unsigned short*)O->ptr, os, Sq, Skv, H, group, scale2, input_pos, vec_ok);
+                           (unsigned short*)O->ptr, os, Sq, Skv, H, group, scale2, input_pos, vec_ok, (int)grid.x);
     set_variant(D == 64 ? "fmha_regstage_q128_kv64_d64" : "fmha_regstage_q128_kv64_d128");
 }
 
@@ -617,7 +619,11 @@ extern "C" int mi_fmha_kernel(const mi_tile_array* Q, const mi_tile_array* K, co
     for (const mi_tile_array* a : {Q, K, V, Out})
         if (a->strides[0] != 1) return MI_E_STRIDE;
     if (Sq > 0x3fffffff || Skv > 0x3fffffff) return MI_E_SHAPE;
-    if (cld(Sq, (int64_t)TILE_M) > MI_MAX_GRID_DIM || B * H > 65535) return MI_E_GRID;
+    // the reference's grid is (cld(Sq, TILE_M), B * H) (fmha.jl:163-165), each below 2^24; the kernels here
+    // use a one-dimensional grid over both
+    if (cld(Sq, (int64_t)TILE_M) > MI_MAX_GRID_DIM || B * H > MI_MAX_GRID_DIM ||
+        cld(Sq, (int64_t)kQB) * B * H > 0x7fffffffLL)
+        return MI_E_GRID;
     if (Sq == 0 || B == 0) return MI_OK;
     if (Skv == 0) return MI_E_SHAPE;
     const bool vec_ok = vec16(Q) && vec16(K) && vec16(V) && vec16(Out);

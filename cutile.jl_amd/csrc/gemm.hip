@@ -45,15 +45,16 @@ template <typename E, typename OutT>
 __global__ __launch_bounds__(256) void gemm16_generic(
     const unsigned short* __restrict__ A, int64_t lda, int64_t sa, const unsigned short* __restrict__ B,
     int64_t ldb, int64_t sb, OutT* __restrict__ C, int64_t ldc, int64_t sc, int M, int N, int K,
-    int tiles_m, bool vecA, bool vecB) {
+    int tiles_m, int tiles_mn, bool vecA, bool vecB) {
     __shared__ __attribute__((aligned(16))) unsigned short As[GK * GA_PITCH];  // [k][m]
     __shared__ __attribute__((aligned(16))) unsigned short Bs[GT * GB_PITCH];  // [n][k]
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int bm = blockIdx.x % tiles_m, bn = blockIdx.x / tiles_m;
+    const int bz = blockIdx.x / (unsigned)tiles_mn, L = blockIdx.x - bz * tiles_mn;   // (tile, batch entry), tiles fastest
+    const int bm = L % tiles_m, bn = L / tiles_m;
     const int64_t m0 = (int64_t)bm * GT, n0 = (int64_t)bn * GT;
-    A += (int64_t)blockIdx.z * sa;
-    B += (int64_t)blockIdx.z * sb;
-    C += (int64_t)blockIdx.z * sc;
+    A += (int64_t)bz * sa;
+    B += (int64_t)bz * sb;
+    C += (int64_t)bz * sc;
     const int wm = (wave & 1) * 32, wn = (wave >> 1) * 32;
 
     const int ak = tid >> 3, am = (tid & 7) * 8;  // A tile: row k, 8 consecutive m
@@ -122,15 +123,16 @@ template <typename E, typename OutT>
 __global__ __launch_bounds__(256) void gemm16_mid(
     const unsigned short* __restrict__ A, int64_t lda, int64_t sa, const unsigned short* __restrict__ B,
     int64_t ldb, int64_t sb, OutT* __restrict__ C, int64_t ldc, int64_t sc, int M, int N, int K,
-    int tiles_m, bool vecA, bool vecB) {
+    int tiles_m, int tiles_mn, bool vecA, bool vecB) {
     __shared__ __attribute__((aligned(16))) unsigned short As[GK * MA_PITCH];  // [k][m]
     __shared__ __attribute__((aligned(16))) unsigned short Bs[MT * MB_PITCH];  // [n][k]
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int bm = blockIdx.x % tiles_m, bn = blockIdx.x / tiles_m;
+    const int bz = blockIdx.x / (unsigned)tiles_mn, L = blockIdx.x - bz * tiles_mn;   // (tile, batch entry), tiles fastest
+    const int bm = L % tiles_m, bn = L / tiles_m;
     const int64_t m0 = (int64_t)bm * MT, n0 = (int64_t)bn * MT;
-    A += (int64_t)blockIdx.z * sa;
-    B += (int64_t)blockIdx.z * sb;
-    C += (int64_t)blockIdx.z * sc;
+    A += (int64_t)bz * sa;
+    B += (int64_t)bz * sb;
+    C += (int64_t)bz * sc;
     const int wm = (wave & 1) * 64, wn = (wave >> 1) * 64;
     const int ak = tid >> 4, am = (tid & 15) * 8;   // A tile: rows k = ak and ak + 16, 8 consecutive m
     const int bnn = tid >> 2, bk = (tid & 3) * 8;   // B tile: columns n = bnn and bnn + 64, 8 consecutive k
@@ -217,15 +219,17 @@ constexpr int FT = 128, FK = 16, F_PITCH = FT + 32;
 __global__ __launch_bounds__(256) void gemm32_kernel(const float* __restrict__ A, int64_t lda, int64_t sa,
                                                      const float* __restrict__ B, int64_t ldb, int64_t sb,
                                                      float* __restrict__ C, int64_t ldc, int64_t sc, int M,
-                                                     int N, int K, int tiles_m, bool vecA, bool vecB) {
+                                                     int N, int K, int tiles_m, int tiles_mn, bool vecA,
+                                                     bool vecB) {
     __shared__ __attribute__((aligned(16))) float As[FK * F_PITCH];  // [k][m]
     __shared__ __attribute__((aligned(16))) float Bs[FK * F_PITCH];  // [k][n]
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int bm = blockIdx.x % tiles_m, bn = blockIdx.x / tiles_m;
+    const int bz = blockIdx.x / (unsigned)tiles_mn, L = blockIdx.x - bz * tiles_mn;   // (tile, batch entry), tiles fastest
+    const int bm = L % tiles_m, bn = L / tiles_m;
     const int64_t m0 = (int64_t)bm * FT, n0 = (int64_t)bn * FT;
-    A += (int64_t)blockIdx.z * sa;
-    B += (int64_t)blockIdx.z * sb;
-    C += (int64_t)blockIdx.z * sc;
+    A += (int64_t)bz * sa;
+    B += (int64_t)bz * sb;
+    C += (int64_t)bz * sc;
     const int wm = (wave & 1) * 64, wn = (wave >> 1) * 64;
     const int ak = tid >> 4, am = (tid & 15) * 4;  // A tile: row k, m = am .. am+3 and 64 + am .. 64 + am+3
     const int bnn = tid & 127, bk = (tid >> 7) * 8;  // B tile: column n, 8 consecutive k; a wave's 64 lanes
@@ -319,9 +323,11 @@ int validate(const mi_tile_array* A, const mi_tile_array* B, const mi_tile_array
     if (ndim == 3) {
         batch = A->sizes[2];
         if (B->sizes[2] != batch || C->sizes[2] != batch) return MI_E_SHAPE;
-        if (batch > 65535) return MI_E_GRID;
+        if (batch > MI_MAX_GRID_DIM) return MI_E_GRID;   // the reference's grid is (cld(M,tm), cld(N,tn), Batch), batchmatmul.jl:78-80
     }
     if (M > 0x7fffffffLL || N > 0x7fffffffLL || K > 0x7fffffffLL) return MI_E_SHAPE;
+    // the kernels number (tile, batch entry) pairs in one grid dimension; their smallest tile is 64 x 64
+    if (cld(M, (int64_t)64) * cld(N, (int64_t)64) * batch > 0x7fffffffLL) return MI_E_GRID;
     if (cld(M, (int64_t)tm) > MI_MAX_GRID_DIM || cld(N, (int64_t)tn) > MI_MAX_GRID_DIM ||
         cld(M, (int64_t)tm) * cld(N, (int64_t)tn) > MI_MAX_GRID_DIM)
         return MI_E_GRID;
@@ -342,9 +348,9 @@ void launch_mid16(const Problem& p, hipStream_t s) {
     const int tiles_m = (int)cld((int64_t)p.M, (int64_t)MT), tiles_n = (int)cld((int64_t)p.N, (int64_t)MT);
     const bool vecA = aligned(p.A, 16) && p.lda % 8 == 0 && p.sa % 8 == 0;
     const bool vecB = aligned(p.B, 16) && p.ldb % 8 == 0 && p.sb % 8 == 0;
-    hipLaunchKernelGGL((gemm16_mid<E, OutT>), dim3((unsigned)(tiles_m * tiles_n), 1, (unsigned)p.batch), dim3(256), 0,
+    hipLaunchKernelGGL((gemm16_mid<E, OutT>), dim3((unsigned)(tiles_m * tiles_n * p.batch)), dim3(256), 0,
                        s, (const unsigned short*)p.A, p.lda, p.sa, (const unsigned short*)p.B, p.ldb, p.sb,
-                       (OutT*)p.C, p.ldc, p.sc, p.M, p.N, p.K, tiles_m, vecA, vecB);
+                       (OutT*)p.C, p.ldc, p.sc, p.M, p.N, p.K, tiles_m, tiles_m * tiles_n, vecA, vecB);
 }
 
 template <typename E, typename OutT>
@@ -352,9 +358,9 @@ void launch_generic16(const Problem& p, hipStream_t s) {
     const int tiles_m = (int)cld((int64_t)p.M, (int64_t)GT), tiles_n = (int)cld((int64_t)p.N, (int64_t)GT);
     const bool vecA = aligned(p.A, 16) && p.lda % 8 == 0 && p.sa % 8 == 0;
     const bool vecB = aligned(p.B, 16) && p.ldb % 8 == 0 && p.sb % 8 == 0;
-    hipLaunchKernelGGL((gemm16_generic<E, OutT>), dim3((unsigned)(tiles_m * tiles_n), 1, (unsigned)p.batch),
+    hipLaunchKernelGGL((gemm16_generic<E, OutT>), dim3((unsigned)(tiles_m * tiles_n * p.batch)),
                        dim3(256), 0, s, (const unsigned short*)p.A, p.lda, p.sa, (const unsigned short*)p.B,
-                       p.ldb, p.sb, (OutT*)p.C, p.ldc, p.sc, p.M, p.N, p.K, tiles_m, vecA, vecB);
+                       p.ldb, p.sb, (OutT*)p.C, p.ldc, p.sc, p.M, p.N, p.K, tiles_m, tiles_m * tiles_n, vecA, vecB);
 }
 
 int run(const Problem& p, hipStream_t s) {
@@ -372,9 +378,9 @@ int run(const Problem& p, hipStream_t s) {
         const int tiles_m = (int)cld((int64_t)p.M, (int64_t)FT), tiles_n = (int)cld((int64_t)p.N, (int64_t)FT);
         const bool vecA = aligned(p.A, 16) && p.lda % 4 == 0 && p.sa % 4 == 0;
         const bool vecB = aligned(p.B, 16) && p.ldb % 4 == 0 && p.sb % 4 == 0;
-        hipLaunchKernelGGL(gemm32_kernel, dim3((unsigned)(tiles_m * tiles_n), 1, (unsigned)p.batch), dim3(256), 0, s,
+        hipLaunchKernelGGL(gemm32_kernel, dim3((unsigned)(tiles_m * tiles_n * p.batch)), dim3(256), 0, s,
                            (const float*)p.A, p.lda, p.sa, (const float*)p.B, p.ldb, p.sb, (float*)p.C, p.ldc, p.sc,
-                           p.M, p.N, p.K, tiles_m, vecA, vecB);
+                           p.M, p.N, p.K, tiles_m, tiles_m * tiles_n, vecA, vecB);
         set_variant("gemm32_128x128x16_mfma32x32x2");
         return launch_status();
     }

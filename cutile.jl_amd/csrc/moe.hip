@@ -391,14 +391,15 @@ template <typename E>
 __global__ __launch_bounds__(256) void silu_and_mul_kernel(const unsigned short* __restrict__ A, int64_t lda,
                                                            const unsigned short* __restrict__ B, int64_t ldb,
                                                            unsigned short* __restrict__ C, int64_t ldc, int rows,
-                                                           bool vec) {
-    const int64_t col = blockIdx.y;
-    const unsigned short* a = A + col * lda;
-    const unsigned short* b = B + col * ldb;
-    unsigned short* c = C + col * ldc;
+                                                           int64_t cols, bool vec) {
     const int i0 = (blockIdx.x * 256 + threadIdx.x) * 8;
     if (i0 >= rows) return;
     auto f = [](float x, float y) { return silu_mul(x, y); };
+    // (the second grid dimension holds at most 65535 workgroups: walk the columns with that stride)
+    for (int64_t col = blockIdx.y; col < cols; col += gridDim.y) {
+    const unsigned short* a = A + col * lda;
+    const unsigned short* b = B + col * ldb;
+    unsigned short* c = C + col * ldc;
     if (vec && i0 + 8 <= rows) {
         s16x8 va = *reinterpret_cast<const s16x8*>(a + i0), vb = *reinterpret_cast<const s16x8*>(b + i0), vc;
 #pragma unroll
@@ -408,20 +409,22 @@ __global__ __launch_bounds__(256) void silu_and_mul_kernel(const unsigned short*
     } else {
         for (int e = 0; e < 8 && i0 + e < rows; ++e) c[i0 + e] = E::cvt(f(E::widen(a[i0 + e]), E::widen(b[i0 + e])));
     }
+    }
 }
 
 // ---- sum over the top-k slots ---------------------------------------------------------------------
 template <typename E>
 __global__ __launch_bounds__(256) void moe_sum_topk_kernel(const unsigned short* __restrict__ in, int64_t s1,
                                                            int64_t s2, unsigned short* __restrict__ out,
-                                                           int64_t ldo, int H, int topk) {
-    const int64_t tok = blockIdx.y;
+                                                           int64_t ldo, int H, int topk, int64_t T) {
     const int h = blockIdx.x * 256 + threadIdx.x;
     if (h >= H) return;
-    const unsigned short* p = in + h + tok * s2;
-    float acc = 0.f;
-    for (int k = 0; k < topk; ++k) acc += E::widen(p[k * s1]);
-    out[h + tok * ldo] = E::cvt(acc);
+    for (int64_t tok = blockIdx.y; tok < T; tok += gridDim.y) {
+        const unsigned short* p = in + h + tok * s2;
+        float acc = 0.f;
+        for (int k = 0; k < topk; ++k) acc += E::widen(p[k * s1]);
+        out[h + tok * ldo] = E::cvt(acc);
+    }
 }
 
 bool is16(int dt) { return dt == MI_F16 || dt == MI_BF16; }
@@ -762,19 +765,18 @@ extern "C" int mi_silu_and_mul_kernel(const mi_tile_array* A, const mi_tile_arra
     if (cols > MI_MAX_GRID_DIM) return MI_E_GRID;
     if (rows == 0 || cols == 0) return MI_OK;
     if (rows > 1 && (A->strides[0] != 1 || B->strides[0] != 1 || C->strides[0] != 1)) return MI_E_STRIDE;
-    if (cols > 65535) return MI_E_UNSUPPORTED;
     const bool vec = aligned(A->ptr, 16) && aligned(B->ptr, 16) && aligned(C->ptr, 16) && A->strides[1] % 8 == 0 &&
                      B->strides[1] % 8 == 0 && C->strides[1] % 8 == 0;
-    dim3 grid((unsigned)cld(rows, (int64_t)2048), (unsigned)cols);
+    dim3 grid((unsigned)cld(rows, (int64_t)2048), (unsigned)(cols < 65535 ? cols : 65535));
     hipStream_t s = (hipStream_t)stream;
     if (A->dtype == MI_F16)
         hipLaunchKernelGGL((silu_and_mul_kernel<F16>), grid, dim3(256), 0, s, (const unsigned short*)A->ptr,
                            A->strides[1], (const unsigned short*)B->ptr, B->strides[1], (unsigned short*)C->ptr,
-                           C->strides[1], (int)rows, vec);
+                           C->strides[1], (int)rows, cols, vec);
     else
         hipLaunchKernelGGL((silu_and_mul_kernel<BF16>), grid, dim3(256), 0, s, (const unsigned short*)A->ptr,
                            A->strides[1], (const unsigned short*)B->ptr, B->strides[1], (unsigned short*)C->ptr,
-                           C->strides[1], (int)rows, vec);
+                           C->strides[1], (int)rows, cols, vec);
     set_variant("silu_and_mul_vec8");
     return launch_status();
 }
@@ -787,17 +789,17 @@ extern "C" int mi_moe_sum_topk(const mi_tile_array* in, const mi_tile_array* out
     if (out->sizes[0] != H || out->sizes[1] != T) return MI_E_SHAPE;
     if (H > 1 && (in->strides[0] != 1 || out->strides[0] != 1)) return MI_E_STRIDE;
     if (H == 0 || T == 0) return MI_OK;
-    if (T > 65535 || H > 0x7fffffff || topk > 0x7fffffff) return MI_E_UNSUPPORTED;
-    dim3 grid((unsigned)cld(H, (int64_t)256), (unsigned)T);
+    if (H > 0x7fffffff || topk > 0x7fffffff) return MI_E_UNSUPPORTED;
+    dim3 grid((unsigned)cld(H, (int64_t)256), (unsigned)(T < 65535 ? T : 65535));
     hipStream_t s = (hipStream_t)stream;
     if (in->dtype == MI_F16)
         hipLaunchKernelGGL((moe_sum_topk_kernel<F16>), grid, dim3(256), 0, s, (const unsigned short*)in->ptr,
                            in->strides[1], in->strides[2], (unsigned short*)out->ptr, out->strides[1], (int)H,
-                           (int)topk);
+                           (int)topk, T);
     else
         hipLaunchKernelGGL((moe_sum_topk_kernel<BF16>), grid, dim3(256), 0, s, (const unsigned short*)in->ptr,
                            in->strides[1], in->strides[2], (unsigned short*)out->ptr, out->strides[1], (int)H,
-                           (int)topk);
+                           (int)topk, T);
     set_variant("moe_sum_topk");
     return launch_status();
 }

@@ -41,9 +41,9 @@ __global__ __launch_bounds__(kBlock) void transpose_kernel(const T* __restrict__
     __shared__ T lds[kTile * kPitch];
 
     const int64_t m0 = (int64_t)blockIdx.x * kTile;  // along x dim 0
-    const int64_t n0 = (int64_t)blockIdx.y * kTile;  // along x dim 1
     const int vi = threadIdx.x % VR, row = threadIdx.x / VR;
-
+    // (the second grid dimension holds at most 65535 workgroups: walk the tile rows along dim 1 with that stride)
+    for (int64_t n0 = (int64_t)blockIdx.y * kTile; n0 < n; n0 += (int64_t)gridDim.y * kTile) {
     // Phase 1: x[m0 + V*vi .. +V-1, n0 + r]  ->  lds[i][j] with i along m, j along n.
 #pragma unroll
     for (int p = 0; p < PASSES; ++p) {
@@ -79,6 +79,8 @@ __global__ __launch_bounds__(kBlock) void transpose_kernel(const T* __restrict__
             for (int q = 0; q < V; ++q)
                 if (gj + q < n && gi < m) y[gj + q + gi * ldy] = lds[i * kPitch + vi * V + q];
         }
+    }
+    __syncthreads();   // the tile is free for the next trip
     }
 }
 
@@ -207,10 +209,10 @@ int launch(const mi_tile_array* x, const mi_tile_array* y, hipStream_t s) {
     const int64_t m = x->sizes[0], n = x->sizes[1];
     const int64_t ldx = x->strides[1], ldy = y->strides[1];
     const int64_t gx = cld(m, (int64_t)kTile), gy = cld(n, (int64_t)kTile);
-    if (gy > 65535 || gx > 0x7fffffffLL) return MI_E_GRID;
+    if (gx > 0x7fffffffLL) return MI_E_GRID;
     const bool vec = (m % V == 0) && (n % V == 0) && (ldx % V == 0) && (ldy % V == 0) &&
                      aligned(x->ptr, 16) && aligned(y->ptr, 16);
-    dim3 grid((unsigned)gx, (unsigned)gy), block(kBlock);
+    dim3 grid((unsigned)gx, (unsigned)(gy < 65535 ? gy : 65535)), block(kBlock);
     if (vec) {
         hipLaunchKernelGGL((transpose_kernel<T, true>), grid, block, 0, s, (const T*)x->ptr, ldx,
                            (T*)y->ptr, ldy, m, n);

@@ -122,9 +122,10 @@ __global__ __launch_bounds__(kBlock) void vadd_2d_kernel(const T* __restrict__ a
                                                          int64_t c0, int64_t c1, int64_t m,
                                                          int64_t n) {
     const int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x;
-    const int64_t j = blockIdx.y;
-    if (i >= m || j >= n) return;
-    c[i * c0 + j * c1] = Vec16<T>::add1(a[i * a0 + j * a1], b[i * b0 + j * b1]);
+    if (i >= m) return;
+    // (the second grid dimension holds at most 65535 workgroups: walk dimension 1 with that stride)
+    for (int64_t j = blockIdx.y; j < n; j += gridDim.y)
+        c[i * c0 + j * c1] = Vec16<T>::add1(a[i * a0 + j * a1], b[i * b0 + j * b1]);
 }
 
 template <typename T>
@@ -177,8 +178,7 @@ int launch_2d(const mi_tile_array* a, const mi_tile_array* b, const mi_tile_arra
               hipStream_t s) {
     const int64_t m = c->sizes[0], n = c->sizes[1];
     if (m == 0 || n == 0) return MI_OK;
-    if (n > 65535) return MI_E_UNSUPPORTED;
-    hipLaunchKernelGGL((vadd_2d_kernel<T>), dim3((unsigned)cld(m, (int64_t)kBlock), (unsigned)n),
+    hipLaunchKernelGGL((vadd_2d_kernel<T>), dim3((unsigned)cld(m, (int64_t)kBlock), (unsigned)(n < 65535 ? n : 65535)),
                        dim3(kBlock), 0, s, (const T*)a->ptr, a->strides[0], a->strides[1],
                        (const T*)b->ptr, b->strides[0], b->strides[1], (T*)c->ptr, c->strides[0],
                        c->strides[1], m, n);

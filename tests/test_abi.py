@@ -115,3 +115,62 @@ def test_host_moe_align_rejects_bad_ids(ct):
     n = ctypes.c_int64()
     assert L.mi_moe_align_tile_size(ids, 2, 2, 4, 4, None, None, ctypes.byref(n)) == ct.MI_E_ARG
     assert L.mi_moe_align_tile_size(ids, 2, 2, 3, 16, None, None, ctypes.byref(n)) == ct.MI_E_TILE
+
+
+def _no_gpu_here():
+    return not torch.cuda.is_available()
+
+
+@pytest.mark.skipif(not _no_gpu_here(), reason="launches with placeholder pointers: only where no GPU can take them")
+def test_dimensions_beyond_65535_pass_the_host_checks(ct):
+    """The reference's grids are flattened and take up to 2^24 - 1 blocks per dimension
+    (src/launch.jl:743,801-807).  Dimensions that this library maps to the second or third grid
+    dimension (at most 65535 workgroups) must not be rejected on the host: tokens * topk columns of
+    silu_and_mul, tokens of the top-k sum, dimension 2 of a strided 2-D vadd, the batch of a batched
+    GEMM, batch * heads of attention.  Without a GPU the launch itself fails with a (positive) HIP
+    status, which is how the test tells "accepted" from a host-side MI_E_* rejection."""
+    L = ct.lib()
+    r = ctypes.byref
+    n = 70_000
+    h16 = ct.MI_F16
+    a = _desc(ct, (64, n), h16); c = _desc(ct, (64, n), h16)
+    assert L.mi_silu_and_mul_kernel(r(a), r(a), r(c), 64, None) > 0
+    assert L.mi_moe_sum_topk(r(_desc(ct, (64, 2, n), h16)), r(_desc(ct, (64, n), h16)), None) > 0
+    v = _desc(ct, (16, n), strides=(2, 32))
+    assert L.mi_vec_add_kernel_2d(r(v), r(v), r(v), 16, 16, None) > 0
+    A = _desc(ct, (8, 8, n), h16)
+    assert L.mi_batch_matmul_kernel(r(A), r(A), r(A), 8, 8, 8, None) > 0
+    q = _desc(ct, (64, 16, 7000, 10), h16)
+    assert L.mi_fmha_kernel(r(q), r(q), r(q), r(q), ctypes.c_float(0.125), 0, 64, 7000, 16, 16, 1, 1, 1, None) > 0
+    # the 24-bit limits of the reference still hold
+    A2 = _desc(ct, (8, 8, 2 ** 24), h16)
+    assert L.mi_batch_matmul_kernel(r(A2), r(A2), r(A2), 8, 8, 8, None) == ct.MI_E_GRID
+
+
+@pytest.mark.skipif(not _no_gpu_here(), reason="launches with placeholder pointers: only where no GPU can take them")
+def test_direct_to_lds_gemms_are_not_chosen_for_descending_or_overlapping_rows(ct):
+    """The direct-to-LDS GEMM kernels compute lane offsets in 32 bits and assume leading dimensions
+    that are at least the row length and positive; a reversed view (negative stride) or overlapping
+    rows must fall to the kernels that index with 64-bit offsets."""
+    L = ct.lib()
+    r = ctypes.byref
+    for dt, bigname in ((ct.MI_F16, "gemm16_big"), (ct.MI_F32, "gemm32_big"), (ct.MI_F8E4M3FN, "gemm8_big")):
+        M = N = K = 2048
+        good = _desc(ct, (M, K), dt); goodB = _desc(ct, (K, N), dt); C = _desc(ct, (M, N), ct.MI_F32)
+        assert L.mi_matmul_kernel(r(good), r(goodB), r(C), 64, 64, 64, None) > 0
+        assert ct.last_variant().startswith(bigname)
+        for bad in (_desc(ct, (M, K), dt, ptr=0x10000000, strides=(1, -M)), _desc(ct, (M, K), dt, strides=(1, M - 16))):
+            assert L.mi_matmul_kernel(r(bad), r(goodB), r(C), 64, 64, 64, None) > 0
+            assert not ct.last_variant().startswith(bigname), ct.last_variant()
+        badC = _desc(ct, (M, N), ct.MI_F32, ptr=0x10000000, strides=(1, -M))
+        assert L.mi_matmul_kernel(r(good), r(goodB), r(badC), 64, 64, 64, None) > 0
+        assert not ct.last_variant().startswith(bigname), ct.last_variant()
+
+
+def test_static_scratch_entry_point_rejects_oversized_problems_on_the_host(ct):
+    """mi_layer_norm_bwd_static: cld(N, 4) * 4 * GROUP_SIZE_M floats must fit the 524288-float static array."""
+    L = ct.lib()
+    r = ctypes.byref
+    X = _desc(ct, (16384, 4)); W = _desc(ct, (16384,)); v = _desc(ct, (4,))
+    assert L.mi_layer_norm_bwd_static(r(X), r(X), r(X), r(W), r(v), r(v), r(W), r(W), 64, 32, 1024, None) == ct.MI_E_SCRATCH
+    assert "scratch" in ct.strerror(ct.MI_E_SCRATCH)

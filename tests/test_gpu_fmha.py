@@ -160,3 +160,16 @@ def test_fmha_full_size(orc):
     ones = torch.ones_like(data.V)
     out1 = fmha.cutile_fmha(data.Q, data.K, ones, causal=True)
     assert torch.all((out1.float() - 1).abs() <= 2e-3)
+
+
+def test_fmha_more_than_65535_batch_heads(ct, orc):
+    """The reference's grid is (cld(Sq, TILE_M), B * H) with up to 2^24 - 1 blocks per dimension
+    (fmha.jl:163-165, src/launch.jl:743): 70 000 (batch, head) pairs of a short sequence."""
+    data = fmha.prepare(batch=10, heads=7000, seq_q=16, seq_kv=16, causal=True)
+    r = fmha.run(data)
+    Q, K, V = (orc.to_julia(t) for t in (data.Q, data.K, data.V))
+    got = orc.to_julia(r.out).astype(np.float64)
+    for b, hs in ((0, slice(0, 3)), (9, slice(6997, 7000)), (9, slice(3552, 3555))):    # pairs 0.., 69997.., 66552..
+        ref = orc.ref_fmha(Q[:, :, hs, b:b + 1], K[:, :, hs, b:b + 1], V[:, :, hs, b:b + 1], causal=True, dtype=np.float64)
+        g = got[:, :, hs, b:b + 1]
+        assert np.all(np.abs(g - ref) <= 2e-2 * (np.abs(ref) + np.abs(ref).max()))

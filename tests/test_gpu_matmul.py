@@ -413,3 +413,17 @@ def test_matmul_full_size_fp8(ct, orc, fmt):
     total = torch.sum(Ct.double()).item()
     expect = float(A.sum(axis=0) @ B.sum(axis=1))
     assert abs(total - expect) <= 1e-4 * np.abs(A).sum(axis=0) @ np.abs(B).sum(axis=1)
+
+
+@pytest.mark.parametrize("T", [torch.float16, torch.float32, torch.float8_e4m3fn])
+def test_batch_matmul_more_than_65535_entries(ct, orc, T):
+    """batch_matmul_kernel's grid is (cld(M,tm), cld(N,tn), Batch) with up to 2^24 - 1 blocks per dimension
+    (batchmatmul.jl:78-80, src/launch.jl:743): 70 000 small entries, integer operands, exact."""
+    rng = np.random.default_rng(21)
+    Bn, M, K, N = 70_000, 16, 16, 8
+    A = rng.integers(-2, 3, (Bn, K, M)).astype(np.float32); B = rng.integers(-2, 3, (Bn, N, K)).astype(np.float32)
+    At = torch.from_numpy(A).to(T).cuda(); Bt = torch.from_numpy(B).to(T).cuda()
+    C = torch.empty((Bn, N, M), dtype=torch.float32, device="cuda")
+    ct.batch_matmul_kernel(At, Bt, C, 16, 8, 16)
+    ref = torch.bmm(torch.from_numpy(B), torch.from_numpy(A))       # torch (N,K) x (K,M) = Julia (A * B)^T
+    assert torch.equal(C.cpu(), ref)

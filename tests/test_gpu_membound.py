@@ -237,3 +237,22 @@ def test_layernorm_full_size(orc):
     close_f32(orc.to_julia(r.DX), DX, tol=2e-5)
     close_f32(orc.to_julia(r.FINAL_DW), DW)
     close_f32(orc.to_julia(r.FINAL_DB), DB)
+
+
+def test_second_dimension_beyond_65535(ct):
+    """A strided 2-D vadd and a transpose whose second dimension exceeds the 65535 workgroups one grid
+    dimension holds here (the reference's grids take 2^24 - 1 blocks per dimension)."""
+    rng = np.random.default_rng(12)
+    n = 70_003
+    A = torch.from_numpy(rng.random((n, 40), dtype=np.float32)).cuda()
+    B = torch.from_numpy(rng.random((n, 40), dtype=np.float32)).cuda()
+    C = torch.zeros(n, 40, device="cuda")
+    ct.vec_add_kernel_2d(A[:, ::2], B[:, ::2], C[:, ::2], 16, 16)     # dimension 0 strided: the element-wise 2-D kernel
+    assert ct.last_variant() == "vadd_2d_strided"
+    assert torch.equal(C[:, ::2], A[:, ::2] + B[:, ::2]) and bool((C[:, 1::2] == 0).all())
+    # one-byte elements take the generic transpose; 64-row tiles along n: 65536 * 64 < n
+    m, nn = 8, 65_540 * 64 + 5
+    x = torch.from_numpy(rng.integers(0, 255, (nn, m), dtype=np.uint8)).cuda().view(torch.float8_e4m3fn)
+    y = torch.empty((m, nn), dtype=torch.uint8, device="cuda").view(torch.float8_e4m3fn)
+    ct.transpose_kernel(x, y, 64, 64)
+    assert torch.equal(y.view(torch.uint8), x.view(torch.uint8).t())

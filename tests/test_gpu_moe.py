@@ -337,3 +337,23 @@ def test_fused_silu_entry_checks_shapes(ct):
     with pytest.raises(ct.MiError) as e:
         ct.fused_moe_silu_kernel(d.hidden_states, d.w1, wrong, d.topk_weights.reshape(-1), tok, exp, 1, False, 16, 128, 64)
     assert e.value.code == ct.MI_E_SHAPE
+
+
+def test_silu_and_topk_sum_beyond_65535_columns(ct, orc):
+    """Prefill sizes: tokens * topk above 65535 (the reference's flattened grids take 2^24 - 1 blocks,
+    src/launch.jl:743).  Checked against the same kernels run on column slices."""
+    rng = np.random.default_rng(4)
+    inter, total = 64, 70_001
+    AB = torch.from_numpy((rng.standard_normal((total, 2 * inter)) * 3).astype(np.float16)).cuda()
+    C = torch.zeros((total, inter), dtype=torch.float16, device="cuda")
+    moe.invoke_silu_and_mul_kernel(AB, C)
+    for lo, hi in ((0, 3), (65_530, 65_545), (total - 4, total)):
+        ref = orc.silu_and_mul(orc.to_julia(AB[lo:hi, :inter]), orc.to_julia(AB[lo:hi, inter:]))
+        check(orc.to_julia(C[lo:hi]), ref, 2e-3)
+    C2 = torch.zeros_like(C)
+    moe.invoke_silu_and_mul_kernel(AB[:60_000], C2[:60_000]); moe.invoke_silu_and_mul_kernel(AB[60_000:], C2[60_000:])
+    assert torch.equal(C, C2)
+    x = torch.from_numpy(rng.standard_normal((total, 2, 64)).astype(np.float16)).cuda()   # Julia (64, 2, total)
+    out = torch.empty((total, 64), dtype=torch.float16, device="cuda")
+    ct.moe_sum_topk(x, out)
+    assert torch.equal(out, x.float().sum(dim=1).to(torch.float16))

@@ -70,17 +70,64 @@ def _back_to_back(fn, nruns):
     return e0.elapsed_time(e1) / nruns
 
 
-def _entry(name, fn, work, unit, bound, peak, dtype, nruns, warmup, extra=None):
+def _entry(name, fn, work, unit, bound, peak, dtype, nruns, warmup, extra=None, cold=None):
+    """``cold``: a list of launches of the same kernel on distinct buffer sets, enough of them that more than
+    the 256 MB memory-side cache holds is touched between two uses of a set; ``frac_cold`` is measured
+    by cycling through them, so that no launch finds its input resident."""
     t = _event_times(fn, nruns, warmup)
-    avg = min(_back_to_back(fn, nruns) for _ in range(2))   # best of two batches: a one-off stall does not define the rate
+    batches = [_back_to_back(fn, nruns) for _ in range(2)]
+    avg = min(batches)   # best of two batches: a one-off stall does not define the rate
     scale = 1e9 if unit == "GB/s" else 1e12
     ach = work / (avg * 1e-3) / scale
     e = {"name": name, "min_ms": round(min(t), 5), "mean_ms": round(sum(t) / len(t), 5), "avg_ms": round(avg, 5),
+         "avg_ms_is": "best of 2 batches of %d back-to-back launches" % nruns,
          "work": work, "achieved": round(ach, 2), "unit": "GB/s" if unit == "GB/s" else "TFLOP/s", "bound": bound,
          "peak": peak, "frac": round(ach / peak, 4), "dtype": dtype}
+    if cold:
+        k = len(cold)
+
+        def cycle():
+            for f in cold:
+                f()
+        cycle()
+        cavg = min(_back_to_back(cycle, max(1, nruns // k)) for _ in range(2)) / k
+        e["avg_ms_cold"] = round(cavg, 5)
+        e["frac_cold"] = round(work / (cavg * 1e-3) / scale / peak, 4)
+        e["cold_sets"] = k
     if extra:
         e.update(extra)
     return e
+
+
+def _shader_clock_mhz():
+    """Current shader clock from the driver's sysfs table (the level marked '*'), or None."""
+    import glob
+    best = None
+    for path in glob.glob("/sys/class/drm/card*/device/pp_dpm_sclk"):
+        try:
+            for line in open(path):
+                if "*" in line:
+                    mhz = int("".join(ch for ch in line.split(":")[1] if ch.isdigit()))
+                    best = mhz if best is None else max(best, mhz)
+        except Exception:
+            pass
+    return best
+
+
+def _clock_under_load(fn, seconds=0.25):
+    """Keep ``fn`` queued for about ``seconds`` and sample the shader clock meanwhile; MHz (median) or None."""
+    import torch
+    samples = []
+    t0 = time.perf_counter()
+    while time.perf_counter() - t0 < seconds:
+        for _ in range(8):
+            fn()
+        c = _shader_clock_mhz()
+        if c is not None:
+            samples.append(c)
+        torch.cuda.synchronize()
+    samples.sort()
+    return samples[len(samples) // 2] if samples else None
 
 
 def _cpu_time(fn, repeats=3):
@@ -127,29 +174,40 @@ def bench_kernels(ct, which, cpu, nruns=NRUNS, warmup=WARMUP):
         del d
     if want("layernorm"):
         for G in (64, 256):
-            d = layernorm.prepare(benchmark=True, GROUP_SIZE_M=G)
-            D = {k: ct.TileArray(getattr(d, k)) for k in ("X", "W", "B", "Y", "Mean", "Rstd", "DY", "DX", "DW_partial",
-                                                          "DB_partial", "Locks", "FINAL_DW", "FINAL_DB")}
+            sets = [layernorm.prepare(benchmark=True, GROUP_SIZE_M=G, seed=1 + i) for i in range(6 if G == 64 else 1)]
+            d = sets[0]
             MN4 = d.M * d.N * 4
 
-            def fwd():
-                ct.layer_norm_fwd(D["X"], D["W"], D["B"], D["Y"], D["Mean"], D["Rstd"], d.eps, 1024)
+            def launches(dd):
+                D = {k: ct.TileArray(getattr(dd, k)) for k in ("X", "W", "B", "Y", "Mean", "Rstd", "DY", "DX", "DW_partial",
+                                                                "DB_partial", "Locks", "FINAL_DW", "FINAL_DB")}
 
-            def bwd():
-                d.partials.zero_()
-                ct.layer_norm_bwd_dx_partial_dwdb(D["DX"], D["DY"], D["DW_partial"], D["DB_partial"], D["X"], D["W"],
-                                                  D["Mean"], D["Rstd"], D["Locks"], G, 1024)
-                ct.layer_norm_bwd_dwdb(D["DW_partial"], D["DB_partial"], D["FINAL_DW"], D["FINAL_DB"], 32, 1024)
+                def fwd():
+                    ct.layer_norm_fwd(D["X"], D["W"], D["B"], D["Y"], D["Mean"], D["Rstd"], dd.eps, 1024)
 
+                def bwd():
+                    dd.partials.zero_()
+                    ct.layer_norm_bwd_dx_partial_dwdb(D["DX"], D["DY"], D["DW_partial"], D["DB_partial"], D["X"], D["W"],
+                                                      D["Mean"], D["Rstd"], D["Locks"], G, 1024)
+                    ct.layer_norm_bwd_dwdb(D["DW_partial"], D["DB_partial"], D["FINAL_DW"], D["FINAL_DB"], 32, 1024)
+                fwd._keep = D
+                return fwd, bwd
+
+            fb = [launches(dd) for dd in sets]
+            fwd, bwd = fb[0]
+            for f, _ in fb:
+                f()     # Mean / Rstd of every set, for its backward
             fwd_bytes = 2 * MN4 + (2 * d.N + 2 * d.M) * 4
             bwd_bytes = 3 * MN4 + (d.N + 2 * d.M) * 4 + 4 * d.N * G * 4 + 2 * d.N * 4
             if G == 64:
                 res["layernorm_fwd"] = _entry("LayerNorm fwd 4096^2 f32", fwd, fwd_bytes, "GB/s", "hbm", HBM_PEAK_GBS,
-                                              "f32", nruns, warmup, {"reference_formula_bytes": 4 * MN4})
+                                              "f32", nruns, warmup, {"reference_formula_bytes": 4 * MN4},
+                                              cold=[f for f, _ in fb])
                 fwd(); res["layernorm_fwd"]["variant"] = ct.last_variant()
             key = "layernorm_bwd" if G == 64 else "layernorm_bwd_G256"
             res[key] = _entry(f"LayerNorm bwd 4096^2 f32, GROUP_SIZE_M={G} (1 fill + 2 kernels)", bwd, bwd_bytes,
-                              "GB/s", "hbm", HBM_PEAK_GBS, "f32", nruns, warmup, {"reference_formula_bytes": 5 * MN4})
+                              "GB/s", "hbm", HBM_PEAK_GBS, "f32", nruns, warmup, {"reference_formula_bytes": 5 * MN4},
+                              cold=[b for _, b in fb] if G == 64 else None)
             if cpu and G == 64:
                 X, W, B, DY = (orc.to_julia(t) for t in (d.X, d.W, d.B, d.DY))
                 sub = slice(0, 512)
@@ -157,28 +215,44 @@ def bench_kernels(ct, which, cpu, nruns=NRUNS, warmup=WARMUP):
                 res["layernorm_fwd"]["cpu_note"] = "numpy 1 thread, 512 of 4096 rows x8"
                 res[key]["cpu_ms"] = round(_cpu_time(lambda: orc.layer_norm_bwd(X[:, sub], W, DY[:, sub], d.eps, dtype=np.float32)) * 8, 1)
                 res[key]["cpu_note"] = "numpy 1 thread, 512 of 4096 rows x8"
-            del d, D
+            del d, sets, fb, fwd, bwd
     if want("softmax"):
-        d = softmax.prepare(benchmark=True)
-        I, O1, O2 = ct.TileArray(d.input), ct.TileArray(d.output_tma), ct.TileArray(d.output_chunked)
+        sets = [softmax.prepare(benchmark=True, seed=2 + i) for i in range(6)]
+        d = sets[0]
         MN4 = d.M * d.N * 4
-        res["softmax_tma"] = _entry("softmax (single tile) 4096^2 f32", lambda: ct.softmax_tma_kernel(O1, I, 4096, d.M),
-                                    2 * MN4, "GB/s", "hbm", HBM_PEAK_GBS, "f32", nruns, warmup)
+        tma, chk = [], []
+        for dd in sets:
+            I, O1, O2 = ct.TileArray(dd.input), ct.TileArray(dd.output_tma), ct.TileArray(dd.output_chunked)
+            tma.append((lambda I=I, O1=O1: ct.softmax_tma_kernel(O1, I, 4096, d.M)))
+            chk.append((lambda I=I, O2=O2: ct.softmax_chunked_kernel(O2, I, d.N, 1024, d.M)))
+        res["softmax_tma"] = _entry("softmax (single tile) 4096^2 f32", tma[0],
+                                    2 * MN4, "GB/s", "hbm", HBM_PEAK_GBS, "f32", nruns, warmup, cold=tma)
         res["softmax_tma"]["variant"] = ct.last_variant()
-        res["softmax_chunked"] = _entry("softmax (chunked) 4096^2 f32",
-                                        lambda: ct.softmax_chunked_kernel(O2, I, d.N, 1024, d.M), 2 * MN4, "GB/s", "hbm",
-                                        HBM_PEAK_GBS, "f32", nruns, warmup, {"reference_formula_bytes": 4 * MN4})
+        res["softmax_chunked"] = _entry("softmax (chunked) 4096^2 f32", chk[0], 2 * MN4, "GB/s", "hbm",
+                                        HBM_PEAK_GBS, "f32", nruns, warmup, {"reference_formula_bytes": 4 * MN4}, cold=chk)
         if cpu:
             x = orc.to_julia(d.input)
             res["softmax_tma"]["cpu_ms"] = round(_cpu_time(lambda: orc.softmax(x[:, :512], dtype=np.float32)) * 8, 1)
             res["softmax_tma"]["cpu_note"] = "numpy 1 thread, 512 of 4096 columns x8"
-        del d
+        del d, sets, tma, chk
+    if want("copy_ref"):
+        # Yardstick for the 64 MB row kernels: a plain 64 MB -> 64 MB copy (the generated Tiled(Y) .= Tiled(X)
+        # kernel) on resident buffers and cycling over six buffer pairs.  What it reaches cold is the ceiling of
+        # any one-pass row kernel of this size on cold input.
+        from cutile_jl_amd import tiled as T
+        n = 1 << 24
+        pairs = [(torch.rand(n, device="cuda"), torch.empty(n, device="cuda")) for _ in range(6)]
+        fns = [(lambda x=x, y=y: T.Tiled(y).assign(T.Tiled(x))) for x, y in pairs]
+        res["copy_ref"] = _entry("yardstick: copy 64 MB -> 64 MB f32 (Tiled(Y) .= Tiled(X))", fns[0], 8 * n, "GB/s", "hbm",
+                                 HBM_PEAK_GBS, "f32", nruns, warmup, cold=fns)
+        del pairs, fns
     if want("matmul"):
         d = matmul.prepare(benchmark=True, T=torch.float16, out_T=torch.float32, dist="normal64")
         A, B, C = ct.TileArray(d.A), ct.TileArray(d.B), ct.TileArray(d.C)
         e = _entry("GEMM 4096^3 f16 -> f32", lambda: ct.matmul_kernel(A, B, C, 64, 64, 64), matmul.metric(d)[0],
                    "TFLOPS", "mfma", 2500.0, "f16", nruns, warmup)
         e["variant"] = ct.last_variant()
+        e["shader_clock_mhz"] = _clock_under_load(lambda: ct.matmul_kernel(A, B, C, 64, 64, 64))
         if cpu:
             a = orc.to_julia(d.A).astype(np.float32); b = orc.to_julia(d.B).astype(np.float32)
             e["cpu_ms"] = round(_cpu_time(lambda: a @ b, repeats=2), 1); e["cpu_note"] = f"numpy/OpenBLAS sgemm on widened inputs, {ncores} threads"
@@ -194,6 +268,7 @@ def bench_kernels(ct, which, cpu, nruns=NRUNS, warmup=WARMUP):
             e = _entry(f"GEMM 4096^3 {nm} x {nm} -> f32 (inputs ~ N(0,1) rounded to fp8)", lambda: ct.matmul_kernel(A, B, C, 64, 64, 64),
                        2.0 * 4096 ** 3, "TFLOPS", "mfma", 5000.0, "fp8", nruns, warmup)
             e["variant"] = ct.last_variant()
+            e["shader_clock_mhz"] = _clock_under_load(lambda: ct.matmul_kernel(A, B, C, 64, 64, 64))
             res[key] = e
             del a8, b8, c8
     if which is not None and "gemm_shapes" in which:
@@ -227,6 +302,7 @@ def bench_kernels(ct, which, cpu, nruns=NRUNS, warmup=WARMUP):
         e = _entry("batched GEMM 8x(1024x512x2048) f32", lambda: ct.batch_matmul_kernel(A, B, C, 128, 128, 64),
                    batchmatmul.metric(d)[0], "TFLOPS", "mfma", 157.3, "f32", nruns, warmup)
         e["variant"] = ct.last_variant()
+        e["shader_clock_mhz"] = _clock_under_load(lambda: ct.batch_matmul_kernel(A, B, C, 128, 128, 64))
         if cpu:
             a = orc.to_julia(d.A); b = orc.to_julia(d.B)
             e["cpu_ms"] = round(_cpu_time(lambda: orc.batch_matmul(a, b, dtype=np.float32), repeats=2), 1)
@@ -244,6 +320,11 @@ def bench_kernels(ct, which, cpu, nruns=NRUNS, warmup=WARMUP):
         e["variant"] = ct.last_variant()
         e["dense_count_flop"] = fmha.metric(d)[0]
         e["tflops_dense_count"] = round(fmha.metric(d)[0] / (e["avg_ms"] * 1e-3) / 1e12, 2)
+        # the reference's timed region is cutile_fmha, which allocates Out (fmha.jl:160,265-267)
+        with_alloc = lambda: fmha.cutile_fmha(d.Q, d.K, d.V, causal=True)
+        with_alloc()
+        e["avg_ms_with_out_alloc"] = round(min(_back_to_back(with_alloc, nruns) for _ in range(2)), 5)
+        e["shader_clock_mhz"] = _clock_under_load(lambda: ct.fmha_kernel(Q, K, V, O, scale, 0, d.d_k, d.heads, 128, 128, 1, True, True))
         if cpu:
             q, k, v = (orc.to_julia(t)[:, :, :, :1] for t in (d.Q, d.K, d.V))
             e["cpu_ms"] = round(_cpu_time(lambda: orc.ref_fmha(q[:, :, :4], k[:, :, :4], v[:, :, :4], causal=True), repeats=2) * 32, 1)
@@ -406,13 +487,20 @@ def bench_kernels(ct, which, cpu, nruns=NRUNS, warmup=WARMUP):
         dev8 = lambda: moe.cutile_moe(d.hidden_states, w1q, w2q, d.topk_weights, d.topk_ids, 128, 128, 64, w1_scale=s1t,
                                       w2_scale=s2t, device_align=True, fuse_silu=True)
         dev8()
+        # two more copies of the e4m3 weights (201 MB each): cycling over three sets touches 400 MB between two
+        # uses of a set, more than the 256 MB memory-side cache keeps
+        copies = [(w1q, w2q)] + [(w1q.clone(), w2q.clone()) for _ in range(2)]
+        cold8 = [(lambda a=a, b=b: moe.cutile_moe(d.hidden_states, a, b, d.topk_weights, d.topk_ids, 128, 128, 64, w1_scale=s1t,
+                                                  w2_scale=s2t, device_align=True, fuse_silu=True)) for a, b in copies]
         try:
             g8, _ = graph_of(dev8)
+            gcold = [graph_of(f)[0].replay for f in cold8]
             res["moe_fp8_device"] = extra(_entry("MoE e4m3 weights top-2, whole cutile_moe on the device (fused SiLU epilogue), HIP graph replay", g8.replay,
-                                                 w8bytes, "GB/s", "hbm", HBM_PEAK_GBS, "fp8 weights / f16 MFMA", nruns, warmup))
+                                                 w8bytes, "GB/s", "hbm", HBM_PEAK_GBS, "fp8 weights / f16 MFMA", nruns, warmup, cold=gcold))
         except Exception as ex:
             res["moe_fp8_device"] = extra(_entry(f"MoE e4m3 weights top-2, device work only (eager; {type(ex).__name__})", dev8,
-                                                 w8bytes, "GB/s", "hbm", HBM_PEAK_GBS, "fp8 weights / f16 MFMA", nruns, warmup))
+                                                 w8bytes, "GB/s", "hbm", HBM_PEAK_GBS, "fp8 weights / f16 MFMA", nruns, warmup, cold=cold8))
+        del copies, cold8
         del d
     torch.cuda.synchronize()
     return res
@@ -513,6 +601,57 @@ def cpu_baseline_headline(sample_rows=4096):
                       "examples' verify() formulas, single-threaded, min of 5 passes"}
 
 
+def _measured_traffic(kernel):
+    """HBM bytes per launch of ``kernel`` from the counter runs recorded under profiles/ (FETCH_SIZE and
+    WRITE_SIZE, scaled as stated there), with the commit they were measured at; (None, None) if absent."""
+    path = os.path.join(ROOT, "profiles", "headline_kernel_hbm_traffic.txt")
+    try:
+        kv = dict(line.split(":", 1) for line in open(path) if ":" in line and not line.startswith("#"))
+        if kernel not in kv.get("kernel", ""):
+            return None, None
+        return int(kv["traffic_bytes_per_launch"].strip()), kv.get("measured_at_commit", "").strip() or None
+    except Exception:
+        return None, None
+
+
+def _host_info():
+    model = None
+    try:
+        for line in open("/proc/cpuinfo"):
+            if line.startswith("model name"):
+                model = line.split(":", 1)[1].strip()
+                break
+    except Exception:
+        pass
+    return {"nproc": os.cpu_count(), "cpu_model": model,
+            "OPENBLAS_NUM_THREADS": os.environ.get("OPENBLAS_NUM_THREADS"), "OMP_NUM_THREADS": os.environ.get("OMP_NUM_THREADS")}
+
+
+# north_star targets: (key in "kernels", figure, target fraction)
+TARGETS = [("vadd", "frac", 0.75), ("layernorm_fwd", "frac_cold", 0.75), ("softmax_tma", "frac_cold", 0.75),
+           ("matmul", "frac", 0.60), ("fmha", "frac", 0.40), ("moe_f16_device_fused", "mfma_frac", 0.40)]
+REPORTED = [("copy_ref", "frac_cold"), ("transpose", "frac"), ("layernorm_bwd", "frac_cold"), ("batchmatmul", "frac"), ("matmul_fp8", "frac"),
+            ("moe_f16_device_fused", "frac"), ("moe_f16", "frac"), ("moe_fp8_device", "frac_cold")]
+
+
+def _summary(kernels):
+    """One compact entry per north_star target (and per reported figure without a target), last in the JSON line."""
+    out = {}
+    for key, fig, target in TARGETS:
+        e = kernels.get(key)
+        if not e or fig not in e:
+            continue
+        peak = 2500.0 if fig == "mfma_frac" else e["peak"]
+        unit = "TFLOP/s" if fig == "mfma_frac" else e["unit"]
+        out[f"{key}.{fig}"] = {"achieved": round(e[fig] * peak, 1), "unit": unit, "frac": e[fig], "target": target,
+                               "pass": bool(e[fig] >= target)}
+    for key, fig in REPORTED:
+        e = kernels.get(key)
+        if e and fig in e:
+            out[f"{key}.{fig}"] = {"achieved": round(e[fig] * e["peak"], 1), "unit": e["unit"], "frac": e[fig], "target": None}
+    return out
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -538,23 +677,28 @@ def main():
     dom = "layer_norm_bwd_dx_partial_dwdb"      # the longest kernel of the step (see stages_ms)
     dom_ms = per_stage["dominant_in_timed_region"]
     ach = work[dom] / (dom_ms * 1e-3) / 1e9
+    traffic, traffic_commit = _measured_traffic(dom)
     out = {
-        "metric": "LayerNorm fwd+bwd + softmax 4096x4096 f32, algorithmic GB/s (the norm/softmax leg of: FMHA/MoE/GEMM TFLOPS + norm/softmax GB/s, % of MI355X roofline; the other legs are under 'kernels')",
+        "metric": "LayerNorm fwd+bwd + softmax 4096x4096 f32, algorithmic GB/s (the norm/softmax leg of: FMHA/MoE/GEMM TFLOPS + norm/softmax GB/s, % of MI355X roofline; the other legs are under 'kernels' and in 'summary')",
         "value": round(total_work / sec_per_step / 1e9, 2), "unit": "GB/s", "n_gpus": 1, "steps": args.steps,
         "warmup": args.warmup, "ms_per_step": round(sec_per_step * 1e3, 5), "higher_is_better": True,
         "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
         "config": {"workload": "configs[1]: row LayerNorm fwd+bwd (y, dx, dgamma, dbeta) + row softmax on 4096x4096 Float32",
-                   "M": 4096, "N": 4096, "eps": 1e-5, "GROUP_SIZE_M": 64, "bytes_per_step": total_work},
+                   "M": 4096, "N": 4096, "eps": 1e-5, "GROUP_SIZE_M": 64, "bytes_per_step": total_work,
+                   "seeds": {"layernorm": 1, "softmax": 2, "matmul": 3, "batchmatmul": 4, "fmha": 5, "moe": 6, "vadd": 0}},
         "roofline": {"bound": "hbm", "achieved": round(ach, 2), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(ach / HBM_PEAK_GBS, 4),
-                     # HBM bytes per launch from rocprofv3 FETCH_SIZE (x2.000) + WRITE_SIZE (x1.000) counter runs,
-                     # calibrated on vadd; summary: profiles/membound_kernels_hbm_traffic_pmc.txt
-                     "traffic": 210371940, "kernel": dom,
+                     # HBM bytes per launch from the rocprofv3 FETCH_SIZE / WRITE_SIZE runs recorded in
+                     # profiles/headline_kernel_hbm_traffic.txt (null if that record is absent)
+                     "traffic": traffic, "traffic_measured_at_commit": traffic_commit, "kernel": dom,
                      "avg_launch_ms": round(dom_ms, 5), "algorithmic_bytes": work[dom]},
         "stages_ms": {k: round(v, 5) for k, v in per_stage.items()},
+        "stages_frac": {k: round(work[k] / (per_stage[k] * 1e-3) / 1e9 / HBM_PEAK_GBS, 4) for k in work if work[k]},
+        "shader_clock_mhz_idle": _shader_clock_mhz(),
     }
     if not args.no_cpu:
         out["cpu_baseline"] = cpu_baseline_headline()
+        out["cpu_baseline"].update(_host_info())
     if args.kernels != "none":
         which = None if args.kernels == "all" else set(args.kernels.split(","))
         out["kernels"] = bench_kernels(ct, which, cpu=not args.no_cpu)
@@ -562,8 +706,11 @@ def main():
         flat = [r for e in out["kernels"].values() for r in e.get("rows", [e])]
         for e in flat:
             cpu = f"  cpu {e['cpu_ms']:10.1f} ms" if "cpu_ms" in e else ""
+            cold = f"  cold {100 * e['frac_cold']:6.2f}%" if "frac_cold" in e else ""
             print(f"{e['name'][:72]:<72} min {e['min_ms']:8.4f}  avg {e['avg_ms']:8.4f} ms  "
-                  f"{e['achieved']:9.1f} {e['unit']:<8} {100 * e['frac']:6.2f}% of {e['bound']} peak{cpu}", file=sys.stderr)
+                  f"{e['achieved']:9.1f} {e['unit']:<8} {100 * e['frac']:6.2f}% of {e['bound']} peak{cold}{cpu}", file=sys.stderr)
+    if "kernels" in out:
+        out["summary"] = _summary(out["kernels"])   # last key: the contract at a glance
     print(json.dumps(out))
 
 

@@ -412,11 +412,15 @@ def bench_kernels(ct, which, cpu, nruns=NRUNS, warmup=WARMUP):
             e["mfma_frac"] = round(e["tflops"] / 2500.0, 5)
             return e
 
-        whole = lambda: moe.cutile_moe(d.hidden_states, d.w1, d.w2, d.topk_weights, d.topk_ids, 128, 128, 64)
-        res["moe_f16"] = extra(_entry("MoE f16 256tok/1024h/32e/2048i top-2, whole cutile_moe (host align + H2D/D2H inside)",
+        whole = lambda: moe.cutile_moe(d.hidden_states, d.w1, d.w2, d.topk_weights, d.topk_ids, 128, 128, 64,
+                                       device_align=False, fuse_silu=False)   # the reference's orchestration, moe.jl:218-257
+        res["moe_f16"] = extra(_entry("MoE f16 256tok/1024h/32e/2048i top-2, cutile_moe as the reference orchestrates it (host sort + H2D/D2H inside, 4 kernels)",
                                       whole, wbytes, "GB/s", "hbm", HBM_PEAK_GBS, "f16", nruns, warmup))
         whole_dev = lambda: moe.cutile_moe(d.hidden_states, d.w1, d.w2, d.topk_weights, d.topk_ids, 128, 128, 64,
-                                           device_align=True)
+                                           device_align=True, fuse_silu=False)
+        default_call = lambda: moe.cutile_moe(d.hidden_states, d.w1, d.w2, d.topk_weights, d.topk_ids, 128, 128, 64)
+        res["moe_f16_default"] = extra(_entry("MoE f16 top-2, cutile_moe with its defaults (token sort on the GPU, SiLU*up fused; eager launches incl. allocations)",
+                                              default_call, wbytes, "GB/s", "hbm", HBM_PEAK_GBS, "f16", nruns, warmup))
         res["moe_f16_device_align"] = extra(_entry("MoE f16 top-2, whole cutile_moe with the token sort on the GPU (no host round trip; eager launches)",
                                                    whole_dev, wbytes, "GB/s", "hbm", HBM_PEAK_GBS, "f16", nruns, warmup))
         dev = whole_dev

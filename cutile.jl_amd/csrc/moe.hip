@@ -16,6 +16,7 @@
 // f16 on their way into LDS (every e4m3 value is exact in f16) and scaled in the epilogue.
 #include "common.h"
 #include <math.h>
+#include <type_traits>
 
 namespace {
 
@@ -90,6 +91,16 @@ __device__ __forceinline__ float silu_mul(float x, float y) {
 
 constexpr int kTT = 32;   // token slots per workgroup (one MFMA row tile)
 
+// Workgroup barrier that waits for the wave's LDS accesses only (lgkmcnt(0); vmcnt and expcnt at their
+// maxima).  __syncthreads() also waits for every global load in flight, which would turn the weight
+// tiles requested one and two steps ahead into synchronous loads.
+__device__ __forceinline__ void lds_barrier() {
+    asm volatile("" ::: "memory");
+    __builtin_amdgcn_s_waitcnt(0xc07f);
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+}
+
 // E: activation/output element traits; W8: weights are E4M3FN bytes (else same type as A).
 // NTW: waves side by side along n (workgroup strip = 32*NTW channels); the other 4/NTW waves
 // split each K step between them and their accumulators are added through LDS at the end.
@@ -108,7 +119,11 @@ constexpr int kTT = 32;   // token slots per workgroup (one MFMA row tile)
 // TS: 32-slot tiles of one expert block that a workgroup multiplies with the same weight tile
 // (wide shapes only).  With more than 32 tokens per expert TS = 2 streams an expert's weights once
 // per 64 tokens instead of once per 32, at the price of one workgroup per CU less.
-template <typename E, bool W8, int NTW, int kKT, bool SILU = false, int TS = 1>
+// FAST: the workgroup's tiles lie wholly inside the arrays and everything is 16-byte aligned (checked on
+// the host for the whole launch): loads without predicates.  A compile-time property, because with both
+// load paths in one loop body the compiler has to wait for every outstanding load at their join, which
+// empties the look-ahead.
+template <typename E, bool W8, int NTW, int kKT, bool SILU = false, int TS = 1, bool FAST = false>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(TS == 1 ? 4 : 3))) void fused_moe_kernel(
     const unsigned short* __restrict__ A, int64_t lda, int num_a_cols, const void* __restrict__ Bv, int64_t ldb,
     int64_t sbe, unsigned short* __restrict__ C, int64_t ldc, int total_tokens,
@@ -172,11 +187,14 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(TS == 1 ? 4
     constexpr int CPRB = kKT / EPB;         // 16-byte global chunks per weight row
     constexpr int NB = kNT * CPRB / 256;    // weight chunks per thread
     constexpr int NA = kTTS * CPR / 256;    // A chunks per thread
-    // Two staging sets for the e4m3 path (its raw tiles are half the size, so two tiles per
-    // workgroup can be in flight at the register cost of one f16 tile); one set otherwise.
-    constexpr int DEPTH = W8 ? 2 : 1;
-    u32x4 breg0[NB], breg1[DEPTH == 2 ? NB : 1];
-    s16x8 areg0[NA], areg1[DEPTH == 2 ? NA : 1];
+    // One staging set: the tile of the next step is requested right after this step's tile has gone to LDS
+    // and is waited for at the next step's LDS write.  Keeping two weight tiles per workgroup in flight was
+    // measured and is markedly slower (52 us against 29 us for the down projection; 46 against 27 us for
+    // the e4m3 gate / up projection): four workgroups per CU already have 64 to 128 KB per CU in flight, and
+    // twice that is the whole L2 of an XCD in outstanding lines.
+    constexpr int DEPTH = 1;
+    u32x4 breg0[NB];
+    s16x8 areg0[NA];
     int a_col[NA];
 #pragma unroll
     for (int i = 0; i < NA; ++i) {
@@ -196,20 +214,15 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(TS == 1 ? 4
     // predicated load is waited for before the other side of its branch may write the same
     // registers, which would leave a lane with one load in flight at a time.  Slots without a token
     // read column 0 there; their accumulator rows are never stored.
-    const bool fast = vecA && vecB && K % kKT == 0 && (SILU ? n0 + kNT / 2 <= half_n : n0 + kNT <= N);
-    auto load_tiles = [&](int k0, u32x4* breg, s16x8* areg) {
-        if (fast) {
+    constexpr bool fast = FAST;
+    auto load_b = [&](int k0, u32x4* breg) {
+        if constexpr (fast) {
 #pragma unroll
             for (int i = 0; i < NB; ++i) {
                 const int id = tid + 256 * i, n = id / CPRB, c = id % CPRB;
                 const int64_t off = k0 + EPB * c + (int64_t)row_of(n) * ldb;
                 breg[i] = W8 ? __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(B8 + off))
                              : __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(B16 + off));
-            }
-#pragma unroll
-            for (int i = 0; i < NA; ++i) {
-                const int gk = k0 + 8 * ((tid + 256 * i) % CPR);
-                areg[i] = *reinterpret_cast<const s16x8*>(A + gk + (int64_t)(a_col[i] < 0 ? 0 : a_col[i]) * lda);
             }
             return;
         }
@@ -235,6 +248,16 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(TS == 1 ? 4
             }
             breg[i] = v;
         }
+    };
+    auto load_a = [&](int k0, s16x8* areg) {
+        if constexpr (fast) {
+#pragma unroll
+            for (int i = 0; i < NA; ++i) {
+                const int gk = k0 + 8 * ((tid + 256 * i) % CPR);
+                areg[i] = *reinterpret_cast<const s16x8*>(A + gk + (int64_t)(a_col[i] < 0 ? 0 : a_col[i]) * lda);
+            }
+            return;
+        }
 #pragma unroll
         for (int i = 0; i < NA; ++i) {
             s16x8 v = {0};
@@ -254,9 +277,26 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(TS == 1 ? 4
     // 8-byte fragment reads of 32 lanes (rows n .. n+31, one half) cover all 64 banks exactly once.
     auto b_sw = [](int n) { return kKT == 128 ? ((n >> 1) & 7) : (n & 15); };
 
-    // One K step: staged tile -> LDS, refill the staging set with the tile DEPTH steps ahead, MFMAs.
-    auto step = [&](int k0, u32x4* breg, s16x8* areg) {
-        __syncthreads();
+    // One K step: staged tiles -> LDS, refill the weight staging set with the tile DEPTH steps ahead and the
+    // activation set with the next tile, MFMAs.
+    // The K tiles are walked from a start that differs from workgroup to workgroup (and wraps): workgroups
+    // that run at the same time would otherwise all read the same few hundred bytes of every weight row
+    // at the same moment, i.e. the same slice of every 4 KB of address space.
+    const int nsteps = (K + kKT - 1) / kKT;
+    // (the narrow shape only: 27.9 against 29.5 us there, 49 against 45 us on the wide shape)
+    const int rot = NTW == 1 ? (int)((unsigned)(3 * expert + grp) % (unsigned)nsteps) : 0;   // (not a function of the strip: the fused-SiLU and the plain kernel then add in the same order)
+    auto k_of = [&](int it) {
+        int st = it + rot;
+        if (st >= nsteps) st -= nsteps;
+        return st * kKT;
+    };
+    // LB / LA: this step requests a weight tile / an activation tile.  Compile-time, and the loops below are
+    // peeled accordingly: after a load that is issued under a run-time condition the compiler has to assume
+    // the older loads are the youngest ones in flight and waits for everything.
+    auto step = [&](int it, u32x4* breg, auto lb, auto la) {
+        constexpr bool LB = decltype(lb)::value, LA = decltype(la)::value;
+        s16x8* areg = areg0;
+        lds_barrier();   // the previous step's fragment reads are done
 #pragma unroll
         for (int i = 0; i < NB; ++i) {
             const int id = tid + 256 * i, n = id / CPRB, c = id % CPRB;
@@ -273,8 +313,12 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(TS == 1 ? 4
             const int id = tid + 256 * i, sl = id / CPR, c = id % CPR;
             *reinterpret_cast<s16x8*>(&As[sl * kKT + 8 * (c ^ (sl & 15))]) = areg[i];
         }
-        __syncthreads();
-        if (k0 + DEPTH * kKT < K) load_tiles(k0 + DEPTH * kKT, breg, areg);
+        lds_barrier();
+        // (activations first: loads return in order, and the next step needs its activations together with a
+        // weight tile requested a step earlier -- were the activations the youngest request, waiting for
+        // them would also wait for the weight tile of the step after)
+        if constexpr (LA) load_a(k_of(it + 1), areg);
+        if constexpr (LB) load_b(k_of(it + DEPTH), breg);
 #pragma unroll
         for (int kq = 0; kq < kKT / 16 / KW; ++kq) {
             const int ks = wk * (kKT / 16 / KW) + kq;
@@ -299,15 +343,14 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(TS == 1 ? 4
             }
         }
     };
-    load_tiles(0, breg0, areg0);
-    if (DEPTH == 2) {
-        if (kKT < K) load_tiles(kKT, breg1, areg1);
-        for (int k0 = 0; k0 < K; k0 += 2 * kKT) {
-            step(k0, breg0, areg0);
-            if (k0 + kKT < K) step(k0 + kKT, breg1, areg1);
-        }
-    } else {
-        for (int k0 = 0; k0 < K; k0 += kKT) step(k0, breg0, areg0);
+    load_a(k_of(0), areg0);
+    load_b(k_of(0), breg0);
+    using Y = std::true_type;
+    using No = std::false_type;
+    {
+        int it = 0;
+        for (; it + 1 < nsteps; ++it) step(it, breg0, Y{}, Y{});
+        step(it, breg0, No{}, No{});
     }
     if (KW > 1) {  // add the K-split partial accumulators: wave (wn, wk) -> wave (wn, 0), one slot tile at a time
         float* red = reinterpret_cast<float*>(Bs_raw);  // 4 waves x 64 lanes x 16 floats = 16 KB <= sizeof(Bs_raw)
@@ -485,7 +528,15 @@ static int fused_moe_impl(const mi_tile_array* A, const mi_tile_array* B, const 
     const bool vecB = aligned(B->ptr, 16) && B->strides[1] % (w8 ? 16 : 8) == 0 && B->strides[2] % (w8 ? 16 : 8) == 0;
     dim3 grid((unsigned)(tiles / ts * n_blocks));
     hipStream_t s = (hipStream_t)stream;
-#define LAUNCH(ET, W8, NTW, KT, ...)                                                                                \
+    // every tile of the launch inside the arrays and 16-byte aligned: the kernels without load predicates
+    const int kt = narrow ? 256 : 128;
+    const bool fast = vecA && vecB && K % kt == 0 && (silu ? (N / 2) % 64 == 0 : N % (narrow ? 32 : 128) == 0);
+#define LAUNCH(ET, W8, NTW, KT, SILU, TS)                                                                           \
+    do {                                                                                                            \
+        if (fast) LAUNCH1(ET, W8, NTW, KT, SILU, TS, true);                                                         \
+        else LAUNCH1(ET, W8, NTW, KT, SILU, TS, false);                                                             \
+    } while (0)
+#define LAUNCH1(ET, W8, NTW, KT, ...)                                                                               \
     hipLaunchKernelGGL((fused_moe_kernel<ET, W8, NTW, KT, ##__VA_ARGS__>), grid, dim3(256), 0, s, (const unsigned short*)A->ptr, \
                        A->strides[1], (int)A->sizes[1], (const void*)B->ptr, B->strides[1], B->strides[2],          \
                        (unsigned short*)C->ptr, C->strides[1], (int)total, (const unsigned short*)topk_weights->ptr, \
@@ -495,10 +546,10 @@ static int fused_moe_impl(const mi_tile_array* A, const mi_tile_array* B, const 
 #define LAUNCH_SHAPE(ET, W8)                                  \
     do {                                                      \
         if (silu && ts == 2) LAUNCH(ET, W8, 4, 128, true, 2); \
-        else if (silu) LAUNCH(ET, W8, 4, 128, true);          \
-        else if (narrow) LAUNCH(ET, W8, 1, 256);              \
+        else if (silu) LAUNCH(ET, W8, 4, 128, true, 1);       \
+        else if (narrow) LAUNCH(ET, W8, 1, 256, false, 1);    \
         else if (ts == 2) LAUNCH(ET, W8, 4, 128, false, 2);   \
-        else LAUNCH(ET, W8, 4, 128);                          \
+        else LAUNCH(ET, W8, 4, 128, false, 1);                \
     } while (0)
     if (A->dtype == MI_F16) {
         if (w8) LAUNCH_SHAPE(F16, true);
@@ -509,6 +560,7 @@ static int fused_moe_impl(const mi_tile_array* A, const mi_tile_array* B, const 
     }
 #undef LAUNCH_SHAPE
 #undef LAUNCH
+#undef LAUNCH1
     if (silu && ts == 2) set_variant(w8 ? "fused_moe_silu_t64_n64x2_k128_w8a16" : "fused_moe_silu_t64_n64x2_k128");
     else if (silu) set_variant(w8 ? "fused_moe_silu_t32_n64x2_k128_w8a16" : "fused_moe_silu_t32_n64x2_k128");
     else if (narrow) set_variant(w8 ? "fused_moe_t32_n32_k256_ksplit4_w8a16" : "fused_moe_t32_n32_k256_ksplit4");

@@ -30,14 +30,16 @@ def invoke_silu_and_mul_kernel(AB, C):
 
 
 def cutile_moe(hidden_states, w1, w2, topk_weights, topk_ids, tile_m, tile_n, tile_k, *, w1_scale=None,
-               w2_scale=None, aligned=None, device_align=False, fuse_silu=False):
+               w2_scale=None, aligned=None, device_align=True, fuse_silu=True):
     """moe.jl:218-257.  Torch shapes (reversed Julia): hidden_states (tokens, hidden); w1
     (E, 2*inter, hidden); w2 (E, hidden, inter); topk_weights / topk_ids (topk, tokens), ids
     1-based int64.  ``aligned`` may carry a precomputed (sorted_token_ids, sorted_expert_ids)
-    pair on the device to skip the host round trip of moe.jl:232-233; ``device_align`` sorts on
-    the GPU instead (fixed-capacity outputs, nothing leaves the device).  ``fuse_silu`` runs the
-    gate / up GEMM with SiLU * up as its epilogue: cache1 and the silu_and_mul launch disappear,
-    the result is bit-identical."""
+    pair on the device to skip the token sort; ``device_align`` (default) sorts on the GPU
+    (fixed-capacity outputs, nothing leaves the device), ``device_align=False`` is the reference's
+    orchestration with the host round trip of moe.jl:232-233.  ``fuse_silu`` (default) runs the gate / up
+    GEMM with SiLU * up as its epilogue: cache1 and the silu_and_mul launch disappear;
+    ``fuse_silu=False`` launches the kernels one by one as moe.jl:234-251 does.  All four combinations
+    give bit-identical results."""
     num_tokens, hidden_size = hidden_states.shape
     num_experts, _, intermediate_size = w2.shape
     topk = topk_ids.shape[0]

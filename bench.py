@@ -510,6 +510,77 @@ def bench_kernels(ct, which, cpu, nruns=NRUNS, warmup=WARMUP):
     return res
 
 
+def parity_errors(ct):
+    """Achieved error of every benchmark configuration against the float64 oracle, on the same seeded inputs
+    the timing legs use (bounded samples where the CPU side would otherwise take minutes).  Per
+    configuration: max_abs; max_rel_scale = max|err| / max|ref|; max_rel_elem = max |err| / |ref| over the
+    elements with |ref| >= 1e-3 max|ref|; the tolerance the configuration states and whether it holds in
+    the form the tests use, |err| <= tol * (|ref| + max|ref|)."""
+    import numpy as np
+    import torch
+    from oracle import cutile_oracle as orc
+    from cutile_jl_amd.examples import vadd, layernorm, softmax, matmul, batchmatmul, fmha, moe
+    J = orc.to_julia
+    out = {}
+
+    def rec(name, got, ref, tol, sample):
+        got = np.asarray(got, dtype=np.float64); ref = np.asarray(ref, dtype=np.float64)
+        err = np.abs(got - ref)
+        scale = float(np.abs(ref).max())
+        big = np.abs(ref) >= 1e-3 * scale
+        out[name] = {"max_abs": float(err.max()), "max_rel_scale": float(err.max() / scale) if scale else 0.0,
+                     "max_rel_elem": float((err[big] / np.abs(ref[big])).max()) if big.any() else 0.0,
+                     "tol": tol, "pass": bool(np.all(err <= tol * (np.abs(ref) + scale))) if tol else bool(err.max() == 0.0),
+                     "sample": sample}
+
+    d = vadd.prepare(benchmark=True)
+    r = vadd.run(d)
+    n = 1 << 24
+    rec("vadd 2^27 f32 (bit-exact)", r.c[:n].cpu().numpy(), d.a[:n].cpu().numpy() + d.b[:n].cpu().numpy(), 0.0, "first 2^24 elements")
+    del d, r
+    d = layernorm.prepare(benchmark=True)
+    r = layernorm.run(d)
+    X, W, B, DY = J(d.X), J(d.W), J(d.B), J(d.DY)
+    Y, mean, rstd = orc.layer_norm_fwd(X, W, B, d.eps)
+    rec("LayerNorm fwd y", J(r.Y), Y, 1e-5, "all 4096 rows")
+    del Y
+    DX, DW, DB = orc.layer_norm_bwd(X, W, DY, d.eps)
+    rec("LayerNorm bwd dx", J(r.DX), DX, 1e-5, "all 4096 rows")
+    rec("LayerNorm bwd dgamma", J(r.FINAL_DW), DW, 1e-5, "all 4096 channels")
+    rec("LayerNorm bwd dbeta", J(r.FINAL_DB), DB, 1e-5, "all 4096 channels")
+    del DX
+    del d, r, X, DY
+    d = softmax.prepare(benchmark=True)
+    r = softmax.run(d)
+    rec("softmax", J(r.output_tma)[:, :256], orc.softmax(J(d.input)[:, :256]), 1e-5, "256 of 4096 columns")
+    del d, r
+    d = matmul.prepare(benchmark=True, T=torch.float16, out_T=torch.float32, dist="normal64")
+    r = matmul.run(d)
+    A = J(d.A).astype(np.float64); Bm = J(d.B).astype(np.float64)
+    rws = [0, 1, 255, 256, 2049, 4095]
+    rec("GEMM 4096^3 f16 -> f32", J(r.C)[rws], A[rws] @ Bm, 2e-2, "6 of 4096 rows of C")
+    del d, r, A, Bm
+    d = batchmatmul.prepare(benchmark=True)
+    r = batchmatmul.run(d)
+    rec("batched GEMM f32", J(r.C)[:, :, 0], J(d.A)[:, :, 0].astype(np.float64) @ J(d.B)[:, :, 0].astype(np.float64), 1e-5, "batch entry 1 of 8")
+    del d, r
+    d = fmha.prepare(benchmark=True)
+    r = fmha.run(d)
+    Q, K, V = (J(t)[:, :, :4, :1] for t in (d.Q, d.K, d.V))
+    rec("causal FMHA f16", J(r.out)[:, :, :4, :1], orc.ref_fmha(Q, K, V, causal=True, dtype=np.float64), 2e-2, "4 of 128 (batch, head) pairs")
+    del d, r
+    d = moe.prepare(benchmark=True, topk=2, router="top2_logits")
+    got = moe.cutile_moe(d.hidden_states, d.w1, d.w2, d.topk_weights, d.topk_ids, 128, 128, 64)
+    rec("MoE f16 top-2", J(got), orc.ref_moe(J(d.hidden_states), J(d.w1), J(d.w2), J(d.topk_weights), J(d.topk_ids), dtype=np.float32), 2e-2, "whole output")
+    q = moe.quantize_weights(d)
+    got = moe.cutile_moe(d.hidden_states, q.w1, q.w2, d.topk_weights, d.topk_ids, 128, 128, 64, w1_scale=q.w1_scale, w2_scale=q.w2_scale)
+    w1d = orc.e4m3fn_decode(J(q.w1.view(torch.uint8))) * J(q.w1_scale)[None]
+    w2d = orc.e4m3fn_decode(J(q.w2.view(torch.uint8))) * J(q.w2_scale)[None]
+    rec("MoE e4m3 weights top-2 (vs ref_moe on the dequantised weights)", J(got),
+        orc.ref_moe(J(d.hidden_states), w1d, w2d, J(d.topk_weights), J(d.topk_ids), dtype=np.float32), 2e-2, "whole output")
+    return out
+
+
 def headline(ct, steps, warmup):
     """configs[1]: LayerNorm fwd+bwd and softmax on 4096x4096 fp32.  Returns seconds per step,
     per-stage average durations from events inside the timed region, and algorithmic bytes."""
@@ -703,6 +774,7 @@ def main():
     if not args.no_cpu:
         out["cpu_baseline"] = cpu_baseline_headline()
         out["cpu_baseline"].update(_host_info())
+        out["errors"] = parity_errors(ct)
     if args.kernels != "none":
         which = None if args.kernels == "all" else set(args.kernels.split(","))
         out["kernels"] = bench_kernels(ct, which, cpu=not args.no_cpu)

@@ -16,6 +16,7 @@ plausible mistake fails a test) is listed in ``tests/test_oracle.py``; summary:
 function               pinned by
 =====================  ======================================================================
 vadd, transpose        closed form (IEEE add / permutation); brute force
+vadd_gather            out-of-bounds known answer of test/device/gather_scatter.jl:75-113; scalar loops
 swizzle_2d             bijection onto the tile grid, brute force; C restatement cross-check
 matmul, batch_matmul   float64 ``@``; 64x16x64 case of test/device/tile.jl:1036-1066 by loops
 layer_norm_*           invariants (zero-mean/unit-var xhat, sum dx = 0, constant row);
@@ -34,8 +35,10 @@ tiled_mapreduce        known answers of test/host/mapreduce.jl (count == 4, any 
 jl_promote             Julia's documented promotion facts (Int32+Int64 -> Int64, Int64+Float32 ->
                        Float32, Float16+Float32 -> Float32, Bool yields, true + true == 2)
 philox2x32, rng_fill   Random123's published known-answer vectors for philox2x32 (7 and 10 rounds);
-                       slot layout by brute-force loops; the reference's own properties
-                       (test/device/random.jl:421-526: uniqueness, disjoint streams, counter carry)
+                       slot layout by brute-force loops, for rand! and for randn! / randexp! (which word
+                       feeds the radius and which the angle, sine / cosine slots, the Float64 counter
+                       pairing); the reference's own properties (test/device/random.jl:421-526:
+                       uniqueness, disjoint streams, counter carry)
 e4m3fn codec           16 round-trip vectors and fma vectors of
                        test/extensions/DLFP8Types.jl:126-141; all 256 codes vs torch.float8_e4m3fn
 e5m2 codec             the same 16 round-trip vectors (DLFP8Types.jl:126-134); all 256 codes and

@@ -61,13 +61,19 @@ def test_vadd_strided_views_and_misaligned(ct, orc):
     assert torch.equal(C[:, :100], A[:, :100] + B[:, :100]) and torch.all(C[:, 100:] == 0)
 
 
-def test_vadd_gather_out_of_bounds_semantics(ct):
+def test_vadd_gather_out_of_bounds_semantics(ct, orc):
     """test/device/gather_scatter.jl:75-113: an out-of-bounds gather lane reads 0, an
     out-of-bounds scatter lane is dropped."""
     a = torch.ones(16, device="cuda"); b = torch.full((32,), 2.0, device="cuda")
     c = torch.zeros(32, device="cuda")
     ct.vec_add_kernel_1d_gather(a, b, c, 32)
     assert torch.all(c[:16] == 3.0) and torch.all(c[16:] == 2.0)
+    rng = np.random.default_rng(8)
+    for na, nb, nc, tile in [(1000, 700, 1500, 256), (33, 1025, 1024, 1024), (5000, 5000, 4097, 512)]:
+        x = torch.from_numpy(rng.random(na, dtype=np.float32)).cuda(); y = torch.from_numpy(rng.random(nb, dtype=np.float32)).cuda()
+        z = torch.full((nc,), -1.0, device="cuda")
+        ct.vec_add_kernel_1d_gather(x, y, z, tile)
+        assert np.array_equal(z.cpu().numpy(), orc.vadd_gather(x.cpu().numpy(), y.cpu().numpy(), nc))
     guard = torch.zeros(48, device="cuda")
     c_small = guard[:16]
     ct.vec_add_kernel_1d_gather(b, b, c_small, 32)
@@ -198,7 +204,7 @@ def test_layernorm_fwd_bwd(orc, M, N, TILE_N, G):
     close_f32(orc.to_julia(r.Y), Y)
     close_f32(orc.to_julia(r.Mean), mean, tol=1e-5 if N > 1 else 1e-5)
     close_f32(orc.to_julia(r.Rstd), rstd)
-    close_f32(orc.to_julia(r.DX), DX, tol=2e-5)
+    close_f32(orc.to_julia(r.DX), DX)
     close_f32(orc.to_julia(r.FINAL_DW), DW)
     close_f32(orc.to_julia(r.FINAL_DB), DB)
     # the reference's own criterion (layernorm.jl:299,311-313)
@@ -234,7 +240,7 @@ def test_layernorm_full_size(orc):
     DX, DW, DB = orc.layer_norm_bwd(X, W, DY, d.eps)
     close_f32(orc.to_julia(r.Y), Y)
     close_f32(orc.to_julia(r.Rstd), rstd)
-    close_f32(orc.to_julia(r.DX), DX, tol=2e-5)
+    close_f32(orc.to_julia(r.DX), DX)
     close_f32(orc.to_julia(r.FINAL_DW), DW)
     close_f32(orc.to_julia(r.FINAL_DB), DB)
 

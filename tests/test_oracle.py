@@ -484,6 +484,18 @@ def test_tiled_mapreduce_reference_cases_and_brute_force(orc):
     assert orc.tiled_mapreduce(None, "add_sum", A, init=100.0)[0] == pytest.approx(100 + A.astype(np.float64).sum(), rel=1e-6)
 
 
+def test_vadd_gather_out_of_bounds_by_brute_force():
+    """vec_add_kernel_1d_gather with arrays of different lengths: an out-of-bounds gather lane reads 0
+    and an out-of-bounds scatter lane is dropped (test/device/gather_scatter.jl:75-113: the lanes past
+    the end of the source come back as 0.0).  Element by element with scalar loops."""
+    assert orc.vadd_gather(np.ones(16, np.float32), np.full(32, 2.0, np.float32), 32).tolist() == [3.0] * 16 + [2.0] * 16
+    rng = np.random.default_rng(3)
+    for na, nb, nc in [(5, 9, 7), (9, 5, 12), (0, 3, 4), (6, 6, 6), (10, 2, 1)]:
+        a = rng.random(na).astype(np.float32); b = rng.random(nb).astype(np.float32)
+        want = [(a[i] if i < na else np.float32(0)) + (b[i] if i < nb else np.float32(0)) for i in range(nc)]
+        assert orc.vadd_gather(a, b, nc).tolist() == [float(w) for w in want]
+
+
 # ---- Philox2x32-7 RNG fills -----------------------------------------------------------------------
 
 def test_philox2x32_random123_known_answers(orc):
@@ -531,6 +543,47 @@ def test_rng_fill_layout_by_brute_force(orc):
     assert orc.rng_fill("u16", n, seed, counter).tolist() == want16[:n]
     assert orc.rng_fill("u8", n, seed, counter).tolist() == want8[:n]
     assert np.array_equal(orc.rng_fill("i32", n, seed, counter).view(np.uint32), orc.rng_fill("u32", n, seed, counter))
+
+
+def test_randn_randexp_layout_by_brute_force(orc):
+    """Which Philox word feeds what in randn! / randexp!, element by element with scalar loops and
+    ``math`` in double precision.  32-bit class (src/language/random.jl:369-380,420-441): call i of a
+    block gives (c1, c2); the radius comes from c2, r = sqrt(-2 log u01(c2)), the angle from c1,
+    2 pi u01(c1); slot i takes r sin, slot 256 + i takes r cos.  Float64 (:386-398,449-480): u1 packs
+    the two words of counter i, u2 those of counter 256 + i; the radius comes from u1 and the angle
+    from u2.  randexp (:500-501) is -log of the rand! value of the same slot.  Swapping the two words,
+    the sine and cosine slots or the counter pairing changes every value; the oracle computes the 32-bit
+    class in Float32, hence the tolerance."""
+    seed, counter, n = 0xCAFEF00D, 0xFFFFFF80, 600          # two blocks, the second partial; the counter wraps
+
+    def call(b, i):
+        key = ((b * orc.PHILOX_W) & 0xFFFFFFFF) ^ seed
+        a, c = orc.philox2x32([(counter + i) & 0xFFFFFFFF], [0], [key])
+        return int(a[0]), int(c[0])
+    u32 = lambda w: w * 2.0 ** -32 + 2.0 ** -33                                   # u01(Float32, ::UInt32), :136-142
+    u64 = lambda w: ((w >> 12) | 1) * 2.0 ** -52                                  # u01(Float64, ::UInt64), :169-174
+    want32, want64 = [0.0] * 1024, [0.0] * 1024
+    for b in range(2):
+        for i in range(256):
+            c1, c2 = call(b, i)
+            r, ang = math.sqrt(-2.0 * math.log(u32(c2))), 2.0 * math.pi * u32(c1)
+            want32[512 * b + i], want32[512 * b + 256 + i] = r * math.sin(ang), r * math.cos(ang)
+            a1, a2 = call(b, i)
+            b1, b2 = call(b, 256 + i)
+            r, ang = math.sqrt(-2.0 * math.log(u64(a1 | (a2 << 32)))), 2.0 * math.pi * u64(b1 | (b2 << 32))
+            want64[512 * b + i], want64[512 * b + 256 + i] = r * math.sin(ang), r * math.cos(ang)
+    got32 = orc.rng_fill("f32", n, seed, counter, "randn").astype(np.float64)
+    np.testing.assert_allclose(got32, want32[:n], rtol=0, atol=2e-5)            # Float32 evaluation of values up to 6.8
+    np.testing.assert_allclose(orc.rng_fill("f64", n, seed, counter, "randn"), want64[:n], rtol=0, atol=1e-12)
+    np.testing.assert_allclose(orc.rng_fill("f16", n, seed, counter, "randn").astype(np.float64), want32[:n], rtol=2e-3, atol=1e-3)
+    # randexp: minus the logarithm of the uniform value in the same slot
+    uni32 = orc.rng_fill("f32", n, seed, counter).astype(np.float64)
+    np.testing.assert_allclose(orc.rng_fill("f32", n, seed, counter, "randexp"), [-math.log(u) for u in uni32], rtol=1e-6, atol=1e-7)
+    uni64 = orc.rng_fill("f64", n, seed, counter)
+    np.testing.assert_allclose(orc.rng_fill("f64", n, seed, counter, "randexp"), [-math.log(u) for u in uni64], rtol=1e-14)
+    # and the uniform floats themselves sit where the raw words do (slot layout of rand!, :262-305)
+    raw = orc.rng_fill("u32", n, seed, counter)
+    np.testing.assert_allclose(uni32, [u32(int(w)) for w in raw], rtol=1e-7)
 
 
 def test_rng_float_conversions_and_reference_properties(orc):

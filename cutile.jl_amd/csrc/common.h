@@ -90,7 +90,7 @@ namespace mi {
 
 constexpr int kWave = 64;
 
-// ---- wave64 reductions (DPP row ops + cross-row permutes via __shfl_xor) --------------
+// ---- wave64 reductions (six butterfly steps of __shfl_xor) -------------------------------
 template <typename T, typename Op>
 __device__ __forceinline__ T wave_reduce(T v, Op op) {
 #pragma unroll

@@ -20,6 +20,7 @@
 // Too few outputs to fill 256 CUs: the reduced range is split over P workgroups that write
 // partials to the caller's workspace and the same kernel shape reduces the P partials (two passes,
 // fixed order, no atomics -- results are reproducible, unlike src/mapreduce.jl:91-108).
+#include <dlfcn.h>
 #include <hip/hiprtc.h>
 #include <mutex>
 #include <string>
@@ -39,44 +40,95 @@ std::unordered_map<std::string, hipFunction_t> g_cache;   // key: device id + ge
 bool g_dry_run = false;                                   // compile only: no module load, no launch
 int g_compiles = 0;
 
+// hiprtc is loaded on first use, so that the ahead-of-time entry points of the library do not depend on
+// libhiprtc.so being present; only the Tiled entry points need it.
+struct Rtc {
+    decltype(&hiprtcCreateProgram) create = nullptr;
+    decltype(&hiprtcCompileProgram) compile = nullptr;
+    decltype(&hiprtcGetProgramLogSize) log_size = nullptr;
+    decltype(&hiprtcGetProgramLog) log = nullptr;
+    decltype(&hiprtcGetCodeSize) code_size = nullptr;
+    decltype(&hiprtcGetCode) code = nullptr;
+    decltype(&hiprtcDestroyProgram) destroy = nullptr;
+    decltype(&hiprtcGetErrorString) error_string = nullptr;
+    bool ok = false;
+};
+const Rtc& rtc() {
+    static const Rtc r = [] {
+        Rtc t;
+        void* h = nullptr;
+        for (const char* name : {"libhiprtc.so", "libhiprtc.so.7", "/opt/rocm/lib/libhiprtc.so"}) {
+            h = dlopen(name, RTLD_NOW | RTLD_GLOBAL);
+            if (h) break;
+        }
+        if (!h) return t;
+#define SYM(field, name) t.field = reinterpret_cast<decltype(t.field)>(dlsym(h, #name))
+        SYM(create, hiprtcCreateProgram);
+        SYM(compile, hiprtcCompileProgram);
+        SYM(log_size, hiprtcGetProgramLogSize);
+        SYM(log, hiprtcGetProgramLog);
+        SYM(code_size, hiprtcGetCodeSize);
+        SYM(code, hiprtcGetCode);
+        SYM(destroy, hiprtcDestroyProgram);
+        SYM(error_string, hiprtcGetErrorString);
+#undef SYM
+        t.ok = t.create && t.compile && t.log_size && t.log && t.code_size && t.code && t.destroy && t.error_string;
+        return t;
+    }();
+    return r;
+}
+
 int compile(const std::string& gen, const char* kernel, hipFunction_t* fn) {
     int dev = 0;
     if (!g_dry_run && hipGetDevice(&dev) != hipSuccess) return (int)hipGetLastError();
     const std::string key = std::to_string(dev) + "#" + gen;
-    std::lock_guard<std::mutex> lock(g_mu);
-    auto it = g_cache.find(key);
-    if (it != g_cache.end()) { *fn = it->second; return MI_OK; }
+    bool dry;
+    {
+        std::lock_guard<std::mutex> lock(g_mu);
+        auto it = g_cache.find(key);
+        if (it != g_cache.end()) { *fn = it->second; return MI_OK; }
+        dry = g_dry_run;
+    }
+    // The compilation itself (a few tenths of a second) runs outside the lock: other threads keep launching
+    // the kernels they already have.  Two threads that meet the same new expression both compile it; the
+    // first to finish enters the cache.
+    const Rtc& R = rtc();
+    if (!R.ok) {
+        fprintf(stderr, "libmi355tile: libhiprtc.so could not be loaded; the Tiled entry points need it\n");
+        return MI_E_UNSUPPORTED;
+    }
     const std::string src = std::string(kDevicePreamble) + gen;
     if (getenv("MI_TILED_DUMP")) fprintf(stderr, "%s\n", gen.c_str());
     hiprtcProgram prog;
-    if (hiprtcCreateProgram(&prog, src.c_str(), "mi_tiled.hip", 0, nullptr, nullptr) != HIPRTC_SUCCESS) return MI_E_UNSUPPORTED;
+    if (R.create(&prog, src.c_str(), "mi_tiled.hip", 0, nullptr, nullptr) != HIPRTC_SUCCESS) return MI_E_UNSUPPORTED;
     const char* opts[] = {"--offload-arch=gfx950", "-O3", "-std=c++17", "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"};
-    const hiprtcResult rc = hiprtcCompileProgram(prog, (int)(sizeof(opts) / sizeof(opts[0])), opts);
+    const hiprtcResult rc = R.compile(prog, (int)(sizeof(opts) / sizeof(opts[0])), opts);
     if (rc != HIPRTC_SUCCESS) {
         size_t n = 0;
-        hiprtcGetProgramLogSize(prog, &n);
+        R.log_size(prog, &n);
         std::string log(n, '\0');
-        if (n) hiprtcGetProgramLog(prog, &log[0]);
+        if (n) R.log(prog, &log[0]);
         fprintf(stderr, "libmi355tile: run-time compilation failed (%s)\n%s\n---- generated source ----\n%s\n",
-                hiprtcGetErrorString(rc), log.c_str(), gen.c_str());
-        hiprtcDestroyProgram(&prog);
+                R.error_string(rc), log.c_str(), gen.c_str());
+        R.destroy(&prog);
         return MI_E_UNSUPPORTED;
     }
-    ++g_compiles;
     hipFunction_t f = nullptr;
-    if (!g_dry_run) {
+    if (!dry) {
         size_t n = 0;
-        hiprtcGetCodeSize(prog, &n);
+        R.code_size(prog, &n);
         std::string code(n, '\0');
-        hiprtcGetCode(prog, &code[0]);
+        R.code(prog, &code[0]);
         hipModule_t mod;
         hipError_t e = hipModuleLoadData(&mod, code.data());   // stays loaded until the process ends
         if (e == hipSuccess) e = hipModuleGetFunction(&f, mod, kernel);
-        if (e != hipSuccess) { hiprtcDestroyProgram(&prog); return (int)e; }
+        if (e != hipSuccess) { R.destroy(&prog); return (int)e; }
     }
-    hiprtcDestroyProgram(&prog);
-    g_cache.emplace(key, f);
-    *fn = f;
+    R.destroy(&prog);
+    std::lock_guard<std::mutex> lock(g_mu);
+    ++g_compiles;
+    auto ins = g_cache.emplace(key, f);
+    *fn = ins.first->second;
     return MI_OK;
 }
 

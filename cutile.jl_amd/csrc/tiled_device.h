@@ -229,12 +229,10 @@ template <int DT> __device__ __forceinline__ car<DT> f_and(car<DT> a, car<DT> b)
 template <int DT> __device__ __forceinline__ car<DT> f_or(car<DT> a, car<DT> b) { return (car<DT>)(a | b); }
 template <int DT> __device__ __forceinline__ car<DT> f_xor(car<DT> a, car<DT> b) { return (car<DT>)(a ^ b); }
 template <int DT> __device__ __forceinline__ car<DT> f_ifelse(bool c, car<DT> a, car<DT> b) { return c ? a : b; }
-// Julia's div (toward zero), rem (sign of the dividend), mod (sign of the divisor), fld, cld.
-template <int DT> __device__ __forceinline__ car<DT> f_divi(car<DT> a, car<DT> b) {
-    if constexpr (DT == DT_F64) return trunc(a / b);
-    else if constexpr (is_flt<DT>) return rnd<DT>(truncf(a / b));
-    else return b == 0 ? (car<DT>)0 : (b == -1 ? -a : a / b);
-}
+// Julia's div (toward zero), rem (sign of the dividend), mod (sign of the divisor), fld, cld.  For floats
+// Julia derives the quotients from the exact remainder, round((x - rem(x, y, r)) / y) (Base div.jl), which
+// differs from rounding x / y where the division itself rounds across an integer (1.0 / 0.1 is 10.0, but
+// div(1.0, 0.1) and fld(1.0, 0.1) are 9.0); mod of an exact multiple takes the sign of the divisor.
 template <int DT> __device__ __forceinline__ car<DT> f_rem(car<DT> a, car<DT> b) {
     if constexpr (DT == DT_F64) return fmod(a, b);
     else if constexpr (is_flt<DT>) return rnd<DT>(fmodf(a, b));
@@ -242,17 +240,25 @@ template <int DT> __device__ __forceinline__ car<DT> f_rem(car<DT> a, car<DT> b)
 }
 template <int DT> __device__ __forceinline__ car<DT> f_mod(car<DT> a, car<DT> b) {
     car<DT> r = f_rem<DT>(a, b);
+    if constexpr (is_flt<DT> || DT == DT_F64) {
+        if (r == (car<DT>)0) return (car<DT>)copysign((double)r, (double)b);
+    }
     if (r != (car<DT>)0 && ((r < (car<DT>)0) != (b < (car<DT>)0))) r = rnd<DT>(r + b);
     return r;
 }
+template <int DT> __device__ __forceinline__ car<DT> f_divi(car<DT> a, car<DT> b) {
+    if constexpr (DT == DT_F64) return rint((a - fmod(a, b)) / b);
+    else if constexpr (is_flt<DT>) return rnd<DT>(rintf((a - f_rem<DT>(a, b)) / b));
+    else return b == 0 ? (car<DT>)0 : (b == -1 ? -a : a / b);
+}
 template <int DT> __device__ __forceinline__ car<DT> f_fld(car<DT> a, car<DT> b) {
-    if constexpr (DT == DT_F64) return floor(a / b);
-    else if constexpr (is_flt<DT>) return rnd<DT>(floorf(a / b));
+    if constexpr (DT == DT_F64) return rint((a - f_mod<DT>(a, b)) / b);
+    else if constexpr (is_flt<DT>) return rnd<DT>(rintf((a - f_mod<DT>(a, b)) / b));
     else { const car<DT> q = f_divi<DT>(a, b); return (b != 0 && (a % (b == -1 ? 1 : b)) != 0 && ((a < 0) != (b < 0))) ? q - 1 : q; }
 }
 template <int DT> __device__ __forceinline__ car<DT> f_cld(car<DT> a, car<DT> b) {
-    if constexpr (DT == DT_F64) return ceil(a / b);
-    else if constexpr (is_flt<DT>) return rnd<DT>(ceilf(a / b));
+    if constexpr (DT == DT_F64) return rint((a - f_mod<DT>(a, -b)) / b);
+    else if constexpr (is_flt<DT>) return rnd<DT>(rintf((a - f_mod<DT>(a, -b)) / b));
     else { const car<DT> q = f_divi<DT>(a, b); return (b != 0 && (a % (b == -1 ? 1 : b)) != 0 && ((a < 0) == (b < 0))) ? q + 1 : q; }
 }
 

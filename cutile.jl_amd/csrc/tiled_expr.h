@@ -32,7 +32,7 @@ enum Rule {
     R_SAME,      // type of the (promoted) arguments
     R_NEG,       // like R_SAME, Bool -> Int64
     R_DIV,       // `/`: integers give Float64, floats promote
-    R_POW,       // `^`: float base keeps its type for integer exponents, otherwise promote
+    R_POW,       // `^`: the base keeps its type for integer / Bool exponents (Julia's ^(x::T, p::Integer)), otherwise promote
     R_FLOAT,     // math functions: integers are converted with float() (Float64), floats keep their type
     R_BOOL,      // predicates and comparisons
     R_LOGIC,     // & | xor !: Bool or integers (bitwise), promote
@@ -251,7 +251,7 @@ static inline int infer_types(Expr& e, const int32_t* leaf_dt, int nl, const int
             case R_DIV: n.dtype = dt_is_float(t) ? t : MI_F64; break;
             case R_POW: {
                 const int b = e.nodes[n.args[0]].dtype, x = e.nodes[n.args[1]].dtype;
-                n.dtype = (dt_is_float(b) && !dt_is_float(x)) ? b : (t == MI_BOOL ? MI_BOOL : t);
+                n.dtype = !dt_is_float(x) ? b : t;   // Int32 ^ Int64 is Int32, Bool ^ Int is Bool, Float32 ^ Int is Float32
                 break;
             }
             case R_FLOAT: n.dtype = dt_is_float(t) ? t : MI_F64; break;
@@ -337,7 +337,7 @@ static inline std::string emit_body(const Expr& e) {
             const Node& a = e.nodes[n.args[k]];
             int want = work;
             if (f.rule == R_IFELSE && k == 0) want = MI_BOOL;
-            if (f.rule == R_POW && k == 1 && dt_is_float(n.dtype) && !dt_is_float(a.dtype)) want = MI_I64;
+            if (f.rule == R_POW && k == 1 && !dt_is_float(a.dtype)) want = MI_I64;
             if (f.rule == R_CONVERT) want = a.dtype;
             if (f.rule == R_SHIFT && k == 1) want = MI_I64;
             if (k) o += ", ";

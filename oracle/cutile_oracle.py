@@ -588,11 +588,15 @@ def tiled_eval(text: str, leaves=(), scalars=()):
             R = "Int64" if T == "Bool" else T
             return (-conv(args[0], R)).astype(_JL_NP[R]), R
         if name == "pow":
+            # ^(x::T, p::Integer) keeps the type of the base (Base intfuncs.jl power_by_squaring; Bool * Bool is
+            # Bool): Int32 ^ Int64 is Int32, Bool ^ Int is Bool, Float32 ^ Int is Float32; otherwise promote
             b, x = args
-            R = b[1] if (b[1] in _JL_FLOATS and x[1] not in _JL_FLOATS) else T
+            R = b[1] if x[1] not in _JL_FLOATS else T
+            if R == "Bool":
+                return np.where(conv(x, "Int64") != 0, b[0], True), R
             if R in _JL_FLOATS:
                 return np.power(conv(b, R), conv(x, R)).astype(_JL_NP[R]), R
-            return np.power(conv(b, R), conv(x, R)).astype(_JL_NP[R]), R
+            return np.power(conv(b, R), conv(x, "Int64")).astype(_JL_NP[R]), R
         if name in _TILED_MATH or name in ("atan2", "hypot"):
             R = T if isf else "Float64"
             # Julia evaluates Float16 functions in Float32 and rounds once (Base math.jl)
@@ -663,8 +667,15 @@ def tiled_eval(text: str, leaves=(), scalars=()):
             R = "Int64" if T == "Bool" else T
             a, b = conv(args[0], R), conv(args[1], R)
             if R in _JL_FLOATS:
-                r = {"div_int": lambda: np.trunc(a / b), "rem": lambda: np.fmod(a, b), "mod": lambda: np.mod(a, b),
-                     "fld": lambda: np.floor(a / b), "cld": lambda: np.ceil(a / b)}[name]()
+                # Base div.jl: the float quotients come from the exact remainder, round((x - rem(x, y, r)) / y);
+                # mod of an exact multiple has the sign of the divisor (Base float.jl)
+                def jmod(x, y):
+                    m = np.fmod(x, y)
+                    m = np.where(m == 0, np.copysign(m, y), np.where((m > 0) != (y > 0), m + y, m))
+                    return m
+                with np.errstate(all="ignore"):
+                    r = {"div_int": lambda: np.rint((a - np.fmod(a, b)) / b), "rem": lambda: np.fmod(a, b), "mod": lambda: jmod(a, b),
+                         "fld": lambda: np.rint((a - jmod(a, b)) / b), "cld": lambda: np.rint((a - jmod(a, -b)) / b)}[name]()
             else:
                 q = np.floor_divide(a, b)
                 r = {"div_int": lambda: np.trunc(a / b).astype(a.dtype), "rem": lambda: np.fmod(a, b),

@@ -216,6 +216,13 @@ TYPE_CASES = [
     ("max(a0,a1)", (torch.int32, torch.int64), "Int64"),
     ("sqrt(abs(a0))", (torch.int32,), "Float64"),
     ("mod(a0,a1)", (torch.int64, torch.int32), "Int64"),
+    ("pow(a0,abs(a1))", (torch.int32, torch.int64), "Int32"),        # ^ keeps the base's type and wraps in it
+    ("pow(a0,abs(a1))", (torch.bool, torch.int32), "Bool"),
+    ("mod(a0,a1)", (torch.float64, torch.float64), "Float64"),       # float quotients from the exact remainder
+    ("fld(a0,a1)", (torch.float64, torch.float64), "Float64"),
+    ("cld(a0,a1)", (torch.float64, torch.float64), "Float64"),
+    ("div_int(a0,a1)", (torch.float64, torch.float64), "Float64"),
+    ("mod(a0,trunc(a1))", (torch.float32, torch.float32), "Float32"),
     ("div_int(a0,a1)", (torch.int32, torch.int32), "Int32"),
     ("fld(a0,a1)", (torch.int32, torch.int32), "Int32"),
     ("cld(a0,a1)", (torch.int64, torch.int64), "Int64"),

@@ -407,6 +407,29 @@ def test_tiled_eval_types_and_values_by_hand(orc):
                        ("rem", [1, -1, 1, -1]), ("mod", [1, 1, -1, -1])):
         v, t = orc.tiled_eval(f"{name}(a0,a1)", (x, y))
         assert t == "Int64" and np.array_equal(v, want), name
+    # the same on floats, answers worked out by hand from Julia's definitions (Base div.jl, float.jl): the quotients
+    # come from the exact remainder, so div(1.0, 0.1) == fld(1.0, 0.1) == 9.0 although 1.0 / 0.1 == 10.0 (rem is
+    # 0.09999999999999995), cld(1.0, 0.1) == 10.0; mod of an exact multiple takes the divisor's sign: mod(4.0, -2.0)
+    # is -0.0, mod(-4.0, 2.0) is 0.0; mod(-1.0, 3.0) == 2.0, mod(1.0, -3.0) == -2.0
+    fx, fy = np.array([1.0, 4.0, -4.0, -1.0, 1.0, 7.5]), np.array([0.1, -2.0, 2.0, 3.0, -3.0, 2.0])
+    for name, want in (("div_int", [9.0, -2.0, -2.0, 0.0, 0.0, 3.0]), ("fld", [9.0, -2.0, -2.0, -1.0, -1.0, 3.0]),
+                       ("cld", [10.0, -2.0, -2.0, 0.0, 0.0, 4.0]), ("mod", [0.09999999999999995, -0.0, 0.0, 2.0, -2.0, 1.5])):
+        v, t = orc.tiled_eval(f"{name}(a0,a1)", (fx, fy))
+        assert t == "Float64" and np.array_equal(v, want), (name, v)
+        assert name != "mod" or np.array_equal(np.signbit(v), np.signbit(want))      # the sign of a zero remainder
+    # ^ keeps the type of the base for integer and Bool exponents (^(x::T, p::Integer), power_by_squaring):
+    # Int32(3)^Int64(4) isa Int32 (and wraps: Int32(2)^40 == 0), true^0 == true^5 == false^0 == true, false^2 == false,
+    # Float32(2)^3 isa Float32; a float exponent promotes: Int32(2)^0.5 isa Float64
+    v, t = orc.tiled_eval("pow(a0,a1)", (np.array([3, 2, -2], np.int32), np.array([4, 40, 3], np.int64)))
+    assert t == "Int32" and np.array_equal(v, [81, 0, -8])
+    v, t = orc.tiled_eval("pow(a0,a1)", (np.array([True, True, False, False]), np.array([0, 5, 0, 2], np.int64)))
+    assert t == "Bool" and np.array_equal(v, [True, True, True, False])
+    v, t = orc.tiled_eval("pow(a0,a1)", (np.array([True, False]), np.array([False, True])))
+    assert t == "Bool" and np.array_equal(v, [True, False])
+    v, t = orc.tiled_eval("pow(a0,a1)", (np.array([2.0], np.float32), np.array([3], np.int32)))
+    assert t == "Float32" and v[0] == 8.0
+    v, t = orc.tiled_eval("pow(a0,a1)", (np.array([2], np.int32), np.array([0.5])))
+    assert t == "Float64" and v[0] == 2.0 ** 0.5
     # Julia's shifts (answers worked out by hand): the value keeps its type; Int32 wraps; a count of the word size
     # or more empties the word (>> keeps the sign); >>> is logical; a negative count shifts the other way
     w = np.array([1, -8, 5, -1, 2 ** 30], np.int32)

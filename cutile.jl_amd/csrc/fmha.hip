@@ -349,7 +349,7 @@ struct FmhaDma {
                     const float p0 = __builtin_amdgcn_exp2f(s[j][kt][r] * scale2 - mj);
                     const float p1 = __builtin_amdgcn_exp2f(s[j][kt][r + 1] * scale2 - mj);
                     const unsigned pk = Pack<E>::pack(p0, p1);
-                    lsum = Pack<E>::sum2(pk, lsum);
+                    lsum = Pack<E>::sum2(pk, p0, p1, lsum);
                     pf[j][kt][r >> 3][(r & 7) >> 1] = pk;
                 }
             st.l[j] = lsum;

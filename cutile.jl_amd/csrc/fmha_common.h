@@ -51,9 +51,13 @@ template <> struct Pack<F16> {
         f16x2 v = {(_Float16)a, (_Float16)b};
         return __builtin_bit_cast(unsigned, v);
     }
-    static __device__ __forceinline__ float sum2(unsigned p, float acc) {
-        const f16x2 one = {(_Float16)1.0f, (_Float16)1.0f};
-        return __builtin_amdgcn_fdot2(__builtin_bit_cast(f16x2, p), one, acc, false);
+    // acc + the two weights of the packed pair pk, as rounded.  Two mixed-precision fma (f16 source, fp32
+    // sum), not a dot2: the dot2 instructions run on the matrix pipe and wait for the MFMA in flight.
+    static __device__ __forceinline__ float sum2(unsigned pk, float, float, float acc) {
+        float r;
+        asm("v_fma_mix_f32 %0, %1, 1.0, %2 op_sel_hi:[1,0,0]" : "=v"(r) : "v"(pk), "v"(acc));
+        asm("v_fma_mix_f32 %0, %1, 1.0, %0 op_sel:[1,0,0] op_sel_hi:[1,0,0]" : "+v"(r) : "v"(pk));
+        return r;
     }
 };
 template <> struct Pack<BF16> {
@@ -61,9 +65,10 @@ template <> struct Pack<BF16> {
         bf16x2 v = {(__bf16)a, (__bf16)b};
         return __builtin_bit_cast(unsigned, v);
     }
-    static __device__ __forceinline__ float sum2(unsigned p, float acc) {
-        const bf16x2 one = {(__bf16)1.0f, (__bf16)1.0f};
-        return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2, p), one, acc, false);
+    // acc + the two weights p0, p1 before rounding (there is no mixed-precision fma for bf16, and widening
+    // the rounded pair would take two more instructions; dot2 is avoided for the reason above).
+    static __device__ __forceinline__ float sum2(unsigned, float p0, float p1, float acc) {
+        return (acc + p0) + p1;
     }
 };
 

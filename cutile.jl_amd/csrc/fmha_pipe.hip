@@ -61,12 +61,11 @@ __device__ __forceinline__ void wait_and_barrier() {
     fence();
 }
 
-// max(a, b, c) as one instruction.  (fmaxf() is preceded by a quieting v_max_f32 x, x, x of every operand the
-// compiler can not prove to be no signalling NaN, and MFMA results are such operands.)
+// max(a, b, c) as one instruction (v_maximum3_f32: the IEEE 754-2019 maximum, which propagates NaN).  fmaxf() is
+// preceded by a quieting v_max_f32 x, x of every operand the compiler can not prove to be no signalling NaN, and
+// MFMA results are such operands; an inline-asm v_max3_f32 makes the compiler put a wait state after every one.
 __device__ __forceinline__ float max3(float a, float b, float c) {
-    float r;
-    asm("v_max3_f32 %0, %1, %2, %3" : "=v"(r) : "v"(a), "v"(b), "v"(c));
-    return r;
+    return __builtin_elementwise_maximum(__builtin_elementwise_maximum(a, b), c);
 }
 
 // max / sum over the lane pair (l, l ^ 32)
@@ -156,7 +155,7 @@ __device__ __forceinline__ void exp_stage1(const f32x16& s, int h, float (&p)[2]
 template <typename E>
 __device__ __forceinline__ void exp_stage2(const float (&p)[2], int h, float& l, unsigned (&pf)[2][4]) {
     const unsigned pk = Pack<E>::pack(p[0], p[1]);
-    l = Pack<E>::sum2(pk, l);
+    l = Pack<E>::sum2(pk, p[0], p[1], l);
     pf[h >> 2][h & 3] = pk;
 }
 
@@ -275,43 +274,36 @@ __device__ __forceinline__ void half_step(const unsigned short* Ks, const unsign
                                : masked_row_max<false>(s_next[jn], 0);
         ++mi;
     };
-    // A: chunk 0 of every stream
+    // the K(j+2) fragments are read once every S MFMA has been issued: the old fragments are free then
+    bool kread = !NEXT;
+    auto after_q = [&]() {
+        if (!kread && qi == nQ) {
+            read_k_frags(Ks, c, (j + 2) & 3, kf);
+            kread = true;
+        }
+    };
+    // A: one MFMA and one exp piece per slot.  First the S MFMAs, then the P.V MFMAs of a chunk as soon as that
+    // chunk's weights exist.
 #pragma unroll
-    for (int sl = 0; sl < 2 * nC; ++sl) {
+    for (int sl = 0; sl < 8 * nC; ++sl) {
         if (qi < nQ) mfma_q();
-        piece();
-        piece();
-        slot_end();
-    }
-    // B: chunk 1; P.V MFMAs of chunk 0 alternate with the remaining S MFMAs, then those P.V MFMAs
-    // of chunk 1 whose weights are complete
-#pragma unroll
-    for (int sl = 0; sl < 4 * nC; ++sl) {
-        if (qi < nQ && (sl % 2 == 0 || p0 == nP)) mfma_q();
         else if (p0 < nP && xi > 4 * ((p0 / 2) + 1)) mfma_p(0, p0++);
         else if (p1 < nP && xi > 4 * nC + 4 * (p1 / 2 + 1)) mfma_p(1, p1++);
+        after_q();
         piece();
         slot_end();
     }
     piece();  // finishes the last pair
-    // C
-    // the K(j+2) fragments are read once every S MFMA has been issued: the old fragments are free then
-    bool kread = !NEXT;
-    if (!kread && qi == nQ) {
-        read_k_frags(Ks, c, (j + 2) & 3, kf);
-        kread = true;
-    }
+    // B: the remaining MFMAs, with the row maxima of S(j+1) between them
+    after_q();
 #pragma unroll
     for (int sl = 0; sl < 2 * nQ + 2 * nP; ++sl) {
         if (qi < nQ) mfma_q();
         else if (p0 < nP) mfma_p(0, p0++);
         else if (p1 < nP) mfma_p(1, p1++);
         else break;
-        if (!kread && qi == nQ) {
-            read_k_frags(Ks, c, (j + 2) & 3, kf);
-            kread = true;
-        }
-        if (qi == nQ && mi < nN && (sl % 2 == 1 || p1 == nP)) maxima();
+        after_q();
+        if (qi == nQ && mi < nN) maxima();
         slot_end();
     }
 #pragma unroll
@@ -392,6 +384,14 @@ __global__ __launch_bounds__(128) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
         }
     }
 
+    // Fill the rings first: the transfers then travel together with the Q loads below instead of after them.
+    issue_k(c, 0);
+    issue_k(c, 1);
+    issue_k(c, 2);
+    issue_v(c, 0);
+    issue_k(c, 3);
+    issue_v(c, 1);
+
     Acc<E> a;
     a.ones = s16x8{0};
     a.ones[0] = hb == 0 ? E::cvt(1.0f) : (short)0;
@@ -415,14 +415,8 @@ __global__ __launch_bounds__(128) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
         a.l[jj] = 0.f;
     }
 
-    // ---- prologue: fill the rings, compute S(0), fetch the K(1) fragments -----------------------
-    issue_k(c, 0);
-    issue_k(c, 1);
-    issue_k(c, 2);
-    issue_v(c, 0);
-    issue_k(c, 3);
-    issue_v(c, 1);
-    wait_and_barrier<kWaitVm4>();  // K(0..2), V(0) have landed
+    // ---- prologue: compute S(0), fetch the K(1) fragments -----------------------------------------
+    wait_and_barrier<kWaitVm0>();  // the first halves (requested before Q, above) have landed
     f32x16 sa[2], sb[2];
     s16x8 kf[4];
     float cand[2];

@@ -5,8 +5,9 @@
 // Work split.  A workgroup is two waves and owns 128 queries of one (batch, head); a wave owns
 // two 32-query MFMA column tiles ("streams").  Without a causal mask the streams are adjacent
 // tiles.  With it, wave w of workgroup qb takes tiles u = 2*qb + w and NT-1-u, so that every
-// wave of the grid has the same number of MFMAs; stream 0 (the early tile) leaves the loop
-// after its diagonal.
+// wave of the grid has the same number of MFMAs; stream 0 (the early tile) is stored after its
+// diagonal, and from then on the long tile takes both streams' slots: two halves per trip ("wide
+// steps", see wide_step below), so that the fixed cost of a trip is paid half as often.
 //
 // K and V travel in halves of 32 keys (4 KB each) through two rings of four LDS slots, filled
 // by direct global->LDS loads three steps ahead of their use.  One step handles one half j:
@@ -175,10 +176,10 @@ constexpr int nth_stream(int m, int k) { return (m & 1) ? k : 1; }
 // A wave issues in order, so the body is laid out as issue slots -- one MFMA followed by the
 // vector work that fits in its shadow, closed by a scheduling barrier -- instead of leaving
 // the interleaving to the compiler:
-//   A: [S(j+1) MFMA] + two exp_pair pieces        while key chunk 0 of every stream is weighted
-//   B: [S(j+1) or P.V MFMA] + one exp_pair piece   while key chunk 1 is weighted; P.V MFMAs of a
-//                                                  chunk follow as soon as its weights exist
-//   C: remaining P.V MFMAs, each followed by the row maxima of one stream of S(j+1)
+//   A: one slot per exp piece: [S(j+1) MFMA, then P.V MFMA of a chunk whose weights exist] + the piece (2 exp2,
+//      pack, row sum: about the time one MFMA takes);
+//   B: the remaining P.V MFMAs, each followed by the row maxima of one stream of S(j+1).
+// The K(j+2) fragments are read as soon as the last S MFMA has been issued.
 template <typename E, int CUR, int NEXT, int MASKN>
 __device__ __forceinline__ void half_step(const unsigned short* Ks, const unsigned short* Vs, Lane& c, Acc<E>& a,
                                           int j, f32x16 (&s_cur)[2], f32x16 (&s_next)[2], s16x8 (&kf)[4],
@@ -310,6 +311,139 @@ __device__ __forceinline__ void half_step(const unsigned short* Ks, const unsign
     while (mi < nN) maxima();
 }
 
+// One wide step: the long tile of a wave (stream 1) alone, over the two halves j and j+1.  Once the early
+// tile is stored, its score buffers, fragments and issue slots would stand empty for the rest of the walk while
+// the fixed cost of a step (barrier, transfers, raise check, fragment reads) stayed the same; instead they take
+// the second half, so that a trip has the shape of a two-stream step and the walk takes half as many trips.
+// Both halves share the stream's state (m, the accumulators); c0 / c1 are S(j) - m / S(j+1) - m, n0 / n1 receive
+// S(j+2) - m / S(j+3) - m, kf[h] holds the K(j+2+h) fragments on entry and the K(j+4+h) fragments on exit,
+// cand[h] the row maxima of c_h on entry and of n_h on exit.  Row sums: half j adds to l[1], half j+1 to l[0].
+// Ring: a trip waits for everything requested one trip ago (K(j+4), K(j+5), V(j+2), V(j+3)), then requests
+// K(j+6), K(j+7) into the slots whose fragments are in registers and V(j+2), V(j+3) into the slots read one trip
+// ago (V(j+2) not in the first wide trip: the narrow steps had requested it already).
+template <typename E, bool NEXT, bool MASK>
+__device__ __forceinline__ void wide_step(const unsigned short* Ks, const unsigned short* Vs, Lane& c, Acc<E>& a,
+                                          int j, bool first, f32x16& c0, f32x16& c1, f32x16& n0, f32x16& n1,
+                                          s16x8 (&kf)[2][4], float (&cand)[2]) {
+    constexpr int nQ = NEXT ? 10 : 0;   // S MFMAs, k-step major over the two halves; "k step" 0 places -m
+    constexpr int nP = 4;               // P.V MFMAs per 16-key chunk, half major
+    {
+        const float cm = __builtin_elementwise_maximum(cand[0], cand[1]);
+        if (__any(cm > a.thr[1])) {
+            const float base = a.thr[1] == -INFINITY ? 0.f : a.m[1];
+            const short mh = E::cvt(fmaxf(a.m[1], base + cm));
+            const float m_new = E::to_f32(mh);
+            const float alpha = __builtin_amdgcn_exp2f(a.m[1] - m_new);
+            const float shift = base - m_new;
+            a.l[0] *= alpha;
+            a.l[1] *= alpha;
+#pragma unroll
+            for (int dt = 0; dt < 2; ++dt)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) a.o[1][dt][r] *= alpha;
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                c0[r] += shift;
+                c1[r] += shift;
+            }
+            a.qm[1][0] = c.hb0 ? (short)(mh ^ (short)0x8000) : (short)0;
+            a.m[1] = m_new;
+            a.thr[1] = kRaise;
+        }
+    }
+    wait_and_barrier<kWaitVm0>();   // everything requested one trip ago has landed, and every wave knows
+    issue_k(c, (j + 2) & 3);        // halves j+6, j+7 (the fragments of j+2, j+3 are in registers)
+    issue_k(c, (j + 3) & 3);
+    if (!first) issue_v(c, (j + 2) & 3);   // half j+2 (the narrow steps had requested it already)
+    issue_v(c, (j + 3) & 3);               // half j+3
+    s16x8 vf[2][2][2];  // [half][16-key chunk][d tile]
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+        const unsigned short* vb = Vs + ((j + h) & 3) * kSlot;
+#pragma unroll
+        for (int ch = 0; ch < 2; ++ch)
+#pragma unroll
+            for (int dt = 0; dt < 2; ++dt) {
+                const unsigned short* p = vb + c.vfo[dt] + 16 * ch * kD;
+                s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16(LDS_PTR(s16x4, p));
+                s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(LDS_PTR(s16x4, p + 8 * kD));
+                vf[h][ch][dt] = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+            }
+    }
+    unsigned pf[2][2][4];   // [half][chunk][pair]
+    slot_end();
+
+    int qi = 0, p0 = 0, p1 = 0, xi = 0;
+    auto mfma_q = [&]() {
+        const int ks = qi / 2, h = qi % 2;
+        f32x16& n = h ? n1 : n0;
+        n = ks == 0 ? E::mfma32(a.ones, a.qm[1], f32x16{0}) : E::mfma32(kf[h][ks - 1], a.qf[1][ks - 1], n);
+        ++qi;
+    };
+    auto mfma_p = [&](int ch, int k) {
+        const int h = k / 2, dt = k % 2;
+        u32x4 pw = {pf[h][ch][0], pf[h][ch][1], pf[h][ch][2], pf[h][ch][3]};
+        a.o[1][dt] = E::mfma32(vf[h][ch][dt], __builtin_bit_cast(s16x8, pw), a.o[1][dt]);
+    };
+    float pa[2], pb[2];
+    auto stage1 = [&](int x, float (&p)[2]) {
+        const int ch = x / 8, h = (x / 4) % 2, pr = 4 * ch + x % 4;
+        exp_stage1(h ? c1 : c0, pr, p);
+    };
+    auto stage2 = [&](int x, const float (&p)[2]) {
+        const int ch = x / 8, h = (x / 4) % 2, pr = 4 * ch + x % 4;
+        exp_stage2<E>(p, pr, a.l[1 - h], pf[h]);
+    };
+    auto piece = [&]() {
+        if (xi % 2 == 0) {
+            if (xi < 16) stage1(xi, pa);
+            if (xi > 0) stage2(xi - 1, pb);
+        } else {
+            if (xi < 16) stage1(xi, pb);
+            stage2(xi - 1, pa);
+        }
+        ++xi;
+    };
+    bool kread = !NEXT;
+    auto after_q = [&]() {
+        if (!kread && qi == nQ) {
+            if (j + 4 < c.nh) {
+                read_k_frags(Ks, c, (j + 4) & 3, kf[0]);
+                read_k_frags(Ks, c, (j + 5) & 3, kf[1]);
+            }
+            kread = true;
+        }
+    };
+#pragma unroll
+    for (int sl = 0; sl < 16; ++sl) {
+        if (qi < nQ) mfma_q();
+        else if (p0 < nP && xi > 4 * ((p0 / 2) + 1)) mfma_p(0, p0++);
+        else if (p1 < nP && xi > 8 + 4 * (p1 / 2 + 1)) mfma_p(1, p1++);
+        after_q();
+        piece();
+        slot_end();
+    }
+    piece();  // finishes the last pair
+    int mi = 0;
+    auto maxima = [&]() {
+        f32x16& n = mi ? n1 : n0;
+        cand[mi] = MASK ? masked_row_max<true>(n, c.q0[1] + c.lim0 - kHK * (j + 2 + mi)) : masked_row_max<false>(n, 0);
+        ++mi;
+    };
+#pragma unroll
+    for (int sl = 0; sl < 2 * nP; ++sl) {
+        if (p0 < nP) mfma_p(0, p0++);
+        else if (p1 < nP) mfma_p(1, p1++);
+        else break;
+        if (NEXT && mi < 2) maxima();
+        slot_end();
+    }
+    if (NEXT) {
+#pragma unroll
+        while (mi < 2) maxima();
+    }
+}
+
 template <typename E, bool CAUSAL>
 __global__ __launch_bounds__(128) __attribute__((amdgpu_waves_per_eu(2, 2))) void fmha_pipe_kernel(
     const unsigned short* __restrict__ Q, Strides qs, const unsigned short* __restrict__ K, Strides ks,
@@ -356,6 +490,10 @@ __global__ __launch_bounds__(128) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     c.ks_base = (unsigned)(size_t)Ks;
     c.vs_base = (unsigned)(size_t)Vs;
     c.wave = wave;
+    // The waves of the second half of the grid land on SIMDs that already host a wave of the first half, and the
+    // instruction arbiter serves the older wave first: the younger one ran 20 % longer.  A raised priority evens
+    // the two out (they have the same amount of work), which shortens the kernel.
+    if (blockIdx.x >= (gridDim.x >> 1)) __builtin_amdgcn_s_setprio(1);
     c.nh = CAUSAL ? NT - 2 * qb : NT;
     c.k_left = c.v_left = c.nh;
     c.hb0 = hb == 0;
@@ -434,8 +572,8 @@ __global__ __launch_bounds__(128) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     issue_v(c, 2);
 
     // Epilogue of one stream: add the two half-row sums, O / l (approximate reciprocal), round, store.
-    auto store_tile = [&](int jj) {
-        const float inv = __builtin_amdgcn_rcpf(xhalf_sum(a.l[jj]));
+    auto store_tile = [&](int jj, float lsum) {
+        const float inv = __builtin_amdgcn_rcpf(xhalf_sum(lsum));
         unsigned short* op = O + (int64_t)my_q[jj] * os.s1;
 #pragma unroll
         for (int dt = 0; dt < 2; ++dt)
@@ -468,17 +606,37 @@ __global__ __launch_bounds__(128) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
         STEP(3, 3, 0, j, sa, sb);
         STEP(3, 2, 1, j + 1, sb, sa);  // (stream 1's mask only bites when its diagonal is two halves away)
         j += 2;
-        store_tile(0);  // stream 0 is complete: its registers are free for the rest of the walk
-        for (; j < nh - 4; j += 2) {
-            STEP(2, 2, -1, j, sa, sb);
-            STEP(2, 2, -1, j + 1, sb, sa);
+        store_tile(0, a.l[0]);  // stream 0 is complete: its registers and issue slots now serve the long tile
+        // ---- wide steps: the long tile over two halves per trip (always an odd number of trips) ------------
+        // S(n1) - m is in sa[1] and the K(n1+1) fragments in kf: compute S(n1+1) - m into sa[0], then fetch
+        // the fragments of the next two halves and request the one transfer the wide schedule still lacks.
+        a.l[0] = 0.f;
+        s16x8 kw[2][4];
+        float wc[2];
+        wc[0] = cand[1];
+        sa[0] = E::mfma32(a.ones, a.qm[1], f32x16{0});
+#pragma unroll
+        for (int s = 0; s < 4; ++s) sa[0] = E::mfma32(kf[s], a.qf[1][s], sa[0]);
+        wc[1] = masked_row_max<true>(sa[0], c.q0[1] + c.lim0 - kHK * (j + 1));
+        wait_and_barrier<kWaitVm0>();
+        read_k_frags(Ks, c, (j + 2) & 3, kw[0]);
+        read_k_frags(Ks, c, (j + 3) & 3, kw[1]);
+        issue_k(c, (j + 1) & 3);  // half j+5
+#define WIDE(NEXT, MASK, jx, first, s0, s1) wide_step<E, NEXT, MASK>(Ks, Vs, c, a, jx, first, s0[1], s0[0], s1[1], s1[0], kw, wc)
+        bool first = true;
+        if (j + 2 < nh) {   // three trips or more: an odd number of plain trips, then the one that masks
+            for (; j + 6 < nh; j += 4) {
+                WIDE(true, false, j, first, sa, sb);
+                WIDE(true, false, j + 2, false, sb, sa);
+                first = false;
+            }
+            WIDE(true, false, j, first, sa, sb);
+            WIDE(true, true, j + 2, false, sb, sa);
+            j += 4;
+            first = false;
         }
-        for (; j < nh - 2; j += 2) {  // at most one trip
-            STEP(2, 2, 1, j, sa, sb);
-            STEP(2, 2, 1, j + 1, sb, sa);
-        }
-        STEP(2, 2, 1, j, sa, sb);
-        STEP(2, 0, -1, j + 1, sb, sa);
+        WIDE(false, false, j, first, sa, sb);
+#undef WIDE
     } else {
         for (; j < nh - 2; j += 2) {
             STEP(3, 3, -1, j, sa, sb);
@@ -492,8 +650,8 @@ __global__ __launch_bounds__(128) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     // workgroup's LDS can be handed to another workgroup.
     __builtin_amdgcn_s_waitcnt(kWaitVm0);
 
-    if (!CAUSAL) store_tile(0);
-    store_tile(1);
+    if (!CAUSAL) store_tile(0, a.l[0]);
+    store_tile(1, CAUSAL ? a.l[0] + a.l[1] : a.l[1]);
 }
 
 bool vec16(const mi_tile_array* a) {

@@ -88,10 +88,13 @@ def test_fmha_strided_views_and_scale(orc):
 @pytest.mark.parametrize("batch,heads,s,causal,qg,T", [
     (1, 4, 512, True, 2, torch.float16), (1, 2, 640, True, 1, torch.float16), (1, 2, 640, False, 1, torch.float16),
     (1, 2, 512, True, 1, torch.bfloat16), (3, 3, 256, True, 1, torch.float16), (1, 8, 1024, False, 8, torch.float16),
+    (1, 2, 128, True, 1, torch.float16), (1, 1, 384, True, 1, torch.float16), (1, 2, 2048, True, 2, torch.bfloat16),
 ])
 def test_fmha_pipelined_kernel_shapes(ct, orc, batch, heads, s, causal, qg, T):
     """Shapes served by the software-pipelined D = 64 kernel (Sq == Skv, multiple of 128): odd numbers
-    of 128-query blocks, (batch*heads) not a multiple of 8, GQA, bf16, and both mask settings."""
+    of 128-query blocks, (batch*heads) not a multiple of 8, GQA, bf16, and both mask settings.  With the
+    causal mask a wave walks its long tile two key halves per trip once its early tile is done: 128 keys give
+    one such trip, 384 up to five, 2048 up to thirty-one."""
     data = fmha.prepare(batch=batch, heads=heads, seq_q=s, seq_kv=s, query_group_size=qg, causal=causal, T=T)
     r = fmha.run(data)
     assert ct.last_variant().startswith("fmha_pipe")

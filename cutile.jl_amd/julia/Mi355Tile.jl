@@ -40,8 +40,9 @@ mi_dtype(::Type{Float16}) = Int32(2)
 mi_dtype(::Type{Int32})   = Int32(5)
 mi_dtype(::Type{Int64})   = Int32(6)
 mi_dtype(::Type{Bool})    = Int32(7)
-# BFloat16 (BFloat16s.jl / Core.BFloat16) = 3 and Float8_E4M3FN (DLFP8Types.jl) = 4: add the
-# methods in a package extension, the way ext/DLFP8TypesExt.jl adds the cuTile mapping.
+# BFloat16 (BFloat16s.jl / Core.BFloat16) = 3, Float8_E4M3FN = 4 and Float8_E5M2 = 10 (DLFP8Types.jl): add the
+# methods in a package extension, the way ext/DLFP8TypesExt.jl adds the cuTile mapping.  matmul_kernel and
+# batch_matmul_kernel take both FP8 types as operands (A and B of the same type, C Float32 / Float16 / BFloat16).
 mi_dtype(T::Type) = T === UInt8 ? Int32(4) :   # raw e4m3fn bytes
                     error("Mi355Tile: unsupported element type $T")
 

@@ -30,6 +30,8 @@
 // re-read the last valid rows / chunks on the way in and clip their stores.  K is walked in whole
 // groups of four steps (128); in the last group the 16-byte chunks at k >= K are fetched from a
 // 16-byte block of zeros instead (both operands, so padding never meets a non-finite value).
+#include <mutex>
+
 #include "gemm_direct.h"
 
 namespace {
@@ -162,7 +164,7 @@ template <typename E, typename OutT, int I, int J>
 __global__ __launch_bounds__(256) void gemm16_big(const unsigned short* __restrict__ A, int64_t lda, int64_t sa,
                                                   const unsigned short* __restrict__ B, int64_t ldb, int64_t sb,
                                                   OutT* __restrict__ C, int64_t ldc, int64_t sc, int M, int N, int K,
-                                                  int tiles_m, int tiles_n, int batch) {
+                                                  int tiles_m, int tiles_n, int batch, int ksplit, int kchunk) {
     constexpr int BTM = 64 * I, STAGE_A = BTM * BK, BTN = 64 * J, STAGE_B = BTN * BK;
     __shared__ __attribute__((aligned(1024))) unsigned short As0[STAGE_A], As1[STAGE_A], As2[STAGE_A], As3[STAGE_A];
     __shared__ __attribute__((aligned(1024))) unsigned short Bs0[STAGE_B], Bs1[STAGE_B], Bs2[STAGE_B], Bs3[STAGE_B];
@@ -171,8 +173,16 @@ __global__ __launch_bounds__(256) void gemm16_big(const unsigned short* __restri
     // One-dimensional grid over (tile, batch).  Workgroups whose ids are congruent mod 8 share an XCD and
     // its L2: give each XCD a contiguous run of (batch-major) tiles, so that it works on neighbouring
     // tiles of as few batch entries as possible.
+    // With a split over K (ksplit > 1) consecutive workgroups are the ksplit parts of one tile; part ks walks
+    // k = ks * kchunk ... and writes its sums to slice (batch entry * ksplit + ks) of C, which is then the
+    // caller's partial-sum buffer.
     const int total = tiles_m * tiles_n, total_all = total * batch;
-    int L = blockIdx.x;
+    int L = blockIdx.x, ks_part = 0;
+    if (ksplit > 1) {
+        ks_part = L % ksplit;
+        L /= ksplit;
+        K = K - ks_part * kchunk < kchunk ? K - ks_part * kchunk : kchunk;
+    }
     if (total_all % 8 == 0) L = (L & 7) * (total_all >> 3) + (L >> 3);
     const int bz = L / total;
     L -= bz * total;
@@ -220,9 +230,10 @@ __global__ __launch_bounds__(256) void gemm16_big(const unsigned short* __restri
     }
     const int64_t lda2 = lda * 2, ldb2 = ldb * 2;
     // wave-uniform byte pointers to this wave's first rows of the k = 0 stage
-    const char* Ab = (const char*)(A + (int64_t)bz * sa + (int64_t)bm * BTM) + (int64_t)(8 / I * wave) * lda2;
-    const char* Bb = (const char*)(B + (int64_t)bz * sb + (int64_t)bn * BTN * ldb) + (int64_t)(16 * wave) * ldb2;
-    C += (int64_t)bz * sc;
+    const int64_t k_first = (int64_t)ks_part * kchunk;
+    const char* Ab = (const char*)(A + (int64_t)bz * sa + (int64_t)bm * BTM) + ((int64_t)(8 / I * wave) + k_first) * lda2;
+    const char* Bb = (const char*)(B + (int64_t)bz * sb + (int64_t)bn * BTN * ldb + k_first) + (int64_t)(16 * wave) * ldb2;
+    C += ((int64_t)bz * ksplit + ks_part) * sc;
     const int64_t a_step = (int64_t)BK * lda2;  // next K step of A: 32 rows down
     const int64_t b_step = (int64_t)BK * 2;     // next K step of B: 32 elements along the row
 
@@ -310,7 +321,127 @@ void launch(const Problem& p, hipStream_t s) {
     const int tiles_m = (p.M + 64 * I - 1) / (64 * I), tiles_n = (p.N + 64 * J - 1) / (64 * J);
     hipLaunchKernelGGL((gemm16_big<E, OutT, I, J>), dim3((unsigned)(tiles_m * tiles_n * p.batch)), dim3(256), 0,
                        s, (const unsigned short*)p.A, p.lda, p.sa, (const unsigned short*)p.B, p.ldb, p.sb,
-                       (OutT*)p.C, p.ldc, p.sc, p.M, p.N, p.K, tiles_m, tiles_n, p.batch);
+                       (OutT*)p.C, p.ldc, p.sc, p.M, p.N, p.K, tiles_m, tiles_n, p.batch, 1, 0);
+}
+
+// ---- split over K for problems with few tiles and a long K ---------------------------------------------------
+// A 512 x 512 x 4096 product is 16 tiles of 128 x 128: sixteen workgroups walk 128 K steps each while 240 CUs
+// idle.  Split into ksplit parts along K, ksplit times as many workgroups walk a part each and write fp32 partial
+// sums; a second kernel adds the parts in fixed order (results do not depend on timing) and converts.  The entry
+// point has no workspace argument (it mirrors the reference's kernel signature), so the partial sums live in a
+// static device array of the library, 16 MiB per GPU.  Launches that use it are ordered by an event when they
+// come from different streams; a stream that is being captured into a graph does not use it.
+constexpr int64_t kSplitFloats = 4 * 1024 * 1024;
+static __device__ __align__(256) float splitk_scratch[kSplitFloats];
+
+template <typename OutT>
+__global__ __launch_bounds__(256) void splitk_reduce(const float* __restrict__ part, int ksplit, OutT* __restrict__ C,
+                                                     int64_t ldc, int64_t sc, int M, int N, int batch, bool bf16) {
+    // one lane: 4 consecutive m of one column (M is a multiple of 8)
+    const int64_t quads = (int64_t)(M / 4) * N * batch;
+    const int64_t MN = (int64_t)M * N;
+    for (int64_t q = (int64_t)blockIdx.x * 256 + threadIdx.x; q < quads; q += (int64_t)gridDim.x * 256) {
+        const int m4 = (int)(q % (M / 4)), n = (int)((q / (M / 4)) % N), bz = (int)(q / ((int64_t)(M / 4) * N));
+        const float* src = part + (int64_t)bz * ksplit * MN + (int64_t)n * M + 4 * m4;
+        // parts added in index order (the result does not depend on timing); four loads in flight at a time
+        f32x4 acc = __builtin_nontemporal_load(reinterpret_cast<const f32x4*>(src));
+        int ks = 1;
+        for (; ks + 4 <= ksplit; ks += 4) {
+            f32x4 v[4];
+#pragma unroll
+            for (int u = 0; u < 4; ++u) v[u] = __builtin_nontemporal_load(reinterpret_cast<const f32x4*>(src + (ks + u) * MN));
+#pragma unroll
+            for (int u = 0; u < 4; ++u) acc += v[u];
+        }
+        for (; ks < ksplit; ++ks) acc += __builtin_nontemporal_load(reinterpret_cast<const f32x4*>(src + ks * MN));
+        OutT* dst = C + (int64_t)bz * sc + (int64_t)n * ldc + 4 * m4;
+        if constexpr (sizeof(OutT) == 4) {
+#pragma unroll
+            for (int e = 0; e < 4; ++e) dst[e] = acc[e];
+        } else {
+#pragma unroll
+            for (int e = 0; e < 4; ++e) dst[e] = bf16 ? BF16::from_f32(acc[e]) : F16::from_f32(acc[e]);
+        }
+    }
+}
+
+struct SplitState {
+    std::mutex mu;
+    float* scratch = nullptr;
+    hipEvent_t done = nullptr;
+    hipStream_t last = nullptr;
+    bool used = false, broken = false;
+};
+SplitState g_split[16];
+
+// Parts and part length for the problem, or 0 if a split does not apply.
+int pick_split(const Problem& p, int* kchunk) {
+    static const int force = [] { const char* e = getenv("MI_GEMM_SPLITK"); return e ? atoi(e) : -1; }();   // 0 = never, n = n parts
+    if (force == 0) return 0;
+    const int64_t tiles = tiles_of(p, 128, 128);
+    if (tiles > 64 || p.K < 1024) return 0;
+    // Estimated times in us: one launch walks K / 32 steps of 0.18 us; the split pays a second launch, the partial
+    // sums written and read again (at about 3 bytes per ns), and walks a part's steps only.
+    const double t_plain = 3.0 + 0.18 * (p.K / 32.0);
+    const double mn_bytes = 4.0 * p.M * p.N * p.batch;
+    int best = 0;
+    double t_best = 0.85 * t_plain;   // (a split has to be clearly better)
+    for (int parts = force > 1 ? force : 2; parts <= (force > 1 ? force : 16); ++parts) {
+        if (parts * tiles > 512) break;
+        const int chunk = ((p.K + parts - 1) / parts + 127) / 128 * 128;        // whole groups of four K steps
+        const int n = (p.K + chunk - 1) / chunk;
+        if (n < 2 || chunk < 256 || p.K - (n - 1) * chunk < 256 || (int64_t)n * p.M * p.N * p.batch > kSplitFloats) continue;
+        const double t = 7.0 + 0.18 * (chunk / 32.0) + (n + 1) * mn_bytes / 3.0e6 + (n * tiles > 256 ? 0.18 * (chunk / 32.0) : 0.0);
+        if (t < t_best || (force > 1 && !best)) {
+            t_best = t;
+            best = n;
+            *kchunk = chunk;
+        }
+    }
+    return best;
+}
+
+template <typename E>
+bool launch_split(const Problem& p, hipStream_t s, int parts, int kchunk) {
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 16) return false;
+    hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
+    if (hipStreamIsCapturing(s, &cap) != hipSuccess || cap != hipStreamCaptureStatusNone) return false;
+    SplitState& st = g_split[dev];
+    std::lock_guard<std::mutex> lock(st.mu);
+    if (st.broken) return false;
+    if (!st.scratch) {
+        if (hipGetSymbolAddress((void**)&st.scratch, HIP_SYMBOL(splitk_scratch)) != hipSuccess ||
+            hipEventCreateWithFlags(&st.done, hipEventDisableTiming) != hipSuccess) {
+            st.broken = true;
+            (void)hipGetLastError();
+            return false;
+        }
+    }
+    // The previous user of the partial sums, if it ran on another stream, has to finish first: an event recorded
+    // on that stream now (it covers everything the stream has been given so far) and awaited by this one.
+    if (st.used && st.last != s) {
+        if (hipEventRecord(st.done, st.last) != hipSuccess || hipStreamWaitEvent(s, st.done, 0) != hipSuccess) {
+            (void)hipGetLastError();
+            return false;
+        }
+    }
+    const int tiles_m = (p.M + 127) / 128, tiles_n = (p.N + 127) / 128;
+    const int64_t MN = (int64_t)p.M * p.N;
+    hipLaunchKernelGGL((gemm16_big<E, float, 2, 2>), dim3((unsigned)(tiles_m * tiles_n * p.batch * parts)), dim3(256), 0, s,
+                       (const unsigned short*)p.A, p.lda, p.sa, (const unsigned short*)p.B, p.ldb, p.sb, st.scratch,
+                       (int64_t)p.M, MN, p.M, p.N, p.K, tiles_m, tiles_n, p.batch, parts, kchunk);
+    const int64_t quads = MN / 4 * p.batch;
+    const unsigned blocks = (unsigned)((quads + 255) / 256 < 2048 ? (quads + 255) / 256 : 2048);
+    if (p.out_dtype == MI_F32)
+        hipLaunchKernelGGL((splitk_reduce<float>), dim3(blocks), dim3(256), 0, s, st.scratch, parts, (float*)p.C, p.ldc,
+                           p.sc, p.M, p.N, p.batch, false);
+    else
+        hipLaunchKernelGGL((splitk_reduce<unsigned short>), dim3(blocks), dim3(256), 0, s, st.scratch, parts,
+                           (unsigned short*)p.C, p.ldc, p.sc, p.M, p.N, p.batch, p.out_dtype == MI_BF16);
+    st.last = s;
+    st.used = true;
+    return true;
 }
 
 }  // namespace
@@ -322,16 +453,31 @@ bool big16_applicable(const Problem& p) {
     if (p.in_dtype != MI_F16 && p.in_dtype != MI_BF16) return false;
     // M and K multiples of 8 (A and B move in 16-byte chunks along m and k), any N
     const int64_t tiles = tiles_of(p, 128, 128);   // (from 16 tiles of 128x128 on, this kernel is no slower than 64x64 tiles)
+    int split = 0, kchunk = 0;
     return p.M % 8 == 0 && p.M >= 8 && p.N >= 1 && p.K % 8 == 0 && p.K >= 256 && aligned(p.A, 16) && aligned(p.B, 16) &&
            p.lda % 8 == 0 && p.ldb % 8 == 0 && p.sa % 8 == 0 && p.sb % 8 == 0 && p.ldc < (1 << 26) &&
            // (the kernel's 32-bit lane offsets assume rows that follow each other upwards in memory)
            p.lda >= p.M && p.ldb >= p.K && p.ldc >= p.M && p.sa >= 0 && p.sb >= 0 && p.sc >= 0 &&
-           p.lda < (1 << 26) && p.ldb < (1 << 26) && tiles >= 16 && tiles < (1 << 30);
+           p.lda < (1 << 26) && p.ldb < (1 << 26) && tiles < (1 << 30) &&
+           // (fewer than 16 tiles only when the split over K multiplies the workgroups)
+           (tiles >= 16 || (split = pick_split(p, &kchunk), (int64_t)split * tiles >= 16));
 }
 
 void big16_launch(const Problem& p, hipStream_t s) {
     const bool f32out = p.out_dtype == MI_F32;
     const int t = pick_direct_tile(p);
+    int kchunk = 0;
+    const int parts = t == 22 ? pick_split(p, &kchunk) : 0;
+    if (parts > 1 && (p.in_dtype == MI_F16 ? launch_split<F16>(p, s, parts, kchunk) : launch_split<BF16>(p, s, parts, kchunk))) {
+        static const char* names[17] = {"", "", "gemm16_big_128x128x32_ring4_splitk2", "gemm16_big_128x128x32_ring4_splitk3",
+            "gemm16_big_128x128x32_ring4_splitk4", "gemm16_big_128x128x32_ring4_splitk5", "gemm16_big_128x128x32_ring4_splitk6",
+            "gemm16_big_128x128x32_ring4_splitk7", "gemm16_big_128x128x32_ring4_splitk8", "gemm16_big_128x128x32_ring4_splitk9",
+            "gemm16_big_128x128x32_ring4_splitk10", "gemm16_big_128x128x32_ring4_splitk11", "gemm16_big_128x128x32_ring4_splitk12",
+            "gemm16_big_128x128x32_ring4_splitk13", "gemm16_big_128x128x32_ring4_splitk14", "gemm16_big_128x128x32_ring4_splitk15",
+            "gemm16_big_128x128x32_ring4_splitk16"};
+        set_variant(names[parts]);
+        return;
+    }
 #define BIG(E, O) (t == 22 ? launch<E, O, 2, 2>(p, s) : t == 42 ? launch<E, O, 4, 2>(p, s) : launch<E, O, 4, 4>(p, s))
     if (p.in_dtype == MI_F16) {
         if (f32out) BIG(F16, float);

@@ -107,6 +107,68 @@ def test_matmul_large_tile_kernel_exact(ct, orc, M, N, K, T, out32, tile):
     assert np.array_equal(orc.to_julia(C).astype(np.float32), ref)
 
 
+@pytest.mark.parametrize("M,N,K,T,out32", [(512, 512, 4096, torch.float16, True), (512, 512, 4096, torch.bfloat16, False),
+                                            (1024, 1024, 8192, torch.float16, False), (256, 256, 4096, torch.float16, True),
+                                            (520, 500, 4000, torch.float16, True), (264, 1001, 3080, torch.bfloat16, False)])
+def test_matmul_split_over_k_exact(ct, orc, M, N, K, T, out32):
+    """Few tiles and a long K: the 128 x 128 direct-to-LDS kernel runs in several parts along K that write fp32
+    partial sums into the library's static scratch, and a second kernel adds the parts in fixed order.  Exact
+    integer sums (K off the part grid, M and N off the tile grid included); A and B are views of buffers whose
+    cells past K hold NaN and C is a view of a larger buffer filled with a sentinel."""
+    rng = np.random.default_rng(M + K)
+    A = rng.integers(-1, 2, (M, K)).astype(np.float32); B = rng.integers(-1, 2, (K, N)).astype(np.float32)
+    Abuf = torch.full((K + 128, M), float("nan"), dtype=T, device="cuda"); Bbuf = torch.full((N, K + 128), float("nan"), dtype=T, device="cuda")
+    Abuf[:K] = orc.from_julia(A).to(T).cuda(); Bbuf[:, :K] = orc.from_julia(B).to(T).cuda()
+    buf = torch.full((N + 3, M + 24), -77.0, dtype=torch.float32 if out32 else T, device="cuda")
+    C = buf[:N, :M]
+    ct.matmul_kernel(Abuf[:K], Bbuf[:, :K], C, 64, 64, 64)
+    assert ct.last_variant().startswith("gemm16_big_128x128x32_ring4_splitk")
+    ref = A @ B
+    assert out32 or np.abs(ref).max() <= (2048 if T == torch.float16 else 256)   # integers the output type holds exactly
+    assert np.array_equal(orc.to_julia(C.contiguous()).astype(np.float32), ref)
+    assert bool((buf[N:] == -77.0).all()) and bool((buf[:, M:] == -77.0).all())
+
+
+def test_matmul_split_over_k_is_reproducible_and_ordered_across_streams(ct, orc):
+    """The parts are added in a fixed order, so two runs give the same bits; launches from two streams share the
+    scratch and are ordered by the library, so alternating between streams still gives every product its own
+    result.  Random f16 data against the float64 product."""
+    rng = np.random.default_rng(21)
+    M = N = 512; K = 4096
+    mats = []
+    for i in range(3):
+        a = (rng.standard_normal((M, K)) / 8).astype(np.float32); b = (rng.standard_normal((K, N)) / 8).astype(np.float32)
+        mats.append((orc.from_julia(a).to(torch.float16).cuda(), orc.from_julia(b).to(torch.float16).cuda()))
+    torch.cuda.synchronize()
+    streams = [torch.cuda.Stream(), torch.cuda.Stream()]
+    outs = [torch.empty((N, M), dtype=torch.float32, device="cuda") for _ in range(6)]
+    for i in range(6):
+        At, Bt = mats[i % 3]
+        ct.matmul_kernel(At, Bt, outs[i], 64, 64, 64, stream=streams[i % 2])
+    assert ct.last_variant().startswith("gemm16_big_128x128x32_ring4_splitk")
+    torch.cuda.synchronize()
+    for i in range(3):
+        assert torch.equal(outs[i], outs[i + 3])
+        At, Bt = mats[i]
+        ref = orc.to_julia(At).astype(np.float64) @ orc.to_julia(Bt).astype(np.float64)
+        got = orc.to_julia(outs[i]).astype(np.float64)
+        assert np.abs(got - ref).max() <= 1e-5 * (np.abs(ref).max() + 1.0) * 4
+
+
+def test_batch_matmul_split_over_k_exact(ct, orc):
+    """Two entries of 512 x 512 x 8192: 32 tiles, split over K as well."""
+    rng = np.random.default_rng(5)
+    Bn, M, N, K = 2, 512, 512, 8192
+    A = rng.integers(-1, 2, (Bn, M, K)).astype(np.float32); B = rng.integers(-1, 2, (Bn, K, N)).astype(np.float32)
+    At = torch.from_numpy(np.ascontiguousarray(A.transpose(0, 2, 1))).to(torch.float16).cuda()   # Julia (M, K, Bn)
+    Bt = torch.from_numpy(np.ascontiguousarray(B.transpose(0, 2, 1))).to(torch.float16).cuda()   # Julia (K, N, Bn)
+    C = torch.empty((Bn, N, M), dtype=torch.float32, device="cuda")
+    ct.batch_matmul_kernel(At, Bt, C, 64, 64, 64)
+    assert ct.last_variant().startswith("gemm16_big_128x128x32_ring4_splitk")
+    got = C.cpu().numpy().transpose(0, 2, 1)
+    assert np.array_equal(got, A @ B)
+
+
 @pytest.mark.parametrize("M,N,K,T,out32,tile", [(2040, 2000, 256, torch.float16, True, "128x128"), (2056, 2311, 384, torch.bfloat16, False, "256x128"),
                                                  (4000, 4001, 256, torch.float16, False, "256x256"), (8, 16385, 256, torch.float16, True, "128x128"),
                                                  (2048, 2048, 264, torch.float16, True, "128x128"), (2040, 2000, 1000, torch.float16, False, "128x128"),

@@ -47,7 +47,8 @@ def eltype(ct, text, leaves=(), scalars=()):
     ("lt(a0,a1)", ("Float32", "Int32"), (), "Bool"),
     ("ifelse(lt(a0,a1),a0,a1)", ("Float32", "Float64"), (), "Float64"),
     ("pow(a0,a1)", ("Float32", "Int64"), (), "Float32"),
-    ("pow(a0,a1)", ("Int32", "Int64"), (), "Int64"),
+    ("pow(a0,a1)", ("Int32", "Int64"), (), "Int32"),           # Julia: ^(x::T, p::Integer) keeps the base type
+    ("pow(a0,a1)", ("Bool", "Int64"), (), "Bool"),
     ("pow(a0,a1)", ("Float32", "Float64"), (), "Float64"),
     ("neg(a0)", ("Bool",), (), "Int64"),
     ("not(a0)", ("Bool",), (), "Bool"),

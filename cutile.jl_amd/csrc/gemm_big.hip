@@ -421,7 +421,14 @@ bool launch_split(const Problem& p, hipStream_t s, int parts, int kchunk) {
     // The previous user of the partial sums, if it ran on another stream, has to finish first: an event recorded
     // on that stream now (it covers everything the stream has been given so far) and awaited by this one.
     if (st.used && st.last != s) {
-        if (hipEventRecord(st.done, st.last) != hipSuccess || hipStreamWaitEvent(s, st.done, 0) != hipSuccess) {
+        bool ordered;
+        if (hipEventRecord(st.done, st.last) == hipSuccess) {
+            ordered = hipStreamWaitEvent(s, st.done, 0) == hipSuccess;
+        } else {   // that stream no longer exists: what it was given is done once the device is idle
+            (void)hipGetLastError();
+            ordered = hipDeviceSynchronize() == hipSuccess;
+        }
+        if (!ordered) {
             (void)hipGetLastError();
             return false;
         }

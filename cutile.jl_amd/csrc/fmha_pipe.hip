@@ -12,12 +12,13 @@
 // K and V travel in halves of 32 keys (4 KB each) through two rings of four LDS slots, filled
 // by direct global->LDS loads three steps ahead of their use.  One step handles one half j:
 //     raise the running maxima if the maxima of S(j) (taken in the previous step) demand it
-//     barrier (publishes the halves issued three steps ago), issue loads of K half j+5, V half j+3
-//     read the V(j) fragments
-//     S(j+1) = K(j+1) . Q   (K fragments already in registers)   |  interleaved, one MFMA per
-//     weights P(j) = exp2(S(j) - m), packed, row sums            |  issue slot, with the
-//     O += V(j) . P(j)      as soon as a 16-key chunk of P exists|  vector work
-//     read the K(j+2) fragments; row maxima of S(j+1)
+//     barrier (publishes the halves issued three steps ago)
+//     sixteen issue slots, each one MFMA -- first the ten of S(j+1) = K(j+1) . Q (K fragments already in
+//     registers), then O += V(j) . P(j) chunk by chunk as soon as a 16-key chunk of P exists -- and one piece
+//     of the weights P(j) = exp2(S(j) - m) (2 exp2, pack, row sum); the step's fixed work rides along a few
+//     instructions per slot: the V(j) fragment reads, the requests for K half j+5 and V half j+3, the
+//     K(j+2) fragment reads, the row maxima of S(j+1) in stages
+//     the last two P.V MFMAs
 // The two score buffers swap roles every step (the loops are unrolled by two), so no register
 // copies are needed.  The global->LDS loads are issued from inline assembly and waited for with
 // explicit vmcnt counts; the compiler sees only the LDS reads.
@@ -126,6 +127,30 @@ __device__ __forceinline__ void issue_v(Lane& c, int slot) {
     if (c.v_left > 0) c.vptr += c.v_half_bytes;
 }
 
+// The same transfers one at a time (PART 0 / 1 of a half), for steps that spread them over their issue slots.
+template <int PART>
+__device__ __forceinline__ void issue_k_part(Lane& c, int slot) {
+    const unsigned lds = c.ks_base + slot * kSlotBytes + c.wave * 1024;
+    if (PART == 0) {
+        dma16(c.kdma, c.kptr, lds);
+    } else {
+        dma16(c.kdma, c.kptr + (c.k_half_bytes >> 1), lds + 2048);
+        c.k_left -= 1;
+        if (c.k_left > 0) c.kptr += c.k_half_bytes;
+    }
+}
+template <int PART>
+__device__ __forceinline__ void issue_v_part(Lane& c, int slot) {
+    const unsigned lds = c.vs_base + slot * kSlotBytes + c.wave * 1024;
+    if (PART == 0) {
+        dma16(c.vdma, c.vptr, lds);
+    } else {
+        dma16(c.vdma, c.vptr + (c.v_half_bytes >> 1), lds + 2048);
+        c.v_left -= 1;
+        if (c.v_left > 0) c.vptr += c.v_half_bytes;
+    }
+}
+
 __device__ __forceinline__ void read_k_frags(const unsigned short* Ks, const Lane& c, int slot, s16x8 (&kf)[4]) {
 #pragma unroll
     for (int ks = 0; ks < 4; ++ks) kf[ks] = *reinterpret_cast<const s16x8*>(Ks + slot * kSlot + c.kfo[ks]);
@@ -143,6 +168,28 @@ __device__ __forceinline__ float masked_row_max(f32x16& s, int lim) {
 #pragma unroll
     for (int r = 3; r < 15; r += 2) mx = max3(mx, s[r], s[r + 1]);
     return xhalf_max(max3(mx, s[15], s[15]));
+}
+
+// The same in three stages of three to four instructions (eleven with the mask), for steps that spread the row
+// maxima over their issue slots: stage 0 and 1 take eight scores each, stage 2 the last one and the other half-wave.
+template <bool MASK, int STAGE>
+__device__ __forceinline__ void row_max_stage(f32x16& s, int lim, float& mx, float& out) {
+    if (MASK && STAGE < 2) {
+#pragma unroll
+        for (int r = 8 * STAGE; r < 8 * STAGE + 8; ++r) s[r] = (8 * (r >> 2) + (r & 3) <= lim) ? s[r] : -INFINITY;
+    }
+    if (STAGE == 0) {
+        mx = max3(s[0], s[1], s[2]);
+        mx = max3(mx, s[3], s[4]);
+        mx = max3(mx, s[5], s[6]);
+    } else if (STAGE == 1) {
+        mx = max3(mx, s[7], s[8]);
+        mx = max3(mx, s[9], s[10]);
+        mx = max3(mx, s[11], s[12]);
+        mx = max3(mx, s[13], s[14]);
+    } else {
+        out = xhalf_max(max3(mx, s[15], s[15]));
+    }
 }
 
 // The weights of one score pair (2h, 2h+1), h = 0..7, are made in two stages that the step below
@@ -217,22 +264,22 @@ __device__ __forceinline__ void half_step(const unsigned short* Ks, const unsign
         }
     }
     wait_and_barrier<kWaitVm8>();
-    issue_k(c, (j + 1) & 3);  // half j+5
-    issue_v(c, (j + 3) & 3);  // half j+3
-    // ---- V(j) fragments ------------------------------------------------------------------------------
-    s16x8 vf[2][2];  // [16-key chunk][d tile]
-    {
-        const unsigned short* vb = Vs + (j & 3) * kSlot;
-#pragma unroll
-        for (int ch = 0; ch < 2; ++ch)
-#pragma unroll
-            for (int dt = 0; dt < 2; ++dt) {
-                const unsigned short* p = vb + c.vfo[dt] + 16 * ch * kD;
-                s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16(LDS_PTR(s16x4, p));
-                s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(LDS_PTR(s16x4, p + 8 * kD));
-                vf[ch][dt] = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
-            }
-    }
+    // The rest of a step's fixed work rides in the issue slots below, a few instructions per slot: under two
+    // waves per SIMD a slot lasts as long as two MFMAs, and a wave needs less than that for its MFMA and its piece.
+    s16x8 vf[2][2];  // V(j) fragments, [16-key chunk][d tile]
+    auto vread = [&](int f) {
+        const int ch = f >> 1, dt = f & 1;
+        const unsigned short* p = Vs + (j & 3) * kSlot + c.vfo[dt] + 16 * ch * kD;
+        s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16(LDS_PTR(s16x4, p));
+        s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(LDS_PTR(s16x4, p + 8 * kD));
+        vf[ch][dt] = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+    };
+    auto dma = [&](int d) {   // halves K(j+5) and V(j+3), two transfers each
+        if (d == 0) issue_k_part<0>(c, (j + 1) & 3);
+        else if (d == 1) issue_k_part<1>(c, (j + 1) & 3);
+        else if (d == 2) issue_v_part<0>(c, (j + 3) & 3);
+        else issue_v_part<1>(c, (j + 3) & 3);
+    };
     unsigned pf[2][2][4];
     slot_end();
 
@@ -269,10 +316,22 @@ __device__ __forceinline__ void half_step(const unsigned short* Ks, const unsign
         }
         ++xi;
     };
-    auto maxima = [&]() {
-        const int jn = nth_stream(NEXT, mi);
-        cand[jn] = MASKN == jn ? masked_row_max<true>(s_next[jn], c.q0[jn] + c.lim0 - kHK * (j + 1))
-                               : masked_row_max<false>(s_next[jn], 0);
+    // row maxima of S(j+1) in stages, stream by stream
+    constexpr int nStages = 3 * nN;
+    constexpr int kMaxStart = nQ + 1;   // the slot after the one that follows the last S MFMA
+    float mx = 0.f;
+    auto max_stage = [&]() {
+        const int jn = nth_stream(NEXT, mi / 3);
+        const int lim = c.q0[jn] + c.lim0 - kHK * (j + 1);
+        if (MASKN == jn) {
+            if (mi % 3 == 0) row_max_stage<true, 0>(s_next[jn], lim, mx, cand[jn]);
+            else if (mi % 3 == 1) row_max_stage<true, 1>(s_next[jn], lim, mx, cand[jn]);
+            else row_max_stage<true, 2>(s_next[jn], lim, mx, cand[jn]);
+        } else {
+            if (mi % 3 == 0) row_max_stage<false, 0>(s_next[jn], lim, mx, cand[jn]);
+            else if (mi % 3 == 1) row_max_stage<false, 1>(s_next[jn], lim, mx, cand[jn]);
+            else row_max_stage<false, 2>(s_next[jn], lim, mx, cand[jn]);
+        }
         ++mi;
     };
     // the K(j+2) fragments are read once every S MFMA has been issued: the old fragments are free then
@@ -284,18 +343,22 @@ __device__ __forceinline__ void half_step(const unsigned short* Ks, const unsign
         }
     };
     // A: one MFMA and one exp piece per slot.  First the S MFMAs, then the P.V MFMAs of a chunk as soon as that
-    // chunk's weights exist.
+    // chunk's weights exist.  Slots 0..3 also read one V fragment each (the first P.V MFMA is in slot 5 at the
+    // earliest), slots 4..7 request one transfer each, and from slot kMaxStart on a slot takes a stage of the maxima.
 #pragma unroll
     for (int sl = 0; sl < 8 * nC; ++sl) {
         if (qi < nQ) mfma_q();
         else if (p0 < nP && xi > 4 * ((p0 / 2) + 1)) mfma_p(0, p0++);
         else if (p1 < nP && xi > 4 * nC + 4 * (p1 / 2 + 1)) mfma_p(1, p1++);
         after_q();
+        if (sl < 4) vread(sl);
+        else if (sl < 8) dma(sl - 4);
+        if (sl >= kMaxStart && mi < nStages) max_stage();
         piece();
         slot_end();
     }
     piece();  // finishes the last pair
-    // B: the remaining MFMAs, with the row maxima of S(j+1) between them
+    // B: the remaining MFMAs, with what is left of the row maxima between them
     after_q();
 #pragma unroll
     for (int sl = 0; sl < 2 * nQ + 2 * nP; ++sl) {
@@ -304,11 +367,11 @@ __device__ __forceinline__ void half_step(const unsigned short* Ks, const unsign
         else if (p1 < nP) mfma_p(1, p1++);
         else break;
         after_q();
-        if (qi == nQ && mi < nN) maxima();
+        if (qi == nQ && mi < nStages) max_stage();
         slot_end();
     }
 #pragma unroll
-    while (mi < nN) maxima();
+    while (mi < nStages) max_stage();
 }
 
 // One wide step: the long tile of a wave (stream 1) alone, over the two halves j and j+1.  Once the early
@@ -352,24 +415,25 @@ __device__ __forceinline__ void wide_step(const unsigned short* Ks, const unsign
         }
     }
     wait_and_barrier<kWaitVm0>();   // everything requested one trip ago has landed, and every wave knows
-    issue_k(c, (j + 2) & 3);        // halves j+6, j+7 (the fragments of j+2, j+3 are in registers)
-    issue_k(c, (j + 3) & 3);
-    if (!first) issue_v(c, (j + 2) & 3);   // half j+2 (the narrow steps had requested it already)
-    issue_v(c, (j + 3) & 3);               // half j+3
+    // As in the narrow step, the fixed work of the trip rides in the issue slots.
     s16x8 vf[2][2][2];  // [half][16-key chunk][d tile]
-#pragma unroll
-    for (int h = 0; h < 2; ++h) {
-        const unsigned short* vb = Vs + ((j + h) & 3) * kSlot;
-#pragma unroll
-        for (int ch = 0; ch < 2; ++ch)
-#pragma unroll
-            for (int dt = 0; dt < 2; ++dt) {
-                const unsigned short* p = vb + c.vfo[dt] + 16 * ch * kD;
-                s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16(LDS_PTR(s16x4, p));
-                s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(LDS_PTR(s16x4, p + 8 * kD));
-                vf[h][ch][dt] = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
-            }
-    }
+    auto vread = [&](int f) {
+        const int h = f >> 2, ch = (f >> 1) & 1, dt = f & 1;
+        const unsigned short* p = Vs + ((j + h) & 3) * kSlot + c.vfo[dt] + 16 * ch * kD;
+        s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16(LDS_PTR(s16x4, p));
+        s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(LDS_PTR(s16x4, p + 8 * kD));
+        vf[h][ch][dt] = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+    };
+    auto dma = [&](int d) {   // K(j+6), K(j+7) (the fragments of j+2, j+3 are in registers), V(j+2), V(j+3)
+        if (d == 0) issue_k_part<0>(c, (j + 2) & 3);
+        else if (d == 1) issue_k_part<1>(c, (j + 2) & 3);
+        else if (d == 2) issue_k_part<0>(c, (j + 3) & 3);
+        else if (d == 3) issue_k_part<1>(c, (j + 3) & 3);
+        else if (d == 4) { if (!first) issue_v_part<0>(c, (j + 2) & 3); }   // (the narrow steps had requested V(j+2) already)
+        else if (d == 5) { if (!first) issue_v_part<1>(c, (j + 2) & 3); }
+        else if (d == 6) issue_v_part<0>(c, (j + 3) & 3);
+        else issue_v_part<1>(c, (j + 3) & 3);
+    };
     unsigned pf[2][2][4];   // [half][chunk][pair]
     slot_end();
 
@@ -404,44 +468,53 @@ __device__ __forceinline__ void wide_step(const unsigned short* Ks, const unsign
         }
         ++xi;
     };
-    bool kread = !NEXT;
-    auto after_q = [&]() {
-        if (!kread && qi == nQ) {
-            if (j + 4 < c.nh) {
-                read_k_frags(Ks, c, (j + 4) & 3, kf[0]);
-                read_k_frags(Ks, c, (j + 5) & 3, kf[1]);
-            }
-            kread = true;
-        }
+    // row maxima of S(j+2), S(j+3) in stages
+    constexpr int nStages = NEXT ? 6 : 0;
+    int mi = 0;
+    float mx = 0.f;
+    auto max_stage = [&]() {
+        const int h = mi / 3;
+        f32x16& n = h ? n1 : n0;
+        const int lim = c.q0[1] + c.lim0 - kHK * (j + 2 + h);
+        if (mi % 3 == 0) row_max_stage<MASK, 0>(n, lim, mx, cand[h]);
+        else if (mi % 3 == 1) row_max_stage<MASK, 1>(n, lim, mx, cand[h]);
+        else row_max_stage<MASK, 2>(n, lim, mx, cand[h]);
+        ++mi;
     };
+    const bool more_k = j + 4 < c.nh;   // (the last trips have no K(j+4), K(j+5) to fetch)
+    // Slots 0..3: two V fragments each (the first P.V MFMA is in slot 5 at the earliest); slots 4..8 and 11..13: one
+    // transfer each; slots 9, 10: the K(j+4) / K(j+5) fragments, each right after the last S MFMA that read the old
+    // ones; from slot 11 on a stage of the maxima.
 #pragma unroll
     for (int sl = 0; sl < 16; ++sl) {
         if (qi < nQ) mfma_q();
         else if (p0 < nP && xi > 4 * ((p0 / 2) + 1)) mfma_p(0, p0++);
         else if (p1 < nP && xi > 8 + 4 * (p1 / 2 + 1)) mfma_p(1, p1++);
-        after_q();
+        if (sl < 4) {
+            vread(2 * sl);
+            vread(2 * sl + 1);
+        } else if (sl < 9) {
+            dma(sl - 4);
+        } else if (sl < 11) {
+            if (NEXT && more_k) read_k_frags(Ks, c, (j + 4 + (sl - 9)) & 3, kf[sl - 9]);
+        } else if (sl < 14) {
+            dma(sl - 6);
+        }
+        if (sl >= 11 && mi < nStages) max_stage();
         piece();
         slot_end();
     }
     piece();  // finishes the last pair
-    int mi = 0;
-    auto maxima = [&]() {
-        f32x16& n = mi ? n1 : n0;
-        cand[mi] = MASK ? masked_row_max<true>(n, c.q0[1] + c.lim0 - kHK * (j + 2 + mi)) : masked_row_max<false>(n, 0);
-        ++mi;
-    };
 #pragma unroll
     for (int sl = 0; sl < 2 * nP; ++sl) {
         if (p0 < nP) mfma_p(0, p0++);
         else if (p1 < nP) mfma_p(1, p1++);
         else break;
-        if (NEXT && mi < 2) maxima();
+        if (mi < nStages) max_stage();
         slot_end();
     }
-    if (NEXT) {
 #pragma unroll
-        while (mi < 2) maxima();
-    }
+    while (mi < nStages) max_stage();
 }
 
 template <typename E, bool CAUSAL>

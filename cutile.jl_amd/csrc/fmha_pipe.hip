@@ -27,7 +27,8 @@
 // only raised when the new maximum exceeds it by more than 8 (a factor 256 in the weights):
 // the result is the same function of the inputs, the weights P stay below 2^8 in the storage
 // type, and the accumulator rescale all but disappears.  Row sums are taken over the rounded
-// weights, i.e. over exactly the values that multiply V.
+// weights, i.e. over exactly the values that multiply V (f16; bf16 has no mixed-precision fma, its
+// row sums take the weights before rounding).
 #include "fmha_common.h"
 
 namespace mi {

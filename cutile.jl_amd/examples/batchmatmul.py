@@ -29,6 +29,13 @@ def run(data, *, tm: int = 128, tn: int = 128, tk: int = 64, nruns: int = 1, war
     return namespace(C=data.C, times=times)
 
 
+
+def run_others(data, *, nruns: int = 1, warmup: int = 0):
+    """batchmatmul.jl:117-146 compares with cuBLAS' strided-batched GEMM; here ``torch.bmm``."""
+    C = torch.empty((data.Batch, data.N, data.M), dtype=data.A.dtype, device=data.A.device)
+    return {"rocBLAS batched (torch.bmm)": time_launches(lambda: torch.bmm(data.B, data.A, out=C), nruns, warmup)}
+
+
 def metric(data):
     """batchmatmul.jl:108-111."""
     return 2 * data.M * data.K * data.N * data.Batch, "TFLOPS"

@@ -57,6 +57,12 @@ def run(data, *, nruns: int = 1, warmup: int = 0):
     return namespace(output=output, times=times)
 
 
+
+def run_others(data, *, nruns: int = 1, warmup: int = 0):
+    """fft.jl:262-279 compares with cuFFT; here rocFFT through ``torch.fft.fft`` over the batch."""
+    return {"rocFFT (torch.fft.fft)": time_launches(lambda: torch.fft.fft(data.input, dim=1), nruns, warmup)}
+
+
 def metric(data):
     """fft.jl:253-256: a latency benchmark, the time itself is the figure."""
     return 0, "us"

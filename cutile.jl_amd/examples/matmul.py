@@ -32,6 +32,14 @@ def run(data, *, tm: int = 64, tn: int = 64, tk: int = 64, nruns: int = 1, warmu
     return namespace(C=data.C, times=times)
 
 
+
+def run_others(data, *, nruns: int = 1, warmup: int = 0):
+    """matmul.jl:112-141 compares with cuBLAS through ``mul!``; here hipBLASLt / rocBLAS through
+    ``torch.matmul`` (Julia C = A * B is torch C^T = B^T A^T on the same bytes; the result has the operands' type)."""
+    C = torch.empty((data.N, data.M), dtype=data.A.dtype, device=data.A.device)
+    return {"hipBLASLt (torch.matmul)": time_launches(lambda: torch.matmul(data.B, data.A, out=C), nruns, warmup)}
+
+
 def metric(data):
     """matmul.jl:103-106."""
     return 2 * data.M * data.N * data.K, "TFLOPS"

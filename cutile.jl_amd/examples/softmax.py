@@ -53,6 +53,22 @@ def run(data, *, tile_tma: int | None = None, tile_chunked: int = 1024, nruns: i
                      times={"cuTile TMA": times_tma, "cuTile Chunked": times_chunked})
 
 
+
+def run_others(data, *, nruns: int = 1, warmup: int = 0):
+    """softmax.jl:205-232 compares with the unfused broadcast formulation on GPUArrays; the same three
+    passes on ``torch``, and ``torch.softmax`` (one fused kernel of the vendor library) beside it."""
+    x = data.input                      # torch (M, N): a Julia column is a torch row
+    out = torch.empty_like(x)
+
+    def broadcast():
+        m = x.amax(dim=1, keepdim=True)
+        e = torch.exp(x - m)
+        torch.div(e, e.sum(dim=1, keepdim=True), out=out)
+
+    return {"torch broadcast": time_launches(broadcast, nruns, warmup),
+            "torch.softmax": time_launches(lambda: torch.softmax(x, dim=1), nruns, warmup)}
+
+
 def metric(data):
     """softmax.jl:190-198."""
     MN = data.M * data.N * 4

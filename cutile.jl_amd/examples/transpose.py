@@ -25,6 +25,14 @@ def run(data, *, tm: int = 64, tn: int = 64, nruns: int = 1, warmup: int = 0):
     return namespace(y=data.y, times=times)
 
 
+
+def run_others(data, *, nruns: int = 1, warmup: int = 0):
+    """transpose.jl:72-123 compares with GPUArrays' ``permutedims!`` (and a naive SIMT kernel); here
+    ``y.copy_(x.t())`` of the library behind ``torch``."""
+    y = torch.empty_like(data.y)
+    return {"torch copy_(x.t())": time_launches(lambda: y.copy_(data.x.t()), nruns, warmup)}
+
+
 def metric(data):
     """transpose.jl:62-66: 1 read + 1 write."""
     return 2 * data.m * data.n * data.x.element_size(), "GB/s"

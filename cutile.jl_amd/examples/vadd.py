@@ -35,6 +35,14 @@ def run(data, *, tile=1024, nruns: int = 1, warmup: int = 0):
     return namespace(c=c, times=times)
 
 
+
+def run_others(data, *, nruns: int = 1, warmup: int = 0):
+    """vadd.jl:141-195 compares with GPUArrays' broadcast (and a SIMT kernel); here the library behind
+    ``torch`` plays that part: ``torch.add`` into a preallocated result."""
+    c = torch.empty_like(data.a)
+    return {"torch.add": time_launches(lambda: torch.add(data.a, data.b, out=c), nruns, warmup)}
+
+
 def metric(data):
     """vadd.jl:131-136: 2 reads + 1 write."""
     n = int(np.prod(data.shape))

@@ -54,5 +54,14 @@ def time_launches(fn, nruns: int, warmup: int) -> list[float]:
     return times
 
 
+def isapprox(x: torch.Tensor, y: torch.Tensor, *, rtol: float | None = None, atol: float = 0.0) -> bool:
+    """Julia's ``isapprox`` for arrays: ``norm(x - y) <= max(atol, rtol * max(norm(x), norm(y)))`` with the
+    2-norm, and ``rtol = sqrt(eps)`` of the element type when neither tolerance is given."""
+    if rtol is None:
+        rtol = float(torch.finfo(x.dtype).eps) ** 0.5 if atol == 0.0 and x.dtype.is_floating_point else 0.0
+    xd, yd = x.double().flatten(), y.double().flatten()
+    return bool(torch.linalg.vector_norm(xd - yd) <= max(atol, rtol * max(torch.linalg.vector_norm(xd), torch.linalg.vector_norm(yd))))
+
+
 def namespace(**kw) -> SimpleNamespace:
     return SimpleNamespace(**kw)

@@ -5,7 +5,7 @@ import numpy as np
 import torch
 
 import cutile_jl_amd as ct
-from ._harness import namespace, rand_uniform, time_launches
+from ._harness import isapprox, namespace, rand_uniform, time_launches
 
 
 def prepare(*, benchmark: bool = False, M: int | None = None, K: int | None = None, N: int | None = None,
@@ -36,6 +36,14 @@ def run_others(data, *, nruns: int = 1, warmup: int = 0):
     return {"rocBLAS batched (torch.bmm)": time_launches(lambda: torch.bmm(data.B, data.A, out=C), nruns, warmup)}
 
 
+
+def verify(data, result) -> None:
+    """batchmatmul.jl:96-107: every batch entry against the host product, ``rtol = 1e-2`` over the whole array."""
+    expected = torch.bmm(data.B.cpu().float(), data.A.cpu().float())
+    got = result.C.cpu().float()
+    assert isapprox(got, expected, rtol=1e-2), f"max diff: {float((got - expected).abs().max())}"
+
+
 def metric(data):
     """batchmatmul.jl:108-111."""
     return 2 * data.M * data.K * data.N * data.Batch, "TFLOPS"
@@ -48,3 +56,23 @@ def smoke(orc):
     got = orc.to_julia(r.C).astype(np.float64)
     assert np.abs(got - ref).max() <= 1e-5 * np.abs(ref).max()
 
+
+def test_batch_matmul(T: torch.dtype, M: int, K: int, N: int, Batch: int, tm: int, tn: int, tk: int, *,
+                      name: str | None = None) -> None:
+    """batchmatmul.jl:152-159."""
+    name = name or (f"batch_matmul ({M} x {K} x {Batch}) @ ({K} x {N} x {Batch}), {str(T).replace('torch.', '')}, "
+                    f"tiles={tm} x {tn} x {tk}")
+    print(f"--- {name} ---")
+    data = prepare(M=M, K=K, N=N, Batch=Batch, T=T)
+    result = run(data, tm=tm, tn=tn, tk=tk)
+    verify(data, result)
+    print("  passed")
+
+
+def main() -> None:
+    """batchmatmul.jl:161-169."""
+    print("--- Batch Matrix Multiplication Examples ---\n")
+    test_batch_matmul(torch.float32, 256, 128, 256, 4, 32, 32, 32)
+    test_batch_matmul(torch.float32, 512, 256, 512, 4, 64, 64, 64)
+    test_batch_matmul(torch.float16, 512, 256, 1024, 4, 128, 256, 64)
+    print("\n--- All batch matmul examples completed ---")

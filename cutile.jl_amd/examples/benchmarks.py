@@ -5,8 +5,8 @@ It finds the example modules of this package, and for each calls ``prepare(bench
 prints one table per example with the minimum and mean time of every implementation and the throughput
 computed from the minimum (benchmarks.jl:26-62,136-183).
 
-    python cutile.jl_amd/examples/benchmarks.py            # every example
-    python cutile.jl_amd/examples/benchmarks.py matmul fmha
+    python cutile.jl_amd/examples benchmarks               # every example
+    python cutile.jl_amd/examples benchmarks matmul fmha
 """
 from __future__ import annotations
 
@@ -111,10 +111,3 @@ def main(*args, file=sys.stdout) -> None:
     print("  Benchmark Complete", file=file)
     print("=" * 72, file=file)
 
-
-if __name__ == "__main__":
-    import os
-    sys.path.insert(0, os.path.dirname(os.path.dirname(os.path.dirname(os.path.abspath(__file__)))))
-    import __graft_entry__ as _g
-    _g.load_package()
-    main(*sys.argv[1:])

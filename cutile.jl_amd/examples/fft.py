@@ -5,7 +5,7 @@ import numpy as np
 import torch
 
 import cutile_jl_amd as ct
-from ._harness import namespace, time_launches, upload
+from ._harness import isapprox, namespace, time_launches, upload
 
 
 def dft_matrix(size: int) -> np.ndarray:
@@ -58,6 +58,16 @@ def run(data, *, nruns: int = 1, warmup: int = 0):
 
 
 
+
+def verify(data, result) -> None:
+    """fft.jl:245-248: against the host FFT along the signal axis (FFTW there, numpy's pocketfft here),
+    ``rtol = 1e-4`` in the norm."""
+    reference = torch.from_numpy(np.fft.fft(data.input.cpu().numpy().astype(np.complex128), axis=1))
+    got = result.output.cpu().to(torch.complex128)
+    err = torch.linalg.vector_norm(torch.view_as_real(got - reference))
+    assert float(err) <= 1e-4 * float(torch.linalg.vector_norm(torch.view_as_real(reference)))
+
+
 def run_others(data, *, nruns: int = 1, warmup: int = 0):
     """fft.jl:262-279 compares with cuFFT; here rocFFT through ``torch.fft.fft`` over the batch."""
     return {"rocFFT (torch.fft.fft)": time_launches(lambda: torch.fft.fft(data.input, dim=1), nruns, warmup)}
@@ -66,3 +76,22 @@ def run_others(data, *, nruns: int = 1, warmup: int = 0):
 def metric(data):
     """fft.jl:253-256: a latency benchmark, the time itself is the figure."""
     return 0, "us"
+
+
+def test_fft(batch: int, factors, *, name: str | None = None) -> None:
+    """fft.jl:285-293."""
+    n = factors[0] * factors[1] * factors[2]
+    name = name or f"fft batch={batch}, size={n}, factors={tuple(factors)}"
+    print(f"--- {name} ---")
+    data = prepare(batch=batch, factors=factors)
+    result = run(data)
+    verify(data, result)
+    print("  passed")
+
+
+def main() -> None:
+    """fft.jl:295-303."""
+    print("--- FFT Examples ---\n")
+    test_fft(64, (8, 8, 8))
+    test_fft(32, (8, 8, 8))
+    print("\n--- All FFT examples completed ---")

@@ -5,7 +5,7 @@ import numpy as np
 import torch
 
 import cutile_jl_amd as ct
-from ._harness import namespace, rand_normal, time_launches
+from ._harness import isapprox, namespace, rand_normal, time_launches
 
 
 def prepare(*, benchmark: bool = False, M: int | None = None, N: int | None = None,
@@ -59,7 +59,45 @@ def run(data, *, TILE_N: int = 1024, TILE_M: int = 32, nruns: int = 1, warmup: i
                      FINAL_DB=d.FINAL_DB, times_fwd=times_fwd, times_bwd=times_bwd)
 
 
+
+def verify(data, result) -> None:
+    """layernorm.jl:284-314: Y, dX, dW, dB against the host formulas in fp32, each ``rtol = 1e-2``.  The Julia
+    arrays are (N, M) with the row along the first axis; the torch tensors are (M, N), the row along dim 1."""
+    X, W, B, DY = data.X.cpu(), data.W.cpu(), data.B.cpu(), data.DY.cpu()
+    N, eps = data.N, data.eps
+    mean = X.sum(dim=1, keepdim=True) / N
+    var = ((X - mean) ** 2).sum(dim=1, keepdim=True) / N
+    rstd = 1.0 / torch.sqrt(var + eps)
+    xhat = (X - mean) * rstd
+    assert isapprox(xhat * W + B, result.Y.cpu(), rtol=1e-2), "Y mismatch"
+    wdy = W * DY
+    c1 = (xhat * wdy).sum(dim=1, keepdim=True) / N
+    c2 = wdy.sum(dim=1, keepdim=True) / N
+    assert isapprox((wdy - (xhat * c1 + c2)) * rstd, result.DX.cpu(), rtol=1e-2), "dX mismatch"
+    assert isapprox((DY * xhat).sum(dim=0), result.FINAL_DW.cpu(), rtol=1e-2), "dW mismatch"
+    assert isapprox(DY.sum(dim=0), result.FINAL_DB.cpu(), rtol=1e-2), "dB mismatch"
+
+
 def metric(data):
     """layernorm.jl:324-332 (the reference's formula, which counts its L2-served re-reads)."""
     MN = data.M * data.N * 4
     return {"cuTile Fwd": (4 * MN, "GB/s"), "cuTile Bwd": (5 * MN, "GB/s")}
+
+
+def test_layernorm(M: int, N: int, TILE_N: int, *, TILE_M: int = 32, eps: float = 1e-5, name: str | None = None) -> None:
+    """layernorm.jl:316-322."""
+    name = name or f"layernorm ({M} x {N}), tile_n={TILE_N}, tile_m={TILE_M}"
+    print(f"--- {name} ---")
+    data = prepare(M=M, N=N, eps=eps)
+    result = run(data, TILE_N=TILE_N, TILE_M=TILE_M)
+    verify(data, result)
+    print("  fwd passed, bwd passed")
+
+
+def main() -> None:
+    """layernorm.jl:340-348."""
+    print("=== LayerNorm Examples (fwd+bwd) ===\n")
+    test_layernorm(256, 256, 256)
+    test_layernorm(512, 512, 512)
+    test_layernorm(1024, 1024, 1024)
+    print("\n=== All layernorm examples completed ===")

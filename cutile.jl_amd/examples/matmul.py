@@ -5,7 +5,7 @@ import numpy as np
 import torch
 
 import cutile_jl_amd as ct
-from ._harness import namespace, rand_normal, rand_uniform, time_launches
+from ._harness import isapprox, namespace, rand_normal, rand_uniform, time_launches
 
 
 def prepare(*, benchmark: bool = False, M: int | None = None, N: int | None = None, K: int | None = None,
@@ -40,6 +40,15 @@ def run_others(data, *, nruns: int = 1, warmup: int = 0):
     return {"hipBLASLt (torch.matmul)": time_launches(lambda: torch.matmul(data.B, data.A, out=C), nruns, warmup)}
 
 
+
+def verify(data, result) -> None:
+    """matmul.jl:98-101: ``isapprox(C, A * B; rtol = 1e-2)`` against the host product (fp32 here for every
+    operand type).  Julia's A * B on the arrays' bytes is torch's B @ A."""
+    expected = data.B.cpu().float() @ data.A.cpu().float()
+    got = result.C.cpu().float()
+    assert isapprox(got, expected, rtol=1e-2), f"max diff: {float((got - expected).abs().max())}"
+
+
 def metric(data):
     """matmul.jl:103-106."""
     return 2 * data.M * data.N * data.K, "TFLOPS"
@@ -52,3 +61,22 @@ def smoke(orc):
     got = orc.to_julia(r.C).astype(np.float64)
     assert np.all(np.abs(got - ref) <= 2e-2 * np.abs(ref) + 2e-2 * np.abs(ref).max() * 1e-2), np.abs(got - ref).max()
 
+
+def test_matmul(T: torch.dtype, M: int, N: int, K: int, tm: int, tn: int, tk: int, *, name: str | None = None) -> None:
+    """matmul.jl:147-154."""
+    name = name or f"matmul ({M} x {K}) @ ({K} x {N}), {str(T).replace('torch.', '')}, tiles={tm} x {tn} x {tk}"
+    print(f"--- {name} ---")
+    data = prepare(M=M, N=N, K=K, T=T)
+    result = run(data, tm=tm, tn=tn, tk=tk)
+    verify(data, result)
+    print("  passed")
+
+
+def main() -> None:
+    """matmul.jl:156-165."""
+    print("--- Matrix Multiplication Examples ---\n")
+    test_matmul(torch.float32, 256, 256, 256, 32, 32, 32)
+    test_matmul(torch.float32, 512, 512, 512, 64, 64, 64)
+    test_matmul(torch.float32, 256, 512, 128, 32, 32, 32)
+    test_matmul(torch.float32, 1024, 1024, 1024, 64, 64, 64)
+    print("\n--- All matmul examples completed ---")

@@ -5,7 +5,7 @@ import numpy as np
 import torch
 
 import cutile_jl_amd as ct
-from ._harness import namespace, rand_normal, time_launches
+from ._harness import isapprox, namespace, rand_normal, time_launches
 
 
 def invoke_fused_moe_kernel(A, B, C, topk_weights, sorted_token_ids, sorted_expert_ids, *, mul_routed_weight,
@@ -140,6 +140,35 @@ def run(data, *, nruns: int = 1, warmup: int = 0, **kw):
     return namespace(out=holder["out"], times=times)
 
 
+
+def ref_moe(hidden_states, w1, w2, topk_weights, topk_ids) -> torch.Tensor:
+    """moe.jl:264-304 on the host in fp32, expert by expert.  Torch shapes (reversed Julia): hidden_states
+    (tokens, hidden); w1 (E, 2*inter, hidden); w2 (E, hidden, inter); topk_weights / topk_ids (topk, tokens),
+    ids 1-based.  Returns (tokens, hidden)."""
+    hs, w1f, w2f = hidden_states.cpu().float(), w1.cpu().float(), w2.cpu().float()
+    tw, ti = topk_weights.cpu().float(), topk_ids.cpu()
+    inter = w2f.shape[2]
+    result = torch.zeros_like(hs)
+    for e in range(w1f.shape[0]):
+        slot, tok = torch.nonzero(ti == e + 1, as_tuple=True)
+        if tok.numel() == 0:
+            continue
+        x = hs[tok]                                            # (count, hidden)
+        gate = x @ w1f[e, :inter].t()                          # (count, inter)
+        up = x @ w1f[e, inter:].t()
+        act = gate / (1.0 + torch.exp(-gate)) * up
+        y = act @ w2f[e].t()                                   # (count, hidden)
+        result.index_add_(0, tok, y * tw[slot, tok].unsqueeze(1))
+    return result
+
+
+def verify(data, result) -> None:
+    """moe.jl:370-374: ``isapprox(Float32.(out), ref_moe(...); rtol = 1e-2, atol = 1e-2)``."""
+    expected = ref_moe(data.hidden_states, data.w1, data.w2, data.topk_weights, data.topk_ids)
+    actual = result.out.cpu().float()
+    assert isapprox(actual, expected, rtol=1e-2, atol=1e-2), f"MoE incorrect! max diff: {float((actual - expected).abs().max())}"
+
+
 def metric(data):
     """moe.jl:377-383."""
     return 2 * data.num_tokens * data.topk * data.hidden_size * data.intermediate_size * 3, "TFLOPS"
@@ -153,3 +182,24 @@ def smoke(orc):
     got = J(r.out).astype(np.float32)
     assert np.abs(got - ref).max() <= 2e-2 * np.abs(ref).max(), np.abs(got - ref).max()
 
+
+def test_moe(num_tokens: int, hidden_size: int, num_experts: int, intermediate_size: int, topk: int, *,
+             T: torch.dtype = torch.float16, name: str | None = None) -> None:
+    """moe.jl:390-399 (the tile constants are those of ``prepare``)."""
+    name = name or (f"moe tokens={num_tokens}, hidden={hidden_size}, experts={num_experts}, inter={intermediate_size}, "
+                    f"topk={topk}, {str(T).replace('torch.', '')}")
+    print(f"--- {name} ---")
+    data = prepare(num_tokens=num_tokens, hidden_size=hidden_size, num_experts=num_experts,
+                   intermediate_size=intermediate_size, topk=topk, T=T)
+    result = run(data)
+    verify(data, result)
+    print("  passed")
+
+
+def main() -> None:
+    """moe.jl:402-411."""
+    print("--- Mixture of Experts Examples ---\n")
+    test_moe(48, 512, 64, 1024, 8)
+    test_moe(128, 512, 32, 1024, 4)
+    test_moe(64, 1024, 64, 2048, 8)
+    print("\n--- All MoE examples completed ---")

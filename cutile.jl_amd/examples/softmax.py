@@ -69,7 +69,42 @@ def run_others(data, *, nruns: int = 1, warmup: int = 0):
             "torch.softmax": time_launches(lambda: torch.softmax(x, dim=1), nruns, warmup)}
 
 
+
+def verify(data, result) -> None:
+    """softmax.jl:175-188: every column of both outputs against exp(x - max) / sum on the host, per column
+    ``atol = 1e-5, rtol = 1e-4`` in the norm (a Julia column is a torch row)."""
+    x = data.input.cpu()
+    e = torch.exp(x - x.amax(dim=1, keepdim=True))
+    expected = (e / e.sum(dim=1, keepdim=True)).double()
+    for label in ("output_tma", "output_chunked"):
+        out = getattr(result, label).cpu().double()
+        err = torch.linalg.vector_norm(out - expected, dim=1)
+        bound = torch.clamp(1e-4 * torch.maximum(torch.linalg.vector_norm(out, dim=1), torch.linalg.vector_norm(expected, dim=1)), min=1e-5)
+        bad = torch.nonzero(err > bound)
+        assert bad.numel() == 0, f"{label} column {int(bad[0]) + 1} mismatch"
+
+
 def metric(data):
     """softmax.jl:190-198."""
     MN = data.M * data.N * 4
     return {"cuTile TMA": (2 * MN, "GB/s"), "cuTile Chunked": (4 * MN, "GB/s")}
+
+
+def test_softmax(M: int, N: int, *, tile_tma: int | None = None, tile_chunked: int = 1024, name: str | None = None) -> None:
+    """softmax.jl:238-245."""
+    tile_tma = next_power_of_2(N) if tile_tma is None else tile_tma
+    name = name or f"softmax ({M} x {N}), tma_tile={tile_tma}, chunked_tile={tile_chunked}"
+    print(f"--- {name} ---")
+    data = prepare(M=M, N=N)
+    result = run(data, tile_tma=tile_tma, tile_chunked=tile_chunked)
+    verify(data, result)
+    print("  tma passed, chunked passed")
+
+
+def main() -> None:
+    """softmax.jl:247-256."""
+    print("--- Softmax Examples ---\n")
+    test_softmax(256, 256)
+    test_softmax(1024, 1024)
+    test_softmax(4096, 4096)
+    print("\n--- All softmax examples completed ---")

@@ -5,7 +5,7 @@ import numpy as np
 import torch
 
 import cutile_jl_amd as ct
-from ._harness import namespace, rand_uniform, time_launches
+from ._harness import isapprox, namespace, rand_uniform, time_launches
 
 
 def prepare(*, benchmark: bool = False, m: int | None = None, n: int | None = None,
@@ -33,6 +33,33 @@ def run_others(data, *, nruns: int = 1, warmup: int = 0):
     return {"torch copy_(x.t())": time_launches(lambda: y.copy_(data.x.t()), nruns, warmup)}
 
 
+
+def verify(data, result) -> None:
+    """transpose.jl:58-60: ``Array(y) ~ transpose(Array(x))``.  The Julia (m, n) array x is the torch (n, m)
+    tensor, so torch sees the same relation: y == x.t()."""
+    assert isapprox(result.y.cpu(), data.x.cpu().t().contiguous())
+
+
 def metric(data):
     """transpose.jl:62-66: 1 read + 1 write."""
     return 2 * data.m * data.n * data.x.element_size(), "GB/s"
+
+
+def test_transpose(T: torch.dtype, m: int, n: int, tm: int, tn: int, *, name: str | None = None) -> None:
+    """transpose.jl:129-136."""
+    name = name or f"transpose ({m} x {n}, {str(T).replace('torch.', '')}, tiles={tm} x {tn})"
+    print(f"--- {name} ---")
+    data = prepare(m=m, n=n, T=T)
+    result = run(data, tm=tm, tn=tn)
+    verify(data, result)
+    print("  passed")
+
+
+def main() -> None:
+    """transpose.jl:138-147."""
+    print("--- Matrix Transposition Examples ---\n")
+    test_transpose(torch.float32, 256, 256, 32, 32)
+    test_transpose(torch.float32, 512, 512, 64, 64)
+    test_transpose(torch.float32, 256, 512, 32, 64)
+    test_transpose(torch.float32, 1024, 1024, 64, 64)
+    print("\n--- All transpose examples completed ---")

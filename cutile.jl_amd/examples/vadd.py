@@ -5,7 +5,7 @@ import numpy as np
 import torch
 
 import cutile_jl_amd as ct
-from ._harness import namespace, rand_uniform, time_launches
+from ._harness import isapprox, namespace, rand_uniform, time_launches
 
 
 def prepare(*, benchmark: bool = False, shape=None, use_gather: bool = False,
@@ -43,7 +43,46 @@ def run_others(data, *, nruns: int = 1, warmup: int = 0):
     return {"torch.add": time_launches(lambda: torch.add(data.a, data.b, out=c), nruns, warmup)}
 
 
+
+def verify(data, result) -> None:
+    """vadd.jl:127-129: ``Array(c) ~ Array(a) + Array(b)`` on the host."""
+    assert isapprox(result.c.cpu(), data.a.cpu() + data.b.cpu())
+
+
 def metric(data):
     """vadd.jl:131-136: 2 reads + 1 write."""
     n = int(np.prod(data.shape))
     return 3 * n * data.a.element_size(), "GB/s"
+
+
+def test_vadd(shape, tile, *, use_gather: bool = False, T: torch.dtype = torch.float32, name: str | None = None) -> None:
+    """vadd.jl:202-217."""
+    tname = str(T).replace("torch.", "")
+    if name is None:
+        if len(shape) == 2:
+            name = f"2D vec_add ({shape[0]} x {shape[1]}, {tname}, tile={tile})"
+        elif use_gather:
+            name = f"1D vec_add gather ({shape[0]} elements, {tname}, tile={tile})"
+        else:
+            name = f"1D vec_add ({shape[0]} elements, {tname}, tile={tile})"
+    print(f"--- {name} ---")
+    data = prepare(shape=shape, use_gather=use_gather, T=T)
+    result = run(data, tile=tile)
+    verify(data, result)
+    print("  passed")
+
+
+def main() -> None:
+    """vadd.jl:219-248: the example's own list of shapes."""
+    print("--- Vector/Matrix Addition Examples ---\n")
+    test_vadd((1_024_000,), 1024)
+    test_vadd((2 ** 20,), 512)
+    test_vadd((2 ** 18,), 512, T=torch.float64)
+    test_vadd((1_024_000,), 1024, T=torch.float16)
+    test_vadd((2048, 1024), (32, 32))
+    test_vadd((1024, 2048), (64, 64))
+    test_vadd((1024, 512), (32, 32), T=torch.float64)
+    test_vadd((1024, 1024), (64, 64), T=torch.float16)
+    test_vadd((1_024_000,), 1024, use_gather=True)
+    test_vadd((2 ** 20,), 512, use_gather=True)
+    print("\n--- All addition examples completed ---")

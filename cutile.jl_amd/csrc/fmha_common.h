@@ -51,6 +51,15 @@ template <> struct Pack<F16> {
         f16x2 v = {(_Float16)a, (_Float16)b};
         return __builtin_bit_cast(unsigned, v);
     }
+    // acc + the eight weights of a 16-key chunk (four packed pairs), as rounded: the pairs are added up in f16
+    // (three packed adds; the weights are at most 2^8, a sum of four stays far below the f16 range, and its
+    // rounding is a quarter of an ulp of the largest weight), the two halves of the result go into the fp32 sum.
+    static constexpr bool kChunkSum = true;
+    static __device__ __forceinline__ float sum_chunk(const unsigned (&q)[4], float acc) {
+        const f16x2 t = (__builtin_bit_cast(f16x2, q[0]) + __builtin_bit_cast(f16x2, q[1])) +
+                        (__builtin_bit_cast(f16x2, q[2]) + __builtin_bit_cast(f16x2, q[3]));
+        return sum2(__builtin_bit_cast(unsigned, t), 0.f, 0.f, acc);
+    }
     // acc + the two weights of the packed pair pk, as rounded.  Two mixed-precision fma (f16 source, fp32
     // sum), not a dot2: the dot2 instructions run on the matrix pipe and wait for the MFMA in flight.
     static __device__ __forceinline__ float sum2(unsigned pk, float, float, float acc) {
@@ -67,6 +76,8 @@ template <> struct Pack<BF16> {
     }
     // acc + the two weights p0, p1 before rounding (there is no mixed-precision fma for bf16, and widening
     // the rounded pair would take two more instructions; dot2 is avoided for the reason above).
+    static constexpr bool kChunkSum = false;
+    static __device__ __forceinline__ float sum_chunk(const unsigned (&)[4], float acc) { return acc; }
     static __device__ __forceinline__ float sum2(unsigned, float p0, float p1, float acc) {
         return (acc + p0) + p1;
     }

@@ -196,7 +196,7 @@ __device__ __forceinline__ void row_max_stage(f32x16& s, int lim, float& mx, flo
 // The weights of one score pair (2h, 2h+1), h = 0..7, are made in two stages that the step below
 // places in consecutive issue slots, so that no instruction waits for the one just before it:
 // stage 1: 2 exp2 of scores that the MFMAs delivered relative to the (possibly stale) running maximum;
-// stage 2: round and pack for the P.V MFMAs, add to the row sum.
+// stage 2: round and pack for the P.V MFMAs, add to the row sum (f16: once per 16-key chunk, see Pack<F16>).
 __device__ __forceinline__ void exp_stage1(const f32x16& s, int h, float (&p)[2]) {
     p[0] = __builtin_amdgcn_exp2f(s[2 * h]);
     p[1] = __builtin_amdgcn_exp2f(s[2 * h + 1]);
@@ -204,8 +204,12 @@ __device__ __forceinline__ void exp_stage1(const f32x16& s, int h, float (&p)[2]
 template <typename E>
 __device__ __forceinline__ void exp_stage2(const float (&p)[2], int h, float& l, unsigned (&pf)[2][4]) {
     const unsigned pk = Pack<E>::pack(p[0], p[1]);
-    l = Pack<E>::sum2(pk, p[0], p[1], l);
     pf[h >> 2][h & 3] = pk;
+    if constexpr (Pack<E>::kChunkSum) {
+        if ((h & 3) == 3) l = Pack<E>::sum_chunk(pf[h >> 2], l);   // the chunk is complete
+    } else {
+        l = Pack<E>::sum2(pk, p[0], p[1], l);
+    }
 }
 
 // Closes an issue slot: nothing is scheduled across it.

@@ -386,7 +386,7 @@ __device__ __forceinline__ void half_step(const unsigned short* Ks, const unsign
 // Both halves share the stream's state (m, the accumulators); c0 / c1 are S(j) - m / S(j+1) - m, n0 / n1 receive
 // S(j+2) - m / S(j+3) - m, kf[h] holds the K(j+2+h) fragments on entry and the K(j+4+h) fragments on exit,
 // cand[h] the row maxima of c_h on entry and of n_h on exit.  Row sums: half j adds to l[1], half j+1 to l[0].
-// Ring: a trip waits for everything requested one trip ago (K(j+4), K(j+5), V(j+2), V(j+3)), then requests
+// Ring: a trip waits for everything requested one trip ago (K(j+4), K(j+5), V(j), V(j+1)), then requests
 // K(j+6), K(j+7) into the slots whose fragments are in registers and V(j+2), V(j+3) into the slots read one trip
 // ago (V(j+2) not in the first wide trip: the narrow steps had requested it already).
 template <typename E, bool NEXT, bool MASK>

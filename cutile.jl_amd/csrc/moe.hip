@@ -174,6 +174,12 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(TS == 1 ? 4
     }
     auto tok_of = [&](int ts, int slot) { return __shfl(my_tok[ts], slot, 64); };
     if (!live || expert < 0 || expert >= num_experts) return;
+    // The routed weight of the lane's slot is requested now and handed round by shuffles in the epilogue: loaded
+    // there (sixteen dependent gathers per lane) it added a memory round trip to the end of every workgroup.
+    unsigned short my_w[TS];
+#pragma unroll
+    for (int ts = 0; ts < TS; ++ts) my_w[ts] = (mul_routed_weight && my_tok[ts]) ? topk_weights[my_tok[ts] - 1] : (unsigned short)0;
+    auto weight_of = [&](int ts, int slot) { return E::widen((unsigned short)__shfl((int)my_w[ts], slot, 64)); };
 
     const unsigned char* B8 = (const unsigned char*)Bv + (int64_t)expert * sbe;
     const unsigned short* B16 = (const unsigned short*)Bv + (int64_t)expert * sbe;
@@ -196,20 +202,6 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(TS == 1 ? 4
     u32x4 breg0[NB];
     s16x8 areg0[NA];
     int a_col[NA];
-#pragma unroll
-    for (int i = 0; i < NA; ++i) {
-        a_col[i] = -1;
-        const int sl = (tid + 256 * i) / CPR;
-        int tok = tok_of(0, sl & 31);
-        if constexpr (TS == 2) {
-            const int tok1 = tok_of(1, sl & 31);
-            if (sl >= kTT) tok = tok1;
-        }
-        if (tok) {
-            const int col = (tok + replicas - 1) / replicas - 1;  // cld(token_id, replicas), 0-based
-            if (col < num_a_cols) a_col[i] = col;
-        }
-    }
     // Workgroups whose whole tile is inside the arrays (the usual case) load without predicates: a
     // predicated load is waited for before the other side of its branch may write the same
     // registers, which would leave a lane with one load in flight at a time.  Slots without a token
@@ -284,7 +276,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(TS == 1 ? 4
     // at the same moment, i.e. the same slice of every 4 KB of address space.
     const int nsteps = (K + kKT - 1) / kKT;
     // (the narrow shape only: 27.9 against 29.5 us there, 49 against 45 us on the wide shape)
-    const int rot = NTW == 1 ? (int)((unsigned)(3 * expert + grp) % (unsigned)nsteps) : 0;   // (not a function of the strip: the fused-SiLU and the plain kernel then add in the same order)
+    const unsigned rot_seed = (unsigned)(3 * expert + grp);
+    const int rot = NTW != 1 ? 0 : (nsteps & (nsteps - 1)) == 0 ? (int)(rot_seed & (unsigned)(nsteps - 1)) : (int)(rot_seed % (unsigned)nsteps);   // (not a function of the strip: the fused-SiLU and the plain kernel then add in the same order)
     auto k_of = [&](int it) {
         int st = it + rot;
         if (st >= nsteps) st -= nsteps;
@@ -343,8 +336,27 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(TS == 1 ? 4
             }
         }
     };
-    load_a(k_of(0), areg0);
+    // The first weight tile only needs the expert and the strip: request it before the columns of the activation
+    // tile are worked out from the token ids.
     load_b(k_of(0), breg0);
+    const bool rep_pow2 = (replicas & (replicas - 1)) == 0;
+    const int rep_shift = __builtin_ctz((unsigned)replicas);
+#pragma unroll
+    for (int i = 0; i < NA; ++i) {
+        a_col[i] = -1;
+        const int sl = (tid + 256 * i) / CPR;
+        int tok = tok_of(0, sl & 31);
+        if constexpr (TS == 2) {
+            const int tok1 = tok_of(1, sl & 31);
+            if (sl >= kTT) tok = tok1;
+        }
+        if (tok) {
+            // cld(token_id, replicas), 0-based (a shift for the usual power of two)
+            const int col = rep_pow2 ? ((tok + replicas - 1) >> rep_shift) - 1 : (tok + replicas - 1) / replicas - 1;
+            if (col < num_a_cols) a_col[i] = col;
+        }
+    }
+    load_a(k_of(0), areg0);
     using Y = std::true_type;
     using No = std::false_type;
     {
@@ -378,8 +390,12 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(TS == 1 ? 4
     for (int ts = 0; ts < TS; ++ts) {
         if (!((live >> ts) & 1u)) continue;   // same decision in every wave
         int toks[16];   // gathered with every lane of the wave active
+        float wts[16];
 #pragma unroll
-        for (int r = 0; r < 16; ++r) toks[r] = tok_of(ts, 8 * (r >> 2) + 4 * hb + (r & 3));
+        for (int r = 0; r < 16; ++r) {
+            toks[r] = tok_of(ts, 8 * (r >> 2) + 4 * hb + (r & 3));
+            wts[r] = mul_routed_weight ? weight_of(ts, 8 * (r >> 2) + 4 * hb + (r & 3)) : 1.f;
+        }
         if constexpr (SILU) {
             const int nt = wn * 32 + (lane & 31);               // tile row of this lane's channel
             const bool ok = row_ok(nt);
@@ -390,7 +406,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(TS == 1 ? 4
             for (int r = 0; r < 16; ++r) {
                 float v = acc[ts][r];
                 if (W8) v *= ch_scale;
-                if (mul_routed_weight && toks[r]) v *= E::widen(topk_weights[toks[r] - 1]);
+                if (mul_routed_weight && toks[r]) v *= wts[r];
                 acc[ts][r] = E::widen(E::cvt(v));
             }
             __syncthreads();   // every wave is done with the operand tiles (and with the previous tile's exchange)
@@ -421,7 +437,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(TS == 1 ? 4
                     if (!tok) continue;
                     float v = acc[ts][r];
                     if (W8) v *= ch_scale;
-                    if (mul_routed_weight) v *= E::widen(topk_weights[tok - 1]);
+                    if (mul_routed_weight) v *= wts[r];
                     C[gn + (int64_t)(tok - 1) * ldc] = E::cvt(v);
                 }
             }

@@ -348,16 +348,19 @@ __device__ __forceinline__ void half_step(const unsigned short* Ks, const unsign
         }
     };
     // A: one MFMA and one exp piece per slot.  First the S MFMAs, then the P.V MFMAs of a chunk as soon as that
-    // chunk's weights exist.  Slots 0..3 also read one V fragment each (the first P.V MFMA is in slot 5 at the
-    // earliest), slots 4..7 request one transfer each, and from slot kMaxStart on a slot takes a stage of the maxima.
+    // chunk's weights exist.  Slots 0..3 also request one transfer and read one V fragment each (the first P.V MFMA
+    // is in slot 5 at the earliest; the transfers are waited for three steps from now, the earlier they leave the
+    // better), and from slot kMaxStart on a slot takes a stage of the maxima.
 #pragma unroll
     for (int sl = 0; sl < 8 * nC; ++sl) {
         if (qi < nQ) mfma_q();
         else if (p0 < nP && xi > 4 * ((p0 / 2) + 1)) mfma_p(0, p0++);
         else if (p1 < nP && xi > 4 * nC + 4 * (p1 / 2 + 1)) mfma_p(1, p1++);
         after_q();
-        if (sl < 4) vread(sl);
-        else if (sl < 8) dma(sl - 4);
+        if (sl < 4) {
+            dma(sl);
+            vread(sl);
+        }
         if (sl >= kMaxStart && mi < nStages) max_stage();
         piece();
         slot_end();
@@ -487,23 +490,20 @@ __device__ __forceinline__ void wide_step(const unsigned short* Ks, const unsign
         ++mi;
     };
     const bool more_k = j + 4 < c.nh;   // (the last trips have no K(j+4), K(j+5) to fetch)
-    // Slots 0..3: two V fragments each (the first P.V MFMA is in slot 5 at the earliest); slots 4..8 and 11..13: one
-    // transfer each; slots 9, 10: the K(j+4) / K(j+5) fragments, each right after the last S MFMA that read the old
+    // Slots 0..7: one transfer each (they are waited for at the head of the next trip: the earlier they leave the
+    // better); slots 0..3: two V fragments each (the first P.V MFMA is in slot 5 at the earliest); slots 9, 10: the K(j+4) / K(j+5) fragments, each right after the last S MFMA that read the old
     // ones; from slot 11 on a stage of the maxima.
 #pragma unroll
     for (int sl = 0; sl < 16; ++sl) {
         if (qi < nQ) mfma_q();
         else if (p0 < nP && xi > 4 * ((p0 / 2) + 1)) mfma_p(0, p0++);
         else if (p1 < nP && xi > 8 + 4 * (p1 / 2 + 1)) mfma_p(1, p1++);
+        if (sl < 8) dma(sl);
         if (sl < 4) {
             vread(2 * sl);
             vread(2 * sl + 1);
-        } else if (sl < 9) {
-            dma(sl - 4);
-        } else if (sl < 11) {
+        } else if (sl >= 9 && sl < 11) {
             if (NEXT && more_k) read_k_frags(Ks, c, (j + 4 + (sl - 9)) & 3, kf[sl - 9]);
-        } else if (sl < 14) {
-            dma(sl - 6);
         }
         if (sl >= 11 && mi < nStages) max_stage();
         piece();

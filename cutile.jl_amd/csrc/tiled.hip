@@ -666,7 +666,10 @@ int plan_pass(const MrShape& sh, int src_dt, int acc_dt, const void* src, const 
     int64_t srcn = 1, nred = 1, nkept = 1;            // products over dimensions 1..3 by role
     for (int d = 0; d < 4; ++d) srcn *= sh.size[d];
     for (int d = 1; d < 4; ++d) (sh.red(d) ? nred : nkept) *= sh.size[d];
-    for (int d = 0; d < 4; ++d) if (sh.size[d] > 0x7fffffffLL) return MI_E_GRID;
+    // Dimensions 1..3 are unpacked with 32-bit divisions in the kernels.  Dimension 0 is walked in 64 bits; what
+    // limits it is the number of vectors (below 2^32 where it is reduced, checked below) or of workgroups.
+    for (int d = 1; d < 4; ++d) if (sh.size[d] > 0x7fffffffLL) return MI_E_GRID;
+    if (nvec0 >= (1ll << 32)) return MI_E_GRID;
     pl->nt = stream_hint(srcn * es);
     pl->UNR = knob_unroll();
     pl->vecd = false;
@@ -738,7 +741,9 @@ int canonical_shape(const mi_tile_array* dest, const mi_tile_array* src, MrShape
         if (s == 1) continue;
         const bool r = ds == 1;
         const int64_t st = stride_of(src, d), dt = r ? 0 : stride_of(dest, d);
-        if (n > 0 && red[n - 1] == r && st == out->sst[n - 1] * out->size[n - 1] && (r || dt == out->dstr[n - 1] * out->size[n - 1])) {
+        // (a fused dimension other than 0 has to stay within 31 bits: the kernels unpack it with 32-bit divisions)
+        if (n > 0 && red[n - 1] == r && st == out->sst[n - 1] * out->size[n - 1] && (r || dt == out->dstr[n - 1] * out->size[n - 1]) &&
+            (n == 1 || out->size[n - 1] * s <= 0x7fffffffLL)) {
             out->size[n - 1] *= s;
             continue;
         }

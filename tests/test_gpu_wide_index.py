@@ -155,3 +155,49 @@ def test_matmul_operand_beyond_2_31_elements(ct):
     for k0 in range(0, K, 8194):                       # in slabs of K: the fp32 copy of A stays small
         ref += B[:, k0:k0 + 8194].float() @ A[k0:k0 + 8194].float()
     assert torch.equal(C, ref)
+
+
+def test_fmha_beyond_2_31_elements(ct, orc):
+    """Q, K, V, Out of 130 x 128 heads x 2048 x 64 Float16 (2^31 + 2^25 elements each), causal.  Checked against
+    the oracle's float64 ref_fmha (examples/fmha.jl:175-220) on the first (batch, head) pair, the pair that starts
+    at element 2^31 and the last one, with the bounds of the attention parity tests."""
+    from cutile_jl_amd.examples import fmha
+    B, H, S, D = 130, 128, 2048, 64
+    assert B * H * S * D > WIDE
+    Q, K, V = (_randn((B, H, S, D), torch.float16, 20 + i) for i in range(3))
+    out = fmha.cutile_fmha(Q, K, V, causal=True)
+    assert ct.last_variant().startswith("fmha_pipe")
+    for b, h in [(0, 0), (WIDE // (H * S * D), 0), (B - 1, H - 1)]:
+        q, k, v = (orc.to_julia(t[b:b + 1, h:h + 1].contiguous()) for t in (Q, K, V))
+        ref = orc.ref_fmha(q, k, v, causal=True, dtype=np.float64)
+        got = orc.to_julia(out[b:b + 1, h:h + 1].contiguous()).astype(np.float64)
+        err = np.abs(got - ref)
+        bound = 2e-2 * (np.abs(ref) + np.abs(ref).max())
+        assert np.all(err <= bound), f"pair ({b}, {h}): max err {err.max():.3e}, worst ratio {np.max(err / bound):.3f}"
+        assert orc.isapprox(got, ref, rtol=1e-2, atol=1e-3)
+
+
+def test_moe_weights_beyond_2_31_elements(ct, orc):
+    """66 experts of 4096 x 8192: w1 has 2^32 + 2^27 elements, w2 2^31 + 2^26, and expert 65 of w2 starts at
+    element 2^31 exactly.  Every token is routed to the last two experts, so the result depends only on weights
+    past that offset; the oracle's float64 ref_moe (examples/moe.jl:264-304) is evaluated on those two experts
+    alone, with the bounds of the MoE parity tests."""
+    from cutile_jl_amd.examples import moe
+    E, H, I, tokens, topk = 66, 4096, 8192, 48, 2
+    assert E * H * I > WIDE and (E - 2) * H * I == WIDE
+    g = torch.Generator(device="cuda").manual_seed(30)
+    w1 = torch.randn((E, 2 * I, H), generator=g, device="cuda", dtype=torch.float16) * 0.02
+    w2 = torch.randn((E, H, I), generator=g, device="cuda", dtype=torch.float16) * 0.02
+    hs = torch.randn((tokens, H), generator=g, device="cuda", dtype=torch.float16)
+    tw = torch.rand((topk, tokens), generator=g, device="cuda", dtype=torch.float32).to(torch.float16)
+    ids = torch.empty((topk, tokens), dtype=torch.int64, device="cuda")
+    ids[0] = E - 1 + (torch.arange(tokens, device="cuda") % 2)        # 1-based: experts 65 and 66, alternating
+    ids[1] = E - (torch.arange(tokens, device="cuda") % 2)
+    out = moe.cutile_moe(hs, w1, w2, tw, ids, 128, 128, 64)
+    J = orc.to_julia
+    ref = orc.ref_moe(J(hs), J(w1[E - 2:].contiguous()), J(w2[E - 2:].contiguous()), J(tw), J(ids - (E - 2)), dtype=np.float64)
+    got = J(out).astype(np.float64)
+    err = np.abs(got - ref)
+    bound = 2e-2 * (np.abs(ref) + np.abs(ref).max())
+    assert np.all(err <= bound), f"max err {err.max():.3e}, worst ratio {np.max(err / bound):.3f}"
+    assert orc.isapprox(got, ref, rtol=1e-2, atol=1e-2)

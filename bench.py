@@ -395,7 +395,7 @@ def bench_kernels(ct, which, cpu, nruns=NRUNS, warmup=WARMUP):
         al = (tok.cuda(), exp.cuda())
 
         def graph_of(fn):
-            """Replayable HIP graph of the device work (zero-fills are fill kernels, no memset nodes)."""
+            """Replayable HIP graph of the device work."""
             s = torch.cuda.Stream()
             s.wait_stream(torch.cuda.current_stream())
             with torch.cuda.stream(s):
@@ -429,7 +429,7 @@ def bench_kernels(ct, which, cpu, nruns=NRUNS, warmup=WARMUP):
             g, gout = graph_of(dev)
             g.replay(); torch.cuda.synchronize()
             assert torch.equal(gout, ref_out), "graph replay differs from eager"
-            res["moe_f16_device"] = extra(_entry("MoE f16 top-2, whole cutile_moe on the device (zero-fill + token sort + 4 kernels), HIP graph replay",
+            res["moe_f16_device"] = extra(_entry("MoE f16 top-2, whole cutile_moe on the device (token sort + 4 kernels), HIP graph replay",
                                                  g.replay, wbytes, "GB/s", "hbm", HBM_PEAK_GBS, "f16", nruns, warmup))
         except Exception as ex:  # graph capture unavailable: fall back to eager launches
             res["moe_f16_device"] = extra(_entry(f"MoE f16 top-2, device work only (eager; graph failed: {type(ex).__name__})",

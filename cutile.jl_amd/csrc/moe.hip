@@ -130,7 +130,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(TS == 1 ? 4
     const unsigned short* __restrict__ topk_weights, const int* __restrict__ sorted_token_ids, int num_slots,
     const int* __restrict__ sorted_expert_ids, const float* __restrict__ b_scale, int64_t ld_scale, int K, int N,
     int num_experts, int replicas, bool mul_routed_weight, int TILE_M, int tile_slots, int n_blocks, bool vecA,
-    bool vecB) {
+    bool vecB, int w_topk, int64_t w_s0, int64_t w_s1) {
     constexpr int kNT = 32 * NTW, KW = 4 / NTW;
     // B tile [n][k], 16-byte chunks XOR-swizzled.  E4M3 weights stay raw bytes here (half the LDS
     // traffic and footprint) and are widened after the fragment read; see b_offset8 below.
@@ -178,7 +178,12 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(TS == 1 ? 4
     // there (sixteen dependent gathers per lane) it added a memory round trip to the end of every workgroup.
     unsigned short my_w[TS];
 #pragma unroll
-    for (int ts = 0; ts < TS; ++ts) my_w[ts] = (mul_routed_weight && my_tok[ts]) ? topk_weights[my_tok[ts] - 1] : (unsigned short)0;
+    for (int ts = 0; ts < TS; ++ts) {
+        // weight of replica t0 = token * w_topk + slot: element (token, slot) of the (num_tokens, topk) matrix
+        // (the flattened, slot-fastest vector of moe.jl:193 is the case w_topk = 1)
+        const int t0 = my_tok[ts] - 1, tk = t0 / w_topk;
+        my_w[ts] = (mul_routed_weight && my_tok[ts]) ? topk_weights[tk * w_s0 + (t0 - tk * w_topk) * w_s1] : (unsigned short)0;
+    }
     auto weight_of = [&](int ts, int slot) { return E::widen((unsigned short)__shfl((int)my_w[ts], slot, 64)); };
 
     const unsigned char* B8 = (const unsigned char*)Bv + (int64_t)expert * sbe;
@@ -497,7 +502,9 @@ static int fused_moe_impl(const mi_tile_array* A, const mi_tile_array* B, const 
     MI_CHECK(check_array(A, 2));
     MI_CHECK(check_array(B, 3));
     MI_CHECK(check_array(C, 2));
-    MI_CHECK(check_array(topk_weights, 1));
+    if (!topk_weights) return MI_E_NULL;
+    if (topk_weights->ndim != 1 && topk_weights->ndim != 2) return MI_E_RANK;
+    MI_CHECK(check_array(topk_weights, topk_weights->ndim));
     MI_CHECK(check_array(sorted_token_ids, 1));
     MI_CHECK(check_array(sorted_expert_ids, 1));
     if (!is16(A->dtype) || C->dtype != A->dtype || topk_weights->dtype != A->dtype) return MI_E_DTYPE;
@@ -513,7 +520,11 @@ static int fused_moe_impl(const mi_tile_array* A, const mi_tile_array* B, const 
     const int64_t slots = sorted_token_ids->sizes[0], total = C->sizes[1];
     const int64_t m_blocks = cld(slots, (int64_t)TILE_M);
     if (sorted_expert_ids->sizes[0] < m_blocks) return MI_E_SHAPE;
-    if (mul_routed_weight && topk_weights->sizes[0] < total) return MI_E_SHAPE;
+    // routed weights: the flattened vector of moe.jl:193, or the (num_tokens, topk) matrix itself with any strides
+    const bool w2d = topk_weights->ndim == 2;
+    const int64_t w_topk = w2d && topk_weights->sizes[1] > 0 ? topk_weights->sizes[1] : 1;
+    if (mul_routed_weight && (w2d ? topk_weights->sizes[0] * topk_weights->sizes[1] != total : topk_weights->sizes[0] < total)) return MI_E_SHAPE;
+    if (w_topk > 0x7fffffff) return MI_E_SHAPE;
     if (w8) {
         MI_CHECK(check_array(b_scale, 2));
         if (b_scale->dtype != MI_F32) return MI_E_DTYPE;
@@ -523,7 +534,7 @@ static int fused_moe_impl(const mi_tile_array* A, const mi_tile_array* B, const 
     if ((K > 1 && (A->strides[0] != 1 || B->strides[0] != 1)) || (N > 1 && C->strides[0] != 1)) return MI_E_STRIDE;
     if (slots > 1 && sorted_token_ids->strides[0] != 1) return MI_E_STRIDE;
     if (m_blocks > 1 && sorted_expert_ids->strides[0] != 1) return MI_E_STRIDE;
-    if (total > 1 && topk_weights->strides[0] != 1) return MI_E_STRIDE;
+    if (!w2d && total > 1 && topk_weights->strides[0] != 1) return MI_E_STRIDE;
     if (K > 0x7fffffff || N > 0x7fffffff || total > 0x7ffffffe || slots > 0x7fffffff) return MI_E_SHAPE;
     if (m_blocks * cld(N, (int64_t)TILE_N) > MI_MAX_GRID_DIM) return MI_E_GRID;
     if (m_blocks == 0 || N == 0) return MI_OK;
@@ -558,7 +569,8 @@ static int fused_moe_impl(const mi_tile_array* A, const mi_tile_array* B, const 
                        (unsigned short*)C->ptr, C->strides[1], (int)total, (const unsigned short*)topk_weights->ptr, \
                        (const int*)sorted_token_ids->ptr, (int)slots, (const int*)sorted_expert_ids->ptr,           \
                        w8 ? (const float*)b_scale->ptr : nullptr, w8 ? b_scale->strides[1] : 0, (int)K, (int)N,     \
-                       (int)E, num_token_replicas, mul_routed_weight != 0, TILE_M, tile_slots, n_blocks, vecA, vecB)
+                       (int)E, num_token_replicas, mul_routed_weight != 0, TILE_M, tile_slots, n_blocks, vecA, vecB,     \
+                       (int)w_topk, w2d ? topk_weights->strides[0] : (int64_t)1, w2d ? topk_weights->strides[1] : (int64_t)0)
 #define LAUNCH_SHAPE(ET, W8)                                  \
     do {                                                      \
         if (silu && ts == 2) LAUNCH(ET, W8, 4, 128, true, 2); \

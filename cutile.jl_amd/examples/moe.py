@@ -10,13 +10,14 @@ from ._harness import isapprox, namespace, rand_normal, time_launches
 
 def invoke_fused_moe_kernel(A, B, C, topk_weights, sorted_token_ids, sorted_expert_ids, *, mul_routed_weight,
                             num_token_replicas, tile_m, tile_n, tile_k, b_scale=None, fuse_silu=False):
-    """moe.jl:186-199.  ``topk_weights`` Julia (num_tokens, topk) = torch (topk, num_tokens);
-    flattened slot-fastest (moe.jl:193).  ``C`` Julia (dim, topk, num_tokens) is flattened to
+    """moe.jl:186-199.  ``topk_weights`` Julia (num_tokens, topk) = torch (topk, num_tokens); the reference
+    flattens it slot-fastest (moe.jl:193).  ``C`` Julia (dim, topk, num_tokens) is flattened to
     (dim, total_tokens) (moe.jl:196)."""
-    topk_weights_flat = topk_weights.t().contiguous().reshape(-1)
     C_flat = C.reshape(C.shape[0] * C.shape[1], C.shape[2]) if C.dim() == 3 else C
     launch = ct.fused_moe_silu_kernel if fuse_silu else ct.fused_moe_kernel
-    launch(A, B, C_flat, topk_weights_flat, sorted_token_ids, sorted_expert_ids, num_token_replicas,
+    # (the library takes the (num_tokens, topk) matrix as it is and looks (token, slot) up in the kernel, which
+    # saves the permuting copy of moe.jl:193 in front of either GEMM; a flattened vector is accepted as well)
+    launch(A, B, C_flat, topk_weights, sorted_token_ids, sorted_expert_ids, num_token_replicas,
            mul_routed_weight, tile_m, tile_n, tile_k, b_scale=b_scale)
 
 
@@ -45,11 +46,14 @@ def cutile_moe(hidden_states, w1, w2, topk_weights, topk_ids, tile_m, tile_n, ti
     topk = topk_ids.shape[0]
     total_tokens = num_tokens * topk
     T, dev = hidden_states.dtype, hidden_states.device
-    # The three zero-initialised caches of moe.jl:228-230 are carved out of one allocation, so
-    # that zeroing them is one fill instead of three.
+    # The three caches of moe.jl:228-230, carved out of one allocation.  The reference zero-fills them; here they
+    # are left as allocated: every column of every cache belongs to one (token, slot) replica, the GEMMs write the
+    # columns of all replicas (only padding slots write nothing, and nothing reads those), so no fill is ever
+    # read.  This holds for expert ids in 1..num_experts, which is what the reference accepts as well
+    # (moe_align_tile_size indexes by them, moe.jl:150-160).
     n1 = 0 if fuse_silu else total_tokens * intermediate_size * 2
     n2, n3 = total_tokens * intermediate_size, total_tokens * hidden_size
-    caches = torch.zeros(n1 + n2 + n3, dtype=T, device=dev)
+    caches = torch.empty(n1 + n2 + n3, dtype=T, device=dev)
     cache1 = None if fuse_silu else caches[:n1].view(num_tokens, topk, intermediate_size * 2)
     cache2 = caches[n1:n1 + n2].view(total_tokens, intermediate_size)
     cache3 = caches[n1 + n2:].view(num_tokens, topk, hidden_size)

@@ -264,7 +264,8 @@ function moe_route_topk(logits, topk_weights, topk_ids; stream::Ptr{Cvoid}=C_NUL
         d[1], d[2], d[3], stream))
 end
 
-# `b_scale` (N, E) Float32 goes with e4m3fn weights only; `nothing` otherwise.
+# `b_scale` (N, E) Float32 goes with e4m3fn weights only; `nothing` otherwise.  `topk_weights` is either the
+# flattened `vec(permutedims(topk_weights))` of moe.jl:193 or the (num_tokens, topk) matrix itself, which saves that copy.
 function fused_moe_kernel(A, B, C, topk_weights, sorted_token_ids, sorted_expert_ids,
                           num_token_replicas::Integer, mul_routed_weight::Bool,
                           TILE_M::Integer, TILE_N::Integer, TILE_K::Integer;

@@ -218,7 +218,9 @@ int mi_moe_align_tile_size_device(const mi_tile_array* topk_ids, int tile_m, int
 int mi_moe_route_topk(const mi_tile_array* logits, const mi_tile_array* topk_weights,
                       const mi_tile_array* topk_ids, void* stream);
 /* fused_moe_kernel (moe.jl:45-105).  A (K,num_tokens), B (K,N,E), C (N,total_tokens),
- * topk_weights (total_tokens,), sorted_token_ids (M_padded,) i32 1-based with sentinel
+ * topk_weights (total_tokens,) -- the slot-fastest flattening `vec(permutedims(topk_weights))` of moe.jl:193 -- or
+ * the (num_tokens, topk) matrix itself with any strides (the kernel then looks element (token, slot) up directly
+ * and the caller saves the permuting copy), sorted_token_ids (M_padded,) i32 1-based with sentinel
  * total_tokens+1, sorted_expert_ids (blocks,) i32 1-based.  A, C, topk_weights f16/bf16.
  * B is f16/bf16, or MI_F8E4M3FN with `b_scale` (N,E) f32 per-output-channel scales
  * (fp8 weights are an extension of this build; b_scale must be NULL otherwise). */

@@ -77,6 +77,20 @@ def test_fused_moe_kernel_alone_with_sentinels(ct, orc):
                 ref[:, f] *= float(w.reshape(-1)[f])
         check(got[:, :total], ref, 2e-2)
         assert np.all(got[:, total:] == 9.0)
+    # The routed weights as the (num_tokens, topk) matrix itself, dense and as a strided view, instead of its
+    # slot-fastest flattening (moe.jl:193): the kernel looks (token, slot) up, the result is the same bit for bit.
+    flat_result = C.clone()
+    w2d = torch.from_numpy(np.ascontiguousarray(w.T)).to(dev)                         # torch (topk, tokens)
+    wide = torch.full((topk + 1, 2 * tokens + 3), float("nan"), dtype=torch.float16, device=dev)
+    wide[:topk, 1:2 * tokens + 1:2] = w2d
+    for wv in (w2d, wide[:topk, 1:2 * tokens + 1:2]):
+        C.fill_(9.0)
+        ct.fused_moe_kernel(orc.from_julia(A).to(dev), orc.from_julia(B).to(dev), C[:total], wv,
+                            torch.from_numpy(tok).to(dev), torch.from_numpy(exp).to(dev), topk, True, tile_m, 128, 64)
+        assert torch.equal(C, flat_result)
+    with pytest.raises(ct.MiError):                                                  # a matrix of the wrong extent
+        ct.fused_moe_kernel(orc.from_julia(A).to(dev), orc.from_julia(B).to(dev), C[:total], w2d[:, :tokens - 1],
+                            torch.from_numpy(tok).to(dev), torch.from_numpy(exp).to(dev), topk, True, tile_m, 128, 64)
 
 
 def test_silu_and_mul_and_topk_sum(ct, orc):

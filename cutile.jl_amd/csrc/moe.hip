@@ -491,6 +491,41 @@ __global__ __launch_bounds__(256) void moe_sum_topk_kernel(const unsigned short*
     }
 }
 
+// The same with eight channels per lane (16-byte loads and stores) and every slot's load issued before the first
+// add; a lane walks (token, channel group) pairs, so a launch has a few hundred workgroups however the two extents
+// are split.  The slots are added in ascending order in fp32, as above: same bits.
+template <typename E, int TOPK>
+__global__ __launch_bounds__(256) void moe_sum_topk_vec_kernel(const unsigned short* __restrict__ in, int64_t s1,
+                                                               int64_t s2, unsigned short* __restrict__ out,
+                                                               int64_t ldo, int hvec, int topk, int64_t items) {
+    typedef unsigned short u16x8 __attribute__((ext_vector_type(8)));
+    for (int64_t it = (int64_t)blockIdx.x * 256 + threadIdx.x; it < items; it += (int64_t)gridDim.x * 256) {
+        const int64_t tok = it / hvec;
+        const int h = (int)(it - tok * hvec) * 8;
+        const unsigned short* p = in + h + tok * s2;
+        float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+        if (TOPK > 0) {
+            u16x8 v[TOPK > 0 ? TOPK : 1];
+#pragma unroll
+            for (int k = 0; k < TOPK; ++k) v[k] = *reinterpret_cast<const u16x8*>(p + k * s1);
+#pragma unroll
+            for (int k = 0; k < TOPK; ++k)
+#pragma unroll
+                for (int e = 0; e < 8; ++e) acc[e] += E::widen(v[k][e]);
+        } else {
+            for (int k = 0; k < topk; ++k) {
+                const u16x8 v = *reinterpret_cast<const u16x8*>(p + k * s1);
+#pragma unroll
+                for (int e = 0; e < 8; ++e) acc[e] += E::widen(v[e]);
+            }
+        }
+        u16x8 o;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) o[e] = E::cvt(acc[e]);
+        *reinterpret_cast<u16x8*>(out + h + tok * ldo) = o;
+    }
+}
+
 bool is16(int dt) { return dt == MI_F16 || dt == MI_BF16; }
 
 }  // namespace
@@ -870,8 +905,30 @@ extern "C" int mi_moe_sum_topk(const mi_tile_array* in, const mi_tile_array* out
     if (H > 1 && (in->strides[0] != 1 || out->strides[0] != 1)) return MI_E_STRIDE;
     if (H == 0 || T == 0) return MI_OK;
     if (H > 0x7fffffff || topk > 0x7fffffff) return MI_E_UNSUPPORTED;
-    dim3 grid((unsigned)cld(H, (int64_t)256), (unsigned)(T < 65535 ? T : 65535));
     hipStream_t s = (hipStream_t)stream;
+    if (H % 8 == 0 && aligned(in->ptr, 16) && aligned(out->ptr, 16) && in->strides[1] % 8 == 0 && in->strides[2] % 8 == 0 &&
+        out->strides[1] % 8 == 0) {
+        const int64_t items = (H / 8) * T;
+        const int64_t blocks = cld(items, (int64_t)256);
+        dim3 vgrid((unsigned)(blocks < 4096 ? blocks : 4096));
+#define SUMV(ET, K)                                                                                                         \
+    hipLaunchKernelGGL((moe_sum_topk_vec_kernel<ET, K>), vgrid, dim3(256), 0, s, (const unsigned short*)in->ptr, in->strides[1], \
+                       in->strides[2], (unsigned short*)out->ptr, out->strides[1], (int)(H / 8), (int)topk, items)
+#define SUMV_K(ET)                       \
+    do {                                 \
+        if (topk == 2) SUMV(ET, 2);      \
+        else if (topk == 4) SUMV(ET, 4); \
+        else if (topk == 8) SUMV(ET, 8); \
+        else SUMV(ET, 0);                \
+    } while (0)
+        if (in->dtype == MI_F16) SUMV_K(F16);
+        else SUMV_K(BF16);
+#undef SUMV_K
+#undef SUMV
+        set_variant("moe_sum_topk_vec8");
+        return launch_status();
+    }
+    dim3 grid((unsigned)cld(H, (int64_t)256), (unsigned)(T < 65535 ? T : 65535));
     if (in->dtype == MI_F16)
         hipLaunchKernelGGL((moe_sum_topk_kernel<F16>), grid, dim3(256), 0, s, (const unsigned short*)in->ptr,
                            in->strides[1], in->strides[2], (unsigned short*)out->ptr, out->strides[1], (int)H,

@@ -106,6 +106,19 @@ def test_silu_and_mul_and_topk_sum(ct, orc):
     out = torch.empty((19, 130), dtype=torch.float16, device="cuda")
     ct.moe_sum_topk(x, out)
     assert torch.equal(out, x.float().sum(dim=1).to(torch.float16))
+    assert ct.last_variant() == "moe_sum_topk"
+    # channel counts that are multiples of eight take 16-byte loads: the unrolled slot counts, a general one, bf16,
+    # and a view whose token stride is padded
+    for topk, H, T, dt in [(2, 1024, 256, torch.float16), (8, 136, 33, torch.float16), (3, 64, 5, torch.float16),
+                           (4, 256, 70, torch.bfloat16), (1, 8, 1, torch.float16)]:
+        x = torch.from_numpy(rng.standard_normal((T, topk + 1, H)).astype(np.float32)).to(dt).cuda()[:, :topk]
+        out = torch.full((T, H + 8), 7.0, dtype=dt, device="cuda")
+        ct.moe_sum_topk(x, out[:, :H])
+        assert ct.last_variant() == "moe_sum_topk_vec8"
+        ref = torch.zeros((T, H), dtype=torch.float32, device="cuda")
+        for k in range(topk):
+            ref += x[:, k].float()                                  # slots in ascending order, fp32
+        assert torch.equal(out[:, :H], ref.to(dt)) and bool((out[:, H:] == 7.0).all())
 
 
 def test_moe_fp8_weights(orc):

@@ -54,7 +54,7 @@ __device__ __forceinline__ void dma16(unsigned voff, const char* sbase, unsigned
 __device__ __forceinline__ void fence() { asm volatile("" ::: "memory"); }
 
 // s_waitcnt immediates (gfx9 encoding): lgkmcnt(0) with vmcnt(N)
-constexpr int kWaitVm0 = 0x0070, kWaitVm4 = 0x0074, kWaitVm8 = 0x0078;
+constexpr int kWaitVm0 = 0x0070, kWaitVm4 = 0x0074, kWaitVm8 = 0x0078, kWaitVm10 = 0x007a;
 
 template <int IMM>
 __device__ __forceinline__ void wait_and_barrier() {
@@ -600,26 +600,43 @@ __global__ __launch_bounds__(128) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
         }
     }
 
-    // Fill the rings first: the transfers then travel together with the Q loads below instead of after them.
+    // Q first, then the ring fill: every load is counted by hand here (the Q loads are inline assembly like the
+    // transfers), so that the wave can go on as soon as what it needs next has landed -- Q with all twelve transfers
+    // still out, S(0) with ten, the K(1) fragments with eight -- instead of once everything has.
+    int my_q[2];
+    u32x4 qraw[2][4];
+#pragma unroll
+    for (int jj = 0; jj < 2; ++jj) {
+        my_q[jj] = 32 * tq[jj] + (lane & 31);
+#pragma unroll
+        for (int s = 0; s < 4; ++s) {
+            const unsigned short* qp = Q + (int64_t)my_q[jj] * qs.s1 + 16 * s + 8 * hb;
+            asm volatile("global_load_dwordx4 %0, %1, off" : "=v"(qraw[jj][s]) : "v"(qp) : "memory");
+        }
+    }
     issue_k(c, 0);
     issue_k(c, 1);
     issue_k(c, 2);
     issue_v(c, 0);
     issue_k(c, 3);
     issue_v(c, 1);
+    // (the registers are operands of the wait, so nothing that reads them is scheduled above it)
+    asm volatile("s_waitcnt vmcnt(12)"
+                 : "+v"(qraw[0][0]), "+v"(qraw[0][1]), "+v"(qraw[0][2]), "+v"(qraw[0][3]), "+v"(qraw[1][0]), "+v"(qraw[1][1]),
+                   "+v"(qraw[1][2]), "+v"(qraw[1][3])
+                 :
+                 : "memory");
 
     Acc<E> a;
     a.ones = s16x8{0};
     a.ones[0] = hb == 0 ? E::cvt(1.0f) : (short)0;
-    int my_q[2];
 #pragma unroll
     for (int jj = 0; jj < 2; ++jj) {
-        my_q[jj] = 32 * tq[jj] + (lane & 31);
 #pragma unroll
         for (int s = 0; s < 4; ++s) {
             // Q * (qk_scale / ln 2), rounded once to the storage type: the S MFMAs then deliver exp2-domain
             // scores (fmha.jl:41,106-110 scales the fp32 products instead; the difference is one rounding of Q)
-            const s16x8 q = *reinterpret_cast<const s16x8*>(Q + (int64_t)my_q[jj] * qs.s1 + 16 * s + 8 * hb);
+            const s16x8 q = __builtin_bit_cast(s16x8, qraw[jj][s]);
 #pragma unroll
             for (int e = 0; e < 8; ++e) a.qf[jj][s][e] = E::cvt(E::to_f32(q[e]) * scale2);
         }
@@ -632,7 +649,7 @@ __global__ __launch_bounds__(128) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     }
 
     // ---- prologue: compute S(0), fetch the K(1) fragments -----------------------------------------
-    wait_and_barrier<kWaitVm0>();  // the first halves (requested before Q, above) have landed
+    wait_and_barrier<kWaitVm10>();  // K(0) has landed, in every wave's part of the slot
     f32x16 sa[2], sb[2];
     s16x8 kf[4];
     float cand[2];
@@ -641,11 +658,12 @@ __global__ __launch_bounds__(128) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     for (int s = 0; s < 4; ++s)
 #pragma unroll
         for (int jj = 0; jj < 2; ++jj) sa[jj] = E::mfma32(kf[s], a.qf[jj][s], s == 0 ? f32x16{0} : sa[jj]);
+    wait_and_barrier<kWaitVm8>();   // K(1)
     read_k_frags(Ks, c, 1, kf);
 #pragma unroll
     for (int jj = 0; jj < 2; ++jj)  // tile 0 has its diagonal in half 0
         cand[jj] = CAUSAL ? masked_row_max<true>(sa[jj], c.q0[jj] + c.lim0) : masked_row_max<false>(sa[jj], 0);
-    wait_and_barrier<kWaitVm4>();  // every wave has read its K(0) fragments: slot 0 is free
+    wait_and_barrier<kWaitVm8>();  // every wave has read its K(0) fragments: slot 0 is free
     issue_k(c, 0);  // half 4
     issue_v(c, 2);
 

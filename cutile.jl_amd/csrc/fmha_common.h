@@ -24,6 +24,21 @@ struct F16 {
         return __builtin_bit_cast(short, h);
     }
     static __device__ __forceinline__ float to_f32(short v) { return (float)__builtin_bit_cast(_Float16, v); }
+    // cvt(to_f32(q[e]) * s) for the eight elements of q: one mixed-precision fma per element (f16 source, fp32
+    // product, rounded once into the low / high half of the result) instead of widen, multiply, narrow
+    static __device__ __forceinline__ s16x8 scale8(s16x8 q, float s) {
+        typedef unsigned u32x4_ __attribute__((ext_vector_type(4)));
+        const u32x4_ in = __builtin_bit_cast(u32x4_, q);
+        u32x4_ out;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            unsigned d;
+            asm("v_fma_mixlo_f16 %0, %1, %2, 0 op_sel_hi:[1,0,0]" : "=v"(d) : "v"(in[i]), "v"(s));
+            asm("v_fma_mixhi_f16 %0, %1, %2, 0 op_sel:[1,0,0] op_sel_hi:[1,0,0]" : "+v"(d) : "v"(in[i]), "v"(s));
+            out[i] = d;
+        }
+        return __builtin_bit_cast(s16x8, out);
+    }
 };
 struct BF16 {
     static __device__ __forceinline__ f32x16 mfma32(s16x8 a, s16x8 b, f32x16 c) {
@@ -36,6 +51,12 @@ struct BF16 {
         return (short)(u >> 16);
     }
     static __device__ __forceinline__ float to_f32(short v) { return __uint_as_float((unsigned)(unsigned short)v << 16); }
+    static __device__ __forceinline__ s16x8 scale8(s16x8 q, float s) {
+        s16x8 r;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) r[e] = cvt(to_f32(q[e]) * s);
+        return r;
+    }
 };
 
 struct Strides {

@@ -636,9 +636,7 @@ __global__ __launch_bounds__(128) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
         for (int s = 0; s < 4; ++s) {
             // Q * (qk_scale / ln 2), rounded once to the storage type: the S MFMAs then deliver exp2-domain
             // scores (fmha.jl:41,106-110 scales the fp32 products instead; the difference is one rounding of Q)
-            const s16x8 q = __builtin_bit_cast(s16x8, qraw[jj][s]);
-#pragma unroll
-            for (int e = 0; e < 8; ++e) a.qf[jj][s][e] = E::cvt(E::to_f32(q[e]) * scale2);
+            a.qf[jj][s] = E::scale8(__builtin_bit_cast(s16x8, qraw[jj][s]), scale2);
         }
 #pragma unroll
         for (int dt = 0; dt < 2; ++dt) a.o[jj][dt] = f32x16{0};

@@ -256,11 +256,14 @@ __device__ __forceinline__ void half_step(const unsigned short* Ks, const unsign
             const float m_new = E::to_f32(mh);
             const float alpha = __builtin_amdgcn_exp2f(a.m[jj] - m_new);
             const float shift = base - m_new;
-            a.l[jj] *= alpha;
+            // (the first raise of a stream finds l = 0 and O = 0: nothing to rescale)
+            if (!__all(a.thr[jj] == -INFINITY)) {
+                a.l[jj] *= alpha;
 #pragma unroll
-            for (int dt = 0; dt < 2; ++dt)
+                for (int dt = 0; dt < 2; ++dt)
 #pragma unroll
-                for (int r = 0; r < 16; ++r) a.o[jj][dt][r] *= alpha;
+                    for (int r = 0; r < 16; ++r) a.o[jj][dt][r] *= alpha;
+            }
 #pragma unroll
             for (int r = 0; r < 16; ++r) s_cur[jj][r] += shift;
             a.qm[jj][0] = c.hb0 ? (short)(mh ^ (short)0x8000) : (short)0;

@@ -525,11 +525,24 @@ __device__ __forceinline__ void wide_step(const unsigned short* Ks, const unsign
     while (mi < nStages) max_stage();
 }
 
+// Division of a workgroup id by a launch constant: a multiply-high with floor(2^32 / d) + 1, which is exact while
+// x * d < 2^32; the host clears `fast` when the grid is too large for that.  (An integer division is some forty
+// instructions, and three of them stand in front of the first load.)
+struct Magic {
+    unsigned m_nqb, m_h, m_group;
+    int fast;
+    __device__ __forceinline__ int div(int x, int d, unsigned m) const {
+        if (!fast) return x / d;
+        return m ? (int)__umulhi((unsigned)x, m) : x;   // (m = 0 stands for d = 1)
+    }
+    static unsigned of(int d) { return d <= 1 ? 0u : (unsigned)((1ull << 32) / (unsigned)d) + 1u; }
+};
+
 template <typename E, bool CAUSAL>
 __global__ __launch_bounds__(128) __attribute__((amdgpu_waves_per_eu(2, 2))) void fmha_pipe_kernel(
     const unsigned short* __restrict__ Q, Strides qs, const unsigned short* __restrict__ K, Strides ks,
     const unsigned short* __restrict__ V, Strides vs, unsigned short* __restrict__ O, Strides os, int S, int H,
-    int group, float scale2, int nqb, int nbh) {
+    int group, float scale2, int nqb, int nbh, Magic mg) {
     __shared__ __attribute__((aligned(1024))) unsigned short Ks[4 * kSlot];
     __shared__ __attribute__((aligned(1024))) unsigned short Vs[4 * kSlot];
 
@@ -542,14 +555,15 @@ __global__ __launch_bounds__(128) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
         const int L = blockIdx.x;
         if (nbh % 8 == 0) {
             const int idx = L >> 3;
-            bh = (L & 7) + 8 * (idx / nqb);
-            qb = idx % nqb;
+            const int q = mg.div(idx, nqb, mg.m_nqb);
+            bh = (L & 7) + 8 * q;
+            qb = idx - q * nqb;
         } else {
-            bh = L / nqb;
-            qb = L % nqb;
+            bh = mg.div(L, nqb, mg.m_nqb);
+            qb = L - bh * nqb;
         }
     }
-    const int batch = bh / H, head = bh % H, kvh = head / group;
+    const int batch = mg.div(bh, H, mg.m_h), head = bh - batch * H, kvh = mg.div(head, group, mg.m_group);
     Q += (int64_t)head * qs.s2 + (int64_t)batch * qs.s3;
     O += (int64_t)head * os.s2 + (int64_t)batch * os.s3;
 
@@ -663,7 +677,8 @@ __global__ __launch_bounds__(128) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     read_k_frags(Ks, c, 1, kf);
 #pragma unroll
     for (int jj = 0; jj < 2; ++jj)  // tile 0 has its diagonal in half 0
-        cand[jj] = CAUSAL ? masked_row_max<true>(sa[jj], c.q0[jj] + c.lim0) : masked_row_max<false>(sa[jj], 0);
+        // (only a tile that starts inside half 0 has its diagonal there; q0 is wave-uniform)
+        cand[jj] = (CAUSAL && c.q0[jj] < kHK) ? masked_row_max<true>(sa[jj], c.q0[jj] + c.lim0) : masked_row_max<false>(sa[jj], 0);
     wait_and_barrier<kWaitVm8>();  // every wave has read its K(0) fragments: slot 0 is free
     issue_k(c, 0);  // half 4
     issue_v(c, 2);
@@ -763,14 +778,17 @@ void launch_e(const Problem& p, hipStream_t stream) {
     const int S = (int)Q->sizes[1];
     const int nqb = S / 128, nbh = (int)(Q->sizes[2] * Q->sizes[3]);
     dim3 grid((unsigned)(nqb * nbh)), blk(128);
+    Magic mg{Magic::of(nqb), Magic::of(p.H), Magic::of(p.group), 0};
+    const int64_t dmax = nqb > p.H ? nqb : p.H;
+    mg.fast = (int64_t)grid.x * (dmax > p.group ? dmax : p.group) < (1ll << 32) ? 1 : 0;
     if (p.causal)
         hipLaunchKernelGGL((fmha_pipe_kernel<E, true>), grid, blk, 0, stream, (const unsigned short*)Q->ptr, qs,
                            (const unsigned short*)K->ptr, ks, (const unsigned short*)V->ptr, vs, (unsigned short*)O->ptr,
-                           os, S, p.H, p.group, p.scale2, nqb, nbh);
+                           os, S, p.H, p.group, p.scale2, nqb, nbh, mg);
     else
         hipLaunchKernelGGL((fmha_pipe_kernel<E, false>), grid, blk, 0, stream, (const unsigned short*)Q->ptr, qs,
                            (const unsigned short*)K->ptr, ks, (const unsigned short*)V->ptr, vs, (unsigned short*)O->ptr,
-                           os, S, p.H, p.group, p.scale2, nqb, nbh);
+                           os, S, p.H, p.group, p.scale2, nqb, nbh, mg);
 }
 
 }  // namespace

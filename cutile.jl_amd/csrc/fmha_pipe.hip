@@ -54,7 +54,7 @@ __device__ __forceinline__ void dma16(unsigned voff, const char* sbase, unsigned
 __device__ __forceinline__ void fence() { asm volatile("" ::: "memory"); }
 
 // s_waitcnt immediates (gfx9 encoding): lgkmcnt(0) with vmcnt(N)
-constexpr int kWaitVm0 = 0x0070, kWaitVm4 = 0x0074, kWaitVm8 = 0x0078, kWaitVm10 = 0x007a;
+constexpr int kWaitVm0 = 0x0070, kWaitVm4 = 0x0074, kWaitVm8 = 0x0078, kWaitVm2 = 0x0072;
 
 template <int IMM>
 __device__ __forceinline__ void wait_and_barrier() {
@@ -617,9 +617,11 @@ __global__ __launch_bounds__(128) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
         }
     }
 
-    // Q first, then the ring fill: every load is counted by hand here (the Q loads are inline assembly like the
-    // transfers), so that the wave can go on as soon as what it needs next has landed -- Q with all twelve transfers
-    // still out, S(0) with ten, the K(1) fragments with eight -- instead of once everything has.
+    // Q first, then the ring fill, in the order of need and spread over the prologue: all the waves of a CU start
+    // together, and what they request before their first MFMA passes through the CU's one 64-byte-per-cycle path to
+    // the L2 (20 KB per wave would be 2 500 cycles; Q, K(0) and K(1) are 12).  Every load is counted by hand here
+    // (the Q loads are inline assembly like the transfers), so that the wave goes on as soon as what it needs next
+    // has landed.
     int my_q[2];
     u32x4 qraw[2][4];
 #pragma unroll
@@ -633,12 +635,8 @@ __global__ __launch_bounds__(128) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     }
     issue_k(c, 0);
     issue_k(c, 1);
-    issue_k(c, 2);
-    issue_v(c, 0);
-    issue_k(c, 3);
-    issue_v(c, 1);
     // (the registers are operands of the wait, so nothing that reads them is scheduled above it)
-    asm volatile("s_waitcnt vmcnt(12)"
+    asm volatile("s_waitcnt vmcnt(4)"
                  : "+v"(qraw[0][0]), "+v"(qraw[0][1]), "+v"(qraw[0][2]), "+v"(qraw[0][3]), "+v"(qraw[1][0]), "+v"(qraw[1][1]),
                    "+v"(qraw[1][2]), "+v"(qraw[1][3])
                  :
@@ -664,7 +662,7 @@ __global__ __launch_bounds__(128) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     }
 
     // ---- prologue: compute S(0), fetch the K(1) fragments -----------------------------------------
-    wait_and_barrier<kWaitVm10>();  // K(0) has landed, in every wave's part of the slot
+    wait_and_barrier<kWaitVm2>();  // K(0) has landed, in every wave's part of the slot
     f32x16 sa[2], sb[2];
     s16x8 kf[4];
     float cand[2];
@@ -673,8 +671,12 @@ __global__ __launch_bounds__(128) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     for (int s = 0; s < 4; ++s)
 #pragma unroll
         for (int jj = 0; jj < 2; ++jj) sa[jj] = E::mfma32(kf[s], a.qf[jj][s], s == 0 ? f32x16{0} : sa[jj]);
-    wait_and_barrier<kWaitVm8>();   // K(1)
+    issue_k(c, 2);
+    issue_v(c, 0);
+    wait_and_barrier<kWaitVm4>();   // K(1)
     read_k_frags(Ks, c, 1, kf);
+    issue_k(c, 3);
+    issue_v(c, 1);
 #pragma unroll
     for (int jj = 0; jj < 2; ++jj)  // tile 0 has its diagonal in half 0
         // (only a tile that starts inside half 0 has its diagonal there; q0 is wave-uniform)

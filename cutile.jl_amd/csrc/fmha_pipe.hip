@@ -731,8 +731,12 @@ __global__ __launch_bounds__(128) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
         sa[0] = E::mfma32(a.ones, a.qm[1], f32x16{0});
 #pragma unroll
         for (int s = 0; s < 4; ++s) sa[0] = E::mfma32(kf[s], a.qf[1][s], sa[0]);
-        wc[1] = masked_row_max<true>(sa[0], c.q0[1] + c.lim0 - kHK * (j + 1));
-        wait_and_barrier<kWaitVm0>();
+        {
+            const int q_rel = c.q0[1] - kHK * (j + 1);   // first query of the tile relative to the half (wave-uniform)
+            wc[1] = q_rel < kHK ? masked_row_max<true>(sa[0], q_rel + c.lim0) : masked_row_max<false>(sa[0], 0);
+        }
+        // K(j+2) and K(j+3) have landed once only the last narrow step's four transfers (K(j+4), V(j+2)) are out
+        wait_and_barrier<kWaitVm4>();
         read_k_frags(Ks, c, (j + 2) & 3, kw[0]);
         read_k_frags(Ks, c, (j + 3) & 3, kw[1]);
         issue_k(c, (j + 1) & 3);  // half j+5

@@ -720,11 +720,9 @@ __global__ __launch_bounds__(128) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
         STEP(3, 3, 0, j, sa, sb);
         STEP(3, 2, 1, j + 1, sb, sa);  // (stream 1's mask only bites when its diagonal is two halves away)
         j += 2;
-        store_tile(0, a.l[0]);  // stream 0 is complete: its registers and issue slots now serve the long tile
         // ---- wide steps: the long tile over two halves per trip (always an odd number of trips) ------------
         // S(n1) - m is in sa[1] and the K(n1+1) fragments in kf: compute S(n1+1) - m into sa[0], then fetch
         // the fragments of the next two halves and request the one transfer the wide schedule still lacks.
-        a.l[0] = 0.f;
         s16x8 kw[2][4];
         float wc[2];
         wc[0] = cand[1];
@@ -737,9 +735,13 @@ __global__ __launch_bounds__(128) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
         }
         // K(j+2) and K(j+3) have landed once only the last narrow step's four transfers (K(j+4), V(j+2)) are out
         wait_and_barrier<kWaitVm4>();
+        issue_k(c, (j + 1) & 3);  // half j+5
+        // Stream 0 is complete: its registers and issue slots now serve the long tile.  (Stored after the wait above:
+        // stores count as outstanding memory operations like the transfers, and are younger than all of them.)
+        store_tile(0, a.l[0]);
+        a.l[0] = 0.f;
         read_k_frags(Ks, c, (j + 2) & 3, kw[0]);
         read_k_frags(Ks, c, (j + 3) & 3, kw[1]);
-        issue_k(c, (j + 1) & 3);  // half j+5
 #define WIDE(NEXT, MASK, jx, first, s0, s1) wide_step<E, NEXT, MASK>(Ks, Vs, c, a, jx, first, s0[1], s0[0], s1[1], s1[0], kw, wc)
         bool first = true;
         if (j + 2 < nh) {   // three trips or more: an odd number of plain trips, then the one that masks

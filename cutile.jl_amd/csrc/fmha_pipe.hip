@@ -54,7 +54,8 @@ __device__ __forceinline__ void dma16(unsigned voff, const char* sbase, unsigned
 __device__ __forceinline__ void fence() { asm volatile("" ::: "memory"); }
 
 // s_waitcnt immediates (gfx9 encoding): lgkmcnt(0) with vmcnt(N)
-constexpr int kWaitVm0 = 0x0070, kWaitVm4 = 0x0074, kWaitVm8 = 0x0078, kWaitVm2 = 0x0072;
+constexpr int kWaitVm0 = 0x0070, kWaitVm4 = 0x0074, kWaitVm8 = 0x0078, kWaitVm2 = 0x0072, kWaitVm6 = 0x0076,
+              kWaitLgkm = 0xc07f;   // lgkmcnt(0) alone
 
 template <int IMM>
 __device__ __forceinline__ void wait_and_barrier() {
@@ -425,7 +426,12 @@ __device__ __forceinline__ void wide_step(const unsigned short* Ks, const unsign
             a.thr[1] = kRaise;
         }
     }
-    wait_and_barrier<kWaitVm0>();   // everything requested one trip ago has landed, and every wave knows
+    // Everything requested one trip ago has landed, and every wave knows.  The first wide trip follows the switch,
+    // which has just waited for all it reads before slot 9 and has since stored the early tile and requested K(j+5):
+    // it only meets the other wave here (both have read their fragments of the slots about to be refilled) and
+    // waits in slot 9, by when stores and request have long returned, for all but this trip's own six transfers.
+    if (first) wait_and_barrier<kWaitLgkm>();
+    else wait_and_barrier<kWaitVm0>();
     // As in the narrow step, the fixed work of the trip rides in the issue slots.
     s16x8 vf[2][2][2];  // [half][16-key chunk][d tile]
     auto vread = [&](int f) {
@@ -506,6 +512,7 @@ __device__ __forceinline__ void wide_step(const unsigned short* Ks, const unsign
             vread(2 * sl);
             vread(2 * sl + 1);
         } else if (sl >= 9 && sl < 11) {
+            if (sl == 9 && first) wait_and_barrier<kWaitVm6>();
             if (NEXT && more_k) read_k_frags(Ks, c, (j + 4 + (sl - 9)) & 3, kf[sl - 9]);
         }
         if (sl >= 11 && mi < nStages) max_stage();

@@ -668,11 +668,11 @@ extern "C" int mi_fused_moe_silu_kernel(const mi_tile_array* A, const mi_tile_ar
 // flattening of topk_ids, examples/moe.jl:148-150): LDS histogram, scan over the experts,
 // then placement in super-blocks of 1024 consecutive replicas (one per lane).  A replica's slot is
 //     cursor[e] + (replicas of e in earlier waves of the super-block) + (those in earlier lanes),
-// the last term from ballots alone, so ids of one expert ascend exactly as the stable sortperm
+// the last term from ballots alone (one per bit of the expert id), so ids of one expert ascend exactly as the stable sortperm
 // of moe.jl:150 orders them.  The outputs have fixed capacity: unused slots hold the sentinel
 // total+1, unused blocks expert 0, which the GEMM kernel skips.
 constexpr int kAlignMaxExperts = 1024;
-constexpr int kAlignThreads = 1024, kAlignWaves = kAlignThreads / 64;
+constexpr int kAlignThreads = 1024, kAlignWaves = kAlignThreads / 64, kAlignCached = 2;
 __global__ __launch_bounds__(kAlignThreads) void moe_align_kernel(const long long* __restrict__ topk_ids, int64_t ld_slot,
                                                         int num_tokens, int topk, int tile_m, int num_experts,
                                                         int* __restrict__ sorted_token_ids, int cap_slots,
@@ -681,6 +681,16 @@ __global__ __launch_bounds__(kAlignThreads) void moe_align_kernel(const long lon
     __shared__ unsigned short tbl[kAlignWaves][kAlignMaxExperts];   // replicas per (wave, expert) of the current super-block (<= 64)
     __shared__ int s_blocks, wave_total[kAlignWaves];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, total = num_tokens * topk;
+    // The ids of the first kAlignCached super-blocks stay in registers between the counting pass and the placing
+    // pass, and are requested before the tables are cleared: one memory round trip instead of three in a row.
+    auto expert_of = [&](int r) {
+        if (r >= total) return -1;
+        const long long v = topk_ids[(r / topk) + (int64_t)(r % topk) * ld_slot];
+        return (v >= 1 && v <= num_experts) ? (int)v - 1 : -1;
+    };
+    int ecache[kAlignCached];
+#pragma unroll
+    for (int i = 0; i < kAlignCached; ++i) ecache[i] = expert_of(tid + kAlignThreads * i);
     for (int e = tid; e < num_experts; e += kAlignThreads) {
         cursor[e] = 0;
 #pragma unroll
@@ -688,9 +698,12 @@ __global__ __launch_bounds__(kAlignThreads) void moe_align_kernel(const long lon
     }
     for (int i = tid; i < cap_slots; i += kAlignThreads) sorted_token_ids[i] = total + 1;
     __syncthreads();
-    for (int r = tid; r < total; r += kAlignThreads) {
-        const long long e = topk_ids[(r / topk) + (int64_t)(r % topk) * ld_slot];
-        if (e >= 1 && e <= num_experts) atomicAdd(&cursor[(int)e - 1], 1);
+#pragma unroll
+    for (int i = 0; i < kAlignCached; ++i)
+        if (ecache[i] >= 0) atomicAdd(&cursor[ecache[i]], 1);
+    for (int r = tid + kAlignThreads * kAlignCached; r < total; r += kAlignThreads) {
+        const int e = expert_of(r);
+        if (e >= 0) atomicAdd(&cursor[e], 1);
     }
     __syncthreads();
     {   // exclusive scan of the experts' block counts (thread e owns expert e): shuffles inside a
@@ -705,7 +718,8 @@ __global__ __launch_bounds__(kAlignThreads) void moe_align_kernel(const long lon
         if (lane == 63) wave_total[wave] = incl;
         __syncthreads();
         int first = incl - nb;
-        for (int w = 0; w < wave; ++w) first += wave_total[w];
+#pragma unroll
+        for (int w = 0; w < kAlignWaves; ++w) first += w < wave ? wave_total[w] : 0;
         if (tid < num_experts) {
             cursor[tid] = first * tile_m;  // first slot of the expert
             for (int b = first; b < first + nb && b < cap_blocks; ++b) sorted_expert_ids[b] = tid + 1;
@@ -716,37 +730,38 @@ __global__ __launch_bounds__(kAlignThreads) void moe_align_kernel(const long lon
     for (int b = s_blocks + tid; b < cap_blocks; b += kAlignThreads) sorted_expert_ids[b] = 0;
 
     const unsigned long long lt = lane ? (~0ull >> (64 - lane)) : 0ull;
+    const int id_bits = 32 - __builtin_clz((unsigned)(num_experts > 1 ? num_experts - 1 : 1));
     for (int r0 = 0; r0 < total; r0 += kAlignThreads) {
         const int r = r0 + tid;
-        int e = -1;
-        if (r < total) {
-            const long long v = topk_ids[(r / topk) + (int64_t)(r % topk) * ld_slot];
-            if (v >= 1 && v <= num_experts) e = (int)v - 1;
+        int e;
+        {
+            const int sb = r0 / kAlignThreads;   // super-block (uniform): the first ones are in registers
+            if (sb == 0) e = ecache[0];
+            else if (sb == 1 && kAlignCached > 1) e = ecache[kAlignCached > 1 ? 1 : 0];
+            else e = expert_of(r);
         }
-        int rank = 0;
-        unsigned long long todo = __ballot(e >= 0);
-        while (todo) {  // one trip per distinct expert of the wave's 64 replicas
-            const int leader = __ffsll((long long)todo) - 1;
-            const int el = __builtin_amdgcn_readlane(e, leader);  // leader comes from a ballot: wave-uniform
-            const unsigned long long m = __ballot(e == el);
-            if (e == el) rank = __popcll(m & lt);
-            if (lane == leader) tbl[wave][el] = (unsigned short)__popcll(m);
-            todo &= ~m;
+        // the lanes of this wave that hold the same expert: one ballot per bit of the expert id
+        unsigned long long m = __ballot(e >= 0);
+        for (int b = 0; b < id_bits; ++b) {
+            const unsigned long long bal = __ballot((e >> b) & 1);
+            m &= ((e >> b) & 1) ? bal : ~bal;
         }
-        __syncthreads();
+        const int rank = __popcll(m & lt);
+        if (e >= 0 && rank == 0) tbl[wave][e] = (unsigned short)__popcll(m);
+        __syncthreads();   // the table is complete, and the cursors of the previous super-block have been advanced
         if (e >= 0) {
             int pos = cursor[e] + rank;
-            for (int w = 0; w < wave; ++w) pos += tbl[w][e];
+#pragma unroll
+            for (int w = 0; w < kAlignWaves; ++w) pos += w < wave ? (int)tbl[w][e] : 0;   // (all sixteen reads in flight)
             if (pos < cap_slots) sorted_token_ids[pos] = r + 1;
         }
-        __syncthreads();
-        // advance the cursors and clear the table: the entries touched are those of this super-block's experts
+        __syncthreads();   // every lane has read the cursors and the table
+        // Advance the cursors and clear the table.  The entries touched are those of this super-block's experts, and
+        // an entry is written by its own wave only (now, and when the next super-block is counted): no third barrier.
         if (e >= 0 && rank == 0) {  // first lane of its expert within the wave
             atomicAdd(&cursor[e], (int)tbl[wave][e]);
+            tbl[wave][e] = 0;
         }
-        __syncthreads();
-        if (e >= 0 && rank == 0) tbl[wave][e] = 0;
-        __syncthreads();
     }
 }
 

@@ -567,8 +567,9 @@ __global__ __launch_bounds__(128) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
             qb = idx - q * nqb;
             // A pair with a late long tile spends more of its walk in wide steps and takes a few per cent longer.
             // An XCD places consecutive workgroups on its 32 CUs in turn, so ids 32 apart share a CU: every
-            // second round of 32 takes the pairs in reverse order, and each CU gets both kinds.
-            if (CAUSAL && ((idx >> 5) & 1)) qb = nqb - 1 - qb;
+            // second round of 32 takes the pairs in reverse order, and each CU gets both kinds.  (Decided by the
+            // first id of the (batch, head) group, so that a group is reversed as a whole: a permutation of its pairs.)
+            if (CAUSAL && (((q * nqb) >> 5) & 1)) qb = nqb - 1 - qb;
         } else {
             bh = mg.div(L, nqb, mg.m_nqb);
             qb = L - bh * nqb;

@@ -17,6 +17,24 @@ pytestmark = pytest.mark.gpu
 from cutile_jl_amd.examples import fmha  # noqa: E402
 
 
+def attend(Q, K, V, **kw):
+    """cutile_fmha into an output buffer filled with NaN beforehand: an element the kernel never writes fails the check."""
+    out = torch.full((Q.shape[0], Q.shape[1], Q.shape[2], V.shape[3]), float("nan"), dtype=Q.dtype, device=Q.device)
+    ret = fmha.cutile_fmha(Q, K, V, out=out, **kw)
+    assert ret is out
+    return out
+
+
+class _Result:
+    def __init__(self, out):
+        self.out = out
+
+
+def run(data):
+    return _Result(attend(data.Q, data.K, data.V, tile_m=data.tile_m, tile_n=data.tile_n,
+                          query_group_size=data.query_group_size, causal=data.causal))
+
+
 def check(orc, out, ref, tol=2e-2):
     got = orc.to_julia(out).astype(np.float64)
     err = np.abs(got - ref)
@@ -34,11 +52,13 @@ def check(orc, out, ref, tol=2e-2):
     (1, 2, 1, 1, 64, True, 1, torch.float16), (1, 2, 130, 64, 64, False, 1, torch.float16),
     (2, 4, 256, 256, 128, True, 1, torch.float16), (1, 2, 100, 300, 128, False, 2, torch.float16),
     (2, 4, 256, 256, 64, True, 1, torch.bfloat16), (1, 2, 192, 192, 128, False, 1, torch.bfloat16),
+    (16, 8, 384, 384, 64, True, 1, torch.float16), (8, 8, 640, 640, 64, True, 1, torch.float16), (4, 4, 896, 896, 64, True, 2, torch.bfloat16),
+    (8, 8, 384, 384, 64, False, 1, torch.float16), (24, 8, 128, 128, 64, True, 1, torch.float16), (8, 16, 1536, 1536, 64, True, 4, torch.float16),
 ])
 def test_fmha_against_ref(orc, batch, heads, sq, skv, d, causal, qg, T):
     data = fmha.prepare(batch=batch, heads=heads, seq_q=sq, seq_kv=skv, d_k=d, d_v=d, query_group_size=qg,
                         causal=causal, T=T)
-    r = fmha.run(data)
+    r = run(data)
     Q, K, V = (orc.to_julia(t) for t in (data.Q, data.K, data.V))
     if causal and sq != skv:
         pytest.skip("ref_fmha's causal mask assumes aligned positions")
@@ -49,7 +69,7 @@ def test_fmha_against_ref(orc, batch, heads, sq, skv, d, causal, qg, T):
 def test_fmha_reference_input_distribution(orc):
     """The reference's own inputs, U(-0.5, 0.5) (fmha.jl:240-242)."""
     data = fmha.prepare(batch=2, heads=8, seq_q=256, seq_kv=256, dist="uniform")
-    r = fmha.run(data)
+    r = run(data)
     ref = orc.ref_fmha(*(orc.to_julia(t) for t in (data.Q, data.K, data.V)), causal=True, dtype=np.float64)
     check(orc, r.out, ref)
 
@@ -58,19 +78,19 @@ def test_fmha_reference_input_distribution(orc):
 def test_fmha_decode_offset(orc, sq, skv, pos):
     """input_pos shifts the query positions (fmha.jl:45-46,66): query i sees keys <= pos + i."""
     data = fmha.prepare(batch=1, heads=4, seq_q=sq, seq_kv=skv, query_group_size=2)
-    out = fmha.cutile_fmha(data.Q, data.K, data.V, input_pos=pos, causal=True, query_group_size=2)
+    out = attend(data.Q, data.K, data.V, input_pos=pos, causal=True, query_group_size=2)
     ref = orc.fmha_general(*(orc.to_julia(t) for t in (data.Q, data.K, data.V)), causal=True, input_pos=pos)
     check(orc, out, ref)
 
 
 def test_fmha_causal_first_row_and_noncausal_limit(orc):
     data = fmha.prepare(batch=1, heads=2, seq_q=256, seq_kv=256)
-    out = fmha.cutile_fmha(data.Q, data.K, data.V, causal=True)
+    out = attend(data.Q, data.K, data.V, causal=True)
     # query 1 attends to key 1 only: output row equals V[:, 1] exactly (softmax weight 1.0)
     assert torch.equal(out[:, :, 0, :], data.V[:, :, 0, :])
     # with input_pos >= Skv the causal kernel sees every key: equals the non-causal kernel bit for bit
-    a = fmha.cutile_fmha(data.Q, data.K, data.V, causal=True, input_pos=256)
-    b = fmha.cutile_fmha(data.Q, data.K, data.V, causal=False)
+    a = attend(data.Q, data.K, data.V, causal=True, input_pos=256)
+    b = attend(data.Q, data.K, data.V, causal=False)
     assert torch.equal(a, b)
 
 
@@ -80,7 +100,7 @@ def test_fmha_strided_views_and_scale(orc):
     B, S, H, D = 2, 192, 4, 64
     packed = torch.from_numpy(rng.standard_normal((B, S, 3, H, D), dtype=np.float32)).to(torch.float16).cuda()
     Q, K, V = (packed[:, :, i].permute(0, 2, 1, 3) for i in range(3))  # torch (B,H,S,D) views, D contiguous
-    out = fmha.cutile_fmha(Q, K, V, causal=True, qk_scale=0.2)
+    out = attend(Q, K, V, causal=True, qk_scale=0.2)
     ref = orc.ref_fmha(orc.to_julia(Q), orc.to_julia(K), orc.to_julia(V), qk_scale=0.2, causal=True, dtype=np.float64)
     check(orc, out, ref)
 
@@ -96,7 +116,7 @@ def test_fmha_pipelined_kernel_shapes(ct, orc, batch, heads, s, causal, qg, T):
     causal mask a wave walks its long tile two key halves per trip once its early tile is done: 128 keys give
     one such trip, 384 up to five, 2048 up to thirty-one."""
     data = fmha.prepare(batch=batch, heads=heads, seq_q=s, seq_kv=s, query_group_size=qg, causal=causal, T=T)
-    r = fmha.run(data)
+    r = run(data)
     assert ct.last_variant().startswith("fmha_pipe")
     ref = orc.ref_fmha(*(orc.to_julia(t) for t in (data.Q, data.K, data.V)), causal=causal, dtype=np.float64)
     check(orc, r.out, ref, 2e-2 if T == torch.float16 else 3e-2)
@@ -131,7 +151,7 @@ def test_fmha_running_maximum_keeps_rising(ct, orc, causal):
     k = (rng.standard_normal((D, S, H, B)).astype(np.float32) * 0.25 + 1.0) * ramp
     v = rng.standard_normal((D, S, H, B)).astype(np.float32)
     Q, K, V = (orc.from_julia(x).to(torch.float16).cuda() for x in (q, k, v))
-    out = fmha.cutile_fmha(Q, K, V, causal=causal)
+    out = attend(Q, K, V, causal=causal)
     assert ct.last_variant().startswith("fmha_pipe")
     ref = orc.ref_fmha(*(orc.to_julia(t) for t in (Q, K, V)), causal=causal, dtype=np.float64)
     check(orc, out, ref)
@@ -152,7 +172,7 @@ def test_fmha_full_size(orc):
     """Benchmark shape 8x16x1024x64 causal: a sample of (batch, head) pairs against float64 and
     the softmax-weights-sum-to-one property via V = ones."""
     data = fmha.prepare(benchmark=True)
-    r = fmha.run(data)
+    r = run(data)
     Q, K, V = (orc.to_julia(t) for t in (data.Q, data.K, data.V))
     got = orc.to_julia(r.out).astype(np.float64)
     for (h, b) in [(0, 0), (15, 7), (7, 3)]:
@@ -161,7 +181,7 @@ def test_fmha_full_size(orc):
         err = np.abs(got[:, :, h, b] - ref[:, :, 0, 0])
         assert np.all(err <= 2e-2 * (np.abs(ref[:, :, 0, 0]) + np.abs(ref).max()))
     ones = torch.ones_like(data.V)
-    out1 = fmha.cutile_fmha(data.Q, data.K, ones, causal=True)
+    out1 = attend(data.Q, data.K, ones, causal=True)
     assert torch.all((out1.float() - 1).abs() <= 2e-3)
 
 
@@ -169,7 +189,7 @@ def test_fmha_more_than_65535_batch_heads(ct, orc):
     """The reference's grid is (cld(Sq, TILE_M), B * H) with up to 2^24 - 1 blocks per dimension
     (fmha.jl:163-165, src/launch.jl:743): 70 000 (batch, head) pairs of a short sequence."""
     data = fmha.prepare(batch=10, heads=7000, seq_q=16, seq_kv=16, causal=True)
-    r = fmha.run(data)
+    r = run(data)
     Q, K, V = (orc.to_julia(t) for t in (data.Q, data.K, data.V))
     got = orc.to_julia(r.out).astype(np.float64)
     for b, hs in ((0, slice(0, 3)), (9, slice(6997, 7000)), (9, slice(3552, 3555))):    # pairs 0.., 69997.., 66552..

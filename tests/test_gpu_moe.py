@@ -167,7 +167,8 @@ def test_moe_full_size_top2(orc):
 
 
 @pytest.mark.parametrize("num_tokens,topk,E,tile_m", [(256, 2, 32, 128), (48, 8, 64, 16), (7, 3, 5, 4), (1, 1, 1, 128),
-                                                      (1000, 4, 9, 32), (130, 2, 1000, 8)])
+                                                      (1000, 4, 9, 32), (130, 2, 1000, 8),
+                                                      (512, 2, 32, 128), (512, 4, 7, 16), (513, 4, 7, 16), (2049, 1, 33, 64)])
 def test_device_align_matches_host_routine(ct, orc, num_tokens, topk, E, tile_m):
     """The one-workgroup counting sort gives the host routine's arrays (stable per-expert order,
     sentinel padding) in the leading part of its fixed-capacity outputs, and marks the rest unused."""

@@ -75,6 +75,26 @@ def test_fmha_random_shapes(ct):
         assert close(out, ref, 3e-2 if dt == torch.bfloat16 else 2e-2), f"B={B} H={H} S={S} group={qg} causal={causal} {dt} {ct.last_variant()}"
 
 
+def test_fmha_random_ragged_shapes(ct):
+    """Sequence lengths off every tile grid, D = 64 and 128, grouped queries: the general kernels (EVEN_K = false).
+    Causal here is the reference's mask with input_pos = 0 (query i sees keys <= i), which is torch's is_causal."""
+    rnd = random.Random(2)
+    for it in range(40):
+        Sq = rnd.choice([1, 2, 17, 63, 64, 65, 100, 128, 130, 200, 257, 300, 511, 700])
+        Skv = rnd.choice([1, 5, 64, 77, 128, 129, 255, 256, 300, 512, 513, 900])
+        causal = rnd.choice([True, False])
+        if causal and Skv < Sq:
+            Skv = Sq
+        D = rnd.choice([64, 128]); qg = rnd.choice([1, 2, 4]); H = rnd.choice([1, 2, 3]) * qg; B = rnd.choice([1, 2, 5])
+        dt = rnd.choice([torch.float16, torch.bfloat16])
+        d = fmha.prepare(batch=B, heads=H, seq_q=Sq, seq_kv=Skv, d_k=D, d_v=D, query_group_size=qg, causal=causal, T=dt, seed=it)
+        out = torch.full_like(d.Q, NAN)
+        fmha.cutile_fmha(d.Q, d.K, d.V, causal=causal, query_group_size=qg, out=out)
+        K = d.K.repeat_interleave(qg, dim=1).float(); V = d.V.repeat_interleave(qg, dim=1).float()
+        ref = F.scaled_dot_product_attention(d.Q.float(), K, V, is_causal=causal)
+        assert close(out, ref, 3e-2 if dt == torch.bfloat16 else 2e-2), f"B={B} H={H} Sq={Sq} Skv={Skv} D={D} group={qg} causal={causal} {dt} {ct.last_variant()}"
+
+
 def test_row_kernels_random_shapes(ct):
     rnd = random.Random(5)
     ns = [1, 3, 7, 64, 100, 255, 256, 257, 1000, 1024, 1500, 4096, 5000, 8192, 12000, 20000]

@@ -39,6 +39,7 @@ constexpr int kD = 64;            // head dimension
 constexpr int kHK = 32;           // keys per half
 constexpr int kSlot = kHK * kD;   // elements per ring slot
 constexpr int kSlotBytes = kSlot * 2;
+constexpr int kPre = 1;           // issue slots of a step that run before its wait and barrier
 constexpr float kRaise = 8.0f;    // raise m only when the new maximum exceeds it by this much
 
 #pragma clang diagnostic ignored "-Winline-asm"  // m0 is named as clobbered on purpose
@@ -272,7 +273,8 @@ __device__ __forceinline__ void half_step(const unsigned short* Ks, const unsign
             a.thr[jj] = kRaise;
         }
     }
-    wait_and_barrier<kWaitVm8>();
+    // (The wait for the transfers and for the other wave stands kPre slots further down: the first S MFMAs and exp
+    // pieces need registers only, and a wave that arrives early does them while it would otherwise idle.)
     // The rest of a step's fixed work rides in the issue slots below, a few instructions per slot: under two
     // waves per SIMD a slot lasts as long as two MFMAs, and a wave needs less than that for its MFMA and its piece.
     s16x8 vf[2][2];  // V(j) fragments, [16-key chunk][d tile]
@@ -352,7 +354,7 @@ __device__ __forceinline__ void half_step(const unsigned short* Ks, const unsign
         }
     };
     // A: one MFMA and one exp piece per slot.  First the S MFMAs, then the P.V MFMAs of a chunk as soon as that
-    // chunk's weights exist.  Slots 0..3 also request one transfer and read one V fragment each (the first P.V MFMA
+    // chunk's weights exist.  Slots kPre..kPre+3 also request one transfer and read one V fragment each (the first P.V MFMA
     // is in slot 5 at the earliest; the transfers are waited for three steps from now, the earlier they leave the
     // better), and from slot kMaxStart on a slot takes a stage of the maxima.
 #pragma unroll
@@ -361,9 +363,10 @@ __device__ __forceinline__ void half_step(const unsigned short* Ks, const unsign
         else if (p0 < nP && xi > 4 * ((p0 / 2) + 1)) mfma_p(0, p0++);
         else if (p1 < nP && xi > 4 * nC + 4 * (p1 / 2 + 1)) mfma_p(1, p1++);
         after_q();
-        if (sl < 4) {
-            dma(sl);
-            vread(sl);
+        if (sl == kPre) wait_and_barrier<kWaitVm8>();
+        if (sl >= kPre && sl < kPre + 4) {
+            dma(sl - kPre);
+            vread(sl - kPre);
         }
         if (sl >= kMaxStart && mi < nStages) max_stage();
         piece();
@@ -430,8 +433,7 @@ __device__ __forceinline__ void wide_step(const unsigned short* Ks, const unsign
     // which has just waited for all it reads before slot 9 and has since stored the early tile and requested K(j+5):
     // it only meets the other wave here (both have read their fragments of the slots about to be refilled) and
     // waits in slot 9, by when stores and request have long returned, for all but this trip's own six transfers.
-    if (first) wait_and_barrier<kWaitLgkm>();
-    else wait_and_barrier<kWaitVm0>();
+    // (As in the narrow step, the wait itself stands kPre slots into the trip.)
     // As in the narrow step, the fixed work of the trip rides in the issue slots.
     s16x8 vf[2][2][2];  // [half][16-key chunk][d tile]
     auto vread = [&](int f) {
@@ -507,10 +509,14 @@ __device__ __forceinline__ void wide_step(const unsigned short* Ks, const unsign
         if (qi < nQ) mfma_q();
         else if (p0 < nP && xi > 4 * ((p0 / 2) + 1)) mfma_p(0, p0++);
         else if (p1 < nP && xi > 8 + 4 * (p1 / 2 + 1)) mfma_p(1, p1++);
-        if (sl < 8) dma(sl);
-        if (sl < 4) {
-            vread(2 * sl);
-            vread(2 * sl + 1);
+        if (sl == kPre) {
+            if (first) wait_and_barrier<kWaitLgkm>();
+            else wait_and_barrier<kWaitVm0>();
+        }
+        if (sl >= kPre && sl < kPre + 8) dma(sl - kPre);
+        if (sl >= kPre && sl < kPre + 4) {
+            vread(2 * (sl - kPre));
+            vread(2 * (sl - kPre) + 1);
         } else if (sl >= 9 && sl < 11) {
             if (sl == 9 && first) wait_and_barrier<kWaitVm6>();
             if (NEXT && more_k) read_k_frags(Ks, c, (j + 4 + (sl - 9)) & 3, kf[sl - 9]);

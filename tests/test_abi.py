@@ -174,3 +174,24 @@ def test_static_scratch_entry_point_rejects_oversized_problems_on_the_host(ct):
     X = _desc(ct, (16384, 4)); W = _desc(ct, (16384,)); v = _desc(ct, (4,))
     assert L.mi_layer_norm_bwd_static(r(X), r(X), r(X), r(W), r(v), r(v), r(W), r(W), 64, 32, 1024, None) == ct.MI_E_SCRATCH
     assert "scratch" in ct.strerror(ct.MI_E_SCRATCH)
+
+
+def test_fused_moe_routed_weight_layouts_are_validated_on_the_host(ct):
+    """The routed weights may be the flattened vector of moe.jl:193 or the (num_tokens, topk) matrix itself; other
+    ranks, a matrix of the wrong extent or element type are refused before anything is launched."""
+    L = ct.lib(); r = ctypes.byref
+    K, N, E, tokens, topk, tile_m = 64, 128, 4, 6, 2, 16
+    total = tokens * topk
+    A = _desc(ct, (K, tokens), ct.MI_F16); B = _desc(ct, (K, N, E), ct.MI_F16); C = _desc(ct, (N, total), ct.MI_F16)
+    tok = _desc(ct, (4 * tile_m,), ct.MI_I32); exp = _desc(ct, (4,), ct.MI_I32)
+    call = lambda w, mul=1: L.mi_fused_moe_kernel(r(A), r(B), r(C), w, r(tok), r(exp), 1, mul, tile_m, 128, 64, None, None)
+    assert call(None) == ct.MI_E_NULL
+    assert call(r(_desc(ct, (tokens, topk, 1), ct.MI_F16))) == ct.MI_E_RANK
+    assert call(r(_desc(ct, (tokens, topk), ct.MI_F32))) == ct.MI_E_DTYPE
+    assert call(r(_desc(ct, (tokens - 1, topk), ct.MI_F16))) == ct.MI_E_SHAPE
+    assert call(r(_desc(ct, (tokens, topk + 1), ct.MI_F16))) == ct.MI_E_SHAPE
+    assert call(r(_desc(ct, (total - 1,), ct.MI_F16))) == ct.MI_E_SHAPE
+    assert call(r(_desc(ct, (total,), ct.MI_F16, strides=(2,)))) == ct.MI_E_STRIDE
+    # weights that are not used (mul_routed_weight = 0) need no particular extent; an empty problem is a no-op
+    C0 = _desc(ct, (0, total), ct.MI_F16, ptr=0); B0 = _desc(ct, (K, 0, E), ct.MI_F16, ptr=0)
+    assert L.mi_fused_moe_kernel(r(A), r(B0), r(C0), r(_desc(ct, (3,), ct.MI_F16)), r(tok), r(exp), 1, 0, tile_m, 128, 64, None, None) == 0

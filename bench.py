@@ -58,16 +58,33 @@ def _event_times(fn, nruns, warmup):
     return out
 
 
-def _back_to_back(fn, nruns):
-    """nruns launches between one pair of events; returns average ms per launch."""
+WARM_MS, TIMED_MS = 5.0, 20.0   # GPU time of the untimed launches in front of a timed batch, and of the batch itself
+
+
+def _batch_counts(nruns, est_ms):
+    if not est_ms:
+        return nruns, nruns
+    return max(nruns, min(1000, int(WARM_MS / est_ms))), max(nruns, min(4000, int(TIMED_MS / est_ms)))
+
+
+def _back_to_back(fn, nruns, est_ms=None):
+    """A batch of launches between one pair of events; returns average ms per launch.  With an estimate of the
+    launch duration the batch lasts about TIMED_MS of GPU time (never fewer than nruns launches) and stands
+    directly behind about WARM_MS of untimed launches of the same kernel, so that it runs at the clocks of a
+    busy GPU: coming from idle, the power management takes milliseconds to settle (the attention kernel takes
+    31-33 us per launch in bursts of 20 to 200 launches from idle and 28.5 us in a run of 2000; the f16 GEMM,
+    which is power-limited, moves the other way)."""
     import torch
     torch.cuda.synchronize()
     e0 = torch.cuda.Event(enable_timing=True); e1 = torch.cuda.Event(enable_timing=True)
+    warm, n = _batch_counts(nruns, est_ms)
+    for _ in range(warm):
+        fn()
     e0.record()
-    for _ in range(nruns):
+    for _ in range(n):
         fn()
     e1.record(); e1.synchronize()
-    return e0.elapsed_time(e1) / nruns
+    return e0.elapsed_time(e1) / n
 
 
 def _entry(name, fn, work, unit, bound, peak, dtype, nruns, warmup, extra=None, cold=None):
@@ -75,12 +92,12 @@ def _entry(name, fn, work, unit, bound, peak, dtype, nruns, warmup, extra=None, 
     the 256 MB memory-side cache holds is touched between two uses of a set; ``frac_cold`` is measured
     by cycling through them, so that no launch finds its input resident."""
     t = _event_times(fn, nruns, warmup)
-    batches = [_back_to_back(fn, nruns) for _ in range(2)]
+    batches = [_back_to_back(fn, nruns, min(t)) for _ in range(2)]
     avg = min(batches)   # best of two batches: a one-off stall does not define the rate
     scale = 1e9 if unit == "GB/s" else 1e12
     ach = work / (avg * 1e-3) / scale
     e = {"name": name, "min_ms": round(min(t), 5), "mean_ms": round(sum(t) / len(t), 5), "avg_ms": round(avg, 5),
-         "avg_ms_is": "best of 2 batches of %d back-to-back launches" % nruns,
+         "avg_ms_is": "best of 2 batches of %d back-to-back launches (about %.0f ms), each directly behind %d untimed ones" % (_batch_counts(nruns, min(t))[1], TIMED_MS, _batch_counts(nruns, min(t))[0]),
          "work": work, "achieved": round(ach, 2), "unit": "GB/s" if unit == "GB/s" else "TFLOP/s", "bound": bound,
          "peak": peak, "frac": round(ach / peak, 4), "dtype": dtype}
     if cold:

@@ -91,6 +91,12 @@ def _entry(name, fn, work, unit, bound, peak, dtype, nruns, warmup, extra=None, 
     """``cold``: a list of launches of the same kernel on distinct buffer sets, enough of them that more than
     the 256 MB memory-side cache holds is touched between two uses of a set; ``frac_cold`` is measured
     by cycling through them, so that no launch finds its input resident."""
+    calls = [0]
+    raw_fn = fn
+
+    def fn():
+        calls[0] += 1
+        return raw_fn()
     t = _event_times(fn, nruns, warmup)
     batches = [_back_to_back(fn, nruns, min(t)) for _ in range(2)]
     avg = min(batches)   # best of two batches: a one-off stall does not define the rate
@@ -100,6 +106,7 @@ def _entry(name, fn, work, unit, bound, peak, dtype, nruns, warmup, extra=None, 
          "avg_ms_is": "best of 2 batches of %d back-to-back launches (about %.0f ms), each directly behind %d untimed ones" % (_batch_counts(nruns, min(t))[1], TIMED_MS, _batch_counts(nruns, min(t))[0]),
          "work": work, "achieved": round(ach, 2), "unit": "GB/s" if unit == "GB/s" else "TFLOP/s", "bound": bound,
          "peak": peak, "frac": round(ach / peak, 4), "dtype": dtype}
+    e["launches"] = calls[0]   # calls of the entry point made for the figures above (warm-up included)
     if cold:
         k = len(cold)
 

@@ -443,7 +443,7 @@ def bench_kernels(ct, which, cpu, nruns=NRUNS, warmup=WARMUP):
         whole_dev = lambda: moe.cutile_moe(d.hidden_states, d.w1, d.w2, d.topk_weights, d.topk_ids, 128, 128, 64,
                                            device_align=True, fuse_silu=False)
         default_call = lambda: moe.cutile_moe(d.hidden_states, d.w1, d.w2, d.topk_weights, d.topk_ids, 128, 128, 64)
-        res["moe_f16_default"] = extra(_entry("MoE f16 top-2, cutile_moe with its defaults (token sort on the GPU, SiLU*up fused; eager launches incl. allocations)",
+        res["moe_f16_default"] = extra(_entry("MoE f16 top-2, cutile_moe with its defaults (token sort on the GPU, SiLU*up fused, down projection adding into the output: 3 launches; eager, incl. allocations)",
                                               default_call, wbytes, "GB/s", "hbm", HBM_PEAK_GBS, "f16", nruns, warmup))
         res["moe_f16_device_align"] = extra(_entry("MoE f16 top-2, whole cutile_moe with the token sort on the GPU (no host round trip; eager launches)",
                                                    whole_dev, wbytes, "GB/s", "hbm", HBM_PEAK_GBS, "f16", nruns, warmup))

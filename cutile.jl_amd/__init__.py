@@ -72,6 +72,7 @@ _SIGNATURES = {
     "mi_fmha_kernel": ([_A, _A, _A, _A, ctypes.c_float, ctypes.c_int32, _i, _i, _i, _i, _i, _i, _i, _vp], _i),
     "mi_fft_kernel": ([_A, _A, _A, _A, _A, _A, _A, _i, _i, _i, _i, _i, _i, _vp], _i),
     "mi_moe_align_tile_size_device": ([_A, _i, _i, _A, _A, _vp], _i),
+    "mi_moe_align_tile_size_device_clear": ([_A, _i, _i, _A, _A, _A, _vp], _i),
     "mi_moe_route_topk": ([_A, _A, _A, _vp], _i),
     "mi_moe_align_tile_size": (
         [ctypes.POINTER(ctypes.c_int64), ctypes.c_int64, ctypes.c_int64, _i, _i,
@@ -79,6 +80,7 @@ _SIGNATURES = {
          ctypes.POINTER(ctypes.c_int64)], _i),
     "mi_fused_moe_kernel": ([_A] * 6 + [_i, _i, _i, _i, _i, _A, _vp], _i),
     "mi_fused_moe_silu_kernel": ([_A] * 6 + [_i, _i, _i, _i, _i, _A, _vp], _i),
+    "mi_fused_moe_accumulate_kernel": ([_A] * 6 + [_i, _i, _i, _A, _vp], _i),
     "mi_silu_and_mul_kernel": ([_A, _A, _A, _i, _vp], _i),
     "mi_moe_sum_topk": ([_A, _A, _vp], _i),
     "mi_tiled_broadcast": ([_A, ctypes.c_char_p, ctypes.POINTER(_A), _i, _vp, _i, _vp], _i),
@@ -313,10 +315,12 @@ def moe_align_capacity(num_tokens: int, topk: int, tile_m: int, num_experts: int
 
 
 def moe_align_tile_size_device(topk_ids, tile_m: int, num_experts: int, sorted_token_ids=None,
-                               sorted_expert_ids=None, stream=None):
+                               sorted_expert_ids=None, stream=None, clear=None):
     """On-device ``moe_align_tile_size`` (no host round trip).  ``topk_ids``: device int64 tensor
     of torch shape (topk, num_tokens).  Returns device int32 tensors of fixed capacity
-    (``moe_align_capacity``); unused slots hold the sentinel, unused blocks expert 0."""
+    (``moe_align_capacity``); unused slots hold the sentinel, unused blocks expert 0.
+    ``clear``: a dense device tensor of whole 16-byte units that the same launch fills with zeros
+    (the output that ``fused_moe_accumulate_kernel`` adds into)."""
     import torch
     topk, num_tokens = topk_ids.shape
     blocks, slots = moe_align_capacity(num_tokens, topk, tile_m, num_experts)
@@ -324,8 +328,12 @@ def moe_align_tile_size_device(topk_ids, tile_m: int, num_experts: int, sorted_t
         sorted_token_ids = torch.empty(slots, dtype=torch.int32, device=topk_ids.device)
     if sorted_expert_ids is None:
         sorted_expert_ids = torch.empty(blocks, dtype=torch.int32, device=topk_ids.device)
-    _call("mi_moe_align_tile_size_device", _ref(topk_ids), tile_m, num_experts, _ref(sorted_token_ids),
-          _ref(sorted_expert_ids), _stream(stream))
+    if clear is None:
+        _call("mi_moe_align_tile_size_device", _ref(topk_ids), tile_m, num_experts, _ref(sorted_token_ids),
+              _ref(sorted_expert_ids), _stream(stream))
+    else:
+        _call("mi_moe_align_tile_size_device_clear", _ref(topk_ids), tile_m, num_experts, _ref(sorted_token_ids),
+              _ref(sorted_expert_ids), _ref(clear), _stream(stream))
     return sorted_token_ids, sorted_expert_ids
 
 
@@ -351,6 +359,17 @@ def fused_moe_kernel(A, B, C, topk_weights, sorted_token_ids, sorted_expert_ids,
     _call("mi_fused_moe_kernel", _ref(A), _ref(B), _ref(C), _ref(topk_weights),
           _ref(sorted_token_ids), _ref(sorted_expert_ids), num_token_replicas,
           int(bool(mul_routed_weight)), TILE_M, TILE_N, TILE_K, _ref(b_scale), _stream(stream))
+
+
+def fused_moe_accumulate_kernel(A, B, Out, topk_weights, sorted_token_ids, sorted_expert_ids, TILE_M: int, TILE_N: int,
+                                TILE_K: int, b_scale=None, stream=None):
+    """The down projection of cutile_moe (fused_moe_kernel with mul_routed_weight, moe.jl:245-251) and the sum over
+    the top-k slots (moe.jl:256) in one launch: ``Out`` (torch (num_tokens, N), zeroed beforehand) receives every
+    replica's weighted row, rounded to the storage type as cache3 would hold it, by memory-side packed atomic adds.
+    top-k of 1 or 2 only (two terms add up the same in either order), ``topk_weights`` as the (num_tokens, topk)
+    matrix, N even."""
+    _call("mi_fused_moe_accumulate_kernel", _ref(A), _ref(B), _ref(Out), _ref(topk_weights), _ref(sorted_token_ids),
+          _ref(sorted_expert_ids), TILE_M, TILE_N, TILE_K, _ref(b_scale), _stream(stream))
 
 
 def fused_moe_silu_kernel(A, B, C, topk_weights, sorted_token_ids, sorted_expert_ids,

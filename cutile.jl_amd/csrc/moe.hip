@@ -42,6 +42,11 @@ struct F16 {
     static __device__ __forceinline__ float widen(unsigned short h) {
         return (float)__builtin_bit_cast(_Float16, h);
     }
+    // *p += the two values packed in `pair` (one memory-side atomic; round to nearest even, denormals kept)
+    static __device__ __forceinline__ void atomic_add2(unsigned short* p, unsigned pair) {
+        typedef _Float16 h2 __attribute__((ext_vector_type(2)));
+        __builtin_amdgcn_global_atomic_fadd_v2f16((h2 __attribute__((address_space(1)))*)p, __builtin_bit_cast(h2, pair));
+    }
 };
 struct BF16 {
     static __device__ __forceinline__ f32x16 mfma32(s16x8 a, s16x8 b, f32x16 c) {
@@ -54,6 +59,10 @@ struct BF16 {
         return (unsigned short)(u >> 16);
     }
     static __device__ __forceinline__ float widen(unsigned short h) { return __uint_as_float(((unsigned)h) << 16); }
+    static __device__ __forceinline__ void atomic_add2(unsigned short* p, unsigned pair) {
+        typedef short s2 __attribute__((ext_vector_type(2)));
+        __builtin_amdgcn_global_atomic_fadd_v2bf16((s2 __attribute__((address_space(1)))*)p, __builtin_bit_cast(s2, pair));
+    }
 };
 
 // Four E4M3FN bytes -> four values of the activation type.  gfx950's FP8 is the OCP E4M3FN
@@ -130,7 +139,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(TS == 1 ? 4
     const unsigned short* __restrict__ topk_weights, const int* __restrict__ sorted_token_ids, int num_slots,
     const int* __restrict__ sorted_expert_ids, const float* __restrict__ b_scale, int64_t ld_scale, int K, int N,
     int num_experts, int replicas, bool mul_routed_weight, int TILE_M, int tile_slots, int n_blocks, bool vecA,
-    bool vecB, int w_topk, int64_t w_s0, int64_t w_s1) {
+    bool vecB, int w_topk, int64_t w_s0, int64_t w_s1, int acc_shift) {
     constexpr int kNT = 32 * NTW, KW = 4 / NTW;
     // B tile [n][k], 16-byte chunks XOR-swizzled.  E4M3 weights stay raw bytes here (half the LDS
     // traffic and footprint) and are widened after the fragment read; see b_offset8 below.
@@ -439,6 +448,26 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(TS == 1 ? 4
                     C[gc + (int64_t)(tok - 1) * ldc] = E::cvt(silu_mul(g, u));
                 }
             }
+        } else if (acc_shift >= 0) {
+            // Accumulating form: C is (N, num_tokens) and column (token_id - 1) >> acc_shift receives the replica's
+            // value as rounded to the storage type, by a packed atomic add of two adjacent channels: lanes 2i and
+            // 2i + 1 exchange their values, the even lane sends the even rows and the odd lane the odd ones.
+            const int gn = n0 + wn * 32 + (lane & 31);
+            float ch_scale = 1.f;
+            if (W8 && gn < N) ch_scale = b_scale[gn + (int64_t)expert * ld_scale];
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const int tok = toks[r];
+                float v = acc[ts][r];
+                if (W8) v *= ch_scale;
+                if (mul_routed_weight) v *= wts[r];
+                const unsigned own = (tok && gn < N) ? (unsigned)E::cvt(v) : 0u;
+                const unsigned nbr = (unsigned)__shfl_xor((int)own, 1, 64);
+                if ((((unsigned)r ^ (unsigned)lane) & 1u) == 0u && tok && gn < N) {
+                    const unsigned pair = (lane & 1) ? (nbr | (own << 16)) : (own | (nbr << 16));
+                    E::atomic_add2(C + (gn & ~1) + (int64_t)((tok - 1) >> acc_shift) * ldc, pair);
+                }
+            }
         } else {
             const int gn = n0 + wn * 32 + (lane & 31);
             if (gn < N) {
@@ -541,7 +570,8 @@ bool is16(int dt) { return dt == MI_F16 || dt == MI_BF16; }
 static int fused_moe_impl(const mi_tile_array* A, const mi_tile_array* B, const mi_tile_array* C,
                           const mi_tile_array* topk_weights, const mi_tile_array* sorted_token_ids,
                           const mi_tile_array* sorted_expert_ids, int num_token_replicas, int mul_routed_weight,
-                          int TILE_M, int TILE_N, int TILE_K, const mi_tile_array* b_scale, bool silu, void* stream) {
+                          int TILE_M, int TILE_N, int TILE_K, const mi_tile_array* b_scale, bool silu, void* stream,
+                          bool accumulate = false) {
     MI_CHECK(check_array(A, 2));
     MI_CHECK(check_array(B, 3));
     MI_CHECK(check_array(C, 2));
@@ -560,7 +590,17 @@ static int fused_moe_impl(const mi_tile_array* A, const mi_tile_array* B, const 
     const int64_t K = B->sizes[0], N = B->sizes[1], E = B->sizes[2];
     if (silu && (N % 2)) return MI_E_SHAPE;
     if (A->sizes[0] != K || C->sizes[0] != (silu ? N / 2 : N)) return MI_E_SHAPE;
-    const int64_t slots = sorted_token_ids->sizes[0], total = C->sizes[1];
+    // accumulating form: C is (N, num_tokens), and the replicas of a token are added into its column
+    int acc_shift = -1;
+    if (accumulate) {
+        if (topk_weights->ndim != 2 || !mul_routed_weight || silu) return MI_E_ARG;
+        const int64_t topk = topk_weights->sizes[1];
+        if (topk != 1 && topk != 2) return MI_E_UNSUPPORTED;   // (two terms add up the same in either order; more would not)
+        if (C->sizes[1] != topk_weights->sizes[0]) return MI_E_SHAPE;
+        if (N % 2 || C->strides[1] % 2 || !aligned(C->ptr, 4)) return MI_E_ALIGN;
+        acc_shift = (int)topk - 1;
+    }
+    const int64_t slots = sorted_token_ids->sizes[0], total = accumulate ? C->sizes[1] * topk_weights->sizes[1] : C->sizes[1];
     const int64_t m_blocks = cld(slots, (int64_t)TILE_M);
     if (sorted_expert_ids->sizes[0] < m_blocks) return MI_E_SHAPE;
     // routed weights: the flattened vector of moe.jl:193, or the (num_tokens, topk) matrix itself with any strides
@@ -618,7 +658,7 @@ static int fused_moe_impl(const mi_tile_array* A, const mi_tile_array* B, const 
                        (const int*)sorted_token_ids->ptr, (int)slots, (const int*)sorted_expert_ids->ptr,           \
                        w8 ? (const float*)b_scale->ptr : nullptr, w8 ? b_scale->strides[1] : 0, (int)K, (int)N,     \
                        (int)E, num_token_replicas, mul_routed_weight != 0, TILE_M, tile_slots, n_blocks, vecA, vecB,     \
-                       (int)w_topk, w2d ? topk_weights->strides[0] : (int64_t)1, w2d ? topk_weights->strides[1] : (int64_t)0)
+                       (int)w_topk, w2d ? topk_weights->strides[0] : (int64_t)1, w2d ? topk_weights->strides[1] : (int64_t)0, acc_shift)
 #define LAUNCH_SHAPE(ET, W8)                                  \
     do {                                                      \
         if (silu && ts == 2) LAUNCH(ET, W8, 4, 128, true, 2); \
@@ -663,6 +703,14 @@ extern "C" int mi_fused_moe_silu_kernel(const mi_tile_array* A, const mi_tile_ar
                           TILE_M, TILE_N, TILE_K, b_scale, true, stream);
 }
 
+extern "C" int mi_fused_moe_accumulate_kernel(const mi_tile_array* A, const mi_tile_array* B, const mi_tile_array* Out,
+                                              const mi_tile_array* topk_weights, const mi_tile_array* sorted_token_ids,
+                                              const mi_tile_array* sorted_expert_ids, int TILE_M, int TILE_N, int TILE_K,
+                                              const mi_tile_array* b_scale, void* stream) {
+    return fused_moe_impl(A, B, Out, topk_weights, sorted_token_ids, sorted_expert_ids, 1, 1, TILE_M, TILE_N, TILE_K, b_scale,
+                          false, stream, true);
+}
+
 // ---- on-device moe_align_tile_size ------------------------------------------------------------
 // One workgroup of sixteen waves.  Counting sort by expert of the replica ids (slot-fastest
 // flattening of topk_ids, examples/moe.jl:148-150): LDS histogram, scan over the experts,
@@ -676,10 +724,18 @@ constexpr int kAlignThreads = 1024, kAlignWaves = kAlignThreads / 64, kAlignCach
 __global__ __launch_bounds__(kAlignThreads) void moe_align_kernel(const long long* __restrict__ topk_ids, int64_t ld_slot,
                                                         int num_tokens, int topk, int tile_m, int num_experts,
                                                         int* __restrict__ sorted_token_ids, int cap_slots,
-                                                        int* __restrict__ sorted_expert_ids, int cap_blocks) {
+                                                        int* __restrict__ sorted_expert_ids, int cap_blocks,
+                                                        u32x4* __restrict__ clear, int64_t clear_n16) {
     __shared__ int cursor[kAlignMaxExperts];      // histogram, then next free slot of every expert
     __shared__ unsigned short tbl[kAlignWaves][kAlignMaxExperts];   // replicas per (wave, expert) of the current super-block (<= 64)
     __shared__ int s_blocks, wave_total[kAlignWaves];
+    // Workgroups past the first only zero their share of the array the caller wants cleared on the way (e.g. the
+    // output that the accumulating down projection adds into); the first one sorts.
+    if (blockIdx.x > 0) {
+        for (int64_t i = (int64_t)(blockIdx.x - 1) * kAlignThreads + threadIdx.x; i < clear_n16; i += (int64_t)(gridDim.x - 1) * kAlignThreads)
+            clear[i] = u32x4{0, 0, 0, 0};
+        return;
+    }
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, total = num_tokens * topk;
     // The ids of the first kAlignCached super-blocks stay in registers between the counting pass and the placing
     // pass, and are requested before the tables are cleared: one memory round trip instead of three in a row.
@@ -765,9 +821,8 @@ __global__ __launch_bounds__(kAlignThreads) void moe_align_kernel(const long lon
     }
 }
 
-extern "C" int mi_moe_align_tile_size_device(const mi_tile_array* topk_ids, int tile_m, int num_experts,
-                                             const mi_tile_array* sorted_token_ids,
-                                             const mi_tile_array* sorted_expert_ids, void* stream) {
+static int moe_align_device_impl(const mi_tile_array* topk_ids, int tile_m, int num_experts, const mi_tile_array* sorted_token_ids,
+                                 const mi_tile_array* sorted_expert_ids, const mi_tile_array* clear, void* stream) {
     MI_CHECK(check_array(topk_ids, 2));
     MI_CHECK(check_array(sorted_token_ids, 1));
     MI_CHECK(check_array(sorted_expert_ids, 1));
@@ -787,12 +842,41 @@ extern "C" int mi_moe_align_tile_size_device(const mi_tile_array* topk_ids, int 
     if ((cap_slots > 1 && sorted_token_ids->strides[0] != 1) || (cap_blocks > 1 && sorted_expert_ids->strides[0] != 1))
         return MI_E_STRIDE;
     if (cap_slots > 0x7fffffff) return MI_E_SHAPE;
-    if (cap_blocks == 0) return MI_OK;
-    hipLaunchKernelGGL(moe_align_kernel, dim3(1), dim3(kAlignThreads), 0, (hipStream_t)stream, (const long long*)topk_ids->ptr,
+    int64_t clear_n16 = 0;
+    if (clear) {   // a dense array of whole 16-byte units
+        MI_CHECK(check_array(clear, clear->ndim));
+        int64_t n = 1, run = 1;
+        for (int d = 0; d < clear->ndim; ++d) {
+            if (clear->sizes[d] > 1 && clear->strides[d] != run) return MI_E_STRIDE;
+            run *= clear->sizes[d];
+            n *= clear->sizes[d];
+        }
+        const int64_t bytes = n * dtype_size(clear->dtype);
+        if (bytes % 16 || !aligned(clear->ptr, 16)) return MI_E_ALIGN;
+        clear_n16 = bytes / 16;
+    }
+    if (cap_blocks == 0 && clear_n16 == 0) return MI_OK;
+    const int64_t clear_wgs = clear_n16 ? (cld(clear_n16, (int64_t)(4 * kAlignThreads)) < 256 ? cld(clear_n16, (int64_t)(4 * kAlignThreads)) : 256) : 0;
+    hipLaunchKernelGGL(moe_align_kernel, dim3((unsigned)(1 + clear_wgs)), dim3(kAlignThreads), 0, (hipStream_t)stream, (const long long*)topk_ids->ptr,
                        topk > 1 ? topk_ids->strides[1] : 0, (int)num_tokens, (int)topk, tile_m, num_experts,
-                       (int*)sorted_token_ids->ptr, (int)cap_slots, (int*)sorted_expert_ids->ptr, (int)cap_blocks);
+                       (int*)sorted_token_ids->ptr, (int)cap_slots, (int*)sorted_expert_ids->ptr, (int)cap_blocks,
+                       clear ? (u32x4*)clear->ptr : nullptr, clear_n16);
     set_variant("moe_align_device_1wg");
     return launch_status();
+}
+
+extern "C" int mi_moe_align_tile_size_device(const mi_tile_array* topk_ids, int tile_m, int num_experts,
+                                             const mi_tile_array* sorted_token_ids,
+                                             const mi_tile_array* sorted_expert_ids, void* stream) {
+    return moe_align_device_impl(topk_ids, tile_m, num_experts, sorted_token_ids, sorted_expert_ids, nullptr, stream);
+}
+
+extern "C" int mi_moe_align_tile_size_device_clear(const mi_tile_array* topk_ids, int tile_m, int num_experts,
+                                                   const mi_tile_array* sorted_token_ids,
+                                                   const mi_tile_array* sorted_expert_ids, const mi_tile_array* clear,
+                                                   void* stream) {
+    if (!clear) return MI_E_NULL;
+    return moe_align_device_impl(topk_ids, tile_m, num_experts, sorted_token_ids, sorted_expert_ids, clear, stream);
 }
 
 // ---- on-device router ---------------------------------------------------------------------------

@@ -31,7 +31,7 @@ def invoke_silu_and_mul_kernel(AB, C):
 
 
 def cutile_moe(hidden_states, w1, w2, topk_weights, topk_ids, tile_m, tile_n, tile_k, *, w1_scale=None,
-               w2_scale=None, aligned=None, device_align=True, fuse_silu=True):
+               w2_scale=None, aligned=None, device_align=True, fuse_silu=True, fuse_sum=None):
     """moe.jl:218-257.  Torch shapes (reversed Julia): hidden_states (tokens, hidden); w1
     (E, 2*inter, hidden); w2 (E, hidden, inter); topk_weights / topk_ids (topk, tokens), ids
     1-based int64.  ``aligned`` may carry a precomputed (sorted_token_ids, sorted_expert_ids)
@@ -39,25 +39,35 @@ def cutile_moe(hidden_states, w1, w2, topk_weights, topk_ids, tile_m, tile_n, ti
     (fixed-capacity outputs, nothing leaves the device), ``device_align=False`` is the reference's
     orchestration with the host round trip of moe.jl:232-233.  ``fuse_silu`` (default) runs the gate / up
     GEMM with SiLU * up as its epilogue: cache1 and the silu_and_mul launch disappear;
-    ``fuse_silu=False`` launches the kernels one by one as moe.jl:234-251 does.  All four combinations
-    give bit-identical results."""
+    ``fuse_silu=False`` launches the kernels one by one as moe.jl:234-251 does.  ``fuse_sum`` (default: whenever
+    it applies -- one or two slots per token, device-side sort, an even hidden size of whole 16-byte rows) lets the
+    down projection add every replica's row into the output itself, which the sort launch has zeroed: cache3 and
+    the top-k sum launch disappear.  All combinations give bit-identical results."""
     num_tokens, hidden_size = hidden_states.shape
     num_experts, _, intermediate_size = w2.shape
     topk = topk_ids.shape[0]
     total_tokens = num_tokens * topk
     T, dev = hidden_states.dtype, hidden_states.device
+    can_fuse_sum = (topk <= 2 and aligned is None and device_align and hidden_size % 8 == 0 and topk_weights.dtype == T)
+    if fuse_sum is None:
+        fuse_sum = can_fuse_sum
+    elif fuse_sum and not can_fuse_sum:
+        raise ValueError("fuse_sum needs top-k <= 2, the device-side sort and a hidden size that is a multiple of 8")
     # The three caches of moe.jl:228-230, carved out of one allocation.  The reference zero-fills them; here they
     # are left as allocated: every column of every cache belongs to one (token, slot) replica, the GEMMs write the
     # columns of all replicas (only padding slots write nothing, and nothing reads those), so no fill is ever
     # read.  This holds for expert ids in 1..num_experts, which is what the reference accepts as well
     # (moe_align_tile_size indexes by them, moe.jl:150-160).
     n1 = 0 if fuse_silu else total_tokens * intermediate_size * 2
-    n2, n3 = total_tokens * intermediate_size, total_tokens * hidden_size
+    n2, n3 = total_tokens * intermediate_size, 0 if fuse_sum else total_tokens * hidden_size
     caches = torch.empty(n1 + n2 + n3, dtype=T, device=dev)
     cache1 = None if fuse_silu else caches[:n1].view(num_tokens, topk, intermediate_size * 2)
     cache2 = caches[n1:n1 + n2].view(total_tokens, intermediate_size)
-    cache3 = caches[n1 + n2:].view(num_tokens, topk, hidden_size)
-    if aligned is None and device_align:
+    cache3 = None if fuse_sum else caches[n1 + n2:].view(num_tokens, topk, hidden_size)
+    out = torch.empty((num_tokens, hidden_size), dtype=T, device=dev)
+    if fuse_sum:
+        sorted_token_ids, sorted_expert_ids = ct.moe_align_tile_size_device(topk_ids, tile_m, num_experts, clear=out)
+    elif aligned is None and device_align:
         sorted_token_ids, sorted_expert_ids = ct.moe_align_tile_size_device(topk_ids, tile_m, num_experts)
     elif aligned is None:
         tok, exp = ct.moe_align_tile_size(topk_ids.cpu(), tile_m, num_experts)
@@ -74,10 +84,13 @@ def cutile_moe(hidden_states, w1, w2, topk_weights, topk_ids, tile_m, tile_n, ti
                                 tile_k=tile_k, b_scale=w1_scale)
         cache1_flat = cache1.reshape(total_tokens, intermediate_size * 2)
         invoke_silu_and_mul_kernel(cache1_flat, cache2)
+    if fuse_sum:
+        ct.fused_moe_accumulate_kernel(cache2, w2, out, topk_weights, sorted_token_ids, sorted_expert_ids, tile_m, tile_n,
+                                       tile_k, b_scale=w2_scale)
+        return out
     invoke_fused_moe_kernel(cache2, w2, cache3, topk_weights, sorted_token_ids, sorted_expert_ids,
                             mul_routed_weight=True, num_token_replicas=1, tile_m=tile_m, tile_n=tile_n,
                             tile_k=tile_k, b_scale=w2_scale)
-    out = torch.empty((num_tokens, hidden_size), dtype=T, device=dev)
     ct.moe_sum_topk(cache3, out)  # sum(cache3; dims=2), moe.jl:256
     return out
 

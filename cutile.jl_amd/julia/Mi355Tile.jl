@@ -264,6 +264,33 @@ function moe_route_topk(logits, topk_weights, topk_ids; stream::Ptr{Cvoid}=C_NUL
         d[1], d[2], d[3], stream))
 end
 
+# The sort of `moe_align_tile_size_device`, which also fills `clear` (a dense device array of whole 16-byte units) with
+# zeros in the same launch: the output that `fused_moe_accumulate_kernel` adds into.
+function moe_align_tile_size_device_clear(topk_ids, tile_m::Integer, num_experts::Integer, sorted_token_ids,
+                                          sorted_expert_ids, clear; stream::Ptr{Cvoid}=C_NULL)
+    d = map(a -> ref(descriptor(a)), (topk_ids, sorted_token_ids, sorted_expert_ids, clear))
+    GC.@preserve topk_ids sorted_token_ids sorted_expert_ids clear check(ccall(
+        (:mi_moe_align_tile_size_device_clear, libmi355tile), Cint,
+        (Ref{MiTileArray}, Cint, Cint, Ref{MiTileArray}, Ref{MiTileArray}, Ref{MiTileArray}, Ptr{Cvoid}),
+        d[1], tile_m, num_experts, d[2], d[3], d[4], stream))
+end
+
+# The down projection and `sum(cache3; dims=2)` (moe.jl:245-256) in one launch: `Out` (N, num_tokens), zeroed
+# beforehand, receives every replica's weighted row by packed atomic adds.  `topk_weights` is the (num_tokens, topk)
+# matrix, topk = 1 or 2.
+function fused_moe_accumulate_kernel(A, B, Out, topk_weights, sorted_token_ids, sorted_expert_ids,
+                                     TILE_M::Integer, TILE_N::Integer, TILE_K::Integer;
+                                     b_scale=nothing, stream::Ptr{Cvoid}=C_NULL)
+    d = map(a -> ref(descriptor(a)), (A, B, Out, topk_weights, sorted_token_ids, sorted_expert_ids))
+    ds = b_scale === nothing ? nothing : ref(descriptor(b_scale))
+    GC.@preserve A B Out topk_weights sorted_token_ids sorted_expert_ids b_scale check(ccall(
+        (:mi_fused_moe_accumulate_kernel, libmi355tile), Cint,
+        (Ref{MiTileArray}, Ref{MiTileArray}, Ref{MiTileArray}, Ref{MiTileArray}, Ref{MiTileArray}, Ref{MiTileArray},
+         Cint, Cint, Cint, Ptr{MiTileArray}, Ptr{Cvoid}),
+        d[1], d[2], d[3], d[4], d[5], d[6], TILE_M, TILE_N, TILE_K,
+        ds === nothing ? NULLDESC : Base.unsafe_convert(Ptr{MiTileArray}, ds), stream))
+end
+
 # `b_scale` (N, E) Float32 goes with e4m3fn weights only; `nothing` otherwise.  `topk_weights` is either the
 # flattened `vec(permutedims(topk_weights))` of moe.jl:193 or the (num_tokens, topk) matrix itself, which saves that copy.
 function fused_moe_kernel(A, B, C, topk_weights, sorted_token_ids, sorted_expert_ids,

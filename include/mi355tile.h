@@ -208,6 +208,13 @@ int mi_moe_align_tile_size(const int64_t* topk_ids, int64_t num_tokens, int64_t 
 int mi_moe_align_tile_size_device(const mi_tile_array* topk_ids, int tile_m, int num_experts,
                                   const mi_tile_array* sorted_token_ids,
                                   const mi_tile_array* sorted_expert_ids, void* stream);
+/* The same, and `clear` (a dense device array of whole 16-byte units, any rank and element type) is filled with zeros
+ * by the same launch: the output that mi_fused_moe_accumulate_kernel adds into, without a fill launch of its own.
+ * No counterpart in the reference (its caches come from CUDA.zeros, moe.jl:228-230). */
+int mi_moe_align_tile_size_device_clear(const mi_tile_array* topk_ids, int tile_m, int num_experts,
+                                        const mi_tile_array* sorted_token_ids,
+                                        const mi_tile_array* sorted_expert_ids, const mi_tile_array* clear,
+                                        void* stream);
 /* Router on the device: topk_ids[t, :] = the topk = size(topk_ids, 2) experts with the largest
  * logits[t, :] in descending order (ties to the lower expert id, NaN ranks as -Inf), 1-based;
  * topk_weights[t, :] = softmax over those topk logits.  logits (num_tokens, num_experts) f32 / f16 /
@@ -229,6 +236,18 @@ int mi_fused_moe_kernel(const mi_tile_array* A, const mi_tile_array* B, const mi
                         const mi_tile_array* sorted_expert_ids, int num_token_replicas,
                         int mul_routed_weight, int TILE_M, int TILE_N, int TILE_K,
                         const mi_tile_array* b_scale, void* stream);
+/* The second grouped GEMM of cutile_moe (moe.jl:245-251: mul_routed_weight = true, num_token_replicas = 1) fused
+ * with the sum over the top-k slots (moe.jl:256): Out (N, num_tokens), zeroed by the caller, receives every replica's
+ * weighted row -- rounded to the activation type first, as cache3 would hold it -- by memory-side packed atomic adds
+ * of two adjacent channels (round to nearest even, denormals kept).  topk_weights must be the (num_tokens, topk)
+ * matrix with topk = 1 or 2: two terms add up the same in either order, so the result is the one mi_fused_moe_kernel +
+ * mi_moe_sum_topk give, bit for bit, and is the same from run to run; MI_E_UNSUPPORTED for more slots.  N even, Out
+ * 4-byte aligned with an even column stride (MI_E_ALIGN).  A (K, num_tokens * topk), B, sorted_*, b_scale as for
+ * mi_fused_moe_kernel. */
+int mi_fused_moe_accumulate_kernel(const mi_tile_array* A, const mi_tile_array* B, const mi_tile_array* Out,
+                                   const mi_tile_array* topk_weights, const mi_tile_array* sorted_token_ids,
+                                   const mi_tile_array* sorted_expert_ids, int TILE_M, int TILE_N, int TILE_K,
+                                   const mi_tile_array* b_scale, void* stream);
 /* The first grouped GEMM of cutile_moe fused with silu_and_mul_kernel (moe.jl:234-251 launch them
  * one after the other through cache1): B holds the gate rows [0, N/2) and the up rows [N/2, N) of
  * every expert, C is (N/2, total_tokens) and receives SiLU(gate) * up.  Both products are rounded

@@ -195,3 +195,24 @@ def test_fused_moe_routed_weight_layouts_are_validated_on_the_host(ct):
     # weights that are not used (mul_routed_weight = 0) need no particular extent; an empty problem is a no-op
     C0 = _desc(ct, (0, total), ct.MI_F16, ptr=0); B0 = _desc(ct, (K, 0, E), ct.MI_F16, ptr=0)
     assert L.mi_fused_moe_kernel(r(A), r(B0), r(C0), r(_desc(ct, (3,), ct.MI_F16)), r(tok), r(exp), 1, 0, tile_m, 128, 64, None, None) == 0
+
+
+def test_accumulating_down_projection_and_clearing_sort_validate_on_the_host(ct):
+    L = ct.lib(); r = ctypes.byref
+    K, N, E, tokens, topk, tile_m = 64, 128, 4, 6, 2, 16
+    A = _desc(ct, (K, tokens * topk), ct.MI_F16); B = _desc(ct, (K, N, E), ct.MI_F16); Out = _desc(ct, (N, tokens), ct.MI_F16)
+    tok = _desc(ct, (4 * tile_m,), ct.MI_I32); exp = _desc(ct, (4,), ct.MI_I32); w = _desc(ct, (tokens, topk), ct.MI_F16)
+    call = lambda a=A, b=B, o=Out, ww=w: L.mi_fused_moe_accumulate_kernel(r(a), r(b), r(o), r(ww), r(tok), r(exp), tile_m, 128, 64, None, None)
+    assert call(ww=_desc(ct, (tokens * topk,), ct.MI_F16)) == ct.MI_E_ARG                 # needs the matrix: top-k is read from it
+    assert call(ww=_desc(ct, (tokens, 3), ct.MI_F16), a=_desc(ct, (K, tokens * 3), ct.MI_F16)) == ct.MI_E_UNSUPPORTED
+    assert call(o=_desc(ct, (N, tokens + 1), ct.MI_F16)) == ct.MI_E_SHAPE
+    assert call(b=_desc(ct, (K, N - 1, E), ct.MI_F16), o=_desc(ct, (N - 1, tokens), ct.MI_F16)) == ct.MI_E_ALIGN   # odd channel count
+    assert call(o=_desc(ct, (N, tokens), ct.MI_F16, ptr=0x1002)) == ct.MI_E_ALIGN
+    assert call(o=_desc(ct, (N, tokens), ct.MI_F16, strides=(1, N + 1))) == ct.MI_E_ALIGN
+    ids = _desc(ct, (tokens, topk), ct.MI_I64)
+    cap_t = _desc(ct, (12 * tile_m,), ct.MI_I32); cap_e = _desc(ct, (12,), ct.MI_I32)
+    clr = lambda c: L.mi_moe_align_tile_size_device_clear(r(ids), tile_m, E, r(cap_t), r(cap_e), c, None)
+    assert clr(None) == ct.MI_E_NULL
+    assert clr(r(_desc(ct, (N - 1, tokens), ct.MI_F16))) == ct.MI_E_ALIGN                 # not whole 16-byte units
+    assert clr(r(_desc(ct, (N, tokens), ct.MI_F16, ptr=0x1008))) == ct.MI_E_ALIGN
+    assert clr(r(_desc(ct, (N, tokens), ct.MI_F16, strides=(1, N + 8)))) == ct.MI_E_STRIDE

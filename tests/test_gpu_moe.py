@@ -394,3 +394,42 @@ def test_silu_and_topk_sum_beyond_65535_columns(ct, orc):
     out = torch.empty((total, 64), dtype=torch.float16, device="cuda")
     ct.moe_sum_topk(x, out)
     assert torch.equal(out, x.float().sum(dim=1).to(torch.float16))
+
+
+@pytest.mark.parametrize("tokens,hidden,experts,inter,topk,T,fp8", [
+    (256, 1024, 32, 2048, 2, torch.float16, False), (256, 1024, 32, 2048, 2, torch.float16, True),
+    (100, 256, 8, 192, 2, torch.bfloat16, False), (33, 128, 3, 64, 1, torch.float16, False),
+    (300, 264, 2, 256, 2, torch.float16, False), (1, 64, 4, 64, 2, torch.bfloat16, True),
+])
+def test_down_projection_that_adds_into_the_output(ct, orc, tokens, hidden, experts, inter, topk, T, fp8):
+    """fuse_sum: the sort launch zeroes the output and the down projection adds every replica's row into it with
+    packed atomic adds (mi_fused_moe_accumulate_kernel) -- three launches, no cache3.  With one or two slots per token
+    the sum does not depend on the order of arrival, and the atomic add rounds like the separate sum does: the result
+    is the unfused one bit for bit, run after run, and is checked against the float64 oracle as well."""
+    d = moe.prepare(num_tokens=tokens, hidden_size=hidden, num_experts=experts, intermediate_size=inter, topk=topk, T=T,
+                    router="top2_logits" if topk == 2 and experts >= 2 else "randperm")
+    kw = {}
+    if fp8:
+        q = moe.quantize_weights(d)
+        w1, w2, kw = q.w1, q.w2, dict(w1_scale=q.w1_scale, w2_scale=q.w2_scale)
+    else:
+        w1, w2 = d.w1, d.w2
+    plain = moe.cutile_moe(d.hidden_states, w1, w2, d.topk_weights, d.topk_ids, 128, 128, 64, fuse_sum=False, **kw)
+    assert ct.last_variant().startswith("moe_sum_topk")
+    for _ in range(3):
+        fused = moe.cutile_moe(d.hidden_states, w1, w2, d.topk_weights, d.topk_ids, 128, 128, 64, fuse_sum=True, **kw)
+        assert ct.last_variant().startswith("fused_moe_t")          # the last launch is the GEMM itself
+        assert torch.equal(fused, plain)
+    default = moe.cutile_moe(d.hidden_states, w1, w2, d.topk_weights, d.topk_ids, 128, 128, 64, **kw)
+    assert torch.equal(default, plain)
+    if not fp8:
+        J = orc.to_julia
+        ref = orc.ref_moe(J(d.hidden_states), J(d.w1), J(d.w2), J(d.topk_weights), J(d.topk_ids), dtype=np.float64)
+        check(J(fused), ref, 2e-2 if T == torch.float16 else 5e-2)
+    # more than two slots: the fused form is refused, the default falls back to the separate sum
+    if experts >= 4:
+        d4 = moe.prepare(num_tokens=tokens, hidden_size=hidden, num_experts=experts, intermediate_size=inter, topk=4, T=T)
+        with pytest.raises(ValueError):
+            moe.cutile_moe(d4.hidden_states, d4.w1, d4.w2, d4.topk_weights, d4.topk_ids, 128, 128, 64, fuse_sum=True)
+        moe.cutile_moe(d4.hidden_states, d4.w1, d4.w2, d4.topk_weights, d4.topk_ids, 128, 128, 64)
+        assert ct.last_variant().startswith("moe_sum_topk")

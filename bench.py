@@ -441,7 +441,7 @@ def bench_kernels(ct, which, cpu, nruns=NRUNS, warmup=WARMUP):
         res["moe_f16"] = extra(_entry("MoE f16 256tok/1024h/32e/2048i top-2, cutile_moe as the reference orchestrates it (host sort + H2D/D2H inside, 4 kernels)",
                                       whole, wbytes, "GB/s", "hbm", HBM_PEAK_GBS, "f16", nruns, warmup))
         whole_dev = lambda: moe.cutile_moe(d.hidden_states, d.w1, d.w2, d.topk_weights, d.topk_ids, 128, 128, 64,
-                                           device_align=True, fuse_silu=False)
+                                           device_align=True, fuse_silu=False, fuse_sum=False)
         default_call = lambda: moe.cutile_moe(d.hidden_states, d.w1, d.w2, d.topk_weights, d.topk_ids, 128, 128, 64)
         res["moe_f16_default"] = extra(_entry("MoE f16 top-2, cutile_moe with its defaults (token sort on the GPU, SiLU*up fused, down projection adding into the output: 3 launches; eager, incl. allocations)",
                                               default_call, wbytes, "GB/s", "hbm", HBM_PEAK_GBS, "f16", nruns, warmup))
@@ -463,12 +463,12 @@ def bench_kernels(ct, which, cpu, nruns=NRUNS, warmup=WARMUP):
         assert torch.equal(fused(), ref_out), "fused SiLU epilogue differs from the separate kernels"
         try:
             gf, _ = graph_of(fused)
-            res["moe_f16_device_fused"] = extra(_entry("MoE f16 top-2 on the device, SiLU*up fused into the gate/up GEMM epilogue (3 kernels + sort), HIP graph replay",
+            res["moe_f16_device_fused"] = extra(_entry("MoE f16 top-2 on the device, SiLU*up fused into the gate/up GEMM epilogue and the top-k sum into the down GEMM (sort + 2 GEMMs), HIP graph replay",
                                                        gf.replay, wbytes, "GB/s", "hbm", HBM_PEAK_GBS, "f16", nruns, warmup))
         except Exception as ex:
             res["moe_f16_device_fused"] = extra(_entry(f"MoE f16 top-2, fused SiLU epilogue (eager; graph failed: {type(ex).__name__})",
                                                        fused, wbytes, "GB/s", "hbm", HBM_PEAK_GBS, "f16", nruns, warmup))
-        # from router logits to output without a host step: router + sort + 3 kernels
+        # from router logits to output without a host step: router + sort + 2 GEMMs
         logits_jl = d.logits.t().contiguous()
         rw = torch.empty_like(d.topk_weights)
         rid = torch.empty_like(d.topk_ids)
@@ -480,7 +480,7 @@ def bench_kernels(ct, which, cpu, nruns=NRUNS, warmup=WARMUP):
         assert torch.equal(rid, d.topk_ids), "device router picks other experts than the host router"
         try:
             gr, _ = graph_of(routed)
-            res["moe_f16_device_routed"] = extra(_entry("MoE f16 top-2 from router logits to output on the device (router + sort + 3 kernels), HIP graph replay",
+            res["moe_f16_device_routed"] = extra(_entry("MoE f16 top-2 from router logits to output on the device (router + sort + 2 GEMMs), HIP graph replay",
                                                         gr.replay, wbytes, "GB/s", "hbm", HBM_PEAK_GBS, "f16", nruns, warmup))
         except Exception as ex:
             res["moe_f16_device_routed"] = extra(_entry(f"MoE f16 top-2 from router logits (eager; graph failed: {type(ex).__name__})",

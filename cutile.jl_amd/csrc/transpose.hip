@@ -3,10 +3,11 @@
 //
 // The result does not depend on the (tm,tn) tile constants, so the physical tiling is the
 // library's.  Two kernels:
-//   * 4-byte elements with every dimension and stride a multiple of 4 (the benchmark case):
-//     128 x 128 tiles of 1024 lanes (64 x 128 of 256 lanes for small matrices), a 4x4 block per
-//     lane transposed in registers, 16-byte traffic through an XOR-swizzled LDS tile in both
-//     directions, workgroup ids walking 8x8 super-tiles (transpose4_kernel);
+//   * 1-, 2-, 4- and 8-byte elements with every dimension and stride a multiple of a 16-byte vector
+//     (the benchmark case is 4-byte: 128 x 128 tiles of 1024 lanes, 64 x 128 of 256 lanes for
+//     small matrices): a V x V block per lane transposed in registers, 16-byte traffic through an
+//     XOR-swizzled LDS tile in both directions, workgroup ids walking 8x8 super-tiles
+//     (transpose_micro_kernel);
 //   * everything else: 64x64 tiles through a padded LDS tile (pitch 65 elements: both the
 //     scattered writes and the gathered reads hit 64 distinct banks), 16-byte global accesses
 //     where alignment allows, element-wise with bounds checks otherwise (transpose_kernel).
@@ -84,26 +85,32 @@ __global__ __launch_bounds__(kBlock) void transpose_kernel(const T* __restrict__
     }
 }
 
-// ---- 4-byte elements, every dimension a multiple of 4: 4x4 register micro-transpose ----------
-// A lane loads a 4(m) x 4(n) block as four 16-byte vectors along m, transposes it in registers,
-// and passes four 16-byte vectors along n through an LDS tile L[m][n] whose 16-byte slots are
-// XOR-swizzled with (m >> 2) so that both the writes (lanes differ in m) and the reads (lanes
-// differ in n) of a quarter-wave cover all 64 banks.  All LDS traffic is 128-bit.
+// ---- every dimension a multiple of a 16-byte vector: V x V register micro-transpose -----------
+// V = 16 / sizeof(T) elements fill a 16-byte vector (2, 4, 8 or 16).  A lane loads a V(m) x V(n) block
+// as V vectors along m, transposes it in registers, and passes V vectors along n through an LDS
+// tile L[m][n] whose 16-byte slots are XOR-swizzled with (m / V) so that both the writes (lanes
+// differ in m) and the reads (lanes differ in n) of a quarter-wave cover all 64 banks.  All LDS
+// traffic is 128-bit.
 // ORDER selects how workgroup ids walk the tile grid (the workgroups that run at the same
 // time decide how large the contiguous spans are that DRAM sees on each side).
 typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
 
-// NT lanes per workgroup.  Two shapes are used: 128 x 128 tiles with 1024 lanes (one 4x4 block per
-// lane) for large matrices -- runs of 512 bytes on both sides, which is what the memory system needs
-// to move a strided run at the rate of a linear copy, and two workgroups fill a CU -- and 64 x 128
-// tiles with 256 lanes (five workgroups per CU) when there are too few tiles for that.
-template <int TM, int TN, bool STREAM = true, int NT = 256>
-__global__ __launch_bounds__(NT) void transpose4_kernel(const unsigned* __restrict__ x, int64_t ldx,
-                                                         unsigned* __restrict__ y, int64_t ldy, int64_t m,
-                                                         int64_t n, int tiles_m, int tiles_n, int order) {
-    __shared__ __attribute__((aligned(16))) unsigned lds[TM * TN];
-    constexpr int MB = TM * TN / (16 * NT);   // 4x4 micro-blocks per lane
-    constexpr int SLOTS = TN / 4;             // 16-byte slots per LDS row
+// NT lanes per workgroup.  For 4-byte elements two shapes are used: 128 x 128 tiles with 1024 lanes
+// (one 4x4 block per lane) for large matrices -- runs of 512 bytes on both sides, which is what the
+// memory system needs to move a strided run at the rate of a linear copy, and two workgroups fill a
+// CU -- and 64 x 128 tiles with 256 lanes (five workgroups per CU) when there are too few tiles for
+// that.  The 2- and 8-byte shapes are chosen the same way (launch_micro).
+template <typename T, int TM, int TN, bool STREAM = true, int NT = 256>
+__global__ __launch_bounds__(NT) void transpose_micro_kernel(const T* __restrict__ x, int64_t ldx,
+                                                              T* __restrict__ y, int64_t ldy, int64_t m,
+                                                              int64_t n, int tiles_m, int tiles_n, int order) {
+    constexpr int V = 16 / sizeof(T);
+    using VT = typename VecOf<T, V>::type;
+    __shared__ __attribute__((aligned(16))) T lds[TM * TN];
+    constexpr int MB = TM * TN / (V * V * NT);   // V x V micro-blocks per lane
+    constexpr int SLOTS = TN / V;                // 16-byte slots per LDS row
+    static_assert(MB >= 1 && MB * V * V * NT == TM * TN, "the lanes must tile the block evenly");
+    static_assert(SLOTS >= 16 && (SLOTS & (SLOTS - 1)) == 0, "a quarter-wave must find 16 distinct slots");
     int bm, bn;
     {
         const int id = blockIdx.x;
@@ -120,38 +127,40 @@ __global__ __launch_bounds__(NT) void transpose4_kernel(const unsigned* __restri
     const int64_t m0 = (int64_t)bm * TM, n0 = (int64_t)bn * TN;
     // A tile that lies wholly inside the matrix is moved without predicates: a predicated load has
     // to be waited for before the other side of its branch may write the same registers, which
-    // would leave a lane with one load in flight instead of four.
+    // would leave a lane with one load in flight instead of V.
     const bool interior = m0 + TM <= m && n0 + TN <= n;
 #pragma unroll
     for (int k = 0; k < MB; ++k) {
         const int b = threadIdx.x + NT * k;
-        const int i4 = b % (TM / 4), j4 = b / (TM / 4);
-        const int64_t gm = m0 + 4 * i4, gn = n0 + 4 * j4;
-        u32x4 r[4] = {};
+        const int iv = b % (TM / V), jv = b / (TM / V);
+        const int64_t gm = m0 + V * iv, gn = n0 + V * jv;
+        VT r[V] = {};
         if (interior) {
 #pragma unroll
-            for (int c = 0; c < 4; ++c) r[c] = ld_global<STREAM>(reinterpret_cast<const u32x4*>(x + gm + (gn + c) * ldx));
+            for (int c = 0; c < V; ++c) r[c] = ld_global<STREAM>(reinterpret_cast<const VT*>(x + gm + (gn + c) * ldx));
         } else if (gm < m) {
 #pragma unroll
-            for (int c = 0; c < 4; ++c)
-                if (gn + c < n) r[c] = ld_global<STREAM>(reinterpret_cast<const u32x4*>(x + gm + (gn + c) * ldx));
+            for (int c = 0; c < V; ++c)
+                if (gn + c < n) r[c] = ld_global<STREAM>(reinterpret_cast<const VT*>(x + gm + (gn + c) * ldx));
         }
 #pragma unroll
-        for (int q = 0; q < 4; ++q) {
-            u32x4 t = {r[0][q], r[1][q], r[2][q], r[3][q]};  // x[m+q, n..n+3]
-            const int row = 4 * i4 + q;
-            *reinterpret_cast<u32x4*>(&lds[row * TN + 4 * (j4 ^ (i4 & (SLOTS - 1)))]) = t;
+        for (int q = 0; q < V; ++q) {
+            VT t;                                            // x[m+q, n..n+V-1]
+#pragma unroll
+            for (int c = 0; c < V; ++c) t[c] = r[c][q];
+            const int row = V * iv + q;
+            *reinterpret_cast<VT*>(&lds[row * TN + V * (jv ^ (iv & (SLOTS - 1)))]) = t;
         }
     }
     __syncthreads();
 #pragma unroll
-    for (int k = 0; k < 4 * MB; ++k) {
+    for (int k = 0; k < V * MB; ++k) {
         const int b = threadIdx.x + NT * k;
-        const int j4 = b % SLOTS, row = b / SLOTS;
-        const int64_t gn = n0 + 4 * j4, gm = m0 + row;
+        const int jv = b % SLOTS, row = b / SLOTS;
+        const int64_t gn = n0 + V * jv, gm = m0 + row;
         if (interior || (gn < n && gm < m)) {
-            u32x4 t = *reinterpret_cast<const u32x4*>(&lds[row * TN + 4 * (j4 ^ ((row >> 2) & (SLOTS - 1)))]);
-            st_global<true>(t, reinterpret_cast<u32x4*>(y + gn + gm * ldy));
+            VT t = *reinterpret_cast<const VT*>(&lds[row * TN + V * (jv ^ ((row / V) & (SLOTS - 1)))]);
+            st_global<true>(t, reinterpret_cast<VT*>(y + gn + gm * ldy));
         }
     }
 }
@@ -177,14 +186,14 @@ int launch4(const mi_tile_array* x, const mi_tile_array* y, hipStream_t s) {
     if (order == 2) blocks = ((tm_ + 7) / 8) * ((tn_ + 7) / 8) * 64;
     if (blocks > 0x7fffffffLL || tm_ > 0x3fffffff || tn_ > 0x3fffffff) return MI_E_GRID;
 #define T4(A, B)                                                                                          \
-    hipLaunchKernelGGL((transpose4_kernel<A, B>), dim3((unsigned)blocks), dim3(256), 0, s,                \
+    hipLaunchKernelGGL((transpose_micro_kernel<unsigned, A, B>), dim3((unsigned)blocks), dim3(256), 0, s,                \
                        (const unsigned*)x->ptr, x->strides[1], (unsigned*)y->ptr, y->strides[1], m, n,    \
                        (int)tm_, (int)tn_, order)
     if (tile == 9) {
         const bool st = stream_hint(2 * m * n * (int64_t)sizeof(unsigned));
-        if (st) hipLaunchKernelGGL((transpose4_kernel<128, 128, true, 1024>), dim3((unsigned)blocks), dim3(1024), 0, s,
+        if (st) hipLaunchKernelGGL((transpose_micro_kernel<unsigned, 128, 128, true, 1024>), dim3((unsigned)blocks), dim3(1024), 0, s,
                                    (const unsigned*)x->ptr, x->strides[1], (unsigned*)y->ptr, y->strides[1], m, n, (int)tm_, (int)tn_, order);
-        else hipLaunchKernelGGL((transpose4_kernel<128, 128, false, 1024>), dim3((unsigned)blocks), dim3(1024), 0, s,
+        else hipLaunchKernelGGL((transpose_micro_kernel<unsigned, 128, 128, false, 1024>), dim3((unsigned)blocks), dim3(1024), 0, s,
                                 (const unsigned*)x->ptr, x->strides[1], (unsigned*)y->ptr, y->strides[1], m, n, (int)tm_, (int)tn_, order);
         set_variant(st ? "transpose4_128x128_t1024_regmicro" : "transpose4_128x128_t1024_regmicro_cached");
     } else if (TM == 64 && TN == 64) { T4(64, 64); set_variant("transpose4_64x64_regmicro"); }
@@ -193,7 +202,7 @@ int launch4(const mi_tile_array* x, const mi_tile_array* y, hipStream_t s) {
     else if (TM == 64 && TN == 256) { T4(64, 256); set_variant("transpose4_64x256_regmicro"); }
     else if (TM == 32 && TN == 128) { T4(32, 128); set_variant("transpose4_32x128_regmicro"); }
     else if (TM == 64 && !stream_hint(2 * m * n * (int64_t)sizeof(unsigned))) {
-        hipLaunchKernelGGL((transpose4_kernel<64, 128, false>), dim3((unsigned)blocks), dim3(256), 0, s,
+        hipLaunchKernelGGL((transpose_micro_kernel<unsigned, 64, 128, false>), dim3((unsigned)blocks), dim3(256), 0, s,
                            (const unsigned*)x->ptr, x->strides[1], (unsigned*)y->ptr, y->strides[1], m, n,
                            (int)tm_, (int)tn_, order);
         set_variant("transpose4_64x128_regmicro_cached");
@@ -201,6 +210,68 @@ int launch4(const mi_tile_array* x, const mi_tile_array* y, hipStream_t s) {
     else { T4(128, 64); set_variant("transpose4_128x64_regmicro"); }
 #undef T4
     return launch_status();
+}
+
+// 2- and 8-byte elements through the same kernel.  `tile` picks the shape (MI_TRANSPOSE_TILE
+// overrides it for tuning): the large shapes keep runs of at least 512 bytes on both sides.
+template <typename T, int TM, int TN, int NT>
+int launch_micro_as(const mi_tile_array* x, const mi_tile_array* y, hipStream_t s, const char* name_stream,
+                    const char* name_cached) {
+    const int64_t m = x->sizes[0], n = x->sizes[1];
+    const int64_t tm_ = cld(m, (int64_t)TM), tn_ = cld(n, (int64_t)TN);
+    const int64_t blocks = ((tm_ + 7) / 8) * ((tn_ + 7) / 8) * 64;
+    if (blocks > 0x7fffffffLL || tm_ > 0x3fffffff || tn_ > 0x3fffffff) return MI_E_GRID;
+    const bool st = stream_hint(2 * m * n * (int64_t)sizeof(T));
+    if (st) hipLaunchKernelGGL((transpose_micro_kernel<T, TM, TN, true, NT>), dim3((unsigned)blocks), dim3(NT), 0, s,
+                               (const T*)x->ptr, x->strides[1], (T*)y->ptr, y->strides[1], m, n, (int)tm_, (int)tn_, 2);
+    else hipLaunchKernelGGL((transpose_micro_kernel<T, TM, TN, false, NT>), dim3((unsigned)blocks), dim3(NT), 0, s,
+                            (const T*)x->ptr, x->strides[1], (T*)y->ptr, y->strides[1], m, n, (int)tm_, (int)tn_, 2);
+    set_variant(st ? name_stream : name_cached);
+    return launch_status();
+}
+
+// measured on MI355X, 8192^2: 8-byte 205 us with 128 x 64 tiles of 1024 lanes (64 x 64 of 256 lanes 221 us; the
+// padded-tile kernel 305 us); 2-byte 51 us with 256 x 256 tiles of 1024 lanes (128 x 128 of 256 lanes 56 us; the
+// padded-tile kernel 67 us).  At 4096^2 the smaller tiles win, there are too few of the large ones to fill the chip.
+int launch8(const mi_tile_array* x, const mi_tile_array* y, hipStream_t s) {
+    const int64_t m = x->sizes[0], n = x->sizes[1];
+    const int64_t t64 = cld(m, (int64_t)64) * cld(n, (int64_t)64);
+    int tile = t64 >= 8192 ? 3 : t64 >= 1024 ? 2 : 0;
+    if (const char* e = getenv("MI_TRANSPOSE_TILE")) tile = atoi(e);
+    switch (tile) {
+        case 1: return launch_micro_as<uint64_t, 64, 128, 1024>(x, y, s, "transpose8_64x128_t1024_regmicro", "transpose8_64x128_t1024_regmicro_cached");
+        case 2: return launch_micro_as<uint64_t, 64, 64, 1024>(x, y, s, "transpose8_64x64_t1024_regmicro", "transpose8_64x64_t1024_regmicro_cached");
+        case 3: return launch_micro_as<uint64_t, 128, 64, 1024>(x, y, s, "transpose8_128x64_t1024_regmicro", "transpose8_128x64_t1024_regmicro_cached");
+        case 4: return launch_micro_as<uint64_t, 32, 128, 256>(x, y, s, "transpose8_32x128_regmicro", "transpose8_32x128_regmicro_cached");
+        default: return launch_micro_as<uint64_t, 64, 64, 256>(x, y, s, "transpose8_64x64_regmicro", "transpose8_64x64_regmicro_cached");
+    }
+}
+
+int launch2(const mi_tile_array* x, const mi_tile_array* y, hipStream_t s) {
+    const int64_t m = x->sizes[0], n = x->sizes[1];
+    const int64_t t128 = cld(m, (int64_t)128) * cld(n, (int64_t)128);
+    int tile = t128 >= 4096 ? 3 : t128 >= 1024 ? 2 : 0;
+    if (const char* e = getenv("MI_TRANSPOSE_TILE")) tile = atoi(e);
+    switch (tile) {
+        case 1: return launch_micro_as<uint16_t, 256, 128, 512>(x, y, s, "transpose2_256x128_t512_regmicro", "transpose2_256x128_t512_regmicro_cached");
+        case 2: return launch_micro_as<uint16_t, 128, 256, 512>(x, y, s, "transpose2_128x256_t512_regmicro", "transpose2_128x256_t512_regmicro_cached");
+        case 3: return launch_micro_as<uint16_t, 256, 256, 1024>(x, y, s, "transpose2_256x256_t1024_regmicro", "transpose2_256x256_t1024_regmicro_cached");
+        case 4: return launch_micro_as<uint16_t, 256, 128, 256>(x, y, s, "transpose2_256x128_regmicro", "transpose2_256x128_regmicro_cached");
+        default: return launch_micro_as<uint16_t, 128, 128, 256>(x, y, s, "transpose2_128x128_regmicro", "transpose2_128x128_regmicro_cached");
+    }
+}
+
+// 1-byte, measured: 16384^2 103 us with 256 x 512 tiles of 512 lanes (256 x 256 of 256 lanes 118 us); 8192^2 22 us
+// with 256 x 256 (24 us with 256 x 512; the padded-tile kernel 46 us)
+int launch1(const mi_tile_array* x, const mi_tile_array* y, hipStream_t s) {
+    const int64_t m = x->sizes[0], n = x->sizes[1];
+    int tile = cld(m, (int64_t)256) * cld(n, (int64_t)256) >= 4096 ? 2 : 0;
+    if (const char* e = getenv("MI_TRANSPOSE_TILE")) tile = atoi(e);
+    switch (tile) {
+        case 1: return launch_micro_as<uint8_t, 512, 256, 512>(x, y, s, "transpose1_512x256_t512_regmicro", "transpose1_512x256_t512_regmicro_cached");
+        case 2: return launch_micro_as<uint8_t, 256, 512, 512>(x, y, s, "transpose1_256x512_t512_regmicro", "transpose1_256x512_t512_regmicro_cached");
+        default: return launch_micro_as<uint8_t, 256, 256, 256>(x, y, s, "transpose1_256x256_regmicro", "transpose1_256x256_regmicro_cached");
+    }
 }
 
 template <typename T>
@@ -241,15 +312,16 @@ extern "C" int mi_transpose_kernel(const mi_tile_array* x, const mi_tile_array* 
     if ((m > 1 && x->strides[0] != 1) || (n > 1 && y->strides[0] != 1)) return MI_E_STRIDE;
     if ((n > 1 && x->strides[1] < m) || (m > 1 && y->strides[1] < n)) return MI_E_STRIDE;
     hipStream_t s = (hipStream_t)stream;
+    // the register micro-transpose moves whole 16-byte vectors of v elements on both sides
+    auto micro = [&](int v) {
+        return m % v == 0 && n % v == 0 && x->strides[1] % v == 0 && y->strides[1] % v == 0 &&
+               aligned(x->ptr, 16) && aligned(y->ptr, 16);
+    };
     switch (dtype_size(x->dtype)) {
-        case 1: return launch<uint8_t>(x, y, s);
-        case 2: return launch<uint16_t>(x, y, s);
-        case 4:
-            if (m % 4 == 0 && n % 4 == 0 && x->strides[1] % 4 == 0 && y->strides[1] % 4 == 0 && aligned(x->ptr, 16) &&
-                aligned(y->ptr, 16))
-                return launch4(x, y, s);
-            return launch<uint32_t>(x, y, s);
-        case 8: return launch<uint64_t>(x, y, s);
+        case 1: return micro(16) ? launch1(x, y, s) : launch<uint8_t>(x, y, s);
+        case 2: return micro(8) ? launch2(x, y, s) : launch<uint16_t>(x, y, s);
+        case 4: return micro(4) ? launch4(x, y, s) : launch<uint32_t>(x, y, s);
+        case 8: return micro(2) ? launch8(x, y, s) : launch<uint64_t>(x, y, s);
         default: return MI_E_DTYPE;
     }
 }

@@ -124,6 +124,37 @@ def test_transpose_padded_leading_dimension(ct):
     assert torch.equal(y, x.T) and torch.all(ybig[:, 40:] == -1.0)
 
 
+@pytest.mark.parametrize("T,isz", [(torch.float8_e4m3fn, 1), (torch.float16, 2), (torch.bfloat16, 2),
+                                   (torch.float32, 4), (torch.float64, 8), (torch.int64, 8)])
+def test_transpose_every_element_size_takes_the_register_path(ct, T, isz):
+    """Random bit patterns (NaN payloads and denormals included) of 1-, 2-, 4- and 8-byte elements
+    through the 16-byte path: whole tiles, ragged edges, skinny matrices, a matrix large enough for
+    the big tiles, and padded leading dimensions on both sides with the padding left untouched."""
+    v = 16 // isz
+    iv = {1: torch.uint8, 2: torch.int16, 4: torch.int32, 8: torch.int64}[isz]
+    g = torch.Generator(device="cuda"); g.manual_seed(100 + isz)
+
+    def bits(r, c):
+        return torch.randint(0, 256, (r, c * isz), device="cuda", generator=g).to(torch.uint8).view(iv)
+
+    for r, c in [(v, v), (8 * v, 24 * v), (256, 512), (1008 // v * v, 528), (2064, 1040), (v, 4096), (4096, v),
+                 (8192, 2048 * v)]:
+        x = bits(r, c)
+        y = torch.zeros(c, r, dtype=iv, device="cuda")
+        ct.transpose_kernel(x.view(T), y.view(T), 64, 64)
+        assert "regmicro" in ct.last_variant(), ct.last_variant()
+        assert torch.equal(y, x.t()), (r, c)
+        xb = bits(r, c + 2 * v); x2 = xb[:, v:v + c]
+        yb = torch.full((c, r + v), 85, dtype=iv, device="cuda"); y2 = yb[:, :r]
+        ct.transpose_kernel(x2.view(T), y2.view(T), 32, 32)
+        assert "regmicro" in ct.last_variant(), ct.last_variant()
+        assert torch.equal(y2, x2.t()) and bool((yb[:, r:] == 85).all()), (r, c)
+    # one element short of a whole vector on either side: the element-wise kernel
+    x = bits(3 * v + 1, 5 * v); y = torch.zeros(5 * v, 3 * v + 1, dtype=iv, device="cuda")
+    ct.transpose_kernel(x.view(T), y.view(T), 64, 64)
+    assert "regmicro" not in ct.last_variant() and torch.equal(y, x.t())
+
+
 def test_transpose_full_size_involution():
     d = transpose.prepare(benchmark=True)
     r = transpose.run(d)

@@ -5,7 +5,7 @@ import numpy as np
 import torch
 
 import cutile_jl_amd as ct
-from ._harness import isapprox, namespace, time_launches, upload
+from ._harness import namespace, time_launches, upload
 
 
 def dft_matrix(size: int) -> np.ndarray:

@@ -83,7 +83,14 @@ __device__ __forceinline__ float xhalf_sum(float v) {
     return __uint_as_float(r[0]) + __uint_as_float(r[1]);
 }
 
-struct Lane {
+// RG: the sequence length is not a multiple of 128 (causal only).  The grid is that of the next multiple; the halves
+// that exist are walked as usual, the last of them re-reads its last row in place of the rows past the end (ragged_offsets),
+// halves past it are never requested (the transfers that would fetch them re-send the last one, as at the end of
+// every walk), and rows past the end are not stored.  Keys past the end lie above the diagonal of every query that
+// exists, so the causal mask removes them.
+template <bool RG>
+struct LaneT {
+    static constexpr bool ragged = RG;
     // wave-uniform
     const char *kptr, *vptr;        // next K / V half to be transferred
     int k_left, v_left;             // halves not yet transferred (the last one is re-sent once they run out)
@@ -97,7 +104,22 @@ struct Lane {
     unsigned vfo[2];                // V fragment element offsets inside a slot, per d tile
     int lim0;                       // (lane % 32) - 4 * (lane / 32)
     int q0[2];                      // first query of each stream (wave-uniform)
+    // RG only
+    bool to_end;                    // (wave-uniform) the walk reaches the last half that exists
+    unsigned kdma_b, vdma_b;        // offset of the lane's 16 bytes in transfer wave+2, relative to the start of the half
+    unsigned k_rg[2], v_rg[2];      // the two offsets for the last half that exists (rows past the end re-read the last row)
 };
+
+// Lane offsets of the two transfers of the last half when rows past `last_row` (0..31) are replaced by that row.
+template <bool IS_V>
+__device__ __forceinline__ void ragged_offsets(int wave, int lane, int last_row, int64_t half_bytes, unsigned& o0, unsigned& o1) {
+    const int key = 8 * wave + (lane >> 3), pos = lane & 7;
+    const unsigned pitch = (unsigned)(half_bytes >> 5);   // bytes per key row
+    const unsigned sw = 16u * (unsigned)(IS_V ? (pos ^ (2 * (key & 3))) : (pos ^ ((key >> 1) & 7)));
+    const int r0 = key < last_row ? key : last_row, r1 = key + 16 < last_row ? key + 16 : last_row;
+    o0 = (unsigned)r0 * pitch + sw;
+    o1 = (unsigned)r1 * pitch + sw;
+}
 
 
 template <typename E>
@@ -115,46 +137,68 @@ struct Acc {
 
 // Transfers the next K (V) half into ring slot `slot`.  Past the last half the same half is sent
 // again into a slot nobody reads, which keeps the count of outstanding transfers uniform.
-__device__ __forceinline__ void issue_k(Lane& c, int slot) {
+// (RG: the selects are wave-uniform conditions on lane offsets -- no branch, the steps keep their layout)
+template <bool RG>
+__device__ __forceinline__ void issue_k(LaneT<RG>& c, int slot) {
     const unsigned lds = c.ks_base + slot * kSlotBytes + c.wave * 1024;
-    dma16(c.kdma, c.kptr, lds);
-    dma16(c.kdma, c.kptr + (c.k_half_bytes >> 1), lds + 2048);
+    if constexpr (RG) {
+        const bool last = c.to_end && c.k_left <= 1;
+        dma16(last ? c.k_rg[0] : c.kdma, c.kptr, lds);
+        dma16(last ? c.k_rg[1] : c.kdma_b, c.kptr, lds + 2048);
+    } else {
+        dma16(c.kdma, c.kptr, lds);
+        dma16(c.kdma, c.kptr + (c.k_half_bytes >> 1), lds + 2048);
+    }
     c.k_left -= 1;
     if (c.k_left > 0) c.kptr += c.k_half_bytes;
 }
-__device__ __forceinline__ void issue_v(Lane& c, int slot) {
+template <bool RG>
+__device__ __forceinline__ void issue_v(LaneT<RG>& c, int slot) {
     const unsigned lds = c.vs_base + slot * kSlotBytes + c.wave * 1024;
-    dma16(c.vdma, c.vptr, lds);
-    dma16(c.vdma, c.vptr + (c.v_half_bytes >> 1), lds + 2048);
+    if constexpr (RG) {
+        const bool last = c.to_end && c.v_left <= 1;
+        dma16(last ? c.v_rg[0] : c.vdma, c.vptr, lds);
+        dma16(last ? c.v_rg[1] : c.vdma_b, c.vptr, lds + 2048);
+    } else {
+        dma16(c.vdma, c.vptr, lds);
+        dma16(c.vdma, c.vptr + (c.v_half_bytes >> 1), lds + 2048);
+    }
     c.v_left -= 1;
     if (c.v_left > 0) c.vptr += c.v_half_bytes;
 }
 
 // The same transfers one at a time (PART 0 / 1 of a half), for steps that spread them over their issue slots.
-template <int PART>
-__device__ __forceinline__ void issue_k_part(Lane& c, int slot) {
+template <int PART, bool RG>
+__device__ __forceinline__ void issue_k_part(LaneT<RG>& c, int slot) {
     const unsigned lds = c.ks_base + slot * kSlotBytes + c.wave * 1024;
+    const bool last = RG && c.to_end && c.k_left <= 1;
     if (PART == 0) {
-        dma16(c.kdma, c.kptr, lds);
+        if constexpr (RG) dma16(last ? c.k_rg[0] : c.kdma, c.kptr, lds);
+        else dma16(c.kdma, c.kptr, lds);
     } else {
-        dma16(c.kdma, c.kptr + (c.k_half_bytes >> 1), lds + 2048);
+        if constexpr (RG) dma16(last ? c.k_rg[1] : c.kdma_b, c.kptr, lds + 2048);
+        else dma16(c.kdma, c.kptr + (c.k_half_bytes >> 1), lds + 2048);
         c.k_left -= 1;
         if (c.k_left > 0) c.kptr += c.k_half_bytes;
     }
 }
-template <int PART>
-__device__ __forceinline__ void issue_v_part(Lane& c, int slot) {
+template <int PART, bool RG>
+__device__ __forceinline__ void issue_v_part(LaneT<RG>& c, int slot) {
     const unsigned lds = c.vs_base + slot * kSlotBytes + c.wave * 1024;
+    const bool last = RG && c.to_end && c.v_left <= 1;
     if (PART == 0) {
-        dma16(c.vdma, c.vptr, lds);
+        if constexpr (RG) dma16(last ? c.v_rg[0] : c.vdma, c.vptr, lds);
+        else dma16(c.vdma, c.vptr, lds);
     } else {
-        dma16(c.vdma, c.vptr + (c.v_half_bytes >> 1), lds + 2048);
+        if constexpr (RG) dma16(last ? c.v_rg[1] : c.vdma_b, c.vptr, lds + 2048);
+        else dma16(c.vdma, c.vptr + (c.v_half_bytes >> 1), lds + 2048);
         c.v_left -= 1;
         if (c.v_left > 0) c.vptr += c.v_half_bytes;
     }
 }
 
-__device__ __forceinline__ void read_k_frags(const unsigned short* Ks, const Lane& c, int slot, s16x8 (&kf)[4]) {
+template <bool RG>
+__device__ __forceinline__ void read_k_frags(const unsigned short* Ks, const LaneT<RG>& c, int slot, s16x8 (&kf)[4]) {
 #pragma unroll
     for (int ks = 0; ks < 4; ++ks) kf[ks] = *reinterpret_cast<const s16x8*>(Ks + slot * kSlot + c.kfo[ks]);
 }
@@ -234,8 +278,8 @@ constexpr int nth_stream(int m, int k) { return (m & 1) ? k : 1; }
 //      pack, row sum: about the time one MFMA takes);
 //   B: the remaining P.V MFMAs, each followed by the row maxima of one stream of S(j+1).
 // The K(j+2) fragments are read as soon as the last S MFMA has been issued.
-template <typename E, int CUR, int NEXT, int MASKN>
-__device__ __forceinline__ void half_step(const unsigned short* Ks, const unsigned short* Vs, Lane& c, Acc<E>& a,
+template <typename E, int CUR, int NEXT, int MASKN, bool RG>
+__device__ __forceinline__ void half_step(const unsigned short* Ks, const unsigned short* Vs, LaneT<RG>& c, Acc<E>& a,
                                           int j, f32x16 (&s_cur)[2], f32x16 (&s_next)[2], s16x8 (&kf)[4],
                                           float (&cand)[2]) {
     constexpr int nC = popcount2(CUR), nN = popcount2(NEXT);
@@ -399,8 +443,8 @@ __device__ __forceinline__ void half_step(const unsigned short* Ks, const unsign
 // Ring: a trip waits for everything requested one trip ago (K(j+4), K(j+5), V(j), V(j+1)), then requests
 // K(j+6), K(j+7) into the slots whose fragments are in registers and V(j+2), V(j+3) into the slots read one trip
 // ago (V(j+2) not in the first wide trip: the narrow steps had requested it already).
-template <typename E, bool NEXT, bool MASK>
-__device__ __forceinline__ void wide_step(const unsigned short* Ks, const unsigned short* Vs, Lane& c, Acc<E>& a,
+template <typename E, bool NEXT, bool MASK, bool RG>
+__device__ __forceinline__ void wide_step(const unsigned short* Ks, const unsigned short* Vs, LaneT<RG>& c, Acc<E>& a,
                                           int j, bool first, f32x16& c0, f32x16& c1, f32x16& n0, f32x16& n1,
                                           s16x8 (&kf)[2][4], float (&cand)[2]) {
     constexpr int nQ = NEXT ? 10 : 0;   // S MFMAs, k-step major over the two halves; "k step" 0 places -m
@@ -551,7 +595,7 @@ struct Magic {
     static unsigned of(int d) { return d <= 1 ? 0u : (unsigned)((1ull << 32) / (unsigned)d) + 1u; }
 };
 
-template <typename E, bool CAUSAL>
+template <typename E, bool CAUSAL, bool RG = false>
 __global__ __launch_bounds__(128) __attribute__((amdgpu_waves_per_eu(2, 2))) void fmha_pipe_kernel(
     const unsigned short* __restrict__ Q, Strides qs, const unsigned short* __restrict__ K, Strides ks,
     const unsigned short* __restrict__ V, Strides vs, unsigned short* __restrict__ O, Strides os, int S, int H,
@@ -585,7 +629,8 @@ __global__ __launch_bounds__(128) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     Q += (int64_t)head * qs.s2 + (int64_t)batch * qs.s3;
     O += (int64_t)head * os.s2 + (int64_t)batch * os.s3;
 
-    const int NT = S / 32;
+    static_assert(CAUSAL || !RG, "keys past the end are only masked by the causal mask");
+    const int NT = 4 * nqb;   // 32-query tiles of the grid (RG: of the sequence rounded up to whole workgroups)
     int tq[2];
     if (CAUSAL) {
         tq[0] = 2 * qb + wave;
@@ -595,7 +640,7 @@ __global__ __launch_bounds__(128) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
         tq[1] = tq[0] + 1;
     }
 
-    Lane c;
+    LaneT<RG> c;
     c.kptr = (const char*)(K + (int64_t)kvh * ks.s2 + (int64_t)batch * ks.s3);
     c.vptr = (const char*)(V + (int64_t)kvh * vs.s2 + (int64_t)batch * vs.s3);
     c.k_half_bytes = (int64_t)kHK * ks.s1 * 2;
@@ -609,6 +654,14 @@ __global__ __launch_bounds__(128) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     if (blockIdx.x >= (gridDim.x >> 1)) __builtin_amdgcn_s_setprio(1);
     c.nh = CAUSAL ? NT - 2 * qb : NT;
     c.k_left = c.v_left = c.nh;
+    c.to_end = false;
+    int last_row = kHK - 1;
+    if constexpr (RG) {
+        const int vh = (S + kHK - 1) / kHK;   // halves that exist
+        c.to_end = c.nh >= vh;
+        if (c.to_end) c.k_left = c.v_left = vh;
+        last_row = S - 1 - kHK * (vh - 1);
+    }
     c.hb0 = hb == 0;
     {
         // transfer `wave` of a half covers keys 8*wave .. 8*wave+7; transfer wave+2 the keys 16 further on,
@@ -618,6 +671,12 @@ __global__ __launch_bounds__(128) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
         const int key = 8 * wave + (lane >> 3), pos = lane & 7;
         c.kdma = (unsigned)(((int64_t)key * ks.s1 + 8 * (pos ^ ((key >> 1) & 7))) * 2);
         c.vdma = (unsigned)(((int64_t)key * vs.s1 + 8 * (pos ^ (2 * (key & 3)))) * 2);
+        if constexpr (RG) {
+            c.kdma_b = c.kdma + (unsigned)(c.k_half_bytes >> 1);
+            c.vdma_b = c.vdma + (unsigned)(c.v_half_bytes >> 1);
+            ragged_offsets<false>(wave, lane, last_row, c.k_half_bytes, c.k_rg[0], c.k_rg[1]);
+            ragged_offsets<true>(wave, lane, last_row, c.v_half_bytes, c.v_rg[0], c.v_rg[1]);
+        }
     }
     c.lim0 = (lane & 31) - 4 * hb;
     c.q0[0] = 32 * tq[0];
@@ -647,7 +706,8 @@ __global__ __launch_bounds__(128) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
         my_q[jj] = 32 * tq[jj] + (lane & 31);
 #pragma unroll
         for (int s = 0; s < 4; ++s) {
-            const unsigned short* qp = Q + (int64_t)my_q[jj] * qs.s1 + 16 * s + 8 * hb;
+            const int row = RG && my_q[jj] >= S ? S - 1 : my_q[jj];   // (queries past the end: any row, never stored)
+            const unsigned short* qp = Q + (int64_t)row * qs.s1 + 16 * s + 8 * hb;
             asm volatile("global_load_dwordx4 %0, %1, off" : "=v"(qraw[jj][s]) : "v"(qp) : "memory");
         }
     }
@@ -706,6 +766,7 @@ __global__ __launch_bounds__(128) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     // Epilogue of one stream: add the two half-row sums, O / l (approximate reciprocal), round, store.
     auto store_tile = [&](int jj, float lsum) {
         const float inv = __builtin_amdgcn_rcpf(xhalf_sum(lsum));
+        if (RG && my_q[jj] >= S) return;
         unsigned short* op = O + (int64_t)my_q[jj] * os.s1;
 #pragma unroll
         for (int dt = 0; dt < 2; ++dt)
@@ -802,12 +863,16 @@ void launch_e(const Problem& p, hipStream_t stream) {
     Strides qs{Q->strides[1], Q->strides[2], Q->strides[3]}, ks{K->strides[1], K->strides[2], K->strides[3]},
         vs{V->strides[1], V->strides[2], V->strides[3]}, os{O->strides[1], O->strides[2], O->strides[3]};
     const int S = (int)Q->sizes[1];
-    const int nqb = S / 128, nbh = (int)(Q->sizes[2] * Q->sizes[3]);
+    const int nqb = (S + 127) / 128, nbh = (int)(Q->sizes[2] * Q->sizes[3]);
     dim3 grid((unsigned)(nqb * nbh)), blk(128);
     Magic mg{Magic::of(nqb), Magic::of(p.H), Magic::of(p.group), 0};
     const int64_t dmax = nqb > p.H ? nqb : p.H;
     mg.fast = (int64_t)grid.x * (dmax > p.group ? dmax : p.group) < (1ll << 32) ? 1 : 0;
-    if (p.causal)
+    if (p.causal && S % 128 != 0)
+        hipLaunchKernelGGL((fmha_pipe_kernel<E, true, true>), grid, blk, 0, stream, (const unsigned short*)Q->ptr, qs,
+                           (const unsigned short*)K->ptr, ks, (const unsigned short*)V->ptr, vs, (unsigned short*)O->ptr,
+                           os, S, p.H, p.group, p.scale2, nqb, nbh, mg);
+    else if (p.causal)
         hipLaunchKernelGGL((fmha_pipe_kernel<E, true>), grid, blk, 0, stream, (const unsigned short*)Q->ptr, qs,
                            (const unsigned short*)K->ptr, ks, (const unsigned short*)V->ptr, vs, (unsigned short*)O->ptr,
                            os, S, p.H, p.group, p.scale2, nqb, nbh, mg);
@@ -823,19 +888,20 @@ bool pipe_applicable(const Problem& p) {
     const mi_tile_array *Q = p.Q, *K = p.K, *V = p.V, *O = p.O;
     if (Q->sizes[0] != kD || V->sizes[0] != kD) return false;
     const int64_t S = Q->sizes[1];
-    if (K->sizes[1] != S || S % 128 != 0 || S < 128) return false;
+    if (K->sizes[1] != S || S < 128) return false;
+    if (S % 128 != 0 && !p.causal) return false;   // (a ragged tail needs a key mask of its own without the causal one)
     if (!(p.scale2 > 0.f)) return false;
     if (p.causal && p.input_pos != 0) return false;
     if (!vec16(Q) || !vec16(K) || !vec16(V) || !vec16(O)) return false;
     if (K->strides[1] >= (1 << 20) || V->strides[1] >= (1 << 20)) return false;
-    if (Q->sizes[2] * Q->sizes[3] * (S / 128) > 0x7fffffff) return false;
+    if (Q->sizes[2] * Q->sizes[3] * ((S + 127) / 128) > 0x7fffffff) return false;
     return true;
 }
 
 void pipe_launch(const Problem& p, hipStream_t stream) {
     if (p.bf16) launch_e<BF16>(p, stream);
     else launch_e<F16>(p, stream);
-    set_variant("fmha_pipe_d64_q128_kv32_ring4");
+    set_variant(p.Q->sizes[1] % 128 ? "fmha_pipe_d64_q128_kv32_ring4_ragged" : "fmha_pipe_d64_q128_kv32_ring4");
 }
 
 }  // namespace fmha

@@ -122,6 +122,36 @@ def test_fmha_pipelined_kernel_shapes(ct, orc, batch, heads, s, causal, qg, T):
     check(orc, r.out, ref, 2e-2 if T == torch.float16 else 3e-2)
 
 
+@pytest.mark.parametrize("batch,heads,s,qg,T", [
+    (1, 8, 129, 1, torch.float16), (2, 3, 160, 1, torch.float16), (1, 8, 191, 4, torch.bfloat16), (1, 2, 193, 1, torch.float16),
+    (1, 4, 255, 2, torch.float16), (1, 8, 257, 1, torch.bfloat16), (1, 2, 333, 1, torch.float16), (1, 16, 500, 1, torch.float16),
+    (2, 8, 647, 2, torch.float16), (1, 2, 1000, 1, torch.float16), (1, 1, 1023, 1, torch.bfloat16), (1, 2, 1025, 1, torch.float16),
+])
+def test_fmha_pipelined_kernel_ragged_causal(ct, orc, batch, heads, s, qg, T):
+    """Causal attention over a sequence that is not a multiple of 128 runs on the pipelined kernel as well: the last
+    key half that exists is partial (its missing rows re-read the last row and fall to the causal mask), halves past
+    it are never fetched, query rows past the end are not stored.  Lengths one past / one short of a half, of a
+    workgroup's 128 queries and of a pair of them; the output sits in a wider buffer whose rows past the end must
+    stay as they were."""
+    data = fmha.prepare(batch=batch, heads=heads, seq_q=s, seq_kv=s, query_group_size=qg, causal=True, T=T)
+    big = torch.full((batch, heads, s + 40, 64), 777.0, dtype=T, device="cuda")
+    out = big[:, :, :s, :]
+    out.fill_(float("nan"))
+    fmha.cutile_fmha(data.Q, data.K, data.V, query_group_size=qg, causal=True, out=out)
+    assert ct.last_variant() == "fmha_pipe_d64_q128_kv32_ring4_ragged"
+    assert bool((big[:, :, s:, :] == 777.0).all())
+    ref = orc.ref_fmha(*(orc.to_julia(t) for t in (data.Q, data.K, data.V)), causal=True, dtype=np.float64)
+    check(orc, out, ref, 2e-2 if T == torch.float16 else 3e-2)
+
+
+def test_fmha_ragged_without_the_causal_mask_takes_the_general_kernel(ct, orc):
+    data = fmha.prepare(batch=1, heads=2, seq_q=200, seq_kv=200, causal=False)
+    r = run(data)
+    assert ct.last_variant().startswith("fmha_dma") or ct.last_variant().startswith("fmha_regstage")
+    ref = orc.ref_fmha(*(orc.to_julia(t) for t in (data.Q, data.K, data.V)), causal=False, dtype=np.float64)
+    check(orc, r.out, ref)
+
+
 @pytest.mark.parametrize("causal", [True, False])
 def test_fmha_pipelined_kernel_strided_views(ct, orc, causal):
     """Q/K/V as views of one packed (B, S, 3, H, D) buffer and Out as a view of a wider buffer: row,

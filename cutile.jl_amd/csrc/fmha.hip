@@ -28,16 +28,28 @@
 // tiles that lie wholly above its own last query.  Masking and the ragged KV tail use -Inf
 // as in the reference (fmha.jl:92-103).
 //
+// Few queries against many keys (decode, chunked prefill): B * H * cld(Sq, 128) workgroups leave most of the chip
+// idle and each walks the whole KV range alone.  The KV tiles of a workgroup are then dealt to `nsplit` workgroups
+// (SPLIT instantiation); each leaves its unnormalised accumulator, running maximum and row sum in a scratch array of
+// the library, and fmha_combine_kernel adds the parts with the usual exp2(m_part - m) weights.  A part may start
+// above a query's diagonal, so a row can go through tiles without a visible key: its maximum stays -Inf and the
+// weights are taken against 0 instead (SAFE), which keeps them at exp2(-Inf) = 0 rather than exp2(-Inf + Inf).
+//
 // FLOPs (causal-exact): 4 * B * H * D * Sq*(Sq+1)/2 for Sq == Skv.
 #include "fmha_common.h"
 #include <stdlib.h>
 #include <string.h>
+
+#include <mutex>
 
 namespace {
 
 using namespace mi;
 using namespace mi::fmha;
 
+
+typedef float f32x2 __attribute__((ext_vector_type(2)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
 
 constexpr int kQB = 128;  // queries per workgroup
 constexpr int kKV = 64;   // keys per LDS tile
@@ -286,7 +298,7 @@ struct FmhaDma {
 
     // JM: bit j set = column tile j takes part in this KV tile (a causal wave drops its early
     // query tile once the keys pass that tile's diagonal).
-    template <int JM>
+    template <int JM, bool SAFE = false>
     static __device__ __forceinline__ void compute(const unsigned short* Ks, const unsigned short* Vs, State& st,
                                                    int kv0, int Skv, float scale2, int lane) {
         const int hb = lane >> 5;
@@ -332,7 +344,8 @@ struct FmhaDma {
             mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
             const float m_new = fmaxf(st.m[j], mx * scale2);
             if (__any(m_new > st.m[j])) {  // some row's max rose: rescale the wave's accumulators
-                const float alpha = __builtin_amdgcn_exp2f(st.m[j] - m_new);
+                // (SAFE: a row that has not seen a key yet keeps l = 0 and o = 0)
+                const float alpha = __builtin_amdgcn_exp2f(st.m[j] - (SAFE && m_new == -INFINITY ? 0.f : m_new));
                 st.l[j] *= alpha;
 #pragma unroll
                 for (int dt = 0; dt < DT; ++dt)
@@ -340,7 +353,7 @@ struct FmhaDma {
                     for (int r = 0; r < 16; ++r) st.o[j][dt][r] *= alpha;
                 st.m[j] = m_new;
             }
-            const float mj = st.m[j];
+            const float mj = SAFE && st.m[j] == -INFINITY ? 0.f : st.m[j];
             float lsum = st.l[j];
 #pragma unroll
             for (int kt = 0; kt < 2; ++kt)
@@ -389,11 +402,13 @@ __device__ __forceinline__ void tile_barrier() {
 // tile grows with its index, so a wave takes one early and one late tile, u and NT-1-u with
 // u = 2*qb + w; every wave then has the same number of MFMAs, and the two waves of a workgroup
 // need the same KV range.  The early tile simply drops out of the KV loop after its diagonal.
-template <typename E, int D, int JT, bool CAUSAL>
+constexpr int kPartPad = 4;   // a part's row: D accumulator values, running maximum, row sum, two unused (16-byte rows)
+
+template <typename E, int D, int JT, bool CAUSAL, bool SPLIT = false>
 __global__ __launch_bounds__(128 * 2 / JT) __attribute__((amdgpu_waves_per_eu(2, 2))) void fmha_fwd_dma_kernel(
     const unsigned short* __restrict__ Q, Strides qs, const unsigned short* __restrict__ K, Strides ks,
     const unsigned short* __restrict__ V, Strides vs, unsigned short* __restrict__ O, Strides os, int Sq, int Skv,
-    int H, int group, float scale2, int input_pos, int nqb, int nbh) {
+    int H, int group, float scale2, int input_pos, int nqb, int nbh, int nsplit = 1, float* __restrict__ part = nullptr) {
     using F = FmhaDma<E, D, JT, CAUSAL>;
     constexpr int NW = F::NW, KSTEPS = F::KSTEPS, DT = F::DT, CH = F::CH, TPW = F::TPW;
     constexpr bool PAIRED = CAUSAL && JT == 2;
@@ -403,9 +418,13 @@ __global__ __launch_bounds__(128 * 2 / JT) __attribute__((amdgpu_waves_per_eu(2,
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     // Workgroup -> (query block, batch*head): ids congruent mod 8 share an XCD; give each XCD
     // whole (batch, head) pairs so their K/V stay in that XCD's L2.  Low block index = most work.
-    int qb, bh;
+    int qb, bh, sp = 0;
     {
-        const int L = blockIdx.x;
+        int L = blockIdx.x;
+        if (SPLIT) {   // the parts of one (query block, batch * head) are nqb * nbh workgroup ids apart
+            sp = L / (nqb * nbh);
+            L -= sp * (nqb * nbh);
+        }
         if (nbh % 8 == 0) {
             const int idx = L >> 3;
             bh = (L & 7) + 8 * (idx / nqb);
@@ -418,7 +437,7 @@ __global__ __launch_bounds__(128 * 2 / JT) __attribute__((amdgpu_waves_per_eu(2,
     }
     const int batch = bh / H, head = bh % H, kvh = head / group;
     Q += (int64_t)head * qs.s2 + (int64_t)batch * qs.s3;
-    O += (int64_t)head * os.s2 + (int64_t)batch * os.s3;
+    if (!SPLIT) O += (int64_t)head * os.s2 + (int64_t)batch * os.s3;
     const char* Kg = (const char*)(K + (int64_t)kvh * ks.s2 + (int64_t)batch * ks.s3);
     const char* Vg = (const char*)(V + (int64_t)kvh * vs.s2 + (int64_t)batch * vs.s3);
 
@@ -488,6 +507,11 @@ __global__ __launch_bounds__(128 * 2 / JT) __attribute__((amdgpu_waves_per_eu(2,
         if (kv_end < 0) kv_end = 0;
     }
     const int ntiles = (kv_end + kKV - 1) / kKV;
+    int t_begin = 0, t_end = ntiles;
+    if (SPLIT) {
+        t_begin = (int)((int64_t)ntiles * sp / nsplit);
+        t_end = (int)((int64_t)ntiles * (sp + 1) / nsplit);
+    }
     const int64_t k_tile_bytes = (int64_t)kKV * ks.s1 * 2, v_tile_bytes = (int64_t)kKV * vs.s1 * 2;
 
     // Rows past the end of K / V in the last tile are never dereferenced: their lanes re-read
@@ -515,24 +539,46 @@ __global__ __launch_bounds__(128 * 2 / JT) __attribute__((amdgpu_waves_per_eu(2,
         if (JT == 2) {
             const bool a0 = tq[0] >= 0 && (!CAUSAL || kv0 <= last_pos[0]);
             const bool a1 = tq[JT - 1] >= 0 && (!CAUSAL || kv0 <= last_pos[JT - 1]);
-            if (a0 && a1) F::template compute<3>(Ksx, Vsx, st, kv0, Skv, scale2, lane);
-            else if (a1) F::template compute<2>(Ksx, Vsx, st, kv0, Skv, scale2, lane);
-            else if (a0) F::template compute<1>(Ksx, Vsx, st, kv0, Skv, scale2, lane);
+            if (a0 && a1) F::template compute<3, SPLIT>(Ksx, Vsx, st, kv0, Skv, scale2, lane);
+            else if (a1) F::template compute<2, SPLIT>(Ksx, Vsx, st, kv0, Skv, scale2, lane);
+            else if (a0) F::template compute<1, SPLIT>(Ksx, Vsx, st, kv0, Skv, scale2, lane);
         } else {
-            if (tq[0] >= 0 && (!CAUSAL || kv0 <= last_pos[0])) F::template compute<1>(Ksx, Vsx, st, kv0, Skv, scale2, lane);
+            if (tq[0] >= 0 && (!CAUSAL || kv0 <= last_pos[0])) F::template compute<1, SPLIT>(Ksx, Vsx, st, kv0, Skv, scale2, lane);
         }
     };
 
-    if (ntiles > 0) issue_tile(0, Ks0, Vs0);
-    for (int t = 0; t < ntiles; t += 2) {
+    if (t_begin < t_end) issue_tile(t_begin, Ks0, Vs0);
+    for (int t = t_begin; t < t_end; t += 2) {
         tile_barrier();  // tile t has landed for every wave; every wave is done with the other stage
-        if (t + 1 < ntiles) issue_tile(t + 1, Ks1, Vs1);
+        if (t + 1 < t_end) issue_tile(t + 1, Ks1, Vs1);
         run_tile(Ks0, Vs0, t * kKV);
-        if (t + 1 < ntiles) {
+        if (t + 1 < t_end) {
             tile_barrier();
-            if (t + 2 < ntiles) issue_tile(t + 2, Ks0, Vs0);
+            if (t + 2 < t_end) issue_tile(t + 2, Ks0, Vs0);
             run_tile(Ks1, Vs1, (t + 1) * kKV);
         }
+    }
+
+    if constexpr (SPLIT) {
+        // ---- this part's unnormalised accumulator, maximum and row sum -> scratch ---------------
+#pragma unroll
+        for (int j = 0; j < JT; ++j) {
+            const float l_tot = st.l[j] + __shfl_xor(st.l[j], 32, 64);
+            if (my_q[j] < Sq) {
+                float* pr = part + (((int64_t)sp * nbh + bh) * Sq + my_q[j]) * (D + kPartPad);
+#pragma unroll
+                for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+                    for (int g = 0; g < 4; ++g) {
+                        f32x4 w;
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) w[e] = st.o[j][dt][4 * g + e];
+                        *reinterpret_cast<f32x4*>(pr + 32 * dt + 8 * g + 4 * hb) = w;
+                    }
+                if (hb == 0) *reinterpret_cast<f32x2*>(pr + D) = f32x2{st.m[j], l_tot};
+            }
+        }
+        return;
     }
 
     // ---- epilogue: add the two half-row sums, O / l (approximate reciprocal), round, store -----
@@ -555,6 +601,107 @@ __global__ __launch_bounds__(128 * 2 / JT) __attribute__((amdgpu_waves_per_eu(2,
     }
 }
 
+// Adds the parts of a split launch: a thread owns four adjacent channels of one query row.
+template <typename E, int D>
+__global__ __launch_bounds__(256) void fmha_combine_kernel(const float* __restrict__ part, int nsplit, int64_t rows,
+                                                           unsigned short* __restrict__ O, Strides os, int Sq, int H) {
+    constexpr int CPRW = D / 4;
+    const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (idx >= rows * CPRW) return;
+    const int64_t row = idx / CPRW;
+    const int c = (int)(idx - row * CPRW);
+    const float* p0 = part + row * (D + kPartPad);
+    const int64_t part_stride = rows * (D + kPartPad);
+    float m = -INFINITY;
+    for (int sp = 0; sp < nsplit; ++sp) m = fmaxf(m, p0[sp * part_stride + D]);
+    f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+    float l = 0.f;
+    for (int sp = 0; sp < nsplit; ++sp) {
+        const float* pr = p0 + sp * part_stride;
+        const float mp = pr[D];
+        if (mp == -INFINITY) continue;   // a part without a visible key for this row
+        const float w = __builtin_amdgcn_exp2f(mp - m);
+        l += w * pr[D + 1];
+        const f32x4 o = *reinterpret_cast<const f32x4*>(pr + 4 * c);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) acc[e] += w * o[e];
+    }
+    const float inv = __builtin_amdgcn_rcpf(l);
+    const int64_t bh = row / Sq;
+    const int q = (int)(row - bh * Sq);
+    const int64_t batch = bh / H, head = bh - batch * H;
+    s16x4 out;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) out[e] = E::cvt(acc[e] * inv);
+    *reinterpret_cast<s16x4*>(O + head * os.s2 + batch * os.s3 + (int64_t)q * os.s1 + 4 * c) = out;
+}
+
+// Scratch of the split launches: one array per GPU, shared by its streams.  A launch that follows one from another
+// stream first waits for an event recorded there; a stream under capture is not given the array.
+constexpr int64_t kPartFloats = 16 * 1024 * 1024;   // 64 MiB
+static __device__ __align__(256) float fmha_part_scratch[kPartFloats];
+struct PartState {
+    std::mutex mu;
+    float* scratch = nullptr;
+    hipEvent_t done = nullptr;
+    hipStream_t last = nullptr;
+    bool used = false, broken = false;
+};
+PartState g_part[16];
+
+// Number of parts for the launch, 0 = no split.
+int pick_parts(int64_t wgs, int64_t rows, int D, int Sq, int Skv, bool causal, int input_pos) {
+    static const int force = [] { const char* e = getenv("MI_FMHA_SPLIT"); return e ? atoi(e) : -1; }();   // 0 = never, n = n parts
+    if (force == 0 || wgs >= 1024) return 0;   // (four workgroups of two or four waves fill a CU)
+    int64_t keys = Skv;   // keys the busiest workgroup walks
+    if (causal && (int64_t)input_pos + Sq < keys) keys = (int64_t)input_pos + Sq;
+    const int64_t tiles = (keys + kKV - 1) / kKV;
+    // Measured, 8 x 16 heads: one query against 4096 keys 28 us with 512 workgroups in all, 33 us with 1024 (64 us unsplit);
+    // 128 queries against 4096 keys 46 us with 1024, 64 us with 384 (104 us unsplit).
+    const int64_t target = Sq <= 32 ? 512 : 1024;
+    int64_t parts = force > 0 ? force : (target + wgs - 1) / wgs;
+    if (parts > tiles / 4) parts = tiles / 4;                              // at least four tiles (256 keys) per part
+    if (parts > 64) parts = 64;
+    while (parts >= 2 && parts * rows * (D + kPartPad) > kPartFloats) --parts;
+    return parts >= 2 ? (int)parts : 0;
+}
+
+// The scratch for a split launch on stream s, ordered after its previous user; nullptr if it can not be had.
+float* acquire_parts(hipStream_t s, std::unique_lock<std::mutex>& lock) {
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 16) return nullptr;
+    hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
+    if (hipStreamIsCapturing(s, &cap) != hipSuccess || cap != hipStreamCaptureStatusNone) return nullptr;
+    PartState& st = g_part[dev];
+    lock = std::unique_lock<std::mutex>(st.mu);
+    if (st.broken) return nullptr;
+    if (!st.scratch) {
+        if (hipGetSymbolAddress((void**)&st.scratch, HIP_SYMBOL(fmha_part_scratch)) != hipSuccess ||
+            hipEventCreateWithFlags(&st.done, hipEventDisableTiming) != hipSuccess) {
+            st.broken = true;
+            st.scratch = nullptr;
+            (void)hipGetLastError();
+            return nullptr;
+        }
+    }
+    if (st.used && st.last != s) {
+        bool ordered;
+        if (hipEventRecord(st.done, st.last) == hipSuccess) {
+            ordered = hipStreamWaitEvent(s, st.done, 0) == hipSuccess;
+        } else {   // that stream no longer exists: what it was given is done once the device is idle
+            (void)hipGetLastError();
+            ordered = hipDeviceSynchronize() == hipSuccess;
+        }
+        if (!ordered) {
+            (void)hipGetLastError();
+            return nullptr;
+        }
+    }
+    st.last = s;
+    st.used = true;
+    return st.scratch;
+}
+
 bool vec16(const mi_tile_array* a) {
     return aligned(a->ptr, 16) && a->strides[1] % 8 == 0 && a->strides[2] % 8 == 0 && a->strides[3] % 8 == 0;
 }
@@ -570,6 +717,26 @@ void launch(dim3 grid, hipStream_t s, bool causal, const mi_tile_array* Q, const
         constexpr int JT = D == 64 ? 2 : 1;
         const int nqb = (int)grid.x, nbh = (int)grid.y;
         dim3 g1((unsigned)(nqb * nbh)), blk(128 * 2 / JT);
+        const int64_t rows = (int64_t)nbh * Sq;
+        if (const int parts = pick_parts((int64_t)nqb * nbh, rows, D, Sq, Skv, causal, input_pos)) {
+            std::unique_lock<std::mutex> lock;
+            if (float* scratch = acquire_parts(s, lock)) {
+                dim3 gs((unsigned)(nqb * nbh * parts));
+                if (causal)
+                    hipLaunchKernelGGL((fmha_fwd_dma_kernel<E, D, JT, true, true>), gs, blk, 0, s, (const unsigned short*)Q->ptr, qs,
+                                       (const unsigned short*)K->ptr, ks, (const unsigned short*)V->ptr, vs,
+                                       (unsigned short*)O->ptr, os, Sq, Skv, H, group, scale2, input_pos, nqb, nbh, parts, scratch);
+                else
+                    hipLaunchKernelGGL((fmha_fwd_dma_kernel<E, D, JT, false, true>), gs, blk, 0, s, (const unsigned short*)Q->ptr, qs,
+                                       (const unsigned short*)K->ptr, ks, (const unsigned short*)V->ptr, vs,
+                                       (unsigned short*)O->ptr, os, Sq, Skv, H, group, scale2, input_pos, nqb, nbh, parts, scratch);
+                const int64_t threads = rows * (D / 4);
+                hipLaunchKernelGGL((fmha_combine_kernel<E, D>), dim3((unsigned)((threads + 255) / 256)), dim3(256), 0, s, scratch, parts,
+                                   rows, (unsigned short*)O->ptr, os, Sq, H);
+                set_variant(D == 64 ? "fmha_dma_q128_kv64_d64_w64q_splitkv" : "fmha_dma_q128_kv64_d128_w32q_splitkv");
+                return;
+            }
+        }
         if (causal)
             hipLaunchKernelGGL((fmha_fwd_dma_kernel<E, D, JT, true>), g1, blk, 0, s, (const unsigned short*)Q->ptr, qs,
                                (const unsigned short*)K->ptr, ks, (const unsigned short*)V->ptr, vs,

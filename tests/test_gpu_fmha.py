@@ -152,6 +152,52 @@ def test_fmha_ragged_without_the_causal_mask_takes_the_general_kernel(ct, orc):
     check(orc, r.out, ref)
 
 
+@pytest.mark.parametrize("batch,heads,sq,skv,qg,causal,pos,d,T", [
+    (2, 4, 1, 1000, 1, True, 999, 64, torch.float16),        # one query at the end of the cache
+    (1, 8, 1, 4096, 4, True, 4095, 64, torch.bfloat16),      # grouped heads
+    (1, 2, 7, 777, 1, True, 770, 64, torch.float16),         # a few queries, ragged cache
+    (1, 4, 130, 2000, 2, True, 1870, 64, torch.float16),     # two query blocks
+    (1, 2, 200, 3000, 1, False, 0, 64, torch.bfloat16),      # no mask
+    (1, 1, 64, 5000, 1, True, 4000, 64, torch.float16),      # the cache ends above every diagonal
+    (1, 2, 512, 600, 1, True, 88, 64, torch.float16),        # the second part starts above the diagonals of the early rows:
+    (1, 2, 512, 512, 1, True, 0, 128, torch.float16),        # they go through it without a visible key
+    (1, 2, 256, 4096, 1, True, 1000, 128, torch.float16),    # D = 128
+    (1, 3, 33, 2049, 1, False, 0, 128, torch.bfloat16),
+    (1, 8, 1, 2048, 2, True, 2047, 128, torch.float16),
+])
+def test_fmha_few_queries_many_keys_split_over_the_keys(ct, orc, batch, heads, sq, skv, qg, causal, pos, d, T):
+    """Decode and chunked-prefill shapes: too few (query block, head) pairs to fill the chip, so the key range of each is
+    dealt to several workgroups and a second kernel adds their parts.  Against the float64 restatement of the kernel's
+    masking rule, into an output inside a wider buffer."""
+    data = fmha.prepare(batch=batch, heads=heads, seq_q=sq, seq_kv=skv, d_k=d, d_v=d, query_group_size=qg, causal=causal, T=T)
+    big = torch.full((batch, heads, sq + 8, d), 777.0, dtype=T, device="cuda")
+    out = big[:, :, :sq, :]
+    out.fill_(float("nan"))
+    fmha.cutile_fmha(data.Q, data.K, data.V, query_group_size=qg, causal=causal, input_pos=pos, out=out)
+    assert ct.last_variant().endswith("_splitkv"), ct.last_variant()
+    assert bool((big[:, :, sq:, :] == 777.0).all())
+    ref = orc.fmha_general(*(orc.to_julia(t) for t in (data.Q, data.K, data.V)), causal=causal, input_pos=pos)
+    check(orc, out, ref, 2e-2 if T == torch.float16 else 3e-2)
+
+
+def test_fmha_split_launches_from_two_streams_are_ordered(ct, orc):
+    """The parts live in one array per GPU: launches that alternate between two streams each get their own result."""
+    datas = [fmha.prepare(batch=1, heads=4, seq_q=1, seq_kv=3000 + 64 * i, causal=True, seed=20 + i) for i in range(3)]
+    refs = [orc.fmha_general(*(orc.to_julia(t) for t in (d.Q, d.K, d.V)), causal=True, input_pos=d.seq_kv - 1) for d in datas]
+    torch.cuda.synchronize()
+    streams = [torch.cuda.Stream(), torch.cuda.Stream()]
+    outs = []
+    for i in range(12):
+        d = datas[i % 3]
+        with torch.cuda.stream(streams[i % 2]):
+            outs.append(fmha.cutile_fmha(d.Q, d.K, d.V, causal=True, input_pos=d.seq_kv - 1))
+            assert ct.last_variant().endswith("_splitkv")
+    torch.cuda.synchronize()
+    for i, o in enumerate(outs):
+        check(orc, o, refs[i % 3])
+        assert torch.equal(o, outs[i % 3])
+
+
 @pytest.mark.parametrize("causal", [True, False])
 def test_fmha_pipelined_kernel_strided_views(ct, orc, causal):
     """Q/K/V as views of one packed (B, S, 3, H, D) buffer and Out as a view of a wider buffer: row,

@@ -35,6 +35,11 @@
 // above a query's diagonal, so a row can go through tiles without a visible key: its maximum stays -Inf and the
 // weights are taken against 0 instead (SAFE), which keeps them at exp2(-Inf) = 0 rather than exp2(-Inf + Inf).
 //
+// Grouped heads with few queries (`pack` = QUERY_GROUP_SIZE when Sq <= 64): the heads that share a K / V head are
+// stacked as rows of one query tile -- row r is query r % Sq of head r / Sq of the group -- so their common keys are
+// read once per group instead of once per head.  Positions are no longer monotonic over a tile's rows; the tile-level
+// decisions (which key tiles a query tile takes part in, which need the mask) use the group's first and last position.
+//
 // FLOPs (causal-exact): 4 * B * H * D * Sq*(Sq+1)/2 for Sq == Skv.
 #include "fmha_common.h"
 #include <stdlib.h>
@@ -408,7 +413,8 @@ template <typename E, int D, int JT, bool CAUSAL, bool SPLIT = false>
 __global__ __launch_bounds__(128 * 2 / JT) __attribute__((amdgpu_waves_per_eu(2, 2))) void fmha_fwd_dma_kernel(
     const unsigned short* __restrict__ Q, Strides qs, const unsigned short* __restrict__ K, Strides ks,
     const unsigned short* __restrict__ V, Strides vs, unsigned short* __restrict__ O, Strides os, int Sq, int Skv,
-    int H, int group, float scale2, int input_pos, int nqb, int nbh, int nsplit = 1, float* __restrict__ part = nullptr) {
+    int H, int group, float scale2, int input_pos, int nqb, int nbh, int pack, int nsplit = 1,
+    float* __restrict__ part = nullptr) {
     using F = FmhaDma<E, D, JT, CAUSAL>;
     constexpr int NW = F::NW, KSTEPS = F::KSTEPS, DT = F::DT, CH = F::CH, TPW = F::TPW;
     constexpr bool PAIRED = CAUSAL && JT == 2;
@@ -435,13 +441,16 @@ __global__ __launch_bounds__(128 * 2 / JT) __attribute__((amdgpu_waves_per_eu(2,
         }
         if (CAUSAL && !PAIRED) qb = nqb - 1 - qb;
     }
-    const int batch = bh / H, head = bh % H, kvh = head / group;
+    // (pack > 1: bh counts (batch, K / V head) pairs, H is their number per batch, and a row carries its head)
+    const int batch = bh / H, hrem = bh % H;
+    const int head = pack > 1 ? hrem * group : hrem, kvh = pack > 1 ? hrem : hrem / group;
+    const int R = Sq * pack;   // query rows of this (batch, head) or (batch, head group)
     Q += (int64_t)head * qs.s2 + (int64_t)batch * qs.s3;
     if (!SPLIT) O += (int64_t)head * os.s2 + (int64_t)batch * os.s3;
     const char* Kg = (const char*)(K + (int64_t)kvh * ks.s2 + (int64_t)batch * ks.s3);
     const char* Vg = (const char*)(V + (int64_t)kvh * vs.s2 + (int64_t)batch * vs.s3);
 
-    const int NT = (Sq + 31) / 32;  // query tiles of 32
+    const int NT = (R + 31) / 32;  // query tiles of 32
     int tq[JT];                     // this wave's query tiles (wave-uniform); -1 = none
     int wg_last_tile;               // highest query tile of the workgroup (bounds the causal KV loop)
     if (PAIRED) {
@@ -461,17 +470,25 @@ __global__ __launch_bounds__(128 * 2 / JT) __attribute__((amdgpu_waves_per_eu(2,
     }
 
     typename F::State st;
-    int my_q[JT], last_pos[JT];
+    int my_q[JT], last_pos[JT];   // my_q: the lane's row, R = none
+    int64_t q_off[JT], o_off[JT];  // element offsets of the row in Q and in Out
 #pragma unroll
     for (int j = 0; j < JT; ++j) {
-        my_q[j] = tq[j] >= 0 ? 32 * tq[j] + (lane & 31) : Sq;
-        st.my_pos[j] = input_pos + my_q[j];
-        st.first_pos[j] = input_pos + 32 * tq[j];
-        last_pos[j] = tq[j] >= 0 ? st.first_pos[j] + 31 : -1;
+        my_q[j] = tq[j] >= 0 ? 32 * tq[j] + (lane & 31) : R;
+        int qi = my_q[j], hq = 0;   // query index and head within the group
+        if (pack > 1) {
+            hq = my_q[j] / Sq;
+            qi = my_q[j] - hq * Sq;
+        }
+        q_off[j] = (int64_t)qi * qs.s1 + (int64_t)hq * qs.s2;
+        o_off[j] = (int64_t)qi * os.s1 + (int64_t)hq * os.s2;
+        st.my_pos[j] = input_pos + qi;
+        st.first_pos[j] = pack > 1 ? input_pos : input_pos + 32 * tq[j];
+        last_pos[j] = tq[j] < 0 ? -1 : pack > 1 ? input_pos + Sq - 1 : st.first_pos[j] + 31;
 #pragma unroll
         for (int s = 0; s < KSTEPS; ++s) {
             s16x8 v = {0};
-            if (my_q[j] < Sq) v = *reinterpret_cast<const s16x8*>(Q + (int64_t)my_q[j] * qs.s1 + 16 * s + 8 * hb);
+            if (my_q[j] < R) v = *reinterpret_cast<const s16x8*>(Q + q_off[j] + 16 * s + 8 * hb);
             st.qf[j][s] = v;
         }
 #pragma unroll
@@ -502,7 +519,7 @@ __global__ __launch_bounds__(128 * 2 / JT) __attribute__((amdgpu_waves_per_eu(2,
 
     int kv_end = Skv;
     if (CAUSAL) {
-        const int lim = input_pos + 32 * (wg_last_tile + 1);  // one past the workgroup's last query position
+        const int lim = input_pos + (pack > 1 ? Sq : 32 * (wg_last_tile + 1));  // one past the workgroup's last query position
         kv_end = lim < Skv ? lim : Skv;
         if (kv_end < 0) kv_end = 0;
     }
@@ -564,8 +581,8 @@ __global__ __launch_bounds__(128 * 2 / JT) __attribute__((amdgpu_waves_per_eu(2,
 #pragma unroll
         for (int j = 0; j < JT; ++j) {
             const float l_tot = st.l[j] + __shfl_xor(st.l[j], 32, 64);
-            if (my_q[j] < Sq) {
-                float* pr = part + (((int64_t)sp * nbh + bh) * Sq + my_q[j]) * (D + kPartPad);
+            if (my_q[j] < R) {
+                float* pr = part + (((int64_t)sp * nbh + bh) * R + my_q[j]) * (D + kPartPad);
 #pragma unroll
                 for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
@@ -585,9 +602,9 @@ __global__ __launch_bounds__(128 * 2 / JT) __attribute__((amdgpu_waves_per_eu(2,
 #pragma unroll
     for (int j = 0; j < JT; ++j) {
         const float l_tot = st.l[j] + __shfl_xor(st.l[j], 32, 64);
-        if (my_q[j] < Sq) {
+        if (my_q[j] < R) {
             const float inv = __builtin_amdgcn_rcpf(l_tot);
-            unsigned short* op = O + (int64_t)my_q[j] * os.s1;
+            unsigned short* op = O + o_off[j];
 #pragma unroll
             for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
@@ -604,7 +621,8 @@ __global__ __launch_bounds__(128 * 2 / JT) __attribute__((amdgpu_waves_per_eu(2,
 // Adds the parts of a split launch: a thread owns four adjacent channels of one query row.
 template <typename E, int D>
 __global__ __launch_bounds__(256) void fmha_combine_kernel(const float* __restrict__ part, int nsplit, int64_t rows,
-                                                           unsigned short* __restrict__ O, Strides os, int Sq, int H) {
+                                                           unsigned short* __restrict__ O, Strides os, int Sq, int H,
+                                                           int pack) {
     constexpr int CPRW = D / 4;
     const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
     if (idx >= rows * CPRW) return;
@@ -627,9 +645,11 @@ __global__ __launch_bounds__(256) void fmha_combine_kernel(const float* __restri
         for (int e = 0; e < 4; ++e) acc[e] += w * o[e];
     }
     const float inv = __builtin_amdgcn_rcpf(l);
-    const int64_t bh = row / Sq;
-    const int q = (int)(row - bh * Sq);
-    const int64_t batch = bh / H, head = bh - batch * H;
+    // a row is (query, head within the group when the group's heads are stacked, head or head group, batch)
+    const int R = Sq * pack;
+    const int64_t bh = row / R;
+    const int r = (int)(row - bh * R), hq = r / Sq, q = r - hq * Sq;
+    const int64_t batch = bh / H, head = (bh - batch * H) * pack + hq;
     s16x4 out;
 #pragma unroll
     for (int e = 0; e < 4; ++e) out[e] = E::cvt(acc[e] * inv);
@@ -715,9 +735,12 @@ void launch(dim3 grid, hipStream_t s, bool causal, const mi_tile_array* Q, const
     const int Sq = (int)Q->sizes[1], Skv = (int)K->sizes[1];
     if (vec_ok && K->strides[1] < (1 << 24) && V->strides[1] < (1 << 24)) {
         constexpr int JT = D == 64 ? 2 : 1;
-        const int nqb = (int)grid.x, nbh = (int)grid.y;
+        // few queries and grouped heads: the heads of a group are stacked in one query tile
+        const int pack = group > 1 && Sq <= 64 ? group : 1;
+        const int Hb = H / pack;                                   // heads, or head groups, per batch
+        const int nqb = pack > 1 ? (Sq * pack + kQB - 1) / kQB : (int)grid.x, nbh = (int)grid.y / pack;
         dim3 g1((unsigned)(nqb * nbh)), blk(128 * 2 / JT);
-        const int64_t rows = (int64_t)nbh * Sq;
+        const int64_t rows = (int64_t)nbh * Sq * pack;
         if (const int parts = pick_parts((int64_t)nqb * nbh, rows, D, Sq, Skv, causal, input_pos)) {
             std::unique_lock<std::mutex> lock;
             if (float* scratch = acquire_parts(s, lock)) {
@@ -725,27 +748,29 @@ void launch(dim3 grid, hipStream_t s, bool causal, const mi_tile_array* Q, const
                 if (causal)
                     hipLaunchKernelGGL((fmha_fwd_dma_kernel<E, D, JT, true, true>), gs, blk, 0, s, (const unsigned short*)Q->ptr, qs,
                                        (const unsigned short*)K->ptr, ks, (const unsigned short*)V->ptr, vs,
-                                       (unsigned short*)O->ptr, os, Sq, Skv, H, group, scale2, input_pos, nqb, nbh, parts, scratch);
+                                       (unsigned short*)O->ptr, os, Sq, Skv, Hb, group, scale2, input_pos, nqb, nbh, pack, parts, scratch);
                 else
                     hipLaunchKernelGGL((fmha_fwd_dma_kernel<E, D, JT, false, true>), gs, blk, 0, s, (const unsigned short*)Q->ptr, qs,
                                        (const unsigned short*)K->ptr, ks, (const unsigned short*)V->ptr, vs,
-                                       (unsigned short*)O->ptr, os, Sq, Skv, H, group, scale2, input_pos, nqb, nbh, parts, scratch);
+                                       (unsigned short*)O->ptr, os, Sq, Skv, Hb, group, scale2, input_pos, nqb, nbh, pack, parts, scratch);
                 const int64_t threads = rows * (D / 4);
                 hipLaunchKernelGGL((fmha_combine_kernel<E, D>), dim3((unsigned)((threads + 255) / 256)), dim3(256), 0, s, scratch, parts,
-                                   rows, (unsigned short*)O->ptr, os, Sq, H);
-                set_variant(D == 64 ? "fmha_dma_q128_kv64_d64_w64q_splitkv" : "fmha_dma_q128_kv64_d128_w32q_splitkv");
+                                   rows, (unsigned short*)O->ptr, os, Sq, Hb, pack);
+                set_variant(pack > 1 ? (D == 64 ? "fmha_dma_q128_kv64_d64_w64q_grouped_splitkv" : "fmha_dma_q128_kv64_d128_w32q_grouped_splitkv")
+                                     : (D == 64 ? "fmha_dma_q128_kv64_d64_w64q_splitkv" : "fmha_dma_q128_kv64_d128_w32q_splitkv"));
                 return;
             }
         }
         if (causal)
             hipLaunchKernelGGL((fmha_fwd_dma_kernel<E, D, JT, true>), g1, blk, 0, s, (const unsigned short*)Q->ptr, qs,
                                (const unsigned short*)K->ptr, ks, (const unsigned short*)V->ptr, vs,
-                               (unsigned short*)O->ptr, os, Sq, Skv, H, group, scale2, input_pos, nqb, nbh);
+                               (unsigned short*)O->ptr, os, Sq, Skv, Hb, group, scale2, input_pos, nqb, nbh, pack);
         else
             hipLaunchKernelGGL((fmha_fwd_dma_kernel<E, D, JT, false>), g1, blk, 0, s, (const unsigned short*)Q->ptr, qs,
                                (const unsigned short*)K->ptr, ks, (const unsigned short*)V->ptr, vs,
-                               (unsigned short*)O->ptr, os, Sq, Skv, H, group, scale2, input_pos, nqb, nbh);
-        set_variant(D == 64 ? "fmha_dma_q128_kv64_d64_w64q" : "fmha_dma_q128_kv64_d128_w32q");
+                               (unsigned short*)O->ptr, os, Sq, Skv, Hb, group, scale2, input_pos, nqb, nbh, pack);
+        set_variant(pack > 1 ? (D == 64 ? "fmha_dma_q128_kv64_d64_w64q_grouped" : "fmha_dma_q128_kv64_d128_w32q_grouped")
+                             : (D == 64 ? "fmha_dma_q128_kv64_d64_w64q" : "fmha_dma_q128_kv64_d128_w32q"));
         return;
     }
     const dim3 g2((unsigned)(grid.x * grid.y));

@@ -184,7 +184,8 @@ int mi_softmax_chunked_kernel(const mi_tile_array* output, const mi_tile_array* 
  * QUERY_GROUP_SIZE, decode offset input_pos, ragged KV tail when !EVEN_K.
  * Few queries against many keys (decode, chunked prefill: fewer than 1024 workgroups of 128 queries) are split over
  * the keys: the parts go through a 64 MiB static device array of the library and a second kernel adds them.  Launches
- * that use the array from different streams are ordered by an event; a stream under capture runs unsplit. */
+ * that use the array from different streams are ordered by an event; a stream under capture runs unsplit.  With
+ * grouped heads and at most 64 queries the heads of a group share a query tile, so their keys are read once. */
 int mi_fmha_kernel(const mi_tile_array* Q, const mi_tile_array* K, const mi_tile_array* V,
                    const mi_tile_array* Out, float qk_scale, int32_t input_pos, int TILE_D,
                    int H, int TILE_M, int TILE_N, int QUERY_GROUP_SIZE, int CAUSAL, int EVEN_K,

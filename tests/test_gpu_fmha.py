@@ -164,6 +164,10 @@ def test_fmha_ragged_without_the_causal_mask_takes_the_general_kernel(ct, orc):
     (1, 2, 256, 4096, 1, True, 1000, 128, torch.float16),    # D = 128
     (1, 3, 33, 2049, 1, False, 0, 128, torch.bfloat16),
     (1, 8, 1, 2048, 2, True, 2047, 128, torch.float16),
+    # grouped heads with few queries: the heads of a group are stacked as rows of one query tile
+    (2, 8, 1, 1300, 8, True, 1299, 64, torch.float16), (1, 16, 64, 640, 4, True, 576, 64, torch.bfloat16),
+    (1, 12, 17, 555, 3, False, 0, 64, torch.float16), (2, 8, 40, 4000, 4, True, 3900, 128, torch.float16),
+    (4, 32, 1, 2048, 4, True, 2047, 64, torch.float16),
 ])
 def test_fmha_few_queries_many_keys_split_over_the_keys(ct, orc, batch, heads, sq, skv, qg, causal, pos, d, T):
     """Decode and chunked-prefill shapes: too few (query block, head) pairs to fill the chip, so the key range of each is
@@ -175,9 +179,23 @@ def test_fmha_few_queries_many_keys_split_over_the_keys(ct, orc, batch, heads, s
     out.fill_(float("nan"))
     fmha.cutile_fmha(data.Q, data.K, data.V, query_group_size=qg, causal=causal, input_pos=pos, out=out)
     assert ct.last_variant().endswith("_splitkv"), ct.last_variant()
+    assert ("_grouped" in ct.last_variant()) == (qg > 1 and sq <= 64)
     assert bool((big[:, :, sq:, :] == 777.0).all())
     ref = orc.fmha_general(*(orc.to_julia(t) for t in (data.Q, data.K, data.V)), causal=causal, input_pos=pos)
     check(orc, out, ref, 2e-2 if T == torch.float16 else 3e-2)
+
+
+@pytest.mark.parametrize("batch,heads,sq,skv,qg,causal,pos,d", [
+    (2, 8, 1, 200, 8, True, 199, 64), (1, 8, 33, 100, 8, True, 10, 64), (3, 6, 5, 130, 2, False, 0, 128), (1, 4, 64, 64, 4, True, 0, 64),
+])
+def test_fmha_grouped_heads_stacked_short_cache(ct, orc, batch, heads, sq, skv, qg, causal, pos, d):
+    """Grouped heads with few queries and too few keys to split: the group's heads as rows of one query tile, one
+    workgroup per (batch, K / V head)."""
+    data = fmha.prepare(batch=batch, heads=heads, seq_q=sq, seq_kv=skv, d_k=d, d_v=d, query_group_size=qg, causal=causal)
+    out = attend(data.Q, data.K, data.V, query_group_size=qg, causal=causal, input_pos=pos)
+    assert ct.last_variant().endswith("_grouped"), ct.last_variant()
+    ref = orc.fmha_general(*(orc.to_julia(t) for t in (data.Q, data.K, data.V)), causal=causal, input_pos=pos)
+    check(orc, out, ref)
 
 
 def test_fmha_split_launches_from_two_streams_are_ordered(ct, orc):

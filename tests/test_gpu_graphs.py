@@ -114,13 +114,20 @@ def test_graph_attention(ct):
     def inputs(seed):
         g = gen(seed)
         h = lambda *s: torch.randn(*s, device="cuda", generator=g).half()
-        return h(2, 8, 512, 64), h(2, 8, 512, 64), h(2, 8, 512, 64), h(1, 4, 200, 64), h(1, 2, 333, 64), h(1, 2, 333, 64)
+        return (h(2, 8, 512, 64), h(2, 8, 512, 64), h(2, 8, 512, 64), h(1, 4, 200, 64), h(1, 2, 333, 64), h(1, 2, 333, 64),
+                h(2, 8, 1, 64), h(2, 2, 3000, 64), h(2, 2, 3000, 64))
 
-    def op(Q, K, V, Q2, K2, V2):
+    def op(Q, K, V, Q2, K2, V2, Q3, K3, V3):
         return (fmha.cutile_fmha(Q, K, V, causal=True), fmha.cutile_fmha(Q, K, V, causal=False),
-                fmha.cutile_fmha(Q2, K2, V2, causal=False, query_group_size=2, tile_m=64, tile_n=64))
+                fmha.cutile_fmha(Q2, K2, V2, causal=False, query_group_size=2, tile_m=64, tile_n=64),
+                fmha.cutile_fmha(Q3, K3, V3, causal=True, input_pos=2999, query_group_size=4))
 
-    replay_check(inputs, op)
+    def compare(got, ref, i):
+        # output 3, one new token against 3000 cached keys: eager deals the keys to several workgroups and adds their
+        # parts, the captured launch walks them in one piece (the library's scratch is not handed to a capturing stream)
+        return torch.allclose(got.float(), ref.float(), rtol=2e-3, atol=2e-3) if i == 3 else torch.equal(got, ref)
+
+    replay_check(inputs, op, compare=compare)
 
 
 @pytest.mark.parametrize("topk", [2, 8])

@@ -618,32 +618,59 @@ __global__ __launch_bounds__(128 * 2 / JT) __attribute__((amdgpu_waves_per_eu(2,
     }
 }
 
-// Adds the parts of a split launch: a thread owns four adjacent channels of one query row.
-template <typename E, int D>
+// Adds the parts of a split launch.  Four adjacent channels of one query row belong to PL threads, which take the
+// parts pl, pl + PL, ... and meet in LDS (with one thread per row and 64 parts the two dependent passes over the
+// parts took 49 us for 32 rows).
+template <typename E, int D, int PL>
 __global__ __launch_bounds__(256) void fmha_combine_kernel(const float* __restrict__ part, int nsplit, int64_t rows,
                                                            unsigned short* __restrict__ O, Strides os, int Sq, int H,
                                                            int pack) {
-    constexpr int CPRW = D / 4;
-    const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
-    if (idx >= rows * CPRW) return;
-    const int64_t row = idx / CPRW;
-    const int c = (int)(idx - row * CPRW);
-    const float* p0 = part + row * (D + kPartPad);
+    constexpr int CPRW = D / 4, TPR = CPRW * PL, RPB = 256 / TPR;
+    static_assert(TPR <= 256 && 256 % TPR == 0, "the threads of a row stay inside the workgroup");
+    __shared__ float s_max[PL > 1 ? 256 : 1];
+    __shared__ float s_acc[PL > 1 ? 256 : 1][5];
+    const int tid = threadIdx.x, c = tid % CPRW, pl = (tid / CPRW) % PL, rl = tid / TPR;
+    const int64_t row = (int64_t)blockIdx.x * RPB + rl;
+    const bool live = row < rows;
+    const float* p0 = part + (live ? row : 0) * (D + kPartPad);
     const int64_t part_stride = rows * (D + kPartPad);
     float m = -INFINITY;
-    for (int sp = 0; sp < nsplit; ++sp) m = fmaxf(m, p0[sp * part_stride + D]);
+    if (live)
+        for (int sp = pl; sp < nsplit; sp += PL) m = fmaxf(m, p0[sp * part_stride + D]);
+    if (PL > 1) {
+        s_max[tid] = m;
+        __syncthreads();
+#pragma unroll
+        for (int i = 0; i < PL; ++i) m = fmaxf(m, s_max[rl * TPR + i * CPRW + c]);
+    }
     f32x4 acc = {0.f, 0.f, 0.f, 0.f};
     float l = 0.f;
-    for (int sp = 0; sp < nsplit; ++sp) {
-        const float* pr = p0 + sp * part_stride;
-        const float mp = pr[D];
-        if (mp == -INFINITY) continue;   // a part without a visible key for this row
-        const float w = __builtin_amdgcn_exp2f(mp - m);
-        l += w * pr[D + 1];
-        const f32x4 o = *reinterpret_cast<const f32x4*>(pr + 4 * c);
+    if (live)
+        for (int sp = pl; sp < nsplit; sp += PL) {
+            const float* pr = p0 + sp * part_stride;
+            const float mp = pr[D];
+            if (mp == -INFINITY) continue;   // a part without a visible key for this row
+            const float w = __builtin_amdgcn_exp2f(mp - m);
+            l += w * pr[D + 1];
+            const f32x4 o = *reinterpret_cast<const f32x4*>(pr + 4 * c);
 #pragma unroll
-        for (int e = 0; e < 4; ++e) acc[e] += w * o[e];
+            for (int e = 0; e < 4; ++e) acc[e] += w * o[e];
+        }
+    if (PL > 1) {
+#pragma unroll
+        for (int e = 0; e < 4; ++e) s_acc[tid][e] = acc[e];
+        s_acc[tid][4] = l;
+        __syncthreads();
+        if (pl != 0) return;
+#pragma unroll
+        for (int i = 1; i < PL; ++i) {
+            const float* o = s_acc[rl * TPR + i * CPRW + c];
+#pragma unroll
+            for (int e = 0; e < 4; ++e) acc[e] += o[e];
+            l += o[4];
+        }
     }
+    if (!live) return;
     const float inv = __builtin_amdgcn_rcpf(l);
     // a row is (query, head within the group when the group's heads are stacked, head or head group, batch)
     const int R = Sq * pack;
@@ -753,9 +780,14 @@ void launch(dim3 grid, hipStream_t s, bool causal, const mi_tile_array* Q, const
                     hipLaunchKernelGGL((fmha_fwd_dma_kernel<E, D, JT, false, true>), gs, blk, 0, s, (const unsigned short*)Q->ptr, qs,
                                        (const unsigned short*)K->ptr, ks, (const unsigned short*)V->ptr, vs,
                                        (unsigned short*)O->ptr, os, Sq, Skv, Hb, group, scale2, input_pos, nqb, nbh, pack, parts, scratch);
-                const int64_t threads = rows * (D / 4);
-                hipLaunchKernelGGL((fmha_combine_kernel<E, D>), dim3((unsigned)((threads + 255) / 256)), dim3(256), 0, s, scratch, parts,
-                                   rows, (unsigned short*)O->ptr, os, Sq, Hb, pack);
+                constexpr int PLMAX = 256 / (D / 4) < 16 ? 256 / (D / 4) : 16;
+#define COMBINE(PL)                                                                                                              \
+    hipLaunchKernelGGL((fmha_combine_kernel<E, D, PL>), dim3((unsigned)((rows * (D / 4) * PL + 255) / 256)), dim3(256), 0, s, scratch, \
+                       parts, rows, (unsigned short*)O->ptr, os, Sq, Hb, pack)
+                if (parts <= 4) COMBINE(1);
+                else if (parts <= 16) COMBINE(4);
+                else COMBINE(PLMAX);
+#undef COMBINE
                 set_variant(pack > 1 ? (D == 64 ? "fmha_dma_q128_kv64_d64_w64q_grouped_splitkv" : "fmha_dma_q128_kv64_d128_w32q_grouped_splitkv")
                                      : (D == 64 ? "fmha_dma_q128_kv64_d64_w64q_splitkv" : "fmha_dma_q128_kv64_d128_w32q_splitkv"));
                 return;

@@ -379,7 +379,9 @@ int pick_split(const Problem& p, int* kchunk) {
     static const int force = [] { const char* e = getenv("MI_GEMM_SPLITK"); return e ? atoi(e) : -1; }();   // 0 = never, n = n parts
     if (force == 0) return 0;
     const int64_t tiles = tiles_of(p, 128, 128);
-    if (tiles > 64 || p.K < 1024) return 0;
+    // (up to half a tile per CU: 2048 x 768 x 8192, 96 tiles, 59 -> 41 us with two parts; 1152 x 1024 x 16384 107 -> 55 us
+    // with three; beyond 128 tiles the estimate below never favours a split)
+    if (tiles > 128 || p.K < 1024) return 0;
     // Estimated times in us: one launch walks K / 32 steps of 0.18 us; the split pays a second launch, the partial
     // sums written and read again (at about 3 bytes per ns), and walks a part's steps only.
     const double t_plain = 3.0 + 0.18 * (p.K / 32.0);

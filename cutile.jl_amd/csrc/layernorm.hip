@@ -241,8 +241,9 @@ __global__ __launch_bounds__(BLOCK) void ln_fwd_pipe_kernel(const float* __restr
 }
 
 // Forward for rows longer than the register-cached variants hold: three passes, the second
-// and third re-reading the row (served by L2 for rows up to a few MB).
-template <int BLOCK>
+// and third re-reading the row (served by L2 for rows up to a few MB).  VEC: every row, W and B are
+// 16-byte aligned and N is a multiple of 4 (16-byte accesses, four per lane in flight).
+template <int BLOCK, bool VEC>
 __global__ __launch_bounds__(BLOCK) void ln_fwd_3pass_kernel(const float* __restrict__ X, int64_t ldx,
                                                              const float* __restrict__ W,
                                                              const float* __restrict__ B,
@@ -251,14 +252,30 @@ __global__ __launch_bounds__(BLOCK) void ln_fwd_3pass_kernel(const float* __rest
                                                              float* __restrict__ Rstd, float eps,
                                                              int64_t N, int64_t M) {
     constexpr int NW = BLOCK / 64;
+    typedef float f4 __attribute__((ext_vector_type(4)));
     __shared__ float red[NW];
+    const int64_t nvec = VEC ? N / 4 : 0;
     for (int64_t m = blockIdx.x; m < M; m += gridDim.x) {
         const float* x = X + m * ldx;
         float s = 0.f;
-        for (int64_t e = threadIdx.x; e < N; e += BLOCK) s += x[e];
+#pragma unroll 4
+        for (int64_t v = threadIdx.x; v < nvec; v += BLOCK) {
+            const f4 r = *reinterpret_cast<const f4*>(x + 4 * v);
+            s += (r[0] + r[1]) + (r[2] + r[3]);
+        }
+        for (int64_t e = 4 * nvec + threadIdx.x; e < N; e += BLOCK) s += x[e];
         const float mean = block_reduce<NW>(s, red, SumOp{}, 0.f) / (float)N;
         float sq = 0.f;
-        for (int64_t e = threadIdx.x; e < N; e += BLOCK) {
+#pragma unroll 4
+        for (int64_t v = threadIdx.x; v < nvec; v += BLOCK) {
+            const f4 r = *reinterpret_cast<const f4*>(x + 4 * v);
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                const float d = r[q] - mean;
+                sq += d * d;
+            }
+        }
+        for (int64_t e = 4 * nvec + threadIdx.x; e < N; e += BLOCK) {
             const float d = x[e] - mean;
             sq += d * d;
         }
@@ -269,7 +286,16 @@ __global__ __launch_bounds__(BLOCK) void ln_fwd_3pass_kernel(const float* __rest
             Rstd[m] = rstd;
         }
         float* y = Y + m * ldy;
-        for (int64_t e = threadIdx.x; e < N; e += BLOCK) y[e] = ((x[e] - mean) * rstd) * W[e] + B[e];
+#pragma unroll 2
+        for (int64_t v = threadIdx.x; v < nvec; v += BLOCK) {
+            const f4 r = *reinterpret_cast<const f4*>(x + 4 * v);
+            const f4 w = *reinterpret_cast<const f4*>(W + 4 * v), bb = *reinterpret_cast<const f4*>(B + 4 * v);
+            f4 o;
+#pragma unroll
+            for (int q = 0; q < 4; ++q) o[q] = ((r[q] - mean) * rstd) * w[q] + bb[q];
+            st_global<true>(o, reinterpret_cast<f4*>(y + 4 * v));
+        }
+        for (int64_t e = 4 * nvec + threadIdx.x; e < N; e += BLOCK) y[e] = ((x[e] - mean) * rstd) * W[e] + B[e];
     }
 }
 
@@ -707,10 +733,17 @@ extern "C" int mi_layer_norm_fwd(const mi_tile_array* X, const mi_tile_array* W,
     float* y = (float*)Y->ptr;
     dim3 grid((unsigned)M);
     if (N > kMaxRegsN) {
-        hipLaunchKernelGGL((ln_fwd_3pass_kernel<256>), grid, dim3(256), 0, s, x, X->strides[1],
-                           (const float*)W->ptr, (const float*)B->ptr, y, Y->strides[1],
-                           (float*)Mean->ptr, (float*)Rstd->ptr, eps, N, M);
-        set_variant("ln_fwd_3pass_b256");
+        const bool vec = N % 4 == 0 && rows_vec_ok(X) && rows_vec_ok(Y) && rows_vec_ok(W) && rows_vec_ok(B);
+        const bool wide = M < 1024;   // few rows: 1024 lanes each
+#define GO(BL, VEC)                                                                                           \
+    hipLaunchKernelGGL((ln_fwd_3pass_kernel<BL, VEC>), grid, dim3(BL), 0, s, x, X->strides[1], (const float*)W->ptr, \
+                       (const float*)B->ptr, y, Y->strides[1], (float*)Mean->ptr, (float*)Rstd->ptr, eps, N, M)
+        if (wide && vec) GO(1024, true);
+        else if (wide) GO(1024, false);
+        else if (vec) GO(256, true);
+        else GO(256, false);
+#undef GO
+        set_variant(wide ? (vec ? "ln_fwd_3pass_b1024_v4" : "ln_fwd_3pass_b1024") : (vec ? "ln_fwd_3pass_b256_v4" : "ln_fwd_3pass_b256"));
         return launch_status();
     }
     const bool al = N % 4 == 0 && rows_vec_ok(X) && rows_vec_ok(Y) && rows_vec_ok(W) && rows_vec_ok(B);

@@ -114,6 +114,9 @@ __global__ __launch_bounds__(BLOCK) void softmax_regs_kernel(T* __restrict__ out
 }
 
 // ---- three-pass kernel: any column length ---------------------------------------------
+// ALIGNED: every column starts on a 16-byte boundary.  Otherwise a column whose input and output sit at the same
+// offset from such a boundary (the usual case: equal leading dimensions) is walked as a scalar head up to the
+// boundary, 16-byte vectors, and a scalar tail; columns that do not, element by element.
 template <typename T, int BLOCK, bool ALIGNED>
 __global__ __launch_bounds__(BLOCK) void softmax_3pass_kernel(T* __restrict__ out, int64_t ldo,
                                                               const T* __restrict__ in, int64_t ldi,
@@ -123,39 +126,57 @@ __global__ __launch_bounds__(BLOCK) void softmax_3pass_kernel(T* __restrict__ ou
     constexpr int NW = BLOCK / 64;
     __shared__ float red[NW];
     const float NEG_INF = -INFINITY;
-    const int64_t nvec = ALIGNED ? L / EV : 0;
 
     for (int64_t col = blockIdx.x; col < M; col += gridDim.x) {
         const T* ip = in + col * ldi;
         T* op = out + col * ldo;
+        int64_t head = 0, nvec = L / EV;
+        if (!ALIGNED) {
+            const uintptr_t ai = (uintptr_t)ip, ao = (uintptr_t)op;
+            if ((ai & 15) == (ao & 15) && ai % sizeof(T) == 0) {
+                head = (int64_t)(((16 - (ai & 15)) & 15) / sizeof(T));
+                if (head > L) head = L;
+                nvec = (L - head) / EV;
+            } else {
+                head = L;
+                nvec = 0;
+            }
+        }
+        const T* ipv = ip + head;
+        T* opv = op + head;
+        const int64_t nscalar = L - nvec * EV;                       // head and tail elements
+        auto at = [&](int64_t e) { return e < head ? e : e + nvec * EV; };   // their positions in the column
         // pass 1: running maximum
         float mx = NEG_INF;
+#pragma unroll 4
         for (int64_t v = threadIdx.x; v < nvec; v += BLOCK) {
-            V raw = *reinterpret_cast<const V*>(ip + v * EV);
+            V raw = *reinterpret_cast<const V*>(ipv + v * EV);
 #pragma unroll
             for (int q = 0; q < EV; ++q) mx = fmaxf(mx, vget<T>(raw, q));
         }
-        for (int64_t e = nvec * EV + threadIdx.x; e < L; e += BLOCK) mx = fmaxf(mx, to_f32<T>(ip[e]));
+        for (int64_t e = threadIdx.x; e < nscalar; e += BLOCK) mx = fmaxf(mx, to_f32<T>(ip[at(e)]));
         mx = block_reduce<NW>(mx, red, MaxOp{}, NEG_INF);
         // pass 2: per-lane partial denominators, one reduction at the end
         float den = 0.f;
+#pragma unroll 4
         for (int64_t v = threadIdx.x; v < nvec; v += BLOCK) {
-            V raw = *reinterpret_cast<const V*>(ip + v * EV);
+            V raw = *reinterpret_cast<const V*>(ipv + v * EV);
 #pragma unroll
             for (int q = 0; q < EV; ++q) den += expf(vget<T>(raw, q) - mx);
         }
-        for (int64_t e = nvec * EV + threadIdx.x; e < L; e += BLOCK) den += expf(to_f32<T>(ip[e]) - mx);
+        for (int64_t e = threadIdx.x; e < nscalar; e += BLOCK) den += expf(to_f32<T>(ip[at(e)]) - mx);
         den = block_reduce<NW>(den, red, SumOp{}, 0.f);
         // pass 3: normalise and store
+#pragma unroll 4
         for (int64_t v = threadIdx.x; v < nvec; v += BLOCK) {
-            V raw = *reinterpret_cast<const V*>(ip + v * EV);
+            V raw = *reinterpret_cast<const V*>(ipv + v * EV);
             V res;
 #pragma unroll
             for (int q = 0; q < EV; ++q) vset<T>(res, q, expf(vget<T>(raw, q) - mx) / den);
-            st_global<true>(res, reinterpret_cast<V*>(op + v * EV));
+            st_global<true>(res, reinterpret_cast<V*>(opv + v * EV));
         }
-        for (int64_t e = nvec * EV + threadIdx.x; e < L; e += BLOCK)
-            op[e] = from_f32<T>(expf(to_f32<T>(ip[e]) - mx) / den);
+        for (int64_t e = threadIdx.x; e < nscalar; e += BLOCK)
+            op[at(e)] = from_f32<T>(expf(to_f32<T>(ip[at(e)]) - mx) / den);
     }
 }
 
@@ -196,14 +217,18 @@ template <typename T>
 int launch_3pass(const mi_tile_array* output, const mi_tile_array* input, int64_t L, hipStream_t s) {
     const int64_t M = input->sizes[1];
     const bool al = vec_ok<T>(output, input);
-    dim3 grid((unsigned)M), block(256);
-    if (al)
-        hipLaunchKernelGGL((softmax_3pass_kernel<T, 256, true>), grid, block, 0, s, (T*)output->ptr,
-                           output->strides[1], (const T*)input->ptr, input->strides[1], L, M);
-    else
-        hipLaunchKernelGGL((softmax_3pass_kernel<T, 256, false>), grid, block, 0, s, (T*)output->ptr,
-                           output->strides[1], (const T*)input->ptr, input->strides[1], L, M);
-    set_variant("softmax_3pass_b256");
+    // (few columns: 1024 lanes each, so that a column has sixteen 16-byte loads per lane-slot in flight, not four)
+    const bool wide = M < 1024;
+    dim3 grid((unsigned)M), block(wide ? 1024 : 256);
+#define GO(B, AL)                                                                                          \
+    hipLaunchKernelGGL((softmax_3pass_kernel<T, B, AL>), grid, block, 0, s, (T*)output->ptr, output->strides[1], \
+                       (const T*)input->ptr, input->strides[1], L, M)
+    if (wide && al) GO(1024, true);
+    else if (wide) GO(1024, false);
+    else if (al) GO(256, true);
+    else GO(256, false);
+#undef GO
+    set_variant(wide ? "softmax_3pass_b1024" : "softmax_3pass_b256");
     return launch_status();
 }
 

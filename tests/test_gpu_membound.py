@@ -184,6 +184,37 @@ def test_softmax_both_kernels(orc, M, N, T):
         np.testing.assert_allclose(g.sum(axis=0), 1.0, rtol=1e-5 if T == torch.float32 else 2e-3)
 
 
+@pytest.mark.parametrize("M,N,T,variant", [
+    (7, 100003, torch.float32, "softmax_3pass_b1024"),     # few long columns, odd length: scalar head, vectors, scalar tail
+    (40, 50257, torch.float16, "softmax_3pass_b1024"), (3, 131075, torch.bfloat16, "softmax_3pass_b1024"),
+    (1100, 16388, torch.float32, "softmax_3pass_b256"), (1030, 16391, torch.float32, "softmax_3pass_b256"),
+])
+def test_softmax_columns_too_long_for_registers(ct, orc, M, N, T, variant):
+    """Columns beyond 16384 four-byte (32768 two-byte) elements take three passes; with fewer than 1024 columns a column
+    gets 1024 lanes, and a column that does not start on a 16-byte boundary is walked as head, vectors and tail."""
+    d = softmax.prepare(M=M, N=N, T=T)
+    out = torch.full_like(d.input, float("nan"))
+    ct.softmax_tma_kernel(out, d.input, 1 << (N - 1).bit_length())
+    assert ct.last_variant() == variant
+    ref = orc.softmax(orc.to_julia(d.input))
+    g = orc.to_julia(out).astype(np.float64)
+    if T == torch.float32:
+        assert np.all(np.abs(g - ref) <= 1e-5 * ref + 1e-12)
+    else:
+        assert np.all(np.abs(g - ref) <= 2e-2 * ref + 1e-7)
+    # views: input and output at the same / at different offsets from a 16-byte boundary
+    if T == torch.float32 and M < 100:
+        xb = torch.randn(M, N + 10, device="cuda"); ob = torch.zeros(M, N + 12, device="cuda")
+        for xo, oo in ((3, 3), (1, 2)):
+            ob.zero_()
+            x, o = xb[:, xo:xo + N], ob[:, oo:oo + N]
+            ct.softmax_tma_kernel(o, x, 1 << (N - 1).bit_length())
+            got = orc.to_julia(o).astype(np.float64)
+            r2 = orc.softmax(orc.to_julia(x))
+            assert np.all(np.abs(got - r2) <= 1e-5 * r2 + 1e-12)
+            assert bool((ob[:, :oo] == 0).all()) and bool((ob[:, oo + N:] == 0).all())
+
+
 def test_softmax_tile_smaller_than_column_and_padding(ct, orc):
     """A TILE_SIZE below N covers rows 1..TILE_SIZE only (softmax.jl:29-38); the chunked
     kernel walks cld(n_elems, TILE)*TILE rows, clipped to the array."""
@@ -241,6 +272,25 @@ def test_layernorm_fwd_bwd(orc, M, N, TILE_N, G):
     # the reference's own criterion (layernorm.jl:299,311-313)
     for got, ref in ((r.Y, Y), (r.DX, DX), (r.FINAL_DW, DW), (r.FINAL_DB, DB)):
         assert orc.isapprox(ref, orc.to_julia(got), rtol=1e-2)
+
+
+@pytest.mark.parametrize("M,N,variant", [(9, 65536, "ln_fwd_3pass_b1024_v4"), (5, 100003, "ln_fwd_3pass_b1024"),
+                                         (1030, 16388, "ln_fwd_3pass_b256_v4"), (1025, 16387, "ln_fwd_3pass_b256")])
+def test_layernorm_fwd_rows_too_long_for_registers(ct, orc, M, N, variant):
+    """Rows beyond 16384 elements: three passes, 16-byte accesses when every row allows them, 1024 lanes per row
+    when there are fewer than 1024 rows."""
+    rng = np.random.default_rng(3)
+    X = torch.from_numpy(rng.standard_normal((M, N), dtype=np.float32)).cuda()
+    W = torch.from_numpy(rng.standard_normal(N, dtype=np.float32)).cuda(); B = torch.from_numpy(rng.standard_normal(N, dtype=np.float32)).cuda()
+    Y = torch.full_like(X, float("nan")); Mean = torch.empty(M, device="cuda"); Rstd = torch.empty(M, device="cuda")
+    ct.layer_norm_fwd(X, W, B, Y, Mean, Rstd, 1e-5, 1024)
+    assert ct.last_variant() == variant
+    x = X.cpu().numpy().astype(np.float64)
+    mean = x.mean(axis=1); var = x.var(axis=1); rstd = 1.0 / np.sqrt(var + 1e-5)
+    ref = (x - mean[:, None]) * rstd[:, None] * W.cpu().numpy().astype(np.float64) + B.cpu().numpy().astype(np.float64)
+    np.testing.assert_allclose(Mean.cpu().numpy(), mean, rtol=0, atol=2e-6)
+    np.testing.assert_allclose(Rstd.cpu().numpy(), rstd, rtol=2e-5)
+    np.testing.assert_allclose(Y.cpu().numpy(), ref, rtol=0, atol=2e-4)
 
 
 def test_layernorm_partials_accumulate_into_caller_buffers(ct, orc):

@@ -95,6 +95,35 @@ def test_fmha_random_ragged_shapes(ct):
         assert close(out, ref, 3e-2 if dt == torch.bfloat16 else 2e-2), f"B={B} H={H} Sq={Sq} Skv={Skv} D={D} group={qg} causal={causal} {dt} {ct.last_variant()}"
 
 
+def test_fmha_random_decode_and_chunked_prefill_shapes(ct):
+    """Few queries at the end of a long cache (input_pos > 0), grouped heads, ragged caches: the kernels that split the
+    keys over several workgroups and stack a head group in one query tile, and the unsplit ones where the cache is short.
+    The mask is the kernel's rule -- query i sits at input_pos + i and sees the keys up to there."""
+    rnd = random.Random(7)
+    seen = set()
+    for it in range(60):
+        Sq = rnd.choice([1, 1, 1, 2, 5, 16, 33, 64, 65, 128, 200, 384])
+        Skv = rnd.choice([64, 100, 257, 1000, 2048, 3001, 4096, 6000])
+        causal = rnd.choice([True, True, False])
+        Skv = max(Skv, Sq)
+        pos = rnd.choice([Skv - Sq, Skv - Sq, 0, (Skv - Sq) // 2]) if causal else 0
+        D = rnd.choice([64, 64, 128]); qg = rnd.choice([1, 2, 4, 8]); H = rnd.choice([1, 2, 4]) * qg; B = rnd.choice([1, 2, 8])
+        dt = rnd.choice([torch.float16, torch.bfloat16])
+        d = fmha.prepare(batch=B, heads=H, seq_q=Sq, seq_kv=Skv, d_k=D, d_v=D, query_group_size=qg, causal=causal, T=dt, seed=100 + it)
+        out = torch.full_like(d.Q, NAN)
+        fmha.cutile_fmha(d.Q, d.K, d.V, causal=causal, input_pos=pos, query_group_size=qg, out=out)
+        seen.add(ct.last_variant())
+        K = d.K.repeat_interleave(qg, dim=1).float(); V = d.V.repeat_interleave(qg, dim=1).float()
+        mask = None
+        if causal:
+            mask = torch.arange(Skv, device="cuda")[None, :] <= (torch.arange(Sq, device="cuda")[:, None] + pos)
+        ref = F.scaled_dot_product_attention(d.Q.float(), K, V, attn_mask=mask)
+        assert close(out, ref, 3e-2 if dt == torch.bfloat16 else 2e-2), \
+            f"B={B} H={H} Sq={Sq} Skv={Skv} pos={pos} D={D} group={qg} causal={causal} {dt} {ct.last_variant()}"
+    assert any(v.endswith("_grouped_splitkv") for v in seen) and any(v.endswith("w64q_splitkv") or v.endswith("w32q_splitkv") for v in seen)
+    assert any(v.endswith("_grouped") for v in seen), seen
+
+
 def test_row_kernels_random_shapes(ct):
     rnd = random.Random(5)
     ns = [1, 3, 7, 64, 100, 255, 256, 257, 1000, 1024, 1500, 4096, 5000, 8192, 12000, 20000]

@@ -28,7 +28,7 @@ def check(got, ref, tol=2e-2):
 @pytest.mark.parametrize("tokens,hidden,experts,inter,topk,router", [
     (48, 512, 64, 1024, 8, "randperm"), (128, 512, 32, 1024, 4, "randperm"), (64, 1024, 64, 2048, 8, "randperm"),
     (256, 512, 32, 512, 2, "top2_logits"), (7, 256, 3, 128, 2, "randperm"), (300, 256, 2, 256, 2, "randperm"),
-    (1, 128, 4, 64, 1, "randperm"),
+    (1, 128, 4, 64, 1, "randperm"), (96, 256, 256, 128, 8, "randperm"), (33, 128, 160, 64, 6, "randperm"),
 ])
 def test_moe_end_to_end(orc, tokens, hidden, experts, inter, topk, router):
     d = moe.prepare(num_tokens=tokens, hidden_size=hidden, num_experts=experts, intermediate_size=inter, topk=topk,

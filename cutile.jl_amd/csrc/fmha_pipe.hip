@@ -83,11 +83,12 @@ __device__ __forceinline__ float xhalf_sum(float v) {
     return __uint_as_float(r[0]) + __uint_as_float(r[1]);
 }
 
-// RG: the sequence length is not a multiple of 128 (causal only).  The grid is that of the next multiple; the halves
-// that exist are walked as usual, the last of them re-reads its last row in place of the rows past the end (ragged_offsets),
-// halves past it are never requested (the transfers that would fetch them re-send the last one, as at the end of
-// every walk), and rows past the end are not stored.  Keys past the end lie above the diagonal of every query that
-// exists, so the causal mask removes them.
+// RG: the sequence length is not a multiple of 128.  The grid is that of the next multiple; the halves that exist are
+// walked as usual, the last of them re-reads its last row in place of the rows past the end (ragged_offsets), halves
+// past it are never requested (the transfers that would fetch them re-send the last one, as at the end of every
+// walk), and rows past the end are not stored.  With the causal mask the keys past the end lie above the diagonal of
+// every query that exists, so that mask removes them; without it the walk ends with the pair of halves that holds
+// the last key, and their scores are masked against the sequence length (MASKN = 2 in half_step).
 template <bool RG>
 struct LaneT {
     static constexpr bool ragged = RG;
@@ -108,6 +109,7 @@ struct LaneT {
     bool to_end;                    // (wave-uniform) the walk reaches the last half that exists
     unsigned kdma_b, vdma_b;        // offset of the lane's 16 bytes in transfer wave+2, relative to the start of the half
     unsigned k_rg[2], v_rg[2];      // the two offsets for the last half that exists (rows past the end re-read the last row)
+    int rag_lim;                    // last key that exists, less the 4 keys the upper half-wave's rows are shifted by
 };
 
 // Lane offsets of the two transfers of the last half when rows past `last_row` (0..31) are replaced by that row.
@@ -268,7 +270,8 @@ constexpr int popcount2(int m) { return (m & 1) + ((m >> 1) & 1); }
 constexpr int nth_stream(int m, int k) { return (m & 1) ? k : 1; }
 
 // One step.  CUR / NEXT: bit jj set = stream jj takes part in half j / half j+1 (NEXT is a
-// subset of CUR).  MASKN: stream whose diagonal may cross half j+1 (-1: none).
+// subset of CUR).  MASKN: stream whose diagonal may cross half j+1 (-1: none; 2: both streams, against the end of a
+// ragged sequence instead of a diagonal).
 // On entry cand[jj] holds the raw row maxima of S(j); on exit those of S(j+1).
 //
 // A wave issues in order, so the body is laid out as issue slots -- one MFMA followed by the
@@ -377,8 +380,8 @@ __device__ __forceinline__ void half_step(const unsigned short* Ks, const unsign
     float mx = 0.f;
     auto max_stage = [&]() {
         const int jn = nth_stream(NEXT, mi / 3);
-        const int lim = c.q0[jn] + c.lim0 - kHK * (j + 1);
-        if (MASKN == jn) {
+        const int lim = (MASKN == 2 ? c.rag_lim : c.q0[jn] + c.lim0) - kHK * (j + 1);
+        if (MASKN == jn || MASKN == 2) {
             if (mi % 3 == 0) row_max_stage<true, 0>(s_next[jn], lim, mx, cand[jn]);
             else if (mi % 3 == 1) row_max_stage<true, 1>(s_next[jn], lim, mx, cand[jn]);
             else row_max_stage<true, 2>(s_next[jn], lim, mx, cand[jn]);
@@ -629,7 +632,6 @@ __global__ __launch_bounds__(128) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     Q += (int64_t)head * qs.s2 + (int64_t)batch * qs.s3;
     O += (int64_t)head * os.s2 + (int64_t)batch * os.s3;
 
-    static_assert(CAUSAL || !RG, "keys past the end are only masked by the causal mask");
     const int NT = 4 * nqb;   // 32-query tiles of the grid (RG: of the sequence rounded up to whole workgroups)
     int tq[2];
     if (CAUSAL) {
@@ -652,7 +654,8 @@ __global__ __launch_bounds__(128) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     // instruction arbiter serves the older wave first: the younger one ran 20 % longer.  A raised priority evens
     // the two out (they have the same amount of work), which shortens the kernel.
     if (blockIdx.x >= (gridDim.x >> 1)) __builtin_amdgcn_s_setprio(1);
-    c.nh = CAUSAL ? NT - 2 * qb : NT;
+    // (ragged, no causal mask: up to the pair of halves that holds the last key)
+    c.nh = CAUSAL ? NT - 2 * qb : RG ? (((S + kHK - 1) / kHK + 1) & ~1) : NT;
     c.k_left = c.v_left = c.nh;
     c.to_end = false;
     int last_row = kHK - 1;
@@ -661,6 +664,7 @@ __global__ __launch_bounds__(128) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
         c.to_end = c.nh >= vh;
         if (c.to_end) c.k_left = c.v_left = vh;
         last_row = S - 1 - kHK * (vh - 1);
+        c.rag_lim = S - 1 - 4 * hb;
     }
     c.hb0 = hb == 0;
     {
@@ -836,6 +840,15 @@ __global__ __launch_bounds__(128) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
         }
         WIDE(false, false, j, first, sa, sb);
 #undef WIDE
+    } else if constexpr (RG) {   // (nh >= 6: at least 129 keys)
+        for (; j < nh - 4; j += 2) {
+            STEP(3, 3, -1, j, sa, sb);
+            STEP(3, 3, -1, j + 1, sb, sa);
+        }
+        STEP(3, 3, -1, j, sa, sb);
+        STEP(3, 3, 2, j + 1, sb, sa);    // S(nh - 2) and S(nh - 1): the halves that may reach past the last key
+        STEP(3, 3, 2, j + 2, sa, sb);
+        STEP(3, 0, -1, j + 3, sb, sa);
     } else {
         for (; j < nh - 2; j += 2) {
             STEP(3, 3, -1, j, sa, sb);
@@ -872,6 +885,10 @@ void launch_e(const Problem& p, hipStream_t stream) {
         hipLaunchKernelGGL((fmha_pipe_kernel<E, true, true>), grid, blk, 0, stream, (const unsigned short*)Q->ptr, qs,
                            (const unsigned short*)K->ptr, ks, (const unsigned short*)V->ptr, vs, (unsigned short*)O->ptr,
                            os, S, p.H, p.group, p.scale2, nqb, nbh, mg);
+    else if (S % 128 != 0)
+        hipLaunchKernelGGL((fmha_pipe_kernel<E, false, true>), grid, blk, 0, stream, (const unsigned short*)Q->ptr, qs,
+                           (const unsigned short*)K->ptr, ks, (const unsigned short*)V->ptr, vs, (unsigned short*)O->ptr,
+                           os, S, p.H, p.group, p.scale2, nqb, nbh, mg);
     else if (p.causal)
         hipLaunchKernelGGL((fmha_pipe_kernel<E, true>), grid, blk, 0, stream, (const unsigned short*)Q->ptr, qs,
                            (const unsigned short*)K->ptr, ks, (const unsigned short*)V->ptr, vs, (unsigned short*)O->ptr,
@@ -889,7 +906,7 @@ bool pipe_applicable(const Problem& p) {
     if (Q->sizes[0] != kD || V->sizes[0] != kD) return false;
     const int64_t S = Q->sizes[1];
     if (K->sizes[1] != S || S < 128) return false;
-    if (S % 128 != 0 && !p.causal) return false;   // (a ragged tail needs a key mask of its own without the causal one)
+    if (S % 128 != 0 && S < 129) return false;
     if (!(p.scale2 > 0.f)) return false;
     if (p.causal && p.input_pos != 0) return false;
     if (!vec16(Q) || !vec16(K) || !vec16(V) || !vec16(O)) return false;

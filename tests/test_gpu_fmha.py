@@ -144,8 +144,28 @@ def test_fmha_pipelined_kernel_ragged_causal(ct, orc, batch, heads, s, qg, T):
     check(orc, out, ref, 2e-2 if T == torch.float16 else 3e-2)
 
 
-def test_fmha_ragged_without_the_causal_mask_takes_the_general_kernel(ct, orc):
-    data = fmha.prepare(batch=1, heads=2, seq_q=200, seq_kv=200, causal=False)
+@pytest.mark.parametrize("batch,heads,s,qg,T", [
+    (1, 8, 129, 1, torch.float16), (2, 3, 161, 1, torch.bfloat16), (1, 8, 192, 4, torch.float16), (1, 2, 197, 1, torch.float16),
+    (1, 4, 225, 2, torch.bfloat16), (1, 8, 257, 1, torch.float16), (1, 2, 577, 1, torch.float16), (1, 2, 1000, 2, torch.float16),
+    (1, 1, 1023, 1, torch.float16), (1, 2, 1025, 1, torch.bfloat16),
+])
+def test_fmha_pipelined_kernel_ragged_without_the_causal_mask(ct, orc, batch, heads, s, qg, T):
+    """Without the causal mask nothing hides the keys past the end: the walk stops with the pair of key halves that
+    holds the last key and masks their scores against the sequence length (an odd number of halves ends with one
+    that is masked as a whole)."""
+    data = fmha.prepare(batch=batch, heads=heads, seq_q=s, seq_kv=s, query_group_size=qg, causal=False, T=T)
+    big = torch.full((batch, heads, s + 40, 64), 777.0, dtype=T, device="cuda")
+    out = big[:, :, :s, :]
+    out.fill_(float("nan"))
+    fmha.cutile_fmha(data.Q, data.K, data.V, query_group_size=qg, causal=False, out=out)
+    assert ct.last_variant() == "fmha_pipe_d64_q128_kv32_ring4_ragged"
+    assert bool((big[:, :, s:, :] == 777.0).all())
+    ref = orc.ref_fmha(*(orc.to_julia(t) for t in (data.Q, data.K, data.V)), causal=False, dtype=np.float64)
+    check(orc, out, ref, 2e-2 if T == torch.float16 else 3e-2)
+
+
+def test_fmha_more_keys_than_queries_takes_the_general_kernel(ct, orc):
+    data = fmha.prepare(batch=1, heads=2, seq_q=200, seq_kv=333, causal=False)
     r = run(data)
     assert ct.last_variant().startswith("fmha_dma") or ct.last_variant().startswith("fmha_regstage")
     ref = orc.ref_fmha(*(orc.to_julia(t) for t in (data.Q, data.K, data.V)), causal=False, dtype=np.float64)

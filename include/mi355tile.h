@@ -90,7 +90,7 @@ const char* mi_last_variant(void);
 
 /* ---- vadd: examples/vadd.jl ------------------------------------------------------- */
 /* vec_add_kernel_1d (vadd.jl:10-17): c = a + b; block `bid` owns elements
- * (bid-1)*tile+1 … bid*tile.  f32 / f64 / f16 / bf16. */
+ * (bid-1)*tile+1 … bid*tile.  f32 / f64 / f16 / bf16, Int32 / Int64 (wrapping, as Julia's +). */
 int mi_vec_add_kernel_1d(const mi_tile_array* a, const mi_tile_array* b, const mi_tile_array* c,
                          int tile, void* stream);
 /* vec_add_kernel_2d (vadd.jl:20-28): same on (tile_x, tile_y) tiles of 2-D arrays. */

@@ -61,6 +61,51 @@ def test_vadd_strided_views_and_misaligned(ct, orc):
     assert torch.equal(C[:, :100], A[:, :100] + B[:, :100]) and torch.all(C[:, 100:] == 0)
 
 
+@pytest.mark.parametrize("T", [torch.float32, torch.float16, torch.bfloat16, torch.float64, torch.int32, torch.int64])
+def test_vadd_views_off_a_16_byte_boundary_and_integers(ct, T):
+    """Views that start 1, 2, 3 or 5 elements past a 16-byte boundary: a head up to the boundary, 16-byte vectors and
+    a tail when all three arrays sit at the same offset, element by element when they do not; the gather kernel with
+    three different lengths; 2-D views of a padded parent.  Integers wrap like Julia's +.  What lies around every
+    destination view stays as it was."""
+    g = torch.Generator(device="cuda"); g.manual_seed(9)
+
+    def rnd(*shape):
+        if T.is_floating_point:
+            return torch.randn(*shape, device="cuda", generator=g).to(T)
+        return (torch.randint(-2 ** 31, 2 ** 31 - 1, shape, device="cuda", generator=g).to(T) * (3 if T == torch.int64 else 1))
+
+    for nn in (1, 3, 4, 5, 17, 1000, 4099, 70001):
+        for off in (0, 1, 2, 3, 5):
+            x, y = rnd(nn + 8), rnd(nn + 8)
+            z = torch.zeros(nn + 8, device="cuda", dtype=T)
+            ct.vec_add_kernel_1d(x[off:off + nn], y[off:off + nn], z[off:off + nn], 1024)
+            assert torch.equal(z[off:off + nn], x[off:off + nn] + y[off:off + nn]), (nn, off, ct.last_variant())
+            assert bool((z[:off] == 0).all()) and bool((z[off + nn:] == 0).all())
+            if nn >= 64:
+                assert ct.last_variant().startswith("vadd_vec16")
+            z.zero_()
+            ct.vec_add_kernel_1d(x[off:off + nn], y[1:1 + nn], z[2:2 + nn], 1024)       # offsets that do not agree
+            assert torch.equal(z[2:2 + nn], x[off:off + nn] + y[1:1 + nn]) and bool((z[:2] == 0).all()) and bool((z[2 + nn:] == 0).all())
+            na, nb = max(1, nn - 3), nn + 5
+            zz = torch.full((nn + 8,), 7, device="cuda", dtype=T)
+            ct.vec_add_kernel_1d_gather(x[off:off + na], y[off:off + nb], zz[off:off + nn], 256)
+            ref = torch.zeros(nn, device="cuda", dtype=T)
+            ref[:na] += x[off:off + na]
+            ref += y[off:off + nb][:nn]
+            assert torch.equal(zz[off:off + nn], ref), (nn, off, ct.last_variant())
+            assert bool((zz[:off] == 7).all()) and bool((zz[off + nn:] == 7).all())
+    v = 16 // torch.empty(0, dtype=T).element_size()
+    for r, cfull, ccols, coff, vec in [(33, 64, 40, 0, True), (100, 1000, 1000 - 2 * v, v, True), (7, 520, 513, 0, True),
+                                       (5, 16, 3, 0, v <= 3), (300, 128, 128, 0, True), (9, 100, 50, 1, False)]:
+        X, Y = rnd(r, cfull), rnd(r, cfull)
+        Z = torch.zeros(r, cfull, device="cuda", dtype=T)
+        ct.vec_add_kernel_2d(X[:, coff:coff + ccols], Y[:, coff:coff + ccols], Z[:, coff:coff + ccols], 32, 32)
+        assert torch.equal(Z[:, coff:coff + ccols], X[:, coff:coff + ccols] + Y[:, coff:coff + ccols]), (r, cfull, ccols, coff)
+        assert bool((Z[:, :coff] == 0).all()) and bool((Z[:, coff + ccols:] == 0).all())
+        if cfull % v == 0:
+            assert (ct.last_variant() != "vadd_2d_strided") == vec, (r, cfull, ccols, coff, ct.last_variant())
+
+
 def test_vadd_gather_out_of_bounds_semantics(ct, orc):
     """test/device/gather_scatter.jl:75-113: an out-of-bounds gather lane reads 0, an
     out-of-bounds scatter lane is dropped."""

@@ -8,8 +8,9 @@
 //     small matrices): a V x V block per lane transposed in registers, 16-byte traffic through an
 //     XOR-swizzled LDS tile in both directions, workgroup ids walking 8x8 super-tiles
 //     (transpose_micro_kernel);
-//   * everything else: 64x64 tiles through a padded LDS tile (pitch 65 elements: both the
-//     scattered writes and the gathered reads hit 64 distinct banks), 16-byte global accesses
+//     sizes that are not multiples of a vector are taken too when the leading dimensions are (edge tiles element-wise);
+//   * everything else: 64x64 (large 2- and 4-byte matrices: 128x128) tiles through a padded LDS tile (pitch + 1
+//     element: both the scattered writes and the gathered reads hit distinct banks), 16-byte global accesses
 //     where alignment allows, element-wise with bounds checks otherwise (transpose_kernel).
 // Algorithmic traffic: 2 * m * n * sizeof(T) bytes.
 #include "common.h"
@@ -19,9 +20,6 @@ namespace {
 
 using namespace mi;
 
-constexpr int kTile = 64;
-constexpr int kBlock = 256;
-constexpr int kPitch = kTile + 1;
 
 template <typename T, int N> struct VecOf {
     typedef T type __attribute__((ext_vector_type(N)));
@@ -30,7 +28,7 @@ template <typename T, int N> struct VecOf {
 // VEC: true  -> every 16-byte vector is either fully inside or fully outside the matrix
 //               and 16-byte aligned (checked on the host);
 //      false -> element-wise accesses with per-element bounds checks.
-template <typename T, bool VEC>
+template <typename T, bool VEC, int kTile = 64, int kBlock = 256>
 __global__ __launch_bounds__(kBlock) void transpose_kernel(const T* __restrict__ x, int64_t ldx,
                                                            T* __restrict__ y, int64_t ldy,
                                                            int64_t m, int64_t n) {
@@ -39,6 +37,7 @@ __global__ __launch_bounds__(kBlock) void transpose_kernel(const T* __restrict__
     constexpr int RP = kBlock / VR;          // tile rows covered per pass
     constexpr int PASSES = kTile / RP;
     using VT = typename VecOf<T, V>::type;
+    constexpr int kPitch = kTile + 1;
     __shared__ T lds[kTile * kPitch];
 
     const int64_t m0 = (int64_t)blockIdx.x * kTile;  // along x dim 0
@@ -100,7 +99,10 @@ typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
 // memory system needs to move a strided run at the rate of a linear copy, and two workgroups fill a
 // CU -- and 64 x 128 tiles with 256 lanes (five workgroups per CU) when there are too few tiles for
 // that.  The 2- and 8-byte shapes are chosen the same way (launch_micro).
-template <typename T, int TM, int TN, bool STREAM = true, int NT = 256>
+// RAGGED: m or n is not a multiple of V (the leading dimensions still are, so every vector inside the matrix is
+// aligned: a view of a padded parent).  Tiles on the edge then load and store the vectors that cross it element by
+// element; interior tiles are unaffected.
+template <typename T, int TM, int TN, bool STREAM = true, int NT = 256, bool RAGGED = false>
 __global__ __launch_bounds__(NT) void transpose_micro_kernel(const T* __restrict__ x, int64_t ldx,
                                                               T* __restrict__ y, int64_t ldy, int64_t m,
                                                               int64_t n, int tiles_m, int tiles_n, int order) {
@@ -141,7 +143,15 @@ __global__ __launch_bounds__(NT) void transpose_micro_kernel(const T* __restrict
         } else if (gm < m) {
 #pragma unroll
             for (int c = 0; c < V; ++c)
-                if (gn + c < n) r[c] = ld_global<STREAM>(reinterpret_cast<const VT*>(x + gm + (gn + c) * ldx));
+                if (gn + c < n) {
+                    if (!RAGGED || gm + V <= m) {
+                        r[c] = ld_global<STREAM>(reinterpret_cast<const VT*>(x + gm + (gn + c) * ldx));
+                    } else {
+#pragma unroll
+                        for (int q = 0; q < V; ++q)
+                            if (gm + q < m) r[c][q] = x[gm + q + (gn + c) * ldx];
+                    }
+                }
         }
 #pragma unroll
         for (int q = 0; q < V; ++q) {
@@ -160,13 +170,27 @@ __global__ __launch_bounds__(NT) void transpose_micro_kernel(const T* __restrict
         const int64_t gn = n0 + V * jv, gm = m0 + row;
         if (interior || (gn < n && gm < m)) {
             VT t = *reinterpret_cast<const VT*>(&lds[row * TN + V * (jv ^ ((row / V) & (SLOTS - 1)))]);
-            st_global<true>(t, reinterpret_cast<VT*>(y + gn + gm * ldy));
+            if (!RAGGED || interior || gn + V <= n) {
+                st_global<true>(t, reinterpret_cast<VT*>(y + gn + gm * ldy));
+            } else {
+#pragma unroll
+                for (int e = 0; e < V; ++e)
+                    if (gn + e < n) y[gn + e + gm * ldy] = t[e];
+            }
         }
     }
 }
 
-int launch4(const mi_tile_array* x, const mi_tile_array* y, hipStream_t s) {
+template <typename T, int TM, int TN, int NT>
+int launch_micro_as(const mi_tile_array* x, const mi_tile_array* y, hipStream_t s, const char* name_stream,
+                    const char* name_cached, bool ragged);
+
+int launch4(const mi_tile_array* x, const mi_tile_array* y, hipStream_t s, bool ragged) {
     const int64_t m = x->sizes[0], n = x->sizes[1];
+    if (ragged)
+        return cld(m, (int64_t)128) * cld(n, (int64_t)128) >= 1024
+                   ? launch_micro_as<unsigned, 128, 128, 1024>(x, y, s, "transpose4_128x128_t1024_regmicro_ragged", "", true)
+                   : launch_micro_as<unsigned, 64, 128, 256>(x, y, s, "transpose4_64x128_regmicro_ragged", "", true);
     // measured best on MI355X for 8192^2 fp32: 128 x 128 tiles of 1024 lanes, 8x8 super-tiles (90 us; 64 x 128
     // tiles of 256 lanes 104 us); the big shape needs enough tiles to keep two workgroups on every CU
     int tile = cld(m, (int64_t)128) * cld(n, (int64_t)128) >= 1024 ? 9 : 2, order = 2;
@@ -216,12 +240,18 @@ int launch4(const mi_tile_array* x, const mi_tile_array* y, hipStream_t s) {
 // overrides it for tuning): the large shapes keep runs of at least 512 bytes on both sides.
 template <typename T, int TM, int TN, int NT>
 int launch_micro_as(const mi_tile_array* x, const mi_tile_array* y, hipStream_t s, const char* name_stream,
-                    const char* name_cached) {
+                    const char* name_cached, bool ragged) {
     const int64_t m = x->sizes[0], n = x->sizes[1];
     const int64_t tm_ = cld(m, (int64_t)TM), tn_ = cld(n, (int64_t)TN);
     const int64_t blocks = ((tm_ + 7) / 8) * ((tn_ + 7) / 8) * 64;
     if (blocks > 0x7fffffffLL || tm_ > 0x3fffffff || tn_ > 0x3fffffff) return MI_E_GRID;
     const bool st = stream_hint(2 * m * n * (int64_t)sizeof(T));
+    if (ragged) {
+        hipLaunchKernelGGL((transpose_micro_kernel<T, TM, TN, true, NT, true>), dim3((unsigned)blocks), dim3(NT), 0, s,
+                           (const T*)x->ptr, x->strides[1], (T*)y->ptr, y->strides[1], m, n, (int)tm_, (int)tn_, 2);
+        set_variant(name_stream);
+        return launch_status();
+    }
     if (st) hipLaunchKernelGGL((transpose_micro_kernel<T, TM, TN, true, NT>), dim3((unsigned)blocks), dim3(NT), 0, s,
                                (const T*)x->ptr, x->strides[1], (T*)y->ptr, y->strides[1], m, n, (int)tm_, (int)tn_, 2);
     else hipLaunchKernelGGL((transpose_micro_kernel<T, TM, TN, false, NT>), dim3((unsigned)blocks), dim3(NT), 0, s,
@@ -233,67 +263,86 @@ int launch_micro_as(const mi_tile_array* x, const mi_tile_array* y, hipStream_t 
 // measured on MI355X, 8192^2: 8-byte 205 us with 128 x 64 tiles of 1024 lanes (64 x 64 of 256 lanes 221 us; the
 // padded-tile kernel 305 us); 2-byte 51 us with 256 x 256 tiles of 1024 lanes (128 x 128 of 256 lanes 56 us; the
 // padded-tile kernel 67 us).  At 4096^2 the smaller tiles win, there are too few of the large ones to fill the chip.
-int launch8(const mi_tile_array* x, const mi_tile_array* y, hipStream_t s) {
+int launch8(const mi_tile_array* x, const mi_tile_array* y, hipStream_t s, bool ragged) {
     const int64_t m = x->sizes[0], n = x->sizes[1];
     const int64_t t64 = cld(m, (int64_t)64) * cld(n, (int64_t)64);
+    if (ragged)
+        return t64 >= 1024 ? launch_micro_as<uint64_t, 64, 64, 1024>(x, y, s, "transpose8_64x64_t1024_regmicro_ragged", "", true)
+                           : launch_micro_as<uint64_t, 64, 64, 256>(x, y, s, "transpose8_64x64_regmicro_ragged", "", true);
     int tile = t64 >= 8192 ? 3 : t64 >= 1024 ? 2 : 0;
     if (const char* e = getenv("MI_TRANSPOSE_TILE")) tile = atoi(e);
     switch (tile) {
-        case 1: return launch_micro_as<uint64_t, 64, 128, 1024>(x, y, s, "transpose8_64x128_t1024_regmicro", "transpose8_64x128_t1024_regmicro_cached");
-        case 2: return launch_micro_as<uint64_t, 64, 64, 1024>(x, y, s, "transpose8_64x64_t1024_regmicro", "transpose8_64x64_t1024_regmicro_cached");
-        case 3: return launch_micro_as<uint64_t, 128, 64, 1024>(x, y, s, "transpose8_128x64_t1024_regmicro", "transpose8_128x64_t1024_regmicro_cached");
-        case 4: return launch_micro_as<uint64_t, 32, 128, 256>(x, y, s, "transpose8_32x128_regmicro", "transpose8_32x128_regmicro_cached");
-        default: return launch_micro_as<uint64_t, 64, 64, 256>(x, y, s, "transpose8_64x64_regmicro", "transpose8_64x64_regmicro_cached");
+        case 1: return launch_micro_as<uint64_t, 64, 128, 1024>(x, y, s, "transpose8_64x128_t1024_regmicro", "transpose8_64x128_t1024_regmicro_cached", false);
+        case 2: return launch_micro_as<uint64_t, 64, 64, 1024>(x, y, s, "transpose8_64x64_t1024_regmicro", "transpose8_64x64_t1024_regmicro_cached", false);
+        case 3: return launch_micro_as<uint64_t, 128, 64, 1024>(x, y, s, "transpose8_128x64_t1024_regmicro", "transpose8_128x64_t1024_regmicro_cached", false);
+        case 4: return launch_micro_as<uint64_t, 32, 128, 256>(x, y, s, "transpose8_32x128_regmicro", "transpose8_32x128_regmicro_cached", false);
+        default: return launch_micro_as<uint64_t, 64, 64, 256>(x, y, s, "transpose8_64x64_regmicro", "transpose8_64x64_regmicro_cached", false);
     }
 }
 
-int launch2(const mi_tile_array* x, const mi_tile_array* y, hipStream_t s) {
+int launch2(const mi_tile_array* x, const mi_tile_array* y, hipStream_t s, bool ragged) {
     const int64_t m = x->sizes[0], n = x->sizes[1];
     const int64_t t128 = cld(m, (int64_t)128) * cld(n, (int64_t)128);
+    if (ragged)
+        return t128 >= 1024 ? launch_micro_as<uint16_t, 128, 256, 512>(x, y, s, "transpose2_128x256_t512_regmicro_ragged", "", true)
+                            : launch_micro_as<uint16_t, 128, 128, 256>(x, y, s, "transpose2_128x128_regmicro_ragged", "", true);
     int tile = t128 >= 4096 ? 3 : t128 >= 1024 ? 2 : 0;
     if (const char* e = getenv("MI_TRANSPOSE_TILE")) tile = atoi(e);
     switch (tile) {
-        case 1: return launch_micro_as<uint16_t, 256, 128, 512>(x, y, s, "transpose2_256x128_t512_regmicro", "transpose2_256x128_t512_regmicro_cached");
-        case 2: return launch_micro_as<uint16_t, 128, 256, 512>(x, y, s, "transpose2_128x256_t512_regmicro", "transpose2_128x256_t512_regmicro_cached");
-        case 3: return launch_micro_as<uint16_t, 256, 256, 1024>(x, y, s, "transpose2_256x256_t1024_regmicro", "transpose2_256x256_t1024_regmicro_cached");
-        case 4: return launch_micro_as<uint16_t, 256, 128, 256>(x, y, s, "transpose2_256x128_regmicro", "transpose2_256x128_regmicro_cached");
-        default: return launch_micro_as<uint16_t, 128, 128, 256>(x, y, s, "transpose2_128x128_regmicro", "transpose2_128x128_regmicro_cached");
+        case 1: return launch_micro_as<uint16_t, 256, 128, 512>(x, y, s, "transpose2_256x128_t512_regmicro", "transpose2_256x128_t512_regmicro_cached", false);
+        case 2: return launch_micro_as<uint16_t, 128, 256, 512>(x, y, s, "transpose2_128x256_t512_regmicro", "transpose2_128x256_t512_regmicro_cached", false);
+        case 3: return launch_micro_as<uint16_t, 256, 256, 1024>(x, y, s, "transpose2_256x256_t1024_regmicro", "transpose2_256x256_t1024_regmicro_cached", false);
+        case 4: return launch_micro_as<uint16_t, 256, 128, 256>(x, y, s, "transpose2_256x128_regmicro", "transpose2_256x128_regmicro_cached", false);
+        default: return launch_micro_as<uint16_t, 128, 128, 256>(x, y, s, "transpose2_128x128_regmicro", "transpose2_128x128_regmicro_cached", false);
     }
 }
 
 // 1-byte, measured: 16384^2 103 us with 256 x 512 tiles of 512 lanes (256 x 256 of 256 lanes 118 us); 8192^2 22 us
 // with 256 x 256 (24 us with 256 x 512; the padded-tile kernel 46 us)
-int launch1(const mi_tile_array* x, const mi_tile_array* y, hipStream_t s) {
+int launch1(const mi_tile_array* x, const mi_tile_array* y, hipStream_t s, bool ragged) {
     const int64_t m = x->sizes[0], n = x->sizes[1];
+    if (ragged) return launch_micro_as<uint8_t, 256, 256, 256>(x, y, s, "transpose1_256x256_regmicro_ragged", "", true);
     int tile = cld(m, (int64_t)256) * cld(n, (int64_t)256) >= 4096 ? 2 : 0;
     if (const char* e = getenv("MI_TRANSPOSE_TILE")) tile = atoi(e);
     switch (tile) {
-        case 1: return launch_micro_as<uint8_t, 512, 256, 512>(x, y, s, "transpose1_512x256_t512_regmicro", "transpose1_512x256_t512_regmicro_cached");
-        case 2: return launch_micro_as<uint8_t, 256, 512, 512>(x, y, s, "transpose1_256x512_t512_regmicro", "transpose1_256x512_t512_regmicro_cached");
-        default: return launch_micro_as<uint8_t, 256, 256, 256>(x, y, s, "transpose1_256x256_regmicro", "transpose1_256x256_regmicro_cached");
+        case 1: return launch_micro_as<uint8_t, 512, 256, 512>(x, y, s, "transpose1_512x256_t512_regmicro", "transpose1_512x256_t512_regmicro_cached", false);
+        case 2: return launch_micro_as<uint8_t, 256, 512, 512>(x, y, s, "transpose1_256x512_t512_regmicro", "transpose1_256x512_t512_regmicro_cached", false);
+        default: return launch_micro_as<uint8_t, 256, 256, 256>(x, y, s, "transpose1_256x256_regmicro", "transpose1_256x256_regmicro_cached", false);
     }
 }
 
-template <typename T>
-int launch(const mi_tile_array* x, const mi_tile_array* y, hipStream_t s) {
+template <typename T, int TILE, int BLOCK>
+int launch_tile(const mi_tile_array* x, const mi_tile_array* y, hipStream_t s) {
     constexpr int V = 16 / sizeof(T);
     const int64_t m = x->sizes[0], n = x->sizes[1];
     const int64_t ldx = x->strides[1], ldy = y->strides[1];
-    const int64_t gx = cld(m, (int64_t)kTile), gy = cld(n, (int64_t)kTile);
+    const int64_t gx = cld(m, (int64_t)TILE), gy = cld(n, (int64_t)TILE);
     if (gx > 0x7fffffffLL) return MI_E_GRID;
     const bool vec = (m % V == 0) && (n % V == 0) && (ldx % V == 0) && (ldy % V == 0) &&
                      aligned(x->ptr, 16) && aligned(y->ptr, 16);
-    dim3 grid((unsigned)gx, (unsigned)(gy < 65535 ? gy : 65535)), block(kBlock);
+    dim3 grid((unsigned)gx, (unsigned)(gy < 65535 ? gy : 65535)), block(BLOCK);
     if (vec) {
-        hipLaunchKernelGGL((transpose_kernel<T, true>), grid, block, 0, s, (const T*)x->ptr, ldx,
+        hipLaunchKernelGGL((transpose_kernel<T, true, TILE, BLOCK>), grid, block, 0, s, (const T*)x->ptr, ldx,
                            (T*)y->ptr, ldy, m, n);
-        set_variant("transpose_lds64_vec16");
+        set_variant(TILE == 64 ? "transpose_lds64_vec16" : "transpose_lds128_vec16");
     } else {
-        hipLaunchKernelGGL((transpose_kernel<T, false>), grid, block, 0, s, (const T*)x->ptr, ldx,
+        hipLaunchKernelGGL((transpose_kernel<T, false, TILE, BLOCK>), grid, block, 0, s, (const T*)x->ptr, ldx,
                            (T*)y->ptr, ldy, m, n);
-        set_variant("transpose_lds64_elem");
+        set_variant(TILE == 64 ? "transpose_lds64_elem" : "transpose_lds128_elem");
     }
     return launch_status();
+}
+
+// Sizes or strides that rule out the register micro-transpose.  Large matrices of 2- and 4-byte elements take
+// 128 x 128 tiles of 1024 lanes (runs of 256 / 512 bytes instead of 128 / 256).
+template <typename T>
+int launch(const mi_tile_array* x, const mi_tile_array* y, hipStream_t s) {
+    int big = sizeof(T) <= 4 && sizeof(T) >= 2 && cld(x->sizes[0], (int64_t)128) * cld(x->sizes[1], (int64_t)128) >= 512;
+    if (const char* e = getenv("MI_TRANSPOSE_FALLBACK_TILE")) big = atoi(e) == 128 && sizeof(T) <= 4;
+    if constexpr (sizeof(T) <= 4) {
+        if (big) return launch_tile<T, 128, 1024>(x, y, s);
+    }
+    return launch_tile<T, 64, 256>(x, y, s);
 }
 
 }  // namespace
@@ -313,15 +362,18 @@ extern "C" int mi_transpose_kernel(const mi_tile_array* x, const mi_tile_array* 
     if ((n > 1 && x->strides[1] < m) || (m > 1 && y->strides[1] < n)) return MI_E_STRIDE;
     hipStream_t s = (hipStream_t)stream;
     // the register micro-transpose moves whole 16-byte vectors of v elements on both sides
+    // 0: not possible; 1: whole vectors everywhere; 2: aligned columns, but m or n is not a multiple of v (edge tiles
+    // move the vectors that cross the edge element by element)
     auto micro = [&](int v) {
-        return m % v == 0 && n % v == 0 && x->strides[1] % v == 0 && y->strides[1] % v == 0 &&
-               aligned(x->ptr, 16) && aligned(y->ptr, 16);
+        if (!((n == 1 || x->strides[1] % v == 0) && (m == 1 || y->strides[1] % v == 0) && aligned(x->ptr, 16) && aligned(y->ptr, 16)))
+            return 0;
+        return m % v == 0 && n % v == 0 ? 1 : 2;
     };
     switch (dtype_size(x->dtype)) {
-        case 1: return micro(16) ? launch1(x, y, s) : launch<uint8_t>(x, y, s);
-        case 2: return micro(8) ? launch2(x, y, s) : launch<uint16_t>(x, y, s);
-        case 4: return micro(4) ? launch4(x, y, s) : launch<uint32_t>(x, y, s);
-        case 8: return micro(2) ? launch8(x, y, s) : launch<uint64_t>(x, y, s);
+        case 1: return micro(16) ? launch1(x, y, s, micro(16) == 2) : launch<uint8_t>(x, y, s);
+        case 2: return micro(8) ? launch2(x, y, s, micro(8) == 2) : launch<uint16_t>(x, y, s);
+        case 4: return micro(4) ? launch4(x, y, s, micro(4) == 2) : launch<uint32_t>(x, y, s);
+        case 8: return micro(2) ? launch8(x, y, s, micro(2) == 2) : launch<uint64_t>(x, y, s);
         default: return MI_E_DTYPE;
     }
 }

@@ -200,6 +200,31 @@ def test_transpose_every_element_size_takes_the_register_path(ct, T, isz):
     assert "regmicro" not in ct.last_variant() and torch.equal(y, x.t())
 
 
+@pytest.mark.parametrize("T,isz", [(torch.float8_e4m3fn, 1), (torch.float16, 2), (torch.float32, 4), (torch.float64, 8)])
+def test_transpose_views_of_a_padded_parent_with_ragged_sizes(ct, T, isz):
+    """Sizes that are not multiples of a 16-byte vector inside parents whose leading dimensions are: the register path
+    with edge tiles that move the vectors crossing the edge element by element.  Small and large tile variants; what
+    lies around the destination view stays as it was.  A dense matrix with such sizes has misaligned columns and takes
+    the padded-tile kernel."""
+    v = 16 // isz
+    iv = {1: torch.uint8, 2: torch.int16, 4: torch.int32, 8: torch.int64}[isz]
+    g = torch.Generator(device="cuda"); g.manual_seed(200 + isz)
+    big = {1: (4100, 4099), 2: (4090, 4093), 4: (4095, 4090), 8: (2051, 2049)}[isz]
+    for r, c in [(1, 1), (3, 5), (v + 1, v + 1), (100, 37), (257, 129), (1000, 999), (130, 4097), big]:
+        R, C = (r + v - 1) // v * v + v, (c + v - 1) // v * v + v
+        xb = torch.randint(0, 256, (R, C * isz), device="cuda", generator=g).to(torch.uint8).view(iv)
+        yb = torch.full((C, R), 85, dtype=iv, device="cuda")
+        x, y = xb[:r, :c], yb[:c, :r]
+        ct.transpose_kernel(x.view(T), y.view(T), 64, 64)
+        assert ct.last_variant().endswith("_regmicro_ragged"), ct.last_variant()
+        assert torch.equal(y, x.t()), (r, c)
+        assert bool((yb[c:, :] == 85).all()) and bool((yb[:, r:] == 85).all()), (r, c)
+    x = torch.randint(0, 256, (1001, 999 * isz), device="cuda", generator=g).to(torch.uint8).view(iv)
+    y = torch.empty(999, 1001, dtype=iv, device="cuda")
+    ct.transpose_kernel(x.view(T), y.view(T), 64, 64)
+    assert ct.last_variant().startswith("transpose_lds") and torch.equal(y, x.t())
+
+
 def test_transpose_full_size_involution():
     d = transpose.prepare(benchmark=True)
     r = transpose.run(d)

@@ -355,6 +355,20 @@ def bench_kernels(ct, which, cpu, nruns=NRUNS, warmup=WARMUP):
             e["cpu_note"] = f"numpy restatement of ref_fmha, 4 of 128 (batch, head) pairs x32, BLAS {ncores} threads"
         res["fmha"] = e
         del d
+        # The same entry point on the other end of its argument range (input_pos, fmha.jl:45-46): one new token per
+        # sequence against a cache of 4096 keys.  Bound by reading the cache once.
+        for key, (B, H, G, Skv) in (("fmha_decode", (8, 16, 1, 4096)), ("fmha_decode_grouped", (32, 32, 4, 2048))):
+            dd = fmha.prepare(batch=B, heads=H, seq_q=1, seq_kv=Skv, query_group_size=G, causal=True)
+            od = torch.empty_like(dd.Q)
+            Qd, Kd, Vd, Od = (ct.TileArray(t) for t in (dd.Q, dd.K, dd.V, od))
+            go = lambda: ct.fmha_kernel(Qd, Kd, Vd, Od, scale, Skv - 1, 64, H, 128, 128, G, True, True)
+            go()
+            nb = (dd.K.numel() + dd.V.numel() + 2 * dd.Q.numel()) * 2
+            ed = _entry(f"FMHA decode: 1 query per sequence at input_pos = {Skv - 1}, {B}x{H} heads in groups of {G}, {Skv} cached keys, f16 "
+                        "(keys split over workgroups + combine kernel: two launches)", go, nb, "GB/s", "hbm", HBM_PEAK_GBS, "f16", nruns, warmup)
+            ed["variant"] = ct.last_variant()
+            res[key] = ed
+            del dd
     if want("fft"):
         d = fft.prepare(benchmark=True)
         F0, F1, F2 = d.factors

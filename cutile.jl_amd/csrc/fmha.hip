@@ -45,7 +45,7 @@
 #include <stdlib.h>
 #include <string.h>
 
-#include <mutex>
+#include "shared_scratch.h"
 
 namespace {
 
@@ -683,18 +683,10 @@ __global__ __launch_bounds__(256) void fmha_combine_kernel(const float* __restri
     *reinterpret_cast<s16x4*>(O + head * os.s2 + batch * os.s3 + (int64_t)q * os.s1 + 4 * c) = out;
 }
 
-// Scratch of the split launches: one array per GPU, shared by its streams.  A launch that follows one from another
-// stream first waits for an event recorded there; a stream under capture is not given the array.
+// Scratch of the split launches (see shared_scratch.h for how its users are ordered).
 constexpr int64_t kPartFloats = 16 * 1024 * 1024;   // 64 MiB
 static __device__ __align__(256) float fmha_part_scratch[kPartFloats];
-struct PartState {
-    std::mutex mu;
-    float* scratch = nullptr;
-    hipEvent_t done = nullptr;
-    hipStream_t last = nullptr;
-    bool used = false, broken = false;
-};
-PartState g_part[16];
+SharedScratch g_part[16];
 
 // Number of parts for the launch, 0 = no split.
 int pick_parts(int64_t wgs, int64_t rows, int D, int Sq, int Skv, bool causal, int input_pos) {
@@ -711,42 +703,6 @@ int pick_parts(int64_t wgs, int64_t rows, int D, int Sq, int Skv, bool causal, i
     if (parts > 64) parts = 64;
     while (parts >= 2 && parts * rows * (D + kPartPad) > kPartFloats) --parts;
     return parts >= 2 ? (int)parts : 0;
-}
-
-// The scratch for a split launch on stream s, ordered after its previous user; nullptr if it can not be had.
-float* acquire_parts(hipStream_t s, std::unique_lock<std::mutex>& lock) {
-    int dev = 0;
-    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 16) return nullptr;
-    hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
-    if (hipStreamIsCapturing(s, &cap) != hipSuccess || cap != hipStreamCaptureStatusNone) return nullptr;
-    PartState& st = g_part[dev];
-    lock = std::unique_lock<std::mutex>(st.mu);
-    if (st.broken) return nullptr;
-    if (!st.scratch) {
-        if (hipGetSymbolAddress((void**)&st.scratch, HIP_SYMBOL(fmha_part_scratch)) != hipSuccess ||
-            hipEventCreateWithFlags(&st.done, hipEventDisableTiming) != hipSuccess) {
-            st.broken = true;
-            st.scratch = nullptr;
-            (void)hipGetLastError();
-            return nullptr;
-        }
-    }
-    if (st.used && st.last != s) {
-        bool ordered;
-        if (hipEventRecord(st.done, st.last) == hipSuccess) {
-            ordered = hipStreamWaitEvent(s, st.done, 0) == hipSuccess;
-        } else {   // that stream no longer exists: what it was given is done once the device is idle
-            (void)hipGetLastError();
-            ordered = hipDeviceSynchronize() == hipSuccess;
-        }
-        if (!ordered) {
-            (void)hipGetLastError();
-            return nullptr;
-        }
-    }
-    st.last = s;
-    st.used = true;
-    return st.scratch;
 }
 
 bool vec16(const mi_tile_array* a) {
@@ -770,7 +726,7 @@ void launch(dim3 grid, hipStream_t s, bool causal, const mi_tile_array* Q, const
         const int64_t rows = (int64_t)nbh * Sq * pack;
         if (const int parts = pick_parts((int64_t)nqb * nbh, rows, D, Sq, Skv, causal, input_pos)) {
             std::unique_lock<std::mutex> lock;
-            if (float* scratch = acquire_parts(s, lock)) {
+            if (float* scratch = (float*)acquire_shared_scratch(g_part, HIP_SYMBOL(fmha_part_scratch), s, lock)) {
                 dim3 gs((unsigned)(nqb * nbh * parts));
                 if (causal)
                     hipLaunchKernelGGL((fmha_fwd_dma_kernel<E, D, JT, true, true>), gs, blk, 0, s, (const unsigned short*)Q->ptr, qs,

@@ -30,9 +30,8 @@
 // re-read the last valid rows / chunks on the way in and clip their stores.  K is walked in whole
 // groups of four steps (128); in the last group the 16-byte chunks at k >= K are fetched from a
 // 16-byte block of zeros instead (both operands, so padding never meets a non-finite value).
-#include <mutex>
-
 #include "gemm_direct.h"
+#include "shared_scratch.h"
 
 namespace {
 
@@ -365,14 +364,7 @@ __global__ __launch_bounds__(256) void splitk_reduce(const float* __restrict__ p
     }
 }
 
-struct SplitState {
-    std::mutex mu;
-    float* scratch = nullptr;
-    hipEvent_t done = nullptr;
-    hipStream_t last = nullptr;
-    bool used = false, broken = false;
-};
-SplitState g_split[16];
+SharedScratch g_split[16];
 
 // Parts and part length for the problem, or 0 if a split does not apply.
 int pick_split(const Problem& p, int* kchunk) {
@@ -405,51 +397,22 @@ int pick_split(const Problem& p, int* kchunk) {
 
 template <typename E>
 bool launch_split(const Problem& p, hipStream_t s, int parts, int kchunk) {
-    int dev = 0;
-    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 16) return false;
-    hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
-    if (hipStreamIsCapturing(s, &cap) != hipSuccess || cap != hipStreamCaptureStatusNone) return false;
-    SplitState& st = g_split[dev];
-    std::lock_guard<std::mutex> lock(st.mu);
-    if (st.broken) return false;
-    if (!st.scratch) {
-        if (hipGetSymbolAddress((void**)&st.scratch, HIP_SYMBOL(splitk_scratch)) != hipSuccess ||
-            hipEventCreateWithFlags(&st.done, hipEventDisableTiming) != hipSuccess) {
-            st.broken = true;
-            (void)hipGetLastError();
-            return false;
-        }
-    }
-    // The previous user of the partial sums, if it ran on another stream, has to finish first: an event recorded
-    // on that stream now (it covers everything the stream has been given so far) and awaited by this one.
-    if (st.used && st.last != s) {
-        bool ordered;
-        if (hipEventRecord(st.done, st.last) == hipSuccess) {
-            ordered = hipStreamWaitEvent(s, st.done, 0) == hipSuccess;
-        } else {   // that stream no longer exists: what it was given is done once the device is idle
-            (void)hipGetLastError();
-            ordered = hipDeviceSynchronize() == hipSuccess;
-        }
-        if (!ordered) {
-            (void)hipGetLastError();
-            return false;
-        }
-    }
+    std::unique_lock<std::mutex> lock;
+    float* scratch = (float*)acquire_shared_scratch(g_split, HIP_SYMBOL(splitk_scratch), s, lock);
+    if (!scratch) return false;
     const int tiles_m = (p.M + 127) / 128, tiles_n = (p.N + 127) / 128;
     const int64_t MN = (int64_t)p.M * p.N;
     hipLaunchKernelGGL((gemm16_big<E, float, 2, 2>), dim3((unsigned)(tiles_m * tiles_n * p.batch * parts)), dim3(256), 0, s,
-                       (const unsigned short*)p.A, p.lda, p.sa, (const unsigned short*)p.B, p.ldb, p.sb, st.scratch,
+                       (const unsigned short*)p.A, p.lda, p.sa, (const unsigned short*)p.B, p.ldb, p.sb, scratch,
                        (int64_t)p.M, MN, p.M, p.N, p.K, tiles_m, tiles_n, p.batch, parts, kchunk);
     const int64_t quads = MN / 4 * p.batch;
     const unsigned blocks = (unsigned)((quads + 255) / 256 < 2048 ? (quads + 255) / 256 : 2048);
     if (p.out_dtype == MI_F32)
-        hipLaunchKernelGGL((splitk_reduce<float>), dim3(blocks), dim3(256), 0, s, st.scratch, parts, (float*)p.C, p.ldc,
+        hipLaunchKernelGGL((splitk_reduce<float>), dim3(blocks), dim3(256), 0, s, scratch, parts, (float*)p.C, p.ldc,
                            p.sc, p.M, p.N, p.batch, false);
     else
-        hipLaunchKernelGGL((splitk_reduce<unsigned short>), dim3(blocks), dim3(256), 0, s, st.scratch, parts,
+        hipLaunchKernelGGL((splitk_reduce<unsigned short>), dim3(blocks), dim3(256), 0, s, scratch, parts,
                            (unsigned short*)p.C, p.ldc, p.sc, p.M, p.N, p.batch, p.out_dtype == MI_BF16);
-    st.last = s;
-    st.used = true;
     return true;
 }
 

@@ -635,8 +635,10 @@ __global__ __launch_bounds__(256) void fmha_combine_kernel(const float* __restri
     const float* p0 = part + (live ? row : 0) * (D + kPartPad);
     const int64_t part_stride = rows * (D + kPartPad);
     float m = -INFINITY;
-    if (live)
+    if (live) {
+#pragma unroll 4
         for (int sp = pl; sp < nsplit; sp += PL) m = fmaxf(m, p0[sp * part_stride + D]);
+    }
     if (PL > 1) {
         s_max[tid] = m;
         __syncthreads();
@@ -645,17 +647,21 @@ __global__ __launch_bounds__(256) void fmha_combine_kernel(const float* __restri
     }
     f32x4 acc = {0.f, 0.f, 0.f, 0.f};
     float l = 0.f;
-    if (live)
+    if (live) {
+        // (a part without a visible key for this row is left out by selects, not by a branch, so that the loads of
+        // the parts can all be in flight together)
+#pragma unroll 4
         for (int sp = pl; sp < nsplit; sp += PL) {
             const float* pr = p0 + sp * part_stride;
-            const float mp = pr[D];
-            if (mp == -INFINITY) continue;   // a part without a visible key for this row
-            const float w = __builtin_amdgcn_exp2f(mp - m);
-            l += w * pr[D + 1];
+            const f32x2 ml = *reinterpret_cast<const f32x2*>(pr + D);
             const f32x4 o = *reinterpret_cast<const f32x4*>(pr + 4 * c);
+            const bool seen = ml[0] != -INFINITY;
+            const float w = seen ? __builtin_amdgcn_exp2f(ml[0] - m) : 0.f;
+            l += seen ? w * ml[1] : 0.f;
 #pragma unroll
-            for (int e = 0; e < 4; ++e) acc[e] += w * o[e];
+            for (int e = 0; e < 4; ++e) acc[e] += seen ? w * o[e] : 0.f;
         }
+    }
     if (PL > 1) {
 #pragma unroll
         for (int e = 0; e < 4; ++e) s_acc[tid][e] = acc[e];

@@ -731,8 +731,8 @@ void launch(dim3 grid, hipStream_t s, bool causal, const mi_tile_array* Q, const
         dim3 g1((unsigned)(nqb * nbh)), blk(128 * 2 / JT);
         const int64_t rows = (int64_t)nbh * Sq * pack;
         if (const int parts = pick_parts((int64_t)nqb * nbh, rows, D, Sq, Skv, causal, input_pos)) {
-            std::unique_lock<std::mutex> lock;
-            if (float* scratch = (float*)acquire_shared_scratch(g_part, HIP_SYMBOL(fmha_part_scratch), s, lock)) {
+            ScratchLease lease;   // ends behind the combine launch
+            if (float* scratch = (float*)lease.acquire(g_part, HIP_SYMBOL(fmha_part_scratch), s)) {
                 dim3 gs((unsigned)(nqb * nbh * parts));
                 if (causal)
                     hipLaunchKernelGGL((fmha_fwd_dma_kernel<E, D, JT, true, true>), gs, blk, 0, s, (const unsigned short*)Q->ptr, qs,
@@ -808,7 +808,7 @@ extern "C" int mi_fmha_kernel(const mi_tile_array* Q, const mi_tile_array* K, co
     // the reference's grid is (cld(Sq, TILE_M), B * H) (fmha.jl:163-165), each below 2^24; the kernels here
     // use a one-dimensional grid over both
     if (cld(Sq, (int64_t)TILE_M) > MI_MAX_GRID_DIM || B * H > MI_MAX_GRID_DIM ||
-        cld(Sq, (int64_t)kQB) * B * H > 0x7fffffffLL)
+        cld(Sq, (int64_t)kQB) * B * H > MI_MAX_GRID_DIM)   // (query block, head) pairs share one grid dimension
         return MI_E_GRID;
     if (Sq == 0 || B == 0) return MI_OK;
     if (Skv == 0) return MI_E_SHAPE;

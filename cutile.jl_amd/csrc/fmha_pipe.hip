@@ -911,7 +911,7 @@ bool pipe_applicable(const Problem& p) {
     if (p.causal && p.input_pos != 0) return false;
     if (!vec16(Q) || !vec16(K) || !vec16(V) || !vec16(O)) return false;
     if (K->strides[1] >= (1 << 20) || V->strides[1] >= (1 << 20)) return false;
-    if (Q->sizes[2] * Q->sizes[3] * ((S + 127) / 128) > 0x7fffffff) return false;
+    if (Q->sizes[2] * Q->sizes[3] * ((S + 127) / 128) > MI_MAX_GRID_DIM) return false;
     return true;
 }
 

@@ -326,8 +326,9 @@ int validate(const mi_tile_array* A, const mi_tile_array* B, const mi_tile_array
         if (batch > MI_MAX_GRID_DIM) return MI_E_GRID;   // the reference's grid is (cld(M,tm), cld(N,tn), Batch), batchmatmul.jl:78-80
     }
     if (M > 0x7fffffffLL || N > 0x7fffffffLL || K > 0x7fffffffLL) return MI_E_SHAPE;
-    // the kernels number (tile, batch entry) pairs in one grid dimension; their smallest tile is 64 x 64
-    if (cld(M, (int64_t)64) * cld(N, (int64_t)64) * batch > 0x7fffffffLL) return MI_E_GRID;
+    // the kernels number (tile, batch entry) pairs in one grid dimension of 256-lane workgroups, and a launch takes
+    // fewer than 2^32 lanes per dimension; their smallest tile is 64 x 64
+    if (cld(M, (int64_t)64) * cld(N, (int64_t)64) * batch > MI_MAX_GRID_DIM) return MI_E_GRID;
     if (cld(M, (int64_t)tm) > MI_MAX_GRID_DIM || cld(N, (int64_t)tn) > MI_MAX_GRID_DIM ||
         cld(M, (int64_t)tm) * cld(N, (int64_t)tn) > MI_MAX_GRID_DIM)
         return MI_E_GRID;

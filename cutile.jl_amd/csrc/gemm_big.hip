@@ -397,8 +397,8 @@ int pick_split(const Problem& p, int* kchunk) {
 
 template <typename E>
 bool launch_split(const Problem& p, hipStream_t s, int parts, int kchunk) {
-    std::unique_lock<std::mutex> lock;
-    float* scratch = (float*)acquire_shared_scratch(g_split, HIP_SYMBOL(splitk_scratch), s, lock);
+    ScratchLease lease;   // ends behind the reduce launch
+    float* scratch = (float*)lease.acquire(g_split, HIP_SYMBOL(splitk_scratch), s);
     if (!scratch) return false;
     const int tiles_m = (p.M + 127) / 128, tiles_n = (p.N + 127) / 128;
     const int64_t MN = (int64_t)p.M * p.N;

@@ -602,13 +602,22 @@ constexpr int kMaxDevices = 64;
 float* g_scratch_ptr[kMaxDevices];
 bool g_scratch_known[kMaxDevices];
 
-// Device address of `scratch` on the current device; positive hipError_t on failure.
-int scratch_ptr(float** out) {
+// Device address of `scratch` on the current device; positive hipError_t on failure.  The lookup
+// (hipGetSymbolAddress may load the code object and is not a stream operation) happens once per
+// device and never while `stream` is being captured: the forward and the three-step backward do
+// it on their first eager call as well, so a capture that holds the static backward finds the
+// address known whenever any LayerNorm entry point has run eagerly on the device before.
+int scratch_ptr(float** out, hipStream_t stream) {
     int dev = 0;
     hipError_t e = hipGetDevice(&dev);
     if (e != hipSuccess) return (int)e;
     if (dev < 0 || dev >= kMaxDevices) return MI_E_UNSUPPORTED;
     if (!__atomic_load_n(&g_scratch_known[dev], __ATOMIC_ACQUIRE)) {
+        hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
+        if (hipStreamIsCapturing(stream, &cap) != hipSuccess || cap != hipStreamCaptureStatusNone) {
+            (void)hipGetLastError();
+            return MI_E_UNSUPPORTED;   // first use on this device inside a capture: call once eagerly before
+        }
         float* p = nullptr;
         e = hipGetSymbolAddress((void**)&p, HIP_SYMBOL(scratch));
         if (e != hipSuccess) return (int)e;
@@ -616,8 +625,20 @@ int scratch_ptr(float** out) {
         g_scratch_ptr[dev] = p;   // every thread that gets here stores the same address
         __atomic_store_n(&g_scratch_known[dev], true, __ATOMIC_RELEASE);
     }
-    *out = g_scratch_ptr[dev];
+    if (out) *out = g_scratch_ptr[dev];
     return MI_OK;
+}
+
+// Called by the other LayerNorm entry points: makes the address known while no capture is on.
+void scratch_warm(void* stream) {
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess) {
+        (void)hipGetLastError();
+        return;
+    }
+    if (dev >= 0 && dev < kMaxDevices && !__atomic_load_n(&g_scratch_known[dev], __ATOMIC_ACQUIRE) &&
+        scratch_ptr(nullptr, (hipStream_t)stream) > 0)
+        (void)hipGetLastError();
 }
 
 // Zero fill as a kernel (a memset node would not survive stream capture and replay on this runtime).
@@ -713,6 +734,7 @@ extern "C" int mi_layer_norm_fwd(const mi_tile_array* X, const mi_tile_array* W,
                                  const mi_tile_array* B, const mi_tile_array* Y,
                                  const mi_tile_array* Mean, const mi_tile_array* Rstd, float eps,
                                  int TILE_N, void* stream) {
+    scratch_warm(stream);
     MI_CHECK(check_f32(X, 2));
     MI_CHECK(check_f32(Y, 2));
     MI_CHECK(check_f32(W, 1));
@@ -763,6 +785,7 @@ extern "C" int mi_layer_norm_bwd_dx_partial_dwdb(
     const mi_tile_array* X, const mi_tile_array* W, const mi_tile_array* Mean,
     const mi_tile_array* Rstd, const mi_tile_array* Locks, int GROUP_SIZE_M, int TILE_N,
     void* stream) {
+    scratch_warm(stream);
     MI_CHECK(check_f32(DX, 2));
     MI_CHECK(check_f32(DY, 2));
     MI_CHECK(check_f32(DW, 2));
@@ -900,7 +923,7 @@ extern "C" int mi_layer_norm_bwd_static(const mi_tile_array* DX, const mi_tile_a
     const int64_t ld = (N + 3) / 4 * 4;
     if (ld * G > kScratchFloats) return MI_E_SCRATCH;
     float* base = nullptr;
-    MI_CHECK(scratch_ptr(&base));
+    MI_CHECK(scratch_ptr(&base, (hipStream_t)stream));
     mi_tile_array dw = {}, db = {};
     dw.ptr = base;
     db.ptr = base + kScratchFloats;

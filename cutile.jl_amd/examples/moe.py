@@ -56,8 +56,10 @@ def cutile_moe(hidden_states, w1, w2, topk_weights, topk_ids, tile_m, tile_n, ti
     # The three caches of moe.jl:228-230, carved out of one allocation.  The reference zero-fills them; here they
     # are left as allocated: every column of every cache belongs to one (token, slot) replica, the GEMMs write the
     # columns of all replicas (only padding slots write nothing, and nothing reads those), so no fill is ever
-    # read.  This holds for expert ids in 1..num_experts, which is what the reference accepts as well
-    # (moe_align_tile_size indexes by them, moe.jl:150-160).
+    # read.  The one exception is a replica whose expert id lies outside 1..num_experts (the reference raises on
+    # those, moe_align_tile_size indexes by them, moe.jl:150-160; the device-side sort drops them): nothing writes
+    # its column of cache3, which the top-k sum reads.  cache3 is therefore zeroed -- by the sort launch itself where
+    # the sort runs on the GPU, by a fill otherwise -- so that such a replica contributes 0 on every path.
     n1 = 0 if fuse_silu else total_tokens * intermediate_size * 2
     n2, n3 = total_tokens * intermediate_size, 0 if fuse_sum else total_tokens * hidden_size
     caches = torch.empty(n1 + n2 + n3, dtype=T, device=dev)
@@ -68,11 +70,16 @@ def cutile_moe(hidden_states, w1, w2, topk_weights, topk_ids, tile_m, tile_n, ti
     if fuse_sum:
         sorted_token_ids, sorted_expert_ids = ct.moe_align_tile_size_device(topk_ids, tile_m, num_experts, clear=out)
     elif aligned is None and device_align:
-        sorted_token_ids, sorted_expert_ids = ct.moe_align_tile_size_device(topk_ids, tile_m, num_experts)
+        clear = cache3 if (cache3.numel() * cache3.element_size()) % 16 == 0 and cache3.data_ptr() % 16 == 0 else None
+        if clear is None:
+            cache3.zero_()
+        sorted_token_ids, sorted_expert_ids = ct.moe_align_tile_size_device(topk_ids, tile_m, num_experts, clear=clear)
     elif aligned is None:
+        cache3.zero_()
         tok, exp = ct.moe_align_tile_size(topk_ids.cpu(), tile_m, num_experts)
         sorted_token_ids, sorted_expert_ids = tok.to(dev), exp.to(dev)
     else:
+        cache3.zero_()
         sorted_token_ids, sorted_expert_ids = aligned
     if fuse_silu:
         invoke_fused_moe_kernel(hidden_states, w1, cache2, topk_weights, sorted_token_ids, sorted_expert_ids,

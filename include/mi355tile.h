@@ -157,7 +157,10 @@ int mi_layer_norm_bwd_dwdb(const mi_tile_array* DW, const mi_tile_array* DB,
  * mi_layer_norm_bwd_dwdb, with the partial slots held in a file-scope device array of the library
  * (4 MiB per GPU, kept until the process ends).  Limit: cld(N,4)*4 * GROUP_SIZE_M <= 524288 floats
  * (N = 8192 with 64 slots), MI_E_SCRATCH beyond.  Every call on a GPU uses that GPU's one array:
- * calls that overlap on one GPU (different streams or threads) race. */
+ * calls that overlap on one GPU (different streams or threads) race.  The array's device address
+ * is looked up once per GPU, outside any stream capture: by the first eager call of this or of
+ * any other mi_layer_norm_* entry point on that GPU.  A call on a capturing stream before that
+ * returns MI_E_UNSUPPORTED (make one eager LayerNorm call first, then capture). */
 int mi_layer_norm_bwd_static(const mi_tile_array* DX, const mi_tile_array* DY, const mi_tile_array* X,
                              const mi_tile_array* W, const mi_tile_array* Mean,
                              const mi_tile_array* Rstd, const mi_tile_array* FINAL_DW,

@@ -145,6 +145,14 @@ def test_dimensions_beyond_65535_pass_the_host_checks(ct):
     # the 24-bit limits of the reference still hold
     A2 = _desc(ct, (8, 8, 2 ** 24), h16)
     assert L.mi_batch_matmul_kernel(r(A2), r(A2), r(A2), 8, 8, 8, None) == ct.MI_E_GRID
+    # ... and so does the launch's own: (tile, batch entry) pairs, or (query block, head) pairs, share one grid
+    # dimension, which takes fewer than 2^32 lanes; a product past that is a host-side MI_E_GRID, not a HIP error
+    A3 = _desc(ct, (128, 128, 2 ** 23), h16)         # 4 tiles of 64 x 64 per entry: 2^25 workgroups of 256 lanes
+    assert L.mi_batch_matmul_kernel(r(A3), r(A3), r(A3), 64, 64, 64, None) == ct.MI_E_GRID
+    A4 = _desc(ct, (128, 128, 2 ** 21), h16)         # 2^23 workgroups: accepted
+    assert L.mi_batch_matmul_kernel(r(A4), r(A4), r(A4), 64, 64, 64, None) > 0
+    q2 = _desc(ct, (64, 128 * 4096, 8192, 1), h16)   # 4096 query blocks x 8192 heads
+    assert L.mi_fmha_kernel(r(q2), r(q2), r(q2), r(q2), ctypes.c_float(0.125), 0, 64, 8192, 128, 128, 1, 1, 1, None) == ct.MI_E_GRID
 
 
 @pytest.mark.skipif(not _no_gpu_here(), reason="launches with placeholder pointers: only where no GPU can take them")

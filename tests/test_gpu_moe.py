@@ -433,3 +433,30 @@ def test_down_projection_that_adds_into_the_output(ct, orc, tokens, hidden, expe
             moe.cutile_moe(d4.hidden_states, d4.w1, d4.w2, d4.topk_weights, d4.topk_ids, 128, 128, 64, fuse_sum=True)
         moe.cutile_moe(d4.hidden_states, d4.w1, d4.w2, d4.topk_weights, d4.topk_ids, 128, 128, 64)
         assert ct.last_variant().startswith("moe_sum_topk")
+
+
+@pytest.mark.parametrize("topk", [2, 4])
+def test_replicas_with_an_expert_id_out_of_range_contribute_nothing(orc, topk):
+    """Expert ids outside 1..num_experts: the reference raises on them (moe_align_tile_size indexes its counters by
+    the id, moe.jl:150-160); the device-side sort drops such replicas.  Whatever path the call then takes (two slots:
+    the down projection adds into the zeroed output; more: cache3 + the top-k sum), a dropped replica has to
+    contribute 0 -- not what an unwritten cache column happens to hold (the tests run with poisoned allocations).
+    The expected output is the oracle's with the dropped replicas' routed weights set to 0."""
+    d = moe.prepare(num_tokens=40, hidden_size=256, num_experts=6, intermediate_size=192, topk=topk)
+    ids = d.topk_ids.clone()
+    ids[0, 3] = 0
+    ids[topk - 1, 17] = d.num_experts + 1
+    ids[1, 29] = -5
+    w_ref = d.topk_weights.clone()
+    bad = (ids < 1) | (ids > d.num_experts)
+    w_ref[bad] = 0
+    ids_ref = torch.where(bad, torch.ones_like(ids), ids)
+    J = orc.to_julia
+    ref = orc.ref_moe(J(d.hidden_states), J(d.w1), J(d.w2), J(w_ref), J(ids_ref), dtype=np.float64)
+    for fuse_silu in (True, False):
+        got = moe.cutile_moe(d.hidden_states, d.w1, d.w2, d.topk_weights, ids, 16, 128, 64, device_align=True, fuse_silu=fuse_silu)
+        assert not torch.isnan(got.float()).any()
+        check(J(got), ref)
+    if topk <= 2:
+        sep = moe.cutile_moe(d.hidden_states, d.w1, d.w2, d.topk_weights, ids, 16, 128, 64, device_align=True, fuse_sum=False)
+        assert torch.equal(sep, got)

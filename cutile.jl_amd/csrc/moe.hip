@@ -15,6 +15,7 @@
 // may be f16/bf16 or OCP FP8 E4M3 with one fp32 scale per (n, expert), which are widened to
 // f16 on their way into LDS (every e4m3 value is exact in f16) and scaled in the epilogue.
 #include "common.h"
+#include "moe_dense.h"
 #include <math.h>
 #include <type_traits>
 
@@ -87,16 +88,7 @@ template <> struct Fp8<BF16> {
     }
 };
 
-// SiLU(x) * y in fp32 with the approximate reciprocal of moe.jl:117-124.  The barrier keeps the
-// fp32 product a value of its own: without it the compiler may fold the final multiply into the
-// conversion to f16 (one rounding instead of two) in one kernel and not in another, and the fused
-// and the separate path would differ in the last bit now and then.
-__device__ __forceinline__ float silu_mul(float x, float y) {
-    const float denom = 1.0f + expf(-x);
-    float p = x * __builtin_amdgcn_rcpf(denom) * y;
-    asm volatile("" : "+v"(p));
-    return p;
-}
+using mi::moe::silu_mul;   // SiLU(x) * y as moe.jl:117-124 computes it, shared with the dense-routing kernel
 
 constexpr int kTT = 32;   // token slots per workgroup (one MFMA row tile)
 
@@ -621,6 +613,25 @@ static int fused_moe_impl(const mi_tile_array* A, const mi_tile_array* B, const 
     if (K > 0x7fffffff || N > 0x7fffffff || total > 0x7ffffffe || slots > 0x7fffffff) return MI_E_SHAPE;
     if (m_blocks * cld(N, (int64_t)TILE_N) > MI_MAX_GRID_DIM) return MI_E_GRID;
     if (m_blocks == 0 || N == 0) return MI_OK;
+    hipStream_t s = (hipStream_t)stream;
+    {   // dense routing: the grouped GEMM on 128 x 128 tiles fed by a ring of LDS stages (moe_dense.hip), same bits
+        mi::moe::DenseArgs d;
+        d.A = (const unsigned short*)A->ptr; d.lda = A->strides[1]; d.num_a_cols = (int)A->sizes[1];
+        d.B = B->ptr; d.ldb = B->strides[1]; d.sbe = B->strides[2];
+        d.C = (unsigned short*)C->ptr; d.ldc = C->strides[1]; d.total_tokens = (int)total;
+        d.topk_weights = (const unsigned short*)topk_weights->ptr; d.w_topk = (int)w_topk;
+        d.w_s0 = w2d ? topk_weights->strides[0] : (int64_t)1; d.w_s1 = w2d ? topk_weights->strides[1] : (int64_t)0;
+        d.sorted_token_ids = (const int*)sorted_token_ids->ptr; d.num_slots = (int)slots;
+        d.sorted_expert_ids = (const int*)sorted_expert_ids->ptr; d.num_blocks = (int)m_blocks;
+        d.b_scale = w8 ? (const float*)b_scale->ptr : nullptr; d.ld_scale = w8 ? b_scale->strides[1] : 0;
+        d.K = (int)K; d.N = (int)N; d.num_experts = (int)E; d.replicas = num_token_replicas;
+        d.mul_routed_weight = mul_routed_weight != 0; d.TILE_M = TILE_M; d.acc_shift = acc_shift;
+        d.bf16 = A->dtype == MI_BF16; d.silu = silu; d.w8 = w8;
+        if (mi::moe::dense_applicable(d)) {
+            mi::moe::dense_launch(d, s);
+            return launch_status();
+        }
+    }
     const int tile_slots = TILE_M < kTT ? TILE_M : kTT;
     const int64_t tiles = m_blocks * (TILE_M / tile_slots);
     // Wide strips (128 channels) when they already give the chip >= ~3 workgroups per CU,
@@ -643,7 +654,6 @@ static int fused_moe_impl(const mi_tile_array* A, const mi_tile_array* B, const 
     const bool vecA = aligned(A->ptr, 16) && A->strides[1] % 8 == 0;
     const bool vecB = aligned(B->ptr, 16) && B->strides[1] % (w8 ? 16 : 8) == 0 && B->strides[2] % (w8 ? 16 : 8) == 0;
     dim3 grid((unsigned)(tiles / ts * n_blocks));
-    hipStream_t s = (hipStream_t)stream;
     // every tile of the launch inside the arrays and 16-byte aligned: the kernels without load predicates
     // (a K step of 512 for the e4m3 down projection, whose steps move half the weight bytes: 29.8 us against 20.4)
     const int kt = narrow ? 256 : 128;

@@ -1,0 +1,520 @@
+// Token-gather grouped GEMM of the MoE for dense routing (fused_moe_kernel, examples/moe.jl:45-105, at the
+// reference example's own routing -- top-8 of 32 experts, moe.jl:311-344 -- and at prefill sizes): with tens to
+// hundreds of tokens per expert the product is no longer a weight stream with a few MFMAs attached (moe.hip) but a
+// GEMM per expert, and takes the big GEMM's structure (gemm_big.hip):
+//
+//   workgroup tile = 128 sorted slots of one expert x 128 weight rows (channels); 4 waves as 2 (slots) x 2
+//   (channels), each 64 x 64 = 2 x 2 MFMA 32x32x16 tiles; K walked in steps of 32 through a ring of four LDS
+//   stages (4 x 16 KB: two workgroups per CU) filled by direct global->LDS transfers with no staging registers;
+//   the token rows of a stage are gathered (every lane of a transfer carries the address of its own token's row),
+//   the weight rows carry the expert's offset; transfers for step s+3 / s+4 are issued between the MFMAs of step s;
+//   one barrier per step that waits for the oldest stage in flight only.
+//
+// Both operands are K-contiguous, so both LDS tiles are [row][32 k] with the 16-byte chunks of a row XOR-swizzled
+// by (row >> 2) & 3, and both fragments are plain 16-byte reads.  The MFMA column operand (lane % 32) carries the
+// channel, so a store of C is a run of 32 consecutive channels; the row operand carries the slot.  k is walked in
+// ascending order with the k <-> lane map of the streaming kernel (moe.hip), so every output element is accumulated
+// in the same order as there and the two kernels give the same bits.
+//
+// 32-slot tiles that hold only padding are never multiplied: a wave whose slots are all padding only takes part in
+// the transfers and barriers.  Workgroups are numbered so that every XCD works on a contiguous range of the blocks
+// in use, strips of one block next to each other: a block's 128 token rows are fetched into that XCD's L2 once, and
+// the two or three blocks of one expert stream its weights at the same time.
+//
+// Epilogues: plain (optionally times the routed weight), SiLU(gate) * up (the tile's 128 weight rows are 64 gate
+// channels and the 64 up channels that go with them, arranged so that a lane holds both halves of an output
+// element), and the accumulating form (packed atomic adds into the token's output column, one or two slots per token).
+#include "gemm_direct.h"
+#include "moe_dense.h"
+
+namespace {
+
+using namespace mi;
+using namespace mi::gemm;
+using mi::moe::DenseArgs;
+
+constexpr int BK = 32;
+constexpr int kRows = 128;            // slots, and weight rows, per workgroup tile
+constexpr int kStage = kRows * BK;    // elements of one operand stage (8 KB)
+constexpr int MODE_PLAIN = 0, MODE_SILU = 1, MODE_ACC = 2;
+
+// Source of every chunk that lies past K.
+__device__ __attribute__((aligned(16))) const unsigned zeros16d[4] = {0u, 0u, 0u, 0u};
+
+__device__ __forceinline__ float widen16(bool bf16, unsigned short h) {
+    return bf16 ? __uint_as_float(((unsigned)h) << 16) : (float)__builtin_bit_cast(_Float16, h);
+}
+
+struct DLane {
+    const char* gT[2];   // global address, at k = 0, of the lane's 16-byte chunk in the wave's two token transfers
+    const char* gW[2];   // the same in its two weight transfers
+    int kC;              // first k, within a stage, of that chunk
+    unsigned fT[2], fW[2];   // LDS element offset of the token / weight fragment of sub-step 0 / 1 (+ 32 * BK per 32-row tile)
+};
+
+struct DFrag {
+    s16x8 t[2], w[2];
+};
+
+// An operand stage is 128 rows x 64 B = eight transfers of 1 KB (16 rows each); wave w takes transfers w and w + 4.
+// TAIL: k_left = K - (first k of the stage); chunks at or past it come from the zero block.
+template <bool TAIL>
+__device__ __forceinline__ void issue2(const char* const (&g)[2], int64_t koff, unsigned short* S, int wave, int kC,
+                                       int k_left) {
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+        const char* p = g[j] + koff;
+        if (TAIL && kC >= k_left) p = (const char*)zeros16d;
+        gload_lds16(p, S + (wave + 4 * j) * 512);
+    }
+}
+
+template <int LIVE>
+__device__ __forceinline__ void load_frags(const unsigned short* Ts, const unsigned short* Ws, const DLane& ln, int ks,
+                                           DFrag& f) {
+    if (LIVE == 0) return;
+#pragma unroll
+    for (int j = 0; j < 2; ++j) f.w[j] = *reinterpret_cast<const s16x8*>(Ws + ln.fW[ks] + 32 * j * BK);
+#pragma unroll
+    for (int i = 0; i < LIVE; ++i) f.t[i] = *reinterpret_cast<const s16x8*>(Ts + ln.fT[ks] + 32 * i * BK);
+}
+
+// SLOT_LANE: the MFMA column operand (lane % 32 of the result) carries the slot and the rows the channel: a lane
+// then holds four consecutive channels of one token's row in four consecutive registers.  Otherwise the lane carries
+// the channel and the rows the slots.  The products and the order in which an element's k are added are the same.
+template <typename E, int LIVE, bool SLOT_LANE>
+__device__ __forceinline__ void mma(const DFrag& f, f32x16 (&acc)[2][2]) {
+#pragma unroll
+    for (int i = 0; i < LIVE; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+            acc[i][j] = SLOT_LANE ? E::mfma32(f.w[j], f.t[i], acc[i][j]) : E::mfma32(f.t[i], f.w[j], acc[i][j]);
+}
+
+// Spread the fragment reads and the two transfers of a half step over its MFMAs.
+template <int LIVE, bool DMA, bool FRAGS>
+__device__ __forceinline__ void interleave() {
+    if constexpr (LIVE == 2) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            __builtin_amdgcn_sched_group_barrier(SG_MFMA, 1, 0);
+            if (FRAGS) __builtin_amdgcn_sched_group_barrier(SG_DSRD, 1, 0);
+            if (DMA && (i & 1) == 0) __builtin_amdgcn_sched_group_barrier(SG_VMEM, 1, 0);
+        }
+    }
+    __builtin_amdgcn_sched_barrier(0);
+}
+
+// One K step of 32 on stage X; the next step's data is in stage Y.
+//   first half : MFMAs of sub-step 0 | read sub-step 1 fragments | token transfers of step s + 3 (into stage TsA)
+//   barrier
+//   second half: MFMAs of sub-step 1 | read the next stage's sub-step 0 fragments | weight transfers of step s + 4 (into WsX)
+template <typename E, int LIVE, bool SLOT_LANE, bool DMA_T, bool DMA_W, int VMCNT, bool LAST, bool TAIL>
+__device__ __forceinline__ void k_step(const unsigned short* TsX, unsigned short* WsX, const unsigned short* TsY,
+                                       const unsigned short* WsY, unsigned short* TsA, int64_t koff3, int wave,
+                                       const DLane& ln, DFrag& f0, DFrag& f1, f32x16 (&acc)[2][2], int k_left3) {
+    if (DMA_T) issue2<TAIL>(ln.gT, koff3, TsA, wave, ln.kC, k_left3);
+    load_frags<LIVE>(TsX, WsX, ln, 1, f1);
+    mma<E, LIVE, SLOT_LANE>(f0, acc);
+    interleave<LIVE, DMA_T, true>();
+    if (!LAST) stage_barrier<VMCNT>();
+    if (DMA_W) issue2<TAIL>(ln.gW, koff3 + 2 * BK, WsX, wave, ln.kC, k_left3 - BK);
+    if (!LAST) load_frags<LIVE>(TsY, WsY, ln, 0, f0);
+    mma<E, LIVE, SLOT_LANE>(f1, acc);
+    interleave<LIVE, DMA_W, !LAST>();
+}
+
+struct Stages {
+    unsigned short *T0, *T1, *T2, *T3, *W0, *W1, *W2, *W3;
+};
+
+constexpr int64_t kStepBytes = BK * 2;   // bytes along a row per K step
+
+// What a tile requests before its first step: stages 0..2 and the weight half of stage 3 (2 + 2 transfers per wave and
+// stage).
+__device__ __forceinline__ void ring_fill(const Stages& st, int wave, const DLane& ln) {
+    issue2<false>(ln.gW, 0, st.W0, wave, ln.kC, 0);
+    issue2<false>(ln.gT, 0, st.T0, wave, ln.kC, 0);
+    issue2<false>(ln.gW, kStepBytes, st.W1, wave, ln.kC, 0);
+    issue2<false>(ln.gT, kStepBytes, st.T1, wave, ln.kC, 0);
+    issue2<false>(ln.gW, 2 * kStepBytes, st.W2, wave, ln.kC, 0);
+    issue2<false>(ln.gT, 2 * kStepBytes, st.T2, wave, ln.kC, 0);
+    issue2<false>(ln.gW, 3 * kStepBytes, st.W3, wave, ln.kC, 0);
+}
+
+// The K walk of one tile whose ring has been filled.  Its first wait leaves the ten youngest transfers in flight:
+// whatever the wave requested before the ring fill (the previous tile's stores, the next tile's token ids) is older
+// and completes first.
+template <typename E, int LIVE, bool SLOT_LANE>
+__device__ __forceinline__ void main_loop(const Stages& st, int K, int wave, const DLane& ln, f32x16 (&acc)[2][2]) {
+    const int KT = 4 * ((K + 4 * BK - 1) / (4 * BK));   // steps, in whole groups of four; >= 8 (K >= 256 is checked on the host)
+    DFrag f0, f1;
+    stage_barrier<2 * 4 + 2>();
+    load_frags<LIVE>(st.T0, st.W0, ln, 0, f0);
+#define KSTEP(X, Y, AA, DT, DW, VM, LAST, TAIL, s)                                                                   \
+    k_step<E, LIVE, SLOT_LANE, DT, DW, (VM) * 4, LAST, TAIL>(st.T##X, st.W##X, st.T##Y, st.W##Y, st.T##AA, (int64_t)((s) + 3) * kStepBytes, \
+                                                  wave, ln, f0, f1, acc, K - ((s) + 3) * BK)
+    int s = 0;
+    for (; s + 12 <= KT; s += 4) {
+        KSTEP(0, 1, 3, true, true, 2, false, false, s);
+        KSTEP(1, 2, 0, true, true, 2, false, false, s + 1);
+        KSTEP(2, 3, 1, true, true, 2, false, false, s + 2);
+        KSTEP(3, 0, 2, true, true, 2, false, false, s + 3);
+    }
+    // the group that requests the last four stages (the only ones that can reach past K)
+    KSTEP(0, 1, 3, true, true, 2, false, true, s);
+    KSTEP(1, 2, 0, true, true, 2, false, true, s + 1);
+    KSTEP(2, 3, 1, true, true, 2, false, true, s + 2);
+    KSTEP(3, 0, 2, true, true, 2, false, true, s + 3);
+    s += 4;
+    // last four steps: only the token half of the final stage is still to be requested
+    KSTEP(0, 1, 3, true, false, 2, false, true, s);
+    KSTEP(1, 2, 0, false, false, 1, false, false, s + 1);
+    KSTEP(2, 3, 1, false, false, 0, false, false, s + 2);
+    KSTEP(3, 0, 2, false, false, 0, true, false, s + 3);
+#undef KSTEP
+}
+
+// Barrier that waits for the wave's LDS accesses only (the transfers, loads and stores in flight stay in flight).
+__device__ __forceinline__ void lds_only_barrier() {
+    asm volatile("" ::: "memory");
+    __builtin_amdgcn_s_waitcnt(0xc07f);
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+}
+
+// What a workgroup reads about a tile ahead of time (raw values: looking at them would wait for the loads).
+struct Meta {
+    int sb, bid_n;          // 128-slot block and channel strip
+    int expert_raw;         // sorted_expert_ids entry (1-based, 0 = unused block)
+    int t0, t1, tm;         // sorted_token_ids entries of the rows of this lane's two transfers / of slot `tid`
+};
+
+// Stores one 32-slot x 32-channel tile held slot-per-lane (o[r]: channel 8 * (r / 4) + 4 * hb + r % 4 of the lane's
+// slot) as 16-byte pieces: four registers are four consecutive channels; the two half-waves of a lane pair (l, l + 32)
+// hold the two halves of every group of eight, and two lane-half swaps per pair of groups leave every lane with eight
+// consecutive channels of its slot's row.  `row`: the slot's output row at the tile's first channel; n_left: channels
+// from there to the end of the row.
+template <typename E>
+__device__ __forceinline__ void store_tile_slot_lane(const float (&o)[16], unsigned short* row, bool valid, int n_left,
+                                                     bool vec_ok, int hb) {
+    unsigned P[4][2];
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+        P[q][0] = (unsigned)E::from_f32(o[4 * q]) | ((unsigned)E::from_f32(o[4 * q + 1]) << 16);
+        P[q][1] = (unsigned)E::from_f32(o[4 * q + 2]) | ((unsigned)E::from_f32(o[4 * q + 3]) << 16);
+    }
+#pragma unroll
+    for (int q = 0; q < 4; q += 2) {
+        // lower half-wave: own group q, then the partner's half of it; upper: the partner's half of group q + 1, then own
+        const auto s0 = __builtin_amdgcn_permlane32_swap(P[q][0], P[q + 1][0], false, false);
+        const auto s1 = __builtin_amdgcn_permlane32_swap(P[q][1], P[q + 1][1], false, false);
+        const u32x4 v = {s0[0], s1[0], s0[1], s1[1]};
+        const int c = 8 * q + 8 * hb;   // first of this lane's eight channels
+        if (valid) {
+            if (vec_ok && c + 8 <= n_left) {
+                __builtin_nontemporal_store(v, reinterpret_cast<u32x4*>(row + c));
+            } else {
+#pragma unroll
+                for (int e = 0; e < 8; ++e)
+                    if (c + e < n_left) row[c + e] = (unsigned short)(v[e >> 1] >> (16 * (e & 1)));
+            }
+        }
+    }
+}
+
+// Stores of one tile.
+template <typename E, int MODE>
+__device__ __forceinline__ void epilogue(const DenseArgs& a, const f32x16 (&acc)[2][2], int nlive, const int* s_tok,
+                                         const float* s_wt, int bid_n, int ws, int wn, int lane, bool vec_ok) {
+    const int hb = lane >> 5;
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+        if (i >= nlive) break;
+        // token and routed weight of slot lane % 32 of this 32-slot tile
+        const int tokv = s_tok[64 * ws + 32 * i + (lane & 31)];
+        const float wtv = s_wt[64 * ws + 32 * i + (lane & 31)];
+        if constexpr (MODE == MODE_SILU) {
+            // lane = slot; register r of the gate tile and of the up tile are the same output channel
+            const int ch0 = bid_n * 64 + 32 * wn;   // the wave's first output channel, < N / 2
+            float o[16];
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                float g = acc[i][0][r], u = acc[i][1][r];
+                if (a.mul_routed_weight) {
+                    g *= wtv;
+                    u *= wtv;
+                }
+                // both halves rounded to the activation type, as the unfused GEMM stores them
+                g = widen16(a.bf16, E::from_f32(g));
+                u = widen16(a.bf16, E::from_f32(u));
+                o[r] = mi::moe::silu_mul(g, u);
+            }
+            store_tile_slot_lane<E>(o, a.C + (int64_t)(tokv ? tokv - 1 : 0) * a.ldc + ch0, tokv != 0, a.N / 2 - ch0, vec_ok, hb);
+        } else if constexpr (MODE == MODE_PLAIN) {
+#pragma unroll
+            for (int j = 0; j < 2; ++j) {
+                const int ch0 = bid_n * kRows + 64 * wn + 32 * j;
+                float o[16];
+#pragma unroll
+                for (int r = 0; r < 16; ++r) o[r] = a.mul_routed_weight ? acc[i][j][r] * wtv : acc[i][j][r];
+                store_tile_slot_lane<E>(o, a.C + (int64_t)(tokv ? tokv - 1 : 0) * a.ldc + ch0, tokv != 0, a.N - ch0, vec_ok, hb);
+            }
+        } else {
+            // lane = channel; rows of a 32 x 32 tile = slots 8 * (r / 4) + 4 * hb + r % 4.  The wave's two MFMA column
+            // tiles are 64 consecutive channels: swapping the upper half of tile 0's register with the lower half of
+            // tile 1's gives one register with all 64 channels of row R and one with those of row R + 4.  Column
+            // (token_id - 1) >> acc_shift receives the replica's value as rounded to the storage type, by a packed
+            // atomic add of two adjacent channels: even lanes send row R, odd lanes row R + 4, each row 128
+            // consecutive bytes.
+            const int gn = bid_n * kRows + 64 * wn + lane;
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const int R = 8 * (r >> 2) + (r & 3);
+                const int tokA = __builtin_amdgcn_readlane(tokv, R), tokB = __builtin_amdgcn_readlane(tokv, R + 4);
+                float v0 = acc[i][0][r], v1 = acc[i][1][r];
+                if (a.mul_routed_weight) {
+                    const float wA = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, wtv), R));
+                    const float wB = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, wtv), R + 4));
+                    const float w = hb ? wB : wA;
+                    v0 *= w;
+                    v1 *= w;
+                }
+                const auto sw = __builtin_amdgcn_permlane32_swap((unsigned)E::from_f32(v0), (unsigned)E::from_f32(v1), false, false);
+                const unsigned rowA = sw[0], rowB = sw[1];   // this lane's channel of row R / of row R + 4
+                const unsigned nbrA = (unsigned)__shfl_xor((int)rowA, 1, 64), nbrB = (unsigned)__shfl_xor((int)rowB, 1, 64);
+                const int tok = (lane & 1) ? tokB : tokA;
+                const unsigned pair = (lane & 1) ? (nbrB | (rowB << 16)) : (rowA | (nbrA << 16));
+                if (tok && gn < a.N)
+                    mi::moe::atomic_add2(a.bf16, a.C + (gn & ~1) + (int64_t)((tok - 1) >> a.acc_shift) * a.ldc, pair);
+            }
+        }
+    }
+}
+
+// Persistent workgroups: the launch has at most two per CU, and each walks the tiles of its XCD's range with a
+// stride.  A tile's stores, and the next tile's ring fill right behind them, are in flight while nothing else of the
+// workgroup is: the next tile's K walk starts as soon as its first stage has landed, and what a tile needs to know
+// (expert, token ids) is requested one tile ahead.
+template <typename E, int MODE>
+__global__ __launch_bounds__(256) void moe_dense_kernel(const DenseArgs a, int n_blocks) {
+    __shared__ __attribute__((aligned(1024))) unsigned short Ts0[kStage], Ts1[kStage], Ts2[kStage], Ts3[kStage];
+    __shared__ __attribute__((aligned(1024))) unsigned short Ws0[kStage], Ws1[kStage], Ws2[kStage], Ws3[kStage];
+    __shared__ int s_tok[2][kRows];      // 1-based replica id of every slot, 0 = no token (two tiles: current and next)
+    __shared__ float s_wt[2][kRows];     // its routed weight (1 where none is applied)
+    __shared__ unsigned s_live[2][2];    // per half of the block: bit i = its 32-slot tile i holds a token
+    const int tid = threadIdx.x, lane = tid & 63, hb = lane >> 5;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int ws = wave & 1, wn = wave >> 1;   // the wave's half of the slots / of the channels
+
+    // Blocks in use: up to and including the last block that names an expert (the on-device sort fills a
+    // fixed-capacity array and marks the rest with expert 0).
+    int used = a.num_blocks;
+    if (a.num_blocks <= 4096) {
+        used = 0;
+        for (int b0 = 0; b0 < a.num_blocks; b0 += 64) {
+            const int b = b0 + lane;
+            const int e = b < a.num_blocks ? a.sorted_expert_ids[b] : 0;
+            const unsigned long long m = __ballot(e >= 1 && e <= a.num_experts);
+            if (m) used = b0 + 64 - __builtin_clzll(m);
+        }
+    }
+    // Workgroup ids congruent mod 8 share an XCD; XCD x takes tiles [x * per, (x + 1) * per) of the (block, strip)
+    // pairs in use, strips of a block consecutive, and its workgroups walk that range with a stride.
+    const int bpb = a.TILE_M / kRows;                       // 128-slot tiles per TILE_M block
+    const int tiles_all = used * bpb * n_blocks;
+    const int per = (tiles_all + 7) >> 3;
+    const int nslot = gridDim.x >> 3;
+    const int lo = (blockIdx.x & 7) * per, hi = lo + per < tiles_all ? lo + per : tiles_all;
+    int cur = lo + (blockIdx.x >> 3);
+    if (cur >= hi) return;
+
+    const int r0 = 16 * wave + (lane >> 2), r1 = 64 + r0;   // rows of this lane's chunks in the wave's two transfers
+    // Tile idx -> (128-slot block, strip).  Blocks of one expert that follow each other form a run (cut at multiples
+    // of 64 blocks, so that one look at 64 expert ids finds it); the tiles of a run are numbered strip-major: all
+    // blocks of the expert for strip 0, then for strip 1, ...  The workgroups of an XCD work on consecutive tiles,
+    // i.e. on a few strips of every block of an expert at a time: a weight strip is fetched into the L2 once for all
+    // of the expert's blocks, and the blocks' token rows stay there while the strips pass.
+    int win = -1, win_e = 0;   // the window of 64 blocks whose expert ids this lane holds one of
+    const int sub_used = used * bpb;
+    auto load_meta = [&](int idx) {
+        Meta m;
+        const int lb = idx / n_blocks, w = lb >> 6, q = lb & 63;
+        if (w != win) {   // (the same decision in every lane)
+            const int b = (w << 6) + lane;
+            win_e = b < sub_used ? a.sorted_expert_ids[b / bpb] : -1;
+            win = w;
+        }
+        const int e_lb = __shfl(win_e, q, 64);
+        const unsigned long long same = __ballot(win_e == e_lb);
+        const unsigned long long below = ~same & ((1ull << q) - 1ull), above = ~same & ~((2ull << q) - 1ull);
+        const int b0 = (w << 6) + (below ? 64 - __builtin_clzll(below) : 0);
+        const int b1 = (w << 6) + ((q < 63 && above) ? __builtin_ctzll(above) : 64);
+        const int nb = b1 - b0, t = idx - b0 * n_blocks;   // 0 <= t < nb * n_blocks
+        m.bid_n = t / nb;
+        m.sb = b0 + (t - m.bid_n * nb);
+        const int slot0 = m.sb * kRows, last = a.num_slots - 1;
+        m.expert_raw = e_lb;
+        m.t0 = a.sorted_token_ids[slot0 + r0 < last ? slot0 + r0 : last];
+        m.t1 = a.sorted_token_ids[slot0 + r1 < last ? slot0 + r1 : last];
+        m.tm = a.sorted_token_ids[slot0 + (tid & 127) < last ? slot0 + (tid & 127) : last];
+        return m;
+    };
+    DLane ln;
+    {
+        const int chunk = (lane & 3) ^ ((lane >> 4) & 3);   // global chunk that belongs at this lane's LDS position
+        ln.kC = 8 * chunk;
+#pragma unroll
+        for (int ks = 0; ks < 2; ++ks) {
+            const int sw = 8 * ((2 * ks + hb) ^ (((lane & 31) >> 2) & 3));
+            ln.fT[ks] = (64 * ws + (lane & 31)) * BK + sw;
+            ln.fW[ks] = (64 * wn + (lane & 31)) * BK + sw;
+        }
+    }
+    // Addresses of a tile's transfers from what was read about it; returns this thread's slot's token (0 = none;
+    // every slot of a block without a valid expert counts as empty, and such a tile reads expert 1's rows).
+    auto setup = [&](const Meta& m, DLane& L) {
+        const int slot0 = m.sb * kRows;
+        int expert = m.expert_raw - 1;
+        const bool ok = expert >= 0 && expert < a.num_experts;
+        if (!ok) expert = 0;
+        auto fix = [&](int raw, int r) { return (ok && slot0 + r < a.num_slots && raw >= 1 && raw <= a.total_tokens) ? raw : 0; };
+        const int t0 = fix(m.t0, r0), t1 = fix(m.t1, r1);
+        const int chunk = L.kC >> 3;
+        const int c0 = t0 ? (t0 - 1) / a.replicas : 0, c1 = t1 ? (t1 - 1) / a.replicas : 0;   // slots without a token read column 0
+        L.gT[0] = (const char*)(a.A + (int64_t)c0 * a.lda + 8 * chunk);
+        L.gT[1] = (const char*)(a.A + (int64_t)c1 * a.lda + 8 * chunk);
+        const unsigned short* Bx = (const unsigned short*)a.B + (int64_t)expert * a.sbe;
+        const int half_n = a.N / 2;
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+            const int R = 64 * j + r0;   // tile row: wave column R / 64, MFMA tile (R / 32) & 1, channel R % 32 of it
+            int row;
+            if (MODE == MODE_SILU) {
+                int ch = m.bid_n * 64 + 32 * (R >> 6) + (R & 31);
+                if (ch > half_n - 1) ch = half_n - 1;
+                row = ((R >> 5) & 1) ? half_n + ch : ch;
+            } else {
+                row = m.bid_n * kRows + R;
+                if (row > a.N - 1) row = a.N - 1;
+            }
+            L.gW[j] = (const char*)(Bx + (int64_t)row * a.ldb + 8 * chunk);
+        }
+        return fix(m.tm, tid & 127);
+    };
+    auto routed_weight = [&](int tm) {
+        float w = 1.f;
+        if (a.mul_routed_weight && tm) {
+            // weight of replica q = token * w_topk + slot: element (token, slot) of the (num_tokens, topk) matrix (the
+            // flattened, slot-fastest vector of moe.jl:193 is the case w_topk = 1)
+            const int q = tm - 1, tk = q / a.w_topk;
+            w = widen16(a.bf16, a.topk_weights[tk * a.w_s0 + (q - tk * a.w_topk) * a.w_s1]);
+        }
+        return w;
+    };
+    auto publish = [&](int p, int tm, float w) {   // waves 0 and 1 hold the 128 slots
+        if (tid < kRows) {
+            s_tok[p][tid] = tm;
+            s_wt[p][tid] = w;
+        }
+        const unsigned long long has = __ballot(tm != 0);
+        if (wave < 2 && lane == 0) s_live[p][wave] = ((has & 0xffffffffull) ? 1u : 0u) | ((has >> 32) ? 2u : 0u);
+    };
+    // (tile 1 of a half without tile 0 does not occur with sorted slots; it is multiplied as two tiles)
+    auto live_of = [&](int p) { const unsigned l = s_live[p][ws]; return l == 0 ? 0 : l == 1 ? 1 : 2; };
+
+    // whole 16-byte pieces of C's rows can be stored as such
+    const bool vec_ok = ((uintptr_t)a.C % 16) == 0 && a.ldc % 8 == 0;
+    const Stages st{Ts0, Ts1, Ts2, Ts3, Ws0, Ws1, Ws2, Ws3};
+    Meta mc = load_meta(cur), mn = mc;
+    int p = 0;
+    {
+        const int tm = setup(mc, ln);
+        publish(0, tm, routed_weight(tm));
+    }
+    __syncthreads();
+    int nlive = live_of(0);
+    int nxt = cur + nslot;
+    bool have_next = nxt < hi;
+    if (have_next) mn = load_meta(nxt);
+    ring_fill(st, wave, ln);
+    for (;;) {
+        f32x16 acc[2][2];
+#pragma unroll
+        for (int i = 0; i < 2; ++i)
+#pragma unroll
+            for (int j = 0; j < 2; ++j) acc[i][j] = f32x16{0};
+        constexpr bool SL = MODE != MODE_ACC;
+        if (nlive == 2) main_loop<E, 2, SL>(st, a.K, wave, ln, acc);
+        else if (nlive == 1) main_loop<E, 1, SL>(st, a.K, wave, ln, acc);
+        else main_loop<E, 0, SL>(st, a.K, wave, ln, acc);
+        // the next tile's addresses and its routed weights (requested now, used after this tile's stores are out)
+        int tmN = 0;
+        float wN = 1.f;
+        if (have_next) {
+            tmN = setup(mn, ln);
+            wN = routed_weight(tmN);
+        }
+        epilogue<E, MODE>(a, acc, nlive, s_tok[p], s_wt[p], mc.bid_n, ws, wn, lane, vec_ok);
+        if (!have_next) break;
+        publish(p ^ 1, tmN, wN);
+        lds_only_barrier();   // every wave is done with the ring's stages, and the next tile's slots are in place
+        p ^= 1;
+        mc = mn;
+        nlive = live_of(p);
+        cur = nxt;
+        nxt += nslot;
+        have_next = nxt < hi;
+        if (have_next) mn = load_meta(nxt);
+        ring_fill(st, wave, ln);
+    }
+}
+
+}  // namespace
+
+namespace mi {
+namespace moe {
+
+bool dense_applicable(const DenseArgs& a) {
+    // MI_MOE_DENSE: 0 = never, 1 = wherever it can run (read at every call, so that one process can compare the kernels)
+    const char* env = getenv("MI_MOE_DENSE");
+    const int force = env ? atoi(env) : -1;
+    if (force == 0 || a.w8) return false;
+    if (a.TILE_M % kRows || a.K % 8 || a.K < 256 || a.N < 1) return false;
+    if (a.silu && (a.N % 2)) return false;
+    if (!aligned(a.A, 16) || !aligned(a.B, 16) || a.lda % 8 || a.ldb % 8 || a.sbe % 8) return false;
+    if (a.lda < 0 || a.ldb < 0) return false;
+    if (cld((int64_t)a.total_tokens, (int64_t)a.replicas) > a.num_a_cols) return false;   // (a replica without a column of A: the streaming kernel feeds it zeros)
+    if (a.acc_shift >= 0 && (a.N % 2)) return false;
+    const int64_t n_blocks = a.silu ? cld((int64_t)a.N / 2, (int64_t)64) : cld((int64_t)a.N, (int64_t)kRows);
+    if ((cld((int64_t)a.num_blocks * (a.TILE_M / kRows) * n_blocks, (int64_t)8) + 1) * 8 > MI_MAX_GRID_DIM) return false;
+    if (force == 1) return true;
+    // dense enough: more than 32 replicas per expert on average (what the streaming kernel's two-tile shape starts at)
+    return (int64_t)a.total_tokens >= 32ll * a.num_experts;
+}
+
+void dense_launch(const DenseArgs& a, hipStream_t s) {
+    const int n_blocks = a.silu ? (int)cld((int64_t)a.N / 2, (int64_t)64) : (int)cld((int64_t)a.N, (int64_t)kRows);
+    const int64_t tiles = (int64_t)a.num_blocks * (a.TILE_M / kRows) * n_blocks;
+    // persistent: two workgroups per CU at most (64 KB of LDS each), a multiple of 8 so that every XCD gets as many
+    const int64_t per_xcd = cld(tiles, (int64_t)8) < 64 ? cld(tiles, (int64_t)8) : 64;
+    const dim3 grid((unsigned)(per_xcd * 8));
+#define LAUNCH(ET, MODE) hipLaunchKernelGGL((moe_dense_kernel<ET, MODE>), grid, dim3(256), 0, s, a, n_blocks)
+    if (a.silu) {
+        if (a.bf16) LAUNCH(BF16, MODE_SILU);
+        else LAUNCH(F16, MODE_SILU);
+        set_variant("fused_moe_dense_silu_t128_n64x2_k32_ring4");
+    } else if (a.acc_shift >= 0) {
+        if (a.bf16) LAUNCH(BF16, MODE_ACC);
+        else LAUNCH(F16, MODE_ACC);
+        set_variant("fused_moe_dense_acc_t128_n128_k32_ring4");
+    } else {
+        if (a.bf16) LAUNCH(BF16, MODE_PLAIN);
+        else LAUNCH(F16, MODE_PLAIN);
+        set_variant("fused_moe_dense_t128_n128_k32_ring4");
+    }
+#undef LAUNCH
+}
+
+}  // namespace moe
+}  // namespace mi

@@ -25,6 +25,25 @@ def check(got, ref, tol=2e-2):
     assert np.all(err <= bound), f"max err {err.max():.3e}, worst ratio {np.max(err / bound):.3f}"
 
 
+class _dense_knob:
+    """MI_MOE_DENSE=0 keeps every launch on the streaming kernels, =1 sends every launch the ring kernel can take to it
+    (the library reads the variable at every call)."""
+    def __init__(self, value):
+        self.value = value
+
+    def __enter__(self):
+        import os
+        self.old = os.environ.get("MI_MOE_DENSE")
+        os.environ["MI_MOE_DENSE"] = self.value
+
+    def __exit__(self, *exc):
+        import os
+        if self.old is None:
+            os.environ.pop("MI_MOE_DENSE", None)
+        else:
+            os.environ["MI_MOE_DENSE"] = self.old
+
+
 @pytest.mark.parametrize("tokens,hidden,experts,inter,topk,router", [
     (48, 512, 64, 1024, 8, "randperm"), (128, 512, 32, 1024, 4, "randperm"), (64, 1024, 64, 2048, 8, "randperm"),
     (256, 512, 32, 512, 2, "top2_logits"), (7, 256, 3, 128, 2, "randperm"), (300, 256, 2, 256, 2, "randperm"),
@@ -290,7 +309,14 @@ def test_dense_routing_two_slot_tiles_per_workgroup(ct, orc):
     experts, moe.jl:311-344): a workgroup then multiplies two 32-slot tiles with the same weight tile.  The wide,
     and the fused-SiLU mainloops have that variant (dense routing always takes wide strips); every element is accumulated in the same order
     as with one tile per workgroup, so fused and separate paths still agree bit for bit, and the result is checked
-    against the float64 oracle.  Includes a small problem with unequal expert loads."""
+    against the float64 oracle.  Includes a small problem with unequal expert loads.  (These are the
+    streaming kernels' shapes for dense routing; they serve blocks smaller than 128 slots and e4m3 weights, and are
+    kept on here by the knob.)"""
+    with _dense_knob("0"):
+        _two_slot_tiles_body(ct, orc)
+
+
+def _two_slot_tiles_body(ct, orc):
     d = moe.prepare(benchmark=True, topk=8)
     tok, exp = ct.moe_align_tile_size_device(d.topk_ids, 128, d.num_experts)
     c1 = torch.zeros(d.num_tokens * 8, 2 * d.intermediate_size, dtype=torch.float16, device="cuda")
@@ -418,7 +444,7 @@ def test_down_projection_that_adds_into_the_output(ct, orc, tokens, hidden, expe
     assert ct.last_variant().startswith("moe_sum_topk")
     for _ in range(3):
         fused = moe.cutile_moe(d.hidden_states, w1, w2, d.topk_weights, d.topk_ids, 128, 128, 64, fuse_sum=True, **kw)
-        assert ct.last_variant().startswith("fused_moe_t")          # the last launch is the GEMM itself
+        assert ct.last_variant().startswith(("fused_moe_t", "fused_moe_dense_acc"))          # the last launch is the GEMM itself
         assert torch.equal(fused, plain)
     default = moe.cutile_moe(d.hidden_states, w1, w2, d.topk_weights, d.topk_ids, 128, 128, 64, **kw)
     assert torch.equal(default, plain)
@@ -460,3 +486,90 @@ def test_replicas_with_an_expert_id_out_of_range_contribute_nothing(orc, topk):
     if topk <= 2:
         sep = moe.cutile_moe(d.hidden_states, d.w1, d.w2, d.topk_weights, ids, 16, 128, 64, device_align=True, fuse_sum=False)
         assert torch.equal(sep, got)
+
+
+def _every_path(d, tile_m, **kw):
+    """cutile_moe over its launch sequences: fused SiLU + accumulating down projection (where top-k allows), fused SiLU
+    + separate sum, and the reference's kernel-by-kernel sequence."""
+    outs = {}
+    a = (d.hidden_states, d.w1, d.w2, d.topk_weights, d.topk_ids, tile_m, 128, 64)
+    if d.topk <= 2 and d.hidden_size % 8 == 0:
+        outs["fused"] = moe.cutile_moe(*a, **kw)
+    outs["fused_silu"] = moe.cutile_moe(*a, fuse_sum=False, **kw)
+    outs["separate"] = moe.cutile_moe(*a, fuse_silu=False, fuse_sum=False, **kw)
+    return outs
+
+
+@pytest.mark.parametrize("shape", [
+    dict(benchmark=True, topk=8),                                                                     # the reference example's routing
+    dict(num_tokens=1024, hidden_size=1024, num_experts=32, intermediate_size=2048, topk=2, router="top2_logits"),
+    dict(num_tokens=300, hidden_size=328, num_experts=3, intermediate_size=200, topk=2),               # K and N off the tile grid
+    dict(num_tokens=700, hidden_size=264, num_experts=5, intermediate_size=96, topk=1),                # one slot per token
+    dict(num_tokens=1024, hidden_size=256, num_experts=160, intermediate_size=128, topk=8),
+    dict(num_tokens=2048, hidden_size=256, num_experts=256, intermediate_size=64, topk=8),
+    dict(num_tokens=400, hidden_size=512, num_experts=4, intermediate_size=256, topk=2, T=torch.bfloat16),
+])
+def test_dense_routing_ring_kernel_gives_the_streaming_kernels_bits(ct, orc, shape):
+    """The grouped GEMM for dense routing (128-slot x 128-channel tiles fed by a ring of LDS stages, persistent
+    workgroups) against the streaming kernels on the same launches: every output element is accumulated over k in
+    the same order by both, so plain, SiLU-fused and accumulating launches have to agree bit for bit; the result is
+    also checked against the float64 oracle.  Shapes: the reference example's own routing (moe.jl:311-344), a prefill
+    batch, sizes off the tile grid (K = 328 ends in a zero-padded group of steps, N = 400 in clipped strips), one slot
+    per token, 160 and 256 experts, bf16."""
+    d = moe.prepare(**shape)
+    J = orc.to_julia
+    with _dense_knob("0"):
+        ref_outs = _every_path(d, 128)
+    names = set()
+    with _dense_knob("1"):
+        outs = _every_path(d, 128)
+        tok, exp = ct.moe_align_tile_size_device(d.topk_ids, 128, d.num_experts)
+        c1 = torch.empty(d.num_tokens * d.topk, 2 * d.intermediate_size, dtype=d.hidden_states.dtype, device="cuda")
+        moe.invoke_fused_moe_kernel(d.hidden_states, d.w1, c1, d.topk_weights, tok, exp, mul_routed_weight=False,
+                                    num_token_replicas=d.topk, tile_m=128, tile_n=128, tile_k=64)
+        names.add(ct.last_variant())
+        c2 = torch.empty(d.num_tokens * d.topk, d.intermediate_size, dtype=d.hidden_states.dtype, device="cuda")
+        moe.invoke_fused_moe_kernel(d.hidden_states, d.w1, c2, d.topk_weights, tok, exp, mul_routed_weight=False,
+                                    num_token_replicas=d.topk, tile_m=128, tile_n=128, tile_k=64, fuse_silu=True)
+        names.add(ct.last_variant())
+    assert names == {"fused_moe_dense_t128_n128_k32_ring4", "fused_moe_dense_silu_t128_n64x2_k32_ring4"}
+    for k in outs:
+        assert not torch.isnan(outs[k].float()).any(), k
+        assert torch.equal(outs[k], ref_outs[k]), k
+        assert torch.equal(outs[k], outs["separate"]), k
+    ref = orc.ref_moe(J(d.hidden_states), J(d.w1), J(d.w2), J(d.topk_weights), J(d.topk_ids), dtype=np.float64)
+    check(J(outs["separate"]), ref, 5e-2 if d.hidden_states.dtype == torch.bfloat16 else 2e-2)
+
+
+def test_dense_ring_kernel_other_block_sizes_sorts_and_output_layouts(ct, orc):
+    """TILE_M = 256 (two 128-slot tiles per block, the second often empty), the host-side sort (exact block count),
+    and an output whose rows are not whole 16-byte pieces (element-wise stores instead of 16-byte ones)."""
+    d = moe.prepare(num_tokens=600, hidden_size=384, num_experts=6, intermediate_size=320, topk=2)
+    J = orc.to_julia
+    ref = orc.ref_moe(J(d.hidden_states), J(d.w1), J(d.w2), J(d.topk_weights), J(d.topk_ids), dtype=np.float64)
+    with _dense_knob("0"):
+        want = moe.cutile_moe(d.hidden_states, d.w1, d.w2, d.topk_weights, d.topk_ids, 128, 128, 64, fuse_sum=False)
+    with _dense_knob("1"):
+        for tile_m, device_align in ((256, True), (256, False), (128, False), (512, True)):
+            got = moe.cutile_moe(d.hidden_states, d.w1, d.w2, d.topk_weights, d.topk_ids, tile_m, 128, 64,
+                                 device_align=device_align, fuse_sum=False)
+            assert torch.equal(got, want), (tile_m, device_align)
+            if device_align:
+                acc = moe.cutile_moe(d.hidden_states, d.w1, d.w2, d.topk_weights, d.topk_ids, tile_m, 128, 64)
+                assert torch.equal(acc, want), tile_m
+        check(J(want), ref)
+        # rows of C that start off a 16-byte boundary: leading dimension 2 * inter + 4 elements
+        total, inter = d.num_tokens * d.topk, d.intermediate_size
+        tok, exp = ct.moe_align_tile_size_device(d.topk_ids, 128, d.num_experts)
+        wide = torch.full((total, 2 * inter + 4), 7.0, dtype=torch.float16, device="cuda")
+        dense_c1 = torch.empty(total, 2 * inter, dtype=torch.float16, device="cuda")
+        for c in (wide[:, :2 * inter], dense_c1):
+            moe.invoke_fused_moe_kernel(d.hidden_states, d.w1, c, d.topk_weights, tok, exp, mul_routed_weight=False,
+                                        num_token_replicas=d.topk, tile_m=128, tile_n=128, tile_k=64)
+            assert ct.last_variant() == "fused_moe_dense_t128_n128_k32_ring4"
+        assert torch.equal(wide[:, :2 * inter], dense_c1)
+        assert bool((wide[:, 2 * inter:] == 7.0).all()), "the kernel wrote past the rows of its output"
+    # 128-slot tiles need TILE_M to be a multiple of 128: smaller blocks stay on the streaming kernels
+    with _dense_knob("1"):
+        moe.cutile_moe(d.hidden_states, d.w1, d.w2, d.topk_weights, d.topk_ids, 64, 128, 64, fuse_sum=False)
+        assert "dense" not in ct.last_variant()

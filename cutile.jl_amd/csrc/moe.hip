@@ -732,7 +732,8 @@ extern "C" int mi_fused_moe_accumulate_kernel(const mi_tile_array* A, const mi_t
 // of moe.jl:150 orders them.  The outputs have fixed capacity: unused slots hold the sentinel
 // total+1, unused blocks expert 0, which the GEMM kernel skips.
 constexpr int kAlignMaxExperts = 1024;
-constexpr int kAlignThreads = 1024, kAlignWaves = kAlignThreads / 64, kAlignCached = 2;
+constexpr int kAlignThreads = 1024, kAlignWaves = kAlignThreads / 64;
+constexpr int kAlignBatch = 8;   // super-blocks whose ids a thread requests together: one memory round trip per batch
 __global__ __launch_bounds__(kAlignThreads) void moe_align_kernel(const long long* __restrict__ topk_ids, int64_t ld_slot,
                                                         int num_tokens, int topk, int tile_m, int num_experts,
                                                         int* __restrict__ sorted_token_ids, int cap_slots,
@@ -749,16 +750,17 @@ __global__ __launch_bounds__(kAlignThreads) void moe_align_kernel(const long lon
         return;
     }
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, total = num_tokens * topk;
-    // The ids of the first kAlignCached super-blocks stay in registers between the counting pass and the placing
-    // pass, and are requested before the tables are cleared: one memory round trip instead of three in a row.
+    // A thread requests the ids of kAlignBatch super-blocks at a time, all loads before the first use: a batch costs one
+    // memory round trip instead of one per super-block.  The first batch (8192 replicas) stays in registers between the
+    // counting pass and the placing pass and is requested before the tables are cleared.
     auto expert_of = [&](int r) {
         if (r >= total) return -1;
         const long long v = topk_ids[(r / topk) + (int64_t)(r % topk) * ld_slot];
         return (v >= 1 && v <= num_experts) ? (int)v - 1 : -1;
     };
-    int ecache[kAlignCached];
+    int ecache[kAlignBatch];
 #pragma unroll
-    for (int i = 0; i < kAlignCached; ++i) ecache[i] = expert_of(tid + kAlignThreads * i);
+    for (int i = 0; i < kAlignBatch; ++i) ecache[i] = expert_of(tid + kAlignThreads * i);
     for (int e = tid; e < num_experts; e += kAlignThreads) {
         cursor[e] = 0;
 #pragma unroll
@@ -767,11 +769,15 @@ __global__ __launch_bounds__(kAlignThreads) void moe_align_kernel(const long lon
     for (int i = tid; i < cap_slots; i += kAlignThreads) sorted_token_ids[i] = total + 1;
     __syncthreads();
 #pragma unroll
-    for (int i = 0; i < kAlignCached; ++i)
+    for (int i = 0; i < kAlignBatch; ++i)
         if (ecache[i] >= 0) atomicAdd(&cursor[ecache[i]], 1);
-    for (int r = tid + kAlignThreads * kAlignCached; r < total; r += kAlignThreads) {
-        const int e = expert_of(r);
-        if (e >= 0) atomicAdd(&cursor[e], 1);
+    for (int r0 = kAlignThreads * kAlignBatch; r0 < total; r0 += kAlignThreads * kAlignBatch) {
+        int eb[kAlignBatch];
+#pragma unroll
+        for (int i = 0; i < kAlignBatch; ++i) eb[i] = expert_of(r0 + tid + kAlignThreads * i);
+#pragma unroll
+        for (int i = 0; i < kAlignBatch; ++i)
+            if (eb[i] >= 0) atomicAdd(&cursor[eb[i]], 1);
     }
     __syncthreads();
     {   // exclusive scan of the experts' block counts (thread e owns expert e): shuffles inside a
@@ -799,36 +805,37 @@ __global__ __launch_bounds__(kAlignThreads) void moe_align_kernel(const long lon
 
     const unsigned long long lt = lane ? (~0ull >> (64 - lane)) : 0ull;
     const int id_bits = 32 - __builtin_clz((unsigned)(num_experts > 1 ? num_experts - 1 : 1));
-    for (int r0 = 0; r0 < total; r0 += kAlignThreads) {
-        const int r = r0 + tid;
-        int e;
-        {
-            const int sb = r0 / kAlignThreads;   // super-block (uniform): the first ones are in registers
-            if (sb == 0) e = ecache[0];
-            else if (sb == 1 && kAlignCached > 1) e = ecache[kAlignCached > 1 ? 1 : 0];
-            else e = expert_of(r);
-        }
-        // the lanes of this wave that hold the same expert: one ballot per bit of the expert id
-        unsigned long long m = __ballot(e >= 0);
-        for (int b = 0; b < id_bits; ++b) {
-            const unsigned long long bal = __ballot((e >> b) & 1);
-            m &= ((e >> b) & 1) ? bal : ~bal;
-        }
-        const int rank = __popcll(m & lt);
-        if (e >= 0 && rank == 0) tbl[wave][e] = (unsigned short)__popcll(m);
-        __syncthreads();   // the table is complete, and the cursors of the previous super-block have been advanced
-        if (e >= 0) {
-            int pos = cursor[e] + rank;
+    for (int b0 = 0; b0 < total; b0 += kAlignThreads * kAlignBatch) {
+        int eb[kAlignBatch];
 #pragma unroll
-            for (int w = 0; w < kAlignWaves; ++w) pos += w < wave ? (int)tbl[w][e] : 0;   // (all sixteen reads in flight)
-            if (pos < cap_slots) sorted_token_ids[pos] = r + 1;
-        }
-        __syncthreads();   // every lane has read the cursors and the table
-        // Advance the cursors and clear the table.  The entries touched are those of this super-block's experts, and
-        // an entry is written by its own wave only (now, and when the next super-block is counted): no third barrier.
-        if (e >= 0 && rank == 0) {  // first lane of its expert within the wave
-            atomicAdd(&cursor[e], (int)tbl[wave][e]);
-            tbl[wave][e] = 0;
+        for (int i = 0; i < kAlignBatch; ++i) eb[i] = b0 == 0 ? ecache[i] : expert_of(b0 + tid + kAlignThreads * i);
+#pragma unroll
+        for (int i = 0; i < kAlignBatch; ++i) {
+            const int r0 = b0 + kAlignThreads * i;
+            if (r0 >= total) break;   // (the same decision in every thread)
+            const int r = r0 + tid, e = eb[i];
+            // the lanes of this wave that hold the same expert: one ballot per bit of the expert id
+            unsigned long long m = __ballot(e >= 0);
+            for (int b = 0; b < id_bits; ++b) {
+                const unsigned long long bal = __ballot((e >> b) & 1);
+                m &= ((e >> b) & 1) ? bal : ~bal;
+            }
+            const int rank = __popcll(m & lt);
+            if (e >= 0 && rank == 0) tbl[wave][e] = (unsigned short)__popcll(m);
+            __syncthreads();   // the table is complete, and the cursors of the previous super-block have been advanced
+            if (e >= 0) {
+                int pos = cursor[e] + rank;
+#pragma unroll
+                for (int w = 0; w < kAlignWaves; ++w) pos += w < wave ? (int)tbl[w][e] : 0;   // (all sixteen reads in flight)
+                if (pos < cap_slots) sorted_token_ids[pos] = r + 1;
+            }
+            __syncthreads();   // every lane has read the cursors and the table
+            // Advance the cursors and clear the table.  The entries touched are those of this super-block's experts, and
+            // an entry is written by its own wave only (now, and when the next super-block is counted): no third barrier.
+            if (e >= 0 && rank == 0) {  // first lane of its expert within the wave
+                atomicAdd(&cursor[e], (int)tbl[wave][e]);
+                tbl[wave][e] = 0;
+            }
         }
     }
 }

@@ -3,27 +3,34 @@
 // hundreds of tokens per expert the product is no longer a weight stream with a few MFMAs attached (moe.hip) but a
 // GEMM per expert, and takes the big GEMM's structure (gemm_big.hip):
 //
-//   workgroup tile = 128 sorted slots of one expert x 128 weight rows (channels); 4 waves as 2 (slots) x 2
-//   (channels), each 64 x 64 = 2 x 2 MFMA 32x32x16 tiles; K walked in steps of 32 through a ring of four LDS
-//   stages (4 x 16 KB: two workgroups per CU) filled by direct global->LDS transfers with no staging registers;
-//   the token rows of a stage are gathered (every lane of a transfer carries the address of its own token's row),
-//   the weight rows carry the expert's offset; transfers for step s+3 / s+4 are issued between the MFMAs of step s;
-//   one barrier per step that waits for the oldest stage in flight only.
+//   workgroup tile = 128 sorted slots of one expert x 64 * J weight rows (channels); 4 waves as 2 (slots) x 2
+//   (channels), each 64 slots x 32 * J channels = 2 x J MFMA 32x32x16 tiles; K walked in steps of 32 through a ring of
+//   LDS stages filled by direct global->LDS transfers with no staging registers (J = 2: four stages of 16 KB, J = 4:
+//   three of 24 KB; two workgroups per CU either way); the token rows of a stage are gathered (every lane of a
+//   transfer carries the address of its own token's row), the weight rows carry the expert's offset; the transfers of
+//   later steps are issued between the MFMAs of a step; one barrier per step that waits for the oldest stage in
+//   flight only.
 //
 // Both operands are K-contiguous, so both LDS tiles are [row][32 k] with the 16-byte chunks of a row XOR-swizzled
-// by (row >> 2) & 3, and both fragments are plain 16-byte reads.  The MFMA column operand (lane % 32) carries the
-// channel, so a store of C is a run of 32 consecutive channels; the row operand carries the slot.  k is walked in
-// ascending order with the k <-> lane map of the streaming kernel (moe.hip), so every output element is accumulated
-// in the same order as there and the two kernels give the same bits.
+// by (row >> 2) & 3, and both fragments are plain 16-byte reads.  What bounds the K walk is the LDS pipe (128 bytes
+// per clock and CU for fragment reads and transfer writes together): with J = 2 a step of two workgroups needs 768
+// of its cycles against 512 of the matrix pipe, with J = 4 1152 against 1024.  k is walked in ascending order with
+// the k <-> lane map of the streaming kernel (moe.hip), whichever operand the lanes of the result carry, so every
+// output element is accumulated in the same order as there and the two kernels give the same bits.
 //
 // 32-slot tiles that hold only padding are never multiplied: a wave whose slots are all padding only takes part in
-// the transfers and barriers.  Workgroups are numbered so that every XCD works on a contiguous range of the blocks
-// in use, strips of one block next to each other: a block's 128 token rows are fetched into that XCD's L2 once, and
-// the two or three blocks of one expert stream its weights at the same time.
+// the transfers and barriers.  Workgroups are persistent (two per CU) and walk the tiles of their XCD's range with a
+// stride; what a tile needs to know (expert, token ids) is requested a tile ahead, and a tile's stores and the next
+// tile's ring fill are issued back to back.  Within a run of blocks of one expert the tiles are numbered strip-major,
+// so the workgroups of an XCD work on a few weight strips of all of the expert's blocks at a time: a strip is
+// fetched into that L2 once, and the blocks' token rows stay there while the strips pass.
 //
-// Epilogues: plain (optionally times the routed weight), SiLU(gate) * up (the tile's 128 weight rows are 64 gate
-// channels and the 64 up channels that go with them, arranged so that a lane holds both halves of an output
-// element), and the accumulating form (packed atomic adds into the token's output column, one or two slots per token).
+// Epilogues: plain (optionally times the routed weight) and SiLU(gate) * up (the tile's weight rows are gate channels
+// and the up channels that go with them, arranged so that a lane holds both halves of an output element) have the
+// slot in the lane: a lane holds runs of four channels of its token's row, two lane-half swaps make them runs of
+// eight, and the stores are 16 bytes per lane.  The accumulating form (packed atomic adds into the token's output
+// column, one or two slots per token) has the channel in the lane, so that an atomic instruction covers whole
+// 128-byte lines.
 #include "gemm_direct.h"
 #include "moe_dense.h"
 
@@ -45,36 +52,40 @@ __device__ __forceinline__ float widen16(bool bf16, unsigned short h) {
     return bf16 ? __uint_as_float(((unsigned)h) << 16) : (float)__builtin_bit_cast(_Float16, h);
 }
 
+// J: MFMA column tiles (32 channels each) per wave.  J = 2: tile of 128 weight rows, ring of four stages of 16 KB;
+// J = 4: 256 weight rows, ring of three stages of 24 KB.  Either way two workgroups fit a CU.
+template <int J>
 struct DLane {
     const char* gT[2];   // global address, at k = 0, of the lane's 16-byte chunk in the wave's two token transfers
-    const char* gW[2];   // the same in its two weight transfers
+    const char* gW[J];   // the same in its J weight transfers
     int kC;              // first k, within a stage, of that chunk
     unsigned fT[2], fW[2];   // LDS element offset of the token / weight fragment of sub-step 0 / 1 (+ 32 * BK per 32-row tile)
 };
 
+template <int J>
 struct DFrag {
-    s16x8 t[2], w[2];
+    s16x8 t[2], w[J];
 };
 
-// An operand stage is 128 rows x 64 B = eight transfers of 1 KB (16 rows each); wave w takes transfers w and w + 4.
+// An operand stage of 64 * N rows x 64 B is 4 * N transfers of 1 KB (16 rows each); wave w takes transfers w, w + 4, ...
 // TAIL: k_left = K - (first k of the stage); chunks at or past it come from the zero block.
-template <bool TAIL>
-__device__ __forceinline__ void issue2(const char* const (&g)[2], int64_t koff, unsigned short* S, int wave, int kC,
+template <bool TAIL, int N>
+__device__ __forceinline__ void issueN(const char* const (&g)[N], int64_t koff, unsigned short* S, int wave, int kC,
                                        int k_left) {
 #pragma unroll
-    for (int j = 0; j < 2; ++j) {
+    for (int j = 0; j < N; ++j) {
         const char* p = g[j] + koff;
         if (TAIL && kC >= k_left) p = (const char*)zeros16d;
         gload_lds16(p, S + (wave + 4 * j) * 512);
     }
 }
 
-template <int LIVE>
-__device__ __forceinline__ void load_frags(const unsigned short* Ts, const unsigned short* Ws, const DLane& ln, int ks,
-                                           DFrag& f) {
+template <int LIVE, int J>
+__device__ __forceinline__ void load_frags(const unsigned short* Ts, const unsigned short* Ws, const DLane<J>& ln, int ks,
+                                           DFrag<J>& f) {
     if (LIVE == 0) return;
 #pragma unroll
-    for (int j = 0; j < 2; ++j) f.w[j] = *reinterpret_cast<const s16x8*>(Ws + ln.fW[ks] + 32 * j * BK);
+    for (int j = 0; j < J; ++j) f.w[j] = *reinterpret_cast<const s16x8*>(Ws + ln.fW[ks] + 32 * j * BK);
 #pragma unroll
     for (int i = 0; i < LIVE; ++i) f.t[i] = *reinterpret_cast<const s16x8*>(Ts + ln.fT[ks] + 32 * i * BK);
 }
@@ -82,46 +93,49 @@ __device__ __forceinline__ void load_frags(const unsigned short* Ts, const unsig
 // SLOT_LANE: the MFMA column operand (lane % 32 of the result) carries the slot and the rows the channel: a lane
 // then holds four consecutive channels of one token's row in four consecutive registers.  Otherwise the lane carries
 // the channel and the rows the slots.  The products and the order in which an element's k are added are the same.
-template <typename E, int LIVE, bool SLOT_LANE>
-__device__ __forceinline__ void mma(const DFrag& f, f32x16 (&acc)[2][2]) {
+template <typename E, int LIVE, bool SLOT_LANE, int J>
+__device__ __forceinline__ void mma(const DFrag<J>& f, f32x16 (&acc)[2][J]) {
 #pragma unroll
     for (int i = 0; i < LIVE; ++i)
 #pragma unroll
-        for (int j = 0; j < 2; ++j)
+        for (int j = 0; j < J; ++j)
             acc[i][j] = SLOT_LANE ? E::mfma32(f.w[j], f.t[i], acc[i][j]) : E::mfma32(f.t[i], f.w[j], acc[i][j]);
 }
 
-// Spread the fragment reads and the two transfers of a half step over its MFMAs.
-template <int LIVE, bool DMA, bool FRAGS>
+// Spread the fragment reads (2 + J) and the transfers (NDMA) of a half step over its 2 * J MFMAs.
+template <int LIVE, int J, int NDMA, bool FRAGS>
 __device__ __forceinline__ void interleave() {
     if constexpr (LIVE == 2) {
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
+        for (int i = 0; i < 2 * J; ++i) {
             __builtin_amdgcn_sched_group_barrier(SG_MFMA, 1, 0);
-            if (FRAGS) __builtin_amdgcn_sched_group_barrier(SG_DSRD, 1, 0);
-            if (DMA && (i & 1) == 0) __builtin_amdgcn_sched_group_barrier(SG_VMEM, 1, 0);
+            if (FRAGS && i < 2 + J) __builtin_amdgcn_sched_group_barrier(SG_DSRD, 1, 0);
+            if (NDMA && (i * NDMA) / (2 * J) != ((i + 1) * NDMA) / (2 * J)) __builtin_amdgcn_sched_group_barrier(SG_VMEM, 1, 0);
         }
     }
     __builtin_amdgcn_sched_barrier(0);
 }
 
 // One K step of 32 on stage X; the next step's data is in stage Y.
-//   first half : MFMAs of sub-step 0 | read sub-step 1 fragments | token transfers of step s + 3 (into stage TsA)
+//   first half : MFMAs of sub-step 0 | read sub-step 1 fragments | token transfers of a later step (into stage TsA)
 //   barrier
-//   second half: MFMAs of sub-step 1 | read the next stage's sub-step 0 fragments | weight transfers of step s + 4 (into WsX)
-template <typename E, int LIVE, bool SLOT_LANE, bool DMA_T, bool DMA_W, int VMCNT, bool LAST, bool TAIL>
+//   second half: MFMAs of sub-step 1 | read the next stage's sub-step 0 fragments | weight transfers of a later step (into WsX)
+// The ring of four stages (J = 2) requests tokens three steps ahead and weights four; the ring of three (J = 4) two
+// and three.  koffT / koffW: byte offsets along a row of the stages requested; k_leftT / k_leftW: K less their first k.
+template <typename E, int LIVE, bool SLOT_LANE, int J, bool DMA_T, bool DMA_W, int VMCNT, bool LAST, bool TAIL>
 __device__ __forceinline__ void k_step(const unsigned short* TsX, unsigned short* WsX, const unsigned short* TsY,
-                                       const unsigned short* WsY, unsigned short* TsA, int64_t koff3, int wave,
-                                       const DLane& ln, DFrag& f0, DFrag& f1, f32x16 (&acc)[2][2], int k_left3) {
-    if (DMA_T) issue2<TAIL>(ln.gT, koff3, TsA, wave, ln.kC, k_left3);
-    load_frags<LIVE>(TsX, WsX, ln, 1, f1);
-    mma<E, LIVE, SLOT_LANE>(f0, acc);
-    interleave<LIVE, DMA_T, true>();
+                                       const unsigned short* WsY, unsigned short* TsA, int64_t koffT, int64_t koffW,
+                                       int wave, const DLane<J>& ln, DFrag<J>& f0, DFrag<J>& f1, f32x16 (&acc)[2][J],
+                                       int k_leftT, int k_leftW) {
+    if (DMA_T) issueN<TAIL, 2>(ln.gT, koffT, TsA, wave, ln.kC, k_leftT);
+    load_frags<LIVE, J>(TsX, WsX, ln, 1, f1);
+    mma<E, LIVE, SLOT_LANE, J>(f0, acc);
+    interleave<LIVE, J, DMA_T ? 2 : 0, true>();
     if (!LAST) stage_barrier<VMCNT>();
-    if (DMA_W) issue2<TAIL>(ln.gW, koff3 + 2 * BK, WsX, wave, ln.kC, k_left3 - BK);
-    if (!LAST) load_frags<LIVE>(TsY, WsY, ln, 0, f0);
-    mma<E, LIVE, SLOT_LANE>(f1, acc);
-    interleave<LIVE, DMA_W, !LAST>();
+    if (DMA_W) issueN<TAIL, J>(ln.gW, koffW, WsX, wave, ln.kC, k_leftW);
+    if (!LAST) load_frags<LIVE, J>(TsY, WsY, ln, 0, f0);
+    mma<E, LIVE, SLOT_LANE, J>(f1, acc);
+    interleave<LIVE, J, DMA_W ? J : 0, !LAST>();
 }
 
 struct Stages {
@@ -130,49 +144,83 @@ struct Stages {
 
 constexpr int64_t kStepBytes = BK * 2;   // bytes along a row per K step
 
-// What a tile requests before its first step: stages 0..2 and the weight half of stage 3 (2 + 2 transfers per wave and
-// stage).
-__device__ __forceinline__ void ring_fill(const Stages& st, int wave, const DLane& ln) {
-    issue2<false>(ln.gW, 0, st.W0, wave, ln.kC, 0);
-    issue2<false>(ln.gT, 0, st.T0, wave, ln.kC, 0);
-    issue2<false>(ln.gW, kStepBytes, st.W1, wave, ln.kC, 0);
-    issue2<false>(ln.gT, kStepBytes, st.T1, wave, ln.kC, 0);
-    issue2<false>(ln.gW, 2 * kStepBytes, st.W2, wave, ln.kC, 0);
-    issue2<false>(ln.gT, 2 * kStepBytes, st.T2, wave, ln.kC, 0);
-    issue2<false>(ln.gW, 3 * kStepBytes, st.W3, wave, ln.kC, 0);
+// What a tile requests before its first step.  Ring of four: stages 0..2 and the weight half of stage 3; ring of three:
+// stages 0, 1 and the weight half of stage 2.
+template <int J>
+__device__ __forceinline__ void ring_fill(const Stages& st, int wave, const DLane<J>& ln) {
+    issueN<false, J>(ln.gW, 0, st.W0, wave, ln.kC, 0);
+    issueN<false, 2>(ln.gT, 0, st.T0, wave, ln.kC, 0);
+    issueN<false, J>(ln.gW, kStepBytes, st.W1, wave, ln.kC, 0);
+    issueN<false, 2>(ln.gT, kStepBytes, st.T1, wave, ln.kC, 0);
+    issueN<false, J>(ln.gW, 2 * kStepBytes, st.W2, wave, ln.kC, 0);
+    if constexpr (J == 2) {
+        issueN<false, 2>(ln.gT, 2 * kStepBytes, st.T2, wave, ln.kC, 0);
+        issueN<false, J>(ln.gW, 3 * kStepBytes, st.W3, wave, ln.kC, 0);
+    }
 }
 
-// The K walk of one tile whose ring has been filled.  Its first wait leaves the ten youngest transfers in flight:
-// whatever the wave requested before the ring fill (the previous tile's stores, the next tile's token ids) is older
-// and completes first.
-template <typename E, int LIVE, bool SLOT_LANE>
-__device__ __forceinline__ void main_loop(const Stages& st, int K, int wave, const DLane& ln, f32x16 (&acc)[2][2]) {
-    const int KT = 4 * ((K + 4 * BK - 1) / (4 * BK));   // steps, in whole groups of four; >= 8 (K >= 256 is checked on the host)
-    DFrag f0, f1;
-    stage_barrier<2 * 4 + 2>();
-    load_frags<LIVE>(st.T0, st.W0, ln, 0, f0);
-#define KSTEP(X, Y, AA, DT, DW, VM, LAST, TAIL, s)                                                                   \
-    k_step<E, LIVE, SLOT_LANE, DT, DW, (VM) * 4, LAST, TAIL>(st.T##X, st.W##X, st.T##Y, st.W##Y, st.T##AA, (int64_t)((s) + 3) * kStepBytes, \
-                                                  wave, ln, f0, f1, acc, K - ((s) + 3) * BK)
-    int s = 0;
-    for (; s + 12 <= KT; s += 4) {
-        KSTEP(0, 1, 3, true, true, 2, false, false, s);
-        KSTEP(1, 2, 0, true, true, 2, false, false, s + 1);
-        KSTEP(2, 3, 1, true, true, 2, false, false, s + 2);
-        KSTEP(3, 0, 2, true, true, 2, false, false, s + 3);
-    }
-    // the group that requests the last four stages (the only ones that can reach past K)
-    KSTEP(0, 1, 3, true, true, 2, false, true, s);
-    KSTEP(1, 2, 0, true, true, 2, false, true, s + 1);
-    KSTEP(2, 3, 1, true, true, 2, false, true, s + 2);
-    KSTEP(3, 0, 2, true, true, 2, false, true, s + 3);
-    s += 4;
-    // last four steps: only the token half of the final stage is still to be requested
-    KSTEP(0, 1, 3, true, false, 2, false, true, s);
-    KSTEP(1, 2, 0, false, false, 1, false, false, s + 1);
-    KSTEP(2, 3, 1, false, false, 0, false, false, s + 2);
-    KSTEP(3, 0, 2, false, false, 0, true, false, s + 3);
+// The K walk of one tile whose ring has been filled.  Its first wait leaves the youngest transfers of the fill in
+// flight (all but stage 0): whatever the wave requested before the ring fill (the previous tile's stores, the next
+// tile's token ids) is older and completes first.
+template <typename E, int LIVE, bool SLOT_LANE, int J>
+__device__ __forceinline__ void main_loop(const Stages& st, int K, int wave, const DLane<J>& ln, f32x16 (&acc)[2][J]) {
+    DFrag<J> f0, f1;
+    constexpr int PER = 2 + J;   // transfers per wave and stage
+    if constexpr (J == 2) {
+        const int KT = 4 * ((K + 4 * BK - 1) / (4 * BK));   // steps, in whole groups of four; >= 8 (K >= 256 is checked on the host)
+        stage_barrier<2 * PER + J>();
+        load_frags<LIVE, J>(st.T0, st.W0, ln, 0, f0);
+#define KSTEP(X, Y, AA, DT, DW, VM, LAST, TAIL, s)                                                                          \
+    k_step<E, LIVE, SLOT_LANE, J, DT, DW, (VM) * PER, LAST, TAIL>(st.T##X, st.W##X, st.T##Y, st.W##Y, st.T##AA,            \
+                                                               (int64_t)((s) + 3) * kStepBytes, (int64_t)((s) + 4) * kStepBytes, \
+                                                               wave, ln, f0, f1, acc, K - ((s) + 3) * BK, K - ((s) + 4) * BK)
+        int s = 0;
+        for (; s + 12 <= KT; s += 4) {
+            KSTEP(0, 1, 3, true, true, 2, false, false, s);
+            KSTEP(1, 2, 0, true, true, 2, false, false, s + 1);
+            KSTEP(2, 3, 1, true, true, 2, false, false, s + 2);
+            KSTEP(3, 0, 2, true, true, 2, false, false, s + 3);
+        }
+        // the group that requests the last four stages (the only ones that can reach past K)
+        KSTEP(0, 1, 3, true, true, 2, false, true, s);
+        KSTEP(1, 2, 0, true, true, 2, false, true, s + 1);
+        KSTEP(2, 3, 1, true, true, 2, false, true, s + 2);
+        KSTEP(3, 0, 2, true, true, 2, false, true, s + 3);
+        s += 4;
+        // last four steps: only the token half of the final stage is still to be requested
+        KSTEP(0, 1, 3, true, false, 2, false, true, s);
+        KSTEP(1, 2, 0, false, false, 1, false, false, s + 1);
+        KSTEP(2, 3, 1, false, false, 0, false, false, s + 2);
+        KSTEP(3, 0, 2, false, false, 0, true, false, s + 3);
 #undef KSTEP
+    } else {
+        // Ring of three: step s requests the tokens of step s + 2 (into the stage freed half a step ago) and, behind
+        // its barrier, the weights of step s + 3 (into its own stage).  At the barrier of step s the transfers
+        // younger than the tokens of step s + 1 are the weights of s + 2 and the tokens of s + 2: J + 2.
+        const int KT = 3 * ((K + 3 * BK - 1) / (3 * BK));   // steps, in whole groups of three (up to two of zeros); >= 9
+        stage_barrier<PER + J>();
+        load_frags<LIVE, J>(st.T0, st.W0, ln, 0, f0);
+#define KSTEP(X, Y, AA, DT, DW, VM, LAST, TAIL, s)                                                                          \
+    k_step<E, LIVE, SLOT_LANE, J, DT, DW, VM, LAST, TAIL>(st.T##X, st.W##X, st.T##Y, st.W##Y, st.T##AA,                    \
+                                                       (int64_t)((s) + 2) * kStepBytes, (int64_t)((s) + 3) * kStepBytes,    \
+                                                       wave, ln, f0, f1, acc, K - ((s) + 2) * BK, K - ((s) + 3) * BK)
+        int s = 0;
+        for (; s + 9 <= KT; s += 3) {
+            KSTEP(0, 1, 2, true, true, PER, false, false, s);
+            KSTEP(1, 2, 0, true, true, PER, false, false, s + 1);
+            KSTEP(2, 0, 1, true, true, PER, false, false, s + 2);
+        }
+        // the group that requests the last stages (the only ones that can reach past K)
+        KSTEP(0, 1, 2, true, true, PER, false, true, s);
+        KSTEP(1, 2, 0, true, true, PER, false, true, s + 1);
+        KSTEP(2, 0, 1, true, true, PER, false, true, s + 2);
+        s += 3;
+        // last three steps: only the tokens of the final stage are still to be requested
+        KSTEP(0, 1, 2, true, false, PER, false, true, s);
+        KSTEP(1, 2, 0, false, false, 0, false, false, s + 1);
+        KSTEP(2, 0, 1, false, false, 0, true, false, s + 2);
+#undef KSTEP
+    }
 }
 
 // Barrier that waits for the wave's LDS accesses only (the transfers, loads and stores in flight stay in flight).
@@ -224,8 +272,8 @@ __device__ __forceinline__ void store_tile_slot_lane(const float (&o)[16], unsig
 }
 
 // Stores of one tile.
-template <typename E, int MODE>
-__device__ __forceinline__ void epilogue(const DenseArgs& a, const f32x16 (&acc)[2][2], int nlive, const int* s_tok,
+template <typename E, int MODE, int J>
+__device__ __forceinline__ void epilogue(const DenseArgs& a, const f32x16 (&acc)[2][J], int nlive, const int* s_tok,
                                          const float* s_wt, int bid_n, int ws, int wn, int lane, bool vec_ok) {
     const int hb = lane >> 5;
 #pragma unroll
@@ -235,58 +283,64 @@ __device__ __forceinline__ void epilogue(const DenseArgs& a, const f32x16 (&acc)
         const int tokv = s_tok[64 * ws + 32 * i + (lane & 31)];
         const float wtv = s_wt[64 * ws + 32 * i + (lane & 31)];
         if constexpr (MODE == MODE_SILU) {
-            // lane = slot; register r of the gate tile and of the up tile are the same output channel
-            const int ch0 = bid_n * 64 + 32 * wn;   // the wave's first output channel, < N / 2
-            float o[16];
+            // lane = slot; register r of gate tile jj and of up tile J / 2 + jj are the same output channel
 #pragma unroll
-            for (int r = 0; r < 16; ++r) {
-                float g = acc[i][0][r], u = acc[i][1][r];
-                if (a.mul_routed_weight) {
-                    g *= wtv;
-                    u *= wtv;
+            for (int jj = 0; jj < J / 2; ++jj) {
+                const int ch0 = bid_n * (32 * J) + 16 * J * wn + 32 * jj;   // first output channel of the pair of tiles, < N / 2
+                float o[16];
+#pragma unroll
+                for (int r = 0; r < 16; ++r) {
+                    float g = acc[i][jj][r], u = acc[i][J / 2 + jj][r];
+                    if (a.mul_routed_weight) {
+                        g *= wtv;
+                        u *= wtv;
+                    }
+                    // both halves rounded to the activation type, as the unfused GEMM stores them
+                    g = widen16(a.bf16, E::from_f32(g));
+                    u = widen16(a.bf16, E::from_f32(u));
+                    o[r] = mi::moe::silu_mul(g, u);
                 }
-                // both halves rounded to the activation type, as the unfused GEMM stores them
-                g = widen16(a.bf16, E::from_f32(g));
-                u = widen16(a.bf16, E::from_f32(u));
-                o[r] = mi::moe::silu_mul(g, u);
+                store_tile_slot_lane<E>(o, a.C + (int64_t)(tokv ? tokv - 1 : 0) * a.ldc + ch0, tokv != 0, a.N / 2 - ch0, vec_ok, hb);
             }
-            store_tile_slot_lane<E>(o, a.C + (int64_t)(tokv ? tokv - 1 : 0) * a.ldc + ch0, tokv != 0, a.N / 2 - ch0, vec_ok, hb);
         } else if constexpr (MODE == MODE_PLAIN) {
 #pragma unroll
-            for (int j = 0; j < 2; ++j) {
-                const int ch0 = bid_n * kRows + 64 * wn + 32 * j;
+            for (int j = 0; j < J; ++j) {
+                const int ch0 = bid_n * (64 * J) + 32 * J * wn + 32 * j;
                 float o[16];
 #pragma unroll
                 for (int r = 0; r < 16; ++r) o[r] = a.mul_routed_weight ? acc[i][j][r] * wtv : acc[i][j][r];
                 store_tile_slot_lane<E>(o, a.C + (int64_t)(tokv ? tokv - 1 : 0) * a.ldc + ch0, tokv != 0, a.N - ch0, vec_ok, hb);
             }
         } else {
-            // lane = channel; rows of a 32 x 32 tile = slots 8 * (r / 4) + 4 * hb + r % 4.  The wave's two MFMA column
-            // tiles are 64 consecutive channels: swapping the upper half of tile 0's register with the lower half of
-            // tile 1's gives one register with all 64 channels of row R and one with those of row R + 4.  Column
-            // (token_id - 1) >> acc_shift receives the replica's value as rounded to the storage type, by a packed
-            // atomic add of two adjacent channels: even lanes send row R, odd lanes row R + 4, each row 128
+            // lane = channel; rows of a 32 x 32 tile = slots 8 * (r / 4) + 4 * hb + r % 4.  Two neighbouring MFMA column
+            // tiles are 64 consecutive channels: swapping the upper half of the first one's register with the lower half
+            // of the second one's gives one register with all 64 channels of row R and one with those of row R + 4.
+            // Column (token_id - 1) >> acc_shift receives the replica's value as rounded to the storage type, by a
+            // packed atomic add of two adjacent channels: even lanes send row R, odd lanes row R + 4, each row 128
             // consecutive bytes.
-            const int gn = bid_n * kRows + 64 * wn + lane;
 #pragma unroll
-            for (int r = 0; r < 16; ++r) {
-                const int R = 8 * (r >> 2) + (r & 3);
-                const int tokA = __builtin_amdgcn_readlane(tokv, R), tokB = __builtin_amdgcn_readlane(tokv, R + 4);
-                float v0 = acc[i][0][r], v1 = acc[i][1][r];
-                if (a.mul_routed_weight) {
-                    const float wA = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, wtv), R));
-                    const float wB = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, wtv), R + 4));
-                    const float w = hb ? wB : wA;
-                    v0 *= w;
-                    v1 *= w;
+            for (int jp = 0; jp < J; jp += 2) {
+                const int gn = bid_n * (64 * J) + 32 * J * wn + 32 * jp + lane;
+#pragma unroll
+                for (int r = 0; r < 16; ++r) {
+                    const int R = 8 * (r >> 2) + (r & 3);
+                    const int tokA = __builtin_amdgcn_readlane(tokv, R), tokB = __builtin_amdgcn_readlane(tokv, R + 4);
+                    float v0 = acc[i][jp][r], v1 = acc[i][jp + 1][r];
+                    if (a.mul_routed_weight) {
+                        const float wA = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, wtv), R));
+                        const float wB = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, wtv), R + 4));
+                        const float w = hb ? wB : wA;
+                        v0 *= w;
+                        v1 *= w;
+                    }
+                    const auto sw = __builtin_amdgcn_permlane32_swap((unsigned)E::from_f32(v0), (unsigned)E::from_f32(v1), false, false);
+                    const unsigned rowA = sw[0], rowB = sw[1];   // this lane's channel of row R / of row R + 4
+                    const unsigned nbrA = (unsigned)__shfl_xor((int)rowA, 1, 64), nbrB = (unsigned)__shfl_xor((int)rowB, 1, 64);
+                    const int tok = (lane & 1) ? tokB : tokA;
+                    const unsigned pair = (lane & 1) ? (nbrB | (rowB << 16)) : (rowA | (nbrA << 16));
+                    if (tok && gn < a.N)
+                        mi::moe::atomic_add2(a.bf16, a.C + (gn & ~1) + (int64_t)((tok - 1) >> a.acc_shift) * a.ldc, pair);
                 }
-                const auto sw = __builtin_amdgcn_permlane32_swap((unsigned)E::from_f32(v0), (unsigned)E::from_f32(v1), false, false);
-                const unsigned rowA = sw[0], rowB = sw[1];   // this lane's channel of row R / of row R + 4
-                const unsigned nbrA = (unsigned)__shfl_xor((int)rowA, 1, 64), nbrB = (unsigned)__shfl_xor((int)rowB, 1, 64);
-                const int tok = (lane & 1) ? tokB : tokA;
-                const unsigned pair = (lane & 1) ? (nbrB | (rowB << 16)) : (rowA | (nbrA << 16));
-                if (tok && gn < a.N)
-                    mi::moe::atomic_add2(a.bf16, a.C + (gn & ~1) + (int64_t)((tok - 1) >> a.acc_shift) * a.ldc, pair);
             }
         }
     }
@@ -296,10 +350,12 @@ __device__ __forceinline__ void epilogue(const DenseArgs& a, const f32x16 (&acc)
 // stride.  A tile's stores, and the next tile's ring fill right behind them, are in flight while nothing else of the
 // workgroup is: the next tile's K walk starts as soon as its first stage has landed, and what a tile needs to know
 // (expert, token ids) is requested one tile ahead.
-template <typename E, int MODE>
-__global__ __launch_bounds__(256) void moe_dense_kernel(const DenseArgs a, int n_blocks) {
-    __shared__ __attribute__((aligned(1024))) unsigned short Ts0[kStage], Ts1[kStage], Ts2[kStage], Ts3[kStage];
-    __shared__ __attribute__((aligned(1024))) unsigned short Ws0[kStage], Ws1[kStage], Ws2[kStage], Ws3[kStage];
+template <typename E, int MODE, int J>
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) void moe_dense_kernel(const DenseArgs a, int n_blocks) {
+    constexpr int kStageW = 64 * J * BK;   // elements of a weight stage: 64 * J rows of 32 k
+    constexpr int kLast = J == 2 ? 1 : 0;  // the ring of three has no fourth stage
+    __shared__ __attribute__((aligned(1024))) unsigned short Ts0[kStage], Ts1[kStage], Ts2[kStage], Ts3[kLast ? kStage : 8];
+    __shared__ __attribute__((aligned(1024))) unsigned short Ws0[kStageW], Ws1[kStageW], Ws2[kStageW], Ws3[kLast ? kStageW : 8];
     __shared__ int s_tok[2][kRows];      // 1-based replica id of every slot, 0 = no token (two tiles: current and next)
     __shared__ float s_wt[2][kRows];     // its routed weight (1 where none is applied)
     __shared__ unsigned s_live[2][2];    // per half of the block: bit i = its 32-slot tile i holds a token
@@ -360,7 +416,7 @@ __global__ __launch_bounds__(256) void moe_dense_kernel(const DenseArgs a, int n
         m.tm = a.sorted_token_ids[slot0 + (tid & 127) < last ? slot0 + (tid & 127) : last];
         return m;
     };
-    DLane ln;
+    DLane<J> ln;
     {
         const int chunk = (lane & 3) ^ ((lane >> 4) & 3);   // global chunk that belongs at this lane's LDS position
         ln.kC = 8 * chunk;
@@ -368,12 +424,12 @@ __global__ __launch_bounds__(256) void moe_dense_kernel(const DenseArgs a, int n
         for (int ks = 0; ks < 2; ++ks) {
             const int sw = 8 * ((2 * ks + hb) ^ (((lane & 31) >> 2) & 3));
             ln.fT[ks] = (64 * ws + (lane & 31)) * BK + sw;
-            ln.fW[ks] = (64 * wn + (lane & 31)) * BK + sw;
+            ln.fW[ks] = (32 * J * wn + (lane & 31)) * BK + sw;
         }
     }
     // Addresses of a tile's transfers from what was read about it; returns this thread's slot's token (0 = none;
     // every slot of a block without a valid expert counts as empty, and such a tile reads expert 1's rows).
-    auto setup = [&](const Meta& m, DLane& L) {
+    auto setup = [&](const Meta& m, DLane<J>& L) {
         const int slot0 = m.sb * kRows;
         int expert = m.expert_raw - 1;
         const bool ok = expert >= 0 && expert < a.num_experts;
@@ -387,15 +443,16 @@ __global__ __launch_bounds__(256) void moe_dense_kernel(const DenseArgs a, int n
         const unsigned short* Bx = (const unsigned short*)a.B + (int64_t)expert * a.sbe;
         const int half_n = a.N / 2;
 #pragma unroll
-        for (int j = 0; j < 2; ++j) {
-            const int R = 64 * j + r0;   // tile row: wave column R / 64, MFMA tile (R / 32) & 1, channel R % 32 of it
+        for (int j = 0; j < J; ++j) {
+            // tile row R: wave column R / (32 * J), MFMA tile (R / 32) % J of it, channel R % 32 of that
+            const int R = 64 * j + r0, wcol = R / (32 * J), tj = (R >> 5) % J;
             int row;
-            if (MODE == MODE_SILU) {
-                int ch = m.bid_n * 64 + 32 * (R >> 6) + (R & 31);
+            if (MODE == MODE_SILU) {   // tiles 0 .. J/2 - 1 of a wave are gate channels, the others the up channels that go with them
+                int ch = m.bid_n * (32 * J) + 16 * J * wcol + 32 * (tj % (J / 2)) + (R & 31);
                 if (ch > half_n - 1) ch = half_n - 1;
-                row = ((R >> 5) & 1) ? half_n + ch : ch;
+                row = tj >= J / 2 ? half_n + ch : ch;
             } else {
-                row = m.bid_n * kRows + R;
+                row = m.bid_n * (64 * J) + R;
                 if (row > a.N - 1) row = a.N - 1;
             }
             L.gW[j] = (const char*)(Bx + (int64_t)row * a.ldb + 8 * chunk);
@@ -437,17 +494,17 @@ __global__ __launch_bounds__(256) void moe_dense_kernel(const DenseArgs a, int n
     int nxt = cur + nslot;
     bool have_next = nxt < hi;
     if (have_next) mn = load_meta(nxt);
-    ring_fill(st, wave, ln);
+    ring_fill<J>(st, wave, ln);
     for (;;) {
-        f32x16 acc[2][2];
+        f32x16 acc[2][J];
 #pragma unroll
         for (int i = 0; i < 2; ++i)
 #pragma unroll
-            for (int j = 0; j < 2; ++j) acc[i][j] = f32x16{0};
+            for (int j = 0; j < J; ++j) acc[i][j] = f32x16{0};
         constexpr bool SL = MODE != MODE_ACC;
-        if (nlive == 2) main_loop<E, 2, SL>(st, a.K, wave, ln, acc);
-        else if (nlive == 1) main_loop<E, 1, SL>(st, a.K, wave, ln, acc);
-        else main_loop<E, 0, SL>(st, a.K, wave, ln, acc);
+        if (nlive == 2) main_loop<E, 2, SL, J>(st, a.K, wave, ln, acc);
+        else if (nlive == 1) main_loop<E, 1, SL, J>(st, a.K, wave, ln, acc);
+        else main_loop<E, 0, SL, J>(st, a.K, wave, ln, acc);
         // the next tile's addresses and its routed weights (requested now, used after this tile's stores are out)
         int tmN = 0;
         float wN = 1.f;
@@ -455,7 +512,7 @@ __global__ __launch_bounds__(256) void moe_dense_kernel(const DenseArgs a, int n
             tmN = setup(mn, ln);
             wN = routed_weight(tmN);
         }
-        epilogue<E, MODE>(a, acc, nlive, s_tok[p], s_wt[p], mc.bid_n, ws, wn, lane, vec_ok);
+        epilogue<E, MODE, J>(a, acc, nlive, s_tok[p], s_wt[p], mc.bid_n, ws, wn, lane, vec_ok);
         if (!have_next) break;
         publish(p ^ 1, tmN, wN);
         lds_only_barrier();   // every wave is done with the ring's stages, and the next tile's slots are in place
@@ -466,7 +523,7 @@ __global__ __launch_bounds__(256) void moe_dense_kernel(const DenseArgs a, int n
         nxt += nslot;
         have_next = nxt < hi;
         if (have_next) mn = load_meta(nxt);
-        ring_fill(st, wave, ln);
+        ring_fill<J>(st, wave, ln);
     }
 }
 
@@ -486,34 +543,55 @@ bool dense_applicable(const DenseArgs& a) {
     if (a.lda < 0 || a.ldb < 0) return false;
     if (cld((int64_t)a.total_tokens, (int64_t)a.replicas) > a.num_a_cols) return false;   // (a replica without a column of A: the streaming kernel feeds it zeros)
     if (a.acc_shift >= 0 && (a.N % 2)) return false;
-    const int64_t n_blocks = a.silu ? cld((int64_t)a.N / 2, (int64_t)64) : cld((int64_t)a.N, (int64_t)kRows);
+    const int64_t n_blocks = a.silu ? cld((int64_t)a.N / 2, (int64_t)64) : cld((int64_t)a.N, (int64_t)kRows);   // (the narrower tile)
     if ((cld((int64_t)a.num_blocks * (a.TILE_M / kRows) * n_blocks, (int64_t)8) + 1) * 8 > MI_MAX_GRID_DIM) return false;
     if (force == 1) return true;
     // dense enough: more than 32 replicas per expert on average (what the streaming kernel's two-tile shape starts at)
     return (int64_t)a.total_tokens >= 32ll * a.num_experts;
 }
 
+// Channels per tile: 256 weight rows per workgroup (four MFMA column tiles per wave, three ring stages) halve the LDS
+// fragment reads per MFMA -- 0.75 KB against 1 KB, and the LDS pipe (128 bytes per clock and CU) is what bounds the
+// K walk of the narrower tile -- and are taken when they still give every workgroup slot of the chip a tile and a
+// half; otherwise 128 rows (two column tiles per wave, four stages).  MI_MOE_DENSE_J = 2 | 4 forces one.
+static int pick_j(const DenseArgs& a) {
+    const char* env = getenv("MI_MOE_DENSE_J");
+    const int force = env ? atoi(env) : 0;
+    if (force == 2 || force == 4) return force;
+    const int64_t strips4 = a.silu ? cld((int64_t)a.N / 2, (int64_t)128) : cld((int64_t)a.N, (int64_t)256);
+    // blocks that hold tokens: at most one partly filled block per expert on top of the full ones
+    const int64_t blocks = cld((int64_t)a.total_tokens, (int64_t)kRows) + a.num_experts / 2;
+    return blocks * strips4 >= 768 ? 4 : 2;
+}
+
 void dense_launch(const DenseArgs& a, hipStream_t s) {
-    const int n_blocks = a.silu ? (int)cld((int64_t)a.N / 2, (int64_t)64) : (int)cld((int64_t)a.N, (int64_t)kRows);
+    const int J = pick_j(a);
+    const int n_blocks = a.silu ? (int)cld((int64_t)a.N / 2, (int64_t)(32 * J)) : (int)cld((int64_t)a.N, (int64_t)(64 * J));
     const int64_t tiles = (int64_t)a.num_blocks * (a.TILE_M / kRows) * n_blocks;
-    // persistent: two workgroups per CU at most (64 KB of LDS each), a multiple of 8 so that every XCD gets as many
+    // persistent: two workgroups per CU at most (64 or 72 KB of LDS each), a multiple of 8 so that every XCD gets as many
     const int64_t per_xcd = cld(tiles, (int64_t)8) < 64 ? cld(tiles, (int64_t)8) : 64;
     const dim3 grid((unsigned)(per_xcd * 8));
-#define LAUNCH(ET, MODE) hipLaunchKernelGGL((moe_dense_kernel<ET, MODE>), grid, dim3(256), 0, s, a, n_blocks)
+#define LAUNCH1(ET, MODE, JJ) hipLaunchKernelGGL((moe_dense_kernel<ET, MODE, JJ>), grid, dim3(256), 0, s, a, n_blocks)
+#define LAUNCH(ET, MODE)              \
+    do {                              \
+        if (J == 4) LAUNCH1(ET, MODE, 4); \
+        else LAUNCH1(ET, MODE, 2);    \
+    } while (0)
     if (a.silu) {
         if (a.bf16) LAUNCH(BF16, MODE_SILU);
         else LAUNCH(F16, MODE_SILU);
-        set_variant("fused_moe_dense_silu_t128_n64x2_k32_ring4");
+        set_variant(J == 4 ? "fused_moe_dense_silu_t128_n128x2_k32_ring3" : "fused_moe_dense_silu_t128_n64x2_k32_ring4");
     } else if (a.acc_shift >= 0) {
         if (a.bf16) LAUNCH(BF16, MODE_ACC);
         else LAUNCH(F16, MODE_ACC);
-        set_variant("fused_moe_dense_acc_t128_n128_k32_ring4");
+        set_variant(J == 4 ? "fused_moe_dense_acc_t128_n256_k32_ring3" : "fused_moe_dense_acc_t128_n128_k32_ring4");
     } else {
         if (a.bf16) LAUNCH(BF16, MODE_PLAIN);
         else LAUNCH(F16, MODE_PLAIN);
-        set_variant("fused_moe_dense_t128_n128_k32_ring4");
+        set_variant(J == 4 ? "fused_moe_dense_t128_n256_k32_ring3" : "fused_moe_dense_t128_n128_k32_ring4");
     }
 #undef LAUNCH
+#undef LAUNCH1
 }
 
 }  // namespace moe

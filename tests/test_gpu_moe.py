@@ -187,7 +187,8 @@ def test_moe_full_size_top2(orc):
 
 @pytest.mark.parametrize("num_tokens,topk,E,tile_m", [(256, 2, 32, 128), (48, 8, 64, 16), (7, 3, 5, 4), (1, 1, 1, 128),
                                                       (1000, 4, 9, 32), (130, 2, 1000, 8),
-                                                      (512, 2, 32, 128), (512, 4, 7, 16), (513, 4, 7, 16), (2049, 1, 33, 64)])
+                                                      (512, 2, 32, 128), (512, 4, 7, 16), (513, 4, 7, 16), (2049, 1, 33, 64),
+                                                      (4096, 2, 32, 128), (4100, 3, 11, 128), (16385, 2, 160, 64)])   # one, two and five batches of ids
 def test_device_align_matches_host_routine(ct, orc, num_tokens, topk, E, tile_m):
     """The one-workgroup counting sort gives the host routine's arrays (stable per-expert order,
     sentinel padding) in the leading part of its fixed-capacity outputs, and marks the rest unused."""
@@ -509,13 +510,16 @@ def _every_path(d, tile_m, **kw):
     dict(num_tokens=2048, hidden_size=256, num_experts=256, intermediate_size=64, topk=8),
     dict(num_tokens=400, hidden_size=512, num_experts=4, intermediate_size=256, topk=2, T=torch.bfloat16),
 ])
-def test_dense_routing_ring_kernel_gives_the_streaming_kernels_bits(ct, orc, shape):
+@pytest.mark.parametrize("J", ["2", "4"])
+def test_dense_routing_ring_kernel_gives_the_streaming_kernels_bits(ct, orc, shape, J, monkeypatch):
     """The grouped GEMM for dense routing (128-slot x 128-channel tiles fed by a ring of LDS stages, persistent
     workgroups) against the streaming kernels on the same launches: every output element is accumulated over k in
     the same order by both, so plain, SiLU-fused and accumulating launches have to agree bit for bit; the result is
     also checked against the float64 oracle.  Shapes: the reference example's own routing (moe.jl:311-344), a prefill
     batch, sizes off the tile grid (K = 328 ends in a zero-padded group of steps, N = 400 in clipped strips), one slot
-    per token, 160 and 256 experts, bf16."""
+    per token, 160 and 256 experts, bf16.  Both tile widths of the ring kernel: 128 weight rows on a ring of four stages
+    (J = 2) and 256 rows on a ring of three (J = 4, whose K walk is padded to whole groups of three steps)."""
+    monkeypatch.setenv("MI_MOE_DENSE_J", J)
     d = moe.prepare(**shape)
     J = orc.to_julia
     with _dense_knob("0"):
@@ -532,7 +536,8 @@ def test_dense_routing_ring_kernel_gives_the_streaming_kernels_bits(ct, orc, sha
         moe.invoke_fused_moe_kernel(d.hidden_states, d.w1, c2, d.topk_weights, tok, exp, mul_routed_weight=False,
                                     num_token_replicas=d.topk, tile_m=128, tile_n=128, tile_k=64, fuse_silu=True)
         names.add(ct.last_variant())
-    assert names == {"fused_moe_dense_t128_n128_k32_ring4", "fused_moe_dense_silu_t128_n64x2_k32_ring4"}
+    assert names in ({"fused_moe_dense_t128_n128_k32_ring4", "fused_moe_dense_silu_t128_n64x2_k32_ring4"},
+                     {"fused_moe_dense_t128_n256_k32_ring3", "fused_moe_dense_silu_t128_n128x2_k32_ring3"}), names
     for k in outs:
         assert not torch.isnan(outs[k].float()).any(), k
         assert torch.equal(outs[k], ref_outs[k]), k
@@ -566,7 +571,7 @@ def test_dense_ring_kernel_other_block_sizes_sorts_and_output_layouts(ct, orc):
         for c in (wide[:, :2 * inter], dense_c1):
             moe.invoke_fused_moe_kernel(d.hidden_states, d.w1, c, d.topk_weights, tok, exp, mul_routed_weight=False,
                                         num_token_replicas=d.topk, tile_m=128, tile_n=128, tile_k=64)
-            assert ct.last_variant() == "fused_moe_dense_t128_n128_k32_ring4"
+            assert ct.last_variant().startswith("fused_moe_dense_t128_")
         assert torch.equal(wide[:, :2 * inter], dense_c1)
         assert bool((wide[:, 2 * inter:] == 7.0).all()), "the kernel wrote past the rows of its output"
     # 128-slot tiles need TILE_M to be a multiple of 128: smaller blocks stay on the streaming kernels

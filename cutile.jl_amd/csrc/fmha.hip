@@ -255,7 +255,12 @@ __global__ __launch_bounds__(256) void fmha_fwd_kernel(const unsigned short* __r
 // fragment read from LDS feeds two MFMAs), for D = 128 four waves of 32 queries.  K and V tiles
 // of 64 keys travel global -> LDS with global_load_lds (no staging registers) into two stages;
 // the transfer of tile t+1 is issued right after the barrier that publishes tile t.
-//   K tile [key][d]: 16-byte chunk c of row `key` at position c ^ (key & 7)
+//   K tile [key][d]: 16-byte chunk c of row `key` at position c ^ ksw(key).  A 16-byte fragment read is served a
+//     quarter-wave (16 consecutive keys) at a time and has to spread those over all 64 banks: with rows of 128 bytes
+//     (D = 64) a row covers half the banks and two neighbouring keys differ in the half, so ksw = (key >> 1) & 7
+//     gives the eight key pairs eight different chunk positions; with rows of 256 bytes (D = 128) every row starts
+//     on bank 0 and ksw = key & 15 gives the sixteen keys sixteen positions.  (key & 7 put keys k and k + 8 of a
+//     quarter-wave on the same banks: two passes per read.)
 //   V tile [key][d]: chunk c at position c ^ ((D/32) * (key & 3)), which spreads the 4 rows x 32
 //     bytes of a transpose-read group over distinct banks.
 // Softmax bookkeeping per lane: running max m (shared by lanes l and l^32 after one exchange
@@ -264,6 +269,11 @@ __global__ __launch_bounds__(256) void fmha_fwd_kernel(const unsigned short* __r
 // weights that multiply V.  The accumulator is rescaled only on tiles where some row's max
 // actually rose.  Workgroups are numbered so that all query tiles of one (batch, head) run
 // on the same XCD and share its K/V in that XCD's L2.
+
+template <int D>
+__device__ __forceinline__ int ksw(int key) {
+    return D == 64 ? (key >> 1) & 7 : key & 15;
+}
 
 __device__ __forceinline__ void gload_lds16(const void* g, void* lds_wave_base) {
     __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)g,
@@ -407,6 +417,9 @@ __device__ __forceinline__ void tile_barrier() {
 // tile grows with its index, so a wave takes one early and one late tile, u and NT-1-u with
 // u = 2*qb + w; every wave then has the same number of MFMAs, and the two waves of a workgroup
 // need the same KV range.  The early tile simply drops out of the KV loop after its diagonal.
+constexpr int kFuseParts = 8;      // most parts that the last-arriving part adds up itself
+constexpr int kFuseRows = 64;      // most rows per (batch, head) for that
+constexpr int kFusePairs = 65536;  // most (query block, batch * head) pairs for that
 constexpr int kPartPad = 4;   // a part's row: D accumulator values, running maximum, row sum, two unused (16-byte rows)
 
 template <typename E, int D, int JT, bool CAUSAL, bool SPLIT = false>
@@ -414,7 +427,7 @@ __global__ __launch_bounds__(128 * 2 / JT) __attribute__((amdgpu_waves_per_eu(2,
     const unsigned short* __restrict__ Q, Strides qs, const unsigned short* __restrict__ K, Strides ks,
     const unsigned short* __restrict__ V, Strides vs, unsigned short* __restrict__ O, Strides os, int Sq, int Skv,
     int H, int group, float scale2, int input_pos, int nqb, int nbh, int pack, int nsplit = 1,
-    float* __restrict__ part = nullptr) {
+    float* __restrict__ part = nullptr, int* __restrict__ arrivals = nullptr) {
     using F = FmhaDma<E, D, JT, CAUSAL>;
     constexpr int NW = F::NW, KSTEPS = F::KSTEPS, DT = F::DT, CH = F::CH, TPW = F::TPW;
     constexpr bool PAIRED = CAUSAL && JT == 2;
@@ -499,7 +512,7 @@ __global__ __launch_bounds__(128 * 2 / JT) __attribute__((amdgpu_waves_per_eu(2,
     {
         const int key = lane & 31;
 #pragma unroll
-        for (int s = 0; s < KSTEPS; ++s) st.kfo[s] = key * D + 8 * ((2 * s + hb) ^ (key & 7));
+        for (int s = 0; s < KSTEPS; ++s) st.kfo[s] = key * D + 8 * ((2 * s + hb) ^ ksw<D>(key));
         const int g = lane >> 4, r = lane & 15;
 #pragma unroll
         for (int dt = 0; dt < DT; ++dt) {
@@ -513,7 +526,7 @@ __global__ __launch_bounds__(128 * 2 / JT) __attribute__((amdgpu_waves_per_eu(2,
     for (int i = 0; i < TPW; ++i) {
         const int t = wave + NW * i;  // transfer index: rows (512/D)*t ... of the tile
         const int key = (512 / D) * t + lane / CH, pos = lane % CH;
-        dl.koff[i] = (unsigned)(((int64_t)key * ks.s1 + 8 * (pos ^ (key & 7))) * 2);
+        dl.koff[i] = (unsigned)(((int64_t)key * ks.s1 + 8 * (pos ^ ksw<D>(key))) * 2);
         dl.voff[i] = (unsigned)(((int64_t)key * vs.s1 + 8 * (pos ^ ((D / 32) * (key & 3)))) * 2);
     }
 
@@ -543,7 +556,7 @@ __global__ __launch_bounds__(128 * 2 / JT) __attribute__((amdgpu_waves_per_eu(2,
                 const int tr = wave + NW * i;
                 int key = (512 / D) * tr + lane / CH;
                 const int pos = lane % CH;
-                const int swk = key & 7, swv = key & 3;
+                const int swk = ksw<D>(key), swv = key & 3;
                 if (t * kKV + key >= Skv) key = Skv - 1 - t * kKV;
                 cl.koff[i] = (unsigned)(((int64_t)key * ks.s1 + 8 * (pos ^ swk)) * 2);
                 cl.voff[i] = (unsigned)(((int64_t)key * vs.s1 + 8 * (pos ^ ((D / 32) * swv))) * 2);
@@ -583,6 +596,22 @@ __global__ __launch_bounds__(128 * 2 / JT) __attribute__((amdgpu_waves_per_eu(2,
             const float l_tot = st.l[j] + __shfl_xor(st.l[j], 32, 64);
             if (my_q[j] < R) {
                 float* pr = part + (((int64_t)sp * nbh + bh) * R + my_q[j]) * (D + kPartPad);
+                if (arrivals) {
+                    // (device-scope stores: written through to where the part that adds them up, on whatever XCD it
+                    // runs, reads them from -- no cache maintenance is needed on either side)
+#pragma unroll
+                    for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+                        for (int g = 0; g < 4; ++g)
+#pragma unroll
+                            for (int e = 0; e < 4; ++e)
+                                __hip_atomic_store(pr + 32 * dt + 8 * g + 4 * hb + e, st.o[j][dt][4 * g + e], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    if (hb == 0) {
+                        __hip_atomic_store(pr + D, st.m[j], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                        __hip_atomic_store(pr + D + 1, l_tot, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    }
+                    continue;
+                }
 #pragma unroll
                 for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
@@ -593,6 +622,63 @@ __global__ __launch_bounds__(128 * 2 / JT) __attribute__((amdgpu_waves_per_eu(2,
                         *reinterpret_cast<f32x4*>(pr + 32 * dt + 8 * g + 4 * hb) = w;
                     }
                 if (hb == 0) *reinterpret_cast<f32x2*>(pr + D) = f32x2{st.m[j], l_tot};
+            }
+        }
+        if (!arrivals) return;   // the parts are added by a launch of their own
+        // ---- the part that arrives last adds the parts (few rows and few parts: decode) ----------
+        // Every part writes its results with device-scope stores, waits until they have been performed, and then
+        // takes a ticket of its (query block, batch * head); the holder of the last ticket knows that all the others
+        // have published theirs.  The counter is left at zero for the next launch.  (Fences are avoided on purpose: a
+        // device-scope fence writes back and invalidates the whole L2 of the XCD, and one per workgroup made the
+        // launch twice as long.)
+        __shared__ int s_last;
+        const int pair = (int)blockIdx.x - sp * (nqb * nbh);
+        __builtin_amdgcn_s_waitcnt(0x0070);   // this wave's stores have been performed (vmcnt(0), lgkmcnt(0))
+        __syncthreads();                      // ... and so have the other waves'
+        if (tid == 0) {
+            const int ticket = __hip_atomic_fetch_add(arrivals + pair, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            s_last = ticket == nsplit - 1;
+            if (s_last) __hip_atomic_store(arrivals + pair, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+        __syncthreads();
+        if (!s_last) return;
+        {
+            constexpr int CPRW = D / 4, NTH = 128 * 2 / JT, RPP = NTH / CPRW;   // threads per row, rows per pass
+            const int c = tid % CPRW;
+            const int64_t part_stride = (int64_t)nbh * R * (D + kPartPad);
+            for (int row = tid / CPRW; row < R; row += RPP) {
+                const float* p0 = part + ((int64_t)bh * R + row) * (D + kPartPad);
+                // one pass with every part's loads in flight together (at most kFuseParts parts); device-scope loads
+                f32x2 ml[kFuseParts];
+                f32x4 o[kFuseParts];
+#pragma unroll
+                for (int q = 0; q < kFuseParts; ++q) {
+                    const float* pr = p0 + (q < nsplit ? q : 0) * part_stride;
+#pragma unroll
+                    for (int e = 0; e < 2; ++e) ml[q][e] = __hip_atomic_load(pr + D + e, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) o[q][e] = __hip_atomic_load(pr + 4 * c + e, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                }
+                float m = -INFINITY;
+#pragma unroll
+                for (int q = 0; q < kFuseParts; ++q) m = q < nsplit ? fmaxf(m, ml[q][0]) : m;
+                f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+                float l = 0.f;
+#pragma unroll
+                for (int q = 0; q < kFuseParts; ++q) {
+                    // (a part without a visible key for this row is left out, as in the combine kernel: same sums)
+                    const bool seen = q < nsplit && ml[q][0] != -INFINITY;
+                    const float w = seen ? __builtin_amdgcn_exp2f(ml[q][0] - m) : 0.f;
+                    l += seen ? w * ml[q][1] : 0.f;
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) acc[e] += seen ? w * o[q][e] : 0.f;
+                }
+                const float inv = __builtin_amdgcn_rcpf(l);
+                const int hq = row / Sq, q = row - hq * Sq;   // head within a stacked group, query
+                s16x4 out;
+#pragma unroll
+                for (int e = 0; e < 4; ++e) out[e] = E::cvt(acc[e] * inv);
+                *reinterpret_cast<s16x4*>(O + (int64_t)(head + hq) * os.s2 + (int64_t)batch * os.s3 + (int64_t)q * os.s1 + 4 * c) = out;
             }
         }
         return;
@@ -692,6 +778,9 @@ __global__ __launch_bounds__(256) void fmha_combine_kernel(const float* __restri
 // Scratch of the split launches (see shared_scratch.h for how its users are ordered).
 constexpr int64_t kPartFloats = 16 * 1024 * 1024;   // 64 MiB
 static __device__ __align__(256) float fmha_part_scratch[kPartFloats];
+// Arrival counters of the parts of a (query block, batch * head) pair; zero between launches (the part that arrives
+// last resets its counter).  Held under the same lease as the part array.
+static __device__ __align__(256) int fmha_part_arrivals[kFusePairs];
 SharedScratch g_part[16];
 
 // Number of parts for the launch, 0 = no split.
@@ -734,14 +823,35 @@ void launch(dim3 grid, hipStream_t s, bool causal, const mi_tile_array* Q, const
             ScratchLease lease;   // ends behind the combine launch
             if (float* scratch = (float*)lease.acquire(g_part, HIP_SYMBOL(fmha_part_scratch), s)) {
                 dim3 gs((unsigned)(nqb * nbh * parts));
+                // Few rows and few parts (one new token per sequence): the part that arrives last adds the parts
+                // itself, and the launch of the combine kernel (4 to 5 us behind a 23 us kernel) goes away.  The
+                // arrival counters are a static array as well; its address is looked up under the lease.
+                int* arrivals = nullptr;
+                static const bool fuse_on = [] { const char* e = getenv("MI_FMHA_FUSE_COMBINE"); return !e || atoi(e) != 0; }();   // 0: always the combine kernel
+                if (fuse_on && parts <= kFuseParts && (int64_t)Sq * pack <= kFuseRows && nqb == 1 && nbh <= kFusePairs) {
+                    static int* arr_ptr[16];
+                    int dev = 0;
+                    if (hipGetDevice(&dev) == hipSuccess && dev >= 0 && dev < 16) {
+                        if (!arr_ptr[dev] && hipGetSymbolAddress((void**)&arr_ptr[dev], HIP_SYMBOL(fmha_part_arrivals)) != hipSuccess) {
+                            arr_ptr[dev] = nullptr;
+                            (void)hipGetLastError();
+                        }
+                        arrivals = arr_ptr[dev];
+                    }
+                }
                 if (causal)
                     hipLaunchKernelGGL((fmha_fwd_dma_kernel<E, D, JT, true, true>), gs, blk, 0, s, (const unsigned short*)Q->ptr, qs,
                                        (const unsigned short*)K->ptr, ks, (const unsigned short*)V->ptr, vs,
-                                       (unsigned short*)O->ptr, os, Sq, Skv, Hb, group, scale2, input_pos, nqb, nbh, pack, parts, scratch);
+                                       (unsigned short*)O->ptr, os, Sq, Skv, Hb, group, scale2, input_pos, nqb, nbh, pack, parts, scratch, arrivals);
                 else
                     hipLaunchKernelGGL((fmha_fwd_dma_kernel<E, D, JT, false, true>), gs, blk, 0, s, (const unsigned short*)Q->ptr, qs,
                                        (const unsigned short*)K->ptr, ks, (const unsigned short*)V->ptr, vs,
-                                       (unsigned short*)O->ptr, os, Sq, Skv, Hb, group, scale2, input_pos, nqb, nbh, pack, parts, scratch);
+                                       (unsigned short*)O->ptr, os, Sq, Skv, Hb, group, scale2, input_pos, nqb, nbh, pack, parts, scratch, arrivals);
+                if (arrivals) {
+                    set_variant(pack > 1 ? (D == 64 ? "fmha_dma_q128_kv64_d64_w64q_grouped_splitkv_fused" : "fmha_dma_q128_kv64_d128_w32q_grouped_splitkv_fused")
+                                         : (D == 64 ? "fmha_dma_q128_kv64_d64_w64q_splitkv_fused" : "fmha_dma_q128_kv64_d128_w32q_splitkv_fused"));
+                    return;
+                }
                 constexpr int PLMAX = 256 / (D / 4) < 16 ? 256 / (D / 4) : 16;
 #define COMBINE(PL)                                                                                                              \
     hipLaunchKernelGGL((fmha_combine_kernel<E, D, PL>), dim3((unsigned)((rows * (D / 4) * PL + 255) / 256)), dim3(256), 0, s, scratch, \

@@ -12,16 +12,21 @@ namespace mi {
 struct SharedScratch {
     std::mutex mu;
     void* ptr = nullptr;
-    hipEvent_t done = nullptr;   // recorded by every user behind its last launch, on its own stream
+    hipEvent_t done = nullptr;   // once several streams use the array: recorded by every holder behind its last launch
+    hipStream_t last = nullptr;  // the previous holder's stream (compared, not used, except once: see acquire)
     bool used = false, broken = false;
+    bool multi = false;          // holders on more than one stream have been seen
 };
 
 // The array as held by one call: `ptr` is null if it can not be had (capturing stream, more than 16 devices, a failing
 // runtime call).  The holder enqueues its kernels while the lease lives, so the order in which streams take the array
-// is the order of their launches.  When the lease ends it records the array's event on the holder's own stream, still
-// under the lock; the next holder makes its stream wait for that event before anything else.  Only the stream of the
-// call at hand is ever touched: a stream that has been destroyed or has gone into capture since it used the array
-// plays no part.
+// is the order of their launches.  As long as every holder has come on the same stream, the stream's own order is all
+// there is to it and no event is touched (an event recorded behind every launch costs 2.5 to 3 us per call: a marker
+// between two kernels of a 25 us loop).  The first holder that comes on another stream switches the array to events
+// for good: from then on a lease that ends records the event on the holder's own stream, still under the lock, and
+// the next holder makes its stream wait for it.  Only that one switch records on the previous holder's stream (whose
+// launches no event covers yet); should that stream be gone or under capture by then, the call at hand is refused
+// the array and runs its unsplit kernel.
 class ScratchLease {
 public:
     ScratchLease() = default;
@@ -29,9 +34,10 @@ public:
     ScratchLease& operator=(const ScratchLease&) = delete;
     ~ScratchLease() {
         if (!ptr_) return;
-        if (hipEventRecord(st_->done, s_) == hipSuccess) {
-            st_->used = true;
-        } else {   // nothing orders the next holder behind this one: the array is not handed out again
+        st_->used = true;
+        st_->last = s_;
+        if (st_->multi && hipEventRecord(st_->done, s_) != hipSuccess) {
+            // nothing orders the next holder behind this one: the array is not handed out again
             (void)hipGetLastError();
             st_->broken = true;
         }
@@ -60,11 +66,21 @@ public:
                 return nullptr;
             }
         }
-        // (a wait for an event recorded on the same stream costs nothing; the handles are not compared, since a
-        // destroyed stream's handle can come back as a new stream's)
-        if (st.used && hipStreamWaitEvent(s, st.done, 0) != hipSuccess) {
-            (void)hipGetLastError();
-            return nullptr;
+        if (st.used && st.multi) {
+            if (hipStreamWaitEvent(s, st.done, 0) != hipSuccess) {
+                (void)hipGetLastError();
+                return nullptr;
+            }
+        } else if (st.used && st.last != s) {
+            st.multi = true;
+            hipStreamCaptureStatus prev = hipStreamCaptureStatusNone;
+            const bool ordered = hipStreamIsCapturing(st.last, &prev) == hipSuccess && prev == hipStreamCaptureStatusNone &&
+                                 hipEventRecord(st.done, st.last) == hipSuccess && hipStreamWaitEvent(s, st.done, 0) == hipSuccess;
+            if (!ordered) {
+                (void)hipGetLastError();
+                st.used = false;   // (whatever that stream was given has long been enqueued; the next holders order themselves by the event)
+                return nullptr;
+            }
         }
         st_ = &st;
         s_ = s;

@@ -120,7 +120,9 @@ def test_fmha_random_decode_and_chunked_prefill_shapes(ct):
         ref = F.scaled_dot_product_attention(d.Q.float(), K, V, attn_mask=mask)
         assert close(out, ref, 3e-2 if dt == torch.bfloat16 else 2e-2), \
             f"B={B} H={H} Sq={Sq} Skv={Skv} pos={pos} D={D} group={qg} causal={causal} {dt} {ct.last_variant()}"
-    assert any(v.endswith("_grouped_splitkv") for v in seen) and any(v.endswith("w64q_splitkv") or v.endswith("w32q_splitkv") for v in seen)
+    split = ("_splitkv", "_splitkv_fused")
+    assert any("_grouped_splitkv" in v for v in seen) and any(v.endswith(tuple("w64q" + e for e in split) + tuple("w32q" + e for e in split)) for v in seen)
+    assert any(v.endswith("_fused") for v in seen) and any(v.endswith("_splitkv") for v in seen), seen
     assert any(v.endswith("_grouped") for v in seen), seen
 
 

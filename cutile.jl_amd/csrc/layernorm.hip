@@ -565,8 +565,11 @@ __global__ __launch_bounds__(BLOCK) void ln_bwd_long_kernel(float* __restrict__ 
 // ---- backward: final reduction over the partial slots -----------------------------------
 // 64 consecutive n per workgroup; its 16 waves split the slots (independent loads, one round
 // trip for GROUP_SIZE_M <= 64), LDS combines them in a fixed order.
-__global__ __launch_bounds__(1024) void ln_dwdb_kernel(const float* __restrict__ DW, int64_t lddw,
-                                                       const float* __restrict__ DB, int64_t lddb,
+// CLEAR: every slot is set to zero once it has been read (the library's own slot array, which
+// the next call then finds ready for its atomic adds).
+template <bool CLEAR>
+__global__ __launch_bounds__(1024) void ln_dwdb_kernel(float* __restrict__ DW, int64_t lddw,
+                                                       float* __restrict__ DB, int64_t lddb,
                                                        float* __restrict__ FDW, float* __restrict__ FDB,
                                                        int64_t N, int G) {
     __shared__ float part[2][16][64];
@@ -578,6 +581,12 @@ __global__ __launch_bounds__(1024) void ln_dwdb_kernel(const float* __restrict__
         for (int g = wq; g < G; g += 16) {
             a += DW[n + g * lddw];
             b += DB[n + g * lddb];
+        }
+        if (CLEAR) {
+            for (int g = wq; g < G; g += 16) {
+                DW[n + g * lddw] = 0.f;
+                DB[n + g * lddb] = 0.f;
+            }
         }
     }
     part[0][wq][lane] = a;
@@ -601,6 +610,7 @@ static __device__ __align__(256) float scratch[2 * kScratchFloats];
 constexpr int kMaxDevices = 64;
 float* g_scratch_ptr[kMaxDevices];
 bool g_scratch_known[kMaxDevices];
+bool g_scratch_dirty[kMaxDevices];   // a call is under way, or one ended before its final kernel was launched
 
 // Device address of `scratch` on the current device; positive hipError_t on failure.  The lookup
 // (hipGetSymbolAddress may load the code object and is not a stream operation) happens once per
@@ -883,9 +893,8 @@ extern "C" int mi_layer_norm_bwd_dx_partial_dwdb(
     return launch_status();
 }
 
-extern "C" int mi_layer_norm_bwd_dwdb(const mi_tile_array* DW, const mi_tile_array* DB,
-                                      const mi_tile_array* FINAL_DW, const mi_tile_array* FINAL_DB,
-                                      int TILE_M, int TILE_N, void* stream) {
+static int dwdb_impl(const mi_tile_array* DW, const mi_tile_array* DB, const mi_tile_array* FINAL_DW,
+                     const mi_tile_array* FINAL_DB, int TILE_M, int TILE_N, bool clear, void* stream) {
     MI_CHECK(check_f32(DW, 2));
     MI_CHECK(check_f32(DB, 2));
     MI_CHECK(check_f32(FINAL_DW, 1));
@@ -897,17 +906,27 @@ extern "C" int mi_layer_norm_bwd_dwdb(const mi_tile_array* DW, const mi_tile_arr
     if (cld(N, (int64_t)TILE_N) > MI_MAX_GRID_DIM) return MI_E_GRID;
     if (N == 0) return MI_OK;
     if (G > 0x7fffffff) return MI_E_SHAPE;
-    hipLaunchKernelGGL(ln_dwdb_kernel, dim3((unsigned)cld(N, (int64_t)64)), dim3(1024), 0,
-                       (hipStream_t)stream, (const float*)DW->ptr, DW->strides[1],
-                       (const float*)DB->ptr, DB->strides[1], (float*)FINAL_DW->ptr,
-                       (float*)FINAL_DB->ptr, N, (int)G);
-    set_variant("ln_dwdb_b1024");
+    const dim3 grid((unsigned)cld(N, (int64_t)64));
+    if (clear)
+        hipLaunchKernelGGL(ln_dwdb_kernel<true>, grid, dim3(1024), 0, (hipStream_t)stream, (float*)DW->ptr, DW->strides[1],
+                           (float*)DB->ptr, DB->strides[1], (float*)FINAL_DW->ptr, (float*)FINAL_DB->ptr, N, (int)G);
+    else
+        hipLaunchKernelGGL(ln_dwdb_kernel<false>, grid, dim3(1024), 0, (hipStream_t)stream, (float*)DW->ptr, DW->strides[1],
+                           (float*)DB->ptr, DB->strides[1], (float*)FINAL_DW->ptr, (float*)FINAL_DB->ptr, N, (int)G);
+    set_variant(clear ? "ln_dwdb_b1024_clear" : "ln_dwdb_b1024");
     return launch_status();
 }
 
-// Backward in one call with the partial slots in the library's static scratch: zero fill,
-// layer_norm_bwd_dx_partial_dwdb, layer_norm_bwd_dwdb (layernorm.jl:245-251 issues the same three
-// steps on buffers its caller allocated, layernorm.jl:226-228).  Calls nothing that allocates.
+extern "C" int mi_layer_norm_bwd_dwdb(const mi_tile_array* DW, const mi_tile_array* DB,
+                                      const mi_tile_array* FINAL_DW, const mi_tile_array* FINAL_DB,
+                                      int TILE_M, int TILE_N, void* stream) {
+    return dwdb_impl(DW, DB, FINAL_DW, FINAL_DB, TILE_M, TILE_N, false, stream);
+}
+
+// Backward in one call with the partial slots in the library's static scratch:
+// layer_norm_bwd_dx_partial_dwdb and layer_norm_bwd_dwdb (layernorm.jl:245-251 issues a zero fill and
+// the same two steps on buffers its caller allocated, layernorm.jl:226-228; here the final kernel
+// leaves the slots zeroed for the next call, so the fill is not a launch).  Calls nothing that allocates.
 extern "C" int mi_layer_norm_bwd_static(const mi_tile_array* DX, const mi_tile_array* DY,
                                         const mi_tile_array* X, const mi_tile_array* W,
                                         const mi_tile_array* Mean, const mi_tile_array* Rstd,
@@ -935,14 +954,21 @@ extern "C" int mi_layer_norm_bwd_static(const mi_tile_array* DX, const mi_tile_a
         a->strides[0] = 1;
         a->strides[1] = ld;
     }
-    if (N > 0) {
-        const int64_t nvec = ld * G / 4;
-        const unsigned blocks = (unsigned)(nvec < 256 * 1024 ? cld(nvec, (int64_t)256) : 1024);
-        hipLaunchKernelGGL(fill_zero_kernel, dim3(blocks), dim3(256), 0, (hipStream_t)stream,
-                           (f32x4*)dw.ptr, (f32x4*)db.ptr, nvec);
+    if (N == 0) return MI_OK;
+    // The array is all zero when the library is loaded, and the final kernel of every call puts back the zeros where it
+    // has read sums: a call normally finds its slots ready and is two launches.  Only after a call that did not get
+    // as far as its final kernel (a failed launch) is the whole array filled first.
+    int dev = 0;
+    (void)hipGetDevice(&dev);
+    if (__atomic_exchange_n(&g_scratch_dirty[dev], true, __ATOMIC_ACQ_REL)) {
+        const int64_t nvec = kScratchFloats / 4;
+        hipLaunchKernelGGL(fill_zero_kernel, dim3(1024), dim3(256), 0, (hipStream_t)stream, (f32x4*)base,
+                           (f32x4*)(base + kScratchFloats), nvec);
         MI_CHECK(launch_status());
     }
     MI_CHECK(mi_layer_norm_bwd_dx_partial_dwdb(DX, DY, &dw, &db, X, W, Mean, Rstd, nullptr, GROUP_SIZE_M,
                                                TILE_N, stream));
-    return mi_layer_norm_bwd_dwdb(&dw, &db, FINAL_DW, FINAL_DB, TILE_M, TILE_N, stream);
+    MI_CHECK(dwdb_impl(&dw, &db, FINAL_DW, FINAL_DB, TILE_M, TILE_N, true, stream));
+    __atomic_store_n(&g_scratch_dirty[dev], false, __ATOMIC_RELEASE);
+    return MI_OK;
 }

@@ -155,7 +155,8 @@ int mi_layer_norm_bwd_dwdb(const mi_tile_array* DW, const mi_tile_array* DB,
  * allocate: code under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc.
  * Same result as zero-filling DW / DB (N, GROUP_SIZE_M), mi_layer_norm_bwd_dx_partial_dwdb and
  * mi_layer_norm_bwd_dwdb, with the partial slots held in a file-scope device array of the library
- * (4 MiB per GPU, kept until the process ends).  Limit: cld(N,4)*4 * GROUP_SIZE_M <= 524288 floats
+ * (4 MiB per GPU, kept until the process ends; the call's last kernel leaves it zeroed for the
+ * next call, so a call is two launches).  Limit: cld(N,4)*4 * GROUP_SIZE_M <= 524288 floats
  * (N = 8192 with 64 slots), MI_E_SCRATCH beyond.  Every call on a GPU uses that GPU's one array:
  * calls that overlap on one GPU (different streams or threads) race.  The array's device address
  * is looked up once per GPU, outside any stream capture: by the first eager call of this or of

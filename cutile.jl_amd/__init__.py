@@ -83,6 +83,7 @@ _SIGNATURES = {
     "mi_fused_moe_accumulate_kernel": ([_A] * 6 + [_i, _i, _i, _A, _vp], _i),
     "mi_silu_and_mul_kernel": ([_A, _A, _A, _i, _vp], _i),
     "mi_moe_sum_topk": ([_A, _A, _vp], _i),
+    "mi_quantize_e4m3fn": ([_A, _A, _A, _A, _vp], _i),
     "mi_tiled_broadcast": ([_A, ctypes.c_char_p, ctypes.POINTER(_A), _i, _vp, _i, _vp], _i),
     "mi_tiled_broadcast_eltype": ([ctypes.c_char_p, ctypes.POINTER(ctypes.c_int32), _i,
                                    ctypes.POINTER(ctypes.c_int32), _i, ctypes.POINTER(ctypes.c_int32)], _i),
@@ -390,6 +391,20 @@ def fused_moe_silu_kernel(A, B, C, topk_weights, sorted_token_ids, sorted_expert
 def silu_and_mul_kernel(A, B, C, TILE_N: int, stream=None):
     """examples/moe.jl:110-128"""
     _call("mi_silu_and_mul_kernel", _ref(A), _ref(B), _ref(C), TILE_N, _stream(stream))
+
+
+def quantize_e4m3fn(x, codes=None, scale=None, workspace=None, stream=None):
+    """Per-tensor E4M3FN codes of a 16-bit activation matrix (torch (columns, K)) and their scale (a 1-element fp32
+    device tensor): the fp8 operand of ``fused_moe_kernel`` with fp8 weights.  Returns (codes, scale)."""
+    import torch
+    if codes is None:
+        codes = torch.empty(x.shape, dtype=torch.float8_e4m3fn, device=x.device)
+    if scale is None:
+        scale = torch.empty(1, dtype=torch.float32, device=x.device)
+    if workspace is None:
+        workspace = torch.empty(1024, dtype=torch.float32, device=x.device)
+    _call("mi_quantize_e4m3fn", _ref(x), _ref(codes), _ref(scale), _ref(workspace), _stream(stream))
+    return codes, scale
 
 
 def moe_sum_topk(inp, out, stream=None):

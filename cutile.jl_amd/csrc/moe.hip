@@ -572,9 +572,13 @@ static int fused_moe_impl(const mi_tile_array* A, const mi_tile_array* B, const 
     MI_CHECK(check_array(topk_weights, topk_weights->ndim));
     MI_CHECK(check_array(sorted_token_ids, 1));
     MI_CHECK(check_array(sorted_expert_ids, 1));
-    if (!is16(A->dtype) || C->dtype != A->dtype || topk_weights->dtype != A->dtype) return MI_E_DTYPE;
+    // activations: 16-bit, or E4M3FN together with E4M3FN weights (fp8 x fp8 on the matrix cores, the operand pairing
+    // of ext/DLFP8TypesExt.jl:15-19); C and the routed weights are 16-bit either way
+    const bool a8 = A->dtype == MI_F8E4M3FN;
+    if (!is16(C->dtype) || topk_weights->dtype != C->dtype) return MI_E_DTYPE;
+    if (!a8 && A->dtype != C->dtype) return MI_E_DTYPE;
     const bool w8 = B->dtype == MI_F8E4M3FN;
-    if (!w8 && B->dtype != A->dtype) return MI_E_DTYPE;
+    if (!w8 && (a8 || B->dtype != A->dtype)) return MI_E_DTYPE;
     if (w8 != (b_scale != nullptr)) return MI_E_ARG;
     if (sorted_token_ids->dtype != MI_I32 || sorted_expert_ids->dtype != MI_I32) return MI_E_DTYPE;
     if (!is_pow2(TILE_M) || !is_pow2(TILE_N) || !is_pow2(TILE_K)) return MI_E_TILE;
@@ -616,7 +620,7 @@ static int fused_moe_impl(const mi_tile_array* A, const mi_tile_array* B, const 
     hipStream_t s = (hipStream_t)stream;
     {   // dense routing: the grouped GEMM on 128 x 128 tiles fed by a ring of LDS stages (moe_dense.hip), same bits
         mi::moe::DenseArgs d;
-        d.A = (const unsigned short*)A->ptr; d.lda = A->strides[1]; d.num_a_cols = (int)A->sizes[1];
+        d.A = A->ptr; d.lda = A->strides[1]; d.num_a_cols = (int)A->sizes[1];
         d.B = B->ptr; d.ldb = B->strides[1]; d.sbe = B->strides[2];
         d.C = (unsigned short*)C->ptr; d.ldc = C->strides[1]; d.total_tokens = (int)total;
         d.topk_weights = (const unsigned short*)topk_weights->ptr; d.w_topk = (int)w_topk;
@@ -626,11 +630,14 @@ static int fused_moe_impl(const mi_tile_array* A, const mi_tile_array* B, const 
         d.b_scale = w8 ? (const float*)b_scale->ptr : nullptr; d.ld_scale = w8 ? b_scale->strides[1] : 0;
         d.K = (int)K; d.N = (int)N; d.num_experts = (int)E; d.replicas = num_token_replicas;
         d.mul_routed_weight = mul_routed_weight != 0; d.TILE_M = TILE_M; d.acc_shift = acc_shift;
-        d.bf16 = A->dtype == MI_BF16; d.silu = silu; d.w8 = w8;
+        d.bf16 = C->dtype == MI_BF16; d.silu = silu; d.w8 = w8; d.a8 = a8;
         if (mi::moe::dense_applicable(d)) {
             mi::moe::dense_launch(d, s);
             return launch_status();
         }
+        // fp8 activations have no other kernel: blocks of 128 slots (or multiples), K a multiple of 16 from 512 up,
+        // rows on 16-byte boundaries
+        if (a8) return MI_E_UNSUPPORTED;
     }
     const int tile_slots = TILE_M < kTT ? TILE_M : kTT;
     const int64_t tiles = m_blocks * (TILE_M / tile_slots);

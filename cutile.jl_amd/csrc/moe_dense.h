@@ -9,7 +9,7 @@ namespace moe {
 
 // One launch of fused_moe_kernel (examples/moe.jl:45-105) as the entry points have validated it.
 struct DenseArgs {
-    const unsigned short* A;       // activations (K, columns), K contiguous
+    const void* A;                 // activations (K, columns), K contiguous: 16-bit, or E4M3FN bytes when a8
     int64_t lda;
     int num_a_cols;
     const void* B;                 // expert weights (K, N, E), K contiguous: 16-bit, or E4M3FN bytes when w8
@@ -30,7 +30,8 @@ struct DenseArgs {
     bool mul_routed_weight;
     int TILE_M;
     int acc_shift;                 // >= 0: accumulate into column (token - 1) >> acc_shift with packed atomic adds
-    bool bf16, silu, w8;
+    bool bf16, silu, w8;           // bf16: C (and the routed weights) are bfloat16, else float16
+    bool a8;                       // activations are E4M3FN as well: fp8 x fp8 MFMA, every channel times its b_scale entry
 };
 
 #ifdef __HIPCC__
@@ -59,8 +60,10 @@ __device__ __forceinline__ void atomic_add2(bool bf16, unsigned short* p, unsign
 }
 #endif
 
-// True if the launch can run on the 128-slot x 128-channel ring kernel (TILE_M a multiple of 128, 16-byte aligned
-// rows, K a multiple of 8 and at least 256) and routing is dense enough for it to pay.
+// True if the launch can run on the 128-slot ring kernel (TILE_M a multiple of 128, 16-byte aligned rows, K a multiple
+// of 8 and at least 256 -- of 16 and at least 512 for fp8 activations) and routing is dense enough for it to pay.
+// 16-bit activations with e4m3 weights are not its case (the streaming kernels widen those); fp8 activations run
+// nowhere else.
 bool dense_applicable(const DenseArgs& a);
 // Launches it and records the variant name.
 void dense_launch(const DenseArgs& a, hipStream_t s);

@@ -138,6 +138,79 @@ __device__ __forceinline__ void k_step(const unsigned short* TsX, unsigned short
     interleave<LIVE, J, DMA_W ? J : 0, !LAST>();
 }
 
+// ---- fp8 x fp8 (E4M3FN activations and weights) on v_mfma_f32_32x32x64_f8f6f4 ------------------------------------
+// A stage has the same bytes as for 16-bit operands (rows of 64 B, four swizzled 16-byte chunks) and therefore twice
+// the k: one stage is one K step of the instruction, whose operand is 32 bytes per lane -- chunks 2 * hb and 2 * hb + 1
+// of the lane's row, two 16-byte reads at the offsets the 16-bit kernel reads in its two sub-steps.  Tokens and weights
+// use the same byte <-> k map, which is all a dot product asks for.  The LDS bytes per MFMA cycle are those of the
+// 16-bit kernel (the instruction takes twice as long and multiplies four times as much), so this is the same loop at
+// twice the K per step.
+typedef int i32x8 __attribute__((ext_vector_type(8)));
+typedef int i32x4 __attribute__((ext_vector_type(4)));
+
+template <int J>
+struct DFrag8 {
+    i32x8 t[2], w[J];
+};
+
+template <int LIVE, int J>
+__device__ __forceinline__ void load_frags8(const unsigned short* Ts, const unsigned short* Ws, const DLane<J>& ln, DFrag8<J>& f) {
+    if (LIVE == 0) return;
+#pragma unroll
+    for (int j = 0; j < J; ++j) {
+        const i32x4 lo = *reinterpret_cast<const i32x4*>(Ws + ln.fW[0] + 32 * j * BK);
+        const i32x4 hi = *reinterpret_cast<const i32x4*>(Ws + ln.fW[1] + 32 * j * BK);
+        f.w[j] = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+    }
+#pragma unroll
+    for (int i = 0; i < LIVE; ++i) {
+        const i32x4 lo = *reinterpret_cast<const i32x4*>(Ts + ln.fT[0] + 32 * i * BK);
+        const i32x4 hi = *reinterpret_cast<const i32x4*>(Ts + ln.fT[1] + 32 * i * BK);
+        f.t[i] = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+    }
+}
+
+// the MFMAs of slot tile I of a step
+template <int LIVE, bool SLOT_LANE, int J, int I>
+__device__ __forceinline__ void mma8(const DFrag8<J>& f, f32x16 (&acc)[2][J]) {
+    if (I >= LIVE) return;
+#pragma unroll
+    for (int j = 0; j < J; ++j)
+        acc[I][j] = SLOT_LANE ? __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(f.w[j], f.t[I], acc[I][j], 0, 0, 0, 0, 0, 0)
+                              : __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(f.t[I], f.w[j], acc[I][j], 0, 0, 0, 0, 0, 0);
+}
+
+template <int LIVE, int J, int NRD, int NDMA>
+__device__ __forceinline__ void interleave8() {
+    if constexpr (LIVE == 2) {
+#pragma unroll
+        for (int i = 0; i < J; ++i) {
+            __builtin_amdgcn_sched_group_barrier(SG_MFMA, 1, 0);
+            if (NRD) __builtin_amdgcn_sched_group_barrier(SG_DSRD, NRD / J, 0);
+            if (NDMA) __builtin_amdgcn_sched_group_barrier(SG_VMEM, NDMA / J > 0 ? NDMA / J : 1, 0);
+        }
+    }
+    __builtin_amdgcn_sched_barrier(0);
+}
+
+// One K step of 64 on stage X, whose fragments are in `cur`; the next step's data is in stage Y.
+//   first half : MFMAs of slot tile 0 | token transfers of step s + 3 (into stage TsA)
+//   barrier
+//   second half: MFMAs of slot tile 1 | read the next stage's fragments into `nxt` | weight transfers of step s + 4 (into WsX)
+template <int LIVE, bool SLOT_LANE, int J, bool DMA_T, bool DMA_W, int VMCNT, bool LAST, bool TAIL>
+__device__ __forceinline__ void k_step8(unsigned short* WsX, const unsigned short* TsY, const unsigned short* WsY,
+                                        unsigned short* TsA, int64_t koffT, int64_t koffW, int wave, const DLane<J>& ln,
+                                        const DFrag8<J>& cur, DFrag8<J>& nxt, f32x16 (&acc)[2][J], int k_leftT, int k_leftW) {
+    if (DMA_T) issueN<TAIL, 2>(ln.gT, koffT, TsA, wave, ln.kC, k_leftT);
+    mma8<LIVE, SLOT_LANE, J, 0>(cur, acc);
+    interleave8<LIVE, J, 0, DMA_T ? 2 : 0>();
+    if (!LAST) stage_barrier<VMCNT>();
+    if (DMA_W) issueN<TAIL, J>(ln.gW, koffW, WsX, wave, ln.kC, k_leftW);
+    if (!LAST) load_frags8<LIVE, J>(TsY, WsY, ln, nxt);
+    mma8<LIVE, SLOT_LANE, J, 1>(cur, acc);
+    interleave8<LIVE, J, LAST ? 0 : 2 * (2 + J), DMA_W ? J : 0>();
+}
+
 struct Stages {
     unsigned short *T0, *T1, *T2, *T3, *W0, *W1, *W2, *W3;
 };
@@ -223,6 +296,38 @@ __device__ __forceinline__ void main_loop(const Stages& st, int K, int wave, con
     }
 }
 
+// The K walk with fp8 operands: the ring of four, a stage per K step of 64.
+template <int LIVE, bool SLOT_LANE, int J>
+__device__ __forceinline__ void main_loop8(const Stages& st, int K, int wave, const DLane<J>& ln, f32x16 (&acc)[2][J]) {
+    static_assert(J == 2, "fp8 operands take the ring of four stages");
+    constexpr int BK8 = 64, PER = 2 + J;
+    const int KT = 4 * ((K + 4 * BK8 - 1) / (4 * BK8));   // steps, in whole groups of four; >= 8 (K >= 512 is checked on the host)
+    DFrag8<J> f0, f1;
+    stage_barrier<2 * PER + J>();
+    load_frags8<LIVE, J>(st.T0, st.W0, ln, f0);
+#define KSTEP(X, Y, AA, CUR, NXT, DT, DW, VM, LAST, TAIL, s)                                                             \
+    k_step8<LIVE, SLOT_LANE, J, DT, DW, (VM) * PER, LAST, TAIL>(st.W##X, st.T##Y, st.W##Y, st.T##AA,                     \
+                                                                (int64_t)((s) + 3) * kStepBytes, (int64_t)((s) + 4) * kStepBytes, \
+                                                                wave, ln, CUR, NXT, acc, K - ((s) + 3) * BK8, K - ((s) + 4) * BK8)
+    int s = 0;
+    for (; s + 12 <= KT; s += 4) {
+        KSTEP(0, 1, 3, f0, f1, true, true, 2, false, false, s);
+        KSTEP(1, 2, 0, f1, f0, true, true, 2, false, false, s + 1);
+        KSTEP(2, 3, 1, f0, f1, true, true, 2, false, false, s + 2);
+        KSTEP(3, 0, 2, f1, f0, true, true, 2, false, false, s + 3);
+    }
+    KSTEP(0, 1, 3, f0, f1, true, true, 2, false, true, s);
+    KSTEP(1, 2, 0, f1, f0, true, true, 2, false, true, s + 1);
+    KSTEP(2, 3, 1, f0, f1, true, true, 2, false, true, s + 2);
+    KSTEP(3, 0, 2, f1, f0, true, true, 2, false, true, s + 3);
+    s += 4;
+    KSTEP(0, 1, 3, f0, f1, true, false, 2, false, true, s);
+    KSTEP(1, 2, 0, f1, f0, false, false, 1, false, false, s + 1);
+    KSTEP(2, 3, 1, f0, f1, false, false, 0, false, false, s + 2);
+    KSTEP(3, 0, 2, f1, f0, false, false, 0, true, false, s + 3);
+#undef KSTEP
+}
+
 // Barrier that waits for the wave's LDS accesses only (the transfers, loads and stores in flight stay in flight).
 __device__ __forceinline__ void lds_only_barrier() {
     asm volatile("" ::: "memory");
@@ -272,10 +377,29 @@ __device__ __forceinline__ void store_tile_slot_lane(const float (&o)[16], unsig
 }
 
 // Stores of one tile.
-template <typename E, int MODE, int J>
+// A8: the products are those of unscaled fp8 codes and every channel is multiplied by its fp32 scale first (scale_of:
+// b_scale entry of a weight row of the tile's expert, 1 for rows past N).
+template <typename E, int MODE, int J, bool A8>
 __device__ __forceinline__ void epilogue(const DenseArgs& a, const f32x16 (&acc)[2][J], int nlive, const int* s_tok,
-                                         const float* s_wt, int bid_n, int ws, int wn, int lane, bool vec_ok) {
+                                         const float* s_wt, int bid_n, int ws, int wn, int lane, bool vec_ok, int expert) {
     const int hb = lane >> 5;
+    auto scale_of = [&](int row) { return (A8 && row < a.N && expert >= 0 && expert < a.num_experts) ? a.b_scale[row + (int64_t)expert * a.ld_scale] : 1.f; };
+    // slot-in-lane layouts: register r of a column tile is weight row (tile's first row) + 8 * (r / 4) + 4 * hb + r % 4
+    float sc[A8 ? J : 1][A8 ? 16 : 1];
+    if constexpr (A8 && MODE != MODE_ACC) {
+#pragma unroll
+        for (int j = 0; j < J; ++j) {
+            int row0;
+            if (MODE == MODE_SILU) row0 = (j >= J / 2 ? a.N / 2 : 0) + bid_n * (32 * J) + 16 * J * wn + 32 * (j % (J / 2));
+            else row0 = bid_n * (64 * J) + 32 * J * wn + 32 * j;
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const int ch = 8 * (r >> 2) + 4 * hb + (r & 3);
+                // (a gate row past N / 2 belongs to no output channel: its scale is never used)
+                sc[j][r] = scale_of(row0 + ch);
+            }
+        }
+    }
 #pragma unroll
     for (int i = 0; i < 2; ++i) {
         if (i >= nlive) break;
@@ -291,6 +415,10 @@ __device__ __forceinline__ void epilogue(const DenseArgs& a, const f32x16 (&acc)
 #pragma unroll
                 for (int r = 0; r < 16; ++r) {
                     float g = acc[i][jj][r], u = acc[i][J / 2 + jj][r];
+                    if constexpr (A8) {
+                        g *= sc[jj][r];
+                        u *= sc[J / 2 + jj][r];
+                    }
                     if (a.mul_routed_weight) {
                         g *= wtv;
                         u *= wtv;
@@ -308,7 +436,11 @@ __device__ __forceinline__ void epilogue(const DenseArgs& a, const f32x16 (&acc)
                 const int ch0 = bid_n * (64 * J) + 32 * J * wn + 32 * j;
                 float o[16];
 #pragma unroll
-                for (int r = 0; r < 16; ++r) o[r] = a.mul_routed_weight ? acc[i][j][r] * wtv : acc[i][j][r];
+                for (int r = 0; r < 16; ++r) {
+                    float v = acc[i][j][r];
+                    if constexpr (A8) v *= sc[j][r];
+                    o[r] = a.mul_routed_weight ? v * wtv : v;
+                }
                 store_tile_slot_lane<E>(o, a.C + (int64_t)(tokv ? tokv - 1 : 0) * a.ldc + ch0, tokv != 0, a.N - ch0, vec_ok, hb);
             }
         } else {
@@ -321,11 +453,18 @@ __device__ __forceinline__ void epilogue(const DenseArgs& a, const f32x16 (&acc)
 #pragma unroll
             for (int jp = 0; jp < J; jp += 2) {
                 const int gn = bid_n * (64 * J) + 32 * J * wn + 32 * jp + lane;
+                // (before the swap a lane holds channel lane % 32 of both column tiles)
+                const int gn0 = bid_n * (64 * J) + 32 * J * wn + 32 * jp + (lane & 31);
+                const float s0 = scale_of(gn0), s1 = scale_of(gn0 + 32);
 #pragma unroll
                 for (int r = 0; r < 16; ++r) {
                     const int R = 8 * (r >> 2) + (r & 3);
                     const int tokA = __builtin_amdgcn_readlane(tokv, R), tokB = __builtin_amdgcn_readlane(tokv, R + 4);
                     float v0 = acc[i][jp][r], v1 = acc[i][jp + 1][r];
+                    if constexpr (A8) {
+                        v0 *= s0;
+                        v1 *= s1;
+                    }
                     if (a.mul_routed_weight) {
                         const float wA = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, wtv), R));
                         const float wB = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, wtv), R + 4));
@@ -350,8 +489,10 @@ __device__ __forceinline__ void epilogue(const DenseArgs& a, const f32x16 (&acc)
 // stride.  A tile's stores, and the next tile's ring fill right behind them, are in flight while nothing else of the
 // workgroup is: the next tile's K walk starts as soon as its first stage has landed, and what a tile needs to know
 // (expert, token ids) is requested one tile ahead.
-template <typename E, int MODE, int J>
+template <typename E, int MODE, int J, bool A8 = false>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) void moe_dense_kernel(const DenseArgs a, int n_blocks) {
+    constexpr int ES = A8 ? 1 : 2;          // bytes per operand element
+    constexpr int EPC = 16 / ES;            // elements per 16-byte chunk
     constexpr int kStageW = 64 * J * BK;   // elements of a weight stage: 64 * J rows of 32 k
     constexpr int kLast = J == 2 ? 1 : 0;  // the ring of three has no fourth stage
     __shared__ __attribute__((aligned(1024))) unsigned short Ts0[kStage], Ts1[kStage], Ts2[kStage], Ts3[kLast ? kStage : 8];
@@ -419,7 +560,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     DLane<J> ln;
     {
         const int chunk = (lane & 3) ^ ((lane >> 4) & 3);   // global chunk that belongs at this lane's LDS position
-        ln.kC = 8 * chunk;
+        ln.kC = EPC * chunk;
 #pragma unroll
         for (int ks = 0; ks < 2; ++ks) {
             const int sw = 8 * ((2 * ks + hb) ^ (((lane & 31) >> 2) & 3));
@@ -436,11 +577,11 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
         if (!ok) expert = 0;
         auto fix = [&](int raw, int r) { return (ok && slot0 + r < a.num_slots && raw >= 1 && raw <= a.total_tokens) ? raw : 0; };
         const int t0 = fix(m.t0, r0), t1 = fix(m.t1, r1);
-        const int chunk = L.kC >> 3;
+        const int chunk = L.kC / EPC;
         const int c0 = t0 ? (t0 - 1) / a.replicas : 0, c1 = t1 ? (t1 - 1) / a.replicas : 0;   // slots without a token read column 0
-        L.gT[0] = (const char*)(a.A + (int64_t)c0 * a.lda + 8 * chunk);
-        L.gT[1] = (const char*)(a.A + (int64_t)c1 * a.lda + 8 * chunk);
-        const unsigned short* Bx = (const unsigned short*)a.B + (int64_t)expert * a.sbe;
+        L.gT[0] = (const char*)a.A + ((int64_t)c0 * a.lda + EPC * chunk) * ES;
+        L.gT[1] = (const char*)a.A + ((int64_t)c1 * a.lda + EPC * chunk) * ES;
+        const char* Bx = (const char*)a.B + (int64_t)expert * a.sbe * ES;
         const int half_n = a.N / 2;
 #pragma unroll
         for (int j = 0; j < J; ++j) {
@@ -455,7 +596,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
                 row = m.bid_n * (64 * J) + R;
                 if (row > a.N - 1) row = a.N - 1;
             }
-            L.gW[j] = (const char*)(Bx + (int64_t)row * a.ldb + 8 * chunk);
+            L.gW[j] = Bx + ((int64_t)row * a.ldb + EPC * chunk) * ES;
         }
         return fix(m.tm, tid & 127);
     };
@@ -502,9 +643,15 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
 #pragma unroll
             for (int j = 0; j < J; ++j) acc[i][j] = f32x16{0};
         constexpr bool SL = MODE != MODE_ACC;
-        if (nlive == 2) main_loop<E, 2, SL, J>(st, a.K, wave, ln, acc);
-        else if (nlive == 1) main_loop<E, 1, SL, J>(st, a.K, wave, ln, acc);
-        else main_loop<E, 0, SL, J>(st, a.K, wave, ln, acc);
+        if constexpr (A8) {
+            if (nlive == 2) main_loop8<2, SL, J>(st, a.K, wave, ln, acc);
+            else if (nlive == 1) main_loop8<1, SL, J>(st, a.K, wave, ln, acc);
+            else main_loop8<0, SL, J>(st, a.K, wave, ln, acc);
+        } else {
+            if (nlive == 2) main_loop<E, 2, SL, J>(st, a.K, wave, ln, acc);
+            else if (nlive == 1) main_loop<E, 1, SL, J>(st, a.K, wave, ln, acc);
+            else main_loop<E, 0, SL, J>(st, a.K, wave, ln, acc);
+        }
         // the next tile's addresses and its routed weights (requested now, used after this tile's stores are out)
         int tmN = 0;
         float wN = 1.f;
@@ -512,7 +659,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
             tmN = setup(mn, ln);
             wN = routed_weight(tmN);
         }
-        epilogue<E, MODE, J>(a, acc, nlive, s_tok[p], s_wt[p], mc.bid_n, ws, wn, lane, vec_ok);
+        epilogue<E, MODE, J, A8>(a, acc, nlive, s_tok[p], s_wt[p], mc.bid_n, ws, wn, lane, vec_ok, mc.expert_raw - 1);
         if (!have_next) break;
         publish(p ^ 1, tmN, wN);
         lds_only_barrier();   // every wave is done with the ring's stages, and the next tile's slots are in place
@@ -536,6 +683,14 @@ bool dense_applicable(const DenseArgs& a) {
     // MI_MOE_DENSE: 0 = never, 1 = wherever it can run (read at every call, so that one process can compare the kernels)
     const char* env = getenv("MI_MOE_DENSE");
     const int force = env ? atoi(env) : -1;
+    if (a.a8) {   // fp8 x fp8: this kernel or none
+        if (!a.w8 || a.TILE_M % kRows || a.K % 16 || a.K < 512 || a.N < 1 || (a.silu && (a.N % 2))) return false;
+        if (!aligned(a.A, 16) || !aligned(a.B, 16) || a.lda % 16 || a.ldb % 16 || a.sbe % 16 || a.lda < 0 || a.ldb < 0) return false;
+        if (cld((int64_t)a.total_tokens, (int64_t)a.replicas) > a.num_a_cols) return false;
+        if (a.acc_shift >= 0 && (a.N % 2)) return false;
+        const int64_t nb8 = a.silu ? cld((int64_t)a.N / 2, (int64_t)64) : cld((int64_t)a.N, (int64_t)kRows);
+        return (cld((int64_t)a.num_blocks * (a.TILE_M / kRows) * nb8, (int64_t)8) + 1) * 8 <= MI_MAX_GRID_DIM;
+    }
     if (force == 0 || a.w8) return false;
     if (a.TILE_M % kRows || a.K % 8 || a.K < 256 || a.N < 1) return false;
     if (a.silu && (a.N % 2)) return false;
@@ -557,6 +712,7 @@ bool dense_applicable(const DenseArgs& a) {
 static int pick_j(const DenseArgs& a) {
     const char* env = getenv("MI_MOE_DENSE_J");
     const int force = env ? atoi(env) : 0;
+    if (a.a8) return 2;
     if (force == 2 || force == 4) return force;
     const int64_t strips4 = a.silu ? cld((int64_t)a.N / 2, (int64_t)128) : cld((int64_t)a.N, (int64_t)256);
     // blocks that hold tokens: at most one partly filled block per expert on top of the full ones
@@ -571,24 +727,25 @@ void dense_launch(const DenseArgs& a, hipStream_t s) {
     // persistent: two workgroups per CU at most (64 or 72 KB of LDS each), a multiple of 8 so that every XCD gets as many
     const int64_t per_xcd = cld(tiles, (int64_t)8) < 64 ? cld(tiles, (int64_t)8) : 64;
     const dim3 grid((unsigned)(per_xcd * 8));
-#define LAUNCH1(ET, MODE, JJ) hipLaunchKernelGGL((moe_dense_kernel<ET, MODE, JJ>), grid, dim3(256), 0, s, a, n_blocks)
-#define LAUNCH(ET, MODE)              \
-    do {                              \
-        if (J == 4) LAUNCH1(ET, MODE, 4); \
-        else LAUNCH1(ET, MODE, 2);    \
+#define LAUNCH1(ET, MODE, JJ, A8) hipLaunchKernelGGL((moe_dense_kernel<ET, MODE, JJ, A8>), grid, dim3(256), 0, s, a, n_blocks)
+#define LAUNCH(ET, MODE)                        \
+    do {                                        \
+        if (a.a8) LAUNCH1(ET, MODE, 2, true);   \
+        else if (J == 4) LAUNCH1(ET, MODE, 4, false); \
+        else LAUNCH1(ET, MODE, 2, false);       \
     } while (0)
     if (a.silu) {
         if (a.bf16) LAUNCH(BF16, MODE_SILU);
         else LAUNCH(F16, MODE_SILU);
-        set_variant(J == 4 ? "fused_moe_dense_silu_t128_n128x2_k32_ring3" : "fused_moe_dense_silu_t128_n64x2_k32_ring4");
+        set_variant(a.a8 ? "fused_moe_dense_silu_t128_n64x2_k64_ring4_w8a8" : J == 4 ? "fused_moe_dense_silu_t128_n128x2_k32_ring3" : "fused_moe_dense_silu_t128_n64x2_k32_ring4");
     } else if (a.acc_shift >= 0) {
         if (a.bf16) LAUNCH(BF16, MODE_ACC);
         else LAUNCH(F16, MODE_ACC);
-        set_variant(J == 4 ? "fused_moe_dense_acc_t128_n256_k32_ring3" : "fused_moe_dense_acc_t128_n128_k32_ring4");
+        set_variant(a.a8 ? "fused_moe_dense_acc_t128_n128_k64_ring4_w8a8" : J == 4 ? "fused_moe_dense_acc_t128_n256_k32_ring3" : "fused_moe_dense_acc_t128_n128_k32_ring4");
     } else {
         if (a.bf16) LAUNCH(BF16, MODE_PLAIN);
         else LAUNCH(F16, MODE_PLAIN);
-        set_variant(J == 4 ? "fused_moe_dense_t128_n256_k32_ring3" : "fused_moe_dense_t128_n128_k32_ring4");
+        set_variant(a.a8 ? "fused_moe_dense_t128_n128_k64_ring4_w8a8" : J == 4 ? "fused_moe_dense_t128_n256_k32_ring3" : "fused_moe_dense_t128_n128_k32_ring4");
     }
 #undef LAUNCH
 #undef LAUNCH1

@@ -30,8 +30,15 @@ def invoke_silu_and_mul_kernel(AB, C):
     ct.silu_and_mul_kernel(A_half, B_half, C, tile_n)
 
 
+def quantize_activations(x):
+    """Per-tensor E4M3FN form of an activation matrix, entirely on the device: codes = round-to-nearest-even of
+    x / scale with scale = max |x| / 448 (1 for an all-zero tensor); returns (codes, scale as a 1-element fp32
+    tensor).  Two launches of the library (``mi_quantize_e4m3fn``)."""
+    return ct.quantize_e4m3fn(x)
+
+
 def cutile_moe(hidden_states, w1, w2, topk_weights, topk_ids, tile_m, tile_n, tile_k, *, w1_scale=None,
-               w2_scale=None, aligned=None, device_align=True, fuse_silu=True, fuse_sum=None):
+               w2_scale=None, aligned=None, device_align=True, fuse_silu=True, fuse_sum=None, fp8_activations=False):
     """moe.jl:218-257.  Torch shapes (reversed Julia): hidden_states (tokens, hidden); w1
     (E, 2*inter, hidden); w2 (E, hidden, inter); topk_weights / topk_ids (topk, tokens), ids
     1-based int64.  ``aligned`` may carry a precomputed (sorted_token_ids, sorted_expert_ids)
@@ -42,12 +49,23 @@ def cutile_moe(hidden_states, w1, w2, topk_weights, topk_ids, tile_m, tile_n, ti
     ``fuse_silu=False`` launches the kernels one by one as moe.jl:234-251 does.  ``fuse_sum`` (default: whenever
     it applies -- one or two slots per token, device-side sort, an even hidden size of whole 16-byte rows) lets the
     down projection add every replica's row into the output itself, which the sort launch has zeroed: cache3 and
-    the top-k sum launch disappear.  All combinations give bit-identical results."""
+    the top-k sum launch disappear.  All combinations give bit-identical results.
+
+    ``fp8_activations`` (with E4M3FN weights and their scales; an extension like the fp8 weights themselves): both
+    grouped GEMMs multiply fp8 by fp8 on the matrix cores, the operand pairing that ext/DLFP8TypesExt.jl:15-19 gives
+    ``mma``.  The activations of either GEMM are quantised per tensor on the device (``quantize_activations``) and
+    their scale is folded into the weights' per-channel scales; needs blocks of 128 slots, the fused SiLU epilogue and
+    hidden / intermediate sizes that are multiples of 16 from 512 up."""
     num_tokens, hidden_size = hidden_states.shape
     num_experts, _, intermediate_size = w2.shape
     topk = topk_ids.shape[0]
     total_tokens = num_tokens * topk
     T, dev = hidden_states.dtype, hidden_states.device
+    if fp8_activations:
+        if w1_scale is None or w2_scale is None or not fuse_silu:
+            raise ValueError("fp8 activations need e4m3 weights with their scales and the fused SiLU epilogue")
+        hidden_states, a_scale = quantize_activations(hidden_states)
+        w1_scale = w1_scale * a_scale
     can_fuse_sum = (topk <= 2 and aligned is None and device_align and hidden_size % 8 == 0 and topk_weights.dtype == T)
     if fuse_sum is None:
         fuse_sum = can_fuse_sum
@@ -91,6 +109,9 @@ def cutile_moe(hidden_states, w1, w2, topk_weights, topk_ids, tile_m, tile_n, ti
                                 tile_k=tile_k, b_scale=w1_scale)
         cache1_flat = cache1.reshape(total_tokens, intermediate_size * 2)
         invoke_silu_and_mul_kernel(cache1_flat, cache2)
+    if fp8_activations:
+        cache2, c_scale = quantize_activations(cache2)
+        w2_scale = w2_scale * c_scale
     if fuse_sum:
         ct.fused_moe_accumulate_kernel(cache2, w2, out, topk_weights, sorted_token_ids, sorted_expert_ids, tile_m, tile_n,
                                        tile_k, b_scale=w2_scale)

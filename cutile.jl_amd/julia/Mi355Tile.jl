@@ -341,6 +341,14 @@ function moe_sum_topk(in, out; stream::Ptr{Cvoid}=C_NULL)
         (Ref{MiTileArray}, Ref{MiTileArray}, Ptr{Cvoid}), d[1], d[2], stream))
 end
 
+"codes (K, columns) E4M3FN and scale[1] = max |x| / 448 of a Float16 / BFloat16 activation matrix x (K, columns):
+the fp8 operand `A` of `fused_moe_kernel` when the expert weights are fp8 as well.  `workspace`: 1024 Float32."
+function quantize_e4m3fn(x, codes, scale, workspace; stream::Ptr{Cvoid}=C_NULL)
+    d = map(a -> ref(descriptor(a)), (x, codes, scale, workspace))
+    GC.@preserve x codes scale workspace check(ccall((:mi_quantize_e4m3fn, libmi355tile), Cint,
+        (Ref{MiTileArray}, Ref{MiTileArray}, Ref{MiTileArray}, Ref{MiTileArray}, Ptr{Cvoid}), d[1], d[2], d[3], d[4], stream))
+end
+
 # ---- examples/fft.jl ----------------------------------------------------------------------
 
 function fft_kernel(x_packed_in, y_packed_out, W0, W1, W2, T0, T1, N::Integer, F0::Integer, F1::Integer,

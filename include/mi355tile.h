@@ -238,7 +238,12 @@ int mi_moe_route_topk(const mi_tile_array* logits, const mi_tile_array* topk_wei
  * and the caller saves the permuting copy), sorted_token_ids (M_padded,) i32 1-based with sentinel
  * total_tokens+1, sorted_expert_ids (blocks,) i32 1-based.  A, C, topk_weights f16/bf16.
  * B is f16/bf16, or MI_F8E4M3FN with `b_scale` (N,E) f32 per-output-channel scales
- * (fp8 weights are an extension of this build; b_scale must be NULL otherwise). */
+ * (fp8 weights are an extension of this build; b_scale must be NULL otherwise).
+ * With fp8 weights A may be MI_F8E4M3FN as well (C and topk_weights stay 16-bit): the products are then formed
+ * by the fp8 matrix instruction, fp8 x fp8 with fp32 accumulation -- the operand pairing ext/DLFP8TypesExt.jl:15-19
+ * gives `mma` -- and every output channel is multiplied by its b_scale entry (fold an activation scale into it).
+ * This form runs on the 128-slot grouped GEMM only: TILE_M a multiple of 128, K a multiple of 16 and at least 512,
+ * rows of A and B on 16-byte boundaries; MI_E_UNSUPPORTED otherwise.  The same holds for the two variants below. */
 int mi_fused_moe_kernel(const mi_tile_array* A, const mi_tile_array* B, const mi_tile_array* C,
                         const mi_tile_array* topk_weights, const mi_tile_array* sorted_token_ids,
                         const mi_tile_array* sorted_expert_ids, int num_token_replicas,
@@ -277,6 +282,14 @@ int mi_silu_and_mul_kernel(const mi_tile_array* A, const mi_tile_array* B,
  * hands to CUDA.jl: out (H, tokens) = sum over dim 2 of in (H, topk, tokens), fp32
  * accumulation in slot order. */
 int mi_moe_sum_topk(const mi_tile_array* in, const mi_tile_array* out, void* stream);
+/* Producer of fp8 activations for the grouped GEMMs above (A of type MI_F8E4M3FN together with fp8 weights: fp8 x fp8
+ * on the matrix cores, the operand pairing of ext/DLFP8TypesExt.jl:15-19; the reference leaves making fp8 operands to
+ * its caller, so this has no counterpart there).  x (K, columns) f16/bf16 -> codes (K, columns) E4M3FN with one scale
+ * for the whole array: scale[0] = max |x| / 448 (1 if x is all zero), codes = round-to-nearest-even of x / scale.
+ * `workspace`: at least 1024 floats of the caller's (partial maxima; nothing to clear).  K a multiple of 8, columns on
+ * 16-byte (x) and 8-byte (codes) boundaries.  Two launches. */
+int mi_quantize_e4m3fn(const mi_tile_array* x, const mi_tile_array* codes, const mi_tile_array* scale,
+                       const mi_tile_array* workspace, void* stream);
 
 /* ---- FFT: examples/fft.jl ------------------------------------------------------------- */
 /* fft_kernel (fft.jl:22-126): batched complex FFT of N = F0*F1*F2 points as three stages of small

@@ -271,9 +271,12 @@ def silu_and_mul(a: np.ndarray, b: np.ndarray, dtype=np.float64) -> np.ndarray:
     return a / (1.0 + np.exp(-a)) * b
 
 
-def ref_moe(hidden_states, w1, w2, topk_weights, topk_ids, dtype=np.float32):
+def ref_moe(hidden_states, w1, w2, topk_weights, topk_ids, dtype=np.float32, mid=None):
     """examples/moe.jl:264-304.  hidden_states (hidden, tokens); w1 (hidden, 2*inter, E);
-    w2 (inter, hidden, E); topk_weights, topk_ids (tokens, topk), ids 1-based."""
+    w2 (inter, hidden, E); topk_weights, topk_ids (tokens, topk), ids 1-based.
+    ``mid``: what a build that quantises the activations between the two projections does to
+    SiLU(gate) * up (a function of the (inter, tokens-of-one-expert) matrix; the reference has
+    no such step and passes None)."""
     hs = hidden_states.astype(dtype); w1 = w1.astype(dtype); w2 = w2.astype(dtype)
     tw = topk_weights.astype(dtype)
     hidden, num_tokens = hs.shape
@@ -289,6 +292,8 @@ def ref_moe(hidden_states, w1, w2, topk_weights, topk_ids, dtype=np.float32):
         gate_out = w1e[:, :inter].T @ tokens
         up_out = w1e[:, inter:].T @ tokens
         silu_out = gate_out / (1.0 + np.exp(-gate_out)) * up_out
+        if mid is not None:
+            silu_out = mid(silu_out).astype(dtype)
         expert_out = w2[:, :, eid - 1].T @ silu_out
         for i, (t, s) in enumerate(zip(tok_idx, slot_idx)):
             result[:, t] += expert_out[:, i] * tw[t, s]

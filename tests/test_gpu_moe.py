@@ -578,3 +578,71 @@ def test_dense_ring_kernel_other_block_sizes_sorts_and_output_layouts(ct, orc):
     with _dense_knob("1"):
         moe.cutile_moe(d.hidden_states, d.w1, d.w2, d.topk_weights, d.topk_ids, 64, 128, 64, fuse_sum=False)
         assert "dense" not in ct.last_variant()
+
+
+@pytest.mark.parametrize("shape,T", [
+    (dict(num_tokens=1024, hidden_size=1024, num_experts=32, intermediate_size=2048, topk=2, router="top2_logits"), torch.float16),
+    (dict(benchmark=True, topk=8), torch.float16),
+    (dict(num_tokens=300, hidden_size=528, num_experts=3, intermediate_size=560, topk=2), torch.bfloat16),   # K = 528, 560: zero-padded last steps
+    (dict(num_tokens=500, hidden_size=512, num_experts=5, intermediate_size=544, topk=1), torch.float16),
+])
+def test_fp8_activations_times_fp8_weights_on_the_matrix_cores(ct, orc, shape, T):
+    """E4M3FN activations x E4M3FN weights (the operand pairing of ext/DLFP8TypesExt.jl:15-19) in both grouped GEMMs of
+    the MoE, fp32 accumulation, per-channel weight scales and per-tensor activation scales.  Oracle (the last row of the
+    fp8 parity plan): ``ref_moe`` in float64 over the dequantised weights and the dequantised activations, with the
+    intermediate rounded to the storage type and quantised exactly as the product does it between the projections
+    (its own codec, pinned by the reference's vectors and by torch's fp8 dtype).  Only the accumulation order differs."""
+    d = moe.prepare(T=T, **shape)
+    q = moe.quantize_weights(d)
+    J = orc.to_julia
+    outs = []
+    for kw in (dict(), dict(fuse_sum=False)):
+        outs.append(moe.cutile_moe(d.hidden_states, q.w1, q.w2, d.topk_weights, d.topk_ids, 128, 128, 64, w1_scale=q.w1_scale,
+                                   w2_scale=q.w2_scale, fp8_activations=True, **kw))
+        assert not torch.isnan(outs[-1].float()).any()
+    assert "w8a8" in ct.last_variant() or ct.last_variant().startswith("moe_sum_topk")
+    if d.topk <= 2:
+        assert torch.equal(outs[0], outs[1])   # the accumulating down projection against cache3 + sum
+    # the oracle's view of the same computation
+    h8, a_scale = moe.quantize_activations(d.hidden_states)
+    hs = orc.e4m3fn_decode(J(h8.view(torch.uint8))) * float(a_scale)
+    # the library's quantiser against the oracle's codec: scale = max |x| / 448 and the quotient x / scale in fp32
+    # (IEEE division), codes = round-to-nearest-even of that quotient.  (With bf16 data many quotients sit exactly on a
+    # rounding boundary, so the quotient has to be formed in the same precision to compare codes one for one.)
+    x32 = J(d.hidden_states).astype(np.float32)
+    assert float(a_scale) == float(np.float32(np.abs(x32).max()) / np.float32(448.0))
+    want = orc.e4m3fn_encode((x32 / np.float32(float(a_scale))).astype(np.float64))
+    assert np.array_equal(want, J(h8.view(torch.uint8)))
+    w1d = orc.e4m3fn_decode(J(q.w1.view(torch.uint8))) * J(q.w1_scale)[None]
+    w2d = orc.e4m3fn_decode(J(q.w2.view(torch.uint8))) * J(q.w2_scale)[None]
+    # the product's cache2: the first projection alone, then its quantisation
+    tok, exp = ct.moe_align_tile_size_device(d.topk_ids, 128, d.num_experts)
+    c2 = torch.empty(d.num_tokens * d.topk, d.intermediate_size, dtype=T, device="cuda")
+    moe.invoke_fused_moe_kernel(h8, q.w1, c2, d.topk_weights, tok, exp, mul_routed_weight=False, num_token_replicas=d.topk,
+                                tile_m=128, tile_n=128, tile_k=64, b_scale=q.w1_scale * a_scale, fuse_silu=True)
+    assert ct.last_variant() == "fused_moe_dense_silu_t128_n64x2_k64_ring4_w8a8"
+    _, c_scale = moe.quantize_activations(c2)
+    c_scale = float(c_scale)
+
+    def mid(x):   # rounded to the storage type, then to e4m3 at the product's per-tensor scale
+        x = orc.bf16_round(x.astype(np.float32)).astype(np.float64) if T == torch.bfloat16 else x.astype(np.float16).astype(np.float64)
+        return orc.e4m3fn_decode(orc.e4m3fn_encode(x / c_scale)) * c_scale
+
+    ref = orc.ref_moe(hs, w1d, w2d, J(d.topk_weights), J(d.topk_ids), dtype=np.float64, mid=mid)
+    check(J(outs[1]), ref, 5e-2 if T == torch.bfloat16 else 2e-2)
+
+
+def test_fp8_activations_are_refused_where_no_kernel_takes_them(ct):
+    d = moe.prepare(num_tokens=64, hidden_size=512, num_experts=4, intermediate_size=512, topk=2)
+    q = moe.quantize_weights(d)
+    h8, _ = moe.quantize_activations(d.hidden_states)
+    tok, exp = ct.moe_align_tile_size_device(d.topk_ids, 64, d.num_experts)
+    c = torch.empty(d.num_tokens * 2, 2 * d.intermediate_size, dtype=torch.float16, device="cuda")
+    with pytest.raises(ct.MiError) as e:    # blocks of 64 slots: only the 128-slot ring kernel multiplies fp8 by fp8
+        moe.invoke_fused_moe_kernel(h8, q.w1, c, d.topk_weights, tok, exp, mul_routed_weight=False, num_token_replicas=2,
+                                    tile_m=64, tile_n=128, tile_k=64, b_scale=q.w1_scale)
+    assert e.value.code == ct.MI_E_UNSUPPORTED
+    with pytest.raises(ct.MiError) as e:    # fp8 activations against 16-bit weights
+        moe.invoke_fused_moe_kernel(h8, d.w1, c, d.topk_weights, tok, exp, mul_routed_weight=False, num_token_replicas=2,
+                                    tile_m=128, tile_n=128, tile_k=64)
+    assert e.value.code == ct.MI_E_DTYPE

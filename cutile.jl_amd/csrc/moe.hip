@@ -16,6 +16,7 @@
 // f16 on their way into LDS (every e4m3 value is exact in f16) and scaled in the epilogue.
 #include "common.h"
 #include "moe_dense.h"
+#include "shared_scratch.h"
 #include <math.h>
 #include <type_traits>
 
@@ -731,120 +732,256 @@ extern "C" int mi_fused_moe_accumulate_kernel(const mi_tile_array* A, const mi_t
 }
 
 // ---- on-device moe_align_tile_size ------------------------------------------------------------
-// One workgroup of sixteen waves.  Counting sort by expert of the replica ids (slot-fastest
-// flattening of topk_ids, examples/moe.jl:148-150): LDS histogram, scan over the experts,
-// then placement in super-blocks of 1024 consecutive replicas (one per lane).  A replica's slot is
-//     cursor[e] + (replicas of e in earlier waves of the super-block) + (those in earlier lanes),
-// the last term from ballots alone (one per bit of the expert id), so ids of one expert ascend exactly as the stable sortperm
-// of moe.jl:150 orders them.  The outputs have fixed capacity: unused slots hold the sentinel
-// total+1, unused blocks expert 0, which the GEMM kernel skips.
+// Counting sort by expert of the replica ids (slot-fastest flattening of topk_ids, examples/moe.jl:148-150), stable:
+// the ids of one expert ascend exactly as the sortperm of moe.jl:150 orders them.
+//
+// A workgroup of sixteen waves sorts a contiguous segment of the replicas, every wave a contiguous part of it:
+//   pass 1: the wave counts its replicas per expert (LDS atomics on its own row of a table);
+//   scan:   thread e turns expert e's sixteen counts into the first slot of every wave's share of the expert;
+//   pass 2: the wave walks its part again, 64 replicas at a time: a replica's slot is the wave's cursor for its expert
+//           plus the number of earlier lanes with the same expert (ballots alone, one per bit of the expert id), and
+//           the first lane of every expert advances the cursor.
+// The passes have no workgroup barrier inside (a wave touches only its own row of the table).
+//
+// One workgroup is one compute unit, and the sort is bound by that unit's instruction issue (10 us at 8192
+// replicas, 40 us at 32768).  Larger batches therefore take two launches of up to 64 workgroups: the first counts
+// every workgroup's segment per expert, and the workgroup that arrives last (a ticket, no waiting) scans the counts
+// into the first slot of every (workgroup, expert) pair, labels the blocks and fills the sentinels' share; the
+// second launch is the one-workgroup kernel per segment with those first slots in place of its own scan.
+// The counts travel through a static array of the library (a captured stream is not given it and sorts with one
+// workgroup).  The outputs have fixed capacity: unused slots hold the sentinel total+1, unused blocks expert 0,
+// which the GEMM kernel skips.
 constexpr int kAlignMaxExperts = 1024;
 constexpr int kAlignThreads = 1024, kAlignWaves = kAlignThreads / 64;
-constexpr int kAlignBatch = 8;   // super-blocks whose ids a thread requests together: one memory round trip per batch
-__global__ __launch_bounds__(kAlignThreads) void moe_align_kernel(const long long* __restrict__ topk_ids, int64_t ld_slot,
-                                                        int num_tokens, int topk, int tile_m, int num_experts,
-                                                        int* __restrict__ sorted_token_ids, int cap_slots,
-                                                        int* __restrict__ sorted_expert_ids, int cap_blocks,
-                                                        u32x4* __restrict__ clear, int64_t clear_n16) {
-    __shared__ int cursor[kAlignMaxExperts];      // histogram, then next free slot of every expert
-    __shared__ unsigned short tbl[kAlignWaves][kAlignMaxExperts];   // replicas per (wave, expert) of the current super-block (<= 64)
+constexpr int kAlignBatch = 8;            // chunks of 64 replicas whose ids a lane requests together: one memory round trip per batch
+constexpr int kAlignMaxWgs = 64;
+constexpr int kAlignPairs = 16384;        // (workgroup, expert) pairs of the two-launch sort
+constexpr int kAlignOneWgReplicas = 8192; // up to here one launch of one workgroup is as fast (10 us either way at 8192)
+// counts [kAlignPairs] | first slot inside the expert [kAlignPairs] | first slot of the expert [kAlignMaxExperts] | ticket
+constexpr int kAlignScratchInts = 2 * kAlignPairs + kAlignMaxExperts + 64;
+static __device__ __align__(256) int moe_align_scratch[kAlignScratchInts];
+static SharedScratch g_align_scratch[16];
+
+struct AlignArgs {
+    const long long* topk_ids;
+    int64_t ld_slot;
+    int num_tokens, topk;
+    float inv_topk;
+    int tile_m, num_experts;
+    int* sorted_token_ids;
+    int cap_slots;
+    int* sorted_expert_ids;
+    int cap_blocks;
+    u32x4* clear;
+    int64_t clear_n16;
+    int sort_wgs;        // workgroups that sort; the ones behind them zero `clear`
+    int wg_chunks;       // chunks of 64 replicas in a workgroup's segment: a multiple of kAlignWaves
+};
+
+// Expert (0-based) of replica r, -1 for a replica at or past `limit` or an id outside 1..num_experts (such a replica takes
+// no slot).  r < 2^22: the float quotient is off by one at most.
+__device__ __forceinline__ int align_expert_of(const AlignArgs& a, int r, int limit) {
+    if (r >= limit) return -1;
+    int tok = (int)((float)r * a.inv_topk), slot = r - tok * a.topk;
+    if (slot < 0) { --tok; slot += a.topk; }
+    if (slot >= a.topk) { ++tok; slot -= a.topk; }
+    const long long v = a.topk_ids[tok + (int64_t)slot * a.ld_slot];
+    return (v >= 1 && v <= a.num_experts) ? (int)v - 1 : -1;
+}
+
+// Exclusive scan over the experts of their block counts (thread e holds expert e's): shuffles inside a wave, the waves'
+// totals through LDS.  Every thread of the workgroup calls it.
+__device__ __forceinline__ int align_scan_blocks(int nb, int* wave_total) {
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    int incl = nb;
+#pragma unroll
+    for (int off = 1; off < 64; off <<= 1) {
+        const int up = __shfl_up(incl, off, 64);
+        if (lane >= off) incl += up;
+    }
+    if (lane == 63) wave_total[wave] = incl;
+    __syncthreads();
+    int first = incl - nb;
+#pragma unroll
+    for (int w = 0; w < kAlignWaves; ++w) first += w < wave ? wave_total[w] : 0;
+    return first;
+}
+
+__device__ __forceinline__ void align_clear(const AlignArgs& a) {
+    const int64_t wgs = gridDim.x - a.sort_wgs;
+    for (int64_t i = (int64_t)(blockIdx.x - a.sort_wgs) * kAlignThreads + threadIdx.x; i < a.clear_n16; i += wgs * kAlignThreads)
+        a.clear[i] = u32x4{0, 0, 0, 0};
+}
+
+// MULTI: the second launch of the two-launch sort (`start`, `rel`: what the first launch left in the static array).
+template <bool MULTI>
+__global__ __launch_bounds__(kAlignThreads) void moe_align_kernel(const AlignArgs a, const int* __restrict__ start,
+                                                                  const int* __restrict__ rel) {
+    __shared__ int tbl[kAlignWaves][kAlignMaxExperts];   // per (wave, expert): count, then next free slot
     __shared__ int s_blocks, wave_total[kAlignWaves];
-    // Workgroups past the first only zero their share of the array the caller wants cleared on the way (e.g. the
-    // output that the accumulating down projection adds into); the first one sorts.
-    if (blockIdx.x > 0) {
-        for (int64_t i = (int64_t)(blockIdx.x - 1) * kAlignThreads + threadIdx.x; i < clear_n16; i += (int64_t)(gridDim.x - 1) * kAlignThreads)
-            clear[i] = u32x4{0, 0, 0, 0};
+    // Workgroups past the sorting ones only zero their share of the array the caller wants cleared on the way (e.g.
+    // the output that the accumulating down projection adds into).
+    if ((int)blockIdx.x >= a.sort_wgs) {
+        align_clear(a);
         return;
     }
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, total = num_tokens * topk;
-    // A thread requests the ids of kAlignBatch super-blocks at a time, all loads before the first use: a batch costs one
-    // memory round trip instead of one per super-block.  The first batch (8192 replicas) stays in registers between the
-    // counting pass and the placing pass and is requested before the tables are cleared.
-    auto expert_of = [&](int r) {
-        if (r >= total) return -1;
-        const long long v = topk_ids[(r / topk) + (int64_t)(r % topk) * ld_slot];
-        return (v >= 1 && v <= num_experts) ? (int)v - 1 : -1;
-    };
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, total = a.num_tokens * a.topk;
+    const int cpw = a.wg_chunks / kAlignWaves;
+    const int seg0 = ((int)blockIdx.x * a.wg_chunks + wave * cpw) * 64, seg1 = seg0 + cpw * 64 < total ? seg0 + cpw * 64 : total;
+    // The ids of the wave's first kAlignBatch chunks stay in registers between the passes (a workgroup's segment of up
+    // to 8192 replicas is read once), and are requested before the table is cleared.
     int ecache[kAlignBatch];
 #pragma unroll
-    for (int i = 0; i < kAlignBatch; ++i) ecache[i] = expert_of(tid + kAlignThreads * i);
-    for (int e = tid; e < num_experts; e += kAlignThreads) {
-        cursor[e] = 0;
+    for (int i = 0; i < kAlignBatch; ++i) ecache[i] = align_expert_of(a, seg0 + 64 * i + lane, seg1);
+    for (int e = tid; e < a.num_experts; e += kAlignThreads) {
 #pragma unroll
         for (int w = 0; w < kAlignWaves; ++w) tbl[w][e] = 0;
     }
-    for (int i = tid; i < cap_slots; i += kAlignThreads) sorted_token_ids[i] = total + 1;
+    if (!MULTI)
+        for (int i = tid; i < a.cap_slots; i += kAlignThreads) a.sorted_token_ids[i] = total + 1;
     __syncthreads();
+    // ---- pass 1
 #pragma unroll
     for (int i = 0; i < kAlignBatch; ++i)
-        if (ecache[i] >= 0) atomicAdd(&cursor[ecache[i]], 1);
-    for (int r0 = kAlignThreads * kAlignBatch; r0 < total; r0 += kAlignThreads * kAlignBatch) {
+        if (ecache[i] >= 0) atomicAdd(&tbl[wave][ecache[i]], 1);
+    for (int r0 = seg0 + 64 * kAlignBatch; r0 < seg1; r0 += 64 * kAlignBatch) {
         int eb[kAlignBatch];
 #pragma unroll
-        for (int i = 0; i < kAlignBatch; ++i) eb[i] = expert_of(r0 + tid + kAlignThreads * i);
+        for (int i = 0; i < kAlignBatch; ++i) eb[i] = align_expert_of(a, r0 + 64 * i + lane, seg1);
 #pragma unroll
         for (int i = 0; i < kAlignBatch; ++i)
-            if (eb[i] >= 0) atomicAdd(&cursor[eb[i]], 1);
+            if (eb[i] >= 0) atomicAdd(&tbl[wave][eb[i]], 1);
     }
     __syncthreads();
-    {   // exclusive scan of the experts' block counts (thread e owns expert e): shuffles inside a
-        // wave, the waves' totals through LDS; then every expert labels its own blocks
-        const int nb = tid < num_experts ? (cursor[tid] + tile_m - 1) / tile_m : 0;
-        int incl = nb;
+    // ---- the first slot of every wave's share of every expert (thread e owns expert e)
+    if (MULTI) {
+        if (tid < a.num_experts) {
+            int slot = start[tid] + rel[(int)blockIdx.x * a.num_experts + tid];
 #pragma unroll
-        for (int off = 1; off < 64; off <<= 1) {
-            const int up = __shfl_up(incl, off, 64);
-            if (lane >= off) incl += up;
+            for (int w = 0; w < kAlignWaves; ++w) {
+                const int c = tbl[w][tid];
+                tbl[w][tid] = slot;
+                slot += c;
+            }
         }
-        if (lane == 63) wave_total[wave] = incl;
-        __syncthreads();
-        int first = incl - nb;
+    } else {
+        int cnt = 0;
+        if (tid < a.num_experts) {
 #pragma unroll
-        for (int w = 0; w < kAlignWaves; ++w) first += w < wave ? wave_total[w] : 0;
-        if (tid < num_experts) {
-            cursor[tid] = first * tile_m;  // first slot of the expert
-            for (int b = first; b < first + nb && b < cap_blocks; ++b) sorted_expert_ids[b] = tid + 1;
+            for (int w = 0; w < kAlignWaves; ++w) cnt += tbl[w][tid];
         }
-        if (tid == kAlignThreads - 1) s_blocks = first + nb < cap_blocks ? first + nb : cap_blocks;
+        const int nb = (cnt + a.tile_m - 1) / a.tile_m;
+        const int first = align_scan_blocks(nb, wave_total);
+        if (tid < a.num_experts) {
+            int slot = first * a.tile_m;
+#pragma unroll
+            for (int w = 0; w < kAlignWaves; ++w) {
+                const int c = tbl[w][tid];
+                tbl[w][tid] = slot;
+                slot += c;
+            }
+            for (int b = first; b < first + nb && b < a.cap_blocks; ++b) a.sorted_expert_ids[b] = tid + 1;
+        }
+        if (tid == kAlignThreads - 1) s_blocks = first + nb < a.cap_blocks ? first + nb : a.cap_blocks;
     }
     __syncthreads();
-    for (int b = s_blocks + tid; b < cap_blocks; b += kAlignThreads) sorted_expert_ids[b] = 0;
+    if (!MULTI)
+        for (int b = s_blocks + tid; b < a.cap_blocks; b += kAlignThreads) a.sorted_expert_ids[b] = 0;
 
+    // ---- pass 2
     const unsigned long long lt = lane ? (~0ull >> (64 - lane)) : 0ull;
-    const int id_bits = 32 - __builtin_clz((unsigned)(num_experts > 1 ? num_experts - 1 : 1));
-    for (int b0 = 0; b0 < total; b0 += kAlignThreads * kAlignBatch) {
+    const int id_bits = 32 - __builtin_clz((unsigned)(a.num_experts > 1 ? a.num_experts - 1 : 1));
+    volatile int* cur = tbl[wave];   // (this wave's row only; its LDS accesses execute in order)
+    for (int b0 = seg0; b0 < seg1; b0 += 64 * kAlignBatch) {
         int eb[kAlignBatch];
 #pragma unroll
-        for (int i = 0; i < kAlignBatch; ++i) eb[i] = b0 == 0 ? ecache[i] : expert_of(b0 + tid + kAlignThreads * i);
+        for (int i = 0; i < kAlignBatch; ++i) eb[i] = b0 == seg0 ? ecache[i] : align_expert_of(a, b0 + 64 * i + lane, seg1);
 #pragma unroll
         for (int i = 0; i < kAlignBatch; ++i) {
-            const int r0 = b0 + kAlignThreads * i;
-            if (r0 >= total) break;   // (the same decision in every thread)
-            const int r = r0 + tid, e = eb[i];
-            // the lanes of this wave that hold the same expert: one ballot per bit of the expert id
+            const int r0 = b0 + 64 * i;
+            if (r0 >= seg1) break;   // (the same decision in every lane)
+            const int r = r0 + lane, e = eb[i];
+            // the lanes of this chunk that hold the same expert: one ballot per bit of the expert id
             unsigned long long m = __ballot(e >= 0);
             for (int b = 0; b < id_bits; ++b) {
                 const unsigned long long bal = __ballot((e >> b) & 1);
                 m &= ((e >> b) & 1) ? bal : ~bal;
             }
             const int rank = __popcll(m & lt);
-            if (e >= 0 && rank == 0) tbl[wave][e] = (unsigned short)__popcll(m);
-            __syncthreads();   // the table is complete, and the cursors of the previous super-block have been advanced
+            int base = 0;
+            if (e >= 0) base = cur[e];
+            // every lane has read its cursor before the first lane of each expert moves it on
+            __builtin_amdgcn_s_waitcnt(0xc07f);
+            __builtin_amdgcn_wave_barrier();
             if (e >= 0) {
-                int pos = cursor[e] + rank;
-#pragma unroll
-                for (int w = 0; w < kAlignWaves; ++w) pos += w < wave ? (int)tbl[w][e] : 0;   // (all sixteen reads in flight)
-                if (pos < cap_slots) sorted_token_ids[pos] = r + 1;
+                if (rank == 0) cur[e] = base + __popcll(m);
+                const int pos = base + rank;
+                if (pos < a.cap_slots) a.sorted_token_ids[pos] = r + 1;
             }
-            __syncthreads();   // every lane has read the cursors and the table
-            // Advance the cursors and clear the table.  The entries touched are those of this super-block's experts, and
-            // an entry is written by its own wave only (now, and when the next super-block is counted): no third barrier.
-            if (e >= 0 && rank == 0) {  // first lane of its expert within the wave
-                atomicAdd(&cursor[e], (int)tbl[wave][e]);
-                tbl[wave][e] = 0;
-            }
+            __builtin_amdgcn_s_waitcnt(0xc07f);
+            __builtin_amdgcn_wave_barrier();
         }
     }
+}
+
+// First launch of the two-launch sort: per-expert counts of every workgroup's segment; the last workgroup to arrive
+// turns them into first slots (scratch: counts | rel | start | ticket, see kAlignScratchInts).
+__global__ __launch_bounds__(kAlignThreads) void moe_align_count_kernel(const AlignArgs a, int* __restrict__ scratch) {
+    __shared__ int hist[kAlignMaxExperts];
+    __shared__ int pairs[kAlignPairs];
+    __shared__ int s_ticket, s_blocks, wave_total[kAlignWaves];
+    if ((int)blockIdx.x >= a.sort_wgs) {
+        align_clear(a);
+        return;
+    }
+    const int tid = threadIdx.x, total = a.num_tokens * a.topk, E = a.num_experts, G = a.sort_wgs;
+    int* counts = scratch;
+    int* rel = scratch + kAlignPairs;
+    int* start = scratch + 2 * kAlignPairs;
+    int* ticket = scratch + 2 * kAlignPairs + kAlignMaxExperts;
+    const int seg0 = (int)blockIdx.x * a.wg_chunks * 64, seg1 = seg0 + a.wg_chunks * 64 < total ? seg0 + a.wg_chunks * 64 : total;
+    for (int e = tid; e < E; e += kAlignThreads) hist[e] = 0;
+    __syncthreads();
+    for (int r0 = seg0; r0 < seg1; r0 += kAlignThreads * 4) {
+        int eb[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) eb[i] = align_expert_of(a, r0 + kAlignThreads * i + tid, seg1);
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+            if (eb[i] >= 0) atomicAdd(&hist[eb[i]], 1);
+    }
+    // this workgroup's share of the sentinels (the second launch writes the ids over them)
+    for (int i = (int)blockIdx.x * kAlignThreads + tid; i < a.cap_slots; i += G * kAlignThreads) a.sorted_token_ids[i] = total + 1;
+    __syncthreads();
+    // Counts go out with device-scope stores and come in with device-scope loads: they pass by the L2 of the writer's
+    // and the reader's XCD, and no cache is written back or invalidated as a fence would have it.
+    if (tid < E) __hip_atomic_store(&counts[(int)blockIdx.x * E + tid], hist[tid], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    __builtin_amdgcn_s_waitcnt(0x0070);   // vmcnt(0): the stores have reached memory
+    __syncthreads();
+    if (tid == 0) s_ticket = __hip_atomic_fetch_add(ticket, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    __syncthreads();
+    if (s_ticket != G - 1) return;
+    if (tid == 0) __hip_atomic_store(ticket, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);   // for the next sort
+    for (int i = tid; i < G * E; i += kAlignThreads) pairs[i] = __hip_atomic_load(&counts[i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    __syncthreads();
+    int cnt = 0;
+    if (tid < E) {
+        for (int g = 0; g < G; ++g) {
+            const int c = pairs[g * E + tid];
+            pairs[g * E + tid] = cnt;
+            cnt += c;
+        }
+    }
+    const int nb = (cnt + a.tile_m - 1) / a.tile_m;
+    const int first = align_scan_blocks(nb, wave_total);
+    if (tid < E) {
+        start[tid] = first * a.tile_m;
+        for (int b = first; b < first + nb && b < a.cap_blocks; ++b) a.sorted_expert_ids[b] = tid + 1;
+    }
+    if (tid == kAlignThreads - 1) s_blocks = first + nb < a.cap_blocks ? first + nb : a.cap_blocks;
+    __syncthreads();
+    for (int i = tid; i < G * E; i += kAlignThreads) rel[i] = pairs[i];
+    for (int b = s_blocks + tid; b < a.cap_blocks; b += kAlignThreads) a.sorted_expert_ids[b] = 0;
 }
 
 static int moe_align_device_impl(const mi_tile_array* topk_ids, int tile_m, int num_experts, const mi_tile_array* sorted_token_ids,
@@ -883,10 +1020,43 @@ static int moe_align_device_impl(const mi_tile_array* topk_ids, int tile_m, int 
     }
     if (cap_blocks == 0 && clear_n16 == 0) return MI_OK;
     const int64_t clear_wgs = clear_n16 ? (cld(clear_n16, (int64_t)(4 * kAlignThreads)) < 256 ? cld(clear_n16, (int64_t)(4 * kAlignThreads)) : 256) : 0;
-    hipLaunchKernelGGL(moe_align_kernel, dim3((unsigned)(1 + clear_wgs)), dim3(kAlignThreads), 0, (hipStream_t)stream, (const long long*)topk_ids->ptr,
-                       topk > 1 ? topk_ids->strides[1] : 0, (int)num_tokens, (int)topk, tile_m, num_experts,
-                       (int*)sorted_token_ids->ptr, (int)cap_slots, (int*)sorted_expert_ids->ptr, (int)cap_blocks,
-                       clear ? (u32x4*)clear->ptr : nullptr, clear_n16);
+    AlignArgs a;
+    a.topk_ids = (const long long*)topk_ids->ptr;
+    a.ld_slot = topk > 1 ? topk_ids->strides[1] : 0;
+    a.num_tokens = (int)num_tokens;
+    a.topk = (int)topk;
+    a.inv_topk = topk > 0 ? 1.0f / (float)topk : 0.f;
+    a.tile_m = tile_m;
+    a.num_experts = num_experts;
+    a.sorted_token_ids = (int*)sorted_token_ids->ptr;
+    a.cap_slots = (int)cap_slots;
+    a.sorted_expert_ids = (int*)sorted_expert_ids->ptr;
+    a.cap_blocks = (int)cap_blocks;
+    a.clear = clear ? (u32x4*)clear->ptr : nullptr;
+    a.clear_n16 = clear_n16;
+    const int64_t chunks = cld(total, (int64_t)64);
+    // Two launches of several workgroups: every workgroup at least 1024 replicas, (workgroup, expert) pairs within the
+    // static array.
+    int64_t wgs = kAlignPairs / num_experts < kAlignMaxWgs ? kAlignPairs / num_experts : kAlignMaxWgs;
+    if (wgs > cld(total, (int64_t)kAlignThreads)) wgs = cld(total, (int64_t)kAlignThreads);
+    if (total > kAlignOneWgReplicas && wgs >= 2 && cap_blocks > 0) {
+        ScratchLease lease;
+        if (int* scratch = (int*)lease.acquire(g_align_scratch, HIP_SYMBOL(moe_align_scratch), (hipStream_t)stream)) {
+            a.wg_chunks = (int)(cld(cld(chunks, wgs), (int64_t)kAlignWaves) * kAlignWaves);
+            a.sort_wgs = (int)cld(chunks, (int64_t)a.wg_chunks);
+            hipLaunchKernelGGL(moe_align_count_kernel, dim3((unsigned)(a.sort_wgs + clear_wgs)), dim3(kAlignThreads), 0, (hipStream_t)stream, a, scratch);
+            const int sort_wgs = a.sort_wgs;
+            a.clear_n16 = 0;   // (the first launch has cleared)
+            hipLaunchKernelGGL(moe_align_kernel<true>, dim3((unsigned)sort_wgs), dim3(kAlignThreads), 0, (hipStream_t)stream, a,
+                               scratch + 2 * kAlignPairs, scratch + kAlignPairs);
+            set_variant("moe_align_device_count_place");
+            return launch_status();
+        }
+    }
+    a.sort_wgs = 1;
+    a.wg_chunks = (int)((chunks > 0 ? cld(chunks, (int64_t)kAlignWaves) : 1) * kAlignWaves);
+    hipLaunchKernelGGL(moe_align_kernel<false>, dim3((unsigned)(1 + clear_wgs)), dim3(kAlignThreads), 0, (hipStream_t)stream, a,
+                       (const int*)nullptr, (const int*)nullptr);
     set_variant("moe_align_device_1wg");
     return launch_status();
 }

@@ -204,8 +204,10 @@ int mi_fmha_kernel(const mi_tile_array* Q, const mi_tile_array* K, const mi_tile
 int mi_moe_align_tile_size(const int64_t* topk_ids, int64_t num_tokens, int64_t topk, int tile_m,
                            int num_experts, int32_t* sorted_token_ids_out,
                            int32_t* sorted_expert_ids_out, int64_t* total_blocks_out);
-/* Device counterpart of moe_align_tile_size: the same stable counting sort, run by one workgroup
- * on `stream`, so that cutile_moe needs no host round trip (the reference copies topk_ids to the
+/* Device counterpart of moe_align_tile_size: the same stable counting sort on `stream` (one launch of one
+ * workgroup up to 8192 replicas; above, two launches of up to 64 workgroups whose per-expert counts meet in a static
+ * array of the library -- a stream under graph capture is not given that array and sorts with one workgroup),
+ * so that cutile_moe needs no host round trip (the reference copies topk_ids to the
  * host, sorts there and copies the result back: moe.jl:232-233).  topk_ids (num_tokens, topk)
  * i64 on the device.  The outputs have fixed capacity, since the block count is only known on
  * the device: sorted_expert_ids needs at least

@@ -188,10 +188,13 @@ def test_moe_full_size_top2(orc):
 @pytest.mark.parametrize("num_tokens,topk,E,tile_m", [(256, 2, 32, 128), (48, 8, 64, 16), (7, 3, 5, 4), (1, 1, 1, 128),
                                                       (1000, 4, 9, 32), (130, 2, 1000, 8),
                                                       (512, 2, 32, 128), (512, 4, 7, 16), (513, 4, 7, 16), (2049, 1, 33, 64),
-                                                      (4096, 2, 32, 128), (4100, 3, 11, 128), (16385, 2, 160, 64)])   # one, two and five batches of ids
+                                                      (4096, 2, 32, 128), (4100, 3, 11, 128),   # one and two batches of ids per wave
+                                                      (16385, 2, 160, 64), (8193, 1, 1000, 8), (40000, 3, 3, 128),   # several workgroups:
+                                                      (70000, 2, 1024, 16), (9000, 7, 64, 128)])                      # 33, 9, 64, 16 and 62 of them
 def test_device_align_matches_host_routine(ct, orc, num_tokens, topk, E, tile_m):
-    """The one-workgroup counting sort gives the host routine's arrays (stable per-expert order,
-    sentinel padding) in the leading part of its fixed-capacity outputs, and marks the rest unused."""
+    """The counting sort (one workgroup, or two launches of several above 8192 replicas) gives the host routine's
+    arrays (stable per-expert order, sentinel padding) in the leading part of its fixed-capacity outputs, and marks
+    the rest unused."""
     rng = np.random.default_rng(num_tokens + topk)
     ids = rng.integers(1, E + 1, size=(topk, num_tokens), dtype=np.int64)   # torch layout of Julia (tokens, topk)
     ids_t = torch.from_numpy(ids)
@@ -202,9 +205,58 @@ def test_device_align_matches_host_routine(ct, orc, num_tokens, topk, E, tile_m)
     assert tok_d.numel() == slots and exp_d.numel() == blocks and nb <= blocks
     assert torch.equal(exp_d[:nb].cpu(), exp_h) and torch.all(exp_d[nb:] == 0)
     assert torch.equal(tok_d[:nb * tile_m].cpu(), tok_h) and torch.all(tok_d[nb * tile_m:] == num_tokens * topk + 1)
+    assert ct.last_variant() == ("moe_align_device_count_place" if num_tokens * topk > 8192 else "moe_align_device_1wg")
     # oracle as a third opinion
     tok_o, exp_o = orc.moe_align_tile_size(ids.T, tile_m, E)
     assert np.array_equal(tok_h.numpy(), tok_o) and np.array_equal(exp_h.numpy(), exp_o)
+
+
+def test_device_align_of_several_workgroups_in_a_row_and_under_capture(ct):
+    """The two-launch sort keeps its counts in an array of the library: a smaller batch after a larger one, a batch
+    with ids outside 1..E and one that clears an array on the way all match the host routine; a capturing stream is
+    not given the array, sorts with one workgroup, and the replayed graph gives the same arrays."""
+    rng = np.random.default_rng(5)
+    E, tile_m = 48, 64
+    for num_tokens, topk, bad in [(30000, 4, False), (5000, 2, False), (12000, 3, True), (9000, 1, False)]:
+        ids = rng.integers(1, E + 1, size=(topk, num_tokens), dtype=np.int64)
+        if bad:
+            ids[rng.random(ids.shape) < 0.1] = 0
+            ids[rng.random(ids.shape) < 0.05] = E + 7
+        ids_t = torch.from_numpy(ids)
+        valid = torch.from_numpy(((ids >= 1) & (ids <= E)).T.reshape(-1))   # replica order: slot fastest
+        junk = torch.full((1024, 33), 3.0, dtype=torch.float16, device="cuda")
+        tok_d, exp_d = ct.moe_align_tile_size_device(ids_t.cuda(), tile_m, E, clear=junk)
+        multi = num_tokens * topk > 8192
+        assert ct.last_variant() == ("moe_align_device_count_place" if multi else "moe_align_device_1wg")
+        assert not junk.any()
+        if not bad:
+            tok_h, exp_h = ct.moe_align_tile_size(ids_t, tile_m, E)
+        else:   # the host routine takes valid ids only: sort the valid replicas, keep their original numbers
+            flat = ids.T.reshape(-1)
+            keep = np.nonzero(valid.numpy())[0]
+            tok_s, exp_h = ct.moe_align_tile_size(torch.from_numpy(flat[keep].reshape(1, -1).copy()), tile_m, E)
+            sentinel = tok_s == keep.size + 1
+            tok_h = torch.from_numpy(keep.astype(np.int32) + 1)[(tok_s.long() - 1).clamp(max=keep.size - 1)]
+            tok_h[sentinel] = num_tokens * topk + 1
+        nb = exp_h.numel()
+        assert torch.equal(exp_d[:nb].cpu(), exp_h) and torch.all(exp_d[nb:] == 0)
+        assert torch.equal(tok_d[:nb * tile_m].cpu(), tok_h) and torch.all(tok_d[nb * tile_m:] == num_tokens * topk + 1)
+    # the last batch again, captured
+    ids_d = ids_t.cuda()
+    tok_g, exp_g = torch.empty_like(tok_d), torch.empty_like(exp_d)
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(side):
+        with torch.cuda.graph(g, stream=side):
+            ct.moe_align_tile_size_device(ids_d, tile_m, E, tok_g, exp_g, stream=side)
+            assert ct.last_variant() == "moe_align_device_1wg"
+    for _ in range(2):
+        tok_g.fill_(-1); exp_g.fill_(-1)
+        torch.cuda.synchronize()
+        g.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(tok_g, tok_d) and torch.equal(exp_g, exp_d)
 
 
 @pytest.mark.parametrize("num_tokens,E,topk,dtype", [(256, 32, 2, torch.float32), (48, 64, 8, torch.float32),

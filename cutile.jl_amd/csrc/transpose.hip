@@ -9,9 +9,9 @@
 //     XOR-swizzled LDS tile in both directions, workgroup ids walking 8x8 super-tiles
 //     (transpose_micro_kernel);
 //     sizes that are not multiples of a vector are taken too when the leading dimensions are (edge tiles element-wise);
-//   * everything else: 64x64 (large 2- and 4-byte matrices: 128x128) tiles through a padded LDS tile (pitch + 1
-//     element: both the scattered writes and the gathered reads hit distinct banks), 16-byte global accesses
-//     where alignment allows, element-wise with bounds checks otherwise (transpose_kernel).
+//   * everything else (columns that start off 16-byte boundaries): 64 x 64 tiles through a padded LDS tile, one element
+//     per lane and access with the lanes of a wave consecutive in memory on both sides, workgroup ids banded by XCD
+//     (transpose_elem_kernel).
 // Algorithmic traffic: 2 * m * n * sizeof(T) bytes.
 #include "common.h"
 #include <stdlib.h>
@@ -25,62 +25,48 @@ template <typename T, int N> struct VecOf {
     typedef T type __attribute__((ext_vector_type(N)));
 };
 
-// VEC: true  -> every 16-byte vector is either fully inside or fully outside the matrix
-//               and 16-byte aligned (checked on the host);
-//      false -> element-wise accesses with per-element bounds checks.
-template <typename T, bool VEC, int kTile = 64, int kBlock = 256>
-__global__ __launch_bounds__(kBlock) void transpose_kernel(const T* __restrict__ x, int64_t ldx,
-                                                           T* __restrict__ y, int64_t ldy,
-                                                           int64_t m, int64_t n) {
-    constexpr int V = 16 / sizeof(T);        // elements per 16-byte vector
-    constexpr int VR = kTile / V;            // vectors per tile row
-    constexpr int RP = kBlock / VR;          // tile rows covered per pass
-    constexpr int PASSES = kTile / RP;
-    using VT = typename VecOf<T, V>::type;
-    constexpr int kPitch = kTile + 1;
-    __shared__ T lds[kTile * kPitch];
-
-    const int64_t m0 = (int64_t)blockIdx.x * kTile;  // along x dim 0
-    const int vi = threadIdx.x % VR, row = threadIdx.x / VR;
-    // (the second grid dimension holds at most 65535 workgroups: walk the tile rows along dim 1 with that stride)
-    for (int64_t n0 = (int64_t)blockIdx.y * kTile; n0 < n; n0 += (int64_t)gridDim.y * kTile) {
-    // Phase 1: x[m0 + V*vi .. +V-1, n0 + r]  ->  lds[i][j] with i along m, j along n.
+// ---- columns that start anywhere: one element per lane and access ------------------------------
+// No 16-byte vector is aligned in every column, so a lane moves single elements, and what keeps the memory system
+// busy is the shape of a wave's access: 64 lanes on 64 consecutive elements of a column, on the load side (lanes
+// along m) and on the store side (lanes along n) alike, with all of a lane's loads issued before the first of them is
+// used.  (The padded-tile kernel above gives a lane V consecutive elements, as its vector form wants them: element
+// by element a wave's access then covers V times the span at 1/V of the density, and the 8191 x 8193 fp32 case ran at
+// 3.0 TB/s.)  The tile sits in LDS with rows of TN + 1 elements: the scattered writes of phase 1 (stride TN + 1
+// elements between lanes) and the linear reads of phase 2 both spread over the banks.
+// A column of a tile starts and ends inside 128-byte lines that the neighbouring tiles along the column share, on the
+// load side (neighbours along m) and on the store side (neighbours along n) alike.  Workgroup ids go round the eight
+// XCDs, each with an L2 of its own: id % 8 therefore selects a band of tile rows along m, and the ids of one XCD walk
+// their band m-fastest, so that the workgroups resident on an XCD at one time cover a compact patch of tiles and both
+// kinds of neighbours meet in the same L2 (a shared line is fetched once and written back whole).
+template <typename T, int TM, int TN, int NT>
+__global__ __launch_bounds__(NT) void transpose_elem_kernel(const T* __restrict__ x, int64_t ldx, T* __restrict__ y,
+                                                            int64_t ldy, int64_t m, int64_t n, int tiles_m, int band) {
+    constexpr int kPitch = TN + 1;
+    __shared__ T lds[TM * kPitch];
+    constexpr int LM = TM < NT ? TM : NT, CJ = NT / LM, P1 = TN / CJ;   // phase 1: LM lanes along m, CJ columns per pass
+    constexpr int LN = TN < NT ? TN : NT, CI = NT / LN, P2 = TM / CI;   // phase 2: LN lanes along n, CI rows per pass
+    static_assert(LM * CJ == NT && CJ * P1 == TN && LN * CI == NT && CI * P2 == TM && LM == TM && LN == TN, "the lanes tile the block");
+    const int xcd = blockIdx.x & 7, seq = blockIdx.x >> 3;
+    const int bm = xcd * band + seq % band;
+    if (bm >= tiles_m || seq % band >= band) return;   // (the last band may be short; the whole workgroup leaves)
+    const int64_t m0 = (int64_t)bm * TM, n0 = (int64_t)(seq / band) * TN;
+    const int i1 = threadIdx.x % LM, j1 = threadIdx.x / LM;
+    const int j2 = threadIdx.x % LN, i2 = threadIdx.x / LN;
+    T v[P1];
+    const bool in_m = m0 + i1 < m;
 #pragma unroll
-    for (int p = 0; p < PASSES; ++p) {
-        const int j = row + p * RP;
-        const int64_t gi = m0 + vi * V, gj = n0 + j;
-        if constexpr (VEC) {
-            if (gi < m && gj < n) {
-                VT v = ld_global<true>(reinterpret_cast<const VT*>(x + gi + gj * ldx));
-#pragma unroll
-                for (int q = 0; q < V; ++q) lds[(vi * V + q) * kPitch + j] = v[q];
-            }
-        } else {
-#pragma unroll
-            for (int q = 0; q < V; ++q)
-                if (gi + q < m && gj < n) lds[(vi * V + q) * kPitch + j] = x[gi + q + gj * ldx];
-        }
+    for (int p = 0; p < P1; ++p) {
+        const int64_t gj = n0 + j1 + p * CJ;
+        v[p] = in_m && gj < n ? x[m0 + i1 + gj * ldx] : T(0);
     }
+#pragma unroll
+    for (int p = 0; p < P1; ++p) lds[i1 * kPitch + j1 + p * CJ] = v[p];
     __syncthreads();
-    // Phase 2: y[n0 + V*vi .. +V-1, m0 + r]  <-  lds[r][V*vi .. ].
+    const bool in_n = n0 + j2 < n;
 #pragma unroll
-    for (int p = 0; p < PASSES; ++p) {
-        const int i = row + p * RP;
-        const int64_t gj = n0 + vi * V, gi = m0 + i;
-        if constexpr (VEC) {
-            if (gj < n && gi < m) {
-                VT v;
-#pragma unroll
-                for (int q = 0; q < V; ++q) v[q] = lds[i * kPitch + vi * V + q];
-                st_global<true>(v, reinterpret_cast<VT*>(y + gj + gi * ldy));
-            }
-        } else {
-#pragma unroll
-            for (int q = 0; q < V; ++q)
-                if (gj + q < n && gi < m) y[gj + q + gi * ldy] = lds[i * kPitch + vi * V + q];
-        }
-    }
-    __syncthreads();   // the tile is free for the next trip
+    for (int p = 0; p < P2; ++p) {
+        const int64_t gi = m0 + i2 + p * CI;
+        if (in_n && gi < m) y[n0 + j2 + gi * ldy] = lds[(i2 + p * CI) * kPitch + j2];
     }
 }
 
@@ -311,38 +297,25 @@ int launch1(const mi_tile_array* x, const mi_tile_array* y, hipStream_t s, bool 
     }
 }
 
-template <typename T, int TILE, int BLOCK>
-int launch_tile(const mi_tile_array* x, const mi_tile_array* y, hipStream_t s) {
-    constexpr int V = 16 / sizeof(T);
+template <typename T, int TM, int TN, int NT>
+int launch_elem(const mi_tile_array* x, const mi_tile_array* y, hipStream_t s, const char* name) {
     const int64_t m = x->sizes[0], n = x->sizes[1];
-    const int64_t ldx = x->strides[1], ldy = y->strides[1];
-    const int64_t gx = cld(m, (int64_t)TILE), gy = cld(n, (int64_t)TILE);
-    if (gx > 0x7fffffffLL) return MI_E_GRID;
-    const bool vec = (m % V == 0) && (n % V == 0) && (ldx % V == 0) && (ldy % V == 0) &&
-                     aligned(x->ptr, 16) && aligned(y->ptr, 16);
-    dim3 grid((unsigned)gx, (unsigned)(gy < 65535 ? gy : 65535)), block(BLOCK);
-    if (vec) {
-        hipLaunchKernelGGL((transpose_kernel<T, true, TILE, BLOCK>), grid, block, 0, s, (const T*)x->ptr, ldx,
-                           (T*)y->ptr, ldy, m, n);
-        set_variant(TILE == 64 ? "transpose_lds64_vec16" : "transpose_lds128_vec16");
-    } else {
-        hipLaunchKernelGGL((transpose_kernel<T, false, TILE, BLOCK>), grid, block, 0, s, (const T*)x->ptr, ldx,
-                           (T*)y->ptr, ldy, m, n);
-        set_variant(TILE == 64 ? "transpose_lds64_elem" : "transpose_lds128_elem");
-    }
+    const int64_t tiles_m = cld(m, (int64_t)TM), tiles_n = cld(n, (int64_t)TN);
+    const int64_t band = cld(tiles_m, (int64_t)8);   // tile rows per XCD
+    if (tiles_m > 0x7fffffffLL || 8 * band * tiles_n > 0x7fffffffLL) return MI_E_GRID;
+    hipLaunchKernelGGL((transpose_elem_kernel<T, TM, TN, NT>), dim3((unsigned)(8 * band * tiles_n)), dim3(NT), 0, s,
+                       (const T*)x->ptr, x->strides[1], (T*)y->ptr, y->strides[1], m, n, (int)tiles_m, (int)band);
+    set_variant(name);
     return launch_status();
 }
 
-// Sizes or strides that rule out the register micro-transpose.  Large matrices of 2- and 4-byte elements take
-// 128 x 128 tiles of 1024 lanes (runs of 256 / 512 bytes instead of 128 / 256).
+// Sizes or strides that rule out the register micro-transpose.
 template <typename T>
 int launch(const mi_tile_array* x, const mi_tile_array* y, hipStream_t s) {
-    int big = sizeof(T) <= 4 && sizeof(T) >= 2 && cld(x->sizes[0], (int64_t)128) * cld(x->sizes[1], (int64_t)128) >= 512;
-    if (const char* e = getenv("MI_TRANSPOSE_FALLBACK_TILE")) big = atoi(e) == 128 && sizeof(T) <= 4;
-    if constexpr (sizeof(T) <= 4) {
-        if (big) return launch_tile<T, 128, 1024>(x, y, s);
-    }
-    return launch_tile<T, 64, 256>(x, y, s);
+    int shape = 0;
+    if (const char* e = getenv("MI_TRANSPOSE_ELEM_TILE")) shape = atoi(e);
+    if (shape == 3) return launch_elem<T, 128, 128, 1024>(x, y, s, "transpose_elem_128x128_t1024");
+    return launch_elem<T, 64, 64, 256>(x, y, s, "transpose_elem_64x64_t256");
 }
 
 }  // namespace

@@ -205,7 +205,7 @@ def test_transpose_views_of_a_padded_parent_with_ragged_sizes(ct, T, isz):
     """Sizes that are not multiples of a 16-byte vector inside parents whose leading dimensions are: the register path
     with edge tiles that move the vectors crossing the edge element by element.  Small and large tile variants; what
     lies around the destination view stays as it was.  A dense matrix with such sizes has misaligned columns and takes
-    the padded-tile kernel."""
+    the element-wise kernel (several bands of tile rows, short last band, ragged last tiles)."""
     v = 16 // isz
     iv = {1: torch.uint8, 2: torch.int16, 4: torch.int32, 8: torch.int64}[isz]
     g = torch.Generator(device="cuda"); g.manual_seed(200 + isz)
@@ -219,10 +219,16 @@ def test_transpose_views_of_a_padded_parent_with_ragged_sizes(ct, T, isz):
         assert ct.last_variant().endswith("_regmicro_ragged"), ct.last_variant()
         assert torch.equal(y, x.t()), (r, c)
         assert bool((yb[c:, :] == 85).all()) and bool((yb[:, r:] == 85).all()), (r, c)
-    x = torch.randint(0, 256, (1001, 999 * isz), device="cuda", generator=g).to(torch.uint8).view(iv)
-    y = torch.empty(999, 1001, dtype=iv, device="cuda")
-    ct.transpose_kernel(x.view(T), y.view(T), 64, 64)
-    assert ct.last_variant().startswith("transpose_lds") and torch.equal(y, x.t())
+    for r, c in [(1001, 999), (3, 2049), (2049, 3), (577, 1), (1, 577), (4097, 67)]:   # torch (r, c) = Julia (c, r)
+        x = torch.randint(0, 256, (r, c * isz), device="cuda", generator=g).to(torch.uint8).view(iv)
+        yb = torch.full((c + 1, r + 2), 85, dtype=iv, device="cuda")
+        y = yb[:c, :r]
+        if c % v == 0 or r == 1:
+            continue   # (aligned columns: not this kernel's case)
+        ct.transpose_kernel(x.view(T), y.view(T), 64, 64)
+        assert ct.last_variant().startswith("transpose_elem_"), ct.last_variant()
+        assert torch.equal(y, x.t()), (r, c)
+        assert bool((yb[c:, :] == 85).all()) and bool((yb[:, r:] == 85).all()), (r, c)
 
 
 def test_transpose_full_size_involution():

@@ -37,6 +37,39 @@ namespace {
 using namespace mi;
 using namespace mi::gemm;
 
+// 16 bytes from an address that is aligned for its elements only.  Global memory takes unaligned vector accesses (a
+// row of a dense matrix whose leading dimension is odd starts anywhere): one instruction either way, where eight
+// 2-byte loads per lane ran a 4095^3 problem at a tenth of the aligned rate.
+template <typename V, typename T>
+__device__ __forceinline__ V ld16(const T* p) {
+    V v;
+    __builtin_memcpy(&v, p, sizeof(V));
+    return v;
+}
+
+// A vector of NE elements of a row at p of which only the first `valid` belong to the matrix (the row ends there; valid
+// may be <= 0 or >= NE); `room` elements from p on lie inside the array (up to the end of its last row).  Where the
+// whole vector is readable it is read whole and the elements past the row's end -- the start of the next row, or the
+// parent's padding -- are zeroed in registers; only at the end of the last row does the tail go element by element.
+// (Element-wise tails on every row made the workgroups on the matrix edge five times slower than the others, and a
+// launch waited for them.)
+template <typename V, int NE, typename T>
+__device__ __forceinline__ V ld_edge(const T* p, int64_t valid, int64_t room) {
+    V v = {0};
+    if (valid <= 0) return v;
+    if (room >= NE) {
+        v = ld16<V>(p);
+#pragma unroll
+        for (int q = 1; q < NE; ++q)
+            if (q >= valid) v[q] = 0;
+    } else {
+#pragma unroll
+        for (int q = 0; q < NE; ++q)
+            if (q < valid) v[q] = p[q];
+    }
+    return v;
+}
+
 // ---- generic 16-bit kernel ---------------------------------------------------------------
 // Workgroup tile 64(m) x 64(n), K step 32, 4 waves as 2x2 of 32x32.
 constexpr int GT = 64, GK = 32, GA_PITCH = GT + 8, GB_PITCH = GK + 8;
@@ -45,7 +78,7 @@ template <typename E, typename OutT>
 __global__ __launch_bounds__(256) void gemm16_generic(
     const unsigned short* __restrict__ A, int64_t lda, int64_t sa, const unsigned short* __restrict__ B,
     int64_t ldb, int64_t sb, OutT* __restrict__ C, int64_t ldc, int64_t sc, int M, int N, int K,
-    int tiles_m, int tiles_mn, bool vecA, bool vecB) {
+    int tiles_m, int tiles_mn) {
     __shared__ __attribute__((aligned(16))) unsigned short As[GK * GA_PITCH];  // [k][m]
     __shared__ __attribute__((aligned(16))) unsigned short Bs[GT * GB_PITCH];  // [n][k]
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -67,20 +100,14 @@ __global__ __launch_bounds__(256) void gemm16_generic(
             const int64_t gm = m0 + am;
             const int gk = k0 + ak;
             if (gk < K) {
-                const unsigned short* p = A + gm + (int64_t)gk * lda;
-                if (vecA && gm + 8 <= M) va = *reinterpret_cast<const s16x8*>(p);
-                else
-#pragma unroll
-                    for (int q = 0; q < 8; ++q) va[q] = (gm + q < M) ? (short)p[q] : (short)0;
+                const int64_t o = gm + (int64_t)gk * lda;
+                va = ld_edge<s16x8, 8>((const short*)A + o, M - gm, (int64_t)(K - 1) * lda + M - o);
             }
             const int64_t gn = n0 + bnn;
             const int gk2 = k0 + bk;
             if (gn < N) {
-                const unsigned short* p = B + gk2 + gn * ldb;
-                if (vecB && gk2 + 8 <= K) vb = *reinterpret_cast<const s16x8*>(p);
-                else
-#pragma unroll
-                    for (int q = 0; q < 8; ++q) vb[q] = (gk2 + q < K) ? (short)p[q] : (short)0;
+                const int64_t o = gk2 + gn * ldb;
+                vb = ld_edge<s16x8, 8>((const short*)B + o, K - gk2, (int64_t)(N - 1) * ldb + K - o);
             }
         }
         __syncthreads();  // previous iteration's fragment reads are done
@@ -108,8 +135,8 @@ __global__ __launch_bounds__(256) void gemm16_generic(
 // Workgroup tile 128(m) x 128(n), K step 32, 4 waves as 2x2 of 64x64 (four 32x32x16 MFMAs per 16
 // k, one LDS fragment read per MFMA).  The next K step's operands are requested into registers
 // before the current step's MFMAs and cross the workgroup barriers in flight (the barriers wait
-// for LDS accesses only).  Any shape: workgroups whose tile is interior and 16-byte aligned load
-// without predicates; the others zero-pad element by element.
+// for LDS accesses only).  Any shape: workgroups whose tile is interior load without predicates (16 bytes
+// per lane, aligned or not); the others zero-pad, element by element where a vector crosses the edge.
 constexpr int MT = 128, MA_PITCH = MT + 8, MB_PITCH = GK + 8;
 
 __device__ __forceinline__ void lds_barrier() {
@@ -123,7 +150,7 @@ template <typename E, typename OutT>
 __global__ __launch_bounds__(256) void gemm16_mid(
     const unsigned short* __restrict__ A, int64_t lda, int64_t sa, const unsigned short* __restrict__ B,
     int64_t ldb, int64_t sb, OutT* __restrict__ C, int64_t ldc, int64_t sc, int M, int N, int K,
-    int tiles_m, int tiles_mn, bool vecA, bool vecB) {
+    int tiles_m, int tiles_mn) {
     __shared__ __attribute__((aligned(16))) unsigned short As[GK * MA_PITCH];  // [k][m]
     __shared__ __attribute__((aligned(16))) unsigned short Bs[MT * MB_PITCH];  // [n][k]
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -136,49 +163,63 @@ __global__ __launch_bounds__(256) void gemm16_mid(
     const int wm = (wave & 1) * 64, wn = (wave >> 1) * 64;
     const int ak = tid >> 4, am = (tid & 15) * 8;   // A tile: rows k = ak and ak + 16, 8 consecutive m
     const int bnn = tid >> 2, bk = (tid & 3) * 8;   // B tile: columns n = bnn and bnn + 64, 8 consecutive k
-    const bool interior = vecA && vecB && m0 + MT <= M && n0 + MT <= N;   // same for the whole workgroup
+    // Workgroups on the M or N edge load like the others wherever that reads existing memory: a row of B past the
+    // last one is replaced by the last one, a vector of A past the end of its row reads on into the next row; what they
+    // bring only reaches elements of C that are never stored.  Left to the element-wise path: the K steps in which
+    // such a vector of A would pass the end of the array (the last rows), and a last K step that is not whole.
+    const int64_t over_m = m0 + MT - M;   // > 0: elements by which the tile's rows overrun the matrix
+    const int64_t bn_row[2] = {n0 + bnn < N ? n0 + bnn : N - 1, n0 + bnn + 64 < N ? n0 + bnn + 64 : N - 1};
 
     f32x16 acc[2][2] = {};
     s16x8 va[2], vb[2];
+    int validA = 8, validB = 8;   // elements of the staged vectors that belong to the matrix
     auto gload = [&](int k0) {
-        if (interior && k0 + GK <= K) {
+        if (k0 + GK <= K && (over_m <= 0 || (lda >= 0 && (int64_t)(K - k0 - GK) * lda >= over_m))) {   // same for the whole workgroup
+            validA = validB = 8;
 #pragma unroll
             for (int h = 0; h < 2; ++h) {
-                va[h] = *reinterpret_cast<const s16x8*>(A + m0 + am + (int64_t)(k0 + ak + 16 * h) * lda);
-                vb[h] = *reinterpret_cast<const s16x8*>(B + k0 + bk + (n0 + bnn + 64 * h) * ldb);
+                va[h] = ld16<s16x8>(A + m0 + am + (int64_t)(k0 + ak + 16 * h) * lda);
+                vb[h] = ld16<s16x8>(B + k0 + bk + bn_row[h] * ldb);
             }
             return;
         }
+        // Edge: whole vectors wherever they are readable; what lies past the end of a row is zeroed when the vector
+        // goes to LDS, a K step later (zeroing it here would wait for the load here, and the edge workgroups, with no
+        // look-ahead left, ran five times longer than the others).
+        const int64_t gm = m0 + am;
+        const int gk2 = k0 + bk;
+        validA = M - gm < 8 ? (M - gm > 0 ? (int)(M - gm) : 0) : 8;
+        validB = K - gk2 < 8 ? (K - gk2 > 0 ? K - gk2 : 0) : 8;
 #pragma unroll
         for (int h = 0; h < 2; ++h) {
             va[h] = vb[h] = s16x8{0};
-            const int64_t gm = m0 + am;
             const int gk = k0 + ak + 16 * h;
-            if (gk < K) {
-                const unsigned short* p = A + gm + (int64_t)gk * lda;
-                if (vecA && gm + 8 <= M) va[h] = *reinterpret_cast<const s16x8*>(p);
-                else
-#pragma unroll
-                    for (int q = 0; q < 8; ++q) va[h][q] = (gm + q < M) ? (short)p[q] : (short)0;
+            if (gk < K && validA > 0) {
+                const int64_t o = gm + (int64_t)gk * lda;
+                if ((int64_t)(K - 1) * lda + M - o >= 8) va[h] = ld16<s16x8>(A + o);
+                else va[h] = ld_edge<s16x8, 8>((const short*)A + o, validA, 0);
             }
             const int64_t gn = n0 + bnn + 64 * h;
-            const int gk2 = k0 + bk;
-            if (gn < N) {
-                const unsigned short* p = B + gk2 + gn * ldb;
-                if (vecB && gk2 + 8 <= K) vb[h] = *reinterpret_cast<const s16x8*>(p);
-                else
-#pragma unroll
-                    for (int q = 0; q < 8; ++q) vb[h][q] = (gk2 + q < K) ? (short)p[q] : (short)0;
+            if (gn < N && validB > 0) {
+                const int64_t o = gk2 + gn * ldb;
+                if ((int64_t)(N - 1) * ldb + K - o >= 8) vb[h] = ld16<s16x8>(B + o);
+                else vb[h] = ld_edge<s16x8, 8>((const short*)B + o, validB, 0);
             }
         }
+    };
+    auto keep = [](s16x8 v, int valid) {
+#pragma unroll
+        for (int q = 1; q < 8; ++q)
+            if (q >= valid) v[q] = 0;
+        return v;
     };
     gload(0);
     for (int k0 = 0; k0 < K; k0 += GK) {
         lds_barrier();  // previous iteration's fragment reads are done
 #pragma unroll
         for (int h = 0; h < 2; ++h) {
-            *reinterpret_cast<s16x8*>(&As[(ak + 16 * h) * MA_PITCH + am]) = va[h];
-            *reinterpret_cast<s16x8*>(&Bs[(bnn + 64 * h) * MB_PITCH + bk]) = vb[h];
+            *reinterpret_cast<s16x8*>(&As[(ak + 16 * h) * MA_PITCH + am]) = validA < 8 ? keep(va[h], validA) : va[h];
+            *reinterpret_cast<s16x8*>(&Bs[(bnn + 64 * h) * MB_PITCH + bk]) = validB < 8 ? keep(vb[h], validB) : vb[h];
         }
         lds_barrier();
         if (k0 + GK < K) gload(k0 + GK);
@@ -219,8 +260,7 @@ constexpr int FT = 128, FK = 16, F_PITCH = FT + 32;
 __global__ __launch_bounds__(256) void gemm32_kernel(const float* __restrict__ A, int64_t lda, int64_t sa,
                                                      const float* __restrict__ B, int64_t ldb, int64_t sb,
                                                      float* __restrict__ C, int64_t ldc, int64_t sc, int M,
-                                                     int N, int K, int tiles_m, int tiles_mn, bool vecA,
-                                                     bool vecB) {
+                                                     int N, int K, int tiles_m, int tiles_mn) {
     __shared__ __attribute__((aligned(16))) float As[FK * F_PITCH];  // [k][m]
     __shared__ __attribute__((aligned(16))) float Bs[FK * F_PITCH];  // [k][n]
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -241,29 +281,24 @@ __global__ __launch_bounds__(256) void gemm32_kernel(const float* __restrict__ A
         {
             const int64_t gm = m0 + am;
             const int gk = k0 + ak;
-            const float* p = A + gm + (int64_t)gk * lda;
-            if (gk < K && vecA && gm + 68 <= M) {
-                f32x4 t0 = *reinterpret_cast<const f32x4*>(p), t1 = *reinterpret_cast<const f32x4*>(p + 64);
-#pragma unroll
-                for (int q = 0; q < 4; ++q) { va[q] = t0[q]; va[4 + q] = t1[q]; }
-            } else {
-#pragma unroll
-                for (int q = 0; q < 8; ++q) {
-                    const int o = (q & 3) + 64 * (q >> 2);
-                    va[q] = (gk < K && gm + o < M) ? p[o] : 0.f;
-                }
+            f32x4 t0 = {0}, t1 = {0};
+            if (gk < K) {
+                const int64_t o = gm + (int64_t)gk * lda, room = (int64_t)(K - 1) * lda + M - o;
+                t0 = ld_edge<f32x4, 4>(A + o, M - gm, room);
+                t1 = ld_edge<f32x4, 4>(A + o + 64, M - gm - 64, room - 64);
             }
+#pragma unroll
+            for (int q = 0; q < 4; ++q) { va[q] = t0[q]; va[4 + q] = t1[q]; }
             const int64_t gn = n0 + bnn;
             const int gk2 = k0 + bk;
-            const float* pb = B + gk2 + gn * ldb;
-            if (gn < N && vecB && gk2 + 8 <= K) {
-                f32x4 t0 = *reinterpret_cast<const f32x4*>(pb), t1 = *reinterpret_cast<const f32x4*>(pb + 4);
-#pragma unroll
-                for (int q = 0; q < 4; ++q) { vb[q] = t0[q]; vb[4 + q] = t1[q]; }
-            } else {
-#pragma unroll
-                for (int q = 0; q < 8; ++q) vb[q] = (gn < N && gk2 + q < K) ? pb[q] : 0.f;
+            t0 = t1 = f32x4{0};
+            if (gn < N) {
+                const int64_t o = gk2 + gn * ldb, room = (int64_t)(N - 1) * ldb + K - o;
+                t0 = ld_edge<f32x4, 4>(B + o, K - gk2, room);
+                t1 = ld_edge<f32x4, 4>(B + o + 4, K - gk2 - 4, room - 4);
             }
+#pragma unroll
+            for (int q = 0; q < 4; ++q) { vb[q] = t0[q]; vb[4 + q] = t1[q]; }
         }
         __syncthreads();
 #pragma unroll
@@ -347,21 +382,17 @@ int validate(const mi_tile_array* A, const mi_tile_array* B, const mi_tile_array
 template <typename E, typename OutT>
 void launch_mid16(const Problem& p, hipStream_t s) {
     const int tiles_m = (int)cld((int64_t)p.M, (int64_t)MT), tiles_n = (int)cld((int64_t)p.N, (int64_t)MT);
-    const bool vecA = aligned(p.A, 16) && p.lda % 8 == 0 && p.sa % 8 == 0;
-    const bool vecB = aligned(p.B, 16) && p.ldb % 8 == 0 && p.sb % 8 == 0;
     hipLaunchKernelGGL((gemm16_mid<E, OutT>), dim3((unsigned)(tiles_m * tiles_n * p.batch)), dim3(256), 0,
                        s, (const unsigned short*)p.A, p.lda, p.sa, (const unsigned short*)p.B, p.ldb, p.sb,
-                       (OutT*)p.C, p.ldc, p.sc, p.M, p.N, p.K, tiles_m, tiles_m * tiles_n, vecA, vecB);
+                       (OutT*)p.C, p.ldc, p.sc, p.M, p.N, p.K, tiles_m, tiles_m * tiles_n);
 }
 
 template <typename E, typename OutT>
 void launch_generic16(const Problem& p, hipStream_t s) {
     const int tiles_m = (int)cld((int64_t)p.M, (int64_t)GT), tiles_n = (int)cld((int64_t)p.N, (int64_t)GT);
-    const bool vecA = aligned(p.A, 16) && p.lda % 8 == 0 && p.sa % 8 == 0;
-    const bool vecB = aligned(p.B, 16) && p.ldb % 8 == 0 && p.sb % 8 == 0;
     hipLaunchKernelGGL((gemm16_generic<E, OutT>), dim3((unsigned)(tiles_m * tiles_n * p.batch)),
                        dim3(256), 0, s, (const unsigned short*)p.A, p.lda, p.sa, (const unsigned short*)p.B,
-                       p.ldb, p.sb, (OutT*)p.C, p.ldc, p.sc, p.M, p.N, p.K, tiles_m, tiles_m * tiles_n, vecA, vecB);
+                       p.ldb, p.sb, (OutT*)p.C, p.ldc, p.sc, p.M, p.N, p.K, tiles_m, tiles_m * tiles_n);
 }
 
 int run(const Problem& p, hipStream_t s) {
@@ -377,11 +408,9 @@ int run(const Problem& p, hipStream_t s) {
             return launch_status();
         }
         const int tiles_m = (int)cld((int64_t)p.M, (int64_t)FT), tiles_n = (int)cld((int64_t)p.N, (int64_t)FT);
-        const bool vecA = aligned(p.A, 16) && p.lda % 4 == 0 && p.sa % 4 == 0;
-        const bool vecB = aligned(p.B, 16) && p.ldb % 4 == 0 && p.sb % 4 == 0;
         hipLaunchKernelGGL(gemm32_kernel, dim3((unsigned)(tiles_m * tiles_n * p.batch)), dim3(256), 0, s,
                            (const float*)p.A, p.lda, p.sa, (const float*)p.B, p.ldb, p.sb, (float*)p.C, p.ldc, p.sc,
-                           p.M, p.N, p.K, tiles_m, tiles_m * tiles_n, vecA, vecB);
+                           p.M, p.N, p.K, tiles_m, tiles_m * tiles_n);
         set_variant("gemm32_128x128x16_mfma32x32x2");
         return launch_status();
     }

@@ -26,10 +26,16 @@
 // Workgroups are numbered so that the tiles resident on one XCD (ids congruent mod 8) form a
 // 4 x 8 block of tiles and share A row panels / B column panels in that XCD's L2.
 //
-// Requires M and K multiples of 8, K >= 256, 16-byte aligned operands.  Tiles that reach past M or N
-// re-read the last valid rows / chunks on the way in and clip their stores.  K is walked in whole
-// groups of four steps (128); in the last group the 16-byte chunks at k >= K are fetched from a
-// 16-byte block of zeros instead (both operands, so padding never meets a non-finite value).
+// Requires K >= 256.  Tiles that reach past M or N re-read the last valid rows / chunks on the way in and clip
+// their stores.  K is walked in whole groups of four steps (128); in the last group the 16-byte chunks at
+// k >= K are fetched from a 16-byte block of zeros instead (both operands, so padding never meets a non-finite value).
+// Rows need no alignment: the transfers take any element-aligned address (a dense matrix with an odd leading
+// dimension: 0.94-1.12 PFLOP/s at 4096^3 against 1.15 with aligned rows).  Sizes that are not multiples of 8:
+//   * K: the transfers cover the whole chunks of 8, k < Kd; the remaining 1 to 8 values of k are one more MFMA step
+//     whose fragments come straight from global memory into registers, element by element with zeros past the edges;
+//   * M: the chunk of A that straddles the end of a row reads on into the next row (its surplus only reaches rows of
+//     C that are never stored); so that no such read passes the end of the array, the last row of A is always
+//     left to the register-fed step (Kd <= K - 1 then).
 #include "gemm_direct.h"
 #include "shared_scratch.h"
 
@@ -163,7 +169,8 @@ template <typename E, typename OutT, int I, int J>
 __global__ __launch_bounds__(256) void gemm16_big(const unsigned short* __restrict__ A, int64_t lda, int64_t sa,
                                                   const unsigned short* __restrict__ B, int64_t ldb, int64_t sb,
                                                   OutT* __restrict__ C, int64_t ldc, int64_t sc, int M, int N, int K,
-                                                  int tiles_m, int tiles_n, int batch, int ksplit, int kchunk) {
+                                                  int tiles_m, int tiles_n, int batch, int ksplit, int kchunk, int kpeel) {
+    // K: the extent the transfers walk (a multiple of 8); kpeel: values of k behind it for the register-fed step
     constexpr int BTM = 64 * I, STAGE_A = BTM * BK, BTN = 64 * J, STAGE_B = BTN * BK;
     __shared__ __attribute__((aligned(1024))) unsigned short As0[STAGE_A], As1[STAGE_A], As2[STAGE_A], As3[STAGE_A];
     __shared__ __attribute__((aligned(1024))) unsigned short Bs0[STAGE_B], Bs1[STAGE_B], Bs2[STAGE_B], Bs3[STAGE_B];
@@ -208,12 +215,12 @@ __global__ __launch_bounds__(256) void gemm16_big(const unsigned short* __restri
             }
         }
         // A transfer: lane -> row lane/(8*I) of its block of 8/I rows, LDS position lane%(8*I); rows
-        // k = 8/I*blk + lane/(8*I).  Chunks of 8 m past the edge re-read the last whole chunk (M is a multiple of 8).
+        // k = 8/I*blk + lane/(8*I).  Chunks of 8 m that start past the edge re-read the last chunk that starts inside.
         const int ka = 8 / I * wave + lane / (8 * I);
         ln.kA = ka;
         ln.kB = 8 * ((lane & 3) ^ ((lane >> 4) & 3));
         int ca = (lane % (8 * I)) ^ (4 * (ka & 3));
-        if (bm * BTM + 8 * ca + 8 > M) ca = (M - bm * BTM) / 8 - 1;
+        if (bm * BTM + 8 * ca >= M) ca = (M - 1 - bm * BTM) / 8;
         ln.goffA = (unsigned)(((int64_t)(lane / (8 * I)) * lda + 8 * ca) * 2);
 #pragma unroll
         for (int ks = 0; ks < 2; ++ks) {
@@ -280,6 +287,28 @@ __global__ __launch_bounds__(256) void gemm16_big(const unsigned short* __restri
     KSTEP(3, 0, 2, false, false, 0, true, false, s + 3);
 #undef KSTEP
 
+    if (kpeel > 0) {   // (same for the whole grid)
+        // k = K .. K + kpeel - 1 as the first values of one 16-wide MFMA step: the lower half-wave holds k 0..7 of its
+        // row of B / column of A, the upper half-wave zeros.
+        const unsigned short* Ap = A + (int64_t)bz * sa + (int64_t)K * lda;
+        const unsigned short* Bp = B + (int64_t)bz * sb + K;
+        Frag fp;
+        const bool lower = lane < 32;
+#pragma unroll
+        for (int j = 0; j < J; ++j) {
+            const int64_t n = (int64_t)bn * BTN + wn + 32 * j + (lane & 31);
+#pragma unroll
+            for (int q = 0; q < 8; ++q) fp.b[j][q] = lower && q < kpeel && n < N ? (short)Bp[n * ldb + q] : (short)0;
+        }
+#pragma unroll
+        for (int i = 0; i < I; ++i) {
+            const int64_t m = (int64_t)bm * BTM + wm + 32 * i + (lane & 31);
+#pragma unroll
+            for (int q = 0; q < 8; ++q) fp.a[i][q] = lower && q < kpeel && m < M ? (short)Ap[m + (int64_t)q * lda] : (short)0;
+        }
+        mma16<E, I, J>(fp, acc);
+    }
+
     // Epilogue.  The lane's own offset (m within the wave tile, plus its 4*hb rows of n) is a
     // 32-bit element offset; the part of n that is uniform across the wave goes into the base.
     const unsigned lane_off = (unsigned)((lane & 31) + (int64_t)(4 * (lane >> 5)) * ldc);
@@ -315,12 +344,16 @@ __global__ __launch_bounds__(256) void gemm16_big(const unsigned short* __restri
     }
 }
 
+// The extent of K that the transfers walk: whole chunks of 8, and not the last row of A when a chunk of A can straddle
+// the end of a row (M not a multiple of 8).
+int dma_extent(const Problem& p) { return p.M % 8 ? (p.K - 1) / 8 * 8 : p.K / 8 * 8; }
+
 template <typename E, typename OutT, int I, int J>
 void launch(const Problem& p, hipStream_t s) {
     const int tiles_m = (p.M + 64 * I - 1) / (64 * I), tiles_n = (p.N + 64 * J - 1) / (64 * J);
     hipLaunchKernelGGL((gemm16_big<E, OutT, I, J>), dim3((unsigned)(tiles_m * tiles_n * p.batch)), dim3(256), 0,
                        s, (const unsigned short*)p.A, p.lda, p.sa, (const unsigned short*)p.B, p.ldb, p.sb,
-                       (OutT*)p.C, p.ldc, p.sc, p.M, p.N, p.K, tiles_m, tiles_n, p.batch, 1, 0);
+                       (OutT*)p.C, p.ldc, p.sc, p.M, p.N, dma_extent(p), tiles_m, tiles_n, p.batch, 1, 0, p.K - dma_extent(p));
 }
 
 // ---- split over K for problems with few tiles and a long K ---------------------------------------------------
@@ -369,7 +402,7 @@ SharedScratch g_split[16];
 // Parts and part length for the problem, or 0 if a split does not apply.
 int pick_split(const Problem& p, int* kchunk) {
     static const int force = [] { const char* e = getenv("MI_GEMM_SPLITK"); return e ? atoi(e) : -1; }();   // 0 = never, n = n parts
-    if (force == 0) return 0;
+    if (force == 0 || p.M % 8 || p.K % 8) return 0;   // (the parts and the kernel that adds them move whole vectors)
     const int64_t tiles = tiles_of(p, 128, 128);
     // (up to half a tile per CU: 2048 x 768 x 8192, 96 tiles, 59 -> 41 us with two parts; 1152 x 1024 x 16384 107 -> 55 us
     // with three; beyond 128 tiles the estimate below never favours a split)
@@ -404,7 +437,7 @@ bool launch_split(const Problem& p, hipStream_t s, int parts, int kchunk) {
     const int64_t MN = (int64_t)p.M * p.N;
     hipLaunchKernelGGL((gemm16_big<E, float, 2, 2>), dim3((unsigned)(tiles_m * tiles_n * p.batch * parts)), dim3(256), 0, s,
                        (const unsigned short*)p.A, p.lda, p.sa, (const unsigned short*)p.B, p.ldb, p.sb, scratch,
-                       (int64_t)p.M, MN, p.M, p.N, p.K, tiles_m, tiles_n, p.batch, parts, kchunk);
+                       (int64_t)p.M, MN, p.M, p.N, p.K, tiles_m, tiles_n, p.batch, parts, kchunk, 0);
     const int64_t quads = MN / 4 * p.batch;
     const unsigned blocks = (unsigned)((quads + 255) / 256 < 2048 ? (quads + 255) / 256 : 2048);
     if (p.out_dtype == MI_F32)
@@ -423,11 +456,9 @@ namespace gemm {
 
 bool big16_applicable(const Problem& p) {
     if (p.in_dtype != MI_F16 && p.in_dtype != MI_BF16) return false;
-    // M and K multiples of 8 (A and B move in 16-byte chunks along m and k), any N
     const int64_t tiles = tiles_of(p, 128, 128);   // (from 16 tiles of 128x128 on, this kernel is no slower than 64x64 tiles)
     int split = 0, kchunk = 0;
-    return p.M % 8 == 0 && p.M >= 8 && p.N >= 1 && p.K % 8 == 0 && p.K >= 256 && aligned(p.A, 16) && aligned(p.B, 16) &&
-           p.lda % 8 == 0 && p.ldb % 8 == 0 && p.sa % 8 == 0 && p.sb % 8 == 0 && p.ldc < (1 << 26) &&
+    return p.M >= 8 && p.N >= 1 && p.K >= 256 + 8 * (p.K % 8 != 0 || p.M % 8 != 0) && p.ldc < (1 << 26) &&
            // (the kernel's 32-bit lane offsets assume rows that follow each other upwards in memory)
            p.lda >= p.M && p.ldb >= p.K && p.ldc >= p.M && p.sa >= 0 && p.sb >= 0 && p.sc >= 0 &&
            p.lda < (1 << 26) && p.ldb < (1 << 26) && tiles < (1 << 30) &&

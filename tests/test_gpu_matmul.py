@@ -67,11 +67,11 @@ def test_matmul_integer_valued_inputs_are_exact(ct, orc):
         assert np.array_equal(orc.to_julia(C), A @ B)
 
 
-@pytest.mark.parametrize("M,N,K,T,out32", [(1504, 1544, 200, torch.float16, True), (1500, 1540, 333, torch.float16, False),
+@pytest.mark.parametrize("M,N,K,T,out32", [(1504, 1544, 200, torch.float16, True), (1500, 1540, 233, torch.float16, False),
                                            (2048, 1100, 96, torch.bfloat16, True), (1536, 1536, 32, torch.float16, True)])
 def test_matmul_mid_tile_kernel_exact(ct, orc, M, N, K, T, out32):
-    """The register-staged 128x128 kernel (shapes the direct-to-LDS kernel does not take: rows that are not
-    16-byte aligned or K below 256; enough tiles to fill half the chip):
+    """The register-staged 128x128 kernel (shapes the direct-to-LDS kernel does not take: K below 256; enough
+    tiles to fill half the chip):
     aligned interior tiles without predicates, ragged edges in M, N and K, rows that are not 16-byte
     aligned (M = 1500), one and many K steps.  Integer-valued operands make every sum exact, so any
     mistake in the tile mapping, the register look-ahead or the fragment reads changes the result."""
@@ -81,7 +81,7 @@ def test_matmul_mid_tile_kernel_exact(ct, orc, M, N, K, T, out32):
     C = torch.empty((N, M), dtype=torch.float32 if out32 else T, device="cuda")
     ct.matmul_kernel(At, Bt, C, 128, 128, 32)
     assert ct.last_variant() == "gemm16_mid_128x128x32"
-    assert np.array_equal(orc.to_julia(C.float()), A @ B)      # (random sums of 333 terms stay far below 2048: exact in f16 too)
+    assert np.array_equal(orc.to_julia(C.float()), A @ B)      # (random sums of 233 terms stay far below 2048: exact in f16 too)
 
 
 @pytest.mark.parametrize("M,N,K,T,out32,tile", [(2048, 2048, 256, torch.float16, True, "128x128"), (2048, 2048, 384, torch.float16, False, "128x128"),
@@ -105,6 +105,49 @@ def test_matmul_large_tile_kernel_exact(ct, orc, M, N, K, T, out32, tile):
     ref = A @ B
     assert out32 or np.abs(ref).max() <= 256  # integers up to 256 are exact in bf16's 8 bits as well
     assert np.array_equal(orc.to_julia(C).astype(np.float32), ref)
+
+
+@pytest.mark.parametrize("M,N,K,T,out32,pad", [
+    (1500, 1540, 333, torch.float16, False, (0, 0)),     # dense, everything ragged: rows of A 4-byte, of B 2-byte aligned
+    (4095, 520, 271, torch.float16, True, (0, 0)),       # odd M: the straddling chunk of A; K - Kd = 7
+    (1501, 1536, 512, torch.bfloat16, True, (0, 0)),     # K a multiple of 8 with odd M: the last 8 rows of A go by registers
+    (1536, 1500, 517, torch.float16, False, (0, 0)),     # M a multiple of 8, K not: B rows misaligned, K - Kd = 5
+    (2048, 2048, 264, torch.float16, True, (3, 5)),      # aligned sizes inside parents with odd leading dimensions
+    (1001, 1003, 1025, torch.bfloat16, False, (1, 2)),
+    (4100, 4097, 265, torch.float16, True, (0, 0)),      # 256 x 128 tiles
+])
+def test_matmul_large_tile_kernel_takes_misaligned_rows_and_ragged_sizes(ct, orc, M, N, K, T, out32, pad):
+    """The direct-to-LDS kernel on rows that are not 16-byte aligned and on M / K that are not multiples of 8 (the K
+    tail and, with a ragged M, the last rows of A are one register-fed MFMA step).  Exact integer sums.  The operands
+    are views: the cells right behind every row of A and B and behind the arrays hold NaN, so a value taken from
+    past an edge shows; C is a view of a buffer filled with a sentinel."""
+    rng = np.random.default_rng(M + K)
+    A = rng.integers(-1, 2, (M, K)).astype(np.float32); B = rng.integers(-2, 3, (K, N)).astype(np.float32)
+    lda, ldb = M + pad[0], K + pad[1]
+    Aflat = torch.full((K * lda + 16,), float("nan"), dtype=T, device="cuda")
+    Bflat = torch.full((N * ldb + 16,), float("nan"), dtype=T, device="cuda")
+    Av = Aflat[:K * lda].view(K, lda)[:, :M]; Bv = Bflat[:N * ldb].view(N, ldb)[:, :K]
+    Av.copy_(orc.from_julia(A).to(T)); Bv.copy_(orc.from_julia(B).to(T))
+    buf = torch.full((N + 2, M + 9), -77.0, dtype=torch.float32 if out32 else T, device="cuda")
+    C = buf[:N, :M]
+    ct.matmul_kernel(Av, Bv, C, 64, 64, 64)
+    assert ct.last_variant().startswith("gemm16_big_") and "splitk" not in ct.last_variant(), ct.last_variant()
+    ref = A @ B
+    assert out32 or np.abs(ref).max() <= (2048 if T == torch.float16 else 256)
+    assert np.array_equal(orc.to_julia(C.contiguous()).astype(np.float32), ref)
+    assert bool((buf[N:] == -77.0).all()) and bool((buf[:, M:] == -77.0).all())
+
+
+def test_batch_matmul_large_tile_kernel_ragged(ct, orc):
+    """The same through mi_batch_matmul_kernel: three dense 1023 x 1030 x 515 products."""
+    rng = np.random.default_rng(11)
+    M, N, K, nb = 1023, 1030, 515, 3
+    A = rng.integers(-1, 2, (M, K, nb)).astype(np.float32); B = rng.integers(-2, 3, (K, N, nb)).astype(np.float32)
+    At = orc.from_julia(A).to(torch.float16).cuda(); Bt = orc.from_julia(B).to(torch.float16).cuda()
+    C = torch.empty((nb, N, M), dtype=torch.float32, device="cuda")
+    ct.batch_matmul_kernel(At, Bt, C, 64, 64, 64)
+    assert ct.last_variant().startswith("gemm16_big_"), ct.last_variant()
+    assert np.array_equal(orc.to_julia(C), np.einsum("mkb,knb->mnb", A, B))
 
 
 @pytest.mark.parametrize("M,N,K,T,out32", [(512, 512, 4096, torch.float16, True), (512, 512, 4096, torch.bfloat16, False),

@@ -10,8 +10,8 @@
 //                  v_mfma_f32_32x32x64_f8f6f4 (K = 64 per instruction, the 5 PFLOP/s rate), K walked in
 //                  steps of 64 bytes through a ring of four 32 KB LDS stages filled by direct
 //                  global->LDS transfers: the data movement of the 16-bit kernel (gemm_big.hip) at one
-//                  byte per element, so a stage carries twice the K.  M and K multiples of 16,
-//                  K >= 512, 16-byte aligned operands.
+//                  byte per element, so a stage carries twice the K.  K >= 512; rows of any alignment, and
+//                  sizes that are not multiples of 16 as in gemm_big.hip (register-fed last K step).
 //   gemm8_generic  64x64 tile, register staged, v_mfma_f32_32x32x16_fp8_fp8: any shape / stride.
 //
 // Operand order inside a K step.  A dot product does not depend on the order of its terms, so the
@@ -241,7 +241,8 @@ template <int FMT, int OD>
 __global__ __launch_bounds__(256) void gemm8_big(const u8* __restrict__ A, int64_t lda, int64_t sa,
                                                  const u8* __restrict__ B, int64_t ldb, int64_t sb,
                                                  typename Out<OD>::T* __restrict__ C, int64_t ldc, int64_t sc, int M,
-                                                 int N, int K, int tiles_m, int tiles_n, int batch) {
+                                                 int N, int K, int tiles_m, int tiles_n, int batch, int kpeel) {
+    // K: the extent the transfers walk (a multiple of 16); kpeel: values of k behind it for the register-fed step
     using OutT = typename Out<OD>::T;
     __shared__ __attribute__((aligned(1024))) u8 As0[STAGE8], As1[STAGE8], As2[STAGE8], As3[STAGE8];
     __shared__ __attribute__((aligned(1024))) u8 Bs0[STAGE8], Bs1[STAGE8], Bs2[STAGE8], Bs3[STAGE8];
@@ -276,11 +277,11 @@ __global__ __launch_bounds__(256) void gemm8_big(const u8* __restrict__ A, int64
         }
         ln.kB = 16 * cb;
         // A transfer: 4 rows of k x 256 bytes; lane -> row lane/16, LDS position lane%16.  Chunks of 16 m
-        // past the edge re-read the last whole chunk (M is a multiple of 16).
+        // that start past the edge re-read the last chunk that starts inside.
         const int ka = 4 * wave + (lane >> 4);
         ln.kA = ka;
         int ca = (lane & 15) ^ (2 * (ka & 7));
-        if (bm * BT8 + 16 * ca + 16 > M) ca = (M - bm * BT8) / 16 - 1;
+        if (bm * BT8 + 16 * ca >= M) ca = (M - 1 - bm * BT8) / 16;
         ln.goffA = (unsigned)((int64_t)(lane >> 4) * lda + 16 * ca);
 #pragma unroll
         for (int t = 0; t < 2; ++t) {
@@ -345,6 +346,36 @@ __global__ __launch_bounds__(256) void gemm8_big(const u8* __restrict__ A, int64
     KSTEP(3, 0, 2, f1, f0, false, false, 0, true, false, s + 3);
 #undef KSTEP
 
+    if (kpeel > 0) {   // (same for the whole grid)
+        // k = K .. K + kpeel - 1 as the first values of one 64-wide MFMA step: the lower half-wave holds k 0..31 of its
+        // row of B / column of A (here: up to 16 values, then zeros), the upper half-wave zeros.
+        const u8* Ap = A + (int64_t)bz * sa + (int64_t)K * lda;
+        const u8* Bp = B + (int64_t)bz * sb + K;
+        const bool lower = lane < 32;
+        auto gather = [&](const u8* p, int64_t step, bool live) {
+            i32x8 v = {0, 0, 0, 0, 0, 0, 0, 0};
+#pragma unroll
+            for (int q = 0; q < 16; ++q) {
+                const unsigned byte = live && q < kpeel ? p[q * step] : 0u;
+                v[q >> 2] |= (int)(byte << (8 * (q & 3)));
+            }
+            return v;
+        };
+        i32x8 pa[4], pb[4];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const int64_t n = (int64_t)bn * BT8 + wn + 32 * j + (lane & 31);
+            pb[j] = gather(Bp + (n < N ? n : 0) * ldb, 1, lower && n < N);
+        }
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int64_t m = (int64_t)bm * BT8 + wm + 32 * i + (lane & 31);
+            pa[i] = gather(Ap + (m < M ? m : 0), lda, lower && m < M);
+        }
+        mma8<FMT, 0>(pa, pb, acc);
+        mma8<FMT, 2>(pa, pb, acc);
+    }
+
     // Epilogue: a half-wave holds 32 consecutive m of one column of C.
     const unsigned lane_off = (unsigned)((lane & 31) + (int64_t)(4 * (lane >> 5)) * ldc);
     OutT* Cw = C + (int64_t)bm * BT8 + wm + ((int64_t)bn * BT8 + wn) * ldc;
@@ -380,9 +411,12 @@ __global__ __launch_bounds__(256) void gemm8_big(const u8* __restrict__ A, int64
 template <int FMT, int OD>
 void launch_big(const Problem& p, hipStream_t s) {
     const int tiles_m = (p.M + BT8 - 1) / BT8, tiles_n = (p.N + BT8 - 1) / BT8;
+    // The extent of K that the transfers walk: whole chunks of 16, and not the last row of A when a chunk of A can
+    // straddle the end of a row (M not a multiple of 16: the chunk then reads on into the next row, which must exist).
+    const int kd = p.M % 16 ? (p.K - 1) / 16 * 16 : p.K / 16 * 16;
     hipLaunchKernelGGL((gemm8_big<FMT, OD>), dim3((unsigned)(tiles_m * tiles_n * p.batch)), dim3(256), 0, s,
                        (const u8*)p.A, p.lda, p.sa, (const u8*)p.B, p.ldb, p.sb, (typename Out<OD>::T*)p.C, p.ldc,
-                       p.sc, p.M, p.N, p.K, tiles_m, tiles_n, p.batch);
+                       p.sc, p.M, p.N, kd, tiles_m, tiles_n, p.batch, p.K - kd);
 }
 
 template <int FMT, int OD>
@@ -405,10 +439,9 @@ void dispatch(const Problem& p, hipStream_t s, bool big) {
 }
 
 bool big8_applicable(const Problem& p) {
-    // M and K multiples of 16 (A and B move in 16-byte chunks along m and k), any N; enough tiles
-    // of 256 x 256 to give every XCD work.
-    return p.M % 16 == 0 && p.M >= 16 && p.N >= 1 && p.K % 16 == 0 && p.K >= 512 && aligned(p.A, 16) &&
-           aligned(p.B, 16) && p.lda % 16 == 0 && p.ldb % 16 == 0 && p.sa % 16 == 0 && p.sb % 16 == 0 &&
+    // Any alignment of the rows, any M, N and K from 512 on (sizes that are not multiples of 16: the K tail, and with a
+    // ragged M the last rows of A, are one register-fed MFMA step); enough tiles of 256 x 256 to give every XCD work.
+    return p.M >= 16 && p.N >= 1 && p.K >= 512 + 16 * (p.M % 16 != 0 || p.K % 16 != 0) &&
            p.lda >= p.M && p.ldb >= p.K && p.ldc >= p.M && p.sa >= 0 && p.sb >= 0 && p.sc >= 0 &&
            p.ldc < (1 << 26) && p.lda < (1 << 27) && p.ldb < (1 << 27) && tiles_of(p, BT8, BT8) >= 8 &&
            tiles_of(p, BT8, BT8) < (1 << 30);

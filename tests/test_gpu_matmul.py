@@ -451,6 +451,30 @@ def test_matmul_fp8_direct_to_lds_kernel_exact(ct, orc, M, N, K, fmt, out):
     assert bool((buf[N:] == -77.0).all()) and bool((buf[:, M:] == -77.0).all())
 
 
+@pytest.mark.parametrize("M,N,K,fmt,out", [(4095, 2100, 529, "e4m3fn", torch.float32), (2049, 2049, 1031, "e5m2", torch.float16),
+                                           (2051, 2048, 1024, "e4m3fn", torch.bfloat16), (2048, 2047, 1025, "e5m2", torch.float32),
+                                           (2048, 2048, 528, "e4m3fn", torch.float32)])
+def test_matmul_fp8_direct_to_lds_kernel_takes_misaligned_rows_and_ragged_sizes(ct, orc, M, N, K, fmt, out):
+    """The fp8 direct-to-LDS kernel on rows that start at odd byte offsets (views at offsets 1 and 3 inside wider buffers) and
+    on M / K that are not multiples of 16: the K tail and, with a ragged M, the last rows of A are one register-fed
+    MFMA step.  Every cell outside the operands holds a NaN code; exact sums; C inside a buffer of sentinels."""
+    rng = np.random.default_rng(M * 3 + K)
+    A = rng.integers(-2, 3, (M, K)) / 2.0; B = rng.integers(-2, 3, (K, N)) / 2.0
+    At, Ac = fp8_tensor(orc, A, fmt); Bt, Bc = fp8_tensor(orc, B, fmt)
+    nan = torch.full((1,), float("nan")).to(FP8[fmt]).view(torch.uint8).item()
+    Abuf = torch.full((K + 3, M + 5), nan, dtype=torch.uint8, device="cuda")
+    Bbuf = torch.full((N + 2, K + 7), nan, dtype=torch.uint8, device="cuda")
+    Abuf[:K, 1:1 + M] = At.view(torch.uint8); Bbuf[:N, 3:3 + K] = Bt.view(torch.uint8)
+    buf = torch.full((N + 3, M + 9), -77.0, dtype=out, device="cuda")
+    C = buf[:N, :M]
+    ct.matmul_kernel(Abuf.view(FP8[fmt])[:K, 1:1 + M], Bbuf.view(FP8[fmt])[:N, 3:3 + K], C, 64, 64, 64)
+    assert ct.last_variant() == "gemm8_big_256x256x64_ring4"
+    ref = orc.fp8_matmul(Ac, Bc, fmt)
+    want = orc.to_julia(orc.from_julia(ref.astype(np.float32)).to(out).float())
+    assert np.array_equal(orc.to_julia(C.contiguous().float()), want)
+    assert bool((buf[N:] == -77.0).all()) and bool((buf[:, M:] == -77.0).all())
+
+
 def test_matmul_fp8_direct_to_lds_kernel_shape_sweep(ct, orc):
     """Sixteen seeded shapes with M, K multiples of 16 (K >= 512) and any N on the fp8 direct-to-LDS
     kernel; exact sums."""

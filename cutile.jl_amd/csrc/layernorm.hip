@@ -524,6 +524,137 @@ __global__ __launch_bounds__(BLOCK * RG) void ln_bwd_rg_kernel(float* __restrict
     }
 }
 
+// Backward for rows of 8192 to 16384 elements (16-byte aligned): 1024 lanes, four vectors of every array per lane.
+// W, dW, dB and the row at hand are 80 registers of a lane's 128; a second row in registers for look-ahead does not
+// fit (it spilled), and without look-ahead the kernel ran at 3.1-3.5 TB/s.  The row in flight therefore lands in LDS:
+// every lane requests its own four vectors of X and of dY with global->LDS transfers (no staging registers), copies
+// them to registers once they have landed, and at once requests the next row into the same places.  A lane reads back
+// only what its own wave's transfers wrote, so the prefetch needs no barrier; the two barriers of a trip belong to the
+// row sums, and they wait for LDS accesses only, so the transfers stay in flight across them.  128 KB of LDS: one
+// workgroup per CU with a whole row (128 KB) in flight.
+// Workgroup (g, s) walks the rows m = g + G*s, stepping by G*S, of partial slot g.
+constexpr int kWideLanes = 1024, kWideVpt = 4, kWideFloats = kWideLanes * kWideVpt * 4;
+__global__ __launch_bounds__(kWideLanes) void ln_bwd_wide_kernel(float* __restrict__ DX, int64_t lddx,
+                                                                 const float* __restrict__ DY, int64_t lddy,
+                                                                 float* __restrict__ DW, int64_t lddw,
+                                                                 float* __restrict__ DB, int64_t lddb,
+                                                                 const float* __restrict__ X, int64_t ldx,
+                                                                 const float* __restrict__ W,
+                                                                 const float* __restrict__ Mean,
+                                                                 const float* __restrict__ Rstd, int N,
+                                                                 int64_t M, int G, int S) {
+    constexpr int NW = kWideLanes / 64, VPT = kWideVpt;
+    __shared__ __attribute__((aligned(1024))) float xs[kWideFloats], ys[kWideFloats];
+    __shared__ float red[2][2 * NW];   // (two sets: a trip's sums are read while the next trip's are not yet written)
+    const int g = blockIdx.x % G, s = blockIdx.x / G;
+    const int lt = threadIdx.x, lane = lt & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(lt >> 6);
+    auto vec = [&](int v) { return (lt + v * kWideLanes) * 4; };
+    float w[VPT][4], dw[VPT][4], db[VPT][4];
+#pragma unroll
+    for (int v = 0; v < VPT; ++v) {
+        const f32x4 t = vec(v) < N ? *reinterpret_cast<const f32x4*>(W + vec(v)) : f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+            w[v][q] = t[q];
+            dw[v][q] = db[v][q] = 0.f;
+        }
+    }
+    // (unpredicated: a vector past the end of the row re-reads the row's last vector and is discarded where it is used)
+    auto request = [&](int64_t m) {
+#pragma unroll
+        for (int v = 0; v < VPT; ++v) {
+            const int col = vec(v) < N ? vec(v) : N - 4;   // N % 4 == 0 here
+            __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(X + m * ldx + col),
+                                             (__attribute__((address_space(3))) void*)(xs + (wave * 64 + v * kWideLanes) * 4), 16, 0, 0);
+            __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(DY + m * lddy + col),
+                                             (__attribute__((address_space(3))) void*)(ys + (wave * 64 + v * kWideLanes) * 4), 16, 0, 0);
+        }
+    };
+    const int64_t step = (int64_t)G * S, m0 = g + (int64_t)G * s;
+    if (m0 < M) request(m0);
+    int set = 0;
+    for (int64_t m = m0; m < M; m += step) {
+        const float mean = Mean[m], rstd = Rstd[m];
+        // this wave's transfers (and the previous trip's stores) are done: vmcnt(0); expcnt and lgkmcnt untouched
+        __builtin_amdgcn_s_waitcnt(0x0f70);
+        asm volatile("" ::: "memory");
+        float x[VPT][4], dy[VPT][4];
+#pragma unroll
+        for (int v = 0; v < VPT; ++v) {
+            const f32x4 tx = *reinterpret_cast<const f32x4*>(xs + vec(v)), ty = *reinterpret_cast<const f32x4*>(ys + vec(v));
+            const bool in = vec(v) < N;
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                x[v][q] = tx[q];
+                dy[v][q] = in ? ty[q] : 0.f;
+            }
+        }
+        // the copies have left LDS before the next row is asked into their places
+        __builtin_amdgcn_s_waitcnt(0xc07f);
+        asm volatile("" ::: "memory");
+        if (m + step < M) request(m + step);
+        float c1 = 0.f, c2 = 0.f;
+#pragma unroll
+        for (int v = 0; v < VPT; ++v) {
+            const bool in = vec(v) < N;
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                const float xhat = in ? (x[v][q] - mean) * rstd : 0.f;
+                const float wdy = w[v][q] * dy[v][q];
+                x[v][q] = xhat;
+                c1 += xhat * wdy;
+                c2 += wdy;
+            }
+        }
+        c1 = wave_reduce(c1, SumOp{});
+        c2 = wave_reduce(c2, SumOp{});
+        if (lane == 0) {
+            red[set][wave] = c1;
+            red[set][NW + wave] = c2;
+        }
+        lds_barrier();
+        c1 = c2 = 0.f;
+#pragma unroll
+        for (int i = 0; i < NW; i += 4) {
+            c1 += (red[set][i] + red[set][i + 1]) + (red[set][i + 2] + red[set][i + 3]);
+            c2 += (red[set][NW + i] + red[set][NW + i + 1]) + (red[set][NW + i + 2] + red[set][NW + i + 3]);
+        }
+        set ^= 1;   // (the next trip writes the other set; the barrier of that trip keeps the one after it behind these reads)
+        c1 /= (float)N;
+        c2 /= (float)N;
+#pragma unroll
+        for (int v = 0; v < VPT; ++v) {
+            f32x4 t;
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                const float xhat = x[v][q], wdy = w[v][q] * dy[v][q];
+                dw[v][q] += dy[v][q] * xhat;
+                db[v][q] += dy[v][q];
+                t[q] = (wdy - (xhat * c1 + c2)) * rstd;
+            }
+            if (vec(v) < N) st_global<true>(t, reinterpret_cast<f32x4*>(DX + m * lddx + vec(v)));
+        }
+    }
+    // flush through LDS (the row buffer is free now) with coalesced atomics, as the other backward kernels do
+    float* dwp = DW + (int64_t)g * lddw;
+    float* dbp = DB + (int64_t)g * lddb;
+#pragma unroll
+    for (int pass = 0; pass < 2; ++pass) {
+        __syncthreads();
+#pragma unroll
+        for (int v = 0; v < VPT; ++v)
+#pragma unroll
+            for (int q = 0; q < 4; ++q) xs[vec(v) + q] = pass == 0 ? dw[v][q] : db[v][q];
+        __syncthreads();
+        float* dst = pass == 0 ? dwp : dbp;
+        for (int c = lt; c < N; c += kWideLanes) {
+            if (S == 1) dst[c] += xs[c];
+            else unsafeAtomicAdd(dst + c, xs[c]);
+        }
+    }
+}
+
 // Backward for rows longer than the register-cached variants hold.
 template <int BLOCK>
 __global__ __launch_bounds__(BLOCK) void ln_bwd_long_kernel(float* __restrict__ DX, int64_t lddx,
@@ -886,6 +1017,16 @@ extern "C" int mi_layer_norm_bwd_dx_partial_dwdb(
         else { RGS(512, 4, 1); set_variant("ln_bwd_regs_b512_v4_rg1"); }
 #undef RGS
 #undef RGK
+    } else if (al && vecs > 2048 && vecs <= kWideFloats / 4 && !one_group && G <= 256) {
+        // one workgroup of 1024 lanes per CU
+        int64_t Sw = cld((int64_t)256, (int64_t)G);
+        if (Sw > rows_per_slot) Sw = rows_per_slot;
+        if (Sw < 1) Sw = 1;
+        hipLaunchKernelGGL(ln_bwd_wide_kernel, dim3((unsigned)(G * Sw)), dim3(kWideLanes), 0, s, (float*)DX->ptr, DX->strides[1],
+                           (const float*)DY->ptr, DY->strides[1], (float*)DW->ptr, DW->strides[1], (float*)DB->ptr,
+                           DB->strides[1], (const float*)X->ptr, X->strides[1], (const float*)W->ptr,
+                           (const float*)Mean->ptr, (const float*)Rstd->ptr, (int)N, M, G, (int)Sw);
+        set_variant("ln_bwd_wide_b1024_v4_lds_lookahead");
     } else if (!al) launch_bwd<false, false>(ARGS);
     else if (stream_in) launch_bwd<true, true>(ARGS);
     else launch_bwd<true, false>(ARGS);

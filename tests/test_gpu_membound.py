@@ -350,6 +350,23 @@ def test_layernorm_fwd_bwd(orc, M, N, TILE_N, G):
         assert orc.isapprox(ref, orc.to_julia(got), rtol=1e-2)
 
 
+@pytest.mark.parametrize("M,N,G", [(300, 12288, 64), (37, 8196, 8), (70, 10240, 256), (3, 16380, 2), (1, 16384, 1), (513, 16384, 64)])
+def test_layernorm_bwd_wide_rows(ct, orc, M, N, G):
+    """Rows of 8192 to 16384 elements: the backward kernel whose row in flight lands in LDS (one, several and more
+    workgroups than rows per partial slot; rows that fill 1024 lanes x 4 vectors and rows that leave lanes idle)."""
+    d = layernorm.prepare(M=M, N=N, GROUP_SIZE_M=G)
+    ct.layer_norm_fwd(d.X, d.W, d.B, d.Y, d.Mean, d.Rstd, d.eps, 1024)
+    d.partials.zero_()
+    ct.layer_norm_bwd_dx_partial_dwdb(d.DX, d.DY, d.DW_partial, d.DB_partial, d.X, d.W, d.Mean, d.Rstd, d.Locks, G, 1024)
+    assert ct.last_variant() == "ln_bwd_wide_b1024_v4_lds_lookahead"
+    ct.layer_norm_bwd_dwdb(d.DW_partial, d.DB_partial, d.FINAL_DW, d.FINAL_DB, 32, 1024)
+    X, W, DY = (orc.to_julia(t) for t in (d.X, d.W, d.DY))
+    DX, DW, DB = orc.layer_norm_bwd(X, W, DY, d.eps)
+    close_f32(orc.to_julia(d.DX), DX)
+    close_f32(orc.to_julia(d.FINAL_DW), DW)
+    close_f32(orc.to_julia(d.FINAL_DB), DB)
+
+
 @pytest.mark.parametrize("M,N,variant", [(9, 65536, "ln_fwd_3pass_b1024_v4"), (5, 100003, "ln_fwd_3pass_b1024"),
                                          (1030, 16388, "ln_fwd_3pass_b256_v4"), (1025, 16387, "ln_fwd_3pass_b256")])
 def test_layernorm_fwd_rows_too_long_for_registers(ct, orc, M, N, variant):

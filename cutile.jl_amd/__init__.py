@@ -84,6 +84,7 @@ _SIGNATURES = {
     "mi_silu_and_mul_kernel": ([_A, _A, _A, _i, _vp], _i),
     "mi_moe_sum_topk": ([_A, _A, _vp], _i),
     "mi_quantize_e4m3fn": ([_A, _A, _A, _A, _vp], _i),
+    "mi_quantize_e4m3fn_fold": ([_A, _A, _A, _A, _A, _A, _vp], _i),
     "mi_tiled_broadcast": ([_A, ctypes.c_char_p, ctypes.POINTER(_A), _i, _vp, _i, _vp], _i),
     "mi_tiled_broadcast_eltype": ([ctypes.c_char_p, ctypes.POINTER(ctypes.c_int32), _i,
                                    ctypes.POINTER(ctypes.c_int32), _i, ctypes.POINTER(ctypes.c_int32)], _i),
@@ -393,9 +394,10 @@ def silu_and_mul_kernel(A, B, C, TILE_N: int, stream=None):
     _call("mi_silu_and_mul_kernel", _ref(A), _ref(B), _ref(C), TILE_N, _stream(stream))
 
 
-def quantize_e4m3fn(x, codes=None, scale=None, workspace=None, stream=None):
+def quantize_e4m3fn(x, codes=None, scale=None, workspace=None, stream=None, fold=None, fold_out=None):
     """Per-tensor E4M3FN codes of a 16-bit activation matrix (torch (columns, K)) and their scale (a 1-element fp32
-    device tensor): the fp8 operand of ``fused_moe_kernel`` with fp8 weights.  Returns (codes, scale)."""
+    device tensor): the fp8 operand of ``fused_moe_kernel`` with fp8 weights.  Returns (codes, scale), or with
+    ``fold`` (a dense fp32 tensor, e.g. the weights' scales) (codes, scale, fold * scale) from the same two launches."""
     import torch
     if codes is None:
         codes = torch.empty(x.shape, dtype=torch.float8_e4m3fn, device=x.device)
@@ -403,6 +405,12 @@ def quantize_e4m3fn(x, codes=None, scale=None, workspace=None, stream=None):
         scale = torch.empty(1, dtype=torch.float32, device=x.device)
     if workspace is None:
         workspace = torch.empty(1024, dtype=torch.float32, device=x.device)
+    if fold is not None:
+        if fold_out is None:
+            fold_out = torch.empty_like(fold)
+        _call("mi_quantize_e4m3fn_fold", _ref(x), _ref(codes), _ref(scale), _ref(workspace), _ref(fold), _ref(fold_out),
+              _stream(stream))
+        return codes, scale, fold_out
     _call("mi_quantize_e4m3fn", _ref(x), _ref(codes), _ref(scale), _ref(workspace), _stream(stream))
     return codes, scale
 

@@ -756,7 +756,8 @@ constexpr int kAlignThreads = 1024, kAlignWaves = kAlignThreads / 64;
 constexpr int kAlignBatch = 8;            // chunks of 64 replicas whose ids a lane requests together: one memory round trip per batch
 constexpr int kAlignMaxWgs = 64;
 constexpr int kAlignPairs = 16384;        // (workgroup, expert) pairs of the two-launch sort
-constexpr int kAlignOneWgReplicas = 8192; // up to here one launch of one workgroup is as fast (10 us either way at 8192)
+constexpr int kAlignOneWgReplicas = 8191; // up to here one launch of one workgroup is the faster sort (8192: 10 us either way, and the
+                                          // workgroups that clear an array on the way have the two launches to hide in)
 // counts [kAlignPairs] | first slot inside the expert [kAlignPairs] | first slot of the expert [kAlignMaxExperts] | ticket
 constexpr int kAlignScratchInts = 2 * kAlignPairs + kAlignMaxExperts + 64;
 static __device__ __align__(256) int moe_align_scratch[kAlignScratchInts];

@@ -40,13 +40,19 @@ template <bool BF16>
 __global__ __launch_bounds__(kQThreads) void quantize_kernel(const unsigned short* __restrict__ x, int64_t ld, int64_t n,
                                                              int64_t rows, unsigned char* __restrict__ q, int64_t ldq,
                                                              const float* __restrict__ partial, int groups,
-                                                             float* __restrict__ scale_out) {
+                                                             float* __restrict__ scale_out,
+                                                             const float* __restrict__ fold_in, float* __restrict__ fold_out,
+                                                             int64_t nfold) {
     __shared__ float red[kQThreads / 64];
     float m = 0.f;
     for (int g = threadIdx.x; g < groups; g += kQThreads) m = fmaxf(m, partial[g]);
     m = block_reduce<kQThreads / 64>(m, red, MaxOp{}, 0.f);
     const float scale = m > 0.f ? m / 448.0f : 1.0f;
     if (blockIdx.x == 0 && threadIdx.x == 0) *scale_out = scale;
+    // the scale folded into an array of the caller's on the way (the weights' per-channel scales of the GEMM that
+    // takes these codes: one multiply there instead of two, and no launch for the product)
+    for (int64_t i = (int64_t)blockIdx.x * kQThreads + threadIdx.x; i < nfold; i += (int64_t)gridDim.x * kQThreads)
+        fold_out[i] = fold_in[i] * scale;
     const int64_t vec_per_row = n / 8, total = vec_per_row * rows;
     for (int64_t i = (int64_t)blockIdx.x * kQThreads + threadIdx.x; i < total; i += (int64_t)gridDim.x * kQThreads) {
         const int64_t r = i / vec_per_row, c = i - r * vec_per_row;
@@ -67,8 +73,21 @@ __global__ __launch_bounds__(kQThreads) void quantize_kernel(const unsigned shor
 
 }  // namespace
 
-extern "C" int mi_quantize_e4m3fn(const mi_tile_array* x, const mi_tile_array* codes, const mi_tile_array* scale,
-                                  const mi_tile_array* workspace, void* stream) {
+static int dense_f32(const mi_tile_array* a, int64_t* n) {
+    MI_CHECK(check_array(a, a->ndim));
+    if (a->dtype != MI_F32) return MI_E_DTYPE;
+    int64_t run = 1;
+    for (int d = 0; d < a->ndim; ++d) {
+        if (a->sizes[d] > 1 && a->strides[d] != run) return MI_E_STRIDE;
+        run *= a->sizes[d];
+    }
+    *n = run;
+    return MI_OK;
+}
+
+static int quantize_impl(const mi_tile_array* x, const mi_tile_array* codes, const mi_tile_array* scale,
+                         const mi_tile_array* workspace, const mi_tile_array* fold_in, const mi_tile_array* fold_out,
+                         void* stream) {
     MI_CHECK(check_array(x, 2));
     MI_CHECK(check_array(codes, 2));
     MI_CHECK(check_array(scale, 1));
@@ -82,7 +101,16 @@ extern "C" int mi_quantize_e4m3fn(const mi_tile_array* x, const mi_tile_array* c
         return MI_E_STRIDE;
     // whole 16-byte pieces of x, 8-byte pieces of the codes
     if (n % 8 || x->strides[1] % 8 || codes->strides[1] % 8 || !aligned(x->ptr, 16) || !aligned(codes->ptr, 8)) return MI_E_ALIGN;
-    if (n == 0 || rows == 0) return MI_OK;
+    int64_t nfold = 0;
+    if (fold_in) {
+        int64_t nout = 0;
+        MI_CHECK(dense_f32(fold_in, &nfold));
+        MI_CHECK(dense_f32(fold_out, &nout));
+        if (nout != nfold) return MI_E_SHAPE;
+    }
+    if (n == 0 || rows == 0) return nfold ? MI_E_SHAPE : MI_OK;
+    const float* fin = fold_in ? (const float*)fold_in->ptr : nullptr;
+    float* fout = fold_out ? (float*)fold_out->ptr : nullptr;
     const int64_t vecs = n / 8 * rows;
     const int groups = (int)(cld(vecs, (int64_t)(4 * kQThreads)) < kQMaxGroups ? cld(vecs, (int64_t)(4 * kQThreads)) : kQMaxGroups);
     hipStream_t s = (hipStream_t)stream;
@@ -90,13 +118,25 @@ extern "C" int mi_quantize_e4m3fn(const mi_tile_array* x, const mi_tile_array* c
         hipLaunchKernelGGL(absmax_kernel<true>, dim3(groups), dim3(kQThreads), 0, s, (const unsigned short*)x->ptr, x->strides[1], n, rows,
                            (float*)workspace->ptr);
         hipLaunchKernelGGL(quantize_kernel<true>, dim3(groups), dim3(kQThreads), 0, s, (const unsigned short*)x->ptr, x->strides[1], n, rows,
-                           (unsigned char*)codes->ptr, codes->strides[1], (const float*)workspace->ptr, groups, (float*)scale->ptr);
+                           (unsigned char*)codes->ptr, codes->strides[1], (const float*)workspace->ptr, groups, (float*)scale->ptr, fin, fout, nfold);
     } else {
         hipLaunchKernelGGL(absmax_kernel<false>, dim3(groups), dim3(kQThreads), 0, s, (const unsigned short*)x->ptr, x->strides[1], n, rows,
                            (float*)workspace->ptr);
         hipLaunchKernelGGL(quantize_kernel<false>, dim3(groups), dim3(kQThreads), 0, s, (const unsigned short*)x->ptr, x->strides[1], n, rows,
-                           (unsigned char*)codes->ptr, codes->strides[1], (const float*)workspace->ptr, groups, (float*)scale->ptr);
+                           (unsigned char*)codes->ptr, codes->strides[1], (const float*)workspace->ptr, groups, (float*)scale->ptr, fin, fout, nfold);
     }
     set_variant("quantize_e4m3fn_per_tensor_2pass");
     return launch_status();
+}
+
+extern "C" int mi_quantize_e4m3fn(const mi_tile_array* x, const mi_tile_array* codes, const mi_tile_array* scale,
+                                  const mi_tile_array* workspace, void* stream) {
+    return quantize_impl(x, codes, scale, workspace, nullptr, nullptr, stream);
+}
+
+extern "C" int mi_quantize_e4m3fn_fold(const mi_tile_array* x, const mi_tile_array* codes, const mi_tile_array* scale,
+                                       const mi_tile_array* workspace, const mi_tile_array* fold_in,
+                                       const mi_tile_array* fold_out, void* stream) {
+    if (!fold_in || !fold_out) return MI_E_NULL;
+    return quantize_impl(x, codes, scale, workspace, fold_in, fold_out, stream);
 }

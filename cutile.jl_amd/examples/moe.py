@@ -54,7 +54,7 @@ def cutile_moe(hidden_states, w1, w2, topk_weights, topk_ids, tile_m, tile_n, ti
     ``fp8_activations`` (with E4M3FN weights and their scales; an extension like the fp8 weights themselves): both
     grouped GEMMs multiply fp8 by fp8 on the matrix cores, the operand pairing that ext/DLFP8TypesExt.jl:15-19 gives
     ``mma``.  The activations of either GEMM are quantised per tensor on the device (``quantize_activations``) and
-    their scale is folded into the weights' per-channel scales; needs blocks of 128 slots, the fused SiLU epilogue and
+    their scale is folded into the weights' per-channel scales by the same launches; needs blocks of 128 slots, the fused SiLU epilogue and
     hidden / intermediate sizes that are multiples of 16 from 512 up."""
     num_tokens, hidden_size = hidden_states.shape
     num_experts, _, intermediate_size = w2.shape
@@ -64,8 +64,7 @@ def cutile_moe(hidden_states, w1, w2, topk_weights, topk_ids, tile_m, tile_n, ti
     if fp8_activations:
         if w1_scale is None or w2_scale is None or not fuse_silu:
             raise ValueError("fp8 activations need e4m3 weights with their scales and the fused SiLU epilogue")
-        hidden_states, a_scale = quantize_activations(hidden_states)
-        w1_scale = w1_scale * a_scale
+        hidden_states, _, w1_scale = ct.quantize_e4m3fn(hidden_states, fold=w1_scale)
     can_fuse_sum = (topk <= 2 and aligned is None and device_align and hidden_size % 8 == 0 and topk_weights.dtype == T)
     if fuse_sum is None:
         fuse_sum = can_fuse_sum
@@ -110,8 +109,7 @@ def cutile_moe(hidden_states, w1, w2, topk_weights, topk_ids, tile_m, tile_n, ti
         cache1_flat = cache1.reshape(total_tokens, intermediate_size * 2)
         invoke_silu_and_mul_kernel(cache1_flat, cache2)
     if fp8_activations:
-        cache2, c_scale = quantize_activations(cache2)
-        w2_scale = w2_scale * c_scale
+        cache2, _, w2_scale = ct.quantize_e4m3fn(cache2, fold=w2_scale)
     if fuse_sum:
         ct.fused_moe_accumulate_kernel(cache2, w2, out, topk_weights, sorted_token_ids, sorted_expert_ids, tile_m, tile_n,
                                        tile_k, b_scale=w2_scale)

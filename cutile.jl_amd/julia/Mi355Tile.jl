@@ -349,6 +349,15 @@ function quantize_e4m3fn(x, codes, scale, workspace; stream::Ptr{Cvoid}=C_NULL)
         (Ref{MiTileArray}, Ref{MiTileArray}, Ref{MiTileArray}, Ref{MiTileArray}, Ptr{Cvoid}), d[1], d[2], d[3], d[4], stream))
 end
 
+"The same, and fold_out .= fold_in .* scale[1] (dense Float32 arrays of one shape: the weights' scales that these
+activations meet) from the same two launches."
+function quantize_e4m3fn_fold(x, codes, scale, workspace, fold_in, fold_out; stream::Ptr{Cvoid}=C_NULL)
+    d = map(a -> ref(descriptor(a)), (x, codes, scale, workspace, fold_in, fold_out))
+    GC.@preserve x codes scale workspace fold_in fold_out check(ccall((:mi_quantize_e4m3fn_fold, libmi355tile), Cint,
+        (Ref{MiTileArray}, Ref{MiTileArray}, Ref{MiTileArray}, Ref{MiTileArray}, Ref{MiTileArray}, Ref{MiTileArray},
+         Ptr{Cvoid}), d[1], d[2], d[3], d[4], d[5], d[6], stream))
+end
+
 # ---- examples/fft.jl ----------------------------------------------------------------------
 
 function fft_kernel(x_packed_in, y_packed_out, W0, W1, W2, T0, T1, N::Integer, F0::Integer, F1::Integer,

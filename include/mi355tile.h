@@ -205,7 +205,7 @@ int mi_moe_align_tile_size(const int64_t* topk_ids, int64_t num_tokens, int64_t 
                            int num_experts, int32_t* sorted_token_ids_out,
                            int32_t* sorted_expert_ids_out, int64_t* total_blocks_out);
 /* Device counterpart of moe_align_tile_size: the same stable counting sort on `stream` (one launch of one
- * workgroup up to 8192 replicas; above, two launches of up to 64 workgroups whose per-expert counts meet in a static
+ * workgroup below 8192 replicas; from there on, two launches of up to 64 workgroups whose per-expert counts meet in a static
  * array of the library -- a stream under graph capture is not given that array and sorts with one workgroup),
  * so that cutile_moe needs no host round trip (the reference copies topk_ids to the
  * host, sorts there and copies the result back: moe.jl:232-233).  topk_ids (num_tokens, topk)
@@ -292,6 +292,12 @@ int mi_moe_sum_topk(const mi_tile_array* in, const mi_tile_array* out, void* str
  * 16-byte (x) and 8-byte (codes) boundaries.  Two launches. */
 int mi_quantize_e4m3fn(const mi_tile_array* x, const mi_tile_array* codes, const mi_tile_array* scale,
                        const mi_tile_array* workspace, void* stream);
+/* The same, and fold_out = fold_in * scale element by element (dense fp32 arrays of one shape, e.g. the (N, E) scales
+ * of the e4m3 weights that these activations meet: the product is what mi_fused_moe_kernel wants as b_scale with fp8
+ * activations, and the second launch writes it on the way).  No counterpart in the reference. */
+int mi_quantize_e4m3fn_fold(const mi_tile_array* x, const mi_tile_array* codes, const mi_tile_array* scale,
+                            const mi_tile_array* workspace, const mi_tile_array* fold_in,
+                            const mi_tile_array* fold_out, void* stream);
 
 /* ---- FFT: examples/fft.jl ------------------------------------------------------------- */
 /* fft_kernel (fft.jl:22-126): batched complex FFT of N = F0*F1*F2 points as three stages of small

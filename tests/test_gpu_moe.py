@@ -192,7 +192,7 @@ def test_moe_full_size_top2(orc):
                                                       (16385, 2, 160, 64), (8193, 1, 1000, 8), (40000, 3, 3, 128),   # several workgroups:
                                                       (70000, 2, 1024, 16), (9000, 7, 64, 128)])                      # 33, 9, 64, 16 and 62 of them
 def test_device_align_matches_host_routine(ct, orc, num_tokens, topk, E, tile_m):
-    """The counting sort (one workgroup, or two launches of several above 8192 replicas) gives the host routine's
+    """The counting sort (one workgroup, or two launches of several from 8192 replicas on) gives the host routine's
     arrays (stable per-expert order, sentinel padding) in the leading part of its fixed-capacity outputs, and marks
     the rest unused."""
     rng = np.random.default_rng(num_tokens + topk)
@@ -205,7 +205,7 @@ def test_device_align_matches_host_routine(ct, orc, num_tokens, topk, E, tile_m)
     assert tok_d.numel() == slots and exp_d.numel() == blocks and nb <= blocks
     assert torch.equal(exp_d[:nb].cpu(), exp_h) and torch.all(exp_d[nb:] == 0)
     assert torch.equal(tok_d[:nb * tile_m].cpu(), tok_h) and torch.all(tok_d[nb * tile_m:] == num_tokens * topk + 1)
-    assert ct.last_variant() == ("moe_align_device_count_place" if num_tokens * topk > 8192 else "moe_align_device_1wg")
+    assert ct.last_variant() == ("moe_align_device_count_place" if num_tokens * topk >= 8192 else "moe_align_device_1wg")
     # oracle as a third opinion
     tok_o, exp_o = orc.moe_align_tile_size(ids.T, tile_m, E)
     assert np.array_equal(tok_h.numpy(), tok_o) and np.array_equal(exp_h.numpy(), exp_o)
@@ -226,7 +226,7 @@ def test_device_align_of_several_workgroups_in_a_row_and_under_capture(ct):
         valid = torch.from_numpy(((ids >= 1) & (ids <= E)).T.reshape(-1))   # replica order: slot fastest
         junk = torch.full((1024, 33), 3.0, dtype=torch.float16, device="cuda")
         tok_d, exp_d = ct.moe_align_tile_size_device(ids_t.cuda(), tile_m, E, clear=junk)
-        multi = num_tokens * topk > 8192
+        multi = num_tokens * topk >= 8192
         assert ct.last_variant() == ("moe_align_device_count_place" if multi else "moe_align_device_1wg")
         assert not junk.any()
         if not bad:
@@ -682,6 +682,23 @@ def test_fp8_activations_times_fp8_weights_on_the_matrix_cores(ct, orc, shape, T
 
     ref = orc.ref_moe(hs, w1d, w2d, J(d.topk_weights), J(d.topk_ids), dtype=np.float64, mid=mid)
     check(J(outs[1]), ref, 5e-2 if T == torch.bfloat16 else 2e-2)
+
+
+def test_quantize_with_the_scale_folded_into_the_weight_scales(ct):
+    """mi_quantize_e4m3fn_fold: the same codes and scale as mi_quantize_e4m3fn, and fold_out = fold_in * scale exactly
+    (one fp32 multiply per element), for f16 and bf16, on a strided view of the activations."""
+    g = torch.Generator(device="cuda"); g.manual_seed(3)
+    for T in (torch.float16, torch.bfloat16):
+        big = (torch.randn(300, 1040, device="cuda", generator=g) * 3).to(T)
+        x = big[:, :1024]
+        w_scale = torch.rand(33, 520, device="cuda", generator=g) + 0.5
+        codes, scale = ct.quantize_e4m3fn(x)
+        codes2, scale2, folded = ct.quantize_e4m3fn(x, fold=w_scale)
+        assert torch.equal(codes.view(torch.uint8), codes2.view(torch.uint8)) and torch.equal(scale, scale2)
+        assert torch.equal(folded, w_scale * scale)
+    with pytest.raises(ct.MiError) as e:
+        ct.quantize_e4m3fn(x, fold=w_scale, fold_out=torch.empty(5, device="cuda"))
+    assert e.value.code == ct.MI_E_SHAPE
 
 
 def test_fp8_activations_are_refused_where_no_kernel_takes_them(ct):

@@ -317,10 +317,14 @@ def bench_kernels(ct, which, cpu, nruns=NRUNS, warmup=WARMUP):
                   ("f16", 1, 2560, 2560, 2560), ("f16", 1, 3072, 3072, 3072), ("f16", 1, 4096, 2048, 4096), ("f16", 1, 4000, 4000, 4000),
                   ("f16", 1, 4096, 4096, 4000), ("f16", 1, 8192, 8192, 8192), ("f16", 4, 512, 1024, 256),
                   ("f32", 1, 256, 256, 256), ("f32", 1, 512, 512, 512), ("f32", 1, 256, 512, 128), ("f32", 1, 1024, 1024, 1024),
-                  ("f32", 1, 2048, 2048, 2048), ("f32", 1, 4096, 4096, 4096), ("f32", 4, 256, 256, 128), ("f32", 4, 512, 512, 256)]
+                  ("f32", 1, 2048, 2048, 2048), ("f32", 1, 4096, 4096, 4096), ("f32", 4, 256, 256, 128), ("f32", 4, 512, 512, 256),
+                  # dense operands whose rows are not 16-byte aligned / sizes that are not multiples of a 16-byte vector
+                  ("f16", 1, 4095, 4096, 4096), ("f16", 1, 4096, 4096, 4095), ("f16", 1, 4095, 4095, 4095), ("f16", 1, 4097, 4096, 4100),
+                  ("f16", 1, 2047, 2048, 200), ("f32", 1, 4095, 4095, 4095),
+                  ("e4m3", 1, 4096, 4096, 4096), ("e4m3", 1, 4095, 4096, 4096), ("e4m3", 1, 4096, 4096, 4095), ("e4m3", 1, 4095, 4095, 4095)]
         rows = []
         for (dt, Bt, M, N, K) in shapes:
-            T = torch.float16 if dt == "f16" else torch.float32
+            T = {"f16": torch.float16, "f32": torch.float32, "e4m3": torch.float8_e4m3fn}[dt]
             a = (torch.randn(Bt, K, M, device="cuda") / 8).to(T); b = (torch.randn(Bt, N, K, device="cuda") / 8).to(T)
             c = torch.empty(Bt, N, M, device="cuda", dtype=torch.float32)
             if Bt == 1:
@@ -330,7 +334,7 @@ def bench_kernels(ct, which, cpu, nruns=NRUNS, warmup=WARMUP):
                 A, B, C = ct.TileArray(a), ct.TileArray(b), ct.TileArray(c)
                 fn = lambda: ct.batch_matmul_kernel(A, B, C, 64, 64, 64)
             e = _entry(f"GEMM {dt} batch {Bt} M={M} N={N} K={K}", fn, 2.0 * Bt * M * N * K, "TFLOPS", "mfma",
-                       2500.0 if dt == "f16" else 157.3, dt, nruns, warmup)
+                       {"f16": 2500.0, "f32": 157.3, "e4m3": 5000.0}[dt], dt, nruns, warmup)
             e["variant"] = ct.last_variant()
             rows.append(e)
         res["gemm_shapes"] = {"name": "GEMM at other shapes (opt-in)", "rows": rows}

@@ -83,6 +83,7 @@ _SIGNATURES = {
     "mi_fused_moe_accumulate_kernel": ([_A] * 6 + [_i, _i, _i, _A, _vp], _i),
     "mi_silu_and_mul_kernel": ([_A, _A, _A, _i, _vp], _i),
     "mi_moe_sum_topk": ([_A, _A, _vp], _i),
+    "mi_scratch_under_capture": ([_i], _i),
     "mi_quantize_e4m3fn": ([_A, _A, _A, _A, _vp], _i),
     "mi_quantize_e4m3fn_fold": ([_A, _A, _A, _A, _A, _A, _vp], _i),
     "mi_tiled_broadcast": ([_A, ctypes.c_char_p, ctypes.POINTER(_A), _i, _vp, _i, _vp], _i),
@@ -124,6 +125,13 @@ def lib() -> ctypes.CDLL:
 
 def strerror(code: int) -> str:
     return lib().mi_strerror(code).decode()
+
+
+def scratch_under_capture(allow: bool) -> bool:
+    """Hand the library's shared static arrays to capturing streams as well (see ``mi_scratch_under_capture``): the
+    caller keeps replays of such graphs apart from one another and from other launches that use the arrays.  Returns
+    the previous setting."""
+    return bool(lib().mi_scratch_under_capture(1 if allow else 0))
 
 
 def last_variant() -> str:

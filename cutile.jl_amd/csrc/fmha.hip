@@ -832,7 +832,9 @@ void launch(dim3 grid, hipStream_t s, bool causal, const mi_tile_array* Q, const
                     static int* arr_ptr[16];
                     int dev = 0;
                     if (hipGetDevice(&dev) == hipSuccess && dev >= 0 && dev < 16) {
-                        if (!arr_ptr[dev] && hipGetSymbolAddress((void**)&arr_ptr[dev], HIP_SYMBOL(fmha_part_arrivals)) != hipSuccess) {
+                        hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;   // (no lookup inside a capture: an eager call has to have made it)
+                        if (!arr_ptr[dev] && hipStreamIsCapturing(s, &cap) == hipSuccess && cap == hipStreamCaptureStatusNone &&
+                            hipGetSymbolAddress((void**)&arr_ptr[dev], HIP_SYMBOL(fmha_part_arrivals)) != hipSuccess) {
                             arr_ptr[dev] = nullptr;
                             (void)hipGetLastError();
                         }

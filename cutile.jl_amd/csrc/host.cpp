@@ -1,6 +1,8 @@
 // Host-only entry points of libmi355tile: version / error strings, the variant record, and
 // the two integer host helpers of the reference's examples (swizzle_2d, moe_align_tile_size).
 #include <algorithm>
+#include <atomic>
+#include <cstdlib>
 #include <cstring>
 #include <numeric>
 #include <vector>
@@ -10,7 +12,17 @@
 namespace mi {
 static thread_local const char* g_variant = "";
 void set_variant(const char* name) { g_variant = name; }
+
+static std::atomic<int> g_scratch_under_capture{[] {
+    const char* e = getenv("MI_SCRATCH_UNDER_CAPTURE");
+    return e && e[0] == '1' ? 1 : 0;
+}()};
+bool scratch_under_capture() { return g_scratch_under_capture.load(std::memory_order_relaxed) != 0; }
 }  // namespace mi
+
+extern "C" int mi_scratch_under_capture(int allow) {
+    return mi::g_scratch_under_capture.exchange(allow ? 1 : 0, std::memory_order_relaxed);
+}
 
 extern "C" int mi_version(void) { return MI355TILE_VERSION; }
 

@@ -1,7 +1,8 @@
 // A static device array of the library that the streams of a GPU share (partial sums of a split GEMM, partial
 // results of split attention).  The library allocates nothing, so such an array is a `static __device__` symbol;
 // launches that use it from different streams are ordered by an event, and a stream under graph capture is not given
-// the array at all (the caller then runs its unsplit kernel).
+// the array at all (the caller then runs its unsplit kernel) unless the caller has promised, through
+// mi_scratch_under_capture, to keep the replays of its graphs apart from one another and from other users of the arrays.
 #pragma once
 #include <mutex>
 
@@ -50,11 +51,20 @@ public:
         int dev = 0;
         if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 16) return nullptr;
         hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
-        if (hipStreamIsCapturing(s, &cap) != hipSuccess || cap != hipStreamCaptureStatusNone) {
+        if (hipStreamIsCapturing(s, &cap) != hipSuccess) {
             (void)hipGetLastError();
             return nullptr;
         }
         SharedScratch& st = per_device[dev];
+        if (cap != hipStreamCaptureStatusNone) {
+            // A launch that is being recorded runs later, as often as the graph is replayed and on whatever stream:
+            // no event of this call can order it.  The array is handed out only if the caller has taken that
+            // ordering upon itself, and only once an eager call has made its address known (the lookup is not
+            // a thing to do inside a capture).  Nothing of the lease's own bookkeeping is touched.
+            if (!scratch_under_capture()) return nullptr;
+            std::unique_lock<std::mutex> lk(st.mu);
+            return st.broken ? nullptr : st.ptr;
+        }
         lock_ = std::unique_lock<std::mutex>(st.mu);
         if (st.broken) return nullptr;
         if (!st.ptr) {

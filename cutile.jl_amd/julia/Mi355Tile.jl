@@ -341,6 +341,11 @@ function moe_sum_topk(in, out; stream::Ptr{Cvoid}=C_NULL)
         (Ref{MiTileArray}, Ref{MiTileArray}, Ptr{Cvoid}), d[1], d[2], stream))
 end
 
+"Hand the library's shared static arrays (split GEMM / attention partials, sort counts) to capturing streams as well;
+the caller keeps replays of such graphs apart from one another and from other launches that use them.  Returns the
+previous setting."
+scratch_under_capture(allow::Bool) = ccall((:mi_scratch_under_capture, libmi355tile), Cint, (Cint,), allow ? 1 : 0) != 0
+
 "codes (K, columns) E4M3FN and scale[1] = max |x| / 448 of a Float16 / BFloat16 activation matrix x (K, columns):
 the fp8 operand `A` of `fused_moe_kernel` when the expert weights are fp8 as well.  `workspace`: 1024 Float32."
 function quantize_e4m3fn(x, codes, scale, workspace; stream::Ptr{Cvoid}=C_NULL)

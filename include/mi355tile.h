@@ -87,6 +87,17 @@ const char* mi_strerror(int code);
 /* Name of the kernel variant chosen by the most recent successful launch on this thread
  * (for profiles and tests; never NULL). */
 const char* mi_last_variant(void);
+/* Some entry points keep partial results in static device arrays of the library that the streams of a GPU share
+ * (the GEMMs split over K, attention split over the keys, the token sort of several workgroups).  Eager launches
+ * that use them from different streams are ordered by the library; a launch recorded into a graph can not be (it
+ * runs later, as often as the graph is replayed), so by default a capturing stream is not given the arrays and
+ * those entry points record their one-piece kernels.  allow != 0 hands the arrays to capturing streams as well: the
+ * caller then sees to it that replays of such graphs overlap neither one another nor any other launch of these entry
+ * points on the device (the usual serving loop, one graph at a time on one stream, does).  The array in question
+ * must have been used by one eager call before (its address is not looked up inside a capture).  Returns the
+ * previous setting; process-wide; also set by MI_SCRATCH_UNDER_CAPTURE=1 in the environment.  No counterpart in the
+ * reference (its launches own their temporaries). */
+int mi_scratch_under_capture(int allow);
 
 /* ---- vadd: examples/vadd.jl ------------------------------------------------------- */
 /* vec_add_kernel_1d (vadd.jl:10-17): c = a + b; block `bid` owns elements

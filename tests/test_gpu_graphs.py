@@ -156,6 +156,48 @@ def test_graph_attention(ct):
     replay_check(inputs, op, compare=compare)
 
 
+def test_graph_with_the_shared_arrays_handed_to_the_capture(ct):
+    """mi_scratch_under_capture(1): the caller keeps its replays apart, and a capturing stream gets what an eager one
+    gets -- attention split over the keys (with the last part adding the parts), the matmul split over K, the token
+    sort of several workgroups.  The recorded variants are the eager ones and every replay equals the eager result
+    bit for bit (split sums are added in a fixed order).  Off again, the one-piece kernels are recorded."""
+    seen = []
+
+    def inputs(seed):
+        g = gen(seed)
+        h = lambda *s: (torch.randn(*s, device="cuda", generator=g) / 4).half()
+        ids = torch.randint(1, 41, (3, 5000), device="cuda", generator=g)
+        return (h(2, 8, 1, 64), h(2, 2, 3000, 64), h(2, 2, 3000, 64), h(4096, 512), h(512, 4096), ids)
+
+    def op(Q, K, V, A, B, ids):
+        o = fmha.cutile_fmha(Q, K, V, causal=True, input_pos=2999, query_group_size=4)
+        seen.append(ct.last_variant())
+        C = torch.empty(512, 512, device="cuda"); ct.matmul_kernel(A, B, C, 64, 64, 64)
+        seen.append(ct.last_variant())
+        tok, exp = ct.moe_align_tile_size_device(ids, 64, 40)
+        seen.append(ct.last_variant())
+        return o, C, tok, exp
+
+    was = ct.scratch_under_capture(True)
+    try:
+        replay_check(inputs, op)
+        # calls in order: warm-up, capture, then one eager call per round
+        assert all("splitkv" in v for v in seen[0::3]) and all("splitk" in v for v in seen[1::3]), seen
+        assert all(v == "moe_align_device_count_place" for v in seen[2::3]), seen
+        ct.scratch_under_capture(False)
+        del seen[:]
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        static = inputs(9)
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.stream(side):
+            with torch.cuda.graph(graph, stream=side):
+                op(*static)
+        assert "splitkv" not in seen[0] and "splitk" not in seen[1] and seen[2] == "moe_align_device_1wg", seen
+    finally:
+        ct.scratch_under_capture(was)
+
+
 @pytest.mark.parametrize("topk", [2, 8])
 def test_graph_moe_with_its_defaults(ct, topk):
     """Token sort on the device, both grouped GEMMs, and for top-2 the down projection that adds into an output the

@@ -50,8 +50,22 @@ template <> __device__ __forceinline__ void vset<__hip_bfloat16>(Raw<__hip_bfloa
     v[q] = *reinterpret_cast<unsigned short*>(&h);
 }
 
+// A 16-byte vector at an address that is aligned for its elements only: global memory takes such accesses, in one
+// instruction (a column of 50257 floats starts anywhere).
+template <typename V, typename T>
+__device__ __forceinline__ V ld_unaligned(const T* p) {
+    V v;
+    __builtin_memcpy(&v, p, sizeof(V));
+    return v;
+}
+template <typename V, typename T>
+__device__ __forceinline__ void st_unaligned(const V& v, T* p) {
+    __builtin_memcpy(p, &v, sizeof(V));
+}
+
 // ---- single-tile kernel: column cached in registers -----------------------------------
-// Capacity BLOCK*VPT*EV elements.  ALIGNED: column bases and L allow 16-byte vectors.
+// Capacity BLOCK*VPT*EV elements.  ALIGNED: every column starts on a 16-byte boundary (plain and streaming vector
+// accesses); otherwise the vectors inside the column move unaligned and only the one across its end element-wise.
 template <typename T, int BLOCK, int VPT, bool ALIGNED, bool STREAM>
 __global__ __launch_bounds__(BLOCK) void softmax_regs_kernel(T* __restrict__ out, int64_t ldo,
                                                              const T* __restrict__ in, int64_t ldi,
@@ -69,8 +83,10 @@ __global__ __launch_bounds__(BLOCK) void softmax_regs_kernel(T* __restrict__ out
 #pragma unroll
         for (int v = 0; v < VPT; ++v) {
             const int e0 = (threadIdx.x + v * BLOCK) * EV;
-            if (ALIGNED && e0 + EV <= L) {
-                V raw = ld_global<STREAM>(reinterpret_cast<const V*>(ip + e0));
+            if (e0 + EV <= L) {
+                V raw;
+                if (ALIGNED) raw = ld_global<STREAM>(reinterpret_cast<const V*>(ip + e0));
+                else raw = ld_unaligned<V>(ip + e0);
 #pragma unroll
                 for (int q = 0; q < EV; ++q) x[v][q] = vget<T>(raw, q);
             } else {
@@ -85,13 +101,28 @@ __global__ __launch_bounds__(BLOCK) void softmax_regs_kernel(T* __restrict__ out
             for (int q = 0; q < EV; ++q) mx = fmaxf(mx, x[v][q]);
         mx = block_reduce<NW>(mx, red, MaxOp{}, NEG_INF);
         float sum = 0.f;
+        if constexpr (BLOCK == 1024) {
+            // One workgroup holds the CU here, so nothing runs under this loop: 64 library exponentials per lane
+            // (about twenty instructions each) were as long as the column's load.  The hardware's 2^x on
+            // (x - max) * log2(e), the product formed by one fma: two instructions, and an error of the argument's
+            // rounding, |x - max| * 2^-24 relative (3e-6 at 50 below the maximum, where the value is 2e-22).
+            const float l2e = 1.4426950408889634f, mxl = mx == NEG_INF ? 0.f : mx * l2e;
 #pragma unroll
-        for (int v = 0; v < VPT; ++v)
+            for (int v = 0; v < VPT; ++v)
 #pragma unroll
-            for (int q = 0; q < EV; ++q) {
-                x[v][q] = expf(x[v][q] - mx);
-                sum += x[v][q];
-            }
+                for (int q = 0; q < EV; ++q) {
+                    x[v][q] = __builtin_amdgcn_exp2f(__builtin_fmaf(x[v][q], l2e, -mxl));
+                    sum += x[v][q];
+                }
+        } else {
+#pragma unroll
+            for (int v = 0; v < VPT; ++v)
+#pragma unroll
+                for (int q = 0; q < EV; ++q) {
+                    x[v][q] = expf(x[v][q] - mx);
+                    sum += x[v][q];
+                }
+        }
         sum = block_reduce<NW>(sum, red, SumOp{}, 0.f);
         // one correctly rounded reciprocal per column, then multiplies: within 1.5 ulp of the
         // element-wise quotient, at a tenth of the instructions
@@ -99,11 +130,12 @@ __global__ __launch_bounds__(BLOCK) void softmax_regs_kernel(T* __restrict__ out
 #pragma unroll
         for (int v = 0; v < VPT; ++v) {
             const int e0 = (threadIdx.x + v * BLOCK) * EV;
-            if (ALIGNED && e0 + EV <= L) {
+            if (e0 + EV <= L) {
                 V raw;
 #pragma unroll
                 for (int q = 0; q < EV; ++q) vset<T>(raw, q, x[v][q] * rsum);
-                st_global<true>(raw, reinterpret_cast<V*>(op + e0));
+                if (ALIGNED) st_global<true>(raw, reinterpret_cast<V*>(op + e0));
+                else st_unaligned<V>(raw, op + e0);
             } else {
 #pragma unroll
                 for (int q = 0; q < EV; ++q)
@@ -156,27 +188,32 @@ __global__ __launch_bounds__(BLOCK) void softmax_3pass_kernel(T* __restrict__ ou
         }
         for (int64_t e = threadIdx.x; e < nscalar; e += BLOCK) mx = fmaxf(mx, to_f32<T>(ip[at(e)]));
         mx = block_reduce<NW>(mx, red, MaxOp{}, NEG_INF);
+        // exp(x - max) as the hardware's 2^x of one fma (see the 1024-lane register kernel): a column this long is
+        // walked by one workgroup per CU, and the library exponential was most of passes 2 and 3
+        const float l2e = 1.4426950408889634f, mxl = mx == NEG_INF ? 0.f : mx * l2e;
+        auto ex = [&](float v) { return __builtin_amdgcn_exp2f(__builtin_fmaf(v, l2e, -mxl)); };
         // pass 2: per-lane partial denominators, one reduction at the end
         float den = 0.f;
 #pragma unroll 4
         for (int64_t v = threadIdx.x; v < nvec; v += BLOCK) {
             V raw = *reinterpret_cast<const V*>(ipv + v * EV);
 #pragma unroll
-            for (int q = 0; q < EV; ++q) den += expf(vget<T>(raw, q) - mx);
+            for (int q = 0; q < EV; ++q) den += ex(vget<T>(raw, q));
         }
-        for (int64_t e = threadIdx.x; e < nscalar; e += BLOCK) den += expf(to_f32<T>(ip[at(e)]) - mx);
+        for (int64_t e = threadIdx.x; e < nscalar; e += BLOCK) den += ex(to_f32<T>(ip[at(e)]));
         den = block_reduce<NW>(den, red, SumOp{}, 0.f);
+        const float rden = 1.0f / den;   // (one reciprocal per column, then multiplies, as in the register kernel)
         // pass 3: normalise and store
 #pragma unroll 4
         for (int64_t v = threadIdx.x; v < nvec; v += BLOCK) {
             V raw = *reinterpret_cast<const V*>(ipv + v * EV);
             V res;
 #pragma unroll
-            for (int q = 0; q < EV; ++q) vset<T>(res, q, expf(vget<T>(raw, q) - mx) / den);
+            for (int q = 0; q < EV; ++q) vset<T>(res, q, ex(vget<T>(raw, q)) * rden);
             st_global<true>(res, reinterpret_cast<V*>(opv + v * EV));
         }
         for (int64_t e = threadIdx.x; e < nscalar; e += BLOCK)
-            op[at(e)] = from_f32<T>(expf(to_f32<T>(ip[at(e)]) - mx) / den);
+            op[at(e)] = from_f32<T>(ex(to_f32<T>(ip[at(e)])) * rden);
     }
 }
 
@@ -203,7 +240,10 @@ template <typename T, int BLOCK, int VPT>
 void launch_regs(const mi_tile_array* output, const mi_tile_array* input, int L, bool al,
                  hipStream_t s) {
     const int64_t M = input->sizes[1];
-    dim3 grid((unsigned)M), block(BLOCK);
+    // The 1024-lane variants hold a CU's registers with one workgroup (two when a lane keeps 32 elements): a workgroup
+    // per CU slot walks the columns, so that the stores of one column, once issued, drain under the loads of the next.
+    const int64_t slots = 256 * (VPT * Raw<T>::EV <= 32 ? 2 : 1);
+    dim3 grid((unsigned)(BLOCK == 1024 && M > slots ? slots : M)), block(BLOCK);
 #define GO(AL, ST)                                                                              \
     hipLaunchKernelGGL((softmax_regs_kernel<T, BLOCK, VPT, AL, ST>), grid, block, 0, s, (T*)output->ptr, \
                        output->strides[1], (const T*)input->ptr, input->strides[1], L, M)
@@ -237,10 +277,18 @@ int launch_3pass(const mi_tile_array* output, const mi_tile_array* input, int64_
 template <typename T>
 int launch_len(const mi_tile_array* output, const mi_tile_array* input, int64_t L64, hipStream_t s) {
     constexpr int EV = Raw<T>::EV;
-    if (L64 > 256 * 16 * EV) return launch_3pass<T>(output, input, L64, s);
+    if (L64 > 65536) return launch_3pass<T>(output, input, L64, s);
     const int L = (int)L64;
+    // (a column that is aligned as a whole: its last vector may still cross the end, which the kernel handles)
     const bool al = vec_ok<T>(output, input);
     const int vecs = (int)cld(L, EV);
+    if (vecs > 256 * 16) {
+        // Up to 65536 elements in the registers of 1024 lanes (64 per lane), one workgroup per CU: one pass over HBM
+        // where the three-pass kernel re-reads the column twice (1024 x 50257 fp32: 121 us).
+        if (L > 32768) { launch_regs<T, 1024, 64 / EV>(output, input, L, al, s); set_variant("softmax_regs_b1024_e64"); }
+        else { launch_regs<T, 1024, 32 / EV>(output, input, L, al, s); set_variant("softmax_regs_b1024_e32"); }
+        return launch_status();
+    }
     if (vecs <= 64) { launch_regs<T, 64, 1>(output, input, L, al, s); set_variant("softmax_regs_b64_v1"); }
     else if (vecs <= 128) { launch_regs<T, 64, 2>(output, input, L, al, s); set_variant("softmax_regs_b64_v2"); }
     else if (vecs <= 256) { launch_regs<T, 64, 4>(output, input, L, al, s); set_variant("softmax_regs_b64_v4"); }   // one wave per column: no barriers

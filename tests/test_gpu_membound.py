@@ -262,12 +262,19 @@ def test_softmax_both_kernels(orc, M, N, T):
 
 @pytest.mark.parametrize("M,N,T,variant", [
     (7, 100003, torch.float32, "softmax_3pass_b1024"),     # few long columns, odd length: scalar head, vectors, scalar tail
-    (40, 50257, torch.float16, "softmax_3pass_b1024"), (3, 131075, torch.bfloat16, "softmax_3pass_b1024"),
-    (1100, 16388, torch.float32, "softmax_3pass_b256"), (1030, 16391, torch.float32, "softmax_3pass_b256"),
+    (3, 131075, torch.bfloat16, "softmax_3pass_b1024"), (1100, 65540, torch.float16, "softmax_3pass_b256"),
+    # up to 65536 elements: the registers of 1024 lanes, 32 or 64 elements per lane, unaligned vectors where the
+    # columns start off 16-byte boundaries
+    (40, 50257, torch.float16, "softmax_regs_b1024_e64"), (50, 50257, torch.float32, "softmax_regs_b1024_e64"),
+    (1100, 16388, torch.float32, "softmax_regs_b1024_e32"), (1030, 16391, torch.float32, "softmax_regs_b1024_e32"),
+    (300, 40000, torch.float32, "softmax_regs_b1024_e64"), (600, 65536, torch.bfloat16, "softmax_regs_b1024_e64"),
+    (9, 32768, torch.float32, "softmax_regs_b1024_e32"),
 ])
 def test_softmax_columns_too_long_for_registers(ct, orc, M, N, T, variant):
-    """Columns beyond 16384 four-byte (32768 two-byte) elements take three passes; with fewer than 1024 columns a column
-    gets 1024 lanes, and a column that does not start on a 16-byte boundary is walked as head, vectors and tail."""
+    """Columns beyond the 256-lane register kernels (16384 four-byte, 32768 two-byte elements): up to 65536 elements
+    the registers of 1024 lanes hold a column (one pass; more columns than workgroup slots are walked by persistent
+    workgroups), beyond that three passes; a column that does not start on a 16-byte boundary moves in unaligned vectors
+    (register kernels) or as head, vectors and tail (three passes)."""
     d = softmax.prepare(M=M, N=N, T=T)
     out = torch.full_like(d.input, float("nan"))
     ct.softmax_tma_kernel(out, d.input, 1 << (N - 1).bit_length())

@@ -50,7 +50,8 @@ __device__ __forceinline__ void block_sum2(float& a, float& b, float* red) {
 // Load / store the lane's VPT 4-element groups of one row.  Out-of-range elements load 0.
 // ALIGNED: 16-byte aligned rows of a multiple of 4 elements, so a group is wholly inside the row or
 // wholly outside and there is no element-wise tail (whose second code path would keep twice the
-// registers alive).
+// registers alive).  Otherwise the groups inside the row move as unaligned vectors and the one across its end
+// element by element.
 template <int BLOCK, int VPT, bool ALIGNED, bool NT>
 __device__ __forceinline__ void load_row(const float* __restrict__ p, int N, float (&r)[VPT][4]) {
 #pragma unroll
@@ -59,6 +60,13 @@ __device__ __forceinline__ void load_row(const float* __restrict__ p, int N, flo
         if constexpr (ALIGNED) {
             f32x4 t = {0.f, 0.f, 0.f, 0.f};
             if (e0 < N) t = ld_global<NT>(reinterpret_cast<const f32x4*>(p + e0));
+#pragma unroll
+            for (int q = 0; q < 4; ++q) r[v][q] = t[q];
+        } else if (e0 + 4 <= N) {
+            // rows that start anywhere: global memory takes a 16-byte access at a 4-byte aligned address, in one
+            // instruction (element by element these rows moved at a third of the aligned rate)
+            f32x4 t;
+            __builtin_memcpy(&t, p + e0, sizeof(t));
 #pragma unroll
             for (int q = 0; q < 4; ++q) r[v][q] = t[q];
         } else {
@@ -77,6 +85,11 @@ __device__ __forceinline__ void store_row(float* __restrict__ p, int N, const fl
 #pragma unroll
             for (int q = 0; q < 4; ++q) t[q] = r[v][q];
             if (e0 < N) st_global<true>(t, reinterpret_cast<f32x4*>(p + e0));
+        } else if (e0 + 4 <= N) {
+            f32x4 t;
+#pragma unroll
+            for (int q = 0; q < 4; ++q) t[q] = r[v][q];
+            __builtin_memcpy(p + e0, &t, sizeof(t));
         } else {
 #pragma unroll
             for (int q = 0; q < 4; ++q)

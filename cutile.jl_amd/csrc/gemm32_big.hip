@@ -23,9 +23,10 @@
 // a lane its four q for one n; A: four 4-byte reads per m tile.  Any pairing of k with (q, h) gives
 // the same sums as long as A and B agree.
 //
-// Requires M and K multiples of 4, K >= 128, 16-byte aligned operands.  Tiles that reach past M or N
-// re-read the last valid rows / chunks on the way in and clip their stores; in the last group of four
-// steps the chunks at k >= K come from a 16-byte block of zeros (both operands).
+// Requires K >= 128.  Tiles that reach past M or N re-read the last valid rows / chunks on the way in and clip
+// their stores; in the last group of four steps the chunks at k >= K come from a 16-byte block of zeros (both
+// operands).  Rows of any (4-byte) alignment; M and K that are not multiples of 4 as in gemm_big.hip: the K tail --
+// and, with a ragged M, the last row of A -- is one register-fed group of MFMAs behind the ring.
 #include "gemm_direct.h"
 
 namespace {
@@ -136,7 +137,8 @@ template <int I, int J>
 __global__ __launch_bounds__(256) void gemm32_big(const float* __restrict__ A, int64_t lda, int64_t sa,
                                                   const float* __restrict__ B, int64_t ldb, int64_t sb,
                                                   float* __restrict__ C, int64_t ldc, int64_t sc, int M, int N, int K,
-                                                  int tiles_m, int tiles_n, int batch) {
+                                                  int tiles_m, int tiles_n, int batch, int kpeel) {
+    // K: the extent the transfers walk (a multiple of 4); kpeel: values of k behind it for the register-fed MFMAs
     constexpr int BTM = 64 * I, STAGE_A = BTM * BK, BTN = 64 * J, STAGE_B = BTN * BK;
     __shared__ __attribute__((aligned(1024))) float As0[STAGE_A], As1[STAGE_A], As2[STAGE_A], As3[STAGE_A];
     __shared__ __attribute__((aligned(1024))) float Bs0[STAGE_B], Bs1[STAGE_B], Bs2[STAGE_B], Bs3[STAGE_B];
@@ -174,14 +176,14 @@ __global__ __launch_bounds__(256) void gemm32_big(const float* __restrict__ A, i
             }
         }
         // A transfer: lane -> row lane/(16*I) of its block of 4/I rows, LDS position lane%(16*I); rows
-        // k = 4/I*blk + lane/(16*I).  Chunks of 4 m past the edge re-read the last whole chunk (M is a multiple of 4).
+        // k = 4/I*blk + lane/(16*I).  Chunks of 4 m that start past the edge re-read the last chunk that starts inside.
         const int r_in = lane / (16 * I);
         ln.kA = 4 / I * wave + r_in;
 #pragma unroll
         for (int j = 0; j < I; ++j) {
             const int k = 4 / I * (wave + 4 * j) + r_in;
             int ca = (lane % (16 * I)) ^ (8 * ((k >> 2) & 1));
-            if (bm * BTM + 4 * ca + 4 > M) ca = (M - bm * BTM) / 4 - 1;
+            if (bm * BTM + 4 * ca >= M) ca = (M - 1 - bm * BTM) / 4;
             ln.goffA[j] = (unsigned)(((int64_t)r_in * lda + 4 * ca) * 4);
         }
 #pragma unroll
@@ -248,6 +250,27 @@ __global__ __launch_bounds__(256) void gemm32_big(const float* __restrict__ A, i
     KSTEP(3, 0, 2, false, false, 0, true, false, s + 3);
 #undef KSTEP
 
+    if (kpeel > 0) {   // (same for the whole grid)
+        // k = K .. K + kpeel - 1 as the q-th k of the lower half-wave in four MFMAs; the upper half-wave holds zeros
+        const float* Ap = A + (int64_t)bz * sa + (int64_t)K * lda;
+        const float* Bp = B + (int64_t)bz * sb + K;
+        Frag fp;
+        const bool lower = lane < 32;
+#pragma unroll
+        for (int j = 0; j < J; ++j) {
+            const int64_t n = (int64_t)bn * BTN + wn + 32 * j + (lane & 31);
+#pragma unroll
+            for (int q = 0; q < 4; ++q) fp.b[j][q] = lower && q < kpeel && n < N ? Bp[n * ldb + q] : 0.f;
+        }
+#pragma unroll
+        for (int i = 0; i < I; ++i) {
+            const int64_t m = (int64_t)bm * BTM + wm + 32 * i + (lane & 31);
+#pragma unroll
+            for (int q = 0; q < 4; ++q) fp.a[i][q] = lower && q < kpeel && m < M ? Ap[m + (int64_t)q * lda] : 0.f;
+        }
+        mma<I, J>(fp, acc);
+    }
+
     // Epilogue.  The lane's own offset (m within the wave tile, plus its 4*h rows of n) is a 32-bit
     // element offset; the part of n that is uniform across the wave goes into the base.
     const unsigned lane_off = (unsigned)((lane & 31) + (int64_t)(4 * (lane >> 5)) * ldc);
@@ -283,9 +306,12 @@ __global__ __launch_bounds__(256) void gemm32_big(const float* __restrict__ A, i
 template <int I, int J>
 void launch(const Problem& p, hipStream_t s) {
     const int tiles_m = (p.M + 64 * I - 1) / (64 * I), tiles_n = (p.N + 64 * J - 1) / (64 * J);
+    // The extent of K that the transfers walk: whole chunks of 4, and not the last row of A when a chunk of A can
+    // straddle the end of a row (M not a multiple of 4: the chunk then reads on into the next row, which must exist).
+    const int kd = p.M % 4 ? (p.K - 1) / 4 * 4 : p.K / 4 * 4;
     hipLaunchKernelGGL((gemm32_big<I, J>), dim3((unsigned)(tiles_m * tiles_n * p.batch)), dim3(256), 0, s,
                        (const float*)p.A, p.lda, p.sa, (const float*)p.B, p.ldb, p.sb, (float*)p.C, p.ldc, p.sc, p.M,
-                       p.N, p.K, tiles_m, tiles_n, p.batch);
+                       p.N, kd, tiles_m, tiles_n, p.batch, p.K - kd);
 }
 
 }  // namespace
@@ -295,9 +321,7 @@ namespace gemm {
 
 bool big32_applicable(const Problem& p) {
     if (p.in_dtype != MI_F32 || p.out_dtype != MI_F32) return false;
-    // M and K multiples of 4 (A and B move in 16-byte chunks along m and k), any N
-    return p.M % 4 == 0 && p.M >= 4 && p.N >= 1 && p.K % 4 == 0 && p.K >= 128 && aligned(p.A, 16) && aligned(p.B, 16) &&
-           p.lda % 4 == 0 && p.ldb % 4 == 0 && p.sa % 4 == 0 && p.sb % 4 == 0 && p.ldc < (1 << 26) &&
+    return p.M >= 4 && p.N >= 1 && p.K >= 128 + 4 * (p.M % 4 != 0 || p.K % 4 != 0) && p.ldc < (1 << 26) &&
            // (the kernel's 32-bit lane offsets assume rows that follow each other upwards in memory)
            p.lda >= p.M && p.ldb >= p.K && p.ldc >= p.M && p.sa >= 0 && p.sb >= 0 && p.sc >= 0 &&
            p.lda < (1 << 26) && p.ldb < (1 << 26) && tiles_of(p, 64, 64) >= 16 &&

@@ -279,6 +279,26 @@ def test_matmul_f32_direct_to_lds_kernel_exact(ct, orc, M, N, K, tile):
     assert bool((buf[N:] == -77.0).all()) and bool((buf[:, M:] == -77.0).all())
 
 
+@pytest.mark.parametrize("M,N,K,pad", [(2041, 2000, 259, (0, 0)), (1001, 1003, 1025, (1, 2)), (2048, 2050, 133, (3, 1)),
+                                        (4095, 519, 132, (0, 0)), (1023, 1030, 515, (0, 0)), (2052, 2049, 128, (5, 5))])
+def test_matmul_f32_direct_to_lds_kernel_takes_misaligned_rows_and_ragged_sizes(ct, orc, M, N, K, pad):
+    """The fp32 direct-to-LDS kernel on rows that are not 16-byte aligned and on M / K that are not multiples of 4 (the K
+    tail and, with a ragged M, the last row of A go through registers).  Exact integer sums; every cell around the
+    operands holds NaN, C is a view of a buffer of sentinels."""
+    rng = np.random.default_rng(M * 5 + K)
+    A = rng.integers(-3, 4, (M, K)).astype(np.float32); B = rng.integers(-3, 4, (K, N)).astype(np.float32)
+    lda, ldb = M + pad[0], K + pad[1]
+    Aflat = torch.full((K * lda + 8,), float("nan"), device="cuda"); Bflat = torch.full((N * ldb + 8,), float("nan"), device="cuda")
+    Av = Aflat[:K * lda].view(K, lda)[:, :M]; Bv = Bflat[:N * ldb].view(N, ldb)[:, :K]
+    Av.copy_(orc.from_julia(A)); Bv.copy_(orc.from_julia(B))
+    buf = torch.full((N + 2, M + 7), -77.0, device="cuda")
+    C = buf[:N, :M]
+    ct.matmul_kernel(Av, Bv, C, 64, 64, 64)
+    assert ct.last_variant().startswith("gemm32_big_"), ct.last_variant()
+    assert np.array_equal(orc.to_julia(C.contiguous()), A @ B)
+    assert bool((buf[N:] == -77.0).all()) and bool((buf[:, M:] == -77.0).all())
+
+
 def test_batch_matmul_large_tile_kernel(ct, orc):
     rng = np.random.default_rng(8)
     M, K, N, Bn = 1024, 256, 1024, 4

@@ -26,6 +26,15 @@ using namespace mi;
 
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 
+// w * dy as a value of its own.  The backward kernels form this product twice, once for the row sums and once for dX;
+// left to the compiler, the second one may be fused into the subtraction that follows (an unrounded product minus a
+// sum of rounded ones), and a row of one element then gets the product's rounding error times rstd instead of 0.
+__device__ __forceinline__ float rounded_product(float a, float b) {
+    float p = a * b;
+    asm volatile("" : "+v"(p));
+    return p;
+}
+
 // Block all-reduce (sum) of two floats at once.
 template <int NWAVES>
 __device__ __forceinline__ void block_sum2(float& a, float& b, float* red) {
@@ -111,11 +120,17 @@ __global__ __launch_bounds__(BLOCK) void ln_fwd_kernel(const float* __restrict__
     __shared__ float red[NW > 1 ? NW : 1];
     const float invN = 1.0f / (float)N;
     for (int64_t m = blockIdx.x; m < M; m += gridDim.x) {
-        float x[VPT][4], w[VPT][4], b[VPT][4];
+        // (eight vectors per lane: W and B are asked for after the reductions, half a row at a time -- with the row
+        // they would be 96 registers of a lane's 128)
+        constexpr bool LATE_WB = VPT >= 8;
+        constexpr int WV = LATE_WB ? VPT / 2 : VPT;
+        float x[VPT][4], w[WV][4], b[WV][4];
         load_row<BLOCK, VPT, ALIGNED, STREAM>(X + m * ldx, N, x);
         // W and B come from L2; asked for now, they arrive while the row is being reduced
-        load_row<BLOCK, VPT, ALIGNED, false>(W, N, w);
-        load_row<BLOCK, VPT, ALIGNED, false>(B, N, b);
+        if constexpr (!LATE_WB) {
+            load_row<BLOCK, VPT, ALIGNED, false>(W, N, w);
+            load_row<BLOCK, VPT, ALIGNED, false>(B, N, b);
+        }
         float s = 0.f;
 #pragma unroll
         for (int v = 0; v < VPT; ++v)
@@ -138,10 +153,26 @@ __global__ __launch_bounds__(BLOCK) void ln_fwd_kernel(const float* __restrict__
             Mean[m] = mean;
             Rstd[m] = rstd;
         }
+        if constexpr (!LATE_WB) {
 #pragma unroll
-        for (int v = 0; v < VPT; ++v)
+            for (int v = 0; v < VPT; ++v)
 #pragma unroll
-            for (int q = 0; q < 4; ++q) x[v][q] = ((x[v][q] - mean) * rstd) * w[v][q] + b[v][q];
+                for (int q = 0; q < 4; ++q) x[v][q] = ((x[v][q] - mean) * rstd) * w[v][q] + b[v][q];
+        } else {
+            const float *Wp = W, *Bp = B;
+            asm volatile("" : "+s"(Wp), "+s"(Bp));   // (opaque per row: the loads stay here instead of being hoisted out of the row loop into registers)
+#pragma unroll
+            for (int half = 0; half < 2; ++half) {
+                // (the second half of the row: the same lanes, WV vectors further on)
+                load_row<BLOCK, WV, ALIGNED, false>(Wp + half * WV * BLOCK * 4, N - half * WV * BLOCK * 4, w);
+                load_row<BLOCK, WV, ALIGNED, false>(Bp + half * WV * BLOCK * 4, N - half * WV * BLOCK * 4, b);
+#pragma unroll
+                for (int v = 0; v < WV; ++v)
+#pragma unroll
+                    for (int q = 0; q < 4; ++q)
+                        x[half * WV + v][q] = ((x[half * WV + v][q] - mean) * rstd) * w[v][q] + b[v][q];
+            }
+        }
         store_row<BLOCK, VPT, ALIGNED, STREAM>(Y + m * ldy, N, x);
     }
     (void)invN;
@@ -360,7 +391,7 @@ __global__ __launch_bounds__(BLOCK) void ln_bwd_kernel(float* __restrict__ DX, i
         for (int v = 0; v < VPT; ++v)
 #pragma unroll
             for (int q = 0; q < 4; ++q) {
-                const float xhat = x[v][q], wdy = w[v][q] * dy[v][q];
+                const float xhat = x[v][q], wdy = rounded_product(w[v][q], dy[v][q]);
                 dw[v][q] += dy[v][q] * xhat;
                 db[v][q] += dy[v][q];
                 x[v][q] = (wdy - (xhat * c1 + c2)) * rstd;
@@ -467,7 +498,7 @@ __global__ __launch_bounds__(BLOCK * RG) void ln_bwd_rg_kernel(float* __restrict
 #pragma unroll
             for (int q = 0; q < 4; ++q) {
                 const float xhat = in ? (x[v][q] - mean) * rstd : 0.f;
-                const float wdy = w[v][q] * dy[v][q];
+                const float wdy = rounded_product(w[v][q], dy[v][q]);
                 x[v][q] = xhat;
                 c1 += xhat * wdy;
                 c2 += wdy;
@@ -496,7 +527,7 @@ __global__ __launch_bounds__(BLOCK * RG) void ln_bwd_rg_kernel(float* __restrict
             f32x4 t;
 #pragma unroll
             for (int q = 0; q < 4; ++q) {
-                const float xhat = x[v][q], wdy = w[v][q] * dy[v][q];
+                const float xhat = x[v][q], wdy = rounded_product(w[v][q], dy[v][q]);
                 dw[v][q] += dy[v][q] * xhat;
                 db[v][q] += dy[v][q];
                 t[q] = (wdy - (xhat * c1 + c2)) * rstd;
@@ -614,7 +645,7 @@ __global__ __launch_bounds__(kWideLanes) void ln_bwd_wide_kernel(float* __restri
 #pragma unroll
             for (int q = 0; q < 4; ++q) {
                 const float xhat = in ? (x[v][q] - mean) * rstd : 0.f;
-                const float wdy = w[v][q] * dy[v][q];
+                const float wdy = rounded_product(w[v][q], dy[v][q]);
                 x[v][q] = xhat;
                 c1 += xhat * wdy;
                 c2 += wdy;
@@ -641,7 +672,7 @@ __global__ __launch_bounds__(kWideLanes) void ln_bwd_wide_kernel(float* __restri
             f32x4 t;
 #pragma unroll
             for (int q = 0; q < 4; ++q) {
-                const float xhat = x[v][q], wdy = w[v][q] * dy[v][q];
+                const float xhat = x[v][q], wdy = rounded_product(w[v][q], dy[v][q]);
                 dw[v][q] += dy[v][q] * xhat;
                 db[v][q] += dy[v][q];
                 t[q] = (wdy - (xhat * c1 + c2)) * rstd;
@@ -687,7 +718,7 @@ __global__ __launch_bounds__(BLOCK) void ln_bwd_long_kernel(float* __restrict__ 
         const float mean = Mean[m], rstd = Rstd[m];
         float c1 = 0.f, c2 = 0.f;
         for (int64_t e = threadIdx.x; e < N; e += BLOCK) {
-            const float xhat = (x[e] - mean) * rstd, wdy = W[e] * dy[e];
+            const float xhat = (x[e] - mean) * rstd, wdy = rounded_product(W[e], dy[e]);
             c1 += xhat * wdy;
             c2 += wdy;
         }
@@ -698,7 +729,7 @@ __global__ __launch_bounds__(BLOCK) void ln_bwd_long_kernel(float* __restrict__ 
         float* dbp = DB + (m % G) * lddb;
         float* dx = DX + m * lddx;
         for (int64_t e = threadIdx.x; e < N; e += BLOCK) {
-            const float xhat = (x[e] - mean) * rstd, wdy = W[e] * dy[e];
+            const float xhat = (x[e] - mean) * rstd, wdy = rounded_product(W[e], dy[e]);
             dx[e] = (wdy - (xhat * c1 + c2)) * rstd;
             unsafeAtomicAdd(dwp + e, dy[e] * xhat);
             unsafeAtomicAdd(dbp + e, dy[e]);
@@ -823,7 +854,7 @@ template <bool ST>
 bool launch_fwd_pipe(int vecs, hipStream_t s, const float* X, int64_t ldx, const float* W, const float* B,
                      float* Y, int64_t ldy, float* Mean, float* Rstd, float eps, int N, int64_t M) {
     static const int wpc = [] { const char* e = getenv("MI_LN_FWD_WPC"); return e ? atoi(e) : 0; }();   // workgroups per CU (tuning; < 0: off)
-    if (wpc < 0) return false;
+    if (wpc < 0 || vecs > 4096) return false;
     const int block = vecs <= 256 ? 64 : vecs <= 1024 ? 256 : vecs <= 2048 ? 512 : 1024;
     // (256-lane workgroups: six per CU measured best, 80 % of the HBM rate on resident input and 64 % on cold
     // input against 78 % and 60 % for one row per workgroup lifetime)
@@ -860,7 +891,8 @@ void launch_fwd(int vecs, dim3 grid, hipStream_t s, const float* X, int64_t ldx,
     else if (vecs <= 512) { FWD(256, 2); set_variant("ln_fwd_regs_b256_v2"); }
     else if (vecs <= 1024) { FWD(256, 4); set_variant("ln_fwd_regs_b256_v4"); }
     else if (vecs <= 2048) { FWD(512, 4); set_variant("ln_fwd_regs_b512_v4"); }      // longer rows: more lanes, not more
-    else { FWD(1024, 4); set_variant("ln_fwd_regs_b1024_v4"); }                       // registers per lane
+    else if (vecs <= 4096) { FWD(1024, 4); set_variant("ln_fwd_regs_b1024_v4"); }    // registers per lane
+    else { FWD(1024, 8); set_variant("ln_fwd_regs_b1024_v8"); }   // up to 32768 elements: x, W and B are 96 of a lane's 128 registers
 
 #undef FWD
 }
@@ -908,7 +940,7 @@ extern "C" int mi_layer_norm_fwd(const mi_tile_array* X, const mi_tile_array* W,
     const float* x = (const float*)X->ptr;
     float* y = (float*)Y->ptr;
     dim3 grid((unsigned)M);
-    if (N > kMaxRegsN) {
+    if (N > 2 * kMaxRegsN) {
         const bool vec = N % 4 == 0 && rows_vec_ok(X) && rows_vec_ok(Y) && rows_vec_ok(W) && rows_vec_ok(B);
         const bool wide = M < 1024;   // few rows: 1024 lanes each
 #define GO(BL, VEC)                                                                                           \

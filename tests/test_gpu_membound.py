@@ -375,10 +375,13 @@ def test_layernorm_bwd_wide_rows(ct, orc, M, N, G):
 
 
 @pytest.mark.parametrize("M,N,variant", [(9, 65536, "ln_fwd_3pass_b1024_v4"), (5, 100003, "ln_fwd_3pass_b1024"),
-                                         (1030, 16388, "ln_fwd_3pass_b256_v4"), (1025, 16387, "ln_fwd_3pass_b256")])
+                                         (1030, 32772, "ln_fwd_3pass_b256_v4"), (1025, 32771, "ln_fwd_3pass_b256"),
+                                         (1030, 16388, "ln_fwd_regs_b1024_v8"), (1025, 16387, "ln_fwd_regs_b1024_v8"),
+                                         (300, 32768, "ln_fwd_regs_b1024_v8"), (7, 20001, "ln_fwd_regs_b1024_v8")])
 def test_layernorm_fwd_rows_too_long_for_registers(ct, orc, M, N, variant):
-    """Rows beyond 16384 elements: three passes, 16-byte accesses when every row allows them, 1024 lanes per row
-    when there are fewer than 1024 rows."""
+    """Rows beyond 16384 elements: up to 32768 in the registers of 1024 lanes (eight vectors per lane, W and B asked
+    for after the reductions), beyond that three passes, 16-byte accesses when every row allows them, 1024 lanes per
+    row when there are fewer than 1024 rows."""
     rng = np.random.default_rng(3)
     X = torch.from_numpy(rng.standard_normal((M, N), dtype=np.float32)).cuda()
     W = torch.from_numpy(rng.standard_normal(N, dtype=np.float32)).cuda(); B = torch.from_numpy(rng.standard_normal(N, dtype=np.float32)).cuda()

@@ -699,6 +699,130 @@ __global__ __launch_bounds__(kWideLanes) void ln_bwd_wide_kernel(float* __restri
     }
 }
 
+// Backward for rows of 16385 to 32768 elements (16-byte aligned): 512 lanes, sixteen vectors of the row per lane.  dW
+// and dB of the lane's 64 columns stay in registers for all the rows of the workgroup (128 of the 256 registers that
+// eight waves per CU leave a lane; with 1024 lanes and 128 registers the kernel spilled) and are flushed
+// once; the row itself does not fit beside them, so it is walked twice -- once for the two row sums, once for dX and
+// the partials, the second time out of the caches -- two vectors of each array at a time.  (The kernel for still
+// longer rows adds every element of every row to the partial slots with an atomic of its own: 1.2-1.6 TB/s at 32768.)
+// Loads are unpredicated (a vector past the end of the row re-reads the row's last vector and is masked where it is
+// used): behind a branch each, the compiler could not order them and spilled 140 registers.
+__global__ __launch_bounds__(512) void ln_bwd_two_pass_kernel(float* __restrict__ DX, int64_t lddx,
+                                                               const float* __restrict__ DY, int64_t lddy,
+                                                               float* __restrict__ DW, int64_t lddw,
+                                                               float* __restrict__ DB, int64_t lddb,
+                                                               const float* __restrict__ X, int64_t ldx,
+                                                               const float* __restrict__ W,
+                                                               const float* __restrict__ Mean,
+                                                               const float* __restrict__ Rstd, int N,
+                                                               int64_t M, int G, int S) {
+    constexpr int BLOCK = 512, NW = BLOCK / 64, VPT = 16, HV = 2;
+    __shared__ float red[2 * NW];
+    __shared__ __attribute__((aligned(16))) float stage[BLOCK * VPT * 4];   // 128 KB: the flush of dW, then of dB
+    const int g = blockIdx.x % G, s = blockIdx.x / G;
+    float dw[VPT][4], db[VPT][4];
+#pragma unroll
+    for (int v = 0; v < VPT; ++v)
+#pragma unroll
+        for (int q = 0; q < 4; ++q) dw[v][q] = db[v][q] = 0.f;
+    auto e0_of = [&](int v) { return ((int)threadIdx.x + v * BLOCK) * 4; };
+    // Vector v of a lane lies v * BLOCK * 16 bytes behind vector 0: that part of the address is the same for the whole
+    // workgroup and goes into the scalar base of the load, the lane's own part is one 32-bit offset for all vectors and
+    // arrays (an address pair per vector and array was 128 registers).  A lane past the end of the row in a vector that
+    // others still have re-reads the row's last vector; vectors that lie past the end for everybody are skipped.
+    const unsigned lane_bytes = threadIdx.x * 16u;
+    auto ldv = [&](const float* row, int v) {
+        const int left = N - v * BLOCK * 4;                         // elements of the row from this vector's first lane on (> 0)
+        const unsigned off = lane_bytes < (unsigned)left * 4u ? lane_bytes : (unsigned)left * 4u - 16u;
+        return *reinterpret_cast<const f32x4*>(reinterpret_cast<const char*>(row + v * BLOCK * 4) + off);
+    };
+    const int nv = (N + BLOCK * 4 - 1) / (BLOCK * 4);               // vectors that hold elements of the row for some lane
+    for (int64_t m = g + (int64_t)G * s; m < M; m += (int64_t)G * S) {
+        const float* xr = X + m * ldx;
+        const float* dyr = DY + m * lddy;
+        const float* Wr = W;
+        asm volatile("" : "+s"(Wr));   // (opaque per row: W is loaded where it is used, not hoisted out of the row loop into registers)
+        const float mean = Mean[m], rstd = Rstd[m];
+        float c1 = 0.f, c2 = 0.f;
+#pragma unroll
+        for (int h = 0; h < VPT / HV; ++h) {
+            __builtin_amdgcn_sched_barrier(0);
+            if (h * HV >= nv) break;   // (the same for the whole workgroup)
+            f32x4 x[HV], dy[HV], w[HV];
+#pragma unroll
+            for (int u = 0; u < HV; ++u) {
+                const int v = h * HV + u < nv ? h * HV + u : nv - 1;
+                x[u] = ldv(xr, v);
+                dy[u] = ldv(dyr, v);
+                w[u] = ldv(Wr, v);
+            }
+#pragma unroll
+            for (int u = 0; u < HV; ++u) {
+                const bool in = e0_of(h * HV + u) < N;
+#pragma unroll
+                for (int q = 0; q < 4; ++q) {
+                    const float xhat = in ? (x[u][q] - mean) * rstd : 0.f;
+                    const float wdy = in ? w[u][q] * dy[u][q] : 0.f;
+                    c1 += xhat * wdy;
+                    c2 += wdy;
+                }
+            }
+        }
+        block_sum2<NW>(c1, c2, red);
+        c1 /= (float)N;
+        c2 /= (float)N;
+        // (opaque again: the second walk loads anew -- as the same loads from the same unwritten addresses the
+        // compiler would keep the first walk's values alive instead, in scratch memory)
+        asm volatile("" : "+s"(xr), "+s"(dyr), "+s"(Wr));
+        float* dxr = DX + m * lddx;
+#pragma unroll
+        for (int h = 0; h < VPT / HV; ++h) {
+            __builtin_amdgcn_sched_barrier(0);
+            if (h * HV >= nv) break;
+            f32x4 x[HV], dy[HV], w[HV];
+#pragma unroll
+            for (int u = 0; u < HV; ++u) {
+                const int v = h * HV + u < nv ? h * HV + u : nv - 1;
+                x[u] = ldv(xr, v);
+                dy[u] = ldv(dyr, v);
+                w[u] = ldv(Wr, v);
+            }
+#pragma unroll
+            for (int u = 0; u < HV; ++u) {
+                const int v = h * HV + u;
+                const bool in = e0_of(v) < N;
+                f32x4 t;
+#pragma unroll
+                for (int q = 0; q < 4; ++q) {
+                    const float dyq = in ? dy[u][q] : 0.f;
+                    const float xhat = in ? (x[u][q] - mean) * rstd : 0.f;
+                    const float wdy = rounded_product(w[u][q], dyq);
+                    dw[v][q] += dyq * xhat;
+                    db[v][q] += dyq;
+                    t[q] = (wdy - (xhat * c1 + c2)) * rstd;
+                }
+                if (in) st_global<true>(t, reinterpret_cast<f32x4*>(reinterpret_cast<char*>(dxr + v * BLOCK * 4) + lane_bytes));
+            }
+        }
+    }
+    float* dwp = DW + (int64_t)g * lddw;
+    float* dbp = DB + (int64_t)g * lddb;
+#pragma unroll
+    for (int pass = 0; pass < 2; ++pass) {
+        __syncthreads();
+#pragma unroll
+        for (int v = 0; v < VPT; ++v)
+#pragma unroll
+            for (int q = 0; q < 4; ++q) stage[e0_of(v) + q] = pass == 0 ? dw[v][q] : db[v][q];
+        __syncthreads();
+        float* dst = pass == 0 ? dwp : dbp;
+        for (int c = threadIdx.x; c < N; c += BLOCK) {
+            if (S == 1) dst[c] += stage[c];
+            else unsafeAtomicAdd(dst + c, stage[c]);
+        }
+    }
+}
+
 // Backward for rows longer than the register-cached variants hold.
 template <int BLOCK>
 __global__ __launch_bounds__(BLOCK) void ln_bwd_long_kernel(float* __restrict__ DX, int64_t lddx,
@@ -998,6 +1122,20 @@ extern "C" int mi_layer_norm_bwd_dx_partial_dwdb(
     if (M == 0) return MI_OK;
     if (N == 0) return MI_E_SHAPE;
     hipStream_t s = (hipStream_t)stream;
+    if (N > kMaxRegsN && N <= 2 * kMaxRegsN && G <= 256 && N % 4 == 0 && rows_vec_ok(X) && rows_vec_ok(DX) && rows_vec_ok(DY) &&
+        rows_vec_ok(W)) {
+        // one workgroup of 512 lanes per CU (128 KB of LDS for the flush)
+        const int64_t rows_per_slot = cld(M, (int64_t)G);
+        int64_t Sw = cld((int64_t)256, (int64_t)G);
+        if (Sw > rows_per_slot) Sw = rows_per_slot;
+        if (Sw < 1) Sw = 1;
+        hipLaunchKernelGGL(ln_bwd_two_pass_kernel, dim3((unsigned)(G * Sw)), dim3(512), 0, s, (float*)DX->ptr,
+                           DX->strides[1], (const float*)DY->ptr, DY->strides[1], (float*)DW->ptr, DW->strides[1],
+                           (float*)DB->ptr, DB->strides[1], (const float*)X->ptr, X->strides[1], (const float*)W->ptr,
+                           (const float*)Mean->ptr, (const float*)Rstd->ptr, (int)N, M, G, (int)Sw);
+        set_variant("ln_bwd_two_pass_b512_v16");
+        return launch_status();
+    }
     if (N > kMaxRegsN) {
         hipLaunchKernelGGL((ln_bwd_long_kernel<256>), dim3((unsigned)M), dim3(256), 0, s,
                            (float*)DX->ptr, DX->strides[1], (const float*)DY->ptr, DY->strides[1],

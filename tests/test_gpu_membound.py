@@ -374,6 +374,27 @@ def test_layernorm_bwd_wide_rows(ct, orc, M, N, G):
     close_f32(orc.to_julia(d.FINAL_DB), DB)
 
 
+@pytest.mark.parametrize("M,N,G,variant", [(130, 32768, 64, "ln_bwd_two_pass_b512_v16"), (37, 16388, 8, "ln_bwd_two_pass_b512_v16"),
+                                           (300, 20000, 256, "ln_bwd_two_pass_b512_v16"), (5, 24580, 1, "ln_bwd_two_pass_b512_v16"),
+                                           (9, 32772, 4, "ln_bwd_long_b256"), (6, 20001, 4, "ln_bwd_long_b256")])
+def test_layernorm_bwd_rows_beyond_the_register_kernels(ct, orc, M, N, G, variant):
+    """Rows of 16385 to 32768 aligned elements: dW / dB of a lane's columns in registers, the row walked twice (vectors
+    that lie past the end of the row for every lane are skipped, the last partly used one is clamped); longer or
+    misaligned rows: the kernel that adds every element to the partial slots."""
+    d = layernorm.prepare(M=M, N=N, GROUP_SIZE_M=G)
+    ct.layer_norm_fwd(d.X, d.W, d.B, d.Y, d.Mean, d.Rstd, d.eps, 1024)
+    d.partials.zero_()
+    d.DX.fill_(float("nan"))
+    ct.layer_norm_bwd_dx_partial_dwdb(d.DX, d.DY, d.DW_partial, d.DB_partial, d.X, d.W, d.Mean, d.Rstd, d.Locks, G, 1024)
+    assert ct.last_variant() == variant
+    ct.layer_norm_bwd_dwdb(d.DW_partial, d.DB_partial, d.FINAL_DW, d.FINAL_DB, 32, 1024)
+    X, W, DY = (orc.to_julia(t) for t in (d.X, d.W, d.DY))
+    DX, DW, DB = orc.layer_norm_bwd(X, W, DY, d.eps)
+    close_f32(orc.to_julia(d.DX), DX)
+    close_f32(orc.to_julia(d.FINAL_DW), DW)
+    close_f32(orc.to_julia(d.FINAL_DB), DB)
+
+
 @pytest.mark.parametrize("M,N,variant", [(9, 65536, "ln_fwd_3pass_b1024_v4"), (5, 100003, "ln_fwd_3pass_b1024"),
                                          (1030, 32772, "ln_fwd_3pass_b256_v4"), (1025, 32771, "ln_fwd_3pass_b256"),
                                          (1030, 16388, "ln_fwd_regs_b1024_v8"), (1025, 16387, "ln_fwd_regs_b1024_v8"),

@@ -707,8 +707,8 @@ bool dense_applicable(const DenseArgs& a) {
 
 // Channels per tile: 256 weight rows per workgroup (four MFMA column tiles per wave, three ring stages) halve the LDS
 // fragment reads per MFMA -- 0.75 KB against 1 KB, and the LDS pipe (128 bytes per clock and CU) is what bounds the
-// K walk of the narrower tile -- and are taken when they still give every workgroup slot of the chip a tile and a
-// half; otherwise 128 rows (two column tiles per wave, four stages).  MI_MOE_DENSE_J = 2 | 4 forces one.
+// K walk of the narrower tile -- and are taken when they still give every workgroup slot of the chip a tile;
+// otherwise 128 rows (two column tiles per wave, four stages).  MI_MOE_DENSE_J = 2 | 4 forces one.
 static int pick_j(const DenseArgs& a) {
     const char* env = getenv("MI_MOE_DENSE_J");
     const int force = env ? atoi(env) : 0;
@@ -717,7 +717,10 @@ static int pick_j(const DenseArgs& a) {
     const int64_t strips4 = a.silu ? cld((int64_t)a.N / 2, (int64_t)128) : cld((int64_t)a.N, (int64_t)256);
     // blocks that hold tokens: at most one partly filled block per expert on top of the full ones
     const int64_t blocks = cld((int64_t)a.total_tokens, (int64_t)kRows) + a.num_experts / 2;
-    return blocks * strips4 >= 768 ? 4 : 2;
+    // (measured, gate / up projection: 256 tokens top-8, 512 such tiles, 62 against 66 us; 1024 top-8 128 / 150; 2048 top-2
+    // 100 / 104; 4096 top-2 137 / 160; 8192 top-2 232 / 264.  The down projection has a quarter of the strips and stays
+    // on 128 channels up to about 16k replicas: 4096 top-2 93 against 99 us.)
+    return blocks * strips4 >= 512 ? 4 : 2;
 }
 
 void dense_launch(const DenseArgs& a, hipStream_t s) {

@@ -117,7 +117,9 @@ def _entry(name, fn, work, unit, bound, peak, dtype, nruns, warmup, extra=None, 
             for f in cold:
                 f()
         cycle()
-        cavg = min(_back_to_back(cycle, max(1, nruns // k)) for _ in range(2)) / k
+        # (batches as long as the warm ones and behind as many untimed launches: three cycles from an idle GPU ran at
+        # the clocks of the ramp, 8-15 % below what the same rotation reaches once they have settled)
+        cavg = min(_back_to_back(cycle, max(1, nruns // k), k * min(t)) for _ in range(2)) / k
         e["avg_ms_cold"] = round(cavg, 5)
         e["frac_cold"] = round(work / (cavg * 1e-3) / scale / peak, 4)
         e["cold_sets"] = k

@@ -172,6 +172,24 @@ def test_matmul_split_over_k_exact(ct, orc, M, N, K, T, out32):
     assert bool((buf[N:] == -77.0).all()) and bool((buf[:, M:] == -77.0).all())
 
 
+@pytest.mark.parametrize("M,N,K,pad", [(512, 512, 4096, (1, 3)), (264, 1001, 3080, (5, 1)), (520, 500, 4000, (2, 2))])
+def test_matmul_split_over_k_on_misaligned_rows(ct, orc, M, N, K, pad):
+    """The split over K with operands whose rows are not 16-byte aligned (views with odd leading dimensions; M and K
+    multiples of 8, as the split wants them): the parts' transfers take the misaligned rows like the plain kernel's.
+    Exact integer sums, NaN around the operands."""
+    rng = np.random.default_rng(M + K + 1)
+    A = rng.integers(-1, 2, (M, K)).astype(np.float32); B = rng.integers(-1, 2, (K, N)).astype(np.float32)
+    lda, ldb = M + pad[0], K + pad[1]
+    Aflat = torch.full((K * lda + 16,), float("nan"), dtype=torch.float16, device="cuda")
+    Bflat = torch.full((N * ldb + 16,), float("nan"), dtype=torch.float16, device="cuda")
+    Av = Aflat[:K * lda].view(K, lda)[:, :M]; Bv = Bflat[:N * ldb].view(N, ldb)[:, :K]
+    Av.copy_(orc.from_julia(A).to(torch.float16)); Bv.copy_(orc.from_julia(B).to(torch.float16))
+    C = torch.full((N, M), -77.0, device="cuda")
+    ct.matmul_kernel(Av, Bv, C, 64, 64, 64)
+    assert ct.last_variant().startswith("gemm16_big_128x128x32_ring4_splitk"), ct.last_variant()
+    assert np.array_equal(orc.to_julia(C), A @ B)
+
+
 def test_matmul_split_over_k_is_reproducible_and_ordered_across_streams(ct, orc):
     """The parts are added in a fixed order, so two runs give the same bits; launches from two streams share the
     scratch and are ordered by the library, so alternating between streams still gives every product its own

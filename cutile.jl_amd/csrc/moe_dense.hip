@@ -366,7 +366,10 @@ __device__ __forceinline__ void store_tile_slot_lane(const float (&o)[16], unsig
         const int c = 8 * q + 8 * hb;   // first of this lane's eight channels
         if (valid) {
             if (vec_ok && c + 8 <= n_left) {
-                __builtin_nontemporal_store(v, reinterpret_cast<u32x4*>(row + c));
+                // (an ordinary store: what is written here is read again by the next launch -- the down projection
+                // or the sum over the slots -- and a streaming store would send it past the L2 it can be found in;
+                // measured 1-7 % on both launches, most at 16 384 tokens)
+                *reinterpret_cast<u32x4*>(row + c) = v;
             } else {
 #pragma unroll
                 for (int e = 0; e < 8; ++e)

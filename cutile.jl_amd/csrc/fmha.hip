@@ -275,9 +275,12 @@ __device__ __forceinline__ int ksw(int key) {
     return D == 64 ? (key >> 1) & 7 : key & 15;
 }
 
+// AUX: the instruction's cache policy bits (0 = default, 2 = non-temporal: the line is the first to leave the L2 and
+// takes no room in the memory-side cache).
+template <int AUX = 0>
 __device__ __forceinline__ void gload_lds16(const void* g, void* lds_wave_base) {
     __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)g,
-                                     (__attribute__((address_space(3))) void*)lds_wave_base, 16, 0, 0);
+                                     (__attribute__((address_space(3))) void*)lds_wave_base, 16, 0, AUX);
 }
 
 template <int D, int NW>
@@ -303,12 +306,20 @@ struct FmhaDma {
         int first_pos[JT];  // position of the first query of column tile j
     };
 
+    template <int AUX>
+    static __device__ __forceinline__ void issue_as(const char* Kg, const char* Vg, unsigned short* Ks,
+                                                    unsigned short* Vs, int wave, const DmaLane<D, NW>& dl) {
+#pragma unroll
+        for (int i = 0; i < TPW; ++i) gload_lds16<AUX>(Kg + dl.koff[i], Ks + (wave + NW * i) * 512);
+#pragma unroll
+        for (int i = 0; i < TPW; ++i) gload_lds16<AUX>(Vg + dl.voff[i], Vs + (wave + NW * i) * 512);
+    }
+    // stream: every key is read by this workgroup alone and the keys of the launch do not fit the memory-side cache
+    // (a KV cache walked once per new token): non-temporal transfers (the host decides, see the launch).
     static __device__ __forceinline__ void issue(const char* Kg, const char* Vg, unsigned short* Ks,
-                                                 unsigned short* Vs, int wave, const DmaLane<D, NW>& dl) {
-#pragma unroll
-        for (int i = 0; i < TPW; ++i) gload_lds16(Kg + dl.koff[i], Ks + (wave + NW * i) * 512);
-#pragma unroll
-        for (int i = 0; i < TPW; ++i) gload_lds16(Vg + dl.voff[i], Vs + (wave + NW * i) * 512);
+                                                 unsigned short* Vs, int wave, const DmaLane<D, NW>& dl, bool stream) {
+        if (stream) issue_as<2>(Kg, Vg, Ks, Vs, wave, dl);
+        else issue_as<0>(Kg, Vg, Ks, Vs, wave, dl);
     }
 
     // JM: bit j set = column tile j takes part in this KV tile (a causal wave drops its early
@@ -426,7 +437,7 @@ template <typename E, int D, int JT, bool CAUSAL, bool SPLIT = false>
 __global__ __launch_bounds__(128 * 2 / JT) __attribute__((amdgpu_waves_per_eu(2, 2))) void fmha_fwd_dma_kernel(
     const unsigned short* __restrict__ Q, Strides qs, const unsigned short* __restrict__ K, Strides ks,
     const unsigned short* __restrict__ V, Strides vs, unsigned short* __restrict__ O, Strides os, int Sq, int Skv,
-    int H, int group, float scale2, int input_pos, int nqb, int nbh, int pack, int nsplit = 1,
+    int H, int group, float scale2, int input_pos, int nqb, int nbh, int pack, int kv_stream, int nsplit = 1,
     float* __restrict__ part = nullptr, int* __restrict__ arrivals = nullptr) {
     using F = FmhaDma<E, D, JT, CAUSAL>;
     constexpr int NW = F::NW, KSTEPS = F::KSTEPS, DT = F::DT, CH = F::CH, TPW = F::TPW;
@@ -548,7 +559,7 @@ __global__ __launch_bounds__(128 * 2 / JT) __attribute__((amdgpu_waves_per_eu(2,
     // the last valid row (the masked scores make the values irrelevant, and finite).
     auto issue_tile = [&](int t, unsigned short* Ksx, unsigned short* Vsx) {
         if ((t + 1) * kKV <= Skv) {
-            F::issue(Kg + t * k_tile_bytes, Vg + t * v_tile_bytes, Ksx, Vsx, wave, dl);
+            F::issue(Kg + t * k_tile_bytes, Vg + t * v_tile_bytes, Ksx, Vsx, wave, dl, kv_stream != 0);
         } else {
             DmaLane<D, NW> cl;
 #pragma unroll
@@ -561,7 +572,7 @@ __global__ __launch_bounds__(128 * 2 / JT) __attribute__((amdgpu_waves_per_eu(2,
                 cl.koff[i] = (unsigned)(((int64_t)key * ks.s1 + 8 * (pos ^ swk)) * 2);
                 cl.voff[i] = (unsigned)(((int64_t)key * vs.s1 + 8 * (pos ^ ((D / 32) * swv))) * 2);
             }
-            F::issue(Kg + t * k_tile_bytes, Vg + t * v_tile_bytes, Ksx, Vsx, wave, cl);
+            F::issue(Kg + t * k_tile_bytes, Vg + t * v_tile_bytes, Ksx, Vsx, wave, cl, kv_stream != 0);
         }
     };
     // Which of the wave's column tiles still see keys of the tile starting at kv0.
@@ -819,6 +830,15 @@ void launch(dim3 grid, hipStream_t s, bool causal, const mi_tile_array* Q, const
         const int nqb = pack > 1 ? (Sq * pack + kQB - 1) / kQB : (int)grid.x, nbh = (int)grid.y / pack;
         dim3 g1((unsigned)(nqb * nbh)), blk(128 * 2 / JT);
         const int64_t rows = (int64_t)nbh * Sq * pack;
+        // Keys that one query block walks alone and that are well beyond what the memory-side cache (256 MB) holds are
+        // streamed.  Measured with the same buffers launch after launch, 16-bit keys of 64 elements: 134 MB 26.8 us
+        // cached / 28.8 streamed, 268 MB 47.3 / 49.7, 537 MB 96.0 / 82.2 (5.6 -> 6.5 TB/s), 32 x 16 heads x 4096 keys
+        // unsplit 91.8 / 78.0 (6.9 TB/s); 134 MB in six rotating sets 30.8 / 28.6.  A caller that knows its cache will not
+        // be read again before it has left the memory-side cache anyway sets MI_FMHA_KV_STREAM = 1 (0 = never; read at
+        // every call).
+        const char* env_kv = getenv("MI_FMHA_KV_STREAM");
+        const int64_t kv_bytes = 2 * (int64_t)(grid.y / group) * Skv * D * 2;
+        const int kv_stream = nqb == 1 && (env_kv ? atoi(env_kv) != 0 : kv_bytes > (320ll << 20)) ? 1 : 0;
         if (const int parts = pick_parts((int64_t)nqb * nbh, rows, D, Sq, Skv, causal, input_pos)) {
             ScratchLease lease;   // ends behind the combine launch
             if (float* scratch = (float*)lease.acquire(g_part, HIP_SYMBOL(fmha_part_scratch), s)) {
@@ -844,11 +864,11 @@ void launch(dim3 grid, hipStream_t s, bool causal, const mi_tile_array* Q, const
                 if (causal)
                     hipLaunchKernelGGL((fmha_fwd_dma_kernel<E, D, JT, true, true>), gs, blk, 0, s, (const unsigned short*)Q->ptr, qs,
                                        (const unsigned short*)K->ptr, ks, (const unsigned short*)V->ptr, vs,
-                                       (unsigned short*)O->ptr, os, Sq, Skv, Hb, group, scale2, input_pos, nqb, nbh, pack, parts, scratch, arrivals);
+                                       (unsigned short*)O->ptr, os, Sq, Skv, Hb, group, scale2, input_pos, nqb, nbh, pack, kv_stream, parts, scratch, arrivals);
                 else
                     hipLaunchKernelGGL((fmha_fwd_dma_kernel<E, D, JT, false, true>), gs, blk, 0, s, (const unsigned short*)Q->ptr, qs,
                                        (const unsigned short*)K->ptr, ks, (const unsigned short*)V->ptr, vs,
-                                       (unsigned short*)O->ptr, os, Sq, Skv, Hb, group, scale2, input_pos, nqb, nbh, pack, parts, scratch, arrivals);
+                                       (unsigned short*)O->ptr, os, Sq, Skv, Hb, group, scale2, input_pos, nqb, nbh, pack, kv_stream, parts, scratch, arrivals);
                 if (arrivals) {
                     set_variant(pack > 1 ? (D == 64 ? "fmha_dma_q128_kv64_d64_w64q_grouped_splitkv_fused" : "fmha_dma_q128_kv64_d128_w32q_grouped_splitkv_fused")
                                          : (D == 64 ? "fmha_dma_q128_kv64_d64_w64q_splitkv_fused" : "fmha_dma_q128_kv64_d128_w32q_splitkv_fused"));
@@ -870,11 +890,11 @@ void launch(dim3 grid, hipStream_t s, bool causal, const mi_tile_array* Q, const
         if (causal)
             hipLaunchKernelGGL((fmha_fwd_dma_kernel<E, D, JT, true>), g1, blk, 0, s, (const unsigned short*)Q->ptr, qs,
                                (const unsigned short*)K->ptr, ks, (const unsigned short*)V->ptr, vs,
-                               (unsigned short*)O->ptr, os, Sq, Skv, Hb, group, scale2, input_pos, nqb, nbh, pack);
+                               (unsigned short*)O->ptr, os, Sq, Skv, Hb, group, scale2, input_pos, nqb, nbh, pack, kv_stream);
         else
             hipLaunchKernelGGL((fmha_fwd_dma_kernel<E, D, JT, false>), g1, blk, 0, s, (const unsigned short*)Q->ptr, qs,
                                (const unsigned short*)K->ptr, ks, (const unsigned short*)V->ptr, vs,
-                               (unsigned short*)O->ptr, os, Sq, Skv, Hb, group, scale2, input_pos, nqb, nbh, pack);
+                               (unsigned short*)O->ptr, os, Sq, Skv, Hb, group, scale2, input_pos, nqb, nbh, pack, kv_stream);
         set_variant(pack > 1 ? (D == 64 ? "fmha_dma_q128_kv64_d64_w64q_grouped" : "fmha_dma_q128_kv64_d128_w32q_grouped")
                              : (D == 64 ? "fmha_dma_q128_kv64_d64_w64q" : "fmha_dma_q128_kv64_d128_w32q"));
         return;

@@ -223,6 +223,28 @@ def test_fmha_grouped_heads_stacked_short_cache(ct, orc, batch, heads, sq, skv, 
     check(orc, out, ref)
 
 
+@pytest.mark.parametrize("batch,heads,sq,skv,qg,pos,d,T", [
+    (2, 4, 1, 1000, 1, 999, 64, torch.float16),        # split over the keys, parts added by the last one to arrive
+    (1, 8, 1, 4096, 4, 4095, 64, torch.bfloat16),      # grouped heads stacked in one query tile
+    (1, 2, 7, 777, 1, 770, 64, torch.float16),         # ragged cache: the last tile's clamped transfers
+    (1, 8, 1, 2048, 2, 2047, 128, torch.float16),      # D = 128
+    (2, 8, 33, 100, 8, 10, 64, torch.float16),         # too few keys to split: one workgroup per (batch, K / V head)
+])
+def test_fmha_key_cache_streamed_with_non_temporal_transfers(ct, orc, monkeypatch, batch, heads, sq, skv, qg, pos, d, T):
+    """A cache that one query block walks alone and that is larger than the memory-side cache is requested with
+    non-temporal transfers; the choice is forced both ways here (MI_FMHA_KV_STREAM), on small caches: the same
+    arithmetic, so the same bits, and the oracle's values."""
+    data = fmha.prepare(batch=batch, heads=heads, seq_q=sq, seq_kv=skv, d_k=d, d_v=d, query_group_size=qg, causal=True, T=T)
+    outs = []
+    for knob in ("0", "1"):
+        monkeypatch.setenv("MI_FMHA_KV_STREAM", knob)
+        outs.append(attend(data.Q, data.K, data.V, query_group_size=qg, causal=True, input_pos=pos))
+        assert ct.last_variant().startswith("fmha_dma_"), ct.last_variant()
+    assert torch.equal(outs[0], outs[1])
+    ref = orc.fmha_general(*(orc.to_julia(t) for t in (data.Q, data.K, data.V)), causal=True, input_pos=pos)
+    check(orc, outs[1], ref, 2e-2 if T == torch.float16 else 3e-2)
+
+
 def test_fmha_split_launches_from_two_streams_are_ordered(ct, orc):
     """The parts live in one array per GPU: launches that alternate between two streams each get their own result."""
     datas = [fmha.prepare(batch=1, heads=4, seq_q=1, seq_kv=3000 + 64 * i, causal=True, seed=20 + i) for i in range(3)]

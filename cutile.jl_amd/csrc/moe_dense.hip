@@ -31,6 +31,8 @@
 // eight, and the stores are 16 bytes per lane.  The accumulating form (packed atomic adds into the token's output
 // column, one or two slots per token) has the channel in the lane, so that an atomic instruction covers whole
 // 128-byte lines.
+#include <type_traits>
+
 #include "gemm_direct.h"
 #include "moe_dense.h"
 
@@ -136,6 +138,62 @@ __device__ __forceinline__ void k_step(const unsigned short* TsX, unsigned short
     if (!LAST) load_frags<LIVE, J>(TsY, WsY, ln, 0, f0);
     mma<E, LIVE, SLOT_LANE, J>(f1, acc);
     interleave<LIVE, J, DMA_W ? J : 0, !LAST>();
+}
+
+// ---- 16-bit operands, 64 k per stage -----------------------------------------------------------------------------
+// The same walk with stages of 64 k: a stage row is a whole 128-byte line, so every line of the operands is requested
+// once, by one transfer (with rows of 64 bytes a line is requested twice, a step apart, and the second request finds
+// the first still on its way).  A transfer is 8 rows x 128 B; chunk c of row r sits at position c ^ ((r >> 1) & 7): the
+// 16 rows of a quarter-wave's fragment read alternate between the two halves of the banks and the eight rows of a
+// half take eight different positions.  Per stage a wave issues four token transfers and 2 * J weight transfers; a K
+// step is four MFMA sub-steps around one barrier.  Twice the LDS per stage: a ring of four (J = 2, 128 KB) or three
+// (J = 4, 144 KB) stages and one workgroup per CU, whose waves have a SIMD's registers to themselves.
+constexpr int BKW = 64;
+constexpr int kStageTW = kRows * BKW;   // elements of a token stage (16 KB)
+
+template <int J>
+struct WLane {
+    const char* gT[4];       // global address, at k = 0, of the lane's 16-byte chunk in the wave's four token transfers
+    const char* gW[2 * J];   // the same in its 2 * J weight transfers
+    int kC;                  // first k, within a stage, of that chunk
+    unsigned fT[4], fW[4];   // LDS element offset of the token / weight fragment of sub-step 0 .. 3 (+ 32 * BKW per 32-row tile)
+};
+
+template <int LIVE, int J>
+__device__ __forceinline__ void load_fragsW(const unsigned short* Ts, const unsigned short* Ws, const WLane<J>& ln, int ss,
+                                            DFrag<J>& f) {
+    if (LIVE == 0) return;
+#pragma unroll
+    for (int j = 0; j < J; ++j) f.w[j] = *reinterpret_cast<const s16x8*>(Ws + ln.fW[ss] + 32 * j * BKW);
+#pragma unroll
+    for (int i = 0; i < LIVE; ++i) f.t[i] = *reinterpret_cast<const s16x8*>(Ts + ln.fT[ss] + 32 * i * BKW);
+}
+
+// One K step of 64 on stage X; the next step's data is in stage Y.
+//   sub-step 0: MFMAs | read sub-step 1 fragments | token transfers of a later step (into stage TsA)
+//   sub-steps 1, 2: MFMAs | read the next sub-step's fragments
+//   barrier
+//   sub-step 3: MFMAs | read the next stage's sub-step 0 fragments | weight transfers of a later step (into WsX)
+template <typename E, int LIVE, bool SLOT_LANE, int J, bool DMA_T, bool DMA_W, int VMCNT, bool LAST, bool TAIL>
+__device__ __forceinline__ void k_stepW(const unsigned short* TsX, unsigned short* WsX, const unsigned short* TsY,
+                                        const unsigned short* WsY, unsigned short* TsA, int64_t koffT, int64_t koffW,
+                                        int wave, const WLane<J>& ln, DFrag<J>& f0, DFrag<J>& f1, f32x16 (&acc)[2][J],
+                                        int k_leftT, int k_leftW) {
+    if (DMA_T) issueN<TAIL, 4>(ln.gT, koffT, TsA, wave, ln.kC, k_leftT);
+    load_fragsW<LIVE, J>(TsX, WsX, ln, 1, f1);
+    mma<E, LIVE, SLOT_LANE, J>(f0, acc);
+    interleave<LIVE, J, DMA_T ? 4 : 0, true>();
+    load_fragsW<LIVE, J>(TsX, WsX, ln, 2, f0);
+    mma<E, LIVE, SLOT_LANE, J>(f1, acc);
+    interleave<LIVE, J, 0, true>();
+    load_fragsW<LIVE, J>(TsX, WsX, ln, 3, f1);
+    mma<E, LIVE, SLOT_LANE, J>(f0, acc);
+    interleave<LIVE, J, 0, true>();
+    if (!LAST) stage_barrier<VMCNT>();
+    if (DMA_W) issueN<TAIL, 2 * J>(ln.gW, koffW, WsX, wave, ln.kC, k_leftW);
+    if (!LAST) load_fragsW<LIVE, J>(TsY, WsY, ln, 0, f0);
+    mma<E, LIVE, SLOT_LANE, J>(f1, acc);
+    interleave<LIVE, J, DMA_W ? 2 * J : 0, !LAST>();
 }
 
 // ---- fp8 x fp8 (E4M3FN activations and weights) on v_mfma_f32_32x32x64_f8f6f4 ------------------------------------
@@ -296,6 +354,77 @@ __device__ __forceinline__ void main_loop(const Stages& st, int K, int wave, con
     }
 }
 
+constexpr int64_t kStepBytesW = BKW * 2;   // bytes along a row per K step of 64
+
+template <int J>
+__device__ __forceinline__ void ring_fillW(const Stages& st, int wave, const WLane<J>& ln) {
+    issueN<false, 2 * J>(ln.gW, 0, st.W0, wave, ln.kC, 0);
+    issueN<false, 4>(ln.gT, 0, st.T0, wave, ln.kC, 0);
+    issueN<false, 2 * J>(ln.gW, kStepBytesW, st.W1, wave, ln.kC, 0);
+    issueN<false, 4>(ln.gT, kStepBytesW, st.T1, wave, ln.kC, 0);
+    issueN<false, 2 * J>(ln.gW, 2 * kStepBytesW, st.W2, wave, ln.kC, 0);
+    if constexpr (J == 2) {
+        issueN<false, 4>(ln.gT, 2 * kStepBytesW, st.T2, wave, ln.kC, 0);
+        issueN<false, 2 * J>(ln.gW, 3 * kStepBytesW, st.W3, wave, ln.kC, 0);
+    }
+}
+
+// The K walk in steps of 64: the rings, the look-ahead and the waits of main_loop with PER = 4 + 2 * J transfers per wave
+// and stage.  K >= 512 is checked on the host (at least two groups of steps, and a ring fill that stays inside K).
+template <typename E, int LIVE, bool SLOT_LANE, int J>
+__device__ __forceinline__ void main_loopW(const Stages& st, int K, int wave, const WLane<J>& ln, f32x16 (&acc)[2][J]) {
+    DFrag<J> f0, f1;
+    constexpr int PER = 4 + 2 * J;
+    if constexpr (J == 2) {
+        const int KT = 4 * ((K + 4 * BKW - 1) / (4 * BKW));
+        stage_barrier<2 * PER + 2 * J>();
+        load_fragsW<LIVE, J>(st.T0, st.W0, ln, 0, f0);
+#define KSTEP(X, Y, AA, DT, DW, VM, LAST, TAIL, s)                                                                          \
+    k_stepW<E, LIVE, SLOT_LANE, J, DT, DW, (VM) * PER, LAST, TAIL>(st.T##X, st.W##X, st.T##Y, st.W##Y, st.T##AA,           \
+                                                                (int64_t)((s) + 3) * kStepBytesW, (int64_t)((s) + 4) * kStepBytesW, \
+                                                                wave, ln, f0, f1, acc, K - ((s) + 3) * BKW, K - ((s) + 4) * BKW)
+        int s = 0;
+        for (; s + 12 <= KT; s += 4) {
+            KSTEP(0, 1, 3, true, true, 2, false, false, s);
+            KSTEP(1, 2, 0, true, true, 2, false, false, s + 1);
+            KSTEP(2, 3, 1, true, true, 2, false, false, s + 2);
+            KSTEP(3, 0, 2, true, true, 2, false, false, s + 3);
+        }
+        KSTEP(0, 1, 3, true, true, 2, false, true, s);
+        KSTEP(1, 2, 0, true, true, 2, false, true, s + 1);
+        KSTEP(2, 3, 1, true, true, 2, false, true, s + 2);
+        KSTEP(3, 0, 2, true, true, 2, false, true, s + 3);
+        s += 4;
+        KSTEP(0, 1, 3, true, false, 2, false, true, s);
+        KSTEP(1, 2, 0, false, false, 1, false, false, s + 1);
+        KSTEP(2, 3, 1, false, false, 0, false, false, s + 2);
+        KSTEP(3, 0, 2, false, false, 0, true, false, s + 3);
+#undef KSTEP
+    } else {
+        const int KT = 3 * ((K + 3 * BKW - 1) / (3 * BKW));
+        stage_barrier<PER + 2 * J>();
+        load_fragsW<LIVE, J>(st.T0, st.W0, ln, 0, f0);
+#define KSTEP(X, Y, AA, DT, DW, VM, LAST, TAIL, s)                                                                          \
+    k_stepW<E, LIVE, SLOT_LANE, J, DT, DW, VM, LAST, TAIL>(st.T##X, st.W##X, st.T##Y, st.W##Y, st.T##AA,                   \
+                                                        (int64_t)((s) + 2) * kStepBytesW, (int64_t)((s) + 3) * kStepBytesW, \
+                                                        wave, ln, f0, f1, acc, K - ((s) + 2) * BKW, K - ((s) + 3) * BKW)
+        int s = 0;
+        for (; s + 9 <= KT; s += 3) {
+            KSTEP(0, 1, 2, true, true, PER, false, false, s);
+            KSTEP(1, 2, 0, true, true, PER, false, false, s + 1);
+            KSTEP(2, 0, 1, true, true, PER, false, false, s + 2);
+        }
+        KSTEP(0, 1, 2, true, true, PER, false, true, s);
+        KSTEP(1, 2, 0, true, true, PER, false, true, s + 1);
+        KSTEP(2, 0, 1, true, true, PER, false, true, s + 2);
+        s += 3;
+        KSTEP(0, 1, 2, true, false, PER, false, true, s);
+        KSTEP(1, 2, 0, false, false, 0, false, false, s + 1);
+        KSTEP(2, 0, 1, false, false, 0, true, false, s + 2);
+#undef KSTEP
+    }
+}
+
 // The K walk with fp8 operands: the ring of four, a stage per K step of 64.
 template <int LIVE, bool SLOT_LANE, int J>
 __device__ __forceinline__ void main_loop8(const Stages& st, int K, int wave, const DLane<J>& ln, f32x16 (&acc)[2][J]) {
@@ -341,6 +470,7 @@ struct Meta {
     int sb, bid_n;          // 128-slot block and channel strip
     int expert_raw;         // sorted_expert_ids entry (1-based, 0 = unused block)
     int t0, t1, tm;         // sorted_token_ids entries of the rows of this lane's two transfers / of slot `tid`
+    int tw[4];              // (stages of 64 k) entries of the rows of this lane's four transfers
 };
 
 // Stores one 32-slot x 32-channel tile held slot-per-lane (o[r]: channel 8 * (r / 4) + 4 * hb + r % 4 of the lane's
@@ -492,13 +622,16 @@ __device__ __forceinline__ void epilogue(const DenseArgs& a, const f32x16 (&acc)
 // stride.  A tile's stores, and the next tile's ring fill right behind them, are in flight while nothing else of the
 // workgroup is: the next tile's K walk starts as soon as its first stage has landed, and what a tile needs to know
 // (expert, token ids) is requested one tile ahead.
-template <typename E, int MODE, int J, bool A8 = false>
-__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) void moe_dense_kernel(const DenseArgs a, int n_blocks) {
+// WIDE: stages of 64 k (16-bit operands only): twice the LDS, one workgroup per CU.
+template <typename E, int MODE, int J, bool A8 = false, bool WIDE = false>
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(WIDE ? 1 : 2, WIDE ? 1 : 2))) void moe_dense_kernel(const DenseArgs a, int n_blocks) {
+    static_assert(!(WIDE && A8), "fp8 stages are 64 k already");
     constexpr int ES = A8 ? 1 : 2;          // bytes per operand element
     constexpr int EPC = 16 / ES;            // elements per 16-byte chunk
-    constexpr int kStageW = 64 * J * BK;   // elements of a weight stage: 64 * J rows of 32 k
+    constexpr int kStageT = WIDE ? kStageTW : kStage;               // elements of a token stage
+    constexpr int kStageW = 64 * J * (WIDE ? BKW : BK);             // elements of a weight stage: 64 * J rows
     constexpr int kLast = J == 2 ? 1 : 0;  // the ring of three has no fourth stage
-    __shared__ __attribute__((aligned(1024))) unsigned short Ts0[kStage], Ts1[kStage], Ts2[kStage], Ts3[kLast ? kStage : 8];
+    __shared__ __attribute__((aligned(1024))) unsigned short Ts0[kStageT], Ts1[kStageT], Ts2[kStageT], Ts3[kLast ? kStageT : 8];
     __shared__ __attribute__((aligned(1024))) unsigned short Ws0[kStageW], Ws1[kStageW], Ws2[kStageW], Ws3[kLast ? kStageW : 8];
     __shared__ int s_tok[2][kRows];      // 1-based replica id of every slot, 0 = no token (two tiles: current and next)
     __shared__ float s_wt[2][kRows];     // its routed weight (1 where none is applied)
@@ -530,6 +663,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     if (cur >= hi) return;
 
     const int r0 = 16 * wave + (lane >> 2), r1 = 64 + r0;   // rows of this lane's chunks in the wave's two transfers
+    const int rw0 = 8 * wave + (lane >> 3);                  // (stages of 64 k) row of its chunk in the first of four transfers, then every 32
     // Tile idx -> (128-slot block, strip).  Blocks of one expert that follow each other form a run (cut at multiples
     // of 64 blocks, so that one look at 64 expert ids finds it); the tiles of a run are numbered strip-major: all
     // blocks of the expert for strip 0, then for strip 1, ...  The workgroups of an XCD work on consecutive tiles,
@@ -555,13 +689,30 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
         m.sb = b0 + (t - m.bid_n * nb);
         const int slot0 = m.sb * kRows, last = a.num_slots - 1;
         m.expert_raw = e_lb;
-        m.t0 = a.sorted_token_ids[slot0 + r0 < last ? slot0 + r0 : last];
-        m.t1 = a.sorted_token_ids[slot0 + r1 < last ? slot0 + r1 : last];
+        if constexpr (WIDE) {
+#pragma unroll
+            for (int j = 0; j < 4; ++j) m.tw[j] = a.sorted_token_ids[slot0 + rw0 + 32 * j < last ? slot0 + rw0 + 32 * j : last];
+        } else {
+            m.t0 = a.sorted_token_ids[slot0 + r0 < last ? slot0 + r0 : last];
+            m.t1 = a.sorted_token_ids[slot0 + r1 < last ? slot0 + r1 : last];
+        }
         m.tm = a.sorted_token_ids[slot0 + (tid & 127) < last ? slot0 + (tid & 127) : last];
         return m;
     };
-    DLane<J> ln;
-    {
+    using LaneT = typename std::conditional<WIDE, WLane<J>, DLane<J>>::type;
+    LaneT ln;
+    if constexpr (WIDE) {
+        // the lane's LDS position in a transfer is lane % 8 of row lane / 8; rows 8 * (wave + 4 * j) + lane / 8 all have
+        // (row >> 1) & 7 = (4 * wave + lane / 16) & 7
+        const int chunk = (lane & 7) ^ ((4 * wave + (lane >> 4)) & 7);
+        ln.kC = EPC * chunk;
+#pragma unroll
+        for (int ss = 0; ss < 4; ++ss) {
+            const int sw = 8 * ((2 * ss + hb) ^ (((lane & 31) >> 1) & 7));   // (tile rows 64 * ws and 32 * J * wn are multiples of 16)
+            ln.fT[ss] = (64 * ws + (lane & 31)) * BKW + sw;
+            ln.fW[ss] = (32 * J * wn + (lane & 31)) * BKW + sw;
+        }
+    } else {
         const int chunk = (lane & 3) ^ ((lane >> 4) & 3);   // global chunk that belongs at this lane's LDS position
         ln.kC = EPC * chunk;
 #pragma unroll
@@ -573,14 +724,40 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     }
     // Addresses of a tile's transfers from what was read about it; returns this thread's slot's token (0 = none;
     // every slot of a block without a valid expert counts as empty, and such a tile reads expert 1's rows).
-    auto setup = [&](const Meta& m, DLane<J>& L) {
+    auto setup = [&](const Meta& m, LaneT& L) {
         const int slot0 = m.sb * kRows;
         int expert = m.expert_raw - 1;
         const bool ok = expert >= 0 && expert < a.num_experts;
         if (!ok) expert = 0;
         auto fix = [&](int raw, int r) { return (ok && slot0 + r < a.num_slots && raw >= 1 && raw <= a.total_tokens) ? raw : 0; };
-        const int t0 = fix(m.t0, r0), t1 = fix(m.t1, r1);
         const int chunk = L.kC / EPC;
+        if constexpr (WIDE) {
+            const char* Bx = (const char*)a.B + (int64_t)expert * a.sbe * ES;
+            const int half_n = a.N / 2;
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const int t = fix(m.tw[j], rw0 + 32 * j);
+                const int c = t ? (t - 1) / a.replicas : 0;   // slots without a token read column 0
+                L.gT[j] = (const char*)a.A + ((int64_t)c * a.lda + EPC * chunk) * ES;
+            }
+#pragma unroll
+            for (int j = 0; j < 2 * J; ++j) {
+                // tile row R: wave column R / (32 * J), MFMA tile (R / 32) % J of it, channel R % 32 of that
+                const int R = 32 * j + rw0, wcol = R / (32 * J), tj = (R >> 5) % J;
+                int row;
+                if (MODE == MODE_SILU) {
+                    int ch = m.bid_n * (32 * J) + 16 * J * wcol + 32 * (tj % (J / 2)) + (R & 31);
+                    if (ch > half_n - 1) ch = half_n - 1;
+                    row = tj >= J / 2 ? half_n + ch : ch;
+                } else {
+                    row = m.bid_n * (64 * J) + R;
+                    if (row > a.N - 1) row = a.N - 1;
+                }
+                L.gW[j] = Bx + ((int64_t)row * a.ldb + EPC * chunk) * ES;
+            }
+            return fix(m.tm, tid & 127);
+        } else {
+        const int t0 = fix(m.t0, r0), t1 = fix(m.t1, r1);
         const int c0 = t0 ? (t0 - 1) / a.replicas : 0, c1 = t1 ? (t1 - 1) / a.replicas : 0;   // slots without a token read column 0
         L.gT[0] = (const char*)a.A + ((int64_t)c0 * a.lda + EPC * chunk) * ES;
         L.gT[1] = (const char*)a.A + ((int64_t)c1 * a.lda + EPC * chunk) * ES;
@@ -602,6 +779,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
             L.gW[j] = Bx + ((int64_t)row * a.ldb + EPC * chunk) * ES;
         }
         return fix(m.tm, tid & 127);
+        }
     };
     auto routed_weight = [&](int tm) {
         float w = 1.f;
@@ -638,7 +816,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     int nxt = cur + nslot;
     bool have_next = nxt < hi;
     if (have_next) mn = load_meta(nxt);
-    ring_fill<J>(st, wave, ln);
+    if constexpr (WIDE) ring_fillW<J>(st, wave, ln);
+    else ring_fill<J>(st, wave, ln);
     for (;;) {
         f32x16 acc[2][J];
 #pragma unroll
@@ -650,6 +829,10 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
             if (nlive == 2) main_loop8<2, SL, J>(st, a.K, wave, ln, acc);
             else if (nlive == 1) main_loop8<1, SL, J>(st, a.K, wave, ln, acc);
             else main_loop8<0, SL, J>(st, a.K, wave, ln, acc);
+        } else if constexpr (WIDE) {
+            if (nlive == 2) main_loopW<E, 2, SL, J>(st, a.K, wave, ln, acc);
+            else if (nlive == 1) main_loopW<E, 1, SL, J>(st, a.K, wave, ln, acc);
+            else main_loopW<E, 0, SL, J>(st, a.K, wave, ln, acc);
         } else {
             if (nlive == 2) main_loop<E, 2, SL, J>(st, a.K, wave, ln, acc);
             else if (nlive == 1) main_loop<E, 1, SL, J>(st, a.K, wave, ln, acc);
@@ -673,7 +856,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
         nxt += nslot;
         have_next = nxt < hi;
         if (have_next) mn = load_meta(nxt);
-        ring_fill<J>(st, wave, ln);
+        if constexpr (WIDE) ring_fillW<J>(st, wave, ln);
+        else ring_fill<J>(st, wave, ln);
     }
 }
 
@@ -731,27 +915,33 @@ void dense_launch(const DenseArgs& a, hipStream_t s) {
     const int n_blocks = a.silu ? (int)cld((int64_t)a.N / 2, (int64_t)(32 * J)) : (int)cld((int64_t)a.N, (int64_t)(64 * J));
     const int64_t tiles = (int64_t)a.num_blocks * (a.TILE_M / kRows) * n_blocks;
     // persistent: two workgroups per CU at most (64 or 72 KB of LDS each), a multiple of 8 so that every XCD gets as many
-    const int64_t per_xcd = cld(tiles, (int64_t)8) < 64 ? cld(tiles, (int64_t)8) : 64;
+    // Stages of 64 k (one workgroup per CU): MI_MOE_DENSE_WIDE = 0 | 1 forces the choice.
+    const char* env_wide = getenv("MI_MOE_DENSE_WIDE");
+    const bool wide = !a.a8 && a.K >= 512 && (env_wide ? atoi(env_wide) != 0 : false);
+    const int64_t cap = wide ? 32 : 64;
+    const int64_t per_xcd = cld(tiles, (int64_t)8) < cap ? cld(tiles, (int64_t)8) : cap;
     const dim3 grid((unsigned)(per_xcd * 8));
-#define LAUNCH1(ET, MODE, JJ, A8) hipLaunchKernelGGL((moe_dense_kernel<ET, MODE, JJ, A8>), grid, dim3(256), 0, s, a, n_blocks)
-#define LAUNCH(ET, MODE)                        \
-    do {                                        \
-        if (a.a8) LAUNCH1(ET, MODE, 2, true);   \
-        else if (J == 4) LAUNCH1(ET, MODE, 4, false); \
-        else LAUNCH1(ET, MODE, 2, false);       \
+#define LAUNCH1(ET, MODE, JJ, A8, WD) hipLaunchKernelGGL((moe_dense_kernel<ET, MODE, JJ, A8, WD>), grid, dim3(256), 0, s, a, n_blocks)
+#define LAUNCH(ET, MODE)                                              \
+    do {                                                              \
+        if (a.a8) LAUNCH1(ET, MODE, 2, true, false);                  \
+        else if (wide && J == 4) LAUNCH1(ET, MODE, 4, false, true);   \
+        else if (wide) LAUNCH1(ET, MODE, 2, false, true);             \
+        else if (J == 4) LAUNCH1(ET, MODE, 4, false, false);          \
+        else LAUNCH1(ET, MODE, 2, false, false);                      \
     } while (0)
     if (a.silu) {
         if (a.bf16) LAUNCH(BF16, MODE_SILU);
         else LAUNCH(F16, MODE_SILU);
-        set_variant(a.a8 ? "fused_moe_dense_silu_t128_n64x2_k64_ring4_w8a8" : J == 4 ? "fused_moe_dense_silu_t128_n128x2_k32_ring3" : "fused_moe_dense_silu_t128_n64x2_k32_ring4");
+        set_variant(a.a8 ? "fused_moe_dense_silu_t128_n64x2_k64_ring4_w8a8" : wide ? (J == 4 ? "fused_moe_dense_silu_t128_n128x2_k64_ring3" : "fused_moe_dense_silu_t128_n64x2_k64_ring4") : J == 4 ? "fused_moe_dense_silu_t128_n128x2_k32_ring3" : "fused_moe_dense_silu_t128_n64x2_k32_ring4");
     } else if (a.acc_shift >= 0) {
         if (a.bf16) LAUNCH(BF16, MODE_ACC);
         else LAUNCH(F16, MODE_ACC);
-        set_variant(a.a8 ? "fused_moe_dense_acc_t128_n128_k64_ring4_w8a8" : J == 4 ? "fused_moe_dense_acc_t128_n256_k32_ring3" : "fused_moe_dense_acc_t128_n128_k32_ring4");
+        set_variant(a.a8 ? "fused_moe_dense_acc_t128_n128_k64_ring4_w8a8" : wide ? (J == 4 ? "fused_moe_dense_acc_t128_n256_k64_ring3" : "fused_moe_dense_acc_t128_n128_k64_ring4") : J == 4 ? "fused_moe_dense_acc_t128_n256_k32_ring3" : "fused_moe_dense_acc_t128_n128_k32_ring4");
     } else {
         if (a.bf16) LAUNCH(BF16, MODE_PLAIN);
         else LAUNCH(F16, MODE_PLAIN);
-        set_variant(a.a8 ? "fused_moe_dense_t128_n128_k64_ring4_w8a8" : J == 4 ? "fused_moe_dense_t128_n256_k32_ring3" : "fused_moe_dense_t128_n128_k32_ring4");
+        set_variant(a.a8 ? "fused_moe_dense_t128_n128_k64_ring4_w8a8" : wide ? (J == 4 ? "fused_moe_dense_t128_n256_k64_ring3" : "fused_moe_dense_t128_n128_k64_ring4") : J == 4 ? "fused_moe_dense_t128_n256_k32_ring3" : "fused_moe_dense_t128_n128_k32_ring4");
     }
 #undef LAUNCH
 #undef LAUNCH1

@@ -562,7 +562,7 @@ def _every_path(d, tile_m, **kw):
     dict(num_tokens=2048, hidden_size=256, num_experts=256, intermediate_size=64, topk=8),
     dict(num_tokens=400, hidden_size=512, num_experts=4, intermediate_size=256, topk=2, T=torch.bfloat16),
 ])
-@pytest.mark.parametrize("J", ["2", "4"])
+@pytest.mark.parametrize("J", ["2", "4", "2wide", "4wide"])
 def test_dense_routing_ring_kernel_gives_the_streaming_kernels_bits(ct, orc, shape, J, monkeypatch):
     """The grouped GEMM for dense routing (128-slot x 128-channel tiles fed by a ring of LDS stages, persistent
     workgroups) against the streaming kernels on the same launches: every output element is accumulated over k in
@@ -570,8 +570,13 @@ def test_dense_routing_ring_kernel_gives_the_streaming_kernels_bits(ct, orc, sha
     also checked against the float64 oracle.  Shapes: the reference example's own routing (moe.jl:311-344), a prefill
     batch, sizes off the tile grid (K = 328 ends in a zero-padded group of steps, N = 400 in clipped strips), one slot
     per token, 160 and 256 experts, bf16.  Both tile widths of the ring kernel: 128 weight rows on a ring of four stages
-    (J = 2) and 256 rows on a ring of three (J = 4, whose K walk is padded to whole groups of three steps)."""
+    (J = 2) and 256 rows on a ring of three (J = 4, whose K walk is padded to whole groups of three steps); and both
+    again with stages of 64 k (whole 128-byte lines per row and transfer; from K = 512 on), forced on for every launch
+    of the "wide" cases and off for the others."""
+    wide = J.endswith("wide")
+    J = J[0]
     monkeypatch.setenv("MI_MOE_DENSE_J", J)
+    monkeypatch.setenv("MI_MOE_DENSE_WIDE", "1" if wide else "0")
     d = moe.prepare(**shape)
     J = orc.to_julia
     with _dense_knob("0"):
@@ -588,8 +593,9 @@ def test_dense_routing_ring_kernel_gives_the_streaming_kernels_bits(ct, orc, sha
         moe.invoke_fused_moe_kernel(d.hidden_states, d.w1, c2, d.topk_weights, tok, exp, mul_routed_weight=False,
                                     num_token_replicas=d.topk, tile_m=128, tile_n=128, tile_k=64, fuse_silu=True)
         names.add(ct.last_variant())
-    assert names in ({"fused_moe_dense_t128_n128_k32_ring4", "fused_moe_dense_silu_t128_n64x2_k32_ring4"},
-                     {"fused_moe_dense_t128_n256_k32_ring3", "fused_moe_dense_silu_t128_n128x2_k32_ring3"}), names
+    k = "k64" if wide and d.hidden_size >= 512 else "k32"
+    assert names in ({f"fused_moe_dense_t128_n128_{k}_ring4", f"fused_moe_dense_silu_t128_n64x2_{k}_ring4"},
+                     {f"fused_moe_dense_t128_n256_{k}_ring3", f"fused_moe_dense_silu_t128_n128x2_{k}_ring3"}), names
     for k in outs:
         assert not torch.isnan(outs[k].float()).any(), k
         assert torch.equal(outs[k], ref_outs[k]), k

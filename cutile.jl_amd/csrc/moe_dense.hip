@@ -159,6 +159,23 @@ struct WLane {
     unsigned fT[4], fW[4];   // LDS element offset of the token / weight fragment of sub-step 0 .. 3 (+ 32 * BKW per 32-row tile)
 };
 
+// The weight transfers of a wide stage, non-temporal where the launch reads every weight line once (one block per
+// expert): a line that is requested as a whole, once, need not stay anywhere behind the transfer.  (With the 64-byte rows
+// of the narrow stages the second half of a line would be fetched from memory again.)
+// (a template parameter, not a run-time flag: a branch around the transfers would end the block of instructions in
+// which they are spread between the MFMAs -- measured, 56.5 -> 65.5 us on the gate / up projection)
+template <bool TAIL, int N, bool STREAM>
+__device__ __forceinline__ void issueWt(const char* const (&g)[N], int64_t koff, unsigned short* S, int wave, int kC,
+                                        int k_left) {
+#pragma unroll
+    for (int j = 0; j < N; ++j) {
+        const char* p = g[j] + koff;
+        if (TAIL && kC >= k_left) p = (const char*)zeros16d;
+        __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)p,
+                                         (__attribute__((address_space(3))) void*)(S + (wave + 4 * j) * 512), 16, 0, STREAM ? 2 : 0);
+    }
+}
+
 template <int LIVE, int J>
 __device__ __forceinline__ void load_fragsW(const unsigned short* Ts, const unsigned short* Ws, const WLane<J>& ln, int ss,
                                             DFrag<J>& f) {
@@ -174,7 +191,7 @@ __device__ __forceinline__ void load_fragsW(const unsigned short* Ts, const unsi
 //   sub-steps 1, 2: MFMAs | read the next sub-step's fragments
 //   barrier
 //   sub-step 3: MFMAs | read the next stage's sub-step 0 fragments | weight transfers of a later step (into WsX)
-template <typename E, int LIVE, bool SLOT_LANE, int J, bool DMA_T, bool DMA_W, int VMCNT, bool LAST, bool TAIL>
+template <typename E, int LIVE, bool SLOT_LANE, int J, bool DMA_T, bool DMA_W, int VMCNT, bool LAST, bool TAIL, bool STREAM>
 __device__ __forceinline__ void k_stepW(const unsigned short* TsX, unsigned short* WsX, const unsigned short* TsY,
                                         const unsigned short* WsY, unsigned short* TsA, int64_t koffT, int64_t koffW,
                                         int wave, const WLane<J>& ln, DFrag<J>& f0, DFrag<J>& f1, f32x16 (&acc)[2][J],
@@ -190,7 +207,7 @@ __device__ __forceinline__ void k_stepW(const unsigned short* TsX, unsigned shor
     mma<E, LIVE, SLOT_LANE, J>(f0, acc);
     interleave<LIVE, J, 0, true>();
     if (!LAST) stage_barrier<VMCNT>();
-    if (DMA_W) issueN<TAIL, 2 * J>(ln.gW, koffW, WsX, wave, ln.kC, k_leftW);
+    if (DMA_W) issueWt<TAIL, 2 * J, STREAM>(ln.gW, koffW, WsX, wave, ln.kC, k_leftW);
     if (!LAST) load_fragsW<LIVE, J>(TsY, WsY, ln, 0, f0);
     mma<E, LIVE, SLOT_LANE, J>(f1, acc);
     interleave<LIVE, J, DMA_W ? 2 * J : 0, !LAST>();
@@ -356,22 +373,22 @@ __device__ __forceinline__ void main_loop(const Stages& st, int K, int wave, con
 
 constexpr int64_t kStepBytesW = BKW * 2;   // bytes along a row per K step of 64
 
-template <int J>
+template <int J, bool STREAM>
 __device__ __forceinline__ void ring_fillW(const Stages& st, int wave, const WLane<J>& ln) {
-    issueN<false, 2 * J>(ln.gW, 0, st.W0, wave, ln.kC, 0);
+    issueWt<false, 2 * J, STREAM>(ln.gW, 0, st.W0, wave, ln.kC, 0);
     issueN<false, 4>(ln.gT, 0, st.T0, wave, ln.kC, 0);
-    issueN<false, 2 * J>(ln.gW, kStepBytesW, st.W1, wave, ln.kC, 0);
+    issueWt<false, 2 * J, STREAM>(ln.gW, kStepBytesW, st.W1, wave, ln.kC, 0);
     issueN<false, 4>(ln.gT, kStepBytesW, st.T1, wave, ln.kC, 0);
-    issueN<false, 2 * J>(ln.gW, 2 * kStepBytesW, st.W2, wave, ln.kC, 0);
+    issueWt<false, 2 * J, STREAM>(ln.gW, 2 * kStepBytesW, st.W2, wave, ln.kC, 0);
     if constexpr (J == 2) {
         issueN<false, 4>(ln.gT, 2 * kStepBytesW, st.T2, wave, ln.kC, 0);
-        issueN<false, 2 * J>(ln.gW, 3 * kStepBytesW, st.W3, wave, ln.kC, 0);
+        issueWt<false, 2 * J, STREAM>(ln.gW, 3 * kStepBytesW, st.W3, wave, ln.kC, 0);
     }
 }
 
 // The K walk in steps of 64: the rings, the look-ahead and the waits of main_loop with PER = 4 + 2 * J transfers per wave
 // and stage.  K >= 512 is checked on the host (at least two groups of steps, and a ring fill that stays inside K).
-template <typename E, int LIVE, bool SLOT_LANE, int J>
+template <typename E, int LIVE, bool SLOT_LANE, int J, bool STREAM>
 __device__ __forceinline__ void main_loopW(const Stages& st, int K, int wave, const WLane<J>& ln, f32x16 (&acc)[2][J]) {
     DFrag<J> f0, f1;
     constexpr int PER = 4 + 2 * J;
@@ -380,7 +397,7 @@ __device__ __forceinline__ void main_loopW(const Stages& st, int K, int wave, co
         stage_barrier<2 * PER + 2 * J>();
         load_fragsW<LIVE, J>(st.T0, st.W0, ln, 0, f0);
 #define KSTEP(X, Y, AA, DT, DW, VM, LAST, TAIL, s)                                                                          \
-    k_stepW<E, LIVE, SLOT_LANE, J, DT, DW, (VM) * PER, LAST, TAIL>(st.T##X, st.W##X, st.T##Y, st.W##Y, st.T##AA,           \
+    k_stepW<E, LIVE, SLOT_LANE, J, DT, DW, (VM) * PER, LAST, TAIL, STREAM>(st.T##X, st.W##X, st.T##Y, st.W##Y, st.T##AA,           \
                                                                 (int64_t)((s) + 3) * kStepBytesW, (int64_t)((s) + 4) * kStepBytesW, \
                                                                 wave, ln, f0, f1, acc, K - ((s) + 3) * BKW, K - ((s) + 4) * BKW)
         int s = 0;
@@ -405,7 +422,7 @@ __device__ __forceinline__ void main_loopW(const Stages& st, int K, int wave, co
         stage_barrier<PER + 2 * J>();
         load_fragsW<LIVE, J>(st.T0, st.W0, ln, 0, f0);
 #define KSTEP(X, Y, AA, DT, DW, VM, LAST, TAIL, s)                                                                          \
-    k_stepW<E, LIVE, SLOT_LANE, J, DT, DW, VM, LAST, TAIL>(st.T##X, st.W##X, st.T##Y, st.W##Y, st.T##AA,                   \
+    k_stepW<E, LIVE, SLOT_LANE, J, DT, DW, VM, LAST, TAIL, STREAM>(st.T##X, st.W##X, st.T##Y, st.W##Y, st.T##AA,                   \
                                                         (int64_t)((s) + 2) * kStepBytesW, (int64_t)((s) + 3) * kStepBytesW, \
                                                         wave, ln, f0, f1, acc, K - ((s) + 2) * BKW, K - ((s) + 3) * BKW)
         int s = 0;
@@ -622,10 +639,12 @@ __device__ __forceinline__ void epilogue(const DenseArgs& a, const f32x16 (&acc)
 // stride.  A tile's stores, and the next tile's ring fill right behind them, are in flight while nothing else of the
 // workgroup is: the next tile's K walk starts as soon as its first stage has landed, and what a tile needs to know
 // (expert, token ids) is requested one tile ahead.
-// WIDE: stages of 64 k (16-bit operands only): twice the LDS, one workgroup per CU.
-template <typename E, int MODE, int J, bool A8 = false, bool WIDE = false>
+// WIDE: stages of 64 k (16-bit operands only): twice the LDS, one workgroup per CU; STREAM: their weight transfers are
+// non-temporal.
+template <typename E, int MODE, int J, bool A8 = false, bool WIDE = false, bool STREAM = false>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(WIDE ? 1 : 2, WIDE ? 1 : 2))) void moe_dense_kernel(const DenseArgs a, int n_blocks) {
     static_assert(!(WIDE && A8), "fp8 stages are 64 k already");
+    static_assert(WIDE || !STREAM, "only whole lines are streamed");
     constexpr int ES = A8 ? 1 : 2;          // bytes per operand element
     constexpr int EPC = 16 / ES;            // elements per 16-byte chunk
     constexpr int kStageT = WIDE ? kStageTW : kStage;               // elements of a token stage
@@ -816,7 +835,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(WIDE ? 1 : 
     int nxt = cur + nslot;
     bool have_next = nxt < hi;
     if (have_next) mn = load_meta(nxt);
-    if constexpr (WIDE) ring_fillW<J>(st, wave, ln);
+    if constexpr (WIDE) ring_fillW<J, STREAM>(st, wave, ln);
     else ring_fill<J>(st, wave, ln);
     for (;;) {
         f32x16 acc[2][J];
@@ -830,9 +849,9 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(WIDE ? 1 : 
             else if (nlive == 1) main_loop8<1, SL, J>(st, a.K, wave, ln, acc);
             else main_loop8<0, SL, J>(st, a.K, wave, ln, acc);
         } else if constexpr (WIDE) {
-            if (nlive == 2) main_loopW<E, 2, SL, J>(st, a.K, wave, ln, acc);
-            else if (nlive == 1) main_loopW<E, 1, SL, J>(st, a.K, wave, ln, acc);
-            else main_loopW<E, 0, SL, J>(st, a.K, wave, ln, acc);
+            if (nlive == 2) main_loopW<E, 2, SL, J, STREAM>(st, a.K, wave, ln, acc);
+            else if (nlive == 1) main_loopW<E, 1, SL, J, STREAM>(st, a.K, wave, ln, acc);
+            else main_loopW<E, 0, SL, J, STREAM>(st, a.K, wave, ln, acc);
         } else {
             if (nlive == 2) main_loop<E, 2, SL, J>(st, a.K, wave, ln, acc);
             else if (nlive == 1) main_loop<E, 1, SL, J>(st, a.K, wave, ln, acc);
@@ -856,7 +875,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(WIDE ? 1 : 
         nxt += nslot;
         have_next = nxt < hi;
         if (have_next) mn = load_meta(nxt);
-        if constexpr (WIDE) ring_fillW<J>(st, wave, ln);
+        if constexpr (WIDE) ring_fillW<J, STREAM>(st, wave, ln);
         else ring_fill<J>(st, wave, ln);
     }
 }
@@ -915,20 +934,37 @@ void dense_launch(const DenseArgs& a, hipStream_t s) {
     const int n_blocks = a.silu ? (int)cld((int64_t)a.N / 2, (int64_t)(32 * J)) : (int)cld((int64_t)a.N, (int64_t)(64 * J));
     const int64_t tiles = (int64_t)a.num_blocks * (a.TILE_M / kRows) * n_blocks;
     // persistent: two workgroups per CU at most (64 or 72 KB of LDS each), a multiple of 8 so that every XCD gets as many
-    // Stages of 64 k (one workgroup per CU): MI_MOE_DENSE_WIDE = 0 | 1 forces the choice.
+    // Stages of 64 k (one workgroup per CU) with non-temporal weight transfers, for launches in which no weight line is
+    // read twice: at most one block per expert.  Measured (us, kernel by kernel and the whole call): 256 tokens top-8 of
+    // 32 experts gate / up 60.6 -> 57-59, down 41.8 -> 34-35, cutile_moe 116.5 -> 106.2 (the same with four rotating
+    // sets of weights).  With two blocks per expert the streamed weights cost 5-10 % instead, and the wide stages with
+    // ordinary transfers gain 3-8 % on the 128-channel tile by the kernels' own durations but lose as much over the
+    // whole call (4096 tokens top-2 231 -> 240, 1024 tokens top-8 215 -> 227): one workgroup per CU starts and ends
+    // a launch more slowly than two.  MI_MOE_DENSE_WIDE = 0 | 1 and MI_MOE_DENSE_STREAM = 0 | 1 (wide stages only) force
+    // the choices.
     const char* env_wide = getenv("MI_MOE_DENSE_WIDE");
-    const bool wide = !a.a8 && a.K >= 512 && (env_wide ? atoi(env_wide) != 0 : false);
+    const char* env_stream = getenv("MI_MOE_DENSE_STREAM");
+    const bool can_wide = !a.a8 && a.K >= 512;
+    // (one block per expert: on average at most 0.8 of a block's slots; weights that would not stay in a cache anyway)
+    const bool one_block = (int64_t)a.total_tokens * 10 <= (int64_t)8 * kRows * a.num_experts;
+    const bool big_weights = (int64_t)a.num_experts * a.N * a.K * 2 >= (64ll << 20);
+    bool stream_w = can_wide && (env_stream ? atoi(env_stream) != 0 : one_block && big_weights);
+    const bool wide = can_wide && (env_wide ? atoi(env_wide) != 0 : stream_w);
+    if (!wide) stream_w = false;
     const int64_t cap = wide ? 32 : 64;
     const int64_t per_xcd = cld(tiles, (int64_t)8) < cap ? cld(tiles, (int64_t)8) : cap;
     const dim3 grid((unsigned)(per_xcd * 8));
-#define LAUNCH1(ET, MODE, JJ, A8, WD) hipLaunchKernelGGL((moe_dense_kernel<ET, MODE, JJ, A8, WD>), grid, dim3(256), 0, s, a, n_blocks)
-#define LAUNCH(ET, MODE)                                              \
-    do {                                                              \
-        if (a.a8) LAUNCH1(ET, MODE, 2, true, false);                  \
-        else if (wide && J == 4) LAUNCH1(ET, MODE, 4, false, true);   \
-        else if (wide) LAUNCH1(ET, MODE, 2, false, true);             \
-        else if (J == 4) LAUNCH1(ET, MODE, 4, false, false);          \
-        else LAUNCH1(ET, MODE, 2, false, false);                      \
+#define LAUNCH1(ET, MODE, JJ, A8, WD, ST) \
+    hipLaunchKernelGGL((moe_dense_kernel<ET, MODE, JJ, A8, WD, ST>), grid, dim3(256), 0, s, a, n_blocks)
+#define LAUNCH(ET, MODE)                                                           \
+    do {                                                                           \
+        if (a.a8) LAUNCH1(ET, MODE, 2, true, false, false);                        \
+        else if (wide && stream_w && J == 4) LAUNCH1(ET, MODE, 4, false, true, true);   \
+        else if (wide && stream_w) LAUNCH1(ET, MODE, 2, false, true, true);        \
+        else if (wide && J == 4) LAUNCH1(ET, MODE, 4, false, true, false);         \
+        else if (wide) LAUNCH1(ET, MODE, 2, false, true, false);                   \
+        else if (J == 4) LAUNCH1(ET, MODE, 4, false, false, false);                \
+        else LAUNCH1(ET, MODE, 2, false, false, false);                            \
     } while (0)
     if (a.silu) {
         if (a.bf16) LAUNCH(BF16, MODE_SILU);

@@ -562,7 +562,7 @@ def _every_path(d, tile_m, **kw):
     dict(num_tokens=2048, hidden_size=256, num_experts=256, intermediate_size=64, topk=8),
     dict(num_tokens=400, hidden_size=512, num_experts=4, intermediate_size=256, topk=2, T=torch.bfloat16),
 ])
-@pytest.mark.parametrize("J", ["2", "4", "2wide", "4wide"])
+@pytest.mark.parametrize("J", ["2", "4", "2wide", "4wide", "2wide_nt", "4wide_nt"])
 def test_dense_routing_ring_kernel_gives_the_streaming_kernels_bits(ct, orc, shape, J, monkeypatch):
     """The grouped GEMM for dense routing (128-slot x 128-channel tiles fed by a ring of LDS stages, persistent
     workgroups) against the streaming kernels on the same launches: every output element is accumulated over k in
@@ -572,8 +572,10 @@ def test_dense_routing_ring_kernel_gives_the_streaming_kernels_bits(ct, orc, sha
     per token, 160 and 256 experts, bf16.  Both tile widths of the ring kernel: 128 weight rows on a ring of four stages
     (J = 2) and 256 rows on a ring of three (J = 4, whose K walk is padded to whole groups of three steps); and both
     again with stages of 64 k (whole 128-byte lines per row and transfer; from K = 512 on), forced on for every launch
-    of the "wide" cases and off for the others."""
-    wide = J.endswith("wide")
+    of the "wide" cases and off for the others; "_nt": their weight transfers non-temporal, as for launches with one
+    block per expert (forced on for every launch; off for "wide")."""
+    wide = "wide" in J
+    monkeypatch.setenv("MI_MOE_DENSE_STREAM", "1" if J.endswith("_nt") else "0")
     J = J[0]
     monkeypatch.setenv("MI_MOE_DENSE_J", J)
     monkeypatch.setenv("MI_MOE_DENSE_WIDE", "1" if wide else "0")

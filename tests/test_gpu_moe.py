@@ -561,6 +561,9 @@ def _every_path(d, tile_m, **kw):
     dict(num_tokens=1024, hidden_size=256, num_experts=160, intermediate_size=128, topk=8),
     dict(num_tokens=2048, hidden_size=256, num_experts=256, intermediate_size=64, topk=8),
     dict(num_tokens=400, hidden_size=512, num_experts=4, intermediate_size=256, topk=2, T=torch.bfloat16),
+    # K of both projections from 512 on and off the grid of the 64-k stages (chunks past K in the last groups of steps)
+    dict(num_tokens=300, hidden_size=520, num_experts=3, intermediate_size=776, topk=2),
+    dict(num_tokens=96, hidden_size=1000, num_experts=4, intermediate_size=584, topk=2, T=torch.bfloat16),
 ])
 @pytest.mark.parametrize("J", ["2", "4", "2wide", "4wide", "2wide_nt", "4wide_nt"])
 def test_dense_routing_ring_kernel_gives_the_streaming_kernels_bits(ct, orc, shape, J, monkeypatch):

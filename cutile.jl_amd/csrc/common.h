@@ -13,6 +13,7 @@ namespace mi {
 
 // Host-side record of which kernel variant the last launch on this thread picked.
 void set_variant(const char* name);
+const char* last_variant_name();   // what the calling thread's last launch set
 // True once the caller has promised (mi_scratch_under_capture) that replays of its graphs neither overlap one another
 // nor other use of the library's shared static arrays on the device: capturing streams are then given those arrays.
 bool scratch_under_capture();

@@ -30,7 +30,10 @@
 // The (tm, tn, tk) tile constants of the reference only fix the block->data mapping and
 // the L2 swizzle; results do not depend on them, and the physical tiling above is chosen
 // for CDNA4.  FLOP count: 2*M*N*K per batch.
+#include <cstdio>
+
 #include "gemm_common.h"
+#include "gemm_direct.h"
 
 namespace {
 
@@ -395,8 +398,75 @@ void launch_generic16(const Problem& p, hipStream_t s) {
                        p.ldb, p.sb, (OutT*)p.C, p.ldc, p.sc, p.M, p.N, p.K, tiles_m, tiles_m * tiles_n);
 }
 
-int run(const Problem& p, hipStream_t s) {
+int run(const Problem& p, hipStream_t s, bool may_split = true);
+
+// A 16-bit product whose tiles are whole rounds of the chip plus a thin strip -- 4097 x 4096 is 16 x 16 tiles of 256 x 256
+// and one more row of sixteen, which costs a second round -- is launched as the product without its last rows and / or
+// columns plus those as one or two small products of their own (disjoint parts of C, one stream, no dependency).  The
+// estimates are the tile choice's (gemm_direct.h); a strip is at most 64 wide and is charged as a small launch.
+// Measured, f16, us: 4096 x 4128 x 4096 166 -> 131, 4160 x 4096 x 4096 165 -> 133, 4097 x 4097 x 4096 220 -> 182,
+// 4097 x 4096 x 4100 247 -> 202, 8200 x 8192 x 4096 558 -> 499 (4096^3: 125).  MI_GEMM_EDGE_SPLIT=0 switches it off.
+bool edge_split(const Problem& p, hipStream_t s, int* status) {
+    static const bool on = [] { const char* e = getenv("MI_GEMM_EDGE_SPLIT"); return !e || atoi(e) != 0; }();
+    if (!on || p.batch != 1 || p.K < 1024 || (p.in_dtype != MI_F16 && p.in_dtype != MI_BF16) || !big16_applicable(p)) return false;
+    int64_t full = 0;
+    (void)pick_direct_tile(p, &full);
+    if (full < 100) return false;   // (less than two rounds of the chip: the estimates are too coarse to split on; 2050 x 2048 x 2048 33.5 -> 39.9 us)
+    const int rM = p.M % 256, rN = p.N % 256;
+    const bool canM = rM > 0 && rM <= 64 && p.M > 512, canN = rN > 0 && rN <= 64 && p.N > 512;
+    constexpr int64_t kStrip = 8;    // a strip: a launch of a few small tiles behind the main one (measured: 6 us at K = 4096)
+    int best = 0;                    // bit 0: without the last rows, bit 1: without the last columns
+    int64_t best_cost = full;
+    for (int c = 1; c <= 3; ++c) {
+        if (((c & 1) && !canM) || ((c & 2) && !canN)) continue;
+        Problem q = p;
+        if (c & 1) q.M -= rM;
+        if (c & 2) q.N -= rN;
+        int64_t cq = 0;
+        (void)pick_direct_tile(q, &cq);
+        cq += kStrip * ((c & 1) + (c >> 1));
+        if (cq < best_cost) {
+            best_cost = cq;
+            best = c;
+        }
+    }
+    if (!best || best_cost * 20 > full * 17) return false;
+    const int64_t esz = 2, csz = p.out_dtype == MI_F32 ? 4 : 2;
+    Problem main = p;
+    if (best & 1) main.M -= rM;
+    if (best & 2) main.N -= rN;
+    int st = run(main, s, false);
+    static thread_local char name[96];
+    snprintf(name, sizeof name, "%s+edge_strips", last_variant_name());
+    if (st == MI_OK && (best & 1)) {   // rows M' .. M - 1 of every column
+        // (at least eight rows, which is what the direct-to-LDS kernel takes: a thinner strip starts inside the main part
+        // and writes those rows of C a second time, behind the main launch on the same stream)
+        const int rows = rM < 8 ? 8 : rM;
+        Problem e = p;
+        e.M = rows;
+        e.A = (const char*)p.A + (int64_t)(p.M - rows) * esz;
+        e.C = (char*)p.C + (int64_t)(p.M - rows) * csz;
+        st = run(e, s, false);
+    }
+    if (st == MI_OK && (best & 2)) {   // columns N' .. N - 1 of the rows above that strip
+        Problem e = p;
+        e.M = main.M;
+        e.N = rN;
+        e.B = (const char*)p.B + (int64_t)main.N * p.ldb * esz;
+        e.C = (char*)p.C + (int64_t)main.N * p.ldc * csz;
+        st = run(e, s, false);
+    }
+    set_variant(name);
+    *status = st;
+    return true;
+}
+
+int run(const Problem& p, hipStream_t s, bool may_split) {
     if (p.M == 0 || p.N == 0 || p.batch == 0) return MI_OK;
+    if (may_split) {
+        int st = MI_OK;
+        if (edge_split(p, s, &st)) return st;
+    }
     static const int force = [] { const char* e = getenv("MI_GEMM_KERNEL"); return e ? atoi(e) : 0; }();   // 1 generic, 2 mid, 3 big
     if (p.in_dtype == MI_F8E4M3FN || p.in_dtype == MI_F8E5M2) {
         fp8_launch(p, s);

@@ -40,13 +40,16 @@ inline int64_t tiles_of(const Problem& p, int btm, int btn) {
 // drops); 256x128 0.42 to 0.51; 128x128 0.33 with one workgroup per CU, 0.58 when CUs hold two.
 // f16 examples (us, 256x256 / 256x128 / 128x128): 1024^3 23 / 15 / 10, 2048^3 40 / 27 / 21,
 // 2560^3 51 / 37 / 46, 4096 x 2048 x 4096 77 / 65 / 74, 3072^3 64 / 83 / 77, 4096^3 119 / 128 / 144.
-inline int pick_direct_tile(const Problem& p) {
+// `cost` (optional): the estimate for the tile chosen, in units of about 1 % of the 4096^3 product's time per 4096 of K.
+inline int pick_direct_tile(const Problem& p, int64_t* cost = nullptr) {
     static const int force = [] { const char* e = getenv("MI_GEMM_BIG_TILE"); return e ? atoi(e) : 0; }();   // 44, 42 or 22
-    if (force == 44 || force == 42 || force == 22) return force;
     const int64_t t44 = tiles_of(p, 256, 256), t42 = tiles_of(p, 256, 128), t22 = tiles_of(p, 128, 128);
     const int64_t c44 = (t44 + 255) / 256 * 90, c42 = (t42 + 255) / 256 * 50;
     const int64_t c22 = t22 <= 256 ? 33 : (t22 + 511) / 512 * 60;
-    return c22 <= c42 && c22 <= c44 ? 22 : c42 <= c44 ? 42 : 44;
+    const int t = c22 <= c42 && c22 <= c44 ? 22 : c42 <= c44 ? 42 : 44;
+    if (cost) *cost = t == 22 ? c22 : t == 42 ? c42 : c44;
+    if (force == 44 || force == 42 || force == 22) return force;
+    return t;
 }
 
 }  // namespace gemm

@@ -12,6 +12,7 @@
 namespace mi {
 static thread_local const char* g_variant = "";
 void set_variant(const char* name) { g_variant = name; }
+const char* last_variant_name() { return g_variant; }
 
 static std::atomic<int> g_scratch_under_capture{[] {
     const char* e = getenv("MI_SCRATCH_UNDER_CAPTURE");

@@ -138,6 +138,33 @@ def test_matmul_large_tile_kernel_takes_misaligned_rows_and_ragged_sizes(ct, orc
     assert bool((buf[N:] == -77.0).all()) and bool((buf[:, M:] == -77.0).all())
 
 
+@pytest.mark.parametrize("M,N,K,T,out32,pad", [
+    (4097, 4096, 1024, torch.float16, True, (0, 0)),      # one row more than 16 x 16 tiles: the strip starts inside the main part
+    (4096, 4100, 1032, torch.float16, False, (0, 0)),     # four columns more
+    (4100, 4130, 1024, torch.bfloat16, True, (3, 1)),     # both, in parents with odd leading dimensions
+    (4160, 4096, 1027, torch.float16, True, (0, 0)),      # 64 rows more, K off the chunks of 8
+])
+def test_matmul_whole_rounds_plus_a_thin_strip_are_launched_apart(ct, orc, M, N, K, T, out32, pad):
+    """A product whose 256 x 256 tiles are whole rounds of the 256 CUs plus a strip of at most 64 rows or columns goes out
+    as the product without the strip(s) and the strip(s) as small products of their own.  Exact integer sums; operands
+    and C are views with NaN / a sentinel behind every row, as in the test above."""
+    rng = np.random.default_rng(M + N)
+    A = rng.integers(-1, 2, (M, K)).astype(np.float32); B = rng.integers(-2, 3, (K, N)).astype(np.float32)
+    lda, ldb = M + pad[0], K + pad[1]
+    Aflat = torch.full((K * lda + 16,), float("nan"), dtype=T, device="cuda")
+    Bflat = torch.full((N * ldb + 16,), float("nan"), dtype=T, device="cuda")
+    Av = Aflat[:K * lda].view(K, lda)[:, :M]; Bv = Bflat[:N * ldb].view(N, ldb)[:, :K]
+    Av.copy_(orc.from_julia(A).to(T)); Bv.copy_(orc.from_julia(B).to(T))
+    buf = torch.full((N + 2, M + 9), -77.0, dtype=torch.float32 if out32 else T, device="cuda")
+    C = buf[:N, :M]
+    ct.matmul_kernel(Av, Bv, C, 64, 64, 64)
+    assert ct.last_variant() == "gemm16_big_256x256x32_ring4+edge_strips", ct.last_variant()
+    ref = A @ B
+    assert out32 or np.abs(ref).max() <= 2048
+    assert np.array_equal(orc.to_julia(C.contiguous()).astype(np.float32), ref)
+    assert bool((buf[N:] == -77.0).all()) and bool((buf[:, M:] == -77.0).all())
+
+
 def test_batch_matmul_large_tile_kernel_ragged(ct, orc):
     """The same through mi_batch_matmul_kernel: three dense 1023 x 1030 x 515 products."""
     rng = np.random.default_rng(11)

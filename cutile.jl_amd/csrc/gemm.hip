@@ -403,18 +403,25 @@ int run(const Problem& p, hipStream_t s, bool may_split = true);
 // A 16-bit product whose tiles are whole rounds of the chip plus a thin strip -- 4097 x 4096 is 16 x 16 tiles of 256 x 256
 // and one more row of sixteen, which costs a second round -- is launched as the product without its last rows and / or
 // columns plus those as one or two small products of their own (disjoint parts of C, one stream, no dependency).  The
-// estimates are the tile choice's (gemm_direct.h); a strip is at most 64 wide and is charged as a small launch.
+// estimates are the tile choice's (gemm_direct.h); a strip is the last tile row / column of 256 or what there is of it.
 // Measured, f16, us: 4096 x 4128 x 4096 166 -> 131, 4160 x 4096 x 4096 165 -> 133, 4097 x 4097 x 4096 220 -> 182,
-// 4097 x 4096 x 4100 247 -> 202, 8200 x 8192 x 4096 558 -> 499 (4096^3: 125).  MI_GEMM_EDGE_SPLIT=0 switches it off.
+// 4097 x 4096 x 4100 247 -> 202, 8200 x 8192 x 4096 558 -> 499, 4352 x 4096 x 4096 165 -> 137, 4096 x 8448 x 4096
+// 287 -> 248 (4096^3: 123).
+// MI_GEMM_EDGE_SPLIT=0 switches it off.
 bool edge_split(const Problem& p, hipStream_t s, int* status) {
     static const bool on = [] { const char* e = getenv("MI_GEMM_EDGE_SPLIT"); return !e || atoi(e) != 0; }();
     if (!on || p.batch != 1 || p.K < 1024 || (p.in_dtype != MI_F16 && p.in_dtype != MI_BF16) || !big16_applicable(p)) return false;
     int64_t full = 0;
     (void)pick_direct_tile(p, &full);
     if (full < 100) return false;   // (less than two rounds of the chip: the estimates are too coarse to split on; 2050 x 2048 x 2048 33.5 -> 39.9 us)
-    const int rM = p.M % 256, rN = p.N % 256;
-    const bool canM = rM > 0 && rM <= 64 && p.M > 512, canN = rN > 0 && rN <= 64 && p.N > 512;
-    constexpr int64_t kStrip = 8;    // a strip: a launch of a few small tiles behind the main one (measured: 6 us at K = 4096)
+    // the last tile row / column of 256, whole or not
+    const int rM = p.M % 256 ? p.M % 256 : 256, rN = p.N % 256 ? p.N % 256 : 256;
+    const bool canM = p.M >= 768, canN = p.N >= 768;
+    // A strip by itself, in the estimates' units, which stand for 1.37 us x K / 4096: its two launches (split over K)
+    // are about 10 us whatever K is, the rest goes with its size (measured at K = 4096, us: 8 ... 64 x 4096 13-14,
+    // 256 x 4096 19, 256 x 8192 31).
+    const int64_t K = p.K;
+    auto strip = [K](int64_t r, int64_t other) { return 30000 / K + r * other * 7 / (256 * 4096); };
     int best = 0;                    // bit 0: without the last rows, bit 1: without the last columns
     int64_t best_cost = full;
     for (int c = 1; c <= 3; ++c) {
@@ -424,13 +431,14 @@ bool edge_split(const Problem& p, hipStream_t s, int* status) {
         if (c & 2) q.N -= rN;
         int64_t cq = 0;
         (void)pick_direct_tile(q, &cq);
-        cq += kStrip * ((c & 1) + (c >> 1));
+        if (c & 1) cq += strip(rM, p.N);
+        if (c & 2) cq += strip(rN, q.M);
         if (cq < best_cost) {
             best_cost = cq;
             best = c;
         }
     }
-    if (!best || best_cost * 20 > full * 17) return false;
+    if (!best || best_cost * 10 > full * 9) return false;
     const int64_t esz = 2, csz = p.out_dtype == MI_F32 ? 4 : 2;
     Problem main = p;
     if (best & 1) main.M -= rM;

@@ -141,13 +141,14 @@ def test_matmul_large_tile_kernel_takes_misaligned_rows_and_ragged_sizes(ct, orc
 @pytest.mark.parametrize("M,N,K,T,out32,pad", [
     (4097, 4096, 1024, torch.float16, True, (0, 0)),      # one row more than 16 x 16 tiles: the strip starts inside the main part
     (4096, 4100, 1032, torch.float16, False, (0, 0)),     # four columns more
-    (4100, 4130, 1024, torch.bfloat16, True, (3, 1)),     # both, in parents with odd leading dimensions
+    (4100, 4130, 2048, torch.bfloat16, True, (3, 1)),     # both, in parents with odd leading dimensions
     (4160, 4096, 1027, torch.float16, True, (0, 0)),      # 64 rows more, K off the chunks of 8
 ])
 def test_matmul_whole_rounds_plus_a_thin_strip_are_launched_apart(ct, orc, M, N, K, T, out32, pad):
-    """A product whose 256 x 256 tiles are whole rounds of the 256 CUs plus a strip of at most 64 rows or columns goes out
-    as the product without the strip(s) and the strip(s) as small products of their own.  Exact integer sums; operands
-    and C are views with NaN / a sentinel behind every row, as in the test above."""
+    """A product whose 256 x 256 tiles are whole rounds of the 256 CUs plus a last row or column of tiles goes out as the
+    product without that strip (or both) and the strip(s) as small products of their own, where the estimates say that
+    saves a round.  Exact integer sums; operands and C are views with NaN / a sentinel behind every row, as in the
+    test above."""
     rng = np.random.default_rng(M + N)
     A = rng.integers(-1, 2, (M, K)).astype(np.float32); B = rng.integers(-2, 3, (K, N)).astype(np.float32)
     lda, ldb = M + pad[0], K + pad[1]

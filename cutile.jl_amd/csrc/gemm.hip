@@ -400,68 +400,88 @@ void launch_generic16(const Problem& p, hipStream_t s) {
 
 int run(const Problem& p, hipStream_t s, bool may_split = true);
 
-// A 16-bit product whose tiles are whole rounds of the chip plus a thin strip -- 4097 x 4096 is 16 x 16 tiles of 256 x 256
-// and one more row of sixteen, which costs a second round -- is launched as the product without its last rows and / or
-// columns plus those as one or two small products of their own (disjoint parts of C, one stream, no dependency).  The
-// estimates are the tile choice's (gemm_direct.h); a strip is the last tile row / column of 256 or what there is of it.
-// Measured, f16, us: 4096 x 4128 x 4096 166 -> 131, 4160 x 4096 x 4096 165 -> 133, 4097 x 4097 x 4096 220 -> 182,
-// 4097 x 4096 x 4100 247 -> 202, 8200 x 8192 x 4096 558 -> 499, 4352 x 4096 x 4096 165 -> 137, 4096 x 8448 x 4096
-// 287 -> 248 (4096^3: 123).
-// MI_GEMM_EDGE_SPLIT=0 switches it off.
+// A 16-bit or fp32 product whose tiles are whole rounds of the chip plus a thin strip -- 4097 x 4096 is 16 x 16 tiles of
+// 256 x 256 and one more row of sixteen, which costs a second round -- is launched as the product without its last row
+// and / or column of tiles plus those as one or two small products of their own (disjoint parts of C, one stream, no
+// dependency).  Estimates in us, from what was measured at 4096^3 and scaled with K: the tile choices' own figures for
+// the whole and the main part, a strip as its launches plus its K walk.  A split has to promise 10 %.  Measured (us,
+// K = 4096 unless given):
+//   f16   4096 x 4128 166 -> 131, 4352 x 4096 165 -> 137, 4097 x 4097 220 -> 182, 4097 x 4096 x 4100 247 -> 202,
+//         4096 x 8448 287 -> 248, 8200 x 8192 558 -> 499 (4096^3: 123); left alone: 4400 x 4096 x 1024 (56; 66 split)
+//   f32   4097 x 4096 1287 -> 1071, 4352 x 4096 1284 -> 1051, 4096 x 4100 x 2048 640 -> 504 (4096^3: 954)
+// Not for fp8, where a second, nearly empty round costs little (4352 x 4096 92 against 59 + 36), and not to take rows
+// off an M that is not a multiple of a chunk: what slows those products is the leading dimension, which a part keeps
+// (f16 4095 x 4096 166 -> 174, e4m3 4100 x 4100 144 -> 169).  MI_GEMM_EDGE_SPLIT=0 switches it off.
 bool edge_split(const Problem& p, hipStream_t s, int* status) {
     static const bool on = [] { const char* e = getenv("MI_GEMM_EDGE_SPLIT"); return !e || atoi(e) != 0; }();
-    if (!on || p.batch != 1 || p.K < 1024 || (p.in_dtype != MI_F16 && p.in_dtype != MI_BF16) || !big16_applicable(p)) return false;
-    int64_t full = 0;
-    (void)pick_direct_tile(p, &full);
-    if (full < 100) return false;   // (less than two rounds of the chip: the estimates are too coarse to split on; 2050 x 2048 x 2048 33.5 -> 39.9 us)
-    // the last tile row / column of 256, whole or not
-    const int rM = p.M % 256 ? p.M % 256 : 256, rN = p.N % 256 ? p.N % 256 : 256;
-    const bool canM = p.M >= 768, canN = p.N >= 768;
-    // A strip by itself, in the estimates' units, which stand for 1.37 us x K / 4096: its two launches (split over K)
-    // are about 10 us whatever K is, the rest goes with its size (measured at K = 4096, us: 8 ... 64 x 4096 13-14,
-    // 256 x 4096 19, 256 x 8192 31).
-    const int64_t K = p.K;
-    auto strip = [K](int64_t r, int64_t other) { return 30000 / K + r * other * 7 / (256 * 4096); };
-    int best = 0;                    // bit 0: without the last rows, bit 1: without the last columns
-    int64_t best_cost = full;
-    for (int c = 1; c <= 3; ++c) {
-        if (((c & 1) && !canM) || ((c & 2) && !canN)) continue;
-        Problem q = p;
-        if (c & 1) q.M -= rM;
-        if (c & 2) q.N -= rN;
-        int64_t cq = 0;
-        (void)pick_direct_tile(q, &cq);
-        if (c & 1) cq += strip(rM, p.N);
-        if (c & 2) cq += strip(rN, q.M);
-        if (cq < best_cost) {
-            best_cost = cq;
-            best = c;
+    if (!on || p.batch != 1 || p.K < 1024 || p.M < 512 || p.N < 512) return false;
+    const bool f16 = p.in_dtype == MI_F16 || p.in_dtype == MI_BF16, f32 = p.in_dtype == MI_F32;
+    if (f16 ? !big16_applicable(p) : f32 ? !big32_applicable(p) : true) return false;
+    const double ks = p.K / 4096.0;
+    const int align = f16 ? 8 : 4;   // rows of A per 16-byte chunk
+    // the whole product or a main part (us)
+    auto whole = [&](const Problem& q) {
+        if (f16) {
+            int64_t c = 0;
+            (void)pick_direct_tile(q, &c);
+            return c * 1.37 * ks;
         }
-    }
-    if (!best || best_cost * 10 > full * 9) return false;
-    const int64_t esz = 2, csz = p.out_dtype == MI_F32 ? 4 : 2;
+        return big32_cost(q) * 59.0 * ks;
+    };
+    // a strip of r rows or columns by itself (us): f16 splits it over K (two launches, 10 us) unless K is off the chunks;
+    // f32 walks K in one launch of small tiles
+    auto strip = [&](int64_t r, int64_t other) {
+        if (f16) return p.K % 8 ? 6.0 + 22.0 * ks : 10.0 + 9.5 * ks * (double)(r * other) / (256.0 * 4096.0);
+        return 4.0 + 62.0 * ks * (other > 8192 ? other / 8192.0 : 1.0);
+    };
+    const double full = whole(p);
+    if (full < (f16 ? 137.0 : 1100.0) * ks) return false;   // (less than about two rounds: the estimates are too coarse)
+    const int rM = p.M % 256 ? p.M % 256 : 256, rN = p.N % 256 ? p.N % 256 : 256;
+    // candidates: rows kept = all | up to the last tile row; columns kept = all | up to the last tile column
+    const int keepM[2] = {p.M, p.M >= 768 ? p.M - rM : p.M};
+    const int keepN[2] = {p.N, p.N >= 768 ? p.N - rN : p.N};
+    int bm = p.M, bn = p.N;
+    double best = full;
+    for (int i = 0; i < 2; ++i)
+        for (int j = 0; j < 2; ++j) {
+            const int m = keepM[i], n = keepN[j];
+            if ((m == p.M && n == p.N) || m < 512 || n < 256) continue;
+            Problem q = p;
+            q.M = m;
+            q.N = n;
+            double t = whole(q);
+            if (m < p.M) t += strip(p.M - m, p.N);
+            if (n < p.N) t += strip(p.N - n, m);
+            if (t < best) {
+                best = t;
+                bm = m;
+                bn = n;
+            }
+        }
+    if (best > 0.9 * full) return false;
+    const int64_t esz = f32 ? 4 : 2, csz = p.out_dtype == MI_F32 ? 4 : 2;
     Problem main = p;
-    if (best & 1) main.M -= rM;
-    if (best & 2) main.N -= rN;
+    main.M = bm;
+    main.N = bn;
     int st = run(main, s, false);
     static thread_local char name[96];
     snprintf(name, sizeof name, "%s+edge_strips", last_variant_name());
-    if (st == MI_OK && (best & 1)) {   // rows M' .. M - 1 of every column
-        // (at least eight rows, which is what the direct-to-LDS kernel takes: a thinner strip starts inside the main part
-        // and writes those rows of C a second time, behind the main launch on the same stream)
-        const int rows = rM < 8 ? 8 : rM;
+    if (st == MI_OK && bm < p.M) {   // rows M' .. M - 1 of every column
+        // (at least a chunk of rows, which is what the direct-to-LDS kernels take: a thinner strip starts inside the main
+        // part and writes those rows of C a second time, behind the main launch on the same stream)
+        const int rows = p.M - bm < align ? align : p.M - bm;
         Problem e = p;
         e.M = rows;
         e.A = (const char*)p.A + (int64_t)(p.M - rows) * esz;
         e.C = (char*)p.C + (int64_t)(p.M - rows) * csz;
         st = run(e, s, false);
     }
-    if (st == MI_OK && (best & 2)) {   // columns N' .. N - 1 of the rows above that strip
+    if (st == MI_OK && bn < p.N) {   // columns N' .. N - 1 of the rows above that strip
         Problem e = p;
-        e.M = main.M;
-        e.N = rN;
-        e.B = (const char*)p.B + (int64_t)main.N * p.ldb * esz;
-        e.C = (char*)p.C + (int64_t)main.N * p.ldc * csz;
+        e.M = bm;
+        e.N = p.N - bn;
+        e.B = (const char*)p.B + (int64_t)bn * p.ldb * esz;
+        e.C = (char*)p.C + (int64_t)bn * p.ldc * csz;
         st = run(e, s, false);
     }
     set_variant(name);

@@ -332,14 +332,22 @@ bool big32_applicable(const Problem& p) {
 // x (MFMAs per wave and step, I*J); co-resident workgroups of the small tiles simply add up.  The
 // smallest tile moves four times the bytes per flop of 128x128 through L2, so it is only taken when it
 // at least halves that cost (1024^3: 64 tiles of 128x128 take 63 us).  Ties go to the larger tile.
-int pick_tile32(const Problem& p) {
+int pick_tile32(const Problem& p, int64_t* cost = nullptr) {
     static const int force = [] { const char* e = getenv("MI_GEMM_BIG_TILE"); return e ? atoi(e) : 0; }();   // 44, 42, 22 or 11
-    if (force == 44 || force == 42 || force == 22 || force == 11) return force;
     auto rounds = [&](int btm, int btn) { return (tiles_of(p, btm, btn) + 255) / 256; };
     const int64_t c44 = rounds(256, 256) * 16, c42 = rounds(256, 128) * 8, c22 = rounds(128, 128) * 4, c11 = rounds(64, 64);
     const int64_t best = c44 <= c42 && c44 <= c22 ? c44 : c42 <= c22 ? c42 : c22;
+    if (cost) *cost = 2 * c11 <= best ? 2 * c11 : best;
+    if (force == 44 || force == 42 || force == 22 || force == 11) return force;
     if (2 * c11 <= best) return 11;
     return best == c44 ? 44 : best == c42 ? 42 : 22;
+}
+
+// The tile choice's estimate: 16 per round of 256 x 256 tiles (the 4096^3 product).
+int64_t big32_cost(const Problem& p) {
+    int64_t c = 0;
+    (void)pick_tile32(p, &c);
+    return c;
 }
 
 void big32_launch(const Problem& p, hipStream_t s) {

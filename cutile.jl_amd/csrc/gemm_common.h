@@ -80,6 +80,7 @@ void big16_launch(const Problem& p, hipStream_t s);
 // gemm32_big.hip: the same for fp32 operands.
 bool big32_applicable(const Problem& p);
 void big32_launch(const Problem& p, hipStream_t s);
+int64_t big32_cost(const Problem& p);   // its tile choice's estimate, 16 = the 4096^3 product per 4096 of K
 // gemm8.hip: fp8 (E4M3FN / E5M2) operands; picks its kernel itself.
 void fp8_launch(const Problem& p, hipStream_t s);
 

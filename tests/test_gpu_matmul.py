@@ -143,6 +143,8 @@ def test_matmul_large_tile_kernel_takes_misaligned_rows_and_ragged_sizes(ct, orc
     (4096, 4100, 1032, torch.float16, False, (0, 0)),     # four columns more
     (4100, 4130, 2048, torch.bfloat16, True, (3, 1)),     # both, in parents with odd leading dimensions
     (4160, 4096, 1027, torch.float16, True, (0, 0)),      # 64 rows more, K off the chunks of 8
+    (4097, 4096, 1024, torch.float32, True, (0, 0)),      # fp32 operands: a strip of four rows, three of them written twice
+    (4096, 4352, 1030, torch.float32, True, (1, 3)),      # a whole last column of tiles
 ])
 def test_matmul_whole_rounds_plus_a_thin_strip_are_launched_apart(ct, orc, M, N, K, T, out32, pad):
     """A product whose 256 x 256 tiles are whole rounds of the 256 CUs plus a last row or column of tiles goes out as the
@@ -159,7 +161,7 @@ def test_matmul_whole_rounds_plus_a_thin_strip_are_launched_apart(ct, orc, M, N,
     buf = torch.full((N + 2, M + 9), -77.0, dtype=torch.float32 if out32 else T, device="cuda")
     C = buf[:N, :M]
     ct.matmul_kernel(Av, Bv, C, 64, 64, 64)
-    assert ct.last_variant() == "gemm16_big_256x256x32_ring4+edge_strips", ct.last_variant()
+    assert ct.last_variant() == ("gemm32_big_256x256x16_ring4" if T == torch.float32 else "gemm16_big_256x256x32_ring4") + "+edge_strips", ct.last_variant()
     ref = A @ B
     assert out32 or np.abs(ref).max() <= 2048
     assert np.array_equal(orc.to_julia(C.contiguous()).astype(np.float32), ref)

@@ -802,7 +802,7 @@ def _host_info():
 TARGETS = [("vadd", "frac", 0.75), ("layernorm_fwd", "frac_cold", 0.75), ("softmax_tma", "frac_cold", 0.75),
            ("matmul", "frac", 0.60), ("fmha", "frac", 0.40), ("moe_f16_default", "mfma_frac", 0.40)]
 REPORTED = [("copy_ref", "frac_cold"), ("copy_ref_runtime", "frac_cold"), ("transpose", "frac"), ("layernorm_bwd", "frac_cold"), ("layernorm_bwd_static", "frac_cold"),
-            ("batchmatmul", "frac"), ("matmul_fp8", "frac"), ("moe_f16_default", "frac"), ("moe_f16_top8_device_fused", "mfma_frac"), ("moe_f16_prefill", "mfma_frac"), ("moe_fp8_prefill", "mfma_frac"),
+            ("batchmatmul", "frac"), ("matmul_fp8", "frac"), ("moe_f16_default", "frac"), ("moe_f16_top8_device_fused", "frac"), ("moe_f16_top8_device_fused", "mfma_frac"), ("moe_f16_prefill", "mfma_frac"), ("moe_fp8_prefill", "mfma_frac"),
             ("moe_fp8_device", "frac_cold"), ("fmha_decode", "frac"), ("fmha_decode_16k", "frac")]
 MAX_LINE_BYTES = 4096   # the last stdout line must stay a small record: a consumer that keeps only the end of stdout still parses it
 
